@@ -1,0 +1,483 @@
+/*
+ * CPU oracle for ESP-DL's quantized operator path.  TEST INFRASTRUCTURE ONLY: see espdl_oracle.h
+ * for who may use it and for the pinning status of every function.
+ *
+ * Each function cites the reference lines it restates (paths relative to the reference tree).
+ */
+#include "espdl_oracle.h"
+
+#include <limits.h>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static int g_threads = 0; /* 0 = leave OpenMP's default */
+
+int espdl_oracle_max_threads(void)
+{
+#ifdef _OPENMP
+    return g_threads > 0 ? g_threads : omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+void espdl_oracle_set_threads(int n)
+{
+    g_threads = n;
+#ifdef _OPENMP
+    if (n > 0)
+        omp_set_num_threads(n);
+#endif
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Integer helpers.
+ * tool::truncate = clamp to the destination type (esp-dl/dl/tool/include/dl_tool.hpp:225-254).
+ * ------------------------------------------------------------------------------------------- */
+static inline int64_t clamp_i64(int64_t v, int64_t lo, int64_t hi)
+{
+    return v < lo ? lo : (v > hi ? hi : v);
+}
+
+/*
+ * tool::shift_and_round<int32_t>  (esp-dl/dl/tool/src/dl_tool.cpp:95-146).
+ * half-up:   shift > 0: (int64(v) + 2^(shift-1)) >> shift, arithmetic shift; the sum is formed in
+ *            64 bits (`half` is int64_t there) and narrowed back to T.
+ *            shift <= 0: int64(v) << -shift, saturated to T.
+ * half-even: shift > 0: q = v >> shift, r = v & (2^shift - 1) (computed in T), bump q when
+ *            r > half, or r == half and q is odd.
+ */
+int32_t espdl_oracle_shift_round_s32(int32_t value, int shift, int round_mode)
+{
+    if (shift <= 0) {
+        /* multiply instead of shifting a negative number: same value, no undefined behaviour */
+        int64_t shifted = (int64_t)value * ((int64_t)1 << -shift);
+        return (int32_t)clamp_i64(shifted, INT32_MIN, INT32_MAX);
+    }
+    if (round_mode == ESPDL_ORACLE_ROUND_HALF_EVEN) {
+        int32_t q = value >> shift;
+        int32_t rem = value & (int32_t)(((uint32_t)1 << shift) - 1u);
+        int32_t half = (int32_t)((uint32_t)1 << (shift - 1));
+        if (rem > half || (rem == half && (q & 1)))
+            q += 1;
+        return q;
+    }
+    int64_t half = (int64_t)1 << (shift - 1);
+    return (int32_t)(((int64_t)value + half) >> shift);
+}
+
+/* tool::shift_and_round<int64_t>: same text with T = int64_t (no widening is available). */
+int64_t espdl_oracle_shift_round_s64(int64_t value, int shift, int round_mode)
+{
+    if (shift <= 0) {
+        return (int64_t)((uint64_t)value << -shift); /* truncate(int64, int64) is the identity */
+    }
+    if (round_mode == ESPDL_ORACLE_ROUND_HALF_EVEN) {
+        int64_t q = value >> shift;
+        int64_t rem = value & (int64_t)(((uint64_t)1 << shift) - 1u);
+        int64_t half = (int64_t)((uint64_t)1 << (shift - 1));
+        if (rem > half || (rem == half && (q & 1)))
+            q += 1;
+        return q;
+    }
+    int64_t half = (int64_t)1 << (shift - 1);
+    return (int64_t)((uint64_t)value + (uint64_t)half) >> shift;
+}
+
+/* Conv::get_output_shape (esp-dl/dl/module/include/dl_module_conv.hpp:90-98). */
+int espdl_oracle_conv_out_h(const espdl_oracle_conv_t *g)
+{
+    return (g->in_h + g->pad_top + g->pad_bottom - g->dil_h * (g->k_h - 1) - 1) / g->stride_h + 1;
+}
+
+int espdl_oracle_conv_out_w(const espdl_oracle_conv_t *g)
+{
+    return (g->in_w + g->pad_left + g->pad_right - g->dil_w * (g->k_w - 1) - 1) / g->stride_w + 1;
+}
+
+static int geometry_ok(const espdl_oracle_conv_t *g, int depthwise)
+{
+    if (g->batch < 0 || g->in_h <= 0 || g->in_w <= 0 || g->in_c <= 0 || g->out_c <= 0)
+        return 0;
+    if (g->k_h <= 0 || g->k_w <= 0 || g->stride_h <= 0 || g->stride_w <= 0 || g->dil_h <= 0 || g->dil_w <= 0)
+        return 0;
+    if (g->pad_top < 0 || g->pad_bottom < 0 || g->pad_left < 0 || g->pad_right < 0)
+        return 0;
+    if (g->n_shift != 1 && g->n_shift != g->out_c)
+        return 0;
+    if (depthwise && g->out_c != g->in_c)
+        return 0;
+    if (g->in_h + g->pad_top + g->pad_bottom - g->dil_h * (g->k_h - 1) - 1 < 0)
+        return 0;
+    if (g->in_w + g->pad_left + g->pad_right - g->dil_w * (g->k_w - 1) - 1 < 0)
+        return 0;
+    return 1;
+}
+
+/*
+ * The reference walks output pixels and, at padded borders, shrinks the filter window to the taps
+ * that fall inside the image (esp-dl/dl/base/dl_base.hpp:951-1138; valid padding :1172-1191), so a
+ * tap outside the image contributes nothing: zero padding.  [k0, k1) below is that in-image tap
+ * range along one axis for the output coordinate `o`.
+ */
+static inline void tap_range(int o, int stride, int pad_head, int dil, int k, int in_size, int *k0, int *k1)
+{
+    int origin = o * stride - pad_head; /* input coordinate of tap 0 */
+    int lo = 0, hi = k;
+    if (origin < 0)
+        lo = (-origin + dil - 1) / dil;
+    /* last tap with origin + t*dil <= in_size - 1 */
+    if (origin + (k - 1) * dil > in_size - 1) {
+        int room = in_size - 1 - origin;
+        hi = room < 0 ? 0 : room / dil + 1;
+    }
+    if (lo > hi)
+        lo = hi;
+    *k0 = lo;
+    *k1 = hi;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Dense convolution, int8.
+ *   MAC      conv2d_11cn / conv2d_33cn / conv2d_hwcn  (esp-dl/dl/base/dl_base_conv2d.cpp:9-163):
+ *            int8 * int8 products accumulated in int32, filter [Cout][kH][kW][Cin].
+ *   epilogue buffer_bias_linear/_relu, buffer_0000_linear/_relu
+ *            (esp-dl/dl/base/dl_base_activate_buffer.hpp:27-36, 61-72, 173-181, 201-210):
+ *            acc += bias (int32) -> shift_and_round(acc, mac_shift) -> ReLU -> truncate to int8.
+ *   mac_shift = out_exp - filter_exp - in_exp (esp-dl/dl/base/dl_base.hpp:260); with a shift per
+ *            output channel the same formula is applied channel-wise.
+ * ------------------------------------------------------------------------------------------- */
+int espdl_oracle_conv2d_s8(const espdl_oracle_conv_t *g, const int8_t *in, const int8_t *filter,
+                           const int32_t *bias, const int32_t *shift, int8_t *out)
+{
+    if (!geometry_ok(g, 0))
+        return -1;
+    const int oh = espdl_oracle_conv_out_h(g), ow = espdl_oracle_conv_out_w(g);
+    const int C = g->in_c, OC = g->out_c, KH = g->k_h, KW = g->k_w;
+    const int64_t in_img = (int64_t)g->in_h * g->in_w * C;
+    const int64_t out_img = (int64_t)oh * ow * OC;
+    const int64_t rows = (int64_t)g->batch * oh;
+
+#pragma omp parallel for schedule(static)
+    for (int64_t row = 0; row < rows; row++) {
+        const int n = (int)(row / oh), oy = (int)(row % oh);
+        const int8_t *img = in + n * in_img;
+        int8_t *dst = out + n * out_img + (int64_t)oy * ow * OC;
+        int ky0, ky1;
+        tap_range(oy, g->stride_h, g->pad_top, g->dil_h, KH, g->in_h, &ky0, &ky1);
+        for (int ox = 0; ox < ow; ox++) {
+            int kx0, kx1;
+            tap_range(ox, g->stride_w, g->pad_left, g->dil_w, KW, g->in_w, &kx0, &kx1);
+            for (int oc = 0; oc < OC; oc++) {
+                const int8_t *f_oc = filter + (int64_t)oc * KH * KW * C;
+                int32_t acc = 0;
+                for (int ky = ky0; ky < ky1; ky++) {
+                    const int iy = oy * g->stride_h - g->pad_top + ky * g->dil_h;
+                    for (int kx = kx0; kx < kx1; kx++) {
+                        const int ix = ox * g->stride_w - g->pad_left + kx * g->dil_w;
+                        const int8_t *px = img + ((int64_t)iy * g->in_w + ix) * C;
+                        const int8_t *fw = f_oc + ((int64_t)ky * KW + kx) * C;
+                        int32_t s = 0;
+                        for (int c = 0; c < C; c++)
+                            s += (int32_t)px[c] * (int32_t)fw[c];
+                        acc += s;
+                    }
+                }
+                if (bias)
+                    acc = (int32_t)((uint32_t)acc + (uint32_t)bias[oc]); /* int32 += int32 */
+                int32_t v = espdl_oracle_shift_round_s32(acc, shift[g->n_shift == 1 ? 0 : oc], g->round_mode);
+                if (g->activation == ESPDL_ORACLE_RELU && v < 0)
+                    v = 0;
+                dst[(int64_t)ox * OC + oc] = (int8_t)clamp_i64(v, INT8_MIN, INT8_MAX);
+            }
+        }
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * Depthwise convolution, int8.
+ *   MAC      depthwise_conv2d_11c1 / _33c1 / _hwc1
+ *            (esp-dl/dl/base/dl_base_depthwise_conv2d.cpp:9-65): acc[c] += in[iy][ix][c] * f[ky][kx][c].
+ *   epilogue the same n_wise functions as the dense path
+ *            (esp-dl/dl/base/dl_base_depthwise_conv2d.cpp:760-805), shift indexed by channel.
+ * ------------------------------------------------------------------------------------------- */
+int espdl_oracle_depthwise_s8(const espdl_oracle_conv_t *g, const int8_t *in, const int8_t *filter,
+                              const int32_t *bias, const int32_t *shift, int8_t *out)
+{
+    if (!geometry_ok(g, 1))
+        return -1;
+    const int oh = espdl_oracle_conv_out_h(g), ow = espdl_oracle_conv_out_w(g);
+    const int C = g->in_c, KH = g->k_h, KW = g->k_w;
+    const int64_t in_img = (int64_t)g->in_h * g->in_w * C;
+    const int64_t out_img = (int64_t)oh * ow * C;
+    const int64_t rows = (int64_t)g->batch * oh;
+
+#pragma omp parallel
+    {
+        int32_t *acc = (int32_t *)malloc(sizeof(int32_t) * (size_t)C);
+#pragma omp for schedule(static)
+        for (int64_t row = 0; row < rows; row++) {
+            const int n = (int)(row / oh), oy = (int)(row % oh);
+            const int8_t *img = in + n * in_img;
+            int8_t *dst = out + n * out_img + (int64_t)oy * ow * C;
+            int ky0, ky1;
+            tap_range(oy, g->stride_h, g->pad_top, g->dil_h, KH, g->in_h, &ky0, &ky1);
+            for (int ox = 0; ox < ow; ox++) {
+                int kx0, kx1;
+                tap_range(ox, g->stride_w, g->pad_left, g->dil_w, KW, g->in_w, &kx0, &kx1);
+                memset(acc, 0, sizeof(int32_t) * (size_t)C);
+                for (int ky = ky0; ky < ky1; ky++) {
+                    const int iy = oy * g->stride_h - g->pad_top + ky * g->dil_h;
+                    for (int kx = kx0; kx < kx1; kx++) {
+                        const int ix = ox * g->stride_w - g->pad_left + kx * g->dil_w;
+                        const int8_t *px = img + ((int64_t)iy * g->in_w + ix) * C;
+                        const int8_t *fw = filter + ((int64_t)ky * KW + kx) * C;
+                        for (int c = 0; c < C; c++)
+                            acc[c] += (int32_t)px[c] * (int32_t)fw[c];
+                    }
+                }
+                for (int c = 0; c < C; c++) {
+                    int32_t a = acc[c];
+                    if (bias)
+                        a = (int32_t)((uint32_t)a + (uint32_t)bias[c]);
+                    int32_t v = espdl_oracle_shift_round_s32(a, shift[g->n_shift == 1 ? 0 : c], g->round_mode);
+                    if (g->activation == ESPDL_ORACLE_RELU && v < 0)
+                        v = 0;
+                    dst[(int64_t)ox * C + c] = (int8_t)clamp_i64(v, INT8_MIN, INT8_MAX);
+                }
+            }
+        }
+        free(acc);
+    }
+    return 0;
+}
+
+/* ---------------------------------------------------------------------------------------------
+ * int16 paths: products are int16*int16 (formed as `int`), accumulator / bias / shift_and_round in
+ * int64 (DL_S16_BUFFER_TYPE, esp-dl/dl/dl_define_private.hpp:15-17;
+ * esp-dl/dl/base/dl_base_conv2d.cpp:875-897, 912-939; dl_base_depthwise_conv2d.cpp:495-519),
+ * output clamped to the int16 range.
+ * ------------------------------------------------------------------------------------------- */
+int espdl_oracle_conv2d_s16(const espdl_oracle_conv_t *g, const int16_t *in, const int16_t *filter,
+                            const int64_t *bias, const int32_t *shift, int16_t *out)
+{
+    if (!geometry_ok(g, 0))
+        return -1;
+    const int oh = espdl_oracle_conv_out_h(g), ow = espdl_oracle_conv_out_w(g);
+    const int C = g->in_c, OC = g->out_c, KH = g->k_h, KW = g->k_w;
+    const int64_t in_img = (int64_t)g->in_h * g->in_w * C;
+    const int64_t out_img = (int64_t)oh * ow * OC;
+    const int64_t rows = (int64_t)g->batch * oh;
+
+#pragma omp parallel for schedule(static)
+    for (int64_t row = 0; row < rows; row++) {
+        const int n = (int)(row / oh), oy = (int)(row % oh);
+        const int16_t *img = in + n * in_img;
+        int16_t *dst = out + n * out_img + (int64_t)oy * ow * OC;
+        int ky0, ky1;
+        tap_range(oy, g->stride_h, g->pad_top, g->dil_h, KH, g->in_h, &ky0, &ky1);
+        for (int ox = 0; ox < ow; ox++) {
+            int kx0, kx1;
+            tap_range(ox, g->stride_w, g->pad_left, g->dil_w, KW, g->in_w, &kx0, &kx1);
+            for (int oc = 0; oc < OC; oc++) {
+                const int16_t *f_oc = filter + (int64_t)oc * KH * KW * C;
+                int64_t acc = 0;
+                for (int ky = ky0; ky < ky1; ky++) {
+                    const int iy = oy * g->stride_h - g->pad_top + ky * g->dil_h;
+                    for (int kx = kx0; kx < kx1; kx++) {
+                        const int ix = ox * g->stride_w - g->pad_left + kx * g->dil_w;
+                        const int16_t *px = img + ((int64_t)iy * g->in_w + ix) * C;
+                        const int16_t *fw = f_oc + ((int64_t)ky * KW + kx) * C;
+                        for (int c = 0; c < C; c++)
+                            acc += (int64_t)((int32_t)px[c] * (int32_t)fw[c]);
+                    }
+                }
+                if (bias)
+                    acc += bias[oc];
+                int64_t v = espdl_oracle_shift_round_s64(acc, shift[g->n_shift == 1 ? 0 : oc], g->round_mode);
+                if (g->activation == ESPDL_ORACLE_RELU && v < 0)
+                    v = 0;
+                dst[(int64_t)ox * OC + oc] = (int16_t)clamp_i64(v, INT16_MIN, INT16_MAX);
+            }
+        }
+    }
+    return 0;
+}
+
+int espdl_oracle_depthwise_s16(const espdl_oracle_conv_t *g, const int16_t *in, const int16_t *filter,
+                               const int64_t *bias, const int32_t *shift, int16_t *out)
+{
+    if (!geometry_ok(g, 1))
+        return -1;
+    const int oh = espdl_oracle_conv_out_h(g), ow = espdl_oracle_conv_out_w(g);
+    const int C = g->in_c, KH = g->k_h, KW = g->k_w;
+    const int64_t in_img = (int64_t)g->in_h * g->in_w * C;
+    const int64_t out_img = (int64_t)oh * ow * C;
+    const int64_t rows = (int64_t)g->batch * oh;
+
+#pragma omp parallel for schedule(static)
+    for (int64_t row = 0; row < rows; row++) {
+        const int n = (int)(row / oh), oy = (int)(row % oh);
+        const int16_t *img = in + n * in_img;
+        int16_t *dst = out + n * out_img + (int64_t)oy * ow * C;
+        int ky0, ky1;
+        tap_range(oy, g->stride_h, g->pad_top, g->dil_h, KH, g->in_h, &ky0, &ky1);
+        for (int ox = 0; ox < ow; ox++) {
+            int kx0, kx1;
+            tap_range(ox, g->stride_w, g->pad_left, g->dil_w, KW, g->in_w, &kx0, &kx1);
+            for (int c = 0; c < C; c++) {
+                int64_t acc = 0;
+                for (int ky = ky0; ky < ky1; ky++) {
+                    const int iy = oy * g->stride_h - g->pad_top + ky * g->dil_h;
+                    for (int kx = kx0; kx < kx1; kx++) {
+                        const int ix = ox * g->stride_w - g->pad_left + kx * g->dil_w;
+                        acc += (int64_t)((int32_t)img[((int64_t)iy * g->in_w + ix) * C + c] *
+                                         (int32_t)filter[((int64_t)ky * KW + kx) * C + c]);
+                    }
+                }
+                if (bias)
+                    acc += bias[c];
+                int64_t v = espdl_oracle_shift_round_s64(acc, shift[g->n_shift == 1 ? 0 : c], g->round_mode);
+                if (g->activation == ESPDL_ORACLE_RELU && v < 0)
+                    v = 0;
+                dst[(int64_t)ox * C + c] = (int16_t)clamp_i64(v, INT16_MIN, INT16_MAX);
+            }
+        }
+    }
+    return 0;
+}
+
+/* lut_s8_c (esp-dl/dl/base/dl_base_lut.cpp:10-15): out = table[(uint8)in ^ 0x80]. */
+void espdl_oracle_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < size; i++)
+        out[i] = table[(uint8_t)in[i] ^ 0x80u];
+}
+
+/*
+ * prelu_11c<int8_t, int16_t> (esp-dl/dl/base/dl_base_prelu.cpp:7-21): for x < 0 the product
+ * int16(x) * int16(alpha[c]) is formed as `int`, shifted with DL_RIGHT_SHIFT (arithmetic right
+ * shift for shift > 0, left shift otherwise; esp-dl/dl/dl_define.hpp:67-69), stored into an int16
+ * temporary, then clamped to int8.  shift comes from get_activation_args
+ * (esp-dl/dl/base/dl_base.hpp:2165-2168).
+ */
+void espdl_oracle_prelu_s8(const int8_t *in, int64_t pixels, int channels, const int8_t *alpha, int shift,
+                           int8_t *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t p = 0; p < pixels; p++) {
+        const int8_t *src = in + p * channels;
+        int8_t *dst = out + p * channels;
+        for (int c = 0; c < channels; c++) {
+            int8_t x = src[c];
+            if (x < 0) {
+                int prod = (int)(int16_t)x * (int)(int16_t)alpha[c];
+                int shifted = shift > 0 ? (prod >> shift) : (int)((unsigned)prod << -shift);
+                int16_t temp = (int16_t)shifted;
+                x = (int8_t)clamp_i64(temp, INT8_MIN, INT8_MAX);
+            }
+            dst[c] = x;
+        }
+    }
+}
+
+/* tool::round(float) = (int)floorf(value + 0.5) with a double literal (esp-dl/dl/tool/src/dl_tool.cpp:72-75). */
+static inline int round_half_up_f32(float v)
+{
+    return (int)floorf((float)((double)v + 0.5));
+}
+
+/* DL_SCALE / DL_RESCALE (esp-dl/dl/dl_define.hpp:75-81) */
+static inline float dl_scale(int e)
+{
+    return e > 0 ? (float)(1 << e) : 1.0f / (float)(1 << -e);
+}
+static inline float dl_rescale(int e)
+{
+    return e > 0 ? 1.0f / (float)(1 << e) : (float)(1 << -e);
+}
+
+/* Relu::forward_template (esp-dl/dl/module/include/dl_module_relu.hpp:65-93). */
+void espdl_oracle_relu_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out)
+{
+    if (in_exp == out_exp) {
+        for (int64_t i = 0; i < size; i++)
+            out[i] = in[i] >= 0 ? in[i] : 0;
+        return;
+    }
+    const float input_scale = dl_scale(in_exp), output_scale = dl_rescale(out_exp);
+    for (int64_t i = 0; i < size; i++) {
+        float temp = (float)in[i] * input_scale;
+        out[i] = temp >= 0 ? (int8_t)clamp_i64(round_half_up_f32(temp * output_scale), INT8_MIN, INT8_MAX) : 0;
+    }
+}
+
+/* Clip::forward_template (esp-dl/dl/module/include/dl_module_clip.hpp:78-90); min/max are quantized scalars. */
+void espdl_oracle_clip_s8(const int8_t *in, int64_t size, int min_q, int max_q, int in_exp, int out_exp,
+                          int8_t *out)
+{
+    const float rescale = dl_scale(in_exp) * dl_rescale(out_exp);
+    for (int64_t i = 0; i < size; i++) {
+        int8_t t = in[i] < min_q ? (int8_t)min_q : (in[i] > max_q ? (int8_t)max_q : in[i]);
+        out[i] = (int8_t)clamp_i64(round_half_up_f32((float)t * rescale), INT8_MIN, INT8_MAX);
+    }
+}
+
+/* c_impl_add_n_n / _n_1 / _1_n (esp-dl/dl/base/dl_base_add.cpp:8-44): clamp(a + b), no exponent handling. */
+void espdl_oracle_add_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size,
+                         int8_t *out)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < size; i++) {
+        int32_t a = in0[len0 == 1 ? 0 : i], b = in1[len1 == 1 ? 0 : i];
+        out[i] = (int8_t)clamp_i64(a + b, INT8_MIN, INT8_MAX);
+    }
+}
+
+/*
+ * GlobalAveragePool = avgpool2d_hwc over the whole image (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54):
+ * int32 sum per channel, then truncate(round(float(sum) * scale)),
+ * scale = DL_SCALE(in_exp) * (1.f / area) * DL_RESCALE(out_exp) evaluated left to right in float32.
+ */
+void espdl_oracle_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
+                                     int8_t *out)
+{
+    const float area_inv = 1.f / (float)(h * w);
+    const float scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < batch; n++) {
+        const int8_t *img = in + (int64_t)n * h * w * c;
+        for (int ch = 0; ch < c; ch++) {
+            int32_t sum = 0;
+            for (int p = 0; p < h * w; p++)
+                sum += img[(int64_t)p * c + ch];
+            out[(int64_t)n * c + ch] = (int8_t)clamp_i64(round_half_up_f32((float)sum * scale), INT8_MIN, INT8_MAX);
+        }
+    }
+}
+
+/*
+ * TensorBase::assign, int8 -> int8 with different exponents
+ * (esp-dl/dl/tensor/src/dl_tensor_base.cpp:362-371; quantize/dequantize :18-42):
+ * quantize(dequantize(x, DL_SCALE(in_exp)), 1.0 / DL_SCALE(out_exp)).
+ */
+void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out)
+{
+    if (in_exp == out_exp) {
+        memmove(out, in, (size_t)size);
+        return;
+    }
+    const float src_scale = dl_scale(in_exp);
+    const float inv_scale = (float)(1.0 / (double)dl_scale(out_exp));
+    for (int64_t i = 0; i < size; i++) {
+        float tmp = (float)in[i] * src_scale;
+        out[i] = (int8_t)clamp_i64(round_half_up_f32(tmp * inv_scale), INT8_MIN, INT8_MAX);
+    }
+}

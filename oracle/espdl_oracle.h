@@ -1,0 +1,100 @@
+/*
+ * CPU oracle for ESP-DL's quantized operator path (portable C, non-PIE).
+ *
+ * TEST INFRASTRUCTURE ONLY.  This is a plain-C restatement of the reference's arithmetic, used
+ * by tests/, by __graft_entry__.smoke() and by bench.py's cpu_baseline leg as the checker and the
+ * timed CPU baseline.  Nothing in the shipped library links, loads or calls it.
+ *
+ * Conventions (as in the reference): activations NHWC, one image = one reference call (the
+ * reference is batch-1; a batch of N is N independent images); conv filter memory is
+ * [Cout][kH][kW][Cin] (esp-dl/dl/base/dl_base_conv2d.cpp:23,64,140), depthwise filter memory is
+ * [kH][kW][C] (esp-dl/dl/base/dl_base_depthwise_conv2d.cpp:46-65); real = q * 2^exponent.
+ *
+ * Pinning status of each function (what fixes its behaviour besides re-reading the reference):
+ *   espdl_oracle_shift_round_*   exhaustive comparison with floor(v/2^s + 1/2) in exact rationals
+ *                                and the half-even ties table                            PINNED
+ *   espdl_oracle_conv2d_s8       reference-held Gemm known answers (c target, 3 files) for the
+ *                                1x1 path, N-major filter layout, bias-before-shift, rounding,
+ *                                ReLU, saturation; brute force + padding/stride/dilation
+ *                                invariants for the windowed path                         PINNED
+ *   espdl_oracle_depthwise_s8    brute force; equality with a grouped conv written as a
+ *                                block-diagonal espdl_oracle_conv2d_s8                    PINNED
+ *   espdl_oracle_conv2d_s16 /
+ *   espdl_oracle_depthwise_s16   brute force in arbitrary-precision integers              PINNED
+ *   per-channel shift            by definition the per-tensor formula applied per output
+ *                                channel (the reference C branch for it is dead code and the
+ *                                shipping semantics live in ESP32-P4 assembly,
+ *                                esp-dl/dl/base/isa/esp32p4/dl_esp32p4_s8.S:57-65); checked as
+ *                                equality with per-tensor runs on single-channel slices   PINNED (to that definition)
+ *   espdl_oracle_lut_s8          known-answer pattern of test_apps/dl_pie_func/main/test_lut.cpp:104-150,
+ *                                identity table                                           PINNED
+ *   espdl_oracle_prelu_s8, _relu_s8, _add_s8   exhaustive over all int8 operand pairs against
+ *                                closed forms in exact integers                           PINNED
+ *   espdl_oracle_clip_s8, _global_avg_pool_s8, _requantize_s8   float32-defined in the reference
+ *                                (floorf(x + 0.5) under -ffast-math); checked against exact
+ *                                rational round-half-up, which fixes every non-tie case; the
+ *                                reference itself could not be built here           PARITY UNPINNED (float ties)
+ */
+#ifndef ESPDL_ORACLE_H
+#define ESPDL_ORACLE_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { ESPDL_ORACLE_ROUND_HALF_UP = 0, ESPDL_ORACLE_ROUND_HALF_EVEN = 1 };
+enum { ESPDL_ORACLE_LINEAR = 0, ESPDL_ORACLE_RELU = 1 };
+
+/* Geometry of one convolution; shared by the s8/s16, dense/depthwise entry points. */
+typedef struct {
+    int batch, in_h, in_w, in_c; /* input  [batch][in_h][in_w][in_c]                      */
+    int out_c;                   /* dense: filters; depthwise: must equal in_c            */
+    int k_h, k_w;
+    int stride_h, stride_w;
+    int dil_h, dil_w;
+    int pad_top, pad_bottom, pad_left, pad_right;
+    int activation; /* ESPDL_ORACLE_LINEAR / ESPDL_ORACLE_RELU                            */
+    int round_mode; /* ESPDL_ORACLE_ROUND_HALF_UP is the portable C path                   */
+    int n_shift;    /* 1 = per-tensor, out_c = one shift per output channel               */
+} espdl_oracle_conv_t;
+
+int32_t espdl_oracle_shift_round_s32(int32_t value, int shift, int round_mode);
+int64_t espdl_oracle_shift_round_s64(int64_t value, int shift, int round_mode);
+
+int espdl_oracle_conv_out_h(const espdl_oracle_conv_t *g);
+int espdl_oracle_conv_out_w(const espdl_oracle_conv_t *g);
+
+/* bias may be NULL.  shift[i] = out_exp - filter_exp[i] - in_exp.  Returns 0, or -1 on bad geometry. */
+int espdl_oracle_conv2d_s8(const espdl_oracle_conv_t *g, const int8_t *in, const int8_t *filter,
+                           const int32_t *bias, const int32_t *shift, int8_t *out);
+int espdl_oracle_depthwise_s8(const espdl_oracle_conv_t *g, const int8_t *in, const int8_t *filter,
+                              const int32_t *bias, const int32_t *shift, int8_t *out);
+int espdl_oracle_conv2d_s16(const espdl_oracle_conv_t *g, const int16_t *in, const int16_t *filter,
+                            const int64_t *bias, const int32_t *shift, int16_t *out);
+int espdl_oracle_depthwise_s16(const espdl_oracle_conv_t *g, const int16_t *in, const int16_t *filter,
+                               const int64_t *bias, const int32_t *shift, int16_t *out);
+
+void espdl_oracle_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out);
+/* alpha has `channels` entries; shift = out_exp - in_exp - alpha_exp. */
+void espdl_oracle_prelu_s8(const int8_t *in, int64_t pixels, int channels, const int8_t *alpha, int shift,
+                           int8_t *out);
+void espdl_oracle_relu_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out);
+void espdl_oracle_clip_s8(const int8_t *in, int64_t size, int min_q, int max_q, int in_exp, int out_exp,
+                          int8_t *out);
+/* Broadcast add: len0 / len1 are `size` or 1 (scalar operand). */
+void espdl_oracle_add_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size,
+                         int8_t *out);
+void espdl_oracle_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
+                                     int8_t *out);
+void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out);
+
+/* Number of worker threads the batch loops use (1 unless built with OpenMP). */
+int espdl_oracle_max_threads(void);
+void espdl_oracle_set_threads(int n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,214 @@
+"""ctypes binding of the CPU oracle (oracle/libespdl_oracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
+leg.  The shipped library never loads it.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libespdl_oracle.so")
+
+ROUND_HALF_UP = 0
+ROUND_HALF_EVEN = 1
+LINEAR = 0
+RELU = 1
+
+
+class ConvGeom(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int) for n in (
+        "batch", "in_h", "in_w", "in_c", "out_c", "k_h", "k_w", "stride_h", "stride_w", "dil_h", "dil_w",
+        "pad_top", "pad_bottom", "pad_left", "pad_right", "activation", "round_mode", "n_shift")]
+
+
+def build():
+    """Compile the oracle with gcc (make -C oracle)."""
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        src_time = max(os.path.getmtime(os.path.join(_HERE, f)) for f in ("espdl_oracle.c", "espdl_oracle.h"))
+        if not os.path.exists(_LIB_PATH) or os.path.getmtime(_LIB_PATH) < src_time:
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        vp, i32, i64 = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+        gp = ctypes.POINTER(ConvGeom)
+        L.espdl_oracle_shift_round_s32.restype = ctypes.c_int32
+        L.espdl_oracle_shift_round_s32.argtypes = [ctypes.c_int32, i32, i32]
+        L.espdl_oracle_shift_round_s64.restype = ctypes.c_int64
+        L.espdl_oracle_shift_round_s64.argtypes = [ctypes.c_int64, i32, i32]
+        for name in ("conv_out_h", "conv_out_w"):
+            f = getattr(L, "espdl_oracle_" + name)
+            f.restype, f.argtypes = i32, [gp]
+        for name in ("conv2d_s8", "depthwise_s8", "conv2d_s16", "depthwise_s16"):
+            f = getattr(L, "espdl_oracle_" + name)
+            f.restype, f.argtypes = i32, [gp, vp, vp, vp, vp, vp]
+        L.espdl_oracle_lut_s8.argtypes = [vp, i64, vp, vp]
+        L.espdl_oracle_prelu_s8.argtypes = [vp, i64, i32, vp, i32, vp]
+        L.espdl_oracle_relu_s8.argtypes = [vp, i64, i32, i32, vp]
+        L.espdl_oracle_clip_s8.argtypes = [vp, i64, i32, i32, i32, i32, vp]
+        L.espdl_oracle_add_s8.argtypes = [vp, i64, vp, i64, i64, vp]
+        L.espdl_oracle_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp]
+        L.espdl_oracle_requantize_s8.argtypes = [vp, i64, i32, i32, vp]
+        L.espdl_oracle_max_threads.restype = i32
+        L.espdl_oracle_set_threads.argtypes = [i32]
+        for name in ("lut_s8", "prelu_s8", "relu_s8", "clip_s8", "add_s8", "global_avg_pool_s8",
+                     "requantize_s8", "set_threads"):
+            getattr(L, "espdl_oracle_" + name).restype = None
+        _lib = L
+    return _lib
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _c(a, dtype):
+    return None if a is None else np.ascontiguousarray(a, dtype=dtype)
+
+
+def set_threads(n):
+    lib().espdl_oracle_set_threads(int(n))
+
+
+def max_threads():
+    return lib().espdl_oracle_max_threads()
+
+
+def shift_round_s32(v, shift, round_mode=ROUND_HALF_UP):
+    return lib().espdl_oracle_shift_round_s32(int(v), int(shift), int(round_mode))
+
+
+def shift_round_s64(v, shift, round_mode=ROUND_HALF_UP):
+    return lib().espdl_oracle_shift_round_s64(int(v), int(shift), int(round_mode))
+
+
+def conv_geom(x_shape, out_c, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), activation=LINEAR,
+              round_mode=ROUND_HALF_UP, n_shift=1):
+    """pads = (top, bottom, left, right), the order ConvOpArgs takes (dl_base.hpp:201-204)."""
+    n, h, w, c = x_shape
+    return ConvGeom(n, h, w, c, out_c, k[0], k[1], stride[0], stride[1], dilation[0], dilation[1],
+                    pads[0], pads[1], pads[2], pads[3], activation, round_mode, n_shift)
+
+
+def out_hw(g):
+    return lib().espdl_oracle_conv_out_h(ctypes.byref(g)), lib().espdl_oracle_conv_out_w(ctypes.byref(g))
+
+
+def _conv(fn, act_dtype, bias_dtype, x, filt, bias, shift, k, stride, dilation, pads, activation, round_mode,
+          depthwise):
+    x = _c(x, act_dtype)
+    assert x.ndim == 4
+    filt = _c(filt, act_dtype)
+    shift = np.atleast_1d(_c(shift, np.int32))
+    out_c = x.shape[3] if depthwise else filt.size // (k[0] * k[1] * x.shape[3])
+    bias = _c(bias, bias_dtype)
+    g = conv_geom(x.shape, out_c, k, stride, dilation, pads, activation, round_mode, shift.size)
+    oh, ow = out_hw(g)
+    out = np.empty((x.shape[0], oh, ow, out_c), dtype=act_dtype)
+    rc = fn(ctypes.byref(g), _ptr(x), _ptr(filt), _ptr(bias), _ptr(shift), _ptr(out))
+    if rc != 0:
+        raise ValueError("oracle rejected the convolution geometry")
+    return out
+
+
+def conv2d_s8(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), activation=LINEAR,
+              round_mode=ROUND_HALF_UP):
+    """x [N,H,W,C] int8, filt memory [OC][kH][kW][C] int8, bias [OC] int32 or None, shift scalar or [OC]."""
+    return _conv(lib().espdl_oracle_conv2d_s8, np.int8, np.int32, x, filt, bias, shift, k, stride, dilation, pads,
+                 activation, round_mode, False)
+
+
+def depthwise_s8(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), activation=LINEAR,
+                 round_mode=ROUND_HALF_UP):
+    """filt memory [kH][kW][C]."""
+    return _conv(lib().espdl_oracle_depthwise_s8, np.int8, np.int32, x, filt, bias, shift, k, stride, dilation,
+                 pads, activation, round_mode, True)
+
+
+def conv2d_s16(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), activation=LINEAR,
+               round_mode=ROUND_HALF_UP):
+    return _conv(lib().espdl_oracle_conv2d_s16, np.int16, np.int64, x, filt, bias, shift, k, stride, dilation,
+                 pads, activation, round_mode, False)
+
+
+def depthwise_s16(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), activation=LINEAR,
+                  round_mode=ROUND_HALF_UP):
+    return _conv(lib().espdl_oracle_depthwise_s16, np.int16, np.int64, x, filt, bias, shift, k, stride, dilation,
+                 pads, activation, round_mode, True)
+
+
+def gemm_s8(x, filt, bias, shift, activation=LINEAR, round_mode=ROUND_HALF_UP):
+    """Gemm / MatMul as the reference runs it: input viewed as {1,1,M,K}, 1x1 conv
+    (esp-dl/dl/module/include/dl_module_gemm.hpp:86-123).  filt memory [N][K]."""
+    x = _c(x, np.int8)
+    k = x.shape[-1]
+    m = x.size // k
+    y = conv2d_s8(x.reshape(1, 1, m, k), filt, bias, shift, (1, 1), activation=activation, round_mode=round_mode)
+    return y.reshape(x.shape[:-1] + (y.shape[-1],))
+
+
+def lut_s8(x, table):
+    x = _c(x, np.int8)
+    table = _c(table, np.int8)
+    assert table.size == 256
+    out = np.empty_like(x)
+    lib().espdl_oracle_lut_s8(_ptr(x), x.size, _ptr(table), _ptr(out))
+    return out
+
+
+def prelu_s8(x, alpha, shift):
+    x = _c(x, np.int8)
+    alpha = _c(alpha, np.int8)
+    c = x.shape[-1]
+    assert alpha.size == c
+    out = np.empty_like(x)
+    lib().espdl_oracle_prelu_s8(_ptr(x), x.size // c, c, _ptr(alpha), int(shift), _ptr(out))
+    return out
+
+
+def relu_s8(x, in_exp=0, out_exp=0):
+    x = _c(x, np.int8)
+    out = np.empty_like(x)
+    lib().espdl_oracle_relu_s8(_ptr(x), x.size, in_exp, out_exp, _ptr(out))
+    return out
+
+
+def clip_s8(x, min_q, max_q, in_exp=0, out_exp=0):
+    x = _c(x, np.int8)
+    out = np.empty_like(x)
+    lib().espdl_oracle_clip_s8(_ptr(x), x.size, int(min_q), int(max_q), in_exp, out_exp, _ptr(out))
+    return out
+
+
+def add_s8(a, b):
+    a = _c(a, np.int8)
+    b = _c(b, np.int8)
+    size = max(a.size, b.size)
+    assert a.size in (1, size) and b.size in (1, size)
+    out = np.empty(a.shape if a.size == size else b.shape, dtype=np.int8)
+    lib().espdl_oracle_add_s8(_ptr(a), a.size, _ptr(b), b.size, size, _ptr(out))
+    return out
+
+
+def global_avg_pool_s8(x, in_exp, out_exp):
+    x = _c(x, np.int8)
+    n, h, w, c = x.shape
+    out = np.empty((n, 1, 1, c), dtype=np.int8)
+    lib().espdl_oracle_global_avg_pool_s8(_ptr(x), n, h, w, c, in_exp, out_exp, _ptr(out))
+    return out
+
+
+def requantize_s8(x, in_exp, out_exp):
+    x = _c(x, np.int8)
+    out = np.empty_like(x)
+    lib().espdl_oracle_requantize_s8(_ptr(x), x.size, in_exp, out_exp, _ptr(out))
+    return out

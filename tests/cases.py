@@ -1,0 +1,64 @@
+"""Shape matrix shared by the oracle tests and the GPU parity tests.
+
+CONV_CASES / DW_CASES restate tools/ops_test/config/op_cfg.toml:14-400 of the reference in NHWC
+terms (aligned, unaligned 22->33 / 27 / 25 channels, filter larger than the input, stride 2,
+asymmetric stride, dilation 3 with padding 12), plus BASELINE config 1 and a few geometries the
+reference shell treats specially (tail-only padding, negative shift).
+Fields: (name, (H, W, C), OC, (kh, kw), stride, dilation, pads(t,b,l,r), bias, relu)
+"""
+
+CONV_CASES = [
+    ("c3_100x50_k3s2_relu", (100, 50, 3), 16, (3, 3), (2, 2), (1, 1), (0, 0, 0, 0), True, True),
+    ("c16_20x20_k1", (20, 20, 16), 32, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("c16_100x50_k1", (100, 50, 16), 32, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("c16_22x22_k5s2p2_relu", (22, 22, 16), 32, (5, 5), (2, 2), (1, 1), (2, 2, 2, 2), True, True),
+    ("c32_19x23_k3s2p1", (19, 23, 32), 16, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, False),
+    ("c22_19x23_k3p1_oc33", (19, 23, 22), 33, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False),
+    ("c16_3x3_k3p1_nobias", (3, 3, 16), 16, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), False, False),
+    ("c27_3x3_k5p2_nobias", (3, 3, 27), 27, (5, 5), (1, 1), (1, 1), (2, 2, 2, 2), False, False),
+    # Conv1D rows of the matrix, as H = 1 images
+    ("c3_1x50_k3s2_relu", (1, 50, 3), 16, (1, 3), (1, 2), (1, 1), (0, 0, 0, 0), True, True),
+    ("c16_1x32_k5s2p2_relu", (1, 32, 16), 32, (1, 5), (1, 2), (1, 1), (0, 0, 2, 2), True, True),
+    ("c22_1x29_k3p1_oc33", (1, 29, 22), 33, (1, 3), (1, 1), (1, 1), (0, 0, 1, 1), True, False),
+    # extra geometries
+    ("c8_9x11_k3s2_tailpad", (9, 11, 8), 12, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), False, False),
+    ("c5_12x12_k3d2p2", (12, 12, 5), 7, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2), True, True),
+    ("c64_14x14_k1_oc96", (14, 14, 64), 96, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
+    ("c24_8x8_k1_oc144", (8, 8, 24), 144, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("c64_8x8_k1s2", (8, 8, 64), 32, (1, 1), (2, 2), (1, 1), (0, 0, 0, 0), True, False),
+    ("c32_10x10_k3p1_oc64_relu", (10, 10, 32), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
+]
+
+# BASELINE config 1: 1x56x56x64 -> 64, 3x3, s1, p1, bias, ReLU, shift 9
+CONFIG1 = ("config1_56x56x64_k3p1_relu", (56, 56, 64), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True)
+
+DW_CASES = [
+    ("dw16_3x3_k3p1_relu", (3, 3, 16), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
+    ("dw16_20x20_k5s12p2_relu", (20, 20, 16), (5, 5), (1, 2), (1, 1), (2, 2, 2, 2), True, True),
+    ("dw25_20x20_k7s12p2_relu", (20, 20, 25), (7, 7), (1, 2), (1, 1), (2, 2, 2, 2), True, True),
+    ("dw32_100x50_k3_relu", (100, 50, 32), (3, 3), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
+    ("dw16_3x3_k5p2_nobias", (3, 3, 16), (5, 5), (1, 1), (1, 1), (2, 2, 2, 2), False, False),
+    ("dw16_9x9_k5d3p12_nobias", (9, 9, 16), (5, 5), (1, 1), (3, 3), (12, 12, 12, 12), False, False),
+    ("dw27_3x3_k5p2_nobias", (3, 3, 27), (5, 5), (1, 1), (1, 1), (2, 2, 2, 2), False, False),
+    ("dw30_1x20_k7s2p2_relu", (1, 20, 30), (1, 7), (1, 2), (1, 1), (0, 0, 2, 2), True, True),
+    ("dw144_14x14_k3p1_relu", (14, 14, 144), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
+    ("dw96_15x15_k3s2p1", (15, 15, 96), (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, False),
+    ("dw8_7x9_k3s2_tailpad", (7, 9, 8), (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), True, False),
+]
+
+GEMM_CASES = [  # (M, K, N, bias, relu)
+    (1, 16, 16, True, True), (1, 31, 32, True, True), (1, 64, 32, True, False),
+    (3, 10, 9, False, False), (32, 10, 35, False, False), (40, 120, 480, True, False),
+    (7, 1280, 1000, True, False), (5, 33, 1, True, True),
+]
+
+
+def rng_int8(rng, shape):
+    import numpy as np
+    return rng.integers(-128, 128, size=shape, dtype=np.int64).astype(np.int8)
+
+
+def typical_shift(k_total):
+    """A requantization shift that keeps outputs spread over the int8 range for uniform int8 operands."""
+    import math
+    return max(1, int(round(math.log2(5461 * math.sqrt(k_total) / 40))))
