@@ -1,0 +1,13 @@
+"""esp-dl_amd: ESP-DL's quantized operator hot path on AMD MI355X (gfx950).
+
+The product is native: `lib/libespdl_hip.so` (HIP kernels behind the C ABI of include/espdl_hip.h)
+and `lib/libespdl_dl.so` (the C++ `dl::` host layer: TensorBase, Module, Model).  This Python
+package is only a thin ctypes driver for tests and benchmarks; PyTorch supplies device memory and
+streams, nothing else.  The directory name is not a Python identifier: import it with
+`importlib.import_module("esp-dl_amd")`.
+"""
+from . import capi  # noqa: F401
+from .capi import (  # noqa: F401
+    ConvDesc, EspdlHipError, LIB_PATH, add_s8, clip_s8, conv2d, conv_out_shape, global_avg_pool_s8, lib, lut_s8,
+    prelu_s8, relu_s8, requantize_s8,
+)

@@ -1,0 +1,60 @@
+"""Builds the gfx950 libraries of this package in-tree with hipcc.
+
+  python esp-dl_amd/build.py            # libespdl_hip.so (kernels + C ABI)
+
+The GPU box runs the prebuilt .so files that travel with the tree; nothing is compiled there.
+"""
+import concurrent.futures
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+OBJ_DIR = os.path.join(HERE, "build")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+KERNEL_SOURCES = ["conv2d_s8_mfma.hip", "depthwise_s8.hip", "conv_s16.hip", "elementwise_s8.hip", "espdl_hip_api.hip"]
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    if r.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s\n%s" % (" ".join(cmd), r.stdout, err))
+    return err
+
+
+def _compile(src, extra=()):
+    obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
+    warn = _run([HIPCC, *HIP_FLAGS, *extra, "-c", src, "-o", obj])
+    return obj, warn
+
+
+def build_kernels(verbose=True):
+    os.makedirs(LIB_DIR, exist_ok=True)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    srcs = [os.path.join(CSRC, s) for s in KERNEL_SOURCES]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        results = list(pool.map(_compile, srcs))
+    for (obj, warn), src in zip(results, srcs):
+        if warn.strip() and verbose:
+            print("[%s]\n%s" % (os.path.basename(src), warn), file=sys.stderr)
+    out = os.path.join(LIB_DIR, "libespdl_hip.so")
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", out, *[o for o, _ in results]])
+    return out
+
+
+def build_all(verbose=True):
+    return [build_kernels(verbose)]
+
+
+if __name__ == "__main__":
+    for lib in build_all():
+        print("built", lib)

@@ -1,0 +1,180 @@
+"""ctypes binding of include/espdl_hip.h (lib/libespdl_hip.so).
+
+Tensors are torch CUDA tensors used as plain device buffers (`data_ptr()`); kernels are enqueued on
+torch's current stream unless another raw stream handle is given.  There is no CPU fallback: if the
+library is missing, `lib()` raises.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libespdl_hip.so")
+
+S8, S16 = 8, 16
+LINEAR, RELU = 0, 1
+ROUND_HALF_UP, ROUND_HALF_EVEN = 0, 1
+
+
+class EspdlHipError(RuntimeError):
+    pass
+
+
+class ConvDesc(ctypes.Structure):
+    """espdl_hip_conv_desc"""
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "dtype", "batch", "in_h", "in_w", "in_c", "out_c", "k_h", "k_w", "stride_h", "stride_w", "dil_h", "dil_w",
+        "pad_top", "pad_bottom", "pad_left", "pad_right", "group", "activation", "round_mode", "n_shift")]
+
+
+_lib = None
+
+
+def lib():
+    """Load libespdl_hip.so; fails loudly when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise EspdlHipError(
+                f"{LIB_PATH} is missing: build it with `python esp-dl_amd/build.py` (no CPU fallback exists)")
+        L = ctypes.CDLL(LIB_PATH)
+        vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
+        dp = ctypes.POINTER(ConvDesc)
+        L.espdl_hip_conv_out_shape.argtypes = [dp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
+        L.espdl_hip_conv2d.argtypes = [dp, vp, vp, vp, vp, vp, vp, vp]
+        L.espdl_hip_lut_s8.argtypes = [vp, i64, vp, vp, vp]
+        L.espdl_hip_prelu_s8.argtypes = [vp, i64, i32, vp, i32, vp, vp]
+        L.espdl_hip_relu_s8.argtypes = [vp, i64, i32, i32, vp, vp]
+        L.espdl_hip_clip_s8.argtypes = [vp, i64, i32, i32, i32, i32, vp, vp]
+        L.espdl_hip_add_s8.argtypes = [ctypes.POINTER(i32 * 4), ctypes.POINTER(i64 * 4), ctypes.POINTER(i64 * 4),
+                                       vp, vp, vp, vp]
+        L.espdl_hip_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp]
+        L.espdl_hip_requantize_s8.argtypes = [vp, i64, i32, i32, vp, vp]
+        for name in ("conv_out_shape", "conv2d", "lut_s8", "prelu_s8", "relu_s8", "clip_s8", "add_s8",
+                     "global_avg_pool_s8", "requantize_s8", "device_cu_count"):
+            getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
+        L.espdl_hip_last_error.restype = ctypes.c_char_p
+        L.espdl_hip_version.restype = ctypes.c_char_p
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise EspdlHipError(f"espdl_hip error {rc}: {lib().espdl_hip_last_error().decode()}")
+
+
+def _stream(stream):
+    if stream is not None:
+        return ctypes.c_void_p(stream)
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def make_desc(x_shape, out_c, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), group=1, activation=LINEAR,
+              round_mode=ROUND_HALF_UP, n_shift=1, dtype=S8):
+    n, h, w, c = x_shape
+    return ConvDesc(dtype, n, h, w, c, out_c, k[0], k[1], stride[0], stride[1], dilation[0], dilation[1],
+                    pads[0], pads[1], pads[2], pads[3], group, activation, round_mode, n_shift)
+
+
+def conv_out_shape(desc):
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    _check(lib().espdl_hip_conv_out_shape(ctypes.byref(desc), ctypes.byref(oh), ctypes.byref(ow)))
+    return oh.value, ow.value
+
+
+def conv2d(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), depthwise=False,
+           activation=LINEAR, round_mode=ROUND_HALF_UP, lut=None, out=None, stream=None):
+    """x [N,H,W,C] int8|int16 CUDA tensor; filt dense [OC][kH][kW][C] or depthwise [kH][kW][C];
+    bias int32|int64 [OC] or None; shift int32 tensor with 1 or OC entries (device)."""
+    import torch
+    dtype = S8 if x.dtype == torch.int8 else S16
+    n, h, w, c = x.shape
+    out_c = c if depthwise else filt.numel() // (k[0] * k[1] * c)
+    desc = make_desc(x.shape, out_c, k, stride, dilation, pads, c if depthwise else 1, activation, round_mode,
+                     shift.numel(), dtype)
+    oh, ow = conv_out_shape(desc)
+    if out is None:
+        out = torch.empty((n, oh, ow, out_c), dtype=x.dtype, device=x.device)
+    _check(lib().espdl_hip_conv2d(ctypes.byref(desc), _p(x), _p(filt), _p(bias), _p(shift), _p(lut), _p(out),
+                                  _stream(stream)))
+    return out
+
+
+def lut_s8(x, table, out=None, stream=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    _check(lib().espdl_hip_lut_s8(_p(x), x.numel(), _p(table), _p(out), _stream(stream)))
+    return out
+
+
+def prelu_s8(x, alpha, shift, out=None, stream=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    c = x.shape[-1]
+    _check(lib().espdl_hip_prelu_s8(_p(x), x.numel() // c, c, _p(alpha), shift, _p(out), _stream(stream)))
+    return out
+
+
+def relu_s8(x, in_exp=0, out_exp=0, out=None, stream=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    _check(lib().espdl_hip_relu_s8(_p(x), x.numel(), in_exp, out_exp, _p(out), _stream(stream)))
+    return out
+
+
+def clip_s8(x, min_q, max_q, in_exp=0, out_exp=0, out=None, stream=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    _check(lib().espdl_hip_clip_s8(_p(x), x.numel(), min_q, max_q, in_exp, out_exp, _p(out), _stream(stream)))
+    return out
+
+
+def _pad4(shape):
+    shape = list(shape)
+    if len(shape) > 4:
+        raise EspdlHipError("add_s8 handles up to 4 dims")
+    return [1] * (4 - len(shape)) + shape
+
+
+def add_s8(a, b, out=None, stream=None):
+    """numpy-style broadcasting add of two contiguous tensors (up to 4 dims)."""
+    import torch
+    sa, sb = _pad4(a.shape), _pad4(b.shape)
+    so = [max(x, y) for x, y in zip(sa, sb)]
+
+    def strides(s):
+        st, acc = [0] * 4, 1
+        for i in range(3, -1, -1):
+            st[i] = acc if s[i] != 1 else 0
+            acc *= s[i]
+        return st
+
+    rank = max(a.dim(), b.dim())
+    if out is None:
+        out = torch.empty(so[4 - rank:] if rank else [], dtype=torch.int8, device=a.device)
+    dims = (ctypes.c_int32 * 4)(*so)
+    s0 = (ctypes.c_int64 * 4)(*strides(sa))
+    s1 = (ctypes.c_int64 * 4)(*strides(sb))
+    _check(lib().espdl_hip_add_s8(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), _p(out),
+                                  _stream(stream)))
+    return out
+
+
+def global_avg_pool_s8(x, in_exp, out_exp, out=None, stream=None):
+    import torch
+    n, h, w, c = x.shape
+    out = torch.empty((n, 1, 1, c), dtype=torch.int8, device=x.device) if out is None else out
+    _check(lib().espdl_hip_global_avg_pool_s8(_p(x), n, h, w, c, in_exp, out_exp, _p(out), _stream(stream)))
+    return out
+
+
+def requantize_s8(x, in_exp, out_exp, out=None, stream=None):
+    import torch
+    out = torch.empty_like(x) if out is None else out
+    _check(lib().espdl_hip_requantize_s8(_p(x), x.numel(), in_exp, out_exp, _p(out), _stream(stream)))
+    return out

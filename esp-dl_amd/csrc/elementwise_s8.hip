@@ -1,0 +1,284 @@
+// Bandwidth-bound int8 element-wise operators for gfx950: LUT, PReLU, ReLU, Clip, Add,
+// GlobalAveragePool, requantize.  Each thread moves 16 bytes per load/store when the tensors are
+// 16-byte aligned; a byte tail (and unaligned tensors) take the scalar path of the same kernel.
+#include "espdl_device.h"
+#include "espdl_kernels.h"
+
+namespace espdl {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+// Launch helper: `vecs` 16-byte vectors handled by the vector path, the remaining `size - 16*vecs`
+// bytes by the scalar path of the first threads.
+inline dim3 grid_for(int64_t size, bool vec_ok, int64_t *vecs)
+{
+    *vecs = vec_ok ? size / 16 : 0;
+    const int64_t tail = size - *vecs * 16;
+    const int64_t threads = (*vecs > tail ? *vecs : tail);
+    return dim3((unsigned)((threads + kBlock - 1) / kBlock));
+}
+
+inline bool aligned16(const void *a, const void *b)
+{
+    return ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b)) & 15) == 0;
+}
+
+// A per-byte functor applied over a flat tensor.
+template <typename F>
+__global__ __launch_bounds__(kBlock) void map_s8_kernel(const int8_t *in, int8_t *out, int64_t size, int64_t vecs, F f)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    f.prepare();
+    if (i < vecs) {
+        const v4i v = reinterpret_cast<const v4i *>(in)[i];
+        v4i r;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const int word = v[w];
+            int o = 0;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const int x = (int)(int8_t)(word >> (8 * b));
+                o |= (f(x, i * 16 + w * 4 + b) & 0xff) << (8 * b);
+            }
+            r[w] = o;
+        }
+        reinterpret_cast<v4i *>(out)[i] = r;
+    }
+    const int64_t t = vecs * 16 + i;
+    if (t < size)
+        out[t] = (int8_t)f((int)in[t], t);
+}
+
+// base::lut_s8_c (esp-dl/dl/base/dl_base_lut.cpp:10-15); the table is copied to LDS once per workgroup.
+struct LutFn {
+    const int8_t *table;
+    __device__ void prepare()
+    {
+        __shared__ int8_t tab[256];
+        tab[threadIdx.x] = table[threadIdx.x];
+        __syncthreads();
+        lds = tab;
+    }
+    __device__ int operator()(int x, int64_t) const { return lds[x + 128]; }
+    const int8_t *lds;
+};
+
+// module::Relu (esp-dl/dl/module/include/dl_module_relu.hpp:65-93)
+struct ReluFn {
+    int same_exp;
+    float in_scale, out_scale;
+    __device__ void prepare() {}
+    __device__ int operator()(int x, int64_t) const
+    {
+        if (same_exp)
+            return x >= 0 ? x : 0;
+        const float temp = (float)x * in_scale;
+        return temp >= 0 ? clamp_s8(round_half_up_f32(temp * out_scale)) : 0;
+    }
+};
+
+// module::Clip (esp-dl/dl/module/include/dl_module_clip.hpp:78-90)
+struct ClipFn {
+    int lo, hi;
+    float rescale;
+    __device__ void prepare() {}
+    __device__ int operator()(int x, int64_t) const
+    {
+        const int t = x < lo ? lo : (x > hi ? hi : x);
+        return clamp_s8(round_half_up_f32((float)t * rescale));
+    }
+};
+
+// TensorBase::assign int8 -> int8 (esp-dl/dl/tensor/src/dl_tensor_base.cpp:362-371, 18-42)
+struct RequantFn {
+    float src_scale, inv_scale;
+    __device__ void prepare() {}
+    __device__ int operator()(int x, int64_t) const
+    {
+        const float tmp = (float)x * src_scale;
+        return clamp_s8(round_half_up_f32(tmp * inv_scale));
+    }
+};
+
+// prelu_11c<int8_t, int16_t> (esp-dl/dl/base/dl_base_prelu.cpp:7-21)
+struct PreluFn {
+    const int8_t *alpha;
+    int channels, shift;
+    __device__ void prepare() {}
+    __device__ int operator()(int x, int64_t idx) const
+    {
+        if (x >= 0)
+            return x;
+        const int prod = x * (int)alpha[idx % channels];
+        const int shifted = shift > 0 ? (prod >> shift) : (int)((unsigned)prod << -shift);
+        return clamp_s8((int)(int16_t)shifted);
+    }
+};
+
+template <typename F>
+hipError_t launch_map(const int8_t *in, int8_t *out, int64_t size, F f, hipStream_t stream)
+{
+    if (size <= 0)
+        return hipSuccess;
+    int64_t vecs;
+    const dim3 grid = grid_for(size, aligned16(in, out), &vecs);
+    hipLaunchKernelGGL(map_s8_kernel<F>, grid, dim3(kBlock), 0, stream, in, out, size, vecs, f);
+    return hipGetLastError();
+}
+
+// c_impl_add_n_n / _n_1 / _1_n (esp-dl/dl/base/dl_base_add.cpp:8-44): clamp(a + b).
+__global__ __launch_bounds__(kBlock) void add_s8_dense_kernel(const int8_t *in0, const int8_t *in1, int8_t *out,
+                                                              int64_t size, int64_t vecs)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < vecs) {
+        const v4i a = reinterpret_cast<const v4i *>(in0)[i];
+        const v4i b = reinterpret_cast<const v4i *>(in1)[i];
+        v4i r;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            int o = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int s = (int)(int8_t)(a[w] >> (8 * k)) + (int)(int8_t)(b[w] >> (8 * k));
+                o |= (clamp_s8(s) & 0xff) << (8 * k);
+            }
+            r[w] = o;
+        }
+        reinterpret_cast<v4i *>(out)[i] = r;
+    }
+    const int64_t t = vecs * 16 + i;
+    if (t < size)
+        out[t] = (int8_t)clamp_s8((int)in0[t] + (int)in1[t]);
+}
+
+struct AddBroadcastArgs {
+    int d[4];
+    long long s0[4], s1[4];
+};
+
+__global__ __launch_bounds__(kBlock) void add_s8_broadcast_kernel(const int8_t *in0, const int8_t *in1, int8_t *out,
+                                                                  int64_t size, AddBroadcastArgs a)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= size)
+        return;
+    int64_t rest = i;
+    const int i3 = (int)(rest % a.d[3]);
+    rest /= a.d[3];
+    const int i2 = (int)(rest % a.d[2]);
+    rest /= a.d[2];
+    const int i1 = (int)(rest % a.d[1]);
+    const int i0 = (int)(rest / a.d[1]);
+    const long long o0 = i0 * a.s0[0] + i1 * a.s0[1] + i2 * a.s0[2] + i3 * a.s0[3];
+    const long long o1 = i0 * a.s1[0] + i1 * a.s1[1] + i2 * a.s1[2] + i3 * a.s1[3];
+    out[i] = (int8_t)clamp_s8((int)in0[o0] + (int)in1[o1]);
+}
+
+// GlobalAveragePool: avgpool2d_hwc with the window covering the image
+// (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54).  One workgroup per (image, 64-channel slab): 64 lanes
+// along channels (contiguous), 4 wavefronts split the pixels, int32 partial sums meet in LDS.
+__global__ __launch_bounds__(kBlock) void global_avg_pool_s8_kernel(const int8_t *in, int8_t *out, int hw, int c,
+                                                                    float scale)
+{
+    __shared__ int partial[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int ch = blockIdx.x * 64 + lane;
+    const int8_t *img = in + (long long)blockIdx.y * hw * c;
+    int sum = 0;
+    if (ch < c)
+        for (int p = wave; p < hw; p += 4)
+            sum += img[(long long)p * c + ch];
+    partial[wave][lane] = sum;
+    __syncthreads();
+    if (wave == 0 && ch < c) {
+        sum = partial[0][lane] + partial[1][lane] + partial[2][lane] + partial[3][lane];
+        out[(long long)blockIdx.y * c + ch] = (int8_t)clamp_s8(round_half_up_f32((float)sum * scale));
+    }
+}
+
+} // namespace
+
+hipError_t launch_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out, hipStream_t stream)
+{
+    return launch_map(in, out, size, LutFn{table, nullptr}, stream);
+}
+
+hipError_t launch_prelu_s8(const int8_t *in, int64_t pixels, int channels, const int8_t *alpha, int shift,
+                           int8_t *out, hipStream_t stream)
+{
+    return launch_map(in, out, pixels * channels, PreluFn{alpha, channels, shift}, stream);
+}
+
+hipError_t launch_relu_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out, hipStream_t stream)
+{
+    return launch_map(in, out, size, ReluFn{in_exp == out_exp, dl_scale(in_exp), dl_rescale(out_exp)}, stream);
+}
+
+hipError_t launch_clip_s8(const int8_t *in, int64_t size, int min_q, int max_q, int in_exp, int out_exp, int8_t *out,
+                          hipStream_t stream)
+{
+    return launch_map(in, out, size, ClipFn{min_q, max_q, dl_scale(in_exp) * dl_rescale(out_exp)}, stream);
+}
+
+hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out,
+                                hipStream_t stream)
+{
+    if (in_exp == out_exp) {
+        if (in == out || size <= 0)
+            return hipSuccess;
+        return hipMemcpyAsync(out, in, (size_t)size, hipMemcpyDeviceToDevice, stream);
+    }
+    const float inv = (float)(1.0 / (double)dl_scale(out_exp));
+    return launch_map(in, out, size, RequantFn{dl_scale(in_exp), inv}, stream);
+}
+
+hipError_t launch_add_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
+                         const int8_t *in1, int8_t *out, hipStream_t stream)
+{
+    const int64_t size = (int64_t)dims[0] * dims[1] * dims[2] * dims[3];
+    if (size <= 0)
+        return hipSuccess;
+    // dense strides of the output shape
+    int64_t dense[4];
+    dense[3] = 1;
+    for (int i = 2; i >= 0; i--)
+        dense[i] = dense[i + 1] * dims[i + 1];
+    bool both_dense = true;
+    for (int i = 0; i < 4; i++)
+        if (dims[i] > 1 && (s0[i] != dense[i] || s1[i] != dense[i]))
+            both_dense = false;
+    if (both_dense) {
+        const bool vec_ok = aligned16(in0, in1) && aligned16(out, out);
+        int64_t vecs;
+        const dim3 grid = grid_for(size, vec_ok, &vecs);
+        hipLaunchKernelGGL(add_s8_dense_kernel, grid, dim3(kBlock), 0, stream, in0, in1, out, size, vecs);
+    } else {
+        AddBroadcastArgs a;
+        for (int i = 0; i < 4; i++) {
+            a.d[i] = dims[i];
+            a.s0[i] = dims[i] > 1 ? s0[i] : 0;
+            a.s1[i] = dims[i] > 1 ? s1[i] : 0;
+        }
+        hipLaunchKernelGGL(add_s8_broadcast_kernel, dim3((unsigned)((size + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           stream, in0, in1, out, size, a);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
+                                     int8_t *out, hipStream_t stream)
+{
+    if (batch <= 0)
+        return hipSuccess;
+    const float area_inv = 1.f / (float)(h * w);
+    const float scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
+    hipLaunchKernelGGL(global_avg_pool_s8_kernel, dim3((unsigned)((c + 63) / 64), (unsigned)batch), dim3(kBlock), 0,
+                       stream, in, out, h * w, c, scale);
+    return hipGetLastError();
+}
+
+} // namespace espdl

@@ -1,0 +1,95 @@
+// Device-side integer helpers shared by the gfx950 kernels.
+//
+// The arithmetic restates tool::shift_and_round / tool::truncate of the reference
+// (esp-dl/dl/tool/src/dl_tool.cpp:95-146; esp-dl/dl/tool/include/dl_tool.hpp:225-254) in forms that
+// need no 64-bit intermediate on the int8 path.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace espdl {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ int clamp_s8(int v)
+{
+    return min(max(v, -128), 127);
+}
+
+// shift_and_round<int32_t> followed by optional ReLU and truncate(int8_t&, .).
+//   shift in 1..31 : floor((v + 2^(s-1)) / 2^s) == (v >> s) + bit(s-1) of v   (no overflow)
+//   shift >= 32    : the 64-bit sum v + 2^(s-1) is non-negative and below 2^s  -> 0
+//   shift <= 0     : saturate(int64(v) << -s); since the result is clamped to int8 afterwards,
+//                    clamping first and shifting by min(-s, 8) gives the same value.
+__device__ __forceinline__ int requant_s8(int v, int shift, bool relu, bool half_even)
+{
+    int q;
+    if (shift > 0) {
+        if (shift > 31) {
+            q = 0;
+        } else if (half_even) {
+            const unsigned mask = (1u << shift) - 1u;
+            const int rem = (int)((unsigned)v & mask);
+            const int half = (int)(1u << (shift - 1));
+            q = v >> shift;
+            q += (rem > half || (rem == half && (q & 1))) ? 1 : 0;
+        } else {
+            q = (v >> shift) + ((v >> (shift - 1)) & 1);
+        }
+    } else {
+        q = clamp_s8(v) << min(-shift, 8);
+    }
+    if (relu)
+        q = max(q, 0);
+    return clamp_s8(q);
+}
+
+// shift_and_round<int64_t> followed by optional ReLU and truncate(int16_t&, .).
+__device__ __forceinline__ int requant_s16(long long v, int shift, bool relu, bool half_even)
+{
+    long long q;
+    if (shift > 0) {
+        if (half_even) {
+            const unsigned long long mask = (1ull << shift) - 1ull;
+            const long long rem = (long long)((unsigned long long)v & mask);
+            const long long half = (long long)(1ull << (shift - 1));
+            q = v >> shift;
+            q += (rem > half || (rem == half && (q & 1))) ? 1 : 0;
+        } else {
+            q = (long long)((unsigned long long)v + (1ull << (shift - 1))) >> shift;
+        }
+    } else {
+        q = (long long)((unsigned long long)v << -shift);
+    }
+    if (relu && q < 0)
+        q = 0;
+    q = q < -32768 ? -32768 : (q > 32767 ? 32767 : q);
+    return (int)q;
+}
+
+// tool::round(float) of the portable build: (int)floorf(value + 0.5) where 0.5 is a double literal,
+// so the sum is formed in double and narrowed to float by floorf's parameter
+// (esp-dl/dl/tool/src/dl_tool.cpp:72-75).
+__device__ __forceinline__ int round_half_up_f32(float v)
+{
+    return (int)floorf((float)((double)v + 0.5));
+}
+
+// DL_SCALE / DL_RESCALE (esp-dl/dl/dl_define.hpp:75-81)
+__host__ __device__ __forceinline__ float dl_scale(int e)
+{
+    return e > 0 ? (float)(1 << e) : 1.0f / (float)(1 << -e);
+}
+__host__ __device__ __forceinline__ float dl_rescale(int e)
+{
+    return e > 0 ? 1.0f / (float)(1 << e) : (float)(1 << -e);
+}
+
+__device__ __forceinline__ int pack4_s8(int a, int b, int c, int d)
+{
+    return (a & 0xff) | ((b & 0xff) << 8) | ((c & 0xff) << 16) | ((d & 0xff) << 24);
+}
+
+} // namespace espdl

@@ -1,0 +1,298 @@
+// extern "C" entry points of libespdl_hip.so (declared in include/espdl_hip.h): argument
+// validation, geometry derivation and kernel dispatch.  No allocation, no synchronization.
+#include "../../include/espdl_hip.h"
+
+#include <climits>
+#include <cstdarg>
+#include <cstdio>
+
+#include "espdl_kernels.h"
+
+namespace {
+
+thread_local char g_last_error[256] = "";
+
+int fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int device_status(hipError_t e, const char *what)
+{
+    if (e == hipSuccess)
+        return ESPDL_HIP_OK;
+    return fail(ESPDL_HIP_EDEVICE, "%s: %s", what, hipGetErrorString(e));
+}
+
+int cu_count_cached()
+{
+    static thread_local int cached_dev = -1;
+    static thread_local int cached_cus = 0;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess)
+        return 0;
+    if (dev != cached_dev) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            cus = 0;
+        cached_dev = dev;
+        cached_cus = cus;
+    }
+    return cached_cus;
+}
+
+// Conv::get_output_shape (esp-dl/dl/module/include/dl_module_conv.hpp:90-98)
+int derive_geometry(const espdl_hip_conv_desc *d, espdl::ConvGeom *g)
+{
+    if (d == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "conv descriptor is NULL");
+    if (d->dtype != ESPDL_HIP_S8 && d->dtype != ESPDL_HIP_S16)
+        return fail(ESPDL_HIP_EINVAL, "dtype %d is neither ESPDL_HIP_S8 nor ESPDL_HIP_S16", d->dtype);
+    if (d->batch < 0 || d->in_h <= 0 || d->in_w <= 0 || d->in_c <= 0 || d->out_c <= 0)
+        return fail(ESPDL_HIP_EINVAL, "bad tensor extents: batch %d in %dx%dx%d out_c %d", d->batch, d->in_h, d->in_w,
+                    d->in_c, d->out_c);
+    if (d->k_h <= 0 || d->k_w <= 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->dil_h <= 0 || d->dil_w <= 0)
+        return fail(ESPDL_HIP_EINVAL, "filter size, stride and dilation must be positive");
+    if (d->pad_top < 0 || d->pad_bottom < 0 || d->pad_left < 0 || d->pad_right < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative padding");
+    if (d->group != 1 && !(d->group == d->in_c && d->out_c == d->in_c))
+        return fail(ESPDL_HIP_ENOTSUP, "group %d: only 1 (dense) or in_c with out_c == in_c (depthwise) are supported",
+                    d->group);
+    if (d->activation != ESPDL_HIP_LINEAR && d->activation != ESPDL_HIP_RELU)
+        return fail(ESPDL_HIP_ENOTSUP, "fused activation %d: only Linear and ReLU exist on this path", d->activation);
+    if (d->round_mode != ESPDL_HIP_ROUND_HALF_UP && d->round_mode != ESPDL_HIP_ROUND_HALF_EVEN)
+        return fail(ESPDL_HIP_EINVAL, "unknown round_mode %d", d->round_mode);
+    if (d->n_shift != 1 && d->n_shift != d->out_c)
+        return fail(ESPDL_HIP_EINVAL, "n_shift %d must be 1 or out_c (%d)", d->n_shift, d->out_c);
+    const long long span_h = (long long)d->in_h + d->pad_top + d->pad_bottom - (long long)d->dil_h * (d->k_h - 1) - 1;
+    const long long span_w = (long long)d->in_w + d->pad_left + d->pad_right - (long long)d->dil_w * (d->k_w - 1) - 1;
+    if (span_h < 0 || span_w < 0)
+        return fail(ESPDL_HIP_EINVAL, "filter window is larger than the padded input");
+    const long long oh = span_h / d->stride_h + 1, ow = span_w / d->stride_w + 1;
+    const long long k_total = (long long)d->k_h * d->k_w * d->in_c;
+    const long long in_elems = (long long)d->batch * d->in_h * d->in_w * d->in_c;
+    const long long out_elems = (long long)d->batch * oh * ow * d->out_c;
+    if (k_total > (1 << 24) || in_elems > (1ll << 40) || out_elems > (1ll << 40) || oh > INT_MAX || ow > INT_MAX ||
+        (long long)d->batch * oh * ow / 64 > INT_MAX / 2)
+        return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    g->batch = d->batch;
+    g->in_h = d->in_h;
+    g->in_w = d->in_w;
+    g->in_c = d->in_c;
+    g->out_c = d->out_c;
+    g->out_h = (int)oh;
+    g->out_w = (int)ow;
+    g->k_h = d->k_h;
+    g->k_w = d->k_w;
+    g->stride_h = d->stride_h;
+    g->stride_w = d->stride_w;
+    g->dil_h = d->dil_h;
+    g->dil_w = d->dil_w;
+    g->pad_top = d->pad_top;
+    g->pad_left = d->pad_left;
+    g->relu = d->activation == ESPDL_HIP_RELU;
+    g->half_even = d->round_mode == ESPDL_HIP_ROUND_HALF_EVEN;
+    g->n_shift = d->n_shift;
+    return ESPDL_HIP_OK;
+}
+
+bool misaligned(const void *p, uintptr_t a)
+{
+    return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0;
+}
+
+} // namespace
+
+extern "C" {
+
+const char *espdl_hip_last_error(void)
+{
+    return g_last_error;
+}
+
+const char *espdl_hip_version(void)
+{
+    return "espdl_hip 0.1 (gfx950)";
+}
+
+int espdl_hip_device_cu_count(void)
+{
+    return cu_count_cached();
+}
+
+int espdl_hip_conv_out_shape(const espdl_hip_conv_desc *desc, int32_t *out_h, int32_t *out_w)
+{
+    espdl::ConvGeom g;
+    const int rc = derive_geometry(desc, &g);
+    if (rc != ESPDL_HIP_OK)
+        return rc;
+    if (out_h)
+        *out_h = g.out_h;
+    if (out_w)
+        *out_w = g.out_w;
+    return ESPDL_HIP_OK;
+}
+
+int espdl_hip_conv2d(const espdl_hip_conv_desc *desc, const void *in, const void *filter, const void *bias,
+                     const int32_t *shift, const int8_t *lut, void *out, void *stream)
+{
+    espdl::ConvGeom g;
+    const int rc = derive_geometry(desc, &g);
+    if (rc != ESPDL_HIP_OK)
+        return rc;
+    if (g.batch == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || filter == nullptr || shift == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in, filter, shift and out must not be NULL");
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const bool depthwise = desc->group != 1;
+    if (desc->dtype == ESPDL_HIP_S8) {
+        if (misaligned(bias, 4) || misaligned(shift, 4))
+            return fail(ESPDL_HIP_EINVAL, "bias and shift must be 4-byte aligned");
+        const int8_t *i8 = static_cast<const int8_t *>(in);
+        const int8_t *f8 = static_cast<const int8_t *>(filter);
+        const int32_t *b32 = static_cast<const int32_t *>(bias);
+        int8_t *o8 = static_cast<int8_t *>(out);
+        if (depthwise)
+            return device_status(espdl::launch_depthwise_s8(g, i8, f8, b32, shift, lut, o8, s), "depthwise_s8");
+        return device_status(espdl::launch_conv2d_s8_mfma(g, i8, f8, b32, shift, lut, o8, cu_count_cached(), s),
+                             "conv2d_s8");
+    }
+    if (lut != nullptr)
+        return fail(ESPDL_HIP_ENOTSUP, "the fused LUT epilogue exists for ESPDL_HIP_S8 only");
+    if (misaligned(in, 2) || misaligned(filter, 2) || misaligned(out, 2) || misaligned(bias, 8) || misaligned(shift, 4))
+        return fail(ESPDL_HIP_EINVAL, "int16 tensors must be 2-byte aligned, int64 bias 8-byte aligned");
+    const int16_t *i16 = static_cast<const int16_t *>(in);
+    const int16_t *f16 = static_cast<const int16_t *>(filter);
+    const int64_t *b64 = static_cast<const int64_t *>(bias);
+    int16_t *o16 = static_cast<int16_t *>(out);
+    if (depthwise)
+        return device_status(espdl::launch_depthwise_s16(g, i16, f16, b64, shift, o16, s), "depthwise_s16");
+    return device_status(espdl::launch_conv2d_s16(g, i16, f16, b64, shift, o16, s), "conv2d_s16");
+}
+
+int espdl_hip_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out, void *stream)
+{
+    if (size < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size");
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || table == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in, table and out must not be NULL");
+    return device_status(espdl::launch_lut_s8(in, size, table, out, reinterpret_cast<hipStream_t>(stream)), "lut_s8");
+}
+
+int espdl_hip_prelu_s8(const int8_t *in, int64_t pixels, int32_t channels, const int8_t *alpha, int32_t shift,
+                       int8_t *out, void *stream)
+{
+    if (pixels < 0 || channels <= 0)
+        return fail(ESPDL_HIP_EINVAL, "bad extents: pixels %lld channels %d", (long long)pixels, channels);
+    if (pixels == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || alpha == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in, alpha and out must not be NULL");
+    if (shift < -15 || shift > 31)
+        return fail(ESPDL_HIP_EINVAL, "prelu shift %d outside [-15, 31]", shift);
+    return device_status(
+        espdl::launch_prelu_s8(in, pixels, channels, alpha, shift, out, reinterpret_cast<hipStream_t>(stream)),
+        "prelu_s8");
+}
+
+static int check_exps(int32_t in_exp, int32_t out_exp)
+{
+    if (in_exp < -30 || in_exp > 30 || out_exp < -30 || out_exp > 30)
+        return fail(ESPDL_HIP_EINVAL, "exponents %d / %d outside [-30, 30]", in_exp, out_exp);
+    return ESPDL_HIP_OK;
+}
+
+int espdl_hip_relu_s8(const int8_t *in, int64_t size, int32_t in_exp, int32_t out_exp, int8_t *out, void *stream)
+{
+    if (size < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size");
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_relu_s8(in, size, in_exp, out_exp, out, reinterpret_cast<hipStream_t>(stream)),
+                         "relu_s8");
+}
+
+int espdl_hip_clip_s8(const int8_t *in, int64_t size, int32_t min_q, int32_t max_q, int32_t in_exp, int32_t out_exp,
+                      int8_t *out, void *stream)
+{
+    if (size < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size");
+    if (min_q < -128 || max_q > 127)
+        return fail(ESPDL_HIP_EINVAL, "clip bounds [%d, %d] are not int8 values", min_q, max_q);
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(
+        espdl::launch_clip_s8(in, size, min_q, max_q, in_exp, out_exp, out, reinterpret_cast<hipStream_t>(stream)),
+        "clip_s8");
+}
+
+int espdl_hip_add_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int8_t *out, void *stream)
+{
+    if (out_dims == nullptr || in0_strides == nullptr || in1_strides == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "dims and strides must not be NULL");
+    long long size = 1;
+    for (int i = 0; i < 4; i++) {
+        if (out_dims[i] < 0 || in0_strides[i] < 0 || in1_strides[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative extent or stride in dim %d", i);
+        size *= out_dims[i];
+        if (size > (1ll << 40))
+            return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    }
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in0 == nullptr || in1 == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in0, in1 and out must not be NULL");
+    return device_status(
+        espdl::launch_add_s8(out_dims, in0_strides, in1_strides, in0, in1, out, reinterpret_cast<hipStream_t>(stream)),
+        "add_s8");
+}
+
+int espdl_hip_global_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t in_exp,
+                                 int32_t out_exp, int8_t *out, void *stream)
+{
+    if (batch < 0 || h <= 0 || w <= 0 || c <= 0 || (long long)h * w > (1 << 23) || batch > 65535)
+        return fail(ESPDL_HIP_EINVAL, "bad extents: batch %d, %dx%dx%d", batch, h, w, c);
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (batch == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_global_avg_pool_s8(in, batch, h, w, c, in_exp, out_exp, out,
+                                                          reinterpret_cast<hipStream_t>(stream)),
+                         "global_avg_pool_s8");
+}
+
+int espdl_hip_requantize_s8(const int8_t *in, int64_t size, int32_t in_exp, int32_t out_exp, int8_t *out,
+                            void *stream)
+{
+    if (size < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size");
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(
+        espdl::launch_requantize_s8(in, size, in_exp, out_exp, out, reinterpret_cast<hipStream_t>(stream)),
+        "requantize_s8");
+}
+
+} // extern "C"

@@ -1,0 +1,45 @@
+// Internal launch interface between the C ABI (espdl_hip_api.hip) and the kernel files.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace espdl {
+
+// Geometry every convolution kernel works from (derived once on the host by the C ABI).
+struct ConvGeom {
+    int batch, in_h, in_w, in_c;
+    int out_c, out_h, out_w;
+    int k_h, k_w, stride_h, stride_w, dil_h, dil_w, pad_top, pad_left;
+    int relu, half_even, n_shift;
+};
+
+// Dense int8 convolution / Gemm as an implicit GEMM on v_mfma_i32_16x16x64_i8.
+hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                 const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
+                                 hipStream_t stream);
+// Largest k_h * k_w * in_c the MFMA kernel accepts (weights of one 64-filter group must fit in LDS).
+int conv2d_s8_mfma_max_k();
+
+hipError_t launch_depthwise_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                               const int32_t *shift, const int8_t *lut, int8_t *out, hipStream_t stream);
+
+hipError_t launch_conv2d_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
+                             const int32_t *shift, int16_t *out, hipStream_t stream);
+hipError_t launch_depthwise_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
+                                const int32_t *shift, int16_t *out, hipStream_t stream);
+
+hipError_t launch_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out, hipStream_t stream);
+hipError_t launch_prelu_s8(const int8_t *in, int64_t pixels, int channels, const int8_t *alpha, int shift,
+                           int8_t *out, hipStream_t stream);
+hipError_t launch_relu_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out, hipStream_t stream);
+hipError_t launch_clip_s8(const int8_t *in, int64_t size, int min_q, int max_q, int in_exp, int out_exp, int8_t *out,
+                          hipStream_t stream);
+hipError_t launch_add_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
+                         const int8_t *in1, int8_t *out, hipStream_t stream);
+hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
+                                     int8_t *out, hipStream_t stream);
+hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out,
+                                hipStream_t stream);
+
+} // namespace espdl

@@ -1,0 +1,135 @@
+/*
+ * espdl_hip.h — C ABI of the MI355X (gfx950) kernels for ESP-DL's quantized operator path.
+ *
+ * Every entry point replaces one kernel-level interface of the reference's portable C path
+ * (esp-dl/dl/base); the reference file:line each one stands in for is cited at its declaration.
+ *
+ * Conventions
+ *   - All data pointers are DEVICE pointers (HBM).  Descriptors are host structs passed by pointer.
+ *   - Activations are NHWC with a leading batch dimension; the reference is batch-1, so a batch of
+ *     N is N independent reference calls on the N images.
+ *   - Dense filter memory is [out_c][k_h][k_w][in_c]; depthwise filter memory is [k_h][k_w][c]
+ *     (the reference's `c`-target layouts, dl_base_conv2d.cpp:23,64,140;
+ *     dl_base_depthwise_conv2d.cpp:46-65).
+ *   - `shift` is int32[n_shift] on the device, n_shift = 1 (per-tensor) or out_c (per-channel);
+ *     shift[i] = out_exponent - filter_exponent[i] - in_exponent (dl_base.hpp:260).
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls are
+ *     asynchronous on that stream and allocate nothing.
+ *   - Return value: ESPDL_HIP_OK (0) or a negative error code; nothing throws.  The message of the
+ *     last error of the calling thread is available from espdl_hip_last_error().
+ *   - Results are bit-exact with the reference's portable C path.  Supported shift range: int8
+ *     paths -31..62 (half-up) / -31..30 (half-even); int16 paths -15..62 (half-up) / -15..62.
+ */
+#ifndef ESPDL_HIP_H
+#define ESPDL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ESPDL_HIP_OK 0
+#define ESPDL_HIP_EINVAL (-22)   /* bad descriptor / null pointer / unsupported geometry */
+#define ESPDL_HIP_ENOTSUP (-95)  /* valid request the library does not implement          */
+#define ESPDL_HIP_EDEVICE (-5)   /* HIP runtime reported an error at launch                */
+
+/* element type of activations and filters: quant_type_t of the reference (dl_define.hpp:94-100) */
+#define ESPDL_HIP_S8 8
+#define ESPDL_HIP_S16 16
+
+/* activation_type_t of the reference (dl_define.hpp:102-108).  The portable C path fuses only
+ * Linear and ReLU into Conv/Gemm (dl_base_conv2d.cpp:1299-1329). */
+#define ESPDL_HIP_LINEAR 0
+#define ESPDL_HIP_RELU 1
+
+/* tool::shift_and_round flavour (dl_tool.cpp:95-146).  HALF_UP is the portable C path;
+ * HALF_EVEN is what ESP32-P4 builds select (dl_define_private.hpp:44-48). */
+#define ESPDL_HIP_ROUND_HALF_UP 0
+#define ESPDL_HIP_ROUND_HALF_EVEN 1
+
+/*
+ * Convolution descriptor: the fields base::ConvOpArgs<T> derives from its tensors and attributes
+ * (esp-dl/dl/base/dl_base.hpp:133-262), plus the batch size.
+ */
+typedef struct espdl_hip_conv_desc {
+    int32_t dtype; /* ESPDL_HIP_S8 or ESPDL_HIP_S16 */
+    int32_t batch, in_h, in_w, in_c;
+    int32_t out_c; /* dense: number of filters; depthwise: must equal in_c */
+    int32_t k_h, k_w;
+    int32_t stride_h, stride_w;
+    int32_t dil_h, dil_w;
+    int32_t pad_top, pad_bottom, pad_left, pad_right; /* ConvOpArgs padding order {t,b,l,r} */
+    int32_t group;      /* 1 = dense conv / Gemm / MatMul; in_c = depthwise (dl_module_conv.hpp:104-119) */
+    int32_t activation; /* ESPDL_HIP_LINEAR / ESPDL_HIP_RELU */
+    int32_t round_mode; /* ESPDL_HIP_ROUND_HALF_UP / ESPDL_HIP_ROUND_HALF_EVEN */
+    int32_t n_shift;    /* 1 or out_c */
+} espdl_hip_conv_desc;
+
+/* Output spatial size, Conv::get_output_shape (esp-dl/dl/module/include/dl_module_conv.hpp:81-102). */
+int espdl_hip_conv_out_shape(const espdl_hip_conv_desc *desc, int32_t *out_h, int32_t *out_w);
+
+/*
+ * Conv2D / DepthwiseConv2D / Gemm / MatMul with fused bias, shift-round, ReLU, saturation and an
+ * optional 256-entry int8 LUT applied to the stored value.
+ * Replaces base::conv2d<int8_t,int32_t,int32_t>, base::conv2d<int16_t,int32_t,int64_t>
+ * (esp-dl/dl/base/dl_base_conv2d.hpp:15-16; dl_base_conv2d.cpp:912-939, 1383-1411) and
+ * base::depthwise_conv2d<...> (esp-dl/dl/base/dl_base_depthwise_conv2d.cpp:495-519, 854-880)
+ * together with conv_operation_shell / dwconv_operation_shell (dl_base.hpp:382-1196, 1209-2107)
+ * and the n_wise epilogues (dl_base_activate_buffer.hpp:10-74, 162-212).
+ *   bias : int32[out_c] (S8) or int64[out_c] (S16), or NULL
+ *   lut  : int8[256] or NULL; S8 only.  out = lut[q + 128] as base::lut_s8 would compute on the
+ *          conv output (dl_base_lut.cpp:10-15), i.e. Conv followed by a LUT module in one pass.
+ * Gemm / MatMul: describe the input as {1, 1, M, K} with a 1x1 filter, as the reference does
+ * (esp-dl/dl/module/include/dl_module_gemm.hpp:86-123).
+ */
+int espdl_hip_conv2d(const espdl_hip_conv_desc *desc, const void *in, const void *filter, const void *bias,
+                     const int32_t *shift, const int8_t *lut, void *out, void *stream);
+
+/* base::lut_s8 (esp-dl/dl/base/dl_base_lut.cpp:10-48): out[i] = table[(uint8)in[i] ^ 0x80]. In-place allowed. */
+int espdl_hip_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out, void *stream);
+
+/* base::prelu<int8_t> (esp-dl/dl/base/dl_base_prelu.cpp:7-21, args dl_base.hpp:2165-2168):
+ * alpha is int8[channels]; shift = out_exp - in_exp - alpha_exp.  In-place allowed. */
+int espdl_hip_prelu_s8(const int8_t *in, int64_t pixels, int32_t channels, const int8_t *alpha, int32_t shift,
+                       int8_t *out, void *stream);
+
+/* module::Relu::forward_template (esp-dl/dl/module/include/dl_module_relu.hpp:65-93). In-place allowed. */
+int espdl_hip_relu_s8(const int8_t *in, int64_t size, int32_t in_exp, int32_t out_exp, int8_t *out, void *stream);
+
+/* module::Clip::forward_template (esp-dl/dl/module/include/dl_module_clip.hpp:78-90); min_q / max_q
+ * are the quantized scalar bounds.  In-place allowed. */
+int espdl_hip_clip_s8(const int8_t *in, int64_t size, int32_t min_q, int32_t max_q, int32_t in_exp,
+                      int32_t out_exp, int8_t *out, void *stream);
+
+/*
+ * base::elemwise_add for int8 (esp-dl/dl/base/dl_base_add.cpp:8-44, 80-153) with the broadcast
+ * description of base::elemwiseArgsType (esp-dl/dl/base/dl_base_elemwise.hpp:19-52): the output is a
+ * dense tensor of up to 4 dims `out_dims` (outermost first, unused leading dims = 1); each input is
+ * addressed with element strides per output dim (0 = broadcast along that dim).
+ * out = clamp(in0 + in1); exponents are not consulted (the exporter matches them).
+ */
+int espdl_hip_add_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int8_t *out, void *stream);
+
+/* GlobalAveragePool over H x W per image and channel: base::avgpool2d_hwc with the filter covering
+ * the whole image (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54). out is [batch][1][1][c]. */
+int espdl_hip_global_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t in_exp,
+                                 int32_t out_exp, int8_t *out, void *stream);
+
+/* TensorBase::assign int8 -> int8 across exponents (esp-dl/dl/tensor/src/dl_tensor_base.cpp:362-371),
+ * which is what a RequantizeLinear node runs. */
+int espdl_hip_requantize_s8(const int8_t *in, int64_t size, int32_t in_exp, int32_t out_exp, int8_t *out,
+                            void *stream);
+
+/* Library / device information. */
+const char *espdl_hip_last_error(void);
+const char *espdl_hip_version(void);
+/* Number of compute units of the current device (0 if none can be queried). */
+int espdl_hip_device_cu_count(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ESPDL_HIP_H */

@@ -1,0 +1,305 @@
+"""GPU parity: every C-ABI entry point against the CPU oracle on the same seeded inputs.
+Bit-exact equality is the bar for all of them (integer / byte work)."""
+import numpy as np
+import pytest
+
+from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, rng_int8, typical_shift
+from gpu_util import announce, espdl, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, depthwise=False, half_even=False, lut=None):
+    m = espdl()
+    act = m.capi.RELU if relu else m.capi.LINEAR
+    rm = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
+    shift = np.atleast_1d(np.asarray(shift, dtype=np.int32))
+    got = m.conv2d(to_dev(x), to_dev(f), to_dev(bias), to_dev(shift), k, stride, dil, pads, depthwise=depthwise,
+                   activation=act, round_mode=rm, lut=to_dev(lut))
+    fn = oracle.depthwise_s8 if depthwise else oracle.conv2d_s8
+    want = fn(x, f, bias, shift, k, stride, dil, pads, oracle.RELU if relu else oracle.LINEAR,
+              oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP)
+    if lut is not None:
+        want = oracle.lut_s8(want, lut)
+    return to_host(got), want
+
+
+def _conv_inputs(case, seed, n, per_channel):
+    name, (h, w, c), oc, k, stride, dil, pads, has_bias, relu = case
+    rng = np.random.default_rng(seed)
+    x = rng_int8(rng, (n, h, w, c))
+    f = rng_int8(rng, (oc, k[0], k[1], c))
+    bias = rng.integers(-4096, 4097, size=oc).astype(np.int32) if has_bias else None
+    base = typical_shift(k[0] * k[1] * c)
+    shift = (base + rng.integers(-2, 3, size=oc)).astype(np.int32) if per_channel else np.int32(base)
+    return x, f, bias, shift, k, stride, dil, pads, relu
+
+
+@pytest.mark.parametrize("case", CONV_CASES, ids=lambda c: c[0])
+@pytest.mark.parametrize("per_channel", [False, True], ids=["per_tensor", "per_channel"])
+def test_conv2d_s8(oracle, case, per_channel):
+    announce(f"conv2d_s8 {case[0]} per_channel={per_channel}")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 101, 3, per_channel)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_conv2d_s8_config1(oracle):
+    """BASELINE config 1: 1x56x56x64 -> 64, 3x3, s1, p1, bias in [-2^12, 2^12], ReLU, shift 9."""
+    announce("conv2d_s8 config1")
+    x, f, bias, _, k, stride, dil, pads, relu = _conv_inputs(CONFIG1, 0xE5D1, 1, False)
+    got, want = _run_conv_s8(oracle, x, f, bias, 9, k, stride, dil, pads, True)
+    assert got.shape == (1, 56, 56, 64)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_conv2d_s8_config1_batched(oracle):
+    announce("conv2d_s8 config1 batch 16")
+    x, f, bias, _, k, stride, dil, pads, relu = _conv_inputs(CONFIG1, 0xE5D2, 16, False)
+    got, want = _run_conv_s8(oracle, x, f, bias, 9, k, stride, dil, pads, True)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("shift", [-3, -1, 0, 1, 31, 33])
+def test_conv2d_s8_shift_range(oracle, shift):
+    announce(f"conv2d_s8 shift={shift}")
+    rng = np.random.default_rng(7)
+    x = rng.integers(-6, 7, size=(2, 5, 5, 8)).astype(np.int8)
+    f = rng.integers(-6, 7, size=(12, 1, 1, 8)).astype(np.int8)
+    bias = rng.integers(-50, 51, size=12).astype(np.int32)
+    if shift > 8:
+        bias = (bias.astype(np.int64) << 24).astype(np.int32)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), False)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", [CONV_CASES[5], CONV_CASES[13]], ids=lambda c: c[0])
+def test_conv2d_s8_half_even(oracle, case):
+    announce(f"conv2d_s8 half-even {case[0]}")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 103, 2, True)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, half_even=True)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_conv2d_s8_fused_lut(oracle):
+    announce("conv2d_s8 + LUT epilogue")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(CONV_CASES[16], 105, 2, True)
+    lut = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, False, lut=lut)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("k_total,oc", [(1280, 1000), (2304, 80), (960, 160), (576, 96)])
+def test_conv2d_s8_large_k(oracle, k_total, oc):
+    """Reduction lengths that exceed one LDS-resident filter chunk, and 1000 filters (not a multiple of 16)."""
+    announce(f"conv2d_s8 large K={k_total} oc={oc}")
+    rng = np.random.default_rng(k_total)
+    x = rng_int8(rng, (1, 1, 37, k_total))
+    f = rng_int8(rng, (oc, 1, 1, k_total))
+    bias = rng.integers(-4096, 4097, size=oc).astype(np.int32)
+    shift = (typical_shift(k_total) + rng.integers(-1, 2, size=oc)).astype(np.int32)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), False)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("m,k,n,has_bias,relu", GEMM_CASES)
+def test_gemm_s8(oracle, m, k, n, has_bias, relu):
+    announce(f"gemm_s8 M={m} K={k} N={n}")
+    rng = np.random.default_rng(107)
+    x = rng_int8(rng, (1, 1, m, k))
+    f = rng_int8(rng, (n, 1, 1, k))
+    bias = rng.integers(-4096, 4097, size=n).astype(np.int32) if has_bias else None
+    shift = (typical_shift(k) + rng.integers(-1, 2, size=n)).astype(np.int32)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), relu)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_gemm_reference_known_answers_on_gpu():
+    """The reference-held Gemm vectors, straight through the C ABI."""
+    import json
+    import os
+    announce("gemm reference fixtures")
+    m = espdl()
+    with open(os.path.join(os.path.dirname(__file__), "golden", "gemm_c_fixtures.json")) as f:
+        cases = json.load(f)
+    for case in cases:
+        _, _, k, n = case["filter_shape"]
+        x = np.array(case["input"], dtype=np.int8).reshape(1, 1, 1, k)
+        w = np.array(case["filter_bytes"], dtype=np.int8)
+        bias = np.array(case["bias"], dtype=np.int32)
+        shift = np.array([case["output_exponent"] - case["filter_exponents"][0] - case["input_exponent"]], np.int32)
+        act = m.capi.RELU if case["activation"] == "Relu" else m.capi.LINEAR
+        got = m.conv2d(to_dev(x), to_dev(w), to_dev(bias), to_dev(shift), (1, 1), activation=act)
+        np.testing.assert_array_equal(to_host(got).ravel(), np.array(case["output"], dtype=np.int8))
+
+
+@pytest.mark.parametrize("case", DW_CASES, ids=lambda c: c[0])
+@pytest.mark.parametrize("per_channel", [False, True], ids=["per_tensor", "per_channel"])
+def test_depthwise_s8(oracle, case, per_channel):
+    announce(f"depthwise_s8 {case[0]} per_channel={per_channel}")
+    name, (h, w, c), k, stride, dil, pads, has_bias, relu = case
+    rng = np.random.default_rng(109)
+    x = rng_int8(rng, (3, h, w, c))
+    f = rng_int8(rng, (k[0], k[1], c))
+    bias = rng.integers(-4096, 4097, size=c).astype(np.int32) if has_bias else None
+    base = typical_shift(k[0] * k[1])
+    shift = (base + rng.integers(-2, 3, size=c)).astype(np.int32) if per_channel else np.int32(base)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, depthwise=True)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_depthwise_s8_config2_shape(oracle):
+    announce("depthwise_s8 56x56x144 batch 4")
+    rng = np.random.default_rng(111)
+    x = rng_int8(rng, (4, 56, 56, 144))
+    f = rng_int8(rng, (3, 3, 144))
+    bias = rng.integers(-4096, 4097, size=144).astype(np.int32)
+    shift = rng.integers(6, 11, size=144).astype(np.int32)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, depthwise=True)
+    np.testing.assert_array_equal(got, want)
+
+
+def _run_conv_s16(oracle, x, f, bias, shift, k, stride, dil, pads, relu, depthwise):
+    m = espdl()
+    act = m.capi.RELU if relu else m.capi.LINEAR
+    got = m.conv2d(to_dev(x), to_dev(f), to_dev(bias), to_dev(np.atleast_1d(shift).astype(np.int32)), k, stride, dil,
+                   pads, depthwise=depthwise, activation=act)
+    fn = oracle.depthwise_s16 if depthwise else oracle.conv2d_s16
+    want = fn(x, f, bias, shift, k, stride, dil, pads, oracle.RELU if relu else oracle.LINEAR)
+    return to_host(got), want
+
+
+@pytest.mark.parametrize("case", [CONV_CASES[1], CONV_CASES[4], CONV_CASES[5], CONV_CASES[7], CONV_CASES[12]],
+                         ids=lambda c: c[0])
+def test_conv2d_s16(oracle, case):
+    announce(f"conv2d_s16 {case[0]}")
+    name, (h, w, c), oc, k, stride, dil, pads, has_bias, relu = case
+    rng = np.random.default_rng(113)
+    x = rng.integers(-32768, 32768, size=(2, h, w, c)).astype(np.int16)
+    f = rng.integers(-32768, 32768, size=(oc, k[0], k[1], c)).astype(np.int16)
+    bias = rng.integers(-2**28, 2**28, size=oc).astype(np.int64) if has_bias else None
+    shift = (typical_shift(k[0] * k[1] * c) + 16 + rng.integers(-2, 3, size=oc)).astype(np.int32)
+    got, want = _run_conv_s16(oracle, x, f, bias, shift, k, stride, dil, pads, relu, False)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", [DW_CASES[1], DW_CASES[2], DW_CASES[5], DW_CASES[10]], ids=lambda c: c[0])
+def test_depthwise_s16(oracle, case):
+    announce(f"depthwise_s16 {case[0]}")
+    name, (h, w, c), k, stride, dil, pads, has_bias, relu = case
+    rng = np.random.default_rng(115)
+    x = rng.integers(-32768, 32768, size=(2, h, w, c)).astype(np.int16)
+    f = rng.integers(-32768, 32768, size=(k[0], k[1], c)).astype(np.int16)
+    bias = rng.integers(-2**28, 2**28, size=c).astype(np.int64) if has_bias else None
+    shift = (typical_shift(k[0] * k[1]) + 16 + rng.integers(-2, 3, size=c)).astype(np.int32)
+    got, want = _run_conv_s16(oracle, x, f, bias, shift, k, stride, dil, pads, relu, True)
+    np.testing.assert_array_equal(got, want)
+
+
+# --------------------------------------------------------------------------- elementwise
+SIZES = [1, 7, 8, 15, 16, 63, 64, 1011, 1024, 100003]
+
+
+@pytest.mark.parametrize("size", SIZES)
+def test_lut_s8(oracle, size):
+    announce(f"lut_s8 size={size}")
+    m = espdl()
+    table = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8)
+    rng = np.random.default_rng(size)
+    x = rng_int8(rng, (size,))
+    edge = np.array([-128, -127, -1, 0, 1, 126, 127], dtype=np.int8)
+    x[:min(size, 7)] = edge[:min(size, 7)]
+    got = to_host(m.lut_s8(to_dev(x), to_dev(table)))
+    np.testing.assert_array_equal(got, oracle.lut_s8(x, table))
+    # in place, and from an address that is not 16-byte aligned
+    import torch
+    buf = torch.zeros(size + 3, dtype=torch.int8, device="cuda")
+    view = buf[3:]
+    view.copy_(torch.from_numpy(x))
+    m.lut_s8(view, to_dev(table), out=view)
+    np.testing.assert_array_equal(to_host(view), oracle.lut_s8(x, table))
+
+
+@pytest.mark.parametrize("shift", [-1, 0, 3, 6])
+def test_prelu_s8(oracle, shift):
+    announce(f"prelu_s8 shift={shift}")
+    m = espdl()
+    xs, _ = np.meshgrid(np.arange(-128, 128), np.arange(-128, 128), indexing="ij")
+    x = xs.astype(np.int8).reshape(1, 16, 16, 256)
+    alpha = np.arange(-128, 128).astype(np.int8)
+    got = to_host(m.prelu_s8(to_dev(x), to_dev(alpha), shift))
+    np.testing.assert_array_equal(got, oracle.prelu_s8(x, alpha, shift))
+    rng = np.random.default_rng(3)
+    x = rng_int8(rng, (1, 20, 20, 20))
+    alpha = rng_int8(rng, (20,))
+    got = to_host(m.prelu_s8(to_dev(x), to_dev(alpha), shift))
+    np.testing.assert_array_equal(got, oracle.prelu_s8(x, alpha, shift))
+
+
+def test_relu_clip_requantize_s8(oracle):
+    announce("relu/clip/requantize")
+    m = espdl()
+    rng = np.random.default_rng(5)
+    x = np.concatenate([np.arange(-128, 128).astype(np.int8), rng_int8(rng, (5000,))])
+    xd = to_dev(x)
+    np.testing.assert_array_equal(to_host(m.relu_s8(xd)), oracle.relu_s8(x))
+    for in_exp, out_exp in ((-6, -5), (-5, -7), (-4, -4), (-7, -3), (-3, -6)):
+        np.testing.assert_array_equal(to_host(m.relu_s8(xd, in_exp, out_exp)), oracle.relu_s8(x, in_exp, out_exp))
+        np.testing.assert_array_equal(to_host(m.clip_s8(xd, 0, 96, in_exp, out_exp)),
+                                      oracle.clip_s8(x, 0, 96, in_exp, out_exp))
+        np.testing.assert_array_equal(to_host(m.clip_s8(xd, -100, 127, in_exp, out_exp)),
+                                      oracle.clip_s8(x, -100, 127, in_exp, out_exp))
+        np.testing.assert_array_equal(to_host(m.requantize_s8(xd, in_exp, out_exp)),
+                                      oracle.requantize_s8(x, in_exp, out_exp))
+
+
+ADD_SHAPES = [
+    ((1, 96, 5, 48), (1, 96, 5, 48)), ((1, 96, 5, 48), (1, 96, 5, 1)), ((1, 96, 5, 1), (1, 96, 5, 48)),
+    ((1, 5, 5, 31), (1, 1, 1, 31)), ((2, 3, 4, 5), (1, 1, 1, 1)), ((1, 1, 4, 5), (2, 3, 4, 5)),
+    ((1, 1, 4, 5), (2, 3, 1, 1)), ((10, 1, 5, 5), (1, 1, 5, 5)), ((1, 512, 7, 7), (1, 512, 7, 7)),
+    ((5,), (1,)), ((2, 5), (2, 1)), ((8, 2, 5), (2, 1)), ((1, 96, 5, 49), (1, 96, 5, 49)),
+    ((4, 56, 56, 24), (4, 56, 56, 24)),
+]
+
+
+@pytest.mark.parametrize("sa,sb", ADD_SHAPES)
+def test_add_s8(oracle, sa, sb):
+    announce(f"add_s8 {sa} + {sb}")
+    m = espdl()
+    rng = np.random.default_rng(len(sa) * 100 + len(sb))
+    a, b = rng_int8(rng, sa), rng_int8(rng, sb)
+    got = to_host(m.add_s8(to_dev(a), to_dev(b)))
+    want = np.clip(a.astype(np.int32) + b.astype(np.int32), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(got, want)
+    if a.size == b.size or a.size == 1 or b.size == 1:
+        np.testing.assert_array_equal(got.ravel(), oracle.add_s8(a, b).ravel())
+
+
+def test_global_avg_pool_s8(oracle):
+    announce("global_avg_pool_s8")
+    m = espdl()
+    rng = np.random.default_rng(9)
+    for shape in ((3, 7, 7, 1280), (2, 5, 3, 33), (1, 1, 1, 8)):
+        x = rng_int8(rng, shape)
+        for in_exp, out_exp in ((-4, -5), (-5, -5), (-3, -6), (-6, -4)):
+            got = to_host(m.global_avg_pool_s8(to_dev(x), in_exp, out_exp))
+            np.testing.assert_array_equal(got, oracle.global_avg_pool_s8(x, in_exp, out_exp))
+    x = np.full((1, 7, 7, 64), 127, dtype=np.int8)
+    x[..., ::2] = -128
+    got = to_host(m.global_avg_pool_s8(to_dev(x), -4, -4))
+    np.testing.assert_array_equal(got, oracle.global_avg_pool_s8(x, -4, -4))
+
+
+def test_bad_arguments_are_rejected():
+    announce("argument validation")
+    m = espdl()
+    import torch
+    x = torch.zeros((1, 2, 2, 4), dtype=torch.int8, device="cuda")
+    f = torch.zeros((4, 5, 5, 4), dtype=torch.int8, device="cuda")
+    s = torch.zeros(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(m.EspdlHipError):
+        m.conv2d(x, f, None, s, (5, 5))  # window larger than the input
+    with pytest.raises(m.EspdlHipError):
+        m.conv2d(x, f, None, torch.zeros(3, dtype=torch.int32, device="cuda"), (1, 1))  # n_shift neither 1 nor out_c
+    empty = torch.zeros((0, 2, 2, 4), dtype=torch.int8, device="cuda")
+    assert m.conv2d(empty, torch.zeros((4, 1, 1, 4), dtype=torch.int8, device="cuda"), None, s, (1, 1)).shape[0] == 0
