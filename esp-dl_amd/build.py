@@ -51,8 +51,38 @@ def build_kernels(verbose=True):
     return out
 
 
+DL_DIR = os.path.join(HERE, "dl")
+DL_SOURCES = ["dl_tensor_base.cpp", "fbs_model.cpp", "dl_model_context.cpp", "dl_module_base.cpp", "dl_model_base.cpp",
+              "espdl_model_capi.cpp"]
+INCLUDE_DIR = os.path.join(os.path.dirname(HERE), "include")
+
+
+def build_host_layer(verbose=True):
+    """libespdl_dl.so: the C++ `dl::` host layer (TensorBase, Module, Model) + its C handle API."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    inc = ["-I" + os.path.join(DL_DIR, "include"), "-I" + INCLUDE_DIR]
+    srcs = [os.path.join(DL_DIR, "src", s) for s in DL_SOURCES]
+
+    def comp(src):
+        obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
+        warn = _run([HIPCC, "-x", "hip", "--offload-arch=" + ARCH, "-O2", "-fPIC", "-std=c++17", "-Wall",
+                     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", *inc, "-c", src, "-o", obj])
+        return obj, warn
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        results = list(pool.map(comp, srcs))
+    for (obj, warn), src in zip(results, srcs):
+        if warn.strip() and verbose:
+            print("[%s]\n%s" % (os.path.basename(src), warn), file=sys.stderr)
+    out = os.path.join(LIB_DIR, "libespdl_dl.so")
+    _run([HIPCC, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", out, *[o for o, _ in results],
+          "-L" + LIB_DIR, "-lespdl_hip", "-Wl,-rpath,$ORIGIN"])
+    return out
+
+
 def build_all(verbose=True):
-    return [build_kernels(verbose)]
+    return [build_kernels(verbose), build_host_layer(verbose)]
 
 
 if __name__ == "__main__":

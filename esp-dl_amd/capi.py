@@ -49,8 +49,9 @@ def lib():
                                        vp, vp, vp, vp]
         L.espdl_hip_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp]
         L.espdl_hip_requantize_s8.argtypes = [vp, i64, i32, i32, vp, vp]
+        L.espdl_hip_requantize.argtypes = [vp, i32, i64, i32, i32, vp, i32, vp]
         for name in ("conv_out_shape", "conv2d", "lut_s8", "prelu_s8", "relu_s8", "clip_s8", "add_s8",
-                     "global_avg_pool_s8", "requantize_s8", "device_cu_count"):
+                     "global_avg_pool_s8", "requantize_s8", "requantize", "device_cu_count"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         L.espdl_hip_last_error.restype = ctypes.c_char_p
         L.espdl_hip_version.restype = ctypes.c_char_p
@@ -177,4 +178,15 @@ def requantize_s8(x, in_exp, out_exp, out=None, stream=None):
     import torch
     out = torch.empty_like(x) if out is None else out
     _check(lib().espdl_hip_requantize_s8(_p(x), x.numel(), in_exp, out_exp, _p(out), _stream(stream)))
+    return out
+
+
+def requantize(x, in_exp, out_exp, out_dtype=None, out=None, stream=None):
+    """int8 / int16 -> int8 / int16 across exponents (TensorBase::assign)."""
+    import torch
+    out_dtype = x.dtype if out_dtype is None else out_dtype
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device) if out is None else out
+    bits = lambda d: S16 if d == torch.int16 else S8  # noqa: E731
+    _check(lib().espdl_hip_requantize(_p(x), bits(x.dtype), x.numel(), in_exp, out_exp, _p(out), bits(out.dtype),
+                                      _stream(stream)))
     return out

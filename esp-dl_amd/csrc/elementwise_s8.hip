@@ -236,6 +236,48 @@ hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int 
     return launch_map(in, out, size, RequantFn{dl_scale(in_exp), inv}, stream);
 }
 
+// TensorBase::assign between int8 / int16 (esp-dl/dl/tensor/src/dl_tensor_base.cpp:321-392).
+template <typename ST, typename DT>
+__global__ __launch_bounds__(kBlock) void requantize_any_kernel(const ST *in, DT *out, int64_t size, int same_exp,
+                                                                float src_scale, float inv_scale)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= size)
+        return;
+    const int lo = sizeof(DT) == 1 ? -128 : -32768, hi = sizeof(DT) == 1 ? 127 : 32767;
+    int q;
+    if (same_exp) {
+        q = (int)in[i];
+    } else {
+        const float tmp = (float)in[i] * src_scale;
+        q = round_half_up_f32(tmp * inv_scale);
+    }
+    out[i] = (DT)min(max(q, lo), hi);
+}
+
+hipError_t launch_requantize_any(const void *in, int in_bits, int64_t size, int in_exp, int out_exp, void *out,
+                                 int out_bits, hipStream_t stream)
+{
+    if (size <= 0)
+        return hipSuccess;
+    const dim3 grid((unsigned)((size + kBlock - 1) / kBlock));
+    const int same = in_exp == out_exp;
+    const float src = dl_scale(in_exp), inv = (float)(1.0 / (double)dl_scale(out_exp));
+    if (in_bits == 8 && out_bits == 16)
+        hipLaunchKernelGGL((requantize_any_kernel<int8_t, int16_t>), grid, dim3(kBlock), 0, stream,
+                           static_cast<const int8_t *>(in), static_cast<int16_t *>(out), size, same, src, inv);
+    else if (in_bits == 16 && out_bits == 8)
+        hipLaunchKernelGGL((requantize_any_kernel<int16_t, int8_t>), grid, dim3(kBlock), 0, stream,
+                           static_cast<const int16_t *>(in), static_cast<int8_t *>(out), size, same, src, inv);
+    else if (in_bits == 16 && out_bits == 16)
+        hipLaunchKernelGGL((requantize_any_kernel<int16_t, int16_t>), grid, dim3(kBlock), 0, stream,
+                           static_cast<const int16_t *>(in), static_cast<int16_t *>(out), size, same, src, inv);
+    else
+        hipLaunchKernelGGL((requantize_any_kernel<int8_t, int8_t>), grid, dim3(kBlock), 0, stream,
+                           static_cast<const int8_t *>(in), static_cast<int8_t *>(out), size, same, src, inv);
+    return hipGetLastError();
+}
+
 hipError_t launch_add_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
                          const int8_t *in1, int8_t *out, hipStream_t stream)
 {

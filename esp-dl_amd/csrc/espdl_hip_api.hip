@@ -295,4 +295,27 @@ int espdl_hip_requantize_s8(const int8_t *in, int64_t size, int32_t in_exp, int3
         "requantize_s8");
 }
 
+int espdl_hip_requantize(const void *in, int32_t in_dtype, int64_t size, int32_t in_exp, int32_t out_exp, void *out,
+                         int32_t out_dtype, void *stream)
+{
+    if (size < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size");
+    if ((in_dtype != ESPDL_HIP_S8 && in_dtype != ESPDL_HIP_S16) || (out_dtype != ESPDL_HIP_S8 && out_dtype != ESPDL_HIP_S16))
+        return fail(ESPDL_HIP_EINVAL, "dtypes must be ESPDL_HIP_S8 or ESPDL_HIP_S16");
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    if ((in_dtype == ESPDL_HIP_S16 && misaligned(in, 2)) || (out_dtype == ESPDL_HIP_S16 && misaligned(out, 2)))
+        return fail(ESPDL_HIP_EINVAL, "int16 tensors must be 2-byte aligned");
+    if (in_dtype == ESPDL_HIP_S8 && out_dtype == ESPDL_HIP_S8)
+        return espdl_hip_requantize_s8(static_cast<const int8_t *>(in), size, in_exp, out_exp,
+                                       static_cast<int8_t *>(out), stream);
+    return device_status(espdl::launch_requantize_any(in, in_dtype, size, in_exp, out_exp, out, out_dtype,
+                                                      reinterpret_cast<hipStream_t>(stream)),
+                         "requantize");
+}
+
 } // extern "C"

@@ -42,4 +42,7 @@ hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, 
 hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out,
                                 hipStream_t stream);
 
+hipError_t launch_requantize_any(const void *in, int in_bits, int64_t size, int in_exp, int out_exp, void *out,
+                                 int out_bits, hipStream_t stream);
+
 } // namespace espdl

@@ -1,0 +1,212 @@
+// dl::module::Conv — Conv2D / DepthwiseConv2D / Conv1D operator object.
+//
+// Mirrors esp-dl/dl/module/include/dl_module_conv.hpp:17-239: attributes (activation, pads
+// {top,bottom,left,right}, dilations, strides, group), get_output_shape (:81-102), forward (:121-162),
+// deserialize with the ONNX pad re-ordering [t,l,b,r] -> [t,b,l,r] (:167-195).  group == 1 is a dense
+// convolution, anything else a depthwise one (:104-119).  forward() derives
+// shift[c] = out_exp - filter_exp[c] - in_exp (esp-dl/dl/base/dl_base.hpp:243-261) and enqueues
+// espdl_hip_conv2d; an optional 256-entry table fuses a following LUT module into the epilogue.
+#pragma once
+
+#include <cassert>
+
+#include "dl_module_base.hpp"
+#include "espdl_hip.h"
+
+namespace dl {
+namespace module {
+
+/// Fill the requantization shifts of a Conv / Gemm / MatMul from the tensors' exponents.
+inline std::vector<int32_t> conv_shifts(TensorBase *output, TensorBase *input, TensorBase *filter, int out_c)
+{
+    std::vector<int32_t> shifts;
+    if (filter->exponent.is_per_channel()) {
+        shifts.resize(out_c);
+        for (int c = 0; c < out_c; c++)
+            shifts[c] = output->exponent.get() - filter->exponent.get(c) - input->exponent.get();
+    } else {
+        shifts.push_back(output->exponent.get() - filter->exponent.get() - input->exponent.get());
+    }
+    return shifts;
+}
+
+class Conv : public Module {
+private:
+    activation_type_t activation;
+    std::vector<int> m_pads;      ///< {top, bottom, left, right} (2-D) or {left, right} (1-D)
+    std::vector<int> m_dilations; ///< {h, w} or {w}
+    std::vector<int> m_strides;   ///< {h, w} or {w}
+    int m_group;
+    TensorBase *m_fused_lut; ///< device int8[256] applied to the stored value, or nullptr (owned)
+    DeviceInts m_shift;
+
+public:
+    Conv(activation_type_t activation = Linear, std::vector<int> pads = {}, std::vector<int> dilations = {},
+         std::vector<int> strides = {}, const char *name = nullptr, int group = 1,
+         quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type),
+        activation(activation),
+        m_pads(pads),
+        m_dilations(dilations),
+        m_strides(strides),
+        m_group(group),
+        m_fused_lut(nullptr)
+    {
+    }
+    ~Conv() { delete m_fused_lut; }
+
+    int get_group() const { return m_group; }
+    activation_type_t get_activation() const { return activation; }
+    /// Take ownership of a LUT (host or device tensor of 256 int8) to apply in the epilogue.
+    void fuse_lut(TensorBase *table)
+    {
+        delete m_fused_lut;
+        m_fused_lut = table;
+    }
+    bool has_fused_lut() const { return m_fused_lut != nullptr; }
+
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        assert(input_shapes.size() >= 2);
+        assert(input_shapes[0].size() == 3 || input_shapes[0].size() == 4);
+        std::vector<int> input_shape = input_shapes[0];
+        std::vector<int> filter_shape = input_shapes[1];
+        std::vector<int> output_shape = input_shape;
+        if (input_shape.size() == 3) {
+            // [N, W, C], filter [kW, Cin, Cout] (dense) / [kW, 1, C] (depthwise)
+            output_shape[1] = (input_shape[1] + m_pads[0] + m_pads[1] - m_dilations[0] * (filter_shape[0] - 1) - 1) /
+                    m_strides[0] +
+                1;
+            output_shape[2] = m_group == 1 ? filter_shape[2] : input_shape[2];
+        } else {
+            output_shape[1] = (input_shape[1] + m_pads[0] + m_pads[1] - m_dilations[0] * (filter_shape[0] - 1) - 1) /
+                    m_strides[0] +
+                1;
+            output_shape[2] = (input_shape[2] + m_pads[2] + m_pads[3] - m_dilations[1] * (filter_shape[1] - 1) - 1) /
+                    m_strides[1] +
+                1;
+            output_shape[3] = m_group == 1 ? filter_shape[3] : input_shape[3];
+        }
+        return {output_shape};
+    }
+
+    int64_t get_macs(std::vector<std::vector<int>> &input_shapes)
+    {
+        std::vector<int> out = get_output_shape(input_shapes)[0];
+        const std::vector<int> &f = input_shapes[1];
+        int64_t pixels = 1;
+        for (size_t i = 0; i + 1 < out.size(); i++)
+            pixels *= out[i];
+        const int64_t taps = out.size() == 3 ? f[0] : (int64_t)f[0] * f[1];
+        const int64_t in_c = m_group == 1 ? input_shapes[0].back() : 1;
+        return pixels * out.back() * taps * in_c;
+    }
+
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *filter = context->get_tensor(m_inputs_index[1]);
+        TensorBase *bias = m_inputs_index.size() == 3 ? context->get_tensor(m_inputs_index[2]) : nullptr;
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!input || !filter || !output || !input->on_device() || !filter->on_device() || !output->on_device() ||
+            (bias && !bias->on_device())) {
+            DL_LOGE("Conv", "%s: tensors must be device tensors", name.c_str());
+            return;
+        }
+
+        espdl_hip_conv_desc d = {};
+        d.dtype = quant_type == QUANT_TYPE_SYMM_16BIT ? ESPDL_HIP_S16 : ESPDL_HIP_S8;
+        d.batch = input->shape[0];
+        if (input->shape.size() == 3) {
+            d.in_h = 1;
+            d.in_w = input->shape[1];
+            d.in_c = input->shape[2];
+            d.out_c = output->shape[2];
+            d.k_h = 1;
+            d.k_w = filter->shape[0];
+            d.stride_h = 1;
+            d.stride_w = m_strides[0];
+            d.dil_h = 1;
+            d.dil_w = m_dilations[0];
+            d.pad_left = m_pads[0];
+            d.pad_right = m_pads[1];
+        } else if (input->shape.size() == 4) {
+            d.in_h = input->shape[1];
+            d.in_w = input->shape[2];
+            d.in_c = input->shape[3];
+            d.out_c = output->shape[3];
+            d.k_h = filter->shape[0];
+            d.k_w = filter->shape[1];
+            d.stride_h = m_strides[0];
+            d.stride_w = m_strides[1];
+            d.dil_h = m_dilations[0];
+            d.dil_w = m_dilations[1];
+            d.pad_top = m_pads[0];
+            d.pad_bottom = m_pads[1];
+            d.pad_left = m_pads[2];
+            d.pad_right = m_pads[3];
+        } else {
+            DL_LOGE("Conv", "Do not support input shape.");
+            return;
+        }
+        d.group = m_group == 1 ? 1 : d.in_c;
+        d.activation = activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR;
+        if (activation != Linear && activation != ReLU) {
+            DL_LOGE("Conv", "%s: only Linear and ReLU can be fused into Conv", name.c_str());
+            return;
+        }
+        d.round_mode = context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP;
+        const std::vector<int32_t> shifts = conv_shifts(output, input, filter, d.out_c);
+        d.n_shift = (int32_t)shifts.size();
+        const int32_t *shift_dev = m_shift.sync(shifts);
+        if (m_fused_lut && !m_fused_lut->on_device()) {
+            TensorBase *dev = m_fused_lut->to_device(context->stream);
+            delete m_fused_lut;
+            m_fused_lut = dev;
+        }
+        const int rc = espdl_hip_conv2d(&d, input->data, filter->data, bias ? bias->data : nullptr, shift_dev,
+                                        m_fused_lut ? static_cast<const int8_t *>(m_fused_lut->data) : nullptr,
+                                        output->data, context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Conv", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        Module *conv_op = nullptr;
+        std::vector<int> pads, strides, dilations;
+        int group = 1;
+        activation_type_t activation_type = Linear;
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "pads", pads);
+        fbs_model->get_operation_attribute(node_name, "strides", strides);
+        fbs_model->get_operation_attribute(node_name, "dilations", dilations);
+        fbs_model->get_operation_attribute(node_name, "group", group);
+        fbs_model->get_operation_attribute(node_name, "activation", activation_type);
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        if (quant_type == QUANT_TYPE_SYMM_8BIT || quant_type == QUANT_TYPE_SYMM_16BIT) {
+            if (pads.size() == 4)
+                pads = {pads[0], pads[2], pads[1], pads[3]}; // ONNX [t,l,b,r] -> [t,b,l,r]
+            else if (pads.size() == 0)
+                pads = {0, 0, 0, 0};
+            if (strides.empty())
+                strides = {1, 1};
+            if (dilations.empty())
+                dilations = {1, 1};
+            conv_op = new Conv(activation_type, pads, dilations, strides, node_name.c_str(), group, quant_type);
+        }
+        return conv_op;
+    }
+
+    void print()
+    {
+        DL_LOGI("Conv", "pads: %s, strides: %s, dilations: %s, group: %d, activation: %s, quant_type: %s%s.",
+                vector_to_string(m_pads).c_str(), vector_to_string(m_strides).c_str(),
+                vector_to_string(m_dilations).c_str(), m_group, activation_type_to_string(activation),
+                quant_type_to_string(quant_type), m_fused_lut ? ", fused LUT" : "");
+    }
+};
+
+} // namespace module
+} // namespace dl

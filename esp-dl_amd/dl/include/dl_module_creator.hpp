@@ -1,0 +1,89 @@
+// dl::module::ModuleCreator: op-type string -> Module factory registry.
+//
+// Same contract as esp-dl/dl/module/include/dl_module_creator.hpp:35-205: a singleton,
+// register_module(op_type, creator), create(fbs_model, op_type, node_name), and
+// register_dl_modules() that installs the built-in operators on first use.  Only the operators on
+// the quantized conv/gemm path exist here; the activation-like op types are accepted when their node
+// carries a `lut` attribute, in which case they become LUT modules exactly as in the reference.
+#pragma once
+
+#include <functional>
+#include <map>
+#include <string>
+
+#include "dl_module_base.hpp"
+#include "dl_module_conv.hpp"
+#include "dl_module_elementwise.hpp"
+#include "dl_module_gemm.hpp"
+
+namespace dl {
+namespace module {
+
+class ModuleCreator {
+public:
+    using Creator = std::function<Module *(fbs::FbsModel *, std::string)>;
+
+    static ModuleCreator *get_instance()
+    {
+        static ModuleCreator instance;
+        return &instance;
+    }
+
+    void register_module(const std::string &op_type, Creator creator) { m_creators[op_type] = creator; }
+
+    Module *create(fbs::FbsModel *fbs_model, const std::string &op_type, const std::string &node_name)
+    {
+        register_dl_modules();
+        auto it = m_creators.find(op_type);
+        return it == m_creators.end() ? nullptr : it->second(fbs_model, node_name);
+    }
+
+    bool is_registered(const std::string &op_type)
+    {
+        register_dl_modules();
+        return m_creators.count(op_type) != 0;
+    }
+
+    void register_dl_modules()
+    {
+        if (!m_creators.empty())
+            return;
+        register_module("Conv", Conv::deserialize);
+        register_module("Gemm", Gemm::deserialize);
+        register_module("MatMul", MatMul::deserialize);
+        register_module("LUT", LUT::deserialize);
+        register_module("Relu", Relu::deserialize);
+        register_module("PRelu", PRelu::deserialize);
+        register_module("Clip", Clip::deserialize);
+        register_module("Add", Add::deserialize);
+        register_module("GlobalAveragePool", GlobalAveragePool::deserialize);
+        register_module("RequantizeLinear", RequantizeLinear::deserialize);
+        register_module("Flatten", Flatten::deserialize);
+        register_module("Squeeze", ShapeView::deserialize_squeeze);
+        register_module("Unsqueeze", ShapeView::deserialize_unsqueeze);
+        register_module("Reshape", ShapeView::deserialize_reshape);
+        // element-wise activations that esp-ppq exports with a precomputed 8-bit table
+        for (const char *op : {"Swish", "HardSwish", "Sigmoid", "HardSigmoid", "Tanh", "Gelu", "Elu", "LeakyRelu",
+                               "Exp", "Log", "Sqrt", "Softplus", "Mish"}) {
+            const std::string op_type = op;
+            register_module(op_type, [op_type](fbs::FbsModel *fbs_model, std::string node_name) -> Module * {
+                quant_type_t quant_type = QUANT_TYPE_NONE;
+                fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+                Module *m = lut_if_present(fbs_model, node_name, quant_type);
+                if (!m)
+                    DL_LOGE("ModuleCreator", "%s (%s) has no 8-bit LUT; the float fallback is not part of this build",
+                            node_name.c_str(), op_type.c_str());
+                return m;
+            });
+        }
+    }
+
+    void clear() { m_creators.clear(); }
+
+private:
+    ModuleCreator() {}
+    std::map<std::string, Creator> m_creators;
+};
+
+} // namespace module
+} // namespace dl

@@ -1,0 +1,534 @@
+// Bandwidth-bound operator objects: LUT, Relu, PRelu, Clip, Add, GlobalAveragePool,
+// RequantizeLinear, Flatten.  Each mirrors the reference module of the same name and enqueues one
+// kernel of include/espdl_hip.h on the context's stream.
+//   LUT                 esp-dl/dl/module/include/dl_module_lut.hpp:15-104
+//   Relu                esp-dl/dl/module/include/dl_module_relu.hpp:13-120
+//   PRelu               esp-dl/dl/module/include/dl_module_prelu.hpp:15-160
+//   Clip                esp-dl/dl/module/include/dl_module_clip.hpp:12-130
+//   Add                 esp-dl/dl/module/include/dl_module_add.hpp:12-110
+//   GlobalAveragePool   esp-dl/dl/module/include/dl_module_global_avg_pool.hpp
+//   RequantizeLinear    esp-dl/dl/module/include/dl_module_requantize_linear.hpp (runs TensorBase::assign)
+//   Flatten             esp-dl/dl/module/include/dl_module_flatten.hpp
+// Activation-like ops whose node carries a `lut` attribute deserialize into a LUT module, as in the
+// reference (esp-dl/dl/module/include/dl_module_clip.hpp:95-113).
+#pragma once
+
+#include <algorithm>
+#include <cassert>
+#include <limits>
+
+#include "dl_module_base.hpp"
+#include "espdl_hip.h"
+
+namespace dl {
+namespace module {
+
+inline bool on_device_all(std::initializer_list<TensorBase *> ts)
+{
+    for (TensorBase *t : ts)
+        if (!t || !t->on_device())
+            return false;
+    return true;
+}
+
+class LUT : public Module {
+private:
+    TensorBase *table; ///< 256 int8 entries, exponent == output exponent (owned)
+
+public:
+    LUT(const char *name = nullptr, TensorBase *table = nullptr,
+        module_inplace_t inplace = MODULE_INPLACE_CHANGED_BUFFER, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, inplace, quant_type), table(table)
+    {
+    }
+    ~LUT() { delete table; }
+
+    /// Hand the table over (for fusing this LUT into the producing Conv); the module keeps nothing.
+    TensorBase *release_table()
+    {
+        TensorBase *t = table;
+        table = nullptr;
+        return t;
+    }
+    TensorBase *get_table() { return table; }
+
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        return {input_shapes[0]};
+    }
+
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT) {
+            DL_LOGE("LUT", "%s: only the 8-bit table is implemented", name.c_str());
+            return;
+        }
+        if (!table || table->get_size() != 256 || !on_device_all({input, output})) {
+            DL_LOGE("LUT", "%s: needs a 256-entry table and device tensors", name.c_str());
+            return;
+        }
+        if (!table->on_device()) {
+            TensorBase *dev = table->to_device(context->stream);
+            delete table;
+            table = dev;
+        }
+        const int rc = espdl_hip_lut_s8(static_cast<const int8_t *>(input->data), input->get_size(),
+                                        static_cast<const int8_t *>(table->data), static_cast<int8_t *>(output->data),
+                                        context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("LUT", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        TensorBase *table = fbs_model->get_operation_lut(node_name);
+        if (table == nullptr) {
+            DL_LOGE("LUT", "Table is null!");
+            return nullptr;
+        }
+        if (quant_type == QUANT_TYPE_SYMM_8BIT)
+            return new LUT(node_name.c_str(), table, MODULE_INPLACE_CHANGED_BUFFER, quant_type);
+        DL_LOGE("LUT", "Only QUANT_TYPE_SYMM_8BIT tables are implemented");
+        delete table;
+        return nullptr;
+    }
+
+    void print() { DL_LOGI("LUT", "quant_type: %s.", quant_type_to_string(quant_type)); }
+};
+
+/// Shared by every activation op: a node with a `lut` attribute becomes a LUT module.
+inline Module *lut_if_present(fbs::FbsModel *fbs_model, const std::string &node_name, quant_type_t quant_type)
+{
+    if (quant_type != QUANT_TYPE_SYMM_8BIT)
+        return nullptr;
+    TensorBase *table = fbs_model->get_operation_lut(node_name);
+    return table ? new LUT(node_name.c_str(), table, MODULE_INPLACE_CHANGED_BUFFER, quant_type) : nullptr;
+}
+
+class Relu : public Module {
+public:
+    Relu(const char *name = nullptr, module_inplace_t inplace = MODULE_INPLACE_CHANGED_BUFFER,
+         quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, inplace, quant_type)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        return {input_shapes[0]};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !on_device_all({input, output})) {
+            DL_LOGE("Relu", "%s: needs int8 device tensors", name.c_str());
+            return;
+        }
+        const int rc = espdl_hip_relu_s8(static_cast<const int8_t *>(input->data), input->get_size(),
+                                         input->exponent.get(), output->exponent.get(),
+                                         static_cast<int8_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Relu", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        Module *op = lut_if_present(fbs_model, node_name, quant_type);
+        return op ? op : new Relu(node_name.c_str(), MODULE_INPLACE_CHANGED_BUFFER, quant_type);
+    }
+    void print() { DL_LOGI("Relu", "quant_type: %s.", quant_type_to_string(quant_type)); }
+};
+
+class PRelu : public Module {
+private:
+    TensorBase *m_alpha; ///< int8 slope per channel, shape [C,1,1] or [1] (owned)
+
+public:
+    PRelu(const char *name = nullptr, TensorBase *alpha = nullptr, module_inplace_t inplace = MODULE_NON_INPLACE,
+          quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, inplace, quant_type), m_alpha(alpha)
+    {
+    }
+    ~PRelu() { delete m_alpha; }
+
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        return {input_shapes[0]};
+    }
+
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !m_alpha || !on_device_all({input, output})) {
+            DL_LOGE("PRelu", "%s: needs int8 device tensors and an alpha", name.c_str());
+            return;
+        }
+        const int channels = input->shape.back();
+        if (m_alpha->get_size() != channels) {
+            // a single slope is broadcast to every channel (dl_module_prelu.hpp:43-62)
+            TensorBase *host = m_alpha->on_device() ? m_alpha->to_host(context->stream) : m_alpha;
+            std::vector<int8_t> spread(channels, host->get_element<int8_t>(0));
+            TensorBase *wide = new TensorBase({channels, 1, 1}, spread.data(), m_alpha->exponent.get(), DATA_TYPE_INT8,
+                                              true, MALLOC_CAP_DEVICE);
+            if (host != m_alpha)
+                delete host;
+            delete m_alpha;
+            m_alpha = wide;
+        }
+        if (!m_alpha->on_device()) {
+            TensorBase *dev = m_alpha->to_device(context->stream);
+            delete m_alpha;
+            m_alpha = dev;
+        }
+        const int shift = output->exponent.get() - input->exponent.get() - m_alpha->exponent.get();
+        const int rc = espdl_hip_prelu_s8(static_cast<const int8_t *>(input->data), input->get_size() / channels,
+                                          channels, static_cast<const int8_t *>(m_alpha->data), shift,
+                                          static_cast<int8_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("PRelu", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        Module *op = lut_if_present(fbs_model, node_name, quant_type);
+        if (op)
+            return op;
+        TensorBase *alpha = fbs_model->get_operation_parameter(node_name, 1);
+        if (!alpha) {
+            DL_LOGE("PRelu", "%s: slope tensor missing", node_name.c_str());
+            return nullptr;
+        }
+        return new PRelu(node_name.c_str(), alpha, MODULE_INPLACE_CHANGED_BUFFER, quant_type);
+    }
+    void print() { DL_LOGI("PRelu", "quant_type: %s.", quant_type_to_string(quant_type)); }
+};
+
+class Clip : public Module {
+public:
+    Clip(const char *name = nullptr, module_inplace_t inplace = MODULE_NON_INPLACE,
+         quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, inplace, quant_type)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        return {input_shapes[0]};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !on_device_all({input, output})) {
+            DL_LOGE("Clip", "%s: needs int8 device tensors", name.c_str());
+            return;
+        }
+        // min / max are quantized scalars held as parameters (read once on the host)
+        if (!m_bounds_read) {
+            m_min = std::numeric_limits<int8_t>::min();
+            m_max = std::numeric_limits<int8_t>::max();
+            for (size_t i = 1; i < m_inputs_index.size() && i < 3; i++) {
+                TensorBase *b = context->get_tensor(m_inputs_index[i]);
+                if (!b)
+                    continue;
+                TensorBase *host = b->on_device() ? b->to_host(context->stream) : b;
+                (i == 1 ? m_min : m_max) = host->get_element<int8_t>(0);
+                if (host != b)
+                    delete host;
+            }
+            m_bounds_read = true;
+        }
+        const int rc = espdl_hip_clip_s8(static_cast<const int8_t *>(input->data), input->get_size(), m_min, m_max,
+                                         input->exponent.get(), output->exponent.get(),
+                                         static_cast<int8_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Clip", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        Module *op = lut_if_present(fbs_model, node_name, quant_type);
+        return op ? op : new Clip(node_name.c_str(), MODULE_INPLACE_CHANGED_BUFFER, quant_type);
+    }
+    void print() { DL_LOGI("Clip", "quant_type: %s.", quant_type_to_string(quant_type)); }
+
+private:
+    bool m_bounds_read = false;
+    int m_min = -128, m_max = 127;
+};
+
+class Add : public Module {
+public:
+    Add(const char *name = nullptr, module_inplace_t inplace = MODULE_NON_INPLACE,
+        quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, inplace, quant_type)
+    {
+    }
+
+    /// numpy-style broadcast of the two shapes (get_elemwise_operation_args merges dims the same way,
+    /// esp-dl/dl/base/dl_base_elemwise.cpp:38-178)
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &a = input_shapes[0], &b = input_shapes[1];
+        const size_t rank = std::max(a.size(), b.size());
+        std::vector<int> out(rank, 1);
+        for (size_t i = 0; i < rank; i++) {
+            const int da = i < rank - a.size() ? 1 : a[i - (rank - a.size())];
+            const int db = i < rank - b.size() ? 1 : b[i - (rank - b.size())];
+            assert(da == db || da == 1 || db == 1);
+            out[i] = std::max(da, db);
+        }
+        return {out};
+    }
+
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input0 = context->get_tensor(m_inputs_index[0]);
+        TensorBase *input1 = context->get_tensor(m_inputs_index[1]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !on_device_all({input0, input1, output}) ||
+            output->shape.size() > 4) {
+            DL_LOGE("Add", "%s: needs int8 device tensors of rank <= 4", name.c_str());
+            return;
+        }
+        int32_t dims[4] = {1, 1, 1, 1};
+        int64_t s0[4] = {0, 0, 0, 0}, s1[4] = {0, 0, 0, 0};
+        const size_t rank = output->shape.size();
+        for (size_t i = 0; i < rank; i++)
+            dims[4 - rank + i] = output->shape[i];
+        auto strides = [&](TensorBase *t, int64_t *s) {
+            const size_t r = t->shape.size();
+            int64_t acc = 1;
+            for (int i = (int)r - 1; i >= 0; i--) {
+                s[4 - r + i] = t->shape[i] == 1 ? 0 : acc;
+                acc *= t->shape[i];
+            }
+        };
+        strides(input0, s0);
+        strides(input1, s1);
+        const int rc = espdl_hip_add_s8(dims, s0, s1, static_cast<const int8_t *>(input0->data),
+                                        static_cast<const int8_t *>(input1->data), static_cast<int8_t *>(output->data),
+                                        context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Add", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        return new Add(node_name.c_str(), MODULE_INPLACE_CHANGED_BUFFER, quant_type);
+    }
+    void print() { DL_LOGI("Add", "quant_type: %s.", quant_type_to_string(quant_type)); }
+};
+
+class GlobalAveragePool : public Module {
+public:
+    GlobalAveragePool(const char *name = nullptr, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        assert(input_shapes[0].size() == 4);
+        return {{input_shapes[0][0], 1, 1, input_shapes[0][3]}};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !on_device_all({input, output}) || input->shape.size() != 4) {
+            DL_LOGE("GlobalAveragePool", "%s: needs int8 NHWC device tensors", name.c_str());
+            return;
+        }
+        const int rc = espdl_hip_global_avg_pool_s8(static_cast<const int8_t *>(input->data), input->shape[0],
+                                                    input->shape[1], input->shape[2], input->shape[3],
+                                                    input->exponent.get(), output->exponent.get(),
+                                                    static_cast<int8_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("GlobalAveragePool", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        return new GlobalAveragePool(node_name.c_str(), quant_type);
+    }
+    void print() { DL_LOGI("GlobalAveragePool", "quant_type: %s.", quant_type_to_string(quant_type)); }
+};
+
+class RequantizeLinear : public Module {
+public:
+    RequantizeLinear(const char *name = nullptr, module_inplace_t inplace = MODULE_NON_INPLACE,
+                     quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, inplace, quant_type)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        return {input_shapes[0]};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) || !output->assign(input, context->stream))
+            DL_LOGE("RequantizeLinear", "%s: assign failed", name.c_str());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        return new RequantizeLinear(node_name.c_str(), MODULE_INPLACE_CHANGED_BUFFER, quant_type);
+    }
+    void print() { DL_LOGI("RequantizeLinear", "quant_type: %s.", quant_type_to_string(quant_type)); }
+};
+
+/// Flatten to [N, rest]: a view, no bytes move (the planner aliases output onto input).
+class Flatten : public Module {
+private:
+    int m_axis;
+
+public:
+    Flatten(const char *name = nullptr, int axis = 1, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_INPLACE_UNCHANGED_BUFFER, quant_type), m_axis(axis)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        int axis = m_axis < 0 ? m_axis + (int)in.size() : m_axis;
+        int outer = 1, inner = 1;
+        for (int i = 0; i < (int)in.size(); i++)
+            (i < axis ? outer : inner) *= in[i];
+        return {{outer, inner}};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (input && output && input->data != output->data)
+            output->copy_from(input, context->stream);
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        int axis = 1;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "axis", axis);
+        return new Flatten(node_name.c_str(), axis, quant_type);
+    }
+    void print() { DL_LOGI("Flatten", "axis: %d, quant_type: %s.", m_axis, quant_type_to_string(quant_type)); }
+};
+
+/// Squeeze / Unsqueeze / Reshape: views that only change the shape (no bytes move).
+///   esp-dl/dl/module/include/dl_module_squeeze.hpp, dl_module_unsqueeze.hpp, dl_module_reshape.hpp
+class ShapeView : public Module {
+public:
+    enum Kind { SQUEEZE, UNSQUEEZE, RESHAPE };
+
+private:
+    Kind m_kind;
+    std::vector<int> m_arg; ///< axes (Squeeze / Unsqueeze) or the per-image target shape with leading 1 (Reshape)
+
+public:
+    ShapeView(const char *name, Kind kind, std::vector<int> arg, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_INPLACE_UNCHANGED_BUFFER, quant_type), m_kind(kind), m_arg(arg)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        std::vector<int> out;
+        const int rank = (int)in.size();
+        if (m_kind == SQUEEZE) {
+            for (int i = 0; i < rank; i++) {
+                bool drop = false;
+                for (int a : m_arg)
+                    if ((a < 0 ? a + rank : a) == i && in[i] == 1)
+                        drop = true;
+                if (m_arg.empty() && in[i] == 1 && i != 0)
+                    drop = true;
+                if (!drop)
+                    out.push_back(in[i]);
+            }
+        } else if (m_kind == UNSQUEEZE) {
+            const int out_rank = rank + (int)m_arg.size();
+            int src = 0;
+            for (int i = 0; i < out_rank; i++) {
+                bool ins = false;
+                for (int a : m_arg)
+                    if ((a < 0 ? a + out_rank : a) == i)
+                        ins = true;
+                out.push_back(ins ? 1 : in[src++]);
+            }
+        } else {
+            int64_t total = 1, known = 1;
+            for (int d : in)
+                total *= d;
+            out = m_arg;
+            if (!out.empty())
+                out[0] = in[0]; // the batch dimension is kept
+            int infer = -1;
+            for (size_t i = 0; i < out.size(); i++) {
+                if (out[i] == -1)
+                    infer = (int)i;
+                else
+                    known *= out[i];
+            }
+            if (infer >= 0)
+                out[infer] = (int)(total / known);
+        }
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (input && output && input->data != output->data)
+            output->copy_from(input, context->stream);
+    }
+    static Module *deserialize_squeeze(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        return make(fbs_model, node_name, SQUEEZE, "axes");
+    }
+    static Module *deserialize_unsqueeze(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        return make(fbs_model, node_name, UNSQUEEZE, "axes");
+    }
+    static Module *deserialize_reshape(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        return make(fbs_model, node_name, RESHAPE, "shape");
+    }
+    void print() { DL_LOGI("ShapeView", "kind %d, arg %s.", (int)m_kind, vector_to_string(m_arg).c_str()); }
+
+private:
+    static Module *make(fbs::FbsModel *fbs_model, const std::string &node_name, Kind kind, const char *key)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        std::vector<int> arg;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, key, arg);
+        return new ShapeView(node_name.c_str(), kind, arg, quant_type);
+    }
+};
+
+} // namespace module
+} // namespace dl

@@ -1,0 +1,707 @@
+#include "dl_model_base.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstring>
+#include <set>
+
+#include "dl_module_creator.hpp"
+
+namespace dl {
+
+namespace {
+const char *TAG = "dl::Model";
+
+bool hip_ok(hipError_t e, const char *what)
+{
+    if (e != hipSuccess) {
+        DL_LOGE(TAG, "%s failed: %s", what, hipGetErrorString(e));
+        return false;
+    }
+    return true;
+}
+
+dtype_t dtype_of(quant_type_t q)
+{
+    switch (q) {
+    case QUANT_TYPE_SYMM_16BIT:
+        return DATA_TYPE_INT16;
+    case QUANT_TYPE_FLOAT32:
+        return DATA_TYPE_FLOAT;
+    default:
+        return DATA_TYPE_INT8;
+    }
+}
+
+// One block of the activation arena.
+struct Block {
+    size_t offset, bytes;
+    int users; // tensors currently living in it
+};
+
+// First-fit free list over a linear arena: the role MemoryManagerGreedy plays in the reference.
+class ArenaPlanner {
+public:
+    size_t alloc(size_t bytes)
+    {
+        bytes = (bytes + 255) & ~(size_t)255;
+        if (bytes == 0)
+            bytes = 256;
+        size_t best = m_free.size();
+        for (size_t i = 0; i < m_free.size(); i++)
+            if (m_free[i].second >= bytes && (best == m_free.size() || m_free[i].second < m_free[best].second))
+                best = i;
+        if (best != m_free.size()) {
+            const size_t off = m_free[best].first;
+            if (m_free[best].second == bytes)
+                m_free.erase(m_free.begin() + best);
+            else {
+                m_free[best].first += bytes;
+                m_free[best].second -= bytes;
+            }
+            return off;
+        }
+        // grow; if the last free range touches the end of the arena, extend it instead
+        if (!m_free.empty() && m_free.back().first + m_free.back().second == m_top) {
+            const size_t off = m_free.back().first;
+            m_top = off + bytes;
+            m_free.pop_back();
+            return off;
+        }
+        const size_t off = m_top;
+        m_top += bytes;
+        return off;
+    }
+    void release(size_t offset, size_t bytes)
+    {
+        bytes = (bytes + 255) & ~(size_t)255;
+        if (bytes == 0)
+            bytes = 256;
+        m_free.push_back({offset, bytes});
+        std::sort(m_free.begin(), m_free.end());
+        for (size_t i = 0; i + 1 < m_free.size();) {
+            if (m_free[i].first + m_free[i].second == m_free[i + 1].first) {
+                m_free[i].second += m_free[i + 1].second;
+                m_free.erase(m_free.begin() + i + 1);
+            } else {
+                i++;
+            }
+        }
+    }
+    size_t top() const { return m_top; }
+
+private:
+    std::vector<std::pair<size_t, size_t>> m_free;
+    size_t m_top = 0;
+};
+
+} // namespace
+
+Model::Model(fbs::FbsModel *fbs_model, int batch, round_mode_t round_mode, void *stream, bool fuse_lut) :
+    m_batch(batch), m_fuse_lut(fuse_lut), m_stream(stream)
+{
+    m_model_context = new ModelContext();
+    m_model_context->owns_tensors = true;
+    m_model_context->round_mode = round_mode;
+    if (!m_stream) {
+        hipStream_t s = nullptr;
+        if (hip_ok(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreateWithFlags")) {
+            m_stream = s;
+            m_own_stream = true;
+        }
+    }
+    m_model_context->stream = m_stream;
+    if (load(fbs_model) == ESP_OK)
+        build(batch);
+}
+
+Model::~Model()
+{
+    disable_graph();
+    if (m_stream)
+        (void)hipStreamSynchronize(static_cast<hipStream_t>(m_stream));
+    for (auto *m : m_execution_plan)
+        delete m;
+    m_execution_plan.clear();
+    delete m_model_context;
+    if (m_own_stream && m_stream)
+        (void)hipStreamDestroy(static_cast<hipStream_t>(m_stream));
+}
+
+esp_err_t Model::load(fbs::FbsModel *fbs_model)
+{
+    if (!fbs_model) {
+        DL_LOGE(TAG, "Fail to load model");
+        return ESP_FAIL;
+    }
+    esp_err_t ret = ESP_OK;
+    m_fbs_model = fbs_model;
+    m_name = fbs_model->get_model_name();
+    m_version = fbs_model->get_model_version();
+    m_doc_string = fbs_model->get_model_doc_string();
+    m_built = false;
+
+    for (auto *m : m_execution_plan)
+        delete m;
+    m_execution_plan.clear();
+    m_model_context->clear();
+    auto *creator = dl::module::ModuleCreator::get_instance();
+    std::vector<std::string> op_inputs, op_outputs;
+    for (const std::string &node_name : fbs_model->topological_sort()) {
+        const std::string op_type = fbs_model->get_operation_type(node_name);
+        if (op_type.empty()) {
+            DL_LOGE(TAG, "Can not find the operation %s", node_name.c_str());
+            ret = ESP_FAIL;
+            break;
+        }
+        dl::module::Module *module = creator->create(fbs_model, op_type, node_name);
+        if (!module) {
+            DL_LOGE(TAG, "Do not support %s, please implement and register it first.", op_type.c_str());
+            ret = ESP_FAIL;
+            break;
+        }
+        m_execution_plan.push_back(module);
+        fbs_model->get_operation_inputs_and_outputs(node_name, op_inputs, op_outputs);
+        for (size_t j = 0; j < op_inputs.size(); j++) {
+            int index;
+            if (fbs_model->is_parameter(op_inputs[j]) || op_inputs[j].empty()) {
+                TensorBase *param = nullptr;
+                if (m_model_context->get_tensor_index(op_inputs[j]) < 0)
+                    param = fbs_model->get_operation_parameter(node_name, (int)j, MALLOC_CAP_DEVICE);
+                index = m_model_context->add_tensor(op_inputs[j], true, param);
+            } else {
+                index = m_model_context->add_tensor(op_inputs[j], false, nullptr);
+            }
+            module->m_inputs_index.push_back(index);
+        }
+        for (size_t j = 0; j < op_outputs.size(); j++)
+            module->m_outputs_index.push_back(m_model_context->add_tensor(op_outputs[j], false, nullptr));
+    }
+    if (ret == ESP_OK && m_fuse_lut)
+        fuse_conv_lut();
+    return ret;
+}
+
+// Conv -> LUT with no other reader of the conv output: the table moves into the conv's epilogue and
+// the conv writes the LUT's output tensor directly.
+void Model::fuse_conv_lut()
+{
+    std::set<std::string> pinned; // tensors that must keep existing
+    for (auto &n : m_fbs_model->get_graph_outputs())
+        pinned.insert(n);
+    for (auto &n : m_fbs_model->get_test_outputs_name())
+        pinned.insert(n);
+    for (size_t i = 0; i < m_execution_plan.size(); i++) {
+        auto *conv = dynamic_cast<dl::module::Conv *>(m_execution_plan[i]);
+        if (!conv || conv->quant_type != QUANT_TYPE_SYMM_8BIT || conv->has_fused_lut())
+            continue;
+        const int mid = conv->m_outputs_index[0];
+        if (pinned.count(m_model_context->get_tensor_name(mid)))
+            continue;
+        int readers = 0;
+        size_t lut_pos = 0;
+        for (size_t j = 0; j < m_execution_plan.size(); j++)
+            for (int in : m_execution_plan[j]->m_inputs_index)
+                if (in == mid) {
+                    readers++;
+                    lut_pos = j;
+                }
+        if (readers != 1)
+            continue;
+        auto *lut = dynamic_cast<dl::module::LUT *>(m_execution_plan[lut_pos]);
+        if (!lut || lut->quant_type != QUANT_TYPE_SYMM_8BIT || !lut->get_table() || lut->get_table()->get_size() != 256)
+            continue;
+        conv->fuse_lut(lut->release_table());
+        conv->m_outputs_index[0] = lut->m_outputs_index[0];
+        delete lut;
+        m_execution_plan.erase(m_execution_plan.begin() + lut_pos);
+        if (lut_pos < i)
+            i--;
+    }
+}
+
+esp_err_t Model::build(int batch)
+{
+    if (!m_fbs_model || batch <= 0)
+        return ESP_FAIL;
+    disable_graph();
+    m_batch = batch;
+    ModelContext *ctx = m_model_context;
+    const int n_var = ctx->get_variable_count();
+
+    // drop activations of a previous build
+    for (int i = 1; i < n_var; i++) {
+        delete ctx->m_variables[i];
+        ctx->m_variables[i] = nullptr;
+    }
+    ctx->root_free();
+
+    // 1. shapes, dtypes and exponents of every variable
+    struct VarInfo {
+        std::vector<int> shape;
+        dtype_t dtype = DATA_TYPE_INT8;
+        int exponent = 0;
+        int first = -1, last = -1; // producing module, last reading module
+        bool known = false;
+        int alias_of = -1; // view of another variable's bytes
+    };
+    std::vector<VarInfo> vars(n_var);
+    const int plan_size = (int)m_execution_plan.size();
+    for (const std::string &name : m_fbs_model->get_graph_inputs()) {
+        const int idx = ctx->get_variable_index(name);
+        if (idx < 0) {
+            DL_LOGE(TAG, "graph input %s feeds no node", name.c_str());
+            return ESP_FAIL;
+        }
+        VarInfo &v = vars[idx];
+        v.shape = m_fbs_model->get_value_info_shape(name);
+        if (v.shape.empty()) {
+            DL_LOGE(TAG, "graph input %s has no shape", name.c_str());
+            return ESP_FAIL;
+        }
+        v.shape[0] *= batch; // exported shapes carry a leading 1
+        v.dtype = m_fbs_model->get_value_info_dtype(name);
+        v.exponent = m_fbs_model->get_value_info_exponent(name);
+        v.known = true;
+        v.first = -1;
+    }
+    for (int i = 0; i < plan_size; i++) {
+        dl::module::Module *m = m_execution_plan[i];
+        std::vector<std::vector<int>> in_shapes;
+        for (int idx : m->m_inputs_index) {
+            if (idx >= CONTEXT_PARAMETER_OFFSET) {
+                TensorBase *p = ctx->get_tensor(idx);
+                in_shapes.push_back(p ? p->shape : std::vector<int>());
+            } else {
+                if (!vars[idx].known) {
+                    DL_LOGE(TAG, "%s reads %s before it is produced", m->name.c_str(), ctx->get_tensor_name(idx).c_str());
+                    return ESP_FAIL;
+                }
+                in_shapes.push_back(vars[idx].shape);
+                vars[idx].last = i;
+            }
+        }
+        std::vector<std::vector<int>> out_shapes = m->get_output_shape(in_shapes);
+        for (size_t j = 0; j < m->m_outputs_index.size(); j++) {
+            const int idx = m->m_outputs_index[j];
+            const std::string name = ctx->get_tensor_name(idx);
+            VarInfo &v = vars[idx];
+            v.shape = out_shapes[j];
+            v.dtype = m_fbs_model->has_value_info(name) ? m_fbs_model->get_value_info_dtype(name) : dtype_of(m->quant_type);
+            if (v.dtype == DATA_TYPE_UNDEFINED)
+                v.dtype = dtype_of(m->quant_type);
+            if (!m_fbs_model->has_value_info(name))
+                DL_LOGW(TAG, "tensor %s has no value_info; exponent 0 assumed", name.c_str());
+            v.exponent = m_fbs_model->get_value_info_exponent(name);
+            v.known = true;
+            v.first = i;
+            if (m->inplace == MODULE_INPLACE_UNCHANGED_BUFFER && j == 0 && m->m_inputs_index[0] < CONTEXT_PARAMETER_OFFSET)
+                v.alias_of = m->m_inputs_index[0];
+        }
+    }
+    for (const std::string &name : m_fbs_model->get_graph_outputs()) {
+        const int idx = ctx->get_variable_index(name);
+        if (idx < 0 || !vars[idx].known) {
+            DL_LOGE(TAG, "graph output %s is not produced", name.c_str());
+            return ESP_FAIL;
+        }
+        vars[idx].last = plan_size; // alive to the end
+    }
+    for (const std::string &name : m_fbs_model->get_test_outputs_name()) {
+        const int idx = ctx->get_variable_index(name);
+        if (idx >= 0)
+            vars[idx].last = plan_size;
+    }
+    // a view keeps its source alive
+    for (int i = n_var - 1; i >= 1; i--)
+        if (vars[i].alias_of >= 0)
+            vars[vars[i].alias_of].last = std::max(vars[vars[i].alias_of].last, vars[i].last);
+
+    // 2. placement
+    auto bytes_of = [&](const VarInfo &v) {
+        size_t n = dtype_sizeof(v.dtype);
+        for (int d : v.shape)
+            n *= (size_t)d;
+        return n;
+    };
+    std::vector<size_t> offset(n_var, 0);
+    std::vector<bool> placed(n_var, false);
+    ArenaPlanner arena;
+    std::set<int> graph_io;
+    for (const std::string &name : m_fbs_model->get_graph_inputs())
+        graph_io.insert(ctx->get_variable_index(name));
+    for (int idx : graph_io) {
+        offset[idx] = arena.alloc(bytes_of(vars[idx]));
+        placed[idx] = true;
+    }
+    auto release_dead = [&](int step) {
+        for (int v = 1; v < n_var; v++)
+            if (placed[v] && vars[v].alias_of < 0 && vars[v].last == step && !graph_io.count(v)) {
+                // views that share the block die no later than their source (made sure above)
+                arena.release(offset[v], bytes_of(vars[v]));
+                placed[v] = false;
+                vars[v].last = -2;
+            }
+    };
+    for (int i = 0; i < plan_size; i++) {
+        dl::module::Module *m = m_execution_plan[i];
+        for (size_t j = 0; j < m->m_outputs_index.size(); j++) {
+            const int idx = m->m_outputs_index[j];
+            VarInfo &v = vars[idx];
+            if (v.alias_of >= 0) {
+                offset[idx] = offset[v.alias_of];
+                continue;
+            }
+            // an in-place module may overwrite its first input when nobody reads that input later
+            const int in0 = m->m_inputs_index.empty() ? -1 : m->m_inputs_index[0];
+            if (m->inplace == MODULE_INPLACE_CHANGED_BUFFER && j == 0 && in0 > 0 && in0 < CONTEXT_PARAMETER_OFFSET &&
+                placed[in0] && vars[in0].alias_of < 0 && vars[in0].last == i && !graph_io.count(in0) &&
+                bytes_of(vars[in0]) == bytes_of(v)) {
+                bool aliased_elsewhere = false;
+                for (int k = 1; k < n_var; k++)
+                    if (vars[k].alias_of == in0)
+                        aliased_elsewhere = true;
+                if (!aliased_elsewhere) {
+                    offset[idx] = offset[in0];
+                    placed[idx] = true;
+                    placed[in0] = false;
+                    vars[in0].last = -2;
+                    continue;
+                }
+            }
+            offset[idx] = arena.alloc(bytes_of(v));
+            placed[idx] = true;
+        }
+        release_dead(i);
+    }
+
+    // 3. materialize
+    if (!ctx->root_alloc(arena.top()))
+        return ESP_FAIL;
+    char *root = static_cast<char *>(ctx->get_device_root());
+    for (int i = 1; i < n_var; i++) {
+        if (!vars[i].known)
+            continue;
+        ctx->m_variables[i] =
+            new TensorBase(vars[i].shape, root + offset[i], vars[i].exponent, vars[i].dtype, false, MALLOC_CAP_DEVICE);
+    }
+    m_inputs.clear();
+    m_outputs.clear();
+    for (const std::string &name : m_fbs_model->get_graph_inputs())
+        m_inputs.emplace(name, get_intermediate(name));
+    for (const std::string &name : m_fbs_model->get_graph_outputs())
+        m_outputs.emplace(name, get_intermediate(name));
+    (void)hipMemsetAsync(root, 0, ctx->get_device_size(), static_cast<hipStream_t>(m_stream));
+    (void)hipStreamSynchronize(static_cast<hipStream_t>(m_stream));
+    m_built = true;
+    return ESP_OK;
+}
+
+void Model::run_async(runtime_mode_t mode)
+{
+    if (!m_built)
+        return;
+    if (m_graph_exec) {
+        (void)hip_ok(hipGraphLaunch(static_cast<hipGraphExec_t>(m_graph_exec), static_cast<hipStream_t>(m_stream)),
+                     "hipGraphLaunch");
+        return;
+    }
+    for (auto *module : m_execution_plan)
+        module->forward(m_model_context, mode);
+}
+
+void Model::synchronize()
+{
+    (void)hip_ok(hipStreamSynchronize(static_cast<hipStream_t>(m_stream)), "hipStreamSynchronize");
+}
+
+void Model::run(runtime_mode_t mode)
+{
+    run_async(mode);
+    synchronize();
+}
+
+void Model::run(TensorBase *input, runtime_mode_t mode)
+{
+    if (m_inputs.size() != 1) {
+        DL_LOGW(TAG, "The inputs of model is not just one! This API will assign data to first input");
+    }
+    TensorBase *model_input = m_inputs.begin()->second;
+    if (!model_input->assign(input, m_stream)) {
+        DL_LOGE(TAG, "Assign input failed");
+        return;
+    }
+    run(mode);
+}
+
+void Model::run(std::map<std::string, TensorBase *> &user_inputs, runtime_mode_t mode,
+                std::map<std::string, TensorBase *> user_outputs)
+{
+    if (user_inputs.size() != m_inputs.size()) {
+        DL_LOGE(TAG, "The size of user_inputs(%zu) don't equal with the size of model inputs(%zu).", user_inputs.size(),
+                m_inputs.size());
+        return;
+    }
+    for (auto &kv : user_inputs) {
+        auto it = m_inputs.find(kv.first);
+        if (it == m_inputs.end() || !it->second->assign(kv.second, m_stream)) {
+            DL_LOGE(TAG, "Assign input %s failed", kv.first.c_str());
+            return;
+        }
+    }
+    run(mode);
+    for (auto &kv : user_outputs) {
+        TensorBase *t = get_intermediate(kv.first);
+        if (!t || !kv.second->assign(t, m_stream))
+            DL_LOGE(TAG, "Assign output %s failed", kv.first.c_str());
+    }
+    synchronize();
+}
+
+void Model::run(int stage_num, int stage_index, runtime_mode_t mode)
+{
+    const int plan_size = (int)m_execution_plan.size();
+    if (stage_num < 1)
+        stage_num = 1;
+    if (stage_index < 0 || stage_index >= stage_num) {
+        DL_LOGE(TAG, "Invalid stage_index(%d), it should be in range [0, %d).", stage_index, stage_num);
+        return;
+    }
+    const int start = stage_index * plan_size / stage_num;
+    const int end = (stage_index + 1) * plan_size / stage_num;
+    for (int i = start; i < end; i++)
+        m_execution_plan[i]->forward(m_model_context, mode);
+    synchronize();
+}
+
+bool Model::enable_graph()
+{
+    if (!m_built || m_graph_exec)
+        return m_graph_exec != nullptr;
+    hipStream_t s = static_cast<hipStream_t>(m_stream);
+    // one eager pass so that every module has uploaded its shifts / tables before capture starts
+    for (auto *module : m_execution_plan)
+        module->forward(m_model_context, RUNTIME_MODE_AUTO);
+    if (!hip_ok(hipStreamSynchronize(s), "hipStreamSynchronize"))
+        return false;
+    if (!hip_ok(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture"))
+        return false;
+    for (auto *module : m_execution_plan)
+        module->forward(m_model_context, RUNTIME_MODE_AUTO);
+    hipGraph_t graph = nullptr;
+    if (!hip_ok(hipStreamEndCapture(s, &graph), "hipStreamEndCapture") || !graph)
+        return false;
+    hipGraphExec_t exec = nullptr;
+    if (!hip_ok(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate")) {
+        (void)hipGraphDestroy(graph);
+        return false;
+    }
+    m_graph = graph;
+    m_graph_exec = exec;
+    return true;
+}
+
+void Model::disable_graph()
+{
+    if (m_graph_exec) {
+        (void)hipStreamSynchronize(static_cast<hipStream_t>(m_stream));
+        (void)hipGraphExecDestroy(static_cast<hipGraphExec_t>(m_graph_exec));
+        m_graph_exec = nullptr;
+    }
+    if (m_graph) {
+        (void)hipGraphDestroy(static_cast<hipGraph_t>(m_graph));
+        m_graph = nullptr;
+    }
+}
+
+esp_err_t Model::test()
+{
+    if (!m_built)
+        return ESP_FAIL;
+    for (auto &kv : m_inputs) {
+        TensorBase *test_input = m_fbs_model->get_test_input_tensor(kv.first);
+        if (!test_input) {
+            DL_LOGE(TAG, "Model input %s doesn't have a corresponding test input.", kv.first.c_str());
+            return ESP_FAIL;
+        }
+        const bool ok = kv.second->assign(test_input, m_stream);
+        delete test_input;
+        if (!ok) {
+            DL_LOGE(TAG, "Assign input failed");
+            return ESP_FAIL;
+        }
+    }
+    std::vector<std::string> names = m_fbs_model->get_test_outputs_name();
+    if (names.empty()) {
+        DL_LOGE(TAG, "The model holds no test outputs");
+        return ESP_FAIL;
+    }
+    for (const std::string &name : names)
+        if (m_model_context->get_tensor_index(name) < 0) {
+            DL_LOGE(TAG, "There's no intermediate result or output named %s in model.", name.c_str());
+            return ESP_FAIL;
+        }
+    // run module by module so that every tested tensor is compared right after it is produced
+    for (auto *module : m_execution_plan) {
+        module->forward(m_model_context, RUNTIME_MODE_SINGLE_CORE);
+        synchronize();
+        for (int index : module->get_outputs_index()) {
+            const std::string out_name = m_model_context->get_tensor_name(index);
+            if (std::find(names.begin(), names.end(), out_name) == names.end())
+                continue;
+            TensorBase *output = m_model_context->get_tensor(index);
+            TensorBase *output_gt = m_fbs_model->get_test_output_tensor(out_name);
+            const float eps = (output->get_dtype() == DATA_TYPE_INT16) ? 1 + 1e-5f : 2e-5f;
+            const bool same = output->equal(output_gt, eps, true);
+            delete output_gt;
+            if (!same) {
+                DL_LOGE(TAG, "Test output %s does not match", out_name.c_str());
+                return ESP_FAIL;
+            }
+        }
+    }
+    DL_LOGI(TAG, "Test Pass!");
+    return ESP_OK;
+}
+
+std::vector<module_info> Model::get_module_info(int repeats)
+{
+    std::vector<module_info> info;
+    if (!m_built)
+        return info;
+    hipStream_t s = static_cast<hipStream_t>(m_stream);
+    hipEvent_t e0, e1;
+    if (!hip_ok(hipEventCreate(&e0), "hipEventCreate") || !hip_ok(hipEventCreate(&e1), "hipEventCreate"))
+        return info;
+    if (repeats < 1)
+        repeats = 1;
+    for (auto *module : m_execution_plan) {
+        module->forward(m_model_context, RUNTIME_MODE_AUTO); // warm
+        (void)hipEventRecord(e0, s);
+        for (int r = 0; r < repeats; r++)
+            module->forward(m_model_context, RUNTIME_MODE_AUTO);
+        (void)hipEventRecord(e1, s);
+        (void)hipEventSynchronize(e1);
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        module_info mi;
+        mi.name = module->name;
+        const std::string op = m_fbs_model->get_operation_type(module->name);
+        mi.type = op;
+        mi.latency_us = ms * 1000.f / repeats;
+        std::vector<std::vector<int>> in_shapes;
+        mi.bytes = 0;
+        for (int idx : module->m_inputs_index) {
+            TensorBase *t = m_model_context->get_tensor(idx);
+            in_shapes.push_back(t ? t->shape : std::vector<int>());
+            if (t)
+                mi.bytes += (int64_t)t->get_bytes();
+        }
+        for (int idx : module->m_outputs_index) {
+            TensorBase *t = m_model_context->get_tensor(idx);
+            if (t)
+                mi.bytes += (int64_t)t->get_bytes();
+        }
+        mi.macs = module->get_macs(in_shapes);
+        info.push_back(mi);
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    return info;
+}
+
+void Model::profile(bool sort_module_by_latency)
+{
+    std::vector<module_info> info = get_module_info();
+    if (sort_module_by_latency)
+        std::sort(info.begin(), info.end(),
+                  [](const module_info &a, const module_info &b) { return a.latency_us > b.latency_us; });
+    double total = 0;
+    for (auto &m : info)
+        total += m.latency_us;
+    std::printf("%-40s %-18s %12s %10s %10s\n", "name", "type", "latency(us)", "TOP/s", "GB/s");
+    for (auto &m : info)
+        std::printf("%-40s %-18s %12.2f %10.2f %10.1f\n", m.name.c_str(), m.type.c_str(), m.latency_us,
+                    m.latency_us > 0 ? 2.0 * m.macs / m.latency_us * 1e-6 : 0.0,
+                    m.latency_us > 0 ? m.bytes / m.latency_us * 1e-3 : 0.0);
+    std::printf("total %.2f us for batch %d\n", total, m_batch);
+    mem_info_t mem = get_memory_info();
+    std::printf("device memory: %zu bytes (activation arena + parameters)\n", mem.device);
+}
+
+mem_info_t Model::get_memory_info()
+{
+    mem_info_t m;
+    m.device = m_model_context->get_variable_memory_size() + m_model_context->get_parameter_memory_size();
+    m.host = 0;
+    return m;
+}
+
+TensorBase *Model::get_input()
+{
+    if (m_inputs.size() != 1)
+        DL_LOGW(TAG, "The inputs of model is not just one! This API will return first input");
+    return m_inputs.empty() ? nullptr : m_inputs.begin()->second;
+}
+
+TensorBase *Model::get_input(const std::string &name)
+{
+    auto it = m_inputs.find(name);
+    return it == m_inputs.end() ? nullptr : it->second;
+}
+
+TensorBase *Model::get_intermediate(const std::string &name)
+{
+    return m_model_context->get_tensor(name);
+}
+
+TensorBase *Model::get_output()
+{
+    if (m_outputs.size() != 1)
+        DL_LOGW(TAG, "The outputs of model is not just one! This API will return first output");
+    return m_outputs.empty() ? nullptr : m_outputs.begin()->second;
+}
+
+TensorBase *Model::get_output(const std::string &name)
+{
+    auto it = m_outputs.find(name);
+    return it == m_outputs.end() ? nullptr : it->second;
+}
+
+std::string Model::get_metadata_prop(const std::string &key)
+{
+    return m_fbs_model ? m_fbs_model->get_model_metadata_prop(key) : std::string();
+}
+
+void Model::print()
+{
+    std::printf("model %s (version %lld), batch %d, %zu modules\n", m_name.c_str(), (long long)m_version, m_batch,
+                m_execution_plan.size());
+    for (auto *module : m_execution_plan) {
+        std::printf("------------------------------- %s\n", module->name.c_str());
+        module->print();
+        for (int idx : module->m_inputs_index) {
+            TensorBase *t = m_model_context->get_tensor(idx);
+            if (t)
+                t->print();
+        }
+        for (int idx : module->m_outputs_index) {
+            TensorBase *t = m_model_context->get_tensor(idx);
+            if (t)
+                t->print();
+        }
+    }
+}
+
+void Model::reset()
+{
+    for (auto *module : m_execution_plan)
+        module->reset();
+    if (m_model_context->get_device_root()) {
+        synchronize();
+        (void)hipMemset(m_model_context->get_device_root(), 0, m_model_context->get_device_size());
+    }
+}
+
+} // namespace dl

@@ -1,0 +1,446 @@
+"""Seeded synthetic graphs in ESP-DL's exported form (what an `.espdl` file holds), for the five
+benchmark configurations: nodes with ONNX-style attributes, int8/int16 initializers with per-tensor
+or per-channel exponents, int32/int64 biases with exponent in_exp + w_exp[c], 8-bit LUT tables,
+value_info exponents.  There are no datasets or trained weights: everything is drawn from
+numpy's PCG64 with the seeds given here.
+
+A GraphSpec is plain data.  `espdl.model.Graph.from_spec` turns it into the native fbs::FbsModel;
+the CPU oracle's graph runner executes the same spec, so both sides see identical bytes.
+
+Layouts follow the reference's `c` target: dense filter initializer dims [kH,kW,Cin,Cout] over
+[Cout][kH][kW][Cin] bytes, depthwise dims [kH,kW,C,1] over [kH][kW][C] bytes, Gemm dims [1,1,K,N]
+over [N][K] bytes (esp-dl/dl/base/dl_base_conv2d.cpp:23,64,140; dl_base_depthwise_conv2d.cpp:46-65).
+"""
+import math
+
+import numpy as np
+
+INT8, INT16, INT32, INT64 = 3, 5, 6, 7
+_NP = {INT8: np.int8, INT16: np.int16, INT32: np.int32, INT64: np.int64}
+
+
+class GraphSpec:
+    def __init__(self, name):
+        self.name = name
+        self.initializers = {}  # name -> (dims, dtype_code, ndarray (bytes as stored), exponents list)
+        self.value_info = {}    # name -> (per-image dims with leading 1, dtype_code, exponent)
+        self.nodes = []         # dicts: name, op_type, inputs, outputs, attrs
+        self.inputs = []
+        self.outputs = []
+        self.macs_per_image = 0
+        self.conv_macs_per_image = 0
+
+    # -- construction helpers ------------------------------------------------------------------
+    def add_init(self, name, dims, dtype, data, exponents):
+        data = np.ascontiguousarray(data, dtype=_NP[dtype])
+        assert data.size == int(np.prod(dims)), (name, dims, data.shape)
+        self.initializers[name] = (list(dims), dtype, data, [int(e) for e in exponents])
+
+    def add_value(self, name, dims, exponent, dtype=INT8):
+        self.value_info[name] = (list(dims), dtype, int(exponent))
+
+    def add_node(self, name, op_type, inputs, outputs, **attrs):
+        self.nodes.append({"name": name, "op_type": op_type, "inputs": list(inputs), "outputs": list(outputs),
+                           "attrs": attrs})
+
+    def shape(self, name):
+        return self.value_info[name][0]
+
+    def exponent(self, name):
+        return self.value_info[name][2]
+
+    def dtype(self, name):
+        return self.value_info[name][1]
+
+    def make_input(self, rng, batch, name=None):
+        """Seeded uniform input for the (single) graph input, whole batch."""
+        name = name or self.inputs[0]
+        dims, dtype, _ = self.value_info[name]
+        shape = [batch * dims[0]] + dims[1:]
+        if dtype == INT16:
+            return rng.integers(-32768, 32768, size=shape, dtype=np.int64).astype(np.int16)
+        return rng.integers(-128, 128, size=shape, dtype=np.int64).astype(np.int8)
+
+
+def typical_shift(k_total):
+    """Shift that maps the accumulator of K uniform-int8 products to a std of about 40."""
+    return max(1, int(round(math.log2(5461.0 * math.sqrt(k_total) / 40.0))))
+
+
+class Builder:
+    """Adds layers to a GraphSpec, tracking the current tensor name."""
+
+    def __init__(self, spec, seed, per_channel=True, w_exp_range=(-10, -6), bits=8):
+        self.g = spec
+        self.rng = np.random.default_rng(seed)
+        self.per_channel = per_channel
+        self.w_exp_range = w_exp_range
+        self.n = 0
+
+    def _name(self, prefix):
+        self.n += 1
+        return "%s_%d" % (prefix, self.n)
+
+    def _w_exps(self, oc, k_total=64):
+        """Per-channel filter exponents.  With an explicit range they are drawn from it; otherwise from
+        [-s-2, -s+2] with s = typical_shift(k_total), so that a layer neither amplifies nor shrinks its
+        input scale (trained networks behave the same way: the shipped MobileNetV2 has filter exponents
+        between -7 and -12 and activations that stay within a few exponents of each other)."""
+        if self.w_exp_range is None:
+            s = typical_shift(k_total)
+            lo, hi = -s - 2, -s + 2
+        else:
+            lo, hi = self.w_exp_range
+        if self.per_channel:
+            return self.rng.integers(lo, hi + 1, size=oc).astype(np.int64)
+        return np.array([(lo + hi) // 2], dtype=np.int64)
+
+    def input(self, name, dims, exponent, dtype=INT8):
+        self.g.add_value(name, dims, exponent, dtype)
+        self.g.inputs.append(name)
+        return name
+
+    def conv(self, x, out_c, k=1, stride=1, pad=None, dilation=1, depthwise=False, relu=False, bias=True,
+             out_exp=None, name=None, s16=False, gain=0):
+        """Conv2D (dense or depthwise).  `gain` lowers the output exponent (finer scale, more saturation)."""
+        g = self.g
+        _, h, w, c = g.shape(x)
+        kh, kw = (k, k) if isinstance(k, int) else k
+        sh, sw = (stride, stride) if isinstance(stride, int) else stride
+        dh, dw = (dilation, dilation) if isinstance(dilation, int) else dilation
+        if pad is None:
+            pad = (dh * (kh - 1) // 2, dh * (kh - 1) // 2, dw * (kw - 1) // 2, dw * (kw - 1) // 2)
+        pt, pb, pl, pr = pad
+        oc = c if depthwise else out_c
+        oh = (h + pt + pb - dh * (kh - 1) - 1) // sh + 1
+        ow = (w + pl + pr - dw * (kw - 1) - 1) // sw + 1
+        name = name or self._name("dwconv" if depthwise else "conv")
+        wdt = INT16 if s16 else INT8
+        lim = 32768 if s16 else 128
+        if depthwise:
+            wt = self.rng.integers(-lim, lim, size=(kh, kw, c))
+            dims = [kh, kw, c, 1]
+            k_total = kh * kw
+        else:
+            wt = self.rng.integers(-lim, lim, size=(oc, kh, kw, c))
+            dims = [kh, kw, c, oc]
+            k_total = kh * kw * c
+        w_exps = self._w_exps(oc, k_total) - (8 if s16 else 0)
+        in_exp = g.exponent(x)
+        if out_exp is None:
+            med = int(np.median(w_exps))
+            out_exp = typical_shift(k_total) + (8 if s16 else 0) + in_exp + med - gain
+        g.add_init(name + ".weight", dims, wdt, wt, w_exps)
+        inputs = [x, name + ".weight"]
+        if bias:
+            if s16:
+                b = self.rng.integers(-2 ** 26, 2 ** 26, size=oc)
+                g.add_init(name + ".bias", [oc], INT64, b, in_exp + w_exps)
+            else:
+                b = self.rng.integers(-4096, 4097, size=oc)
+                g.add_init(name + ".bias", [oc], INT32, b, in_exp + w_exps)
+            inputs.append(name + ".bias")
+        y = name + "_out"
+        g.add_value(y, [1, oh, ow, oc], out_exp, INT16 if s16 else INT8)
+        # pads attribute in ONNX order [t, l, b, r] (Conv::deserialize re-orders it)
+        g.add_node(name, "Conv", inputs, [y], pads=[pt, pl, pb, pr], strides=[sh, sw], dilations=[dh, dw],
+                   group=(c if depthwise else 1), activation=("Relu" if relu else "Linear"),
+                   quant_type=("S16" if s16 else "S8"))
+        macs = oh * ow * oc * k_total
+        g.macs_per_image += macs
+        g.conv_macs_per_image += macs
+        return y
+
+    def gemm(self, x, out_f, relu=False, bias=True, out_exp=None, name=None, matmul=False):
+        g = self.g
+        dims = g.shape(x)
+        k = dims[-1]
+        name = name or self._name("matmul" if matmul else "gemm")
+        wt = self.rng.integers(-128, 128, size=(out_f, k))
+        w_exps = self._w_exps(out_f, k)
+        in_exp = g.exponent(x)
+        if out_exp is None:
+            out_exp = typical_shift(k) + in_exp + int(np.median(w_exps))
+        g.add_init(name + ".weight", [1, 1, k, out_f], INT8, wt, w_exps)
+        inputs = [x, name + ".weight"]
+        if bias and not matmul:
+            b = self.rng.integers(-4096, 4097, size=out_f)
+            g.add_init(name + ".bias", [out_f], INT32, b, in_exp + w_exps)
+            inputs.append(name + ".bias")
+        y = name + "_out"
+        g.add_value(y, dims[:-1] + [out_f], out_exp)
+        g.add_node(name, "MatMul" if matmul else "Gemm", inputs, [y], activation=("Relu" if relu else "Linear"),
+                   quant_type="S8")
+        g.macs_per_image += int(np.prod(dims[1:-1])) * k * out_f if len(dims) > 2 else k * out_f
+        return y
+
+    def lut(self, x, fn, op_type="LUT", out_exp=None, name=None):
+        """8-bit table activation: table[i] = clip(round(fn((i-128) * 2^in_exp) / 2^out_exp))."""
+        g = self.g
+        name = name or self._name(op_type.lower())
+        in_exp = g.exponent(x)
+        out_exp = in_exp if out_exp is None else out_exp
+        table = make_lut(fn, in_exp, out_exp)
+        g.add_init(name + ".lut", [256], INT8, table, [out_exp])
+        y = name + "_out"
+        g.add_value(y, g.shape(x), out_exp)
+        g.add_node(name, op_type, [x], [y], lut=name + ".lut", quant_type="S8")
+        return y
+
+    def clip(self, x, lo_q, hi_q, out_exp=None, name=None):
+        g = self.g
+        name = name or self._name("clip")
+        e = g.exponent(x)
+        g.add_init(name + ".min", [1], INT8, [lo_q], [e])
+        g.add_init(name + ".max", [1], INT8, [hi_q], [e])
+        y = name + "_out"
+        g.add_value(y, g.shape(x), e if out_exp is None else out_exp)
+        g.add_node(name, "Clip", [x, name + ".min", name + ".max"], [y], quant_type="S8")
+        return y
+
+    def relu(self, x, name=None):
+        g = self.g
+        name = name or self._name("relu")
+        y = name + "_out"
+        g.add_value(y, g.shape(x), g.exponent(x))
+        g.add_node(name, "Relu", [x], [y], quant_type="S8")
+        return y
+
+    def prelu(self, x, name=None, alpha_exp=-7, out_exp=None):
+        g = self.g
+        name = name or self._name("prelu")
+        c = g.shape(x)[-1]
+        alpha = self.rng.integers(-128, 128, size=c)
+        g.add_init(name + ".slope", [c, 1, 1], INT8, alpha, [alpha_exp])
+        y = name + "_out"
+        g.add_value(y, g.shape(x), g.exponent(x) if out_exp is None else out_exp)
+        g.add_node(name, "PRelu", [x, name + ".slope"], [y], quant_type="S8")
+        return y
+
+    def requantize(self, x, out_exp, name=None):
+        g = self.g
+        name = name or self._name("requant")
+        y = name + "_out"
+        g.add_value(y, g.shape(x), out_exp, g.dtype(x))
+        g.add_node(name, "RequantizeLinear", [x], [y], quant_type="S8")
+        return y
+
+    def add(self, a, b, name=None):
+        """Residual add at matched exponents: the operand with the other exponent is requantized first,
+        which is what the exporter does by inserting RequantizeLinear."""
+        g = self.g
+        name = name or self._name("add")
+        ea, eb = g.exponent(a), g.exponent(b)
+        if ea != eb:
+            a = self.requantize(a, eb)
+        y = name + "_out"
+        g.add_value(y, g.shape(b), eb)
+        g.add_node(name, "Add", [a, b], [y], quant_type="S8")
+        return y
+
+    def global_avg_pool(self, x, out_exp=None, name=None):
+        g = self.g
+        name = name or self._name("gap")
+        n, h, w, c = g.shape(x)
+        y = name + "_out"
+        # the mean of roughly uniform values shrinks by about sqrt(area): keep resolution
+        e = g.exponent(x) - max(0, int(round(math.log2(math.sqrt(h * w))))) + 1 if out_exp is None else out_exp
+        g.add_value(y, [1, 1, 1, c], e)
+        g.add_node(name, "GlobalAveragePool", [x], [y], quant_type="S8")
+        return y
+
+    def flatten(self, x, name=None):
+        g = self.g
+        name = name or self._name("flatten")
+        dims = g.shape(x)
+        y = name + "_out"
+        g.add_value(y, [1, int(np.prod(dims[1:]))], g.exponent(x))
+        g.add_node(name, "Flatten", [x], [y], axis=1, quant_type="S8")
+        return y
+
+    def output(self, x):
+        self.g.outputs.append(x)
+        return x
+
+
+def make_lut(fn, in_exp, out_exp):
+    """Closed form of the exporter's 8-bit tables: entry i is fn at real input (i - 128) * 2^in_exp,
+    divided by 2^out_exp, rounded to nearest and clipped to int8."""
+    x = (np.arange(256, dtype=np.float64) - 128.0) * (2.0 ** in_exp)
+    y = np.asarray(fn(x), dtype=np.float64) / (2.0 ** out_exp)
+    return np.clip(np.rint(y), -128, 127).astype(np.int8)
+
+
+def silu(x):
+    with np.errstate(over="ignore"):
+        return x / (1.0 + np.exp(-x))
+
+
+def hardswish(x):
+    return x * np.clip(x + 3.0, 0.0, 6.0) / 6.0
+
+
+def relu6(x):
+    return np.clip(x, 0.0, 6.0)
+
+
+# ------------------------------------------------------------------------------------------------
+# The five benchmark configurations
+# ------------------------------------------------------------------------------------------------
+def config1_single_conv(seed=0xE5D1):
+    """int8 Conv2D 1x56x56x64 -> 64, 3x3, s1, p1, per-tensor exponents in -7 / w -8 / out -6, bias, ReLU."""
+    g = GraphSpec("config1_single_conv")
+    b = Builder(g, seed, per_channel=False, w_exp_range=(-8, -8))
+    x = b.input("input", [1, 56, 56, 64], -7)
+    y = b.conv(x, 64, k=3, stride=1, relu=True, out_exp=-6, name="conv")
+    b.output(y)
+    return g
+
+
+def config2_mbv2_block(seed=0xE5D2):
+    """MobileNetV2 inverted residual, 56x56x24: 1x1 -> 144, ReLU6 as Clip, dw 3x3 s1, 1x1 -> 24, residual Add."""
+    g = GraphSpec("config2_mbv2_block")
+    b = Builder(g, seed, per_channel=True)
+    x = b.input("input", [1, 56, 56, 24], -5)
+    e = b.conv(x, 144, k=1, name="expand")
+    six = min(127, int(round(6.0 / 2.0 ** g.exponent(e)))) if g.exponent(e) < 0 else 6
+    e = b.clip(e, 0, max(1, six), name="relu6_a")
+    d = b.conv(e, 144, k=3, depthwise=True, name="dw")
+    six = min(127, int(round(6.0 / 2.0 ** g.exponent(d)))) if g.exponent(d) < 0 else 6
+    d = b.clip(d, 0, max(1, six), name="relu6_b")
+    p = b.conv(d, 24, k=1, name="project")
+    y = b.add(x, p, name="residual")
+    b.output(y)
+    return g
+
+
+MBV2_TABLE = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]
+
+
+def config3_mobilenetv2(seed=0xE5D3, resolution=224, num_classes=1000, width=1.0):
+    """MobileNetV2-1.0 as ESP-DL runs it: ReLU fused into Conv (ReLU6 was replaced by ReLU before
+    quantization), project convs Linear, residual Adds, GlobalAveragePool, Flatten, Gemm head."""
+    g = GraphSpec("config3_mobilenetv2_%d" % resolution)
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, resolution, resolution, 3], -6)
+    x = b.conv(x, int(32 * width), k=3, stride=2, relu=True, name="stem")
+    cin = int(32 * width)
+    blk = 0
+    for t, c, n, s in MBV2_TABLE:
+        c = int(c * width)
+        for i in range(n):
+            stride = s if i == 0 else 1
+            blk += 1
+            skip = x
+            h = x
+            if t != 1:
+                h = b.conv(h, cin * t, k=1, relu=True, name="b%d_expand" % blk)
+            h = b.conv(h, cin * t, k=3, stride=stride, depthwise=True, relu=True, name="b%d_dw" % blk)
+            h = b.conv(h, c, k=1, relu=False, name="b%d_project" % blk)
+            if stride == 1 and cin == c:
+                h = b.add(skip, h, name="b%d_add" % blk)
+            x = h
+            cin = c
+    x = b.conv(x, int(1280 * max(1.0, width)), k=1, relu=True, name="head_conv")
+    x = b.global_avg_pool(x, name="gap")
+    x = b.flatten(x, name="flatten")
+    x = b.gemm(x, num_classes, name="classifier")
+    b.output(x)
+    return g
+
+
+def c3k2_like(b, x, c_out, name):
+    """YOLO11-style C3k2 / C2f block without Split/Concat (those data-movement ops are outside the
+    conv/gemm path): 1x1 reduce, two 3x3 bottleneck convs with SiLU tables and a residual Add, 1x1 fuse."""
+    g = b.g
+    h = b.conv(x, c_out // 2, k=1, name=name + "_cv1")
+    h = b.lut(h, silu, "Swish", name=name + "_cv1_act")
+    m = b.conv(h, c_out // 2, k=3, name=name + "_m1")
+    m = b.lut(m, silu, "Swish", name=name + "_m1_act")
+    m = b.conv(m, c_out // 2, k=3, name=name + "_m2")
+    m = b.lut(m, silu, "Swish", name=name + "_m2_act")
+    h = b.add(h, m, name=name + "_add")
+    y = b.conv(h, c_out, k=1, name=name + "_cv2")
+    return b.lut(y, silu, "Swish", name=name + "_cv2_act")
+
+
+def config4_yolo_style(seed=0xE5D4, resolution=640):
+    """YOLO11n-style detector trunk: int8 Conv backbone with SiLU as 8-bit LUT after every conv
+    (conv -> LUT pairs, as in the exported YOLO11n), strided 3x3 downsampling, bottleneck blocks
+    with residual Adds, and an int16 detection head (int16 weights and activations, int64 bias).
+    Concat / Split / Resize / MaxPool of the real graph are data movement outside the conv/gemm/LUT
+    path and are left out; channel widths follow YOLO11n (16-32-64-128-256)."""
+    g = GraphSpec("config4_yolo_style_%d" % resolution)
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, resolution, resolution, 3], -6)
+
+    def cbs(x, c, k, s, name):
+        y = b.conv(x, c, k=k, stride=s, name=name)
+        return b.lut(y, silu, "Swish", name=name + "_act")
+
+    x = cbs(x, 16, 3, 2, "p1")     # 320
+    x = cbs(x, 32, 3, 2, "p2")     # 160
+    x = c3k2_like(b, x, 64, "c2")
+    x = cbs(x, 64, 3, 2, "p3")     # 80
+    x = c3k2_like(b, x, 128, "c3")
+    p3 = x
+    x = cbs(x, 128, 3, 2, "p4")    # 40
+    x = c3k2_like(b, x, 128, "c4")
+    p4 = x
+    x = cbs(x, 256, 3, 2, "p5")    # 20
+    x = c3k2_like(b, x, 256, "c5")
+    p5 = x
+    # detection head per scale: int8 3x3 conv + SiLU, then int16 box branch (requantize to int16,
+    # int16 3x3 conv, int16 1x1 conv) and an int8 class branch
+    for i, (p, c) in enumerate(((p3, 64), (p4, 64), (p5, 64))):
+        h = cbs(p, c, 3, 1, "head%d_cv" % i)
+        h16 = "head%d_s16_in" % i
+        g.add_value(h16, g.shape(h), g.exponent(h) - 8, INT16)
+        g.add_node("head%d_to_s16" % i, "RequantizeLinear", [h], [h16], quant_type="S16")
+        box = b.conv(h16, c, k=3, s16=True, name="head%d_box1" % i)
+        box = b.conv(box, 64, k=1, s16=True, name="head%d_box2" % i)
+        b.output(box)
+        cls = cbs(h, 80, 1, 1, "head%d_cls1" % i)
+        cls = b.conv(cls, 80, k=1, name="head%d_cls2" % i)
+        b.output(cls)
+    return g
+
+
+def config5_ocr_style(seed=0xE5D5):
+    """PP-OCR-style text-line recognizer on 48x320x3 crops: conv backbone (3x3 and depthwise-separable
+    stages, hardswish tables) down to a 1x40x120 sequence, two int8 Gemm/MatMul layers
+    120 -> 480 -> 120 with LUT activation, and a 120 -> 6625 int8 Gemm classifier."""
+    g = GraphSpec("config5_ocr_style")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 48, 320, 3], -6)
+
+    def cbh(x, c, k, s, name, depthwise=False):
+        y = b.conv(x, c, k=k, stride=s, depthwise=depthwise, name=name)
+        return b.lut(y, hardswish, "HardSwish", name=name + "_act")
+
+    x = cbh(x, 16, 3, (2, 2), "stem")                  # 24 x 160
+    for i, (c, s) in enumerate(((32, (2, 2)), (64, (2, 2)), (120, (2, 1)), (120, (3, 1)))):
+        x = cbh(x, None, 3, s, "s%d_dw" % i, depthwise=True)
+        x = cbh(x, c, 1, 1, "s%d_pw" % i)
+    # now [1, 1, 40, 120]: a sequence of 40 steps of 120 features
+    _, h, w, c = g.shape(x)
+    assert (h, w, c) == (1, 40, 120), (h, w, c)
+    seq = "sequence"
+    g.add_value(seq, [1, 40, 120], g.exponent(x))
+    g.add_node("to_sequence", "Squeeze", [x], [seq], axes=[1], quant_type="S8")
+    y = b.gemm(seq, 480, name="fc1")
+    y = b.lut(y, hardswish, "HardSwish", name="fc1_act")
+    y = b.gemm(y, 120, name="fc2", matmul=True)
+    y = b.lut(y, hardswish, "HardSwish", name="fc2_act")
+    y = b.gemm(y, 6625, name="classifier")
+    b.output(y)
+    return g
+
+
+CONFIGS = {
+    1: config1_single_conv,
+    2: config2_mbv2_block,
+    3: config3_mobilenetv2,
+    4: config4_yolo_style,
+    5: config5_ocr_style,
+}

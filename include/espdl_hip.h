@@ -123,6 +123,14 @@ int espdl_hip_global_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int
 int espdl_hip_requantize_s8(const int8_t *in, int64_t size, int32_t in_exp, int32_t out_exp, int8_t *out,
                             void *stream);
 
+/* TensorBase::assign between int8 / int16 tensors of any two exponents
+ * (esp-dl/dl/tensor/src/dl_tensor_base.cpp:321-392): same exponent widens (int8 -> int16) or saturates
+ * (int16 -> int8); different exponents run quantize(dequantize(x)) in float32 with round-half-up.
+ * in_dtype / out_dtype are ESPDL_HIP_S8 or ESPDL_HIP_S16.  This is the int8 <-> int16 boundary of a
+ * mixed-precision graph. */
+int espdl_hip_requantize(const void *in, int32_t in_dtype, int64_t size, int32_t in_exp, int32_t out_exp, void *out,
+                         int32_t out_dtype, void *stream);
+
 /* Library / device information. */
 const char *espdl_hip_last_error(void);
 const char *espdl_hip_version(void);

@@ -1,0 +1,90 @@
+"""Runs a zoo.GraphSpec on the CPU oracle, node by node.  TEST INFRASTRUCTURE ONLY (see espdl_oracle.h).
+
+It mirrors what dl::Model does with the same spec: per node, read attributes the way the reference's
+Module::deserialize does (pads arrive in ONNX order [t,l,b,r] and are re-ordered to [t,b,l,r],
+esp-dl/dl/module/include/dl_module_conv.hpp:186-190), derive shift[c] = out_exp - w_exp[c] - in_exp
+(esp-dl/dl/base/dl_base.hpp:243-261) and call the oracle function of the operator.
+"""
+import numpy as np
+
+import espdl_oracle as oracle
+
+INT8, INT16 = 3, 5
+
+
+def _shift(spec, node, x_name, w_name, y_name):
+    w_exps = np.array(spec.initializers[w_name][3], dtype=np.int64)
+    return (spec.exponent(y_name) - w_exps - spec.exponent(x_name)).astype(np.int32)
+
+
+def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
+    """inputs: {name: ndarray for the whole batch}.  Returns {tensor name: ndarray}."""
+    t = dict(inputs)
+    for node in spec.nodes:
+        op, a = node["op_type"], node["attrs"]
+        ins, outs = node["inputs"], node["outputs"]
+        x = t[ins[0]]
+        y_name = outs[0]
+        if op == "Conv":
+            dims, wdt, w, _ = spec.initializers[ins[1]]
+            bias = spec.initializers[ins[2]][2] if len(ins) > 2 else None
+            kh, kw = dims[0], dims[1]
+            pt, pl, pb, pr = a["pads"]
+            shift = _shift(spec, node, ins[0], ins[1], y_name)
+            act = oracle.RELU if a.get("activation", "Linear") == "Relu" else oracle.LINEAR
+            depthwise = a.get("group", 1) != 1
+            s16 = a.get("quant_type") == "S16"
+            fn = {(False, False): oracle.conv2d_s8, (True, False): oracle.depthwise_s8,
+                  (False, True): oracle.conv2d_s16, (True, True): oracle.depthwise_s16}[(depthwise, s16)]
+            y = fn(x, w, bias, shift, (kh, kw), tuple(a["strides"]), tuple(a["dilations"]), (pt, pb, pl, pr), act,
+                   round_mode)
+        elif op in ("Gemm", "MatMul"):
+            w = spec.initializers[ins[1]][2]
+            bias = spec.initializers[ins[2]][2] if len(ins) > 2 else None
+            shift = _shift(spec, node, ins[0], ins[1], y_name)
+            act = oracle.RELU if a.get("activation", "Linear") == "Relu" else oracle.LINEAR
+            y = oracle.gemm_s8(x, w, bias, shift, activation=act, round_mode=round_mode)
+        elif "lut" in a:
+            y = oracle.lut_s8(x, spec.initializers[a["lut"]][2])
+        elif op == "Relu":
+            y = oracle.relu_s8(x, spec.exponent(ins[0]), spec.exponent(y_name))
+        elif op == "PRelu":
+            alpha_dims, _, alpha, alpha_exp = spec.initializers[ins[1]]
+            shift = spec.exponent(y_name) - spec.exponent(ins[0]) - alpha_exp[0]
+            y = oracle.prelu_s8(x, alpha, shift)
+        elif op == "Clip":
+            lo = int(spec.initializers[ins[1]][2].ravel()[0]) if len(ins) > 1 else -128
+            hi = int(spec.initializers[ins[2]][2].ravel()[0]) if len(ins) > 2 else 127
+            y = oracle.clip_s8(x, lo, hi, spec.exponent(ins[0]), spec.exponent(y_name))
+        elif op == "Add":
+            b = t[ins[1]]
+            assert x.shape == b.shape, "the graph runner only needs same-shape residual adds"
+            y = oracle.add_s8(x, b)
+        elif op == "GlobalAveragePool":
+            y = oracle.global_avg_pool_s8(x, spec.exponent(ins[0]), spec.exponent(y_name))
+        elif op == "RequantizeLinear":
+            y = requantize(x, spec.exponent(ins[0]), spec.exponent(y_name), spec.dtype(y_name))
+        elif op == "Flatten":
+            y = x.reshape(x.shape[0], -1)
+        elif op == "Squeeze":
+            y = np.squeeze(x, axis=tuple(a["axes"]))
+        else:
+            raise NotImplementedError(op)
+        t[y_name] = y
+    return t if keep_all else {k: t[k] for k in spec.outputs}
+
+
+def requantize(x, in_exp, out_exp, out_dtype_code):
+    """TensorBase::assign across exponents / widths (esp-dl/dl/tensor/src/dl_tensor_base.cpp:321-392):
+    same exponent -> widen or saturate; otherwise quantize(dequantize(x)) in float32 with round-half-up."""
+    out_np = np.int16 if out_dtype_code == INT16 else np.int8
+    lo, hi = (-32768, 32767) if out_dtype_code == INT16 else (-128, 127)
+    if x.dtype == np.int8 and out_np == np.int8:
+        return oracle.requantize_s8(x, in_exp, out_exp)
+    if in_exp == out_exp:
+        return np.clip(x.astype(np.int32), lo, hi).astype(out_np)
+    src_scale = np.float32(2.0 ** in_exp)
+    inv_scale = np.float32(1.0 / np.float32(2.0 ** out_exp))
+    tmp = x.astype(np.float32) * src_scale
+    q = np.floor((tmp * inv_scale).astype(np.float64) + 0.5).astype(np.float32)
+    return np.clip(q.astype(np.int64), lo, hi).astype(out_np)
