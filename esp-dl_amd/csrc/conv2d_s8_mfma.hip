@@ -20,9 +20,19 @@
 // read straight from global memory, 16 bytes per lane:
 //   B_VEC16   in_c % 16 == 0: the 16 k positions of a lane lie inside one filter tap -> one
 //             aligned 16-byte load, or zeros when the tap falls into the padding;
-//   B_POINT   1x1 filter without padding and in_c % 4 == 0: k is the channel index, the load may
-//             run past in_c into the next pixel (those positions meet zero weights);
+//   B_POINT   1x1 filter without padding: k is the channel index; one (possibly unaligned) 16-byte
+//             load that may run past in_c into the next pixel (those positions meet zero weights);
+//   B_ROWSEG  dilation_w == 1: the k_w * in_c bytes of one filter row are contiguous in the input, so
+//             the reduction axis is re-ordered as (ky, j) with every row segment padded to a
+//             multiple of 16; a lane's chunk is one unaligned 16-byte load, masked at the left and
+//             right image borders (the 3-channel stem convolutions run this way);
 //   B_GATHER  anything else: byte gather.
+// Epilogue.  When every shift of the workgroup's filters lies in 1..31, rounding is half-up and
+// |bias + 2^(s-1)| + K * 2^14 cannot overflow, the accumulator starts at bias + 2^(s-1) and a value
+// costs about three VALU instructions: t = (acc << max(0, 8-s)) >> max(0, s-8) carries the result in
+// bits 8.. of t, v_cvt_pk_i16_i32 saturates two of them to int16 (which saturates the int8 result
+// held in the high byte), and one v_perm_b32 gathers four high bytes into the output dword.
+// Otherwise the general shift_and_round restatement runs.
 // A workgroup is persistent: it keeps its filter chunk in LDS and walks pixel sets with a grid
 // stride.  If 64 filters x K do not fit the LDS budget, K is processed in chunks that are re-staged
 // between barriers while the accumulators stay in registers.
@@ -33,7 +43,7 @@ namespace espdl {
 
 namespace {
 
-enum { B_VEC16 = 0, B_POINT = 1, B_GATHER = 2 };
+enum { B_VEC16 = 0, B_POINT = 1, B_GATHER = 2, B_ROWSEG = 3 };
 
 constexpr int kThreads = 256;            // 4 wavefronts
 constexpr int kLdsSoftBudget = 64 * 1024; // two workgroups per CU
@@ -47,7 +57,9 @@ struct MfmaConvArgs {
     const int8_t *lut;
     int8_t *out;
     ConvGeom g;
-    int K;                // k_h * k_w * in_c
+    int K;                // length of the reduction axis as the MFMA sees it (k_h * seg_pad for B_ROWSEG)
+    int seg_len;          // B_ROWSEG: k_w * in_c, bytes of one filter row
+    int seg_pad;          // B_ROWSEG: seg_len rounded up to a multiple of 16
     int ksteps;           // ceil(K / 64)
     int ks_per_chunk;     // k steps resident in LDS at a time (== ksteps when everything fits)
     int n_kchunks;        // ceil(ksteps / ks_per_chunk)
@@ -81,7 +93,16 @@ __device__ __forceinline__ void stage_weights(const MfmaConvArgs &a, v4i *wts, i
             const int i = l & 15, gk = l >> 4;
             const int oc = gbase + 4 * nt * (i >> 2) + 4 * t + (i & 3);
             const int k = (ks_begin + ks) * 64 + gk * 16;
-            if (oc < OC && k < K) {
+            if (oc < OC && k < K && a.seg_pad > 0) {
+                // (ky, j) ordering: filter row ky starts at k = ky * seg_pad and holds seg_len bytes
+                const int ky = k / a.seg_pad, j0 = k - ky * a.seg_pad;
+                const int8_t *src = a.w + ((size_t)oc * a.g.k_h + ky) * a.seg_len + j0;
+                unsigned int words[4] = {0, 0, 0, 0};
+                const int n = min(16, a.seg_len - j0);
+                for (int b = 0; b < n; b++)
+                    words[b >> 2] |= (unsigned int)(unsigned char)src[b] << ((b & 3) * 8);
+                val = v4i{(int)words[0], (int)words[1], (int)words[2], (int)words[3]};
+            } else if (oc < OC && k < K) {
                 const int8_t *src = a.w + (size_t)oc * K + k;
                 if ((K & 15) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15) == 0) {
                     val = *reinterpret_cast<const v4i *>(src);
@@ -110,8 +131,7 @@ __device__ __forceinline__ v4i load_b(const MfmaConvArgs &a, bool valid, long lo
         // iy0 / ix0 are the input coordinates themselves (no padding, single tap)
         const long long off = img_off + ((long long)iy0 * g.in_w + ix0) * g.in_c + k;
         if (off + 16 <= a.in_bytes) {
-            const int *s = reinterpret_cast<const int *>(a.in + off);
-            r = v4i{s[0], s[1], s[2], s[3]};
+            __builtin_memcpy(&r, a.in + off, 16); // one dwordx4 load; gfx950 global loads need no alignment
         } else {
             unsigned int words[4] = {0, 0, 0, 0};
             const int n = min(16, a.K - k);
@@ -127,6 +147,37 @@ __device__ __forceinline__ v4i load_b(const MfmaConvArgs &a, bool valid, long lo
         const int iy = iy0 + ky * g.dil_h, ix = ix0 + kx * g.dil_w;
         if ((unsigned)iy < (unsigned)g.in_h && (unsigned)ix < (unsigned)g.in_w)
             r = *reinterpret_cast<const v4i *>(a.in + img_off + ((long long)iy * g.in_w + ix) * g.in_c + c0);
+        return r;
+    }
+    if (BMODE == B_ROWSEG) {
+        const int ky = k / a.seg_pad, j0 = k - ky * a.seg_pad;
+        const int iy = iy0 + ky * g.dil_h;
+        if ((unsigned)iy >= (unsigned)g.in_h)
+            return r;
+        // valid bytes of this chunk: those whose input column lies inside the image
+        const int row_lo = -ix0 * g.in_c, row_hi = (g.in_w - ix0) * g.in_c; // j range inside the image
+        const int nlo = min(max(row_lo - j0, 0), 16), nhi = min(max(row_hi - j0, 0), 16);
+        if (nlo >= nhi)
+            return r;
+        const long long off = img_off + ((long long)iy * g.in_w + ix0) * g.in_c + j0;
+        if (off >= 0 && off + 16 <= a.in_bytes) {
+            __builtin_memcpy(&r, a.in + off, 16);
+            if (nlo > 0 || nhi < 16) {
+#pragma unroll
+                for (int w = 0; w < 4; w++) {
+                    const int hi_n = min(max(nhi - 4 * w, 0), 4), lo_n = min(max(nlo - 4 * w, 0), 4);
+                    const unsigned hi_m = hi_n >= 4 ? 0xffffffffu : ((1u << (8 * hi_n)) - 1u);
+                    const unsigned lo_m = lo_n >= 4 ? 0xffffffffu : ((1u << (8 * lo_n)) - 1u);
+                    r[w] = (int)((unsigned)r[w] & hi_m & ~lo_m);
+                }
+            }
+        } else {
+            unsigned int words[4] = {0, 0, 0, 0};
+            const int stop = min(nhi, a.seg_len - j0);
+            for (int b = nlo; b < stop; b++)
+                words[b >> 2] |= (unsigned int)(unsigned char)a.in[off + b] << ((b & 3) * 8);
+            r = v4i{(int)words[0], (int)words[1], (int)words[2], (int)words[3]};
+        }
         return r;
     }
     // B_GATHER
@@ -157,8 +208,8 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
     extern __shared__ __align__(16) unsigned char smem[];
     const int gpc = a.groups_per_chunk;
     v4i *wts = reinterpret_cast<v4i *>(smem);
-    int *bias_l = reinterpret_cast<int *>(smem + (size_t)gpc * a.ks_per_chunk * 4096);
-    int *shift_l = bias_l + gpc * 64;
+    int *init_l = reinterpret_cast<int *>(smem + (size_t)gpc * a.ks_per_chunk * 4096); // accumulator start value
+    int *shift_l = init_l + gpc * 64; // fast epilogue: lsh | rsh << 8; general epilogue: the raw shift
     int8_t *lut_l = reinterpret_cast<int8_t *>(shift_l + gpc * 64);
 
     const ConvGeom &g = a.g;
@@ -169,15 +220,43 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
     const int g_count = min(gpc, a.n_groups - g_first);
     const bool relu = g.relu != 0, half_even = g.half_even != 0, has_lut = a.lut != nullptr;
 
+    // Can this workgroup's filters take the short epilogue?  Every shift in 1..31, and the sum
+    // bias + 2^(s-1) + (k_h*k_w*in_c products of at most 2^14) must fit int32 even after the left
+    // shift by max(0, 8-s) that the short form applies.
+    const long long mac_bound = (long long)g.k_h * g.k_w * g.in_c * 16384;
+    int ok_local = half_even ? 0 : 1;
     for (int c = tid; c < g_count * 64; c += kThreads) {
         const int oc = g_first * 64 + c;
-        bias_l[c] = (a.bias != nullptr && oc < OC) ? a.bias[oc] : 0;
-        shift_l[c] = oc < OC ? a.shift[g.n_shift == 1 ? 0 : oc] : 0;
+        if (oc < OC) {
+            const int s = a.shift[g.n_shift == 1 ? 0 : oc];
+            const long long b = a.bias != nullptr ? (long long)a.bias[oc] : 0;
+            if (s < 1 || s > 31) {
+                ok_local = 0;
+            } else {
+                const long long start = b + (1ll << (s - 1));
+                const long long mag = (start < 0 ? -start : start) + mac_bound;
+                if (mag >= (1ll << (31 - max(0, 8 - s))))
+                    ok_local = 0;
+            }
+        }
     }
     if (has_lut)
         lut_l[tid] = a.lut[tid];
     if (a.n_kchunks == 1)
         stage_weights(a, wts, g_first, g_count, 0, a.ksteps);
+    const bool fast = __syncthreads_and(ok_local) != 0;
+    for (int c = tid; c < g_count * 64; c += kThreads) {
+        const int oc = g_first * 64 + c;
+        int init = 0, sh = fast ? (8 << 8) : 0;
+        if (oc < OC) {
+            const int s = a.shift[g.n_shift == 1 ? 0 : oc];
+            const int b = a.bias != nullptr ? a.bias[oc] : 0;
+            init = fast ? b + (1 << (s - 1)) : b;
+            sh = fast ? (max(0, 8 - s) | (max(0, s - 8) << 8)) : s;
+        }
+        init_l[c] = init;
+        shift_l[c] = sh;
+    }
     __syncthreads();
 
     const long long out_hw = (long long)g.out_h * g.out_w;
@@ -213,12 +292,17 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
         for (int gi = 0; gi < g_count; gi++) {
             const int gbase = (g_first + gi) * 64;
             const int nt = group_tiles(OC, gbase);
+            // accumulators start at bias (+ rounding constant on the short path): integer addition
+            // wraps associatively, so adding it first or last gives the same 32-bit value
+            const int c_local = gi * 64 + 4 * nt * quad;
             v4i acc[PT][4];
 #pragma unroll
-            for (int p = 0; p < PT; p++)
+            for (int t = 0; t < 4; t++) {
+                const v4i start = t < nt ? *reinterpret_cast<const v4i *>(init_l + c_local + 4 * t) : v4i{0, 0, 0, 0};
 #pragma unroll
-                for (int t = 0; t < 4; t++)
-                    acc[p][t] = v4i{0, 0, 0, 0};
+                for (int p = 0; p < PT; p++)
+                    acc[p][t] = start;
+            }
 
             if (KSC > 0) {
 #pragma unroll
@@ -266,8 +350,11 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
             }
 
             // epilogue: this lane owns output channels [c_lane, c_lane + 4*nt) of pixel pix[p]
-            const int c_local = gi * 64 + 4 * nt * quad;
             const int c_lane = gbase + 4 * nt * quad;
+            v4i ss[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+                ss[t] = t < nt ? *reinterpret_cast<const v4i *>(shift_l + c_local + 4 * t) : v4i{0, 0, 0, 0};
 #pragma unroll
             for (int p = 0; p < PT; p++) {
                 int words[4];
@@ -275,16 +362,29 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
                 for (int t = 0; t < 4; t++) {
                     words[t] = 0;
                     if (t < nt) {
-                        const v4i bb = *reinterpret_cast<const v4i *>(bias_l + c_local + 4 * t);
-                        const v4i ss = *reinterpret_cast<const v4i *>(shift_l + c_local + 4 * t);
-                        int q[4];
+                        if (fast) {
+                            int tv[4];
 #pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            q[r] = requant_s8(acc[p][t][r] + bb[r], ss[r], relu, half_even);
-                            if (has_lut)
-                                q[r] = lut_l[q[r] + 128];
+                            for (int r = 0; r < 4; r++) {
+                                const int sh = ss[t][r];
+                                int v = (int)((unsigned)acc[p][t][r] << (sh & 31)) >> (sh >> 8);
+                                tv[r] = relu ? max(v, 0) : v;
+                            }
+                            const int p01 = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(tv[0], tv[1]));
+                            const int p23 = __builtin_bit_cast(int, __builtin_amdgcn_cvt_pk_i16(tv[2], tv[3]));
+                            words[t] = (int)__builtin_amdgcn_perm((unsigned)p23, (unsigned)p01, 0x07050301u);
+                        } else {
+                            int q[4];
+#pragma unroll
+                            for (int r = 0; r < 4; r++)
+                                q[r] = requant_s8(acc[p][t][r], ss[t][r], relu, half_even);
+                            words[t] = pack4_s8(q[0], q[1], q[2], q[3]);
                         }
-                        words[t] = pack4_s8(q[0], q[1], q[2], q[3]);
+                        if (has_lut) {
+                            const int w = words[t];
+                            words[t] = pack4_s8(lut_l[(int)(int8_t)w + 128], lut_l[(int)(int8_t)(w >> 8) + 128],
+                                                lut_l[(int)(int8_t)(w >> 16) + 128], lut_l[(w >> 24) + 128]);
+                        }
                     }
                 }
                 if (!pv[p])
@@ -357,7 +457,22 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     a.lut = lut;
     a.out = out;
     a.g = g;
+    const bool aligned16 = ((reinterpret_cast<uintptr_t>(in) & 15) == 0);
+    int bmode = B_GATHER;
+    if ((g.in_c & 15) == 0 && aligned16)
+        bmode = B_VEC16;
+    else if (g.k_h == 1 && g.k_w == 1 && g.pad_top == 0 && g.pad_left == 0 && (g.out_h - 1) * g.stride_h < g.in_h &&
+             (g.out_w - 1) * g.stride_w < g.in_w)
+        bmode = B_POINT;
+    else if (g.dil_w == 1)
+        bmode = B_ROWSEG;
+    a.seg_len = a.seg_pad = 0;
     a.K = g.k_h * g.k_w * g.in_c;
+    if (bmode == B_ROWSEG) {
+        a.seg_len = g.k_w * g.in_c;
+        a.seg_pad = (a.seg_len + 15) & ~15;
+        a.K = g.k_h * a.seg_pad;
+    }
     a.ksteps = (a.K + 63) / 64;
     a.n_groups = (g.out_c + 63) / 64;
     a.npix = (long long)g.batch * g.out_h * g.out_w;
@@ -397,20 +512,13 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
         gx &= ~7;
     dim3 grid((unsigned)gx, (unsigned)n_chunks, 1);
 
-    const bool aligned16 = ((reinterpret_cast<uintptr_t>(in) & 15) == 0);
-    int bmode = B_GATHER;
-    if ((g.in_c & 15) == 0 && aligned16)
-        bmode = B_VEC16;
-    else if (g.k_h == 1 && g.k_w == 1 && g.pad_top == 0 && g.pad_left == 0 && (g.in_c & 3) == 0 &&
-             ((reinterpret_cast<uintptr_t>(in) & 3) == 0) &&
-             (g.out_h - 1) * g.stride_h < g.in_h && (g.out_w - 1) * g.stride_w < g.in_w)
-        bmode = B_POINT;
-
     switch (bmode) {
     case B_VEC16:
         return launch_pt<B_VEC16>(a, pt, ksc, grid, lds, stream);
     case B_POINT:
         return launch_pt<B_POINT>(a, pt, ksc, grid, lds, stream);
+    case B_ROWSEG:
+        return launch_pt<B_ROWSEG>(a, pt, ksc, grid, lds, stream);
     default:
         return launch_pt<B_GATHER>(a, pt, ksc, grid, lds, stream);
     }
