@@ -17,9 +17,12 @@ OBJ_DIR = os.path.join(HERE, "build")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
-             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             # keep MFMA accumulators in ordinary VGPRs: no v_accvgpr_read/write around the epilogue
+             "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
-KERNEL_SOURCES = ["conv2d_s8_mfma.hip", "depthwise_s8.hip", "conv_s16.hip", "elementwise_s8.hip", "espdl_hip_api.hip"]
+KERNEL_SOURCES = ["conv2d_s8_mfma.hip", "conv2d_s8_mfma_vec16.hip", "conv2d_s8_mfma_point.hip",
+                  "conv2d_s8_mfma_rowseg.hip", "conv2d_s8_mfma_gather.hip", "depthwise_s8.hip", "depthwise_s8_mfma.hip", "conv_s16.hip", "elementwise_s8.hip", "espdl_hip_api.hip"]
 
 
 def _run(cmd):

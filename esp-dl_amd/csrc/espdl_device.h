@@ -87,6 +87,53 @@ __host__ __device__ __forceinline__ float dl_rescale(int e)
     return e > 0 ? 1.0f / (float)(1 << e) : (float)(1 << -e);
 }
 
+typedef short v2s __attribute__((ext_vector_type(2)));
+
+// Short requantization of four accumulators that already hold bias + 2^(s-1): after the shifts the
+// result q sits in bits 8.. of t; v_cvt_pk_i16_i32 saturates t to int16, which saturates q to int8
+// in the high byte; ReLU is one packed max on the int16 pairs; v_perm_b32 gathers the four high bytes.
+// USE_LSH: some shift is below 8, so the value is first shifted left by max(0, 8-s).
+template <bool USE_LSH>
+__device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk)
+{
+    int t[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int v = USE_LSH ? (int)((unsigned)acc[r] << lsh[r]) : acc[r];
+        t[r] = v >> rsh[r];
+    }
+    // floor_pk holds the lower clamp twice as int16: 0 for ReLU, -32768 (no effect) otherwise
+    const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
+    const v2s p01 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(t[0], t[1]), floor2);
+    const v2s p23 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(t[2], t[3]), floor2);
+    return (int)__builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, p23), (unsigned)__builtin_bit_cast(int, p01),
+                                      0x07050301u);
+}
+
+// Division of a 31-bit unsigned number by a launch-invariant divisor: q = (mulhi(n, m) + n) >> s
+// with m = floor(2^32 * (2^s - d) / d) + 1, s = ceil(log2 d)  (Granlund-Montgomery; exact for
+// every n < 2^31).  The host fills the struct, the device spends three instructions.
+struct FastDiv {
+    unsigned int m, s, d;
+};
+
+inline FastDiv make_fastdiv(unsigned int d)
+{
+    FastDiv f;
+    f.d = d;
+    unsigned int s = 0;
+    while ((1ull << s) < d)
+        s++;
+    f.s = s;
+    f.m = (unsigned int)(((1ull << 32) * ((1ull << s) - d)) / d + 1);
+    return f;
+}
+
+__device__ __forceinline__ unsigned int fastdiv(unsigned int n, const FastDiv &f)
+{
+    return (__umulhi(n, f.m) + n) >> f.s;
+}
+
 __device__ __forceinline__ int pack4_s8(int a, int b, int c, int d)
 {
     return (a & 0xff) | ((b & 0xff) << 8) | ((c & 0xff) << 16) | ((d & 0xff) << 24);

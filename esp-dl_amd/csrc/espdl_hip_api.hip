@@ -77,7 +77,7 @@ int derive_geometry(const espdl_hip_conv_desc *d, espdl::ConvGeom *g)
     const long long in_elems = (long long)d->batch * d->in_h * d->in_w * d->in_c;
     const long long out_elems = (long long)d->batch * oh * ow * d->out_c;
     if (k_total > (1 << 24) || in_elems > (1ll << 40) || out_elems > (1ll << 40) || oh > INT_MAX || ow > INT_MAX ||
-        (long long)d->batch * oh * ow / 64 > INT_MAX / 2)
+        (long long)d->batch * oh * ow > INT_MAX - 65536 || oh * ow > INT_MAX / 2)
         return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
     g->batch = d->batch;
     g->in_h = d->in_h;
@@ -157,8 +157,12 @@ int espdl_hip_conv2d(const espdl_hip_conv_desc *desc, const void *in, const void
         const int8_t *f8 = static_cast<const int8_t *>(filter);
         const int32_t *b32 = static_cast<const int32_t *>(bias);
         int8_t *o8 = static_cast<int8_t *>(out);
-        if (depthwise)
+        if (depthwise) {
+            if (espdl::depthwise_s8_mfma_supports(g, in, out))
+                return device_status(espdl::launch_depthwise_s8_mfma(g, i8, f8, b32, shift, lut, o8, cu_count_cached(), s),
+                                     "depthwise_s8_mfma");
             return device_status(espdl::launch_depthwise_s8(g, i8, f8, b32, shift, lut, o8, s), "depthwise_s8");
+        }
         return device_status(espdl::launch_conv2d_s8_mfma(g, i8, f8, b32, shift, lut, o8, cu_count_cached(), s),
                              "conv2d_s8");
     }

@@ -18,11 +18,15 @@ struct ConvGeom {
 hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                  const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
                                  hipStream_t stream);
-// Largest k_h * k_w * in_c the MFMA kernel accepts (weights of one 64-filter group must fit in LDS).
-int conv2d_s8_mfma_max_k();
 
 hipError_t launch_depthwise_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                const int32_t *shift, const int8_t *lut, int8_t *out, hipStream_t stream);
+
+// Depthwise on the matrix pipe with a diagonal operand A (up to 12 taps, channels % 16 == 0).
+bool depthwise_s8_mfma_supports(const ConvGeom &g, const void *in, const void *out);
+hipError_t launch_depthwise_s8_mfma(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                    const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
+                                    hipStream_t stream);
 
 hipError_t launch_conv2d_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
                              const int32_t *shift, int16_t *out, hipStream_t stream);
