@@ -67,11 +67,23 @@ def cpu_baseline(pkg, spec, threads_all):
     out["single_thread_sample"] = "%d images in %.2f s" % (n1, t1)
     # all cores: OpenMP over batch*rows inside every oracle call
     oracle.set_threads(threads_all)
-    nall = max(threads_all, min(512, int(round(10.0 * threads_all / max(t_one, 1e-3)))))
-    x = spec.make_input(rng, nall)
+    # size the sample from a short multi-thread pass so that the timed one takes about 15 s
+    ncal = 4 * threads_all
+    x = spec.make_input(rng, ncal)
     t0 = time.perf_counter()
     graph_runner.run(spec, {spec.inputs[0]: x}, keep_all=False)
-    tall = time.perf_counter() - t0
+    t_cal = time.perf_counter() - t0
+    nall = max(threads_all, min(8192, int(round(15.0 * ncal / max(t_cal, 1e-3)))))
+    nall -= nall % threads_all
+    chunk = 256  # images per oracle call: bounds host memory (activations of every layer are kept per call)
+    done, tall = 0, 0.0
+    while done < nall:
+        n = min(chunk, nall - done)
+        x = spec.make_input(rng, n)
+        t0 = time.perf_counter()
+        graph_runner.run(spec, {spec.inputs[0]: x}, keep_all=False)
+        tall += time.perf_counter() - t0
+        done += n
     gmacs = spec.macs_per_image * nall / tall / 1e9
     return {
         "value": nall / tall, "unit": "images/s", "cores": threads_all, "kind": "port",
@@ -91,6 +103,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of HIP-graph replay")
     ap.add_argument("--profile-repeats", type=int, default=5)
+    ap.add_argument("--copy-mib", type=int, default=0,
+                    help="also run one plain device copy of this many MiB (a kernel of known traffic, the "
+                         "yardstick for FETCH_SIZE / WRITE_SIZE counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (images are independent, "
@@ -105,6 +120,13 @@ def main():
     torch.cuda.set_device(0)
     pkg = importlib.import_module("esp-dl_amd")
     pkg.lib()  # fails loudly when the HIP library is missing
+
+    if args.copy_mib > 0:
+        src = torch.randint(-128, 128, (args.copy_mib << 20,), dtype=torch.int8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.add(src, 1, out=dst)  # an element-wise kernel: reads and writes copy_mib MiB each
+        torch.cuda.synchronize()
+        del src, dst
 
     spec = pkg.zoo.CONFIGS[args.config]()
     batch = args.batch

@@ -10,7 +10,6 @@ using namespace mfma_conv;
 
 namespace {
 constexpr int kLdsPerWorkgroup = 64 * 1024; // dynamic LDS a workgroup may ask for without opting in
-constexpr int kLdsPerCu = 160 * 1024;       // gfx950
 } // namespace
 
 hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
@@ -91,20 +90,8 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     a.fd_k_w = make_fastdiv((unsigned)g.k_w);
     a.fd_seg_pad = make_fastdiv((unsigned)(a.seg_pad > 0 ? a.seg_pad : 1));
 
-    // persistent grid: as many workgroups per CU as LDS and registers allow (at most 8), split over
-    // the filter chunks; gridDim.x a multiple of 8 so that workgroups sharing a pixel set (same x,
-    // different filter chunk) land on the same XCD
-    int per_cu = (int)(kLdsPerCu / lds);
-    const int b_regs = (ksc > 0 ? ksc : 4) * pt * 4 * ((ksc > 0 && ksc * pt <= 16) ? 2 : 1);
-    const int vgpr_est = 48 + 16 * pt + b_regs;
-    per_cu = min(per_cu, max(1, 512 / vgpr_est));
-    per_cu = max(1, min(per_cu, 8));
-    int gx = max(1, (cus * per_cu) / n_chunks);
-    if (gx > a.n_sets)
-        gx = a.n_sets;
-    if (gx >= 8)
-        gx &= ~7;
-    dim3 grid((unsigned)gx, (unsigned)n_chunks, 1);
+    // persistent grid: sized by launch_variant from the residency of the chosen kernel variant
+    const GridPlan grid{cus, n_chunks};
 
     switch (bmode) {
     case B_VEC16:

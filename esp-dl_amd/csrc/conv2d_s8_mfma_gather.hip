@@ -5,7 +5,7 @@
 namespace espdl {
 namespace mfma_conv {
 
-hipError_t launch_gather(const MfmaConvArgs &a, int pt, int ksc, dim3 grid, size_t lds, hipStream_t stream)
+hipError_t launch_gather(const MfmaConvArgs &a, int pt, int ksc, GridPlan grid, size_t lds, hipStream_t stream)
 {
     (void)ksc;
     return pt == 2 ? launch_variant<B_GATHER, 2, 0>(a, grid, lds, stream)

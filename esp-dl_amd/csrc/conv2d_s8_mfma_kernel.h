@@ -428,19 +428,19 @@ __device__ __forceinline__ void run_group(const MfmaConvArgs &a, const WaveCtx &
 // The persistent loop over pixel sets with one epilogue flavour compiled in.
 template <int BMODE, int PT, int KSC, bool FAST, bool USE_LSH>
 __device__ __forceinline__ void run_sets(const MfmaConvArgs &a, const WaveCtx &w, int wave, int g_first, int g_count,
-                                         int set, PixelRef (&px)[PT], v4i (&bc)[PT][KSC > 0 ? KSC : 1])
+                                         const TileSeq &seq, PixelRef (&px)[PT], v4i (&bc)[PT][KSC > 0 ? KSC : 1])
 {
     constexpr bool kDoubleBuffer = KSC > 0 && KSC * PT <= 16;
     const int OC = a.g.out_c;
-    for (; set < a.n_sets; set += gridDim.x) {
+    for (int set = seq.first; set < seq.end; set += seq.step) {
         if constexpr (KSC == 0)
             decode_set<BMODE, PT>(a, set, wave, w.col, px);
         // operands of the next pixel set: issued now, consumed in the next iteration
         PixelRef px_next[PT];
         v4i bn[PT][kDoubleBuffer ? KSC : 1];
-        const int set_next = set + gridDim.x;
+        const int set_next = set + seq.step;
         if constexpr (kDoubleBuffer) {
-            if (set_next < a.n_sets) {
+            if (set_next < seq.end) {
                 decode_set<BMODE, PT>(a, set_next, wave, w.col, px_next);
                 load_all_b<BMODE, PT, KSC>(a, px_next, w.quad, bn);
             }
@@ -529,9 +529,10 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
     // first pixel set: get its operand loads going before anything else
     PixelRef px[PT];
     v4i bc[PT][KSC > 0 ? KSC : 1];
-    const int set = blockIdx.x;
+    const TileSeq seq = xcd_tile_sequence(a.n_sets);
+    const int set = seq.first;
     if constexpr (KSC > 0) {
-        if (set < a.n_sets) {
+        if (set < seq.end) {
             decode_set<BMODE, PT>(a, set, wave, col, px);
             load_all_b<BMODE, PT, KSC>(a, px, quad, bc);
         }
@@ -598,17 +599,32 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
     w.floor_pk = w.relu ? 0 : (int)0x80008000u;
     w.stage_out = a.stage_out != 0;
     if (fast && !use_lsh)
-        run_sets<BMODE, PT, KSC, true, false>(a, w, wave, g_first, g_count, set, px, bc);
+        run_sets<BMODE, PT, KSC, true, false>(a, w, wave, g_first, g_count, seq, px, bc);
     else if (fast)
-        run_sets<BMODE, PT, KSC, true, true>(a, w, wave, g_first, g_count, set, px, bc);
+        run_sets<BMODE, PT, KSC, true, true>(a, w, wave, g_first, g_count, seq, px, bc);
     else
-        run_sets<BMODE, PT, KSC, false, false>(a, w, wave, g_first, g_count, set, px, bc);
+        run_sets<BMODE, PT, KSC, false, false>(a, w, wave, g_first, g_count, seq, px, bc);
 }
 
+// What the host planner knows; the grid itself is sized per kernel variant from the number of
+// workgroups of that variant a CU can hold (registers and LDS), so that the persistent grid is
+// resident all at once: a grid larger than that would run in rounds, the last one partly empty.
+struct GridPlan {
+    int cus;      // compute units of the device
+    int n_chunks; // filter chunks = gridDim.y
+};
+
 template <int BMODE, int PT, int KSC>
-hipError_t launch_variant(const MfmaConvArgs &a, dim3 grid, size_t lds, hipStream_t stream)
+hipError_t launch_variant(const MfmaConvArgs &a, GridPlan plan, size_t lds, hipStream_t stream)
 {
-    hipLaunchKernelGGL((conv2d_s8_mfma_kernel<BMODE, PT, KSC>), grid, dim3(kThreads), lds, stream, a);
+    const int per_cu = resident_workgroups_per_cu(conv2d_s8_mfma_kernel<BMODE, PT, KSC>, kThreads, lds);
+    int gx = max(1, (plan.cus * per_cu) / plan.n_chunks);
+    if (gx > a.n_sets)
+        gx = a.n_sets;
+    if (gx >= 8)
+        gx &= ~7; // blockIdx.x % 8 is then the XCD of a workgroup, for every blockIdx.y
+    hipLaunchKernelGGL((conv2d_s8_mfma_kernel<BMODE, PT, KSC>), dim3((unsigned)gx, (unsigned)plan.n_chunks),
+                       dim3(kThreads), lds, stream, a);
     return hipGetLastError();
 }
 
@@ -623,7 +639,7 @@ inline int pick_ksc(int ksteps)
 }
 
 template <int BMODE, int PT>
-hipError_t launch_ksc(const MfmaConvArgs &a, int ksc, dim3 grid, size_t lds, hipStream_t stream)
+hipError_t launch_ksc(const MfmaConvArgs &a, int ksc, GridPlan grid, size_t lds, hipStream_t stream)
 {
     switch (ksc) {
     case 1:
@@ -650,10 +666,10 @@ hipError_t launch_ksc(const MfmaConvArgs &a, int ksc, dim3 grid, size_t lds, hip
 }
 
 // Per operand-B mode entry points, each compiled in its own translation unit.
-hipError_t launch_vec16(const MfmaConvArgs &a, int pt, int ksc, dim3 grid, size_t lds, hipStream_t stream);
-hipError_t launch_point(const MfmaConvArgs &a, int pt, int ksc, dim3 grid, size_t lds, hipStream_t stream);
-hipError_t launch_rowseg(const MfmaConvArgs &a, int pt, int ksc, dim3 grid, size_t lds, hipStream_t stream);
-hipError_t launch_gather(const MfmaConvArgs &a, int pt, int ksc, dim3 grid, size_t lds, hipStream_t stream);
+hipError_t launch_vec16(const MfmaConvArgs &a, int pt, int ksc, GridPlan grid, size_t lds, hipStream_t stream);
+hipError_t launch_point(const MfmaConvArgs &a, int pt, int ksc, GridPlan grid, size_t lds, hipStream_t stream);
+hipError_t launch_rowseg(const MfmaConvArgs &a, int pt, int ksc, GridPlan grid, size_t lds, hipStream_t stream);
+hipError_t launch_gather(const MfmaConvArgs &a, int pt, int ksc, GridPlan grid, size_t lds, hipStream_t stream);
 
 } // namespace mfma_conv
 } // namespace espdl

@@ -4,7 +4,7 @@
 namespace espdl {
 namespace mfma_conv {
 
-hipError_t launch_vec16(const MfmaConvArgs &a, int pt, int ksc, dim3 grid, size_t lds, hipStream_t stream)
+hipError_t launch_vec16(const MfmaConvArgs &a, int pt, int ksc, GridPlan grid, size_t lds, hipStream_t stream)
 {
     return pt == 2 ? launch_ksc<B_VEC16, 2>(a, ksc, grid, lds, stream) : launch_ksc<B_VEC16, 1>(a, ksc, grid, lds, stream);
 }

@@ -117,10 +117,11 @@ __device__ __forceinline__ void dw_block(const DwMfmaArgs &a, unsigned char *sme
         }
     }
 
-    int set = blockIdx.x;
+    const TileSeq seq = xcd_tile_sequence(a.n_sets);
+    int set = seq.first;
     DwPixel px;
     v4i b[kKs][NT];
-    if (set < a.n_sets) {
+    if (set < seq.end) {
         dw_decode(a, set, wave, col, px);
         dw_load<NT>(a, px, cb, dy, dx, b);
     }
@@ -175,11 +176,11 @@ __device__ __forceinline__ void dw_block(const DwMfmaArgs &a, unsigned char *sme
         ls[t] = *reinterpret_cast<const v4i *>(lsh_l + 4 * NT * quad + 4 * t);
     }
 
-    for (; set < a.n_sets; set += gridDim.x) {
+    for (; set < seq.end; set += seq.step) {
         DwPixel px_next;
         v4i bn[kKs][NT];
-        const int set_next = set + gridDim.x;
-        if (set_next < a.n_sets) {
+        const int set_next = set + seq.step;
+        if (set_next < seq.end) {
             dw_decode(a, set_next, wave, col, px_next);
             dw_load<NT>(a, px_next, cb, dy, dx, bn);
         }
@@ -295,14 +296,15 @@ hipError_t launch_depthwise_s8_mfma(const ConvGeom &g, const int8_t *in, const i
     a.fd_out_w = make_fastdiv((unsigned)g.out_w);
     a.fd_k_w = make_fastdiv((unsigned)g.k_w);
     const int cus = cu_count > 0 ? cu_count : 256;
-    // persistent: about 8 workgroups per CU over all channel blocks; x a multiple of 8 so that the
-    // channel blocks of one pixel set share an XCD (and its L2) 
-    int gx = max(1, (cus * 8) / a.n_cblk);
+    // persistent: as many workgroups as are resident at once, over all channel blocks; x a multiple of 8 so that
+    // blockIdx.x % 8 is the XCD of a workgroup (see xcd_tile_sequence)
+    const size_t lds = (size_t)kKs * 4 * 1024 + 3 * 64 * sizeof(int) + 256;
+    const int per_cu = resident_workgroups_per_cu(depthwise_s8_mfma_kernel, kThreads, lds);
+    int gx = max(1, (cus * per_cu) / a.n_cblk);
     if (gx > a.n_sets)
         gx = a.n_sets;
     if (gx >= 8)
         gx &= ~7;
-    const size_t lds = (size_t)kKs * 4 * 1024 + 3 * 64 * sizeof(int) + 256;
     hipLaunchKernelGGL(depthwise_s8_mfma_kernel, dim3((unsigned)gx, (unsigned)a.n_cblk), dim3(kThreads), lds, stream, a);
     return hipGetLastError();
 }

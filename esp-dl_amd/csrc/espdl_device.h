@@ -6,6 +6,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <mutex>
+#include <vector>
 #include <stdint.h>
 
 namespace espdl {
@@ -137,6 +139,67 @@ __device__ __forceinline__ unsigned int fastdiv(unsigned int n, const FastDiv &f
 __device__ __forceinline__ int pack4_s8(int a, int b, int c, int d)
 {
     return (a & 0xff) | ((b & 0xff) << 8) | ((c & 0xff) << 16) | ((d & 0xff) << 24);
+}
+
+// Tile sequence of one workgroup of a persistent grid.  The hardware deals workgroups to the eight
+// XCDs round-robin by their linear id, and every XCD has its own L2.  Striding tiles by gridDim.x
+// would therefore spread neighbouring tiles (which share input rows through the filter window) over
+// all eight L2s and each of them would fetch those rows from memory again.  Instead XCD x owns the
+// contiguous eighth [x * per, (x + 1) * per) of the tiles and its workgroups stride through that
+// range, so rows shared between neighbouring tiles are found in the L2 that already holds them.
+// Needs gridDim.x % 8 == 0 (gridDim.y slices then keep blockIdx.x % 8 as the XCD); otherwise the
+// plain strided sequence is used.
+struct TileSeq {
+    int first, step, end;
+};
+
+__device__ __forceinline__ TileSeq xcd_tile_sequence(int n_tiles)
+{
+    TileSeq s;
+    if ((gridDim.x & 7u) == 0) {
+        const int per = (n_tiles + 7) >> 3;
+        const int xcd = blockIdx.x & 7;
+        s.first = xcd * per + (int)(blockIdx.x >> 3);
+        s.step = (int)(gridDim.x >> 3);
+        s.end = min(n_tiles, (xcd + 1) * per);
+    } else {
+        s.first = blockIdx.x;
+        s.step = gridDim.x;
+        s.end = n_tiles;
+    }
+    return s;
+}
+
+// Workgroups of `kernel` (block size `threads`, `lds` bytes of dynamic LDS) that fit on one CU at
+// the same time, as the runtime computes it from the kernel's register and LDS use; clamped to
+// [1, 8].  Host only.  Looked up once per (kernel, lds) and remembered.
+template <typename Kernel>
+inline int resident_workgroups_per_cu(Kernel kernel, int threads, size_t lds)
+{
+    struct Entry {
+        const void *fn;
+        size_t lds;
+        int n;
+    };
+    static std::mutex mu;
+    static std::vector<Entry> seen;
+    const void *fn = reinterpret_cast<const void *>(kernel);
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        for (const Entry &e : seen)
+            if (e.fn == fn && e.lds == lds)
+                return e.n;
+    }
+    int n = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, lds) != hipSuccess || n < 1) {
+        (void)hipGetLastError();
+        n = 1;
+    }
+    if (n > 8)
+        n = 8;
+    std::lock_guard<std::mutex> lock(mu);
+    seen.push_back(Entry{fn, lds, n});
+    return n;
 }
 
 } // namespace espdl

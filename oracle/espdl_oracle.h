@@ -30,10 +30,17 @@
  *                                identity table                                           PINNED
  *   espdl_oracle_prelu_s8, _relu_s8, _add_s8   exhaustive over all int8 operand pairs against
  *                                closed forms in exact integers                           PINNED
- *   espdl_oracle_clip_s8, _global_avg_pool_s8, _requantize_s8   float32-defined in the reference
- *                                (floorf(x + 0.5) under -ffast-math); checked against exact
- *                                rational round-half-up, which fixes every non-tie case; the
- *                                reference itself could not be built here           PARITY UNPINNED (float ties)
+ *   espdl_oracle_clip_s8, _relu_s8 (exponent change), _requantize_s8   float32-defined in the reference
+ *                                (floorf(x * 2^k + 0.5)); for int8/int16 x and power-of-two
+ *                                scales every intermediate is exactly representable, so the
+ *                                result is fixed by the mathematics: checked exhaustively
+ *                                against round-half-up in exact rationals                 PINNED
+ *   espdl_oracle_global_avg_pool_s8   float32 mean times a float scale under -ffast-math in the
+ *                                reference; the restatement is checked against exact rational
+ *                                round-half-up, which fixes every case whose exact value is not
+ *                                within float rounding error of a tie; the reference itself
+ *                                cannot be built here (every translation unit needs ESP-IDF
+ *                                headers that are absent)                   PARITY UNPINNED (near-ties)
  */
 #ifndef ESPDL_ORACLE_H
 #define ESPDL_ORACLE_H
