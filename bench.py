@@ -30,6 +30,16 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E, published
 PEAK_INT8_TOPS = 5000.0      # MI355X dense int8 MFMA, published (5.0 POP/s)
 MACHINE_BALANCE = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)  # OP per byte
 
+# HBM bytes per launch (average over the launches of a step) of the default workload, from two
+# rocprofv3 counter runs of this program (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0: the factors a
+# 256 MiB element-wise kernel of known traffic gave in the same runs).  Only valid for config 3 at
+# batch 256; any other workload reports null.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
+    "depthwise_s8": (2 * 34040.0 + 37922.4) * 1024,
+    "conv2d_s8_mfma": (2 * 10972.8 + 30566.2) * 1024,
+    "elementwise_s8": None,
+}
+
 
 def kernel_family(info, spec_nodes):
     """Map a module to the kernel that runs it."""
@@ -184,6 +194,8 @@ def main():
     else:
         roofline = {"kernel": dom, "bound": "hbm", "achieved": kd["GBps"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": kd["hbm_frac"], "traffic": None}
+    if args.config == 3 and batch == 256:
+        roofline["traffic"] = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(dom)
     roofline["launches_per_step"] = kd["launches_per_step"]
     roofline["avg_launch_us"] = kd["avg_launch_us"]
     roofline["algorithmic_per_launch"] = (kd["algorithmic_ops_per_step"] if roofline["bound"] == "mfma"
