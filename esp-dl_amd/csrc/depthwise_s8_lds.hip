@@ -1,0 +1,512 @@
+// Depthwise int8 convolution for gfx950 with the input tile staged in LDS (channels % 16 == 0, up to
+// 12 filter taps).
+//
+// What it computes is depthwise_conv2d_33c1 / _hwc1 (esp-dl/dl/base/dl_base_depthwise_conv2d.cpp:19-65)
+// under dwconv_operation_shell's window clipping (esp-dl/dl/base/dl_base.hpp:1852-2102) and the n_wise
+// epilogue (esp-dl/dl/base/dl_base_activate_buffer.hpp:27-36, 61-72, 173-181, 201-210).
+//
+// The operator moves two bytes per nine multiply-accumulates, so it has to run at memory speed, and
+// that decides the structure:
+//   * Every input byte is read from global memory once per tile, as part of a contiguous run:
+//     a workgroup copies the (th*s + halo) x (tw*s + halo) x (16*gc channels) input patch of its
+//     output tile into LDS with 16-byte loads of consecutive addresses (a pixel's channel chunk is
+//     contiguous, a patch row is contiguous when the chunk is the whole pixel).  Out-of-image
+//     positions are written as zeros, which is the reference's window clipping.  The patch of the
+//     next tile is in flight (in registers) while the current one is computed.
+//   * The byte products run on v_mfma_i32_16x16x64_i8 with a diagonal operand A (rows = 16 channels,
+//     reduction axis = (tap, channel), A[i][(tap, c)] = w[tap][i] if c == i): three MFMAs finish 16
+//     pixels x 16 channels x up to 12 taps, and operand B is one 16-byte LDS read per lane and k
+//     step, at patch offset (pixel) + (tap) + 16 * group.  The vector ALU is left with three adds
+//     and the epilogue per MFMA tile.
+//   * MFMA tiles are taken group-major and split evenly over the four wavefronts; a wavefront
+//     rebuilds operand A and its per-channel constants only when the channel group changes.
+//   * Results go to an LDS copy of the output tile and leave as 16-byte stores of consecutive
+//     addresses.
+// A workgroup is persistent over tiles; tiles of one XCD are contiguous in memory (xcd_tile_sequence).
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include "espdl_device.h"
+#include "espdl_kernels.h"
+
+namespace espdl {
+
+namespace {
+
+constexpr int kThreads = 512; // 8 wavefronts share one patch: fewer chunks (registers) per thread
+constexpr int kWaves = kThreads / 64;
+constexpr int kKs = 3;     // k steps of 4 taps
+constexpr int kMaxIn = 5;  // 16-byte patch chunks per thread
+constexpr int kMaxOut = 4; // 16-byte output chunks per thread
+
+struct DwLdsArgs {
+    const int8_t *in;
+    const int8_t *w;
+    const int32_t *bias;
+    const int32_t *shift;
+    const int8_t *lut;
+    int8_t *out;
+    ConvGeom g;
+    int taps;
+    int th, tw;         // output tile, pixels
+    int ph, pw;         // input patch, pixels
+    int gc;             // channel groups of 16 per workgroup (divides in_c / 16)
+    int cs;             // LDS pixel stride of the patch, bytes (an odd number of 16-byte units)
+    int cso;            // LDS pixel stride of the output tile, bytes
+    int np;             // pixel tiles of 16 per output tile
+    int tiles_x, tiles_y;
+    int n_units;        // batch * tiles_y * tiles_x
+    int n_in_chunks;    // ph * pw * gc
+    int n_out_chunks;   // th * tw * gc
+    int tiles_per_wave; // ceil(gc * np / kWaves)
+    FastDiv fd_tiles_x, fd_tiles_yx, fd_pwgc, fd_gc, fd_tw, fd_np;
+    // LDS layout, byte offsets
+    int off_patch, off_out, off_a, off_init, off_ss, off_ls, off_pixtab, off_lut;
+};
+
+struct UnitPos {
+    int n, y0, x0; // image, first output row / column of the tile
+};
+
+__device__ __forceinline__ UnitPos dw_unit(const DwLdsArgs &a, int unit)
+{
+    UnitPos u;
+    const unsigned n = fastdiv((unsigned)unit, a.fd_tiles_yx);
+    const unsigned rem = (unsigned)unit - n * a.fd_tiles_yx.d;
+    const unsigned ty = fastdiv(rem, a.fd_tiles_x);
+    u.n = (int)n;
+    u.y0 = (int)ty * a.th;
+    u.x0 = (int)(rem - ty * a.fd_tiles_x.d) * a.tw;
+    return u;
+}
+
+// Patch chunks of this thread for one tile: global -> registers (zeros outside the image).
+__device__ __forceinline__ void dw_fetch(const DwLdsArgs &a, const UnitPos &u, int cc0, const int (&rel)[kMaxIn],
+                                         const int (&rc)[kMaxIn], v4i (&pv)[kMaxIn])
+{
+    const ConvGeom &g = a.g;
+    const int iy0 = u.y0 * g.stride_h - g.pad_top, ix0 = u.x0 * g.stride_w - g.pad_left;
+    const int8_t *base = a.in + (((long long)u.n * g.in_h + iy0) * g.in_w + ix0) * g.in_c + cc0;
+#pragma unroll
+    for (int i = 0; i < kMaxIn; i++) {
+        if (i * kThreads < a.n_in_chunks) { // uniform
+            const int iy = iy0 + (rc[i] & 0xffff), ix = ix0 + (rc[i] >> 16);
+            const bool ok = rc[i] >= 0 && (unsigned)iy < (unsigned)g.in_h && (unsigned)ix < (unsigned)g.in_w;
+            pv[i] = ok ? *reinterpret_cast<const v4i *>(base + rel[i]) : v4i{0, 0, 0, 0};
+        }
+    }
+}
+
+template <bool FAST, bool USE_LSH>
+__device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *smem, int wave, int lane,
+                                           const int (&tapoff)[kKs], int floor_pk)
+{
+    const ConvGeom &g = a.g;
+    const int col = lane & 15, quad = lane >> 4;
+    const bool relu = g.relu != 0, half_even = g.half_even != 0, has_lut = a.lut != nullptr;
+    const int *a_l = reinterpret_cast<const int *>(smem + a.off_a);
+    const int *pixtab = reinterpret_cast<const int *>(smem + a.off_pixtab);
+    const int8_t *lut_l = reinterpret_cast<const int8_t *>(smem + a.off_lut);
+    const unsigned char *patch = smem + a.off_patch;
+    unsigned char *out_l = smem + a.off_out;
+
+    const int t_end = min((wave + 1) * a.tiles_per_wave, a.gc * a.np);
+    int t = wave * a.tiles_per_wave;
+    if (t >= t_end)
+        return;
+    int grp = (int)fastdiv((unsigned)t, a.fd_np);
+    int p = t - grp * a.np;
+
+    const int sel = col >> 2; // dword of the 16-byte operand A vector that holds this row's weight
+    v4i aop[kKs], init, ss, ls;
+    auto load_group = [&](int gi) {
+#pragma unroll
+        for (int ks = 0; ks < kKs; ks++) {
+            const int d = a_l[(gi * kKs + ks) * 64 + lane];
+            aop[ks] = v4i{sel == 0 ? d : 0, sel == 1 ? d : 0, sel == 2 ? d : 0, sel == 3 ? d : 0};
+        }
+        const int ch = 16 * gi + 4 * quad;
+        init = *reinterpret_cast<const v4i *>(smem + a.off_init + 4 * ch);
+        ss = *reinterpret_cast<const v4i *>(smem + a.off_ss + 4 * ch);
+        ls = *reinterpret_cast<const v4i *>(smem + a.off_ls + 4 * ch);
+    };
+    int grp_loaded = -1;
+
+    v4i b[kKs];
+    {
+        const int po = pixtab[p * 16 + col] + 16 * grp;
+#pragma unroll
+        for (int ks = 0; ks < kKs; ks++)
+            b[ks] = *reinterpret_cast<const v4i *>(patch + po + tapoff[ks]);
+    }
+    const int out_lane = col * a.cso + 4 * quad;
+    for (; t < t_end; t++) {
+        if (grp != grp_loaded) { // uniform; once per np tiles
+            load_group(grp);
+            grp_loaded = grp;
+        }
+        int p_next = p + 1, grp_next = grp;
+        if (p_next == a.np) {
+            p_next = 0;
+            grp_next = grp + 1;
+        }
+        const int out_off = out_lane + p * 16 * a.cso + 16 * grp;
+        v4i acc = init;
+#pragma unroll
+        for (int ks = 0; ks < kKs; ks++)
+            if (4 * ks < a.taps)
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], acc, 0, 0, 0);
+        // operand B of the next tile of this wavefront is read while this one is in the matrix pipe
+        if (t + 1 < t_end) {
+            const int po = pixtab[p_next * 16 + col] + 16 * grp_next;
+#pragma unroll
+            for (int ks = 0; ks < kKs; ks++)
+                b[ks] = *reinterpret_cast<const v4i *>(patch + po + tapoff[ks]);
+        }
+        int word;
+        if (FAST) {
+            word = pack_fast4<USE_LSH>(acc, ls, ss, floor_pk);
+        } else {
+            int q[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                q[r] = requant_s8(acc[r], ss[r], relu, half_even);
+            word = pack4_s8(q[0], q[1], q[2], q[3]);
+        }
+        if (has_lut)
+            word = pack4_s8(lut_l[(int)(int8_t)word + 128], lut_l[(int)(int8_t)(word >> 8) + 128],
+                            lut_l[(int)(int8_t)(word >> 16) + 128], lut_l[(word >> 24) + 128]);
+        *reinterpret_cast<int *>(out_l + out_off) = word;
+        p = p_next;
+        grp = grp_next;
+    }
+}
+
+__global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwLdsArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const ConvGeom &g = a.g;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int quad = lane >> 4;
+    const int C = g.in_c;
+    const int cc0 = blockIdx.y * a.gc * 16; // first channel of this workgroup's chunk
+    const int cw = a.gc * 16;
+    const bool half_even = g.half_even != 0;
+
+    // per-thread chunk descriptors: the tile geometry is the same for every tile
+    int in_rel[kMaxIn], in_lds[kMaxIn], in_rc[kMaxIn];
+#pragma unroll
+    for (int i = 0; i < kMaxIn; i++) {
+        const int k = tid + i * kThreads;
+        if (k < a.n_in_chunks) {
+            const unsigned prow = fastdiv((unsigned)k, a.fd_pwgc);
+            const unsigned rem = (unsigned)k - prow * a.fd_pwgc.d;
+            const unsigned pcol = fastdiv(rem, a.fd_gc);
+            const unsigned c16 = rem - pcol * a.fd_gc.d;
+            in_rel[i] = (int)((prow * g.in_w + pcol) * C + c16 * 16);
+            in_lds[i] = (int)((prow * a.pw + pcol) * a.cs + c16 * 16);
+            in_rc[i] = (int)(prow | (pcol << 16));
+        } else {
+            in_rel[i] = 0;
+            in_lds[i] = -1;
+            in_rc[i] = -1;
+        }
+    }
+    int out_rel[kMaxOut], out_lds[kMaxOut], out_rc[kMaxOut];
+#pragma unroll
+    for (int i = 0; i < kMaxOut; i++) {
+        const int k = tid + i * kThreads;
+        if (k < a.n_out_chunks) {
+            const unsigned q = fastdiv((unsigned)k, a.fd_gc);
+            const unsigned c16 = (unsigned)k - q * a.fd_gc.d;
+            const unsigned py = fastdiv(q, a.fd_tw);
+            const unsigned px = q - py * a.fd_tw.d;
+            out_rel[i] = (int)((py * g.out_w + px) * C + c16 * 16);
+            out_lds[i] = (int)(q * a.cso + c16 * 16);
+            out_rc[i] = (int)(py | (px << 16));
+        } else {
+            out_rel[i] = 0;
+            out_lds[i] = 0;
+            out_rc[i] = -1;
+        }
+    }
+
+    const TileSeq seq = xcd_tile_sequence(a.n_units);
+    int unit = seq.first;
+    v4i pv[kMaxIn];
+    UnitPos u = {0, 0, 0};
+    if (unit < seq.end) {
+        u = dw_unit(a, unit);
+        dw_fetch(a, u, cc0, in_rel, in_rc, pv);
+    }
+
+    // tables: diagonal operand A as one dword per (group, k step, lane); start values and shifts;
+    // patch offset of every output pixel of the tile; the LUT
+    int *a_l = reinterpret_cast<int *>(smem + a.off_a);
+    for (int e = tid; e < a.gc * kKs * 64; e += kThreads) {
+        const int l = e & 63, ks = (e >> 6) % kKs, gi = e / (64 * kKs);
+        const int i = l & 15, tap = 4 * ks + (l >> 4);
+        int d = 0;
+        if (tap < a.taps)
+            d = (int)(unsigned char)a.w[(long long)tap * C + cc0 + 16 * gi + i] << (8 * (i & 3));
+        a_l[e] = d;
+    }
+    // start values and shifts: every thread owns at most one channel of the chunk (16 * gc <= 256)
+    const long long mac_bound = (long long)a.taps * 16384;
+    int ok_local = half_even ? 0 : 1;
+    int lsh_local = 0;
+    int my_s = 0, my_b = 0;
+    if (tid < cw) {
+        my_s = a.shift[g.n_shift == 1 ? 0 : cc0 + tid];
+        my_b = a.bias != nullptr ? a.bias[cc0 + tid] : 0;
+        if (my_s < 1 || my_s > 31) {
+            ok_local = 0;
+        } else {
+            const long long start = (long long)my_b + (1ll << (my_s - 1));
+            if ((start < 0 ? -start : start) + mac_bound >= (1ll << (31 - max(0, 8 - my_s))))
+                ok_local = 0;
+            if (my_s < 8)
+                lsh_local = 1;
+        }
+    }
+    const bool fast = __syncthreads_and(ok_local) != 0;
+    const bool use_lsh = __syncthreads_or(lsh_local) != 0;
+    {
+        if (tid < cw) {
+            reinterpret_cast<int *>(smem + a.off_init)[tid] = fast ? my_b + (1 << (my_s - 1)) : my_b;
+            reinterpret_cast<int *>(smem + a.off_ss)[tid] = fast ? max(0, my_s - 8) : my_s;
+            reinterpret_cast<int *>(smem + a.off_ls)[tid] = fast ? max(0, 8 - my_s) : 0;
+        }
+        int *pixtab = reinterpret_cast<int *>(smem + a.off_pixtab);
+        for (int q = tid; q < a.np * 16; q += kThreads) {
+            int off = 0;
+            if (q < a.th * a.tw) {
+                const unsigned py = fastdiv((unsigned)q, a.fd_tw);
+                const unsigned px = (unsigned)q - py * a.fd_tw.d;
+                off = (int)((py * g.stride_h * a.pw + px * g.stride_w) * a.cs);
+            }
+            pixtab[q] = off;
+        }
+        if (a.lut != nullptr && tid < 256)
+            reinterpret_cast<int8_t *>(smem + a.off_lut)[tid] = a.lut[tid];
+    }
+    // tap offsets of this lane's quad inside the patch
+    int tapoff[kKs];
+#pragma unroll
+    for (int ks = 0; ks < kKs; ks++) {
+        const int tap = 4 * ks + quad;
+        tapoff[ks] = 0;
+        if (tap < a.taps) {
+            const int ky = tap / g.k_w, kx = tap - ky * g.k_w;
+            tapoff[ks] = (ky * g.dil_h * a.pw + kx * g.dil_w) * a.cs;
+        }
+    }
+    const int floor_pk = g.relu ? 0 : (int)0x80008000u;
+
+    for (; unit < seq.end; unit += seq.step) {
+        // patch of this tile: registers -> LDS
+#pragma unroll
+        for (int i = 0; i < kMaxIn; i++)
+            if (i * kThreads < a.n_in_chunks && in_lds[i] >= 0)
+                *reinterpret_cast<v4i *>(smem + a.off_patch + in_lds[i]) = pv[i];
+        __syncthreads();
+        const UnitPos u_cur = u;
+        const int unit_next = unit + seq.step;
+        if (unit_next < seq.end) {
+            u = dw_unit(a, unit_next);
+            dw_fetch(a, u, cc0, in_rel, in_rc, pv); // in flight during the compute phase
+        }
+
+        if (fast && !use_lsh)
+            dw_compute<true, false>(a, smem, wave, lane, tapoff, floor_pk);
+        else if (fast)
+            dw_compute<true, true>(a, smem, wave, lane, tapoff, floor_pk);
+        else
+            dw_compute<false, false>(a, smem, wave, lane, tapoff, floor_pk);
+        __syncthreads();
+
+        // output tile: LDS -> global, consecutive 16-byte pieces
+        const int rows = min(a.th, g.out_h - u_cur.y0), cols = min(a.tw, g.out_w - u_cur.x0);
+        int8_t *obase = a.out + (((long long)u_cur.n * g.out_h + u_cur.y0) * g.out_w + u_cur.x0) * C + cc0;
+#pragma unroll
+        for (int i = 0; i < kMaxOut; i++) {
+            if (i * kThreads < a.n_out_chunks) { // uniform
+                const int py = out_rc[i] & 0xffff, px = out_rc[i] >> 16;
+                if (out_rc[i] >= 0 && py < rows && px < cols)
+                    *reinterpret_cast<v4i *>(obase + out_rel[i]) =
+                        *reinterpret_cast<const v4i *>(smem + a.off_out + out_lds[i]);
+            }
+        }
+        // the next iteration's patch stores touch only the patch area; its output stores come after
+        // the barrier that follows them, by which time these reads have completed
+    }
+}
+
+struct DwLdsPlan {
+    bool ok;
+    DwLdsArgs a;
+    size_t lds;
+    int n_cchunk;
+};
+
+constexpr int kLdsBudget = 80 * 1024; // two workgroups of 8 wavefronts per CU (160 KB of LDS)
+
+// Tile choice: the cheapest (patch bytes read per output byte, with a penalty for tiles too small
+// to amortize the per-tile barriers) among the candidates that fit the LDS and register budgets.
+DwLdsPlan dw_lds_plan(const ConvGeom &g)
+{
+    DwLdsPlan best;
+    best.ok = false;
+    const int G = g.in_c / 16;
+    const int taps = g.k_h * g.k_w;
+    const int halo_h = (g.k_h - 1) * g.dil_h + 1, halo_w = (g.k_w - 1) * g.dil_w + 1;
+    double best_cost = 1e30;
+    static const int sizes[] = {1, 2, 3, 4, 6, 7, 8, 12, 14, 16, 24, 28, 32, 56, 64, 112};
+    std::vector<int> cand_h, cand_w;
+    for (int v : sizes) {
+        if (v < g.out_h)
+            cand_h.push_back(v);
+        if (v < g.out_w)
+            cand_w.push_back(v);
+    }
+    cand_h.push_back(g.out_h);
+    cand_w.push_back(g.out_w);
+    for (int gc = 1; gc <= min(G, 16); gc++) {
+        if (G % gc != 0)
+            continue;
+        const int cs = 16 * ((gc & 1) ? gc : gc + 1); // odd number of 16-byte units: conflict-free LDS reads
+        const int cso = cs;
+        for (int the : cand_h) {
+            for (int twe : cand_w) {
+                const int ph = (the - 1) * g.stride_h + halo_h, pw = (twe - 1) * g.stride_w + halo_w;
+                const int np = (the * twe + 15) / 16;
+                const long long n_in = (long long)ph * pw * gc, n_out = (long long)the * twe * gc;
+                if (n_in > kMaxIn * kThreads || n_out > kMaxOut * kThreads || ph > 0xffff || pw > 0x7fff)
+                    continue;
+                const size_t patch = (size_t)ph * pw * cs + 16 * 16; // reads of padded pixel slots stay inside
+                const size_t outb = (size_t)np * 16 * cso;
+                const size_t tables = (size_t)gc * kKs * 64 * 4 + (size_t)gc * 16 * 12 + (size_t)np * 16 * 4 + 256;
+                const size_t lds = patch + outb + tables + 64;
+                if (lds > (size_t)kLdsBudget)
+                    continue;
+                const int per_cu = (int)std::min<size_t>(2, (size_t)(160 * 1024) / lds); // 2 x 8 wavefronts fill a CU
+                const double mfma_tiles = (double)np * gc;
+                // bytes through the memory system per output byte, relative
+                double cost = (double)ph * pw / ((double)the * twe) + 1.0;
+                cost *= (double)(np * 16) / (the * twe);           // idle MFMA columns also idle the LDS reads
+                cost *= 1.0 + 12.0 / mfma_tiles;                    // barriers and table walks per tile
+                cost *= per_cu >= 2 ? 1.0 : 1.6; // latency hiding needs co-resident tiles
+                // a pixel's channel chunk should cover whole 128-byte lines unless it is the whole pixel
+                if (gc < G && gc * 16 < 128)
+                    cost *= 1.0 + 0.5 * (128.0 / (gc * 16) - 1.0);
+                // partial tiles at the image edges
+                const int ty = (g.out_h + the - 1) / the, tx = (g.out_w + twe - 1) / twe;
+                cost *= (double)(ty * the) * (tx * twe) / ((double)g.out_h * g.out_w);
+                if (cost < best_cost) {
+                    best_cost = cost;
+                    best.ok = true;
+                    DwLdsArgs &a = best.a;
+                    a.taps = taps;
+                    a.th = the;
+                    a.tw = twe;
+                    a.ph = ph;
+                    a.pw = pw;
+                    a.gc = gc;
+                    a.cs = cs;
+                    a.cso = cso;
+                    a.np = np;
+                    a.tiles_y = ty;
+                    a.tiles_x = tx;
+                    a.n_in_chunks = (int)n_in;
+                    a.n_out_chunks = (int)n_out;
+                    a.tiles_per_wave = (gc * np + kWaves - 1) / kWaves;
+                    size_t off = 0;
+                    a.off_patch = (int)off;
+                    off += (patch + 15) & ~(size_t)15;
+                    a.off_out = (int)off;
+                    off += outb;
+                    a.off_a = (int)off;
+                    off += (size_t)gc * kKs * 64 * 4;
+                    a.off_init = (int)off;
+                    off += (size_t)gc * 16 * 4;
+                    a.off_ss = (int)off;
+                    off += (size_t)gc * 16 * 4;
+                    a.off_ls = (int)off;
+                    off += (size_t)gc * 16 * 4;
+                    a.off_pixtab = (int)off;
+                    off += (size_t)np * 16 * 4;
+                    a.off_lut = (int)off;
+                    off += 256;
+                    best.lds = off;
+                    best.n_cchunk = G / gc;
+                }
+            }
+        }
+    }
+    return best;
+}
+
+} // namespace
+
+bool depthwise_s8_lds_supports(const ConvGeom &g, const void *in, const void *out)
+{
+    if ((g.in_c & 15) != 0 || g.k_h * g.k_w > 4 * kKs ||
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) != 0)
+        return false;
+    // 32-bit offsets inside one image
+    if ((long long)g.in_h * g.in_w * g.in_c >= (1ll << 30) || (long long)g.out_h * g.out_w * g.out_c >= (1ll << 30))
+        return false;
+    return dw_lds_plan(g).ok;
+}
+
+hipError_t launch_depthwise_s8_lds(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                   const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
+                                   hipStream_t stream)
+{
+    if ((long long)g.batch * g.out_h * g.out_w == 0)
+        return hipSuccess;
+    DwLdsPlan plan = dw_lds_plan(g);
+    if (!plan.ok)
+        return hipErrorInvalidValue;
+    DwLdsArgs &a = plan.a;
+    a.in = in;
+    a.w = filter;
+    a.bias = bias;
+    a.shift = shift;
+    a.lut = lut;
+    a.out = out;
+    a.g = g;
+    const long long units = (long long)g.batch * a.tiles_y * a.tiles_x;
+    if (units > 0x7fffffff)
+        return hipErrorInvalidValue;
+    a.n_units = (int)units;
+    a.fd_tiles_x = make_fastdiv((unsigned)a.tiles_x);
+    a.fd_tiles_yx = make_fastdiv((unsigned)(a.tiles_y * a.tiles_x));
+    a.fd_pwgc = make_fastdiv((unsigned)(a.pw * a.gc));
+    a.fd_gc = make_fastdiv((unsigned)a.gc);
+    a.fd_tw = make_fastdiv((unsigned)a.tw);
+    a.fd_np = make_fastdiv((unsigned)a.np);
+    const int cus = cu_count > 0 ? cu_count : 256;
+    static const hipError_t lds_opt_in = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(depthwise_s8_lds_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+    if (lds_opt_in != hipSuccess)
+        return lds_opt_in;
+    const int per_cu = resident_workgroups_per_cu(depthwise_s8_lds_kernel, kThreads, plan.lds);
+    int gx = max(1, (cus * per_cu) / plan.n_cchunk);
+    if (gx > a.n_units)
+        gx = a.n_units;
+    if (gx >= 8)
+        gx &= ~7;
+    static const bool trace = getenv("ESPDL_HIP_TRACE") != nullptr;
+    if (trace)
+        fprintf(stderr, "depthwise_s8_lds: %dx%dx%d s%d tile %dx%d patch %dx%d gc %d np %d lds %zu per_cu %d grid %dx%d units %d\n",
+                g.in_h, g.in_w, g.in_c, g.stride_h, a.th, a.tw, a.ph, a.pw, a.gc, a.np, plan.lds, per_cu, gx, plan.n_cchunk,
+                a.n_units);
+    hipLaunchKernelGGL(depthwise_s8_lds_kernel, dim3((unsigned)gx, (unsigned)plan.n_cchunk), dim3(kThreads), plan.lds,
+                       stream, a);
+    return hipGetLastError();
+}
+
+} // namespace espdl

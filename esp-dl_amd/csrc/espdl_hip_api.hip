@@ -158,6 +158,9 @@ int espdl_hip_conv2d(const espdl_hip_conv_desc *desc, const void *in, const void
         const int32_t *b32 = static_cast<const int32_t *>(bias);
         int8_t *o8 = static_cast<int8_t *>(out);
         if (depthwise) {
+            if (espdl::depthwise_s8_lds_supports(g, in, out))
+                return device_status(espdl::launch_depthwise_s8_lds(g, i8, f8, b32, shift, lut, o8, cu_count_cached(), s),
+                                     "depthwise_s8_lds");
             if (espdl::depthwise_s8_mfma_supports(g, in, out))
                 return device_status(espdl::launch_depthwise_s8_mfma(g, i8, f8, b32, shift, lut, o8, cu_count_cached(), s),
                                      "depthwise_s8_mfma");

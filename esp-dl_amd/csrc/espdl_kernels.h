@@ -28,6 +28,13 @@ hipError_t launch_depthwise_s8_mfma(const ConvGeom &g, const int8_t *in, const i
                                     const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
                                     hipStream_t stream);
 
+// Depthwise with the input tile staged in LDS (contiguous global reads and writes) and the products
+// on the matrix pipe; same shape limits as the direct form.
+bool depthwise_s8_lds_supports(const ConvGeom &g, const void *in, const void *out);
+hipError_t launch_depthwise_s8_lds(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                   const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
+                                   hipStream_t stream);
+
 hipError_t launch_conv2d_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
                              const int32_t *shift, int16_t *out, hipStream_t stream);
 hipError_t launch_depthwise_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
