@@ -159,6 +159,45 @@ def test_depthwise_s8_config2_shape(oracle):
     np.testing.assert_array_equal(got, want)
 
 
+# Geometries aimed at the LDS-tile depthwise kernel: tiles that do not divide the image, channel
+# counts whose 16-channel groups split unevenly over workgroups, every tap count up to 12, dilation,
+# asymmetric padding, shifts below 8 (left-shift form of the short epilogue), the general epilogue
+# (half-even, shift 0 / 32), a fused LUT, per-tensor shift.
+# Fields: (name, (N, H, W, C), (kh, kw), stride, dilation, pads, bias, relu, shift_lo, shift_hi, half_even, lut, per_tensor)
+DW_TILE_CASES = [
+    ("n3_61x45x48_k3p1", (3, 61, 45, 48), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 7, 11, False, False, False),
+    ("n2_31x29x32_k3s2p1", (2, 31, 29, 32), (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, False, 8, 12, False, False, False),
+    ("n2_33x37x272_k3p1", (2, 33, 37, 272), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 6, 10, False, False, False),
+    ("n5_14x14x512_k3p1", (5, 14, 14, 512), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 9, 12, False, False, False),
+    ("n9_7x7x960_k3p1", (9, 7, 7, 960), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 9, 12, False, False, False),
+    ("n2_40x24x64_k3d2p2", (2, 40, 24, 64), (3, 3), (1, 1), (2, 2), (2, 2, 2, 2), True, True, 8, 11, False, False, False),
+    ("n2_25x40x16_k2x2_tailpad", (2, 25, 40, 16), (2, 2), (1, 1), (1, 1), (0, 1, 0, 1), False, False, 5, 9, False, False, False),
+    ("n2_20x33x80_k3x4_s12", (2, 20, 33, 80), (3, 4), (1, 2), (1, 1), (1, 1, 2, 1), True, True, 8, 12, False, False, False),
+    ("n2_1x100x48_k1x3p1", (2, 1, 100, 48), (1, 3), (1, 1), (1, 1), (0, 0, 1, 1), True, False, 6, 9, False, False, False),
+    ("n2_19x19x96_k3p1_halfeven", (2, 19, 19, 96), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 7, 11, True, False, False),
+    ("n2_19x19x96_k3p1_wide_shifts", (2, 19, 19, 96), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False, 0, 33, False, False, False),
+    ("n2_28x28x192_k3s2p1_lut", (2, 28, 28, 192), (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, True, 8, 11, False, True, False),
+    ("n2_56x56x144_k3p1_per_tensor", (2, 56, 56, 144), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 9, 9, False, False, True),
+    ("n1_112x112x32_k3p1", (1, 112, 112, 32), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 8, 11, False, False, False),
+    ("n1_112x112x96_k3s2_tailpad", (1, 112, 112, 96), (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), True, True, 8, 11, False, False, False),
+]
+
+
+@pytest.mark.parametrize("case", DW_TILE_CASES, ids=lambda c: c[0])
+def test_depthwise_s8_tiles(oracle, case):
+    announce(f"depthwise_s8 tiles {case[0]}")
+    name, (n, h, w, c), k, stride, dil, pads, has_bias, relu, s_lo, s_hi, half_even, with_lut, per_tensor = case
+    rng = np.random.default_rng(0xD3 + len(name))
+    x = rng_int8(rng, (n, h, w, c))
+    f = rng_int8(rng, (k[0], k[1], c))
+    bias = rng.integers(-4096, 4097, size=c).astype(np.int32) if has_bias else None
+    shift = np.int32(s_lo) if per_tensor else rng.integers(s_lo, s_hi + 1, size=c).astype(np.int32)
+    lut = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8) if with_lut else None
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, depthwise=True,
+                             half_even=half_even, lut=lut)
+    np.testing.assert_array_equal(got, want)
+
+
 def _run_conv_s16(oracle, x, f, bias, shift, k, stride, dil, pads, relu, depthwise):
     m = espdl()
     act = m.capi.RELU if relu else m.capi.LINEAR
