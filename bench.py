@@ -113,6 +113,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of HIP-graph replay")
     ap.add_argument("--profile-repeats", type=int, default=5)
+    ap.add_argument("--layers", action="store_true", help="print the per-module timing table to stderr")
     ap.add_argument("--copy-mib", type=int, default=0,
                     help="also run one plain device copy of this many MiB (a kernel of known traffic, the "
                          "yardstick for FETCH_SIZE / WRITE_SIZE counter runs)")
@@ -168,6 +169,10 @@ def main():
     fam = {}
     for info in mdl.profile(repeats=args.profile_repeats):
         f = kernel_family(info, nodes)
+        if args.layers:
+            print("%-28s %-8s %-16s %9.2f us %8.1f GB/s %8.2f TOP/s" % (
+                info["name"], info["type"], f, info["latency_us"], info["bytes"] / max(info["latency_us"], 1e-3) * 1e-3,
+                2.0 * info["macs"] / max(info["latency_us"], 1e-3) * 1e-6), file=sys.stderr)
         d = fam.setdefault(f, {"us": 0.0, "macs": 0, "bytes": 0, "launches": 0})
         d["us"] += info["latency_us"]
         d["macs"] += info["macs"]
