@@ -26,6 +26,20 @@ class ConvDesc(ctypes.Structure):
         "pad_top", "pad_bottom", "pad_left", "pad_right", "group", "activation", "round_mode", "n_shift")]
 
 
+class MbconvDesc(ctypes.Structure):
+    """espdl_hip_mbconv_desc"""
+    _fields_ = [(n, ctypes.c_int32) for n in (
+        "batch", "in_h", "in_w", "in_c", "exp_c", "out_c", "has_expand", "k_h", "k_w", "stride_h", "stride_w",
+        "dil_h", "dil_w", "pad_top", "pad_bottom", "pad_left", "pad_right", "act_expand", "act_dw", "act_project",
+        "round_mode", "n_shift_expand", "n_shift_dw", "n_shift_project")]
+
+
+class MbconvWeights(ctypes.Structure):
+    """espdl_hip_mbconv_weights"""
+    _fields_ = [(n, ctypes.c_void_p) for n in (
+        "w_expand", "b_expand", "s_expand", "w_dw", "b_dw", "s_dw", "w_project", "b_project", "s_project")]
+
+
 _lib = None
 
 
@@ -50,6 +64,12 @@ def lib():
         L.espdl_hip_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp]
         L.espdl_hip_requantize_s8.argtypes = [vp, i64, i32, i32, vp, vp]
         L.espdl_hip_requantize.argtypes = [vp, i32, i64, i32, i32, vp, i32, vp]
+        mp = ctypes.POINTER(MbconvDesc)
+        L.espdl_hip_mbconv_out_shape.argtypes = [mp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
+        L.espdl_hip_mbconv_s8_supported.argtypes = [mp]
+        L.espdl_hip_mbconv_s8.argtypes = [mp, vp, ctypes.POINTER(MbconvWeights), vp, vp, vp]
+        for name in ("mbconv_out_shape", "mbconv_s8_supported", "mbconv_s8"):
+            getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         for name in ("conv_out_shape", "conv2d", "lut_s8", "prelu_s8", "relu_s8", "clip_s8", "add_s8",
                      "global_avg_pool_s8", "requantize_s8", "requantize", "device_cu_count"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
@@ -103,6 +123,31 @@ def conv2d(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 
         out = torch.empty((n, oh, ow, out_c), dtype=x.dtype, device=x.device)
     _check(lib().espdl_hip_conv2d(ctypes.byref(desc), _p(x), _p(filt), _p(bias), _p(shift), _p(lut), _p(out),
                                   _stream(stream)))
+    return out
+
+
+def mbconv_s8(x, expand, dw, project, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), relus=(True, True, False),
+              residual=None, round_mode=ROUND_HALF_UP, out=None, stream=None):
+    """Fused inverted-residual block.  expand / dw / project are (filter, bias, shift) triples of CUDA
+    tensors (expand may be None); filters as for conv2d: [E][C], [kH][kW][E], [OC][E]."""
+    import torch
+    n, h, w, c = x.shape
+    wd, bd, sd = dw
+    wp, bp, sp = project
+    exp_c = wd.numel() // (k[0] * k[1])
+    out_c = wp.numel() // exp_c
+    we, be, se = expand if expand is not None else (None, None, None)
+    desc = MbconvDesc(n, h, w, c, exp_c, out_c, 0 if expand is None else 1, k[0], k[1], stride[0], stride[1],
+                      dilation[0], dilation[1], pads[0], pads[1], pads[2], pads[3],
+                      RELU if relus[0] else LINEAR, RELU if relus[1] else LINEAR, RELU if relus[2] else LINEAR,
+                      round_mode, 1 if se is None else se.numel(), sd.numel(), sp.numel())
+    oh, ow = ctypes.c_int32(), ctypes.c_int32()
+    _check(lib().espdl_hip_mbconv_out_shape(ctypes.byref(desc), ctypes.byref(oh), ctypes.byref(ow)))
+    if out is None:
+        out = torch.empty((n, oh.value, ow.value, out_c), dtype=torch.int8, device=x.device)
+    wts = MbconvWeights(_p(we), _p(be), _p(se), _p(wd), _p(bd), _p(sd), _p(wp), _p(bp), _p(sp))
+    _check(lib().espdl_hip_mbconv_s8(ctypes.byref(desc), _p(x), ctypes.byref(wts), _p(residual), _p(out),
+                                     _stream(stream)))
     return out
 
 

@@ -326,3 +326,119 @@ int espdl_hip_requantize(const void *in, int32_t in_dtype, int64_t size, int32_t
 }
 
 } // extern "C"
+
+namespace {
+
+// Fills the geometry part of MbconvParams; pointers are set by the caller.
+int mbconv_geometry(const espdl_hip_mbconv_desc *d, espdl::MbconvParams *p)
+{
+    if (d == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "null descriptor");
+    if (d->batch < 0 || d->in_h <= 0 || d->in_w <= 0 || d->in_c <= 0 || d->exp_c <= 0 || d->out_c <= 0 || d->k_h <= 0 ||
+        d->k_w <= 0 || d->stride_h <= 0 || d->stride_w <= 0 || d->dil_h <= 0 || d->dil_w <= 0 || d->pad_top < 0 ||
+        d->pad_bottom < 0 || d->pad_left < 0 || d->pad_right < 0)
+        return fail(ESPDL_HIP_EINVAL, "bad mbconv geometry");
+    if (!d->has_expand && d->exp_c != d->in_c)
+        return fail(ESPDL_HIP_EINVAL, "without an expand stage exp_c must equal in_c");
+    const int eff_h = (d->k_h - 1) * d->dil_h + 1, eff_w = (d->k_w - 1) * d->dil_w + 1;
+    const int span_h = d->in_h + d->pad_top + d->pad_bottom - eff_h, span_w = d->in_w + d->pad_left + d->pad_right - eff_w;
+    if (span_h < 0 || span_w < 0)
+        return fail(ESPDL_HIP_EINVAL, "depthwise filter larger than the padded input");
+    if ((d->has_expand && d->n_shift_expand != 1 && d->n_shift_expand != d->exp_c) ||
+        (d->n_shift_dw != 1 && d->n_shift_dw != d->exp_c) || (d->n_shift_project != 1 && d->n_shift_project != d->out_c))
+        return fail(ESPDL_HIP_EINVAL, "n_shift_* must be 1 or the channel count of the stage");
+    p->batch = d->batch;
+    p->in_h = d->in_h;
+    p->in_w = d->in_w;
+    p->in_c = d->in_c;
+    p->exp_c = d->exp_c;
+    p->out_c = d->out_c;
+    p->out_h = span_h / d->stride_h + 1;
+    p->out_w = span_w / d->stride_w + 1;
+    p->k_h = d->k_h;
+    p->k_w = d->k_w;
+    p->stride_h = d->stride_h;
+    p->stride_w = d->stride_w;
+    p->dil_h = d->dil_h;
+    p->dil_w = d->dil_w;
+    p->pad_top = d->pad_top;
+    p->pad_left = d->pad_left;
+    p->relu_expand = d->act_expand == ESPDL_HIP_RELU;
+    p->relu_dw = d->act_dw == ESPDL_HIP_RELU;
+    p->relu_project = d->act_project == ESPDL_HIP_RELU;
+    p->half_even = d->round_mode == ESPDL_HIP_ROUND_HALF_EVEN;
+    p->n_s_expand = d->n_shift_expand;
+    p->n_s_dw = d->n_shift_dw;
+    p->n_s_project = d->n_shift_project;
+    if ((long long)p->batch * p->out_h * p->out_w > 0x7fffffffll - 65536)
+        return fail(ESPDL_HIP_EINVAL, "too many output pixels");
+    return ESPDL_HIP_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int espdl_hip_mbconv_out_shape(const espdl_hip_mbconv_desc *desc, int32_t *out_h, int32_t *out_w)
+{
+    espdl::MbconvParams p = {};
+    const int rc = mbconv_geometry(desc, &p);
+    if (rc != ESPDL_HIP_OK)
+        return rc;
+    if (out_h)
+        *out_h = p.out_h;
+    if (out_w)
+        *out_w = p.out_w;
+    return ESPDL_HIP_OK;
+}
+
+int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
+{
+    espdl::MbconvParams p = {};
+    if (mbconv_geometry(desc, &p) != ESPDL_HIP_OK)
+        return 0;
+    // any 16-byte aligned non-null value stands for the pointers the plan looks at
+    static const int8_t *const aligned = reinterpret_cast<const int8_t *>(uintptr_t(256));
+    p.in = aligned;
+    p.out = const_cast<int8_t *>(aligned);
+    p.w_expand = desc->has_expand ? aligned : nullptr;
+    p.w_dw = aligned;
+    p.w_project = aligned;
+    return espdl::mbconv_s8_fused_supports(p) ? 1 : 0;
+}
+
+int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *w,
+                        const int8_t *residual, int8_t *out, void *stream)
+{
+    espdl::MbconvParams p = {};
+    const int rc = mbconv_geometry(desc, &p);
+    if (rc != ESPDL_HIP_OK)
+        return rc;
+    if (p.batch == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr || w == nullptr || w->w_dw == nullptr || w->s_dw == nullptr ||
+        w->w_project == nullptr || w->s_project == nullptr || (desc->has_expand && (w->w_expand == nullptr || w->s_expand == nullptr)))
+        return fail(ESPDL_HIP_EINVAL, "in, out, filters and shifts must not be NULL");
+    if (misaligned(in, 4) || misaligned(out, 4) || misaligned(residual, 4) || misaligned(w->w_project, 16) ||
+        misaligned(w->w_expand, 4) || misaligned(w->b_expand, 4) || misaligned(w->s_expand, 4) || misaligned(w->b_dw, 4) ||
+        misaligned(w->s_dw, 4) || misaligned(w->b_project, 4) || misaligned(w->s_project, 4))
+        return fail(ESPDL_HIP_EINVAL, "activations, expand filter, biases and shifts must be 4-byte aligned, the project filter 16-byte aligned");
+    p.in = in;
+    p.residual = residual;
+    p.out = out;
+    p.w_expand = desc->has_expand ? w->w_expand : nullptr;
+    p.b_expand = w->b_expand;
+    p.s_expand = w->s_expand;
+    p.w_dw = w->w_dw;
+    p.b_dw = w->b_dw;
+    p.s_dw = w->s_dw;
+    p.w_project = w->w_project;
+    p.b_project = w->b_project;
+    p.s_project = w->s_project;
+    if (!espdl::mbconv_s8_fused_supports(p))
+        return fail(ESPDL_HIP_ENOTSUP, "this block shape is not covered by the fused kernel");
+    return device_status(espdl::launch_mbconv_s8_fused(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                         "mbconv_s8_fused");
+}
+
+} // extern "C"

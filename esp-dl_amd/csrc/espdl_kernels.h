@@ -35,6 +35,28 @@ hipError_t launch_depthwise_s8_lds(const ConvGeom &g, const int8_t *in, const in
                                    const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
                                    hipStream_t stream);
 
+// Inverted-residual block as one kernel: [1x1 expand conv] -> depthwise conv -> 1x1 project conv
+// [-> saturating Add of `residual`].  w_expand == nullptr means there is no expand stage
+// (exp_c == in_c).  Filters are in the layouts of the separate kernels; every shift array has 1 or
+// <channels> entries.
+struct MbconvParams {
+    const int8_t *in;
+    const int8_t *residual; // same shape as out, or nullptr
+    int8_t *out;
+    const int8_t *w_expand; // [exp_c][in_c]
+    const int32_t *b_expand, *s_expand;
+    const int8_t *w_dw; // [k_h][k_w][exp_c]
+    const int32_t *b_dw, *s_dw;
+    const int8_t *w_project; // [out_c][exp_c]
+    const int32_t *b_project, *s_project;
+    int n_s_expand, n_s_dw, n_s_project;
+    int batch, in_h, in_w, in_c, exp_c, out_c, out_h, out_w;
+    int k_h, k_w, stride_h, stride_w, dil_h, dil_w, pad_top, pad_left;
+    int relu_expand, relu_dw, relu_project, half_even;
+};
+bool mbconv_s8_fused_supports(const MbconvParams &p);
+hipError_t launch_mbconv_s8_fused(const MbconvParams &p, int cu_count, hipStream_t stream);
+
 hipError_t launch_conv2d_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
                              const int32_t *shift, int16_t *out, hipStream_t stream);
 hipError_t launch_depthwise_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,

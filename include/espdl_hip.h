@@ -131,6 +131,46 @@ int espdl_hip_requantize_s8(const int8_t *in, int64_t size, int32_t in_exp, int3
 int espdl_hip_requantize(const void *in, int32_t in_dtype, int64_t size, int32_t in_exp, int32_t out_exp, void *out,
                          int32_t out_dtype, void *stream);
 
+/*
+ * Inverted-residual block in one launch: [1x1 Conv] -> depthwise Conv -> 1x1 Conv [-> Add].
+ * No single reference function does this; it runs the same sequence of module::Conv::forward
+ * (esp-dl/dl/module/include/dl_module_conv.hpp:121-162) and module::Add::forward
+ * (esp-dl/dl/base/dl_base_add.cpp:34-44) calls as the separate entry points above, with the int8 result
+ * of every stage formed exactly as espdl_hip_conv2d forms it, but keeps the expanded activation in
+ * on-chip memory.  Results are bit-identical to the separate calls.
+ *   has_expand = 0: the block starts at the depthwise stage and exp_c must equal in_c.
+ *   Filters use the layouts of espdl_hip_conv2d: expand [exp_c][in_c], depthwise [k_h][k_w][exp_c],
+ *   project [out_c][exp_c]; biases int32 or NULL; shifts int32[1 or channels] per stage.
+ *   residual: int8 tensor of the output's shape added with saturation after the project stage, or NULL.
+ * Needs exp_c % 16 == 0, in_c % 4 == 0, out_c % 4 == 0, at most 12 depthwise taps, in_c <= 256,
+ * out_c <= 384; espdl_hip_mbconv_s8_supported() answers for a descriptor (1 = yes), and
+ * espdl_hip_mbconv_s8 returns ESPDL_HIP_ENOTSUP where it does not apply.
+ */
+typedef struct espdl_hip_mbconv_desc {
+    int32_t batch, in_h, in_w, in_c;
+    int32_t exp_c, out_c;
+    int32_t has_expand;
+    int32_t k_h, k_w, stride_h, stride_w, dil_h, dil_w;               /* depthwise stage */
+    int32_t pad_top, pad_bottom, pad_left, pad_right;                 /* depthwise stage */
+    int32_t act_expand, act_dw, act_project;                          /* ESPDL_HIP_LINEAR / ESPDL_HIP_RELU */
+    int32_t round_mode;
+    int32_t n_shift_expand, n_shift_dw, n_shift_project;              /* 1 or channels of the stage */
+} espdl_hip_mbconv_desc;
+
+typedef struct espdl_hip_mbconv_weights {
+    const int8_t *w_expand;
+    const int32_t *b_expand, *s_expand;
+    const int8_t *w_dw;
+    const int32_t *b_dw, *s_dw;
+    const int8_t *w_project;
+    const int32_t *b_project, *s_project;
+} espdl_hip_mbconv_weights;
+
+int espdl_hip_mbconv_out_shape(const espdl_hip_mbconv_desc *desc, int32_t *out_h, int32_t *out_w);
+int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc);
+int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *weights,
+                        const int8_t *residual, int8_t *out, void *stream);
+
 /* Library / device information. */
 const char *espdl_hip_last_error(void);
 const char *espdl_hip_version(void);

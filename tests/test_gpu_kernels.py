@@ -342,3 +342,57 @@ def test_bad_arguments_are_rejected():
         m.conv2d(x, f, None, torch.zeros(3, dtype=torch.int32, device="cuda"), (1, 1))  # n_shift neither 1 nor out_c
     empty = torch.zeros((0, 2, 2, 4), dtype=torch.int8, device="cuda")
     assert m.conv2d(empty, torch.zeros((4, 1, 1, 4), dtype=torch.int8, device="cuda"), None, s, (1, 1)).shape[0] == 0
+
+
+# --------------------------------------------------------------------------- fused inverted-residual block
+# (name, (N, H, W, Cin), Ce (None = no expand stage), Cout, k, stride, pads, residual, half_even, per_tensor)
+MBCONV_CASES = [
+    ("b8_14x14_64_384_64_res", (3, 14, 14, 64), 384, 64, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
+    ("b3_56x56_24_144_24_res", (2, 56, 56, 24), 144, 24, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
+    ("b2_40x40_16_96_24_s2", (2, 40, 40, 16), 96, 24, (3, 3), (2, 2), (1, 1, 1, 1), False, False, False),
+    ("b1_30x30_32_noexp_16", (2, 30, 30, 32), None, 16, (3, 3), (1, 1), (1, 1, 1, 1), False, False, False),
+    ("b17_7x7_160_960_320", (5, 7, 7, 160), 960, 320, (3, 3), (1, 1), (1, 1, 1, 1), False, False, False),
+    ("b14_14x14_96_576_160_s2", (3, 14, 14, 96), 576, 160, (3, 3), (2, 2), (1, 1, 1, 1), False, False, False),
+    ("ragged_19x23_32_80_48_res", (2, 19, 23, 32), 80, 48, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
+    ("tailpad_17x17_32_96_32_s2", (2, 17, 17, 32), 96, 32, (3, 3), (2, 2), (0, 1, 0, 1), False, False, False),
+    ("halfeven_14x14_32_192_32_res", (2, 14, 14, 32), 192, 32, (3, 3), (1, 1), (1, 1, 1, 1), True, True, False),
+    ("pertensor_28x28_32_192_64", (2, 28, 28, 32), 192, 64, (3, 3), (1, 1), (1, 1, 1, 1), False, False, True),
+]
+
+
+@pytest.mark.parametrize("case", MBCONV_CASES, ids=lambda c: c[0])
+def test_mbconv_s8_fused(oracle, case):
+    announce(f"mbconv_s8 {case[0]}")
+    name, (n, h, w, cin), ce, cout, k, stride, pads, with_res, half_even, per_tensor = case
+    m = espdl()
+    rng = np.random.default_rng(0xB10C + len(name))
+    rm_o = oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP
+    rm_g = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
+
+    def stage(oc, kk, fshape):
+        f = rng_int8(rng, fshape)
+        b = rng.integers(-4096, 4097, size=oc).astype(np.int32)
+        base = typical_shift(kk)
+        s = np.full(1, base, np.int32) if per_tensor else (base + rng.integers(-2, 3, size=oc)).astype(np.int32)
+        return f, b, s
+
+    x = rng_int8(rng, (n, h, w, cin))
+    cur = x
+    expand = None
+    e = cin
+    if ce is not None:
+        e = ce
+        expand = stage(e, cin, (e, 1, 1, cin))
+        cur = oracle.conv2d_s8(cur, expand[0], expand[1], expand[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.RELU, rm_o)
+    dw = stage(e, k[0] * k[1], (k[0], k[1], e))
+    cur = oracle.depthwise_s8(cur, dw[0], dw[1], dw[2], k, stride, (1, 1), pads, oracle.RELU, rm_o)
+    proj = stage(cout, e, (cout, 1, 1, e))
+    cur = oracle.conv2d_s8(cur, proj[0], proj[1], proj[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.LINEAR, rm_o)
+    res = None
+    if with_res:
+        res = rng_int8(rng, cur.shape)
+        cur = oracle.add_s8(cur, res)
+    dev = lambda t: None if t is None else tuple(to_dev(a) for a in t)  # noqa: E731
+    got = m.mbconv_s8(to_dev(x), dev(expand), dev(dw), dev(proj), k, stride, (1, 1), pads, (True, True, False),
+                      residual=to_dev(res), round_mode=rm_g)
+    np.testing.assert_array_equal(to_host(got), cur)
