@@ -41,7 +41,6 @@ constexpr int kWaves = kThreads / 64;
 constexpr int kKsDw = 3;    // depthwise k steps of 4 taps
 constexpr int kMaxKse = 4;  // expand k steps of 64 input channels (in_c <= 256)
 constexpr int kMaxAcc = 10; // project accumulator tiles per wavefront
-constexpr int kMaxCtIn = 3; // expand column tiles (16 patch pixels) per wavefront
 constexpr int kMaxWe = 2;   // 16-byte expand-filter units per thread and chunk
 constexpr int kMaxWp = 3;   // 16-byte project-filter units per thread and chunk
 constexpr int kEs = 80;     // pixel stride of E and D in LDS: 64 channels + 16 (odd number of 16-byte units)
@@ -65,7 +64,7 @@ struct MbArgs {
     FastDiv fd_tiles_x, fd_tiles_yx, fd_pw, fd_tw, fd_nct_out, fd_in_vecs, fd_out_vecs;
     int in_vecs, out_vecs; // pieces per pixel
     // LDS layout (byte offsets)
-    int off_x, off_e, off_d, off_out, off_we, off_wp, off_wd, off_ce, off_cd, off_cp, off_pixtab;
+    int off_x, off_e, off_d, off_out, off_we, off_wp, off_wd, off_ce, off_cd, off_cp, off_pixtab, off_rctab, off_slottab;
 };
 
 struct TilePos {
@@ -212,12 +211,30 @@ __device__ __forceinline__ void mb_store_weights(const MbArgs &a, int chunk, int
     }
 }
 
+// Requantize four accumulators with the stage constants held in registers.
+__device__ __forceinline__ int mb_pack_r(const v4i &acc, const v4i &ss, const v4i &ls, bool fast, bool relu,
+                                         bool half_even, int floor_pk)
+{
+    if (fast)
+        return pack_fast4<true>(acc, ls, ss, floor_pk);
+    int q[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+        q[r] = requant_s8(acc[r], ss[r], relu, half_even);
+    return pack4_s8(q[0], q[1], q[2], q[3]);
+}
+
+constexpr int kMaxCtE = 12; // expand column tiles per wavefront (two wavefronts share a row tile)
+constexpr int kMaxCtD = 8;  // depthwise column tiles per wavefront (two wavefronts share a channel group)
+constexpr int kAccBatch = 5;
+
 __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const MbconvParams &p = a.p;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 15, quad = lane >> 4;
+    const int sub = wave & 3, half = wave >> 2; // row tile / channel group of this wavefront, and which half of the columns
     const bool half_even = p.half_even != 0;
     const int ec_pad = a.n_chunks * 64; // expanded channels padded to whole chunks
     const int oc_pad = a.nrt * 16;
@@ -242,7 +259,7 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
                                        (long long)p.exp_c * 16384, half_even, tid);
     for (int i = tid; i < a.taps * p.exp_c; i += kThreads)
         smem[a.off_wd + i] = (unsigned char)p.w_dw[i];
-    // stage the depthwise reads from: E (stride kEs) or, without expand, the input patch (stride xs)
+    // the depthwise stage reads from E (stride kEs) or, without expand, from the input patch (stride xs)
     const int dw_stride = a.has_expand ? kEs : a.xs;
     for (int q = tid; q < a.nct_out * 16; q += kThreads) {
         int off = 0;
@@ -252,6 +269,23 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
             off = (int)((qy * p.stride_h * a.pw + qx * p.stride_w) * dw_stride);
         }
         pixtab[q] = off;
+    }
+    // project accumulator tile t -> (row tile | column tile << 8); read back inside the loops so that
+    // the per-tile addresses are formed where they are used instead of living in registers throughout
+    int *slottab = reinterpret_cast<int *>(smem + a.off_slottab);
+    for (int t = tid; t < kMaxAcc * kWaves; t += kThreads) {
+        const int rt = (int)fastdiv((unsigned)t, a.fd_nct_out);
+        slottab[t] = t < a.n_acc ? (rt | ((t - rt * a.nct_out) << 8)) : 0;
+    }
+    // (row | col << 16) of every patch pixel, -1 past the patch
+    int *rctab = reinterpret_cast<int *>(smem + a.off_rctab);
+    for (int q = tid; q < a.nct_in * 16; q += kThreads) {
+        int rc = -1;
+        if (q < a.p_in) {
+            const unsigned py = fastdiv((unsigned)q, a.fd_pw);
+            rc = (int)(py | (((unsigned)q - py * a.fd_pw.d) << 16));
+        }
+        rctab[q] = rc;
     }
     int tapoff[kKsDw];
 #pragma unroll
@@ -266,18 +300,9 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
     const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
     const int floor_d = p.relu_dw ? 0 : (int)0x80008000u;
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
-    // patch pixel (row, col) of this lane's column in each of its expand column tiles
-    int ct_rc[kMaxCtIn];
-#pragma unroll
-    for (int s = 0; s < kMaxCtIn; s++) {
-        const int pix = (wave + s * kWaves) * 16 + col;
-        ct_rc[s] = -1;
-        if (pix < a.p_in) {
-            const unsigned py = fastdiv((unsigned)pix, a.fd_pw);
-            ct_rc[s] = (int)(py | (((unsigned)pix - py * a.fd_pw.d) << 16));
-        }
-    }
     __syncthreads();
+    // patch pixel (row | col << 16) of this lane in each of the wavefront's expand column tiles
+    // is recomputed per tile into a bit mask of the pixels that lie inside the image
 
     const TileSeq seq = xcd_tile_sequence(a.n_units);
     for (int unit = seq.first; unit < seq.end; unit += seq.step) {
@@ -307,14 +332,13 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
                     *reinterpret_cast<int *>(dst) = ok ? *reinterpret_cast<const int *>(src) : 0;
             }
         }
-
         // ---- project accumulators start at bias (+ rounding constant)
         v4i acc[kMaxAcc];
 #pragma unroll
         for (int s = 0; s < kMaxAcc; s++) {
             const int t = wave + s * kWaves;
             if (t < a.n_acc) {
-                const int rt = (int)fastdiv((unsigned)t, a.fd_nct_out);
+                const int rt = slottab[t] & 0xff;
                 acc[s] = *reinterpret_cast<const v4i *>(cst_p + 16 * rt + 4 * quad);
             }
         }
@@ -330,86 +354,129 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
             if (chunk + 1 < a.n_chunks)
                 mb_fetch_weights(a, chunk + 1, tid, we_r, wp_r); // in flight during this chunk's stages
 
-            // ---- 2a. expand: E[patch pixel][4*ng*q + 4*t + r]
+            // ---- 2a. expand: this wavefront owns row tile `sub` (channels e0 + 4*ng*q + 4*sub + r of
+            // lane quad q) and every second column tile; E[patch pixel][4*ng*q + 4*sub + r]
             if (a.has_expand) {
+                if (sub < ng) {
+                    const int c = e0 + 4 * ng * quad + 4 * sub;
+                    const v4i init = *reinterpret_cast<const v4i *>(cst_e + c);
+                    const v4i ss = *reinterpret_cast<const v4i *>(cst_e + ec_pad + c);
+                    const v4i ls = *reinterpret_cast<const v4i *>(cst_e + 2 * ec_pad + c);
+                    v4i aop[kMaxKse];
 #pragma unroll
-                for (int s = 0; s < kMaxCtIn; s++) {
-                    const int ct = wave + s * kWaves;
-                    if (ct < a.nct_in) { // uniform per wavefront
-                        v4i b[kMaxKse];
+                    for (int ks = 0; ks < kMaxKse; ks++)
+                        if (ks < a.kse)
+                            aop[ks] = *reinterpret_cast<const v4i *>(smem + a.off_we + 16 * ((ks * ng + sub) * 64 + lane));
+                    const unsigned char *bsrc = x_l + col * a.xs + 16 * quad;
+                    unsigned char *dst = e_l + col * kEs + 4 * ng * quad + 4 * sub;
+                    v4i b[kMaxKse];
 #pragma unroll
-                        for (int ks = 0; ks < kMaxKse; ks++)
-                            if (ks < a.kse)
-                                b[ks] = *reinterpret_cast<const v4i *>(x_l + (ct * 16 + col) * a.xs + 64 * ks + 16 * quad);
-                        bool inside = false;
-                        if (ct_rc[s] >= 0) {
-                            const int iy = iy0 + (ct_rc[s] & 0xffff), ix = ix0 + (ct_rc[s] >> 16);
-                            inside = (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
-                        }
-                        unsigned char *dst = e_l + (ct * 16 + col) * kEs + 4 * ng * quad;
-                        for (int t = 0; t < ng; t++) {
-                            const int c = e0 + 4 * ng * quad + 4 * t;
-                            v4i r = *reinterpret_cast<const v4i *>(cst_e + c);
+                    for (int ks = 0; ks < kMaxKse; ks++)
+                        if (ks < a.kse)
+                            b[ks] = *reinterpret_cast<const v4i *>(bsrc + half * 16 * a.xs + 64 * ks);
+#pragma unroll 1
+                    for (int s = 0; s < kMaxCtE; s++) {
+                        const int ct = half + 2 * s;
+                        if (ct >= a.nct_in) // uniform per wavefront
+                            break;
+                        {
+                            v4i r = init;
 #pragma unroll
                             for (int ks = 0; ks < kMaxKse; ks++)
-                                if (ks < a.kse) {
-                                    const v4i aop = *reinterpret_cast<const v4i *>(smem + a.off_we + 16 * ((ks * ng + t) * 64 + lane));
-                                    r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[ks], r, 0, 0, 0);
-                                }
-                            const int word = mb_pack(r, cst_e, ec_pad, c, fast_e, p.relu_expand != 0, half_even, floor_e);
-                            *reinterpret_cast<int *>(dst + 4 * t) = inside ? word : 0;
+                                if (ks < a.kse)
+                                    r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], r, 0, 0, 0);
+                            if (ct + 2 < a.nct_in) {
+#pragma unroll
+                                for (int ks = 0; ks < kMaxKse; ks++)
+                                    if (ks < a.kse)
+                                        b[ks] = *reinterpret_cast<const v4i *>(bsrc + (ct + 2) * 16 * a.xs + 64 * ks);
+                            }
+                            const int word = mb_pack_r(r, ss, ls, fast_e, p.relu_expand != 0, half_even, floor_e);
+                            // outside the image the expanded activation is the depthwise zero padding
+                            const int rc = rctab[ct * 16 + col];
+                            const int iy = iy0 + (rc & 0xffff), ix = ix0 + (rc >> 16);
+                            const bool inside = rc >= 0 && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
+                            *reinterpret_cast<int *>(dst + ct * 16 * kEs) = inside ? word : 0;
                         }
                     }
                 }
                 __syncthreads();
             }
 
-            // ---- 2b. depthwise: D[tile pixel][16*g + 4*q + r]
+            // ---- 2b. depthwise: this wavefront owns channel group `sub` and every second column tile;
+            // D[tile pixel][16*sub + 4*q + r]
             {
-                const unsigned char *src_l = a.has_expand ? e_l : x_l + e0;
-                const int n_t = ng * a.nct_out;
-                const int sel = col >> 2;
-                int grp_loaded = -1;
-                v4i aop[kKsDw];
-                for (int t = wave; t < n_t; t += kWaves) {
-                    const int g = (int)fastdiv((unsigned)t, a.fd_nct_out);
-                    const int ct = t - g * a.nct_out;
-                    if (g != grp_loaded) {
+                if (sub < ng) {
+                    const unsigned char *src_l = (a.has_expand ? e_l : x_l + e0) + 16 * sub;
+                    const int sel = col >> 2;
+                    v4i aop[kKsDw];
 #pragma unroll
-                        for (int ks = 0; ks < kKsDw; ks++) {
-                            const int tap = 4 * ks + quad;
-                            int d = 0;
-                            if (tap < a.taps)
-                                d = (int)smem[a.off_wd + tap * p.exp_c + e0 + 16 * g + col] << (8 * (col & 3));
-                            aop[ks] = v4i{sel == 0 ? d : 0, sel == 1 ? d : 0, sel == 2 ? d : 0, sel == 3 ? d : 0};
-                        }
-                        grp_loaded = g;
+                    for (int ks = 0; ks < kKsDw; ks++) {
+                        const int tap = 4 * ks + quad;
+                        int d = 0;
+                        if (tap < a.taps)
+                            d = (int)smem[a.off_wd + tap * p.exp_c + e0 + 16 * sub + col] << (8 * (col & 3));
+                        aop[ks] = v4i{sel == 0 ? d : 0, sel == 1 ? d : 0, sel == 2 ? d : 0, sel == 3 ? d : 0};
                     }
-                    const int c = e0 + 16 * g + 4 * quad;
-                    v4i r = *reinterpret_cast<const v4i *>(cst_d + c);
-                    const int po = pixtab[ct * 16 + col] + 16 * g;
+                    const int c = e0 + 16 * sub + 4 * quad;
+                    const v4i init = *reinterpret_cast<const v4i *>(cst_d + c);
+                    const v4i ss = *reinterpret_cast<const v4i *>(cst_d + ec_pad + c);
+                    const v4i ls = *reinterpret_cast<const v4i *>(cst_d + 2 * ec_pad + c);
+                    unsigned char *dst = d_l + col * kEs + 16 * sub + 4 * quad;
+                    v4i b[kKsDw];
+                    {
+                        const int po = pixtab[min(half, a.nct_out - 1) * 16 + col];
 #pragma unroll
-                    for (int ks = 0; ks < kKsDw; ks++)
-                        if (4 * ks < a.taps) {
-                            const v4i b = *reinterpret_cast<const v4i *>(src_l + po + tapoff[ks]);
-                            r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b, r, 0, 0, 0);
+                        for (int ks = 0; ks < kKsDw; ks++)
+                            b[ks] = *reinterpret_cast<const v4i *>(src_l + po + tapoff[ks]);
+                    }
+                    // patch offset of the lane's pixel in the column tile after this one (two ahead of the reads)
+                    int po_next = pixtab[min(half + 2, a.nct_out - 1) * 16 + col];
+#pragma unroll 1
+                    for (int s = 0; s < kMaxCtD; s++) {
+                        const int ct = half + 2 * s;
+                        if (ct >= a.nct_out) // uniform per wavefront
+                            break;
+                        {
+                            v4i r = init;
+#pragma unroll
+                            for (int ks = 0; ks < kKsDw; ks++)
+                                if (4 * ks < a.taps)
+                                    r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], r, 0, 0, 0);
+                            if (ct + 2 < a.nct_out) {
+#pragma unroll
+                                for (int ks = 0; ks < kKsDw; ks++)
+                                    b[ks] = *reinterpret_cast<const v4i *>(src_l + po_next + tapoff[ks]);
+                                po_next = pixtab[min(ct + 4, a.nct_out - 1) * 16 + col];
+                            }
+                            const int word = mb_pack_r(r, ss, ls, fast_d, p.relu_dw != 0, half_even, floor_d);
+                            *reinterpret_cast<int *>(dst + ct * 16 * kEs) = word;
                         }
-                    const int word = mb_pack(r, cst_d, ec_pad, c, fast_d, p.relu_dw != 0, half_even, floor_d);
-                    *reinterpret_cast<int *>(d_l + (ct * 16 + col) * kEs + 16 * g + 4 * quad) = word;
+                    }
                 }
                 __syncthreads();
             }
 
-            // ---- 2c. project: acc[rt][ct] += Wp[rt][chunk] x D[ct]
+            // ---- 2c. project: acc[rt][ct] += Wp[rt][chunk] x D[ct]; operands of a batch of tiles are
+            // all requested before the first MFMA of the batch
 #pragma unroll
-            for (int s = 0; s < kMaxAcc; s++) {
-                const int t = wave + s * kWaves;
-                if (t < a.n_acc) {
-                    const int rt = (int)fastdiv((unsigned)t, a.fd_nct_out);
-                    const int ct = t - rt * a.nct_out;
-                    const v4i aop = *reinterpret_cast<const v4i *>(smem + a.off_wp + 16 * (rt * 64 + lane));
-                    const v4i b = *reinterpret_cast<const v4i *>(d_l + (ct * 16 + col) * kEs + 16 * quad);
-                    acc[s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b, acc[s], 0, 0, 0);
+            for (int s0 = 0; s0 < kMaxAcc; s0 += kAccBatch) {
+                if (wave + s0 * kWaves < a.n_acc) { // uniform per wavefront
+                    v4i aop[kAccBatch], b[kAccBatch];
+#pragma unroll
+                    for (int j = 0; j < kAccBatch; j++) {
+                        const int t = wave + (s0 + j) * kWaves;
+                        if (t < a.n_acc) {
+                            const int e = slottab[t];
+                            const int rt = e & 0xff, ct = e >> 8;
+                            aop[j] = *reinterpret_cast<const v4i *>(smem + a.off_wp + 16 * (rt * 64 + lane));
+                            b[j] = *reinterpret_cast<const v4i *>(d_l + (ct * 16 + col) * kEs + 16 * quad);
+                        }
+                    }
+#pragma unroll
+                    for (int j = 0; j < kAccBatch; j++)
+                        if (wave + (s0 + j) * kWaves < a.n_acc)
+                            acc[s0 + j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[j], b[j], acc[s0 + j], 0, 0, 0);
                 }
             }
         }
@@ -420,8 +487,8 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
         for (int s = 0; s < kMaxAcc; s++) {
             const int t = wave + s * kWaves;
             if (t < a.n_acc) {
-                const int rt = (int)fastdiv((unsigned)t, a.fd_nct_out);
-                const int ct = t - rt * a.nct_out;
+                const int e = slottab[t];
+                const int rt = e & 0xff, ct = e >> 8;
                 const int c = 16 * rt + 4 * quad;
                 const int word = mb_pack(acc[s], cst_p, oc_pad, c, fast_p, p.relu_project != 0, half_even, floor_p);
                 *reinterpret_cast<int *>(out_l + (ct * 16 + col) * a.os + c) = word;
@@ -458,8 +525,7 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
                 }
             }
         }
-        // the barrier at the top of the next tile's chunk 0 orders these LDS reads before the next
-        // patch copy only if the patch copy comes after it: so wait here
+        // the output tile aliases the patch area: its reads finish before the next patch copy
         __syncthreads();
     }
 }
@@ -549,7 +615,7 @@ MbPlan mb_plan(const MbconvParams &p)
             a.nrt = (p.out_c + 15) / 16;
             a.n_acc = a.nrt * a.nct_out;
             a.os = odd16(a.nrt * 16);
-            if (a.nct_in > kMaxCtIn * kWaves || a.n_acc > kMaxAcc * kWaves)
+            if (a.nct_in > 2 * kMaxCtE || a.nct_out > 2 * kMaxCtD || a.n_acc > kMaxAcc * kWaves)
                 continue;
             if (a.kse * 4 * 64 > kMaxWe * kThreads || a.nrt * 64 > kMaxWp * kThreads)
                 continue;
@@ -580,6 +646,10 @@ MbPlan mb_plan(const MbconvParams &p)
             off += (size_t)3 * a.nrt * 16 * 4;
             a.off_pixtab = (int)off;
             off += (size_t)a.nct_out * 16 * 4;
+            a.off_rctab = (int)off;
+            off += (size_t)a.nct_in * 16 * 4;
+            a.off_slottab = (int)off;
+            off += (size_t)kMaxAcc * kWaves * 4;
             if (off > lds_limit())
                 continue;
             const int per_cu = off <= 80 * 1024 ? 2 : 1;
