@@ -58,10 +58,20 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     // as fit; if even one group does not fit, K is chunked.
     const int fixed = 256;
     const int per_group_full = a.ksteps * 4096 + 768;
+    const int cus = cu_count > 0 ? cu_count : 256;
+    // With few pixel sets per CU a workgroup lives for a handful of sets and the launch is bound by
+    // the latency of staging its filters and of its first loads, not by bandwidth: then smaller filter
+    // chunks (more, shorter-lived workgroups per CU; the input is re-read per chunk, from L2) win.
+    const long long sets64 = (a.npix + 63) / 64;
+    const int budget = sets64 < (long long)cus * 16 ? 40 * 1024 : kLdsPerWorkgroup;
     if (per_group_full + fixed <= kLdsPerWorkgroup) {
         a.ks_per_chunk = a.ksteps;
         a.n_kchunks = 1;
-        a.groups_per_chunk = min(a.n_groups, max(1, (kLdsPerWorkgroup - fixed) / per_group_full));
+        int gpc = min(a.n_groups, max(1, (budget - fixed) / per_group_full));
+        // equal chunks: the slowest chunk sets the time
+        const int chunks = (a.n_groups + gpc - 1) / gpc;
+        gpc = (a.n_groups + chunks - 1) / chunks;
+        a.groups_per_chunk = gpc;
     } else {
         a.ks_per_chunk = (kLdsPerWorkgroup - fixed - 768) / 4096;
         a.n_kchunks = (a.ksteps + a.ks_per_chunk - 1) / a.ks_per_chunk;
@@ -72,7 +82,6 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
 
     // register plan: hold the whole reduction axis when it is short enough; two pixel tiles per wave
     // (half the LDS traffic per MFMA) when there are enough pixels and registers
-    const int cus = cu_count > 0 ? cu_count : 256;
     int ksc = a.n_kchunks == 1 ? pick_ksc(a.ksteps) : 0;
     if (bmode == B_GATHER)
         ksc = 0;
