@@ -64,6 +64,17 @@ struct DwLdsArgs {
     FastDiv fd_tiles_x, fd_tiles_yx, fd_pwgc, fd_gc, fd_tw, fd_np;
     // LDS layout, byte offsets
     int off_patch, off_out, off_a, off_init, off_ss, off_ls, off_pixtab, off_lut;
+    // optional 1x1 project convolution (+ residual Add) applied to the depthwise result of the tile
+    // while it is still in LDS; needs every channel in one workgroup (gc == in_c / 16)
+    DwProject pj;
+    int p_nrt;          // row tiles of 16 project filters
+    int p_ks;           // k steps of 64 depthwise channels
+    int p_os;           // LDS pixel stride of the project result, bytes
+    int p_vec;          // bytes per store piece of the project result: 16 or 4
+    int p_vecs;         // pieces per pixel
+    int n_pout_chunks;  // th * tw * p_vecs
+    FastDiv fd_pvecs;
+    int off_wp, off_cp, off_pout;
 };
 
 struct UnitPos {
@@ -184,6 +195,7 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
     }
 }
 
+template <bool PROJ>
 __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwLdsArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -218,7 +230,15 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
 #pragma unroll
     for (int i = 0; i < kMaxOut; i++) {
         const int k = tid + i * kThreads;
-        if (k < a.n_out_chunks) {
+        if (PROJ && k < a.n_pout_chunks) {
+            const unsigned q = fastdiv((unsigned)k, a.fd_pvecs);
+            const unsigned v = (unsigned)k - q * a.fd_pvecs.d;
+            const unsigned py = fastdiv(q, a.fd_tw);
+            const unsigned px = q - py * a.fd_tw.d;
+            out_rel[i] = (int)((py * g.out_w + px) * a.pj.out_c + v * a.p_vec);
+            out_lds[i] = (int)(q * a.p_os + v * a.p_vec);
+            out_rc[i] = (int)(py | (px << 16));
+        } else if (!PROJ && k < a.n_out_chunks) {
             const unsigned q = fastdiv((unsigned)k, a.fd_gc);
             const unsigned c16 = (unsigned)k - q * a.fd_gc.d;
             const unsigned py = fastdiv(q, a.fd_tw);
@@ -305,6 +325,46 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
     }
     const int floor_pk = g.relu ? 0 : (int)0x80008000u;
 
+    // project stage: filters in MFMA operand-A order (row i of row tile rt is filter 16*rt + i, the
+    // lane's 16 k positions are depthwise channels 64*ks + 16*gk ...; zeros past out_c and past C),
+    // and the stage's [start value | shift | left shift] table
+    bool fast_p = false;
+    int floor_p = 0;
+    if (PROJ) {
+        const DwProject &pj = a.pj;
+        for (int e = tid; e < a.p_nrt * a.p_ks * 64; e += kThreads) {
+            const int l = e & 63, ks = (e >> 6) % a.p_ks, rt = (e >> 6) / a.p_ks;
+            const int f = 16 * rt + (l & 15), k0 = 64 * ks + 16 * (l >> 4);
+            v4i w = {0, 0, 0, 0};
+            if (f < pj.out_c && k0 < C)
+                w = *reinterpret_cast<const v4i *>(pj.w + (long long)f * C + k0);
+            *reinterpret_cast<v4i *>(smem + a.off_wp + 16 * e) = w;
+        }
+        const int ocp = a.p_nrt * 16;
+        const long long bound = (long long)C * 16384;
+        int okp = half_even ? 0 : 1;
+        int ps = 0, pb = 0;
+        if (tid < pj.out_c) {
+            ps = pj.shift[pj.n_shift == 1 ? 0 : tid];
+            pb = pj.bias != nullptr ? pj.bias[tid] : 0;
+            if (ps < 1 || ps > 31) {
+                okp = 0;
+            } else {
+                const long long start = (long long)pb + (1ll << (ps - 1));
+                if ((start < 0 ? -start : start) + bound >= (1ll << (31 - max(0, 8 - ps))))
+                    okp = 0;
+            }
+        }
+        fast_p = __syncthreads_and(okp) != 0;
+        int *cp = reinterpret_cast<int *>(smem + a.off_cp);
+        if (tid < ocp) {
+            cp[tid] = (fast_p && tid < pj.out_c) ? pb + (1 << (ps - 1)) : pb;
+            cp[ocp + tid] = fast_p ? max(0, ps - 8) : ps;
+            cp[2 * ocp + tid] = fast_p ? max(0, 8 - ps) : 0;
+        }
+        floor_p = pj.relu ? 0 : (int)0x80008000u;
+    }
+
     for (; unit < seq.end; unit += seq.step) {
         // patch of this tile: registers -> LDS
 #pragma unroll
@@ -327,20 +387,86 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
             dw_compute<false, false>(a, smem, wave, lane, tapoff, floor_pk);
         __syncthreads();
 
-        // output tile: LDS -> global, consecutive 16-byte pieces
-        const int rows = min(a.th, g.out_h - u_cur.y0), cols = min(a.tw, g.out_w - u_cur.x0);
-        int8_t *obase = a.out + (((long long)u_cur.n * g.out_h + u_cur.y0) * g.out_w + u_cur.x0) * C + cc0;
+        if (PROJ) {
+            // 1x1 project convolution of the tile: rows = filters, columns = tile pixels, reduction
+            // over the depthwise channels, operand B straight from the depthwise result in LDS
+            const DwProject &pj = a.pj;
+            const int col = lane & 15;
+            const int ocp = a.p_nrt * 16;
+            const int *cp = reinterpret_cast<const int *>(smem + a.off_cp);
+            const int n_t = a.p_nrt * a.np;
+            for (int t = wave; t < n_t; t += kWaves) {
+                const int rt = (int)fastdiv((unsigned)t, a.fd_np);
+                const int ct = t - rt * a.np;
+                const int c = 16 * rt + 4 * quad;
+                v4i r = *reinterpret_cast<const v4i *>(cp + c);
+                const unsigned char *bsrc = smem + a.off_out + (ct * 16 + col) * a.cso + 16 * quad;
+                const unsigned char *asrc = smem + a.off_wp + 16 * (rt * a.p_ks * 64 + lane);
+                for (int ks = 0; ks < a.p_ks; ks++) {
+                    const v4i aop = *reinterpret_cast<const v4i *>(asrc + 1024 * ks);
+                    const v4i b = *reinterpret_cast<const v4i *>(bsrc + 64 * ks);
+                    r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b, r, 0, 0, 0);
+                }
+                const v4i ss = *reinterpret_cast<const v4i *>(cp + ocp + c);
+                int word;
+                if (fast_p) {
+                    const v4i ls = *reinterpret_cast<const v4i *>(cp + 2 * ocp + c);
+                    word = pack_fast4<true>(r, ls, ss, floor_p);
+                } else {
+                    int q[4];
 #pragma unroll
-        for (int i = 0; i < kMaxOut; i++) {
-            if (i * kThreads < a.n_out_chunks) { // uniform
-                const int py = out_rc[i] & 0xffff, px = out_rc[i] >> 16;
-                if (out_rc[i] >= 0 && py < rows && px < cols)
-                    *reinterpret_cast<v4i *>(obase + out_rel[i]) =
-                        *reinterpret_cast<const v4i *>(smem + a.off_out + out_lds[i]);
+                    for (int k = 0; k < 4; k++)
+                        q[k] = requant_s8(r[k], ss[k], pj.relu != 0, half_even);
+                    word = pack4_s8(q[0], q[1], q[2], q[3]);
+                }
+                *reinterpret_cast<int *>(smem + a.off_pout + (ct * 16 + col) * a.p_os + c) = word;
+            }
+            __syncthreads();
+        }
+
+        // result tile: LDS -> global, consecutive pieces
+        const int rows = min(a.th, g.out_h - u_cur.y0), cols = min(a.tw, g.out_w - u_cur.x0);
+        if (PROJ) {
+            const DwProject &pj = a.pj;
+            const long long gbase = (((long long)u_cur.n * g.out_h + u_cur.y0) * g.out_w + u_cur.x0) * pj.out_c;
+#pragma unroll
+            for (int i = 0; i < kMaxOut; i++) {
+                if (i * kThreads < a.n_pout_chunks) { // uniform
+                    const int py = out_rc[i] & 0xffff, px = out_rc[i] >> 16;
+                    if (out_rc[i] >= 0 && py < rows && px < cols) {
+                        const long long go = gbase + out_rel[i];
+                        if (a.p_vec == 16) {
+                            v4i w = *reinterpret_cast<const v4i *>(smem + a.off_pout + out_lds[i]);
+                            if (pj.residual != nullptr) {
+                                const v4i rv = *reinterpret_cast<const v4i *>(pj.residual + go);
+#pragma unroll
+                                for (int d = 0; d < 4; d++)
+                                    w[d] = sat_add4_s8(w[d], rv[d]);
+                            }
+                            *reinterpret_cast<v4i *>(pj.out + go) = w;
+                        } else {
+                            int w = *reinterpret_cast<const int *>(smem + a.off_pout + out_lds[i]);
+                            if (pj.residual != nullptr)
+                                w = sat_add4_s8(w, *reinterpret_cast<const int *>(pj.residual + go));
+                            *reinterpret_cast<int *>(pj.out + go) = w;
+                        }
+                    }
+                }
+            }
+        } else {
+            int8_t *obase = a.out + (((long long)u_cur.n * g.out_h + u_cur.y0) * g.out_w + u_cur.x0) * C + cc0;
+#pragma unroll
+            for (int i = 0; i < kMaxOut; i++) {
+                if (i * kThreads < a.n_out_chunks) { // uniform
+                    const int py = out_rc[i] & 0xffff, px = out_rc[i] >> 16;
+                    if (out_rc[i] >= 0 && py < rows && px < cols)
+                        *reinterpret_cast<v4i *>(obase + out_rel[i]) =
+                            *reinterpret_cast<const v4i *>(smem + a.off_out + out_lds[i]);
+                }
             }
         }
-        // the next iteration's patch stores touch only the patch area; its output stores come after
-        // the barrier that follows them, by which time these reads have completed
+        // the next iteration's patch stores touch only the patch area; its stores to the result tiles
+        // come after the barrier that follows them, by which time these reads have completed
     }
 }
 
@@ -355,7 +481,7 @@ constexpr int kLdsBudget = 80 * 1024; // two workgroups of 8 wavefronts per CU (
 
 // Tile choice: the cheapest (patch bytes read per output byte, with a penalty for tiles too small
 // to amortize the per-tile barriers) among the candidates that fit the LDS and register budgets.
-DwLdsPlan dw_lds_plan(const ConvGeom &g)
+DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr)
 {
     DwLdsPlan best;
     best.ok = false;
@@ -373,8 +499,21 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g)
     }
     cand_h.push_back(g.out_h);
     cand_w.push_back(g.out_w);
+    const bool proj = pj != nullptr && pj->w != nullptr;
+    int p_nrt = 0, p_ks = 0, p_os = 0, p_vec = 16, p_vecs = 0;
+    if (proj) {
+        if (G > 16 || pj->out_c > 384 || (pj->out_c & 3) != 0)
+            return best;
+        p_nrt = (pj->out_c + 15) / 16;
+        p_ks = (g.in_c + 63) / 64;
+        p_os = 16 * ((p_nrt & 1) ? p_nrt : p_nrt + 1);
+        const bool al16 = (pj->out_c & 15) == 0 && (reinterpret_cast<uintptr_t>(pj->out) & 15) == 0 &&
+            (pj->residual == nullptr || (reinterpret_cast<uintptr_t>(pj->residual) & 15) == 0);
+        p_vec = al16 ? 16 : 4;
+        p_vecs = pj->out_c / p_vec;
+    }
     for (int gc = 1; gc <= min(G, 16); gc++) {
-        if (G % gc != 0)
+        if (G % gc != 0 || (proj && gc != G))
             continue;
         const int cs = 16 * ((gc & 1) ? gc : gc + 1); // odd number of 16-byte units: conflict-free LDS reads
         const int cso = cs;
@@ -386,9 +525,14 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g)
                 if (n_in > kMaxIn * kThreads || n_out > kMaxOut * kThreads || ph > 0xffff || pw > 0x7fff)
                     continue;
                 const size_t patch = (size_t)ph * pw * cs + 16 * 16; // reads of padded pixel slots stay inside
-                const size_t outb = (size_t)np * 16 * cso;
+                // the project stage reads whole 64-channel k steps: slack after the last pixel
+                const size_t outb = (size_t)np * 16 * cso + (proj ? 256 : 0);
+                const size_t pbytes = proj ? (size_t)p_nrt * p_ks * 1024 + (size_t)3 * p_nrt * 64 + (size_t)np * 16 * p_os : 0;
+                const long long n_pout = (long long)the * twe * p_vecs;
+                if (proj && n_pout > kMaxOut * kThreads)
+                    continue;
                 const size_t tables = (size_t)gc * kKs * 64 * 4 + (size_t)gc * 16 * 12 + (size_t)np * 16 * 4 + 256;
-                const size_t lds = patch + outb + tables + 64;
+                const size_t lds = patch + outb + tables + pbytes + 64;
                 if (lds > (size_t)kLdsBudget)
                     continue;
                 const int per_cu = (int)std::min<size_t>(2, (size_t)(160 * 1024) / lds); // 2 x 8 wavefronts fill a CU
@@ -439,6 +583,18 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g)
                     off += (size_t)np * 16 * 4;
                     a.off_lut = (int)off;
                     off += 256;
+                    a.p_nrt = p_nrt;
+                    a.p_ks = p_ks;
+                    a.p_os = p_os;
+                    a.p_vec = p_vec;
+                    a.p_vecs = p_vecs;
+                    a.n_pout_chunks = (int)n_pout;
+                    a.off_wp = (int)off;
+                    off += (size_t)p_nrt * p_ks * 1024;
+                    a.off_cp = (int)off;
+                    off += (size_t)3 * p_nrt * 64;
+                    a.off_pout = (int)off;
+                    off += proj ? (size_t)np * 16 * p_os : 0;
                     best.lds = off;
                     best.n_cchunk = G / gc;
                 }
@@ -461,6 +617,47 @@ bool depthwise_s8_lds_supports(const ConvGeom &g, const void *in, const void *ou
     return dw_lds_plan(g).ok;
 }
 
+namespace {
+
+template <bool PROJ>
+hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
+{
+    DwLdsArgs &a = plan.a;
+    const ConvGeom &g = a.g;
+    const long long units = (long long)g.batch * a.tiles_y * a.tiles_x;
+    if (units > 0x7fffffff)
+        return hipErrorInvalidValue;
+    a.n_units = (int)units;
+    a.fd_tiles_x = make_fastdiv((unsigned)a.tiles_x);
+    a.fd_tiles_yx = make_fastdiv((unsigned)(a.tiles_y * a.tiles_x));
+    a.fd_pwgc = make_fastdiv((unsigned)(a.pw * a.gc));
+    a.fd_gc = make_fastdiv((unsigned)a.gc);
+    a.fd_tw = make_fastdiv((unsigned)a.tw);
+    a.fd_np = make_fastdiv((unsigned)a.np);
+    a.fd_pvecs = make_fastdiv((unsigned)max(1, a.p_vecs));
+    const int cus = cu_count > 0 ? cu_count : 256;
+    static const hipError_t lds_opt_in = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ>),
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+    if (lds_opt_in != hipSuccess)
+        return lds_opt_in;
+    const int per_cu = resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ>, kThreads, plan.lds);
+    int gx = max(1, (cus * per_cu) / plan.n_cchunk);
+    if (gx > a.n_units)
+        gx = a.n_units;
+    if (gx >= 8)
+        gx &= ~7;
+    static const bool trace = getenv("ESPDL_HIP_TRACE") != nullptr;
+    if (trace)
+        fprintf(stderr, "depthwise_s8_lds%s: %dx%dx%d s%d tile %dx%d patch %dx%d gc %d np %d lds %zu per_cu %d grid %dx%d units %d\n",
+                PROJ ? "+project" : "", g.in_h, g.in_w, g.in_c, g.stride_h, a.th, a.tw, a.ph, a.pw, a.gc, a.np, plan.lds,
+                per_cu, gx, plan.n_cchunk, a.n_units);
+    hipLaunchKernelGGL(depthwise_s8_lds_kernel<PROJ>, dim3((unsigned)gx, (unsigned)plan.n_cchunk), dim3(kThreads),
+                       plan.lds, stream, a);
+    return hipGetLastError();
+}
+
+} // namespace
+
 hipError_t launch_depthwise_s8_lds(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                    const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
                                    hipStream_t stream)
@@ -478,35 +675,39 @@ hipError_t launch_depthwise_s8_lds(const ConvGeom &g, const int8_t *in, const in
     a.lut = lut;
     a.out = out;
     a.g = g;
-    const long long units = (long long)g.batch * a.tiles_y * a.tiles_x;
-    if (units > 0x7fffffff)
+    a.pj = DwProject{};
+    return dw_lds_launch<false>(plan, cu_count, stream);
+}
+
+bool depthwise_project_s8_supports(const ConvGeom &g, const void *in, const DwProject &pj)
+{
+    if ((g.in_c & 15) != 0 || g.k_h * g.k_w > 4 * kKs || pj.w == nullptr ||
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(pj.w)) & 15) != 0 ||
+        ((reinterpret_cast<uintptr_t>(pj.out) | reinterpret_cast<uintptr_t>(pj.residual)) & 3) != 0)
+        return false;
+    if ((long long)g.in_h * g.in_w * g.in_c >= (1ll << 30) || (long long)g.out_h * g.out_w * pj.out_c >= (1ll << 30))
+        return false;
+    return dw_lds_plan(g, &pj).ok;
+}
+
+hipError_t launch_depthwise_project_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                       const int32_t *shift, const DwProject &pj, int cu_count, hipStream_t stream)
+{
+    if ((long long)g.batch * g.out_h * g.out_w == 0)
+        return hipSuccess;
+    DwLdsPlan plan = dw_lds_plan(g, &pj);
+    if (!plan.ok)
         return hipErrorInvalidValue;
-    a.n_units = (int)units;
-    a.fd_tiles_x = make_fastdiv((unsigned)a.tiles_x);
-    a.fd_tiles_yx = make_fastdiv((unsigned)(a.tiles_y * a.tiles_x));
-    a.fd_pwgc = make_fastdiv((unsigned)(a.pw * a.gc));
-    a.fd_gc = make_fastdiv((unsigned)a.gc);
-    a.fd_tw = make_fastdiv((unsigned)a.tw);
-    a.fd_np = make_fastdiv((unsigned)a.np);
-    const int cus = cu_count > 0 ? cu_count : 256;
-    static const hipError_t lds_opt_in = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(depthwise_s8_lds_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
-    if (lds_opt_in != hipSuccess)
-        return lds_opt_in;
-    const int per_cu = resident_workgroups_per_cu(depthwise_s8_lds_kernel, kThreads, plan.lds);
-    int gx = max(1, (cus * per_cu) / plan.n_cchunk);
-    if (gx > a.n_units)
-        gx = a.n_units;
-    if (gx >= 8)
-        gx &= ~7;
-    static const bool trace = getenv("ESPDL_HIP_TRACE") != nullptr;
-    if (trace)
-        fprintf(stderr, "depthwise_s8_lds: %dx%dx%d s%d tile %dx%d patch %dx%d gc %d np %d lds %zu per_cu %d grid %dx%d units %d\n",
-                g.in_h, g.in_w, g.in_c, g.stride_h, a.th, a.tw, a.ph, a.pw, a.gc, a.np, plan.lds, per_cu, gx, plan.n_cchunk,
-                a.n_units);
-    hipLaunchKernelGGL(depthwise_s8_lds_kernel, dim3((unsigned)gx, (unsigned)plan.n_cchunk), dim3(kThreads), plan.lds,
-                       stream, a);
-    return hipGetLastError();
+    DwLdsArgs &a = plan.a;
+    a.in = in;
+    a.w = filter;
+    a.bias = bias;
+    a.shift = shift;
+    a.lut = nullptr;
+    a.out = nullptr;
+    a.g = g;
+    a.pj = pj;
+    return dw_lds_launch<true>(plan, cu_count, stream);
 }
 
 } // namespace espdl

@@ -112,6 +112,19 @@ __device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const 
                                       0x07050301u);
 }
 
+// int8 x 4 saturating add of two packed dwords
+__device__ __forceinline__ int sat_add4_s8(int x, int y)
+{
+    int r = 0;
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        int s = (int)(int8_t)(x >> (8 * b)) + (int)(int8_t)(y >> (8 * b));
+        s = s < -128 ? -128 : (s > 127 ? 127 : s);
+        r |= (s & 0xff) << (8 * b);
+    }
+    return r;
+}
+
 // Division of a 31-bit unsigned number by a launch-invariant divisor: q = (mulhi(n, m) + n) >> s
 // with m = floor(2^32 * (2^s - d) / d) + 1, s = ceil(log2 d)  (Granlund-Montgomery; exact for
 // every n < 2^31).  The host fills the struct, the device spends three instructions.

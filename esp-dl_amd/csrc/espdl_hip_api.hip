@@ -375,6 +375,37 @@ int mbconv_geometry(const espdl_hip_mbconv_desc *d, espdl::MbconvParams *p)
     return ESPDL_HIP_OK;
 }
 
+// Depthwise geometry and project description of a block without expand stage.
+void dwproject_from(const espdl::MbconvParams &p, espdl::ConvGeom *g, espdl::DwProject *pj)
+{
+    g->batch = p.batch;
+    g->in_h = p.in_h;
+    g->in_w = p.in_w;
+    g->in_c = p.in_c;
+    g->out_c = p.in_c;
+    g->out_h = p.out_h;
+    g->out_w = p.out_w;
+    g->k_h = p.k_h;
+    g->k_w = p.k_w;
+    g->stride_h = p.stride_h;
+    g->stride_w = p.stride_w;
+    g->dil_h = p.dil_h;
+    g->dil_w = p.dil_w;
+    g->pad_top = p.pad_top;
+    g->pad_left = p.pad_left;
+    g->relu = p.relu_dw;
+    g->half_even = p.half_even;
+    g->n_shift = p.n_s_dw;
+    pj->w = p.w_project;
+    pj->bias = p.b_project;
+    pj->shift = p.s_project;
+    pj->n_shift = p.n_s_project;
+    pj->relu = p.relu_project;
+    pj->out_c = p.out_c;
+    pj->residual = p.residual;
+    pj->out = p.out;
+}
+
 } // namespace
 
 extern "C" {
@@ -404,6 +435,13 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
     p.w_expand = desc->has_expand ? aligned : nullptr;
     p.w_dw = aligned;
     p.w_project = aligned;
+    if (!desc->has_expand) {
+        espdl::ConvGeom g;
+        espdl::DwProject pj;
+        dwproject_from(p, &g, &pj);
+        if (espdl::depthwise_project_s8_supports(g, p.in, pj))
+            return 1;
+    }
     return espdl::mbconv_s8_fused_supports(p) ? 1 : 0;
 }
 
@@ -435,6 +473,15 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
     p.w_project = w->w_project;
     p.b_project = w->b_project;
     p.s_project = w->s_project;
+    if (!desc->has_expand) {
+        espdl::ConvGeom g;
+        espdl::DwProject pj;
+        dwproject_from(p, &g, &pj);
+        if (espdl::depthwise_project_s8_supports(g, p.in, pj))
+            return device_status(espdl::launch_depthwise_project_s8(g, p.in, p.w_dw, p.b_dw, p.s_dw, pj, cu_count_cached(),
+                                                                    reinterpret_cast<hipStream_t>(stream)),
+                                 "depthwise_project_s8");
+    }
     if (!espdl::mbconv_s8_fused_supports(p))
         return fail(ESPDL_HIP_ENOTSUP, "this block shape is not covered by the fused kernel");
     return device_status(espdl::launch_mbconv_s8_fused(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),

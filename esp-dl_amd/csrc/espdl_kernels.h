@@ -28,6 +28,15 @@ hipError_t launch_depthwise_s8_mfma(const ConvGeom &g, const int8_t *in, const i
                                     const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
                                     hipStream_t stream);
 
+// 1x1 project convolution (+ saturating residual Add) fused behind a depthwise convolution.
+struct DwProject {
+    const int8_t *w; // [out_c][channels of the depthwise stage]
+    const int32_t *bias, *shift;
+    int n_shift, relu, out_c;
+    const int8_t *residual; // shape of out, or nullptr
+    int8_t *out;
+};
+
 // Depthwise with the input tile staged in LDS (contiguous global reads and writes) and the products
 // on the matrix pipe; same shape limits as the direct form.
 bool depthwise_s8_lds_supports(const ConvGeom &g, const void *in, const void *out);
@@ -56,6 +65,12 @@ struct MbconvParams {
 };
 bool mbconv_s8_fused_supports(const MbconvParams &p);
 hipError_t launch_mbconv_s8_fused(const MbconvParams &p, int cu_count, hipStream_t stream);
+
+// Depthwise -> 1x1 project [-> Add] in one launch of the LDS-tile depthwise kernel: the depthwise
+// result never leaves LDS.  Needs at most 256 depthwise channels.
+bool depthwise_project_s8_supports(const ConvGeom &g, const void *in, const DwProject &pj);
+hipError_t launch_depthwise_project_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                       const int32_t *shift, const DwProject &pj, int cu_count, hipStream_t stream);
 
 hipError_t launch_conv2d_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
                              const int32_t *shift, int16_t *out, hipStream_t stream);

@@ -83,19 +83,6 @@ __device__ __forceinline__ TilePos mb_tile(const MbArgs &a, int unit)
     return u;
 }
 
-// int8 x 4 saturating add of two packed dwords
-__device__ __forceinline__ int sat_add4_s8(int x, int y)
-{
-    int r = 0;
-#pragma unroll
-    for (int b = 0; b < 4; b++) {
-        int s = (int)(int8_t)(x >> (8 * b)) + (int)(int8_t)(y >> (8 * b));
-        s = s < -128 ? -128 : (s > 127 ? 127 : s);
-        r |= (s & 0xff) << (8 * b);
-    }
-    return r;
-}
-
 // Requantize four accumulators of one lane (channels c..c+3) to a packed dword.
 __device__ __forceinline__ int mb_pack(const v4i &acc, const int *cst, int stride, int c, bool fast, bool relu,
                                        bool half_even, int floor_pk)

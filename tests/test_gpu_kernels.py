@@ -357,6 +357,12 @@ MBCONV_CASES = [
     ("tailpad_17x17_32_96_32_s2", (2, 17, 17, 32), 96, 32, (3, 3), (2, 2), (0, 1, 0, 1), False, False, False),
     ("halfeven_14x14_32_192_32_res", (2, 14, 14, 32), 192, 32, (3, 3), (1, 1), (1, 1, 1, 1), True, True, False),
     ("pertensor_28x28_32_192_64", (2, 28, 28, 32), 192, 64, (3, 3), (1, 1), (1, 1, 1, 1), False, False, True),
+    # no expand stage: depthwise -> project [-> Add] inside the LDS-tile depthwise kernel
+    ("dwp_56x56_144_24_res", (2, 56, 56, 144), None, 24, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
+    ("dwp_57x41_96_24_s2", (2, 57, 41, 96), None, 24, (3, 3), (2, 2), (1, 1, 1, 1), False, False, False),
+    ("dwp_28x28_192_64_s2", (3, 28, 28, 192), None, 64, (3, 3), (2, 2), (0, 1, 0, 1), False, False, False),
+    ("dwp_20x20_256_48_res_halfeven", (2, 20, 20, 256), None, 48, (3, 3), (1, 1), (1, 1, 1, 1), True, True, False),
+    ("dwp_112x112_32_16", (1, 112, 112, 32), None, 16, (3, 3), (1, 1), (1, 1, 1, 1), False, False, True),
 ]
 
 
