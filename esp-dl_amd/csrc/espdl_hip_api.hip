@@ -440,7 +440,7 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
         espdl::DwProject pj;
         dwproject_from(p, &g, &pj);
         if (espdl::depthwise_project_s8_supports(g, p.in, pj))
-            return 1;
+            return 2;
     }
     return espdl::mbconv_s8_fused_supports(p) ? 1 : 0;
 }

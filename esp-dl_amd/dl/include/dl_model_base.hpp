@@ -27,12 +27,15 @@ struct module_info {
     int64_t bytes;    ///< bytes of the tensors it reads and writes (each counted once)
 };
 
+enum { FUSE_CONV_LUT = 1, FUSE_DW_PROJECT = 2 };
+
 class Model {
 public:
     /// The model does not take ownership of `fbs_model`.  `stream` is a hipStream_t (nullptr: the
-    /// model creates its own).  `fuse_lut` folds a LUT that directly follows a Conv into its epilogue.
+    /// model creates its own).  `fuse` is a bit mask of graph fusions: FUSE_CONV_LUT folds a LUT that directly follows a Conv
+    /// into its epilogue, FUSE_DW_PROJECT runs depthwise Conv -> 1x1 Conv [-> Add] as one kernel.
     Model(fbs::FbsModel *fbs_model, int batch = 1, round_mode_t round_mode = ROUND_MODE_HALF_UP, void *stream = nullptr,
-          bool fuse_lut = true);
+          int fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT);
     virtual ~Model();
     Model(const Model &) = delete;
     Model &operator=(const Model &) = delete;
@@ -82,6 +85,7 @@ public:
 
 private:
     void fuse_conv_lut();
+    void fuse_dw_project();
 
     fbs::FbsModel *m_fbs_model = nullptr;
     std::vector<dl::module::Module *> m_execution_plan;
@@ -90,7 +94,7 @@ private:
     std::string m_name, m_doc_string;
     int64_t m_version = 0;
     int m_batch = 1;
-    bool m_fuse_lut = true;
+    int m_fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT;
     void *m_stream = nullptr;
     bool m_own_stream = false;
     void *m_graph = nullptr;      // hipGraph_t

@@ -39,6 +39,14 @@ private:
     int m_group;
     TensorBase *m_fused_lut; ///< device int8[256] applied to the stored value, or nullptr (owned)
     DeviceInts m_shift;
+    // A depthwise Conv may absorb the 1x1 Conv that follows it (and the Add after that): the three
+    // run as one kernel and the depthwise result stays on chip.  The absorbed modules' parameter
+    // indices are appended to m_inputs_index at the positions below.
+    bool m_has_project = false;
+    activation_type_t m_project_activation = Linear;
+    int m_mid_exponent = 0;      ///< exponent of the (no longer materialized) depthwise output
+    int m_project_filter_pos = -1, m_project_bias_pos = -1, m_residual_pos = -1;
+    DeviceInts m_shift_project;
 
 public:
     Conv(activation_type_t activation = Linear, std::vector<int> pads = {}, std::vector<int> dilations = {},
@@ -64,6 +72,34 @@ public:
         m_fused_lut = table;
     }
     bool has_fused_lut() const { return m_fused_lut != nullptr; }
+    bool has_fused_project() const { return m_has_project; }
+    const std::vector<int> &get_pads() const { return m_pads; }
+    const std::vector<int> &get_strides() const { return m_strides; }
+    const std::vector<int> &get_dilations() const { return m_dilations; }
+    /// Absorb a following 1x1 Conv (filter / bias indices, activation) and optionally the other
+    /// operand of the Add after it.  The caller re-points m_outputs_index at the final tensor.
+    void fuse_project(int filter_index, int bias_index, activation_type_t act, int mid_exponent, int residual_index)
+    {
+        m_has_project = true;
+        m_project_activation = act;
+        m_mid_exponent = mid_exponent;
+        m_project_filter_pos = (int)m_inputs_index.size();
+        m_inputs_index.push_back(filter_index);
+        if (bias_index >= 0) {
+            m_project_bias_pos = (int)m_inputs_index.size();
+            m_inputs_index.push_back(bias_index);
+        }
+        if (residual_index >= 0) {
+            m_residual_pos = (int)m_inputs_index.size();
+            m_inputs_index.push_back(residual_index);
+        }
+    }
+    /// Position of the depthwise bias in m_inputs_index, or -1.
+    int own_bias_pos() const
+    {
+        const int own = m_has_project ? m_project_filter_pos : (int)m_inputs_index.size();
+        return own == 3 ? 2 : -1;
+    }
 
     std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
     {
@@ -86,6 +122,8 @@ public:
                     m_strides[1] +
                 1;
             output_shape[3] = m_group == 1 ? filter_shape[3] : input_shape[3];
+            if (m_has_project)
+                output_shape[3] = input_shapes[m_project_filter_pos][3];
         }
         return {output_shape};
     }
@@ -99,6 +137,8 @@ public:
             pixels *= out[i];
         const int64_t taps = out.size() == 3 ? f[0] : (int64_t)f[0] * f[1];
         const int64_t in_c = m_group == 1 ? input_shapes[0].back() : 1;
+        if (m_has_project) // depthwise over the input channels + 1x1 over them
+            return pixels * input_shapes[0].back() * taps + pixels * out.back() * input_shapes[0].back();
         return pixels * out.back() * taps * in_c;
     }
 
@@ -107,8 +147,12 @@ public:
         (void)mode;
         TensorBase *input = context->get_tensor(m_inputs_index[0]);
         TensorBase *filter = context->get_tensor(m_inputs_index[1]);
-        TensorBase *bias = m_inputs_index.size() == 3 ? context->get_tensor(m_inputs_index[2]) : nullptr;
+        TensorBase *bias = own_bias_pos() >= 0 ? context->get_tensor(m_inputs_index[own_bias_pos()]) : nullptr;
         TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (m_has_project) {
+            forward_with_project(context, input, filter, bias, output);
+            return;
+        }
         if (!input || !filter || !output || !input->on_device() || !filter->on_device() || !output->on_device() ||
             (bias && !bias->on_device())) {
             DL_LOGE("Conv", "%s: tensors must be device tensors", name.c_str());
@@ -168,6 +212,70 @@ public:
         const int rc = espdl_hip_conv2d(&d, input->data, filter->data, bias ? bias->data : nullptr, shift_dev,
                                         m_fused_lut ? static_cast<const int8_t *>(m_fused_lut->data) : nullptr,
                                         output->data, context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Conv", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+
+    /// depthwise -> 1x1 project [-> Add] through espdl_hip_mbconv_s8 (has_expand = 0)
+    void forward_with_project(ModelContext *context, TensorBase *input, TensorBase *filter, TensorBase *bias,
+                              TensorBase *output)
+    {
+        TensorBase *pfilter = context->get_tensor(m_inputs_index[m_project_filter_pos]);
+        TensorBase *pbias = m_project_bias_pos >= 0 ? context->get_tensor(m_inputs_index[m_project_bias_pos]) : nullptr;
+        TensorBase *residual = m_residual_pos >= 0 ? context->get_tensor(m_inputs_index[m_residual_pos]) : nullptr;
+        if (!input || !filter || !output || !pfilter || !input->on_device() || !filter->on_device() ||
+            !output->on_device() || !pfilter->on_device() || (bias && !bias->on_device()) ||
+            (pbias && !pbias->on_device()) || (residual && !residual->on_device()) || input->shape.size() != 4) {
+            DL_LOGE("Conv", "%s: fused depthwise+project needs 4-D device tensors", name.c_str());
+            return;
+        }
+        espdl_hip_mbconv_desc d = {};
+        d.batch = input->shape[0];
+        d.in_h = input->shape[1];
+        d.in_w = input->shape[2];
+        d.in_c = input->shape[3];
+        d.exp_c = d.in_c;
+        d.out_c = output->shape[3];
+        d.has_expand = 0;
+        d.k_h = filter->shape[0];
+        d.k_w = filter->shape[1];
+        d.stride_h = m_strides[0];
+        d.stride_w = m_strides[1];
+        d.dil_h = m_dilations[0];
+        d.dil_w = m_dilations[1];
+        d.pad_top = m_pads[0];
+        d.pad_bottom = m_pads[1];
+        d.pad_left = m_pads[2];
+        d.pad_right = m_pads[3];
+        d.act_dw = activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR;
+        d.act_project = m_project_activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR;
+        d.round_mode = context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP;
+        std::vector<int32_t> s_dw, s_pj;
+        if (filter->exponent.is_per_channel()) {
+            for (int c = 0; c < d.in_c; c++)
+                s_dw.push_back(m_mid_exponent - filter->exponent.get(c) - input->exponent.get());
+        } else {
+            s_dw.push_back(m_mid_exponent - filter->exponent.get() - input->exponent.get());
+        }
+        if (pfilter->exponent.is_per_channel()) {
+            for (int c = 0; c < d.out_c; c++)
+                s_pj.push_back(output->exponent.get() - pfilter->exponent.get(c) - m_mid_exponent);
+        } else {
+            s_pj.push_back(output->exponent.get() - pfilter->exponent.get() - m_mid_exponent);
+        }
+        d.n_shift_expand = 1;
+        d.n_shift_dw = (int32_t)s_dw.size();
+        d.n_shift_project = (int32_t)s_pj.size();
+        espdl_hip_mbconv_weights w = {};
+        w.w_dw = static_cast<const int8_t *>(filter->data);
+        w.b_dw = bias ? static_cast<const int32_t *>(bias->data) : nullptr;
+        w.s_dw = m_shift.sync(s_dw);
+        w.w_project = static_cast<const int8_t *>(pfilter->data);
+        w.b_project = pbias ? static_cast<const int32_t *>(pbias->data) : nullptr;
+        w.s_project = m_shift_project.sync(s_pj);
+        const int rc = espdl_hip_mbconv_s8(&d, static_cast<const int8_t *>(input->data), &w,
+                                           residual ? static_cast<const int8_t *>(residual->data) : nullptr,
+                                           static_cast<int8_t *>(output->data), context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("Conv", "%s: %s", name.c_str(), espdl_hip_last_error());
     }

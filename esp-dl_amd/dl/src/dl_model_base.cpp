@@ -1,4 +1,5 @@
 #include "dl_model_base.hpp"
+#include "espdl_hip.h"
 
 #include <hip/hip_runtime.h>
 
@@ -98,8 +99,8 @@ private:
 
 } // namespace
 
-Model::Model(fbs::FbsModel *fbs_model, int batch, round_mode_t round_mode, void *stream, bool fuse_lut) :
-    m_batch(batch), m_fuse_lut(fuse_lut), m_stream(stream)
+Model::Model(fbs::FbsModel *fbs_model, int batch, round_mode_t round_mode, void *stream, int fuse) :
+    m_batch(batch), m_fuse(fuse), m_stream(stream)
 {
     m_model_context = new ModelContext();
     m_model_context->owns_tensors = true;
@@ -178,8 +179,10 @@ esp_err_t Model::load(fbs::FbsModel *fbs_model)
         for (size_t j = 0; j < op_outputs.size(); j++)
             module->m_outputs_index.push_back(m_model_context->add_tensor(op_outputs[j], false, nullptr));
     }
-    if (ret == ESP_OK && m_fuse_lut)
+    if (ret == ESP_OK && (m_fuse & FUSE_CONV_LUT))
         fuse_conv_lut();
+    if (ret == ESP_OK && (m_fuse & FUSE_DW_PROJECT))
+        fuse_dw_project();
     return ret;
 }
 
@@ -218,6 +221,122 @@ void Model::fuse_conv_lut()
         m_execution_plan.erase(m_execution_plan.begin() + lut_pos);
         if (lut_pos < i)
             i--;
+    }
+}
+
+// depthwise Conv -> 1x1 Conv [-> Add]: when the depthwise output has no other reader (and, for the
+// Add, the project output has none either) the chain becomes one module that keeps the depthwise
+// result on chip (espdl_hip_mbconv_s8 without expand stage).  Every value is formed exactly as the
+// separate modules form it, so results do not change.  The fused module takes the place of the last
+// module it absorbs, so everything it reads (the Add's other operand included) is produced before it.
+void Model::fuse_dw_project()
+{
+    std::set<std::string> pinned;
+    for (auto &n : m_fbs_model->get_graph_outputs())
+        pinned.insert(n);
+    for (auto &n : m_fbs_model->get_test_outputs_name())
+        pinned.insert(n);
+    auto single_reader = [&](int tensor, size_t *pos) {
+        int readers = 0;
+        for (size_t j = 0; j < m_execution_plan.size(); j++)
+            for (int in : m_execution_plan[j]->m_inputs_index)
+                if (in == tensor) {
+                    readers++;
+                    *pos = j;
+                }
+        return readers == 1 && !pinned.count(m_model_context->get_tensor_name(tensor));
+    };
+    for (size_t i = 0; i < m_execution_plan.size(); i++) {
+        auto *dw = dynamic_cast<dl::module::Conv *>(m_execution_plan[i]);
+        if (!dw || dw->quant_type != QUANT_TYPE_SYMM_8BIT || dw->get_group() == 1 || dw->has_fused_lut() ||
+            dw->has_fused_project() || dw->get_pads().size() != 4)
+            continue;
+        const int mid = dw->m_outputs_index[0];
+        size_t pj_pos = 0;
+        if (!single_reader(mid, &pj_pos) || pj_pos <= i)
+            continue;
+        auto *pj = dynamic_cast<dl::module::Conv *>(m_execution_plan[pj_pos]);
+        if (!pj || pj->quant_type != QUANT_TYPE_SYMM_8BIT || pj->get_group() != 1 || pj->has_fused_lut() ||
+            pj->has_fused_project() || pj->m_inputs_index[0] != mid)
+            continue;
+        TensorBase *pf = m_model_context->get_tensor(pj->m_inputs_index[1]);
+        TensorBase *df = m_model_context->get_tensor(dw->m_inputs_index[1]);
+        const std::vector<int> in_shape = m_fbs_model->get_value_info_shape(m_model_context->get_tensor_name(dw->m_inputs_index[0]));
+        if (!pf || !df || pf->shape.size() != 4 || df->shape.size() != 4 || pf->shape[0] != 1 || pf->shape[1] != 1 ||
+            in_shape.size() != 4)
+            continue;
+        bool plain = true; // 1x1, stride 1, no padding, no dilation
+        for (int v : pj->get_pads())
+            plain = plain && v == 0;
+        for (int v : pj->get_strides())
+            plain = plain && v == 1;
+        for (int v : pj->get_dilations())
+            plain = plain && v == 1;
+        if (!plain)
+            continue;
+        espdl_hip_mbconv_desc d = {};
+        d.batch = 1;
+        d.in_h = in_shape[1];
+        d.in_w = in_shape[2];
+        d.in_c = in_shape[3];
+        d.exp_c = d.in_c;
+        d.out_c = pf->shape[3];
+        d.k_h = df->shape[0];
+        d.k_w = df->shape[1];
+        d.stride_h = dw->get_strides()[0];
+        d.stride_w = dw->get_strides()[1];
+        d.dil_h = dw->get_dilations()[0];
+        d.dil_w = dw->get_dilations()[1];
+        d.pad_top = dw->get_pads()[0];
+        d.pad_bottom = dw->get_pads()[1];
+        d.pad_left = dw->get_pads()[2];
+        d.pad_right = dw->get_pads()[3];
+        d.n_shift_expand = d.n_shift_dw = d.n_shift_project = 1;
+        // only where the depthwise+project kernel applies (answer 2): that form beats separate launches
+        if (pf->shape[2] != d.in_c || espdl_hip_mbconv_s8_supported(&d) != 2)
+            continue;
+
+        // optional Add behind the project conv
+        int out_index = pj->m_outputs_index[0];
+        int residual = -1;
+        size_t last_pos = pj_pos, add_pos = 0;
+        dl::module::Add *add = nullptr;
+        if (single_reader(out_index, &add_pos) && add_pos > pj_pos) {
+            add = dynamic_cast<dl::module::Add *>(m_execution_plan[add_pos]);
+            if (add && add->quant_type == QUANT_TYPE_SYMM_8BIT && add->m_inputs_index.size() == 2 &&
+                add->m_inputs_index[0] != add->m_inputs_index[1]) {
+                const int other = add->m_inputs_index[0] == out_index ? add->m_inputs_index[1] : add->m_inputs_index[0];
+                const std::string other_name = m_model_context->get_tensor_name(other);
+                const std::string out_name = m_model_context->get_tensor_name(out_index);
+                if (other < CONTEXT_PARAMETER_OFFSET && m_fbs_model->has_value_info(other_name) &&
+                    m_fbs_model->get_value_info_shape(other_name) == m_fbs_model->get_value_info_shape(out_name)) {
+                    residual = other;
+                    out_index = add->m_outputs_index[0];
+                    last_pos = add_pos;
+                } else {
+                    add = nullptr;
+                }
+            } else {
+                add = nullptr;
+            }
+        }
+        const int mid_exp = m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(mid));
+        dw->fuse_project(pj->m_inputs_index[1], pj->m_inputs_index.size() == 3 ? pj->m_inputs_index[2] : -1,
+                         pj->get_activation(), mid_exp, residual);
+        dw->m_outputs_index[0] = out_index;
+        // the fused module moves to the slot of the last absorbed module
+        m_execution_plan[last_pos] = dw;
+        if (add) {
+            delete add;
+            if (last_pos != pj_pos) {
+                delete pj;
+                m_execution_plan.erase(m_execution_plan.begin() + pj_pos);
+            }
+        } else {
+            delete pj;
+        }
+        m_execution_plan.erase(m_execution_plan.begin() + i);
+        i--;
     }
 }
 

@@ -139,13 +139,13 @@ int espdl_graph_add_test_output(espdl_graph *g, const char *name, const int32_t 
     return 0;
 }
 
-espdl_model *espdl_model_create(espdl_graph *g, int32_t batch, int32_t round_mode, void *stream, int32_t fuse_lut)
+espdl_model *espdl_model_create(espdl_graph *g, int32_t batch, int32_t round_mode, void *stream, int32_t fuse)
 {
     if (!g || batch <= 0)
         return nullptr;
     espdl_model *m = new espdl_model();
     m->model = new dl::Model(&g->fbs, batch, round_mode == 1 ? dl::ROUND_MODE_HALF_EVEN : dl::ROUND_MODE_HALF_UP, stream,
-                             fuse_lut != 0);
+                             (int)fuse);
     if (m->model->get_outputs().empty() || m->model->get_module_count() == 0) {
         delete m->model;
         delete m;

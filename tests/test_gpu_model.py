@@ -35,14 +35,14 @@ def _check_all(spec, mdl, want, skip_missing=True):
     return checked
 
 
-def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False):
+def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fuse_blocks=True):
     m, zoo, model, runner = _mods()
     import espdl_oracle as oracle
     rng = np.random.default_rng(seed)
     x = spec.make_input(rng, batch)
     want = runner.run(spec, {spec.inputs[0]: x}, oracle.ROUND_HALF_EVEN if round_mode else oracle.ROUND_HALF_UP)
     g = model.Graph.from_spec(spec)
-    mdl = model.Model(g, batch, round_mode=round_mode, fuse_lut=fuse_lut)
+    mdl = model.Model(g, batch, round_mode=round_mode, fuse_lut=fuse_lut, fuse_blocks=fuse_blocks)
     mdl.set_input(spec.inputs[0], x)
     if graph:
         assert mdl.enable_graph()
@@ -165,7 +165,7 @@ def test_config4_yolo_style(oracle, fuse):
     announce(f"model config4 160px fuse={fuse}")
     _, zoo, _, _ = _mods()
     spec = zoo.config4_yolo_style(resolution=160)
-    mdl, want, _ = _run_config(spec, 2, 8, fuse_lut=fuse)
+    mdl, want, _ = _run_config(spec, 2, 8, fuse_lut=fuse, fuse_blocks=fuse)
     assert len(spec.outputs) == 6
     for name in spec.outputs:
         got = mdl.get_tensor(name, _np_dtype(spec, name))
@@ -209,3 +209,20 @@ def test_unknown_operator_fails_to_load():
     spec.nodes[0]["op_type"] = "NoSuchOp"
     with pytest.raises(model.EspdlModelError):
         model.Model(model.Graph.from_spec(spec), 1)
+
+
+@pytest.mark.parametrize("fuse_blocks", [True, False], ids=["fused_blocks", "separate_modules"])
+def test_mobilenetv2_block_fusion(oracle, fuse_blocks):
+    """depthwise -> project [-> Add] chains run as one module or as separate ones: same logits, and the
+    fused plan is shorter (only blocks with at most 256 expanded channels fuse)."""
+    announce(f"model config3 96px fuse_blocks={fuse_blocks}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.config3_mobilenetv2(resolution=96, num_classes=100)
+    mdl, want, _ = _run_config(spec, 3, 21, fuse_blocks=fuse_blocks)
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
+    if fuse_blocks:
+        assert mdl.module_count() < len(spec.nodes)
+    else:
+        assert mdl.module_count() == len(spec.nodes)
+    mdl.close()
