@@ -12,19 +12,21 @@
 //   Add               saturating int8 add without rescale (esp-dl/dl/base/dl_base_add.cpp:34-44)
 // so a fused block is bit-identical to running Conv, Conv, Conv, Add modules one after the other.
 //
-// A workgroup (8 wavefronts) owns a th x tw tile of the block's output in one image and walks the
-// expanded channels in chunks of 64:
-//   1. the input patch (tile + filter halo, all input channels) is copied to LDS once;
-//   2. per chunk: the chunk's expand filters and project filter columns are staged in LDS in MFMA
-//      operand order (the next chunk's are already in flight in registers);
-//      expand   = MFMA GEMM  [64 filters] x [patch pixels] over the input channels -> E (LDS, int8);
-//                 positions outside the image are forced to zero: the depthwise zero padding pads the
-//                 *expanded* activation;
-//      depthwise= MFMA with a diagonal operand A, operand B straight from E            -> D (LDS, int8);
-//      project  = MFMA GEMM  [out_c filters] x [tile pixels], K = the chunk's 64 channels, accumulated
-//                 over the chunks in registers;
-//   3. project epilogue -> LDS -> (+ residual read from global) -> contiguous 16-byte global stores.
-// Without an expand stage (first block of MobileNetV2) the depthwise stage reads the input patch.
+// The kernel is built for blocks at small spatial sizes (14x14, 7x7 in MobileNetV2), where separate
+// kernels are bound by launch and start-up latency, not by bandwidth.  A workgroup of 16 wavefronts
+// owns a th x tw tile of the block's output in one image:
+//   1. the input patch (tile + filter halo, all input channels) is copied to LDS;
+//   2. the expanded channels are walked in chunks of 64:
+//      expand    MFMA GEMM [64 filters] x [patch pixels] over the input channels -> E (LDS, int8, two
+//                buffers); positions outside the image are forced to zero, because the depthwise zero
+//                padding pads the *expanded* activation; operand A comes straight from the filter in
+//                global memory (L2), requested one chunk ahead;
+//      depthwise MFMA with a diagonal operand A, operand B straight from E -> D (LDS, int8, all chunks);
+//      expand(c) and depthwise(c - 1) share one barrier;
+//   3. project   MFMA GEMM [out_c filters] x [tile pixels] over all expanded channels from D, operand A
+//                straight from the filter in global memory, one k step ahead;
+//   4. epilogue -> LDS -> (+ residual read from global) -> contiguous global stores.
+// Without an expand stage the depthwise stage reads the input patch.
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -36,35 +38,36 @@ namespace espdl {
 
 namespace {
 
-constexpr int kThreads = 512;
+constexpr int kThreads = 1024;
 constexpr int kWaves = kThreads / 64;
-constexpr int kKsDw = 3;    // depthwise k steps of 4 taps
-constexpr int kMaxKse = 4;  // expand k steps of 64 input channels (in_c <= 256)
-constexpr int kMaxAcc = 10; // project accumulator tiles per wavefront
-constexpr int kMaxWe = 2;   // 16-byte expand-filter units per thread and chunk
-constexpr int kMaxWp = 3;   // 16-byte project-filter units per thread and chunk
-constexpr int kEs = 80;     // pixel stride of E and D in LDS: 64 channels + 16 (odd number of 16-byte units)
+constexpr int kParts = kWaves / 4; // wavefronts that share a row tile / channel group split the column tiles
+constexpr int kKsDw = 3;           // depthwise k steps of 4 taps
+constexpr int kMaxKse = 3;         // expand k steps of 64 input channels (in_c <= 192)
+constexpr int kMaxAcc = 5;         // project accumulator tiles per wavefront
+constexpr int kEs = 80;            // pixel stride of E in LDS: 64 channels + 16 (odd number of 16-byte units)
 
 struct MbArgs {
     MbconvParams p;
     int has_expand;
     int taps;
     int th, tw, ph, pw;
-    int p_in, p_out;       // pixels of the patch / of the tile
-    int nct_in, nct_out;   // column tiles of 16 pixels
-    int xs;                // LDS pixel stride of the input patch, bytes
-    int kse;               // expand k steps
-    int n_chunks;          // chunks of 64 expanded channels
-    int nrt;               // project row tiles of 16 filters
-    int n_acc;             // nrt * nct_out
-    int os;                // LDS pixel stride of the output tile, bytes
-    int out_vec;           // bytes per output store piece: 16 or 4
-    int in_vec;            // bytes per input load piece: 16 or 4
+    int p_in, p_out;     // pixels of the patch / of the tile
+    int nct_in, nct_out; // column tiles of 16 pixels
+    int xs;              // LDS pixel stride of the input patch, bytes
+    int ds;              // LDS pixel stride of D, bytes
+    int kse;             // expand k steps
+    int ksp;             // project k steps (chunks of 64 expanded channels)
+    int n_chunks;        // = ksp
+    int nrt;             // project row tiles of 16 filters
+    int n_acc;           // nrt * nct_out
+    int os;              // LDS pixel stride of the output tile, bytes
+    int out_vec;         // bytes per output store piece: 16 or 4
+    int in_vec;          // bytes per input load piece: 16 or 4
+    int in_vecs, out_vecs;
     int tiles_x, tiles_y, n_units;
     FastDiv fd_tiles_x, fd_tiles_yx, fd_pw, fd_tw, fd_nct_out, fd_in_vecs, fd_out_vecs;
-    int in_vecs, out_vecs; // pieces per pixel
     // LDS layout (byte offsets)
-    int off_x, off_e, off_d, off_out, off_we, off_wp, off_wd, off_ce, off_cd, off_cp, off_pixtab, off_rctab, off_slottab;
+    int off_x, off_e, off_d, off_out, off_wd, off_ce, off_cd, off_cp, off_pixtab, off_rctab;
 };
 
 struct TilePos {
@@ -83,121 +86,6 @@ __device__ __forceinline__ TilePos mb_tile(const MbArgs &a, int unit)
     return u;
 }
 
-// Requantize four accumulators of one lane (channels c..c+3) to a packed dword.
-__device__ __forceinline__ int mb_pack(const v4i &acc, const int *cst, int stride, int c, bool fast, bool relu,
-                                       bool half_even, int floor_pk)
-{
-    // cst: [init | shift | lsh] arrays of `stride` ints each
-    const v4i ss = *reinterpret_cast<const v4i *>(cst + stride + c);
-    if (fast) {
-        const v4i ls = *reinterpret_cast<const v4i *>(cst + 2 * stride + c);
-        return pack_fast4<true>(acc, ls, ss, floor_pk);
-    }
-    int q[4];
-#pragma unroll
-    for (int r = 0; r < 4; r++)
-        q[r] = requant_s8(acc[r], ss[r], relu, half_even);
-    return pack4_s8(q[0], q[1], q[2], q[3]);
-}
-
-// Fill one stage's constant table [init | shift | lsh] for `n` channels (padded to `stride`), and
-// decide whether the short epilogue is valid for all of them.  Returns the flag; contains barriers.
-__device__ __forceinline__ bool mb_fill_consts(int *cst, int stride, int n, const int32_t *bias, const int32_t *shift,
-                                               int n_shift, long long mac_bound, bool half_even, int tid)
-{
-    int ok_local = half_even ? 0 : 1;
-    for (int c = tid; c < n; c += kThreads) {
-        const int s = shift[n_shift == 1 ? 0 : c];
-        const long long bv = bias != nullptr ? (long long)bias[c] : 0;
-        if (s < 1 || s > 31) {
-            ok_local = 0;
-        } else {
-            const long long start = bv + (1ll << (s - 1));
-            if ((start < 0 ? -start : start) + mac_bound >= (1ll << (31 - max(0, 8 - s))))
-                ok_local = 0;
-        }
-    }
-    const bool fast = __syncthreads_and(ok_local) != 0;
-    for (int c = tid; c < stride; c += kThreads) {
-        int s = 0, bv = 0;
-        if (c < n) {
-            s = shift[n_shift == 1 ? 0 : c];
-            bv = bias != nullptr ? bias[c] : 0;
-        }
-        cst[c] = (fast && c < n) ? bv + (1 << (s - 1)) : bv;
-        cst[stride + c] = fast ? max(0, s - 8) : s;
-        cst[2 * stride + c] = fast ? max(0, 8 - s) : 0;
-    }
-    return fast;
-}
-
-// Filter units of one chunk: global -> registers.
-__device__ __forceinline__ void mb_fetch_weights(const MbArgs &a, int chunk, int tid, v4i (&we)[kMaxWe],
-                                                 v4i (&wp)[kMaxWp])
-{
-    const MbconvParams &p = a.p;
-    const int e0 = chunk * 64;
-    const int ng = min(4, (p.exp_c - e0) >> 4);
-    if (a.has_expand) {
-        // unit u = (ks * ng + t) * 64 + lane: row i of tile t is channel e0 + 4*ng*(i/4) + 4*t + i%4,
-        // the lane's 16 k positions are input channels 64*ks + 16*gk ...
-#pragma unroll
-        for (int j = 0; j < kMaxWe; j++) {
-            const int u = tid + j * kThreads;
-            we[j] = v4i{0, 0, 0, 0};
-            if (u < a.kse * ng * 64) {
-                const int lane = u & 63, t = (u >> 6) % ng, ks = (u >> 6) / ng;
-                const int i = lane & 15, gk = lane >> 4;
-                const int ch = e0 + 4 * ng * (i >> 2) + 4 * t + (i & 3);
-                const int k0 = 64 * ks + 16 * gk;
-                const int8_t *src = p.w_expand + (long long)ch * p.in_c + k0;
-                if (a.in_vec == 16) {
-                    if (k0 < p.in_c)
-                        we[j] = *reinterpret_cast<const v4i *>(src);
-                } else {
-#pragma unroll
-                    for (int d = 0; d < 4; d++)
-                        if (k0 + 4 * d < p.in_c)
-                            we[j][d] = *reinterpret_cast<const int *>(src + 4 * d);
-                }
-            }
-        }
-    }
-    // project: unit u = rt * 64 + lane: row i is filter 16*rt + i, k positions are expanded channels
-    // e0 + 16*gk ... (zeros past exp_c and past out_c)
-#pragma unroll
-    for (int j = 0; j < kMaxWp; j++) {
-        const int u = tid + j * kThreads;
-        wp[j] = v4i{0, 0, 0, 0};
-        if (u < a.nrt * 64) {
-            const int lane = u & 63, rt = u >> 6;
-            const int f = 16 * rt + (lane & 15), e = e0 + 16 * (lane >> 4);
-            if (f < p.out_c && e < p.exp_c)
-                wp[j] = *reinterpret_cast<const v4i *>(p.w_project + (long long)f * p.exp_c + e);
-        }
-    }
-}
-
-__device__ __forceinline__ void mb_store_weights(const MbArgs &a, int chunk, int tid, unsigned char *smem,
-                                                 const v4i (&we)[kMaxWe], const v4i (&wp)[kMaxWp])
-{
-    const int ng = min(4, (a.p.exp_c - chunk * 64) >> 4);
-    if (a.has_expand) {
-#pragma unroll
-        for (int j = 0; j < kMaxWe; j++) {
-            const int u = tid + j * kThreads;
-            if (u < a.kse * ng * 64)
-                *reinterpret_cast<v4i *>(smem + a.off_we + 16 * u) = we[j];
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < kMaxWp; j++) {
-        const int u = tid + j * kThreads;
-        if (u < a.nrt * 64)
-            *reinterpret_cast<v4i *>(smem + a.off_wp + 16 * u) = wp[j];
-    }
-}
-
 // Requantize four accumulators with the stage constants held in registers.
 __device__ __forceinline__ int mb_pack_r(const v4i &acc, const v4i &ss, const v4i &ls, bool fast, bool relu,
                                          bool half_even, int floor_pk)
@@ -211,41 +99,108 @@ __device__ __forceinline__ int mb_pack_r(const v4i &acc, const v4i &ss, const v4
     return pack4_s8(q[0], q[1], q[2], q[3]);
 }
 
-constexpr int kMaxCtE = 12; // expand column tiles per wavefront (two wavefronts share a row tile)
-constexpr int kMaxCtD = 8;  // depthwise column tiles per wavefront (two wavefronts share a channel group)
-constexpr int kAccBatch = 5;
+// Is the short epilogue valid for this channel?  (shift in 1..31, no overflow of the start value plus
+// the largest possible sum of products, also after the left shift the short form may apply)
+__device__ __forceinline__ bool mb_short_ok(int s, int bias, long long mac_bound)
+{
+    if (s < 1 || s > 31)
+        return false;
+    const long long start = (long long)bias + (1ll << (s - 1));
+    return (start < 0 ? -start : start) + mac_bound < (1ll << (31 - max(0, 8 - s)));
+}
 
-__global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbArgs a)
+__device__ __forceinline__ void mb_put_consts(int *cst, int stride, int c, bool valid, bool fast, int s, int b)
+{
+    cst[c] = (fast && valid) ? b + (1 << (s - 1)) : b;
+    cst[stride + c] = fast ? max(0, s - 8) : s;
+    cst[2 * stride + c] = fast ? max(0, 8 - s) : 0;
+}
+
+// Operand A of the expand stage for one chunk, straight from the filter: row i of row tile `sub` is
+// channel e0 + 4*ng*(i/4) + 4*sub + i%4 (so that a lane ends up with 4 consecutive channels per row
+// tile and 4*ng consecutive channels over the row tiles); the lane's 16 k positions are input channels
+// 64*ks + 16*gk ... (zeros past in_c).
+__device__ __forceinline__ void mb_load_we(const MbArgs &a, int chunk, int sub, int lane, v4i (&aop)[kMaxKse])
+{
+    const MbconvParams &p = a.p;
+    const int e0 = chunk * 64;
+    const int ng = min(4, (p.exp_c - e0) >> 4);
+    const int i = lane & 15, gk = lane >> 4;
+#pragma unroll
+    for (int ks = 0; ks < kMaxKse; ks++) {
+        aop[ks] = v4i{0, 0, 0, 0};
+        if (ks < a.kse && sub < ng) {
+            const int ch = e0 + 4 * ng * (i >> 2) + 4 * sub + (i & 3);
+            const int k0 = 64 * ks + 16 * gk;
+            const int8_t *src = p.w_expand + (long long)ch * p.in_c + k0;
+            if (k0 < p.in_c) // in_c % 16 == 0: the 16 positions are all inside or all outside
+                aop[ks] = *reinterpret_cast<const v4i *>(src);
+        }
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void mbconv_s8_fused_kernel(const MbArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const MbconvParams &p = a.p;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 15, quad = lane >> 4;
-    const int sub = wave & 3, half = wave >> 2; // row tile / channel group of this wavefront, and which half of the columns
+    const int sub = wave & 3, part = wave >> 2; // row tile / channel group, and which share of the column tiles
     const bool half_even = p.half_even != 0;
-    const int ec_pad = a.n_chunks * 64; // expanded channels padded to whole chunks
+    const int ec_pad = a.n_chunks * 64;
     const int oc_pad = a.nrt * 16;
 
     int *cst_e = reinterpret_cast<int *>(smem + a.off_ce); // [3][ec_pad]
     int *cst_d = reinterpret_cast<int *>(smem + a.off_cd); // [3][ec_pad]
     int *cst_p = reinterpret_cast<int *>(smem + a.off_cp); // [3][oc_pad]
     int *pixtab = reinterpret_cast<int *>(smem + a.off_pixtab);
+    int *rctab = reinterpret_cast<int *>(smem + a.off_rctab);
     unsigned char *x_l = smem + a.off_x;
-    unsigned char *e_l = smem + a.off_e;
     unsigned char *d_l = smem + a.off_d;
     unsigned char *out_l = smem + a.off_out;
 
-    // ---- once per workgroup: constants of the three stages, depthwise filter, pixel table
-    bool fast_e = false;
-    if (a.has_expand)
-        fast_e = mb_fill_consts(cst_e, ec_pad, p.exp_c, p.b_expand, p.s_expand, p.n_s_expand,
-                                (long long)p.in_c * 16384, half_even, tid);
-    const bool fast_d = mb_fill_consts(cst_d, ec_pad, p.exp_c, p.b_dw, p.s_dw, p.n_s_dw, (long long)a.taps * 16384,
-                                       half_even, tid);
-    const bool fast_p = mb_fill_consts(cst_p, oc_pad, p.out_c, p.b_project, p.s_project, p.n_s_project,
-                                       (long long)p.exp_c * 16384, half_even, tid);
-    for (int i = tid; i < a.taps * p.exp_c; i += kThreads)
-        smem[a.off_wd + i] = (unsigned char)p.w_dw[i];
+    // ---- once per workgroup.  Every thread owns one expanded channel (exp_c <= 1024) and one output
+    // channel: one round of global reads, then the three "short epilogue valid" votes.
+    bool fast_e, fast_d, fast_p;
+    {
+        int s_e = 0, b_e = 0, s_d = 0, b_d = 0, s_p = 0, b_p = 0;
+        int bad = 0;
+        if (tid < p.exp_c) {
+            if (a.has_expand) {
+                s_e = p.s_expand[p.n_s_expand == 1 ? 0 : tid];
+                b_e = p.b_expand != nullptr ? p.b_expand[tid] : 0;
+            }
+            s_d = p.s_dw[p.n_s_dw == 1 ? 0 : tid];
+            b_d = p.b_dw != nullptr ? p.b_dw[tid] : 0;
+        }
+        if (tid < p.out_c) {
+            s_p = p.s_project[p.n_s_project == 1 ? 0 : tid];
+            b_p = p.b_project != nullptr ? p.b_project[tid] : 0;
+        }
+        for (int i = tid; i < a.taps * p.exp_c; i += kThreads)
+            smem[a.off_wd + i] = (unsigned char)p.w_dw[i];
+        if (tid < p.exp_c) {
+            if (a.has_expand && !mb_short_ok(s_e, b_e, (long long)p.in_c * 16384))
+                bad |= 1;
+            if (!mb_short_ok(s_d, b_d, (long long)a.taps * 16384))
+                bad |= 2;
+        }
+        if (tid < p.out_c && !mb_short_ok(s_p, b_p, (long long)p.exp_c * 16384))
+            bad |= 4;
+        if (half_even)
+            bad = 7;
+        // the vote is a logical OR of a predicate, so one vote per stage
+        fast_e = __syncthreads_or(bad & 1) == 0;
+        fast_d = __syncthreads_or(bad & 2) == 0;
+        fast_p = __syncthreads_or(bad & 4) == 0;
+        if (tid < ec_pad) {
+            if (a.has_expand)
+                mb_put_consts(cst_e, ec_pad, tid, tid < p.exp_c, fast_e, s_e, b_e);
+            mb_put_consts(cst_d, ec_pad, tid, tid < p.exp_c, fast_d, s_d, b_d);
+        }
+        if (tid < oc_pad)
+            mb_put_consts(cst_p, oc_pad, tid, tid < p.out_c, fast_p, s_p, b_p);
+    }
     // the depthwise stage reads from E (stride kEs) or, without expand, from the input patch (stride xs)
     const int dw_stride = a.has_expand ? kEs : a.xs;
     for (int q = tid; q < a.nct_out * 16; q += kThreads) {
@@ -257,15 +212,7 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
         }
         pixtab[q] = off;
     }
-    // project accumulator tile t -> (row tile | column tile << 8); read back inside the loops so that
-    // the per-tile addresses are formed where they are used instead of living in registers throughout
-    int *slottab = reinterpret_cast<int *>(smem + a.off_slottab);
-    for (int t = tid; t < kMaxAcc * kWaves; t += kThreads) {
-        const int rt = (int)fastdiv((unsigned)t, a.fd_nct_out);
-        slottab[t] = t < a.n_acc ? (rt | ((t - rt * a.nct_out) << 8)) : 0;
-    }
     // (row | col << 16) of every patch pixel, -1 past the patch
-    int *rctab = reinterpret_cast<int *>(smem + a.off_rctab);
     for (int q = tid; q < a.nct_in * 16; q += kThreads) {
         int rc = -1;
         if (q < a.p_in) {
@@ -287,18 +234,25 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
     const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
     const int floor_d = p.relu_dw ? 0 : (int)0x80008000u;
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
-    __syncthreads();
-    // patch pixel (row | col << 16) of this lane in each of the wavefront's expand column tiles
-    // is recomputed per tile into a bit mask of the pixels that lie inside the image
 
     const TileSeq seq = xcd_tile_sequence(a.n_units);
     for (int unit = seq.first; unit < seq.end; unit += seq.step) {
         const TilePos u = mb_tile(a, unit);
         const int iy0 = u.y0 * p.stride_h - p.pad_top, ix0 = u.x0 * p.stride_w - p.pad_left;
+        // Lane and wavefront ids pass through an opaque copy once per tile: everything derived from
+        // them below (operand addresses, accumulator-tile assignment) is then formed where it is used
+        // instead of being hoisted out of the tile loop and held in registers throughout.
+        int lane_t = lane, wave_v = wave;
+        asm volatile("" : "+v"(lane_t), "+v"(wave_v));
+        const int wave = __builtin_amdgcn_readfirstlane(wave_v);
+        const int lane = lane_t;
+        const int col = lane & 15, quad = lane >> 4;
+        const int sub = wave & 3, part = wave >> 2;
 
-        // ---- filters of chunk 0 on their way while the patch is copied
-        v4i we_r[kMaxWe], wp_r[kMaxWp];
-        mb_fetch_weights(a, 0, tid, we_r, wp_r);
+        // expand operands of chunk 0 are requested before the patch copy
+        v4i we_cur[kMaxKse];
+        if (a.has_expand)
+            mb_load_we(a, 0, sub, lane, we_cur);
 
         // ---- 1. input patch -> LDS (zeros outside the image)
         {
@@ -313,88 +267,70 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
                 const bool ok = (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
                 const int8_t *src = base + ((long long)py * p.in_w + px) * p.in_c + v * a.in_vec;
                 unsigned char *dst = x_l + pix * a.xs + v * a.in_vec;
-                if (a.in_vec == 16)
-                    *reinterpret_cast<v4i *>(dst) = ok ? *reinterpret_cast<const v4i *>(src) : v4i{0, 0, 0, 0};
-                else
-                    *reinterpret_cast<int *>(dst) = ok ? *reinterpret_cast<const int *>(src) : 0;
+                *reinterpret_cast<v4i *>(dst) = ok ? *reinterpret_cast<const v4i *>(src) : v4i{0, 0, 0, 0};
             }
         }
-        // ---- project accumulators start at bias (+ rounding constant)
-        v4i acc[kMaxAcc];
+        __syncthreads(); // patch (and, first tile, the tables) visible
+
+        // ---- 2. chunks of 64 expanded channels.  Pipeline: iteration c runs expand(c) and
+        // depthwise(c - 1), which touch different E buffers; one barrier per iteration.
+        for (int chunk = 0; chunk <= a.n_chunks; chunk++) {
+            if (a.has_expand && chunk < a.n_chunks) {
+                const int e0 = chunk * 64;
+                const int ng = min(4, (p.exp_c - e0) >> 4);
+                v4i aop[kMaxKse];
 #pragma unroll
-        for (int s = 0; s < kMaxAcc; s++) {
-            const int t = wave + s * kWaves;
-            if (t < a.n_acc) {
-                const int rt = slottab[t] & 0xff;
-                acc[s] = *reinterpret_cast<const v4i *>(cst_p + 16 * rt + 4 * quad);
-            }
-        }
-
-        for (int chunk = 0; chunk < a.n_chunks; chunk++) {
-            const int e0 = chunk * 64;
-            const int ng = min(4, (p.exp_c - e0) >> 4);
-            // the previous chunk's project reads of D and of the filters, and (chunk 0) the previous
-            // tile's output copy, are finished before the filters are overwritten
-            __syncthreads();
-            mb_store_weights(a, chunk, tid, smem, we_r, wp_r);
-            __syncthreads();
-            if (chunk + 1 < a.n_chunks)
-                mb_fetch_weights(a, chunk + 1, tid, we_r, wp_r); // in flight during this chunk's stages
-
-            // ---- 2a. expand: this wavefront owns row tile `sub` (channels e0 + 4*ng*q + 4*sub + r of
-            // lane quad q) and every second column tile; E[patch pixel][4*ng*q + 4*sub + r]
-            if (a.has_expand) {
+                for (int ks = 0; ks < kMaxKse; ks++)
+                    aop[ks] = we_cur[ks];
+                if (chunk + 1 < a.n_chunks)
+                    mb_load_we(a, chunk + 1, sub, lane, we_cur); // in flight during this chunk
                 if (sub < ng) {
                     const int c = e0 + 4 * ng * quad + 4 * sub;
                     const v4i init = *reinterpret_cast<const v4i *>(cst_e + c);
                     const v4i ss = *reinterpret_cast<const v4i *>(cst_e + ec_pad + c);
                     const v4i ls = *reinterpret_cast<const v4i *>(cst_e + 2 * ec_pad + c);
-                    v4i aop[kMaxKse];
-#pragma unroll
-                    for (int ks = 0; ks < kMaxKse; ks++)
-                        if (ks < a.kse)
-                            aop[ks] = *reinterpret_cast<const v4i *>(smem + a.off_we + 16 * ((ks * ng + sub) * 64 + lane));
                     const unsigned char *bsrc = x_l + col * a.xs + 16 * quad;
-                    unsigned char *dst = e_l + col * kEs + 4 * ng * quad + 4 * sub;
+                    unsigned char *dst = smem + a.off_e + (chunk & 1) * (a.nct_in * 16 * kEs) + col * kEs + 4 * ng * quad + 4 * sub;
                     v4i b[kMaxKse];
+                    int rc = -1;
+                    if (part < a.nct_in) {
 #pragma unroll
-                    for (int ks = 0; ks < kMaxKse; ks++)
-                        if (ks < a.kse)
-                            b[ks] = *reinterpret_cast<const v4i *>(bsrc + half * 16 * a.xs + 64 * ks);
+                        for (int ks = 0; ks < kMaxKse; ks++)
+                            if (ks < a.kse)
+                                b[ks] = *reinterpret_cast<const v4i *>(bsrc + part * 16 * a.xs + 64 * ks);
+                        rc = rctab[part * 16 + col];
+                    }
 #pragma unroll 1
-                    for (int s = 0; s < kMaxCtE; s++) {
-                        const int ct = half + 2 * s;
-                        if (ct >= a.nct_in) // uniform per wavefront
-                            break;
-                        {
-                            v4i r = init;
+                    for (int ct = part; ct < a.nct_in; ct += kParts) {
+                        v4i r = init;
+#pragma unroll
+                        for (int ks = 0; ks < kMaxKse; ks++)
+                            if (ks < a.kse)
+                                r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], r, 0, 0, 0);
+                        const int rc_cur = rc;
+                        if (ct + kParts < a.nct_in) {
 #pragma unroll
                             for (int ks = 0; ks < kMaxKse; ks++)
                                 if (ks < a.kse)
-                                    r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], r, 0, 0, 0);
-                            if (ct + 2 < a.nct_in) {
-#pragma unroll
-                                for (int ks = 0; ks < kMaxKse; ks++)
-                                    if (ks < a.kse)
-                                        b[ks] = *reinterpret_cast<const v4i *>(bsrc + (ct + 2) * 16 * a.xs + 64 * ks);
-                            }
-                            const int word = mb_pack_r(r, ss, ls, fast_e, p.relu_expand != 0, half_even, floor_e);
-                            // outside the image the expanded activation is the depthwise zero padding
-                            const int rc = rctab[ct * 16 + col];
-                            const int iy = iy0 + (rc & 0xffff), ix = ix0 + (rc >> 16);
-                            const bool inside = rc >= 0 && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
-                            *reinterpret_cast<int *>(dst + ct * 16 * kEs) = inside ? word : 0;
+                                    b[ks] = *reinterpret_cast<const v4i *>(bsrc + (ct + kParts) * 16 * a.xs + 64 * ks);
+                            rc = rctab[(ct + kParts) * 16 + col];
                         }
+                        const int word = mb_pack_r(r, ss, ls, fast_e, p.relu_expand != 0, half_even, floor_e);
+                        // outside the image the expanded activation is the depthwise zero padding
+                        const int iy = iy0 + (rc_cur & 0xffff), ix = ix0 + (rc_cur >> 16);
+                        const bool inside = rc_cur >= 0 && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
+                        *reinterpret_cast<int *>(dst + ct * 16 * kEs) = inside ? word : 0;
                     }
                 }
-                __syncthreads();
             }
-
-            // ---- 2b. depthwise: this wavefront owns channel group `sub` and every second column tile;
-            // D[tile pixel][16*sub + 4*q + r]
-            {
-                if (sub < ng) {
-                    const unsigned char *src_l = (a.has_expand ? e_l : x_l + e0) + 16 * sub;
+            // depthwise of the previous chunk (with expand) / of this chunk (without)
+            const int dchunk = a.has_expand ? chunk - 1 : chunk;
+            if (dchunk >= 0 && dchunk < a.n_chunks) {
+                const int e0 = dchunk * 64;
+                const int ng = min(4, (p.exp_c - e0) >> 4);
+                if (sub < ng && part < a.nct_out) {
+                    const unsigned char *src_l = (a.has_expand ? smem + a.off_e + (dchunk & 1) * (a.nct_in * 16 * kEs)
+                                                               : x_l + e0) + 16 * sub;
                     const int sel = col >> 2;
                     v4i aop[kKsDw];
 #pragma unroll
@@ -409,76 +345,96 @@ __global__ __launch_bounds__(kThreads, 2) void mbconv_s8_fused_kernel(const MbAr
                     const v4i init = *reinterpret_cast<const v4i *>(cst_d + c);
                     const v4i ss = *reinterpret_cast<const v4i *>(cst_d + ec_pad + c);
                     const v4i ls = *reinterpret_cast<const v4i *>(cst_d + 2 * ec_pad + c);
-                    unsigned char *dst = d_l + col * kEs + 16 * sub + 4 * quad;
+                    unsigned char *dst = d_l + col * a.ds + c;
                     v4i b[kKsDw];
                     {
-                        const int po = pixtab[min(half, a.nct_out - 1) * 16 + col];
+                        const int po = pixtab[part * 16 + col];
 #pragma unroll
                         for (int ks = 0; ks < kKsDw; ks++)
                             b[ks] = *reinterpret_cast<const v4i *>(src_l + po + tapoff[ks]);
                     }
-                    // patch offset of the lane's pixel in the column tile after this one (two ahead of the reads)
-                    int po_next = pixtab[min(half + 2, a.nct_out - 1) * 16 + col];
+                    int po_next = pixtab[min(part + kParts, a.nct_out - 1) * 16 + col];
 #pragma unroll 1
-                    for (int s = 0; s < kMaxCtD; s++) {
-                        const int ct = half + 2 * s;
-                        if (ct >= a.nct_out) // uniform per wavefront
-                            break;
-                        {
-                            v4i r = init;
+                    for (int ct = part; ct < a.nct_out; ct += kParts) {
+                        v4i r = init;
+#pragma unroll
+                        for (int ks = 0; ks < kKsDw; ks++)
+                            if (4 * ks < a.taps)
+                                r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], r, 0, 0, 0);
+                        if (ct + kParts < a.nct_out) {
 #pragma unroll
                             for (int ks = 0; ks < kKsDw; ks++)
-                                if (4 * ks < a.taps)
-                                    r = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], r, 0, 0, 0);
-                            if (ct + 2 < a.nct_out) {
-#pragma unroll
-                                for (int ks = 0; ks < kKsDw; ks++)
-                                    b[ks] = *reinterpret_cast<const v4i *>(src_l + po_next + tapoff[ks]);
-                                po_next = pixtab[min(ct + 4, a.nct_out - 1) * 16 + col];
-                            }
-                            const int word = mb_pack_r(r, ss, ls, fast_d, p.relu_dw != 0, half_even, floor_d);
-                            *reinterpret_cast<int *>(dst + ct * 16 * kEs) = word;
+                                b[ks] = *reinterpret_cast<const v4i *>(src_l + po_next + tapoff[ks]);
+                            po_next = pixtab[min(ct + 2 * kParts, a.nct_out - 1) * 16 + col];
                         }
+                        const int word = mb_pack_r(r, ss, ls, fast_d, p.relu_dw != 0, half_even, floor_d);
+                        *reinterpret_cast<int *>(dst + ct * 16 * a.ds) = word;
                     }
                 }
-                __syncthreads();
             }
-
-            // ---- 2c. project: acc[rt][ct] += Wp[rt][chunk] x D[ct]; operands of a batch of tiles are
-            // all requested before the first MFMA of the batch
-#pragma unroll
-            for (int s0 = 0; s0 < kMaxAcc; s0 += kAccBatch) {
-                if (wave + s0 * kWaves < a.n_acc) { // uniform per wavefront
-                    v4i aop[kAccBatch], b[kAccBatch];
-#pragma unroll
-                    for (int j = 0; j < kAccBatch; j++) {
-                        const int t = wave + (s0 + j) * kWaves;
-                        if (t < a.n_acc) {
-                            const int e = slottab[t];
-                            const int rt = e & 0xff, ct = e >> 8;
-                            aop[j] = *reinterpret_cast<const v4i *>(smem + a.off_wp + 16 * (rt * 64 + lane));
-                            b[j] = *reinterpret_cast<const v4i *>(d_l + (ct * 16 + col) * kEs + 16 * quad);
-                        }
-                    }
-#pragma unroll
-                    for (int j = 0; j < kAccBatch; j++)
-                        if (wave + (s0 + j) * kWaves < a.n_acc)
-                            acc[s0 + j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[j], b[j], acc[s0 + j], 0, 0, 0);
-                }
-            }
+            __syncthreads();
         }
 
-        // ---- 3. project epilogue -> LDS tile (aliases the patch / E / D area) -> global
-        __syncthreads();
+        // ---- 3. project: acc[rt][ct] = sum over all expanded channels, operand A from global memory,
+        // one k step ahead
+        {
+            v4i acc[kMaxAcc];
+            int arow[kMaxAcc], boff[kMaxAcc];
 #pragma unroll
-        for (int s = 0; s < kMaxAcc; s++) {
-            const int t = wave + s * kWaves;
-            if (t < a.n_acc) {
-                const int e = slottab[t];
-                const int rt = e & 0xff, ct = e >> 8;
-                const int c = 16 * rt + 4 * quad;
-                const int word = mb_pack(acc[s], cst_p, oc_pad, c, fast_p, p.relu_project != 0, half_even, floor_p);
-                *reinterpret_cast<int *>(out_l + (ct * 16 + col) * a.os + c) = word;
+            for (int s = 0; s < kMaxAcc; s++) {
+                const int t = min(wave + s * kWaves, a.n_acc - 1);
+                const int rt = (int)fastdiv((unsigned)t, a.fd_nct_out);
+                const int ct = t - rt * a.nct_out;
+                arow[s] = 16 * rt + col; // filter of this lane's row
+                boff[s] = (ct * 16 + col) * a.ds + 16 * quad;
+                acc[s] = *reinterpret_cast<const v4i *>(cst_p + 16 * rt + 4 * quad);
+            }
+            auto load_wp = [&](int ks, v4i(&w)[kMaxAcc]) {
+#pragma unroll
+                for (int s = 0; s < kMaxAcc; s++) {
+                    w[s] = v4i{0, 0, 0, 0};
+                    const int e = 64 * ks + 16 * quad;
+                    if (wave + s * kWaves < a.n_acc && arow[s] < p.out_c && e < p.exp_c)
+                        w[s] = *reinterpret_cast<const v4i *>(p.w_project + (long long)arow[s] * p.exp_c + e);
+                }
+            };
+            v4i wa[kMaxAcc], wb[kMaxAcc];
+            load_wp(0, wa);
+#pragma unroll 1
+            for (int ks = 0; ks < a.ksp; ks += 2) {
+                if (ks + 1 < a.ksp)
+                    load_wp(ks + 1, wb);
+#pragma unroll
+                for (int s = 0; s < kMaxAcc; s++)
+                    if (wave + s * kWaves < a.n_acc) {
+                        const v4i b = *reinterpret_cast<const v4i *>(d_l + boff[s] + 64 * ks);
+                        acc[s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa[s], b, acc[s], 0, 0, 0);
+                    }
+                if (ks + 1 < a.ksp) {
+                    if (ks + 2 < a.ksp)
+                        load_wp(ks + 2, wa);
+#pragma unroll
+                    for (int s = 0; s < kMaxAcc; s++)
+                        if (wave + s * kWaves < a.n_acc) {
+                            const v4i b = *reinterpret_cast<const v4i *>(d_l + boff[s] + 64 * (ks + 1));
+                            acc[s] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wb[s], b, acc[s], 0, 0, 0);
+                        }
+                }
+            }
+            // ---- 4. epilogue -> LDS tile.  It aliases the patch / E area, which nobody reads after the
+            // last barrier of step 2.
+#pragma unroll
+            for (int s = 0; s < kMaxAcc; s++) {
+                const int t = wave + s * kWaves;
+                if (t < a.n_acc) {
+                    const int rt = (int)fastdiv((unsigned)t, a.fd_nct_out);
+                    const int ct = t - rt * a.nct_out;
+                    const int c = 16 * rt + 4 * quad;
+                    const v4i ss = *reinterpret_cast<const v4i *>(cst_p + oc_pad + c);
+                    const v4i ls = *reinterpret_cast<const v4i *>(cst_p + 2 * oc_pad + c);
+                    const int word = mb_pack_r(acc[s], ss, ls, fast_p, p.relu_project != 0, half_even, floor_p);
+                    *reinterpret_cast<int *>(out_l + (ct * 16 + col) * a.os + c) = word;
+                }
             }
         }
         __syncthreads();
@@ -563,7 +519,8 @@ MbPlan mb_plan(const MbconvParams &p)
     MbPlan best;
     best.ok = false;
     const bool has_expand = p.w_expand != nullptr;
-    if ((p.exp_c & 15) != 0 || (p.in_c & 3) != 0 || (p.out_c & 3) != 0 || p.k_h * p.k_w > 4 * kKsDw)
+    if ((p.exp_c & 15) != 0 || (p.in_c & 15) != 0 || (p.out_c & 3) != 0 || p.k_h * p.k_w > 4 * kKsDw ||
+        p.exp_c > kThreads || p.out_c > 384 || (reinterpret_cast<uintptr_t>(p.w_project) & 15) != 0)
         return best;
     if (!has_expand && (p.in_c != p.exp_c))
         return best;
@@ -590,8 +547,9 @@ MbPlan mb_plan(const MbconvParams &p)
             a.p_out = a.th * a.tw;
             a.nct_in = (a.p_in + 15) / 16;
             a.nct_out = (a.p_out + 15) / 16;
-            a.in_vec = (p.in_c & 15) == 0 && (reinterpret_cast<uintptr_t>(p.in) & 15) == 0 &&
-                    (!has_expand || (reinterpret_cast<uintptr_t>(p.w_expand) & 15) == 0) ? 16 : 4;
+            if ((reinterpret_cast<uintptr_t>(p.in) & 15) != 0 || (has_expand && (reinterpret_cast<uintptr_t>(p.w_expand) & 15) != 0))
+                continue;
+            a.in_vec = 16;
             a.out_vec = (p.out_c & 15) == 0 && (reinterpret_cast<uintptr_t>(p.out) & 15) == 0 &&
                     (p.residual == nullptr || (reinterpret_cast<uintptr_t>(p.residual) & 15) == 0) ? 16 : 4;
             a.in_vecs = p.in_c / a.in_vec;
@@ -599,29 +557,25 @@ MbPlan mb_plan(const MbconvParams &p)
             a.xs = odd16(p.in_c);
             a.kse = has_expand ? (p.in_c + 63) / 64 : 0;
             a.n_chunks = (p.exp_c + 63) / 64;
+            a.ksp = a.n_chunks;
+            a.ds = odd16(a.n_chunks * 64);
             a.nrt = (p.out_c + 15) / 16;
             a.n_acc = a.nrt * a.nct_out;
             a.os = odd16(a.nrt * 16);
-            if (a.nct_in > 2 * kMaxCtE || a.nct_out > 2 * kMaxCtD || a.n_acc > kMaxAcc * kWaves)
+            if (a.n_acc > kMaxAcc * kWaves || a.ph > 0xffff || a.pw > 0x7fff)
                 continue;
-            if (a.kse * 4 * 64 > kMaxWe * kThreads || a.nrt * 64 > kMaxWp * kThreads)
-                continue;
-            // LDS: [patch | E | D] (the output tile aliases this area), filters, tables
+            // LDS: [patch | E (two buffers)] (the output tile aliases this area), D, tables
             size_t off = 0;
             a.off_x = (int)off;
             off += (size_t)a.nct_in * 16 * a.xs + 64 * kMaxKse; // expand k padding may read past the last pixel
             a.off_e = (int)off;
             if (has_expand)
-                off += (size_t)a.nct_in * 16 * kEs + 64;
-            a.off_d = (int)off;
-            off += (size_t)a.nct_out * 16 * kEs;
+                off += (size_t)2 * a.nct_in * 16 * kEs + 64;
             a.off_out = 0;
             off = std::max(off, (size_t)a.nct_out * 16 * a.os);
             off = (off + 15) & ~(size_t)15;
-            a.off_we = (int)off;
-            off += (size_t)a.kse * 4 * 64 * 16;
-            a.off_wp = (int)off;
-            off += (size_t)a.nrt * 64 * 16;
+            a.off_d = (int)off;
+            off += (size_t)a.nct_out * 16 * a.ds + 64;
             a.off_wd = (int)off;
             off += ((size_t)a.taps * p.exp_c + 15) & ~(size_t)15;
             a.off_ce = (int)off;
@@ -635,20 +589,17 @@ MbPlan mb_plan(const MbconvParams &p)
             off += (size_t)a.nct_out * 16 * 4;
             a.off_rctab = (int)off;
             off += (size_t)a.nct_in * 16 * 4;
-            a.off_slottab = (int)off;
-            off += (size_t)kMaxAcc * kWaves * 4;
             if (off > lds_limit())
                 continue;
-            const int per_cu = off <= 80 * 1024 ? 2 : 1;
             a.tiles_y = (p.out_h + a.th - 1) / a.th;
             a.tiles_x = (p.out_w + a.tw - 1) / a.tw;
-            // cost per output pixel: expand work on the patch, depthwise and project on the padded
-            // tile, per-chunk filter staging and barriers amortized over the tile, edge waste
+            // work per output pixel: expand on the patch, depthwise and project on the padded tile, a
+            // fixed cost per chunk (barrier) and per tile, edge waste
             const double px = (double)a.p_out;
-            double cost = (has_expand ? 1.0 * a.nct_in * 16 * a.kse : 0.0) + 3.0 * a.nct_out * 16 + 0.3 * a.nct_out * 16 * a.nrt;
-            cost += 600.0; // barriers and filter staging per chunk, in the same unit
+            double cost = (has_expand ? 1.0 * a.nct_in * 16 * a.kse : 0.0) + 3.0 * a.nct_out * 16 +
+                0.3 * a.nct_out * 16 * a.nrt;
+            cost = cost * a.n_chunks + 300.0 * a.n_chunks + 1500.0;
             cost /= px;
-            cost *= per_cu == 2 ? 1.0 : 1.5;
             cost *= (double)(a.tiles_y * a.th) * (a.tiles_x * a.tw) / ((double)p.out_h * p.out_w);
             if (cost < best_cost) {
                 best_cost = cost;

@@ -142,8 +142,8 @@ int espdl_hip_requantize(const void *in, int32_t in_dtype, int64_t size, int32_t
  *   Filters use the layouts of espdl_hip_conv2d: expand [exp_c][in_c], depthwise [k_h][k_w][exp_c],
  *   project [out_c][exp_c]; biases int32 or NULL; shifts int32[1 or channels] per stage.
  *   residual: int8 tensor of the output's shape added with saturation after the project stage, or NULL.
- * Needs exp_c % 16 == 0, in_c % 4 == 0, out_c % 4 == 0, at most 12 depthwise taps, in_c <= 256,
- * out_c <= 384; espdl_hip_mbconv_s8_supported() answers for a descriptor: 0 = no, 1 = yes (general
+ * Needs exp_c % 16 == 0, in_c % 16 == 0, out_c % 4 == 0, at most 12 depthwise taps, in_c <= 192,
+ * exp_c <= 1024, out_c <= 384, 16-byte aligned input and filters; espdl_hip_mbconv_s8_supported() answers for a descriptor: 0 = no, 1 = yes (general
  * fused kernel), 2 = yes, through the depthwise+project kernel (no expand stage, at most 256
  * channels), which is the form that is faster than separate launches today.
  * espdl_hip_mbconv_s8 returns ESPDL_HIP_ENOTSUP where it does not apply.

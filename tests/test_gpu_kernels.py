@@ -348,7 +348,7 @@ def test_bad_arguments_are_rejected():
 # (name, (N, H, W, Cin), Ce (None = no expand stage), Cout, k, stride, pads, residual, half_even, per_tensor)
 MBCONV_CASES = [
     ("b8_14x14_64_384_64_res", (3, 14, 14, 64), 384, 64, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
-    ("b3_56x56_24_144_24_res", (2, 56, 56, 24), 144, 24, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
+    ("b3_56x56_32_144_24_res", (2, 56, 56, 32), 144, 24, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
     ("b2_40x40_16_96_24_s2", (2, 40, 40, 16), 96, 24, (3, 3), (2, 2), (1, 1, 1, 1), False, False, False),
     ("b1_30x30_32_noexp_16", (2, 30, 30, 32), None, 16, (3, 3), (1, 1), (1, 1, 1, 1), False, False, False),
     ("b17_7x7_160_960_320", (5, 7, 7, 160), 960, 320, (3, 3), (1, 1), (1, 1, 1, 1), False, False, False),
@@ -402,3 +402,33 @@ def test_mbconv_s8_fused(oracle, case):
     got = m.mbconv_s8(to_dev(x), dev(expand), dev(dw), dev(proj), k, stride, (1, 1), pads, (True, True, False),
                       residual=to_dev(res), round_mode=rm_g)
     np.testing.assert_array_equal(to_host(got), cur)
+
+
+@pytest.mark.parametrize("general_stage", [0, 1, 2], ids=["expand_general", "dw_general", "project_general"])
+def test_mbconv_s8_mixed_epilogues(oracle, general_stage):
+    """One stage has shifts outside 1..31 (general shift_and_round form), the other two take the
+    short epilogue: the per-stage choice must not leak between stages."""
+    announce(f"mbconv_s8 mixed epilogues, general stage {general_stage}")
+    m = espdl()
+    rng = np.random.default_rng(77 + general_stage)
+    n, h, w, cin, ce, cout = 2, 14, 14, 32, 320, 48
+    x = rng_int8(rng, (n, h, w, cin))
+
+    def stage(idx, oc, kk, fshape):
+        f = rng_int8(rng, fshape)
+        b = rng.integers(-4096, 4097, size=oc).astype(np.int32)
+        s = (typical_shift(kk) + rng.integers(-2, 3, size=oc)).astype(np.int32)
+        if idx == general_stage:
+            s[::7] = 0
+            s[3::11] = 33
+        return f, b, s
+
+    ex = stage(0, ce, cin, (ce, 1, 1, cin))
+    dw = stage(1, ce, 9, (3, 3, ce))
+    pj = stage(2, cout, ce, (cout, 1, 1, ce))
+    cur = oracle.conv2d_s8(x, ex[0], ex[1], ex[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.RELU)
+    cur = oracle.depthwise_s8(cur, dw[0], dw[1], dw[2], (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), oracle.RELU)
+    want = oracle.conv2d_s8(cur, pj[0], pj[1], pj[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.LINEAR)
+    dev = lambda t: tuple(to_dev(a) for a in t)  # noqa: E731
+    got = m.mbconv_s8(to_dev(x), dev(ex), dev(dw), dev(pj), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), (True, True, False))
+    np.testing.assert_array_equal(to_host(got), want)
