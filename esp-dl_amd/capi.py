@@ -55,6 +55,8 @@ def lib():
         dp = ctypes.POINTER(ConvDesc)
         L.espdl_hip_conv_out_shape.argtypes = [dp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
         L.espdl_hip_conv2d.argtypes = [dp, vp, vp, vp, vp, vp, vp, vp]
+        L.espdl_hip_conv2d_add.argtypes = [dp, vp, vp, vp, vp, vp, vp, vp, vp]
+        L.espdl_hip_conv2d_add.restype = ctypes.c_int
         L.espdl_hip_lut_s8.argtypes = [vp, i64, vp, vp, vp]
         L.espdl_hip_prelu_s8.argtypes = [vp, i64, i32, vp, i32, vp, vp]
         L.espdl_hip_relu_s8.argtypes = [vp, i64, i32, i32, vp, vp]
@@ -109,7 +111,7 @@ def conv_out_shape(desc):
 
 
 def conv2d(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), depthwise=False,
-           activation=LINEAR, round_mode=ROUND_HALF_UP, lut=None, out=None, stream=None):
+           activation=LINEAR, round_mode=ROUND_HALF_UP, lut=None, out=None, stream=None, residual=None):
     """x [N,H,W,C] int8|int16 CUDA tensor; filt dense [OC][kH][kW][C] or depthwise [kH][kW][C];
     bias int32|int64 [OC] or None; shift int32 tensor with 1 or OC entries (device)."""
     import torch
@@ -121,8 +123,8 @@ def conv2d(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 
     oh, ow = conv_out_shape(desc)
     if out is None:
         out = torch.empty((n, oh, ow, out_c), dtype=x.dtype, device=x.device)
-    _check(lib().espdl_hip_conv2d(ctypes.byref(desc), _p(x), _p(filt), _p(bias), _p(shift), _p(lut), _p(out),
-                                  _stream(stream)))
+    _check(lib().espdl_hip_conv2d_add(ctypes.byref(desc), _p(x), _p(filt), _p(bias), _p(shift), _p(lut), _p(residual),
+                                      _p(out), _stream(stream)))
     return out
 
 

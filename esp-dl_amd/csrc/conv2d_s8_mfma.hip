@@ -13,8 +13,8 @@ constexpr int kLdsPerWorkgroup = 64 * 1024; // dynamic LDS a workgroup may ask f
 } // namespace
 
 hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
-                                 const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
-                                 hipStream_t stream)
+                                 const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
+                                 int cu_count, hipStream_t stream)
 {
     MfmaConvArgs a;
     a.in = in;
@@ -22,6 +22,7 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     a.bias = bias;
     a.shift = shift;
     a.lut = lut;
+    a.res = residual;
     a.out = out;
     a.g = g;
     a.npix = (long long)g.batch * g.out_h * g.out_w;
@@ -50,7 +51,7 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     }
     a.ksteps = (a.K + 63) / 64;
     a.n_groups = (g.out_c + 63) / 64;
-    const uintptr_t out_addr = reinterpret_cast<uintptr_t>(out);
+    const uintptr_t out_addr = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(residual);
     a.out_vec = ((g.out_c & 15) == 0 && (out_addr & 15) == 0) ? 16 : (((g.out_c & 3) == 0 && (out_addr & 3) == 0) ? 4 : 1);
 
     // LDS plan: per resident filter group ksteps * 4 KiB of weights + 512 B of start values / shifts,
@@ -89,7 +90,7 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     a.n_sets = (int)((a.npix + 64 * pt - 1) / (64 * pt));
     // contiguous output: needs every filter group in one chunk, 4-byte aligned rows and room in LDS
     const size_t out_tiles = (size_t)4 * 16 * pt * g.out_c;
-    a.stage_out = (n_chunks == 1 && a.out_vec >= 4 && (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+    a.stage_out = (n_chunks == 1 && a.out_vec >= 4 && (out_addr & 15) == 0 &&
                    lds + out_tiles <= 40 * 1024) ? 1 : 0;
     if (a.stage_out)
         lds += out_tiles;

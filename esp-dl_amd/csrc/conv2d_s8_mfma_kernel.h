@@ -57,6 +57,7 @@ struct MfmaConvArgs {
     const int32_t *bias;
     const int32_t *shift;
     const int8_t *lut;
+    const int8_t *res; // tensor of the output's shape added with saturation to the stored value, or nullptr
     int8_t *out;
     ConvGeom g;
     int K;                // length of the reduction axis as the MFMA sees it (k_h * seg_pad for B_ROWSEG)
@@ -407,20 +408,36 @@ __device__ __forceinline__ void run_group(const MfmaConvArgs &a, const WaveCtx &
         }
         if (!px[p].valid)
             continue;
-        int8_t *dst = a.out + (long long)px[p].pix * OC + c_lane;
+        const long long goff = (long long)px[p].pix * OC + c_lane;
+        int8_t *dst = a.out + goff;
         if (NT == 4 && a.out_vec == 16) {
-            *reinterpret_cast<v4i *>(dst) = v4i{words[0], words[NT > 1 ? 1 : 0], words[NT > 2 ? 2 : 0], words[NT > 3 ? 3 : 0]};
+            v4i v = {words[0], words[NT > 1 ? 1 : 0], words[NT > 2 ? 2 : 0], words[NT > 3 ? 3 : 0]};
+            if (a.res != nullptr) {
+                const v4i r = *reinterpret_cast<const v4i *>(a.res + goff);
+#pragma unroll
+                for (int d = 0; d < 4; d++)
+                    v[d] = sat_add4_s8(v[d], r[d]);
+            }
+            *reinterpret_cast<v4i *>(dst) = v;
         } else if (a.out_vec >= 4) {
 #pragma unroll
             for (int t = 0; t < NT; t++)
-                if (c_lane + 4 * t < OC)
-                    *reinterpret_cast<int *>(dst + 4 * t) = words[t];
+                if (c_lane + 4 * t < OC) {
+                    int v = words[t];
+                    if (a.res != nullptr)
+                        v = sat_add4_s8(v, *reinterpret_cast<const int *>(a.res + goff + 4 * t));
+                    *reinterpret_cast<int *>(dst + 4 * t) = v;
+                }
         } else {
 #pragma unroll
             for (int t = 0; t < NT; t++)
                 for (int r = 0; r < 4; r++)
-                    if (c_lane + 4 * t + r < OC)
-                        dst[4 * t + r] = (int8_t)(words[t] >> (8 * r));
+                    if (c_lane + 4 * t + r < OC) {
+                        int v = (int)(int8_t)(words[t] >> (8 * r));
+                        if (a.res != nullptr)
+                            v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
+                        dst[4 * t + r] = (int8_t)v;
+                    }
         }
     }
 }
@@ -475,12 +492,22 @@ __device__ __forceinline__ void run_sets(const MfmaConvArgs &a, const WaveCtx &w
             int8_t *gdst = a.out + first;
             for (int off = w.lane * 16; off < tile_bytes; off += 64 * 16) {
                 if (first + off + 16 <= total) {
-                    const v4i v = *reinterpret_cast<const v4i *>(w.my_tile + off);
+                    v4i v = *reinterpret_cast<const v4i *>(w.my_tile + off);
+                    if (a.res != nullptr) {
+                        const v4i r = *reinterpret_cast<const v4i *>(a.res + first + off);
+#pragma unroll
+                        for (int d = 0; d < 4; d++)
+                            v[d] = sat_add4_s8(v[d], r[d]);
+                    }
                     *reinterpret_cast<v4i *>(gdst + off) = v;
                 } else {
                     for (int b = 0; b < 16; b++)
-                        if (first + off + b < total)
-                            gdst[off + b] = (int8_t)w.my_tile[off + b];
+                        if (first + off + b < total) {
+                            int v = (int)(int8_t)w.my_tile[off + b];
+                            if (a.res != nullptr)
+                                v = clamp_s8(v + (int)a.res[first + off + b]);
+                            gdst[off + b] = (int8_t)v;
+                        }
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");

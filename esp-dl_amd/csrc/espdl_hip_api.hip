@@ -140,6 +140,12 @@ int espdl_hip_conv_out_shape(const espdl_hip_conv_desc *desc, int32_t *out_h, in
 int espdl_hip_conv2d(const espdl_hip_conv_desc *desc, const void *in, const void *filter, const void *bias,
                      const int32_t *shift, const int8_t *lut, void *out, void *stream)
 {
+    return espdl_hip_conv2d_add(desc, in, filter, bias, shift, lut, nullptr, out, stream);
+}
+
+int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const void *filter, const void *bias,
+                         const int32_t *shift, const int8_t *lut, const int8_t *residual, void *out, void *stream)
+{
     espdl::ConvGeom g;
     const int rc = derive_geometry(desc, &g);
     if (rc != ESPDL_HIP_OK)
@@ -157,6 +163,8 @@ int espdl_hip_conv2d(const espdl_hip_conv_desc *desc, const void *in, const void
         const int8_t *f8 = static_cast<const int8_t *>(filter);
         const int32_t *b32 = static_cast<const int32_t *>(bias);
         int8_t *o8 = static_cast<int8_t *>(out);
+        if (residual != nullptr && depthwise)
+            return fail(ESPDL_HIP_ENOTSUP, "the fused residual Add exists for dense int8 convolutions only");
         if (depthwise) {
             if (espdl::depthwise_s8_lds_supports(g, in, out))
                 return device_status(espdl::launch_depthwise_s8_lds(g, i8, f8, b32, shift, lut, o8, cu_count_cached(), s),
@@ -166,11 +174,11 @@ int espdl_hip_conv2d(const espdl_hip_conv_desc *desc, const void *in, const void
                                      "depthwise_s8_mfma");
             return device_status(espdl::launch_depthwise_s8(g, i8, f8, b32, shift, lut, o8, s), "depthwise_s8");
         }
-        return device_status(espdl::launch_conv2d_s8_mfma(g, i8, f8, b32, shift, lut, o8, cu_count_cached(), s),
+        return device_status(espdl::launch_conv2d_s8_mfma(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
                              "conv2d_s8");
     }
-    if (lut != nullptr)
-        return fail(ESPDL_HIP_ENOTSUP, "the fused LUT epilogue exists for ESPDL_HIP_S8 only");
+    if (lut != nullptr || residual != nullptr)
+        return fail(ESPDL_HIP_ENOTSUP, "the fused LUT / residual epilogues exist for ESPDL_HIP_S8 only");
     if (misaligned(in, 2) || misaligned(filter, 2) || misaligned(out, 2) || misaligned(bias, 8) || misaligned(shift, 4))
         return fail(ESPDL_HIP_EINVAL, "int16 tensors must be 2-byte aligned, int64 bias 8-byte aligned");
     const int16_t *i16 = static_cast<const int16_t *>(in);

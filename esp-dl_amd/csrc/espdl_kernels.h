@@ -16,8 +16,8 @@ struct ConvGeom {
 
 // Dense int8 convolution / Gemm as an implicit GEMM on v_mfma_i32_16x16x64_i8.
 hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
-                                 const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count,
-                                 hipStream_t stream);
+                                 const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
+                                 int cu_count, hipStream_t stream);
 
 hipError_t launch_depthwise_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                const int32_t *shift, const int8_t *lut, int8_t *out, hipStream_t stream);

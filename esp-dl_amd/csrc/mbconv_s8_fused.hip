@@ -144,8 +144,7 @@ __global__ __launch_bounds__(kThreads) void mbconv_s8_fused_kernel(const MbArgs 
     extern __shared__ __align__(16) unsigned char smem[];
     const MbconvParams &p = a.p;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int col = lane & 15, quad = lane >> 4;
-    const int sub = wave & 3, part = wave >> 2; // row tile / channel group, and which share of the column tiles
+    const int quad = lane >> 4;
     const bool half_even = p.half_even != 0;
     const int ec_pad = a.n_chunks * 64;
     const int oc_pad = a.nrt * 16;

@@ -27,13 +27,15 @@ struct module_info {
     int64_t bytes;    ///< bytes of the tensors it reads and writes (each counted once)
 };
 
-enum { FUSE_CONV_LUT = 1, FUSE_DW_PROJECT = 2 };
+enum { FUSE_CONV_LUT = 1, FUSE_DW_PROJECT = 2, FUSE_CONV_ADD = 4 };
 
 class Model {
 public:
     /// The model does not take ownership of `fbs_model`.  `stream` is a hipStream_t (nullptr: the
     /// model creates its own).  `fuse` is a bit mask of graph fusions: FUSE_CONV_LUT folds a LUT that directly follows a Conv
-    /// into its epilogue, FUSE_DW_PROJECT runs depthwise Conv -> 1x1 Conv [-> Add] as one kernel.
+    /// into its epilogue, FUSE_DW_PROJECT runs depthwise Conv -> 1x1 Conv [-> Add] as one kernel,
+    /// FUSE_CONV_ADD folds the Add behind a dense Conv into its epilogue (off by default: measured
+    /// slightly slower than the separate Add kernel on MobileNetV2, whose residual tensors are small).
     Model(fbs::FbsModel *fbs_model, int batch = 1, round_mode_t round_mode = ROUND_MODE_HALF_UP, void *stream = nullptr,
           int fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT);
     virtual ~Model();
@@ -86,6 +88,7 @@ public:
 private:
     void fuse_conv_lut();
     void fuse_dw_project();
+    void fuse_conv_add();
 
     fbs::FbsModel *m_fbs_model = nullptr;
     std::vector<dl::module::Module *> m_execution_plan;

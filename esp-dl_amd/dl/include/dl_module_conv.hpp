@@ -46,6 +46,7 @@ private:
     activation_type_t m_project_activation = Linear;
     int m_mid_exponent = 0;      ///< exponent of the (no longer materialized) depthwise output
     int m_project_filter_pos = -1, m_project_bias_pos = -1, m_residual_pos = -1;
+    int m_own_inputs = 0; ///< inputs of the Conv itself when a plain residual Add was absorbed
     DeviceInts m_shift_project;
 
 public:
@@ -94,10 +95,18 @@ public:
             m_inputs_index.push_back(residual_index);
         }
     }
+    /// Absorb the Add that follows a dense Conv: `residual_index` is the Add's other operand.
+    void fuse_residual(int residual_index)
+    {
+        m_own_inputs = (int)m_inputs_index.size();
+        m_residual_pos = (int)m_inputs_index.size();
+        m_inputs_index.push_back(residual_index);
+    }
+    bool has_fused_residual() const { return m_residual_pos >= 0; }
     /// Position of the depthwise bias in m_inputs_index, or -1.
     int own_bias_pos() const
     {
-        const int own = m_has_project ? m_project_filter_pos : (int)m_inputs_index.size();
+        const int own = m_has_project ? m_project_filter_pos : (m_own_inputs > 0 ? m_own_inputs : (int)m_inputs_index.size());
         return own == 3 ? 2 : -1;
     }
 
@@ -209,9 +218,15 @@ public:
             delete m_fused_lut;
             m_fused_lut = dev;
         }
-        const int rc = espdl_hip_conv2d(&d, input->data, filter->data, bias ? bias->data : nullptr, shift_dev,
-                                        m_fused_lut ? static_cast<const int8_t *>(m_fused_lut->data) : nullptr,
-                                        output->data, context->stream);
+        TensorBase *residual = m_residual_pos >= 0 ? context->get_tensor(m_inputs_index[m_residual_pos]) : nullptr;
+        if (residual && !residual->on_device()) {
+            DL_LOGE("Conv", "%s: the residual must be a device tensor", name.c_str());
+            return;
+        }
+        const int rc = espdl_hip_conv2d_add(&d, input->data, filter->data, bias ? bias->data : nullptr, shift_dev,
+                                            m_fused_lut ? static_cast<const int8_t *>(m_fused_lut->data) : nullptr,
+                                            residual ? static_cast<const int8_t *>(residual->data) : nullptr, output->data,
+                                            context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("Conv", "%s: %s", name.c_str(), espdl_hip_last_error());
     }

@@ -183,6 +183,8 @@ esp_err_t Model::load(fbs::FbsModel *fbs_model)
         fuse_conv_lut();
     if (ret == ESP_OK && (m_fuse & FUSE_DW_PROJECT))
         fuse_dw_project();
+    if (ret == ESP_OK && (m_fuse & FUSE_CONV_ADD))
+        fuse_conv_add();
     return ret;
 }
 
@@ -335,6 +337,53 @@ void Model::fuse_dw_project()
         } else {
             delete pj;
         }
+        m_execution_plan.erase(m_execution_plan.begin() + i);
+        i--;
+    }
+}
+
+// dense Conv -> Add with no other reader of the conv output: the Add's other operand becomes the
+// conv's residual input and the conv writes the Add's output (espdl_hip_conv2d_add).  The fused module
+// takes the Add's place in the plan, so the other operand is produced before it.
+void Model::fuse_conv_add()
+{
+    std::set<std::string> pinned;
+    for (auto &n : m_fbs_model->get_graph_outputs())
+        pinned.insert(n);
+    for (auto &n : m_fbs_model->get_test_outputs_name())
+        pinned.insert(n);
+    for (size_t i = 0; i < m_execution_plan.size(); i++) {
+        auto *conv = dynamic_cast<dl::module::Conv *>(m_execution_plan[i]);
+        if (!conv || conv->quant_type != QUANT_TYPE_SYMM_8BIT || conv->get_group() != 1 || conv->has_fused_project() ||
+            conv->has_fused_residual())
+            continue;
+        const int mid = conv->m_outputs_index[0];
+        if (pinned.count(m_model_context->get_tensor_name(mid)))
+            continue;
+        int readers = 0;
+        size_t add_pos = 0;
+        for (size_t j = 0; j < m_execution_plan.size(); j++)
+            for (int in : m_execution_plan[j]->m_inputs_index)
+                if (in == mid) {
+                    readers++;
+                    add_pos = j;
+                }
+        if (readers != 1 || add_pos <= i)
+            continue;
+        auto *add = dynamic_cast<dl::module::Add *>(m_execution_plan[add_pos]);
+        if (!add || add->quant_type != QUANT_TYPE_SYMM_8BIT || add->m_inputs_index.size() != 2 ||
+            add->m_inputs_index[0] == add->m_inputs_index[1])
+            continue;
+        const int other = add->m_inputs_index[0] == mid ? add->m_inputs_index[1] : add->m_inputs_index[0];
+        const std::string other_name = m_model_context->get_tensor_name(other);
+        const std::string mid_name = m_model_context->get_tensor_name(mid);
+        if (other >= CONTEXT_PARAMETER_OFFSET || !m_fbs_model->has_value_info(other_name) ||
+            m_fbs_model->get_value_info_shape(other_name) != m_fbs_model->get_value_info_shape(mid_name))
+            continue;
+        conv->fuse_residual(other);
+        conv->m_outputs_index[0] = add->m_outputs_index[0];
+        delete add;
+        m_execution_plan[add_pos] = conv;
         m_execution_plan.erase(m_execution_plan.begin() + i);
         i--;
     }

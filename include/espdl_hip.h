@@ -87,6 +87,15 @@ int espdl_hip_conv_out_shape(const espdl_hip_conv_desc *desc, int32_t *out_h, in
 int espdl_hip_conv2d(const espdl_hip_conv_desc *desc, const void *in, const void *filter, const void *bias,
                      const int32_t *shift, const int8_t *lut, void *out, void *stream);
 
+/*
+ * espdl_hip_conv2d followed by base::elemwise_add of `residual` (esp-dl/dl/base/dl_base_add.cpp:34-44) in
+ * the same launch: out = clamp_int8(conv_result + residual), where conv_result is the int8 value
+ * espdl_hip_conv2d would have stored (after the optional LUT) and residual has the output's shape.
+ * Dense int8 convolutions only (group 1); residual == NULL is plain espdl_hip_conv2d.
+ */
+int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const void *filter, const void *bias,
+                         const int32_t *shift, const int8_t *lut, const int8_t *residual, void *out, void *stream);
+
 /* base::lut_s8 (esp-dl/dl/base/dl_base_lut.cpp:10-48): out[i] = table[(uint8)in[i] ^ 0x80]. In-place allowed. */
 int espdl_hip_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out, void *stream);
 

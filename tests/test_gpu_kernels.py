@@ -9,18 +9,23 @@ from gpu_util import announce, espdl, to_dev, to_host
 pytestmark = pytest.mark.gpu
 
 
-def _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, depthwise=False, half_even=False, lut=None):
+def _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, depthwise=False, half_even=False, lut=None,
+                 residual_seed=None):
     m = espdl()
     act = m.capi.RELU if relu else m.capi.LINEAR
     rm = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
     shift = np.atleast_1d(np.asarray(shift, dtype=np.int32))
-    got = m.conv2d(to_dev(x), to_dev(f), to_dev(bias), to_dev(shift), k, stride, dil, pads, depthwise=depthwise,
-                   activation=act, round_mode=rm, lut=to_dev(lut))
     fn = oracle.depthwise_s8 if depthwise else oracle.conv2d_s8
     want = fn(x, f, bias, shift, k, stride, dil, pads, oracle.RELU if relu else oracle.LINEAR,
               oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP)
     if lut is not None:
         want = oracle.lut_s8(want, lut)
+    residual = None
+    if residual_seed is not None:  # Conv -> Add in one launch
+        residual = rng_int8(np.random.default_rng(residual_seed), want.shape)
+        want = oracle.add_s8(want, residual)
+    got = m.conv2d(to_dev(x), to_dev(f), to_dev(bias), to_dev(shift), k, stride, dil, pads, depthwise=depthwise,
+                   activation=act, round_mode=rm, lut=to_dev(lut), residual=to_dev(residual))
     return to_host(got), want
 
 
@@ -41,6 +46,17 @@ def test_conv2d_s8(oracle, case, per_channel):
     announce(f"conv2d_s8 {case[0]} per_channel={per_channel}")
     x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 101, 3, per_channel)
     got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", [CONV_CASES[1], CONV_CASES[2], CONV_CASES[4], CONV_CASES[5], CONV_CASES[11], CONFIG1],
+                         ids=lambda c: c[0])
+def test_conv2d_s8_residual(oracle, case):
+    """Conv followed by a saturating Add of a tensor of the output's shape, in the conv's epilogue:
+    16-byte, 4-byte and byte store paths, direct and LDS-staged output."""
+    announce(f"conv2d_s8 + residual {case[0]}")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 131, 3, True)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, residual_seed=5)
     np.testing.assert_array_equal(got, want)
 
 

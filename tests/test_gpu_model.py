@@ -35,14 +35,14 @@ def _check_all(spec, mdl, want, skip_missing=True):
     return checked
 
 
-def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fuse_blocks=True):
+def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fuse_blocks=True, fuse_add=False):
     m, zoo, model, runner = _mods()
     import espdl_oracle as oracle
     rng = np.random.default_rng(seed)
     x = spec.make_input(rng, batch)
     want = runner.run(spec, {spec.inputs[0]: x}, oracle.ROUND_HALF_EVEN if round_mode else oracle.ROUND_HALF_UP)
     g = model.Graph.from_spec(spec)
-    mdl = model.Model(g, batch, round_mode=round_mode, fuse_lut=fuse_lut, fuse_blocks=fuse_blocks)
+    mdl = model.Model(g, batch, round_mode=round_mode, fuse_lut=fuse_lut, fuse_blocks=fuse_blocks, fuse_add=fuse_add)
     mdl.set_input(spec.inputs[0], x)
     if graph:
         assert mdl.enable_graph()
@@ -226,3 +226,17 @@ def test_mobilenetv2_block_fusion(oracle, fuse_blocks):
     else:
         assert mdl.module_count() == len(spec.nodes)
     mdl.close()
+
+
+def test_mobilenetv2_conv_add_fusion(oracle):
+    """Residual Adds folded into the project convolutions' epilogues (optional fusion): same logits."""
+    announce("model config3 96px fuse_add")
+    _, zoo, _, _ = _mods()
+    spec = zoo.config3_mobilenetv2(resolution=96, num_classes=100)
+    mdl, want, _ = _run_config(spec, 3, 22, fuse_add=True)
+    plain, _, _ = _run_config(spec, 3, 22)
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
+    assert mdl.module_count() < plain.module_count()
+    mdl.close()
+    plain.close()
