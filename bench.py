@@ -35,8 +35,8 @@ MACHINE_BALANCE = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)  # OP per byte
 # 256 MiB element-wise kernel of known traffic gave in the same runs).  Only valid for config 3 at
 # batch 256; any other workload reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "depthwise_s8": (2 * 34040.0 + 37922.4) * 1024,
-    "conv2d_s8_mfma": (2 * 10972.8 + 30566.2) * 1024,
+    "depthwise_s8": (7 * (2 * 55393.4 + 15715.5) + 10 * (2 * 9880.8 + 17404.8)) / 17 * 1024,
+    "conv2d_s8_mfma": (2 * 6669.5 + 33968.3) * 1024,
     "elementwise_s8": None,
 }
 
