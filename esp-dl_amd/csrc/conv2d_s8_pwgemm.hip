@@ -1,0 +1,277 @@
+// Pointwise (1x1, stride 1, unpadded) int8 convolution / Gemm as a tiled GEMM for layers with few
+// pixels per compute unit.
+//
+// What it computes is conv2d_11cn (esp-dl/dl/base/dl_base_conv2d.cpp:9-33) with the n_wise epilogue
+// (esp-dl/dl/base/dl_base_activate_buffer.hpp:27-36, 61-72, 173-181, 201-210), exactly as the
+// implicit-GEMM kernel in conv2d_s8_mfma_kernel.h does.
+//
+// Why a second kernel: the implicit-GEMM kernel keeps a whole 64-filter group (K x 64 bytes) resident
+// in LDS per workgroup and walks pixel sets under it, which is right when a workgroup sees thousands of
+// pixels.  At 14x14 and 7x7 a workgroup sees one or two pixel sets, and its time is the latency of
+// staging up to 60 KB of filters before the first MFMA.  Here both operands stream through LDS in
+// k steps of 64 with a register/LDS double buffer, so the first MFMA starts after one k step:
+//   workgroup tile = 128 pixels x 64*NG filters, 4 wavefronts, wavefront = 32 pixels x all filters;
+//   per k step: 128 x 64 B of pixels and 64*NG x 64 B of filters go global -> registers (one step
+//   ahead) -> LDS rows of 80 bytes (odd number of 16-byte units: conflict-free operand reads);
+//   one barrier per k step; MFMA operands are plain 16-byte LDS reads.
+// The filter -> tile-row permutation (row i of tile t is filter 16*(i/4) + 4*t + i%4 of the group)
+// leaves every lane with 16 consecutive output channels per pixel: one 16-byte store.
+#include "espdl_device.h"
+#include "espdl_kernels.h"
+
+namespace espdl {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kTileM = 128; // pixels per workgroup
+constexpr int kRow = 80;    // LDS row: 64 k bytes + 16
+
+struct PwArgs {
+    const int8_t *in;  // [M][K]
+    const int8_t *w;   // [N][K]
+    const int32_t *bias;
+    const int32_t *shift;
+    const int8_t *lut;
+    const int8_t *res;
+    int8_t *out;       // [M][N]
+    long long M;
+    int K, N;
+    int ksteps;
+    int relu, half_even, n_shift;
+    int out_vec; // 16, 4 or 1
+};
+
+template <int NG>
+__global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs a)
+{
+    constexpr int TN = 64 * NG;
+    constexpr int kPiecesB = kTileM * 4 / kThreads; // 16-byte pieces of the pixel tile per thread and k step (2)
+    constexpr int kPiecesA = TN * 4 / kThreads;     // ... of the filter tile (1 or 2)
+    __shared__ __align__(16) unsigned char b_l[2][kTileM * kRow];
+    __shared__ __align__(16) unsigned char a_l[2][TN * kRow];
+    __shared__ int cst[3][TN]; // start value | shift | left shift
+    __shared__ int8_t lut_l[256];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 15, quad = lane >> 4;
+    const long long m0 = (long long)blockIdx.x * kTileM;
+    const int n0 = blockIdx.y * TN;
+    const bool relu = a.relu != 0, half_even = a.half_even != 0, has_lut = a.lut != nullptr;
+
+    // piece p of a tile: row p / 4, 16-byte quarter p % 4 of the 64-byte k step
+    auto fetch = [&](int ks, v4i(&pb)[kPiecesB], v4i(&pa)[kPiecesA]) {
+        const int k0 = 64 * ks;
+#pragma unroll
+        for (int j = 0; j < kPiecesB; j++) {
+            const int p = tid + j * kThreads;
+            const long long m = m0 + (p >> 2);
+            const int k = k0 + 16 * (p & 3);
+            pb[j] = (m < a.M && k < a.K) ? *reinterpret_cast<const v4i *>(a.in + m * a.K + k) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int j = 0; j < kPiecesA; j++) {
+            const int p = tid + j * kThreads;
+            const int n = n0 + (p >> 2);
+            const int k = k0 + 16 * (p & 3);
+            pa[j] = (n < a.N && k < a.K) ? *reinterpret_cast<const v4i *>(a.w + (long long)n * a.K + k) : v4i{0, 0, 0, 0};
+        }
+    };
+    auto stash = [&](int buf, const v4i(&pb)[kPiecesB], const v4i(&pa)[kPiecesA]) {
+#pragma unroll
+        for (int j = 0; j < kPiecesB; j++) {
+            const int p = tid + j * kThreads;
+            *reinterpret_cast<v4i *>(&b_l[buf][(p >> 2) * kRow + 16 * (p & 3)]) = pb[j];
+        }
+#pragma unroll
+        for (int j = 0; j < kPiecesA; j++) {
+            const int p = tid + j * kThreads;
+            *reinterpret_cast<v4i *>(&a_l[buf][(p >> 2) * kRow + 16 * (p & 3)]) = pa[j];
+        }
+    };
+
+    v4i pb[kPiecesB], pa[kPiecesA];
+    fetch(0, pb, pa);
+
+    // epilogue constants of the workgroup's filters; the short form needs every shift in 1..31 and no
+    // possible overflow of bias + 2^(s-1) + K products
+    const long long mac_bound = (long long)a.K * 16384;
+    int ok_local = half_even ? 0 : 1;
+    int my_s = 0, my_b = 0;
+    if (tid < TN) {
+        const int n = n0 + tid;
+        if (n < a.N) {
+            my_s = a.shift[a.n_shift == 1 ? 0 : n];
+            my_b = a.bias != nullptr ? a.bias[n] : 0;
+            if (my_s < 1 || my_s > 31) {
+                ok_local = 0;
+            } else {
+                const long long start = (long long)my_b + (1ll << (my_s - 1));
+                if ((start < 0 ? -start : start) + mac_bound >= (1ll << (31 - max(0, 8 - my_s))))
+                    ok_local = 0;
+            }
+        }
+    }
+    if (has_lut)
+        lut_l[tid] = a.lut[tid];
+    const bool fast = __syncthreads_and(ok_local) != 0;
+    if (tid < TN) {
+        const bool valid = n0 + tid < a.N;
+        cst[0][tid] = (fast && valid) ? my_b + (1 << (my_s - 1)) : my_b;
+        cst[1][tid] = fast ? max(0, my_s - 8) : my_s;
+        cst[2][tid] = fast ? max(0, 8 - my_s) : 0;
+    }
+    stash(0, pb, pa);
+    __syncthreads();
+
+    // accumulators: 2 pixel tiles x 4*NG filter tiles, started at bias (+ rounding constant)
+    v4i acc[2][4 * NG];
+#pragma unroll
+    for (int g = 0; g < NG; g++)
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            // rows 4*quad .. 4*quad+3 of tile t are filters 64*g + 16*quad + 4*t + r
+            const v4i init = *reinterpret_cast<const v4i *>(&cst[0][64 * g + 16 * quad + 4 * t]);
+            acc[0][4 * g + t] = init;
+            acc[1][4 * g + t] = init;
+        }
+
+    // operand A row of this lane in tile t of group g: filter 64*g + 16*(col/4) + 4*t + col%4
+    const int a_row0 = 16 * (col >> 2) + (col & 3);
+    for (int ks = 0; ks < a.ksteps; ks++) {
+        const int buf = ks & 1;
+        if (ks + 1 < a.ksteps)
+            fetch(ks + 1, pb, pa); // in flight during this step's MFMAs
+        v4i b[2];
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+            b[c] = *reinterpret_cast<const v4i *>(&b_l[buf][(32 * wave + 16 * c + col) * kRow + 16 * quad]);
+#pragma unroll
+        for (int g = 0; g < NG; g++)
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const v4i aop = *reinterpret_cast<const v4i *>(&a_l[buf][(64 * g + a_row0 + 4 * t) * kRow + 16 * quad]);
+                acc[0][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[0], acc[0][4 * g + t], 0, 0, 0);
+                acc[1][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[1], acc[1][4 * g + t], 0, 0, 0);
+            }
+        if (ks + 1 < a.ksteps) {
+            // the other buffer was last read in step ks - 1, which every wavefront finished before
+            // the barrier at the end of that step
+            stash(buf ^ 1, pb, pa);
+            __syncthreads();
+        }
+    }
+
+    // epilogue: lane (col, quad) holds, per pixel tile and group, filters 64*g + 16*quad + [0, 16)
+    const int floor_pk = relu ? 0 : (int)0x80008000u;
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+        const long long m = m0 + 32 * wave + 16 * c + col;
+#pragma unroll
+        for (int g = 0; g < NG; g++) {
+            const int n = n0 + 64 * g + 16 * quad;
+            int words[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const v4i ss = *reinterpret_cast<const v4i *>(&cst[1][64 * g + 16 * quad + 4 * t]);
+                if (fast) {
+                    const v4i ls = *reinterpret_cast<const v4i *>(&cst[2][64 * g + 16 * quad + 4 * t]);
+                    words[t] = pack_fast4<true>(acc[c][4 * g + t], ls, ss, floor_pk);
+                } else {
+                    int q[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        q[r] = requant_s8(acc[c][4 * g + t][r], ss[r], relu, half_even);
+                    words[t] = pack4_s8(q[0], q[1], q[2], q[3]);
+                }
+                if (has_lut) {
+                    const int v = words[t];
+                    words[t] = pack4_s8(lut_l[(int)(int8_t)v + 128], lut_l[(int)(int8_t)(v >> 8) + 128],
+                                        lut_l[(int)(int8_t)(v >> 16) + 128], lut_l[(v >> 24) + 128]);
+                }
+            }
+            if (m >= a.M || n >= a.N)
+                continue;
+            const long long goff = m * a.N + n;
+            if (a.out_vec == 16 && n + 16 <= a.N) {
+                v4i v = {words[0], words[1], words[2], words[3]};
+                if (a.res != nullptr) {
+                    const v4i r = *reinterpret_cast<const v4i *>(a.res + goff);
+#pragma unroll
+                    for (int d = 0; d < 4; d++)
+                        v[d] = sat_add4_s8(v[d], r[d]);
+                }
+                *reinterpret_cast<v4i *>(a.out + goff) = v;
+            } else if (a.out_vec >= 4) {
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    if (n + 4 * t + 4 <= a.N) {
+                        int v = words[t];
+                        if (a.res != nullptr)
+                            v = sat_add4_s8(v, *reinterpret_cast<const int *>(a.res + goff + 4 * t));
+                        *reinterpret_cast<int *>(a.out + goff + 4 * t) = v;
+                    }
+            } else {
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    for (int r = 0; r < 4; r++)
+                        if (n + 4 * t + r < a.N) {
+                            int v = (int)(int8_t)(words[t] >> (8 * r));
+                            if (a.res != nullptr)
+                                v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
+                            a.out[goff + 4 * t + r] = (int8_t)v;
+                        }
+            }
+        }
+    }
+}
+
+} // namespace
+
+// Flat pointwise geometry with 16-byte aligned rows; worth it when a workgroup of the implicit-GEMM
+// kernel would see only a few pixel sets.
+bool conv2d_s8_pwgemm_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count)
+{
+    const bool flat = g.k_h == 1 && g.k_w == 1 && g.stride_h == 1 && g.stride_w == 1 && g.pad_top == 0 &&
+        g.pad_left == 0 && g.out_h == g.in_h && g.out_w == g.in_w;
+    if (!flat || (g.in_c & 15) != 0 || g.in_c < 64 || g.out_c < 32 ||
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) != 0)
+        return false;
+    const long long npix = (long long)g.batch * g.out_h * g.out_w;
+    const int cus = cu_count > 0 ? cu_count : 256;
+    return npix > 0 && (npix + 63) / 64 < (long long)cus * 16 && (npix + kTileM - 1) / kTileM <= 0x7fffffffll;
+}
+
+hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                   const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
+                                   hipStream_t stream)
+{
+    PwArgs a;
+    a.in = in;
+    a.w = filter;
+    a.bias = bias;
+    a.shift = shift;
+    a.lut = lut;
+    a.res = residual;
+    a.out = out;
+    a.M = (long long)g.batch * g.out_h * g.out_w;
+    a.K = g.in_c;
+    a.N = g.out_c;
+    a.ksteps = (a.K + 63) / 64;
+    a.relu = g.relu;
+    a.half_even = g.half_even;
+    a.n_shift = g.n_shift;
+    const uintptr_t oaddr = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(residual);
+    a.out_vec = ((a.N & 15) == 0 && (oaddr & 15) == 0) ? 16 : (((a.N & 3) == 0 && (oaddr & 3) == 0) ? 4 : 1);
+    if (a.M == 0)
+        return hipSuccess;
+    const unsigned gx = (unsigned)((a.M + kTileM - 1) / kTileM);
+    if (a.N <= 64) {
+        hipLaunchKernelGGL(conv2d_s8_pwgemm_kernel<1>, dim3(gx, (unsigned)((a.N + 63) / 64)), dim3(kThreads), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL(conv2d_s8_pwgemm_kernel<2>, dim3(gx, (unsigned)((a.N + 127) / 128)), dim3(kThreads), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+} // namespace espdl

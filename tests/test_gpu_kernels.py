@@ -118,6 +118,40 @@ def test_conv2d_s8_large_k(oracle, k_total, oc):
     np.testing.assert_array_equal(got, want)
 
 
+# Pointwise layers with few pixels and K % 16 == 0, K >= 64, N >= 32 take the tiled-GEMM kernel:
+# (pixels (n, h, w), K, N): pixel tails (M % 128), filter tails (N % 128, % 16, % 4, odd), K tails (K % 64),
+# many k steps, one k step.
+PWGEMM_CASES = [
+    ((2, 14, 14), 64, 384), ((3, 7, 7), 960, 160), ((1, 7, 7), 960, 320), ((2, 14, 14), 576, 96),
+    ((1, 1, 256), 1280, 1000), ((1, 5, 9), 80, 40), ((2, 3, 5), 112, 33), ((1, 1, 1), 64, 32),
+    ((1, 13, 11), 144, 200), ((4, 14, 14), 96, 576), ((1, 7, 7), 320, 1280),
+]
+
+
+@pytest.mark.parametrize("case", PWGEMM_CASES, ids=lambda c: "x".join(map(str, c[0])) + f"_k{c[1]}_n{c[2]}")
+@pytest.mark.parametrize("variant", ["plain", "relu_pc", "half_even", "lut", "residual", "low_shift"])
+def test_conv2d_s8_pointwise_tiled_gemm(oracle, case, variant):
+    (n, h, w), kk, oc = case
+    announce(f"conv2d_s8 pointwise tiled gemm {case} {variant}")
+    rng = np.random.default_rng(4242 + kk + oc)
+    x = rng_int8(rng, (n, h, w, kk))
+    f = rng_int8(rng, (oc, 1, 1, kk))
+    bias = rng.integers(-4096, 4097, size=oc).astype(np.int32) if variant != "plain" else None
+    base = typical_shift(kk)
+    shift = np.int32(base)
+    if variant in ("relu_pc", "residual", "half_even"):
+        shift = (base + rng.integers(-2, 3, size=oc)).astype(np.int32)
+    if variant == "low_shift":  # some shifts below 8 (left-shift form) and one outside 1..31 (general form)
+        shift = rng.integers(3, 12, size=oc).astype(np.int32)
+        if oc > 40:
+            shift[37] = 0
+    lut = rng_int8(rng, (256,)) if variant == "lut" else None
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), variant == "relu_pc",
+                             half_even=variant == "half_even", lut=lut,
+                             residual_seed=77 if variant == "residual" else None)
+    np.testing.assert_array_equal(got, want)
+
+
 @pytest.mark.parametrize("m,k,n,has_bias,relu", GEMM_CASES)
 def test_gemm_s8(oracle, m, k, n, has_bias, relu):
     announce(f"gemm_s8 M={m} K={k} N={n}")
