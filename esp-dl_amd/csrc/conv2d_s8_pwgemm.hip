@@ -10,8 +10,8 @@
 // pixels.  At 14x14 and 7x7 a workgroup sees one or two pixel sets, and its time is the latency of
 // staging up to 60 KB of filters before the first MFMA.  Here both operands stream through LDS in
 // k steps of 64 with a register/LDS double buffer, so the first MFMA starts after one k step:
-//   workgroup tile = 128 pixels x 64*NG filters, 4 wavefronts, wavefront = 32 pixels x all filters;
-//   per k step: 128 x 64 B of pixels and 64*NG x 64 B of filters go global -> registers (one step
+//   workgroup tile = 64*PT pixels x 64*NG filters, 4 wavefronts, wavefront = 16*PT pixels x all filters;
+//   per k step: 64*PT x 64 B of pixels and 64*NG x 64 B of filters go global -> registers (one step
 //   ahead) -> LDS rows of 80 bytes (odd number of 16-byte units: conflict-free operand reads);
 //   one barrier per k step; MFMA operands are plain 16-byte LDS reads.
 // The filter -> tile-row permutation (row i of tile t is filter 16*(i/4) + 4*t + i%4 of the group)
@@ -24,7 +24,6 @@ namespace espdl {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kTileM = 128; // pixels per workgroup
 constexpr int kRow = 80;    // LDS row: 64 k bytes + 16
 
 struct PwArgs {
@@ -42,10 +41,11 @@ struct PwArgs {
     int out_vec; // 16, 4 or 1
 };
 
-template <int NG>
+template <int NG, int PT>
 __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs a)
 {
     constexpr int TN = 64 * NG;
+    constexpr int kTileM = 64 * PT; // pixels per workgroup, 16 * PT per wavefront
     constexpr int kPiecesB = kTileM * 4 / kThreads; // 16-byte pieces of the pixel tile per thread and k step (2)
     constexpr int kPiecesA = TN * 4 / kThreads;     // ... of the filter tile (1 or 2)
     __shared__ __align__(16) unsigned char b_l[2][kTileM * kRow];
@@ -125,15 +125,16 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     __syncthreads();
 
     // accumulators: 2 pixel tiles x 4*NG filter tiles, started at bias (+ rounding constant)
-    v4i acc[2][4 * NG];
+    v4i acc[PT][4 * NG];
 #pragma unroll
     for (int g = 0; g < NG; g++)
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             // rows 4*quad .. 4*quad+3 of tile t are filters 64*g + 16*quad + 4*t + r
             const v4i init = *reinterpret_cast<const v4i *>(&cst[0][64 * g + 16 * quad + 4 * t]);
-            acc[0][4 * g + t] = init;
-            acc[1][4 * g + t] = init;
+#pragma unroll
+            for (int c = 0; c < PT; c++)
+                acc[c][4 * g + t] = init;
         }
 
     // operand A row of this lane in tile t of group g: filter 64*g + 16*(col/4) + 4*t + col%4
@@ -142,17 +143,18 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
         const int buf = ks & 1;
         if (ks + 1 < a.ksteps)
             fetch(ks + 1, pb, pa); // in flight during this step's MFMAs
-        v4i b[2];
+        v4i b[PT];
 #pragma unroll
-        for (int c = 0; c < 2; c++)
-            b[c] = *reinterpret_cast<const v4i *>(&b_l[buf][(32 * wave + 16 * c + col) * kRow + 16 * quad]);
+        for (int c = 0; c < PT; c++)
+            b[c] = *reinterpret_cast<const v4i *>(&b_l[buf][(16 * PT * wave + 16 * c + col) * kRow + 16 * quad]);
 #pragma unroll
         for (int g = 0; g < NG; g++)
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const v4i aop = *reinterpret_cast<const v4i *>(&a_l[buf][(64 * g + a_row0 + 4 * t) * kRow + 16 * quad]);
-                acc[0][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[0], acc[0][4 * g + t], 0, 0, 0);
-                acc[1][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[1], acc[1][4 * g + t], 0, 0, 0);
+#pragma unroll
+                for (int c = 0; c < PT; c++)
+                    acc[c][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[c], acc[c][4 * g + t], 0, 0, 0);
             }
         if (ks + 1 < a.ksteps) {
             // the other buffer was last read in step ks - 1, which every wavefront finished before
@@ -165,8 +167,8 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     // epilogue: lane (col, quad) holds, per pixel tile and group, filters 64*g + 16*quad + [0, 16)
     const int floor_pk = relu ? 0 : (int)0x80008000u;
 #pragma unroll
-    for (int c = 0; c < 2; c++) {
-        const long long m = m0 + 32 * wave + 16 * c + col;
+    for (int c = 0; c < PT; c++) {
+        const long long m = m0 + 16 * PT * wave + 16 * c + col;
 #pragma unroll
         for (int g = 0; g < NG; g++) {
             const int n = n0 + 64 * g + 16 * quad;
@@ -201,7 +203,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
                     for (int d = 0; d < 4; d++)
                         v[d] = sat_add4_s8(v[d], r[d]);
                 }
-                *reinterpret_cast<v4i *>(a.out + goff) = v;
+                __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(a.out + goff));
             } else if (a.out_vec >= 4) {
 #pragma unroll
                 for (int t = 0; t < 4; t++)
@@ -239,12 +241,12 @@ bool conv2d_s8_pwgemm_supports(const ConvGeom &g, const void *in, const void *fi
         return false;
     const long long npix = (long long)g.batch * g.out_h * g.out_w;
     const int cus = cu_count > 0 ? cu_count : 256;
-    return npix > 0 && (npix + 63) / 64 < (long long)cus * 16 && (npix + kTileM - 1) / kTileM <= 0x7fffffffll;
+    return npix > 0 && (npix + 63) / 64 < (long long)cus * 16 && (npix + 63) / 64 <= 0x7fffffffll;
 }
 
 hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                    const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
-                                   hipStream_t stream)
+                                   int cu_count, hipStream_t stream)
 {
     PwArgs a;
     a.in = in;
@@ -265,12 +267,15 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
     a.out_vec = ((a.N & 15) == 0 && (oaddr & 15) == 0) ? 16 : (((a.N & 3) == 0 && (oaddr & 3) == 0) ? 4 : 1);
     if (a.M == 0)
         return hipSuccess;
-    const unsigned gx = (unsigned)((a.M + kTileM - 1) / kTileM);
-    if (a.N <= 64) {
-        hipLaunchKernelGGL(conv2d_s8_pwgemm_kernel<1>, dim3(gx, (unsigned)((a.N + 63) / 64)), dim3(kThreads), 0, stream, a);
-    } else {
-        hipLaunchKernelGGL(conv2d_s8_pwgemm_kernel<2>, dim3(gx, (unsigned)((a.N + 127) / 128)), dim3(kThreads), 0, stream, a);
-    }
+    // 64-filter tiles: measured faster than 128 on every MobileNetV2 layer (more, shorter workgroups).
+    // 128-pixel tiles unless that leaves fewer than 1.5 workgroups per compute unit.
+    const unsigned gy = (unsigned)((a.N + 63) / 64);
+    const long long tiles128 = (a.M + 127) / 128;
+    const int cus = cu_count > 0 ? cu_count : 256;
+    if (tiles128 * gy * 2 < 3ll * cus)
+        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1>), dim3((unsigned)((a.M + 63) / 64), gy), dim3(kThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2>), dim3((unsigned)tiles128, gy), dim3(kThreads), 0, stream, a);
     return hipGetLastError();
 }
 

@@ -24,7 +24,7 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
 bool conv2d_s8_pwgemm_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count);
 hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                    const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
-                                   hipStream_t stream);
+                                   int cu_count, hipStream_t stream);
 
 hipError_t launch_depthwise_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                const int32_t *shift, const int8_t *lut, int8_t *out, hipStream_t stream);
