@@ -481,3 +481,149 @@ void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int 
         out[i] = (int8_t)clamp_i64(round_half_up_f32(tmp * inv_scale), INT8_MIN, INT8_MAX);
     }
 }
+
+/* ---------------------------------------------------------------------------------------------
+ * Data-movement operators of the detection necks (Concat, Split, Transpose, Resize, MaxPool).
+ * ------------------------------------------------------------------------------------------- */
+
+/* Concat along an axis (esp-dl/dl/module/include/dl_module_concat.hpp:56-108): loop_times =
+ * product of the dims before the axis; input j contributes copy_nums[j] = product of its dims
+ * from the axis on, per loop.  elem_size in bytes. */
+void espdl_oracle_concat(const void *const *inputs, int n_inputs, const int64_t *copy_nums, int64_t loop_times,
+                         int elem_size, void *out)
+{
+    char *o = (char *)out;
+    for (int64_t i = 0; i < loop_times; i++)
+        for (int j = 0; j < n_inputs; j++) {
+            const int64_t bytes = copy_nums[j] * elem_size;
+            memcpy(o, (const char *)inputs[j] + i * bytes, (size_t)bytes);
+            o += bytes;
+        }
+}
+
+/* One output of Split (esp-dl/dl/module/include/dl_module_split.hpp:84-93): for each of the
+ * num_slices outer positions copy out_axis * slice_size elements that start at element
+ * (n * in_axis + slice_index) * slice_size. */
+void espdl_oracle_split_slice(const void *in, int64_t slice_index, int64_t num_slices, int64_t slice_size,
+                              int64_t in_axis, int64_t out_axis, int elem_size, void *out)
+{
+    for (int64_t n = 0; n < num_slices; n++) {
+        const int64_t in_off = (n * in_axis + slice_index) * slice_size;
+        const int64_t out_off = n * out_axis * slice_size;
+        memcpy((char *)out + out_off * elem_size, (const char *)in + in_off * elem_size,
+               (size_t)(slice_size * out_axis * elem_size));
+    }
+}
+
+/* Transpose (esp-dl/dl/tensor/src/dl_tensor_base.cpp:722-812): out.shape[i] = in.shape[perm[i]],
+ * out[index permuted] = in[index].  Up to 8 dims; perm entries already non-negative. */
+int espdl_oracle_transpose(const void *in, const int *shape, int dims, const int *perm, int elem_size, void *out)
+{
+    if (dims < 1 || dims > 8)
+        return -1;
+    int64_t in_stride[8], out_stride[8], out_shape[8], total = 1;
+    in_stride[dims - 1] = 1;
+    for (int i = dims - 2; i >= 0; i--)
+        in_stride[i] = in_stride[i + 1] * shape[i + 1];
+    for (int i = 0; i < dims; i++) {
+        if (perm[i] < 0 || perm[i] >= dims)
+            return -1;
+        out_shape[i] = shape[perm[i]];
+        total *= shape[i];
+    }
+    out_stride[dims - 1] = 1;
+    for (int i = dims - 2; i >= 0; i--)
+        out_stride[i] = out_stride[i + 1] * out_shape[i + 1];
+    int64_t idx[8] = {0};
+    for (int64_t e = 0; e < total; e++) { /* e walks the input in memory order */
+        int64_t o = 0;
+        for (int i = 0; i < dims; i++)
+            o += idx[perm[i]] * out_stride[i];
+        memcpy((char *)out + o * elem_size, (const char *)in + e * elem_size, (size_t)elem_size);
+        for (int i = dims - 1; i >= 0; i--) {
+            if (++idx[i] < shape[i])
+                break;
+            idx[i] = 0;
+        }
+    }
+    (void)in_stride;
+    return 0;
+}
+
+/* Resize, nearest, int8 NHWC (esp-dl/dl/base/dl_base_resize.cpp:7-34 per pixel, :236-268 the
+ * coordinate loops, esp-dl/dl/base/dl_base_resize.hpp:37-92 the arguments).  scale_h / scale_w are
+ * the float32 scales of the module; the exact-2x path replicates each input pixel into a 2x2 block,
+ * every other scale uses in = min((int)(out * (1 / scale)), len - 1) in float32 ("asymmetric").
+ * Value: round((float)x * output_scale / (1 << output_shift)) with round = floorf(v + 0.5), stored
+ * to int8 by C conversion (no saturation in the reference: wraps when the exponent shrinks). */
+void espdl_oracle_resize_nearest_s8(const int8_t *in, int batch, int h, int w, int c, int out_h, int out_w,
+                                    float scale_h, float scale_w, int in_exp, int out_exp, int8_t *out)
+{
+    int output_shift = out_exp - in_exp, output_scale = 1;
+    if (output_shift < 0) {
+        output_scale = 1 << (-output_shift);
+        output_shift = 0;
+    }
+    const float scale_h_inv = 1 / scale_h, scale_w_inv = 1 / scale_w;
+    const int exact2 = scale_h == 2 && scale_w == 2;
+    for (int n = 0; n < batch; n++) {
+        const int8_t *img = in + (int64_t)n * h * w * c;
+        int8_t *oimg = out + (int64_t)n * out_h * out_w * c;
+        for (int y = 0; y < out_h; y++) {
+            int in_y = exact2 ? y / 2 : (int)(y * scale_h_inv);
+            if (in_y > h - 1)
+                in_y = h - 1;
+            for (int x = 0; x < out_w; x++) {
+                int in_x = exact2 ? x / 2 : (int)(x * scale_w_inv);
+                if (in_x > w - 1)
+                    in_x = w - 1;
+                const int8_t *src = img + ((int64_t)in_y * w + in_x) * c;
+                int8_t *dst = oimg + ((int64_t)y * out_w + x) * c;
+                for (int k = 0; k < c; k++) {
+                    const float v = (float)src[k] * (float)output_scale / (float)(1 << output_shift);
+                    dst[k] = (int8_t)(int)floorf(v + 0.5f);
+                }
+            }
+        }
+    }
+}
+
+/* MaxPool, NHWC (esp-dl/dl/base/dl_base_max_pool2d.cpp:9-29 on the window clipped to the image as
+ * the pool shell does; output size esp-dl/dl/module/include/dl_module_max_pool.hpp:42-49).  No
+ * rescale: output exponent = input exponent.  elem_size 1 (int8) or 2 (int16). */
+int espdl_oracle_max_pool(const void *in, int elem_size, int batch, int h, int w, int c, int k_h, int k_w,
+                          int stride_h, int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right,
+                          void *out)
+{
+    const int out_h = (h + pad_top + pad_bottom - k_h) / stride_h + 1;
+    const int out_w = (w + pad_left + pad_right - k_w) / stride_w + 1;
+    if (elem_size != 1 && elem_size != 2)
+        return -1;
+    for (int n = 0; n < batch; n++)
+        for (int oy = 0; oy < out_h; oy++)
+            for (int ox = 0; ox < out_w; ox++)
+                for (int k = 0; k < c; k++) {
+                    int best = 0, have = 0;
+                    for (int ky = 0; ky < k_h; ky++) {
+                        const int iy = oy * stride_h - pad_top + ky;
+                        if (iy < 0 || iy >= h)
+                            continue;
+                        for (int kx = 0; kx < k_w; kx++) {
+                            const int ix = ox * stride_w - pad_left + kx;
+                            if (ix < 0 || ix >= w)
+                                continue;
+                            const int64_t off = (((int64_t)n * h + iy) * w + ix) * c + k;
+                            const int v = elem_size == 1 ? ((const int8_t *)in)[off] : ((const int16_t *)in)[off];
+                            if (!have || v > best)
+                                best = v;
+                            have = 1;
+                        }
+                    }
+                    const int64_t ooff = (((int64_t)n * out_h + oy) * out_w + ox) * c + k;
+                    if (elem_size == 1)
+                        ((int8_t *)out)[ooff] = (int8_t)best;
+                    else
+                        ((int16_t *)out)[ooff] = (int16_t)best;
+                }
+    return 0;
+}

@@ -41,6 +41,14 @@
  *                                within float rounding error of a tie; the reference itself
  *                                cannot be built here (every translation unit needs ESP-IDF
  *                                headers that are absent)                   PARITY UNPINNED (near-ties)
+ *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
+ *                                numpy.split / numpy.transpose on random shapes           PINNED
+ *   espdl_oracle_max_pool        equality with scipy.ndimage.maximum_filter (minimum-value border)
+ *                                sampled at the window centres, and brute force            PINNED
+ *   espdl_oracle_resize_nearest_s8   coordinates: numpy.repeat for integer scales, exact rational
+ *                                floor(o / scale) for the others where float32 is exact; values:
+ *                                the already pinned round-half-up shift for a growing exponent,
+ *                                x * 2^k wrapped to int8 for a shrinking one               PINNED
  */
 #ifndef ESPDL_ORACLE_H
 #define ESPDL_ORACLE_H
@@ -96,6 +104,18 @@ void espdl_oracle_add_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int
 void espdl_oracle_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
                                      int8_t *out);
 void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out);
+
+/* Data-movement operators (see the .c file for the reference lines each one follows). */
+void espdl_oracle_concat(const void *const *inputs, int n_inputs, const int64_t *copy_nums, int64_t loop_times,
+                         int elem_size, void *out);
+void espdl_oracle_split_slice(const void *in, int64_t slice_index, int64_t num_slices, int64_t slice_size,
+                              int64_t in_axis, int64_t out_axis, int elem_size, void *out);
+int espdl_oracle_transpose(const void *in, const int *shape, int dims, const int *perm, int elem_size, void *out);
+void espdl_oracle_resize_nearest_s8(const int8_t *in, int batch, int h, int w, int c, int out_h, int out_w,
+                                    float scale_h, float scale_w, int in_exp, int out_exp, int8_t *out);
+int espdl_oracle_max_pool(const void *in, int elem_size, int batch, int h, int w, int c, int k_h, int k_w,
+                          int stride_h, int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right,
+                          void *out);
 
 /* Number of worker threads the batch loops use (1 unless built with OpenMP). */
 int espdl_oracle_max_threads(void);

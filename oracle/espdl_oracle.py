@@ -58,6 +58,14 @@ def lib():
         L.espdl_oracle_add_s8.argtypes = [vp, i64, vp, i64, i64, vp]
         L.espdl_oracle_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp]
         L.espdl_oracle_requantize_s8.argtypes = [vp, i64, i32, i32, vp]
+        L.espdl_oracle_concat.argtypes = [vp, i32, vp, i64, i32, vp]
+        L.espdl_oracle_split_slice.argtypes = [vp, i64, i64, i64, i64, i64, i32, vp]
+        L.espdl_oracle_transpose.restype = i32
+        L.espdl_oracle_transpose.argtypes = [vp, vp, i32, vp, i32, vp]
+        L.espdl_oracle_resize_nearest_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, ctypes.c_float, ctypes.c_float,
+                                                     i32, i32, vp]
+        L.espdl_oracle_max_pool.restype = i32
+        L.espdl_oracle_max_pool.argtypes = [vp, i32] + [i32] * 12 + [vp]
         L.espdl_oracle_max_threads.restype = i32
         L.espdl_oracle_set_threads.argtypes = [i32]
         for name in ("lut_s8", "prelu_s8", "relu_s8", "clip_s8", "add_s8", "global_avg_pool_s8",
@@ -211,4 +219,81 @@ def requantize_s8(x, in_exp, out_exp):
     x = _c(x, np.int8)
     out = np.empty_like(x)
     lib().espdl_oracle_requantize_s8(_ptr(x), x.size, in_exp, out_exp, _ptr(out))
+    return out
+
+
+def concat(arrays, axis):
+    """Concat as the reference runs it: per outer index, one contiguous run from each input
+    (esp-dl/dl/module/include/dl_module_concat.hpp:56-108)."""
+    arrays = [np.ascontiguousarray(a) for a in arrays]
+    dt = arrays[0].dtype
+    nd = arrays[0].ndim
+    axis = axis + nd if axis < 0 else axis
+    loop_times = int(np.prod(arrays[0].shape[:axis], dtype=np.int64))
+    copy_nums = np.array([int(np.prod(a.shape[axis:], dtype=np.int64)) for a in arrays], dtype=np.int64)
+    shape = list(arrays[0].shape)
+    shape[axis] = sum(a.shape[axis] for a in arrays)
+    out = np.empty(shape, dtype=dt)
+    ptrs = (ctypes.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+    lib().espdl_oracle_concat(ptrs, len(arrays), _ptr(copy_nums), loop_times, dt.itemsize, _ptr(out))
+    return out
+
+
+def split(x, axis, sizes):
+    """Split into consecutive pieces of the given sizes along axis
+    (esp-dl/dl/module/include/dl_module_split.hpp:84-152)."""
+    x = np.ascontiguousarray(x)
+    axis = axis + x.ndim if axis < 0 else axis
+    num_slices = int(np.prod(x.shape[:axis], dtype=np.int64))
+    slice_size = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    outs, start = [], 0
+    for sz in sizes:
+        shape = list(x.shape)
+        shape[axis] = int(sz)
+        out = np.empty(shape, dtype=x.dtype)
+        lib().espdl_oracle_split_slice(_ptr(x), start, num_slices, slice_size, x.shape[axis], int(sz), x.dtype.itemsize,
+                                       _ptr(out))
+        outs.append(out)
+        start += int(sz)
+    return outs
+
+
+def transpose(x, perm=None):
+    x = np.ascontiguousarray(x)
+    perm = list(range(x.ndim - 1, -1, -1)) if not perm else [p + x.ndim if p < 0 else p for p in perm]
+    out = np.empty([x.shape[p] for p in perm], dtype=x.dtype)
+    shape = np.array(x.shape, dtype=np.int32)
+    permv = np.array(perm, dtype=np.int32)
+    rc = lib().espdl_oracle_transpose(_ptr(x), _ptr(shape), x.ndim, _ptr(permv), x.dtype.itemsize, _ptr(out))
+    assert rc == 0
+    return out
+
+
+def resize_out_hw(h, w, scale_h, scale_w):
+    """Output size as esp-dl/dl/module/include/dl_module_resize.hpp:66-70 computes it from scales."""
+    return int(h * np.float32(scale_h)), int(w * np.float32(scale_w))
+
+
+def resize_nearest_s8(x, scale_h, scale_w, in_exp=0, out_exp=0, out_hw=None):
+    x = _c(x, np.int8)
+    n, h, w, c = x.shape
+    oh, ow = out_hw if out_hw is not None else resize_out_hw(h, w, scale_h, scale_w)
+    out = np.empty((n, oh, ow, c), dtype=np.int8)
+    lib().espdl_oracle_resize_nearest_s8(_ptr(x), n, h, w, c, oh, ow, float(scale_h), float(scale_w), in_exp, out_exp,
+                                         _ptr(out))
+    return out
+
+
+def max_pool(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0)):
+    """pads = (top, bottom, left, right).  int8 or int16 NHWC."""
+    x = np.ascontiguousarray(x)
+    assert x.dtype in (np.int8, np.int16)
+    n, h, w, c = x.shape
+    pt, pb, pl, pr = pads
+    oh = (h + pt + pb - kernel[0]) // strides[0] + 1
+    ow = (w + pl + pr - kernel[1]) // strides[1] + 1
+    out = np.empty((n, oh, ow, c), dtype=x.dtype)
+    rc = lib().espdl_oracle_max_pool(_ptr(x), x.dtype.itemsize, n, h, w, c, kernel[0], kernel[1], strides[0], strides[1],
+                                     pt, pb, pl, pr, _ptr(out))
+    assert rc == 0
     return out

@@ -1,0 +1,121 @@
+"""Pins the oracle's data-movement operators (Concat, Split, Transpose, Resize-nearest, MaxPool) against
+library routines and exact arithmetic.  No GPU needed."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+from scipy import ndimage
+
+import bruteforce as bf
+
+
+def _rand(rng, shape, dtype=np.int8):
+    info = np.iinfo(dtype)
+    return rng.integers(info.min, info.max + 1, size=shape).astype(dtype)
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("axis", [0, 1, 2, 3, -1])
+def test_concat_is_numpy_concatenate(oracle, dtype, axis):
+    rng = np.random.default_rng(5)
+    base = [2, 3, 5, 7]
+    arrays = []
+    for extent in (4, 1, 9):
+        shape = list(base)
+        shape[axis] = extent
+        arrays.append(_rand(rng, shape, dtype))
+    np.testing.assert_array_equal(oracle.concat(arrays, axis), np.concatenate(arrays, axis=axis))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("axis,sizes", [(3, [16, 16]), (3, [5, 20, 7]), (1, [1, 2]), (0, [2]), (-2, [3, 1, 1])])
+def test_split_is_numpy_split(oracle, dtype, axis, sizes):
+    rng = np.random.default_rng(6)
+    shape = [2, 3, 5, 32]
+    shape[axis] = sum(sizes)
+    x = _rand(rng, shape, dtype)
+    want = np.split(x, np.cumsum(sizes)[:-1], axis=axis)
+    got = oracle.split(x, axis, sizes)
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        np.testing.assert_array_equal(g, w)
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16, np.int32])
+@pytest.mark.parametrize("shape,perm", [
+    ((2, 3, 4, 5), (0, 3, 1, 2)), ((2, 3, 4, 5), (0, 2, 3, 1)), ((2, 3, 4, 5), None), ((7, 9), (1, 0)),
+    ((3, 1, 1, 8), (0, 3, 1, 2)), ((2, 3, 4), (-1, 0, 1)), ((2, 2, 3, 2, 5), (4, 0, 3, 1, 2)), ((6,), (0,)),
+])
+def test_transpose_is_numpy_transpose(oracle, dtype, shape, perm):
+    rng = np.random.default_rng(7)
+    x = _rand(rng, shape, dtype)
+    np.testing.assert_array_equal(oracle.transpose(x, perm), np.transpose(x, perm))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("kernel,strides,pads", [
+    ((5, 5), (1, 1), (2, 2, 2, 2)), ((2, 2), (2, 2), (0, 0, 0, 0)), ((3, 3), (2, 2), (1, 1, 1, 1)),
+    ((3, 2), (1, 2), (1, 0, 0, 1)), ((1, 1), (1, 1), (0, 0, 0, 0)), ((3, 3), (1, 1), (0, 0, 0, 0)),
+])
+def test_max_pool_matches_brute_force(oracle, dtype, kernel, strides, pads):
+    rng = np.random.default_rng(8)
+    x = _rand(rng, (2, 9, 8, 5), dtype)
+    got = oracle.max_pool(x, kernel, strides, pads)
+    pt, pb, pl, pr = pads
+    lo = np.iinfo(dtype).min
+    padded = np.full((2, 9 + pt + pb, 8 + pl + pr, 5), lo, dtype=dtype)  # clipped window == minimum-value padding
+    padded[:, pt:pt + 9, pl:pl + 8, :] = x
+    oh = (9 + pt + pb - kernel[0]) // strides[0] + 1
+    ow = (8 + pl + pr - kernel[1]) // strides[1] + 1
+    want = np.empty((2, oh, ow, 5), dtype=dtype)
+    for oy in range(oh):
+        for ox in range(ow):
+            win = padded[:, oy * strides[0]:oy * strides[0] + kernel[0], ox * strides[1]:ox * strides[1] + kernel[1], :]
+            want[:, oy, ox, :] = win.max(axis=(1, 2))
+    np.testing.assert_array_equal(got, want)
+
+
+def test_max_pool_5x5_same_is_scipy_maximum_filter(oracle):
+    """The SPPF pooling (5x5, stride 1, pad 2) is a maximum filter with a minimum-value border."""
+    rng = np.random.default_rng(9)
+    x = _rand(rng, (3, 20, 20, 6))
+    want = ndimage.maximum_filter(x, size=(1, 5, 5, 1), mode="constant", cval=-128)
+    np.testing.assert_array_equal(oracle.max_pool(x, (5, 5), (1, 1), (2, 2, 2, 2)), want)
+
+
+def test_resize_nearest_integer_scales_are_numpy_repeat(oracle):
+    rng = np.random.default_rng(10)
+    x = _rand(rng, (2, 5, 7, 6))
+    for sh, sw in ((2, 2), (1, 2), (3, 1), (2, 4), (1, 1)):
+        want = np.repeat(np.repeat(x, sh, axis=1), sw, axis=2)
+        np.testing.assert_array_equal(oracle.resize_nearest_s8(x, sh, sw), want)
+
+
+@pytest.mark.parametrize("scale_h,scale_w", [(1.5, 2.5), (0.5, 0.5), (0.75, 1.25), (2.0, 3.0)])
+def test_resize_nearest_coordinates_are_floor_of_exact_quotient(oracle, scale_h, scale_w):
+    """Scales with an exact binary reciprocal or small numerators: float32 (int)(o * (1 / s)) equals
+    floor(o / s) computed in rationals, clipped to the last row / column."""
+    rng = np.random.default_rng(11)
+    x = _rand(rng, (1, 8, 12, 3))
+    got = oracle.resize_nearest_s8(x, scale_h, scale_w)
+    oh, ow = int(8 * scale_h), int(12 * scale_w)
+    assert got.shape == (1, oh, ow, 3)
+    for oy in range(oh):
+        iy = min(int(Fraction(oy) / Fraction(scale_h)), 7)
+        for ox in range(ow):
+            ix = min(int(Fraction(ox) / Fraction(scale_w)), 11)
+            np.testing.assert_array_equal(got[0, oy, ox], x[0, iy, ix])
+
+
+def test_resize_nearest_values_exhaustive(oracle):
+    """All 256 int8 inputs: a larger output exponent is the round-half-up shift (pinned separately);
+    a smaller one multiplies by 2^k and wraps to int8, as the reference's unsaturated store does."""
+    x = np.arange(-128, 128, dtype=np.int8).reshape(1, 16, 16, 1)
+    for d in range(0, 8):
+        got = oracle.resize_nearest_s8(x, 1, 1, in_exp=-5, out_exp=-5 + d).ravel()
+        want = [bf.round_half_up_exact(int(v), d) if d > 0 else int(v) for v in x.ravel()]
+        np.testing.assert_array_equal(got, np.array(want, dtype=np.int64).astype(np.int8))
+    for d in range(1, 4):
+        got = oracle.resize_nearest_s8(x, 1, 1, in_exp=-5, out_exp=-5 - d).ravel()
+        want = ((x.ravel().astype(np.int64) << d) & 0xff).astype(np.uint8).view(np.int8)
+        np.testing.assert_array_equal(got, want)
