@@ -66,6 +66,14 @@ def lib():
         L.espdl_hip_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp]
         L.espdl_hip_requantize_s8.argtypes = [vp, i64, i32, i32, vp, vp]
         L.espdl_hip_requantize.argtypes = [vp, i32, i64, i32, i32, vp, i32, vp]
+        f32 = ctypes.c_float
+        L.espdl_hip_concat.argtypes = [i32, vp, vp, i64, vp, vp]
+        L.espdl_hip_copy_rows.argtypes = [vp, i64, vp, i64, i64, i64, vp]
+        L.espdl_hip_transpose.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
+        L.espdl_hip_resize_nearest_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, vp, vp]
+        L.espdl_hip_max_pool.argtypes = [vp, i32] + [i32] * 12 + [vp, vp]
+        for name in ("concat", "copy_rows", "transpose", "resize_nearest_s8", "max_pool"):
+            getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         mp = ctypes.POINTER(MbconvDesc)
         L.espdl_hip_mbconv_out_shape.argtypes = [mp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
         L.espdl_hip_mbconv_s8_supported.argtypes = [mp]
@@ -236,4 +244,83 @@ def requantize(x, in_exp, out_exp, out_dtype=None, out=None, stream=None):
     bits = lambda d: S16 if d == torch.int16 else S8  # noqa: E731
     _check(lib().espdl_hip_requantize(_p(x), bits(x.dtype), x.numel(), in_exp, out_exp, _p(out), bits(out.dtype),
                                       _stream(stream)))
+    return out
+
+
+def _prod(xs):
+    n = 1
+    for x in xs:
+        n *= int(x)
+    return n
+
+
+def concat(tensors, axis, out=None, stream=None):
+    """Concat of contiguous device tensors along axis (any element type)."""
+    import torch
+    nd = tensors[0].dim()
+    axis = axis + nd if axis < 0 else axis
+    esize = tensors[0].element_size()
+    shape = list(tensors[0].shape)
+    shape[axis] = sum(int(t.shape[axis]) for t in tensors)
+    out = torch.empty(shape, dtype=tensors[0].dtype, device=tensors[0].device) if out is None else out
+    n = len(tensors)
+    ptrs = (ctypes.c_void_p * n)(*[t.data_ptr() for t in tensors])
+    nbytes = (ctypes.c_int64 * n)(*[_prod(t.shape[axis:]) * esize for t in tensors])
+    _check(lib().espdl_hip_concat(n, ptrs, nbytes, _prod(shape[:axis]), _p(out), _stream(stream)))
+    return out
+
+
+def split(x, axis, sizes, stream=None):
+    """Consecutive pieces of the given sizes along axis, each a new contiguous tensor."""
+    import torch
+    axis = axis + x.dim() if axis < 0 else axis
+    esize = x.element_size()
+    num_slices, slice_size = _prod(x.shape[:axis]), _prod(x.shape[axis + 1:])
+    outs, start = [], 0
+    for sz in sizes:
+        shape = list(x.shape)
+        shape[axis] = int(sz)
+        out = torch.empty(shape, dtype=x.dtype, device=x.device)
+        row = slice_size * int(sz) * esize
+        _check(lib().espdl_hip_copy_rows(ctypes.c_void_p(x.data_ptr() + start * slice_size * esize),
+                                         slice_size * int(x.shape[axis]) * esize, _p(out), row, row, num_slices,
+                                         _stream(stream)))
+        outs.append(out)
+        start += int(sz)
+    return outs
+
+
+def transpose(x, perm=None, out=None, stream=None):
+    import torch
+    nd = x.dim()
+    perm = list(perm) if perm else []
+    full = [p + nd if p < 0 else p for p in perm] if perm else list(range(nd - 1, -1, -1))
+    out = torch.empty([x.shape[p] for p in full], dtype=x.dtype, device=x.device) if out is None else out
+    shape = (ctypes.c_int32 * nd)(*x.shape)
+    pv = (ctypes.c_int32 * max(1, len(perm)))(*perm) if perm else None
+    _check(lib().espdl_hip_transpose(_p(x), shape, nd, pv, len(perm), x.element_size(), _p(out), _stream(stream)))
+    return out
+
+
+def resize_nearest_s8(x, scale_h, scale_w, in_exp=0, out_exp=0, out_hw=None, out=None, stream=None):
+    import numpy as np
+    import torch
+    n, h, w, c = x.shape
+    oh, ow = out_hw if out_hw is not None else (int(h * np.float32(scale_h)), int(w * np.float32(scale_w)))
+    out = torch.empty((n, oh, ow, c), dtype=torch.int8, device=x.device) if out is None else out
+    _check(lib().espdl_hip_resize_nearest_s8(_p(x), n, h, w, c, oh, ow, float(scale_h), float(scale_w), in_exp, out_exp,
+                                             _p(out), _stream(stream)))
+    return out
+
+
+def max_pool(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0), out=None, stream=None):
+    """pads = (top, bottom, left, right); x int8 or int16 NHWC."""
+    import torch
+    n, h, w, c = x.shape
+    pt, pb, pl, pr = pads
+    oh = (h + pt + pb - kernel[0]) // strides[0] + 1
+    ow = (w + pl + pr - kernel[1]) // strides[1] + 1
+    out = torch.empty((n, max(oh, 0), max(ow, 0), c), dtype=x.dtype, device=x.device) if out is None else out
+    _check(lib().espdl_hip_max_pool(_p(x), S16 if x.dtype == torch.int16 else S8, n, h, w, c, kernel[0], kernel[1],
+                                    strides[0], strides[1], pt, pb, pl, pr, _p(out), _stream(stream)))
     return out

@@ -7,6 +7,7 @@
 #include <cstdio>
 
 #include "espdl_kernels.h"
+#include <vector>
 
 namespace {
 
@@ -334,6 +335,125 @@ int espdl_hip_requantize(const void *in, int32_t in_dtype, int64_t size, int32_t
     return device_status(espdl::launch_requantize_any(in, in_dtype, size, in_exp, out_exp, out, out_dtype,
                                                       reinterpret_cast<hipStream_t>(stream)),
                          "requantize");
+}
+
+int espdl_hip_concat(int32_t n_inputs, const void *const *inputs, const int64_t *copy_bytes, int64_t loop_times,
+                     void *out, void *stream)
+{
+    if (n_inputs < 0 || loop_times < 0 || (n_inputs > 0 && (inputs == nullptr || copy_bytes == nullptr)))
+        return fail(ESPDL_HIP_EINVAL, "bad concat arguments");
+    std::vector<long long> bytes((size_t)n_inputs);
+    long long total = 0;
+    for (int j = 0; j < n_inputs; j++) {
+        if (copy_bytes[j] < 0 || (copy_bytes[j] > 0 && inputs[j] == nullptr))
+            return fail(ESPDL_HIP_EINVAL, "concat input %d: null pointer or negative size", j);
+        bytes[(size_t)j] = copy_bytes[j];
+        total += copy_bytes[j];
+    }
+    if (total == 0 || loop_times == 0)
+        return ESPDL_HIP_OK;
+    if (out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "out must not be NULL");
+    return device_status(espdl::launch_concat(n_inputs, inputs, bytes.data(), loop_times, out, cu_count_cached(),
+                                              reinterpret_cast<hipStream_t>(stream)),
+                         "concat");
+}
+
+int espdl_hip_copy_rows(const void *src, int64_t src_pitch, void *dst, int64_t dst_pitch, int64_t row_bytes,
+                        int64_t rows, void *stream)
+{
+    if (rows < 0 || row_bytes < 0 || src_pitch < 0 || dst_pitch < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size or pitch");
+    if (rows == 0 || row_bytes == 0)
+        return ESPDL_HIP_OK;
+    if (src == nullptr || dst == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "src and dst must not be NULL");
+    if (rows > 1 && (src_pitch < row_bytes || dst_pitch < row_bytes))
+        return fail(ESPDL_HIP_EINVAL, "pitches must be at least row_bytes");
+    return device_status(espdl::launch_copy_rows(src, src_pitch, dst, dst_pitch, row_bytes, rows, cu_count_cached(),
+                                                 reinterpret_cast<hipStream_t>(stream)),
+                         "copy_rows");
+}
+
+int espdl_hip_transpose(const void *in, const int32_t *shape, int32_t dims, const int32_t *perm, int32_t n_perm,
+                        int32_t elem_size, void *out, void *stream)
+{
+    if (dims < 1 || dims > 8 || shape == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "transpose handles 1..8 dims");
+    if (elem_size != 1 && elem_size != 2 && elem_size != 4)
+        return fail(ESPDL_HIP_EINVAL, "elem_size must be 1, 2 or 4");
+    if (n_perm != 0 && (n_perm != dims || perm == nullptr))
+        return fail(ESPDL_HIP_EINVAL, "perm must have one entry per dim (or none)");
+    int p[8], sh[8];
+    bool seen[8] = {false, false, false, false, false, false, false, false};
+    long long total = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative extent");
+        sh[i] = shape[i];
+        total *= shape[i];
+        int v = n_perm == 0 ? dims - 1 - i : perm[i];
+        if (v < 0)
+            v += dims;
+        if (v < 0 || v >= dims || seen[v])
+            return fail(ESPDL_HIP_EINVAL, "perm is not a permutation of the dims");
+        seen[v] = true;
+        p[i] = v;
+    }
+    if (total == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    if (misaligned(in, (size_t)elem_size) || misaligned(out, (size_t)elem_size))
+        return fail(ESPDL_HIP_EINVAL, "tensors must be aligned to the element size");
+    return device_status(espdl::launch_transpose(in, sh, dims, p, elem_size, out, cu_count_cached(),
+                                                 reinterpret_cast<hipStream_t>(stream)),
+                         "transpose");
+}
+
+int espdl_hip_resize_nearest_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t out_h,
+                                int32_t out_w, float scale_h, float scale_w, int32_t in_exp, int32_t out_exp,
+                                int8_t *out, void *stream)
+{
+    if (batch < 0 || h <= 0 || w <= 0 || c <= 0 || out_h < 0 || out_w < 0 || !(scale_h > 0) || !(scale_w > 0))
+        return fail(ESPDL_HIP_EINVAL, "bad resize geometry");
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (out_exp - in_exp > 30 || in_exp - out_exp > 30)
+        return fail(ESPDL_HIP_EINVAL, "exponent difference out of range");
+    if ((long long)batch * out_h * out_w == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_resize_nearest_s8(in, batch, h, w, c, out_h, out_w, scale_h, scale_w, in_exp,
+                                                         out_exp, out, cu_count_cached(),
+                                                         reinterpret_cast<hipStream_t>(stream)),
+                         "resize_nearest_s8");
+}
+
+int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h,
+                       int32_t k_w, int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom,
+                       int32_t pad_left, int32_t pad_right, void *out, void *stream)
+{
+    if (dtype != ESPDL_HIP_S8 && dtype != ESPDL_HIP_S16)
+        return fail(ESPDL_HIP_EINVAL, "dtype must be ESPDL_HIP_S8 or ESPDL_HIP_S16");
+    if (batch < 0 || h <= 0 || w <= 0 || c <= 0 || k_h <= 0 || k_w <= 0 || stride_h <= 0 || stride_w <= 0 || pad_top < 0 ||
+        pad_bottom < 0 || pad_left < 0 || pad_right < 0)
+        return fail(ESPDL_HIP_EINVAL, "bad max_pool geometry");
+    if (h + pad_top + pad_bottom < k_h || w + pad_left + pad_right < k_w)
+        return fail(ESPDL_HIP_EINVAL, "window larger than the padded image");
+    const int out_h = (h + pad_top + pad_bottom - k_h) / stride_h + 1, out_w = (w + pad_left + pad_right - k_w) / stride_w + 1;
+    if (batch == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    const int esize = dtype == ESPDL_HIP_S8 ? 1 : 2;
+    if (misaligned(in, (size_t)esize) || misaligned(out, (size_t)esize))
+        return fail(ESPDL_HIP_EINVAL, "int16 tensors must be 2-byte aligned");
+    return device_status(espdl::launch_max_pool(in, esize, batch, h, w, c, k_h, k_w, stride_h, stride_w, pad_top, pad_left,
+                                                out_h, out_w, out, cu_count_cached(),
+                                                reinterpret_cast<hipStream_t>(stream)),
+                         "max_pool");
 }
 
 } // extern "C"

@@ -100,4 +100,18 @@ hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int 
 hipError_t launch_requantize_any(const void *in, int in_bits, int64_t size, int in_exp, int out_exp, void *out,
                                  int out_bits, hipStream_t stream);
 
+// Data-movement operators (layout_ops.hip).
+hipError_t launch_copy_rows(const void *src, long long src_pitch, void *dst, long long dst_pitch, long long row_bytes,
+                            long long rows, int cu_count, hipStream_t stream);
+hipError_t launch_concat(int n_inputs, const void *const *inputs, const long long *copy_bytes, long long loop_times,
+                         void *out, int cu_count, hipStream_t stream);
+hipError_t launch_transpose(const void *in, const int *shape, int dims, const int *perm, int elem_size, void *out,
+                            int cu_count, hipStream_t stream);
+hipError_t launch_resize_nearest_s8(const int8_t *in, int batch, int h, int w, int c, int out_h, int out_w, float scale_h,
+                                    float scale_w, int in_exp, int out_exp, int8_t *out, int cu_count,
+                                    hipStream_t stream);
+hipError_t launch_max_pool(const void *in, int elem_size, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
+                           int stride_w, int pad_top, int pad_left, int out_h, int out_w, void *out, int cu_count,
+                           hipStream_t stream);
+
 } // namespace espdl

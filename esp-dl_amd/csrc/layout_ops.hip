@@ -1,0 +1,496 @@
+// Data-movement operators of detection necks for gfx950: Concat, Split (row copies), Transpose,
+// Resize (nearest) and MaxPool.  All are HBM-bound byte movers: every path moves 16 bytes per thread
+// when pointers, pitches and channel counts allow, and falls back to narrower accesses otherwise.
+//
+// Reference behaviour:
+//   Concat     esp-dl/dl/module/include/dl_module_concat.hpp:86-108  (loop_times x one run per input)
+//   Split      esp-dl/dl/module/include/dl_module_split.hpp:84-93    (num_slices runs per output)
+//   Transpose  esp-dl/dl/tensor/src/dl_tensor_base.cpp:722-812
+//   Resize     esp-dl/dl/base/dl_base_resize.cpp:7-34, 236-268 (nearest; "asymmetric" coordinates)
+//   MaxPool    esp-dl/dl/base/dl_base_max_pool2d.cpp:9-29 on the window clipped to the image
+#include "espdl_device.h"
+#include "espdl_kernels.h"
+
+namespace espdl {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kMaxSeg = 8;
+
+// ------------------------------------------------------------------------------------------------
+// Row copies: `rows` runs of `row_bytes` bytes, run r at src + r * src_pitch -> dst + r * dst_pitch.
+// ------------------------------------------------------------------------------------------------
+struct RowSeg {
+    const char *src;
+    char *dst;
+    long long src_pitch, dst_pitch, row_bytes;
+    int vec;        // bytes per access: 16, 4 or 1
+    FastDiv per_row; // accesses per row
+};
+struct RowCopyArgs {
+    RowSeg seg[kMaxSeg];
+    long long rows;
+};
+
+__global__ __launch_bounds__(kBlock) void copy_rows_kernel(const RowCopyArgs a)
+{
+    const RowSeg &s = a.seg[blockIdx.y];
+    const long long total = a.rows * s.per_row.d;
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < total; i += (long long)gridDim.x * kBlock) {
+        long long r;
+        unsigned c;
+        if (total <= 0x7fffffffll) { // range in which fastdiv is exact
+            r = fastdiv((unsigned)i, s.per_row);
+            c = (unsigned)i - (unsigned)r * s.per_row.d;
+        } else {
+            r = i / s.per_row.d;
+            c = (unsigned)(i - r * s.per_row.d);
+        }
+        const char *sp = s.src + r * s.src_pitch + (long long)c * s.vec;
+        char *dp = s.dst + r * s.dst_pitch + (long long)c * s.vec;
+        if (s.vec == 16)
+            *reinterpret_cast<v4i *>(dp) = *reinterpret_cast<const v4i *>(sp);
+        else if (s.vec == 4)
+            *reinterpret_cast<int *>(dp) = *reinterpret_cast<const int *>(sp);
+        else
+            *dp = *sp;
+    }
+}
+
+inline int widest_access(const void *a, const void *b, long long p0, long long p1, long long n)
+{
+    const uintptr_t m = reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(b) | (uintptr_t)p0 | (uintptr_t)p1 |
+        (uintptr_t)n;
+    return (m & 15) == 0 ? 16 : ((m & 3) == 0 ? 4 : 1);
+}
+
+inline bool fill_seg(RowSeg &s, const void *src, long long src_pitch, void *dst, long long dst_pitch, long long row_bytes)
+{
+    s.src = static_cast<const char *>(src);
+    s.dst = static_cast<char *>(dst);
+    s.src_pitch = src_pitch;
+    s.dst_pitch = dst_pitch;
+    s.row_bytes = row_bytes;
+    s.vec = widest_access(src, dst, src_pitch, dst_pitch, row_bytes);
+    const long long per_row = row_bytes / s.vec;
+    if (per_row > 0x7fffffffll)
+        return false;
+    s.per_row = make_fastdiv((unsigned)std::max<long long>(per_row, 1));
+    return true;
+}
+
+inline unsigned blocks_for(long long work, int cu_count)
+{
+    const long long want = (work + kBlock - 1) / kBlock;
+    const long long cap = (long long)(cu_count > 0 ? cu_count : 256) * 32; // grid-stride beyond this
+    return (unsigned)std::max<long long>(1, std::min(want, cap));
+}
+
+// ------------------------------------------------------------------------------------------------
+// Transpose.  Dimensions are first simplified on the host (size-1 dims dropped, dims that stay
+// adjacent merged).  If the innermost dim stays innermost the copy is a gather of contiguous runs
+// (general kernel, coalesced on both sides); otherwise a 32x32 tile goes through LDS so that reads
+// run along the input's innermost dim and writes along the output's.
+// ------------------------------------------------------------------------------------------------
+constexpr int kMaxDims = 8;
+struct TransposeArgs {
+    const char *in;
+    char *out;
+    int dims, esize;
+    long long total;
+    int out_shape[kMaxDims];       // output extents, outermost first
+    long long in_stride[kMaxDims]; // element stride in the input of output dim i
+    // tiled path: a = input innermost dim, b = the input dim that becomes the output's innermost
+    int ext_a, ext_b;
+    long long a_out_stride, b_in_stride;
+    int n_batch_dims;
+    int batch_shape[kMaxDims];
+    long long batch_in_stride[kMaxDims], batch_out_stride[kMaxDims];
+    int tiles_a, tiles_b;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transpose_general_kernel(const TransposeArgs a)
+{
+    const T *in = reinterpret_cast<const T *>(a.in);
+    T *out = reinterpret_cast<T *>(a.out);
+    for (long long o = (long long)blockIdx.x * kBlock + threadIdx.x; o < a.total; o += (long long)gridDim.x * kBlock) {
+        long long rem = o, src = 0;
+        for (int d = a.dims - 1; d >= 0; d--) {
+            const long long q = rem / a.out_shape[d];
+            src += (rem - q * a.out_shape[d]) * a.in_stride[d];
+            rem = q;
+        }
+        out[o] = in[src];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void transpose_tiled_kernel(const TransposeArgs a)
+{
+    __shared__ T tile[32][33];
+    const T *in = reinterpret_cast<const T *>(a.in);
+    T *out = reinterpret_cast<T *>(a.out);
+    long long blk = blockIdx.x;
+    const int ta = (int)(blk % a.tiles_a);
+    blk /= a.tiles_a;
+    const int tb = (int)(blk % a.tiles_b);
+    blk /= a.tiles_b;
+    long long in_base = 0, out_base = 0;
+    for (int d = a.n_batch_dims - 1; d >= 0; d--) {
+        const long long q = blk / a.batch_shape[d];
+        const long long i = blk - q * a.batch_shape[d];
+        in_base += i * a.batch_in_stride[d];
+        out_base += i * a.batch_out_stride[d];
+        blk = q;
+    }
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5; // 32 x 8 threads
+    const int a0 = ta * 32, b0 = tb * 32;
+#pragma unroll
+    for (int r = ty; r < 32; r += 8)
+        if (b0 + r < a.ext_b && a0 + tx < a.ext_a)
+            tile[r][tx] = in[in_base + (long long)(b0 + r) * a.b_in_stride + (a0 + tx)];
+    __syncthreads();
+#pragma unroll
+    for (int r = ty; r < 32; r += 8)
+        if (a0 + r < a.ext_a && b0 + tx < a.ext_b)
+            out[out_base + (long long)(a0 + r) * a.a_out_stride + (b0 + tx)] = tile[tx][r];
+}
+
+// ------------------------------------------------------------------------------------------------
+// Resize (nearest) and MaxPool: one thread per (output pixel, channel vector).
+// ------------------------------------------------------------------------------------------------
+struct ResizeArgs {
+    const int8_t *in;
+    int8_t *out;
+    int h, w, c, out_h, out_w;
+    float scale_h_inv, scale_w_inv;
+    int exact2;
+    int rshift, lshift; // value = wrap8((x + round) >> rshift) or wrap8(x << lshift)
+    int vec;            // channels per thread: 16 or 1
+    FastDiv fd_cv, fd_ow, fd_oh;
+    long long total;
+};
+
+__device__ __forceinline__ int resize_value(int x, int rshift, int lshift)
+{
+    // round((float)x * 2^lshift / 2^rshift) with round = floor(v + 0.5): exact in integers
+    return rshift > 0 ? (x + (1 << (rshift - 1))) >> rshift : x << lshift;
+}
+
+__global__ __launch_bounds__(kBlock) void resize_nearest_s8_kernel(const ResizeArgs a)
+{
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < a.total; i += (long long)gridDim.x * kBlock) {
+        // i = ((n * out_h + y) * out_w + x) * cv + v; the host refuses totals of 2^31 and more
+        const unsigned pix = fastdiv((unsigned)i, a.fd_cv);
+        const unsigned v = (unsigned)i - pix * a.fd_cv.d;
+        const unsigned row = fastdiv(pix, a.fd_ow);
+        const unsigned x = pix - row * a.fd_ow.d;
+        const unsigned n = fastdiv(row, a.fd_oh);
+        const unsigned y = row - n * a.fd_oh.d;
+        int in_y = a.exact2 ? (int)(y >> 1) : (int)((float)y * a.scale_h_inv);
+        int in_x = a.exact2 ? (int)(x >> 1) : (int)((float)x * a.scale_w_inv);
+        in_y = min(in_y, a.h - 1);
+        in_x = min(in_x, a.w - 1);
+        const long long src = (((long long)n * a.h + in_y) * a.w + in_x) * a.c + (long long)v * a.vec;
+        const long long dst = (long long)pix * a.c + (long long)v * a.vec;
+        if (a.vec == 16) {
+            v4i d = *reinterpret_cast<const v4i *>(a.in + src);
+            if (a.rshift | a.lshift) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    int o = 0;
+#pragma unroll
+                    for (int b = 0; b < 4; b++)
+                        o |= (resize_value((int)(int8_t)(d[k] >> (8 * b)), a.rshift, a.lshift) & 0xff) << (8 * b);
+                    d[k] = o;
+                }
+            }
+            *reinterpret_cast<v4i *>(a.out + dst) = d;
+        } else {
+            a.out[dst] = (int8_t)resize_value((int)a.in[src], a.rshift, a.lshift);
+        }
+    }
+}
+
+struct PoolArgs {
+    const char *in;
+    char *out;
+    int h, w, c, out_h, out_w;
+    int k_h, k_w, stride_h, stride_w, pad_top, pad_left;
+    int vec; // elements per thread: 16 / 8 (vector path) or 1
+    FastDiv fd_cv, fd_ow, fd_oh;
+    long long total;
+};
+
+typedef signed char v16c __attribute__((ext_vector_type(16)));
+typedef short v8s __attribute__((ext_vector_type(8)));
+
+template <typename T, typename V>
+__global__ __launch_bounds__(kBlock) void max_pool_kernel(const PoolArgs a)
+{
+    const T *in = reinterpret_cast<const T *>(a.in);
+    T *out = reinterpret_cast<T *>(a.out);
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < a.total; i += (long long)gridDim.x * kBlock) {
+        const unsigned pix = fastdiv((unsigned)i, a.fd_cv);
+        const unsigned v = (unsigned)i - pix * a.fd_cv.d;
+        const unsigned row = fastdiv(pix, a.fd_ow);
+        const unsigned x = pix - row * a.fd_ow.d;
+        const unsigned n = fastdiv(row, a.fd_oh);
+        const unsigned y = row - n * a.fd_oh.d;
+        const int iy0 = (int)y * a.stride_h - a.pad_top, ix0 = (int)x * a.stride_w - a.pad_left;
+        const int ky0 = max(0, -iy0), ky1 = min(a.k_h, a.h - iy0);
+        const int kx0 = max(0, -ix0), kx1 = min(a.k_w, a.w - ix0);
+        const long long img = (long long)n * a.h * a.w;
+        const long long dst = (long long)pix * a.c + (long long)v * a.vec;
+        if (a.vec > 1) {
+            V best = {}; // an empty clipped window (pads >= kernel) stores zeros
+            bool have = false;
+            for (int ky = ky0; ky < ky1; ky++)
+                for (int kx = kx0; kx < kx1; kx++) {
+                    const V cur = *reinterpret_cast<const V *>(in + (img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.c +
+                                                               (long long)v * a.vec);
+                    best = have ? __builtin_elementwise_max(best, cur) : cur;
+                    have = true;
+                }
+            *reinterpret_cast<V *>(out + dst) = best;
+        } else {
+            int best = 0;
+            bool have = false;
+            for (int ky = ky0; ky < ky1; ky++)
+                for (int kx = kx0; kx < kx1; kx++) {
+                    const int cur = in[(img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.c + v];
+                    best = have ? max(best, cur) : cur;
+                    have = true;
+                }
+            out[dst] = (T)best;
+        }
+    }
+}
+
+} // namespace
+
+hipError_t launch_copy_rows(const void *src, long long src_pitch, void *dst, long long dst_pitch, long long row_bytes,
+                            long long rows, int cu_count, hipStream_t stream)
+{
+    if (rows <= 0 || row_bytes <= 0)
+        return hipSuccess;
+    RowCopyArgs a;
+    a.rows = rows;
+    if (!fill_seg(a.seg[0], src, src_pitch, dst, dst_pitch, row_bytes))
+        return hipErrorInvalidValue;
+    hipLaunchKernelGGL(copy_rows_kernel, dim3(blocks_for(rows * a.seg[0].per_row.d, cu_count), 1), dim3(kBlock), 0, stream,
+                       a);
+    return hipGetLastError();
+}
+
+hipError_t launch_concat(int n_inputs, const void *const *inputs, const long long *copy_bytes, long long loop_times,
+                         void *out, int cu_count, hipStream_t stream)
+{
+    long long total = 0;
+    for (int j = 0; j < n_inputs; j++)
+        total += copy_bytes[j];
+    if (loop_times <= 0 || total <= 0)
+        return hipSuccess;
+    long long prefix = 0;
+    for (int j0 = 0; j0 < n_inputs; j0 += kMaxSeg) {
+        RowCopyArgs a;
+        a.rows = loop_times;
+        int n = 0;
+        long long most = 0;
+        for (int j = j0; j < n_inputs && n < kMaxSeg; j++) {
+            if (copy_bytes[j] > 0) {
+                if (!fill_seg(a.seg[n], inputs[j], copy_bytes[j], static_cast<char *>(out) + prefix, total, copy_bytes[j]))
+                    return hipErrorInvalidValue;
+                most = std::max<long long>(most, loop_times * a.seg[n].per_row.d);
+                n++;
+            }
+            prefix += copy_bytes[j];
+        }
+        if (n > 0)
+            hipLaunchKernelGGL(copy_rows_kernel, dim3(blocks_for(most, cu_count), (unsigned)n), dim3(kBlock), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_transpose(const void *in, const int *shape, int dims, const int *perm, int elem_size, void *out,
+                            int cu_count, hipStream_t stream)
+{
+    // simplify: drop extent-1 dims, then merge input dims that are adjacent and in order in the output
+    int s_shape[kMaxDims], s_perm[kMaxDims], n = 0;
+    {
+        int keep[kMaxDims], newidx[kMaxDims];
+        for (int i = 0; i < dims; i++) {
+            keep[i] = shape[i] != 1;
+            newidx[i] = keep[i] ? n : -1;
+            if (keep[i])
+                s_shape[n++] = shape[i];
+        }
+        int m = 0;
+        for (int i = 0; i < dims; i++)
+            if (keep[perm[i]])
+                s_perm[m++] = newidx[perm[i]];
+    }
+    long long total = 1;
+    for (int i = 0; i < dims; i++)
+        total *= shape[i];
+    if (total == 0)
+        return hipSuccess;
+    bool merged = true;
+    while (merged && n > 1) {
+        merged = false;
+        for (int i = 0; i + 1 < n; i++)
+            if (s_perm[i + 1] == s_perm[i] + 1) { // input dims p, p+1 stay adjacent: one dim
+                const int p = s_perm[i];
+                s_shape[p] *= s_shape[p + 1];
+                for (int k = p + 1; k + 1 < n; k++)
+                    s_shape[k] = s_shape[k + 1];
+                for (int k = i + 1; k + 1 < n; k++)
+                    s_perm[k] = s_perm[k + 1];
+                n--;
+                for (int k = 0; k < n; k++)
+                    if (s_perm[k] > p)
+                        s_perm[k]--;
+                merged = true;
+                break;
+            }
+    }
+    if (n <= 1) // identity
+        return hipMemcpyAsync(out, in, (size_t)(total * elem_size), hipMemcpyDeviceToDevice, stream);
+
+    TransposeArgs a = {};
+    a.in = static_cast<const char *>(in);
+    a.out = static_cast<char *>(out);
+    a.dims = n;
+    a.esize = elem_size;
+    a.total = total;
+    long long in_stride[kMaxDims], out_stride[kMaxDims];
+    in_stride[n - 1] = 1;
+    for (int i = n - 2; i >= 0; i--)
+        in_stride[i] = in_stride[i + 1] * s_shape[i + 1];
+    for (int i = 0; i < n; i++) {
+        a.out_shape[i] = s_shape[s_perm[i]];
+        a.in_stride[i] = in_stride[s_perm[i]];
+    }
+    out_stride[n - 1] = 1;
+    for (int i = n - 2; i >= 0; i--)
+        out_stride[i] = out_stride[i + 1] * a.out_shape[i + 1];
+
+    if (s_perm[n - 1] != n - 1) {
+        // tiled path
+        const int da = n - 1, db = s_perm[n - 1];
+        int pos_a = 0;
+        for (int i = 0; i < n; i++)
+            if (s_perm[i] == da)
+                pos_a = i;
+        a.ext_a = s_shape[da];
+        a.ext_b = s_shape[db];
+        a.a_out_stride = out_stride[pos_a];
+        a.b_in_stride = in_stride[db];
+        a.tiles_a = (a.ext_a + 31) / 32;
+        a.tiles_b = (a.ext_b + 31) / 32;
+        long long blocks = (long long)a.tiles_a * a.tiles_b;
+        for (int i = 0; i < n; i++) { // the other dims, in output order
+            const int d = s_perm[i];
+            if (d == da || d == db)
+                continue;
+            a.batch_shape[a.n_batch_dims] = s_shape[d];
+            a.batch_in_stride[a.n_batch_dims] = in_stride[d];
+            a.batch_out_stride[a.n_batch_dims] = out_stride[i];
+            a.n_batch_dims++;
+            blocks *= s_shape[d];
+        }
+        if (blocks > 0x7fffffffll)
+            return hipErrorInvalidValue;
+        const dim3 grid((unsigned)blocks);
+        if (elem_size == 1)
+            hipLaunchKernelGGL(transpose_tiled_kernel<int8_t>, grid, dim3(kBlock), 0, stream, a);
+        else if (elem_size == 2)
+            hipLaunchKernelGGL(transpose_tiled_kernel<int16_t>, grid, dim3(kBlock), 0, stream, a);
+        else
+            hipLaunchKernelGGL(transpose_tiled_kernel<int32_t>, grid, dim3(kBlock), 0, stream, a);
+        return hipGetLastError();
+    }
+    const dim3 grid(blocks_for(total, cu_count));
+    if (elem_size == 1)
+        hipLaunchKernelGGL(transpose_general_kernel<int8_t>, grid, dim3(kBlock), 0, stream, a);
+    else if (elem_size == 2)
+        hipLaunchKernelGGL(transpose_general_kernel<int16_t>, grid, dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL(transpose_general_kernel<int32_t>, grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_resize_nearest_s8(const int8_t *in, int batch, int h, int w, int c, int out_h, int out_w, float scale_h,
+                                    float scale_w, int in_exp, int out_exp, int8_t *out, int cu_count,
+                                    hipStream_t stream)
+{
+    ResizeArgs a;
+    a.in = in;
+    a.out = out;
+    a.h = h;
+    a.w = w;
+    a.c = c;
+    a.out_h = out_h;
+    a.out_w = out_w;
+    a.scale_h_inv = 1 / scale_h;
+    a.scale_w_inv = 1 / scale_w;
+    a.exact2 = scale_h == 2 && scale_w == 2;
+    const int d = out_exp - in_exp;
+    a.rshift = d > 0 ? d : 0;
+    a.lshift = d < 0 ? -d : 0;
+    const bool vec_ok = (c & 15) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    a.vec = vec_ok ? 16 : 1;
+    const int cv = c / a.vec;
+    a.total = (long long)batch * out_h * out_w * cv;
+    if (a.total <= 0)
+        return hipSuccess;
+    if (a.total > 0x7fffffffll) // fastdiv range
+        return hipErrorInvalidValue;
+    a.fd_cv = make_fastdiv((unsigned)cv);
+    a.fd_ow = make_fastdiv((unsigned)out_w);
+    a.fd_oh = make_fastdiv((unsigned)out_h);
+    hipLaunchKernelGGL(resize_nearest_s8_kernel, dim3(blocks_for(a.total, cu_count)), dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_max_pool(const void *in, int elem_size, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
+                           int stride_w, int pad_top, int pad_left, int out_h, int out_w, void *out, int cu_count,
+                           hipStream_t stream)
+{
+    PoolArgs a;
+    a.in = static_cast<const char *>(in);
+    a.out = static_cast<char *>(out);
+    a.h = h;
+    a.w = w;
+    a.c = c;
+    a.out_h = out_h;
+    a.out_w = out_w;
+    a.k_h = k_h;
+    a.k_w = k_w;
+    a.stride_h = stride_h;
+    a.stride_w = stride_w;
+    a.pad_top = pad_top;
+    a.pad_left = pad_left;
+    const int per_vec = 16 / elem_size;
+    const bool vec_ok = (c % per_vec) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    a.vec = vec_ok ? per_vec : 1;
+    const int cv = c / a.vec;
+    a.total = (long long)batch * out_h * out_w * cv;
+    if (a.total <= 0)
+        return hipSuccess;
+    if (a.total > 0x7fffffffll) // fastdiv range
+        return hipErrorInvalidValue;
+    a.fd_cv = make_fastdiv((unsigned)cv);
+    a.fd_ow = make_fastdiv((unsigned)out_w);
+    a.fd_oh = make_fastdiv((unsigned)out_h);
+    const dim3 grid(blocks_for(a.total, cu_count));
+    if (elem_size == 1)
+        hipLaunchKernelGGL((max_pool_kernel<int8_t, v16c>), grid, dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL((max_pool_kernel<int16_t, v8s>), grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+} // namespace espdl

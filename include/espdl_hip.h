@@ -141,6 +141,46 @@ int espdl_hip_requantize(const void *in, int32_t in_dtype, int64_t size, int32_t
                          int32_t out_dtype, void *stream);
 
 /*
+ * module::Concat::forward_template (esp-dl/dl/module/include/dl_module_concat.hpp:86-108): for each of
+ * the loop_times outer positions (product of the dims before the axis) one contiguous run from every
+ * input in turn; copy_bytes[j] = bytes input j contributes per position (product of its dims from the
+ * axis on, times the element size).  `inputs` and `copy_bytes` are host arrays of n_inputs entries read
+ * during the call; inputs[j] are device pointers.  Any element type.
+ */
+int espdl_hip_concat(int32_t n_inputs, const void *const *inputs, const int64_t *copy_bytes, int64_t loop_times,
+                     void *out, void *stream);
+
+/* `rows` runs of row_bytes bytes, run r from src + r * src_pitch to dst + r * dst_pitch.  One output of
+ * module::Split (esp-dl/dl/module/include/dl_module_split.hpp:84-93) is this with rows = num_slices,
+ * row_bytes = slice_size * out_axis * sizeof(T), src_pitch = slice_size * in_axis * sizeof(T),
+ * src = input + slice_index * slice_size * sizeof(T), dst_pitch = row_bytes. */
+int espdl_hip_copy_rows(const void *src, int64_t src_pitch, void *dst, int64_t dst_pitch, int64_t row_bytes,
+                        int64_t rows, void *stream);
+
+/* TensorBase::transpose (esp-dl/dl/tensor/src/dl_tensor_base.cpp:722-812): out.shape[i] =
+ * shape[perm[i]].  1..8 dims, elem_size 1, 2 or 4 bytes; perm entries may be negative (counted from
+ * the end) and n_perm = 0 reverses the dims.  shape and perm are host arrays. */
+int espdl_hip_transpose(const void *in, const int32_t *shape, int32_t dims, const int32_t *perm, int32_t n_perm,
+                        int32_t elem_size, void *out, void *stream);
+
+/* base::resize<int8_t> in nearest mode (esp-dl/dl/base/dl_base_resize.cpp:7-34, 236-268; arguments
+ * esp-dl/dl/base/dl_base_resize.hpp:37-92) on [batch][h][w][c] -> [batch][out_h][out_w][c].
+ * scale_h / scale_w are the module's float scales (output / input); exactly 2 x 2 replicates pixels,
+ * any other scale maps coordinates with in = min((int)(out * (1 / scale)), len - 1).  A different
+ * output exponent rescales with round-half-up and, like the reference, without saturation. */
+int espdl_hip_resize_nearest_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t out_h,
+                                int32_t out_w, float scale_h, float scale_w, int32_t in_exp, int32_t out_exp,
+                                int8_t *out, void *stream);
+
+/* base::max_pool2d (esp-dl/dl/base/dl_base_max_pool2d.cpp:9-29) over the window clipped to the image;
+ * output size (h + pad_top + pad_bottom - k_h) / stride_h + 1 and likewise for the width
+ * (esp-dl/dl/module/include/dl_module_max_pool.hpp:42-49).  dtype ESPDL_HIP_S8 or ESPDL_HIP_S16; the
+ * exponent is unchanged.  out is [batch][out_h][out_w][c]. */
+int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h,
+                       int32_t k_w, int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom,
+                       int32_t pad_left, int32_t pad_right, void *out, void *stream);
+
+/*
  * Inverted-residual block in one launch: [1x1 Conv] -> depthwise Conv -> 1x1 Conv [-> Add].
  * No single reference function does this; it runs the same sequence of module::Conv::forward
  * (esp-dl/dl/module/include/dl_module_conv.hpp:121-162) and module::Add::forward

@@ -1,0 +1,117 @@
+"""Concat / Split / Transpose / Resize-nearest / MaxPool on the GPU against the CPU oracle (bit-exact)."""
+import numpy as np
+import pytest
+
+from gpu_util import announce, espdl, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(rng, shape, dtype=np.int8):
+    info = np.iinfo(dtype)
+    return rng.integers(info.min, info.max + 1, size=shape).astype(dtype)
+
+
+CONCAT_CASES = [
+    # (base shape, axis, extents along the axis)
+    ((2, 20, 20, 0), 3, [64, 64, 64, 64]),      # SPPF: four 16-byte aligned runs
+    ((2, 40, 40, 0), 3, [128, 64]),              # FPN: upsampled + skip
+    ((3, 7, 5, 0), 3, [5, 11, 16]),              # byte paths
+    ((2, 0, 9, 8), 1, [3, 1, 6]),                # an outer axis
+    ((0, 4, 4, 16), 0, [1, 2]),                  # batch axis: one run per input
+    ((1, 4, 4, 0), -1, [4] * 11),                # more inputs than one launch takes
+]
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("case", CONCAT_CASES, ids=lambda c: f"{c[0]}_ax{c[1]}")
+def test_concat(oracle, case, dtype):
+    base, axis, extents = case
+    announce(f"concat {case} {dtype.__name__}")
+    rng = np.random.default_rng(21)
+    arrays = []
+    for e in extents:
+        shape = list(base)
+        shape[axis] = e
+        arrays.append(_rand(rng, shape, dtype))
+    got = to_host(espdl().concat([to_dev(a) for a in arrays], axis))
+    np.testing.assert_array_equal(got, oracle.concat(arrays, axis))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("shape,axis,sizes", [
+    ((2, 20, 20, 128), 3, [64, 64]), ((2, 9, 9, 48), 3, [5, 20, 23]), ((4, 6, 5, 8), 1, [1, 2, 3]),
+    ((5, 3, 3, 4), 0, [2, 3]), ((1, 1, 1, 32), -1, [16, 16]),
+])
+def test_split(oracle, shape, axis, sizes, dtype):
+    announce(f"split {shape} axis {axis} {sizes} {dtype.__name__}")
+    x = _rand(np.random.default_rng(22), shape, dtype)
+    got = espdl().split(to_dev(x), axis, sizes)
+    want = oracle.split(x, axis, sizes)
+    assert len(got) == len(want)
+    for g, w in zip(got, want):
+        np.testing.assert_array_equal(to_host(g), w)
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16, np.int32])
+@pytest.mark.parametrize("shape,perm", [
+    ((2, 20, 20, 64), (0, 3, 1, 2)), ((2, 64, 20, 20), (0, 2, 3, 1)), ((3, 5, 7, 9), None), ((37, 65), (1, 0)),
+    ((4, 1, 1, 1280), (0, 3, 1, 2)), ((2, 3, 4, 5), (0, 1, 2, 3)), ((2, 3, 4, 5), (1, 0, 2, 3)),
+    ((2, 2, 3, 2, 5), (4, 0, 3, 1, 2)), ((2, 3, 33, 40), (0, 1, 3, 2)), ((6,), (0,)), ((2, 3, 4), (-1, 0, 1)),
+])
+def test_transpose(oracle, shape, perm, dtype):
+    announce(f"transpose {shape} {perm} {dtype.__name__}")
+    x = _rand(np.random.default_rng(23), shape, dtype)
+    got = to_host(espdl().transpose(to_dev(x), perm))
+    np.testing.assert_array_equal(got, oracle.transpose(x, perm))
+
+
+@pytest.mark.parametrize("shape,scales,exps", [
+    ((2, 20, 20, 128), (2, 2), (-4, -4)), ((2, 10, 10, 64), (2, 2), (-4, -3)), ((1, 7, 5, 3), (2, 2), (-4, -4)),
+    ((2, 8, 12, 16), (1.5, 2.5), (-4, -4)), ((2, 8, 12, 5), (0.5, 0.5), (-5, -3)), ((1, 6, 6, 32), (3, 1), (-4, -6)),
+    ((1, 9, 9, 16), (1, 1), (0, 2)),
+])
+def test_resize_nearest_s8(oracle, shape, scales, exps):
+    announce(f"resize nearest {shape} x{scales} exps {exps}")
+    x = _rand(np.random.default_rng(24), shape)
+    got = to_host(espdl().resize_nearest_s8(to_dev(x), scales[0], scales[1], exps[0], exps[1]))
+    np.testing.assert_array_equal(got, oracle.resize_nearest_s8(x, scales[0], scales[1], exps[0], exps[1]))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("shape,kernel,strides,pads", [
+    ((2, 20, 20, 128), (5, 5), (1, 1), (2, 2, 2, 2)), ((2, 16, 16, 24), (2, 2), (2, 2), (0, 0, 0, 0)),
+    ((3, 9, 8, 5), (3, 3), (2, 2), (1, 1, 1, 1)), ((1, 11, 7, 16), (3, 2), (1, 2), (1, 0, 0, 1)),
+    ((2, 5, 5, 8), (5, 5), (1, 1), (0, 0, 0, 0)), ((1, 1, 30, 40), (1, 3), (1, 1), (0, 0, 1, 1)),
+])
+def test_max_pool(oracle, shape, kernel, strides, pads, dtype):
+    announce(f"max_pool {shape} k{kernel} s{strides} p{pads} {dtype.__name__}")
+    x = _rand(np.random.default_rng(25), shape, dtype)
+    got = to_host(espdl().max_pool(to_dev(x), kernel, strides, pads))
+    np.testing.assert_array_equal(got, oracle.max_pool(x, kernel, strides, pads))
+
+
+def test_sppf_pool_chain_idempotence():
+    """Size-independent property at full batch: three chained 5x5/1 pools equal one 13x13/1 pool, and
+    pooling is monotone (output >= input)."""
+    import torch
+    m = espdl()
+    announce("max_pool chain 256x20x20x128")
+    x = torch.randint(-128, 128, (256, 20, 20, 128), dtype=torch.int8, device="cuda")
+    p1 = m.max_pool(x, (5, 5), (1, 1), (2, 2, 2, 2))
+    p3 = m.max_pool(m.max_pool(p1, (5, 5), (1, 1), (2, 2, 2, 2)), (5, 5), (1, 1), (2, 2, 2, 2))
+    big = m.max_pool(x, (13, 13), (1, 1), (6, 6, 6, 6))
+    assert torch.equal(p3, big)
+    assert bool((p1 >= x).all())
+
+
+def test_bad_layout_arguments_are_rejected():
+    import torch
+    m = espdl()
+    x = torch.zeros((1, 4, 4, 8), dtype=torch.int8, device="cuda")
+    with pytest.raises(m.EspdlHipError):
+        m.transpose(x, (0, 1, 1, 2))
+    with pytest.raises(m.EspdlHipError):
+        m.max_pool(x, (7, 7))
+    with pytest.raises(m.EspdlHipError):
+        m.resize_nearest_s8(x, 0.0, 2.0, out_hw=(4, 8))
