@@ -15,6 +15,7 @@
 #include "dl_module_conv.hpp"
 #include "dl_module_elementwise.hpp"
 #include "dl_module_gemm.hpp"
+#include "dl_module_layout.hpp"
 
 namespace dl {
 namespace module {
@@ -62,6 +63,11 @@ public:
         register_module("Squeeze", ShapeView::deserialize_squeeze);
         register_module("Unsqueeze", ShapeView::deserialize_unsqueeze);
         register_module("Reshape", ShapeView::deserialize_reshape);
+        register_module("Concat", Concat::deserialize);
+        register_module("Split", Split::deserialize);
+        register_module("Transpose", Transpose::deserialize);
+        register_module("Resize", Resize::deserialize);
+        register_module("MaxPool", MaxPool::deserialize);
         // element-wise activations that esp-ppq exports with a precomputed 8-bit table
         for (const char *op : {"Swish", "HardSwish", "Sigmoid", "HardSigmoid", "Tanh", "Gelu", "Elu", "LeakyRelu",
                                "Exp", "Log", "Sqrt", "Softplus", "Mish"}) {

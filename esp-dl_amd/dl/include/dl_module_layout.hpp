@@ -1,0 +1,397 @@
+// Data-movement operator objects: Concat, Split, Transpose, Resize, MaxPool.  Each mirrors the
+// reference module of the same name (same attributes, shape rules and error behaviour) and enqueues
+// kernels of include/espdl_hip.h on the context's stream.
+//   Concat     esp-dl/dl/module/include/dl_module_concat.hpp:14-127
+//   Split      esp-dl/dl/module/include/dl_module_split.hpp:14-177
+//   Transpose  esp-dl/dl/module/include/dl_module_transpose.hpp:12-88
+//   Resize     esp-dl/dl/module/include/dl_module_resize.hpp:14-180 (nearest mode)
+//   MaxPool    esp-dl/dl/module/include/dl_module_max_pool.hpp:13-131
+#pragma once
+
+#include <cassert>
+#include <cstring>
+
+#include "dl_module_base.hpp"
+#include "dl_module_elementwise.hpp"
+#include "espdl_hip.h"
+
+namespace dl {
+namespace module {
+
+class Concat : public Module {
+private:
+    int m_axis;
+
+public:
+    Concat(const char *name = nullptr, int axis = 0, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_axis(axis)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        assert(!input_shapes.empty());
+        const int dims = (int)input_shapes[0].size();
+        if (m_axis < 0)
+            m_axis += dims;
+        assert(m_axis >= 0 && m_axis < dims);
+        std::vector<int> out = input_shapes[0];
+        out[m_axis] = 0;
+        for (auto &s : input_shapes) {
+            assert((int)s.size() == dims);
+            out[m_axis] += s[m_axis];
+        }
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!output || !output->on_device()) {
+            DL_LOGE("Concat", "%s: needs device tensors", name.c_str());
+            return;
+        }
+        const size_t esize = output->get_dtype_bytes();
+        std::vector<const void *> ptrs;
+        std::vector<int64_t> bytes;
+        int64_t loop_times = 1;
+        for (size_t j = 0; j < m_inputs_index.size(); j++) {
+            TensorBase *input = context->get_tensor(m_inputs_index[j]);
+            if (!input || !input->on_device() || input->dtype != output->dtype) {
+                DL_LOGE("Concat", "%s: input %d is missing, on the host or of another type", name.c_str(), (int)j);
+                return;
+            }
+            int64_t n = 1;
+            for (int i = m_axis; i < (int)input->shape.size(); i++)
+                n *= input->shape[i];
+            if (j == 0)
+                for (int i = 0; i < m_axis; i++)
+                    loop_times *= input->shape[i];
+            ptrs.push_back(input->data);
+            bytes.push_back(n * (int64_t)esize);
+        }
+        const int rc =
+            espdl_hip_concat((int32_t)ptrs.size(), ptrs.data(), bytes.data(), loop_times, output->data, context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Concat", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        int axis = 0;
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "axis", axis);
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        return new Concat(node_name.c_str(), axis, quant_type);
+    }
+    void print() { DL_LOGI("Concat", "axis: %d, quant_type: %s.", m_axis, quant_type_to_string(quant_type)); }
+};
+
+/// With a `split` parameter the outputs take those extents.  Without one the reference makes
+/// ceil(extent / num_outputs) outputs of num_outputs elements each (the last one takes the rest):
+/// the attribute acts as the piece size there, and this class does the same.
+class Split : public Module {
+private:
+    std::vector<int64_t> m_split;
+    int m_axis;
+    int m_num_outputs;
+
+public:
+    Split(const std::vector<int64_t> &split = {}, int axis = 0, int num_outputs = -1, const char *name = nullptr,
+          quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_split(split), m_axis(axis), m_num_outputs(num_outputs)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        assert(!input_shapes[0].empty());
+        if (m_axis < 0)
+            m_axis += (int)input_shapes[0].size();
+        const int extent = input_shapes[0][m_axis];
+        std::vector<std::vector<int>> out;
+        if (!m_split.empty()) {
+            int64_t total = 0;
+            for (int64_t s : m_split) {
+                out.push_back(input_shapes[0]);
+                out.back()[m_axis] = (int)s;
+                total += s;
+            }
+            assert(total == extent);
+            (void)total;
+        } else {
+            assert(m_num_outputs > 0);
+            const int n = (extent + m_num_outputs - 1) / m_num_outputs;
+            for (int i = 0; i < n; i++) {
+                out.push_back(input_shapes[0]);
+                out.back()[m_axis] = i + 1 < n ? m_num_outputs : extent - (n - 1) * m_num_outputs;
+            }
+        }
+        return out;
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        if (!input || !input->on_device() || input->shape.empty()) {
+            DL_LOGE("Split", "%s: needs a device tensor of at least one dim", name.c_str());
+            return;
+        }
+        int64_t num_slices = 1, slice_size = 1;
+        for (int i = 0; i < m_axis; i++)
+            num_slices *= input->shape[i];
+        for (int i = m_axis + 1; i < (int)input->shape.size(); i++)
+            slice_size *= input->shape[i];
+        const int64_t esize = (int64_t)input->get_dtype_bytes();
+        const int64_t in_axis = input->shape[m_axis];
+        int64_t slice_index = 0;
+        for (size_t i = 0; i < m_outputs_index.size(); i++) {
+            TensorBase *output = context->get_tensor(m_outputs_index[i]);
+            if (!output || !output->on_device() || output->dtype != input->dtype) {
+                DL_LOGE("Split", "%s: output %d is missing, on the host or of another type", name.c_str(), (int)i);
+                return;
+            }
+            const int64_t out_axis = output->shape[m_axis];
+            const int64_t row = slice_size * out_axis * esize;
+            const int rc = espdl_hip_copy_rows(static_cast<const char *>(input->data) + slice_index * slice_size * esize,
+                                               slice_size * in_axis * esize, output->data, row, row, num_slices,
+                                               context->stream);
+            if (rc != ESPDL_HIP_OK)
+                DL_LOGE("Split", "%s: %s", name.c_str(), espdl_hip_last_error());
+            slice_index += out_axis;
+        }
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        int axis = 0, num_outputs = -1;
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "axis", axis);
+        fbs_model->get_operation_attribute(node_name, "num_outputs", num_outputs);
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        std::vector<int64_t> split;
+        TensorBase *t = fbs_model->get_operation_parameter(node_name, 1);
+        if (t) {
+            if (t->dtype == DATA_TYPE_INT64) {
+                const int64_t *p = t->get_element_ptr<int64_t>();
+                split.assign(p, p + t->get_size());
+            } else if (t->dtype == DATA_TYPE_INT32) {
+                const int32_t *p = t->get_element_ptr<int32_t>();
+                split.assign(p, p + t->get_size());
+            }
+            delete t;
+        }
+        return new Split(split, axis, num_outputs, node_name.c_str(), quant_type);
+    }
+    void print()
+    {
+        DL_LOGI("Split", "axis: %d, pieces: %d, quant_type: %s.", m_axis, (int)m_split.size(),
+                quant_type_to_string(quant_type));
+    }
+};
+
+class Transpose : public Module {
+private:
+    std::vector<int> m_perm;
+
+public:
+    Transpose(const char *name = nullptr, quant_type_t quant_type = QUANT_TYPE_NONE, std::vector<int> perm = {}) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_perm(perm)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const int dims = (int)input_shapes[0].size();
+        assert((int)m_perm.size() == dims || m_perm.empty());
+        if (m_perm.empty())
+            for (int i = dims - 1; i >= 0; i--)
+                m_perm.push_back(i);
+        std::vector<int> out;
+        for (int i = 0; i < dims; i++) {
+            if (m_perm[i] < 0)
+                m_perm[i] += dims;
+            out.push_back(input_shapes[0][m_perm[i]]);
+        }
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) || input->dtype != output->dtype) {
+            DL_LOGE("Transpose", "%s: needs device tensors of one type", name.c_str());
+            return;
+        }
+        const int rc = espdl_hip_transpose(input->data, input->shape.data(), (int32_t)input->shape.size(), m_perm.data(),
+                                           (int32_t)m_perm.size(), (int32_t)input->get_dtype_bytes(), output->data,
+                                           context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Transpose", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        std::vector<int> perm;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "perm", perm);
+        return new Transpose(node_name.c_str(), quant_type, perm);
+    }
+    void print() { DL_LOGI("Transpose", "dims: %d, quant_type: %s.", (int)m_perm.size(), quant_type_to_string(quant_type)); }
+};
+
+/// Nearest mode on int8 NHWC / NWC tensors.  Scales and sizes are in the exporter's NCHW order
+/// (scales[2] = height, scales[3] = width), as in the reference.
+class Resize : public Module {
+private:
+    std::string m_mode;
+    std::vector<float> m_scales;
+    std::vector<int64_t> m_sizes;
+
+public:
+    Resize(const char *name = nullptr, const std::string &mode = "nearest", const std::vector<float> &scales = {},
+           const std::vector<int64_t> &sizes = {}, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_mode(mode), m_scales(scales), m_sizes(sizes)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        assert(in.size() == 3 || in.size() == 4);
+        std::vector<int> out = in;
+        if (!m_sizes.empty()) {
+            std::vector<float> scales(in.size(), 1.0f);
+            out[1] = (int)m_sizes[2];
+            scales[2] = out[1] / (float)in[1];
+            if (in.size() == 4) {
+                out[2] = (int)m_sizes[3];
+                scales[3] = out[2] / (float)in[2];
+            }
+            m_scales.swap(scales);
+        } else {
+            assert(m_scales.size() == in.size());
+            out[1] = (int)(in[1] * m_scales[2]);
+            if (in.size() == 4)
+                out[2] = (int)(in[2] * m_scales[3]);
+        }
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !on_device_all({input, output}) || m_mode != "nearest") {
+            DL_LOGE("Resize", "%s: this build resizes int8 device tensors in nearest mode only", name.c_str());
+            return;
+        }
+        const bool nwc = input->shape.size() == 3;
+        // NWC runs as one row: height 1, height scale 1 (esp-dl/dl/base/dl_base_resize.hpp:39-51)
+        const int h = nwc ? 1 : input->shape[1], w = nwc ? input->shape[1] : input->shape[2];
+        const int c = nwc ? input->shape[2] : input->shape[3];
+        const int oh = nwc ? 1 : output->shape[1], ow = nwc ? output->shape[1] : output->shape[2];
+        const float sh = nwc ? 1.0f : m_scales[2], sw = nwc ? m_scales[2] : m_scales[3];
+        const int rc = espdl_hip_resize_nearest_s8(static_cast<const int8_t *>(input->data), input->shape[0], h, w, c, oh,
+                                                   ow, sh, sw, input->exponent.get(), output->exponent.get(),
+                                                   static_cast<int8_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Resize", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        std::string mode = "nearest";
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "mode", mode);
+        std::vector<float> scales;
+        TensorBase *st = fbs_model->get_operation_parameter(node_name, 2);
+        if (st && st->dtype == DATA_TYPE_FLOAT) {
+            const float *p = st->get_element_ptr<float>();
+            scales.assign(p, p + st->get_size());
+        }
+        delete st;
+        std::vector<int64_t> sizes;
+        TensorBase *zt = fbs_model->get_operation_parameter(node_name, 3);
+        if (zt && zt->dtype == DATA_TYPE_INT64) {
+            const int64_t *p = zt->get_element_ptr<int64_t>();
+            sizes.assign(p, p + zt->get_size());
+        }
+        delete zt;
+        if (quant_type != QUANT_TYPE_SYMM_8BIT && quant_type != QUANT_TYPE_SYMM_16BIT)
+            return nullptr;
+        return new Resize(node_name.c_str(), mode, scales, sizes, quant_type);
+    }
+    void print() { DL_LOGI("Resize", "mode: %s, quant_type: %s.", m_mode.c_str(), quant_type_to_string(quant_type)); }
+};
+
+class MaxPool : public Module {
+private:
+    std::vector<int> m_filter_shape;
+    std::vector<int> m_padding; ///< [top, bottom, left, right] (NWC: [head, tail])
+    std::vector<int> m_strides;
+
+public:
+    MaxPool(const char *name = nullptr, const std::vector<int> &filter_shape = {2, 2},
+            const std::vector<int> &padding = {0, 0, 0, 0}, const std::vector<int> &strides = {1, 1},
+            quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_filter_shape(filter_shape), m_padding(padding), m_strides(strides)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        assert(in.size() == 3 || in.size() == 4);
+        std::vector<int> out = in;
+        out[1] = (in[1] + m_padding[0] + m_padding[1] - m_filter_shape[0]) / m_strides[0] + 1;
+        if (in.size() == 4)
+            out[2] = (in[2] + m_padding[2] + m_padding[3] - m_filter_shape[1]) / m_strides[1] + 1;
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) ||
+            (quant_type != QUANT_TYPE_SYMM_8BIT && quant_type != QUANT_TYPE_SYMM_16BIT)) {
+            DL_LOGE("MaxPool", "%s: needs int8 / int16 device tensors", name.c_str());
+            return;
+        }
+        const bool nwc = input->shape.size() == 3;
+        const int h = nwc ? 1 : input->shape[1], w = nwc ? input->shape[1] : input->shape[2];
+        const int c = nwc ? input->shape[2] : input->shape[3];
+        const int kh = nwc ? 1 : m_filter_shape[0], kw = nwc ? m_filter_shape[0] : m_filter_shape[1];
+        const int sh = nwc ? 1 : m_strides[0], sw = nwc ? m_strides[0] : m_strides[1];
+        const int pt = nwc ? 0 : m_padding[0], pb = nwc ? 0 : m_padding[1];
+        const int pl = nwc ? m_padding[0] : m_padding[2], pr = nwc ? m_padding[1] : m_padding[3];
+        const int rc = espdl_hip_max_pool(input->data, quant_type == QUANT_TYPE_SYMM_8BIT ? ESPDL_HIP_S8 : ESPDL_HIP_S16,
+                                          input->shape[0], h, w, c, kh, kw, sh, sw, pt, pb, pl, pr, output->data,
+                                          context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("MaxPool", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        std::vector<int> kernel_shape, pads, strides;
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "kernel_shape", kernel_shape);
+        fbs_model->get_operation_attribute(node_name, "pads", pads);
+        fbs_model->get_operation_attribute(node_name, "strides", strides);
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT && quant_type != QUANT_TYPE_SYMM_16BIT)
+            return nullptr;
+        if (kernel_shape.empty())
+            return nullptr;
+        if (pads.size() == 4) // ONNX [top, left, bottom, right] -> [top, bottom, left, right]
+            pads = {pads[0], pads[2], pads[1], pads[3]};
+        else if (pads.empty())
+            pads = {0, 0, 0, 0};
+        if (strides.empty())
+            strides.assign(kernel_shape.size(), 1);
+        return new MaxPool(node_name.c_str(), kernel_shape, pads, strides, quant_type);
+    }
+    void print()
+    {
+        DL_LOGI("MaxPool", "kernel: %dx%d, quant_type: %s.", m_filter_shape[0], m_filter_shape.size() > 1 ? m_filter_shape[1] : 1,
+                quant_type_to_string(quant_type));
+    }
+};
+
+} // namespace module
+} // namespace dl

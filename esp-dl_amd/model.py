@@ -67,7 +67,7 @@ def _dims(d):
     return (ctypes.c_int32 * len(d))(*[int(v) for v in d]), len(d)
 
 
-_NP_OF = {3: np.int8, 5: np.int16, 6: np.int32, 7: np.int64}
+_NP_OF = {1: np.float32, 3: np.int8, 5: np.int16, 6: np.int32, 7: np.int64}
 
 
 class Graph:

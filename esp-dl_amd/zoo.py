@@ -15,8 +15,8 @@ import math
 
 import numpy as np
 
-INT8, INT16, INT32, INT64 = 3, 5, 6, 7
-_NP = {INT8: np.int8, INT16: np.int16, INT32: np.int32, INT64: np.int64}
+FLOAT, INT8, INT16, INT32, INT64 = 1, 3, 5, 6, 7
+_NP = {FLOAT: np.float32, INT8: np.int8, INT16: np.int16, INT32: np.int32, INT64: np.int64}
 
 
 class GraphSpec:
@@ -40,6 +40,7 @@ class GraphSpec:
         self.value_info[name] = (list(dims), dtype, int(exponent))
 
     def add_node(self, name, op_type, inputs, outputs, **attrs):
+        assert all(n["name"] != name for n in self.nodes), "duplicate node name " + name
         self.nodes.append({"name": name, "op_type": op_type, "inputs": list(inputs), "outputs": list(outputs),
                            "attrs": attrs})
 
@@ -258,6 +259,68 @@ class Builder:
         g.add_node(name, "Flatten", [x], [y], axis=1, quant_type="S8")
         return y
 
+    def max_pool(self, x, k, stride=1, pad=None, name=None):
+        g = self.g
+        name = name or self._name("maxpool")
+        _, h, w, c = g.shape(x)
+        pad = k // 2 if pad is None else pad
+        oh, ow = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+        y = name + "_out"
+        g.add_value(y, [1, oh, ow, c], g.exponent(x), g.dtype(x))
+        g.add_node(name, "MaxPool", [x], [y], kernel_shape=[k, k], pads=[pad, pad, pad, pad], strides=[stride, stride],
+                   quant_type="S8")
+        return y
+
+    def concat(self, xs, axis=3, name=None):
+        """Concat at one exponent: inputs at another exponent are requantized to the coarsest one first,
+        as the exporter does."""
+        g = self.g
+        name = name or self._name("concat")
+        e = max(g.exponent(x) for x in xs)
+        xs = [x if g.exponent(x) == e else self.requantize(x, e, name="%s_rq%d" % (name, i)) for i, x in enumerate(xs)]
+        dims = list(g.shape(xs[0]))
+        dims[axis] = sum(g.shape(x)[axis] for x in xs)
+        y = name + "_out"
+        g.add_value(y, dims, e, g.dtype(xs[0]))
+        g.add_node(name, "Concat", xs, [y], axis=axis, quant_type="S8")
+        return y
+
+    def split(self, x, sizes, axis=3, name=None):
+        g = self.g
+        name = name or self._name("split")
+        g.add_init(name + ".split", [len(sizes)], INT64, sizes, [0])
+        outs = []
+        for i, sz in enumerate(sizes):
+            dims = list(g.shape(x))
+            dims[axis] = int(sz)
+            y = "%s_out%d" % (name, i)
+            g.add_value(y, dims, g.exponent(x), g.dtype(x))
+            outs.append(y)
+        g.add_node(name, "Split", [x, name + ".split"], outs, axis=axis, quant_type="S8")
+        return outs
+
+    def resize_nearest(self, x, scale=2, out_exp=None, name=None):
+        g = self.g
+        name = name or self._name("resize")
+        _, h, w, c = g.shape(x)
+        g.add_init(name + ".scales", [4], FLOAT, [1.0, 1.0, float(scale), float(scale)], [0])
+        y = name + "_out"
+        g.add_value(y, [1, int(h * np.float32(scale)), int(w * np.float32(scale)), c],
+                    g.exponent(x) if out_exp is None else out_exp, g.dtype(x))
+        # ONNX inputs: X, roi (absent), scales
+        g.add_node(name, "Resize", [x, "", name + ".scales"], [y], mode="nearest",
+                   coordinate_transformation_mode="asymmetric", quant_type="S8")
+        return y
+
+    def transpose(self, x, perm, name=None):
+        g = self.g
+        name = name or self._name("transpose")
+        dims = g.shape(x)
+        y = name + "_out"
+        g.add_value(y, [dims[p] for p in perm], g.exponent(x), g.dtype(x))
+        g.add_node(name, "Transpose", [x], [y], perm=list(perm), quant_type="S8")
+        return y
+
     def output(self, x):
         self.g.outputs.append(x)
         return x
@@ -350,26 +413,42 @@ def config3_mobilenetv2(seed=0xE5D3, resolution=224, num_classes=1000, width=1.0
 
 
 def c3k2_like(b, x, c_out, name):
-    """YOLO11-style C3k2 / C2f block without Split/Concat (those data-movement ops are outside the
-    conv/gemm path): 1x1 reduce, two 3x3 bottleneck convs with SiLU tables and a residual Add, 1x1 fuse."""
-    g = b.g
-    h = b.conv(x, c_out // 2, k=1, name=name + "_cv1")
+    """YOLO11-style C3k2 / C2f block: 1x1 conv, Split into two halves, a bottleneck (two 3x3 convs with
+    SiLU tables and a residual Add) on the second half, Concat of both halves and the bottleneck output,
+    1x1 fuse."""
+    h = b.conv(x, c_out, k=1, name=name + "_cv1")
     h = b.lut(h, silu, "Swish", name=name + "_cv1_act")
-    m = b.conv(h, c_out // 2, k=3, name=name + "_m1")
+    a, c = b.split(h, [c_out // 2, c_out // 2], name=name + "_split")
+    m = b.conv(c, c_out // 2, k=3, name=name + "_m1")
     m = b.lut(m, silu, "Swish", name=name + "_m1_act")
     m = b.conv(m, c_out // 2, k=3, name=name + "_m2")
     m = b.lut(m, silu, "Swish", name=name + "_m2_act")
-    h = b.add(h, m, name=name + "_add")
-    y = b.conv(h, c_out, k=1, name=name + "_cv2")
+    m = b.add(c, m, name=name + "_add")
+    cat = b.concat([a, c, m], name=name + "_cat")
+    y = b.conv(cat, c_out, k=1, name=name + "_cv2")
+    return b.lut(y, silu, "Swish", name=name + "_cv2_act")
+
+
+def sppf_like(b, x, c_out, name):
+    """SPPF: 1x1 reduce, three chained 5x5 stride-1 max pools, Concat of all four, 1x1 fuse."""
+    c = b.g.shape(x)[3] // 2
+    h = b.conv(x, c, k=1, name=name + "_cv1")
+    h = b.lut(h, silu, "Swish", name=name + "_cv1_act")
+    m1 = b.max_pool(h, 5, name=name + "_m1")
+    m2 = b.max_pool(m1, 5, name=name + "_m2")
+    m3 = b.max_pool(m2, 5, name=name + "_m3")
+    cat = b.concat([h, m1, m2, m3], name=name + "_cat")
+    y = b.conv(cat, c_out, k=1, name=name + "_cv2")
     return b.lut(y, silu, "Swish", name=name + "_cv2_act")
 
 
 def config4_yolo_style(seed=0xE5D4, resolution=640):
     """YOLO11n-style detector trunk: int8 Conv backbone with SiLU as 8-bit LUT after every conv
     (conv -> LUT pairs, as in the exported YOLO11n), strided 3x3 downsampling, bottleneck blocks
-    with residual Adds, and an int16 detection head (int16 weights and activations, int64 bias).
-    Concat / Split / Resize / MaxPool of the real graph are data movement outside the conv/gemm/LUT
-    path and are left out; channel widths follow YOLO11n (16-32-64-128-256)."""
+    (Split -> bottleneck with residual Add -> Concat), SPPF (chained 5x5 max pools + Concat), an FPN
+    top-down path (nearest Resize x2 + Concat with the skip), an NCHW Transpose of one class output,
+    and an int16 detection head (int16 weights and activations, int64 bias).  Channel widths follow
+    YOLO11n (16-32-64-128-256)."""
     g = GraphSpec("config4_yolo_style_%d" % resolution)
     b = Builder(g, seed, per_channel=True, w_exp_range=None)
     x = b.input("input", [1, resolution, resolution, 3], -6)
@@ -389,7 +468,12 @@ def config4_yolo_style(seed=0xE5D4, resolution=640):
     p4 = x
     x = cbs(x, 256, 3, 2, "p5")    # 20
     x = c3k2_like(b, x, 256, "c5")
-    p5 = x
+    p5 = sppf_like(b, x, 256, "sppf")
+    # FPN top-down: upsample, concatenate with the skip, fuse
+    up = b.resize_nearest(p5, 2, name="up5")
+    p4 = c3k2_like(b, b.concat([up, p4], name="fpn4_join"), 128, "fpn4")
+    up = b.resize_nearest(p4, 2, name="up4")
+    p3 = c3k2_like(b, b.concat([up, p3], name="fpn3_join"), 64, "fpn3")
     # detection head per scale: int8 3x3 conv + SiLU, then int16 box branch (requantize to int16,
     # int16 3x3 conv, int16 1x1 conv) and an int8 class branch
     for i, (p, c) in enumerate(((p3, 64), (p4, 64), (p5, 64))):
@@ -402,6 +486,8 @@ def config4_yolo_style(seed=0xE5D4, resolution=640):
         b.output(box)
         cls = cbs(h, 80, 1, 1, "head%d_cls1" % i)
         cls = b.conv(cls, 80, k=1, name="head%d_cls2" % i)
+        if i == 2:  # one output in the NCHW layout detection post-processing reads
+            cls = b.transpose(cls, (0, 3, 1, 2), name="head%d_cls_nchw" % i)
         b.output(cls)
     return g
 

@@ -68,6 +68,21 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             y = x.reshape(x.shape[0], -1)
         elif op == "Squeeze":
             y = np.squeeze(x, axis=tuple(a["axes"]))
+        elif op == "MaxPool":
+            pt, pl, pb, pr = a["pads"]
+            y = oracle.max_pool(x, tuple(a["kernel_shape"]), tuple(a["strides"]), (pt, pb, pl, pr))
+        elif op == "Concat":
+            y = oracle.concat([t[n] for n in ins], a["axis"])
+        elif op == "Split":
+            sizes = [int(v) for v in spec.initializers[ins[1]][2].ravel()]
+            for name, piece in zip(outs, oracle.split(x, a["axis"], sizes)):
+                t[name] = piece
+            continue
+        elif op == "Resize":
+            scales = spec.initializers[ins[2]][2].ravel()
+            y = oracle.resize_nearest_s8(x, scales[2], scales[3], spec.exponent(ins[0]), spec.exponent(y_name))
+        elif op == "Transpose":
+            y = oracle.transpose(x, list(a["perm"]))
         else:
             raise NotImplementedError(op)
         t[y_name] = y

@@ -178,6 +178,33 @@ def test_config4_yolo_style(oracle, fuse):
     mdl.close()
 
 
+def test_config4_neck_data_movement_tensors(oracle):
+    """Every Split / Concat / MaxPool / Resize / Transpose output of the detector graph, kept alive as
+    test outputs, equals the oracle's (C3k2 split+concat, SPPF pool chain, FPN upsample+concat)."""
+    announce("model config4 160px neck tensors")
+    m, zoo, model, runner = _mods()
+    import espdl_oracle as oracle_mod
+    spec = zoo.config4_yolo_style(resolution=160)
+    batch = 3
+    x = spec.make_input(np.random.default_rng(12), batch)
+    want = runner.run(spec, {spec.inputs[0]: x}, oracle_mod.ROUND_HALF_UP)
+    names = [o for n in spec.nodes if n["op_type"] in ("Split", "Concat", "MaxPool", "Resize", "Transpose")
+             for o in n["outputs"]]
+    assert len(names) >= 25
+    g = model.Graph.from_spec(spec, test_outputs={n: want[n][:1] for n in names})
+    mdl = model.Model(g, batch)
+    mdl.set_input(spec.inputs[0], x)
+    mdl.run()
+    for n in names:
+        np.testing.assert_array_equal(mdl.get_tensor(n, _np_dtype(spec, n)), want[n], err_msg=n)
+    # under a captured graph as well
+    assert mdl.enable_graph()
+    mdl.run()
+    for n in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(n, _np_dtype(spec, n)), want[n], err_msg=n)
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()
