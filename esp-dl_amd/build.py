@@ -56,7 +56,7 @@ def build_kernels(verbose=True):
 
 
 DL_DIR = os.path.join(HERE, "dl")
-DL_SOURCES = ["dl_tensor_base.cpp", "fbs_model.cpp", "dl_model_context.cpp", "dl_module_base.cpp", "dl_model_base.cpp",
+DL_SOURCES = ["dl_tensor_base.cpp", "fbs_model.cpp", "fbs_loader.cpp", "dl_model_context.cpp", "dl_module_base.cpp", "dl_model_base.cpp",
               "espdl_model_capi.cpp"]
 INCLUDE_DIR = os.path.join(os.path.dirname(HERE), "include")
 

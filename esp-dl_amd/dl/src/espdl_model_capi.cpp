@@ -1,10 +1,12 @@
 // C handle API of include/espdl_model.h over fbs::FbsModel and dl::Model.
 #include "espdl_model.h"
 
+#include <cstring>
 #include <string>
 #include <vector>
 
 #include "dl_model_base.hpp"
+#include "fbs_loader.hpp"
 
 struct espdl_graph {
     fbs::FbsModel fbs;
@@ -34,6 +36,84 @@ espdl_graph *espdl_graph_create(const char *name)
 void espdl_graph_destroy(espdl_graph *g)
 {
     delete g;
+}
+
+static thread_local std::string g_load_error;
+
+static espdl_graph *graph_from_loader(fbs::FbsLoader &loader, int32_t model_index)
+{
+    fbs::FbsModel *m = loader.load(model_index);
+    if (!m) {
+        g_load_error = loader.last_error();
+        return nullptr;
+    }
+    espdl_graph *g = new espdl_graph();
+    g->fbs = std::move(*m);
+    delete m;
+    g_load_error.clear();
+    return g;
+}
+
+espdl_graph *espdl_graph_load_file(const char *path, int32_t model_index)
+{
+    fbs::FbsLoader loader(path, fbs::MODEL_LOCATION_IN_SDCARD);
+    return graph_from_loader(loader, model_index);
+}
+
+espdl_graph *espdl_graph_load_memory(const void *data, int64_t size, int32_t model_index)
+{
+    fbs::FbsLoader loader(data, size > 0 ? (size_t)size : 0);
+    return graph_from_loader(loader, model_index);
+}
+
+const char *espdl_graph_load_error(void)
+{
+    return g_load_error.c_str();
+}
+
+int32_t espdl_graph_input_count(espdl_graph *g)
+{
+    return g ? (int32_t)g->fbs.get_graph_inputs().size() : -1;
+}
+
+int32_t espdl_graph_output_count(espdl_graph *g)
+{
+    return g ? (int32_t)g->fbs.get_graph_outputs().size() : -1;
+}
+
+static const char *io_name(espdl_graph *g, bool input, int32_t index)
+{
+    static thread_local std::string name;
+    if (!g)
+        return nullptr;
+    const std::vector<std::string> names = input ? g->fbs.get_graph_inputs() : g->fbs.get_graph_outputs();
+    if (index < 0 || index >= (int32_t)names.size())
+        return nullptr;
+    name = names[(size_t)index];
+    return name.c_str();
+}
+
+int64_t espdl_graph_initializer_bytes(espdl_graph *g, const char *name, void *dst, int64_t capacity)
+{
+    if (!g || !name || !g->fbs.is_parameter(name))
+        return -1;
+    const void *raw = g->fbs.get_tensor_raw_data(name);
+    size_t bytes = dl::dtype_sizeof(g->fbs.get_tensor_dtype(name));
+    for (int d : g->fbs.get_tensor_shape(name))
+        bytes *= (size_t)d;
+    if (dst && capacity >= (int64_t)bytes && raw)
+        std::memcpy(dst, raw, bytes);
+    return (int64_t)bytes;
+}
+
+const char *espdl_graph_input_name(espdl_graph *g, int32_t index)
+{
+    return io_name(g, true, index);
+}
+
+const char *espdl_graph_output_name(espdl_graph *g, int32_t index)
+{
+    return io_name(g, false, index);
 }
 
 int espdl_graph_add_initializer(espdl_graph *g, const char *name, const int32_t *dims, int32_t n_dims, int32_t dtype,

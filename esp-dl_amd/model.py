@@ -57,6 +57,17 @@ def lib():
         L.espdl_model_get_tensor.argtypes = [vp, cp, vp, i64]
         L.espdl_model_device_bytes.restype = i64
         L.espdl_model_device_bytes.argtypes = [vp]
+        L.espdl_graph_load_file.restype = vp
+        L.espdl_graph_load_file.argtypes = [cp, i32]
+        L.espdl_graph_load_memory.restype = vp
+        L.espdl_graph_load_memory.argtypes = [vp, ctypes.c_int64, i32]
+        L.espdl_graph_load_error.restype = cp
+        for nm in ("input", "output"):
+            getattr(L, "espdl_graph_%s_count" % nm).argtypes = [vp]
+            getattr(L, "espdl_graph_%s_name" % nm).argtypes = [vp, i32]
+            getattr(L, "espdl_graph_%s_name" % nm).restype = cp
+        L.espdl_graph_initializer_bytes.restype = ctypes.c_int64
+        L.espdl_graph_initializer_bytes.argtypes = [vp, cp, vp, ctypes.c_int64]
         L.espdl_model_stream.restype = vp
         L.espdl_model_stream.argtypes = [vp]
         _lib = L
@@ -122,6 +133,40 @@ class Graph:
                 L.espdl_graph_add_test_output(g.h, name.encode(), d, nd, dtype, arr.ctypes.data_as(ctypes.c_void_p),
                                               exp)
         return g
+
+    @classmethod
+    def from_file(cls, path, model_index=0):
+        """Read an `.espdl` container with the native loader (no GPU needed)."""
+        g = cls.__new__(cls)
+        g.h = lib().espdl_graph_load_file(os.fsencode(path), model_index)
+        if not g.h:
+            raise EspdlModelError("%s: %s" % (path, lib().espdl_graph_load_error().decode()))
+        return g
+
+    @classmethod
+    def from_bytes(cls, blob, model_index=0):
+        g = cls.__new__(cls)
+        g.h = lib().espdl_graph_load_memory(blob, len(blob), model_index)
+        if not g.h:
+            raise EspdlModelError(lib().espdl_graph_load_error().decode())
+        return g
+
+    def initializer(self, name, dtype=np.int8):
+        """Bytes of a constant tensor as the kernels will read it (flat array of dtype)."""
+        n = lib().espdl_graph_initializer_bytes(self.h, name.encode(), None, 0)
+        if n < 0:
+            raise KeyError(name)
+        out = np.empty(n // np.dtype(dtype).itemsize, dtype=dtype)
+        lib().espdl_graph_initializer_bytes(self.h, name.encode(), out.ctypes.data_as(ctypes.c_void_p), n)
+        return out
+
+    def input_names(self):
+        L = lib()
+        return [L.espdl_graph_input_name(self.h, i).decode() for i in range(L.espdl_graph_input_count(self.h))]
+
+    def output_names(self):
+        L = lib()
+        return [L.espdl_graph_output_name(self.h, i).decode() for i in range(L.espdl_graph_output_count(self.h))]
 
     def __del__(self):
         if getattr(self, "h", None) and _lib is not None:

@@ -35,6 +35,22 @@ typedef struct espdl_model espdl_model;
 
 espdl_graph *espdl_graph_create(const char *name);
 void espdl_graph_destroy(espdl_graph *g);
+/* A graph read from an `.espdl` container (what fbs::FbsLoader::load does,
+ * esp-dl/fbs_loader/src/fbs_loader.cpp:276-360): EDL1 / EDL2 files and PDL1 / PDL2 packages (model_index
+ * selects the model, 0 for single-model files), plain payloads only.  Filters stored in the blocked
+ * ESP32-S3 / ESP32-P4 order are rewritten to the N-major order the kernels read.  Embedded test vectors
+ * become the graph's test inputs / outputs.  NULL on failure, reason in espdl_graph_load_error(). */
+espdl_graph *espdl_graph_load_file(const char *path, int32_t model_index);
+espdl_graph *espdl_graph_load_memory(const void *data, int64_t size, int32_t model_index);
+const char *espdl_graph_load_error(void);
+int32_t espdl_graph_input_count(espdl_graph *g);
+int32_t espdl_graph_output_count(espdl_graph *g);
+/* Copies the bytes of a constant tensor (after any re-layout) into dst when capacity allows; returns
+ * its size in bytes, -1 when there is no such initializer. */
+int64_t espdl_graph_initializer_bytes(espdl_graph *g, const char *name, void *dst, int64_t capacity);
+/* Valid until the next call on this thread. */
+const char *espdl_graph_input_name(espdl_graph *g, int32_t index);
+const char *espdl_graph_output_name(espdl_graph *g, int32_t index);
 /* A constant tensor (filter, bias, LUT, PReLU slope, Clip bound); `data` is a host buffer that is copied. */
 int espdl_graph_add_initializer(espdl_graph *g, const char *name, const int32_t *dims, int32_t n_dims, int32_t dtype,
                                 const void *data, const int32_t *exponents, int32_t n_exponents);
