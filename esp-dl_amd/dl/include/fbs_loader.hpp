@@ -8,10 +8,10 @@
 //
 // What load() does beyond copying fields:
 //   * filters stored for the ESP32-S3 / ESP32-P4 targets in the blocked order the vector units read
-//     ("(N/16)HWC16", "N16HWC16", "(N/16)WC16", "(N/8)HWC8", tail "…_UNALIGNED": blocks of 16 (int8) or
-//     8 (int16) output channels, channel index innermost, then the N % block remaining filters as
-//     [H][W][C][rest]) are rewritten into the N-major order of the `c` target, [N][H][W][C], which is
-//     what the kernels of this repository read;
+//     ("(N/16)HWC16", "N16HWC16", "(N/16)WC16", "(N/8)HWC8", "..._UNALIGNED": blocks of 16 (int8) or
+//     8 (int16) filters with the filter index innermost, then the N % block remaining filters in plain
+//     filter-major order; depthwise filters are blocked over their channels) are rewritten into the
+//     order of the `c` target, [N][H][W][C] (depthwise [H][W][C]), which the kernels here read;
 //   * encrypted payloads (mode 1, AES-128) are refused.
 #pragma once
 

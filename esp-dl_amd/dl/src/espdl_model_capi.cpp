@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "dl_model_base.hpp"
+#include "dl_module_creator.hpp"
 #include "fbs_loader.hpp"
 
 struct espdl_graph {
@@ -104,6 +105,28 @@ int64_t espdl_graph_initializer_bytes(espdl_graph *g, const char *name, void *ds
     if (dst && capacity >= (int64_t)bytes && raw)
         std::memcpy(dst, raw, bytes);
     return (int64_t)bytes;
+}
+
+int32_t espdl_graph_node_count(espdl_graph *g)
+{
+    return g ? (int32_t)g->fbs.topological_sort().size() : -1;
+}
+
+const char *espdl_graph_node_op_type(espdl_graph *g, int32_t index)
+{
+    static thread_local std::string op;
+    if (!g)
+        return nullptr;
+    const std::vector<std::string> order = g->fbs.topological_sort();
+    if (index < 0 || index >= (int32_t)order.size())
+        return nullptr;
+    op = g->fbs.get_operation_type(order[(size_t)index]);
+    return op.c_str();
+}
+
+int32_t espdl_module_is_registered(const char *op_type)
+{
+    return op_type && dl::module::ModuleCreator::get_instance()->is_registered(op_type) ? 1 : 0;
 }
 
 const char *espdl_graph_input_name(espdl_graph *g, int32_t index)

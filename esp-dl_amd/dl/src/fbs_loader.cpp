@@ -3,6 +3,7 @@
 
 #include <cstdio>
 #include <cstring>
+#include <set>
 
 namespace fbs {
 
@@ -212,20 +213,28 @@ int layout_block(const std::string &doc)
     return 0;
 }
 
-// [N/B][spatial][C][B] + [spatial][C][N % B]  ->  [N][spatial][C]; dims are [spatial..., C, N].
-bool unblock_filter(RawTensor &t, int block)
+// [N/B][spatial][C][B] followed by the N % B remaining filters in plain [rest][spatial][C] order
+//   ->  [N][spatial][C].
+// dims are [spatial..., C, N]; a depthwise filter ([spatial..., C, 1]) is blocked over its C filters of
+// one input channel each and ends up as the `c` target's [spatial][C].
+// The S3 / P4 files of the reference's Gemm fixtures hold the same weights as their `c` files, which
+// fixes the body order; the order of the remainder and of depthwise filters is fixed by the shipped
+// MobileNetV2 (N = 24 and depthwise layers): only this reading reproduces the top-5 classes that
+// examples/mobilenetv2_cls/README.md lists for its cat.jpg.
+bool unblock_filter(RawTensor &t, int block, bool depthwise)
 {
     if (t.dims.size() < 2)
         return false;
     const size_t esize = dl::dtype_sizeof(t.dtype);
-    const size_t n = (size_t)t.dims.back(), c = (size_t)t.dims[t.dims.size() - 2];
+    const size_t last = (size_t)t.dims.back(), prev = (size_t)t.dims[t.dims.size() - 2];
+    const size_t n = depthwise ? last * prev : last, c = depthwise ? 1 : prev;
     size_t sp = 1;
     for (size_t i = 0; i + 2 < t.dims.size(); i++)
         sp *= (size_t)t.dims[i];
     if (t.bytes.size() != n * sp * c * esize)
         return false;
-    const size_t nb = n / (size_t)block, tail = n % (size_t)block;
-    std::vector<uint8_t> out(t.bytes.size());
+    const size_t nb = n / (size_t)block;
+    std::vector<uint8_t> nmajor(t.bytes.size());
     const uint8_t *src = t.bytes.data();
     for (size_t b = 0; b < nb; b++)
         for (size_t s = 0; s < sp; s++)
@@ -233,17 +242,20 @@ bool unblock_filter(RawTensor &t, int block)
                 for (size_t j = 0; j < (size_t)block; j++) {
                     const size_t from = (((b * sp + s) * c + k) * block + j) * esize;
                     const size_t to = (((b * block + j) * sp + s) * c + k) * esize;
-                    std::memcpy(&out[to], src + from, esize);
+                    std::memcpy(&nmajor[to], src + from, esize);
                 }
-    const uint8_t *tsrc = src + nb * block * sp * c * esize;
-    for (size_t s = 0; s < sp; s++)
-        for (size_t k = 0; k < c; k++)
-            for (size_t j = 0; j < tail; j++) {
-                const size_t from = ((s * c + k) * tail + j) * esize;
-                const size_t to = (((nb * block + j) * sp + s) * c + k) * esize;
-                std::memcpy(&out[to], tsrc + from, esize);
-            }
-    t.bytes.swap(out);
+    const size_t done = nb * block * sp * c * esize;
+    std::memcpy(nmajor.data() + done, src + done, t.bytes.size() - done); // remainder: already filter-major
+    if (depthwise) {
+        // [C][spatial] -> [spatial][C]
+        std::vector<uint8_t> hwc(t.bytes.size());
+        for (size_t ch = 0; ch < n; ch++)
+            for (size_t s = 0; s < sp; s++)
+                std::memcpy(&hwc[(s * n + ch) * esize], &nmajor[(ch * sp + s) * esize], esize);
+        t.bytes.swap(hwc);
+    } else {
+        t.bytes.swap(nmajor);
+    }
     return true;
 }
 
@@ -443,12 +455,27 @@ FbsModel *FbsLoader::parse(const Entry &e, const uint8_t *key)
         return nullptr;
     };
 
+    // filters of grouped (depthwise) convolutions are blocked over their channels: find them first
+    std::set<std::string> depthwise_filters;
+    for (Table n : graph.tables(0)) {
+        if (n.string(3) != "Conv")
+            continue;
+        int64_t group = 1;
+        for (Table a : n.tables(5))
+            if (a.string(0) == "group" && a.scalar<int32_t>(3, 0) == 2) {
+                const size_t p = a.field(5);
+                group = p ? buf.rd<int64_t>(p) : 1;
+            }
+        const std::vector<std::string> ins = n.strings(0);
+        if (group != 1 && ins.size() > 1)
+            depthwise_filters.insert(ins[1]);
+    }
     for (Table t : graph.tables(2)) {
         RawTensor r = read_tensor(t);
         if (!r.ok)
             return fail("initializer " + r.name + ": unreadable tensor");
         const int block = layout_block(r.doc);
-        if (block && !unblock_filter(r, block))
+        if (block && !unblock_filter(r, block, depthwise_filters.count(r.name) != 0))
             return fail("initializer " + r.name + ": blocked layout does not fit its dims");
         out->add_initializer(r.name, r.dims, r.dtype, r.bytes.data(), r.exponents);
     }

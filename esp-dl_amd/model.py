@@ -68,6 +68,10 @@ def lib():
             getattr(L, "espdl_graph_%s_name" % nm).restype = cp
         L.espdl_graph_initializer_bytes.restype = ctypes.c_int64
         L.espdl_graph_initializer_bytes.argtypes = [vp, cp, vp, ctypes.c_int64]
+        L.espdl_graph_node_count.argtypes = [vp]
+        L.espdl_graph_node_op_type.argtypes = [vp, i32]
+        L.espdl_graph_node_op_type.restype = cp
+        L.espdl_module_is_registered.argtypes = [cp]
         L.espdl_model_stream.restype = vp
         L.espdl_model_stream.argtypes = [vp]
         _lib = L
@@ -160,6 +164,10 @@ class Graph:
         lib().espdl_graph_initializer_bytes(self.h, name.encode(), out.ctypes.data_as(ctypes.c_void_p), n)
         return out
 
+    def op_types(self):
+        L = lib()
+        return [L.espdl_graph_node_op_type(self.h, i).decode() for i in range(L.espdl_graph_node_count(self.h))]
+
     def input_names(self):
         L = lib()
         return [L.espdl_graph_input_name(self.h, i).decode() for i in range(L.espdl_graph_input_count(self.h))]
@@ -172,6 +180,10 @@ class Graph:
         if getattr(self, "h", None) and _lib is not None:
             _lib.espdl_graph_destroy(self.h)
             self.h = None
+
+
+def is_registered(op_type):
+    return bool(lib().espdl_module_is_registered(op_type.encode()))
 
 
 class Model:

@@ -48,6 +48,11 @@ int32_t espdl_graph_output_count(espdl_graph *g);
 /* Copies the bytes of a constant tensor (after any re-layout) into dst when capacity allows; returns
  * its size in bytes, -1 when there is no such initializer. */
 int64_t espdl_graph_initializer_bytes(espdl_graph *g, const char *name, void *dst, int64_t capacity);
+/* Nodes in execution order, and whether an operator type has a module in this build
+ * (ModuleCreator::register_module adds more, esp-dl/dl/module/include/dl_module_creator.hpp:107). */
+int32_t espdl_graph_node_count(espdl_graph *g);
+const char *espdl_graph_node_op_type(espdl_graph *g, int32_t index);
+int32_t espdl_module_is_registered(const char *op_type);
 /* Valid until the next call on this thread. */
 const char *espdl_graph_input_name(espdl_graph *g, int32_t index);
 const char *espdl_graph_output_name(espdl_graph *g, int32_t index);

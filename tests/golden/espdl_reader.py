@@ -140,7 +140,27 @@ def _attribute(a):
 
 
 def _value_info(v):
-    return {"name": v.string(0), "exponents": v.vector_i64(3)}
+    """ValueInfo: 0 name, 1 value_info_type (TypeInfo: 0 union tag, 1 value -> TensorTypeAndShape:
+    0 elem_type, 1 shape -> TensorShape.dim[] -> Dimension.value -> DimensionValue.dim_value), 3 exponents."""
+    out = {"name": v.string(0), "exponents": v.vector_i64(3), "dtype": 0, "dims": []}
+    p = v.field(1)
+    ti = v.table(1)
+    if p is None or ti is None:
+        return out
+    tag = ti.field(0)
+    if tag is None or ti.b.u8(tag) != 1:
+        return out
+    tts = ti.table(1)
+    if tts is None:
+        return out
+    out["dtype"] = tts.scalar_i32(0)
+    shape = tts.table(1)
+    if shape is not None:
+        for dim in shape.vector_tables(0):
+            dv = dim.table(0)
+            p = None if dv is None else dv.field(1)
+            out["dims"].append(int(dv.b.i64(p)) if p is not None else 1)
+    return out
 
 
 def read_espdl(path):

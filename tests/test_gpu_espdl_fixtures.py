@@ -50,3 +50,43 @@ def test_reference_fixture_batched(path):
         want = np.repeat(tout["data"].reshape(tout["dims"]), 5, axis=0)
         np.testing.assert_array_equal(mdl.get_tensor(name).reshape(want.shape), want, err_msg=name)
     mdl.close()
+
+
+def _extra_models():
+    """More `.espdl` files (e.g. the reference's model zoo) can be named through ESPDL_EXTRA_MODELS, a
+    directory; they are too large to keep as fixtures, so without the variable only the committed
+    files run."""
+    d = os.environ.get("ESPDL_EXTRA_MODELS")
+    return sorted(glob.glob(os.path.join(d, "*.espdl"))) if d else []
+
+
+@pytest.mark.parametrize("path", FIXTURES + _extra_models(), ids=os.path.basename)
+def test_loaded_graph_matches_oracle_on_random_input(path):
+    """Native loader -> dl::Model on the GPU against Python walker -> GraphSpec -> CPU oracle, on a seeded
+    random batch: every graph output bit-exact (covers graphs whose files carry no test vectors)."""
+    announce("espdl graph vs oracle " + os.path.basename(path))
+    sys.path.insert(0, HERE)
+    import espdl_spec
+    import graph_runner
+    import espdl_oracle as oracle
+    spec, _ = espdl_spec.spec_from_espdl(path)
+    model = importlib.import_module("esp-dl_amd").model
+    unsupported = sorted({n["op_type"] for n in spec.nodes if not model.is_registered(n["op_type"])})
+    if unsupported:
+        pytest.skip("operators without a module in this build: " + ", ".join(unsupported))
+    rm = _round_mode(path)
+    batch = 3
+    x = spec.make_input(np.random.default_rng(77), batch)
+    want = graph_runner.run(spec, {spec.inputs[0]: x}, oracle.ROUND_HALF_EVEN if rm else oracle.ROUND_HALF_UP,
+                            keep_all=False)
+    g = model.Graph.from_file(path)
+    for fuse in (True, False):
+        mdl = model.Model(g, batch, round_mode=rm, fuse_lut=fuse, fuse_blocks=fuse)
+        mdl.set_input(spec.inputs[0], x)
+        mdl.run()
+        for name in spec.outputs:
+            dt = np.int16 if spec.dtype(name) == 5 else np.int8
+            got = mdl.get_tensor(name, dt)
+            np.testing.assert_array_equal(got.reshape(want[name].shape), want[name], err_msg=f"{name} fuse={fuse}")
+            assert want[name].min() < want[name].max()
+        mdl.close()
