@@ -284,7 +284,7 @@ struct WaveCtx {
 // One group of NT filter tiles (16*NT filters) for the wave's PT pixel tiles: MFMA over the K steps
 // resident in registers (KSC > 0) or streamed (KSC == 0), then the epilogue.  NT is a compile-time
 // constant so that the tile loops carry no run-time tests.
-template <int BMODE, int PT, int KSC, bool FAST, bool USE_LSH, int NT>
+template <int BMODE, int PT, int KSC, bool FAST, int USE_LSH, int NT>
 __device__ __forceinline__ void run_group(const MfmaConvArgs &a, const WaveCtx &w, const PixelRef (&px)[PT],
                                           const v4i (&bc)[PT][KSC > 0 ? KSC : 1], int gi, int gbase, int g_first,
                                           int g_count)
@@ -443,7 +443,7 @@ __device__ __forceinline__ void run_group(const MfmaConvArgs &a, const WaveCtx &
 }
 
 // The persistent loop over pixel sets with one epilogue flavour compiled in.
-template <int BMODE, int PT, int KSC, bool FAST, bool USE_LSH>
+template <int BMODE, int PT, int KSC, bool FAST, int USE_LSH>
 __device__ __forceinline__ void run_sets(const MfmaConvArgs &a, const WaveCtx &w, int wave, int g_first, int g_count,
                                          const TileSeq &seq, PixelRef (&px)[PT], v4i (&bc)[PT][KSC > 0 ? KSC : 1])
 {
@@ -533,7 +533,10 @@ __device__ __forceinline__ void run_sets(const MfmaConvArgs &a, const WaveCtx &w
 
 // KSC > 0: the whole reduction axis (at most KSC k steps) is held in registers per pixel tile.
 // KSC == 0: k steps are streamed four at a time (any K, including K chunks re-staged in LDS).
-template <int BMODE, int PT, int KSC>
+// HE: the round-half-even build of the kernel.  A separate kernel, not one more branch of this one: the
+// register allocation of a kernel is that of its heaviest branch, and the half-even epilogue would cost
+// the half-up build a wavefront of occupancy.
+template <int BMODE, int PT, int KSC, bool HE>
 __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConvArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -569,7 +572,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
     // bias + 2^(s-1) + (k_h*k_w*in_c products of at most 2^14) must fit int32 even after the left
     // shift by max(0, 8-s) that the short form applies.
     const long long mac_bound = (long long)g.k_h * g.k_w * g.in_c * 16384;
-    int ok_local = half_even ? 0 : 1;
+    int ok_local = 1;
     int lsh_local = 0;
     for (int c = tid; c < g_count * 64; c += kThreads) {
         const int oc = g_first * 64 + c;
@@ -625,12 +628,21 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
     w.has_lut = has_lut;
     w.floor_pk = w.relu ? 0 : (int)0x80008000u;
     w.stage_out = a.stage_out != 0;
-    if (fast && !use_lsh)
-        run_sets<BMODE, PT, KSC, true, false>(a, w, wave, g_first, g_count, seq, px, bc);
-    else if (fast)
-        run_sets<BMODE, PT, KSC, true, true>(a, w, wave, g_first, g_count, seq, px, bc);
-    else
-        run_sets<BMODE, PT, KSC, false, false>(a, w, wave, g_first, g_count, seq, px, bc);
+    // epilogue mode of pack_fast4: 0 plain (every shift >= 8), 1 with the left shift, 2 the same with
+    // round-half-even
+    if (HE) {
+        if (fast)
+            run_sets<BMODE, PT, KSC, true, 2>(a, w, wave, g_first, g_count, seq, px, bc);
+        else
+            run_sets<BMODE, PT, KSC, false, 0>(a, w, wave, g_first, g_count, seq, px, bc);
+    } else {
+        if (fast && !use_lsh)
+            run_sets<BMODE, PT, KSC, true, 0>(a, w, wave, g_first, g_count, seq, px, bc);
+        else if (fast)
+            run_sets<BMODE, PT, KSC, true, 1>(a, w, wave, g_first, g_count, seq, px, bc);
+        else
+            run_sets<BMODE, PT, KSC, false, 0>(a, w, wave, g_first, g_count, seq, px, bc);
+    }
 }
 
 // What the host planner knows; the grid itself is sized per kernel variant from the number of
@@ -641,18 +653,25 @@ struct GridPlan {
     int n_chunks; // filter chunks = gridDim.y
 };
 
-template <int BMODE, int PT, int KSC>
-hipError_t launch_variant(const MfmaConvArgs &a, GridPlan plan, size_t lds, hipStream_t stream)
+template <int BMODE, int PT, int KSC, bool HE>
+hipError_t launch_variant_he(const MfmaConvArgs &a, GridPlan plan, size_t lds, hipStream_t stream)
 {
-    const int per_cu = resident_workgroups_per_cu(conv2d_s8_mfma_kernel<BMODE, PT, KSC>, kThreads, lds);
+    const int per_cu = resident_workgroups_per_cu(conv2d_s8_mfma_kernel<BMODE, PT, KSC, HE>, kThreads, lds);
     int gx = max(1, (plan.cus * per_cu) / plan.n_chunks);
     if (gx > a.n_sets)
         gx = a.n_sets;
     if (gx >= 8)
         gx &= ~7; // blockIdx.x % 8 is then the XCD of a workgroup, for every blockIdx.y
-    hipLaunchKernelGGL((conv2d_s8_mfma_kernel<BMODE, PT, KSC>), dim3((unsigned)gx, (unsigned)plan.n_chunks),
+    hipLaunchKernelGGL((conv2d_s8_mfma_kernel<BMODE, PT, KSC, HE>), dim3((unsigned)gx, (unsigned)plan.n_chunks),
                        dim3(kThreads), lds, stream, a);
     return hipGetLastError();
+}
+
+template <int BMODE, int PT, int KSC>
+hipError_t launch_variant(const MfmaConvArgs &a, GridPlan plan, size_t lds, hipStream_t stream)
+{
+    return a.g.half_even ? launch_variant_he<BMODE, PT, KSC, true>(a, plan, lds, stream)
+                         : launch_variant_he<BMODE, PT, KSC, false>(a, plan, lds, stream);
 }
 
 // Smallest register-resident variant that holds `ksteps` k steps (0 = streamed).

@@ -16,6 +16,8 @@
 //   one barrier per k step; MFMA operands are plain 16-byte LDS reads.
 // The filter -> tile-row permutation (row i of tile t is filter 16*(i/4) + 4*t + i%4 of the group)
 // leaves every lane with 16 consecutive output channels per pixel: one 16-byte store.
+#include <type_traits>
+
 #include "espdl_device.h"
 #include "espdl_kernels.h"
 
@@ -96,7 +98,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     // epilogue constants of the workgroup's filters; the short form needs every shift in 1..31 and no
     // possible overflow of bias + 2^(s-1) + K products
     const long long mac_bound = (long long)a.K * 16384;
-    int ok_local = half_even ? 0 : 1;
+    int ok_local = 1;
     int my_s = 0, my_b = 0;
     if (tid < TN) {
         const int n = n0 + tid;
@@ -166,66 +168,73 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
 
     // epilogue: lane (col, quad) holds, per pixel tile and group, filters 64*g + 16*quad + [0, 16)
     const int floor_pk = relu ? 0 : (int)0x80008000u;
-#pragma unroll
-    for (int c = 0; c < PT; c++) {
-        const long long m = m0 + 16 * PT * wave + 16 * c + col;
-#pragma unroll
-        for (int g = 0; g < NG; g++) {
-            const int n = n0 + 64 * g + 16 * quad;
-            int words[4];
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                const v4i ss = *reinterpret_cast<const v4i *>(&cst[1][64 * g + 16 * quad + 4 * t]);
-                if (fast) {
-                    const v4i ls = *reinterpret_cast<const v4i *>(&cst[2][64 * g + 16 * quad + 4 * t]);
-                    words[t] = pack_fast4<true>(acc[c][4 * g + t], ls, ss, floor_pk);
-                } else {
-                    int q[4];
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        q[r] = requant_s8(acc[c][4 * g + t][r], ss[r], relu, half_even);
-                    words[t] = pack4_s8(q[0], q[1], q[2], q[3]);
-                }
-                if (has_lut) {
-                    const int v = words[t];
-                    words[t] = pack4_s8(lut_l[(int)(int8_t)v + 128], lut_l[(int)(int8_t)(v >> 8) + 128],
-                                        lut_l[(int)(int8_t)(v >> 16) + 128], lut_l[(v >> 24) + 128]);
-                }
-            }
-            if (m >= a.M || n >= a.N)
-                continue;
-            const long long goff = m * a.N + n;
-            if (a.out_vec == 16 && n + 16 <= a.N) {
-                v4i v = {words[0], words[1], words[2], words[3]};
-                if (a.res != nullptr) {
-                    const v4i r = *reinterpret_cast<const v4i *>(a.res + goff);
-#pragma unroll
-                    for (int d = 0; d < 4; d++)
-                        v[d] = sat_add4_s8(v[d], r[d]);
-                }
-                __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(a.out + goff));
-            } else if (a.out_vec >= 4) {
-#pragma unroll
-                for (int t = 0; t < 4; t++)
-                    if (n + 4 * t + 4 <= a.N) {
-                        int v = words[t];
-                        if (a.res != nullptr)
-                            v = sat_add4_s8(v, *reinterpret_cast<const int *>(a.res + goff + 4 * t));
-                        *reinterpret_cast<int *>(a.out + goff + 4 * t) = v;
+    // one straight-line copy per rounding mode (pack_fast4 mode 1: half up, 2: half even)
+    auto epilogue = [&](auto mode) {
+    #pragma unroll
+        for (int c = 0; c < PT; c++) {
+            const long long m = m0 + 16 * PT * wave + 16 * c + col;
+    #pragma unroll
+            for (int g = 0; g < NG; g++) {
+                const int n = n0 + 64 * g + 16 * quad;
+                int words[4];
+    #pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const v4i ss = *reinterpret_cast<const v4i *>(&cst[1][64 * g + 16 * quad + 4 * t]);
+                    if (fast) {
+                        const v4i ls = *reinterpret_cast<const v4i *>(&cst[2][64 * g + 16 * quad + 4 * t]);
+                        words[t] = pack_fast4<decltype(mode)::value>(acc[c][4 * g + t], ls, ss, floor_pk);
+                    } else {
+                        int q[4];
+    #pragma unroll
+                        for (int r = 0; r < 4; r++)
+                            q[r] = requant_s8(acc[c][4 * g + t][r], ss[r], relu, half_even);
+                        words[t] = pack4_s8(q[0], q[1], q[2], q[3]);
                     }
-            } else {
-#pragma unroll
-                for (int t = 0; t < 4; t++)
-                    for (int r = 0; r < 4; r++)
-                        if (n + 4 * t + r < a.N) {
-                            int v = (int)(int8_t)(words[t] >> (8 * r));
+                    if (has_lut) {
+                        const int v = words[t];
+                        words[t] = pack4_s8(lut_l[(int)(int8_t)v + 128], lut_l[(int)(int8_t)(v >> 8) + 128],
+                                            lut_l[(int)(int8_t)(v >> 16) + 128], lut_l[(v >> 24) + 128]);
+                    }
+                }
+                if (m >= a.M || n >= a.N)
+                    continue;
+                const long long goff = m * a.N + n;
+                if (a.out_vec == 16 && n + 16 <= a.N) {
+                    v4i v = {words[0], words[1], words[2], words[3]};
+                    if (a.res != nullptr) {
+                        const v4i r = *reinterpret_cast<const v4i *>(a.res + goff);
+    #pragma unroll
+                        for (int d = 0; d < 4; d++)
+                            v[d] = sat_add4_s8(v[d], r[d]);
+                    }
+                    __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(a.out + goff));
+                } else if (a.out_vec >= 4) {
+    #pragma unroll
+                    for (int t = 0; t < 4; t++)
+                        if (n + 4 * t + 4 <= a.N) {
+                            int v = words[t];
                             if (a.res != nullptr)
-                                v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
-                            a.out[goff + 4 * t + r] = (int8_t)v;
+                                v = sat_add4_s8(v, *reinterpret_cast<const int *>(a.res + goff + 4 * t));
+                            *reinterpret_cast<int *>(a.out + goff + 4 * t) = v;
                         }
+                } else {
+    #pragma unroll
+                    for (int t = 0; t < 4; t++)
+                        for (int r = 0; r < 4; r++)
+                            if (n + 4 * t + r < a.N) {
+                                int v = (int)(int8_t)(words[t] >> (8 * r));
+                                if (a.res != nullptr)
+                                    v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
+                                a.out[goff + 4 * t + r] = (int8_t)v;
+                            }
+                }
             }
         }
-    }
+    };
+    if (half_even)
+        epilogue(std::integral_constant<int, 2>{});
+    else
+        epilogue(std::integral_constant<int, 1>{});
 }
 
 } // namespace

@@ -110,7 +110,7 @@ __device__ __forceinline__ void dw_fetch(const DwLdsArgs &a, const UnitPos &u, i
     }
 }
 
-template <bool FAST, bool USE_LSH>
+template <bool FAST, int USE_LSH>
 __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *smem, int wave, int lane,
                                            const int (&tapoff)[kKs], int floor_pk)
 {
@@ -195,7 +195,8 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
     }
 }
 
-template <bool PROJ>
+// HE: the round-half-even build (a separate kernel so that the half-up build keeps its register count).
+template <bool PROJ, bool HE>
 __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwLdsArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -275,7 +276,7 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
     }
     // start values and shifts: every thread owns at most one channel of the chunk (16 * gc <= 256)
     const long long mac_bound = (long long)a.taps * 16384;
-    int ok_local = half_even ? 0 : 1;
+    int ok_local = 1;
     int lsh_local = 0;
     int my_s = 0, my_b = 0;
     if (tid < cw) {
@@ -342,7 +343,7 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
         }
         const int ocp = a.p_nrt * 16;
         const long long bound = (long long)C * 16384;
-        int okp = half_even ? 0 : 1;
+        int okp = 1;
         int ps = 0, pb = 0;
         if (tid < pj.out_c) {
             ps = pj.shift[pj.n_shift == 1 ? 0 : tid];
@@ -379,12 +380,16 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
             dw_fetch(a, u, cc0, in_rel, in_rc, pv); // in flight during the compute phase
         }
 
-        if (fast && !use_lsh)
-            dw_compute<true, false>(a, smem, wave, lane, tapoff, floor_pk);
+        // epilogue mode of pack_fast4: 0 plain (every shift >= 8), 1 with the left shift, 2 the same with
+        // round-half-even
+        if (fast && HE)
+            dw_compute<true, 2>(a, smem, wave, lane, tapoff, floor_pk);
+        else if (fast && !use_lsh)
+            dw_compute<true, 0>(a, smem, wave, lane, tapoff, floor_pk);
         else if (fast)
-            dw_compute<true, true>(a, smem, wave, lane, tapoff, floor_pk);
+            dw_compute<true, 1>(a, smem, wave, lane, tapoff, floor_pk);
         else
-            dw_compute<false, false>(a, smem, wave, lane, tapoff, floor_pk);
+            dw_compute<false, 0>(a, smem, wave, lane, tapoff, floor_pk);
         __syncthreads();
 
         if (PROJ) {
@@ -411,7 +416,7 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
                 int word;
                 if (fast_p) {
                     const v4i ls = *reinterpret_cast<const v4i *>(cp + 2 * ocp + c);
-                    word = pack_fast4<true>(r, ls, ss, floor_p);
+                    word = pack_fast4<HE ? 2 : 1>(r, ls, ss, floor_p);
                 } else {
                     int q[4];
 #pragma unroll
@@ -636,11 +641,18 @@ hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
     a.fd_np = make_fastdiv((unsigned)a.np);
     a.fd_pvecs = make_fastdiv((unsigned)max(1, a.p_vecs));
     const int cus = cu_count > 0 ? cu_count : 256;
-    static const hipError_t lds_opt_in = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ>),
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+    static const hipError_t lds_opt_in = [] {
+        const hipError_t e0 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, false>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, true>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
+        return e0 != hipSuccess ? e0 : e1;
+    }();
     if (lds_opt_in != hipSuccess)
         return lds_opt_in;
-    const int per_cu = resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ>, kThreads, plan.lds);
+    const bool he = g.half_even != 0;
+    const int per_cu = he ? resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, true>, kThreads, plan.lds)
+                          : resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, false>, kThreads, plan.lds);
     int gx = max(1, (cus * per_cu) / plan.n_cchunk);
     if (gx > a.n_units)
         gx = a.n_units;
@@ -651,8 +663,12 @@ hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
         fprintf(stderr, "depthwise_s8_lds%s: %dx%dx%d s%d tile %dx%d patch %dx%d gc %d np %d lds %zu per_cu %d grid %dx%d units %d\n",
                 PROJ ? "+project" : "", g.in_h, g.in_w, g.in_c, g.stride_h, a.th, a.tw, a.ph, a.pw, a.gc, a.np, plan.lds,
                 per_cu, gx, plan.n_cchunk, a.n_units);
-    hipLaunchKernelGGL(depthwise_s8_lds_kernel<PROJ>, dim3((unsigned)gx, (unsigned)plan.n_cchunk), dim3(kThreads),
-                       plan.lds, stream, a);
+    if (he)
+        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, true>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
+                           dim3(kThreads), plan.lds, stream, a);
+    else
+        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, false>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
+                           dim3(kThreads), plan.lds, stream, a);
     return hipGetLastError();
 }
 

@@ -142,7 +142,7 @@ __device__ __forceinline__ void dw_block(const DwMfmaArgs &a, unsigned char *sme
     }
     // epilogue constants; the short form needs every shift in 1..31 and no possible overflow
     const long long mac_bound = (long long)a.taps * 16384;
-    int ok_local = half_even ? 0 : 1;
+    int ok_local = 1;
     for (int c = tid; c < 16 * NT; c += kThreads) {
         const int s = a.shift[g.n_shift == 1 ? 0 : cb + c];
         const long long bv = a.bias != nullptr ? (long long)a.bias[cb + c] : 0;
@@ -212,7 +212,7 @@ __device__ __forceinline__ void dw_block(const DwMfmaArgs &a, unsigned char *sme
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 if (fast) {
-                    words[t] = pack_fast4<true>(acc[t], ls[t], ss[t], floor_pk);
+                    words[t] = half_even ? pack_fast4<2>(acc[t], ls[t], ss[t], floor_pk) : pack_fast4<1>(acc[t], ls[t], ss[t], floor_pk);
                 } else {
                     int q[4];
 #pragma unroll

@@ -94,15 +94,29 @@ typedef short v2s __attribute__((ext_vector_type(2)));
 // Short requantization of four accumulators that already hold bias + 2^(s-1): after the shifts the
 // result q sits in bits 8.. of t; v_cvt_pk_i16_i32 saturates t to int16, which saturates q to int8
 // in the high byte; ReLU is one packed max on the int16 pairs; v_perm_b32 gathers the four high bytes.
-// USE_LSH: some shift is below 8, so the value is first shifted left by max(0, 8-s).
-template <bool USE_LSH>
-__device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk)
+// MODE 0: every shift is at least 8, round half up.  MODE 1: some shift is below 8, so the value is
+// first shifted left by max(0, 8-s).  MODE 2: as 1 with round-half-even.  MODE 3: as 1, half-even
+// when `he` is set (a run-time choice, for kernels whose register budget rules out one more
+// compiled copy of their main loop).  Half-up and half-even
+// differ only at exact ties, where half-up gives q + 1 and half-even the even one of q, q + 1;
+// acc = value + 2^(s-1) is a tie iff its low s bits are zero, so the half-even result is the half-up
+// result minus one when that holds and the half-up result is odd (the rule of
+// esp-dl/dl/tool/src/dl_tool.cpp:95-119, stated on acc instead of the value).
+template <int MODE>
+__device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk, bool he = false)
 {
     int t[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        const int v = USE_LSH ? (int)((unsigned)acc[r] << lsh[r]) : acc[r];
+        const int v = MODE != 0 ? (int)((unsigned)acc[r] << lsh[r]) : acc[r];
         t[r] = v >> rsh[r];
+        if (MODE == 2 || (MODE == 3 && he)) {
+            // t = q * 256 + (top 8 fraction bits); the other fraction bits left with the shift by rsh.
+            // All fraction bits are zero iff putting q back in place gives v again.  Written with rsh
+            // only, so that no further per-channel constant has to live across the pixel loop.
+            const bool tie = (int)((unsigned)(t[r] & ~0xff) << rsh[r]) == v;
+            t[r] -= tie ? (t[r] & 0x100) : 0;
+        }
     }
     // floor_pk holds the lower clamp twice as int16: 0 for ReLU, -32768 (no effect) otherwise
     const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);

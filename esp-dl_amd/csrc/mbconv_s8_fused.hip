@@ -91,7 +91,7 @@ __device__ __forceinline__ int mb_pack_r(const v4i &acc, const v4i &ss, const v4
                                          bool half_even, int floor_pk)
 {
     if (fast)
-        return pack_fast4<true>(acc, ls, ss, floor_pk);
+        return half_even ? pack_fast4<2>(acc, ls, ss, floor_pk) : pack_fast4<1>(acc, ls, ss, floor_pk);
     int q[4];
 #pragma unroll
     for (int r = 0; r < 4; r++)
@@ -186,8 +186,6 @@ __global__ __launch_bounds__(kThreads) void mbconv_s8_fused_kernel(const MbArgs 
         }
         if (tid < p.out_c && !mb_short_ok(s_p, b_p, (long long)p.exp_c * 16384))
             bad |= 4;
-        if (half_even)
-            bad = 7;
         // the vote is a logical OR of a predicate, so one vote per stage
         fast_e = __syncthreads_or(bad & 1) == 0;
         fast_d = __syncthreads_or(bad & 2) == 0;

@@ -152,6 +152,35 @@ def test_conv2d_s8_pointwise_tiled_gemm(oracle, case, variant):
     np.testing.assert_array_equal(got, want)
 
 
+# Round-half-even differs from half-up only at exact ties; small operands and small shifts make ties
+# frequent (a quarter to a half of all outputs), on every kernel route that has the short epilogue.
+@pytest.mark.parametrize("route", ["dense3x3", "pointwise_tiled", "pointwise_large", "depthwise", "depthwise_s2"])
+@pytest.mark.parametrize("shift_lo,shift_hi", [(1, 3), (2, 9), (8, 10)])
+def test_half_even_ties(oracle, route, shift_lo, shift_hi):
+    announce(f"half-even ties {route} shifts {shift_lo}..{shift_hi}")
+    rng = np.random.default_rng(900 + shift_lo)
+    dw = route.startswith("depthwise")
+    if route == "dense3x3":
+        shape, oc, k, stride, pads = (2, 12, 12, 16), 32, (3, 3), (1, 1), (1, 1, 1, 1)
+    elif route == "pointwise_tiled":
+        shape, oc, k, stride, pads = (2, 9, 9, 64), 48, (1, 1), (1, 1), (0, 0, 0, 0)
+    elif route == "pointwise_large":
+        shape, oc, k, stride, pads = (2, 9, 9, 24), 40, (1, 1), (1, 1), (0, 0, 0, 0)
+    elif route == "depthwise":
+        shape, oc, k, stride, pads = (2, 14, 14, 32), 32, (3, 3), (1, 1), (1, 1, 1, 1)
+    else:
+        shape, oc, k, stride, pads = (2, 15, 15, 48), 48, (3, 3), (2, 2), (1, 1, 1, 1)
+    x = rng.integers(-4, 5, size=shape).astype(np.int8)
+    f = rng.integers(-4, 5, size=(k[0], k[1], shape[3]) if dw else (oc, k[0], k[1], shape[3])).astype(np.int8)
+    bias = rng.integers(-8, 9, size=oc).astype(np.int32)
+    shift = rng.integers(shift_lo, shift_hi + 1, size=oc).astype(np.int32)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, (1, 1), pads, False, depthwise=dw, half_even=True)
+    np.testing.assert_array_equal(got, want)
+    up, _ = _run_conv_s8(oracle, x, f, bias, shift, k, stride, (1, 1), pads, False, depthwise=dw, half_even=False)
+    if shift_hi <= 9:
+        assert (up != got).mean() > 0.01  # the two modes really differ on this input
+
+
 @pytest.mark.parametrize("m,k,n,has_bias,relu", GEMM_CASES)
 def test_gemm_s8(oracle, m, k, n, has_bias, relu):
     announce(f"gemm_s8 M={m} K={k} N={n}")
