@@ -35,8 +35,8 @@ MACHINE_BALANCE = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)  # OP per byte
 # 256 MiB element-wise kernel of known traffic gave in the same runs).  Only valid for config 3 at
 # batch 256; any other workload reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "depthwise_s8": (7 * (2 * 55393.4 + 15715.5) + 10 * (2 * 9880.8 + 17404.8)) / 17 * 1024,
-    "conv2d_s8_mfma": (2 * 6669.5 + 33968.3) * 1024,
+    "depthwise_s8": (7 * (2 * 55393.8 + 15717.6) + 10 * (2 * 9887.8 + 17404.8)) / 17 * 1024,
+    "conv2d_s8": (2 * 8334.9 + 35596.5) * 1024,
     "elementwise_s8": None,
 }
 
@@ -45,11 +45,11 @@ def kernel_family(info, spec_nodes):
     """Map a module to the kernel that runs it."""
     node = spec_nodes.get(info["name"])
     if info["type"] in ("Gemm", "MatMul"):
-        return "conv2d_s8_mfma"
+        return "conv2d_s8"
     if info["type"] == "Conv":
         if node and node["attrs"].get("quant_type") == "S16":
             return "depthwise_s16" if node["attrs"].get("group", 1) != 1 else "conv2d_s16"
-        return "depthwise_s8" if node and node["attrs"].get("group", 1) != 1 else "conv2d_s8_mfma"
+        return "depthwise_s8" if node and node["attrs"].get("group", 1) != 1 else "conv2d_s8"
     if info["type"] in ("Flatten", "Squeeze", "Reshape", "Unsqueeze"):
         return "view"
     return "elementwise_s8"
@@ -193,7 +193,7 @@ def main():
                       "ops_per_byte": round(ai, 1)}
     dom = max(kernels, key=lambda k: kernels[k]["us_per_step"])
     kd = kernels[dom]
-    if dom in ("conv2d_s8_mfma",) and kd["ops_per_byte"] > MACHINE_BALANCE:
+    if dom in ("conv2d_s8",) and kd["ops_per_byte"] > MACHINE_BALANCE:
         roofline = {"kernel": dom, "bound": "mfma", "achieved": kd["TOPs"], "peak": PEAK_INT8_TOPS,
                     "unit": "TOP/s", "frac": kd["mfma_frac"], "traffic": None}
     else:
