@@ -63,6 +63,9 @@ def lib():
         L.espdl_hip_clip_s8.argtypes = [vp, i64, i32, i32, i32, i32, vp, vp]
         L.espdl_hip_add_s8.argtypes = [ctypes.POINTER(i32 * 4), ctypes.POINTER(i64 * 4), ctypes.POINTER(i64 * 4),
                                        vp, vp, vp, vp]
+        L.espdl_hip_mul_s8.argtypes = [ctypes.POINTER(i32 * 4), ctypes.POINTER(i64 * 4), ctypes.POINTER(i64 * 4),
+                                       vp, vp, i32, i32, vp, vp]
+        L.espdl_hip_mul_s8.restype = ctypes.c_int
         L.espdl_hip_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp]
         L.espdl_hip_requantize_s8.argtypes = [vp, i64, i32, i32, vp, vp]
         L.espdl_hip_requantize.argtypes = [vp, i32, i64, i32, i32, vp, i32, vp]
@@ -197,8 +200,7 @@ def _pad4(shape):
     return [1] * (4 - len(shape)) + shape
 
 
-def add_s8(a, b, out=None, stream=None):
-    """numpy-style broadcasting add of two contiguous tensors (up to 4 dims)."""
+def _broadcast(a, b, out):
     import torch
     sa, sb = _pad4(a.shape), _pad4(b.shape)
     so = [max(x, y) for x, y in zip(sa, sb)]
@@ -213,11 +215,22 @@ def add_s8(a, b, out=None, stream=None):
     rank = max(a.dim(), b.dim())
     if out is None:
         out = torch.empty(so[4 - rank:] if rank else [], dtype=torch.int8, device=a.device)
-    dims = (ctypes.c_int32 * 4)(*so)
-    s0 = (ctypes.c_int64 * 4)(*strides(sa))
-    s1 = (ctypes.c_int64 * 4)(*strides(sb))
+    return (ctypes.c_int32 * 4)(*so), (ctypes.c_int64 * 4)(*strides(sa)), (ctypes.c_int64 * 4)(*strides(sb)), out
+
+
+def add_s8(a, b, out=None, stream=None):
+    """numpy-style broadcasting add of two contiguous tensors (up to 4 dims)."""
+    dims, s0, s1, out = _broadcast(a, b, out)
     _check(lib().espdl_hip_add_s8(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), _p(out),
                                   _stream(stream)))
+    return out
+
+
+def mul_s8(a, b, shift, round_mode=ROUND_HALF_UP, out=None, stream=None):
+    """numpy-style broadcasting product; shift = out_exp - a_exp - b_exp."""
+    dims, s0, s1, out = _broadcast(a, b, out)
+    _check(lib().espdl_hip_mul_s8(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), int(shift),
+                                  round_mode, _p(out), _stream(stream)))
     return out
 
 

@@ -130,8 +130,23 @@ hipError_t launch_map(const int8_t *in, int8_t *out, int64_t size, F f, hipStrea
 }
 
 // c_impl_add_n_n / _n_1 / _1_n (esp-dl/dl/base/dl_base_add.cpp:8-44): clamp(a + b).
-__global__ __launch_bounds__(kBlock) void add_s8_dense_kernel(const int8_t *in0, const int8_t *in1, int8_t *out,
-                                                              int64_t size, int64_t vecs)
+// Binary element-wise operators on two int8 tensors: Op::apply(a, b) per element.
+//   AddOp  elemwise_add, c_impl_add_n_n (esp-dl/dl/base/dl_base_add.cpp:8-44): clamp(a + b)
+//   MulOp  elemwise_mul, c_impl_mul_n_n (esp-dl/dl/base/dl_base_mul.cpp:33-46): the product rescaled by
+//          2^-(out_exp - e0 - e1) with round-half-up (the float expression there is exact for these
+//          operands) or, for the ESP32-P4 behaviour, round-half-even; then clamped
+struct AddOp {
+    __device__ __forceinline__ int apply(int a, int b) const { return clamp_s8(a + b); }
+};
+struct MulOp {
+    int shift;
+    bool half_even;
+    __device__ __forceinline__ int apply(int a, int b) const { return requant_s8(a * b, shift, false, half_even); }
+};
+
+template <typename Op>
+__global__ __launch_bounds__(kBlock) void binary_s8_dense_kernel(const int8_t *in0, const int8_t *in1, int8_t *out,
+                                                                 int64_t size, int64_t vecs, Op op)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < vecs) {
@@ -142,26 +157,25 @@ __global__ __launch_bounds__(kBlock) void add_s8_dense_kernel(const int8_t *in0,
         for (int w = 0; w < 4; w++) {
             int o = 0;
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const int s = (int)(int8_t)(a[w] >> (8 * k)) + (int)(int8_t)(b[w] >> (8 * k));
-                o |= (clamp_s8(s) & 0xff) << (8 * k);
-            }
+            for (int k = 0; k < 4; k++)
+                o |= (op.apply((int)(int8_t)(a[w] >> (8 * k)), (int)(int8_t)(b[w] >> (8 * k))) & 0xff) << (8 * k);
             r[w] = o;
         }
         reinterpret_cast<v4i *>(out)[i] = r;
     }
     const int64_t t = vecs * 16 + i;
     if (t < size)
-        out[t] = (int8_t)clamp_s8((int)in0[t] + (int)in1[t]);
+        out[t] = (int8_t)op.apply((int)in0[t], (int)in1[t]);
 }
 
-struct AddBroadcastArgs {
+struct BroadcastArgs {
     int d[4];
     long long s0[4], s1[4];
 };
 
-__global__ __launch_bounds__(kBlock) void add_s8_broadcast_kernel(const int8_t *in0, const int8_t *in1, int8_t *out,
-                                                                  int64_t size, AddBroadcastArgs a)
+template <typename Op>
+__global__ __launch_bounds__(kBlock) void binary_s8_broadcast_kernel(const int8_t *in0, const int8_t *in1, int8_t *out,
+                                                                     int64_t size, BroadcastArgs a, Op op)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= size)
@@ -175,7 +189,41 @@ __global__ __launch_bounds__(kBlock) void add_s8_broadcast_kernel(const int8_t *
     const int i0 = (int)(rest / a.d[1]);
     const long long o0 = i0 * a.s0[0] + i1 * a.s0[1] + i2 * a.s0[2] + i3 * a.s0[3];
     const long long o1 = i0 * a.s1[0] + i1 * a.s1[1] + i2 * a.s1[2] + i3 * a.s1[3];
-    out[i] = (int8_t)clamp_s8((int)in0[o0] + (int)in1[o1]);
+    out[i] = (int8_t)op.apply((int)in0[o0], (int)in1[o1]);
+}
+
+template <typename Op>
+hipError_t launch_binary_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
+                            const int8_t *in1, int8_t *out, Op op, hipStream_t stream)
+{
+    const int64_t size = (int64_t)dims[0] * dims[1] * dims[2] * dims[3];
+    if (size <= 0)
+        return hipSuccess;
+    // dense strides of the output shape
+    int64_t dense[4];
+    dense[3] = 1;
+    for (int i = 2; i >= 0; i--)
+        dense[i] = dense[i + 1] * dims[i + 1];
+    bool both_dense = true;
+    for (int i = 0; i < 4; i++)
+        if (dims[i] > 1 && (s0[i] != dense[i] || s1[i] != dense[i]))
+            both_dense = false;
+    if (both_dense) {
+        const bool vec_ok = aligned16(in0, in1) && aligned16(out, out);
+        int64_t vecs;
+        const dim3 grid = grid_for(size, vec_ok, &vecs);
+        hipLaunchKernelGGL(binary_s8_dense_kernel<Op>, grid, dim3(kBlock), 0, stream, in0, in1, out, size, vecs, op);
+    } else {
+        BroadcastArgs a;
+        for (int i = 0; i < 4; i++) {
+            a.d[i] = dims[i];
+            a.s0[i] = dims[i] > 1 ? s0[i] : 0;
+            a.s1[i] = dims[i] > 1 ? s1[i] : 0;
+        }
+        hipLaunchKernelGGL(binary_s8_broadcast_kernel<Op>, dim3((unsigned)((size + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           stream, in0, in1, out, size, a, op);
+    }
+    return hipGetLastError();
 }
 
 // GlobalAveragePool: avgpool2d_hwc with the window covering the image
@@ -281,34 +329,13 @@ hipError_t launch_requantize_any(const void *in, int in_bits, int64_t size, int 
 hipError_t launch_add_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
                          const int8_t *in1, int8_t *out, hipStream_t stream)
 {
-    const int64_t size = (int64_t)dims[0] * dims[1] * dims[2] * dims[3];
-    if (size <= 0)
-        return hipSuccess;
-    // dense strides of the output shape
-    int64_t dense[4];
-    dense[3] = 1;
-    for (int i = 2; i >= 0; i--)
-        dense[i] = dense[i + 1] * dims[i + 1];
-    bool both_dense = true;
-    for (int i = 0; i < 4; i++)
-        if (dims[i] > 1 && (s0[i] != dense[i] || s1[i] != dense[i]))
-            both_dense = false;
-    if (both_dense) {
-        const bool vec_ok = aligned16(in0, in1) && aligned16(out, out);
-        int64_t vecs;
-        const dim3 grid = grid_for(size, vec_ok, &vecs);
-        hipLaunchKernelGGL(add_s8_dense_kernel, grid, dim3(kBlock), 0, stream, in0, in1, out, size, vecs);
-    } else {
-        AddBroadcastArgs a;
-        for (int i = 0; i < 4; i++) {
-            a.d[i] = dims[i];
-            a.s0[i] = dims[i] > 1 ? s0[i] : 0;
-            a.s1[i] = dims[i] > 1 ? s1[i] : 0;
-        }
-        hipLaunchKernelGGL(add_s8_broadcast_kernel, dim3((unsigned)((size + kBlock - 1) / kBlock)), dim3(kBlock), 0,
-                           stream, in0, in1, out, size, a);
-    }
-    return hipGetLastError();
+    return launch_binary_s8(dims, s0, s1, in0, in1, out, AddOp{}, stream);
+}
+
+hipError_t launch_mul_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
+                         const int8_t *in1, int shift, int half_even, int8_t *out, hipStream_t stream)
+{
+    return launch_binary_s8(dims, s0, s1, in0, in1, out, MulOp{shift, half_even != 0}, stream);
 }
 
 hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,

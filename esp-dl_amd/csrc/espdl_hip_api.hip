@@ -282,6 +282,34 @@ int espdl_hip_add_s8(const int32_t out_dims[4], const int64_t in0_strides[4], co
         "add_s8");
 }
 
+int espdl_hip_mul_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int32_t mul_shift, int32_t round_mode, int8_t *out,
+                     void *stream)
+{
+    if (out_dims == nullptr || in0_strides == nullptr || in1_strides == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "dims and strides must not be NULL");
+    if (mul_shift < -60 || mul_shift > 60)
+        return fail(ESPDL_HIP_EINVAL, "mul_shift %d outside [-60, 60]", mul_shift);
+    if (round_mode != ESPDL_HIP_ROUND_HALF_UP && round_mode != ESPDL_HIP_ROUND_HALF_EVEN)
+        return fail(ESPDL_HIP_EINVAL, "bad round_mode %d", round_mode);
+    long long size = 1;
+    for (int i = 0; i < 4; i++) {
+        if (out_dims[i] < 0 || in0_strides[i] < 0 || in1_strides[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative extent or stride in dim %d", i);
+        size *= out_dims[i];
+        if (size > (1ll << 40))
+            return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    }
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in0 == nullptr || in1 == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in0, in1 and out must not be NULL");
+    return device_status(espdl::launch_mul_s8(out_dims, in0_strides, in1_strides, in0, in1, mul_shift,
+                                              round_mode == ESPDL_HIP_ROUND_HALF_EVEN, out,
+                                              reinterpret_cast<hipStream_t>(stream)),
+                         "mul_s8");
+}
+
 int espdl_hip_global_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t in_exp,
                                  int32_t out_exp, int8_t *out, void *stream)
 {

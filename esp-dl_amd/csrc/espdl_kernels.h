@@ -92,6 +92,8 @@ hipError_t launch_clip_s8(const int8_t *in, int64_t size, int min_q, int max_q, 
                           hipStream_t stream);
 hipError_t launch_add_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
                          const int8_t *in1, int8_t *out, hipStream_t stream);
+hipError_t launch_mul_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
+                         const int8_t *in1, int shift, int half_even, int8_t *out, hipStream_t stream);
 hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
                                      int8_t *out, hipStream_t stream);
 hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out,

@@ -17,17 +17,21 @@ namespace dl {
 namespace module {
 
 /// Fill the requantization shifts of a Conv / Gemm / MatMul from the tensors' exponents.
-inline std::vector<int32_t> conv_shifts(TensorBase *output, TensorBase *input, TensorBase *filter, int out_c)
+inline std::vector<int32_t> conv_shifts(int out_exponent, TensorBase *input, TensorBase *filter, int out_c)
 {
     std::vector<int32_t> shifts;
     if (filter->exponent.is_per_channel()) {
         shifts.resize(out_c);
         for (int c = 0; c < out_c; c++)
-            shifts[c] = output->exponent.get() - filter->exponent.get(c) - input->exponent.get();
+            shifts[c] = out_exponent - filter->exponent.get(c) - input->exponent.get();
     } else {
-        shifts.push_back(output->exponent.get() - filter->exponent.get() - input->exponent.get());
+        shifts.push_back(out_exponent - filter->exponent.get() - input->exponent.get());
     }
     return shifts;
+}
+inline std::vector<int32_t> conv_shifts(TensorBase *output, TensorBase *input, TensorBase *filter, int out_c)
+{
+    return conv_shifts(output->exponent.get(), input, filter, out_c);
 }
 
 class Conv : public Module {
@@ -45,6 +49,7 @@ private:
     bool m_has_project = false;
     activation_type_t m_project_activation = Linear;
     int m_mid_exponent = 0;      ///< exponent of the (no longer materialized) depthwise output
+    int m_lut_in_exponent = 0;   ///< exponent of the conv result that indexes a fused LUT
     int m_project_filter_pos = -1, m_project_bias_pos = -1, m_residual_pos = -1;
     int m_own_inputs = 0; ///< inputs of the Conv itself when a plain residual Add was absorbed
     DeviceInts m_shift_project;
@@ -67,10 +72,14 @@ public:
     int get_group() const { return m_group; }
     activation_type_t get_activation() const { return activation; }
     /// Take ownership of a LUT (host or device tensor of 256 int8) to apply in the epilogue.
-    void fuse_lut(TensorBase *table)
+    /// `table_in_exponent` is the exponent of the value the table is indexed with, i.e. of this
+    /// convolution's own (no longer materialized) output: the requantization shift is derived from it,
+    /// not from the exponent of the tensor the table's result is stored to.
+    void fuse_lut(TensorBase *table, int table_in_exponent)
     {
         delete m_fused_lut;
         m_fused_lut = table;
+        m_lut_in_exponent = table_in_exponent;
     }
     bool has_fused_lut() const { return m_fused_lut != nullptr; }
     bool has_fused_project() const { return m_has_project; }
@@ -210,7 +219,8 @@ public:
             return;
         }
         d.round_mode = context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP;
-        const std::vector<int32_t> shifts = conv_shifts(output, input, filter, d.out_c);
+        const std::vector<int32_t> shifts =
+            conv_shifts(m_fused_lut ? m_lut_in_exponent : output->exponent.get(), input, filter, d.out_c);
         d.n_shift = (int32_t)shifts.size();
         const int32_t *shift_dev = m_shift.sync(shifts);
         if (m_fused_lut && !m_fused_lut->on_device()) {

@@ -57,6 +57,7 @@ public:
         register_module("PRelu", PRelu::deserialize);
         register_module("Clip", Clip::deserialize);
         register_module("Add", Add::deserialize);
+        register_module("Mul", Mul::deserialize);
         register_module("GlobalAveragePool", GlobalAveragePool::deserialize);
         register_module("RequantizeLinear", RequantizeLinear::deserialize);
         register_module("Flatten", Flatten::deserialize);

@@ -304,9 +304,25 @@ public:
             DL_LOGE("Add", "%s: needs int8 device tensors of rank <= 4", name.c_str());
             return;
         }
-        int32_t dims[4] = {1, 1, 1, 1};
-        int64_t s0[4] = {0, 0, 0, 0}, s1[4] = {0, 0, 0, 0};
+        int32_t dims[4];
+        int64_t s0[4], s1[4];
+        broadcast_layout(input0, input1, output, dims, s0, s1);
+        const int rc = espdl_hip_add_s8(dims, s0, s1, static_cast<const int8_t *>(input0->data),
+                                        static_cast<const int8_t *>(input1->data), static_cast<int8_t *>(output->data),
+                                        context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Add", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+
+    /// Output extents padded to 4 dims and element strides of both inputs per output dim (0 = broadcast).
+    static void broadcast_layout(TensorBase *input0, TensorBase *input1, TensorBase *output, int32_t dims[4],
+                                 int64_t s0[4], int64_t s1[4])
+    {
         const size_t rank = output->shape.size();
+        for (int i = 0; i < 4; i++) {
+            dims[i] = 1;
+            s0[i] = s1[i] = 0;
+        }
         for (size_t i = 0; i < rank; i++)
             dims[4 - rank + i] = output->shape[i];
         auto strides = [&](TensorBase *t, int64_t *s) {
@@ -319,11 +335,6 @@ public:
         };
         strides(input0, s0);
         strides(input1, s1);
-        const int rc = espdl_hip_add_s8(dims, s0, s1, static_cast<const int8_t *>(input0->data),
-                                        static_cast<const int8_t *>(input1->data), static_cast<int8_t *>(output->data),
-                                        context->stream);
-        if (rc != ESPDL_HIP_OK)
-            DL_LOGE("Add", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
 
     static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
@@ -333,6 +344,48 @@ public:
         return new Add(node_name.c_str(), MODULE_INPLACE_CHANGED_BUFFER, quant_type);
     }
     void print() { DL_LOGI("Add", "quant_type: %s.", quant_type_to_string(quant_type)); }
+};
+
+/// Mul with numpy-style broadcasting (esp-dl/dl/module/include/dl_module_mul.hpp, base::elemwise_mul).
+/// Rounds like the rest of the model: half up for the portable C path, half even when the context
+/// runs ESP32-P4 semantics (the P4 kernels of this operator set the hardware rounding that way).
+class Mul : public Add {
+public:
+    Mul(const char *name = nullptr, module_inplace_t inplace = MODULE_NON_INPLACE,
+        quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Add(name, inplace, quant_type)
+    {
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input0 = context->get_tensor(m_inputs_index[0]);
+        TensorBase *input1 = context->get_tensor(m_inputs_index[1]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !on_device_all({input0, input1, output}) ||
+            output->shape.size() > 4) {
+            DL_LOGE("Mul", "%s: needs int8 device tensors of rank <= 4", name.c_str());
+            return;
+        }
+        int32_t dims[4];
+        int64_t s0[4], s1[4];
+        broadcast_layout(input0, input1, output, dims, s0, s1);
+        const int shift = output->exponent.get() - input0->exponent.get() - input1->exponent.get();
+        const int rc = espdl_hip_mul_s8(dims, s0, s1, static_cast<const int8_t *>(input0->data),
+                                        static_cast<const int8_t *>(input1->data), shift,
+                                        context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN
+                                                                                    : ESPDL_HIP_ROUND_HALF_UP,
+                                        static_cast<int8_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Mul", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        return new Mul(node_name.c_str(), MODULE_INPLACE_CHANGED_BUFFER, quant_type);
+    }
+    void print() { DL_LOGI("Mul", "quant_type: %s.", quant_type_to_string(quant_type)); }
 };
 
 class GlobalAveragePool : public Module {

@@ -217,7 +217,8 @@ void Model::fuse_conv_lut()
         auto *lut = dynamic_cast<dl::module::LUT *>(m_execution_plan[lut_pos]);
         if (!lut || lut->quant_type != QUANT_TYPE_SYMM_8BIT || !lut->get_table() || lut->get_table()->get_size() != 256)
             continue;
-        conv->fuse_lut(lut->release_table());
+        conv->fuse_lut(lut->release_table(),
+                       m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(mid)));
         conv->m_outputs_index[0] = lut->m_outputs_index[0];
         delete lut;
         m_execution_plan.erase(m_execution_plan.begin() + lut_pos);

@@ -239,6 +239,19 @@ class Builder:
         g.add_node(name, "Add", [a, b], [y], quant_type="S8")
         return y
 
+    def mul(self, a, b, out_exp=None, name=None):
+        """Element-wise product (numpy broadcasting).  Default output exponent keeps the larger operand's
+        scale when the other one is a gate in [0, 1)."""
+        g = self.g
+        name = name or self._name("mul")
+        y = name + "_out"
+        sa, sb = g.shape(a), g.shape(b)
+        rank = max(len(sa), len(sb))
+        pa, pb = [1] * (rank - len(sa)) + sa, [1] * (rank - len(sb)) + sb
+        g.add_value(y, [max(u, v) for u, v in zip(pa, pb)], g.exponent(a) if out_exp is None else out_exp)
+        g.add_node(name, "Mul", [a, b], [y], quant_type="S8")
+        return y
+
     def global_avg_pool(self, x, out_exp=None, name=None):
         g = self.g
         name = name or self._name("gap")
@@ -530,3 +543,23 @@ CONFIGS = {
     4: config4_yolo_style,
     5: config5_ocr_style,
 }
+
+
+def gated_block(seed=0xE5D6):
+    """Conv blocks with x * sigmoid(x) written as Sigmoid (8-bit LUT) + Mul, a squeeze-and-excitation
+    gate (GlobalAveragePool -> 1x1 Conv -> Sigmoid LUT -> Mul broadcast over H x W) and a residual Add:
+    the operator mix of the reference's exported streaming / SE models."""
+    g = GraphSpec("gated_block")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 20, 20, 32], -5)
+    h = b.conv(x, 64, k=3, name="c1")
+    s = b.lut(h, lambda v: 1.0 / (1.0 + np.exp(-v)), "Sigmoid", out_exp=-7, name="c1_sig")
+    h = b.mul(h, s, name="c1_gate")                      # same shape
+    sq = b.global_avg_pool(h, name="se_pool")
+    sq = b.conv(sq, 64, k=1, name="se_fc")
+    sq = b.lut(sq, lambda v: 1.0 / (1.0 + np.exp(-v)), "Sigmoid", out_exp=-7, name="se_sig")
+    h = b.mul(h, sq, name="se_scale")                    # [1,20,20,64] * [1,1,1,64]
+    y = b.conv(h, 32, k=1, name="c2")
+    y = b.add(x, y, name="res")
+    b.output(y)
+    return g

@@ -122,6 +122,17 @@ int espdl_hip_clip_s8(const int8_t *in, int64_t size, int32_t min_q, int32_t max
 int espdl_hip_add_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
                      const int8_t *in0, const int8_t *in1, int8_t *out, void *stream);
 
+/*
+ * base::elemwise_mul for int8 (esp-dl/dl/base/dl_base_mul.cpp:33-46, 83-160), same broadcast description
+ * as espdl_hip_add_s8.  mul_shift = out_exp - in0_exp - in1_exp (elemwiseArgsType::mul_shift,
+ * dl_base_elemwise.cpp:167): out = clamp(round(in0 * in1 / 2^mul_shift)); a negative shift multiplies.
+ * ESPDL_HIP_ROUND_HALF_UP is the portable C path; ESPDL_HIP_ROUND_HALF_EVEN is how the ESP32-P4 kernels
+ * of the reference round this operator.
+ */
+int espdl_hip_mul_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int32_t mul_shift, int32_t round_mode, int8_t *out,
+                     void *stream);
+
 /* GlobalAveragePool over H x W per image and channel: base::avgpool2d_hwc with the filter covering
  * the whole image (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54). out is [batch][1][1][c]. */
 int espdl_hip_global_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t in_exp,

@@ -442,6 +442,31 @@ void espdl_oracle_add_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int
 }
 
 /*
+ * Mul, int8 (esp-dl/dl/base/dl_base_mul.cpp:9-46, 130-141; scales dl_base_elemwise.cpp:167-171):
+ * out = truncate(round(float(a * b) * rescale)), rescale = DL_SCALE(e0) * DL_SCALE(e1) * DL_RESCALE(eout),
+ * a product of powers of two, passed here as shift = eout - e0 - e1 (rescale = 2^-shift).  The portable C
+ * path rounds half up (tool::round).  round_mode half-even restates what the ESP32-P4 kernels do for this
+ * operator (they configure the hardware rounding, dl_base_mul.cpp:90): shift_and_round half-even of the
+ * integer product.  len0 / len1 are `size` or 1 (scalar operand).
+ */
+void espdl_oracle_mul_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size, int shift,
+                         int round_mode, int8_t *out)
+{
+    const float rescale = dl_rescale(shift); /* 2^-shift */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < size; i++) {
+        const int32_t a = in0[len0 == 1 ? 0 : i], b = in1[len1 == 1 ? 0 : i];
+        const int32_t prod = a * b;
+        int64_t q;
+        if (round_mode == ESPDL_ORACLE_ROUND_HALF_EVEN && shift > 0)
+            q = espdl_oracle_shift_round_s32(prod, shift, ESPDL_ORACLE_ROUND_HALF_EVEN);
+        else
+            q = (int64_t)floorf((float)prod * rescale + 0.5f);
+        out[i] = (int8_t)clamp_i64(q, INT8_MIN, INT8_MAX);
+    }
+}
+
+/*
  * GlobalAveragePool = avgpool2d_hwc over the whole image (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54):
  * int32 sum per channel, then truncate(round(float(sum) * scale)),
  * scale = DL_SCALE(in_exp) * (1.f / area) * DL_RESCALE(out_exp) evaluated left to right in float32.

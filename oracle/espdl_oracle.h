@@ -41,6 +41,8 @@
  *                                within float rounding error of a tie; the reference itself
  *                                cannot be built here (every translation unit needs ESP-IDF
  *                                headers that are absent)                   PARITY UNPINNED (near-ties)
+ *   espdl_oracle_mul_s8          exhaustive over all int8 operand pairs and shifts -4..14 against round-half-up
+ *                                (and the half-even table) of the exact product in rationals        PINNED
  *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
  *                                numpy.split / numpy.transpose on random shapes           PINNED
  *   espdl_oracle_max_pool        equality with scipy.ndimage.maximum_filter (minimum-value border)
@@ -101,6 +103,9 @@ void espdl_oracle_clip_s8(const int8_t *in, int64_t size, int min_q, int max_q, 
 /* Broadcast add: len0 / len1 are `size` or 1 (scalar operand). */
 void espdl_oracle_add_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size,
                          int8_t *out);
+/* shift = out_exp - in0_exp - in1_exp; operands broadcast as in espdl_oracle_add_s8. */
+void espdl_oracle_mul_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size, int shift,
+                         int round_mode, int8_t *out);
 void espdl_oracle_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
                                      int8_t *out);
 void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out);

@@ -58,6 +58,7 @@ def lib():
         L.espdl_oracle_add_s8.argtypes = [vp, i64, vp, i64, i64, vp]
         L.espdl_oracle_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp]
         L.espdl_oracle_requantize_s8.argtypes = [vp, i64, i32, i32, vp]
+        L.espdl_oracle_mul_s8.argtypes = [vp, i64, vp, i64, i64, i32, i32, vp]
         L.espdl_oracle_concat.argtypes = [vp, i32, vp, i64, i32, vp]
         L.espdl_oracle_split_slice.argtypes = [vp, i64, i64, i64, i64, i64, i32, vp]
         L.espdl_oracle_transpose.restype = i32
@@ -204,6 +205,17 @@ def add_s8(a, b):
     assert a.size in (1, size) and b.size in (1, size)
     out = np.empty(a.shape if a.size == size else b.shape, dtype=np.int8)
     lib().espdl_oracle_add_s8(_ptr(a), a.size, _ptr(b), b.size, size, _ptr(out))
+    return out
+
+
+def mul_s8(a, b, shift, round_mode=ROUND_HALF_UP):
+    """Element-wise product; a scalar operand broadcasts.  shift = out_exp - a_exp - b_exp."""
+    a = _c(a, np.int8)
+    b = _c(b, np.int8)
+    size = max(a.size, b.size)
+    assert a.size in (1, size) and b.size in (1, size)
+    out = np.empty(a.shape if a.size == size else b.shape, dtype=np.int8)
+    lib().espdl_oracle_mul_s8(_ptr(a), a.size, _ptr(b), b.size, size, int(shift), int(round_mode), _ptr(out))
     return out
 
 

@@ -60,6 +60,12 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             b = t[ins[1]]
             assert x.shape == b.shape, "the graph runner only needs same-shape residual adds"
             y = oracle.add_s8(x, b)
+        elif op == "Mul":
+            b = t[ins[1]]
+            shift = spec.exponent(y_name) - spec.exponent(ins[0]) - spec.exponent(ins[1])
+            if x.shape != b.shape:  # broadcast explicitly: the oracle takes equal sizes or a scalar
+                x, b = np.broadcast_arrays(x, b)
+            y = oracle.mul_s8(np.ascontiguousarray(x), np.ascontiguousarray(b), shift, round_mode)
         elif op == "GlobalAveragePool":
             y = oracle.global_avg_pool_s8(x, spec.exponent(ins[0]), spec.exponent(y_name))
         elif op == "RequantizeLinear":

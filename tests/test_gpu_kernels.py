@@ -393,6 +393,20 @@ def test_add_s8(oracle, sa, sb):
         np.testing.assert_array_equal(got.ravel(), oracle.add_s8(a, b).ravel())
 
 
+@pytest.mark.parametrize("sa,sb", ADD_SHAPES, ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shift,half_even", [(7, False), (7, True), (1, True), (0, False), (-2, False), (12, False)])
+def test_mul_s8(oracle, sa, sb, shift, half_even):
+    announce(f"mul_s8 {sa} * {sb} shift {shift} half_even={half_even}")
+    m = espdl()
+    rng = np.random.default_rng(31)
+    a, b = rng_int8(rng, sa), rng_int8(rng, sb)
+    ab, bb = np.broadcast_arrays(a, b)
+    want = oracle.mul_s8(np.ascontiguousarray(ab), np.ascontiguousarray(bb), shift,
+                         oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP)
+    got = to_host(m.mul_s8(to_dev(a), to_dev(b), shift, m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP))
+    np.testing.assert_array_equal(got, want)
+
+
 def test_global_avg_pool_s8(oracle):
     announce("global_avg_pool_s8")
     m = espdl()

@@ -205,6 +205,19 @@ def test_config4_neck_data_movement_tensors(oracle):
     mdl.close()
 
 
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+def test_gated_block_with_mul(oracle, round_mode):
+    """Sigmoid LUT + Mul gates (same-shape and broadcast over H x W), both rounding modes."""
+    announce(f"model gated_block round_mode={round_mode}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.gated_block()
+    mdl, want, _ = _run_config(spec, 4, 21, round_mode=round_mode)
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
+        assert want[name].min() < want[name].max()
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()

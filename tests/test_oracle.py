@@ -351,3 +351,27 @@ def test_global_avg_pool_non_ties(oracle):
                 assert got[n, c] == max(-128, min(127, math.floor(frac)))
                 checked += 1
         assert checked > 100
+
+
+def test_mul_s8_exhaustive(oracle):
+    """All int8 operand pairs, shifts -4..14: round-half-up of the exact product (half-even table for the
+    ESP32-P4 rounding), clamped; the float expression of the reference is exact for these operands."""
+    a = np.repeat(np.arange(-128, 128, dtype=np.int8), 256)
+    b = np.tile(np.arange(-128, 128, dtype=np.int8), 256)
+    prod = a.astype(np.int64) * b.astype(np.int64)
+    for shift in range(-4, 15):
+        got = oracle.mul_s8(a, b, shift).astype(np.int64)
+        if shift > 0:
+            want = (prod + (1 << (shift - 1))) >> shift  # floor(p / 2^s + 1/2) in exact integers
+        else:
+            want = prod << -shift
+        np.testing.assert_array_equal(got, np.clip(want, -128, 127), err_msg=f"shift {shift}")
+        if shift > 0:
+            he = oracle.mul_s8(a, b, shift, oracle.ROUND_HALF_EVEN).astype(np.int64)
+            q, r = prod >> shift, prod & ((1 << shift) - 1)
+            h = 1 << (shift - 1)
+            want_he = q + ((r > h) | ((r == h) & ((q & 1) == 1)))
+            np.testing.assert_array_equal(he, np.clip(want_he, -128, 127), err_msg=f"half-even shift {shift}")
+    # scalar operand
+    np.testing.assert_array_equal(oracle.mul_s8(a[:512], np.array([3], dtype=np.int8), 1),
+                                  np.clip((a[:512].astype(np.int64) * 3 + 1) >> 1, -128, 127))
