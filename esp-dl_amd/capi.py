@@ -75,7 +75,9 @@ def lib():
         L.espdl_hip_transpose.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
         L.espdl_hip_resize_nearest_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, vp, vp]
         L.espdl_hip_max_pool.argtypes = [vp, i32] + [i32] * 12 + [vp, vp]
-        for name in ("concat", "copy_rows", "transpose", "resize_nearest_s8", "max_pool"):
+        L.espdl_hip_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp, vp]
+        L.espdl_hip_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp, vp]
+        for name in ("concat", "copy_rows", "transpose", "resize_nearest_s8", "max_pool", "avg_pool_s8", "slice"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         mp = ctypes.POINTER(MbconvDesc)
         L.espdl_hip_mbconv_out_shape.argtypes = [mp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
@@ -336,4 +338,28 @@ def max_pool(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0), out=None, stream=None
     out = torch.empty((n, max(oh, 0), max(ow, 0), c), dtype=x.dtype, device=x.device) if out is None else out
     _check(lib().espdl_hip_max_pool(_p(x), S16 if x.dtype == torch.int16 else S8, n, h, w, c, kernel[0], kernel[1],
                                     strides[0], strides[1], pt, pb, pl, pr, _p(out), _stream(stream)))
+    return out
+
+
+def avg_pool_s8(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0), in_exp=0, out_exp=0, out=None, stream=None):
+    """pads = (top, bottom, left, right); x int8 NHWC."""
+    import torch
+    n, h, w, c = x.shape
+    pt, pb, pl, pr = pads
+    oh = (h + pt + pb - kernel[0]) // strides[0] + 1
+    ow = (w + pl + pr - kernel[1]) // strides[1] + 1
+    out = torch.empty((n, max(oh, 0), max(ow, 0), c), dtype=torch.int8, device=x.device) if out is None else out
+    _check(lib().espdl_hip_avg_pool_s8(_p(x), n, h, w, c, kernel[0], kernel[1], strides[0], strides[1], pt, pb, pl, pr,
+                                       in_exp, out_exp, _p(out), _stream(stream)))
+    return out
+
+
+def slice_(x, start, step, out_shape, out=None, stream=None):
+    """out[i...] = x[start + i * step ...]; start / step / out_shape have one entry per dim of x."""
+    import torch
+    nd = x.dim()
+    out = torch.empty(list(out_shape), dtype=x.dtype, device=x.device) if out is None else out
+    arr = lambda v: (ctypes.c_int32 * nd)(*[int(t) for t in v])  # noqa: E731
+    _check(lib().espdl_hip_slice(_p(x), arr(x.shape), nd, arr(start), arr(step), arr(out_shape), x.element_size(),
+                                 _p(out), _stream(stream)))
     return out

@@ -484,6 +484,59 @@ int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, 
                          "max_pool");
 }
 
+int espdl_hip_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,
+                          int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom, int32_t pad_left,
+                          int32_t pad_right, int32_t in_exp, int32_t out_exp, int8_t *out, void *stream)
+{
+    if (batch < 0 || h <= 0 || w <= 0 || c <= 0 || k_h <= 0 || k_w <= 0 || stride_h <= 0 || stride_w <= 0 || pad_top < 0 ||
+        pad_bottom < 0 || pad_left < 0 || pad_right < 0 || (long long)k_h * k_w > (1 << 23))
+        return fail(ESPDL_HIP_EINVAL, "bad avg_pool geometry");
+    if (h + pad_top + pad_bottom < k_h || w + pad_left + pad_right < k_w)
+        return fail(ESPDL_HIP_EINVAL, "window larger than the padded image");
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    const int out_h = (h + pad_top + pad_bottom - k_h) / stride_h + 1, out_w = (w + pad_left + pad_right - k_w) / stride_w + 1;
+    if (batch == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_avg_pool_s8(in, batch, h, w, c, k_h, k_w, stride_h, stride_w, pad_top, pad_left,
+                                                   out_h, out_w, in_exp, out_exp, out, cu_count_cached(),
+                                                   reinterpret_cast<hipStream_t>(stream)),
+                         "avg_pool_s8");
+}
+
+int espdl_hip_slice(const void *in, const int32_t *shape, int32_t dims, const int32_t *start, const int32_t *step,
+                    const int32_t *out_shape, int32_t elem_size, void *out, void *stream)
+{
+    if (dims < 1 || dims > 8 || shape == nullptr || start == nullptr || step == nullptr || out_shape == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "slice handles 1..8 dims");
+    if (elem_size != 1 && elem_size != 2 && elem_size != 4)
+        return fail(ESPDL_HIP_EINVAL, "elem_size must be 1, 2 or 4");
+    int sh[8], st[8], sp[8], os[8];
+    long long total = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0 || out_shape[i] < 0 || step[i] < 1 || start[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "dim %d: negative extent or start, or step below 1", i);
+        if (out_shape[i] > 0 && (long long)start[i] + (long long)(out_shape[i] - 1) * step[i] >= shape[i])
+            return fail(ESPDL_HIP_EINVAL, "dim %d: the slice leaves the tensor", i);
+        sh[i] = shape[i];
+        st[i] = start[i];
+        sp[i] = step[i];
+        os[i] = out_shape[i];
+        total *= out_shape[i];
+    }
+    if (total == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    if (misaligned(in, (size_t)elem_size) || misaligned(out, (size_t)elem_size))
+        return fail(ESPDL_HIP_EINVAL, "tensors must be aligned to the element size");
+    return device_status(espdl::launch_slice(in, sh, dims, st, sp, os, elem_size, out, cu_count_cached(),
+                                             reinterpret_cast<hipStream_t>(stream)),
+                         "slice");
+}
+
 } // extern "C"
 
 namespace {

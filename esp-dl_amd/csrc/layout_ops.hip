@@ -269,6 +269,63 @@ __global__ __launch_bounds__(kBlock) void max_pool_kernel(const PoolArgs a)
     }
 }
 
+// AveragePool (esp-dl/dl/base/dl_base_avg_pool2d.cpp:28-54): int32 sums over the clipped window, one
+// float multiply, round half up, clamp.  One thread per (output pixel, 16 channels) or per element.
+struct AvgPoolArgs {
+    PoolArgs p;
+    float scale;
+};
+
+__global__ __launch_bounds__(kBlock) void avg_pool_s8_kernel(const AvgPoolArgs args)
+{
+    const PoolArgs &a = args.p;
+    const int8_t *in = reinterpret_cast<const int8_t *>(a.in);
+    int8_t *out = reinterpret_cast<int8_t *>(a.out);
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < a.total; i += (long long)gridDim.x * kBlock) {
+        const unsigned pix = fastdiv((unsigned)i, a.fd_cv);
+        const unsigned v = (unsigned)i - pix * a.fd_cv.d;
+        const unsigned row = fastdiv(pix, a.fd_ow);
+        const unsigned x = pix - row * a.fd_ow.d;
+        const unsigned n = fastdiv(row, a.fd_oh);
+        const unsigned y = row - n * a.fd_oh.d;
+        const int iy0 = (int)y * a.stride_h - a.pad_top, ix0 = (int)x * a.stride_w - a.pad_left;
+        const int ky0 = max(0, -iy0), ky1 = min(a.k_h, a.h - iy0);
+        const int kx0 = max(0, -ix0), kx1 = min(a.k_w, a.w - ix0);
+        const long long img = (long long)n * a.h * a.w;
+        const long long dst = (long long)pix * a.c + (long long)v * a.vec;
+        if (a.vec == 16) {
+            int sum[16];
+#pragma unroll
+            for (int k = 0; k < 16; k++)
+                sum[k] = 0;
+            for (int ky = ky0; ky < ky1; ky++)
+                for (int kx = kx0; kx < kx1; kx++) {
+                    const v4i cur = *reinterpret_cast<const v4i *>(in + (img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.c +
+                                                                   (long long)v * 16);
+#pragma unroll
+                    for (int k = 0; k < 16; k++)
+                        sum[k] += (int)(int8_t)(cur[k >> 2] >> (8 * (k & 3)));
+                }
+            v4i r;
+#pragma unroll
+            for (int wd = 0; wd < 4; wd++) {
+                int o = 0;
+#pragma unroll
+                for (int b = 0; b < 4; b++)
+                    o |= (clamp_s8(round_half_up_f32((float)sum[4 * wd + b] * args.scale)) & 0xff) << (8 * b);
+                r[wd] = o;
+            }
+            *reinterpret_cast<v4i *>(out + dst) = r;
+        } else {
+            int sum = 0;
+            for (int ky = ky0; ky < ky1; ky++)
+                for (int kx = kx0; kx < kx1; kx++)
+                    sum += in[(img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.c + v];
+            out[dst] = (int8_t)clamp_s8(round_half_up_f32((float)sum * args.scale));
+        }
+    }
+}
+
 } // namespace
 
 hipError_t launch_copy_rows(const void *src, long long src_pitch, void *dst, long long dst_pitch, long long row_bytes,
@@ -490,6 +547,76 @@ hipError_t launch_max_pool(const void *in, int elem_size, int batch, int h, int 
         hipLaunchKernelGGL((max_pool_kernel<int8_t, v16c>), grid, dim3(kBlock), 0, stream, a);
     else
         hipLaunchKernelGGL((max_pool_kernel<int16_t, v8s>), grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
+                              int stride_w, int pad_top, int pad_left, int out_h, int out_w, int in_exp, int out_exp,
+                              int8_t *out, int cu_count, hipStream_t stream)
+{
+    AvgPoolArgs args;
+    PoolArgs &a = args.p;
+    a.in = reinterpret_cast<const char *>(in);
+    a.out = reinterpret_cast<char *>(out);
+    a.h = h;
+    a.w = w;
+    a.c = c;
+    a.out_h = out_h;
+    a.out_w = out_w;
+    a.k_h = k_h;
+    a.k_w = k_w;
+    a.stride_h = stride_h;
+    a.stride_w = stride_w;
+    a.pad_top = pad_top;
+    a.pad_left = pad_left;
+    const bool vec_ok = (c & 15) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    a.vec = vec_ok ? 16 : 1;
+    const int cv = c / a.vec;
+    a.total = (long long)batch * out_h * out_w * cv;
+    if (a.total <= 0)
+        return hipSuccess;
+    if (a.total > 0x7fffffffll) // fastdiv range
+        return hipErrorInvalidValue;
+    a.fd_cv = make_fastdiv((unsigned)cv);
+    a.fd_ow = make_fastdiv((unsigned)out_w);
+    a.fd_oh = make_fastdiv((unsigned)out_h);
+    // the scale the reference forms, left to right in float32
+    const float area_inv = 1.f / (float)(k_h * k_w);
+    args.scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
+    hipLaunchKernelGGL(avg_pool_s8_kernel, dim3(blocks_for(a.total, cu_count)), dim3(kBlock), 0, stream, args);
+    return hipGetLastError();
+}
+
+// Slice with positive steps: a gather whose element strides are the input strides times the steps.
+hipError_t launch_slice(const void *in, const int *shape, int dims, const int *start, const int *step, const int *out_shape,
+                        int elem_size, void *out, int cu_count, hipStream_t stream)
+{
+    TransposeArgs a = {};
+    long long in_stride[kMaxDims];
+    in_stride[dims - 1] = 1;
+    for (int i = dims - 2; i >= 0; i--)
+        in_stride[i] = in_stride[i + 1] * shape[i + 1];
+    long long base = 0, total = 1;
+    for (int i = 0; i < dims; i++) {
+        base += (long long)start[i] * in_stride[i];
+        a.out_shape[i] = out_shape[i];
+        a.in_stride[i] = in_stride[i] * step[i];
+        total *= out_shape[i];
+    }
+    if (total <= 0)
+        return hipSuccess;
+    a.in = static_cast<const char *>(in) + base * elem_size;
+    a.out = static_cast<char *>(out);
+    a.dims = dims;
+    a.esize = elem_size;
+    a.total = total;
+    const dim3 grid(blocks_for(total, cu_count));
+    if (elem_size == 1)
+        hipLaunchKernelGGL(transpose_general_kernel<int8_t>, grid, dim3(kBlock), 0, stream, a);
+    else if (elem_size == 2)
+        hipLaunchKernelGGL(transpose_general_kernel<int16_t>, grid, dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL(transpose_general_kernel<int32_t>, grid, dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 

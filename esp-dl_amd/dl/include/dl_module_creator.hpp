@@ -69,6 +69,8 @@ public:
         register_module("Transpose", Transpose::deserialize);
         register_module("Resize", Resize::deserialize);
         register_module("MaxPool", MaxPool::deserialize);
+        register_module("AveragePool", AveragePool::deserialize);
+        register_module("Slice", Slice::deserialize);
         // element-wise activations that esp-ppq exports with a precomputed 8-bit table
         for (const char *op : {"Swish", "HardSwish", "Sigmoid", "HardSigmoid", "Tanh", "Gelu", "Elu", "LeakyRelu",
                                "Exp", "Log", "Sqrt", "Softplus", "Mish"}) {

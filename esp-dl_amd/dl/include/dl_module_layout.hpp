@@ -1,4 +1,5 @@
-// Data-movement operator objects: Concat, Split, Transpose, Resize, MaxPool.  Each mirrors the
+// Data-movement and pooling operator objects: Concat, Split, Transpose, Resize, MaxPool, AveragePool,
+// Slice.  Each mirrors the
 // reference module of the same name (same attributes, shape rules and error behaviour) and enqueues
 // kernels of include/espdl_hip.h on the context's stream.
 //   Concat     esp-dl/dl/module/include/dl_module_concat.hpp:14-127
@@ -6,8 +7,11 @@
 //   Transpose  esp-dl/dl/module/include/dl_module_transpose.hpp:12-88
 //   Resize     esp-dl/dl/module/include/dl_module_resize.hpp:14-180 (nearest mode)
 //   MaxPool    esp-dl/dl/module/include/dl_module_max_pool.hpp:13-131
+//   AveragePool esp-dl/dl/module/include/dl_module_average_pool.hpp
+//   Slice      esp-dl/dl/module/include/dl_module_slice.hpp
 #pragma once
 
+#include <algorithm>
 #include <cassert>
 #include <cstring>
 
@@ -391,6 +395,165 @@ public:
         DL_LOGI("MaxPool", "kernel: %dx%d, quant_type: %s.", m_filter_shape[0], m_filter_shape.size() > 1 ? m_filter_shape[1] : 1,
                 quant_type_to_string(quant_type));
     }
+};
+
+/// AveragePool on int8 NHWC / NWC tensors, portable C path arithmetic
+/// (esp-dl/dl/module/include/dl_module_average_pool.hpp; attributes as MaxPool; `ceil_mode` and
+/// `count_include_pad` are read by neither the reference's shape rule nor its C kernel).
+class AveragePool : public Module {
+private:
+    std::vector<int> m_kernel_shape, m_pads, m_strides;
+
+public:
+    AveragePool(const char *name = nullptr, const std::vector<int> &kernel_shape = {2, 2},
+                const std::vector<int> &pads = {0, 0, 0, 0}, const std::vector<int> &strides = {1, 1},
+                quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_kernel_shape(kernel_shape), m_pads(pads), m_strides(strides)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        assert(in.size() == 3 || in.size() == 4);
+        std::vector<int> out = in;
+        out[1] = (in[1] + m_pads[0] + m_pads[1] - m_kernel_shape[0]) / m_strides[0] + 1;
+        if (in.size() == 4)
+            out[2] = (in[2] + m_pads[2] + m_pads[3] - m_kernel_shape[1]) / m_strides[1] + 1;
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) || quant_type != QUANT_TYPE_SYMM_8BIT) {
+            DL_LOGE("AveragePool", "%s: needs int8 device tensors", name.c_str());
+            return;
+        }
+        const bool nwc = input->shape.size() == 3;
+        const int h = nwc ? 1 : input->shape[1], w = nwc ? input->shape[1] : input->shape[2];
+        const int c = nwc ? input->shape[2] : input->shape[3];
+        const int kh = nwc ? 1 : m_kernel_shape[0], kw = nwc ? m_kernel_shape[0] : m_kernel_shape[1];
+        const int sh = nwc ? 1 : m_strides[0], sw = nwc ? m_strides[0] : m_strides[1];
+        const int pt = nwc ? 0 : m_pads[0], pb = nwc ? 0 : m_pads[1];
+        const int pl = nwc ? m_pads[0] : m_pads[2], pr = nwc ? m_pads[1] : m_pads[3];
+        const int rc = espdl_hip_avg_pool_s8(static_cast<const int8_t *>(input->data), input->shape[0], h, w, c, kh, kw, sh,
+                                             sw, pt, pb, pl, pr, input->exponent.get(), output->exponent.get(),
+                                             static_cast<int8_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("AveragePool", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        std::vector<int> kernel_shape, pads, strides;
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "kernel_shape", kernel_shape);
+        fbs_model->get_operation_attribute(node_name, "pads", pads);
+        fbs_model->get_operation_attribute(node_name, "strides", strides);
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        if (kernel_shape.empty())
+            return nullptr;
+        if (pads.size() == 4) // ONNX [top, left, bottom, right] -> [top, bottom, left, right]
+            pads = {pads[0], pads[2], pads[1], pads[3]};
+        else if (pads.empty())
+            pads.assign(kernel_shape.size() * 2, 0);
+        if (strides.empty())
+            strides.assign(kernel_shape.size(), 1);
+        return new AveragePool(node_name.c_str(), kernel_shape, pads, strides, quant_type);
+    }
+    void print() { DL_LOGI("AveragePool", "kernel dims: %d, quant_type: %s.", (int)m_kernel_shape.size(), quant_type_to_string(quant_type)); }
+};
+
+/// Slice with positive steps (esp-dl/dl/module/include/dl_module_slice.hpp; ONNX index rules: negative
+/// starts / ends count from the end, both are clamped to the extent).
+class Slice : public Module {
+private:
+    std::vector<int64_t> m_start, m_end, m_axes, m_step;
+    std::vector<int> m_norm_start, m_norm_step;
+
+    bool normalize(const std::vector<int> &shape, std::vector<int> *out_shape)
+    {
+        const int nd = (int)shape.size();
+        m_norm_start.assign(nd, 0);
+        m_norm_step.assign(nd, 1);
+        *out_shape = shape;
+        for (size_t i = 0; i < m_start.size(); i++) {
+            const int ax = m_axes.empty() ? (int)i : (int)((m_axes[i] + nd) % nd);
+            const int64_t st = m_step.empty() ? 1 : m_step[i];
+            if (ax < 0 || ax >= nd || st < 1)
+                return false;
+            const int64_t dim = shape[ax];
+            int64_t s = m_start[i], e = m_end[i];
+            s = s < 0 ? s + dim : s;
+            e = e < 0 ? e + dim : e;
+            s = std::min<int64_t>(std::max<int64_t>(s, 0), dim);
+            e = std::min<int64_t>(std::max<int64_t>(e, 0), dim);
+            m_norm_start[ax] = (int)s;
+            m_norm_step[ax] = (int)st;
+            (*out_shape)[ax] = e > s ? (int)((e - s + st - 1) / st) : 0;
+        }
+        return true;
+    }
+
+public:
+    Slice(const char *name = nullptr, const std::vector<int64_t> &start = {}, const std::vector<int64_t> &end = {},
+          const std::vector<int64_t> &axes = {}, const std::vector<int64_t> &step = {},
+          quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_start(start), m_end(end), m_axes(axes), m_step(step)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        std::vector<int> out;
+        if (!normalize(input_shapes[0], &out)) {
+            DL_LOGE("Slice", "%s: bad axes or a step below 1 (negative steps are not part of this build)", name.c_str());
+            return {input_shapes[0]};
+        }
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) || input->dtype != output->dtype) {
+            DL_LOGE("Slice", "%s: needs device tensors of one type", name.c_str());
+            return;
+        }
+        std::vector<int> out_shape;
+        if (!normalize(input->shape, &out_shape) || out_shape != output->shape) {
+            DL_LOGE("Slice", "%s: output shape does not match the slice", name.c_str());
+            return;
+        }
+        const int rc = espdl_hip_slice(input->data, input->shape.data(), (int32_t)input->shape.size(), m_norm_start.data(),
+                                       m_norm_step.data(), out_shape.data(), (int32_t)input->get_dtype_bytes(),
+                                       output->data, context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Slice", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        std::vector<int64_t> v[4];
+        for (int k = 0; k < 4; k++) {
+            TensorBase *t = fbs_model->get_operation_parameter(node_name, k + 1);
+            if (!t)
+                continue;
+            if (t->dtype == DATA_TYPE_INT64) {
+                const int64_t *p = t->get_element_ptr<int64_t>();
+                v[k].assign(p, p + t->get_size());
+            } else if (t->dtype == DATA_TYPE_INT32) {
+                const int32_t *p = t->get_element_ptr<int32_t>();
+                v[k].assign(p, p + t->get_size());
+            }
+            delete t;
+        }
+        if (v[0].empty() || v[0].size() != v[1].size())
+            return nullptr;
+        return new Slice(node_name.c_str(), v[0], v[1], v[2], v[3], quant_type);
+    }
+    void print() { DL_LOGI("Slice", "axes: %d, quant_type: %s.", (int)m_start.size(), quant_type_to_string(quant_type)); }
 };
 
 } // namespace module

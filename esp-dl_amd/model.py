@@ -144,7 +144,7 @@ class Graph:
         g = cls.__new__(cls)
         g.h = lib().espdl_graph_load_file(os.fsencode(path), model_index)
         if not g.h:
-            raise EspdlModelError("%s: %s" % (path, lib().espdl_graph_load_error().decode()))
+            raise EspdlModelError("%s: %s" % (path, lib().espdl_graph_load_error().decode("utf-8", "replace")))
         return g
 
     @classmethod
@@ -152,7 +152,7 @@ class Graph:
         g = cls.__new__(cls)
         g.h = lib().espdl_graph_load_memory(blob, len(blob), model_index)
         if not g.h:
-            raise EspdlModelError(lib().espdl_graph_load_error().decode())
+            raise EspdlModelError(lib().espdl_graph_load_error().decode("utf-8", "replace"))
         return g
 
     def initializer(self, name, dtype=np.int8):

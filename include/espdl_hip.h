@@ -191,6 +191,21 @@ int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, 
                        int32_t k_w, int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom,
                        int32_t pad_left, int32_t pad_right, void *out, void *stream);
 
+/* base::avg_pool2d<int8_t> on the portable C path (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54 under the
+ * shell of dl_base_pool2d.hpp:439-560): sum over the window clipped to the image, times
+ * 2^in_exp * (1 / (k_h * k_w)) * 2^-out_exp in float32 (the divisor is the full window also at the borders),
+ * round half up, clamp.  Output size as espdl_hip_max_pool. */
+int espdl_hip_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,
+                          int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom, int32_t pad_left,
+                          int32_t pad_right, int32_t in_exp, int32_t out_exp, int8_t *out, void *stream);
+
+/* TensorBase::slice for positive steps (esp-dl/dl/base/dl_base_shape.cpp:68-120 gives the shape rule):
+ * out[i0, i1, ...] = in[start[0] + i0 * step[0], start[1] + i1 * step[1], ...].  The caller passes
+ * normalized values per dim (0 <= start, step >= 1, out_shape) for all `dims` dims of the input;
+ * host arrays.  1..8 dims, elem_size 1, 2 or 4. */
+int espdl_hip_slice(const void *in, const int32_t *shape, int32_t dims, const int32_t *start, const int32_t *step,
+                    const int32_t *out_shape, int32_t elem_size, void *out, void *stream);
+
 /*
  * Inverted-residual block in one launch: [1x1 Conv] -> depthwise Conv -> 1x1 Conv [-> Add].
  * No single reference function does this; it runs the same sequence of module::Conv::forward

@@ -489,6 +489,75 @@ void espdl_oracle_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, 
 }
 
 /*
+ * AveragePool, int8 NHWC (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54 under the pool shell of
+ * dl_base_pool2d.hpp:439-560): int32 sum over the window clipped to the image, then
+ * truncate(round(float(sum) * scale)) with scale = DL_SCALE(in_exp) * (1.f / area) * DL_RESCALE(out_exp)
+ * evaluated left to right in float32.  On the portable C path `area` stays k_h * k_w for every window,
+ * clipped or not (args.avg_pool_area is set once, dl_base_pool2d.hpp:132).  Output size as MaxPool.
+ */
+void espdl_oracle_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
+                              int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,
+                              int out_exp, int8_t *out)
+{
+    const int out_h = (h + pad_top + pad_bottom - k_h) / stride_h + 1;
+    const int out_w = (w + pad_left + pad_right - k_w) / stride_w + 1;
+    const float area_inv = 1.f / (float)(k_h * k_w);
+    const float scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
+#pragma omp parallel for schedule(static)
+    for (int n = 0; n < batch; n++)
+        for (int oy = 0; oy < out_h; oy++)
+            for (int ox = 0; ox < out_w; ox++)
+                for (int k = 0; k < c; k++) {
+                    int32_t sum = 0;
+                    for (int ky = 0; ky < k_h; ky++) {
+                        const int iy = oy * stride_h - pad_top + ky;
+                        if (iy < 0 || iy >= h)
+                            continue;
+                        for (int kx = 0; kx < k_w; kx++) {
+                            const int ix = ox * stride_w - pad_left + kx;
+                            if (ix < 0 || ix >= w)
+                                continue;
+                            sum += in[(((int64_t)n * h + iy) * w + ix) * c + k];
+                        }
+                    }
+                    out[(((int64_t)n * out_h + oy) * out_w + ox) * c + k] =
+                        (int8_t)clamp_i64(round_half_up_f32((float)sum * scale), INT8_MIN, INT8_MAX);
+                }
+}
+
+/*
+ * Slice with ONNX semantics (what base::get_slice_shape, esp-dl/dl/base/dl_base_shape.cpp:68-120, and
+ * TensorBase::slice compute for positive steps): per listed axis take indices start, start + step, ...
+ * below end.  starts / ends / steps here are already normalized to 0 <= start < dim, step >= 1 and the
+ * output extent out_shape[axis]; every other axis is copied whole.  Up to 8 dims.
+ */
+int espdl_oracle_slice(const void *in, const int *shape, int dims, const int *start, const int *step,
+                       const int *out_shape, int elem_size, void *out)
+{
+    if (dims < 1 || dims > 8)
+        return -1;
+    int64_t in_stride[8], total = 1;
+    in_stride[dims - 1] = 1;
+    for (int i = dims - 2; i >= 0; i--)
+        in_stride[i] = in_stride[i + 1] * shape[i + 1];
+    for (int i = 0; i < dims; i++)
+        total *= out_shape[i];
+    int64_t idx[8] = {0};
+    for (int64_t e = 0; e < total; e++) {
+        int64_t src = 0;
+        for (int i = 0; i < dims; i++)
+            src += ((int64_t)start[i] + idx[i] * step[i]) * in_stride[i];
+        memcpy((char *)out + e * elem_size, (const char *)in + src * elem_size, (size_t)elem_size);
+        for (int i = dims - 1; i >= 0; i--) {
+            if (++idx[i] < out_shape[i])
+                break;
+            idx[i] = 0;
+        }
+    }
+    return 0;
+}
+
+/*
  * TensorBase::assign, int8 -> int8 with different exponents
  * (esp-dl/dl/tensor/src/dl_tensor_base.cpp:362-371; quantize/dequantize :18-42):
  * quantize(dequantize(x, DL_SCALE(in_exp)), 1.0 / DL_SCALE(out_exp)).

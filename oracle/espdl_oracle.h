@@ -43,6 +43,10 @@
  *                                headers that are absent)                   PARITY UNPINNED (near-ties)
  *   espdl_oracle_mul_s8          exhaustive over all int8 operand pairs and shifts -4..14 against round-half-up
  *                                (and the half-even table) of the exact product in rationals        PINNED
+ *   espdl_oracle_avg_pool_s8     float32 scale as espdl_oracle_global_avg_pool_s8: exact rational round-half-up away
+ *                                from ties; the reference's streaming-model fixtures (S3 and P4 exports with
+ *                                embedded outputs) pass through it                  PARITY UNPINNED (near-ties)
+ *   espdl_oracle_slice           equality with numpy basic slicing                                   PINNED
  *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
  *                                numpy.split / numpy.transpose on random shapes           PINNED
  *   espdl_oracle_max_pool        equality with scipy.ndimage.maximum_filter (minimum-value border)
@@ -108,6 +112,11 @@ void espdl_oracle_mul_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int
                          int round_mode, int8_t *out);
 void espdl_oracle_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
                                      int8_t *out);
+void espdl_oracle_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
+                              int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,
+                              int out_exp, int8_t *out);
+int espdl_oracle_slice(const void *in, const int *shape, int dims, const int *start, const int *step,
+                       const int *out_shape, int elem_size, void *out);
 void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out);
 
 /* Data-movement operators (see the .c file for the reference lines each one follows). */

@@ -59,6 +59,9 @@ def lib():
         L.espdl_oracle_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp]
         L.espdl_oracle_requantize_s8.argtypes = [vp, i64, i32, i32, vp]
         L.espdl_oracle_mul_s8.argtypes = [vp, i64, vp, i64, i64, i32, i32, vp]
+        L.espdl_oracle_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp]
+        L.espdl_oracle_slice.restype = i32
+        L.espdl_oracle_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp]
         L.espdl_oracle_concat.argtypes = [vp, i32, vp, i64, i32, vp]
         L.espdl_oracle_split_slice.argtypes = [vp, i64, i64, i64, i64, i64, i32, vp]
         L.espdl_oracle_transpose.restype = i32
@@ -307,5 +310,46 @@ def max_pool(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0)):
     out = np.empty((n, oh, ow, c), dtype=x.dtype)
     rc = lib().espdl_oracle_max_pool(_ptr(x), x.dtype.itemsize, n, h, w, c, kernel[0], kernel[1], strides[0], strides[1],
                                      pt, pb, pl, pr, _ptr(out))
+    assert rc == 0
+    return out
+
+
+def avg_pool_s8(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0), in_exp=0, out_exp=0):
+    """pads = (top, bottom, left, right).  int8 NHWC."""
+    x = _c(x, np.int8)
+    n, h, w, c = x.shape
+    pt, pb, pl, pr = pads
+    oh = (h + pt + pb - kernel[0]) // strides[0] + 1
+    ow = (w + pl + pr - kernel[1]) // strides[1] + 1
+    out = np.empty((n, oh, ow, c), dtype=np.int8)
+    lib().espdl_oracle_avg_pool_s8(_ptr(x), n, h, w, c, kernel[0], kernel[1], strides[0], strides[1], pt, pb, pl, pr,
+                                   in_exp, out_exp, _ptr(out))
+    return out
+
+
+def normalize_slice(shape, starts, ends, axes=None, steps=None):
+    """ONNX Slice bookkeeping for positive steps -> (start, step, out_shape) per dim."""
+    nd = len(shape)
+    start, step, out_shape = [0] * nd, [1] * nd, list(shape)
+    for i in range(len(starts)):
+        ax = i if axes is None or len(axes) == 0 else (int(axes[i]) + nd) % nd
+        st = 1 if steps is None or len(steps) == 0 else int(steps[i])
+        assert st >= 1, "negative steps are not part of this build"
+        dim = shape[ax]
+        s, e = int(starts[i]), int(ends[i])
+        s = s + dim if s < 0 else s
+        e = e + dim if e < 0 else e
+        s, e = min(max(s, 0), dim), min(max(e, 0), dim)
+        start[ax], step[ax], out_shape[ax] = s, st, max(0, -(-(e - s) // st))
+    return start, step, out_shape
+
+
+def slice_(x, starts, ends, axes=None, steps=None):
+    x = np.ascontiguousarray(x)
+    start, step, out_shape = normalize_slice(x.shape, starts, ends, axes, steps)
+    out = np.empty(out_shape, dtype=x.dtype)
+    i32 = lambda v: np.array(v, dtype=np.int32)  # noqa: E731
+    sh, st, sp, os_ = i32(x.shape), i32(start), i32(step), i32(out_shape)
+    rc = lib().espdl_oracle_slice(_ptr(x), _ptr(sh), x.ndim, _ptr(st), _ptr(sp), _ptr(os_), x.dtype.itemsize, _ptr(out))
     assert rc == 0
     return out

@@ -28,16 +28,20 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
         if op == "Conv":
             dims, wdt, w, _ = spec.initializers[ins[1]]
             bias = spec.initializers[ins[2]][2] if len(ins) > 2 else None
-            kh, kw = dims[0], dims[1]
-            pt, pl, pb, pr = a["pads"]
             shift = _shift(spec, node, ins[0], ins[1], y_name)
             act = oracle.RELU if a.get("activation", "Linear") == "Relu" else oracle.LINEAR
             depthwise = a.get("group", 1) != 1
             s16 = a.get("quant_type") == "S16"
             fn = {(False, False): oracle.conv2d_s8, (True, False): oracle.depthwise_s8,
                   (False, True): oracle.conv2d_s16, (True, True): oracle.depthwise_s16}[(depthwise, s16)]
-            y = fn(x, w, bias, shift, (kh, kw), tuple(a["strides"]), tuple(a["dilations"]), (pt, pb, pl, pr), act,
-                   round_mode)
+            if x.ndim == 3:  # Conv1d on NWC runs as one image row (dl_module_conv.hpp: 3-D inputs)
+                pl, pr = a["pads"]
+                y = fn(x[:, None], w, bias, shift, (1, dims[0]), (1, a["strides"][0]), (1, a["dilations"][0]),
+                       (0, 0, pl, pr), act, round_mode)[:, 0]
+            else:
+                pt, pl, pb, pr = a["pads"]
+                y = fn(x, w, bias, shift, (dims[0], dims[1]), tuple(a["strides"]), tuple(a["dilations"]),
+                       (pt, pb, pl, pr), act, round_mode)
         elif op in ("Gemm", "MatMul"):
             w = spec.initializers[ins[1]][2]
             bias = spec.initializers[ins[2]][2] if len(ins) > 2 else None
@@ -74,6 +78,18 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             y = x.reshape(x.shape[0], -1)
         elif op == "Squeeze":
             y = np.squeeze(x, axis=tuple(a["axes"]))
+        elif op == "AveragePool":
+            k, st, pads = list(a["kernel_shape"]), list(a.get("strides") or [1] * len(a["kernel_shape"])), list(a.get("pads") or [])
+            if x.ndim == 3:  # NWC runs as one row
+                pl, pr = pads if pads else (0, 0)
+                y = oracle.avg_pool_s8(x[:, None], (1, k[0]), (1, st[0]), (0, 0, pl, pr), spec.exponent(ins[0]),
+                                       spec.exponent(y_name))[:, 0]
+            else:
+                pt, pl, pb, pr = pads if pads else (0, 0, 0, 0)
+                y = oracle.avg_pool_s8(x, tuple(k), tuple(st), (pt, pb, pl, pr), spec.exponent(ins[0]), spec.exponent(y_name))
+        elif op == "Slice":
+            par = [spec.initializers[n][2].ravel() if n in spec.initializers else None for n in (ins[1:5] + [None] * 4)[:4]]
+            y = oracle.slice_(x, par[0], par[1], par[2], par[3])
         elif op == "MaxPool":
             pt, pl, pb, pr = a["pads"]
             y = oracle.max_pool(x, tuple(a["kernel_shape"]), tuple(a["strides"]), (pt, pb, pl, pr))

@@ -5,6 +5,9 @@ source code.  Run in the development container:  python tests/golden/copy_espdl_
 
   test_apps/esp-dl/models/{c,esp32s3,esp32p4}/Gemm/*.espdl   one int8 Gemm each, three targets
   examples/tutorial/how_to_run_model/main/models/{s3,p4}/model.espdl   three chained int8 Gemms
+  examples/tutorial/how_to_deploy_streaming_model/test_streaming_model/main/models/{esp32s3,esp32p4}/model.espdl
+      a Conv1d network: dense and dilated depthwise Conv1d, Sigmoid tables, Mul, Add, AveragePool,
+      Transpose, Slice, Flatten, Gemm
 """
 import glob
 import os
@@ -25,6 +28,11 @@ def main():
     for target in ("s3", "p4"):
         src = os.path.join(REF, "examples/tutorial/how_to_run_model/main/models", target, "model.espdl")
         shutil.copyfile(src, os.path.join(OUT, "gemm_chain_%s.espdl" % target))
+        n += 1
+    for target in ("esp32s3", "esp32p4"):
+        src = os.path.join(REF, "examples/tutorial/how_to_deploy_streaming_model/test_streaming_model/main/models",
+                           target, "model.espdl")
+        shutil.copyfile(src, os.path.join(OUT, "conv1d_net_%s.espdl" % target))
         n += 1
     print("copied", n, "files to", OUT)
 

@@ -23,23 +23,15 @@ def _py_reader():
     return espdl_reader
 
 
-def _n_major(t):
-    """Python restatement of the blocked layout -> [N][spatial][C] (dims are [spatial..., C, N])."""
-    dims, data, doc = t["dims"], t["data"].ravel(), t["doc"] or ""
-    if "16" not in doc:
-        return data
-    n, c = dims[-1], dims[-2]
-    sp = int(np.prod(dims[:-2]))
-    nb, tail = n // 16, n % 16
-    out = np.zeros((n, sp, c), dtype=data.dtype)
-    out[:nb * 16] = data[:nb * 16 * sp * c].reshape(nb, sp, c, 16).transpose(0, 3, 1, 2).reshape(nb * 16, sp, c)
-    if tail:
-        out[nb * 16:] = data[nb * 16 * sp * c:].reshape(tail, sp, c)  # remainder: plain filter-major
-    return out.ravel()
+def _spec(path):
+    import sys
+    sys.path.insert(0, HERE)
+    import espdl_spec
+    return espdl_spec.spec_from_espdl(path)[0]
 
 
 def test_fixtures_are_present():
-    assert len(FIXTURES) == 11
+    assert len(FIXTURES) == 13
 
 
 @pytest.mark.parametrize("path", FIXTURES, ids=os.path.basename)
@@ -49,9 +41,8 @@ def test_loader_matches_python_reader(path):
     assert g.input_names() == [v["name"] for v in ref["inputs"]]
     assert g.output_names() == [v["name"] for v in ref["outputs"]]
     np_of = {3: np.int8, 5: np.int16, 6: np.int32, 7: np.int64, 1: np.float32}
-    for name, t in ref["initializers"].items():
-        got = g.initializer(name, np_of[t["dtype"]])
-        np.testing.assert_array_equal(got, _n_major(t), err_msg=name)
+    for name, (dims, dtype, data, _) in _spec(path).initializers.items():
+        np.testing.assert_array_equal(g.initializer(name, np_of[dtype]), np.asarray(data).ravel(), err_msg=name)
 
 
 def test_blocked_and_plain_targets_hold_the_same_filters():
@@ -70,7 +61,7 @@ def test_blocked_and_plain_targets_hold_the_same_filters():
 
 def test_damaged_files_are_refused_not_crashed_on():
     model = _model_mod()
-    blob = open(FIXTURES[3], "rb").read()
+    blob = open([f for f in FIXTURES if "gemm_chain_s3" in f][0], "rb").read()
     with pytest.raises(model.EspdlModelError):
         model.Graph.from_bytes(b"XXXX" + blob[4:])
     with pytest.raises(model.EspdlModelError):

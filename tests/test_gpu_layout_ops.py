@@ -91,6 +91,33 @@ def test_max_pool(oracle, shape, kernel, strides, pads, dtype):
     np.testing.assert_array_equal(got, oracle.max_pool(x, kernel, strides, pads))
 
 
+@pytest.mark.parametrize("shape,kernel,strides,pads,exps", [
+    ((2, 1, 24, 32), (1, 3), (1, 1), (0, 0, 2, 0), (-6, -7)), ((2, 14, 14, 64), (3, 3), (1, 1), (1, 1, 1, 1), (-5, -5)),
+    ((3, 16, 16, 24), (2, 2), (2, 2), (0, 0, 0, 0), (-4, -5)), ((2, 7, 7, 1280), (7, 7), (1, 1), (0, 0, 0, 0), (-3, -4)),
+    ((1, 9, 11, 5), (3, 2), (2, 1), (1, 0, 0, 1), (-5, -3)),
+])
+def test_avg_pool_s8(oracle, shape, kernel, strides, pads, exps):
+    announce(f"avg_pool {shape} k{kernel} s{strides} p{pads} exps {exps}")
+    x = _rand(np.random.default_rng(26), shape)
+    got = to_host(espdl().avg_pool_s8(to_dev(x), kernel, strides, pads, exps[0], exps[1]))
+    np.testing.assert_array_equal(got, oracle.avg_pool_s8(x, kernel, strides, pads, exps[0], exps[1]))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("shape,starts,ends,axes,steps", [
+    ((2, 16, 24), [-3], [2 ** 63 - 1], [2], [1]), ((2, 5, 10, 8), [1], [4], [1], [2]),
+    ((2, 5, 10, 8), [0, 2, 1], [1, 9, 100], [0, 2, 3], [1, 3, 1]), ((3, 4, 4, 64), [0], [64], [-1], [4]),
+    ((6,), [2], [5], None, None),
+])
+def test_slice(oracle, shape, starts, ends, axes, steps, dtype):
+    announce(f"slice {shape} {starts}:{ends} axes {axes} steps {steps} {dtype.__name__}")
+    x = _rand(np.random.default_rng(27), shape, dtype)
+    want = oracle.slice_(x, starts, ends, axes, steps)
+    start, step, out_shape = oracle.normalize_slice(x.shape, starts, ends, axes, steps)
+    got = to_host(espdl().slice_(to_dev(x), start, step, out_shape))
+    np.testing.assert_array_equal(got, want)
+
+
 def test_sppf_pool_chain_idempotence():
     """Size-independent property at full batch: three chained 5x5/1 pools equal one 13x13/1 pool, and
     pooling is monotone (output >= input)."""

@@ -119,3 +119,46 @@ def test_resize_nearest_values_exhaustive(oracle):
         got = oracle.resize_nearest_s8(x, 1, 1, in_exp=-5, out_exp=-5 - d).ravel()
         want = ((x.ravel().astype(np.int64) << d) & 0xff).astype(np.uint8).view(np.int8)
         np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("sl", [
+    (np.s_[:, :, -3:], [-3], [2 ** 63 - 1], [2], [1]), (np.s_[:, 1:4:2], [1], [4], [1], [2]),
+    (np.s_[0:1, :, 2:9:3, 1:], [0, 2, 1], [1, 9, 100], [0, 2, 3], [1, 3, 1]), (np.s_[:, :, :, ::4], [0], [64], [-1], [4]),
+])
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+def test_slice_is_numpy_slicing(oracle, sl, dtype):
+    idx, starts, ends, axes, steps = sl
+    x = _rand(np.random.default_rng(12), (2, 5, 10, 8), dtype)
+    np.testing.assert_array_equal(oracle.slice_(x, starts, ends, axes, steps), x[idx])
+
+
+@pytest.mark.parametrize("kernel,strides,pads,exps", [
+    ((1, 3), (1, 1), (0, 0, 2, 0), (-6, -7)), ((3, 3), (1, 1), (1, 1, 1, 1), (-5, -5)), ((2, 2), (2, 2), (0, 0, 0, 0), (-4, -5)),
+    ((7, 7), (1, 1), (0, 0, 0, 0), (-3, -4)), ((3, 2), (2, 1), (1, 0, 0, 1), (-5, -3)),
+])
+def test_avg_pool_matches_exact_mean_away_from_ties(oracle, kernel, strides, pads, exps):
+    """Clipped-window sum divided by the FULL window area, scaled by 2^(in_exp - out_exp), rounded half up:
+    the exact rational value decides every output that is not within float32 error of a tie."""
+    rng = np.random.default_rng(13)
+    x = _rand(rng, (2, 9, 11, 5))
+    got = oracle.avg_pool_s8(x, kernel, strides, pads, exps[0], exps[1]).astype(int)
+    pt, pb, pl, pr = pads
+    padded = np.zeros((2, 9 + pt + pb, 11 + pl + pr, 5), dtype=np.int64)
+    padded[:, pt:pt + 9, pl:pl + 11] = x
+    oh, ow = got.shape[1], got.shape[2]
+    area = kernel[0] * kernel[1]
+    checked = 0
+    for oy in range(oh):
+        for ox in range(ow):
+            win = padded[:, oy * strides[0]:oy * strides[0] + kernel[0], ox * strides[1]:ox * strides[1] + kernel[1]]
+            sums = win.sum(axis=(1, 2))
+            for n in range(2):
+                for k in range(5):
+                    exact = Fraction(int(sums[n, k]), area) * Fraction(2) ** (exps[0] - exps[1])
+                    frac = exact - (exact.numerator // exact.denominator)
+                    if abs(frac - Fraction(1, 2)) < Fraction(1, 10000):
+                        continue  # a (near-)tie: float32 may fall either way
+                    want = min(127, max(-128, (exact + Fraction(1, 2)).__floor__()))
+                    assert got[n, oy, ox, k] == want, (n, oy, ox, k)
+                    checked += 1
+    assert checked > 50
