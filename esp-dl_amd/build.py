@@ -85,8 +85,22 @@ def build_host_layer(verbose=True):
     return out
 
 
+def build_api_check(verbose=True):
+    """lib/espdl_api_check: a small C++ program written against the host layer's public headers
+    (tests/cpp/api_check.cpp); the GPU tests run it on the `.espdl` fixtures."""
+    src = os.path.join(os.path.dirname(HERE), "tests", "cpp", "api_check.cpp")
+    out = os.path.join(LIB_DIR, "espdl_api_check")
+    warn = _run([HIPCC, "-x", "hip", "--offload-arch=" + ARCH, "-O1", "-std=c++17", "-Wall",
+                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                 "-I" + os.path.join(DL_DIR, "include"), "-I" + INCLUDE_DIR, src, "-o", out,
+                 "-L" + LIB_DIR, "-lespdl_dl", "-lespdl_hip", "-Wl,-rpath,$ORIGIN"])
+    if warn.strip() and verbose:
+        print("[api_check.cpp]\n%s" % warn, file=sys.stderr)
+    return out
+
+
 def build_all(verbose=True):
-    return [build_kernels(verbose), build_host_layer(verbose)]
+    return [build_kernels(verbose), build_host_layer(verbose), build_api_check(verbose)]
 
 
 if __name__ == "__main__":

@@ -371,6 +371,27 @@ def test_relu_clip_requantize_s8(oracle):
                                       oracle.requantize_s8(x, in_exp, out_exp))
 
 
+@pytest.mark.parametrize("src,dst", [("s8", "s16"), ("s16", "s8"), ("s16", "s16")])
+def test_requantize_across_widths(oracle, src, dst):
+    """TensorBase::assign between int8 and int16 tensors: same exponent widens / saturates, different
+    exponents go through quantize(dequantize(x)) in float32 (oracle/graph_runner.requantize)."""
+    import torch
+    import graph_runner
+    announce(f"requantize {src} -> {dst}")
+    m = espdl()
+    rng = np.random.default_rng(6)
+    if src == "s8":
+        x = np.concatenate([np.arange(-128, 128).astype(np.int8), rng_int8(rng, (4099,))])
+    else:
+        x = np.concatenate([np.arange(-32768, 32768, 7), rng.integers(-32768, 32768, size=4099)]).astype(np.int16)
+    code = 5 if dst == "s16" else 3
+    tdt = torch.int16 if dst == "s16" else torch.int8
+    for in_exp, out_exp in ((-6, -6), (-6, -14), (-14, -6), (-7, -3), (-3, -9), (-12, -13)):
+        want = graph_runner.requantize(x, in_exp, out_exp, code)
+        got = to_host(m.requantize(to_dev(x), in_exp, out_exp, out_dtype=tdt))
+        np.testing.assert_array_equal(got, want, err_msg=f"{in_exp}->{out_exp}")
+
+
 ADD_SHAPES = [
     ((1, 96, 5, 48), (1, 96, 5, 48)), ((1, 96, 5, 48), (1, 96, 5, 1)), ((1, 96, 5, 1), (1, 96, 5, 48)),
     ((1, 5, 5, 31), (1, 1, 1, 31)), ((2, 3, 4, 5), (1, 1, 1, 1)), ((1, 1, 4, 5), (2, 3, 4, 5)),
