@@ -19,7 +19,8 @@ FIXTURES = sorted(glob.glob(os.path.join(HERE, "golden", "espdl", "*.espdl")))
 @pytest.mark.parametrize("path", [p for p in FIXTURES if "chain" in p or "conv1d" in p or "gemm_c_" in p],
                          ids=os.path.basename)
 def test_cpp_program_runs_fixture(path):
-    assert os.path.exists(BIN), "run `python esp-dl_amd/build.py` first"
+    if not os.path.exists(BIN):
+        pytest.skip("esp-dl_amd/lib/espdl_api_check is not built (python esp-dl_amd/build.py builds it)")
     announce("C++ api_check " + os.path.basename(path))
     round_mode = "1" if "p4" in os.path.basename(path) else "0"
     r = subprocess.run([BIN, path, round_mode], capture_output=True, text=True, timeout=120)
