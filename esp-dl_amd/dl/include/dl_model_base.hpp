@@ -34,10 +34,9 @@ public:
     /// The model does not take ownership of `fbs_model`.  `stream` is a hipStream_t (nullptr: the
     /// model creates its own).  `fuse` is a bit mask of graph fusions: FUSE_CONV_LUT folds a LUT that directly follows a Conv
     /// into its epilogue, FUSE_DW_PROJECT runs depthwise Conv -> 1x1 Conv [-> Add] as one kernel,
-    /// FUSE_CONV_ADD folds the Add behind a dense Conv into its epilogue (off by default: measured
-    /// slightly slower than the separate Add kernel on MobileNetV2, whose residual tensors are small).
+    /// FUSE_CONV_ADD folds the Add behind a dense Conv into its epilogue.  All are exact and on by default.
     Model(fbs::FbsModel *fbs_model, int batch = 1, round_mode_t round_mode = ROUND_MODE_HALF_UP, void *stream = nullptr,
-          int fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT);
+          int fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT | FUSE_CONV_ADD);
     virtual ~Model();
     Model(const Model &) = delete;
     Model &operator=(const Model &) = delete;
@@ -97,7 +96,7 @@ private:
     std::string m_name, m_doc_string;
     int64_t m_version = 0;
     int m_batch = 1;
-    int m_fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT;
+    int m_fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT | FUSE_CONV_ADD;
     void *m_stream = nullptr;
     bool m_own_stream = false;
     void *m_graph = nullptr;      // hipGraph_t

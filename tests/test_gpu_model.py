@@ -35,7 +35,7 @@ def _check_all(spec, mdl, want, skip_missing=True):
     return checked
 
 
-def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fuse_blocks=True, fuse_add=False):
+def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fuse_blocks=True, fuse_add=True):
     m, zoo, model, runner = _mods()
     import espdl_oracle as oracle
     rng = np.random.default_rng(seed)
@@ -165,7 +165,7 @@ def test_config4_yolo_style(oracle, fuse):
     announce(f"model config4 160px fuse={fuse}")
     _, zoo, _, _ = _mods()
     spec = zoo.config4_yolo_style(resolution=160)
-    mdl, want, _ = _run_config(spec, 2, 8, fuse_lut=fuse, fuse_blocks=fuse)
+    mdl, want, _ = _run_config(spec, 2, 8, fuse_lut=fuse, fuse_blocks=fuse, fuse_add=fuse)
     assert len(spec.outputs) == 6
     for name in spec.outputs:
         got = mdl.get_tensor(name, _np_dtype(spec, name))
@@ -258,7 +258,7 @@ def test_mobilenetv2_block_fusion(oracle, fuse_blocks):
     announce(f"model config3 96px fuse_blocks={fuse_blocks}")
     _, zoo, _, _ = _mods()
     spec = zoo.config3_mobilenetv2(resolution=96, num_classes=100)
-    mdl, want, _ = _run_config(spec, 3, 21, fuse_blocks=fuse_blocks)
+    mdl, want, _ = _run_config(spec, 3, 21, fuse_blocks=fuse_blocks, fuse_add=fuse_blocks)
     for name in spec.outputs:
         np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
     if fuse_blocks:
@@ -269,14 +269,15 @@ def test_mobilenetv2_block_fusion(oracle, fuse_blocks):
 
 
 def test_mobilenetv2_conv_add_fusion(oracle):
-    """Residual Adds folded into the project convolutions' epilogues (optional fusion): same logits."""
+    """Residual Adds folded into the project convolutions' epilogues, and not: same logits."""
     announce("model config3 96px fuse_add")
     _, zoo, _, _ = _mods()
     spec = zoo.config3_mobilenetv2(resolution=96, num_classes=100)
     mdl, want, _ = _run_config(spec, 3, 22, fuse_add=True)
-    plain, _, _ = _run_config(spec, 3, 22)
+    plain, _, _ = _run_config(spec, 3, 22, fuse_add=False)
     for name in spec.outputs:
         np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
+        np.testing.assert_array_equal(plain.get_tensor(name), want[name], err_msg=name)
     assert mdl.module_count() < plain.module_count()
     mdl.close()
     plain.close()
