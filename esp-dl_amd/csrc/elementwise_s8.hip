@@ -227,24 +227,45 @@ hipError_t launch_binary_s8(const int32_t dims[4], const int64_t s0[4], const in
 }
 
 // GlobalAveragePool: avgpool2d_hwc with the window covering the image
-// (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54).  One workgroup per (image, 64-channel slab): 64 lanes
-// along channels (contiguous), 4 wavefronts split the pixels, int32 partial sums meet in LDS.
+// (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54).  One workgroup per (image, slab of 64 x VEC channels):
+// lane l owns VEC consecutive channels (one VEC-byte load per pixel, adjacent lanes adjacent bytes, so a
+// wavefront reads whole contiguous runs of a pixel row), the 4 wavefronts split the pixels, int32
+// partial sums meet in LDS.  VEC = 16 when the channel count and pointers allow, else 1.
+template <int VEC>
 __global__ __launch_bounds__(kBlock) void global_avg_pool_s8_kernel(const int8_t *in, int8_t *out, int hw, int c,
                                                                     float scale)
 {
-    __shared__ int partial[4][64];
+    __shared__ int partial[4][64 * VEC];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int ch = blockIdx.x * 64 + lane;
+    const int ch = (blockIdx.x * 64 + lane) * VEC;
     const int8_t *img = in + (long long)blockIdx.y * hw * c;
-    int sum = 0;
-    if (ch < c)
-        for (int p = wave; p < hw; p += 4)
-            sum += img[(long long)p * c + ch];
-    partial[wave][lane] = sum;
+    int sum[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; k++)
+        sum[k] = 0;
+    if (ch < c) {
+        for (int p = wave; p < hw; p += 4) {
+            if (VEC == 16) {
+                const v4i v = *reinterpret_cast<const v4i *>(img + (long long)p * c + ch);
+#pragma unroll
+                for (int k = 0; k < VEC; k++)
+                    sum[k] += (int)(int8_t)(v[k >> 2] >> (8 * (k & 3)));
+            } else {
+                sum[0] += img[(long long)p * c + ch];
+            }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; k++)
+        partial[wave][lane * VEC + k] = sum[k];
     __syncthreads();
-    if (wave == 0 && ch < c) {
-        sum = partial[0][lane] + partial[1][lane] + partial[2][lane] + partial[3][lane];
-        out[(long long)blockIdx.y * c + ch] = (int8_t)clamp_s8(round_half_up_f32((float)sum * scale));
+    // 256 threads finish 64 * VEC channels
+    for (int e = threadIdx.x; e < 64 * VEC; e += kBlock) {
+        const int oc = blockIdx.x * 64 * VEC + e;
+        if (oc < c) {
+            const int total = partial[0][e] + partial[1][e] + partial[2][e] + partial[3][e];
+            out[(long long)blockIdx.y * c + oc] = (int8_t)clamp_s8(round_half_up_f32((float)total * scale));
+        }
     }
 }
 
@@ -345,8 +366,12 @@ hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, 
         return hipSuccess;
     const float area_inv = 1.f / (float)(h * w);
     const float scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
-    hipLaunchKernelGGL(global_avg_pool_s8_kernel, dim3((unsigned)((c + 63) / 64), (unsigned)batch), dim3(kBlock), 0,
-                       stream, in, out, h * w, c, scale);
+    if ((c & 15) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0)
+        hipLaunchKernelGGL(global_avg_pool_s8_kernel<16>, dim3((unsigned)((c + 1023) / 1024), (unsigned)batch), dim3(kBlock),
+                           0, stream, in, out, h * w, c, scale);
+    else
+        hipLaunchKernelGGL(global_avg_pool_s8_kernel<1>, dim3((unsigned)((c + 63) / 64), (unsigned)batch), dim3(kBlock), 0,
+                           stream, in, out, h * w, c, scale);
     return hipGetLastError();
 }
 
