@@ -77,7 +77,9 @@ def lib():
         L.espdl_hip_max_pool.argtypes = [vp, i32] + [i32] * 12 + [vp, vp]
         L.espdl_hip_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp, vp]
         L.espdl_hip_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp, vp]
-        for name in ("concat", "copy_rows", "transpose", "resize_nearest_s8", "max_pool", "avg_pool_s8", "slice"):
+        L.espdl_hip_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
+        for name in ("concat", "copy_rows", "transpose", "resize_nearest_s8", "max_pool", "avg_pool_s8", "slice",
+                     "reduce_mean_s8"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         mp = ctypes.POINTER(MbconvDesc)
         L.espdl_hip_mbconv_out_shape.argtypes = [mp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
@@ -363,3 +365,15 @@ def slice_(x, start, step, out_shape, out=None, stream=None):
     _check(lib().espdl_hip_slice(_p(x), arr(x.shape), nd, arr(start), arr(step), arr(out_shape), x.element_size(),
                                  _p(out), _stream(stream)))
     return out
+
+
+def reduce_mean_s8(x, axes, keepdims=True, in_exp=0, out_exp=0, stream=None):
+    import torch
+    nd = x.dim()
+    axes = [a + nd if a < 0 else a for a in (axes if len(axes) else range(nd))]
+    flags = [1 if i in axes else 0 for i in range(nd)]
+    kept = [int(x.shape[i]) for i in range(nd) if not flags[i]]
+    out = torch.empty(kept if kept else [1], dtype=torch.int8, device=x.device)
+    _check(lib().espdl_hip_reduce_mean_s8(_p(x), (ctypes.c_int32 * nd)(*x.shape), nd, (ctypes.c_int32 * nd)(*flags),
+                                          in_exp, out_exp, _p(out), _stream(stream)))
+    return out.reshape([1 if flags[i] else int(x.shape[i]) for i in range(nd)]) if keepdims else out

@@ -537,6 +537,37 @@ int espdl_hip_slice(const void *in, const int32_t *shape, int32_t dims, const in
                          "slice");
 }
 
+int espdl_hip_reduce_mean_s8(const int8_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
+                             int32_t in_exp, int32_t out_exp, int8_t *out, void *stream)
+{
+    if (dims < 1 || dims > 8 || shape == nullptr || reduce_flag == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "reduce_mean handles 1..8 dims");
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    int sh[8], fl[8];
+    long long total = 1, count = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative extent");
+        sh[i] = shape[i];
+        fl[i] = reduce_flag[i] != 0;
+        total *= shape[i];
+        if (fl[i])
+            count *= shape[i];
+        if (total > (1ll << 40))
+            return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    }
+    if (total == 0)
+        return ESPDL_HIP_OK;
+    if (count > (1 << 23))
+        return fail(ESPDL_HIP_ENOTSUP, "more than 2^23 elements per mean: the int32 sum could overflow");
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_reduce_mean_s8(in, sh, dims, fl, in_exp, out_exp, out, cu_count_cached(),
+                                                      reinterpret_cast<hipStream_t>(stream)),
+                         "reduce_mean_s8");
+}
+
 } // extern "C"
 
 namespace {

@@ -122,4 +122,7 @@ hipError_t launch_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, 
 hipError_t launch_slice(const void *in, const int *shape, int dims, const int *start, const int *step, const int *out_shape,
                         int elem_size, void *out, int cu_count, hipStream_t stream);
 
+hipError_t launch_reduce_mean_s8(const int8_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
+                                 int out_exp, int8_t *out, int cu_count, hipStream_t stream);
+
 } // namespace espdl

@@ -326,6 +326,42 @@ __global__ __launch_bounds__(kBlock) void avg_pool_s8_kernel(const AvgPoolArgs a
     }
 }
 
+// ReduceMean (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:16-45): one thread per output element
+// walks the reduced axes; the float expression is the reference's, left to right.
+struct ReduceArgs {
+    const int8_t *in;
+    int8_t *out;
+    int n_kept, n_red;
+    int kept_shape[kMaxDims], red_shape[kMaxDims];
+    long long kept_stride[kMaxDims], red_stride[kMaxDims];
+    long long n_out, count;
+    float input_scale, output_scale;
+};
+
+__global__ __launch_bounds__(kBlock) void reduce_mean_s8_kernel(const ReduceArgs a)
+{
+    for (long long o = (long long)blockIdx.x * kBlock + threadIdx.x; o < a.n_out; o += (long long)gridDim.x * kBlock) {
+        long long rem = o, base = 0;
+        for (int d = a.n_kept - 1; d >= 0; d--) {
+            const long long q = rem / a.kept_shape[d];
+            base += (rem - q * a.kept_shape[d]) * a.kept_stride[d];
+            rem = q;
+        }
+        int sum = 0;
+        for (long long r = 0; r < a.count; r++) {
+            long long rr = r, off = base;
+            for (int d = a.n_red - 1; d >= 0; d--) {
+                const long long q = rr / a.red_shape[d];
+                off += (rr - q * a.red_shape[d]) * a.red_stride[d];
+                rr = q;
+            }
+            sum += a.in[off];
+        }
+        const float v = (float)sum * a.input_scale / (float)a.count * a.output_scale;
+        a.out[o] = (int8_t)clamp_s8(round_half_up_f32(v));
+    }
+}
+
 } // namespace
 
 hipError_t launch_copy_rows(const void *src, long long src_pitch, void *dst, long long dst_pitch, long long row_bytes,
@@ -617,6 +653,37 @@ hipError_t launch_slice(const void *in, const int *shape, int dims, const int *s
         hipLaunchKernelGGL(transpose_general_kernel<int16_t>, grid, dim3(kBlock), 0, stream, a);
     else
         hipLaunchKernelGGL(transpose_general_kernel<int32_t>, grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_reduce_mean_s8(const int8_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
+                                 int out_exp, int8_t *out, int cu_count, hipStream_t stream)
+{
+    ReduceArgs a = {};
+    long long stride[kMaxDims];
+    stride[dims - 1] = 1;
+    for (int i = dims - 2; i >= 0; i--)
+        stride[i] = stride[i + 1] * shape[i + 1];
+    a.n_out = 1;
+    a.count = 1;
+    for (int i = 0; i < dims; i++) {
+        if (reduce_flag[i]) {
+            a.red_shape[a.n_red] = shape[i];
+            a.red_stride[a.n_red++] = stride[i];
+            a.count *= shape[i];
+        } else {
+            a.kept_shape[a.n_kept] = shape[i];
+            a.kept_stride[a.n_kept++] = stride[i];
+            a.n_out *= shape[i];
+        }
+    }
+    if (a.n_out <= 0 || a.count <= 0)
+        return hipSuccess;
+    a.in = in;
+    a.out = out;
+    a.input_scale = dl_scale(in_exp);
+    a.output_scale = dl_rescale(out_exp);
+    hipLaunchKernelGGL(reduce_mean_s8_kernel, dim3(blocks_for(a.n_out, cu_count)), dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 

@@ -52,6 +52,8 @@ private:
     int m_lut_in_exponent = 0;   ///< exponent of the conv result that indexes a fused LUT
     int m_project_filter_pos = -1, m_project_bias_pos = -1, m_residual_pos = -1;
     int m_own_inputs = 0; ///< inputs of the Conv itself when a plain residual Add was absorbed
+    bool m_has_pre_add_exponent = false;
+    int m_pre_add_exponent = 0; ///< exponent of the tensor an absorbed Add used to read from this module
     DeviceInts m_shift_project;
 
 public:
@@ -88,8 +90,13 @@ public:
     const std::vector<int> &get_dilations() const { return m_dilations; }
     /// Absorb a following 1x1 Conv (filter / bias indices, activation) and optionally the other
     /// operand of the Add after it.  The caller re-points m_outputs_index at the final tensor.
-    void fuse_project(int filter_index, int bias_index, activation_type_t act, int mid_exponent, int residual_index)
+    void fuse_project(int filter_index, int bias_index, activation_type_t act, int mid_exponent, int residual_index,
+                      int project_out_exponent = 0)
     {
+        if (residual_index >= 0) {
+            m_has_pre_add_exponent = true;
+            m_pre_add_exponent = project_out_exponent;
+        }
         m_has_project = true;
         m_project_activation = act;
         m_mid_exponent = mid_exponent;
@@ -104,9 +111,14 @@ public:
             m_inputs_index.push_back(residual_index);
         }
     }
-    /// Absorb the Add that follows a dense Conv: `residual_index` is the Add's other operand.
-    void fuse_residual(int residual_index)
+    /// Absorb the Add that follows a dense Conv: `residual_index` is the Add's other operand and
+    /// `own_out_exponent` the exponent of the tensor the Conv used to write.  The Add sums stored integers
+    /// whatever the exponents of its operands and result are (esp-dl/dl/base/dl_base_add.cpp:35-44), so the
+    /// Conv keeps requantizing to its own exponent, not to the one of the tensor it now writes.
+    void fuse_residual(int residual_index, int own_out_exponent)
     {
+        m_has_pre_add_exponent = true;
+        m_pre_add_exponent = own_out_exponent;
         m_own_inputs = (int)m_inputs_index.size();
         m_residual_pos = (int)m_inputs_index.size();
         m_inputs_index.push_back(residual_index);
@@ -220,7 +232,9 @@ public:
         }
         d.round_mode = context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP;
         const std::vector<int32_t> shifts =
-            conv_shifts(m_fused_lut ? m_lut_in_exponent : output->exponent.get(), input, filter, d.out_c);
+            conv_shifts(m_fused_lut ? m_lut_in_exponent
+                                    : (m_has_pre_add_exponent ? m_pre_add_exponent : output->exponent.get()),
+                        input, filter, d.out_c);
         d.n_shift = (int32_t)shifts.size();
         const int32_t *shift_dev = m_shift.sync(shifts);
         if (m_fused_lut && !m_fused_lut->on_device()) {
@@ -282,11 +296,12 @@ public:
         } else {
             s_dw.push_back(m_mid_exponent - filter->exponent.get() - input->exponent.get());
         }
+        const int pj_out_exponent = m_has_pre_add_exponent ? m_pre_add_exponent : output->exponent.get();
         if (pfilter->exponent.is_per_channel()) {
             for (int c = 0; c < d.out_c; c++)
-                s_pj.push_back(output->exponent.get() - pfilter->exponent.get(c) - m_mid_exponent);
+                s_pj.push_back(pj_out_exponent - pfilter->exponent.get(c) - m_mid_exponent);
         } else {
-            s_pj.push_back(output->exponent.get() - pfilter->exponent.get() - m_mid_exponent);
+            s_pj.push_back(pj_out_exponent - pfilter->exponent.get() - m_mid_exponent);
         }
         d.n_shift_expand = 1;
         d.n_shift_dw = (int32_t)s_dw.size();

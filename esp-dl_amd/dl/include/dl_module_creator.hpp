@@ -71,6 +71,7 @@ public:
         register_module("MaxPool", MaxPool::deserialize);
         register_module("AveragePool", AveragePool::deserialize);
         register_module("Slice", Slice::deserialize);
+        register_module("ReduceMean", ReduceMean::deserialize);
         // element-wise activations that esp-ppq exports with a precomputed 8-bit table
         for (const char *op : {"Swish", "HardSwish", "Sigmoid", "HardSigmoid", "Tanh", "Gelu", "Elu", "LeakyRelu",
                                "Exp", "Log", "Sqrt", "Softplus", "Mish"}) {

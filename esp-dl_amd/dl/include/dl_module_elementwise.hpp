@@ -499,6 +499,7 @@ public:
 private:
     Kind m_kind;
     std::vector<int> m_arg; ///< axes (Squeeze / Unsqueeze) or the per-image target shape with leading 1 (Reshape)
+    bool m_allowzero = false;
 
 public:
     ShapeView(const char *name, Kind kind, std::vector<int> arg, quant_type_t quant_type = QUANT_TYPE_NONE) :
@@ -536,6 +537,11 @@ public:
             for (int d : in)
                 total *= d;
             out = m_arg;
+            // a 0 copies the input extent unless allowzero is set
+            // (esp-dl/dl/module/include/dl_module_reshape.hpp:46-61)
+            for (size_t i = 0; i < out.size(); i++)
+                if (out[i] == 0 && !m_allowzero && i < in.size())
+                    out[i] = in[i];
             if (!out.empty())
                 out[0] = in[0]; // the batch dimension is kept
             int infer = -1;
@@ -579,6 +585,31 @@ private:
         std::vector<int> arg;
         fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
         fbs_model->get_operation_attribute(node_name, key, arg);
+        if (arg.empty()) {
+            // exported graphs carry the axes / target shape as the second operand, an integer initializer
+            // (esp-dl/dl/module/include/dl_module_reshape.hpp:107-118)
+            TensorBase *t = fbs_model->get_operation_parameter(node_name, 1);
+            if (t && t->dtype == DATA_TYPE_INT64) {
+                const int64_t *p = t->get_element_ptr<int64_t>();
+                for (int i = 0; i < t->get_size(); i++)
+                    arg.push_back((int)p[i]);
+            } else if (t && t->dtype == DATA_TYPE_INT32) {
+                const int32_t *p = t->get_element_ptr<int32_t>();
+                arg.assign(p, p + t->get_size());
+            }
+            delete t;
+        }
+        if (kind == RESHAPE) {
+            int allowzero = 0;
+            fbs_model->get_operation_attribute(node_name, "allowzero", allowzero);
+            if (arg.empty()) {
+                DL_LOGE("Reshape", "%s: no target shape (attribute or integer initializer)", node_name.c_str());
+                return nullptr;
+            }
+            ShapeView *op = new ShapeView(node_name.c_str(), kind, arg, quant_type);
+            op->m_allowzero = allowzero != 0;
+            return op;
+        }
         return new ShapeView(node_name.c_str(), kind, arg, quant_type);
     }
 };

@@ -60,8 +60,9 @@ public:
     std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
     {
         std::vector<int> filter_shape = input_shapes[1];
-        assert(filter_shape.size() == 4 && filter_shape[0] == 1 && filter_shape[1] == 1);
-        assert(input_shapes[0].back() == filter_shape[2]);
+        if (input_shapes[0].empty() || filter_shape.size() != 4 || filter_shape[0] != 1 || filter_shape[1] != 1 ||
+            input_shapes[0].back() != filter_shape[2])
+            return {{}}; // an empty shape makes Model::build fail with the node's name
         std::vector<int> output_shape = input_shapes[0];
         output_shape.back() = filter_shape[3];
         return {output_shape};

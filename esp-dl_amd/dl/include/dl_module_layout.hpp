@@ -1,5 +1,5 @@
 // Data-movement and pooling operator objects: Concat, Split, Transpose, Resize, MaxPool, AveragePool,
-// Slice.  Each mirrors the
+// Slice, ReduceMean.  Each mirrors the
 // reference module of the same name (same attributes, shape rules and error behaviour) and enqueues
 // kernels of include/espdl_hip.h on the context's stream.
 //   Concat     esp-dl/dl/module/include/dl_module_concat.hpp:14-127
@@ -9,6 +9,7 @@
 //   MaxPool    esp-dl/dl/module/include/dl_module_max_pool.hpp:13-131
 //   AveragePool esp-dl/dl/module/include/dl_module_average_pool.hpp
 //   Slice      esp-dl/dl/module/include/dl_module_slice.hpp
+//   ReduceMean esp-dl/dl/module/include/dl_module_reduce_mean.hpp, dl_module_reduce_base.hpp
 #pragma once
 
 #include <algorithm>
@@ -554,6 +555,98 @@ public:
         return new Slice(node_name.c_str(), v[0], v[1], v[2], v[3], quant_type);
     }
     void print() { DL_LOGI("Slice", "axes: %d, quant_type: %s.", (int)m_start.size(), quant_type_to_string(quant_type)); }
+};
+
+/// ReduceMean on int8 tensors (esp-dl/dl/module/include/dl_module_reduce_mean.hpp, axes handling of
+/// dl_module_reduce_base.hpp:262-298: `axes` is the second input; empty axes reduce everything unless
+/// `noop_with_empty_axes` is set).
+class ReduceMean : public Module {
+private:
+    int m_keepdims;
+    std::vector<int64_t> m_axes;
+    int m_noop_with_empty_axes;
+
+    std::vector<int32_t> flags_for(size_t rank) const
+    {
+        std::vector<int32_t> f(rank, 0);
+        if (m_axes.empty()) {
+            if (!m_noop_with_empty_axes)
+                f.assign(rank, 1);
+            return f;
+        }
+        for (int64_t a : m_axes) {
+            const int64_t ax = a < 0 ? a + (int64_t)rank : a;
+            if (ax >= 0 && ax < (int64_t)rank)
+                f[(size_t)ax] = 1;
+        }
+        return f;
+    }
+
+public:
+    ReduceMean(const char *name = nullptr, int keepdims = 1, const std::vector<int64_t> &axes = {},
+               int noop_with_empty_axes = 0, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_keepdims(keepdims), m_axes(axes),
+        m_noop_with_empty_axes(noop_with_empty_axes)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        const std::vector<int32_t> f = flags_for(in.size());
+        std::vector<int> out;
+        for (size_t i = 0; i < in.size(); i++) {
+            if (!f[i])
+                out.push_back(in[i]);
+            else if (m_keepdims)
+                out.push_back(1);
+        }
+        if (out.empty())
+            out.push_back(1);
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) || quant_type != QUANT_TYPE_SYMM_8BIT || input->shape.size() > 8) {
+            DL_LOGE("ReduceMean", "%s: needs int8 device tensors of at most 8 dims", name.c_str());
+            return;
+        }
+        const std::vector<int32_t> f = flags_for(input->shape.size());
+        const int rc = espdl_hip_reduce_mean_s8(static_cast<const int8_t *>(input->data), input->shape.data(),
+                                                (int32_t)input->shape.size(), f.data(), input->exponent.get(),
+                                                output->exponent.get(), static_cast<int8_t *>(output->data),
+                                                context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("ReduceMean", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        int keepdims = 1, noop = 0;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "keepdims", keepdims);
+        fbs_model->get_operation_attribute(node_name, "noop_with_empty_axes", noop);
+        std::vector<int64_t> axes;
+        TensorBase *t = fbs_model->get_operation_parameter(node_name, 1);
+        if (t) {
+            if (t->dtype == DATA_TYPE_INT64) {
+                const int64_t *p = t->get_element_ptr<int64_t>();
+                axes.assign(p, p + t->get_size());
+            } else if (t->dtype == DATA_TYPE_INT32) {
+                const int32_t *p = t->get_element_ptr<int32_t>();
+                axes.assign(p, p + t->get_size());
+            }
+            delete t;
+        } else {
+            std::vector<int> attr_axes; // older exports carry the axes as an attribute
+            if (fbs_model->get_operation_attribute(node_name, "axes", attr_axes) == ESP_OK)
+                axes.assign(attr_axes.begin(), attr_axes.end());
+        }
+        return new ReduceMean(node_name.c_str(), keepdims, axes, noop, quant_type);
+    }
+    void print() { DL_LOGI("ReduceMean", "keepdims: %d, quant_type: %s.", m_keepdims, quant_type_to_string(quant_type)); }
 };
 
 } // namespace module

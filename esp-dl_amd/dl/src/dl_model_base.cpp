@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <cstring>
 #include <set>
+#include <typeinfo>
 
 #include "dl_module_creator.hpp"
 
@@ -188,6 +189,13 @@ esp_err_t Model::load(fbs::FbsModel *fbs_model)
     return ret;
 }
 
+// The module as an Add, or nullptr: classes derived from Add (Mul) share its operand handling but
+// not its arithmetic, so they must never be absorbed as a residual addition.
+static dl::module::Add *plain_add(dl::module::Module *m)
+{
+    return m && typeid(*m) == typeid(dl::module::Add) ? static_cast<dl::module::Add *>(m) : nullptr;
+}
+
 // Conv -> LUT with no other reader of the conv output: the table moves into the conv's epilogue and
 // the conv writes the LUT's output tensor directly.
 void Model::fuse_conv_lut()
@@ -305,7 +313,7 @@ void Model::fuse_dw_project()
         size_t last_pos = pj_pos, add_pos = 0;
         dl::module::Add *add = nullptr;
         if (single_reader(out_index, &add_pos) && add_pos > pj_pos) {
-            add = dynamic_cast<dl::module::Add *>(m_execution_plan[add_pos]);
+            add = plain_add(m_execution_plan[add_pos]);
             if (add && add->quant_type == QUANT_TYPE_SYMM_8BIT && add->m_inputs_index.size() == 2 &&
                 add->m_inputs_index[0] != add->m_inputs_index[1]) {
                 const int other = add->m_inputs_index[0] == out_index ? add->m_inputs_index[1] : add->m_inputs_index[0];
@@ -324,8 +332,9 @@ void Model::fuse_dw_project()
             }
         }
         const int mid_exp = m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(mid));
+        const int pj_out_exp = m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(pj->m_outputs_index[0]));
         dw->fuse_project(pj->m_inputs_index[1], pj->m_inputs_index.size() == 3 ? pj->m_inputs_index[2] : -1,
-                         pj->get_activation(), mid_exp, residual);
+                         pj->get_activation(), mid_exp, residual, pj_out_exp);
         dw->m_outputs_index[0] = out_index;
         // the fused module moves to the slot of the last absorbed module
         m_execution_plan[last_pos] = dw;
@@ -371,7 +380,7 @@ void Model::fuse_conv_add()
                 }
         if (readers != 1 || add_pos <= i)
             continue;
-        auto *add = dynamic_cast<dl::module::Add *>(m_execution_plan[add_pos]);
+        auto *add = plain_add(m_execution_plan[add_pos]);
         if (!add || add->quant_type != QUANT_TYPE_SYMM_8BIT || add->m_inputs_index.size() != 2 ||
             add->m_inputs_index[0] == add->m_inputs_index[1])
             continue;
@@ -381,7 +390,7 @@ void Model::fuse_conv_add()
         if (other >= CONTEXT_PARAMETER_OFFSET || !m_fbs_model->has_value_info(other_name) ||
             m_fbs_model->get_value_info_shape(other_name) != m_fbs_model->get_value_info_shape(mid_name))
             continue;
-        conv->fuse_residual(other);
+        conv->fuse_residual(other, m_fbs_model->get_value_info_exponent(mid_name));
         conv->m_outputs_index[0] = add->m_outputs_index[0];
         delete add;
         m_execution_plan[add_pos] = conv;
@@ -452,6 +461,16 @@ esp_err_t Model::build(int batch)
             }
         }
         std::vector<std::vector<int>> out_shapes = m->get_output_shape(in_shapes);
+        bool shapes_ok = out_shapes.size() >= m->m_outputs_index.size();
+        for (size_t j = 0; shapes_ok && j < m->m_outputs_index.size(); j++) {
+            shapes_ok = !out_shapes[j].empty();
+            for (int d : out_shapes[j])
+                shapes_ok = shapes_ok && d > 0;
+        }
+        if (!shapes_ok) {
+            DL_LOGE(TAG, "module %s cannot derive its output shape from its inputs", m->name.c_str());
+            return ESP_FAIL;
+        }
         for (size_t j = 0; j < m->m_outputs_index.size(); j++) {
             const int idx = m->m_outputs_index[j];
             const std::string name = ctx->get_tensor_name(idx);

@@ -226,16 +226,17 @@ class Builder:
         g.add_node(name, "RequantizeLinear", [x], [y], quant_type="S8")
         return y
 
-    def add(self, a, b, name=None):
+    def add(self, a, b, name=None, out_exp=None):
         """Residual add at matched exponents: the operand with the other exponent is requantized first,
-        which is what the exporter does by inserting RequantizeLinear."""
+        which is what the exporter does by inserting RequantizeLinear.  `out_exp` labels the result with
+        another exponent, as some exported graphs do; the operator still sums the stored integers."""
         g = self.g
         name = name or self._name("add")
         ea, eb = g.exponent(a), g.exponent(b)
         if ea != eb:
             a = self.requantize(a, eb)
         y = name + "_out"
-        g.add_value(y, g.shape(b), eb)
+        g.add_value(y, g.shape(b), eb if out_exp is None else out_exp)
         g.add_node(name, "Add", [a, b], [y], quant_type="S8")
         return y
 
@@ -270,6 +271,47 @@ class Builder:
         y = name + "_out"
         g.add_value(y, [1, int(np.prod(dims[1:]))], g.exponent(x))
         g.add_node(name, "Flatten", [x], [y], axis=1, quant_type="S8")
+        return y
+
+    def reduce_mean(self, x, axes, keepdims=True, out_exp=None, name=None):
+        """ReduceMean with the axes as an INT64 initializer operand, as exported graphs carry them."""
+        g = self.g
+        name = name or self._name("mean")
+        dims = g.shape(x)
+        norm = [a % len(dims) for a in axes]
+        count = int(np.prod([dims[a] for a in norm]))
+        out = [1 if i in norm else d for i, d in enumerate(dims)] if keepdims else \
+            [d for i, d in enumerate(dims) if i not in norm]
+        e = g.exponent(x) - max(0, int(round(math.log2(math.sqrt(count))))) + 1 if out_exp is None else out_exp
+        g.add_init(name + ".axes", [len(axes)], INT64, list(axes), [0])
+        y = name + "_out"
+        g.add_value(y, out, e)
+        g.add_node(name, "ReduceMean", [x, name + ".axes"], [y], keepdims=1 if keepdims else 0, noop_with_empty_axes=0,
+                   quant_type="S8")
+        return y
+
+    def avg_pool(self, x, k, stride=1, pad=0, out_exp=None, name=None):
+        g = self.g
+        name = name or self._name("avgpool")
+        _, h, w, c = g.shape(x)
+        oh, ow = (h + 2 * pad - k) // stride + 1, (w + 2 * pad - k) // stride + 1
+        y = name + "_out"
+        g.add_value(y, [1, oh, ow, c], g.exponent(x) if out_exp is None else out_exp)
+        g.add_node(name, "AveragePool", [x], [y], kernel_shape=[k, k], strides=[stride, stride],
+                   pads=[pad, pad, pad, pad], quant_type="S8")
+        return y
+
+    def reshape(self, x, shape, name=None):
+        """Reshape with the per-image target shape (leading 1, one -1 allowed) as an INT64 initializer operand."""
+        g = self.g
+        name = name or self._name("reshape")
+        total = int(np.prod(g.shape(x)))
+        known = int(np.prod([d for d in shape if d != -1]))
+        out = [total // known if d == -1 else d for d in shape]
+        g.add_init(name + ".shape", [len(shape)], INT64, list(shape), [0])
+        y = name + "_out"
+        g.add_value(y, out, g.exponent(x), g.dtype(x))
+        g.add_node(name, "Reshape", [x, name + ".shape"], [y], allowzero=0, quant_type="S8")
         return y
 
     def max_pool(self, x, k, stride=1, pad=None, name=None):
@@ -561,5 +603,31 @@ def gated_block(seed=0xE5D6):
     h = b.mul(h, sq, name="se_scale")                    # [1,20,20,64] * [1,1,1,64]
     y = b.conv(h, 32, k=1, name="c2")
     y = b.add(x, y, name="res")
+    b.output(y)
+    # detection-style score head: two single-channel Conv -> Sigmoid branches multiplied together (each
+    # Conv's only reader is its LUT, and each LUT's only reader is the Mul)
+    sig = lambda v: 1.0 / (1.0 + np.exp(-v))
+    p = b.lut(b.conv(h, 1, k=1, name="score_cls"), sig, "Sigmoid", out_exp=-7, name="score_cls_sig")
+    q = b.lut(b.conv(h, 1, k=5, name="score_obj"), sig, "Sigmoid", out_exp=-7, name="score_obj_sig")
+    b.output(b.mul(p, q, name="score"))
+    return g
+
+
+def pooled_embedding(seed=0xE5D7):
+    """Conv -> AveragePool -> Conv -> ReduceMean over H x W (axes as an initializer operand) -> Transpose to
+    N,C,1,1 -> Reshape [1,-1] (shape as an initializer operand) -> Gemm: the tail of the reference's exported
+    re-identification / embedding models."""
+    g = GraphSpec("pooled_embedding")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 24, 12, 16], -5)
+    h = b.conv(x, 32, k=3, relu=True, name="c1")
+    h = b.avg_pool(h, 2, stride=2, name="pool")
+    h = b.conv(h, 128, k=1, relu=True, name="c2")
+    r = b.conv(h, 128, k=1, out_exp=g.exponent(h), name="c3")
+    h = b.add(h, r, out_exp=g.exponent(h) - 1, name="res")   # the Add's result carries its own exponent
+    h = b.reduce_mean(h, [1, 2], keepdims=True, name="mean")
+    h = b.transpose(h, [0, 3, 1, 2], name="to_nchw")
+    h = b.reshape(h, [1, -1], name="view")
+    y = b.gemm(h, 64, relu=True, name="fc")
     b.output(y)
     return g

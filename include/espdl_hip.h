@@ -199,6 +199,13 @@ int espdl_hip_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w,
                           int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom, int32_t pad_left,
                           int32_t pad_right, int32_t in_exp, int32_t out_exp, int8_t *out, void *stream);
 
+/* module::ReduceMean for int8 (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:16-45): mean over the
+ * axes whose reduce_flag is non-zero, out = clamp(round(sum * 2^in_exp / count * 2^-out_exp)) in float32.
+ * `out` holds the kept axes in order (keepdims changes only the shape).  shape and reduce_flag are host
+ * arrays of `dims` entries, 1..8 dims. */
+int espdl_hip_reduce_mean_s8(const int8_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
+                             int32_t in_exp, int32_t out_exp, int8_t *out, void *stream);
+
 /* TensorBase::slice for positive steps (esp-dl/dl/base/dl_base_shape.cpp:68-120 gives the shape rule):
  * out[i0, i1, ...] = in[start[0] + i0 * step[0], start[1] + i1 * step[1], ...].  The caller passes
  * normalized values per dim (0 <= start, step >= 1, out_shape) for all `dims` dims of the input;

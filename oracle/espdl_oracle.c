@@ -526,6 +526,55 @@ void espdl_oracle_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, 
 }
 
 /*
+ * ReduceMean, int8 (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:16-45 over the loops of
+ * dl_module_reduce_base.hpp:121-260): int32 sum over the flagged axes, then
+ * truncate(round(sum * DL_SCALE(in_exp) / count * DL_RESCALE(out_exp))) in float32, left to right,
+ * count = number of summed elements.  `out` holds the kept axes in order (keepdims only changes the
+ * shape, not the bytes).  Up to 8 dims.
+ */
+int espdl_oracle_reduce_mean_s8(const int8_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
+                                int out_exp, int8_t *out)
+{
+    if (dims < 1 || dims > 8)
+        return -1;
+    int64_t stride[8], total = 1, count = 1;
+    stride[dims - 1] = 1;
+    for (int i = dims - 2; i >= 0; i--)
+        stride[i] = stride[i + 1] * shape[i + 1];
+    for (int i = 0; i < dims; i++) {
+        total *= shape[i];
+        if (reduce_flag[i])
+            count *= shape[i];
+    }
+    if (total == 0)
+        return 0;
+    const int64_t n_out = total / count;
+    int32_t *sums = (int32_t *)calloc((size_t)n_out, sizeof(int32_t));
+    if (!sums)
+        return -1;
+    int64_t idx[8] = {0};
+    for (int64_t e = 0; e < total; e++) {
+        int64_t o = 0;
+        for (int i = 0; i < dims; i++)
+            if (!reduce_flag[i])
+                o = o * shape[i] + idx[i];
+        sums[o] += in[e];
+        for (int i = dims - 1; i >= 0; i--) {
+            if (++idx[i] < shape[i])
+                break;
+            idx[i] = 0;
+        }
+    }
+    const float input_scale = dl_scale(in_exp), output_scale = dl_rescale(out_exp);
+    for (int64_t o = 0; o < n_out; o++)
+        out[o] = (int8_t)clamp_i64(round_half_up_f32((float)sums[o] * input_scale / (float)count * output_scale),
+                                   INT8_MIN, INT8_MAX);
+    free(sums);
+    (void)stride;
+    return 0;
+}
+
+/*
  * Slice with ONNX semantics (what base::get_slice_shape, esp-dl/dl/base/dl_base_shape.cpp:68-120, and
  * TensorBase::slice compute for positive steps): per listed axis take indices start, start + step, ...
  * below end.  starts / ends / steps here are already normalized to 0 <= start < dim, step >= 1 and the

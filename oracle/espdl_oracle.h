@@ -46,6 +46,8 @@
  *   espdl_oracle_avg_pool_s8     float32 scale as espdl_oracle_global_avg_pool_s8: exact rational round-half-up away
  *                                from ties; the reference's streaming-model fixtures (S3 and P4 exports with
  *                                embedded outputs) pass through it                  PARITY UNPINNED (near-ties)
+ *   espdl_oracle_reduce_mean_s8  float32 as the two above: exact rational mean, round half up, away from ties
+ *                                                                                   PARITY UNPINNED (near-ties)
  *   espdl_oracle_slice           equality with numpy basic slicing                                   PINNED
  *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
  *                                numpy.split / numpy.transpose on random shapes           PINNED
@@ -115,6 +117,8 @@ void espdl_oracle_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, 
 void espdl_oracle_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                               int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,
                               int out_exp, int8_t *out);
+int espdl_oracle_reduce_mean_s8(const int8_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
+                                int out_exp, int8_t *out);
 int espdl_oracle_slice(const void *in, const int *shape, int dims, const int *start, const int *step,
                        const int *out_shape, int elem_size, void *out);
 void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out);

@@ -60,6 +60,8 @@ def lib():
         L.espdl_oracle_requantize_s8.argtypes = [vp, i64, i32, i32, vp]
         L.espdl_oracle_mul_s8.argtypes = [vp, i64, vp, i64, i64, i32, i32, vp]
         L.espdl_oracle_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp]
+        L.espdl_oracle_reduce_mean_s8.restype = i32
+        L.espdl_oracle_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp]
         L.espdl_oracle_slice.restype = i32
         L.espdl_oracle_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp]
         L.espdl_oracle_concat.argtypes = [vp, i32, vp, i64, i32, vp]
@@ -352,4 +354,19 @@ def slice_(x, starts, ends, axes=None, steps=None):
     sh, st, sp, os_ = i32(x.shape), i32(start), i32(step), i32(out_shape)
     rc = lib().espdl_oracle_slice(_ptr(x), _ptr(sh), x.ndim, _ptr(st), _ptr(sp), _ptr(os_), x.dtype.itemsize, _ptr(out))
     assert rc == 0
+    return out
+
+
+def reduce_mean_s8(x, axes, keepdims=True, in_exp=0, out_exp=0):
+    x = _c(x, np.int8)
+    nd = x.ndim
+    axes = [a + nd if a < 0 else a for a in (axes if len(axes) else range(nd))]
+    flags = np.array([1 if i in axes else 0 for i in range(nd)], dtype=np.int32)
+    kept = [x.shape[i] for i in range(nd) if not flags[i]]
+    out = np.empty(kept if kept else [1], dtype=np.int8)
+    shape = np.array(x.shape, dtype=np.int32)
+    rc = lib().espdl_oracle_reduce_mean_s8(_ptr(x), _ptr(shape), nd, _ptr(flags), in_exp, out_exp, _ptr(out))
+    assert rc == 0
+    if keepdims:
+        out = out.reshape([1 if flags[i] else x.shape[i] for i in range(nd)])
     return out

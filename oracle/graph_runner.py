@@ -20,6 +20,17 @@ def _shift(spec, node, x_name, w_name, y_name):
 def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
     """inputs: {name: ndarray for the whole batch}.  Returns {tensor name: ndarray}."""
     t = dict(inputs)
+
+    def operand(name):
+        """An activation, or a constant operand (initializer) as stored."""
+        if name in t:
+            return t[name]
+        dims, _, data, _ = spec.initializers[name]
+        return np.asarray(data).reshape(dims)
+
+    def exponent_of(name):
+        return spec.exponent(name) if name in spec.value_info else int(spec.initializers[name][3][0])
+
     for node in spec.nodes:
         op, a = node["op_type"], node["attrs"]
         ins, outs = node["inputs"], node["outputs"]
@@ -61,12 +72,15 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             hi = int(spec.initializers[ins[2]][2].ravel()[0]) if len(ins) > 2 else 127
             y = oracle.clip_s8(x, lo, hi, spec.exponent(ins[0]), spec.exponent(y_name))
         elif op == "Add":
-            b = t[ins[1]]
-            assert x.shape == b.shape, "the graph runner only needs same-shape residual adds"
-            y = oracle.add_s8(x, b)
+            # the C path adds the stored integers and saturates, whatever the exponents say
+            # (esp-dl/dl/base/dl_base_add.cpp:35-44); the exporter gives all three the same exponent
+            b = operand(ins[1])
+            if x.shape != b.shape:
+                x, b = np.broadcast_arrays(x, b)
+            y = oracle.add_s8(np.ascontiguousarray(x), np.ascontiguousarray(b))
         elif op == "Mul":
-            b = t[ins[1]]
-            shift = spec.exponent(y_name) - spec.exponent(ins[0]) - spec.exponent(ins[1])
+            b = operand(ins[1])
+            shift = spec.exponent(y_name) - exponent_of(ins[0]) - exponent_of(ins[1])
             if x.shape != b.shape:  # broadcast explicitly: the oracle takes equal sizes or a scalar
                 x, b = np.broadcast_arrays(x, b)
             y = oracle.mul_s8(np.ascontiguousarray(x), np.ascontiguousarray(b), shift, round_mode)
@@ -76,8 +90,18 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             y = requantize(x, spec.exponent(ins[0]), spec.exponent(y_name), spec.dtype(y_name))
         elif op == "Flatten":
             y = x.reshape(x.shape[0], -1)
-        elif op == "Squeeze":
-            y = np.squeeze(x, axis=tuple(a["axes"]))
+        elif op in ("Squeeze", "Unsqueeze"):
+            axes = a["axes"] if "axes" in a else [int(v) for v in spec.initializers[ins[1]][2].ravel()]
+            y = np.squeeze(x, axis=tuple(axes)) if op == "Squeeze" else np.expand_dims(x, tuple(axes))
+        elif op == "Reshape":
+            # exported target shapes are per image (leading 1); a batch keeps its own leading extent
+            shape = [int(v) for v in spec.initializers[ins[1]][2].ravel()]
+            per_image = x.size // x.shape[0]
+            rest = [d if d != 0 else x.shape[i] for i, d in enumerate(shape)][1:]
+            if -1 in rest:
+                known = int(np.prod([d for d in rest if d != -1]))
+                rest[rest.index(-1)] = per_image // max(1, known)
+            y = x.reshape([x.shape[0]] + rest)
         elif op == "AveragePool":
             k, st, pads = list(a["kernel_shape"]), list(a.get("strides") or [1] * len(a["kernel_shape"])), list(a.get("pads") or [])
             if x.ndim == 3:  # NWC runs as one row
@@ -87,6 +111,13 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             else:
                 pt, pl, pb, pr = pads if pads else (0, 0, 0, 0)
                 y = oracle.avg_pool_s8(x, tuple(k), tuple(st), (pt, pb, pl, pr), spec.exponent(ins[0]), spec.exponent(y_name))
+        elif op == "ReduceMean":
+            axes = spec.initializers[ins[1]][2].ravel() if len(ins) > 1 and ins[1] in spec.initializers else a.get("axes", [])
+            if len(axes) == 0 and a.get("noop_with_empty_axes", 0):
+                y = x
+            else:
+                y = oracle.reduce_mean_s8(x, [int(v) for v in axes], bool(a.get("keepdims", 1)), spec.exponent(ins[0]),
+                                          spec.exponent(y_name))
         elif op == "Slice":
             par = [spec.initializers[n][2].ravel() if n in spec.initializers else None for n in (ins[1:5] + [None] * 4)[:4]]
             y = oracle.slice_(x, par[0], par[1], par[2], par[3])

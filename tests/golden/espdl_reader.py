@@ -111,10 +111,18 @@ def _tensor(t):
     data = None
     p, n = t.vector(8)  # raw_data: [AlignedBytes], 16 bytes each
     np_dtype = _DTYPES.get(dtype)
+    count = int(np.prod(dims)) if dims else 1
     if p is not None and np_dtype is not None:
-        count = int(np.prod(dims)) if dims else 1
         raw = bytes(t.b.d[p:p + 16 * n])
         data = np.frombuffer(raw, dtype=np_dtype, count=count).reshape(dims if dims else ())
+    elif np_dtype is not None:
+        # small tensors may be written as typed arrays: 2 float_data, 3 int32_data, 5 int64_data
+        field = {1: 2, 6: 3, 7: 5}.get(dtype)
+        if field is not None:
+            q, m = t.vector(field)
+            if q is not None and m >= count:
+                raw = bytes(t.b.d[q:q + np.dtype(np_dtype).itemsize * count])
+                data = np.frombuffer(raw, dtype=np_dtype, count=count).reshape(dims if dims else ())
     return {"name": name, "dims": dims, "dtype": dtype, "doc": doc, "exponents": exps, "data": data}
 
 

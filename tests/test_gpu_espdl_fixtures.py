@@ -77,8 +77,11 @@ def test_loaded_graph_matches_oracle_on_random_input(path):
     rm = _round_mode(path)
     batch = 3
     x = spec.make_input(np.random.default_rng(77), batch)
-    want = graph_runner.run(spec, {spec.inputs[0]: x}, oracle.ROUND_HALF_EVEN if rm else oracle.ROUND_HALF_UP,
-                            keep_all=False)
+    try:
+        want = graph_runner.run(spec, {spec.inputs[0]: x}, oracle.ROUND_HALF_EVEN if rm else oracle.ROUND_HALF_UP,
+                                keep_all=False)
+    except NotImplementedError as e:
+        pytest.skip("the oracle's graph runner does not cover this graph: %s" % e)
     g = model.Graph.from_file(path)
     for fuse in (True, False):
         mdl = model.Model(g, batch, round_mode=rm, fuse_lut=fuse, fuse_blocks=fuse)

@@ -118,6 +118,17 @@ def test_slice(oracle, shape, starts, ends, axes, steps, dtype):
     np.testing.assert_array_equal(got, want)
 
 
+@pytest.mark.parametrize("shape,axes,keepdims,exps", [
+    ((4, 7, 7, 64), [1, 2], True, (-4, -5)), ((3, 40, 120), [-1], True, (-5, -5)), ((2, 3, 4, 5), [0, 2], False, (-3, -4)),
+    ((4, 9), [], True, (-6, -6)), ((2, 6, 10), [1], False, (-5, -7)), ((2, 1, 40, 96), [2], True, (-4, -4)),
+])
+def test_reduce_mean_s8(oracle, shape, axes, keepdims, exps):
+    announce(f"reduce_mean {shape} axes {axes} keepdims {keepdims} exps {exps}")
+    x = _rand(np.random.default_rng(28), shape)
+    got = to_host(espdl().reduce_mean_s8(to_dev(x), axes, keepdims, exps[0], exps[1]))
+    np.testing.assert_array_equal(got, oracle.reduce_mean_s8(x, axes, keepdims, exps[0], exps[1]))
+
+
 def test_sppf_pool_chain_idempotence():
     """Size-independent property at full batch: three chained 5x5/1 pools equal one 13x13/1 pool, and
     pooling is monotone (output >= input)."""

@@ -218,6 +218,20 @@ def test_gated_block_with_mul(oracle, round_mode):
     mdl.close()
 
 
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+def test_pooled_embedding_tail(oracle, round_mode):
+    """AveragePool, ReduceMean and Reshape whose axes / shape arrive as initializer operands, then Gemm."""
+    announce(f"model pooled_embedding round_mode={round_mode}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.pooled_embedding()
+    mdl, want, _ = _run_config(spec, 5, 33, round_mode=round_mode)
+    got = mdl.get_tensor(spec.outputs[0])
+    assert got.shape == (5, 64)
+    np.testing.assert_array_equal(got, want[spec.outputs[0]])
+    assert want[spec.outputs[0]].min() < want[spec.outputs[0]].max()
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()

@@ -162,3 +162,26 @@ def test_avg_pool_matches_exact_mean_away_from_ties(oracle, kernel, strides, pad
                     assert got[n, oy, ox, k] == want, (n, oy, ox, k)
                     checked += 1
     assert checked > 50
+
+
+@pytest.mark.parametrize("shape,axes,keepdims,exps", [
+    ((2, 7, 7, 16), [1, 2], True, (-4, -5)), ((3, 5, 8), [-1], True, (-5, -5)), ((2, 3, 4, 5), [0, 2], False, (-3, -4)),
+    ((4, 9), [], True, (-6, -6)), ((2, 6, 10), [1], False, (-5, -7)),
+])
+def test_reduce_mean_matches_exact_mean_away_from_ties(oracle, shape, axes, keepdims, exps):
+    x = _rand(np.random.default_rng(14), shape)
+    got = oracle.reduce_mean_s8(x, axes, keepdims, exps[0], exps[1])
+    nd = len(shape)
+    ax = tuple(a % nd for a in axes) if axes else tuple(range(nd))
+    sums = x.astype(np.int64).sum(axis=ax, keepdims=keepdims)
+    count = int(np.prod([shape[a] for a in ax]))
+    assert got.shape == (sums.shape if sums.shape else (1,))
+    checked = 0
+    for g, sm in zip(got.ravel(), sums.ravel()):
+        exact = Fraction(int(sm), count) * Fraction(2) ** (exps[0] - exps[1])
+        frac = exact - (exact.numerator // exact.denominator)
+        if abs(frac - Fraction(1, 2)) < Fraction(1, 10000):
+            continue
+        assert int(g) == min(127, max(-128, (exact + Fraction(1, 2)).__floor__()))
+        checked += 1
+    assert checked > 0
