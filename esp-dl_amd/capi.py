@@ -78,8 +78,12 @@ def lib():
         L.espdl_hip_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp, vp]
         L.espdl_hip_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp, vp]
         L.espdl_hip_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
+        L.espdl_hip_softmax_s8.argtypes = [vp, i64, i64, i64, i32, vp, vp]
+        L.espdl_hip_quantize_f32.argtypes = [vp, i64, i32, i32, vp, vp]
+        L.espdl_hip_dequantize_f32.argtypes = [vp, i64, i32, i32, vp, vp]
+        L.espdl_hip_matmul_s8.argtypes = [vp, vp, i32, i32, i32, vp, vp, vp, i32, i32, i32, vp, vp]
         for name in ("concat", "copy_rows", "transpose", "resize_nearest_s8", "max_pool", "avg_pool_s8", "slice",
-                     "reduce_mean_s8"):
+                     "reduce_mean_s8", "softmax_s8", "quantize_f32", "dequantize_f32", "matmul_s8"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         mp = ctypes.POINTER(MbconvDesc)
         L.espdl_hip_mbconv_out_shape.argtypes = [mp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
@@ -377,3 +381,50 @@ def reduce_mean_s8(x, axes, keepdims=True, in_exp=0, out_exp=0, stream=None):
     _check(lib().espdl_hip_reduce_mean_s8(_p(x), (ctypes.c_int32 * nd)(*x.shape), nd, (ctypes.c_int32 * nd)(*flags),
                                           in_exp, out_exp, _p(out), _stream(stream)))
     return out.reshape([1 if flags[i] else int(x.shape[i]) for i in range(nd)]) if keepdims else out
+
+
+def softmax_s8(x, axis=-1, in_exp=0, stream=None):
+    """int8 tensor -> float32 softmax along `axis` (espdl_hip_softmax_s8)."""
+    import torch
+    import math
+    axis = axis % x.dim()
+    outer = math.prod(int(d) for d in x.shape[:axis])
+    inner = math.prod(int(d) for d in x.shape[axis + 1:])
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _check(lib().espdl_hip_softmax_s8(_p(x), outer, int(x.shape[axis]), inner, in_exp, _p(out), _stream(stream)))
+    return out
+
+
+def quantize_f32(x, out_exp, dtype=None, stream=None):
+    import torch
+    dtype = dtype or torch.int8
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    _check(lib().espdl_hip_quantize_f32(_p(x), x.numel(), out_exp, out.element_size(), _p(out), _stream(stream)))
+    return out
+
+
+def dequantize_f32(x, in_exp, stream=None):
+    import torch
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    _check(lib().espdl_hip_dequantize_f32(_p(x), x.numel(), in_exp, x.element_size(), _p(out), _stream(stream)))
+    return out
+
+
+def matmul_s8(a, b, shift, activation=0, round_mode=0, stream=None):
+    """a [..., M, K] x b [..., K, N] with up to two broadcast leading dims (espdl_hip_matmul_s8)."""
+    import torch
+    assert a.dim() >= 2 and b.dim() >= 2 and a.dim() <= 4 and b.dim() <= 4 and a.shape[-1] == b.shape[-2]
+    la = [1] * (4 - a.dim()) + [int(d) for d in a.shape[:-2]]
+    lb = [1] * (4 - b.dim()) + [int(d) for d in b.shape[:-2]]
+    lead = [max(la[0], lb[0]), max(la[1], lb[1])]
+    m, k, n = int(a.shape[-2]), int(a.shape[-1]), int(b.shape[-1])
+
+    def strides(l, mat):
+        return [0 if l[0] == 1 else l[1] * mat, 0 if l[1] == 1 else mat]
+
+    rank = max(a.dim(), b.dim())
+    out = torch.empty(lead[4 - rank:] + [m, n] if rank > 2 else [m, n], dtype=torch.int8, device=a.device)
+    _check(lib().espdl_hip_matmul_s8(_p(a), _p(b), m, k, n, (ctypes.c_int32 * 2)(*lead),
+                                     (ctypes.c_int64 * 2)(*strides(la, m * k)), (ctypes.c_int64 * 2)(*strides(lb, k * n)),
+                                     shift, activation, round_mode, _p(out), _stream(stream)))
+    return out

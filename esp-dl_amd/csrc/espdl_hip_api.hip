@@ -731,4 +731,89 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
                          "mbconv_s8_fused");
 }
 
+int espdl_hip_softmax_s8(const int8_t *in, int64_t outer, int64_t len, int64_t inner, int32_t in_exp, float *out,
+                         void *stream)
+{
+    if (outer < 0 || len < 0 || inner < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative extent");
+    if (check_exps(in_exp, 0) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (outer == 0 || len == 0 || inner == 0)
+        return ESPDL_HIP_OK;
+    if (outer > (1ll << 40) / len || outer * len > (1ll << 40) / inner)
+        return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_softmax_s8(in, outer, len, inner, in_exp, out, cu_count_cached(),
+                                                  reinterpret_cast<hipStream_t>(stream)),
+                         "softmax_s8");
+}
+
+int espdl_hip_quantize_f32(const float *in, int64_t size, int32_t out_exp, int32_t elem_size, void *out, void *stream)
+{
+    if (size < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size");
+    if (elem_size != 1 && elem_size != 2)
+        return fail(ESPDL_HIP_EINVAL, "elem_size must be 1 (int8) or 2 (int16)");
+    if (check_exps(0, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_quantize_f32(in, size, out_exp, elem_size, out, cu_count_cached(),
+                                                    reinterpret_cast<hipStream_t>(stream)),
+                         "quantize_f32");
+}
+
+int espdl_hip_dequantize_f32(const void *in, int64_t size, int32_t in_exp, int32_t elem_size, float *out, void *stream)
+{
+    if (size < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size");
+    if (elem_size != 1 && elem_size != 2)
+        return fail(ESPDL_HIP_EINVAL, "elem_size must be 1 (int8) or 2 (int16)");
+    if (check_exps(in_exp, 0) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_dequantize_f32(in, size, in_exp, elem_size, out, cu_count_cached(),
+                                                      reinterpret_cast<hipStream_t>(stream)),
+                         "dequantize_f32");
+}
+
+int espdl_hip_matmul_s8(const int8_t *a, const int8_t *b, int32_t m, int32_t k, int32_t n, const int32_t lead[2],
+                        const int64_t a_stride[2], const int64_t b_stride[2], int32_t shift, int32_t activation,
+                        int32_t round_mode, int8_t *out, void *stream)
+{
+    if (lead == nullptr || a_stride == nullptr || b_stride == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "lead, a_stride and b_stride must not be NULL");
+    if (m < 0 || k < 0 || n < 0 || lead[0] < 0 || lead[1] < 0 || a_stride[0] < 0 || a_stride[1] < 0 || b_stride[0] < 0 ||
+        b_stride[1] < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative extent or stride");
+    if (activation != ESPDL_HIP_LINEAR && activation != ESPDL_HIP_RELU)
+        return fail(ESPDL_HIP_EINVAL, "activation must be ESPDL_HIP_LINEAR or ESPDL_HIP_RELU");
+    if (round_mode != ESPDL_HIP_ROUND_HALF_UP && round_mode != ESPDL_HIP_ROUND_HALF_EVEN)
+        return fail(ESPDL_HIP_EINVAL, "unknown round mode %d", round_mode);
+    if (shift < -31 || shift > 62)
+        return fail(ESPDL_HIP_EINVAL, "shift %d outside [-31, 62]", shift);
+    if (m == 0 || n == 0 || lead[0] == 0 || lead[1] == 0)
+        return ESPDL_HIP_OK;
+    if ((long long)lead[0] * lead[1] > 65535)
+        return fail(ESPDL_HIP_ENOTSUP, "more than 65535 matrix pairs in one call");
+    if (k > (1 << 16))
+        return fail(ESPDL_HIP_ENOTSUP, "k above 65536: the int32 accumulator could overflow");
+    if ((long long)m * n > 0x7fffffffll || (long long)m * k > 0x7fffffffll || (long long)k * n > 0x7fffffffll)
+        return fail(ESPDL_HIP_ENOTSUP, "matrix too large for this build");
+    if (a == nullptr || b == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "a, b and out must not be NULL");
+    const int ld[2] = {lead[0], lead[1]};
+    const long long as[2] = {a_stride[0], a_stride[1]}, bs[2] = {b_stride[0], b_stride[1]};
+    return device_status(espdl::launch_matmul_s8(a, b, m, k, n, ld, as, bs, shift, activation == ESPDL_HIP_RELU,
+                                                 round_mode == ESPDL_HIP_ROUND_HALF_EVEN, out,
+                                                 reinterpret_cast<hipStream_t>(stream)),
+                         "matmul_s8");
+}
+
 } // extern "C"

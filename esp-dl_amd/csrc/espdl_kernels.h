@@ -125,4 +125,15 @@ hipError_t launch_slice(const void *in, const int *shape, int dims, const int *s
 hipError_t launch_reduce_mean_s8(const int8_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
                                  int out_exp, int8_t *out, int cu_count, hipStream_t stream);
 
+// attention_ops.hip
+hipError_t launch_softmax_s8(const int8_t *in, long long outer, long long len, long long inner, int in_exp, float *out,
+                             int cu_count, hipStream_t stream);
+hipError_t launch_quantize_f32(const float *in, long long size, int out_exp, int elem_size, void *out, int cu_count,
+                               hipStream_t stream);
+hipError_t launch_dequantize_f32(const void *in, long long size, int in_exp, int elem_size, float *out, int cu_count,
+                                 hipStream_t stream);
+hipError_t launch_matmul_s8(const int8_t *a, const int8_t *b, int m, int k, int n, const int lead[2],
+                            const long long a_stride[2], const long long b_stride[2], int shift, bool relu, bool half_even,
+                            int8_t *out, hipStream_t stream);
+
 } // namespace espdl

@@ -72,6 +72,11 @@ public:
         register_module("AveragePool", AveragePool::deserialize);
         register_module("Slice", Slice::deserialize);
         register_module("ReduceMean", ReduceMean::deserialize);
+        register_module("Softmax", Softmax::deserialize);
+        // both are TensorBase::assign between a float32 and a quantized tensor
+        // (esp-dl/dl/module/include/dl_module_creator.hpp:154-155)
+        register_module("QuantizeLinear", RequantizeLinear::deserialize);
+        register_module("DequantizeLinear", RequantizeLinear::deserialize);
         // element-wise activations that esp-ppq exports with a precomputed 8-bit table
         for (const char *op : {"Swish", "HardSwish", "Sigmoid", "HardSigmoid", "Tanh", "Gelu", "Elu", "LeakyRelu",
                                "Exp", "Log", "Sqrt", "Softplus", "Mish"}) {

@@ -124,6 +124,26 @@ public:
     std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
     {
         const std::vector<int> &a = input_shapes[0], &b = input_shapes[1];
+        if (batched_rhs(b)) {
+            // both operands carry leading dims: numpy-style broadcast of up to two of them
+            // (esp-dl/dl/module/include/dl_module_matmul.hpp: the rank-3 and rank-4 branches)
+            if (a.size() < 2 || a.size() > 4 || a.back() != b[b.size() - 2])
+                return {{}};
+            int la[2], lb[2];
+            leading(a, la);
+            leading(b, lb);
+            for (int i = 0; i < 2; i++)
+                if (la[i] != lb[i] && la[i] != 1 && lb[i] != 1)
+                    return {{}};
+            std::vector<int> out;
+            const size_t rank = std::max(a.size(), b.size());
+            if (rank == 4)
+                out.push_back(std::max(la[0], lb[0]));
+            out.push_back(std::max(la[1], lb[1]));
+            out.push_back(a[a.size() - 2]);
+            out.push_back(b.back());
+            return {out};
+        }
         // right-hand side: [K, N] matrix, or the [1, 1, K, N] filter view of it
         const int k = b.size() == 4 ? b[2] : b[0];
         const int n = b.size() == 4 ? b[3] : (b.size() == 2 ? b[1] : 1);
@@ -136,22 +156,72 @@ public:
 
     int64_t get_macs(std::vector<std::vector<int>> &input_shapes)
     {
-        int64_t total = 1;
-        for (int d : input_shapes[0])
+        const std::vector<int> out = get_output_shape(input_shapes)[0];
+        if (out.empty() || input_shapes[0].empty())
+            return 0;
+        int64_t total = input_shapes[0].back(); // k multiply-accumulates per output element
+        for (int d : out)
             total *= d;
-        return total * get_output_shape(input_shapes)[0].back();
+        return total;
     }
 
     void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
     {
         (void)mode;
         TensorBase *rhs = context->get_tensor(m_inputs_index[1]);
-        if (m_inputs_index[1] < CONTEXT_PARAMETER_OFFSET || !rhs || (rhs->shape.size() != 2 && rhs->shape.size() != 4)) {
-            DL_LOGE("MatMul", "%s: only a constant right-hand side of rank 2 is implemented", name.c_str());
+        if (rhs && m_inputs_index[1] < CONTEXT_PARAMETER_OFFSET) {
+            forward_activations(context, context->get_tensor(m_inputs_index[0]), rhs,
+                                context->get_tensor(m_outputs_index[0]));
+            return;
+        }
+        if (!rhs || (rhs->shape.size() != 2 && rhs->shape.size() != 4)) {
+            DL_LOGE("MatMul", "%s: a constant right-hand side must have rank 2 (or its rank-4 filter view)", name.c_str());
             return;
         }
         gemm_forward("MatMul", name, quant_type, m_activation, context, context->get_tensor(m_inputs_index[0]), rhs,
                      nullptr, context->get_tensor(m_outputs_index[0]), m_shift);
+    }
+
+    /// True when the right-hand side is a stack of matrices (an activation), not one [K, N] matrix.
+    static bool batched_rhs(const std::vector<int> &b)
+    {
+        return b.size() == 3 || (b.size() == 4 && (b[0] != 1 || b[1] != 1));
+    }
+    /// The two leading extents of a rank 2..4 operand, padded with 1 in front.
+    static void leading(const std::vector<int> &s, int lead[2])
+    {
+        lead[0] = s.size() == 4 ? s[0] : 1;
+        lead[1] = s.size() >= 3 ? s[s.size() - 3] : 1;
+    }
+
+    /// Both operands are activations: every pair of matrices runs as the reference's 1x1 convolution
+    /// with one shift (espdl_hip_matmul_s8).
+    void forward_activations(ModelContext *context, TensorBase *a, TensorBase *b, TensorBase *output)
+    {
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !a || !output || !a->on_device() || !b->on_device() ||
+            !output->on_device() || a->shape.size() < 2 || a->shape.size() > 4 || b->shape.size() < 2 ||
+            b->shape.size() > 4 || a->shape.back() != b->shape[b->shape.size() - 2]) {
+            DL_LOGE("MatMul", "%s: two activations need int8 device tensors of rank 2..4 with matching inner extent",
+                    name.c_str());
+            return;
+        }
+        int la[2], lb[2];
+        leading(a->shape, la);
+        leading(b->shape, lb);
+        const int32_t m = a->shape[a->shape.size() - 2], k = a->shape.back(), n = b->shape.back();
+        const int32_t lead[2] = {std::max(la[0], lb[0]), std::max(la[1], lb[1])};
+        const int64_t mk = (int64_t)m * k, kn = (int64_t)k * n;
+        const int64_t as[2] = {la[0] == 1 ? 0 : la[1] * mk, la[1] == 1 ? 0 : mk};
+        const int64_t bs[2] = {lb[0] == 1 ? 0 : lb[1] * kn, lb[1] == 1 ? 0 : kn};
+        const int shift = output->exponent.get() - a->exponent.get() - b->exponent.get();
+        const int rc = espdl_hip_matmul_s8(static_cast<const int8_t *>(a->data), static_cast<const int8_t *>(b->data), m, k,
+                                           n, lead, as, bs, shift,
+                                           m_activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR,
+                                           context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN
+                                                                                       : ESPDL_HIP_ROUND_HALF_UP,
+                                           static_cast<int8_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("MatMul", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
 
     static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)

@@ -649,5 +649,57 @@ public:
     void print() { DL_LOGI("ReduceMean", "keepdims: %d, quant_type: %s.", m_keepdims, quant_type_to_string(quant_type)); }
 };
 
+/// Softmax on an int8 tensor with a float32 result (esp-dl/dl/module/include/dl_module_softmax.hpp,
+/// forward_lut): the exported graphs follow it with QuantizeLinear.
+class Softmax : public Module {
+private:
+    int m_axis;
+
+public:
+    Softmax(const char *name = nullptr, int axis = -1, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_axis(axis)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        return {input_shapes[0]};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type != QUANT_TYPE_SYMM_8BIT || !input || !output || !input->on_device() || !output->on_device() ||
+            input->dtype != DATA_TYPE_INT8 || output->dtype != DATA_TYPE_FLOAT || input->shape.empty()) {
+            DL_LOGE("Softmax", "%s: needs an int8 device input and a float32 device output", name.c_str());
+            return;
+        }
+        const int rank = (int)input->shape.size();
+        const int axis = m_axis < 0 ? m_axis + rank : m_axis;
+        if (axis < 0 || axis >= rank) {
+            DL_LOGE("Softmax", "%s: axis %d outside rank %d", name.c_str(), m_axis, rank);
+            return;
+        }
+        int64_t outer = 1, inner = 1;
+        for (int i = 0; i < axis; i++)
+            outer *= input->shape[i];
+        for (int i = axis + 1; i < rank; i++)
+            inner *= input->shape[i];
+        const int rc = espdl_hip_softmax_s8(static_cast<const int8_t *>(input->data), outer, input->shape[axis], inner,
+                                            input->exponent.get(), static_cast<float *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Softmax", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        int axis = -1;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "axis", axis);
+        return new Softmax(node_name.c_str(), axis, quant_type);
+    }
+    void print() { DL_LOGI("Softmax", "axis: %d, quant_type: %s.", m_axis, quant_type_to_string(quant_type)); }
+};
+
 } // namespace module
 } // namespace dl

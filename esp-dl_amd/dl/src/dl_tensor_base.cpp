@@ -275,6 +275,16 @@ bool TensorBase::assign(TensorBase *tensor, void *stream)
     }
     const bool ints = (dtype == DATA_TYPE_INT8 || dtype == DATA_TYPE_INT16) &&
         (tensor->dtype == DATA_TYPE_INT8 || tensor->dtype == DATA_TYPE_INT16);
+    // float32 <-> quantized on the device (QuantizeLinear / DequantizeLinear,
+    // esp-dl/dl/tensor/src/dl_tensor_base.cpp:251-268 and :286-299)
+    if (on_device() && tensor->on_device()) {
+        if (tensor->dtype == DATA_TYPE_FLOAT && (dtype == DATA_TYPE_INT8 || dtype == DATA_TYPE_INT16))
+            return espdl_hip_quantize_f32(static_cast<const float *>(tensor->data), size, exponent,
+                                          dtype == DATA_TYPE_INT8 ? 1 : 2, data, stream) == ESPDL_HIP_OK;
+        if (dtype == DATA_TYPE_FLOAT && (tensor->dtype == DATA_TYPE_INT8 || tensor->dtype == DATA_TYPE_INT16))
+            return espdl_hip_dequantize_f32(tensor->data, size, tensor->exponent, tensor->dtype == DATA_TYPE_INT8 ? 1 : 2,
+                                            static_cast<float *>(data), stream) == ESPDL_HIP_OK;
+    }
     if (!ints) {
         DL_LOGE("TensorBase::assign", "unsupported conversion %s -> %s", dtype_to_string(tensor->dtype),
                 dtype_to_string(dtype));

@@ -314,6 +314,38 @@ class Builder:
         g.add_node(name, "Reshape", [x, name + ".shape"], [y], allowzero=0, quant_type="S8")
         return y
 
+    def softmax(self, x, axis=-1, name=None):
+        """Softmax with a float32 result, as the exporter leaves it (QuantizeLinear follows)."""
+        g = self.g
+        name = name or self._name("softmax")
+        y = name + "_out"
+        g.add_value(y, g.shape(x), 0, FLOAT)
+        g.add_node(name, "Softmax", [x], [y], axis=axis, quant_type="S8")
+        return y
+
+    def quantize(self, x, out_exp, name=None):
+        g = self.g
+        name = name or self._name("quantize")
+        y = name + "_out"
+        g.add_value(y, g.shape(x), out_exp, INT8)
+        g.add_node(name, "QuantizeLinear", [x], [y], quant_type="S8")
+        return y
+
+    def matmul_act(self, a, b, out_exp=None, name=None):
+        """MatMul of two activations (rank 3 or 4, equal leading dims or 1)."""
+        g = self.g
+        name = name or self._name("matmul")
+        sa, sb = g.shape(a), g.shape(b)
+        assert sa[-1] == sb[-2]
+        lead = [max(p, q) for p, q in zip(sa[:-2], sb[:-2])]
+        if out_exp is None:
+            out_exp = typical_shift(sa[-1]) + g.exponent(a) + g.exponent(b)
+        y = name + "_out"
+        g.add_value(y, lead + [sa[-2], sb[-1]], out_exp)
+        g.add_node(name, "MatMul", [a, b], [y], activation="Linear", quant_type="S8")
+        g.macs_per_image += int(np.prod(lead[1:])) * sa[-2] * sa[-1] * sb[-1]
+        return y
+
     def max_pool(self, x, k, stride=1, pad=None, name=None):
         g = self.g
         name = name or self._name("maxpool")
@@ -630,4 +662,37 @@ def pooled_embedding(seed=0xE5D7):
     h = b.reshape(h, [1, -1], name="view")
     y = b.gemm(h, 64, relu=True, name="fc")
     b.output(y)
+    return g
+
+
+def attention_block(seed=0xE5D8, hw=10, heads=2, key_dim=16, head_dim=32):
+    """The position-sensitive attention block of the reference's exported YOLO11n graphs: a 1x1 Conv makes
+    q, k and v, Reshape / Split / Transpose bring them to [1, heads, ., hw*hw], q^T x k is scaled (Mul by a
+    constant), Softmax leaves a float32 tensor that QuantizeLinear turns back into int8, v x attn^T is
+    reshaped to the feature map, a depthwise positional Conv of v is added and a 1x1 Conv projects."""
+    g = GraphSpec("attention_block")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    c = heads * head_dim
+    per_head = 2 * key_dim + head_dim
+    n = hw * hw
+    x = b.input("input", [1, hw, hw, c], -4)
+    qkv = b.conv(x, heads * per_head, k=1, name="qkv")                  # [1, hw, hw, heads*per_head]
+    qkv = b.transpose(qkv, [0, 3, 1, 2], name="qkv_nchw")               # [1, heads*per_head, hw, hw]
+    qkv = b.reshape(qkv, [1, heads, per_head, n], name="qkv_heads")     # [1, heads, per_head, n]
+    q, k, v = b.split(qkv, [key_dim, key_dim, head_dim], axis=2, name="qkv_split")
+    qt = b.transpose(q, [0, 1, 3, 2], name="q_t")                        # [1, heads, n, key_dim]
+    attn = b.matmul_act(qt, k, name="qk")                                # [1, heads, n, n]
+    g.add_init("attn_scale", [1], INT8, [91], [-9])                      # ~ key_dim ** -0.5 at exponent -9
+    y = "attn_scaled_out"
+    g.add_value(y, g.shape(attn), -3)
+    g.add_node("attn_scaled", "Mul", [attn, "attn_scale"], [y], quant_type="S8")
+    attn = b.quantize(b.softmax(y, axis=-1, name="attn_softmax"), -8, name="attn_q")
+    attn_t = b.transpose(attn, [0, 1, 3, 2], name="attn_t")              # [1, heads, n, n]
+    o = b.matmul_act(v, attn_t, out_exp=g.exponent(v), name="av")                               # [1, heads, head_dim, n]
+    o = b.reshape(o, [1, c, hw, hw], name="o_map")
+    o = b.transpose(o, [0, 2, 3, 1], name="o_nhwc")                      # [1, hw, hw, c]
+    vmap = b.transpose(b.reshape(v, [1, c, hw, hw], name="v_map"), [0, 2, 3, 1], name="v_nhwc")
+    pe = b.conv(vmap, c, k=3, depthwise=True, name="pe")
+    o = b.add(o, pe, name="o_pe")
+    b.output(b.conv(o, c, k=1, name="proj"))
     return g

@@ -206,6 +206,31 @@ int espdl_hip_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w,
 int espdl_hip_reduce_mean_s8(const int8_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
                              int32_t in_exp, int32_t out_exp, int8_t *out, void *stream);
 
+/* module::Softmax on an int8 tensor (Softmax::forward_lut, esp-dl/dl/module/include/dl_module_softmax.hpp:148-217):
+ * the tensor is viewed as [outer][len][inner] and normalized along len; out is float32 of the same
+ * layout, out = T[q] / sum_i T[q_i] with T[q] = expf(2^in_exp * q), the sum taken in float32 in index
+ * order.  No maximum is subtracted, as in the reference's int8 path. */
+int espdl_hip_softmax_s8(const int8_t *in, int64_t outer, int64_t len, int64_t inner, int32_t in_exp, float *out,
+                         void *stream);
+
+/* QuantizeLinear: TensorBase::assign from float32 (esp-dl/dl/tensor/src/dl_tensor_base.cpp:251-268):
+ * out = clamp(round_half_up(in * 2^-out_exp)).  elem_size 1 writes int8, 2 writes int16. */
+int espdl_hip_quantize_f32(const float *in, int64_t size, int32_t out_exp, int32_t elem_size, void *out, void *stream);
+
+/* DequantizeLinear: TensorBase::assign into float32 (dl_tensor_base.cpp:286-299): out = in * 2^in_exp.
+ * elem_size 1 reads int8, 2 reads int16. */
+int espdl_hip_dequantize_f32(const void *in, int64_t size, int32_t in_exp, int32_t elem_size, float *out, void *stream);
+
+/* module::MatMul with two int8 activations (batched branches of MatMul::forward_template,
+ * esp-dl/dl/module/include/dl_module_matmul.hpp): for each of lead[0] x lead[1] leading index pairs
+ * out[z0][z1] = a[z0][z1] ([m][k]) x b[z0][z1] ([k][n]), each run as the reference's 1x1 convolution with
+ * one shift = out_exp - a_exp - b_exp, ESPDL_HIP_LINEAR / _RELU and the given round mode.  a_stride and
+ * b_stride give each operand's element stride per leading dim (0 broadcasts that operand); out is dense
+ * [lead[0]][lead[1]][m][n].  lead[0] * lead[1] <= 65535. */
+int espdl_hip_matmul_s8(const int8_t *a, const int8_t *b, int32_t m, int32_t k, int32_t n, const int32_t lead[2],
+                        const int64_t a_stride[2], const int64_t b_stride[2], int32_t shift, int32_t activation,
+                        int32_t round_mode, int8_t *out, void *stream);
+
 /* TensorBase::slice for positive steps (esp-dl/dl/base/dl_base_shape.cpp:68-120 gives the shape rule):
  * out[i0, i1, ...] = in[start[0] + i0 * step[0], start[1] + i1 * step[1], ...].  The caller passes
  * normalized values per dim (0 <= start, step >= 1, out_shape) for all `dims` dims of the input;

@@ -625,6 +625,58 @@ void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int 
     }
 }
 
+/*
+ * Softmax on an int8 tensor, float32 result (Softmax::forward_lut,
+ * esp-dl/dl/module/include/dl_module_softmax.hpp:148-217): a 256-entry table
+ * expf(DL_SCALE(in_exp) * (i - 128)) (tool::gen_lut_8bit, esp-dl/dl/tool/src/dl_tool.cpp:258-268), the
+ * row sum accumulated in float32 in index order, then one division per element.  No maximum is
+ * subtracted on this path.  The tensor is viewed as [outer][len][inner], softmax along len.
+ */
+void espdl_oracle_softmax_s8(const int8_t *in, int64_t outer, int64_t len, int64_t inner, int in_exp, float *out)
+{
+    float table[256];
+    const float scale = dl_scale(in_exp);
+    for (int i = 0; i < 256; i++)
+        table[i] = expf(scale * (float)(i - 128));
+    for (int64_t o = 0; o < outer; o++)
+        for (int64_t k = 0; k < inner; k++) {
+            const int8_t *src = in + o * len * inner + k;
+            float *dst = out + o * len * inner + k;
+            float sum = 0.f;
+            for (int64_t i = 0; i < len; i++) {
+                dst[i * inner] = table[(int)src[i * inner] + 128];
+                sum += dst[i * inner];
+            }
+            for (int64_t i = 0; i < len; i++)
+                dst[i * inner] = dst[i * inner] / sum;
+        }
+}
+
+/*
+ * QuantizeLinear = TensorBase::assign from a float32 tensor
+ * (esp-dl/dl/tensor/src/dl_tensor_base.cpp:251-268, quantize :17-29): clip(round(v * DL_RESCALE(out_exp))).
+ * elem_size 1 writes int8, 2 writes int16.
+ */
+void espdl_oracle_quantize_f32(const float *in, int64_t size, int out_exp, int elem_size, void *out)
+{
+    const float inv_scale = dl_rescale(out_exp);
+    for (int64_t i = 0; i < size; i++) {
+        const int q = round_half_up_f32(in[i] * inv_scale);
+        if (elem_size == 1)
+            ((int8_t *)out)[i] = (int8_t)clamp_i64(q, INT8_MIN, INT8_MAX);
+        else
+            ((int16_t *)out)[i] = (int16_t)clamp_i64(q, INT16_MIN, INT16_MAX);
+    }
+}
+
+/* DequantizeLinear = TensorBase::assign into a float32 tensor (dl_tensor_base.cpp:286-299): v * DL_SCALE(in_exp). */
+void espdl_oracle_dequantize_f32(const void *in, int64_t size, int in_exp, int elem_size, float *out)
+{
+    const float scale = dl_scale(in_exp);
+    for (int64_t i = 0; i < size; i++)
+        out[i] = (elem_size == 1 ? (float)((const int8_t *)in)[i] : (float)((const int16_t *)in)[i]) * scale;
+}
+
 /* ---------------------------------------------------------------------------------------------
  * Data-movement operators of the detection necks (Concat, Split, Transpose, Resize, MaxPool).
  * ------------------------------------------------------------------------------------------- */

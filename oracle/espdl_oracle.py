@@ -62,6 +62,12 @@ def lib():
         L.espdl_oracle_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp]
         L.espdl_oracle_reduce_mean_s8.restype = i32
         L.espdl_oracle_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp]
+        L.espdl_oracle_softmax_s8.restype = None
+        L.espdl_oracle_softmax_s8.argtypes = [vp, i64, i64, i64, i32, vp]
+        L.espdl_oracle_quantize_f32.restype = None
+        L.espdl_oracle_quantize_f32.argtypes = [vp, i64, i32, i32, vp]
+        L.espdl_oracle_dequantize_f32.restype = None
+        L.espdl_oracle_dequantize_f32.argtypes = [vp, i64, i32, i32, vp]
         L.espdl_oracle_slice.restype = i32
         L.espdl_oracle_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp]
         L.espdl_oracle_concat.argtypes = [vp, i32, vp, i64, i32, vp]
@@ -168,6 +174,48 @@ def gemm_s8(x, filt, bias, shift, activation=LINEAR, round_mode=ROUND_HALF_UP):
     m = x.size // k
     y = conv2d_s8(x.reshape(1, 1, m, k), filt, bias, shift, (1, 1), activation=activation, round_mode=round_mode)
     return y.reshape(x.shape[:-1] + (y.shape[-1],))
+
+
+def matmul_s8(a, b, shift, activation=LINEAR, round_mode=ROUND_HALF_UP):
+    """MatMul of two activations: every [M,K] x [K,N] pair of the broadcast leading dims runs as a 1x1
+    convolution whose filter is the second operand (esp-dl/dl/module/include/dl_module_matmul.hpp: the
+    batched branches build {1,1,K,N} filter views and call base::conv2d per matrix); one shift for all."""
+    a, b = _c(a, np.int8), _c(b, np.int8)
+    assert a.ndim >= 2 and b.ndim >= 2 and a.shape[-1] == b.shape[-2]
+    lead = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
+    m, k, n = a.shape[-2], a.shape[-1], b.shape[-1]
+    ab = np.broadcast_to(a, lead + (m, k)).reshape(-1, m, k)
+    bb = np.broadcast_to(b, lead + (k, n)).reshape(-1, k, n)
+    out = np.empty((ab.shape[0], m, n), dtype=np.int8)
+    sh = np.array([shift], dtype=np.int32)
+    for i in range(ab.shape[0]):
+        out[i] = gemm_s8(ab[i], np.ascontiguousarray(bb[i].T), None, sh, activation=activation, round_mode=round_mode)
+    return out.reshape(lead + (m, n))
+
+
+def softmax_s8(x, axis=-1, in_exp=0):
+    x = _c(x, np.int8)
+    axis = axis % x.ndim
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    out = np.empty(x.shape, dtype=np.float32)
+    lib().espdl_oracle_softmax_s8(_ptr(x), outer, x.shape[axis], inner, int(in_exp), _ptr(out))
+    return out
+
+
+def quantize_f32(x, out_exp, dtype=np.int8):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, dtype=dtype)
+    lib().espdl_oracle_quantize_f32(_ptr(x), x.size, int(out_exp), out.itemsize, _ptr(out))
+    return out
+
+
+def dequantize_f32(x, in_exp):
+    x = np.ascontiguousarray(x)
+    assert x.dtype in (np.int8, np.int16)
+    out = np.empty(x.shape, dtype=np.float32)
+    lib().espdl_oracle_dequantize_f32(_ptr(x), x.size, int(in_exp), x.itemsize, _ptr(out))
+    return out
 
 
 def lut_s8(x, table):

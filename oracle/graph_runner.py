@@ -53,6 +53,20 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
                 pt, pl, pb, pr = a["pads"]
                 y = fn(x, w, bias, shift, (dims[0], dims[1]), tuple(a["strides"]), tuple(a["dilations"]),
                        (pt, pb, pl, pr), act, round_mode)
+        elif op == "MatMul" and ins[1] in t:
+            # two activations: per matrix pair a 1x1 convolution with one shift
+            shift = spec.exponent(y_name) - spec.exponent(ins[0]) - spec.exponent(ins[1])
+            act = oracle.RELU if a.get("activation", "Linear") == "Relu" else oracle.LINEAR
+            y = oracle.matmul_s8(x, t[ins[1]], shift, act, round_mode)
+        elif op == "Softmax":
+            if x.dtype != np.int8:
+                raise NotImplementedError("Softmax on " + str(x.dtype))
+            y = oracle.softmax_s8(x, a.get("axis", -1), spec.exponent(ins[0]))
+        elif op in ("QuantizeLinear", "DequantizeLinear") or (op == "RequantizeLinear" and x.dtype == np.float32):
+            if x.dtype == np.float32:
+                y = oracle.quantize_f32(x, spec.exponent(y_name), np.int16 if spec.dtype(y_name) == INT16 else np.int8)
+            else:
+                y = oracle.dequantize_f32(x, spec.exponent(ins[0]))
         elif op in ("Gemm", "MatMul"):
             w = spec.initializers[ins[1]][2]
             bias = spec.initializers[ins[2]][2] if len(ins) > 2 else None
@@ -60,6 +74,8 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             act = oracle.RELU if a.get("activation", "Linear") == "Relu" else oracle.LINEAR
             y = oracle.gemm_s8(x, w, bias, shift, activation=act, round_mode=round_mode)
         elif "lut" in a:
+            if x.dtype != np.int8 or spec.initializers[a["lut"]][2].size != 256:
+                raise NotImplementedError("16-bit LUT")
             y = oracle.lut_s8(x, spec.initializers[a["lut"]][2])
         elif op == "Relu":
             y = oracle.relu_s8(x, spec.exponent(ins[0]), spec.exponent(y_name))

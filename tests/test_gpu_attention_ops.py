@@ -1,0 +1,138 @@
+"""Softmax (int8 -> float32), QuantizeLinear / DequantizeLinear and activation x activation MatMul on the GPU
+against the CPU oracle.  Integer results are bit-exact.  The float32 softmax is compared bit for bit too: both
+sides build the 256-entry table with the host C library's expf, add the row in index order in float32 and
+divide once per element in IEEE float32."""
+import numpy as np
+import pytest
+
+from gpu_util import announce, espdl, to_dev, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand(rng, shape, dtype=np.int8):
+    info = np.iinfo(dtype)
+    return rng.integers(info.min, info.max + 1, size=shape).astype(dtype)
+
+
+SOFTMAX_CASES = [
+    # (shape, axis, in_exp)
+    ((2, 2, 400, 400), -1, -3),   # the attention map of the exported YOLO11n graphs at 640 x 640
+    ((3, 2, 100, 100), -1, -3),
+    ((5, 7, 33), -1, -4),         # odd row length
+    ((300, 1), -1, -2),           # rows of one element
+    ((2, 1000, 6), -1, -5),       # many short rows
+    ((4, 3000), -1, -4),          # rows longer than one staging buffer line
+    ((2, 40000), -1, -6),         # rows too long for LDS staging: strided path with inner == 1
+    ((2, 16, 20, 20), 1, -3),     # softmax over channels of an NCHW map (DFL-style)
+    ((3, 9, 5), 0, -4),
+    ((2, 5, 7, 3), 2, -4),
+]
+
+
+@pytest.mark.parametrize("case", SOFTMAX_CASES, ids=lambda c: f"{c[0]}_ax{c[1]}")
+def test_softmax_s8(oracle, case):
+    shape, axis, in_exp = case
+    announce(f"softmax_s8 {case}")
+    x = _rand(np.random.default_rng(41), shape)
+    got = to_host(espdl().softmax_s8(to_dev(x), axis, in_exp))
+    want = oracle.softmax_s8(x, axis, in_exp)
+    assert got.dtype == np.float32
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_softmax_empty():
+    announce("softmax_s8 empty")
+    import torch
+    out = espdl().softmax_s8(torch.empty((0, 8), dtype=torch.int8, device="cuda"), -1, -3)
+    assert tuple(out.shape) == (0, 8)
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("out_exp", [-9, -7, 0, 3])
+def test_quantize_f32(oracle, dtype, out_exp):
+    announce(f"quantize_f32 {dtype.__name__} exp {out_exp}")
+    import torch
+    rng = np.random.default_rng(42)
+    info = np.iinfo(dtype)
+    scale = 2.0 ** out_exp
+    x = np.concatenate([(rng.standard_normal(100003) * info.max * scale * 0.7).astype(np.float32),
+                        ((np.arange(-300, 300) + 0.5) * scale).astype(np.float32),
+                        rng.random(5000, dtype=np.float32)])
+    got = to_host(espdl().quantize_f32(to_dev(x), out_exp, torch.int8 if dtype == np.int8 else torch.int16))
+    np.testing.assert_array_equal(got, oracle.quantize_f32(x, out_exp, dtype))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+def test_dequantize_f32(oracle, dtype):
+    announce(f"dequantize_f32 {dtype.__name__}")
+    x = _rand(np.random.default_rng(43), (7, 1001), dtype)
+    for e in (-12, -3, 0, 4):
+        got = to_host(espdl().dequantize_f32(to_dev(x), e))
+        np.testing.assert_array_equal(got.view(np.uint32), oracle.dequantize_f32(x, e).view(np.uint32))
+
+
+def test_softmax_then_quantize_matches_reference_chain(oracle):
+    """Softmax -> QuantizeLinear as the exported attention blocks chain them."""
+    announce("softmax + quantize chain")
+    x = _rand(np.random.default_rng(44), (2, 2, 400, 400))
+    m = espdl()
+    got = to_host(m.quantize_f32(m.softmax_s8(to_dev(x), -1, -3), -9))
+    np.testing.assert_array_equal(got, oracle.quantize_f32(oracle.softmax_s8(x, -1, -3), -9))
+    assert got.max() > 0
+
+
+MATMUL_CASES = [
+    # (a shape, b shape, shift)
+    ((2, 2, 400, 32), (2, 2, 32, 400), 9),     # q^T x k of the exported attention block
+    ((2, 2, 64, 400), (2, 2, 400, 400), 8),    # v x attn^T
+    ((3, 1, 5, 7), (1, 4, 7, 3), 6),           # both leading dims broadcast, tiles mostly empty
+    ((2, 65, 33), (2, 33, 130), 7),            # rank 3, extents just past one tile / chunk
+    ((4, 9, 64), (1, 64, 64), 9),              # rank 3, right operand broadcast
+    ((17, 100), (100, 19), 8),                 # plain matrices
+    ((1, 1, 1, 1), (1, 1, 1, 1), 1),
+    ((2, 3, 8, 16), (2, 3, 16, 8), 0),         # shift 0: saturation only
+    ((2, 3, 8, 16), (2, 3, 16, 8), -2),        # left shift
+]
+
+
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+@pytest.mark.parametrize("case", MATMUL_CASES, ids=lambda c: f"{c[0]}x{c[1]}_s{c[2]}")
+def test_matmul_s8(oracle, case, round_mode):
+    sa, sb, shift = case
+    announce(f"matmul_s8 {case} round_mode={round_mode}")
+    rng = np.random.default_rng(45)
+    a, b = _rand(rng, sa), _rand(rng, sb)
+    for act in (oracle.LINEAR, oracle.RELU):
+        got = to_host(espdl().matmul_s8(to_dev(a), to_dev(b), shift, act, round_mode))
+        want = oracle.matmul_s8(a, b, shift, act, round_mode)
+        np.testing.assert_array_equal(got, want.reshape(got.shape))
+
+
+def test_matmul_rounding_ties(oracle):
+    """Accumulators that sit exactly on .5 after the shift: the two rounding modes differ there."""
+    announce("matmul_s8 ties")
+    a = np.zeros((1, 1, 64, 4), dtype=np.int8)
+    a[0, 0, :, 0] = np.arange(-32, 32)
+    b = np.zeros((1, 1, 4, 64), dtype=np.int8)
+    b[0, 0, 0, :] = 1
+    up = to_host(espdl().matmul_s8(to_dev(a), to_dev(b), 1, 0, 0))
+    even = to_host(espdl().matmul_s8(to_dev(a), to_dev(b), 1, 0, 1))
+    np.testing.assert_array_equal(up, oracle.matmul_s8(a, b, 1, 0, 0))
+    np.testing.assert_array_equal(even, oracle.matmul_s8(a, b, 1, 0, 1))
+    assert not np.array_equal(up, even)
+
+
+def test_matmul_rejects_bad_arguments():
+    announce("matmul_s8 argument checks")
+    import ctypes
+    import torch
+    m = espdl()
+    a = torch.zeros((2, 4), dtype=torch.int8, device="cuda")
+    lead = (ctypes.c_int32 * 2)(70000, 1)
+    z = (ctypes.c_int64 * 2)(0, 0)
+    rc = m.lib().espdl_hip_matmul_s8(a.data_ptr(), a.data_ptr(), 2, 4, 2, lead, z, z, 7, 0, 0, a.data_ptr(), None)
+    assert rc != 0 and b"65535" in m.lib().espdl_hip_last_error()
+    lead = (ctypes.c_int32 * 2)(1, 1)
+    assert m.lib().espdl_hip_matmul_s8(a.data_ptr(), a.data_ptr(), 2, 4, 2, lead, z, z, 7, 5, 0, a.data_ptr(), None) != 0
+    assert m.lib().espdl_hip_matmul_s8(a.data_ptr(), None, 2, 4, 2, lead, z, z, 7, 0, 0, a.data_ptr(), None) != 0

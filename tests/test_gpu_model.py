@@ -232,6 +232,19 @@ def test_pooled_embedding_tail(oracle, round_mode):
     mdl.close()
 
 
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+def test_attention_block(oracle, round_mode):
+    """MatMul of two activations, Mul by a constant, Softmax to float32, QuantizeLinear back to int8."""
+    announce(f"model attention_block round_mode={round_mode}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.attention_block()
+    mdl, want, _ = _run_config(spec, 3, 35, round_mode=round_mode)
+    got = mdl.get_tensor(spec.outputs[0])
+    np.testing.assert_array_equal(got, want[spec.outputs[0]])
+    assert want[spec.outputs[0]].min() < want[spec.outputs[0]].max()
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()

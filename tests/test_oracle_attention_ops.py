@@ -1,0 +1,117 @@
+"""Pins the oracle's Softmax (int8 -> float32), QuantizeLinear / DequantizeLinear and activation x activation
+MatMul against library routines and exact arithmetic.  No GPU needed."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+from scipy import special
+
+
+def _rand(rng, shape, dtype=np.int8):
+    info = np.iinfo(dtype)
+    return rng.integers(info.min, info.max + 1, size=shape).astype(dtype)
+
+
+@pytest.mark.parametrize("axis", [-1, 0, 1, 2])
+@pytest.mark.parametrize("in_exp", [-5, -3, 0])
+def test_softmax_is_scipy_softmax_within_float32(oracle, axis, in_exp):
+    """Closed form: the real softmax of the dequantized values.  The reference subtracts no maximum on its
+    int8 path, so at exponent 0 float32 overflows above e^88 and underflows below e^-87; the inputs stay
+    inside that range here."""
+    rng = np.random.default_rng(31)
+    x = _rand(rng, (3, 4, 9, 6))
+    if in_exp == 0:
+        x = np.clip(x, -60, 60).astype(np.int8)
+    got = oracle.softmax_s8(x, axis, in_exp)
+    want = special.softmax(x.astype(np.float64) * 2.0 ** in_exp, axis=axis)
+    assert got.dtype == np.float32 and got.shape == x.shape
+    np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-30)  # float32 underflows below ~1e-38
+    np.testing.assert_allclose(got.sum(axis=axis), 1.0, atol=1e-5)
+
+
+def test_softmax_sums_in_index_order_in_float32(oracle):
+    """The order of the float32 additions is part of the result.  numpy's cumsum adds strictly left to
+    right, so its last element is the reference's row sum; a pairwise or float64 sum differs in the low
+    bits on rows this long.  The table entries come from the C library's expf called directly."""
+    import ctypes
+    import ctypes.util
+    libm = ctypes.CDLL(ctypes.util.find_library("m"))
+    libm.expf.restype = ctypes.c_float
+    libm.expf.argtypes = [ctypes.c_float]
+    scale = np.float32(2.0 ** -3)
+    table = np.array([libm.expf(float(scale * np.float32(q))) for q in range(-128, 128)], dtype=np.float32)
+    rng = np.random.default_rng(32)
+    x = _rand(rng, (64, 400))
+    e = table[x.astype(np.int32) + 128]
+    row_sum = np.cumsum(e, axis=1, dtype=np.float32)[:, -1:]
+    np.testing.assert_array_equal(oracle.softmax_s8(x, -1, -3), e / row_sum)
+    # the check above has teeth: a float64 row sum gives different float32 quotients somewhere
+    assert not np.array_equal(e / e.sum(axis=1, dtype=np.float64, keepdims=True).astype(np.float32), e / row_sum)
+
+
+def test_softmax_axis_views_agree(oracle):
+    """Softmax along a middle axis equals softmax along the last axis of the transposed tensor, bit for bit."""
+    rng = np.random.default_rng(33)
+    x = _rand(rng, (2, 5, 7, 3))
+    a = oracle.softmax_s8(x, 1, -4)
+    b = oracle.softmax_s8(np.ascontiguousarray(np.moveaxis(x, 1, -1)), -1, -4)
+    np.testing.assert_array_equal(a, np.moveaxis(b, -1, 1))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("out_exp", [-9, -7, 0, 2])
+def test_quantize_is_round_half_up_of_the_scaled_value(oracle, dtype, out_exp):
+    rng = np.random.default_rng(34)
+    info = np.iinfo(dtype)
+    scale = 2.0 ** out_exp
+    x = (rng.standard_normal(4000) * info.max * scale * 0.7).astype(np.float32)
+    # exact ties and the saturation edges
+    ties = ((np.arange(-40, 40) + 0.5) * scale).astype(np.float32)
+    edges = np.array([info.max + 0.49, info.max + 0.5, info.min - 0.5, info.min - 0.51, 3e4, -3e4], dtype=np.float64) * scale
+    x = np.concatenate([x, ties, edges.astype(np.float32)])
+    got = oracle.quantize_f32(x, out_exp, dtype)
+    want = [min(max(int(np.floor(Fraction(float(v)) / Fraction(scale) + Fraction(1, 2))), info.min), info.max) for v in x]
+    np.testing.assert_array_equal(got, np.array(want, dtype=dtype))
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+def test_dequantize_is_exact_scaling(oracle, dtype):
+    rng = np.random.default_rng(35)
+    x = _rand(rng, (5, 33), dtype)
+    for e in (-12, -3, 0, 4):
+        np.testing.assert_array_equal(oracle.dequantize_f32(x, e), (x.astype(np.float64) * 2.0 ** e).astype(np.float32))
+
+
+def _shift_round(v, shift, half_even):
+    v = np.asarray(v, dtype=np.int64)
+    if shift <= 0:
+        return v << -shift
+    q, r = v >> shift, v & ((1 << shift) - 1)
+    h = 1 << (shift - 1)
+    up = (r > h) | ((r == h) & ((q & 1) == 1)) if half_even else (r >= h)
+    return q + up
+
+
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+@pytest.mark.parametrize("shapes", [((2, 3, 5, 8), (2, 3, 8, 6)), ((1, 3, 5, 8), (2, 1, 8, 6)), ((4, 5, 16), (4, 16, 3)),
+                                    ((7, 9), (9, 2))], ids=str)
+def test_matmul_is_numpy_matmul_then_shift_round(oracle, shapes, round_mode):
+    rng = np.random.default_rng(36)
+    a, b = _rand(rng, shapes[0]), _rand(rng, shapes[1])
+    exact = a.astype(np.int64) @ b.astype(np.int64)
+    for shift, act in ((7, oracle.LINEAR), (10, oracle.RELU), (1, oracle.LINEAR), (13, oracle.LINEAR)):
+        got = oracle.matmul_s8(a, b, shift, act, round_mode)
+        want = _shift_round(exact, shift, round_mode == 1)
+        if act == oracle.RELU:
+            want = np.maximum(want, 0)
+        np.testing.assert_array_equal(got, np.clip(want, -128, 127).astype(np.int8))
+    assert got.shape == exact.shape
+
+
+def test_matmul_transposed_operand_is_not_confused(oracle):
+    """a x b differs from a x b^T for a square b: guards against reading the second operand [n][k]."""
+    rng = np.random.default_rng(37)
+    a, b = _rand(rng, (6, 6)), _rand(rng, (6, 6))
+    got = oracle.matmul_s8(a, b, 8)
+    np.testing.assert_array_equal(got, np.clip(_shift_round(a.astype(np.int64) @ b.astype(np.int64), 8, False), -128, 127))
+    assert not np.array_equal(got, np.clip(_shift_round(a.astype(np.int64) @ b.T.astype(np.int64), 8, False), -128, 127))
