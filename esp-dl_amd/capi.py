@@ -78,6 +78,8 @@ def lib():
         L.espdl_hip_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp, vp]
         L.espdl_hip_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp, vp]
         L.espdl_hip_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
+        L.espdl_hip_lut_s16.argtypes = [vp, i64, vp, i32, i32, vp, vp]
+        L.espdl_hip_lut_s16.restype = ctypes.c_int
         L.espdl_hip_softmax_s8.argtypes = [vp, i64, i64, i64, i32, vp, vp]
         L.espdl_hip_quantize_f32.argtypes = [vp, i64, i32, i32, vp, vp]
         L.espdl_hip_dequantize_f32.argtypes = [vp, i64, i32, i32, vp, vp]
@@ -427,4 +429,11 @@ def matmul_s8(a, b, shift, activation=0, round_mode=0, stream=None):
     _check(lib().espdl_hip_matmul_s8(_p(a), _p(b), m, k, n, (ctypes.c_int32 * 2)(*lead),
                                      (ctypes.c_int64 * 2)(*strides(la, m * k)), (ctypes.c_int64 * 2)(*strides(lb, k * n)),
                                      shift, activation, round_mode, _p(out), _stream(stream)))
+    return out
+
+
+def lut_s16(x, table, round_mode=0, stream=None):
+    import torch
+    out = torch.empty_like(x)
+    _check(lib().espdl_hip_lut_s16(_p(x), x.numel(), _p(table), table.numel(), round_mode, _p(out), _stream(stream)))
     return out

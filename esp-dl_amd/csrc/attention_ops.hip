@@ -104,6 +104,34 @@ __global__ __launch_bounds__(kThreads) void dequantize_f32_kernel(const T *__res
         out[i] = (float)in[i] * scale;
 }
 
+// base::lut_s16_nearest_neighbor with lut_index (esp-dl/dl/base/dl_base_lut.cpp:49-77).  Tables of up to
+// 8193 entries are copied to LDS once per workgroup; larger ones are read through the caches.
+template <bool LDS_TABLE>
+__global__ __launch_bounds__(kThreads) void lut_s16_kernel(const int16_t *__restrict__ in, long long size,
+                                                           const int16_t *__restrict__ table, int table_size, int shift,
+                                                           int p4_ties, int16_t *__restrict__ out)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int16_t *t = table;
+    if (LDS_TABLE) {
+        int16_t *tl = reinterpret_cast<int16_t *>(smem);
+        for (int i = threadIdx.x; i < table_size; i += kThreads)
+            tl[i] = table[i];
+        __syncthreads();
+        t = tl;
+    }
+    for (long long i = (long long)blockIdx.x * kThreads + threadIdx.x; i < size; i += (long long)gridDim.x * kThreads) {
+        const unsigned value = (unsigned)(unsigned short)in[i] ^ 0x8000u;
+        unsigned index = value >> shift;
+        if (shift > 0) {
+            const unsigned remainder = value & ((1u << shift) - 1u), half = 1u << (shift - 1);
+            if (p4_ties ? (remainder > half || (remainder == half && (index & 1u))) : (remainder >= half))
+                index++;
+        }
+        out[i] = t[index];
+    }
+}
+
 struct MatMulArgs {
     const int8_t *a, *b;
     int8_t *out;
@@ -258,6 +286,19 @@ hipError_t launch_dequantize_f32(const void *in, long long size, int in_exp, int
     else
         dequantize_f32_kernel<int16_t><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(
             static_cast<const int16_t *>(in), size, scale, out);
+    return hipGetLastError();
+}
+
+hipError_t launch_lut_s16(const int16_t *in, long long size, const int16_t *table, int table_size, int shift, bool p4_ties,
+                          int16_t *out, int cu_count, hipStream_t stream)
+{
+    const long long blocks = min((size + kThreads - 1) / kThreads, (long long)cu_count * 8);
+    if (table_size <= 8193)
+        lut_s16_kernel<true><<<dim3((unsigned)blocks), dim3(kThreads), (size_t)table_size * 2, stream>>>(
+            in, size, table, table_size, shift, p4_ties ? 1 : 0, out);
+    else
+        lut_s16_kernel<false><<<dim3((unsigned)blocks), dim3(kThreads), 0, stream>>>(in, size, table, table_size, shift,
+                                                                                      p4_ties ? 1 : 0, out);
     return hipGetLastError();
 }
 

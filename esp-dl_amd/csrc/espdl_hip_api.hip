@@ -731,6 +731,30 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
                          "mbconv_s8_fused");
 }
 
+int espdl_hip_lut_s16(const int16_t *in, int64_t size, const int16_t *table, int32_t table_size, int32_t round_mode,
+                      int16_t *out, void *stream)
+{
+    if (size < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative size");
+    if (round_mode != ESPDL_HIP_ROUND_HALF_UP && round_mode != ESPDL_HIP_ROUND_HALF_EVEN)
+        return fail(ESPDL_HIP_EINVAL, "unknown round mode %d", round_mode);
+    int shift = -1;
+    if (table_size == 65536)
+        shift = 0;
+    for (int s = 0; s <= 15 && shift < 0; s++)
+        if (table_size == (65536 >> s) + 1)
+            shift = s;
+    if (shift < 0)
+        return fail(ESPDL_HIP_EINVAL, "table of %d entries: need 65536 / 2^n + 1 (n = 0..15) or 65536", table_size);
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr || table == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in, table and out must not be NULL");
+    return device_status(espdl::launch_lut_s16(in, size, table, table_size, shift, round_mode == ESPDL_HIP_ROUND_HALF_EVEN,
+                                               out, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                         "lut_s16");
+}
+
 int espdl_hip_softmax_s8(const int8_t *in, int64_t outer, int64_t len, int64_t inner, int32_t in_exp, float *out,
                          void *stream)
 {

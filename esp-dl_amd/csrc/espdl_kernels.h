@@ -132,6 +132,8 @@ hipError_t launch_quantize_f32(const float *in, long long size, int out_exp, int
                                hipStream_t stream);
 hipError_t launch_dequantize_f32(const void *in, long long size, int in_exp, int elem_size, float *out, int cu_count,
                                  hipStream_t stream);
+hipError_t launch_lut_s16(const int16_t *in, long long size, const int16_t *table, int table_size, int shift, bool p4_ties,
+                          int16_t *out, int cu_count, hipStream_t stream);
 hipError_t launch_matmul_s8(const int8_t *a, const int8_t *b, int m, int k, int n, const int lead[2],
                             const long long a_stride[2], const long long b_stride[2], int shift, bool relu, bool half_even,
                             int8_t *out, hipStream_t stream);

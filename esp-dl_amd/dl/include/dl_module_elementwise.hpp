@@ -62,8 +62,12 @@ public:
         (void)mode;
         TensorBase *input = context->get_tensor(m_inputs_index[0]);
         TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (quant_type == QUANT_TYPE_SYMM_16BIT) {
+            forward_s16(context, input, output);
+            return;
+        }
         if (quant_type != QUANT_TYPE_SYMM_8BIT) {
-            DL_LOGE("LUT", "%s: only the 8-bit table is implemented", name.c_str());
+            DL_LOGE("LUT", "%s: only 8-bit and 16-bit tables are implemented", name.c_str());
             return;
         }
         if (!table || table->get_size() != 256 || !on_device_all({input, output})) {
@@ -82,6 +86,30 @@ public:
             DL_LOGE("LUT", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
 
+    /// int16: the table samples the function every 65536 / (entries - 1) input steps and the nearest entry is
+    /// taken (esp-dl/dl/module/include/dl_module_lut.hpp:61-74); the ESP32-P4 tie rule goes with the
+    /// context's half-even mode.
+    void forward_s16(ModelContext *context, TensorBase *input, TensorBase *output)
+    {
+        if (!table || table->dtype != DATA_TYPE_INT16 || !on_device_all({input, output}) ||
+            input->dtype != DATA_TYPE_INT16 || output->dtype != DATA_TYPE_INT16) {
+            DL_LOGE("LUT", "%s: the 16-bit form needs an int16 table and int16 device tensors", name.c_str());
+            return;
+        }
+        if (!table->on_device()) {
+            TensorBase *dev = table->to_device(context->stream);
+            delete table;
+            table = dev;
+        }
+        const int rc = espdl_hip_lut_s16(static_cast<const int16_t *>(input->data), input->get_size(),
+                                         static_cast<const int16_t *>(table->data), table->get_size(),
+                                         context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN
+                                                                                     : ESPDL_HIP_ROUND_HALF_UP,
+                                         static_cast<int16_t *>(output->data), context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("LUT", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+
     static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
     {
         quant_type_t quant_type = QUANT_TYPE_NONE;
@@ -91,9 +119,9 @@ public:
             DL_LOGE("LUT", "Table is null!");
             return nullptr;
         }
-        if (quant_type == QUANT_TYPE_SYMM_8BIT)
+        if (quant_type == QUANT_TYPE_SYMM_8BIT || (quant_type == QUANT_TYPE_SYMM_16BIT && table->dtype == DATA_TYPE_INT16))
             return new LUT(node_name.c_str(), table, MODULE_INPLACE_CHANGED_BUFFER, quant_type);
-        DL_LOGE("LUT", "Only QUANT_TYPE_SYMM_8BIT tables are implemented");
+        DL_LOGE("LUT", "Only 8-bit tables and int16 tables of 16-bit nodes are implemented");
         delete table;
         return nullptr;
     }
@@ -104,9 +132,13 @@ public:
 /// Shared by every activation op: a node with a `lut` attribute becomes a LUT module.
 inline Module *lut_if_present(fbs::FbsModel *fbs_model, const std::string &node_name, quant_type_t quant_type)
 {
-    if (quant_type != QUANT_TYPE_SYMM_8BIT)
+    if (quant_type != QUANT_TYPE_SYMM_8BIT && quant_type != QUANT_TYPE_SYMM_16BIT)
         return nullptr;
     TensorBase *table = fbs_model->get_operation_lut(node_name);
+    if (table && quant_type == QUANT_TYPE_SYMM_16BIT && table->dtype != DATA_TYPE_INT16) {
+        delete table;
+        return nullptr;
+    }
     return table ? new LUT(node_name.c_str(), table, MODULE_INPLACE_CHANGED_BUFFER, quant_type) : nullptr;
 }
 

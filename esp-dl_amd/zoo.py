@@ -188,6 +188,22 @@ class Builder:
         g.add_node(name, op_type, [x], [y], lut=name + ".lut", quant_type="S8")
         return y
 
+    def lut_s16(self, x, fn, points=2048, op_type="LUT", out_exp=None, name=None):
+        """16-bit table activation: `points` + 1 samples of fn, one every 65536 / points input steps;
+        the operator takes the nearest sample."""
+        g = self.g
+        name = name or self._name(op_type.lower())
+        in_exp = g.exponent(x)
+        out_exp = in_exp if out_exp is None else out_exp
+        step = 65536 // points
+        q = (np.arange(points + 1, dtype=np.int64) * step - 32768).astype(np.float64)
+        table = np.clip(np.floor(fn(q * 2.0 ** in_exp) / 2.0 ** out_exp + 0.5), -32768, 32767).astype(np.int16)
+        g.add_init(name + ".lut", [points + 1], INT16, table, [out_exp])
+        y = name + "_out"
+        g.add_value(y, g.shape(x), out_exp, INT16)
+        g.add_node(name, op_type, [x], [y], lut=name + ".lut", quant_type="S16")
+        return y
+
     def clip(self, x, lo_q, hi_q, out_exp=None, name=None):
         g = self.g
         name = name or self._name("clip")
@@ -562,13 +578,14 @@ def config4_yolo_style(seed=0xE5D4, resolution=640):
     up = b.resize_nearest(p4, 2, name="up4")
     p3 = c3k2_like(b, b.concat([up, p3], name="fpn3_join"), 64, "fpn3")
     # detection head per scale: int8 3x3 conv + SiLU, then int16 box branch (requantize to int16,
-    # int16 3x3 conv, int16 1x1 conv) and an int8 class branch
+    # int16 3x3 conv, SiLU through a 2049-entry int16 table, int16 1x1 conv) and an int8 class branch
     for i, (p, c) in enumerate(((p3, 64), (p4, 64), (p5, 64))):
         h = cbs(p, c, 3, 1, "head%d_cv" % i)
         h16 = "head%d_s16_in" % i
         g.add_value(h16, g.shape(h), g.exponent(h) - 8, INT16)
         g.add_node("head%d_to_s16" % i, "RequantizeLinear", [h], [h16], quant_type="S16")
         box = b.conv(h16, c, k=3, s16=True, name="head%d_box1" % i)
+        box = b.lut_s16(box, silu, name="head%d_box1_silu" % i)
         box = b.conv(box, 64, k=1, s16=True, name="head%d_box2" % i)
         b.output(box)
         cls = cbs(h, 80, 1, 1, "head%d_cls1" % i)

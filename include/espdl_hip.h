@@ -206,6 +206,14 @@ int espdl_hip_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w,
 int espdl_hip_reduce_mean_s8(const int8_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
                              int32_t in_exp, int32_t out_exp, int8_t *out, void *stream);
 
+/* module::LUT for int16 (esp-dl/dl/module/include/dl_module_lut.hpp:61-74; base::lut_s16_nearest_neighbor and
+ * lut_index, esp-dl/dl/base/dl_base_lut.cpp:49-77): `table` (device) holds table_size = 65536 / step + 1
+ * entries, step a power of two, or 65536 entries; out = table[round((in + 32768) / step)].  Ties go up with
+ * ESPDL_HIP_ROUND_HALF_UP (portable C path) and to the even index with ESPDL_HIP_ROUND_HALF_EVEN (the
+ * ESP32-P4 build). */
+int espdl_hip_lut_s16(const int16_t *in, int64_t size, const int16_t *table, int32_t table_size, int32_t round_mode,
+                      int16_t *out, void *stream);
+
 /* module::Softmax on an int8 tensor (Softmax::forward_lut, esp-dl/dl/module/include/dl_module_softmax.hpp:148-217):
  * the tensor is viewed as [outer][len][inner] and normalized along len; out is float32 of the same
  * layout, out = T[q] / sum_i T[q_i] with T[q] = expf(2^in_exp * q), the sum taken in float32 in index

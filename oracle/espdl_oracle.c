@@ -677,6 +677,40 @@ void espdl_oracle_dequantize_f32(const void *in, int64_t size, int in_exp, int e
         out[i] = (elem_size == 1 ? (float)((const int8_t *)in)[i] : (float)((const int16_t *)in)[i]) * scale;
 }
 
+/*
+ * LUT on int16 (LUT::forward, esp-dl/dl/module/include/dl_module_lut.hpp:61-74, with
+ * base::lut_s16_nearest_neighbor and lut_index, esp-dl/dl/base/dl_base_lut.cpp:49-77): the table holds
+ * table_size = 65536 / step + 1 entries (step a power of two), or 65536 entries for step 1.  The input is
+ * biased to 0..65535, divided by step and rounded to the nearest entry: ties go up on the portable C path
+ * and to the even index when p4_ties is set (the ESP32-P4 build).
+ */
+int espdl_oracle_lut_s16(const int16_t *in, int64_t size, const int16_t *table, int table_size, int p4_ties,
+                         int16_t *out)
+{
+    if (table_size < 2)
+        return -1;
+    const int step = 65536 / (table_size - 1);
+    if (step < 1 || (step & (step - 1)) != 0)
+        return -1;
+    if (step == 1) {
+        for (int64_t i = 0; i < size; i++)
+            out[i] = table[(int)in[i] + 32768];
+        return 0;
+    }
+    int shift = 0;
+    while ((1 << shift) < step)
+        shift++;
+    for (int64_t i = 0; i < size; i++) {
+        const uint32_t value = (uint32_t)(uint16_t)in[i] ^ 0x8000u;
+        uint32_t index = value >> shift;
+        const uint32_t remainder = value & ((1u << shift) - 1u), half = 1u << (shift - 1);
+        if (p4_ties ? (remainder > half || (remainder == half && (index & 1u))) : (remainder >= half))
+            index++;
+        out[i] = table[index];
+    }
+    return 0;
+}
+
 /* ---------------------------------------------------------------------------------------------
  * Data-movement operators of the detection necks (Concat, Split, Transpose, Resize, MaxPool).
  * ------------------------------------------------------------------------------------------- */

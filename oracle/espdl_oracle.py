@@ -62,6 +62,8 @@ def lib():
         L.espdl_oracle_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp]
         L.espdl_oracle_reduce_mean_s8.restype = i32
         L.espdl_oracle_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp]
+        L.espdl_oracle_lut_s16.restype = i32
+        L.espdl_oracle_lut_s16.argtypes = [vp, i64, vp, i32, i32, vp]
         L.espdl_oracle_softmax_s8.restype = None
         L.espdl_oracle_softmax_s8.argtypes = [vp, i64, i64, i64, i32, vp]
         L.espdl_oracle_quantize_f32.restype = None
@@ -224,6 +226,15 @@ def lut_s8(x, table):
     assert table.size == 256
     out = np.empty_like(x)
     lib().espdl_oracle_lut_s8(_ptr(x), x.size, _ptr(table), _ptr(out))
+    return out
+
+
+def lut_s16(x, table, p4_ties=False):
+    x = _c(x, np.int16)
+    table = _c(table, np.int16)
+    out = np.empty_like(x)
+    rc = lib().espdl_oracle_lut_s16(_ptr(x), x.size, _ptr(table), table.size, 1 if p4_ties else 0, _ptr(out))
+    assert rc == 0, "table size must be 65536 / 2^n + 1 (or 65536)"
     return out
 
 

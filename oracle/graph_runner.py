@@ -74,9 +74,10 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             act = oracle.RELU if a.get("activation", "Linear") == "Relu" else oracle.LINEAR
             y = oracle.gemm_s8(x, w, bias, shift, activation=act, round_mode=round_mode)
         elif "lut" in a:
-            if x.dtype != np.int8 or spec.initializers[a["lut"]][2].size != 256:
-                raise NotImplementedError("16-bit LUT")
-            y = oracle.lut_s8(x, spec.initializers[a["lut"]][2])
+            if x.dtype == np.int16:
+                y = oracle.lut_s16(x, spec.initializers[a["lut"]][2], p4_ties=(round_mode == oracle.ROUND_HALF_EVEN))
+            else:
+                y = oracle.lut_s8(x, spec.initializers[a["lut"]][2])
         elif op == "Relu":
             y = oracle.relu_s8(x, spec.exponent(ins[0]), spec.exponent(y_name))
         elif op == "PRelu":

@@ -136,3 +136,23 @@ def test_matmul_rejects_bad_arguments():
     lead = (ctypes.c_int32 * 2)(1, 1)
     assert m.lib().espdl_hip_matmul_s8(a.data_ptr(), a.data_ptr(), 2, 4, 2, lead, z, z, 7, 5, 0, a.data_ptr(), None) != 0
     assert m.lib().espdl_hip_matmul_s8(a.data_ptr(), None, 2, 4, 2, lead, z, z, 7, 0, 0, a.data_ptr(), None) != 0
+
+
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["ties_up", "ties_even"])
+@pytest.mark.parametrize("entries", [65536, 65537, 32769, 2049, 257, 3])
+def test_lut_s16(oracle, entries, round_mode):
+    announce(f"lut_s16 entries={entries} round_mode={round_mode}")
+    rng = np.random.default_rng(46)
+    table = _rand(rng, (entries,), np.int16)
+    x = np.concatenate([np.arange(-32768, 32768, dtype=np.int16), _rand(rng, (100003,), np.int16)])
+    got = to_host(espdl().lut_s16(to_dev(x), to_dev(table), round_mode))
+    np.testing.assert_array_equal(got, oracle.lut_s16(x, table, round_mode == 1))
+
+
+def test_lut_s16_rejects_odd_table_sizes():
+    announce("lut_s16 argument checks")
+    import torch
+    m = espdl()
+    x = torch.zeros(8, dtype=torch.int16, device="cuda")
+    with pytest.raises(m.EspdlHipError):
+        m.lut_s16(x, torch.zeros(1000, dtype=torch.int16, device="cuda"))

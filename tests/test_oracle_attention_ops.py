@@ -115,3 +115,27 @@ def test_matmul_transposed_operand_is_not_confused(oracle):
     got = oracle.matmul_s8(a, b, 8)
     np.testing.assert_array_equal(got, np.clip(_shift_round(a.astype(np.int64) @ b.astype(np.int64), 8, False), -128, 127))
     assert not np.array_equal(got, np.clip(_shift_round(a.astype(np.int64) @ b.T.astype(np.int64), 8, False), -128, 127))
+
+
+@pytest.mark.parametrize("p4_ties", [False, True], ids=["ties_up", "ties_even"])
+@pytest.mark.parametrize("entries", [65536, 65537, 2049, 257, 3])
+def test_lut_s16_takes_the_nearest_sample(oracle, entries, p4_ties):
+    """All 65536 inputs against exact rational arithmetic: index = round((x + 32768) / step)."""
+    rng = np.random.default_rng(38)
+    table = _rand(rng, (entries,), np.int16)
+    x = np.arange(-32768, 32768, dtype=np.int16)
+    step = 65536 // (entries - 1)
+    want = np.empty(65536, dtype=np.int16)
+    for i, v in enumerate(range(65536)):
+        q = Fraction(v, step)
+        idx = int(np.floor(q))
+        frac = q - idx
+        if frac > Fraction(1, 2) or (frac == Fraction(1, 2) and (idx % 2 == 1 if p4_ties else True)):
+            idx += 1
+        want[i] = table[idx]
+    np.testing.assert_array_equal(oracle.lut_s16(x, table, p4_ties), want)
+
+
+def test_lut_s16_rejects_odd_table_sizes(oracle):
+    with pytest.raises(AssertionError):
+        oracle.lut_s16(np.zeros(4, dtype=np.int16), np.zeros(1000, dtype=np.int16))
