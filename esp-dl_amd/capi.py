@@ -78,6 +78,8 @@ def lib():
         L.espdl_hip_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp, vp]
         L.espdl_hip_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp, vp]
         L.espdl_hip_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
+        L.espdl_hip_insert_zeros.argtypes = [vp] + [i32] * 9 + [vp, vp]
+        L.espdl_hip_insert_zeros.restype = ctypes.c_int
         L.espdl_hip_lut_s16.argtypes = [vp, i64, vp, i32, i32, vp, vp]
         L.espdl_hip_lut_s16.restype = ctypes.c_int
         L.espdl_hip_softmax_s8.argtypes = [vp, i64, i64, i64, i32, vp, vp]
@@ -436,4 +438,18 @@ def lut_s16(x, table, round_mode=0, stream=None):
     import torch
     out = torch.empty_like(x)
     _check(lib().espdl_hip_lut_s16(_p(x), x.numel(), _p(table), table.numel(), round_mode, _p(out), _stream(stream)))
+    return out
+
+
+def insert_zeros(x, stride, output_padding=(0, 0), stream=None):
+    """x [N, H, W, C] (or [N, L, C]) -> zeros with x at every stride-th position (espdl_hip_insert_zeros)."""
+    import torch
+    one_d = x.dim() == 3
+    n, h, w, c = (int(x.shape[0]), int(x.shape[1]), 1, int(x.shape[2])) if one_d else [int(d) for d in x.shape]
+    sh, sw = (stride[0], 1) if one_d else stride
+    ph, pw = (output_padding[0], 0) if one_d else output_padding
+    oh = max(0, h + (sh - 1) * (h - 1) + ph) if h else 0
+    ow = max(0, w + (sw - 1) * (w - 1) + pw) if w else 0
+    out = torch.empty([n, oh, c] if one_d else [n, oh, ow, c], dtype=x.dtype, device=x.device)
+    _check(lib().espdl_hip_insert_zeros(_p(x), x.element_size(), n, h, w, c, sh, sw, ph, pw, _p(out), _stream(stream)))
     return out

@@ -731,6 +731,30 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
                          "mbconv_s8_fused");
 }
 
+int espdl_hip_insert_zeros(const void *in, int32_t elem_size, int32_t batch, int32_t h, int32_t w, int32_t c,
+                           int32_t stride_h, int32_t stride_w, int32_t output_padding_h, int32_t output_padding_w,
+                           void *out, void *stream)
+{
+    if (elem_size != 1 && elem_size != 2 && elem_size != 4)
+        return fail(ESPDL_HIP_EINVAL, "elem_size must be 1, 2 or 4");
+    if (batch < 0 || h < 0 || w < 0 || c < 0)
+        return fail(ESPDL_HIP_EINVAL, "negative extent");
+    if (stride_h < 1 || stride_w < 1 || output_padding_h < 0 || output_padding_w < 0)
+        return fail(ESPDL_HIP_EINVAL, "strides must be >= 1 and output paddings >= 0");
+    if (batch == 0 || h == 0 || w == 0 || c == 0)
+        return ESPDL_HIP_OK;
+    const long long out_h = h + (long long)(stride_h - 1) * (h - 1) + output_padding_h;
+    const long long out_w = w + (long long)(stride_w - 1) * (w - 1) + output_padding_w;
+    if (out_h > 0x7fffffffll || out_w > 0x7fffffffll || (long long)batch * out_h > 0x7fffffffll / out_w ||
+        (long long)batch * out_h * out_w > 0x7fffffffll / ((long long)c * elem_size))
+        return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_insert_zeros(in, elem_size, batch, h, w, c, stride_h, stride_w, (int)out_h, (int)out_w,
+                                                    out, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                         "insert_zeros");
+}
+
 int espdl_hip_lut_s16(const int16_t *in, int64_t size, const int16_t *table, int32_t table_size, int32_t round_mode,
                       int16_t *out, void *stream)
 {

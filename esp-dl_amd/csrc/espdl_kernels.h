@@ -125,6 +125,9 @@ hipError_t launch_slice(const void *in, const int *shape, int dims, const int *s
 hipError_t launch_reduce_mean_s8(const int8_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
                                  int out_exp, int8_t *out, int cu_count, hipStream_t stream);
 
+hipError_t launch_insert_zeros(const void *in, int elem_size, int batch, int h, int w, int c, int stride_h, int stride_w,
+                               int out_h, int out_w, void *out, int cu_count, hipStream_t stream);
+
 // attention_ops.hip
 hipError_t launch_softmax_s8(const int8_t *in, long long outer, long long len, long long inner, int in_exp, float *out,
                              int cu_count, hipStream_t stream);

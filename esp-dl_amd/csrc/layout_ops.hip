@@ -214,6 +214,40 @@ __global__ __launch_bounds__(kBlock) void resize_nearest_s8_kernel(const ResizeA
     }
 }
 
+struct InsertZerosArgs {
+    const char *in;
+    char *out;
+    int h, w, out_h, out_w, stride_h, stride_w;
+    int pixel_bytes, vec; // bytes per pixel (channels * element size) and bytes per lane (16, 4 or 1)
+    long long total;
+    FastDiv fd_cv, fd_ow, fd_oh;
+};
+
+// InsertZeros::forward_template (esp-dl/dl/module/include/dl_module_insert_zeros.hpp): input pixel (h, w)
+// lands on output pixel (h * stride_h, w * stride_w); every other output pixel is zero.  Written as a
+// gather over the output so that each byte is stored once.
+__global__ __launch_bounds__(kBlock) void insert_zeros_kernel(const InsertZerosArgs a)
+{
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < a.total; i += (long long)gridDim.x * kBlock) {
+        const unsigned pix = fastdiv((unsigned)i, a.fd_cv);
+        const unsigned v = (unsigned)i - pix * a.fd_cv.d;
+        const unsigned row = fastdiv(pix, a.fd_ow);
+        const unsigned x = pix - row * a.fd_ow.d;
+        const unsigned n = fastdiv(row, a.fd_oh);
+        const unsigned y = row - n * a.fd_oh.d;
+        const unsigned iy = y / (unsigned)a.stride_h, ix = x / (unsigned)a.stride_w;
+        const bool hit = iy * a.stride_h == y && ix * a.stride_w == x && iy < (unsigned)a.h && ix < (unsigned)a.w;
+        const long long src = (((long long)n * a.h + iy) * a.w + ix) * a.pixel_bytes + (long long)v * a.vec;
+        const long long dst = (long long)pix * a.pixel_bytes + (long long)v * a.vec;
+        if (a.vec == 16)
+            *reinterpret_cast<v4i *>(a.out + dst) = hit ? *reinterpret_cast<const v4i *>(a.in + src) : v4i{0, 0, 0, 0};
+        else if (a.vec == 4)
+            *reinterpret_cast<int *>(a.out + dst) = hit ? *reinterpret_cast<const int *>(a.in + src) : 0;
+        else
+            a.out[dst] = hit ? a.in[src] : (char)0;
+    }
+}
+
 struct PoolArgs {
     const char *in;
     char *out;
@@ -545,6 +579,34 @@ hipError_t launch_resize_nearest_s8(const int8_t *in, int batch, int h, int w, i
     a.fd_ow = make_fastdiv((unsigned)out_w);
     a.fd_oh = make_fastdiv((unsigned)out_h);
     hipLaunchKernelGGL(resize_nearest_s8_kernel, dim3(blocks_for(a.total, cu_count)), dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launch_insert_zeros(const void *in, int elem_size, int batch, int h, int w, int c, int stride_h, int stride_w,
+                               int out_h, int out_w, void *out, int cu_count, hipStream_t stream)
+{
+    InsertZerosArgs a;
+    a.in = static_cast<const char *>(in);
+    a.out = static_cast<char *>(out);
+    a.h = h;
+    a.w = w;
+    a.out_h = out_h;
+    a.out_w = out_w;
+    a.stride_h = stride_h;
+    a.stride_w = stride_w;
+    a.pixel_bytes = c * elem_size;
+    const uintptr_t align = reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out);
+    a.vec = (a.pixel_bytes % 16 == 0 && (align & 15) == 0) ? 16 : ((a.pixel_bytes % 4 == 0 && (align & 3) == 0) ? 4 : 1);
+    const int cv = a.pixel_bytes / a.vec;
+    a.total = (long long)batch * out_h * out_w * cv;
+    if (a.total <= 0)
+        return hipSuccess;
+    if (a.total > 0x7fffffffll) // fastdiv range
+        return hipErrorInvalidValue;
+    a.fd_cv = make_fastdiv((unsigned)cv);
+    a.fd_ow = make_fastdiv((unsigned)out_w);
+    a.fd_oh = make_fastdiv((unsigned)out_h);
+    hipLaunchKernelGGL(insert_zeros_kernel, dim3(blocks_for(a.total, cu_count)), dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 

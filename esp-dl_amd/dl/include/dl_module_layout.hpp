@@ -649,6 +649,76 @@ public:
     void print() { DL_LOGI("ReduceMean", "keepdims: %d, quant_type: %s.", m_keepdims, quant_type_to_string(quant_type)); }
 };
 
+/// InsertZeros on [N, spatial..., C] tensors with one or two spatial dims
+/// (esp-dl/dl/module/include/dl_module_insert_zeros.hpp): the exporter writes a transposed convolution as
+/// InsertZeros followed by an ordinary Conv.
+class InsertZeros : public Module {
+private:
+    std::vector<int> m_stride, m_output_padding;
+
+    void normalize(size_t spatial)
+    {
+        if (m_stride.size() == 1 && spatial > 1)
+            m_stride.assign(spatial, m_stride[0]);
+        if (m_output_padding.size() == 1 && spatial > 1)
+            m_output_padding.assign(spatial, m_output_padding[0]);
+    }
+
+public:
+    InsertZeros(const char *name = nullptr, const std::vector<int> &stride = {1}, const std::vector<int> &output_padding = {0},
+                quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_stride(stride), m_output_padding(output_padding)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        if (in.size() != 3 && in.size() != 4)
+            return {{}};
+        const size_t spatial = in.size() - 2;
+        normalize(spatial);
+        if (m_stride.size() != spatial || m_output_padding.size() != spatial)
+            return {{}};
+        std::vector<int> out = in;
+        for (size_t i = 0; i < spatial; i++)
+            out[1 + i] = in[1 + i] + (m_stride[i] - 1) * (in[1 + i] - 1) + m_output_padding[i];
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) || (input->shape.size() != 3 && input->shape.size() != 4) ||
+            input->dtype != output->dtype) {
+            DL_LOGE("InsertZeros", "%s: needs device tensors of rank 3 or 4 and one dtype", name.c_str());
+            return;
+        }
+        const bool one_d = input->shape.size() == 3;
+        normalize(input->shape.size() - 2);
+        const int rc = espdl_hip_insert_zeros(input->data, (int32_t)input->get_dtype_bytes(), input->shape[0], input->shape[1],
+                                              one_d ? 1 : input->shape[2], input->shape.back(), m_stride[0],
+                                              one_d ? 1 : m_stride[1], m_output_padding[0],
+                                              one_d ? 0 : m_output_padding[1], output->data, context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("InsertZeros", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        std::vector<int> stride = {1}, output_padding = {0};
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "stride", stride);
+        fbs_model->get_operation_attribute(node_name, "output_padding", output_padding);
+        if (stride.empty())
+            stride = {1};
+        if (output_padding.empty())
+            output_padding = {0};
+        return new InsertZeros(node_name.c_str(), stride, output_padding, quant_type);
+    }
+    void print() { DL_LOGI("InsertZeros", "stride: %s, quant_type: %s.", vector_to_string(m_stride).c_str(), quant_type_to_string(quant_type)); }
+};
+
 /// Softmax on an int8 tensor with a float32 result (esp-dl/dl/module/include/dl_module_softmax.hpp,
 /// forward_lut): the exported graphs follow it with QuantizeLinear.
 class Softmax : public Module {

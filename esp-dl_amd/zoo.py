@@ -330,6 +330,16 @@ class Builder:
         g.add_node(name, "Reshape", [x, name + ".shape"], [y], allowzero=0, quant_type="S8")
         return y
 
+    def insert_zeros(self, x, stride=2, name=None):
+        """The zero-stuffing half of a transposed convolution; a Conv follows."""
+        g = self.g
+        name = name or self._name("insert_zeros")
+        _, h, w, c = g.shape(x)
+        y = name + "_out"
+        g.add_value(y, [1, h + (stride - 1) * (h - 1), w + (stride - 1) * (w - 1), c], g.exponent(x), g.dtype(x))
+        g.add_node(name, "InsertZeros", [x], [y], stride=[stride, stride], output_padding=[0, 0], quant_type="S8")
+        return y
+
     def softmax(self, x, axis=-1, name=None):
         """Softmax with a float32 result, as the exporter leaves it (QuantizeLinear follows)."""
         g = self.g
@@ -653,6 +663,9 @@ def gated_block(seed=0xE5D6):
     y = b.conv(h, 32, k=1, name="c2")
     y = b.add(x, y, name="res")
     b.output(y)
+    # transposed convolution as exported: InsertZeros, then a Conv whose padding restores 2x the size
+    up = b.conv(b.insert_zeros(h, 2, name="up_zeros"), 16, k=2, pad=(1, 1, 1, 1), name="up_conv")
+    b.output(up)
     # detection-style score head: two single-channel Conv -> Sigmoid branches multiplied together (each
     # Conv's only reader is its LUT, and each LUT's only reader is the Mul)
     sig = lambda v: 1.0 / (1.0 + np.exp(-v))

@@ -206,6 +206,14 @@ int espdl_hip_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w,
 int espdl_hip_reduce_mean_s8(const int8_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
                              int32_t in_exp, int32_t out_exp, int8_t *out, void *stream);
 
+/* module::InsertZeros (esp-dl/dl/module/include/dl_module_insert_zeros.hpp; the exporter places it in front of
+ * a Conv to express a transposed convolution): in is [batch][h][w][c] of elem_size-byte elements, out is
+ * [batch][out_h][out_w][c] with out_h = h + (stride_h - 1) * (h - 1) + output_padding_h (same for w);
+ * out[n][y * stride_h][x * stride_w] = in[n][y][x], every other element 0.  1-D tensors pass w = 1. */
+int espdl_hip_insert_zeros(const void *in, int32_t elem_size, int32_t batch, int32_t h, int32_t w, int32_t c,
+                           int32_t stride_h, int32_t stride_w, int32_t output_padding_h, int32_t output_padding_w,
+                           void *out, void *stream);
+
 /* module::LUT for int16 (esp-dl/dl/module/include/dl_module_lut.hpp:61-74; base::lut_s16_nearest_neighbor and
  * lut_index, esp-dl/dl/base/dl_base_lut.cpp:49-77): `table` (device) holds table_size = 65536 / step + 1
  * entries, step a power of two, or 65536 entries; out = table[round((in + 32768) / step)].  Ties go up with

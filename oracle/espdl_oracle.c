@@ -678,6 +678,22 @@ void espdl_oracle_dequantize_f32(const void *in, int64_t size, int in_exp, int e
 }
 
 /*
+ * InsertZeros::forward_template (esp-dl/dl/module/include/dl_module_insert_zeros.hpp): the output is cleared,
+ * then input pixel (h, w) is copied to output pixel (h * stride_h, w * stride_w).
+ */
+void espdl_oracle_insert_zeros(const void *in, int elem_size, int batch, int h, int w, int c, int stride_h, int stride_w,
+                               int out_h, int out_w, void *out)
+{
+    const size_t px = (size_t)c * (size_t)elem_size;
+    memset(out, 0, (size_t)batch * out_h * out_w * px);
+    for (int n = 0; n < batch; n++)
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++)
+                memcpy((char *)out + (((size_t)n * out_h + (size_t)y * stride_h) * out_w + (size_t)x * stride_w) * px,
+                       (const char *)in + (((size_t)n * h + y) * w + x) * px, px);
+}
+
+/*
  * LUT on int16 (LUT::forward, esp-dl/dl/module/include/dl_module_lut.hpp:61-74, with
  * base::lut_s16_nearest_neighbor and lut_index, esp-dl/dl/base/dl_base_lut.cpp:49-77): the table holds
  * table_size = 65536 / step + 1 entries (step a power of two), or 65536 entries for step 1.  The input is

@@ -122,6 +122,8 @@ int espdl_oracle_reduce_mean_s8(const int8_t *in, const int *shape, int dims, co
 int espdl_oracle_slice(const void *in, const int *shape, int dims, const int *start, const int *step,
                        const int *out_shape, int elem_size, void *out);
 void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out);
+void espdl_oracle_insert_zeros(const void *in, int elem_size, int batch, int h, int w, int c, int stride_h, int stride_w,
+                               int out_h, int out_w, void *out);
 int espdl_oracle_lut_s16(const int16_t *in, int64_t size, const int16_t *table, int table_size, int p4_ties,
                          int16_t *out);
 void espdl_oracle_softmax_s8(const int8_t *in, int64_t outer, int64_t len, int64_t inner, int in_exp, float *out);

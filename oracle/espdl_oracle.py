@@ -62,6 +62,8 @@ def lib():
         L.espdl_oracle_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp]
         L.espdl_oracle_reduce_mean_s8.restype = i32
         L.espdl_oracle_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp]
+        L.espdl_oracle_insert_zeros.restype = None
+        L.espdl_oracle_insert_zeros.argtypes = [vp] + [i32] * 9 + [vp]
         L.espdl_oracle_lut_s16.restype = i32
         L.espdl_oracle_lut_s16.argtypes = [vp, i64, vp, i32, i32, vp]
         L.espdl_oracle_softmax_s8.restype = None
@@ -226,6 +228,16 @@ def lut_s8(x, table):
     assert table.size == 256
     out = np.empty_like(x)
     lib().espdl_oracle_lut_s8(_ptr(x), x.size, _ptr(table), _ptr(out))
+    return out
+
+
+def insert_zeros(x, stride, output_padding=(0, 0)):
+    x = np.ascontiguousarray(x)
+    n, h, w, c = x.shape
+    oh = h + (stride[0] - 1) * (h - 1) + output_padding[0]
+    ow = w + (stride[1] - 1) * (w - 1) + output_padding[1]
+    out = np.empty((n, oh, ow, c), dtype=x.dtype)
+    lib().espdl_oracle_insert_zeros(_ptr(x), x.itemsize, n, h, w, c, stride[0], stride[1], oh, ow, _ptr(out))
     return out
 
 

@@ -151,6 +151,14 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
         elif op == "Resize":
             scales = spec.initializers[ins[2]][2].ravel()
             y = oracle.resize_nearest_s8(x, scales[2], scales[3], spec.exponent(ins[0]), spec.exponent(y_name))
+        elif op == "InsertZeros":
+            st, op_pad = list(a["stride"]), list(a.get("output_padding") or [0])
+            if x.ndim == 3:
+                y = oracle.insert_zeros(x[:, :, None], (st[0], 1), (op_pad[0], 0))[:, :, 0]
+            else:
+                st = st * 2 if len(st) == 1 else st
+                op_pad = op_pad * 2 if len(op_pad) == 1 else op_pad
+                y = oracle.insert_zeros(x, st, op_pad)
         elif op == "Transpose":
             y = oracle.transpose(x, list(a["perm"]))
         else:

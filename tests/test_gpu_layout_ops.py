@@ -153,3 +153,31 @@ def test_bad_layout_arguments_are_rejected():
         m.max_pool(x, (7, 7))
     with pytest.raises(m.EspdlHipError):
         m.resize_nearest_s8(x, 0.0, 2.0, out_hw=(4, 8))
+
+
+INSERT_ZEROS_CASES = [
+    # (shape, stride, output_padding)
+    ((2, 80, 80, 64), (2, 2), (0, 0)),     # the mask branch of the exported segmentation graphs
+    ((1, 23, 17, 16), (2, 2), (0, 0)),
+    ((3, 5, 4, 3), (3, 1), (1, 0)),        # byte path, mixed strides, output padding
+    ((2, 7, 9, 6), (2, 4), (1, 3)),        # 4-byte path for int16
+    ((2, 6, 6, 8), (1, 1), (0, 0)),        # stride 1: a copy
+    ((0, 4, 4, 16), (2, 2), (0, 0)),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("case", INSERT_ZEROS_CASES, ids=lambda c: f"{c[0]}_s{c[1]}_p{c[2]}")
+def test_insert_zeros(oracle, case, dtype):
+    shape, stride, pad = case
+    announce(f"insert_zeros {case} {dtype.__name__}")
+    x = _rand(np.random.default_rng(29), shape, dtype)
+    got = to_host(espdl().insert_zeros(to_dev(x), stride, pad))
+    np.testing.assert_array_equal(got, oracle.insert_zeros(x, stride, pad))
+
+
+def test_insert_zeros_one_spatial_dim(oracle):
+    announce("insert_zeros NWC")
+    x = _rand(np.random.default_rng(30), (3, 11, 5))
+    got = to_host(espdl().insert_zeros(to_dev(x), (3,), (2,)))
+    np.testing.assert_array_equal(got, oracle.insert_zeros(x[:, :, None], (3, 1), (2, 0))[:, :, 0])

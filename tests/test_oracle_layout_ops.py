@@ -185,3 +185,19 @@ def test_reduce_mean_matches_exact_mean_away_from_ties(oracle, shape, axes, keep
         assert int(g) == min(127, max(-128, (exact + Fraction(1, 2)).__floor__()))
         checked += 1
     assert checked > 0
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("stride,pad", [((2, 2), (0, 0)), ((3, 1), (1, 0)), ((1, 1), (0, 2)), ((2, 4), (1, 3))])
+def test_insert_zeros_is_strided_assignment(oracle, dtype, stride, pad):
+    """numpy statement of the operator: zeros, then out[:, ::sh, ::sw] = x; equivalently the adjoint of a
+    strided slice, which is how a transposed convolution's input is prepared."""
+    rng = np.random.default_rng(39)
+    x = _rand(rng, (2, 5, 4, 3), dtype)
+    got = oracle.insert_zeros(x, stride, pad)
+    oh = 5 + (stride[0] - 1) * 4 + pad[0]
+    ow = 4 + (stride[1] - 1) * 3 + pad[1]
+    want = np.zeros((2, oh, ow, 3), dtype=dtype)
+    want[:, :(5 - 1) * stride[0] + 1:stride[0], :(4 - 1) * stride[1] + 1:stride[1]] = x
+    np.testing.assert_array_equal(got, want)
+    np.testing.assert_array_equal(got[:, ::stride[0], ::stride[1]][:, :5, :4], x)
