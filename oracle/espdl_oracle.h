@@ -49,6 +49,21 @@
  *   espdl_oracle_reduce_mean_s8  float32 as the two above: exact rational mean, round half up, away from ties
  *                                                                                   PARITY UNPINNED (near-ties)
  *   espdl_oracle_slice           equality with numpy basic slicing                                   PINNED
+ *   espdl_oracle_softmax_s8      float32: within 2e-6 relative of scipy.special.softmax of the dequantized values;
+ *                                the order-sensitive part (the float32 row sum in index order, one IEEE division
+ *                                per element) bit for bit against numpy.cumsum / numpy division on the table the
+ *                                host C library's expf gives.  The device the reference targets computes that
+ *                                table with its own libm (newlib), whose expf may differ from glibc's in the last
+ *                                place, so against that device the claim is the tolerance, not the bits
+ *                                                                                   PINNED (to float32 tolerance)
+ *   espdl_oracle_quantize_f32, _dequantize_f32   exact rational round-half-up of v * 2^-e incl. ties and the
+ *                                saturation edges; exact scaling                                     PINNED
+ *   matmul_s8 (espdl_oracle.py)  built from espdl_oracle_conv2d_s8 exactly as the reference builds it from
+ *                                base::conv2d; checked against numpy integer matmul with broadcasting followed by
+ *                                the pinned shift-round, and against the transposed-operand mistake   PINNED
+ *   espdl_oracle_lut_s16         all 65536 inputs against round((x + 32768) / step) in exact rationals for both tie
+ *                                rules and five table sizes                                          PINNED
+ *   espdl_oracle_insert_zeros    equality with numpy strided assignment into zeros                   PINNED
  *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
  *                                numpy.split / numpy.transpose on random shapes           PINNED
  *   espdl_oracle_max_pool        equality with scipy.ndimage.maximum_filter (minimum-value border)
