@@ -22,6 +22,9 @@
 //     rebuilds operand A and its per-channel constants only when the channel group changes.
 //   * Results go to an LDS copy of the output tile and leave as 16-byte stores of consecutive
 //     addresses.
+//   * Optional stages around the depthwise one, all on the tile while it is in LDS: a 1x1 project
+//     convolution (+ residual Add) behind it, and a 1x1 expand convolution in front of it that computes
+//     the patch from a patch of the block input (at most 64 channels) instead of reading it.
 // A workgroup is persistent over tiles; tiles of one XCD are contiguous in memory (xcd_tile_sequence).
 #include <algorithm>
 #include <cstdio>
@@ -40,6 +43,7 @@ constexpr int kWaves = kThreads / 64;
 constexpr int kKs = 3;     // k steps of 4 taps
 constexpr int kMaxIn = 5;  // 16-byte patch chunks per thread
 constexpr int kMaxOut = 4; // 16-byte output chunks per thread
+constexpr int kMaxX = 4;   // dwords of the expand stage's input patch per thread
 
 struct DwLdsArgs {
     const int8_t *in;
@@ -75,6 +79,15 @@ struct DwLdsArgs {
     int n_pout_chunks;  // th * tw * p_vecs
     FastDiv fd_pvecs;
     int off_wp, off_cp, off_pout;
+    // optional 1x1 expand convolution in front: the patch is computed from a patch of the block input
+    // (ex.c0 <= 64 channels) instead of being read, so the expanded tensor never exists in memory
+    DwExpand ex;
+    int xs;              // LDS pixel stride of the block-input patch, bytes (an odd number of 16-byte units)
+    int x_units;         // 16-byte units of a pixel that hold data: ceil(c0 / 16)
+    int n_x_dwords;      // ph * pw * c0 / 4
+    int n_xpt;           // pixel tiles of 16 in the patch
+    FastDiv fd_xdw, fd_pw, fd_nxg;
+    int off_xin, off_xrc, off_we, off_ce;
 };
 
 struct UnitPos {
@@ -106,6 +119,93 @@ __device__ __forceinline__ void dw_fetch(const DwLdsArgs &a, const UnitPos &u, i
             const int iy = iy0 + (rc[i] & 0xffff), ix = ix0 + (rc[i] >> 16);
             const bool ok = rc[i] >= 0 && (unsigned)iy < (unsigned)g.in_h && (unsigned)ix < (unsigned)g.in_w;
             pv[i] = ok ? *reinterpret_cast<const v4i *>(base + rel[i]) : v4i{0, 0, 0, 0};
+        }
+    }
+}
+
+// Block-input patch dwords of this thread for one tile (expand form): global -> registers.
+__device__ __forceinline__ void dw_fetch_x(const DwLdsArgs &a, const UnitPos &u, const int (&rel)[kMaxX],
+                                           const int (&rc)[kMaxX], int (&xv)[kMaxX])
+{
+    const ConvGeom &g = a.g;
+    const int iy0 = u.y0 * g.stride_h - g.pad_top, ix0 = u.x0 * g.stride_w - g.pad_left;
+    const int8_t *base = a.ex.x + (((long long)u.n * g.in_h + iy0) * g.in_w + ix0) * a.ex.c0;
+#pragma unroll
+    for (int i = 0; i < kMaxX; i++) {
+        if (i * kThreads < a.n_x_dwords) { // uniform
+            const int iy = iy0 + (rc[i] & 0xffff), ix = ix0 + (rc[i] >> 16);
+            const bool ok = rc[i] >= 0 && (unsigned)iy < (unsigned)g.in_h && (unsigned)ix < (unsigned)g.in_w;
+            xv[i] = ok ? *reinterpret_cast<const int *>(base + rel[i]) : 0;
+        }
+    }
+}
+
+// Expand stage of one tile: patch[pixel][channel] = act(requant(w_e[channel] . x[pixel] + bias)) for the
+// pixels of the patch that lie inside the image, zero for the others (the depthwise stage's window
+// clipping).  Rows = 16 expanded channels, columns = 16 patch pixels, one MFMA per tile (c0 <= 64).
+// A wavefront takes units of four pixel tiles of one channel tile, so that four independent
+// load -> MFMA -> requantize -> store chains are in flight.  INTERIOR: the whole patch lies inside the
+// image, no per-pixel test (pixel slots past the patch fall into slack the patch area keeps for them).
+template <int MODE, bool INTERIOR> // MODE: pack_fast4 mode, or -1 for the general epilogue
+__device__ __forceinline__ void dw_expand(const DwLdsArgs &a, unsigned char *smem, int wave, int lane, const UnitPos &u,
+                                          int floor_e)
+{
+    const ConvGeom &g = a.g;
+    const int col = lane & 15, quad = lane >> 4;
+    const int iy0 = u.y0 * g.stride_h - g.pad_top, ix0 = u.x0 * g.stride_w - g.pad_left;
+    const int *xrc = reinterpret_cast<const int *>(smem + a.off_xrc);
+    const int *ce = reinterpret_cast<const int *>(smem + a.off_ce);
+    const unsigned char *xin = smem + a.off_xin + col * a.xs + 16 * quad;
+    unsigned char *patch = smem + a.off_patch + col * a.cs + 4 * quad;
+    const int cw = a.gc * 16;
+    const int n_xg = (a.n_xpt + 3) >> 2;
+    const int n_units = a.gc * n_xg;
+    const bool has_k = quad < a.x_units;
+    // the wavefront index is the same in every lane: say so, so that the unit walk and its guards are scalar
+    for (int unit = __builtin_amdgcn_readfirstlane(wave); unit < n_units; unit += kWaves) {
+        const int ct = (int)fastdiv((unsigned)unit, a.fd_nxg);
+        const int pt0 = (unit - ct * n_xg) * 4;
+        const int cnt = min(4, a.n_xpt - pt0); // uniform
+        const v4i aop = *reinterpret_cast<const v4i *>(smem + a.off_we + 16 * (ct * 64 + lane));
+        const int ch = 16 * ct + 4 * quad;
+        const v4i init = *reinterpret_cast<const v4i *>(ce + ch);
+        const v4i ss = *reinterpret_cast<const v4i *>(ce + cw + ch);
+        const v4i ls = *reinterpret_cast<const v4i *>(ce + 2 * cw + ch);
+        v4i b[4], acc[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            b[j] = v4i{0, 0, 0, 0};
+            if (j < cnt && has_k)
+                b[j] = *reinterpret_cast<const v4i *>(xin + (pt0 + j) * 16 * a.xs);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (j < cnt)
+                acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[j], init, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (j < cnt) {
+                int word;
+                if constexpr (MODE >= 0) {
+                    word = pack_fast4<MODE>(acc[j], ls, ss, floor_e);
+                } else {
+                    int q[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        q[r] = requant_s8(acc[j][r], ss[r], a.ex.relu != 0, g.half_even != 0);
+                    word = pack4_s8(q[0], q[1], q[2], q[3]);
+                }
+                int *dst = reinterpret_cast<int *>(patch + (pt0 + j) * 16 * a.cs + 16 * ct);
+                if constexpr (INTERIOR) {
+                    *dst = word;
+                } else {
+                    const int prc = xrc[(pt0 + j) * 16 + col];
+                    if (prc >= 0) {
+                        const int iy = iy0 + (prc & 0xffff), ix = ix0 + (prc >> 16);
+                        *dst = ((unsigned)iy < (unsigned)g.in_h && (unsigned)ix < (unsigned)g.in_w) ? word : 0;
+                    }
+                }
+            }
         }
     }
 }
@@ -196,7 +296,7 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
 }
 
 // HE: the round-half-even build (a separate kernel so that the half-up build keeps its register count).
-template <bool PROJ, bool HE>
+template <bool PROJ, bool HE, bool EXP>
 __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwLdsArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -225,6 +325,24 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
             in_rel[i] = 0;
             in_lds[i] = -1;
             in_rc[i] = -1;
+        }
+    }
+    int x_rel[kMaxX], x_lds[kMaxX], x_rc[kMaxX];
+#pragma unroll
+    for (int i = 0; i < kMaxX; i++) {
+        const int k = tid + i * kThreads;
+        if (EXP && k < a.n_x_dwords) {
+            const unsigned q = fastdiv((unsigned)k, a.fd_xdw);
+            const unsigned d = (unsigned)k - q * a.fd_xdw.d;
+            const unsigned prow = fastdiv(q, a.fd_pw);
+            const unsigned pcol = q - prow * a.fd_pw.d;
+            x_rel[i] = (int)((prow * g.in_w + pcol) * a.ex.c0 + 4 * d);
+            x_lds[i] = (int)(q * a.xs + 4 * d);
+            x_rc[i] = (int)(prow | (pcol << 16));
+        } else {
+            x_rel[i] = 0;
+            x_lds[i] = -1;
+            x_rc[i] = -1;
         }
     }
     int out_rel[kMaxOut], out_lds[kMaxOut], out_rc[kMaxOut];
@@ -257,10 +375,14 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
     const TileSeq seq = xcd_tile_sequence(a.n_units);
     int unit = seq.first;
     v4i pv[kMaxIn];
+    int xv[kMaxX];
     UnitPos u = {0, 0, 0};
     if (unit < seq.end) {
         u = dw_unit(a, unit);
-        dw_fetch(a, u, cc0, in_rel, in_rc, pv);
+        if (EXP)
+            dw_fetch_x(a, u, x_rel, x_rc, xv);
+        else
+            dw_fetch(a, u, cc0, in_rel, in_rc, pv);
     }
 
     // tables: diagonal operand A as one dword per (group, k step, lane); start values and shifts;
@@ -366,18 +488,88 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
         floor_p = pj.relu ? 0 : (int)0x80008000u;
     }
 
+    // expand stage: filters in MFMA operand-A order (row i of channel tile ct is expanded channel
+    // cc0 + 16*ct + i, the lane's 16 k positions are block-input channels 16*quad ...; zeros past c0), the
+    // [start value | shift | left shift] table, the (row, column) of every patch pixel, and a cleared
+    // block-input patch (its bytes past c0 stay zero)
+    bool fast_e = false;
+    int floor_e = 0;
+    if (EXP) {
+        const DwExpand &ex = a.ex;
+        for (int e = tid; e < a.gc * 64 * 16; e += kThreads) {
+            const int byte = e & 15, l = (e >> 4) & 63, ct = e >> 10;
+            const int ch = cc0 + 16 * ct + (l & 15), k = 16 * (l >> 4) + byte;
+            smem[a.off_we + e] = k < ex.c0 ? (unsigned char)ex.w[(long long)ch * ex.c0 + k] : (unsigned char)0;
+        }
+        const long long bound = (long long)ex.c0 * 16384;
+        int oke = 1;
+        int es = 0, eb = 0;
+        if (tid < cw) {
+            es = ex.shift[ex.n_shift == 1 ? 0 : cc0 + tid];
+            eb = ex.bias != nullptr ? ex.bias[cc0 + tid] : 0;
+            if (es < 1 || es > 31) {
+                oke = 0;
+            } else {
+                const long long start = (long long)eb + (1ll << (es - 1));
+                if ((start < 0 ? -start : start) + bound >= (1ll << (31 - max(0, 8 - es))))
+                    oke = 0;
+            }
+        }
+        fast_e = __syncthreads_and(oke) != 0;
+        int *ce = reinterpret_cast<int *>(smem + a.off_ce);
+        if (tid < cw) {
+            ce[tid] = fast_e ? eb + (1 << (es - 1)) : eb;
+            ce[cw + tid] = fast_e ? max(0, es - 8) : es;
+            ce[2 * cw + tid] = fast_e ? max(0, 8 - es) : 0;
+        }
+        int *xrc = reinterpret_cast<int *>(smem + a.off_xrc);
+        for (int q = tid; q < a.n_xpt * 16; q += kThreads) {
+            int v = -1;
+            if (q < a.ph * a.pw) {
+                const unsigned prow = fastdiv((unsigned)q, a.fd_pw);
+                v = (int)(prow | (((unsigned)q - prow * a.fd_pw.d) << 16));
+            }
+            xrc[q] = v;
+        }
+        for (int e = tid; e < a.n_xpt * 16 * a.xs / 4; e += kThreads)
+            reinterpret_cast<int *>(smem + a.off_xin)[e] = 0;
+        floor_e = ex.relu ? 0 : (int)0x80008000u;
+        __syncthreads(); // the cleared patch must not overtake the first tile's stores below
+    }
+
     for (; unit < seq.end; unit += seq.step) {
         // patch of this tile: registers -> LDS
+        if (EXP) {
 #pragma unroll
-        for (int i = 0; i < kMaxIn; i++)
-            if (i * kThreads < a.n_in_chunks && in_lds[i] >= 0)
-                *reinterpret_cast<v4i *>(smem + a.off_patch + in_lds[i]) = pv[i];
+            for (int i = 0; i < kMaxX; i++)
+                if (i * kThreads < a.n_x_dwords && x_lds[i] >= 0)
+                    *reinterpret_cast<int *>(smem + a.off_xin + x_lds[i]) = xv[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kMaxIn; i++)
+                if (i * kThreads < a.n_in_chunks && in_lds[i] >= 0)
+                    *reinterpret_cast<v4i *>(smem + a.off_patch + in_lds[i]) = pv[i];
+        }
         __syncthreads();
         const UnitPos u_cur = u;
         const int unit_next = unit + seq.step;
         if (unit_next < seq.end) {
             u = dw_unit(a, unit_next);
-            dw_fetch(a, u, cc0, in_rel, in_rc, pv); // in flight during the compute phase
+            if (EXP)
+                dw_fetch_x(a, u, x_rel, x_rc, xv); // in flight during the compute phases
+            else
+                dw_fetch(a, u, cc0, in_rel, in_rc, pv);
+        }
+        if (EXP) {
+            const int py0 = u_cur.y0 * g.stride_h - g.pad_top, px0 = u_cur.x0 * g.stride_w - g.pad_left;
+            const bool interior = py0 >= 0 && px0 >= 0 && py0 + a.ph <= g.in_h && px0 + a.pw <= g.in_w;
+            if (fast_e && interior)
+                dw_expand<HE ? 2 : 1, true>(a, smem, wave, lane, u_cur, floor_e);
+            else if (fast_e)
+                dw_expand<HE ? 2 : 1, false>(a, smem, wave, lane, u_cur, floor_e);
+            else
+                dw_expand<-1, false>(a, smem, wave, lane, u_cur, floor_e);
+            __syncthreads();
         }
 
         // epilogue mode of pack_fast4: 0 plain (every shift >= 8), 1 with the left shift, 2 the same with
@@ -486,7 +678,13 @@ constexpr int kLdsBudget = 80 * 1024; // two workgroups of 8 wavefronts per CU (
 
 // Tile choice: the cheapest (patch bytes read per output byte, with a penalty for tiles too small
 // to amortize the per-tile barriers) among the candidates that fit the LDS and register budgets.
-DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr)
+// pixel tiles of 16 in a patch when an expand stage fills it, else 0
+int expand_n_xpt(int ph, int pw, const DwExpand *ex)
+{
+    return ex != nullptr && ex->w != nullptr ? (ph * pw + 15) / 16 : 0;
+}
+
+DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr, const DwExpand *ex = nullptr)
 {
     DwLdsPlan best;
     best.ok = false;
@@ -517,6 +715,14 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr)
         p_vec = al16 ? 16 : 4;
         p_vecs = pj->out_c / p_vec;
     }
+    const bool expand = ex != nullptr && ex->w != nullptr;
+    int x_units = 0, xs = 0;
+    if (expand) {
+        if (ex->c0 < 4 || ex->c0 > 64 || (ex->c0 & 3) != 0)
+            return best;
+        x_units = (ex->c0 + 15) / 16;
+        xs = 16 * ((x_units & 1) ? x_units : x_units + 1);
+    }
     for (int gc = 1; gc <= min(G, 16); gc++) {
         if (G % gc != 0 || (proj && gc != G))
             continue;
@@ -527,9 +733,15 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr)
                 const int ph = (the - 1) * g.stride_h + halo_h, pw = (twe - 1) * g.stride_w + halo_w;
                 const int np = (the * twe + 15) / 16;
                 const long long n_in = (long long)ph * pw * gc, n_out = (long long)the * twe * gc;
-                if (n_in > kMaxIn * kThreads || n_out > kMaxOut * kThreads || ph > 0xffff || pw > 0x7fff)
+                if ((!expand && n_in > kMaxIn * kThreads) || n_out > kMaxOut * kThreads || ph > 0xffff || pw > 0x7fff)
                     continue;
-                const size_t patch = (size_t)ph * pw * cs + 16 * 16; // reads of padded pixel slots stay inside
+                const long long n_x = expand ? (long long)ph * pw * (ex->c0 / 4) : 0;
+                const int n_xpt = expand ? (ph * pw + 15) / 16 : 0;
+                if (n_x > kMaxX * kThreads)
+                    continue;
+                const size_t xbytes = expand ? (size_t)n_xpt * 16 * xs + (size_t)n_xpt * 16 * 4 + (size_t)gc * 1024 + (size_t)gc * 16 * 12 : 0;
+                // reads of padded pixel slots stay inside; the expand stage also writes whole pixel tiles
+                const size_t patch = (size_t)std::max(ph * pw, expand_n_xpt(ph, pw, ex) * 16) * cs + 16 * 16;
                 // the project stage reads whole 64-channel k steps: slack after the last pixel
                 const size_t outb = (size_t)np * 16 * cso + (proj ? 256 : 0);
                 const size_t pbytes = proj ? (size_t)p_nrt * p_ks * 1024 + (size_t)3 * p_nrt * 64 + (size_t)np * 16 * p_os : 0;
@@ -537,7 +749,7 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr)
                 if (proj && n_pout > kMaxOut * kThreads)
                     continue;
                 const size_t tables = (size_t)gc * kKs * 64 * 4 + (size_t)gc * 16 * 12 + (size_t)np * 16 * 4 + 256;
-                const size_t lds = patch + outb + tables + pbytes + 64;
+                const size_t lds = patch + outb + tables + pbytes + xbytes + 64;
                 if (lds > (size_t)kLdsBudget)
                     continue;
                 const int per_cu = (int)std::min<size_t>(2, (size_t)(160 * 1024) / lds); // 2 x 8 wavefronts fill a CU
@@ -600,6 +812,19 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr)
                     off += (size_t)3 * p_nrt * 64;
                     a.off_pout = (int)off;
                     off += proj ? (size_t)np * 16 * p_os : 0;
+                    off = (off + 15) & ~(size_t)15;
+                    a.xs = xs;
+                    a.x_units = x_units;
+                    a.n_x_dwords = (int)n_x;
+                    a.n_xpt = n_xpt;
+                    a.off_xin = (int)off;
+                    off += expand ? (size_t)n_xpt * 16 * xs : 0;
+                    a.off_xrc = (int)off;
+                    off += expand ? (size_t)n_xpt * 16 * 4 : 0;
+                    a.off_we = (int)off;
+                    off += expand ? (size_t)gc * 1024 : 0;
+                    a.off_ce = (int)off;
+                    off += expand ? (size_t)gc * 16 * 12 : 0;
                     best.lds = off;
                     best.n_cchunk = G / gc;
                 }
@@ -624,7 +849,7 @@ bool depthwise_s8_lds_supports(const ConvGeom &g, const void *in, const void *ou
 
 namespace {
 
-template <bool PROJ>
+template <bool PROJ, bool EXP = false>
 hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
 {
     DwLdsArgs &a = plan.a;
@@ -640,19 +865,22 @@ hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
     a.fd_tw = make_fastdiv((unsigned)a.tw);
     a.fd_np = make_fastdiv((unsigned)a.np);
     a.fd_pvecs = make_fastdiv((unsigned)max(1, a.p_vecs));
+    a.fd_xdw = make_fastdiv((unsigned)max(1, a.ex.c0 / 4));
+    a.fd_pw = make_fastdiv((unsigned)a.pw);
+    a.fd_nxg = make_fastdiv((unsigned)max(1, (a.n_xpt + 3) / 4));
     const int cus = cu_count > 0 ? cu_count : 256;
     static const hipError_t lds_opt_in = [] {
-        const hipError_t e0 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, false>),
+        const hipError_t e0 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, false, EXP>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
-        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, true>),
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, true, EXP>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
         return e0 != hipSuccess ? e0 : e1;
     }();
     if (lds_opt_in != hipSuccess)
         return lds_opt_in;
     const bool he = g.half_even != 0;
-    const int per_cu = he ? resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, true>, kThreads, plan.lds)
-                          : resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, false>, kThreads, plan.lds);
+    const int per_cu = he ? resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, true, EXP>, kThreads, plan.lds)
+                          : resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, false, EXP>, kThreads, plan.lds);
     int gx = max(1, (cus * per_cu) / plan.n_cchunk);
     if (gx > a.n_units)
         gx = a.n_units;
@@ -660,14 +888,14 @@ hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
         gx &= ~7;
     static const bool trace = getenv("ESPDL_HIP_TRACE") != nullptr;
     if (trace)
-        fprintf(stderr, "depthwise_s8_lds%s: %dx%dx%d s%d tile %dx%d patch %dx%d gc %d np %d lds %zu per_cu %d grid %dx%d units %d\n",
-                PROJ ? "+project" : "", g.in_h, g.in_w, g.in_c, g.stride_h, a.th, a.tw, a.ph, a.pw, a.gc, a.np, plan.lds,
+        fprintf(stderr, "depthwise_s8_lds%s%s: %dx%dx%d s%d tile %dx%d patch %dx%d gc %d np %d lds %zu per_cu %d grid %dx%d units %d\n",
+                EXP ? "expand+" : "", PROJ ? "+project" : "", g.in_h, g.in_w, g.in_c, g.stride_h, a.th, a.tw, a.ph, a.pw, a.gc, a.np, plan.lds,
                 per_cu, gx, plan.n_cchunk, a.n_units);
     if (he)
-        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, true>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
+        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, true, EXP>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
                            dim3(kThreads), plan.lds, stream, a);
     else
-        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, false>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
+        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, false, EXP>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
                            dim3(kThreads), plan.lds, stream, a);
     return hipGetLastError();
 }
@@ -692,6 +920,7 @@ hipError_t launch_depthwise_s8_lds(const ConvGeom &g, const int8_t *in, const in
     a.out = out;
     a.g = g;
     a.pj = DwProject{};
+    a.ex = DwExpand{};
     return dw_lds_launch<false>(plan, cu_count, stream);
 }
 
@@ -723,7 +952,41 @@ hipError_t launch_depthwise_project_s8(const ConvGeom &g, const int8_t *in, cons
     a.out = nullptr;
     a.g = g;
     a.pj = pj;
+    a.ex = DwExpand{};
     return dw_lds_launch<true>(plan, cu_count, stream);
+}
+
+bool expand_depthwise_project_s8_supports(const ConvGeom &g, const DwExpand &ex, const DwProject &pj)
+{
+    if ((g.in_c & 15) != 0 || g.k_h * g.k_w > 4 * kKs || pj.w == nullptr || ex.w == nullptr || ex.x == nullptr ||
+        (reinterpret_cast<uintptr_t>(pj.w) & 15) != 0 || (reinterpret_cast<uintptr_t>(ex.x) & 3) != 0 ||
+        ((reinterpret_cast<uintptr_t>(pj.out) | reinterpret_cast<uintptr_t>(pj.residual)) & 3) != 0)
+        return false;
+    if ((long long)g.in_h * g.in_w * ex.c0 >= (1ll << 30) || (long long)g.out_h * g.out_w * pj.out_c >= (1ll << 30))
+        return false;
+    return dw_lds_plan(g, &pj, &ex).ok;
+}
+
+hipError_t launch_expand_depthwise_project_s8(const ConvGeom &g, const DwExpand &ex, const int8_t *filter,
+                                              const int32_t *bias, const int32_t *shift, const DwProject &pj,
+                                              int cu_count, hipStream_t stream)
+{
+    if ((long long)g.batch * g.out_h * g.out_w == 0)
+        return hipSuccess;
+    DwLdsPlan plan = dw_lds_plan(g, &pj, &ex);
+    if (!plan.ok)
+        return hipErrorInvalidValue;
+    DwLdsArgs &a = plan.a;
+    a.in = nullptr;
+    a.w = filter;
+    a.bias = bias;
+    a.shift = shift;
+    a.lut = nullptr;
+    a.out = nullptr;
+    a.g = g;
+    a.pj = pj;
+    a.ex = ex;
+    return dw_lds_launch<true, true>(plan, cu_count, stream);
 }
 
 } // namespace espdl

@@ -649,6 +649,21 @@ void dwproject_from(const espdl::MbconvParams &p, espdl::ConvGeom *g, espdl::DwP
     pj->out = p.out;
 }
 
+// The same for a block with expand stage: the depthwise stage works on exp_c channels.
+void expand_dwproject_from(const espdl::MbconvParams &p, espdl::ConvGeom *g, espdl::DwProject *pj, espdl::DwExpand *ex)
+{
+    dwproject_from(p, g, pj);
+    g->in_c = p.exp_c;
+    g->out_c = p.exp_c;
+    ex->x = p.in;
+    ex->w = p.w_expand;
+    ex->bias = p.b_expand;
+    ex->shift = p.s_expand;
+    ex->n_shift = p.n_s_expand;
+    ex->relu = p.relu_expand;
+    ex->c0 = p.in_c;
+}
+
 } // namespace
 
 extern "C" {
@@ -684,6 +699,14 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
         dwproject_from(p, &g, &pj);
         if (espdl::depthwise_project_s8_supports(g, p.in, pj))
             return 2;
+    }
+    if (desc->has_expand) {
+        espdl::ConvGeom g;
+        espdl::DwProject pj;
+        espdl::DwExpand ex;
+        expand_dwproject_from(p, &g, &pj, &ex);
+        if (espdl::expand_depthwise_project_s8_supports(g, ex, pj))
+            return 3;
     }
     return espdl::mbconv_s8_fused_supports(p) ? 1 : 0;
 }
@@ -724,6 +747,16 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
             return device_status(espdl::launch_depthwise_project_s8(g, p.in, p.w_dw, p.b_dw, p.s_dw, pj, cu_count_cached(),
                                                                     reinterpret_cast<hipStream_t>(stream)),
                                  "depthwise_project_s8");
+    }
+    if (desc->has_expand) {
+        espdl::ConvGeom g;
+        espdl::DwProject pj;
+        espdl::DwExpand ex;
+        expand_dwproject_from(p, &g, &pj, &ex);
+        if (espdl::expand_depthwise_project_s8_supports(g, ex, pj))
+            return device_status(espdl::launch_expand_depthwise_project_s8(g, ex, p.w_dw, p.b_dw, p.s_dw, pj, cu_count_cached(),
+                                                                           reinterpret_cast<hipStream_t>(stream)),
+                                 "expand_depthwise_project_s8");
     }
     if (!espdl::mbconv_s8_fused_supports(p))
         return fail(ESPDL_HIP_ENOTSUP, "this block shape is not covered by the fused kernel");

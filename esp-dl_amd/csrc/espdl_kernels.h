@@ -44,6 +44,15 @@ struct DwProject {
     int8_t *out;
 };
 
+// 1x1 expand convolution fused in front of a depthwise convolution: the depthwise kernel computes its input
+// patch from `x` ([batch][in_h][in_w][c0], c0 <= 64 and a multiple of 4) instead of reading it.
+struct DwExpand {
+    const int8_t *x;
+    const int8_t *w; // [depthwise channels][c0]
+    const int32_t *bias, *shift;
+    int n_shift, relu, c0;
+};
+
 // Depthwise with the input tile staged in LDS (contiguous global reads and writes) and the products
 // on the matrix pipe; same shape limits as the direct form.
 bool depthwise_s8_lds_supports(const ConvGeom &g, const void *in, const void *out);
@@ -78,6 +87,13 @@ hipError_t launch_mbconv_s8_fused(const MbconvParams &p, int cu_count, hipStream
 bool depthwise_project_s8_supports(const ConvGeom &g, const void *in, const DwProject &pj);
 hipError_t launch_depthwise_project_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                        const int32_t *shift, const DwProject &pj, int cu_count, hipStream_t stream);
+
+// 1x1 expand -> depthwise -> 1x1 project [-> Add] in one launch of the same kernel: neither the expanded
+// tensor nor the depthwise result exists in memory.  Needs at most 256 expanded channels and c0 <= 64.
+bool expand_depthwise_project_s8_supports(const ConvGeom &g, const DwExpand &ex, const DwProject &pj);
+hipError_t launch_expand_depthwise_project_s8(const ConvGeom &g, const DwExpand &ex, const int8_t *filter,
+                                              const int32_t *bias, const int32_t *shift, const DwProject &pj,
+                                              int cu_count, hipStream_t stream);
 
 hipError_t launch_conv2d_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
                              const int32_t *shift, int16_t *out, hipStream_t stream);

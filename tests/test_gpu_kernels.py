@@ -471,6 +471,15 @@ MBCONV_CASES = [
     ("tailpad_17x17_32_96_32_s2", (2, 17, 17, 32), 96, 32, (3, 3), (2, 2), (0, 1, 0, 1), False, False, False),
     ("halfeven_14x14_32_192_32_res", (2, 14, 14, 32), 192, 32, (3, 3), (1, 1), (1, 1, 1, 1), True, True, False),
     ("pertensor_28x28_32_192_64", (2, 28, 28, 32), 192, 64, (3, 3), (1, 1), (1, 1, 1, 1), False, False, True),
+    # expand -> depthwise -> project [-> Add] inside the LDS-tile depthwise kernel (block input <= 64 channels,
+    # at most 256 expanded channels): 24 input channels (one and a half 16-byte units), 64 (four units),
+    # 4 (a quarter unit), 48 expanded channels in a 20-channel-wide ragged image
+    ("edp_56x56_24_144_24_res", (2, 56, 56, 24), 144, 24, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
+    ("edp_56x56_24_144_32_s2", (2, 56, 56, 24), 144, 32, (3, 3), (2, 2), (0, 1, 0, 1), False, False, False),
+    ("edp_112x112_16_96_24_s2", (1, 112, 112, 16), 96, 24, (3, 3), (2, 2), (0, 1, 0, 1), False, False, False),
+    ("edp_14x14_64_256_64_res_halfeven", (3, 14, 14, 64), 256, 64, (3, 3), (1, 1), (1, 1, 1, 1), True, True, False),
+    ("edp_9x11_4_16_8", (2, 9, 11, 4), 16, 8, (3, 3), (1, 1), (1, 1, 1, 1), False, False, True),
+    ("edp_13x20_20_48_20_res", (2, 13, 20, 20), 48, 20, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
     # no expand stage: depthwise -> project [-> Add] inside the LDS-tile depthwise kernel
     ("dwp_56x56_144_24_res", (2, 56, 56, 144), None, 24, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
     ("dwp_57x41_96_24_s2", (2, 57, 41, 96), None, 24, (3, 3), (2, 2), (1, 1, 1, 1), False, False, False),
@@ -518,14 +527,15 @@ def test_mbconv_s8_fused(oracle, case):
     np.testing.assert_array_equal(to_host(got), cur)
 
 
+@pytest.mark.parametrize("ce", [320, 192], ids=["e320_block_kernel", "e192_lds_tile_kernel"])
 @pytest.mark.parametrize("general_stage", [0, 1, 2], ids=["expand_general", "dw_general", "project_general"])
-def test_mbconv_s8_mixed_epilogues(oracle, general_stage):
+def test_mbconv_s8_mixed_epilogues(oracle, general_stage, ce):
     """One stage has shifts outside 1..31 (general shift_and_round form), the other two take the
     short epilogue: the per-stage choice must not leak between stages."""
-    announce(f"mbconv_s8 mixed epilogues, general stage {general_stage}")
+    announce(f"mbconv_s8 mixed epilogues, general stage {general_stage}, {ce} expanded channels")
     m = espdl()
     rng = np.random.default_rng(77 + general_stage)
-    n, h, w, cin, ce, cout = 2, 14, 14, 32, 320, 48
+    n, h, w, cin, cout = 2, 14, 14, 32, 48
     x = rng_int8(rng, (n, h, w, cin))
 
     def stage(idx, oc, kk, fshape):
