@@ -35,8 +35,8 @@ MACHINE_BALANCE = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)  # OP per byte
 # 256 MiB element-wise kernel of known traffic gave in the same runs).  Only valid for config 3 at
 # batch 256; any other workload reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "depthwise_s8": (7 * (2 * 55393.8 + 15717.6) + 10 * (2 * 9887.8 + 17404.8)) / 17 * 1024,
-    "conv2d_s8": (2 * 8334.9 + 35596.5) * 1024,
+    "depthwise_s8": (7 * (2 * 55383.5 + 15715.0) + 10 * (2 * 9882.0 + 17404.8)) / 17 * 1024,
+    "conv2d_s8": (2 * 8794.2 + 35695.7) * 1024,
     "elementwise_s8": None,
 }
 
