@@ -677,6 +677,111 @@ void espdl_oracle_dequantize_f32(const void *in, int64_t size, int in_exp, int e
         out[i] = (elem_size == 1 ? (float)((const int8_t *)in)[i] : (float)((const int16_t *)in)[i]) * scale;
 }
 
+/* ---------------------------------------------------------------------------------------------
+ * int16 forms of the element-wise and pooling operators (the int16 PP-OCR recognizer uses them).
+ * ------------------------------------------------------------------------------------------- */
+
+/* Add, int16 (c_impl_add_n_n<int16_t>, esp-dl/dl/base/dl_base_add.cpp:33-44): saturating integer add. */
+void espdl_oracle_add_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size,
+                          int16_t *out)
+{
+    for (int64_t i = 0; i < size; i++) {
+        const int32_t a = in0[len0 == 1 ? 0 : i], b = in1[len1 == 1 ? 0 : i];
+        out[i] = (int16_t)clamp_i64(a + b, INT16_MIN, INT16_MAX);
+    }
+}
+
+/*
+ * Mul, int16 (c_impl_mul_n_n<int16_t>, esp-dl/dl/base/dl_base_mul.cpp:33-46): the int32 product is
+ * converted to float32 (rounding to nearest even above 2^24), scaled by 2^-shift and rounded with
+ * tool::round.  Half-even mode restates the ESP32-P4 kernels as for int8: shift_and_round half-even of
+ * the exact product.
+ */
+void espdl_oracle_mul_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size, int shift,
+                          int round_mode, int16_t *out)
+{
+    const float rescale = dl_rescale(shift);
+    for (int64_t i = 0; i < size; i++) {
+        const int32_t a = in0[len0 == 1 ? 0 : i], b = in1[len1 == 1 ? 0 : i];
+        const int32_t prod = a * b; /* at most 2^30 in magnitude */
+        int64_t q;
+        if (round_mode == ESPDL_ORACLE_ROUND_HALF_EVEN && shift > 0)
+            q = espdl_oracle_shift_round_s32(prod, shift, ESPDL_ORACLE_ROUND_HALF_EVEN);
+        else
+            q = round_half_up_f32((float)prod * rescale);
+        out[i] = (int16_t)clamp_i64(q, INT16_MIN, INT16_MAX);
+    }
+}
+
+/* AveragePool, int16 (avgpool2d_hwc<int16_t, int32_t>, esp-dl/dl/base/dl_base_avg_pool2d.cpp:28-54, :87). */
+void espdl_oracle_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
+                               int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,
+                               int out_exp, int16_t *out)
+{
+    const int out_h = (h + pad_top + pad_bottom - k_h) / stride_h + 1;
+    const int out_w = (w + pad_left + pad_right - k_w) / stride_w + 1;
+    const float area_inv = 1.f / (float)(k_h * k_w);
+    const float scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
+    for (int n = 0; n < batch; n++)
+        for (int oy = 0; oy < out_h; oy++)
+            for (int ox = 0; ox < out_w; ox++)
+                for (int k = 0; k < c; k++) {
+                    int32_t sum = 0;
+                    for (int ky = 0; ky < k_h; ky++) {
+                        const int iy = oy * stride_h - pad_top + ky;
+                        if (iy < 0 || iy >= h)
+                            continue;
+                        for (int kx = 0; kx < k_w; kx++) {
+                            const int ix = ox * stride_w - pad_left + kx;
+                            if (ix < 0 || ix >= w)
+                                continue;
+                            sum += in[(((int64_t)n * h + iy) * w + ix) * c + k];
+                        }
+                    }
+                    out[(((int64_t)n * out_h + oy) * out_w + ox) * c + k] =
+                        (int16_t)clamp_i64(round_half_up_f32((float)sum * scale), INT16_MIN, INT16_MAX);
+                }
+}
+
+/* ReduceMean, int16 (reduce<int64_t, int16_t>, esp-dl/dl/module/include/dl_module_reduce_mean.hpp:18-45, :54-56). */
+int espdl_oracle_reduce_mean_s16(const int16_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
+                                 int out_exp, int16_t *out)
+{
+    if (dims < 1 || dims > 8)
+        return -1;
+    int64_t total = 1, count = 1;
+    for (int i = 0; i < dims; i++) {
+        total *= shape[i];
+        if (reduce_flag[i])
+            count *= shape[i];
+    }
+    if (total == 0)
+        return 0;
+    const int64_t n_out = total / count;
+    int64_t *sums = (int64_t *)calloc((size_t)n_out, sizeof(int64_t));
+    if (!sums)
+        return -1;
+    int64_t idx[8] = {0};
+    for (int64_t e = 0; e < total; e++) {
+        int64_t o = 0;
+        for (int i = 0; i < dims; i++)
+            if (!reduce_flag[i])
+                o = o * shape[i] + idx[i];
+        sums[o] += in[e];
+        for (int i = dims - 1; i >= 0; i--) {
+            if (++idx[i] < shape[i])
+                break;
+            idx[i] = 0;
+        }
+    }
+    const float input_scale = dl_scale(in_exp), output_scale = dl_rescale(out_exp);
+    for (int64_t o = 0; o < n_out; o++)
+        out[o] = (int16_t)clamp_i64(round_half_up_f32((float)sums[o] * input_scale / (float)count * output_scale),
+                                    INT16_MIN, INT16_MAX);
+    free(sums);
+    return 0;
+}
+
 /*
  * InsertZeros::forward_template (esp-dl/dl/module/include/dl_module_insert_zeros.hpp): the output is cleared,
  * then input pixel (h, w) is copied to output pixel (h * stride_h, w * stride_w).

@@ -64,6 +64,12 @@
  *   espdl_oracle_lut_s16         all 65536 inputs against round((x + 32768) / step) in exact rationals for both tie
  *                                rules and five table sizes                                          PINNED
  *   espdl_oracle_insert_zeros    equality with numpy strided assignment into zeros                   PINNED
+ *   espdl_oracle_add_s16         numpy saturating add                                               PINNED
+ *   espdl_oracle_mul_s16         numpy: int64 product -> float32 (round to nearest even) -> exact power-of-two
+ *                                scaling -> exact rational round half up; half-even mode against the pinned
+ *                                integer shift-round                                                  PINNED
+ *   espdl_oracle_avg_pool_s16, _reduce_mean_s16   as their int8 forms: exact rationals away from ties
+ *                                                                                   PARITY UNPINNED (near-ties)
  *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
  *                                numpy.split / numpy.transpose on random shapes           PINNED
  *   espdl_oracle_max_pool        equality with scipy.ndimage.maximum_filter (minimum-value border)
@@ -137,6 +143,15 @@ int espdl_oracle_reduce_mean_s8(const int8_t *in, const int *shape, int dims, co
 int espdl_oracle_slice(const void *in, const int *shape, int dims, const int *start, const int *step,
                        const int *out_shape, int elem_size, void *out);
 void espdl_oracle_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out);
+void espdl_oracle_add_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size,
+                          int16_t *out);
+void espdl_oracle_mul_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size, int shift,
+                          int round_mode, int16_t *out);
+void espdl_oracle_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
+                               int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,
+                               int out_exp, int16_t *out);
+int espdl_oracle_reduce_mean_s16(const int16_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
+                                 int out_exp, int16_t *out);
 void espdl_oracle_insert_zeros(const void *in, int elem_size, int batch, int h, int w, int c, int stride_h, int stride_w,
                                int out_h, int out_w, void *out);
 int espdl_oracle_lut_s16(const int16_t *in, int64_t size, const int16_t *table, int table_size, int p4_ties,

@@ -62,6 +62,14 @@ def lib():
         L.espdl_oracle_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp]
         L.espdl_oracle_reduce_mean_s8.restype = i32
         L.espdl_oracle_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp]
+        L.espdl_oracle_add_s16.restype = None
+        L.espdl_oracle_add_s16.argtypes = [vp, i64, vp, i64, i64, vp]
+        L.espdl_oracle_mul_s16.restype = None
+        L.espdl_oracle_mul_s16.argtypes = [vp, i64, vp, i64, i64, i32, i32, vp]
+        L.espdl_oracle_avg_pool_s16.restype = None
+        L.espdl_oracle_avg_pool_s16.argtypes = [vp] + [i32] * 14 + [vp]
+        L.espdl_oracle_reduce_mean_s16.restype = i32
+        L.espdl_oracle_reduce_mean_s16.argtypes = [vp, vp, i32, vp, i32, i32, vp]
         L.espdl_oracle_insert_zeros.restype = None
         L.espdl_oracle_insert_zeros.argtypes = [vp] + [i32] * 9 + [vp]
         L.espdl_oracle_lut_s16.restype = i32
@@ -295,6 +303,26 @@ def mul_s8(a, b, shift, round_mode=ROUND_HALF_UP):
     return out
 
 
+def add_s16(a, b):
+    a = _c(a, np.int16)
+    b = _c(b, np.int16)
+    size = max(a.size, b.size)
+    assert a.size in (1, size) and b.size in (1, size)
+    out = np.empty(a.shape if a.size == size else b.shape, dtype=np.int16)
+    lib().espdl_oracle_add_s16(_ptr(a), a.size, _ptr(b), b.size, size, _ptr(out))
+    return out
+
+
+def mul_s16(a, b, shift, round_mode=ROUND_HALF_UP):
+    a = _c(a, np.int16)
+    b = _c(b, np.int16)
+    size = max(a.size, b.size)
+    assert a.size in (1, size) and b.size in (1, size)
+    out = np.empty(a.shape if a.size == size else b.shape, dtype=np.int16)
+    lib().espdl_oracle_mul_s16(_ptr(a), a.size, _ptr(b), b.size, size, int(shift), int(round_mode), _ptr(out))
+    return out
+
+
 def global_avg_pool_s8(x, in_exp, out_exp):
     x = _c(x, np.int8)
     n, h, w, c = x.shape
@@ -397,6 +425,33 @@ def avg_pool_s8(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0), in_exp=0, out_exp=
     out = np.empty((n, oh, ow, c), dtype=np.int8)
     lib().espdl_oracle_avg_pool_s8(_ptr(x), n, h, w, c, kernel[0], kernel[1], strides[0], strides[1], pt, pb, pl, pr,
                                    in_exp, out_exp, _ptr(out))
+    return out
+
+
+def avg_pool_s16(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0), in_exp=0, out_exp=0):
+    x = _c(x, np.int16)
+    n, h, w, c = x.shape
+    pt, pb, pl, pr = pads
+    oh = (h + pt + pb - kernel[0]) // strides[0] + 1
+    ow = (w + pl + pr - kernel[1]) // strides[1] + 1
+    out = np.empty((n, oh, ow, c), dtype=np.int16)
+    lib().espdl_oracle_avg_pool_s16(_ptr(x), n, h, w, c, kernel[0], kernel[1], strides[0], strides[1], pt, pb, pl, pr,
+                                    in_exp, out_exp, _ptr(out))
+    return out
+
+
+def reduce_mean_s16(x, axes, keepdims=True, in_exp=0, out_exp=0):
+    x = _c(x, np.int16)
+    nd = x.ndim
+    axes = [a + nd if a < 0 else a for a in (axes if len(axes) else range(nd))]
+    flags = np.array([1 if i in axes else 0 for i in range(nd)], dtype=np.int32)
+    kept = [x.shape[i] for i in range(nd) if not flags[i]]
+    out = np.empty(kept if kept else [1], dtype=np.int16)
+    shape = np.array(x.shape, dtype=np.int32)
+    rc = lib().espdl_oracle_reduce_mean_s16(_ptr(x), _ptr(shape), nd, _ptr(flags), in_exp, out_exp, _ptr(out))
+    assert rc == 0
+    if keepdims:
+        out = out.reshape([1 if flags[i] else x.shape[i] for i in range(nd)])
     return out
 
 

@@ -72,7 +72,13 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             bias = spec.initializers[ins[2]][2] if len(ins) > 2 else None
             shift = _shift(spec, node, ins[0], ins[1], y_name)
             act = oracle.RELU if a.get("activation", "Linear") == "Relu" else oracle.LINEAR
-            y = oracle.gemm_s8(x, w, bias, shift, activation=act, round_mode=round_mode)
+            if x.dtype == np.int16:  # the same 1x1 convolution view, int16 x int16 -> int64
+                k = x.shape[-1]
+                y = oracle.conv2d_s16(x.reshape(1, 1, x.size // k, k), w, bias, shift, (1, 1), activation=act,
+                                      round_mode=round_mode)
+                y = y.reshape(x.shape[:-1] + (y.shape[-1],))
+            else:
+                y = oracle.gemm_s8(x, w, bias, shift, activation=act, round_mode=round_mode)
         elif "lut" in a:
             if x.dtype == np.int16:
                 y = oracle.lut_s16(x, spec.initializers[a["lut"]][2], p4_ties=(round_mode == oracle.ROUND_HALF_EVEN))
@@ -94,13 +100,15 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             b = operand(ins[1])
             if x.shape != b.shape:
                 x, b = np.broadcast_arrays(x, b)
-            y = oracle.add_s8(np.ascontiguousarray(x), np.ascontiguousarray(b))
+            add = oracle.add_s16 if x.dtype == np.int16 else oracle.add_s8
+            y = add(np.ascontiguousarray(x), np.ascontiguousarray(b))
         elif op == "Mul":
             b = operand(ins[1])
             shift = spec.exponent(y_name) - exponent_of(ins[0]) - exponent_of(ins[1])
             if x.shape != b.shape:  # broadcast explicitly: the oracle takes equal sizes or a scalar
                 x, b = np.broadcast_arrays(x, b)
-            y = oracle.mul_s8(np.ascontiguousarray(x), np.ascontiguousarray(b), shift, round_mode)
+            mul = oracle.mul_s16 if x.dtype == np.int16 else oracle.mul_s8
+            y = mul(np.ascontiguousarray(x), np.ascontiguousarray(b), shift, round_mode)
         elif op == "GlobalAveragePool":
             y = oracle.global_avg_pool_s8(x, spec.exponent(ins[0]), spec.exponent(y_name))
         elif op == "RequantizeLinear":
@@ -121,20 +129,22 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
             y = x.reshape([x.shape[0]] + rest)
         elif op == "AveragePool":
             k, st, pads = list(a["kernel_shape"]), list(a.get("strides") or [1] * len(a["kernel_shape"])), list(a.get("pads") or [])
+            avg_pool = oracle.avg_pool_s16 if x.dtype == np.int16 else oracle.avg_pool_s8
             if x.ndim == 3:  # NWC runs as one row
                 pl, pr = pads if pads else (0, 0)
-                y = oracle.avg_pool_s8(x[:, None], (1, k[0]), (1, st[0]), (0, 0, pl, pr), spec.exponent(ins[0]),
+                y = avg_pool(x[:, None], (1, k[0]), (1, st[0]), (0, 0, pl, pr), spec.exponent(ins[0]),
                                        spec.exponent(y_name))[:, 0]
             else:
                 pt, pl, pb, pr = pads if pads else (0, 0, 0, 0)
-                y = oracle.avg_pool_s8(x, tuple(k), tuple(st), (pt, pb, pl, pr), spec.exponent(ins[0]), spec.exponent(y_name))
+                y = avg_pool(x, tuple(k), tuple(st), (pt, pb, pl, pr), spec.exponent(ins[0]), spec.exponent(y_name))
         elif op == "ReduceMean":
             axes = spec.initializers[ins[1]][2].ravel() if len(ins) > 1 and ins[1] in spec.initializers else a.get("axes", [])
             if len(axes) == 0 and a.get("noop_with_empty_axes", 0):
                 y = x
             else:
-                y = oracle.reduce_mean_s8(x, [int(v) for v in axes], bool(a.get("keepdims", 1)), spec.exponent(ins[0]),
-                                          spec.exponent(y_name))
+                reduce_mean = oracle.reduce_mean_s16 if x.dtype == np.int16 else oracle.reduce_mean_s8
+                y = reduce_mean(x, [int(v) for v in axes], bool(a.get("keepdims", 1)), spec.exponent(ins[0]),
+                                spec.exponent(y_name))
         elif op == "Slice":
             par = [spec.initializers[n][2].ravel() if n in spec.initializers else None for n in (ins[1:5] + [None] * 4)[:4]]
             y = oracle.slice_(x, par[0], par[1], par[2], par[3])

@@ -139,3 +139,55 @@ def test_lut_s16_takes_the_nearest_sample(oracle, entries, p4_ties):
 def test_lut_s16_rejects_odd_table_sizes(oracle):
     with pytest.raises(AssertionError):
         oracle.lut_s16(np.zeros(4, dtype=np.int16), np.zeros(1000, dtype=np.int16))
+
+
+def test_add_s16_saturates(oracle):
+    rng = np.random.default_rng(50)
+    a, b = _rand(rng, (3, 1000), np.int16), _rand(rng, (3, 1000), np.int16)
+    want = np.clip(a.astype(np.int32) + b.astype(np.int32), -32768, 32767).astype(np.int16)
+    np.testing.assert_array_equal(oracle.add_s16(a, b), want)
+    np.testing.assert_array_equal(oracle.add_s16(a, b[:1, :1]), np.clip(a.astype(np.int32) + int(b[0, 0]), -32768, 32767))
+
+
+@pytest.mark.parametrize("shift", [0, 7, 12, 15, 20])
+def test_mul_s16_goes_through_float32(oracle, shift):
+    """Half up: the product passes through float32 (numpy's int64 -> float32 conversion rounds to nearest
+    even, as the C conversion does), is scaled by an exact power of two and rounded half up in exact
+    rationals.  Half even: integer shift-round of the exact product."""
+    rng = np.random.default_rng(51)
+    a, b = _rand(rng, (20000,), np.int16), _rand(rng, (20000,), np.int16)
+    a[:4], b[:4] = [-32768, 32767, -32768, 4097], [-32768, 32767, 32767, 4099]
+    prod = a.astype(np.int64) * b.astype(np.int64)
+    as_f32 = prod.astype(np.float32)
+    want = [min(max(int(np.floor(Fraction(float(v)) / (1 << shift) + Fraction(1, 2))), -32768), 32767) for v in as_f32]
+    np.testing.assert_array_equal(oracle.mul_s16(a, b, shift, oracle.ROUND_HALF_UP), np.array(want, dtype=np.int16))
+    if shift > 0:
+        even = np.clip(_shift_round(prod, shift, True), -32768, 32767).astype(np.int16)
+        np.testing.assert_array_equal(oracle.mul_s16(a, b, shift, oracle.ROUND_HALF_EVEN), even)
+    if shift == 0:  # above 2^24 the float32 detour is visible: some products change
+        assert np.any(as_f32.astype(np.int64) != prod)
+
+
+def test_avg_pool_and_reduce_mean_s16_are_exact_means_away_from_ties(oracle):
+    rng = np.random.default_rng(52)
+    x = _rand(rng, (2, 9, 8, 5), np.int16)
+    got = oracle.avg_pool_s16(x, (3, 3), (2, 2), (1, 1, 1, 1), -10, -9)
+    pad = np.pad(x.astype(np.int64), ((0, 0), (1, 1), (1, 1), (0, 0)))
+    checked = 0
+    for oy in range(got.shape[1]):
+        for ox in range(got.shape[2]):
+            s = pad[:, 2 * oy:2 * oy + 3, 2 * ox:2 * ox + 3].sum(axis=(1, 2))
+            for n in range(2):
+                for c in range(5):
+                    exact = Fraction(int(s[n, c]), 9) / 2  # 2^-10 / 2^-9
+                    if abs((exact - np.floor(exact)) - Fraction(1, 2)) > Fraction(1, 1000):
+                        assert got[n, oy, ox, c] == min(max(int(np.floor(exact + Fraction(1, 2))), -32768), 32767)
+                        checked += 1
+    assert checked > 150
+    r = oracle.reduce_mean_s16(x, [1, 2], True, -10, -12)
+    s = x.astype(np.int64).sum(axis=(1, 2))
+    for n in range(2):
+        for c in range(5):
+            exact = Fraction(int(s[n, c]), 72) * 4
+            if abs((exact - np.floor(exact)) - Fraction(1, 2)) > Fraction(1, 1000):
+                assert r[n, 0, 0, c] == min(max(int(np.floor(exact + Fraction(1, 2))), -32768), 32767)
