@@ -78,6 +78,12 @@ def lib():
         L.espdl_hip_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp, vp]
         L.espdl_hip_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp, vp]
         L.espdl_hip_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
+        L.espdl_hip_add_s16.argtypes = [vp, vp, vp, vp, vp, vp, vp]
+        L.espdl_hip_mul_s16.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp]
+        L.espdl_hip_avg_pool_s16.argtypes = [vp] + [i32] * 14 + [vp, vp]
+        L.espdl_hip_reduce_mean_s16.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
+        for name in ("add_s16", "mul_s16", "avg_pool_s16", "reduce_mean_s16"):
+            getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         L.espdl_hip_insert_zeros.argtypes = [vp] + [i32] * 9 + [vp, vp]
         L.espdl_hip_insert_zeros.restype = ctypes.c_int
         L.espdl_hip_lut_s16.argtypes = [vp, i64, vp, i32, i32, vp, vp]
@@ -453,3 +459,49 @@ def insert_zeros(x, stride, output_padding=(0, 0), stream=None):
     out = torch.empty([n, oh, c] if one_d else [n, oh, ow, c], dtype=x.dtype, device=x.device)
     _check(lib().espdl_hip_insert_zeros(_p(x), x.element_size(), n, h, w, c, sh, sw, ph, pw, _p(out), _stream(stream)))
     return out
+
+
+def _broadcast16(a, b):
+    import torch
+    dims, s0, s1, _ = _broadcast(a, b, a)  # strides only; the result is allocated below
+    rank = max(a.dim(), b.dim())
+    so = [int(d) for d in dims]
+    return dims, s0, s1, torch.empty(so[4 - rank:] if rank else [], dtype=torch.int16, device=a.device)
+
+
+def add_s16(a, b, stream=None):
+    dims, s0, s1, out = _broadcast16(a, b)
+    _check(lib().espdl_hip_add_s16(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), _p(out),
+                                   _stream(stream)))
+    return out
+
+
+def mul_s16(a, b, shift, round_mode=ROUND_HALF_UP, stream=None):
+    dims, s0, s1, out = _broadcast16(a, b)
+    _check(lib().espdl_hip_mul_s16(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), int(shift),
+                                   round_mode, _p(out), _stream(stream)))
+    return out
+
+
+def avg_pool_s16(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0), in_exp=0, out_exp=0, stream=None):
+    import torch
+    n, h, w, c = x.shape
+    pt, pb, pl, pr = pads
+    oh = (h + pt + pb - kernel[0]) // strides[0] + 1
+    ow = (w + pl + pr - kernel[1]) // strides[1] + 1
+    out = torch.empty((n, max(oh, 0), max(ow, 0), c), dtype=torch.int16, device=x.device)
+    _check(lib().espdl_hip_avg_pool_s16(_p(x), n, h, w, c, kernel[0], kernel[1], strides[0], strides[1], pt, pb, pl, pr,
+                                        in_exp, out_exp, _p(out), _stream(stream)))
+    return out
+
+
+def reduce_mean_s16(x, axes, keepdims=True, in_exp=0, out_exp=0, stream=None):
+    import torch
+    nd = x.dim()
+    axes = [a + nd if a < 0 else a for a in (axes if len(axes) else range(nd))]
+    flags = [1 if i in axes else 0 for i in range(nd)]
+    kept = [int(x.shape[i]) for i in range(nd) if not flags[i]]
+    out = torch.empty(kept if kept else [1], dtype=torch.int16, device=x.device)
+    _check(lib().espdl_hip_reduce_mean_s16(_p(x), (ctypes.c_int32 * nd)(*x.shape), nd, (ctypes.c_int32 * nd)(*flags),
+                                           in_exp, out_exp, _p(out), _stream(stream)))
+    return out.reshape([1 if flags[i] else int(x.shape[i]) for i in range(nd)]) if keepdims else out

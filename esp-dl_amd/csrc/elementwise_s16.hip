@@ -1,0 +1,215 @@
+// int16 forms of Add, Mul, AveragePool and ReduceMean for gfx950.  They serve the int16 heads and the int16
+// text recognizer of the reference's model files: small tensors, so one element per lane and plain loops.
+//
+// Add: c_impl_add_n_n<int16_t> (esp-dl/dl/base/dl_base_add.cpp:33-44), saturating integer add.
+// Mul: c_impl_mul_n_n<int16_t> (esp-dl/dl/base/dl_base_mul.cpp:33-46): the int32 product goes through
+//      float32, is scaled by 2^-shift and rounded half up; with ESP32-P4 semantics the exact product is
+//      shifted and rounded half to even.
+// AveragePool: avgpool2d_hwc<int16_t, int32_t> (esp-dl/dl/base/dl_base_avg_pool2d.cpp:28-54).
+// ReduceMean: reduce<int64_t, int16_t> (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:18-56).
+#include "espdl_device.h"
+#include "espdl_kernels.h"
+
+namespace espdl {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ int clamp_s16(int v)
+{
+    return min(max(v, -32768), 32767);
+}
+
+struct Binary16Args {
+    const int16_t *in0, *in1;
+    int16_t *out;
+    int dims[4];
+    long long s0[4], s1[4];
+    long long total;
+    int shift, half_even;
+    float rescale;
+};
+
+template <bool MUL>
+__global__ __launch_bounds__(kThreads) void binary_s16_kernel(const Binary16Args a)
+{
+    for (long long i = (long long)blockIdx.x * kThreads + threadIdx.x; i < a.total; i += (long long)gridDim.x * kThreads) {
+        long long rem = i, o0 = 0, o1 = 0;
+#pragma unroll
+        for (int d = 3; d >= 0; d--) {
+            const long long q = rem / a.dims[d];
+            const long long idx = rem - q * a.dims[d];
+            o0 += idx * a.s0[d];
+            o1 += idx * a.s1[d];
+            rem = q;
+        }
+        const int x = a.in0[o0], y = a.in1[o1];
+        int r;
+        if (MUL) {
+            const int prod = x * y; // at most 2^30 in magnitude
+            if (a.half_even && a.shift > 0) {
+                const long long q = (long long)prod >> a.shift;
+                const long long frac = (long long)prod & ((1ll << a.shift) - 1), half = 1ll << (a.shift - 1);
+                r = (int)min(max(q + ((frac > half || (frac == half && (q & 1))) ? 1 : 0), -32768ll), 32767ll);
+            } else {
+                r = clamp_s16(round_half_up_f32((float)prod * a.rescale));
+            }
+        } else {
+            r = clamp_s16(x + y);
+        }
+        a.out[i] = (int16_t)r;
+    }
+}
+
+struct Pool16Args {
+    const int16_t *in;
+    int16_t *out;
+    int h, w, c, out_h, out_w, k_h, k_w, stride_h, stride_w, pad_top, pad_left;
+    long long total;
+    float scale;
+};
+
+__global__ __launch_bounds__(kThreads) void avg_pool_s16_kernel(const Pool16Args a)
+{
+    for (long long i = (long long)blockIdx.x * kThreads + threadIdx.x; i < a.total; i += (long long)gridDim.x * kThreads) {
+        const long long pix = i / a.c;
+        const int ch = (int)(i - pix * a.c);
+        const long long row = pix / a.out_w;
+        const int x = (int)(pix - row * a.out_w);
+        const long long n = row / a.out_h;
+        const int y = (int)(row - n * a.out_h);
+        const int iy0 = y * a.stride_h - a.pad_top, ix0 = x * a.stride_w - a.pad_left;
+        int sum = 0;
+        for (int ky = max(0, -iy0); ky < min(a.k_h, a.h - iy0); ky++)
+            for (int kx = max(0, -ix0); kx < min(a.k_w, a.w - ix0); kx++)
+                sum += a.in[((n * a.h + iy0 + ky) * a.w + ix0 + kx) * a.c + ch];
+        a.out[i] = (int16_t)clamp_s16(round_half_up_f32((float)sum * a.scale));
+    }
+}
+
+struct Reduce16Args {
+    const int16_t *in;
+    int16_t *out;
+    int n_kept, n_red;
+    int kept_shape[8], red_shape[8];
+    long long kept_stride[8], red_stride[8];
+    long long n_out, count;
+    float input_scale, output_scale;
+};
+
+__global__ __launch_bounds__(kThreads) void reduce_mean_s16_kernel(const Reduce16Args a)
+{
+    for (long long o = (long long)blockIdx.x * kThreads + threadIdx.x; o < a.n_out; o += (long long)gridDim.x * kThreads) {
+        long long rem = o, base = 0;
+        for (int d = a.n_kept - 1; d >= 0; d--) {
+            const long long q = rem / a.kept_shape[d];
+            base += (rem - q * a.kept_shape[d]) * a.kept_stride[d];
+            rem = q;
+        }
+        long long sum = 0;
+        for (long long r = 0; r < a.count; r++) {
+            long long rr = r, off = base;
+            for (int d = a.n_red - 1; d >= 0; d--) {
+                const long long q = rr / a.red_shape[d];
+                off += (rr - q * a.red_shape[d]) * a.red_stride[d];
+                rr = q;
+            }
+            sum += a.in[off];
+        }
+        const float v = (float)sum * a.input_scale / (float)a.count * a.output_scale;
+        a.out[o] = (int16_t)clamp_s16(round_half_up_f32(v));
+    }
+}
+
+unsigned blocks_for(long long total, int cu_count)
+{
+    return (unsigned)max(1ll, min((total + kThreads - 1) / kThreads, (long long)max(1, cu_count) * 16));
+}
+
+} // namespace
+
+hipError_t launch_binary_s16(bool mul, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int16_t *in0,
+                             const int16_t *in1, int shift, bool half_even, int16_t *out, int cu_count, hipStream_t stream)
+{
+    Binary16Args a = {};
+    a.in0 = in0;
+    a.in1 = in1;
+    a.out = out;
+    a.total = 1;
+    for (int i = 0; i < 4; i++) {
+        a.dims[i] = dims[i];
+        a.s0[i] = s0[i];
+        a.s1[i] = s1[i];
+        a.total *= dims[i];
+    }
+    if (a.total <= 0)
+        return hipSuccess;
+    a.shift = shift;
+    a.half_even = half_even;
+    a.rescale = dl_rescale(shift);
+    if (mul)
+        binary_s16_kernel<true><<<dim3(blocks_for(a.total, cu_count)), dim3(kThreads), 0, stream>>>(a);
+    else
+        binary_s16_kernel<false><<<dim3(blocks_for(a.total, cu_count)), dim3(kThreads), 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+hipError_t launch_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
+                               int stride_w, int pad_top, int pad_left, int out_h, int out_w, int in_exp, int out_exp,
+                               int16_t *out, int cu_count, hipStream_t stream)
+{
+    Pool16Args a = {};
+    a.in = in;
+    a.out = out;
+    a.h = h;
+    a.w = w;
+    a.c = c;
+    a.out_h = out_h;
+    a.out_w = out_w;
+    a.k_h = k_h;
+    a.k_w = k_w;
+    a.stride_h = stride_h;
+    a.stride_w = stride_w;
+    a.pad_top = pad_top;
+    a.pad_left = pad_left;
+    a.total = (long long)batch * out_h * out_w * c;
+    if (a.total <= 0)
+        return hipSuccess;
+    const float area_inv = 1.f / (float)(k_h * k_w);
+    a.scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
+    avg_pool_s16_kernel<<<dim3(blocks_for(a.total, cu_count)), dim3(kThreads), 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+hipError_t launch_reduce_mean_s16(const int16_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
+                                  int out_exp, int16_t *out, int cu_count, hipStream_t stream)
+{
+    Reduce16Args a = {};
+    a.in = in;
+    a.out = out;
+    long long stride[8];
+    stride[dims - 1] = 1;
+    for (int i = dims - 2; i >= 0; i--)
+        stride[i] = stride[i + 1] * shape[i + 1];
+    a.n_out = 1;
+    a.count = 1;
+    for (int i = 0; i < dims; i++) {
+        if (reduce_flag[i]) {
+            a.red_shape[a.n_red] = shape[i];
+            a.red_stride[a.n_red++] = stride[i];
+            a.count *= shape[i];
+        } else {
+            a.kept_shape[a.n_kept] = shape[i];
+            a.kept_stride[a.n_kept++] = stride[i];
+            a.n_out *= shape[i];
+        }
+    }
+    if (a.n_out <= 0 || a.count <= 0)
+        return hipSuccess;
+    a.input_scale = dl_scale(in_exp);
+    a.output_scale = dl_rescale(out_exp);
+    reduce_mean_s16_kernel<<<dim3(blocks_for(a.n_out, cu_count)), dim3(kThreads), 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+} // namespace espdl

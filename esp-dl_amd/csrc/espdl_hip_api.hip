@@ -764,6 +764,96 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
                          "mbconv_s8_fused");
 }
 
+static int binary_s16(bool mul, const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int32_t mul_shift, int32_t round_mode, int16_t *out,
+                      void *stream)
+{
+    if (out_dims == nullptr || in0_strides == nullptr || in1_strides == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "dims and strides must not be NULL");
+    if (mul_shift < -30 || mul_shift > 30)
+        return fail(ESPDL_HIP_EINVAL, "mul_shift %d outside [-30, 30]", mul_shift);
+    if (round_mode != ESPDL_HIP_ROUND_HALF_UP && round_mode != ESPDL_HIP_ROUND_HALF_EVEN)
+        return fail(ESPDL_HIP_EINVAL, "bad round_mode %d", round_mode);
+    long long size = 1;
+    for (int i = 0; i < 4; i++) {
+        if (out_dims[i] < 0 || in0_strides[i] < 0 || in1_strides[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative extent or stride in dim %d", i);
+        size *= out_dims[i];
+        if (size > (1ll << 40))
+            return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    }
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in0 == nullptr || in1 == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in0, in1 and out must not be NULL");
+    return device_status(espdl::launch_binary_s16(mul, out_dims, in0_strides, in1_strides, in0, in1, mul_shift,
+                                                  round_mode == ESPDL_HIP_ROUND_HALF_EVEN, out, cu_count_cached(),
+                                                  reinterpret_cast<hipStream_t>(stream)),
+                         mul ? "mul_s16" : "add_s16");
+}
+
+int espdl_hip_add_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int16_t *out, void *stream)
+{
+    return binary_s16(false, out_dims, in0_strides, in1_strides, in0, in1, 0, ESPDL_HIP_ROUND_HALF_UP, out, stream);
+}
+
+int espdl_hip_mul_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int32_t mul_shift, int32_t round_mode, int16_t *out,
+                      void *stream)
+{
+    return binary_s16(true, out_dims, in0_strides, in1_strides, in0, in1, mul_shift, round_mode, out, stream);
+}
+
+int espdl_hip_avg_pool_s16(const int16_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,
+                           int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom, int32_t pad_left,
+                           int32_t pad_right, int32_t in_exp, int32_t out_exp, int16_t *out, void *stream)
+{
+    if (batch < 0 || h <= 0 || w <= 0 || c <= 0 || k_h <= 0 || k_w <= 0 || stride_h <= 0 || stride_w <= 0 || pad_top < 0 ||
+        pad_bottom < 0 || pad_left < 0 || pad_right < 0 || (long long)k_h * k_w > (1 << 15))
+        return fail(ESPDL_HIP_EINVAL, "bad avg_pool geometry");
+    if (h + pad_top + pad_bottom < k_h || w + pad_left + pad_right < k_w)
+        return fail(ESPDL_HIP_EINVAL, "window larger than the padded image");
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    const int out_h = (h + pad_top + pad_bottom - k_h) / stride_h + 1, out_w = (w + pad_left + pad_right - k_w) / stride_w + 1;
+    if (batch == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_avg_pool_s16(in, batch, h, w, c, k_h, k_w, stride_h, stride_w, pad_top, pad_left,
+                                                    out_h, out_w, in_exp, out_exp, out, cu_count_cached(),
+                                                    reinterpret_cast<hipStream_t>(stream)),
+                         "avg_pool_s16");
+}
+
+int espdl_hip_reduce_mean_s16(const int16_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
+                              int32_t in_exp, int32_t out_exp, int16_t *out, void *stream)
+{
+    if (dims < 1 || dims > 8 || shape == nullptr || reduce_flag == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "reduce_mean handles 1..8 dims");
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    int sh[8], fl[8];
+    long long total = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative extent");
+        sh[i] = shape[i];
+        fl[i] = reduce_flag[i] != 0;
+        total *= shape[i];
+        if (total > (1ll << 40))
+            return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    }
+    if (total == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    return device_status(espdl::launch_reduce_mean_s16(in, sh, dims, fl, in_exp, out_exp, out, cu_count_cached(),
+                                                       reinterpret_cast<hipStream_t>(stream)),
+                         "reduce_mean_s16");
+}
+
 int espdl_hip_insert_zeros(const void *in, int32_t elem_size, int32_t batch, int32_t h, int32_t w, int32_t c,
                            int32_t stride_h, int32_t stride_w, int32_t output_padding_h, int32_t output_padding_w,
                            void *out, void *stream)

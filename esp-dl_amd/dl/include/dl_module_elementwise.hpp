@@ -331,17 +331,21 @@ public:
         TensorBase *input0 = context->get_tensor(m_inputs_index[0]);
         TensorBase *input1 = context->get_tensor(m_inputs_index[1]);
         TensorBase *output = context->get_tensor(m_outputs_index[0]);
-        if (quant_type != QUANT_TYPE_SYMM_8BIT || !on_device_all({input0, input1, output}) ||
-            output->shape.size() > 4) {
-            DL_LOGE("Add", "%s: needs int8 device tensors of rank <= 4", name.c_str());
+        if ((quant_type != QUANT_TYPE_SYMM_8BIT && quant_type != QUANT_TYPE_SYMM_16BIT) ||
+            !on_device_all({input0, input1, output}) || output->shape.size() > 4) {
+            DL_LOGE("Add", "%s: needs int8 or int16 device tensors of rank <= 4", name.c_str());
             return;
         }
         int32_t dims[4];
         int64_t s0[4], s1[4];
         broadcast_layout(input0, input1, output, dims, s0, s1);
-        const int rc = espdl_hip_add_s8(dims, s0, s1, static_cast<const int8_t *>(input0->data),
-                                        static_cast<const int8_t *>(input1->data), static_cast<int8_t *>(output->data),
-                                        context->stream);
+        const int rc = quant_type == QUANT_TYPE_SYMM_16BIT
+            ? espdl_hip_add_s16(dims, s0, s1, static_cast<const int16_t *>(input0->data),
+                                static_cast<const int16_t *>(input1->data), static_cast<int16_t *>(output->data),
+                                context->stream)
+            : espdl_hip_add_s8(dims, s0, s1, static_cast<const int8_t *>(input0->data),
+                               static_cast<const int8_t *>(input1->data), static_cast<int8_t *>(output->data),
+                               context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("Add", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
@@ -394,20 +398,23 @@ public:
         TensorBase *input0 = context->get_tensor(m_inputs_index[0]);
         TensorBase *input1 = context->get_tensor(m_inputs_index[1]);
         TensorBase *output = context->get_tensor(m_outputs_index[0]);
-        if (quant_type != QUANT_TYPE_SYMM_8BIT || !on_device_all({input0, input1, output}) ||
-            output->shape.size() > 4) {
-            DL_LOGE("Mul", "%s: needs int8 device tensors of rank <= 4", name.c_str());
+        if ((quant_type != QUANT_TYPE_SYMM_8BIT && quant_type != QUANT_TYPE_SYMM_16BIT) ||
+            !on_device_all({input0, input1, output}) || output->shape.size() > 4) {
+            DL_LOGE("Mul", "%s: needs int8 or int16 device tensors of rank <= 4", name.c_str());
             return;
         }
         int32_t dims[4];
         int64_t s0[4], s1[4];
         broadcast_layout(input0, input1, output, dims, s0, s1);
         const int shift = output->exponent.get() - input0->exponent.get() - input1->exponent.get();
-        const int rc = espdl_hip_mul_s8(dims, s0, s1, static_cast<const int8_t *>(input0->data),
-                                        static_cast<const int8_t *>(input1->data), shift,
-                                        context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN
-                                                                                    : ESPDL_HIP_ROUND_HALF_UP,
-                                        static_cast<int8_t *>(output->data), context->stream);
+        const int32_t rm = context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP;
+        const int rc = quant_type == QUANT_TYPE_SYMM_16BIT
+            ? espdl_hip_mul_s16(dims, s0, s1, static_cast<const int16_t *>(input0->data),
+                                static_cast<const int16_t *>(input1->data), shift, rm,
+                                static_cast<int16_t *>(output->data), context->stream)
+            : espdl_hip_mul_s8(dims, s0, s1, static_cast<const int8_t *>(input0->data),
+                               static_cast<const int8_t *>(input1->data), shift, rm, static_cast<int8_t *>(output->data),
+                               context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("Mul", "%s: %s", name.c_str(), espdl_hip_last_error());
     }

@@ -427,8 +427,8 @@ public:
         (void)mode;
         TensorBase *input = context->get_tensor(m_inputs_index[0]);
         TensorBase *output = context->get_tensor(m_outputs_index[0]);
-        if (!on_device_all({input, output}) || quant_type != QUANT_TYPE_SYMM_8BIT) {
-            DL_LOGE("AveragePool", "%s: needs int8 device tensors", name.c_str());
+        if (!on_device_all({input, output}) || (quant_type != QUANT_TYPE_SYMM_8BIT && quant_type != QUANT_TYPE_SYMM_16BIT)) {
+            DL_LOGE("AveragePool", "%s: needs int8 or int16 device tensors", name.c_str());
             return;
         }
         const bool nwc = input->shape.size() == 3;
@@ -438,9 +438,13 @@ public:
         const int sh = nwc ? 1 : m_strides[0], sw = nwc ? m_strides[0] : m_strides[1];
         const int pt = nwc ? 0 : m_pads[0], pb = nwc ? 0 : m_pads[1];
         const int pl = nwc ? m_pads[0] : m_pads[2], pr = nwc ? m_pads[1] : m_pads[3];
-        const int rc = espdl_hip_avg_pool_s8(static_cast<const int8_t *>(input->data), input->shape[0], h, w, c, kh, kw, sh,
-                                             sw, pt, pb, pl, pr, input->exponent.get(), output->exponent.get(),
-                                             static_cast<int8_t *>(output->data), context->stream);
+        const int rc = quant_type == QUANT_TYPE_SYMM_16BIT
+            ? espdl_hip_avg_pool_s16(static_cast<const int16_t *>(input->data), input->shape[0], h, w, c, kh, kw, sh, sw, pt,
+                                     pb, pl, pr, input->exponent.get(), output->exponent.get(),
+                                     static_cast<int16_t *>(output->data), context->stream)
+            : espdl_hip_avg_pool_s8(static_cast<const int8_t *>(input->data), input->shape[0], h, w, c, kh, kw, sh, sw, pt,
+                                    pb, pl, pr, input->exponent.get(), output->exponent.get(),
+                                    static_cast<int8_t *>(output->data), context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("AveragePool", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
@@ -609,15 +613,19 @@ public:
         (void)mode;
         TensorBase *input = context->get_tensor(m_inputs_index[0]);
         TensorBase *output = context->get_tensor(m_outputs_index[0]);
-        if (!on_device_all({input, output}) || quant_type != QUANT_TYPE_SYMM_8BIT || input->shape.size() > 8) {
-            DL_LOGE("ReduceMean", "%s: needs int8 device tensors of at most 8 dims", name.c_str());
+        if (!on_device_all({input, output}) || (quant_type != QUANT_TYPE_SYMM_8BIT && quant_type != QUANT_TYPE_SYMM_16BIT) ||
+            input->shape.size() > 8) {
+            DL_LOGE("ReduceMean", "%s: needs int8 or int16 device tensors of at most 8 dims", name.c_str());
             return;
         }
         const std::vector<int32_t> f = flags_for(input->shape.size());
-        const int rc = espdl_hip_reduce_mean_s8(static_cast<const int8_t *>(input->data), input->shape.data(),
-                                                (int32_t)input->shape.size(), f.data(), input->exponent.get(),
-                                                output->exponent.get(), static_cast<int8_t *>(output->data),
-                                                context->stream);
+        const int rc = quant_type == QUANT_TYPE_SYMM_16BIT
+            ? espdl_hip_reduce_mean_s16(static_cast<const int16_t *>(input->data), input->shape.data(),
+                                        (int32_t)input->shape.size(), f.data(), input->exponent.get(),
+                                        output->exponent.get(), static_cast<int16_t *>(output->data), context->stream)
+            : espdl_hip_reduce_mean_s8(static_cast<const int8_t *>(input->data), input->shape.data(),
+                                       (int32_t)input->shape.size(), f.data(), input->exponent.get(),
+                                       output->exponent.get(), static_cast<int8_t *>(output->data), context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("ReduceMean", "%s: %s", name.c_str(), espdl_hip_last_error());
     }

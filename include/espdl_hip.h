@@ -206,6 +206,24 @@ int espdl_hip_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w,
 int espdl_hip_reduce_mean_s8(const int8_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
                              int32_t in_exp, int32_t out_exp, int8_t *out, void *stream);
 
+/* int16 forms.  espdl_hip_add_s16: c_impl_add_n_n<int16_t> (esp-dl/dl/base/dl_base_add.cpp:33-44), saturating
+ * add.  espdl_hip_mul_s16: c_impl_mul_n_n<int16_t> (esp-dl/dl/base/dl_base_mul.cpp:33-46): the int32 product is
+ * converted to float32, scaled by 2^-mul_shift and rounded half up (ESPDL_HIP_ROUND_HALF_UP), or shifted and
+ * rounded half to even as an integer (ESPDL_HIP_ROUND_HALF_EVEN, the ESP32-P4 kernels).  Broadcast description
+ * as espdl_hip_add_s8.  espdl_hip_avg_pool_s16: avgpool2d_hwc<int16_t, int32_t> (dl_base_avg_pool2d.cpp:28-54,
+ * :87), arguments as espdl_hip_avg_pool_s8.  espdl_hip_reduce_mean_s16: reduce<int64_t, int16_t>
+ * (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:18-56), arguments as espdl_hip_reduce_mean_s8. */
+int espdl_hip_add_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int16_t *out, void *stream);
+int espdl_hip_mul_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int32_t mul_shift, int32_t round_mode, int16_t *out,
+                      void *stream);
+int espdl_hip_avg_pool_s16(const int16_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,
+                           int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom, int32_t pad_left,
+                           int32_t pad_right, int32_t in_exp, int32_t out_exp, int16_t *out, void *stream);
+int espdl_hip_reduce_mean_s16(const int16_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
+                              int32_t in_exp, int32_t out_exp, int16_t *out, void *stream);
+
 /* module::InsertZeros (esp-dl/dl/module/include/dl_module_insert_zeros.hpp; the exporter places it in front of
  * a Conv to express a transposed convolution): in is [batch][h][w][c] of elem_size-byte elements, out is
  * [batch][out_h][out_w][c] with out_h = h + (stride_h - 1) * (h - 1) + output_padding_h (same for w);

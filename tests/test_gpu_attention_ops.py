@@ -156,3 +156,41 @@ def test_lut_s16_rejects_odd_table_sizes():
     x = torch.zeros(8, dtype=torch.int16, device="cuda")
     with pytest.raises(m.EspdlHipError):
         m.lut_s16(x, torch.zeros(1000, dtype=torch.int16, device="cuda"))
+
+
+def test_add_s16(oracle):
+    announce("add_s16")
+    rng = np.random.default_rng(60)
+    a, b = _rand(rng, (3, 7, 33), np.int16), _rand(rng, (3, 7, 33), np.int16)
+    np.testing.assert_array_equal(to_host(espdl().add_s16(to_dev(a), to_dev(b))), oracle.add_s16(a, b))
+    # broadcast over the last axis
+    c = _rand(rng, (3, 7, 1), np.int16)
+    want = np.clip(a.astype(np.int32) + c.astype(np.int32), -32768, 32767).astype(np.int16)
+    np.testing.assert_array_equal(to_host(espdl().add_s16(to_dev(a), to_dev(c))), want)
+
+
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+@pytest.mark.parametrize("shift", [0, 7, 13, 15, 22])
+def test_mul_s16(oracle, shift, round_mode):
+    announce(f"mul_s16 shift={shift} round_mode={round_mode}")
+    rng = np.random.default_rng(61)
+    a, b = _rand(rng, (50021,), np.int16), _rand(rng, (50021,), np.int16)
+    a[:4], b[:4] = [-32768, 32767, -32768, 4097], [-32768, 32767, 32767, 4099]
+    got = to_host(espdl().mul_s16(to_dev(a), to_dev(b), shift, round_mode))
+    np.testing.assert_array_equal(got, oracle.mul_s16(a, b, shift, round_mode))
+    s = _rand(rng, (1,), np.int16)
+    got = to_host(espdl().mul_s16(to_dev(a), to_dev(s), shift, round_mode))
+    np.testing.assert_array_equal(got, oracle.mul_s16(a, s, shift, round_mode))
+
+
+def test_avg_pool_and_reduce_mean_s16(oracle):
+    announce("avg_pool_s16 / reduce_mean_s16")
+    rng = np.random.default_rng(62)
+    x = _rand(rng, (3, 12, 9, 20), np.int16)
+    for k, st, pads, ei, eo in (((3, 3), (2, 2), (1, 1, 1, 1), -10, -9), ((2, 2), (2, 2), (0, 0, 0, 0), -12, -12),
+                                ((1, 9), (1, 1), (0, 0, 0, 0), -8, -11)):
+        got = to_host(espdl().avg_pool_s16(to_dev(x), k, st, pads, ei, eo))
+        np.testing.assert_array_equal(got, oracle.avg_pool_s16(x, k, st, pads, ei, eo))
+    for axes, keep in (([1, 2], True), ([3], False), ([0, 2], True), ([], True)):
+        got = to_host(espdl().reduce_mean_s16(to_dev(x), axes, keep, -10, -12))
+        np.testing.assert_array_equal(got, oracle.reduce_mean_s16(x, axes, keep, -10, -12))
