@@ -726,3 +726,34 @@ def attention_block(seed=0xE5D8, hw=10, heads=2, key_dim=16, head_dim=32):
     o = b.add(o, pe, name="o_pe")
     b.output(b.conv(o, c, k=1, name="proj"))
     return g
+
+
+def int16_tail(seed=0xE5D9):
+    """int8 Conv -> RequantizeLinear to int16 -> int16 Conv -> int16 table (SiLU) -> int16 Add (residual) ->
+    int16 Mul by a constant -> int16 AveragePool -> int16 ReduceMean -> int16 Gemm: the operator mix of the
+    reference's int16 text recognizer."""
+    g = GraphSpec("int16_tail")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 12, 16, 16], -5)
+    h = b.conv(x, 32, k=3, relu=True, name="c1")
+    h16 = "to_s16_out"
+    g.add_value(h16, g.shape(h), g.exponent(h) - 8, INT16)
+    g.add_node("to_s16", "RequantizeLinear", [h], [h16], quant_type="S16")
+    c2 = b.conv(h16, 32, k=1, s16=True, out_exp=g.exponent(h16) + 3, name="c2")
+    act = b.lut_s16(c2, silu, name="c2_silu")
+    res = "res_out"
+    g.add_value(res, g.shape(act), g.exponent(act), INT16)
+    g.add_node("res", "Add", [act, c2], [res], quant_type="S16")
+    g.add_init("gain", [1], INT16, [23170], [-15])       # ~ 0.707 at exponent -15
+    sc = "scaled_out"
+    g.add_value(sc, g.shape(res), g.exponent(res), INT16)
+    g.add_node("scaled", "Mul", [res, "gain"], [sc], quant_type="S16")
+    ap = "pool_out"
+    g.add_value(ap, [1, 6, 8, 32], g.exponent(sc), INT16)
+    g.add_node("pool", "AveragePool", [sc], [ap], kernel_shape=[2, 2], strides=[2, 2], pads=[0, 0, 0, 0], quant_type="S16")
+    g.add_init("mean.axes", [1], INT64, [1], [0])
+    mn = "mean_out"
+    g.add_value(mn, [1, 1, 8, 32], g.exponent(ap) - 1, INT16)
+    g.add_node("mean", "ReduceMean", [ap, "mean.axes"], [mn], keepdims=1, noop_with_empty_axes=0, quant_type="S16")
+    g.outputs.append(mn)
+    return g

@@ -245,6 +245,19 @@ def test_attention_block(oracle, round_mode):
     mdl.close()
 
 
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+def test_int16_tail(oracle, round_mode):
+    """int16 table, Add, Mul by a constant, AveragePool and ReduceMean behind an int8 -> int16 requantize."""
+    announce(f"model int16_tail round_mode={round_mode}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.int16_tail()
+    mdl, want, _ = _run_config(spec, 3, 37, round_mode=round_mode)
+    got = mdl.get_tensor(spec.outputs[0], np.int16)
+    np.testing.assert_array_equal(got, want[spec.outputs[0]])
+    assert want[spec.outputs[0]].min() < want[spec.outputs[0]].max()
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()
