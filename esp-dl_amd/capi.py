@@ -82,7 +82,9 @@ def lib():
         L.espdl_hip_mul_s16.argtypes = [vp, vp, vp, vp, vp, i32, i32, vp, vp]
         L.espdl_hip_avg_pool_s16.argtypes = [vp] + [i32] * 14 + [vp, vp]
         L.espdl_hip_reduce_mean_s16.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
-        for name in ("add_s16", "mul_s16", "avg_pool_s16", "reduce_mean_s16"):
+        L.espdl_hip_sub_s16.argtypes = [vp, vp, vp, vp, vp, vp, vp]
+        L.espdl_hip_div_s16.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp]
+        for name in ("add_s16", "mul_s16", "sub_s16", "div_s16", "avg_pool_s16", "reduce_mean_s16"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         L.espdl_hip_insert_zeros.argtypes = [vp] + [i32] * 9 + [vp, vp]
         L.espdl_hip_insert_zeros.restype = ctypes.c_int
@@ -505,3 +507,18 @@ def reduce_mean_s16(x, axes, keepdims=True, in_exp=0, out_exp=0, stream=None):
     _check(lib().espdl_hip_reduce_mean_s16(_p(x), (ctypes.c_int32 * nd)(*x.shape), nd, (ctypes.c_int32 * nd)(*flags),
                                            in_exp, out_exp, _p(out), _stream(stream)))
     return out.reshape([1 if flags[i] else int(x.shape[i]) for i in range(nd)]) if keepdims else out
+
+
+def sub_s16(a, b, stream=None):
+    dims, s0, s1, out = _broadcast16(a, b)
+    _check(lib().espdl_hip_sub_s16(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), _p(out),
+                                   _stream(stream)))
+    return out
+
+
+def div_s16(a, b, shift, stream=None):
+    """shift = out_exp - a_exp + b_exp."""
+    dims, s0, s1, out = _broadcast16(a, b)
+    _check(lib().espdl_hip_div_s16(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), int(shift),
+                                   _p(out), _stream(stream)))
+    return out

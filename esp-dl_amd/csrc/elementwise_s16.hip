@@ -5,6 +5,7 @@
 // Mul: c_impl_mul_n_n<int16_t> (esp-dl/dl/base/dl_base_mul.cpp:33-46): the int32 product goes through
 //      float32, is scaled by 2^-shift and rounded half up; with ESP32-P4 semantics the exact product is
 //      shifted and rounded half to even.
+// Sub: c_impl_sub_n_n<int16_t> (esp-dl/dl/base/dl_base_sub.cpp:33-43).  Div: esp-dl/dl/base/dl_base_div.cpp, float32.
 // AveragePool: avgpool2d_hwc<int16_t, int32_t> (esp-dl/dl/base/dl_base_avg_pool2d.cpp:28-54).
 // ReduceMean: reduce<int64_t, int16_t> (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:18-56).
 #include "espdl_device.h"
@@ -30,7 +31,8 @@ struct Binary16Args {
     float rescale;
 };
 
-template <bool MUL>
+// OP: 0 add, 1 mul, 2 sub, 3 div
+template <int OP>
 __global__ __launch_bounds__(kThreads) void binary_s16_kernel(const Binary16Args a)
 {
     for (long long i = (long long)blockIdx.x * kThreads + threadIdx.x; i < a.total; i += (long long)gridDim.x * kThreads) {
@@ -45,7 +47,29 @@ __global__ __launch_bounds__(kThreads) void binary_s16_kernel(const Binary16Args
         }
         const int x = a.in0[o0], y = a.in1[o1];
         int r;
-        if (MUL) {
+        if (OP == 3) {
+            // c_impl_div_n_n / _n_1 / _1_n (esp-dl/dl/base/dl_base_div.cpp:92-112, 141-163, 175-195): float32, the
+            // order of the two operations depends on which operand is constant along the innermost axis
+            if (x == 0) {
+                r = 0;
+            } else if (y == 0) {
+                r = x > 0 ? 32767 : -32768;
+            } else {
+                float v;
+                if (a.shift == 1) {
+                    const float q = a.rescale / (float)y;
+                    v = (float)x * q;
+                } else if (a.shift == 2) {
+                    const float q = (float)x * a.rescale;
+                    v = q / (float)y;
+                } else {
+                    v = (float)x * a.rescale / (float)y;
+                }
+                r = clamp_s16(round_half_up_f32(v));
+            }
+        } else if (OP == 2) {
+            r = clamp_s16(x - y);
+        } else if (OP == 1) {
             const int prod = x * y; // at most 2^30 in magnitude
             if (a.half_even && a.shift > 0) {
                 const long long q = (long long)prod >> a.shift;
@@ -128,7 +152,7 @@ unsigned blocks_for(long long total, int cu_count)
 
 } // namespace
 
-hipError_t launch_binary_s16(bool mul, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int16_t *in0,
+hipError_t launch_binary_s16(int op, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int16_t *in0,
                              const int16_t *in1, int shift, bool half_even, int16_t *out, int cu_count, hipStream_t stream)
 {
     Binary16Args a = {};
@@ -147,10 +171,24 @@ hipError_t launch_binary_s16(bool mul, const int32_t dims[4], const int64_t s0[4
     a.shift = shift;
     a.half_even = half_even;
     a.rescale = dl_rescale(shift);
-    if (mul)
-        binary_s16_kernel<true><<<dim3(blocks_for(a.total, cu_count)), dim3(kThreads), 0, stream>>>(a);
-    else
-        binary_s16_kernel<false><<<dim3(blocks_for(a.total, cu_count)), dim3(kThreads), 0, stream>>>(a);
+    const dim3 grid(blocks_for(a.total, cu_count));
+    if (op == 3) {
+        // the loop form: 1 = divisor constant along the innermost axis longer than 1, 2 = dividend constant
+        int form = 1;
+        for (int d = 3; d >= 0; d--)
+            if (dims[d] > 1) {
+                form = s1[d] == 0 ? 1 : (s0[d] == 0 ? 2 : 0);
+                break;
+            }
+        a.shift = form;
+        binary_s16_kernel<3><<<grid, dim3(kThreads), 0, stream>>>(a);
+    } else if (op == 2) {
+        binary_s16_kernel<2><<<grid, dim3(kThreads), 0, stream>>>(a);
+    } else if (op == 1) {
+        binary_s16_kernel<1><<<grid, dim3(kThreads), 0, stream>>>(a);
+    } else {
+        binary_s16_kernel<0><<<grid, dim3(kThreads), 0, stream>>>(a);
+    }
     return hipGetLastError();
 }
 

@@ -764,7 +764,7 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
                          "mbconv_s8_fused");
 }
 
-static int binary_s16(bool mul, const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+static int binary_s16(int op, const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
                       const int16_t *in0, const int16_t *in1, int32_t mul_shift, int32_t round_mode, int16_t *out,
                       void *stream)
 {
@@ -786,23 +786,36 @@ static int binary_s16(bool mul, const int32_t out_dims[4], const int64_t in0_str
         return ESPDL_HIP_OK;
     if (in0 == nullptr || in1 == nullptr || out == nullptr)
         return fail(ESPDL_HIP_EINVAL, "in0, in1 and out must not be NULL");
-    return device_status(espdl::launch_binary_s16(mul, out_dims, in0_strides, in1_strides, in0, in1, mul_shift,
+    static const char *const names[4] = {"add_s16", "mul_s16", "sub_s16", "div_s16"};
+    return device_status(espdl::launch_binary_s16(op, out_dims, in0_strides, in1_strides, in0, in1, mul_shift,
                                                   round_mode == ESPDL_HIP_ROUND_HALF_EVEN, out, cu_count_cached(),
                                                   reinterpret_cast<hipStream_t>(stream)),
-                         mul ? "mul_s16" : "add_s16");
+                         names[op & 3]);
 }
 
 int espdl_hip_add_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
                       const int16_t *in0, const int16_t *in1, int16_t *out, void *stream)
 {
-    return binary_s16(false, out_dims, in0_strides, in1_strides, in0, in1, 0, ESPDL_HIP_ROUND_HALF_UP, out, stream);
+    return binary_s16(0, out_dims, in0_strides, in1_strides, in0, in1, 0, ESPDL_HIP_ROUND_HALF_UP, out, stream);
 }
 
 int espdl_hip_mul_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
                       const int16_t *in0, const int16_t *in1, int32_t mul_shift, int32_t round_mode, int16_t *out,
                       void *stream)
 {
-    return binary_s16(true, out_dims, in0_strides, in1_strides, in0, in1, mul_shift, round_mode, out, stream);
+    return binary_s16(1, out_dims, in0_strides, in1_strides, in0, in1, mul_shift, round_mode, out, stream);
+}
+
+int espdl_hip_sub_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int16_t *out, void *stream)
+{
+    return binary_s16(2, out_dims, in0_strides, in1_strides, in0, in1, 0, ESPDL_HIP_ROUND_HALF_UP, out, stream);
+}
+
+int espdl_hip_div_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int32_t div_shift, int16_t *out, void *stream)
+{
+    return binary_s16(3, out_dims, in0_strides, in1_strides, in0, in1, div_shift, ESPDL_HIP_ROUND_HALF_UP, out, stream);
 }
 
 int espdl_hip_avg_pool_s16(const int16_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,

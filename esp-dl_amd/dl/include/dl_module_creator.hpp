@@ -58,6 +58,8 @@ public:
         register_module("Clip", Clip::deserialize);
         register_module("Add", Add::deserialize);
         register_module("Mul", Mul::deserialize);
+        register_module("Sub", SubDiv::deserialize_sub);
+        register_module("Div", SubDiv::deserialize_div);
         register_module("GlobalAveragePool", GlobalAveragePool::deserialize);
         register_module("RequantizeLinear", RequantizeLinear::deserialize);
         register_module("Flatten", Flatten::deserialize);

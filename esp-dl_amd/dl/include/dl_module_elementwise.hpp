@@ -427,6 +427,57 @@ public:
     void print() { DL_LOGI("Mul", "quant_type: %s.", quant_type_to_string(quant_type)); }
 };
 
+/// Sub and Div on int16 tensors with numpy-style broadcasting (esp-dl/dl/module/include/dl_module_sub.hpp,
+/// dl_module_div.hpp over base::elemwise_sub / base::elemwise_div).
+class SubDiv : public Add {
+private:
+    bool m_div;
+
+public:
+    SubDiv(bool div, const char *name = nullptr, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Add(name, MODULE_NON_INPLACE, quant_type), m_div(div)
+    {
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input0 = context->get_tensor(m_inputs_index[0]);
+        TensorBase *input1 = context->get_tensor(m_inputs_index[1]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        const char *tag = m_div ? "Div" : "Sub";
+        if (quant_type != QUANT_TYPE_SYMM_16BIT || !on_device_all({input0, input1, output}) || output->shape.size() > 4) {
+            DL_LOGE(tag, "%s: needs int16 device tensors of rank <= 4", name.c_str());
+            return;
+        }
+        int32_t dims[4];
+        int64_t s0[4], s1[4];
+        broadcast_layout(input0, input1, output, dims, s0, s1);
+        const int rc = m_div
+            ? espdl_hip_div_s16(dims, s0, s1, static_cast<const int16_t *>(input0->data),
+                                static_cast<const int16_t *>(input1->data),
+                                output->exponent.get() - input0->exponent.get() + input1->exponent.get(),
+                                static_cast<int16_t *>(output->data), context->stream)
+            : espdl_hip_sub_s16(dims, s0, s1, static_cast<const int16_t *>(input0->data),
+                                static_cast<const int16_t *>(input1->data), static_cast<int16_t *>(output->data),
+                                context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE(tag, "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize_sub(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        return new SubDiv(false, node_name.c_str(), quant_type);
+    }
+    static Module *deserialize_div(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        return new SubDiv(true, node_name.c_str(), quant_type);
+    }
+    void print() { DL_LOGI(m_div ? "Div" : "Sub", "quant_type: %s.", quant_type_to_string(quant_type)); }
+};
+
 class GlobalAveragePool : public Module {
 public:
     GlobalAveragePool(const char *name = nullptr, quant_type_t quant_type = QUANT_TYPE_NONE) :

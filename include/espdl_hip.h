@@ -218,6 +218,15 @@ int espdl_hip_add_s16(const int32_t out_dims[4], const int64_t in0_strides[4], c
 int espdl_hip_mul_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
                       const int16_t *in0, const int16_t *in1, int32_t mul_shift, int32_t round_mode, int16_t *out,
                       void *stream);
+/* base::elemwise_sub for int16 (esp-dl/dl/base/dl_base_sub.cpp:33-43): saturating in0 - in1. */
+int espdl_hip_sub_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int16_t *out, void *stream);
+/* base::elemwise_div for int16 (esp-dl/dl/base/dl_base_div.cpp:66-68, 92-112, 141-163, 175-195, 244-252): float32,
+ * div_shift = out_exp - in0_exp + in1_exp; out = round(in0 * 2^-div_shift / in1), evaluated in the order of the
+ * reference loop that matches the broadcast (divisor constant along the innermost axis: in0 * (2^-s / in1);
+ * dividend constant: (in0 * 2^-s) / in1); in0 == 0 gives 0, in1 == 0 the int16 extreme of in0's sign. */
+int espdl_hip_div_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                      const int16_t *in0, const int16_t *in1, int32_t div_shift, int16_t *out, void *stream);
 int espdl_hip_avg_pool_s16(const int16_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,
                            int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom, int32_t pad_left,
                            int32_t pad_right, int32_t in_exp, int32_t out_exp, int16_t *out, void *stream);

@@ -713,6 +713,48 @@ void espdl_oracle_mul_s16(const int16_t *in0, int64_t len0, const int16_t *in1, 
     }
 }
 
+/* Sub, int16 (c_impl_sub_n_n<int16_t>, esp-dl/dl/base/dl_base_sub.cpp:33-43): saturating integer subtraction. */
+void espdl_oracle_sub_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size,
+                          int16_t *out)
+{
+    for (int64_t i = 0; i < size; i++) {
+        const int32_t a = in0[len0 == 1 ? 0 : i], b = in1[len1 == 1 ? 0 : i];
+        out[i] = (int16_t)clamp_i64(a - b, INT16_MIN, INT16_MAX);
+    }
+}
+
+/*
+ * Div, int16 (esp-dl/dl/base/dl_base_div.cpp:66-68, 92-112, 141-163, 175-195): float32 arithmetic whose
+ * order depends on which operand is constant along the innermost axis.  rescale = 2^-shift with
+ * shift = out_exp - in0_exp + in1_exp.  form 0 (both vary): round(a * rescale / b); form 1 (divisor
+ * constant): round(a * (rescale / b)); form 2 (dividend constant): round((a * rescale) / b).  a == 0 gives
+ * 0, b == 0 gives the int16 extreme of a's sign.  Operands are passed already broadcast to `size`.
+ */
+void espdl_oracle_div_s16(const int16_t *in0, const int16_t *in1, int64_t size, int shift, int form, int16_t *out)
+{
+    const float rescale = dl_rescale(shift);
+    for (int64_t i = 0; i < size; i++) {
+        const int16_t a = in0[i], b = in1[i];
+        if (a == 0) {
+            out[i] = 0;
+        } else if (b == 0) {
+            out[i] = a > 0 ? INT16_MAX : INT16_MIN;
+        } else {
+            float v;
+            if (form == 1) {
+                const float r = rescale / (float)b;
+                v = (float)a * r;
+            } else if (form == 2) {
+                const float r = (float)a * rescale;
+                v = r / (float)b;
+            } else {
+                v = (float)a * rescale / (float)b;
+            }
+            out[i] = (int16_t)clamp_i64(round_half_up_f32(v), INT16_MIN, INT16_MAX);
+        }
+    }
+}
+
 /* AveragePool, int16 (avgpool2d_hwc<int16_t, int32_t>, esp-dl/dl/base/dl_base_avg_pool2d.cpp:28-54, :87). */
 void espdl_oracle_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                                int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,

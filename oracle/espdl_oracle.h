@@ -68,6 +68,10 @@
  *   espdl_oracle_mul_s16         numpy: int64 product -> float32 (round to nearest even) -> exact power-of-two
  *                                scaling -> exact rational round half up; half-even mode against the pinned
  *                                integer shift-round                                                  PINNED
+ *   espdl_oracle_sub_s16         numpy saturating subtraction                                        PINNED
+ *   espdl_oracle_div_s16         numpy float32 arithmetic in the same order for each of the three forms (IEEE
+ *                                operations, so the order is the whole content), and within one unit of the exact
+ *                                rational quotient                                                   PINNED
  *   espdl_oracle_avg_pool_s16, _reduce_mean_s16   as their int8 forms: exact rationals away from ties
  *                                                                                   PARITY UNPINNED (near-ties)
  *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
@@ -147,6 +151,9 @@ void espdl_oracle_add_s16(const int16_t *in0, int64_t len0, const int16_t *in1, 
                           int16_t *out);
 void espdl_oracle_mul_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size, int shift,
                           int round_mode, int16_t *out);
+void espdl_oracle_sub_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size,
+                          int16_t *out);
+void espdl_oracle_div_s16(const int16_t *in0, const int16_t *in1, int64_t size, int shift, int form, int16_t *out);
 void espdl_oracle_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                                int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,
                                int out_exp, int16_t *out);

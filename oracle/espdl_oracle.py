@@ -66,6 +66,10 @@ def lib():
         L.espdl_oracle_add_s16.argtypes = [vp, i64, vp, i64, i64, vp]
         L.espdl_oracle_mul_s16.restype = None
         L.espdl_oracle_mul_s16.argtypes = [vp, i64, vp, i64, i64, i32, i32, vp]
+        L.espdl_oracle_sub_s16.restype = None
+        L.espdl_oracle_sub_s16.argtypes = [vp, i64, vp, i64, i64, vp]
+        L.espdl_oracle_div_s16.restype = None
+        L.espdl_oracle_div_s16.argtypes = [vp, vp, i64, i32, i32, vp]
         L.espdl_oracle_avg_pool_s16.restype = None
         L.espdl_oracle_avg_pool_s16.argtypes = [vp] + [i32] * 14 + [vp]
         L.espdl_oracle_reduce_mean_s16.restype = i32
@@ -310,6 +314,39 @@ def add_s16(a, b):
     assert a.size in (1, size) and b.size in (1, size)
     out = np.empty(a.shape if a.size == size else b.shape, dtype=np.int16)
     lib().espdl_oracle_add_s16(_ptr(a), a.size, _ptr(b), b.size, size, _ptr(out))
+    return out
+
+
+def sub_s16(a, b):
+    a = _c(a, np.int16)
+    b = _c(b, np.int16)
+    size = max(a.size, b.size)
+    assert a.size in (1, size) and b.size in (1, size)
+    out = np.empty(a.shape if a.size == size else b.shape, dtype=np.int16)
+    lib().espdl_oracle_sub_s16(_ptr(a), a.size, _ptr(b), b.size, size, _ptr(out))
+    return out
+
+
+def div_form(shape_a, shape_b):
+    """Which of the reference's three loops runs: 1 if the divisor is constant along the innermost axis of the
+    result that is longer than 1, 2 if the dividend is, else 0."""
+    out = np.broadcast_shapes(tuple(shape_a), tuple(shape_b))
+    rank = len(out)
+    pa = (1,) * (rank - len(shape_a)) + tuple(shape_a)
+    pb = (1,) * (rank - len(shape_b)) + tuple(shape_b)
+    for d in range(rank - 1, -1, -1):
+        if out[d] > 1:
+            return 1 if pb[d] == 1 else (2 if pa[d] == 1 else 0)
+    return 1
+
+
+def div_s16(a, b, shift):
+    """numpy-broadcast quotient; shift = out_exp - a_exp + b_exp."""
+    form = div_form(np.shape(a), np.shape(b))
+    a, b = np.broadcast_arrays(np.asarray(a, dtype=np.int16), np.asarray(b, dtype=np.int16))
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    out = np.empty(a.shape, dtype=np.int16)
+    lib().espdl_oracle_div_s16(_ptr(a), _ptr(b), a.size, int(shift), form, _ptr(out))
     return out
 
 

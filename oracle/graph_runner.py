@@ -102,6 +102,18 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
                 x, b = np.broadcast_arrays(x, b)
             add = oracle.add_s16 if x.dtype == np.int16 else oracle.add_s8
             y = add(np.ascontiguousarray(x), np.ascontiguousarray(b))
+        elif op == "Sub":
+            b = operand(ins[1])
+            if x.dtype != np.int16:
+                raise NotImplementedError("Sub on " + str(x.dtype))
+            if x.shape != b.shape:
+                x, b = np.broadcast_arrays(x, b)
+            y = oracle.sub_s16(np.ascontiguousarray(x), np.ascontiguousarray(b))
+        elif op == "Div":
+            b = operand(ins[1])
+            if x.dtype != np.int16:
+                raise NotImplementedError("Div on " + str(x.dtype))
+            y = oracle.div_s16(x, b, spec.exponent(y_name) - exponent_of(ins[0]) + exponent_of(ins[1]))
         elif op == "Mul":
             b = operand(ins[1])
             shift = spec.exponent(y_name) - exponent_of(ins[0]) - exponent_of(ins[1])

@@ -194,3 +194,25 @@ def test_avg_pool_and_reduce_mean_s16(oracle):
     for axes, keep in (([1, 2], True), ([3], False), ([0, 2], True), ([], True)):
         got = to_host(espdl().reduce_mean_s16(to_dev(x), axes, keep, -10, -12))
         np.testing.assert_array_equal(got, oracle.reduce_mean_s16(x, axes, keep, -10, -12))
+
+
+def test_sub_s16(oracle):
+    announce("sub_s16")
+    rng = np.random.default_rng(63)
+    a, b = _rand(rng, (2, 286, 800), np.int16), _rand(rng, (2, 1, 800), np.int16)
+    want = np.clip(a.astype(np.int32) - b.astype(np.int32), -32768, 32767).astype(np.int16)
+    np.testing.assert_array_equal(to_host(espdl().sub_s16(to_dev(a), to_dev(b))), want)
+    np.testing.assert_array_equal(to_host(espdl().sub_s16(to_dev(a), to_dev(a))), oracle.sub_s16(a, a))
+
+
+@pytest.mark.parametrize("shapes", [((4, 3000), (4, 3000)), ((2, 800), (1,)), ((4, 300), (4, 1)), ((1,), (4, 300)),
+                                    ((4, 1), (4, 300))], ids=str)
+@pytest.mark.parametrize("shift", [-3, 0, 3, 9])
+def test_div_s16(oracle, shapes, shift):
+    announce(f"div_s16 {shapes} shift={shift}")
+    rng = np.random.default_rng(64)
+    a, b = _rand(rng, shapes[0], np.int16), _rand(rng, shapes[1], np.int16)
+    a.flat[0] = 0
+    b.flat[-1] = 0
+    got = to_host(espdl().div_s16(to_dev(a), to_dev(b), shift))
+    np.testing.assert_array_equal(got, oracle.div_s16(a, b, shift))

@@ -191,3 +191,36 @@ def test_avg_pool_and_reduce_mean_s16_are_exact_means_away_from_ties(oracle):
             exact = Fraction(int(s[n, c]), 72) * 4
             if abs((exact - np.floor(exact)) - Fraction(1, 2)) > Fraction(1, 1000):
                 assert r[n, 0, 0, c] == min(max(int(np.floor(exact + Fraction(1, 2))), -32768), 32767)
+
+
+def test_sub_s16_saturates(oracle):
+    rng = np.random.default_rng(53)
+    a, b = _rand(rng, (3, 1000), np.int16), _rand(rng, (3, 1000), np.int16)
+    want = np.clip(a.astype(np.int32) - b.astype(np.int32), -32768, 32767).astype(np.int16)
+    np.testing.assert_array_equal(oracle.sub_s16(a, b), want)
+
+
+@pytest.mark.parametrize("shapes,form", [(((4, 300), (4, 300)), 0), (((4, 300), (1,)), 1), (((4, 300), (4, 1)), 1),
+                                         (((1,), (4, 300)), 2), (((4, 1), (4, 300)), 2)], ids=str)
+@pytest.mark.parametrize("shift", [-3, 0, 5])
+def test_div_s16_is_float32_arithmetic_in_the_reference_order(oracle, shapes, form, shift):
+    """IEEE float32 operations in numpy, in the order of the loop that the broadcast selects; and within one
+    unit of the exact quotient, which a wrong shift sign or swapped operands would miss by far."""
+    rng = np.random.default_rng(54)
+    a, b = _rand(rng, shapes[0], np.int16), _rand(rng, shapes[1], np.int16)
+    a.flat[0] = 0
+    b.flat[-1] = 0
+    assert oracle.div_form(shapes[0], shapes[1]) == form
+    got = oracle.div_s16(a, b, shift)
+    af, bf = np.broadcast_arrays(a.astype(np.float32), b.astype(np.float32))
+    r = np.float32(2.0 ** -shift)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        v = af * (r / bf) if form == 1 else ((af * r) / bf if form == 2 else af * r / bf)
+    q = np.floor(v.astype(np.float64) + 0.5)
+    want = np.clip(np.nan_to_num(q, nan=0.0, posinf=32767, neginf=-32768), -32768, 32767).astype(np.int16)
+    want = np.where(af == 0, 0, np.where(bf == 0, np.where(af > 0, 32767, -32768), want)).astype(np.int16)
+    np.testing.assert_array_equal(got, want)
+    ok = (af != 0) & (bf != 0)
+    exact = af[ok].astype(np.float64) * 2.0 ** -shift / bf[ok].astype(np.float64)
+    inside = np.abs(exact) < 32000
+    assert np.all(np.abs(got[ok][inside] - exact[inside]) <= 1.0)
