@@ -51,6 +51,11 @@ public:
     }
     virtual void print() {}
     virtual void reset() {}
+    /// A module that carries data from one forward to the next saves it in hold_state and puts it back in
+    /// restore_state: the model brackets passes whose results are discarded (the warm-up before a graph
+    /// capture, profiling passes) with the two calls, on `stream`.
+    virtual void hold_state(void *stream) { (void)stream; }
+    virtual void restore_state(void *stream) { (void)stream; }
     /// Multiply-accumulates one forward performs for the given input shapes (0 for data movement);
     /// used by Model::profile to report achieved int8 OP/s.
     virtual int64_t get_macs(std::vector<std::vector<int>> &input_shapes)

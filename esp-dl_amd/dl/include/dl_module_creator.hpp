@@ -75,6 +75,7 @@ public:
         register_module("Slice", Slice::deserialize);
         register_module("ReduceMean", ReduceMean::deserialize);
         register_module("InsertZeros", InsertZeros::deserialize);
+        register_module("StreamingCache", StreamingCache::deserialize);
         register_module("Softmax", Softmax::deserialize);
         // both are TensorBase::assign between a float32 and a quantized tensor
         // (esp-dl/dl/module/include/dl_module_creator.hpp:154-155)

@@ -657,6 +657,114 @@ public:
     void print() { DL_LOGI("ReduceMean", "keepdims: %d, quant_type: %s.", m_keepdims, quant_type_to_string(quant_type)); }
 };
 
+/// StreamingCache (esp-dl/dl/module/include/dl_module_streaming_cache.hpp): the output is the last
+/// window_size - 1 frames of the previous call followed by this call's frames; the cache starts as zeros.
+/// The reference copies whole byte blocks of its single image, which is a concatenation along axis 1;
+/// here every image of the batch carries its own cache and the same block copies run once per image.
+class StreamingCache : public Module {
+private:
+    int m_window_size, m_frame_axis;
+    TensorBase *m_cache = nullptr; ///< [batch][cache bytes per image], device
+    TensorBase *m_held = nullptr;  ///< copy of the cache while a discarded pass runs
+    bool m_held_valid = false;
+
+public:
+    StreamingCache(const char *name = nullptr, int window_size = 1, int frame_axis = 1,
+                   quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_window_size(window_size), m_frame_axis(frame_axis)
+    {
+    }
+    ~StreamingCache()
+    {
+        delete m_cache;
+        delete m_held;
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        std::vector<int> out = input_shapes[0];
+        const int axis = m_frame_axis < 0 ? m_frame_axis + (int)out.size() : m_frame_axis;
+        if (axis != 1 || out.size() < 2 || m_window_size < 1)
+            return {{}}; // the block copies below are a concatenation only along axis 1
+        out[1] += m_window_size - 1;
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) || input->shape.size() < 2 || input->dtype != output->dtype) {
+            DL_LOGE("StreamingCache", "%s: needs device tensors of one dtype", name.c_str());
+            return;
+        }
+        const int64_t batch = input->shape[0];
+        const int64_t in_bytes = (int64_t)input->get_bytes() / std::max<int64_t>(1, batch);
+        const int64_t frame_bytes = in_bytes / std::max(1, input->shape[1]);
+        const int64_t cache_bytes = frame_bytes * (m_window_size - 1);
+        if (cache_bytes == 0) {
+            output->copy_from(input, context->stream);
+            return;
+        }
+        if (m_cache == nullptr || m_cache->get_bytes() != (size_t)(batch * cache_bytes)) {
+            delete m_cache;
+            m_cache = new TensorBase({(int)batch, (int)cache_bytes}, nullptr, 0, DATA_TYPE_INT8, true, MALLOC_CAP_DEVICE);
+            if (!m_cache->data) { // a null element pointer asks for zero-filled storage
+                DL_LOGE("StreamingCache", "%s: cannot allocate the cache", name.c_str());
+                return;
+            }
+        }
+        char *out = static_cast<char *>(output->data);
+        const int64_t out_bytes = cache_bytes + in_bytes;
+        int rc = espdl_hip_copy_rows(m_cache->data, cache_bytes, out, out_bytes, cache_bytes, batch, context->stream);
+        if (rc == ESPDL_HIP_OK)
+            rc = espdl_hip_copy_rows(input->data, in_bytes, out + cache_bytes, out_bytes, in_bytes, batch, context->stream);
+        if (rc == ESPDL_HIP_OK)
+            rc = espdl_hip_copy_rows(out + in_bytes, out_bytes, m_cache->data, cache_bytes, cache_bytes, batch, context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("StreamingCache", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    /// Forget the frames seen so far.
+    void reset()
+    {
+        if (m_cache && m_cache->data)
+            m_cache->memset(0, nullptr);
+    }
+    void hold_state(void *stream)
+    {
+        m_held_valid = false;
+        if (!m_cache || !m_cache->data)
+            return; // nothing seen yet: restore_state clears whatever the discarded pass leaves
+        if (!m_held || m_held->get_bytes() != m_cache->get_bytes()) {
+            delete m_held;
+            m_held = new TensorBase(m_cache->shape, nullptr, 0, DATA_TYPE_INT8, true, MALLOC_CAP_DEVICE);
+        }
+        m_held_valid = m_held->copy_from(m_cache, stream);
+    }
+    void restore_state(void *stream)
+    {
+        if (!m_cache || !m_cache->data)
+            return;
+        if (m_held_valid && m_held && m_held->get_bytes() == m_cache->get_bytes())
+            m_cache->copy_from(m_held, stream);
+        else
+            m_cache->memset(0, stream);
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        int window_size = 1, frame_axis = 1;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "window_size", window_size);
+        fbs_model->get_operation_attribute(node_name, "frame_axis", frame_axis);
+        return new StreamingCache(node_name.c_str(), window_size, frame_axis, quant_type);
+    }
+    void print()
+    {
+        DL_LOGI("StreamingCache", "window_size: %d, frame_axis: %d, quant_type: %s.", m_window_size, m_frame_axis,
+                quant_type_to_string(quant_type));
+    }
+};
+
 /// InsertZeros on [N, spatial..., C] tensors with one or two spatial dims
 /// (esp-dl/dl/module/include/dl_module_insert_zeros.hpp): the exporter writes a transposed convolution as
 /// InsertZeros followed by an ordinary Conv.

@@ -668,9 +668,14 @@ bool Model::enable_graph()
     if (!m_built || m_graph_exec)
         return m_graph_exec != nullptr;
     hipStream_t s = static_cast<hipStream_t>(m_stream);
-    // one eager pass so that every module has uploaded its shifts / tables before capture starts
+    // one eager pass so that every module has uploaded its shifts / tables before capture starts; modules that
+    // carry data between passes (StreamingCache) get it back afterwards, the pass counts for nothing
+    for (auto *module : m_execution_plan)
+        module->hold_state(m_stream);
     for (auto *module : m_execution_plan)
         module->forward(m_model_context, RUNTIME_MODE_AUTO);
+    for (auto *module : m_execution_plan)
+        module->restore_state(m_stream);
     if (!hip_ok(hipStreamSynchronize(s), "hipStreamSynchronize"))
         return false;
     if (!hip_ok(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture"))
@@ -765,11 +770,13 @@ std::vector<module_info> Model::get_module_info(int repeats)
     if (repeats < 1)
         repeats = 1;
     for (auto *module : m_execution_plan) {
+        module->hold_state(m_stream); // timing passes leave no trace in modules that carry data between passes
         module->forward(m_model_context, RUNTIME_MODE_AUTO); // warm
         (void)hipEventRecord(e0, s);
         for (int r = 0; r < repeats; r++)
             module->forward(m_model_context, RUNTIME_MODE_AUTO);
         (void)hipEventRecord(e1, s);
+        module->restore_state(m_stream);
         (void)hipEventSynchronize(e1);
         float ms = 0.f;
         (void)hipEventElapsedTime(&ms, e0, e1);

@@ -17,9 +17,11 @@ def _shift(spec, node, x_name, w_name, y_name):
     return (spec.exponent(y_name) - w_exps - spec.exponent(x_name)).astype(np.int32)
 
 
-def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
-    """inputs: {name: ndarray for the whole batch}.  Returns {tensor name: ndarray}."""
+def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None):
+    """inputs: {name: ndarray for the whole batch}.  Returns {tensor name: ndarray}.  `state` (a dict the
+    caller keeps between calls) holds the frames StreamingCache nodes carry from one call to the next."""
     t = dict(inputs)
+    state = {} if state is None else state
 
     def operand(name):
         """An activation, or a constant operand (initializer) as stored."""
@@ -173,6 +175,17 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True):
         elif op == "Resize":
             scales = spec.initializers[ins[2]][2].ravel()
             y = oracle.resize_nearest_s8(x, scales[2], scales[3], spec.exponent(ins[0]), spec.exponent(y_name))
+        elif op == "StreamingCache":
+            # esp-dl/dl/module/include/dl_module_streaming_cache.hpp: [previous window_size - 1 frames | input]
+            # along axis 1, zeros before the first call; the last frames of the result are kept
+            keep = a.get("window_size", 1) - 1
+            if a.get("frame_axis", 1) % x.ndim != 1:
+                raise NotImplementedError("StreamingCache along axis %d" % a.get("frame_axis", 1))
+            prev = state.get(node["name"])
+            if prev is None:
+                prev = np.zeros((x.shape[0], keep) + x.shape[2:], dtype=x.dtype)
+            y = np.concatenate([prev, x], axis=1)
+            state[node["name"]] = y[:, y.shape[1] - keep:].copy()
         elif op == "InsertZeros":
             st, op_pad = list(a["stride"]), list(a.get("output_padding") or [0])
             if x.ndim == 3:

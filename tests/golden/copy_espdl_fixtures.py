@@ -7,7 +7,8 @@ source code.  Run in the development container:  python tests/golden/copy_espdl_
   examples/tutorial/how_to_run_model/main/models/{s3,p4}/model.espdl   three chained int8 Gemms
   examples/tutorial/how_to_deploy_streaming_model/test_streaming_model/main/models/{esp32s3,esp32p4}/model.espdl
       a Conv1d network: dense and dilated depthwise Conv1d, Sigmoid tables, Mul, Add, AveragePool,
-      Transpose, Slice, Flatten, Gemm
+      Transpose, Slice, Flatten, Gemm; and streaming_model.espdl beside it, the same network with StreamingCache
+      nodes for chunk-by-chunk inference
 """
 import glob
 import os
@@ -33,6 +34,10 @@ def main():
         src = os.path.join(REF, "examples/tutorial/how_to_deploy_streaming_model/test_streaming_model/main/models",
                            target, "model.espdl")
         shutil.copyfile(src, os.path.join(OUT, "conv1d_net_%s.espdl" % target))
+        n += 1
+        # the same network exported for frame-by-frame use: StreamingCache nodes in front of every windowed operator
+        shutil.copyfile(src.replace("model.espdl", "streaming_model.espdl"),
+                        os.path.join(OUT, "conv1d_net_streaming_%s.espdl" % target))
         n += 1
     print("copied", n, "files to", OUT)
 

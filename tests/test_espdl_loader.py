@@ -31,7 +31,7 @@ def _spec(path):
 
 
 def test_fixtures_are_present():
-    assert len(FIXTURES) == 13
+    assert len(FIXTURES) == 15
 
 
 @pytest.mark.parametrize("path", FIXTURES, ids=os.path.basename)

@@ -22,7 +22,48 @@ def _round_mode(path):
     return 1 if "p4" in os.path.basename(path) else 0
 
 
-@pytest.mark.parametrize("path", FIXTURES, ids=os.path.basename)
+# the streaming exports carry no embedded vectors: they are checked step by step against the oracle below
+WITH_VECTORS = [p for p in FIXTURES if "streaming" not in os.path.basename(p)]
+
+
+@pytest.mark.parametrize("path", [p for p in FIXTURES if "streaming" in os.path.basename(p)], ids=os.path.basename)
+def test_streaming_model_carries_frames_between_calls(path):
+    """StreamingCache: five consecutive chunks through one dl::Model (eager, then HIP-graph replays) against
+    the oracle's graph runner keeping the same state; every image of the batch has its own history."""
+    announce("espdl streaming " + os.path.basename(path))
+    sys.path.insert(0, HERE)
+    import espdl_spec
+    import graph_runner
+    import espdl_oracle as oracle
+    spec, _ = espdl_spec.spec_from_espdl(path)
+    model = importlib.import_module("esp-dl_amd").model
+    rm = _round_mode(path)
+    batch = 3
+    rng = np.random.default_rng(78)
+    mdl = model.Model(model.Graph.from_file(path), batch, round_mode=rm)
+    state = {}
+    outs = []
+    for step in range(5):
+        if step == 2:
+            assert mdl.enable_graph()
+        x = spec.make_input(rng, batch)
+        want = graph_runner.run(spec, {spec.inputs[0]: x}, oracle.ROUND_HALF_EVEN if rm else oracle.ROUND_HALF_UP,
+                                keep_all=False, state=state)
+        mdl.set_input(spec.inputs[0], x)
+        mdl.run()
+        for name in spec.outputs:
+            np.testing.assert_array_equal(mdl.get_tensor(name).reshape(want[name].shape), want[name],
+                                          err_msg=f"{name} step {step}")
+        outs.append(want[spec.outputs[0]].copy())
+    # the history matters: the same chunk gives another result once earlier frames are in the caches
+    x = spec.make_input(np.random.default_rng(79), batch)
+    fresh = graph_runner.run(spec, {spec.inputs[0]: x}, keep_all=False, state={})
+    carried = graph_runner.run(spec, {spec.inputs[0]: x}, keep_all=False, state=state)
+    assert not np.array_equal(fresh[spec.outputs[0]], carried[spec.outputs[0]])
+    mdl.close()
+
+
+@pytest.mark.parametrize("path", WITH_VECTORS, ids=os.path.basename)
 def test_reference_fixture_passes_model_test(path):
     announce("espdl fixture " + os.path.basename(path))
     model = importlib.import_module("esp-dl_amd").model
