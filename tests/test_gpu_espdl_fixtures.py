@@ -132,5 +132,6 @@ def test_loaded_graph_matches_oracle_on_random_input(path):
             dt = np.int16 if spec.dtype(name) == 5 else np.int8
             got = mdl.get_tensor(name, dt)
             np.testing.assert_array_equal(got.reshape(want[name].shape), want[name], err_msg=f"{name} fuse={fuse}")
-            assert want[name].min() < want[name].max()
         mdl.close()
+    # not a comparison of constants (single score maps of some detectors do saturate on noise)
+    assert any(want[name].min() < want[name].max() for name in spec.outputs)
