@@ -23,6 +23,7 @@ struct SoftmaxArgs {
     long long outer, len, inner;
     int rows_per_block; // rows staged per workgroup (softmax axis innermost)
     int row_stride;     // padded LDS bytes per row
+    FastDiv fd_len;     // element index -> row, without an integer division per element
     float table[256];
 };
 
@@ -44,21 +45,34 @@ __global__ __launch_bounds__(kThreads) void softmax_s8_rows_kernel(const Softmax
         const int8_t *src = a.in + row0 * len;
         __syncthreads(); // table ready / previous span consumed
         for (int e = tid; e < rows_here * len; e += kThreads) {
-            const int r = e / len;
+            const int r = (int)fastdiv((unsigned)e, a.fd_len);
             rows[r * a.row_stride + (e - r * len)] = src[e];
         }
         __syncthreads();
         if (tid < rows_here) {
+            // four values per LDS read, their table entries fetched together; only the additions form a chain,
+            // and they stay in index order
             const int8_t *row = rows + tid * a.row_stride;
+            const int *row4 = reinterpret_cast<const int *>(row);
             float sum = 0.f;
-            for (int i = 0; i < len; i++)
+            int i = 0;
+            for (; i + 4 <= len; i += 4) {
+                const int q = row4[i >> 2];
+                const float t0 = table[(int)(int8_t)q + 128], t1 = table[(int)(int8_t)(q >> 8) + 128];
+                const float t2 = table[(int)(int8_t)(q >> 16) + 128], t3 = table[(q >> 24) + 128];
+                sum += t0;
+                sum += t1;
+                sum += t2;
+                sum += t3;
+            }
+            for (; i < len; i++)
                 sum += table[(int)row[i] + 128];
             sums[tid] = sum;
         }
         __syncthreads();
         float *dst = a.out + row0 * len;
         for (int e = tid; e < rows_here * len; e += kThreads) {
-            const int r = e / len;
+            const int r = (int)fastdiv((unsigned)e, a.fd_len);
             dst[e] = table[(int)rows[r * a.row_stride + (e - r * len)] + 128] / sums[r];
         }
     }
@@ -139,6 +153,7 @@ struct MatMulArgs {
     int lead[2];                 // broadcast leading extents of the result (outer, inner)
     long long a_stride[2], b_stride[2]; // element strides of each operand per leading dim (0 = broadcast)
     int shift, relu, half_even;
+    int vec_a, vec_b; // rows of a (k long) / b (n long) can be read with 8- / 4-byte loads
 };
 
 constexpr int kTile = 64;  // output tile edge
@@ -170,26 +185,42 @@ __global__ __launch_bounds__(kThreads) void matmul_s8_kernel(const MatMulArgs p)
 
     for (int k0 = 0; k0 < p.k; k0 += kChunk) {
         __syncthreads();
-        // A tile: 64 rows x 32 k, k fastest in memory; 8 consecutive k per lane
+        // A tile: 64 rows x 32 k, k fastest in memory; 8 consecutive k per lane (one 8-byte load when the
+        // row length and the base allow it)
         {
             const int r = tid >> 2, kk = (tid & 3) * 8;
             const int gm = m0 + r;
+            if (p.vec_a && gm < p.m && k0 + kk + 8 <= p.k) {
+                const int2 v = *reinterpret_cast<const int2 *>(A + (long long)gm * p.k + k0 + kk);
+                *reinterpret_cast<int *>(&as[r][kk]) = v.x; // LDS rows are 36 bytes apart: 4-byte aligned only
+                *reinterpret_cast<int *>(&as[r][kk + 4]) = v.y;
+            } else {
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int gk = k0 + kk + e;
-                as[r][kk + e] = (gm < p.m && gk < p.k) ? A[(long long)gm * p.k + gk] : (int8_t)0;
+                for (int e = 0; e < 8; e++) {
+                    const int gk = k0 + kk + e;
+                    as[r][kk + e] = (gm < p.m && gk < p.k) ? A[(long long)gm * p.k + gk] : (int8_t)0;
+                }
             }
         }
-        // B tile: 32 k x 64 n, n fastest in memory; lanes walk n so loads coalesce, stores transpose
-        {
-            const int c = tid & 63, kq = tid >> 6; // 4 groups of 8 k
-            const int gn = n0 + c;
+        // B tile: 32 k x 64 n, n fastest in memory; a lane loads four neighbouring n of one k row (or single
+        // bytes at the edges) and stores them transposed
+        for (int it = tid; it < kChunk * (kTile / 4); it += kThreads) {
+            const int kk = it >> 4, c4 = (it & 15) * 4;
+            const int gk = k0 + kk, gn = n0 + c4;
+            int v = 0;
+            if (gk < p.k) {
+                if (p.vec_b && gn + 4 <= p.n) {
+                    v = *reinterpret_cast<const int *>(B + (long long)gk * p.n + gn);
+                } else {
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int kk = kq * 8 + e;
-                const int gk = k0 + kk;
-                bs[c][kk] = (gn < p.n && gk < p.k) ? B[(long long)gk * p.n + gn] : (int8_t)0;
+                    for (int e = 0; e < 4; e++)
+                        if (gn + e < p.n)
+                            v |= (int)(unsigned char)B[(long long)gk * p.n + gn + e] << (8 * e);
+                }
             }
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                bs[c4 + e][kk] = (int8_t)(v >> (8 * e));
         }
         __syncthreads();
 #pragma unroll
@@ -246,6 +277,7 @@ hipError_t launch_softmax_s8(const int8_t *in, long long outer, long long len, l
         rows = (int)min((long long)rows, outer);
         a.rows_per_block = rows;
         a.row_stride = stride;
+        a.fd_len = make_fastdiv((unsigned)len);
         const size_t lds = 256 * sizeof(float) + (size_t)rows * sizeof(float) + (size_t)rows * stride;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(softmax_s8_rows_kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -321,6 +353,8 @@ hipError_t launch_matmul_s8(const int8_t *a, const int8_t *b, int m, int k, int 
     p.shift = shift;
     p.relu = relu;
     p.half_even = half_even;
+    p.vec_a = (k % 8) == 0 && (reinterpret_cast<uintptr_t>(a) & 7) == 0 && (a_stride[0] % 8) == 0 && (a_stride[1] % 8) == 0;
+    p.vec_b = (n % 4) == 0 && (reinterpret_cast<uintptr_t>(b) & 3) == 0 && (b_stride[0] % 4) == 0 && (b_stride[1] % 4) == 0;
     const dim3 grid((unsigned)((n + kTile - 1) / kTile), (unsigned)((m + kTile - 1) / kTile), (unsigned)(lead[0] * lead[1]));
     matmul_s8_kernel<<<grid, dim3(kThreads), 0, stream>>>(p);
     return hipGetLastError();

@@ -24,6 +24,7 @@ struct S16Args {
     ConvGeom g;
     int oc_quads;
     long long n_items;
+    int vec8; // channels % 8 == 0 and 16-byte aligned tensors: 16-byte loads
 };
 
 __global__ __launch_bounds__(256) void conv2d_s16_kernel(const S16Args a)
@@ -54,7 +55,28 @@ __global__ __launch_bounds__(256) void conv2d_s16_kernel(const S16Args a)
                 continue;
             const int16_t *px = img + ((long long)iy * g.in_w + ix) * C;
             const int16_t *fw = a.w + (long long)oc0 * ftap + ((long long)ky * g.k_w + kx) * C;
-            for (int c = 0; c < C; c++) {
+            int c = 0;
+            if (a.vec8 && oc0 + 3 < OC) {
+                // eight channels per 16-byte load of the pixel and of each of the four filters; every product
+                // goes into the 64-bit accumulator with one multiply-add
+                for (; c + 8 <= C; c += 8) {
+                    const v4i xv = *reinterpret_cast<const v4i *>(px + c);
+                    v4i wv[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        wv[r] = *reinterpret_cast<const v4i *>(fw + r * ftap + c);
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+                        const long long x0 = (short)xv[d], x1 = xv[d] >> 16;
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            acc[r] += x0 * (long long)(short)wv[r][d];
+                            acc[r] += x1 * (long long)(wv[r][d] >> 16);
+                        }
+                    }
+                }
+            }
+            for (; c < C; c++) {
                 const int v = px[c];
 #pragma unroll
                 for (int r = 0; r < 4; r++)
@@ -111,8 +133,9 @@ __global__ __launch_bounds__(256) void depthwise_s16_kernel(const S16Args a)
 hipError_t launch_conv2d_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
                              const int32_t *shift, int16_t *out, hipStream_t stream)
 {
-    S16Args a{in, filter, bias, shift, out, g, (g.out_c + 3) / 4, 0};
+    S16Args a{in, filter, bias, shift, out, g, (g.out_c + 3) / 4, 0, 0};
     a.n_items = (long long)g.batch * g.out_h * g.out_w * a.oc_quads;
+    a.vec8 = (g.in_c % 8) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) == 0;
     if (a.n_items == 0)
         return hipSuccess;
     hipLaunchKernelGGL(conv2d_s16_kernel, dim3((unsigned)((a.n_items + 255) / 256)), dim3(256), 0, stream, a);
@@ -122,7 +145,7 @@ hipError_t launch_conv2d_s16(const ConvGeom &g, const int16_t *in, const int16_t
 hipError_t launch_depthwise_s16(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
                                 const int32_t *shift, int16_t *out, hipStream_t stream)
 {
-    S16Args a{in, filter, bias, shift, out, g, 0, 0};
+    S16Args a{in, filter, bias, shift, out, g, 0, 0, 0};
     a.n_items = (long long)g.batch * g.out_h * g.out_w * g.in_c;
     if (a.n_items == 0)
         return hipSuccess;

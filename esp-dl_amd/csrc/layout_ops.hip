@@ -369,30 +369,46 @@ struct ReduceArgs {
     int kept_shape[kMaxDims], red_shape[kMaxDims];
     long long kept_stride[kMaxDims], red_stride[kMaxDims];
     long long n_out, count;
+    int lanes; // lanes per output: a power of two, 1..64
     float input_scale, output_scale;
 };
 
+// Each output is summed by `a.lanes` lanes of one wavefront (a power of two up to 64): neighbouring lanes hold
+// neighbouring outputs, the lanes of one output sit 64 / lanes apart and walk the reduced elements with that
+// stride; integer partial sums are combined with cross-lane adds, so the order does not matter.
 __global__ __launch_bounds__(kBlock) void reduce_mean_s8_kernel(const ReduceArgs a)
 {
-    for (long long o = (long long)blockIdx.x * kBlock + threadIdx.x; o < a.n_out; o += (long long)gridDim.x * kBlock) {
-        long long rem = o, base = 0;
-        for (int d = a.n_kept - 1; d >= 0; d--) {
-            const long long q = rem / a.kept_shape[d];
-            base += (rem - q * a.kept_shape[d]) * a.kept_stride[d];
-            rem = q;
-        }
+    const int per_wave = 64 / a.lanes; // outputs per wavefront
+    const int lane = threadIdx.x & 63;
+    const int o_local = lane % per_wave, part = lane / per_wave;
+    const long long waves = ((long long)gridDim.x * kBlock) >> 6;
+    const long long n_groups = (a.n_out + per_wave - 1) / per_wave;
+    for (long long grp = ((long long)blockIdx.x * kBlock + threadIdx.x) >> 6; grp < n_groups; grp += waves) {
+        const long long o = grp * per_wave + o_local;
         int sum = 0;
-        for (long long r = 0; r < a.count; r++) {
-            long long rr = r, off = base;
-            for (int d = a.n_red - 1; d >= 0; d--) {
-                const long long q = rr / a.red_shape[d];
-                off += (rr - q * a.red_shape[d]) * a.red_stride[d];
-                rr = q;
+        if (o < a.n_out) {
+            long long rem = o, base = 0;
+            for (int d = a.n_kept - 1; d >= 0; d--) {
+                const long long q = rem / a.kept_shape[d];
+                base += (rem - q * a.kept_shape[d]) * a.kept_stride[d];
+                rem = q;
             }
-            sum += a.in[off];
+            for (long long r = part; r < a.count; r += a.lanes) {
+                long long rr = r, off = base;
+                for (int d = a.n_red - 1; d >= 0; d--) {
+                    const long long q = rr / a.red_shape[d];
+                    off += (rr - q * a.red_shape[d]) * a.red_stride[d];
+                    rr = q;
+                }
+                sum += a.in[off];
+            }
         }
-        const float v = (float)sum * a.input_scale / (float)a.count * a.output_scale;
-        a.out[o] = (int8_t)clamp_s8(round_half_up_f32(v));
+        for (int step = 32; step >= per_wave; step >>= 1)
+            sum += __shfl_xor(sum, step, 64);
+        if (o < a.n_out && part == 0) {
+            const float v = (float)sum * a.input_scale / (float)a.count * a.output_scale;
+            a.out[o] = (int8_t)clamp_s8(round_half_up_f32(v));
+        }
     }
 }
 
@@ -745,7 +761,11 @@ hipError_t launch_reduce_mean_s8(const int8_t *in, const int *shape, int dims, c
     a.out = out;
     a.input_scale = dl_scale(in_exp);
     a.output_scale = dl_rescale(out_exp);
-    hipLaunchKernelGGL(reduce_mean_s8_kernel, dim3(blocks_for(a.n_out, cu_count)), dim3(kBlock), 0, stream, a);
+    // enough lanes per output to occupy the device when there are few outputs and long sums
+    a.lanes = 1;
+    while (a.lanes < 64 && a.n_out * a.lanes < (long long)max(1, cu_count) * 2048 && a.count >= 4ll * a.lanes)
+        a.lanes *= 2;
+    hipLaunchKernelGGL(reduce_mean_s8_kernel, dim3(blocks_for(a.n_out * a.lanes, cu_count)), dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 
