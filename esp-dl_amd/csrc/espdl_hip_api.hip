@@ -191,6 +191,9 @@ int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const 
     int16_t *o16 = static_cast<int16_t *>(out);
     if (depthwise)
         return device_status(espdl::launch_depthwise_s16(g, i16, f16, b64, shift, o16, s), "depthwise_s16");
+    if (espdl::conv2d_s16_mfma_supports(g, i16, f16, o16))
+        return device_status(espdl::launch_conv2d_s16_mfma(g, i16, f16, b64, shift, o16, cu_count_cached(), s),
+                             "conv2d_s16_mfma");
     return device_status(espdl::launch_conv2d_s16(g, i16, f16, b64, shift, o16, s), "conv2d_s16");
 }
 

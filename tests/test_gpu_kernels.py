@@ -262,6 +262,50 @@ DW_TILE_CASES = [
 ]
 
 
+S16_MFMA_CASES = [
+    # (name, (n, h, w, c), out_c, k, stride, dil, pads, relu, half_even, values)
+    ("pw_80x80_96_64", (2, 40, 40, 96), 64, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False, "random"),
+    ("c3_20x20_256_16", (2, 20, 20, 256), 16, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False, "random"),
+    ("c3_13x11_16_16", (3, 13, 11, 16), 16, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), False, True, "random"),
+    ("pw_7x9_80_80", (2, 7, 9, 80), 80, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), False, False, "random"),
+    ("pw_9x5_16_4", (2, 9, 5, 16), 4, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), False, False, "random"),
+    ("c3s2_17x15_32_70", (2, 17, 15, 32), 70, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), True, False, "random"),
+    ("c3d2_12x12_48_33", (1, 12, 12, 48), 33, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2), False, True, "random"),
+    ("pw_6x6_384_256", (2, 6, 6, 384), 256, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False, "random"),
+    # every digit at its extremes: all -32768, all 32767, and the 7-bit boundaries
+    ("extremes_min", (1, 5, 5, 64), 32, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), False, False, "min"),
+    ("extremes_max", (1, 5, 5, 64), 32, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), False, False, "max"),
+    ("extremes_edges", (1, 6, 6, 32), 16, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), False, False, "edges"),
+]
+
+
+@pytest.mark.parametrize("case", S16_MFMA_CASES, ids=lambda c: c[0])
+def test_conv2d_s16_matrix_pipe(oracle, case):
+    """int16 convolutions whose input channels are a multiple of 16 run as 7-bit digit products on the int8
+    MFMA; the 64-bit sums must come out exact whatever the digits are."""
+    announce(f"conv2d_s16 mfma {case[0]}")
+    name, (n, h, w, c), oc, k, stride, dil, pads, relu, half_even, values = case
+    rng = np.random.default_rng(0x516 + len(name))
+    if values == "random":
+        x = rng.integers(-32768, 32768, size=(n, h, w, c)).astype(np.int16)
+        f = rng.integers(-32768, 32768, size=(oc, k[0], k[1], c)).astype(np.int16)
+    else:
+        pool = {"min": [-32768], "max": [32767],
+                "edges": [-32768, -16385, -16384, -129, -128, -1, 0, 1, 127, 128, 16383, 16384, 32767]}[values]
+        x = rng.choice(pool, size=(n, h, w, c)).astype(np.int16)
+        f = rng.choice(pool, size=(oc, k[0], k[1], c)).astype(np.int16)
+    bias = rng.integers(-2**40, 2**40, size=oc).astype(np.int64)
+    shift = (typical_shift(k[0] * k[1] * c) + 16 + rng.integers(-2, 3, size=oc)).astype(np.int32)
+    m = espdl()
+    rm_g = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
+    rm_o = oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP
+    got = m.conv2d(to_dev(x), to_dev(f), to_dev(bias), to_dev(shift), k, stride, dil, pads,
+                   activation=m.capi.RELU if relu else m.capi.LINEAR, round_mode=rm_g)
+    want = oracle.conv2d_s16(x, f, bias, shift, k, stride, dil, pads, oracle.RELU if relu else oracle.LINEAR, rm_o)
+    np.testing.assert_array_equal(to_host(got), want)
+    assert want.min() < want.max()
+
+
 @pytest.mark.parametrize("case", DW_TILE_CASES, ids=lambda c: c[0])
 def test_depthwise_s8_tiles(oracle, case):
     announce(f"depthwise_s8 tiles {case[0]}")
