@@ -84,7 +84,9 @@ def lib():
         L.espdl_hip_reduce_mean_s16.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
         L.espdl_hip_sub_s16.argtypes = [vp, vp, vp, vp, vp, vp, vp]
         L.espdl_hip_div_s16.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp]
-        for name in ("add_s16", "mul_s16", "sub_s16", "div_s16", "avg_pool_s16", "reduce_mean_s16"):
+        L.espdl_hip_sub_s8.argtypes = [vp, vp, vp, vp, vp, vp, vp]
+        L.espdl_hip_div_s8.argtypes = [vp, vp, vp, vp, vp, i32, vp, vp]
+        for name in ("add_s16", "mul_s16", "sub_s16", "div_s16", "avg_pool_s16", "reduce_mean_s16", "sub_s8", "div_s8"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         L.espdl_hip_insert_zeros.argtypes = [vp] + [i32] * 9 + [vp, vp]
         L.espdl_hip_insert_zeros.restype = ctypes.c_int
@@ -463,12 +465,12 @@ def insert_zeros(x, stride, output_padding=(0, 0), stream=None):
     return out
 
 
-def _broadcast16(a, b):
+def _broadcast16(a, b, dtype=None):
     import torch
     dims, s0, s1, _ = _broadcast(a, b, a)  # strides only; the result is allocated below
     rank = max(a.dim(), b.dim())
     so = [int(d) for d in dims]
-    return dims, s0, s1, torch.empty(so[4 - rank:] if rank else [], dtype=torch.int16, device=a.device)
+    return dims, s0, s1, torch.empty(so[4 - rank:] if rank else [], dtype=dtype or torch.int16, device=a.device)
 
 
 def add_s16(a, b, stream=None):
@@ -513,6 +515,23 @@ def sub_s16(a, b, stream=None):
     dims, s0, s1, out = _broadcast16(a, b)
     _check(lib().espdl_hip_sub_s16(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), _p(out),
                                    _stream(stream)))
+    return out
+
+
+def sub_s8(a, b, stream=None):
+    import torch
+    dims, s0, s1, out = _broadcast16(a, b, torch.int8)
+    _check(lib().espdl_hip_sub_s8(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), _p(out),
+                                  _stream(stream)))
+    return out
+
+
+def div_s8(a, b, shift, stream=None):
+    """shift = out_exp - a_exp + b_exp."""
+    import torch
+    dims, s0, s1, out = _broadcast16(a, b, torch.int8)
+    _check(lib().espdl_hip_div_s8(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), int(shift),
+                                  _p(out), _stream(stream)))
     return out
 
 

@@ -1,11 +1,14 @@
-// int16 forms of Add, Mul, AveragePool and ReduceMean for gfx950.  They serve the int16 heads and the int16
-// text recognizer of the reference's model files: small tensors, so one element per lane and plain loops.
+// int16 forms of Add, Mul, AveragePool and ReduceMean, and Sub / Div for int8 and int16, for gfx950.  They serve
+// the int16 heads and the int16 text recognizer of the reference's model files: small tensors, so one element per
+// lane and plain loops.
 //
 // Add: c_impl_add_n_n<int16_t> (esp-dl/dl/base/dl_base_add.cpp:33-44), saturating integer add.
 // Mul: c_impl_mul_n_n<int16_t> (esp-dl/dl/base/dl_base_mul.cpp:33-46): the int32 product goes through
 //      float32, is scaled by 2^-shift and rounded half up; with ESP32-P4 semantics the exact product is
 //      shifted and rounded half to even.
-// Sub: c_impl_sub_n_n<int16_t> (esp-dl/dl/base/dl_base_sub.cpp:33-43).  Div: esp-dl/dl/base/dl_base_div.cpp, float32.
+// Sub: c_impl_sub_n_n<feature_t> (esp-dl/dl/base/dl_base_sub.cpp:33-43).  Div: esp-dl/dl/base/dl_base_div.cpp, float32;
+//      the int8 form with a single-element operand goes through a 256-entry table there (create_div_lut, :8-46),
+//      whose entries are the same float32 expressions except for 0 / 0 with a single-element dividend (-128).
 // AveragePool: avgpool2d_hwc<int16_t, int32_t> (esp-dl/dl/base/dl_base_avg_pool2d.cpp:28-54).
 // ReduceMean: reduce<int64_t, int16_t> (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:18-56).
 #include "espdl_device.h"
@@ -21,20 +24,22 @@ __device__ __forceinline__ int clamp_s16(int v)
     return min(max(v, -32768), 32767);
 }
 
-struct Binary16Args {
-    const int16_t *in0, *in1;
-    int16_t *out;
+template <typename T>
+struct BinaryArgs {
+    const T *in0, *in1;
+    T *out;
     int dims[4];
     long long s0[4], s1[4];
     long long total;
-    int shift, half_even;
+    int shift, half_even, zero_by_zero;
     float rescale;
 };
 
-// OP: 0 add, 1 mul, 2 sub, 3 div
-template <int OP>
-__global__ __launch_bounds__(kThreads) void binary_s16_kernel(const Binary16Args a)
+// OP: 0 add, 1 mul, 2 sub, 3 div.  Add and Mul are instantiated for int16 only (int8 has kernels of its own).
+template <typename T, int OP>
+__global__ __launch_bounds__(kThreads) void binary_kernel(const BinaryArgs<T> a)
 {
+    constexpr int lo = sizeof(T) == 1 ? -128 : -32768, hi = sizeof(T) == 1 ? 127 : 32767;
     for (long long i = (long long)blockIdx.x * kThreads + threadIdx.x; i < a.total; i += (long long)gridDim.x * kThreads) {
         long long rem = i, o0 = 0, o1 = 0;
 #pragma unroll
@@ -51,9 +56,9 @@ __global__ __launch_bounds__(kThreads) void binary_s16_kernel(const Binary16Args
             // c_impl_div_n_n / _n_1 / _1_n (esp-dl/dl/base/dl_base_div.cpp:92-112, 141-163, 175-195): float32, the
             // order of the two operations depends on which operand is constant along the innermost axis
             if (x == 0) {
-                r = 0;
+                r = y == 0 ? a.zero_by_zero : 0;
             } else if (y == 0) {
-                r = x > 0 ? 32767 : -32768;
+                r = x > 0 ? hi : lo;
             } else {
                 float v;
                 if (a.shift == 1) {
@@ -65,10 +70,10 @@ __global__ __launch_bounds__(kThreads) void binary_s16_kernel(const Binary16Args
                 } else {
                     v = (float)x * a.rescale / (float)y;
                 }
-                r = clamp_s16(round_half_up_f32(v));
+                r = min(max(round_half_up_f32(v), lo), hi);
             }
         } else if (OP == 2) {
-            r = clamp_s16(x - y);
+            r = min(max(x - y, lo), hi);
         } else if (OP == 1) {
             const int prod = x * y; // at most 2^30 in magnitude
             if (a.half_even && a.shift > 0) {
@@ -81,7 +86,7 @@ __global__ __launch_bounds__(kThreads) void binary_s16_kernel(const Binary16Args
         } else {
             r = clamp_s16(x + y);
         }
-        a.out[i] = (int16_t)r;
+        a.out[i] = (T)r;
     }
 }
 
@@ -152,10 +157,13 @@ unsigned blocks_for(long long total, int cu_count)
 
 } // namespace
 
-hipError_t launch_binary_s16(int op, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int16_t *in0,
-                             const int16_t *in1, int shift, bool half_even, int16_t *out, int cu_count, hipStream_t stream)
+namespace {
+
+template <typename T>
+hipError_t launch_binary(int op, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const T *in0, const T *in1,
+                         int shift, bool half_even, T *out, int cu_count, hipStream_t stream)
 {
-    Binary16Args a = {};
+    BinaryArgs<T> a = {};
     a.in0 = in0;
     a.in1 = in1;
     a.out = out;
@@ -173,23 +181,47 @@ hipError_t launch_binary_s16(int op, const int32_t dims[4], const int64_t s0[4],
     a.rescale = dl_rescale(shift);
     const dim3 grid(blocks_for(a.total, cu_count));
     if (op == 3) {
-        // the loop form: 1 = divisor constant along the innermost axis longer than 1, 2 = dividend constant
-        int form = 1;
+        // the loop form: 1 = divisor constant along the innermost axis longer than 1, 2 = dividend constant.  With
+        // every axis of length 1 the reference tests the divisor first for int16 (dl_base_div.cpp:248-252) and the
+        // dividend first for int8 (:212-224).
+        int form = sizeof(T) == 1 ? 2 : 1;
+        bool single_dividend = true;
         for (int d = 3; d >= 0; d--)
             if (dims[d] > 1) {
                 form = s1[d] == 0 ? 1 : (s0[d] == 0 ? 2 : 0);
                 break;
             }
+        for (int d = 0; d < 4; d++)
+            single_dividend = single_dividend && (dims[d] == 1 || s0[d] == 0);
         a.shift = form;
-        binary_s16_kernel<3><<<grid, dim3(kThreads), 0, stream>>>(a);
+        // int8, one-element dividend: entry 128 of the reference's table (dl_base_div.cpp:19-24) is -128 for 0 / 0
+        a.zero_by_zero = (sizeof(T) == 1 && single_dividend) ? -128 : 0;
+        binary_kernel<T, 3><<<grid, dim3(kThreads), 0, stream>>>(a);
     } else if (op == 2) {
-        binary_s16_kernel<2><<<grid, dim3(kThreads), 0, stream>>>(a);
-    } else if (op == 1) {
-        binary_s16_kernel<1><<<grid, dim3(kThreads), 0, stream>>>(a);
+        binary_kernel<T, 2><<<grid, dim3(kThreads), 0, stream>>>(a);
+    } else if constexpr (sizeof(T) == 2) {
+        if (op == 1)
+            binary_kernel<T, 1><<<grid, dim3(kThreads), 0, stream>>>(a);
+        else
+            binary_kernel<T, 0><<<grid, dim3(kThreads), 0, stream>>>(a);
     } else {
-        binary_s16_kernel<0><<<grid, dim3(kThreads), 0, stream>>>(a);
+        return hipErrorInvalidValue;
     }
     return hipGetLastError();
+}
+
+} // namespace
+
+hipError_t launch_binary_s16(int op, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int16_t *in0,
+                             const int16_t *in1, int shift, bool half_even, int16_t *out, int cu_count, hipStream_t stream)
+{
+    return launch_binary<int16_t>(op, dims, s0, s1, in0, in1, shift, half_even, out, cu_count, stream);
+}
+
+hipError_t launch_subdiv_s8(bool div, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
+                            const int8_t *in1, int shift, int8_t *out, int cu_count, hipStream_t stream)
+{
+    return launch_binary<int8_t>(div ? 3 : 2, dims, s0, s1, in0, in1, shift, false, out, cu_count, stream);
 }
 
 hipError_t launch_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,

@@ -821,6 +821,42 @@ int espdl_hip_div_s16(const int32_t out_dims[4], const int64_t in0_strides[4], c
     return binary_s16(3, out_dims, in0_strides, in1_strides, in0, in1, div_shift, ESPDL_HIP_ROUND_HALF_UP, out, stream);
 }
 
+static int subdiv_s8(bool div, const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int32_t div_shift, int8_t *out, void *stream)
+{
+    if (out_dims == nullptr || in0_strides == nullptr || in1_strides == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "dims and strides must not be NULL");
+    if (div_shift < -30 || div_shift > 30)
+        return fail(ESPDL_HIP_EINVAL, "div_shift %d outside [-30, 30]", div_shift);
+    long long size = 1;
+    for (int i = 0; i < 4; i++) {
+        if (out_dims[i] < 0 || in0_strides[i] < 0 || in1_strides[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative extent or stride in dim %d", i);
+        size *= out_dims[i];
+        if (size > (1ll << 40))
+            return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    }
+    if (size == 0)
+        return ESPDL_HIP_OK;
+    if (in0 == nullptr || in1 == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in0, in1 and out must not be NULL");
+    return device_status(espdl::launch_subdiv_s8(div, out_dims, in0_strides, in1_strides, in0, in1, div_shift, out,
+                                                 cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                         div ? "div_s8" : "sub_s8");
+}
+
+int espdl_hip_sub_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int8_t *out, void *stream)
+{
+    return subdiv_s8(false, out_dims, in0_strides, in1_strides, in0, in1, 0, out, stream);
+}
+
+int espdl_hip_div_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int32_t div_shift, int8_t *out, void *stream)
+{
+    return subdiv_s8(true, out_dims, in0_strides, in1_strides, in0, in1, div_shift, out, stream);
+}
+
 int espdl_hip_avg_pool_s16(const int16_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,
                            int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom, int32_t pad_left,
                            int32_t pad_right, int32_t in_exp, int32_t out_exp, int16_t *out, void *stream)

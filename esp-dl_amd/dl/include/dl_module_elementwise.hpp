@@ -445,21 +445,29 @@ public:
         TensorBase *input1 = context->get_tensor(m_inputs_index[1]);
         TensorBase *output = context->get_tensor(m_outputs_index[0]);
         const char *tag = m_div ? "Div" : "Sub";
-        if (quant_type != QUANT_TYPE_SYMM_16BIT || !on_device_all({input0, input1, output}) || output->shape.size() > 4) {
-            DL_LOGE(tag, "%s: needs int16 device tensors of rank <= 4", name.c_str());
+        const bool s8 = quant_type == QUANT_TYPE_SYMM_8BIT;
+        if ((!s8 && quant_type != QUANT_TYPE_SYMM_16BIT) || !on_device_all({input0, input1, output}) ||
+            output->shape.size() > 4) {
+            DL_LOGE(tag, "%s: needs int8 or int16 device tensors of rank <= 4", name.c_str());
             return;
         }
         int32_t dims[4];
         int64_t s0[4], s1[4];
         broadcast_layout(input0, input1, output, dims, s0, s1);
-        const int rc = m_div
-            ? espdl_hip_div_s16(dims, s0, s1, static_cast<const int16_t *>(input0->data),
-                                static_cast<const int16_t *>(input1->data),
-                                output->exponent.get() - input0->exponent.get() + input1->exponent.get(),
-                                static_cast<int16_t *>(output->data), context->stream)
-            : espdl_hip_sub_s16(dims, s0, s1, static_cast<const int16_t *>(input0->data),
-                                static_cast<const int16_t *>(input1->data), static_cast<int16_t *>(output->data),
-                                context->stream);
+        const int div_shift = output->exponent.get() - input0->exponent.get() + input1->exponent.get();
+        int rc;
+        if (s8) {
+            const int8_t *a = static_cast<const int8_t *>(input0->data), *b = static_cast<const int8_t *>(input1->data);
+            int8_t *y = static_cast<int8_t *>(output->data);
+            rc = m_div ? espdl_hip_div_s8(dims, s0, s1, a, b, div_shift, y, context->stream)
+                       : espdl_hip_sub_s8(dims, s0, s1, a, b, y, context->stream);
+        } else {
+            const int16_t *a = static_cast<const int16_t *>(input0->data),
+                          *b = static_cast<const int16_t *>(input1->data);
+            int16_t *y = static_cast<int16_t *>(output->data);
+            rc = m_div ? espdl_hip_div_s16(dims, s0, s1, a, b, div_shift, y, context->stream)
+                       : espdl_hip_sub_s16(dims, s0, s1, a, b, y, context->stream);
+        }
         if (rc != ESPDL_HIP_OK)
             DL_LOGE(tag, "%s: %s", name.c_str(), espdl_hip_last_error());
     }

@@ -728,6 +728,35 @@ def attention_block(seed=0xE5D8, hw=10, heads=2, key_dim=16, head_dim=32):
     return g
 
 
+def centered_ratio(seed=0xE5DA):
+    """int8 Sub and Div in all of the reference's forms: features minus their spatial mean (broadcast Sub), the
+    result over a one-element constant (divisor table), over a second feature map (element by element, zeros
+    from its ReLU included) and a one-element constant over that map (dividend table)."""
+    g = GraphSpec("centered_ratio")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 14, 14, 16], -5)
+    f = b.conv(x, 32, k=3, name="features")
+    m = b.reduce_mean(f, [1, 2], out_exp=g.exponent(f), name="spatial_mean")
+    ctr = "centered_out"
+    g.add_value(ctr, g.shape(f), g.exponent(f))
+    g.add_node("centered", "Sub", [f, m], [ctr], quant_type="S8")
+    g.add_init("three", [1], INT8, [3], [0])
+    third = "third_out"
+    g.add_value(third, g.shape(f), g.exponent(ctr) - 1)
+    g.add_node("third", "Div", [ctr, "three"], [third], quant_type="S8")
+    d = b.conv(x, 32, k=3, relu=True, name="denominator")
+    ratio = "ratio_out"
+    g.add_value(ratio, g.shape(f), -4)
+    g.add_node("ratio", "Div", [third, d], [ratio], quant_type="S8")
+    g.add_init("numerator", [1], INT8, [100], [-6])
+    inv = "inverse_out"
+    g.add_value(inv, g.shape(f), -4)
+    g.add_node("inverse", "Div", ["numerator", d], [inv], quant_type="S8")
+    g.outputs.append(ratio)
+    g.outputs.append(inv)
+    return g
+
+
 def int16_tail(seed=0xE5D9):
     """int8 Conv -> RequantizeLinear to int16 -> int16 Conv -> int16 table (SiLU) -> int16 Add (residual) ->
     int16 Mul by a constant -> int16 AveragePool -> int16 ReduceMean -> int16 Gemm: the operator mix of the

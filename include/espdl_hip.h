@@ -227,6 +227,16 @@ int espdl_hip_sub_s16(const int32_t out_dims[4], const int64_t in0_strides[4], c
  * dividend constant: (in0 * 2^-s) / in1); in0 == 0 gives 0, in1 == 0 the int16 extreme of in0's sign. */
 int espdl_hip_div_s16(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
                       const int16_t *in0, const int16_t *in1, int32_t div_shift, int16_t *out, void *stream);
+/* base::elemwise_sub and base::elemwise_div for int8 (esp-dl/dl/base/dl_base_sub.cpp:33-43;
+ * esp-dl/dl/base/dl_base_div.cpp:8-46, 66-70, 92-130, 141-175, 208-224).  Sub saturates in0 - in1 to int8.  Div is
+ * the float32 arithmetic of espdl_hip_div_s16 with int8 limits; where an operand is a one-element tensor the
+ * reference reads a 256-entry table built from the same expressions, which differs in one entry only: a
+ * one-element dividend of 0 over a divisor of 0 gives -128.  A one-element divisor of 0 is undefined in the
+ * reference (a float infinity converted to int); here it gives the int8 extreme of in0's sign, 0 for in0 == 0. */
+int espdl_hip_sub_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int8_t *out, void *stream);
+int espdl_hip_div_s8(const int32_t out_dims[4], const int64_t in0_strides[4], const int64_t in1_strides[4],
+                     const int8_t *in0, const int8_t *in1, int32_t div_shift, int8_t *out, void *stream);
 int espdl_hip_avg_pool_s16(const int16_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,
                            int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom, int32_t pad_left,
                            int32_t pad_right, int32_t in_exp, int32_t out_exp, int16_t *out, void *stream);

@@ -755,6 +755,76 @@ void espdl_oracle_div_s16(const int16_t *in0, const int16_t *in1, int64_t size, 
     }
 }
 
+/* Sub, int8 (c_impl_sub_n_n<int8_t>, esp-dl/dl/base/dl_base_sub.cpp:33-43): saturating integer subtraction. */
+void espdl_oracle_sub_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size, int8_t *out)
+{
+    for (int64_t i = 0; i < size; i++) {
+        const int32_t a = in0[len0 == 1 ? 0 : i], b = in1[len1 == 1 ? 0 : i];
+        out[i] = (int8_t)clamp_i64(a - b, INT8_MIN, INT8_MAX);
+    }
+}
+
+/*
+ * Div, int8 (esp-dl/dl/base/dl_base_div.cpp:8-46, 66-70, 92-130, 141-175, 208-224).  The three loops are those
+ * of the int16 form with int8 limits.  When an operand tensor has one element the reference reads a 256-entry
+ * table instead (create_div_lut); this function builds that table the way the reference does and reads it
+ * (table_operand: 0 no table, 1 the dividend is the one element, 2 the divisor is).  A one-element divisor of 0
+ * makes the reference convert an infinity to int, which is undefined; here that entry follows the loop form
+ * (the int8 extreme of the dividend's sign).  Operands are passed already broadcast to `size`.
+ */
+void espdl_oracle_div_s8(const int8_t *in0, const int8_t *in1, int64_t size, int shift, int form, int table_operand,
+                         int8_t *out)
+{
+    const float rescale = dl_rescale(shift);
+    if (table_operand && size > 0) {
+        int8_t table[256];
+        if (table_operand == 1) {
+            const float in0_float = (float)in0[0] * rescale;
+            for (int i = -128; i <= 127; i++) {
+                if (i == 0)
+                    table[i + 128] = in0_float > 0 ? INT8_MAX : INT8_MIN;
+                else
+                    table[i + 128] = (int8_t)clamp_i64(round_half_up_f32(in0_float / (float)i), INT8_MIN, INT8_MAX);
+            }
+            for (int64_t i = 0; i < size; i++)
+                out[i] = table[in1[i] + 128];
+        } else {
+            if (in1[0] == 0) {
+                for (int i = -128; i <= 127; i++)
+                    table[i + 128] = i == 0 ? 0 : (i > 0 ? INT8_MAX : INT8_MIN);
+            } else {
+                const float scale = rescale / (float)in1[0];
+                for (int i = -128; i <= 127; i++)
+                    table[i + 128] =
+                        i == 0 ? 0 : (int8_t)clamp_i64(round_half_up_f32((float)i * scale), INT8_MIN, INT8_MAX);
+            }
+            for (int64_t i = 0; i < size; i++)
+                out[i] = table[in0[i] + 128];
+        }
+        return;
+    }
+    for (int64_t i = 0; i < size; i++) {
+        const int8_t a = in0[i], b = in1[i];
+        if (a == 0) {
+            out[i] = 0;
+        } else if (b == 0) {
+            out[i] = a > 0 ? INT8_MAX : INT8_MIN;
+        } else {
+            float v;
+            if (form == 1) {
+                const float r = rescale / (float)b;
+                v = (float)a * r;
+            } else if (form == 2) {
+                const float r = (float)a * rescale;
+                v = r / (float)b;
+            } else {
+                v = (float)a * rescale / (float)b;
+            }
+            out[i] = (int8_t)clamp_i64(round_half_up_f32(v), INT8_MIN, INT8_MAX);
+        }
+    }
+}
+
 /* AveragePool, int16 (avgpool2d_hwc<int16_t, int32_t>, esp-dl/dl/base/dl_base_avg_pool2d.cpp:28-54, :87). */
 void espdl_oracle_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                                int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,

@@ -72,6 +72,9 @@
  *   espdl_oracle_div_s16         numpy float32 arithmetic in the same order for each of the three forms (IEEE
  *                                operations, so the order is the whole content), and within one unit of the exact
  *                                rational quotient                                                   PINNED
+ *   espdl_oracle_sub_s8          numpy saturating subtraction                                        PINNED
+ *   espdl_oracle_div_s8          as _div_s16 for the three loop forms; the table forms against a table built in
+ *                                numpy float32 from the reference's two expressions, entry by entry   PINNED
  *   espdl_oracle_avg_pool_s16, _reduce_mean_s16   as their int8 forms: exact rationals away from ties
  *                                                                                   PARITY UNPINNED (near-ties)
  *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
@@ -154,6 +157,9 @@ void espdl_oracle_mul_s16(const int16_t *in0, int64_t len0, const int16_t *in1, 
 void espdl_oracle_sub_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size,
                           int16_t *out);
 void espdl_oracle_div_s16(const int16_t *in0, const int16_t *in1, int64_t size, int shift, int form, int16_t *out);
+void espdl_oracle_sub_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size, int8_t *out);
+void espdl_oracle_div_s8(const int8_t *in0, const int8_t *in1, int64_t size, int shift, int form, int table_operand,
+                         int8_t *out);
 void espdl_oracle_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                                int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,
                                int out_exp, int16_t *out);

@@ -69,6 +69,10 @@ def lib():
         L.espdl_oracle_sub_s16.restype = None
         L.espdl_oracle_sub_s16.argtypes = [vp, i64, vp, i64, i64, vp]
         L.espdl_oracle_div_s16.restype = None
+        L.espdl_oracle_sub_s8.restype = None
+        L.espdl_oracle_sub_s8.argtypes = [vp, i64, vp, i64, i64, vp]
+        L.espdl_oracle_div_s8.restype = None
+        L.espdl_oracle_div_s8.argtypes = [vp, vp, i64, i32, i32, i32, vp]
         L.espdl_oracle_div_s16.argtypes = [vp, vp, i64, i32, i32, vp]
         L.espdl_oracle_avg_pool_s16.restype = None
         L.espdl_oracle_avg_pool_s16.argtypes = [vp] + [i32] * 14 + [vp]
@@ -327,9 +331,10 @@ def sub_s16(a, b):
     return out
 
 
-def div_form(shape_a, shape_b):
+def div_form(shape_a, shape_b, all_ones=1):
     """Which of the reference's three loops runs: 1 if the divisor is constant along the innermost axis of the
-    result that is longer than 1, 2 if the dividend is, else 0."""
+    result that is longer than 1, 2 if the dividend is, else 0.  A result of one element takes `all_ones`: the
+    int16 dispatcher tests the divisor first, the int8 one the dividend."""
     out = np.broadcast_shapes(tuple(shape_a), tuple(shape_b))
     rank = len(out)
     pa = (1,) * (rank - len(shape_a)) + tuple(shape_a)
@@ -337,7 +342,30 @@ def div_form(shape_a, shape_b):
     for d in range(rank - 1, -1, -1):
         if out[d] > 1:
             return 1 if pb[d] == 1 else (2 if pa[d] == 1 else 0)
-    return 1
+    return all_ones
+
+
+def sub_s8(a, b):
+    a = _c(a, np.int8)
+    b = _c(b, np.int8)
+    size = max(a.size, b.size)
+    assert a.size in (1, size) and b.size in (1, size)
+    out = np.empty(a.shape if a.size == size else b.shape, dtype=np.int8)
+    lib().espdl_oracle_sub_s8(_ptr(a), a.size, _ptr(b), b.size, size, _ptr(out))
+    return out
+
+
+def div_s8(a, b, shift):
+    """numpy-broadcast quotient; shift = out_exp - a_exp + b_exp.  A one-element operand selects the reference's
+    table form, the dividend first (esp-dl/dl/base/dl_base_div.cpp:17, 33, 212-224)."""
+    a, b = np.asarray(a, dtype=np.int8), np.asarray(b, dtype=np.int8)
+    table_operand = 1 if a.size == 1 else (2 if b.size == 1 else 0)
+    form = div_form(a.shape, b.shape, all_ones=2)
+    a, b = np.broadcast_arrays(a, b)
+    a, b = np.ascontiguousarray(a), np.ascontiguousarray(b)
+    out = np.empty(a.shape, dtype=np.int8)
+    lib().espdl_oracle_div_s8(_ptr(a), _ptr(b), a.size, int(shift), form, table_operand, _ptr(out))
+    return out
 
 
 def div_s16(a, b, shift):

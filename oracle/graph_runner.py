@@ -36,7 +36,7 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None
     for node in spec.nodes:
         op, a = node["op_type"], node["attrs"]
         ins, outs = node["inputs"], node["outputs"]
-        x = t[ins[0]]
+        x = operand(ins[0])
         y_name = outs[0]
         if op == "Conv":
             dims, wdt, w, _ = spec.initializers[ins[1]]
@@ -106,16 +106,14 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None
             y = add(np.ascontiguousarray(x), np.ascontiguousarray(b))
         elif op == "Sub":
             b = operand(ins[1])
-            if x.dtype != np.int16:
-                raise NotImplementedError("Sub on " + str(x.dtype))
             if x.shape != b.shape:
                 x, b = np.broadcast_arrays(x, b)
-            y = oracle.sub_s16(np.ascontiguousarray(x), np.ascontiguousarray(b))
+            sub = oracle.sub_s16 if x.dtype == np.int16 else oracle.sub_s8
+            y = sub(np.ascontiguousarray(x), np.ascontiguousarray(b))
         elif op == "Div":
             b = operand(ins[1])
-            if x.dtype != np.int16:
-                raise NotImplementedError("Div on " + str(x.dtype))
-            y = oracle.div_s16(x, b, spec.exponent(y_name) - exponent_of(ins[0]) + exponent_of(ins[1]))
+            div = oracle.div_s16 if x.dtype == np.int16 else oracle.div_s8
+            y = div(x, b, spec.exponent(y_name) - exponent_of(ins[0]) + exponent_of(ins[1]))
         elif op == "Mul":
             b = operand(ins[1])
             shift = spec.exponent(y_name) - exponent_of(ins[0]) - exponent_of(ins[1])

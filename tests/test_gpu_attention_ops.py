@@ -216,3 +216,41 @@ def test_div_s16(oracle, shapes, shift):
     b.flat[-1] = 0
     got = to_host(espdl().div_s16(to_dev(a), to_dev(b), shift))
     np.testing.assert_array_equal(got, oracle.div_s16(a, b, shift))
+
+
+def test_sub_s8(oracle):
+    announce("sub_s8")
+    rng = np.random.default_rng(65)
+    a, b = _rand(rng, (2, 286, 800), np.int8), _rand(rng, (2, 1, 800), np.int8)
+    want = np.clip(a.astype(np.int32) - b.astype(np.int32), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(to_host(espdl().sub_s8(to_dev(a), to_dev(b))), want)
+    np.testing.assert_array_equal(to_host(espdl().sub_s8(to_dev(a), to_dev(a))), oracle.sub_s8(a, a))
+
+
+@pytest.mark.parametrize("shapes", [((4, 3000), (4, 3000)), ((2, 800), (1,)), ((4, 300), (4, 1)), ((1,), (4, 300)),
+                                    ((4, 1), (4, 300)), ((1, 1), (1,))], ids=str)
+@pytest.mark.parametrize("shift", [-3, 0, 3, 6])
+def test_div_s8(oracle, shapes, shift):
+    """Loop forms and both table forms of the reference, zero operands included (a one-element divisor of zero is
+    undefined there and left out)."""
+    announce(f"div_s8 {shapes} shift={shift}")
+    rng = np.random.default_rng(66)
+    for scalar0 in (0, 1):
+        a, b = _rand(rng, shapes[0], np.int8), _rand(rng, shapes[1], np.int8)
+        a.flat[0] = 0 if scalar0 == 0 else 37
+        b.flat[-1] = 0
+        if b.size == 1:
+            b.flat[0] = -5
+        b.flat[0] = 0 if b.size > 1 else b.flat[0]
+        got = to_host(espdl().div_s8(to_dev(a), to_dev(b), shift))
+        np.testing.assert_array_equal(got, oracle.div_s8(a, b, shift))
+
+
+def test_div_s8_one_element_operands(oracle):
+    announce("div_s8 one-element operands")
+    zero = np.array([0], np.int8)
+    got = to_host(espdl().div_s8(to_dev(zero), to_dev(zero), 0))
+    np.testing.assert_array_equal(got, oracle.div_s8(zero, zero, 0))
+    assert got[0] == -128
+    z16 = np.array([0], np.int16)
+    assert to_host(espdl().div_s16(to_dev(z16), to_dev(z16), 0))[0] == 0

@@ -258,6 +258,19 @@ def test_int16_tail(oracle, round_mode):
     mdl.close()
 
 
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+def test_centered_ratio(oracle, round_mode):
+    """int8 Sub (broadcast) and Div in its loop and both table forms, through dl::Model."""
+    announce(f"model centered_ratio round_mode={round_mode}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.centered_ratio()
+    mdl, want, _ = _run_config(spec, 3, 39, round_mode=round_mode)
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want[name])
+        assert len(np.unique(want[name])) > 8
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()

@@ -224,3 +224,71 @@ def test_div_s16_is_float32_arithmetic_in_the_reference_order(oracle, shapes, fo
     exact = af[ok].astype(np.float64) * 2.0 ** -shift / bf[ok].astype(np.float64)
     inside = np.abs(exact) < 32000
     assert np.all(np.abs(got[ok][inside] - exact[inside]) <= 1.0)
+
+
+def test_sub_s8_saturates(oracle):
+    rng = np.random.default_rng(55)
+    a, b = _rand(rng, (3, 1000), np.int8), _rand(rng, (3, 1000), np.int8)
+    want = np.clip(a.astype(np.int32) - b.astype(np.int32), -128, 127).astype(np.int8)
+    np.testing.assert_array_equal(oracle.sub_s8(a, b), want)
+    np.testing.assert_array_equal(oracle.sub_s8(a, np.array([-128], np.int8)),
+                                  np.clip(a.astype(np.int32) + 128, -128, 127).astype(np.int8))
+
+
+@pytest.mark.parametrize("shapes,form", [(((4, 300), (4, 300)), 0), (((4, 300), (4, 1)), 1), (((4, 1), (4, 300)), 2)],
+                         ids=str)
+@pytest.mark.parametrize("shift", [-3, 0, 4])
+def test_div_s8_loop_forms_are_float32_arithmetic_in_the_reference_order(oracle, shapes, form, shift):
+    """No one-element operand, so the reference runs its loops (dl_base_div.cpp:92-112, 141-163, 175-195): IEEE
+    float32 operations in numpy in the same order, and within one unit of the exact quotient."""
+    rng = np.random.default_rng(56)
+    a, b = _rand(rng, shapes[0], np.int8), _rand(rng, shapes[1], np.int8)
+    a.flat[0] = 0
+    b.flat[-1] = 0
+    got = oracle.div_s8(a, b, shift)
+    af, bf = np.broadcast_arrays(a.astype(np.float32), b.astype(np.float32))
+    r = np.float32(2.0 ** -shift)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        v = af * (r / bf) if form == 1 else ((af * r) / bf if form == 2 else af * r / bf)
+    q = np.floor(v.astype(np.float64) + 0.5)
+    want = np.clip(np.nan_to_num(q, nan=0.0, posinf=127, neginf=-128), -128, 127).astype(np.int8)
+    want = np.where(af == 0, 0, np.where(bf == 0, np.where(af > 0, 127, -128), want)).astype(np.int8)
+    np.testing.assert_array_equal(got, want)
+    ok = (af != 0) & (bf != 0)
+    exact = af[ok].astype(np.float64) * 2.0 ** -shift / bf[ok].astype(np.float64)
+    inside = np.abs(exact) < 120
+    assert np.all(np.abs(got[ok][inside] - exact[inside]) <= 1.0)
+
+
+@pytest.mark.parametrize("shift", [-3, 0, 2, 5])
+@pytest.mark.parametrize("scalar", [-128, -77, -1, 0, 1, 5, 127])
+def test_div_s8_table_forms_follow_create_div_lut(oracle, scalar, shift):
+    """A one-element operand makes the reference read a table (dl_base_div.cpp:8-46): rebuilt here entry by entry
+    in numpy float32 from its two expressions, over all 256 values of the other operand."""
+    r = np.float32(2.0 ** -shift)
+    other = np.arange(-128, 128, dtype=np.int8).reshape(2, 128)
+    i = other.astype(np.float32)
+    one = np.array([scalar], np.int8)
+
+    def rounded(v):
+        return np.clip(np.floor(v.astype(np.float64) + 0.5), -128, 127).astype(np.int8)
+
+    # one-element dividend: table[i] = round((in0 * rescale) / i), entry 0 by the sign of in0 * rescale
+    in0_float = np.float32(scalar) * r
+    with np.errstate(divide="ignore", invalid="ignore"):
+        want = rounded(np.where(other == 0, np.float32(1), in0_float / i))
+    want = np.where(other == 0, 127 if in0_float > 0 else -128, want).astype(np.int8)
+    np.testing.assert_array_equal(oracle.div_s8(one, other, shift), want)
+    # one-element divisor: table[i] = round(i * (rescale / in1)), entry 0 is 0
+    if scalar != 0:
+        want = rounded(i * (r / np.float32(scalar)))
+        want = np.where(other == 0, 0, want).astype(np.int8)
+        np.testing.assert_array_equal(oracle.div_s8(other, one, shift), want)
+
+
+def test_div_s8_one_element_result_uses_the_dividend_table(oracle):
+    # both operands have one element: create_div_lut and elemwise_div test the dividend first
+    assert oracle.div_s8(np.array([0], np.int8), np.array([0], np.int8), 0)[0] == -128
+    assert oracle.div_s8(np.array([[0]], np.int8), np.array([[0, 3]], np.int8), 0).tolist() == [[-128, 0]]
+    assert oracle.div_s8(np.array([[0, 3]], np.int8), np.array([[0, 3]], np.int8), 0).tolist() == [[0, 1]]
+    assert oracle.div_form((1,), (1,), all_ones=2) == 2 and oracle.div_form((1,), (1,)) == 1
