@@ -21,6 +21,8 @@ typedef int esp_err_t;
 #define DL_LOGW(tag, fmt, ...) std::fprintf(stderr, "W (%s) " fmt "\n", tag, ##__VA_ARGS__)
 #define DL_LOGI(tag, fmt, ...) std::fprintf(stdout, "I (%s) " fmt "\n", tag, ##__VA_ARGS__)
 
+#define DL_MAX(x, y) (((x) < (y)) ? (y) : (x))
+#define DL_MIN(x, y) (((x) < (y)) ? (x) : (y))
 #define DL_CLIP(x, low, high) (((x) < (low)) ? (low) : (((x) > (high)) ? (high) : (x)))
 #define DL_SCALE(exponent) (((exponent) > 0) ? (float)(1 << (exponent)) : ((float)1.0 / (float)(1 << -(exponent))))
 #define DL_RESCALE(exponent) (((exponent) > 0) ? ((float)1.0 / (float)(1 << (exponent))) : (float)(1 << -(exponent)))

@@ -16,6 +16,7 @@
 #include "dl_module_elementwise.hpp"
 #include "dl_module_gemm.hpp"
 #include "dl_module_layout.hpp"
+#include "dl_module_unary.hpp"
 
 namespace dl {
 namespace module {
@@ -81,16 +82,30 @@ public:
         // (esp-dl/dl/module/include/dl_module_creator.hpp:154-155)
         register_module("QuantizeLinear", RequantizeLinear::deserialize);
         register_module("DequantizeLinear", RequantizeLinear::deserialize);
-        // element-wise activations that esp-ppq exports with a precomputed 8-bit table
-        for (const char *op : {"Swish", "HardSwish", "Sigmoid", "HardSigmoid", "Tanh", "Gelu", "Elu", "LeakyRelu",
-                               "Exp", "Log", "Sqrt", "Softplus", "Mish"}) {
+        // element-wise activations: a node with a precomputed table becomes a LUT, otherwise the reference's
+        // float32 expression is evaluated per possible input (dl_module_unary.hpp)
+        register_module("Sigmoid", UnaryMath::deserialize<UNARY_SIGMOID>);
+        register_module("Tanh", UnaryMath::deserialize<UNARY_TANH>);
+        register_module("HardSwish", UnaryMath::deserialize<UNARY_HARD_SWISH>);
+        register_module("Elu", UnaryMath::deserialize<UNARY_ELU>);
+        register_module("Exp", UnaryMath::deserialize<UNARY_EXP>);
+        register_module("Log", UnaryMath::deserialize<UNARY_LOG>);
+        register_module("Sqrt", UnaryMath::deserialize<UNARY_SQRT>);
+        register_module("LeakyRelu", UnaryMath::deserialize<UNARY_LEAKY_RELU>);
+        register_module("Neg", UnaryMath::deserialize<UNARY_NEG>);
+        register_module("Swish", UnaryMath::deserialize<UNARY_SWISH>);
+        register_module("HardSigmoid", UnaryMath::deserialize<UNARY_HARD_SIGMOID>);
+        // Identity is output->assign(input) (esp-dl/dl/module/include/dl_module_identity.hpp:34-42)
+        register_module("Identity", RequantizeLinear::deserialize);
+        // exported only with a table (esp-dl/dl/module/include/dl_module_creator.hpp:151)
+        for (const char *op : {"Gelu", "Softplus", "Mish"}) {
             const std::string op_type = op;
             register_module(op_type, [op_type](fbs::FbsModel *fbs_model, std::string node_name) -> Module * {
                 quant_type_t quant_type = QUANT_TYPE_NONE;
                 fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
                 Module *m = lut_if_present(fbs_model, node_name, quant_type);
                 if (!m)
-                    DL_LOGE("ModuleCreator", "%s (%s) has no 8-bit LUT; the float fallback is not part of this build",
+                    DL_LOGE("ModuleCreator", "%s (%s) has no table; only the table form is implemented",
                             node_name.c_str(), op_type.c_str());
                 return m;
             });

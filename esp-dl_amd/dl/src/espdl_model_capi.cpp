@@ -200,6 +200,18 @@ int espdl_graph_node_set_int(espdl_graph *g, const char *node, const char *key, 
     return 0;
 }
 
+int espdl_graph_node_set_float(espdl_graph *g, const char *node, const char *key, float value)
+{
+    fbs::Node *n = g ? g->fbs.get_node(node) : nullptr;
+    if (!n)
+        return -1;
+    fbs::Attribute a;
+    a.kind = fbs::Attribute::FLOAT;
+    a.f = value;
+    n->attributes[key] = a;
+    return 0;
+}
+
 int espdl_graph_node_set_ints(espdl_graph *g, const char *node, const char *key, const int64_t *values, int32_t count)
 {
     fbs::Node *n = g ? g->fbs.get_node(node) : nullptr;

@@ -33,6 +33,7 @@ def lib():
         L.espdl_graph_add_output.argtypes = [vp, cp]
         L.espdl_graph_add_node.argtypes = [vp, cp, cp, ctypes.POINTER(cp), i32, ctypes.POINTER(cp), i32]
         L.espdl_graph_node_set_int.argtypes = [vp, cp, cp, i64]
+        L.espdl_graph_node_set_float.argtypes = [vp, cp, cp, ctypes.c_float]
         L.espdl_graph_node_set_ints.argtypes = [vp, cp, cp, ctypes.POINTER(i64), i32]
         L.espdl_graph_node_set_string.argtypes = [vp, cp, cp, cp]
         L.espdl_graph_add_test_input.argtypes = [vp, cp, pi32, i32, i32, vp, i32]
@@ -121,6 +122,8 @@ class Graph:
                 elif isinstance(val, (list, tuple)):
                     arr = (ctypes.c_int64 * len(val))(*[int(v) for v in val])
                     L.espdl_graph_node_set_ints(g.h, nm, key.encode(), arr, len(val))
+                elif isinstance(val, float):
+                    L.espdl_graph_node_set_float(g.h, nm, key.encode(), val)
                 else:
                     L.espdl_graph_node_set_int(g.h, nm, key.encode(), int(val))
         if test_input is not None:

@@ -757,6 +757,49 @@ def centered_ratio(seed=0xE5DA):
     return g
 
 
+def activation_chain(seed=0xE5DB, s16=False):
+    """Every activation module that the reference evaluates in float32 per element, without tables in the file:
+    Conv -> Sigmoid / Tanh / HardSwish / Elu / LeakyRelu / Swish / HardSigmoid / Neg branches summed pairwise,
+    then Exp, Sqrt and Log on tensors whose sign suits them, and an Identity that changes the exponent."""
+    g = GraphSpec("activation_chain_s16" if s16 else "activation_chain")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    qt, dt = ("S16", INT16) if s16 else ("S8", INT8)
+    bits = 15 if s16 else 7
+    x = b.input("input", [1, 10, 10, 16], -5)
+    f = b.conv(x, 32, k=3, name="features")              # spans roughly [-4, 4) at its exponent
+    fe = g.exponent(f)
+    if s16:
+        f16 = "features_s16"
+        g.add_value(f16, g.shape(f), fe - 8, INT16)
+        g.add_node("to_s16", "RequantizeLinear", [f], [f16], quant_type="S16")
+        f = b.conv(f16, 32, k=1, s16=True, out_exp=fe - 8, name="mixed")   # int16 values, not multiples of 256
+        fe = fe - 8
+    span = fe + bits                                      # the input covers [-2^span, 2^span)
+
+    def unary(op, src, out_exp, name, **attrs):
+        y = name + "_out"
+        g.add_value(y, g.shape(src), out_exp, dt)
+        g.add_node(name, op, [src], [y], quant_type=qt, **attrs)
+        return y
+
+    outs = [unary("Sigmoid", f, -bits, "sigmoid"),
+            unary("Tanh", f, -bits, "tanh"),
+            unary("HardSwish", f, span - bits, "hard_swish"),
+            unary("Elu", f, span - bits, "elu", alpha=0.75),
+            unary("LeakyRelu", f, span - bits, "leaky_relu", alpha=0.1),
+            unary("Swish", f, span - bits, "swish"),
+            unary("HardSigmoid", f, -bits, "hard_sigmoid", alpha=0.25, beta=0.5),
+            unary("HardSigmoid", f, -bits, "hard_sigmoid_default"),
+            unary("Neg", f, fe, "neg")]
+    small = unary("Identity", f, fe + 2, "quarter")       # a requantize by assign
+    outs.append(unary("Exp", outs[1], 2 - bits, "exp"))   # exp(tanh) in (0.36, 2.72)
+    pos = unary("Sigmoid", small, -bits, "gate")
+    outs.append(unary("Sqrt", pos, -bits, "sqrt"))
+    outs.append(unary("Log", pos, 3 - bits, "log"))       # log(sigmoid) in (-4.1, 0)
+    g.outputs.extend(outs)
+    return g
+
+
 def int16_tail(seed=0xE5D9):
     """int8 Conv -> RequantizeLinear to int16 -> int16 Conv -> int16 table (SiLU) -> int16 Add (residual) ->
     int16 Mul by a constant -> int16 AveragePool -> int16 ReduceMean -> int16 Gemm: the operator mix of the

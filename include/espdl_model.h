@@ -67,6 +67,7 @@ int espdl_graph_add_output(espdl_graph *g, const char *name);
 int espdl_graph_add_node(espdl_graph *g, const char *name, const char *op_type, const char *const *inputs,
                          int32_t n_inputs, const char *const *outputs, int32_t n_outputs);
 int espdl_graph_node_set_int(espdl_graph *g, const char *node, const char *key, int64_t value);
+int espdl_graph_node_set_float(espdl_graph *g, const char *node, const char *key, float value);
 int espdl_graph_node_set_ints(espdl_graph *g, const char *node, const char *key, const int64_t *values, int32_t n);
 int espdl_graph_node_set_string(espdl_graph *g, const char *node, const char *key, const char *value);
 /* Known-answer vectors checked by espdl_model_test (whole-batch tensors). */

@@ -825,6 +825,114 @@ void espdl_oracle_div_s8(const int8_t *in0, const int8_t *in1, int64_t size, int
     }
 }
 
+/*
+ * The activation modules that compute in float32 per element: Sigmoid, Tanh, HardSwish, Elu, Exp, Log, Sqrt,
+ * LeakyRelu, Swish, HardSigmoid, and the integer Neg.  All of them (int8 and int16 alike) are
+ *     out = truncate(tool::round(f(q * DL_SCALE(in_exp)) * DL_RESCALE(out_exp)))
+ * with f written exactly as the module writes it, float / double promotions included:
+ *   sigmoid(x) = (float)(1.0 / (1.0 + expf(-x)))            esp-dl/dl/math/include/dl_math.hpp:200-203
+ *   tanh(x)    = 2 * sigmoid(2 * x) - 1                      dl_math.hpp:205-208
+ *   Sigmoid    dl_module_sigmoid.hpp:33-52                   Tanh       dl_module_tanh.hpp:47-66
+ *   HardSwish  max(0, min(1, 0.166667 * x + 0.5)) * x in double, stored to float   dl_module_hard_swish.hpp:66-76
+ *   Elu        x >= 0 ? x : alpha * (expf(x) - 1)            dl_module_elu.hpp:68-82
+ *   Exp, Log, Sqrt   expf / logf / sqrtf                     dl_module_exp.hpp:62-72, _log.hpp:61-71, _sqrt.hpp:61-71
+ *   LeakyRelu  x >= 0 ? x * rescale : x * rescale * alpha    dl_module_leaky_relu.hpp:74-87
+ *   Swish      sigmoid(x) * x                                dl_module_swish.hpp:66-76
+ *   HardSigmoid max(0, min(1, alpha * x + beta)) in float    dl_module_hard_sigmoid.hpp:74-84
+ *   Neg        -q, the minimum maps to the maximum           dl_module_neg.hpp:57-86
+ * tool::round is floorf(v + 0.5) in the portable build and round_half_even((double)v) in the ESP32-P4 build
+ * (esp-dl/dl/tool/src/dl_tool.cpp:50-91).  Where f is not a number (Log or Sqrt of a negative input) or infinite
+ * the reference converts it to int, which is undefined: this restatement gives 0 for NaN and saturates infinities.
+ */
+static int round_half_even_f64(double value)
+{
+    const double rounded = value < 0 ? value - 0.5 : value + 0.5;
+    int int_part = (int)rounded;
+    if (fabs(rounded - int_part) < 1e-6 && (int_part & 1) != 0)
+        int_part += value < 0 ? 1 : -1;
+    return int_part;
+}
+
+static float oracle_sigmoid(float x)
+{
+    return 1.0 / (1.0 + expf(-x));
+}
+
+static int64_t unary_value(int kind, int q, float in_scale, float out_scale, float alpha, float beta, int round_mode,
+                           int lo, int hi)
+{
+    float temp = (float)q * in_scale, v;
+    switch (kind) {
+    case ESPDL_ORACLE_UNARY_SIGMOID:
+        v = oracle_sigmoid(temp) * out_scale;
+        break;
+    case ESPDL_ORACLE_UNARY_TANH:
+        temp = 2 * oracle_sigmoid(2 * temp) - 1;
+        v = temp * out_scale;
+        break;
+    case ESPDL_ORACLE_UNARY_HARD_SWISH: {
+        const double gate = 0.166667 * temp + 0.5;
+        const double clipped = gate > 1 ? 1 : (gate < 0 ? 0 : gate);
+        temp = clipped * temp;
+        v = temp * out_scale;
+        break;
+    }
+    case ESPDL_ORACLE_UNARY_ELU:
+        v = temp >= 0 ? temp * out_scale : alpha * (expf(temp) - 1) * out_scale;
+        break;
+    case ESPDL_ORACLE_UNARY_EXP:
+        v = expf(temp) * out_scale;
+        break;
+    case ESPDL_ORACLE_UNARY_LOG:
+        v = logf(temp) * out_scale;
+        break;
+    case ESPDL_ORACLE_UNARY_SQRT:
+        v = sqrtf(temp) * out_scale;
+        break;
+    case ESPDL_ORACLE_UNARY_LEAKY_RELU:
+        v = temp >= 0 ? temp * out_scale : temp * out_scale * alpha;
+        break;
+    case ESPDL_ORACLE_UNARY_SWISH:
+        temp = oracle_sigmoid(temp) * temp;
+        v = temp * out_scale;
+        break;
+    case ESPDL_ORACLE_UNARY_HARD_SIGMOID: {
+        const float gate = alpha * temp + beta;
+        temp = gate > 1 ? 1 : (gate < 0 ? 0 : gate);
+        v = temp * out_scale;
+        break;
+    }
+    case ESPDL_ORACLE_UNARY_NEG:
+        return q == lo ? hi : -q;
+    default:
+        return 0;
+    }
+    if (isnan(v))
+        return 0;
+    if (v >= 2147483520.f)
+        return hi;
+    if (v <= -2147483520.f)
+        return lo;
+    const int r = round_mode == ESPDL_ORACLE_ROUND_HALF_EVEN ? round_half_even_f64((double)v) : round_half_up_f32(v);
+    return clamp_i64(r, lo, hi);
+}
+
+void espdl_oracle_unary_s8(int kind, const int8_t *in, int64_t size, int in_exp, int out_exp, float alpha, float beta,
+                           int round_mode, int8_t *out)
+{
+    const float in_scale = dl_scale(in_exp), out_scale = dl_rescale(out_exp);
+    for (int64_t i = 0; i < size; i++)
+        out[i] = (int8_t)unary_value(kind, in[i], in_scale, out_scale, alpha, beta, round_mode, INT8_MIN, INT8_MAX);
+}
+
+void espdl_oracle_unary_s16(int kind, const int16_t *in, int64_t size, int in_exp, int out_exp, float alpha, float beta,
+                            int round_mode, int16_t *out)
+{
+    const float in_scale = dl_scale(in_exp), out_scale = dl_rescale(out_exp);
+    for (int64_t i = 0; i < size; i++)
+        out[i] = (int16_t)unary_value(kind, in[i], in_scale, out_scale, alpha, beta, round_mode, INT16_MIN, INT16_MAX);
+}
+
 /* AveragePool, int16 (avgpool2d_hwc<int16_t, int32_t>, esp-dl/dl/base/dl_base_avg_pool2d.cpp:28-54, :87). */
 void espdl_oracle_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                                int stride_w, int pad_top, int pad_bottom, int pad_left, int pad_right, int in_exp,

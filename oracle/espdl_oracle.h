@@ -72,6 +72,11 @@
  *   espdl_oracle_div_s16         numpy float32 arithmetic in the same order for each of the three forms (IEEE
  *                                operations, so the order is the whole content), and within one unit of the exact
  *                                rational quotient                                                   PINNED
+ *   espdl_oracle_unary_s8, _s16  every function against its closed form in numpy float64 (within one output unit
+ *                                everywhere, equal away from rounding ties), the float / double promotions of
+ *                                HardSwish and sigmoid against numpy operations of those widths; expf / logf
+ *                                are the host libm's, which may differ from the target's in the last bit
+ *                                                                       PARITY UNPINNED (libm last-bit, near-ties)
  *   espdl_oracle_sub_s8          numpy saturating subtraction                                        PINNED
  *   espdl_oracle_div_s8          as _div_s16 for the three loop forms; the table forms against a table built in
  *                                numpy float32 from the reference's two expressions, entry by entry   PINNED
@@ -157,6 +162,23 @@ void espdl_oracle_mul_s16(const int16_t *in0, int64_t len0, const int16_t *in1, 
 void espdl_oracle_sub_s16(const int16_t *in0, int64_t len0, const int16_t *in1, int64_t len1, int64_t size,
                           int16_t *out);
 void espdl_oracle_div_s16(const int16_t *in0, const int16_t *in1, int64_t size, int shift, int form, int16_t *out);
+enum {
+    ESPDL_ORACLE_UNARY_SIGMOID = 0,
+    ESPDL_ORACLE_UNARY_TANH = 1,
+    ESPDL_ORACLE_UNARY_HARD_SWISH = 2,
+    ESPDL_ORACLE_UNARY_ELU = 3,
+    ESPDL_ORACLE_UNARY_EXP = 4,
+    ESPDL_ORACLE_UNARY_LOG = 5,
+    ESPDL_ORACLE_UNARY_SQRT = 6,
+    ESPDL_ORACLE_UNARY_LEAKY_RELU = 7,
+    ESPDL_ORACLE_UNARY_NEG = 8,
+    ESPDL_ORACLE_UNARY_SWISH = 9,
+    ESPDL_ORACLE_UNARY_HARD_SIGMOID = 10
+};
+void espdl_oracle_unary_s8(int kind, const int8_t *in, int64_t size, int in_exp, int out_exp, float alpha, float beta,
+                           int round_mode, int8_t *out);
+void espdl_oracle_unary_s16(int kind, const int16_t *in, int64_t size, int in_exp, int out_exp, float alpha, float beta,
+                            int round_mode, int16_t *out);
 void espdl_oracle_sub_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size, int8_t *out);
 void espdl_oracle_div_s8(const int8_t *in0, const int8_t *in1, int64_t size, int shift, int form, int table_operand,
                          int8_t *out);

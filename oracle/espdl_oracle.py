@@ -69,6 +69,10 @@ def lib():
         L.espdl_oracle_sub_s16.restype = None
         L.espdl_oracle_sub_s16.argtypes = [vp, i64, vp, i64, i64, vp]
         L.espdl_oracle_div_s16.restype = None
+        L.espdl_oracle_unary_s8.restype = None
+        L.espdl_oracle_unary_s8.argtypes = [i32, vp, i64, i32, i32, ctypes.c_float, ctypes.c_float, i32, vp]
+        L.espdl_oracle_unary_s16.restype = None
+        L.espdl_oracle_unary_s16.argtypes = [i32, vp, i64, i32, i32, ctypes.c_float, ctypes.c_float, i32, vp]
         L.espdl_oracle_sub_s8.restype = None
         L.espdl_oracle_sub_s8.argtypes = [vp, i64, vp, i64, i64, vp]
         L.espdl_oracle_div_s8.restype = None
@@ -343,6 +347,27 @@ def div_form(shape_a, shape_b, all_ones=1):
         if out[d] > 1:
             return 1 if pb[d] == 1 else (2 if pa[d] == 1 else 0)
     return all_ones
+
+
+UNARY_KINDS = {"Sigmoid": 0, "Tanh": 1, "HardSwish": 2, "Elu": 3, "Exp": 4, "Log": 5, "Sqrt": 6, "LeakyRelu": 7,
+               "Neg": 8, "Swish": 9, "HardSigmoid": 10}
+# default attribute values of the reference's deserializers (dl_module_elu.hpp:92, dl_module_leaky_relu.hpp:99,
+# dl_module_hard_sigmoid.hpp: alpha 0.2, beta 0.5)
+UNARY_DEFAULTS = {"Elu": (1.0, 0.0), "LeakyRelu": (0.01, 0.0), "HardSigmoid": (0.2, 0.5)}
+
+
+def unary(op_type, x, in_exp, out_exp, alpha=None, beta=None, round_mode=ROUND_HALF_UP):
+    """The float32-per-element activation modules and Neg, int8 or int16 by the dtype of x."""
+    x = np.ascontiguousarray(x)
+    assert x.dtype in (np.int8, np.int16)
+    da, db = UNARY_DEFAULTS.get(op_type, (0.0, 0.0))
+    alpha = da if alpha is None else alpha
+    beta = db if beta is None else beta
+    out = np.empty_like(x)
+    fn = lib().espdl_oracle_unary_s8 if x.dtype == np.int8 else lib().espdl_oracle_unary_s16
+    fn(UNARY_KINDS[op_type], _ptr(x), x.size, int(in_exp), int(out_exp), float(alpha), float(beta), int(round_mode),
+       _ptr(out))
+    return out
 
 
 def sub_s8(a, b):

@@ -104,6 +104,10 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None
                 x, b = np.broadcast_arrays(x, b)
             add = oracle.add_s16 if x.dtype == np.int16 else oracle.add_s8
             y = add(np.ascontiguousarray(x), np.ascontiguousarray(b))
+        elif op in oracle.UNARY_KINDS:
+            y = oracle.unary(op, x, exponent_of(ins[0]), spec.exponent(y_name), a.get("alpha"), a.get("beta"), round_mode)
+        elif op == "Identity":  # output->assign(input): a requantize when the exponents differ
+            y = requantize(x, spec.exponent(ins[0]), spec.exponent(y_name), spec.dtype(y_name))
         elif op == "Sub":
             b = operand(ins[1])
             if x.shape != b.shape:

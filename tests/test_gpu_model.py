@@ -271,6 +271,22 @@ def test_centered_ratio(oracle, round_mode):
     mdl.close()
 
 
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+@pytest.mark.parametrize("s16", [False, True], ids=["s8", "s16"])
+def test_activation_chain(oracle, s16, round_mode):
+    """Sigmoid, Tanh, HardSwish, Elu, LeakyRelu, Swish, HardSigmoid, Neg, Exp, Sqrt, Log and Identity nodes
+    without tables in the file: the module evaluates the reference's float32 expression per possible input."""
+    announce(f"model activation_chain s16={s16} round_mode={round_mode}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.activation_chain(s16=s16)
+    mdl, want, _ = _run_config(spec, 3, 41, round_mode=round_mode)
+    for name in spec.outputs:
+        got = mdl.get_tensor(name, np.int16) if s16 else mdl.get_tensor(name)
+        np.testing.assert_array_equal(got, want[name], err_msg=name)
+        assert len(np.unique(want[name])) > 20, name
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()
