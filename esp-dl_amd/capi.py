@@ -90,6 +90,8 @@ def lib():
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         L.espdl_hip_insert_zeros.argtypes = [vp] + [i32] * 9 + [vp, vp]
         L.espdl_hip_insert_zeros.restype = ctypes.c_int
+        L.espdl_hip_pad.argtypes = [vp, vp, i32, vp, i32, i32, i32, vp, vp]
+        L.espdl_hip_pad.restype = ctypes.c_int
         L.espdl_hip_lut_s16.argtypes = [vp, i64, vp, i32, i32, vp, vp]
         L.espdl_hip_lut_s16.restype = ctypes.c_int
         L.espdl_hip_softmax_s8.argtypes = [vp, i64, i64, i64, i32, vp, vp]
@@ -515,6 +517,21 @@ def sub_s16(a, b, stream=None):
     dims, s0, s1, out = _broadcast16(a, b)
     _check(lib().espdl_hip_sub_s16(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), _p(out),
                                    _stream(stream)))
+    return out
+
+
+PAD_MODES = {"constant": 0, "edge": 1, "reflect": 2}
+
+
+def pad(x, pads, mode="constant", value=0, stream=None):
+    """pads: the leading pad of every axis, then the trailing pad of every axis (espdl_hip_pad)."""
+    import torch
+    nd = x.dim()
+    assert len(pads) == 2 * nd
+    out = torch.empty([int(x.shape[i]) + int(pads[i]) + int(pads[i + nd]) for i in range(nd)], dtype=x.dtype,
+                      device=x.device)
+    _check(lib().espdl_hip_pad(_p(x), (ctypes.c_int32 * nd)(*x.shape), nd, (ctypes.c_int32 * (2 * nd))(*pads),
+                               PAD_MODES[mode], int(value), x.element_size(), _p(out), _stream(stream)))
     return out
 
 

@@ -540,6 +540,46 @@ int espdl_hip_slice(const void *in, const int32_t *shape, int32_t dims, const in
                          "slice");
 }
 
+int espdl_hip_pad(const void *in, const int32_t *shape, int32_t dims, const int32_t *pads, int32_t mode,
+                  int32_t constant_value, int32_t elem_size, void *out, void *stream)
+{
+    if (dims < 1 || dims > 8 || shape == nullptr || pads == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "pad handles 1..8 dims");
+    if (elem_size != 1 && elem_size != 2 && elem_size != 4)
+        return fail(ESPDL_HIP_EINVAL, "elem_size must be 1, 2 or 4");
+    if (mode != ESPDL_HIP_PAD_CONSTANT && mode != ESPDL_HIP_PAD_EDGE && mode != ESPDL_HIP_PAD_REFLECT)
+        return fail(ESPDL_HIP_EINVAL, "unknown pad mode %d", mode);
+    int sh[8], pd[16];
+    long long total = 1, in_total = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0 || pads[i] < 0 || pads[i + dims] < 0)
+            return fail(ESPDL_HIP_EINVAL, "dim %d: negative extent or pad", i);
+        if (mode == ESPDL_HIP_PAD_REFLECT && (pads[i] > shape[i] - 1 || pads[i + dims] > shape[i] - 1) &&
+            (pads[i] || pads[i + dims]))
+            return fail(ESPDL_HIP_EINVAL, "dim %d: a reflected pad must be shorter than the axis", i);
+        if (mode == ESPDL_HIP_PAD_EDGE && shape[i] == 0 && (pads[i] || pads[i + dims]))
+            return fail(ESPDL_HIP_EINVAL, "dim %d: no edge to repeat on an empty axis", i);
+        sh[i] = shape[i];
+        pd[i] = pads[i];
+        pd[i + dims] = pads[i + dims];
+        in_total *= shape[i];
+        total *= (long long)shape[i] + pads[i] + pads[i + dims];
+        if (total > (1ll << 40))
+            return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    }
+    if (total == 0)
+        return ESPDL_HIP_OK;
+    if (out == nullptr || (in == nullptr && in_total > 0))
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    if (in_total == 0 && mode != ESPDL_HIP_PAD_CONSTANT)
+        return fail(ESPDL_HIP_EINVAL, "only a constant pad can fill from an empty tensor");
+    if (misaligned(in, (size_t)elem_size) || misaligned(out, (size_t)elem_size))
+        return fail(ESPDL_HIP_EINVAL, "tensors must be aligned to the element size");
+    return device_status(espdl::launch_pad(in, sh, dims, pd, mode, constant_value, elem_size, out, cu_count_cached(),
+                                           reinterpret_cast<hipStream_t>(stream)),
+                         "pad");
+}
+
 int espdl_hip_reduce_mean_s8(const int8_t *in, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
                              int32_t in_exp, int32_t out_exp, int8_t *out, void *stream)
 {

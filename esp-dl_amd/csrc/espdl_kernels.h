@@ -139,6 +139,8 @@ hipError_t launch_max_pool(const void *in, int elem_size, int batch, int h, int 
 hipError_t launch_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                               int stride_w, int pad_top, int pad_left, int out_h, int out_w, int in_exp, int out_exp,
                               int8_t *out, int cu_count, hipStream_t stream);
+hipError_t launch_pad(const void *in, const int *shape, int dims, const int *pads, int mode, int value, int elem_size,
+                      void *out, int cu_count, hipStream_t stream);
 hipError_t launch_slice(const void *in, const int *shape, int dims, const int *start, const int *step, const int *out_shape,
                         int elem_size, void *out, int cu_count, hipStream_t stream);
 

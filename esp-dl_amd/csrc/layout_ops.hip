@@ -734,6 +734,76 @@ hipError_t launch_slice(const void *in, const int *shape, int dims, const int *s
     return hipGetLastError();
 }
 
+// Pad (esp-dl/dl/base/dl_base_pad.cpp:19-260, TensorBase::pad esp-dl/dl/tensor/src/dl_tensor_base.cpp:1225-1299):
+// every axis is padded on its own, so an output coordinate maps to an input coordinate axis by axis.
+// mode 0 constant, 1 edge (clamp), 2 reflect (mirror without repeating the border element).
+struct PadArgs {
+    const char *in;
+    char *out;
+    int dims, mode, value;
+    int out_shape[kMaxDims], in_shape[kMaxDims], before[kMaxDims];
+    long long in_stride[kMaxDims];
+    long long total;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void pad_kernel(const PadArgs a)
+{
+    const T *in = reinterpret_cast<const T *>(a.in);
+    T *out = reinterpret_cast<T *>(a.out);
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < a.total; i += (long long)gridDim.x * kBlock) {
+        long long rem = i, off = 0;
+        bool outside = false;
+        for (int d = a.dims - 1; d >= 0; d--) {
+            const long long q = rem / a.out_shape[d];
+            int x = (int)(rem - q * a.out_shape[d]) - a.before[d];
+            rem = q;
+            const int n = a.in_shape[d];
+            if (x < 0 || x >= n) {
+                if (a.mode == 0)
+                    outside = true;
+                else if (a.mode == 1)
+                    x = x < 0 ? 0 : n - 1;
+                else
+                    x = x < 0 ? -x : 2 * (n - 1) - x;
+            }
+            off += (long long)x * a.in_stride[d];
+        }
+        out[i] = outside ? (T)a.value : in[off];
+    }
+}
+
+hipError_t launch_pad(const void *in, const int *shape, int dims, const int *pads, int mode, int value, int elem_size,
+                      void *out, int cu_count, hipStream_t stream)
+{
+    PadArgs a = {};
+    a.in = static_cast<const char *>(in);
+    a.out = static_cast<char *>(out);
+    a.dims = dims;
+    a.mode = mode;
+    a.value = value;
+    a.total = 1;
+    long long stride = 1;
+    for (int d = dims - 1; d >= 0; d--) {
+        a.in_shape[d] = shape[d];
+        a.before[d] = pads[d];
+        a.out_shape[d] = shape[d] + pads[d] + pads[d + dims];
+        a.in_stride[d] = stride;
+        stride *= shape[d];
+        a.total *= a.out_shape[d];
+    }
+    if (a.total <= 0)
+        return hipSuccess;
+    const dim3 grid(blocks_for(a.total, cu_count));
+    if (elem_size == 1)
+        hipLaunchKernelGGL(pad_kernel<int8_t>, grid, dim3(kBlock), 0, stream, a);
+    else if (elem_size == 2)
+        hipLaunchKernelGGL(pad_kernel<int16_t>, grid, dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL(pad_kernel<int32_t>, grid, dim3(kBlock), 0, stream, a);
+    return hipGetLastError();
+}
+
 hipError_t launch_reduce_mean_s8(const int8_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
                                  int out_exp, int8_t *out, int cu_count, hipStream_t stream)
 {

@@ -76,6 +76,7 @@ public:
         register_module("Slice", Slice::deserialize);
         register_module("ReduceMean", ReduceMean::deserialize);
         register_module("InsertZeros", InsertZeros::deserialize);
+        register_module("Pad", Pad::deserialize);
         register_module("StreamingCache", StreamingCache::deserialize);
         register_module("Softmax", Softmax::deserialize);
         // both are TensorBase::assign between a float32 and a quantized tensor

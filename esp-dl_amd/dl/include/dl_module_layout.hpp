@@ -835,6 +835,93 @@ public:
     void print() { DL_LOGI("InsertZeros", "stride: %s, quant_type: %s.", vector_to_string(m_stride).c_str(), quant_type_to_string(quant_type)); }
 };
 
+/// Pad (esp-dl/dl/module/include/dl_module_pad.hpp:12-100): pads and the optional constant are initializer
+/// operands; the constant is read as the tensor's element type, whatever its own exponent says
+/// (TensorBase::pad, esp-dl/dl/tensor/src/dl_tensor_base.cpp:1231-1234).
+class Pad : public Module {
+private:
+    std::vector<int> m_pads;
+    int m_mode;
+    int m_constant;
+
+public:
+    Pad(const std::vector<int> &pads, int mode, int constant, const char *name = nullptr,
+        quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_pads(pads), m_mode(mode), m_constant(constant)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        if (m_pads.size() != 2 * in.size() || in.empty() || in.size() > 8)
+            return {{}};
+        std::vector<int> out = in;
+        for (size_t i = 0; i < in.size(); i++) {
+            if (m_pads[i] < 0 || m_pads[i + in.size()] < 0)
+                return {{}};
+            out[i] = in[i] + m_pads[i] + m_pads[i + in.size()];
+        }
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        if (!on_device_all({input, output}) || input->dtype != output->dtype ||
+            m_pads.size() != 2 * input->shape.size()) {
+            DL_LOGE("Pad", "%s: needs device tensors of one dtype and two pads per axis", name.c_str());
+            return;
+        }
+        const int rc = espdl_hip_pad(input->data, input->shape.data(), (int32_t)input->shape.size(), m_pads.data(), m_mode,
+                                     m_constant, (int32_t)input->get_dtype_bytes(), output->data, context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Pad", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        std::string mode_name = "constant";
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "mode", mode_name);
+        int mode;
+        if (mode_name == "constant")
+            mode = ESPDL_HIP_PAD_CONSTANT;
+        else if (mode_name == "edge")
+            mode = ESPDL_HIP_PAD_EDGE;
+        else if (mode_name == "reflect")
+            mode = ESPDL_HIP_PAD_REFLECT;
+        else {
+            DL_LOGE("Pad", "%s: mode %s is not supported", node_name.c_str(), mode_name.c_str());
+            return nullptr;
+        }
+        std::vector<int> pads;
+        TensorBase *t = fbs_model->get_operation_parameter(node_name, 1);
+        if (!t || t->dtype != DATA_TYPE_INT64) {
+            DL_LOGE("Pad", "%s: pads must be an int64 initializer", node_name.c_str());
+            delete t;
+            return nullptr;
+        }
+        for (int i = 0; i < t->get_size(); i++)
+            pads.push_back((int)t->get_element_ptr<int64_t>()[i]);
+        delete t;
+        int constant = 0;
+        if (TensorBase *c = fbs_model->get_operation_parameter(node_name, 2)) {
+            if (c->get_size() > 0) {
+                if (c->dtype == DATA_TYPE_INT8)
+                    constant = c->get_element_ptr<int8_t>()[0];
+                else if (c->dtype == DATA_TYPE_INT16)
+                    constant = c->get_element_ptr<int16_t>()[0];
+                else if (c->dtype == DATA_TYPE_INT32)
+                    constant = c->get_element_ptr<int32_t>()[0];
+            }
+            delete c;
+        }
+        return new Pad(pads, mode, constant, node_name.c_str(), quant_type);
+    }
+    void print() { DL_LOGI("Pad", "pads: %s, quant_type: %s.", vector_to_string(m_pads).c_str(), quant_type_to_string(quant_type)); }
+};
+
 /// Softmax on an int8 tensor with a float32 result (esp-dl/dl/module/include/dl_module_softmax.hpp,
 /// forward_lut): the exported graphs follow it with QuantizeLinear.
 class Softmax : public Module {

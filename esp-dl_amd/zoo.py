@@ -800,6 +800,35 @@ def activation_chain(seed=0xE5DB, s16=False):
     return g
 
 
+def padded_convs(seed=0xE5DC):
+    """Explicit Pad nodes in the three modes of the reference in front of unpadded convolutions: reflect (H, W by
+    2), edge (1 and 2, unequal sides) and constant with a non-zero value (also along channels)."""
+    g = GraphSpec("padded_convs")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 12, 12, 16], -5)
+
+    def pad(src, pads, mode, name, value=None):
+        dims = g.shape(src)
+        nd = len(dims)
+        y = name + "_out"
+        g.add_init(name + ".pads", [2 * nd], INT64, pads, [0])
+        ins = [src, name + ".pads"]
+        if value is not None:
+            g.add_init(name + ".value", [1], INT8, [value], [g.exponent(src)])
+            ins.append(name + ".value")
+        g.add_value(y, [dims[i] + pads[i] + pads[i + nd] for i in range(nd)], g.exponent(src))
+        g.add_node(name, "Pad", ins, [y], mode=mode, quant_type="S8")
+        return y
+
+    h = pad(x, [0, 2, 2, 0, 0, 2, 2, 0], "reflect", "mirror")
+    h = b.conv(h, 32, k=5, pad=(0, 0, 0, 0), relu=True, name="c1")
+    h = pad(h, [0, 1, 2, 0, 0, 2, 1, 0], "edge", "border")
+    h = b.conv(h, 32, k=3, pad=(0, 0, 0, 0), depthwise=True, name="dw")
+    h = pad(h, [0, 1, 1, 3, 0, 1, 1, 5], "constant", "frame", value=-3)
+    b.output(b.conv(h, 24, k=3, pad=(0, 0, 0, 0), name="c2"))
+    return g
+
+
 def int16_tail(seed=0xE5D9):
     """int8 Conv -> RequantizeLinear to int16 -> int16 Conv -> int16 table (SiLU) -> int16 Add (residual) ->
     int16 Mul by a constant -> int16 AveragePool -> int16 ReduceMean -> int16 Gemm: the operator mix of the

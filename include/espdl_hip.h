@@ -251,6 +251,16 @@ int espdl_hip_insert_zeros(const void *in, int32_t elem_size, int32_t batch, int
                            int32_t stride_h, int32_t stride_w, int32_t output_padding_h, int32_t output_padding_w,
                            void *out, void *stream);
 
+/* module::Pad = TensorBase::pad (esp-dl/dl/module/include/dl_module_pad.hpp:33-40;
+ * esp-dl/dl/tensor/src/dl_tensor_base.cpp:1225-1299; base::pad1D..pad4D, esp-dl/dl/base/dl_base_pad.cpp:19-260).
+ * `shape` has `dims` (1..8) extents, `pads` 2 * dims entries: the leading pad of every axis, then the trailing pad
+ * of every axis (the ONNX order the reference keeps).  out has extents shape[i] + pads[i] + pads[i + dims].
+ * ESPDL_HIP_PAD_CONSTANT fills with constant_value (converted to the element type), ESPDL_HIP_PAD_EDGE repeats
+ * the border element, ESPDL_HIP_PAD_REFLECT mirrors about it (pads shorter than the axis).  elem_size 1, 2, 4. */
+enum { ESPDL_HIP_PAD_CONSTANT = 0, ESPDL_HIP_PAD_EDGE = 1, ESPDL_HIP_PAD_REFLECT = 2 };
+int espdl_hip_pad(const void *in, const int32_t *shape, int32_t dims, const int32_t *pads, int32_t mode,
+                  int32_t constant_value, int32_t elem_size, void *out, void *stream);
+
 /* module::LUT for int16 (esp-dl/dl/module/include/dl_module_lut.hpp:61-74; base::lut_s16_nearest_neighbor and
  * lut_index, esp-dl/dl/base/dl_base_lut.cpp:49-77): `table` (device) holds table_size = 65536 / step + 1
  * entries, step a power of two, or 65536 entries; out = table[round((in + 32768) / step)].  Ties go up with

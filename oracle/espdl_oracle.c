@@ -755,6 +755,62 @@ void espdl_oracle_div_s16(const int16_t *in0, const int16_t *in1, int64_t size, 
     }
 }
 
+/*
+ * Pad (TensorBase::pad, esp-dl/dl/tensor/src/dl_tensor_base.cpp:1225-1299; base::pad1D and pad_head_and_tail,
+ * esp-dl/dl/base/dl_base_pad.cpp:19-64, 108-183): the innermost axis is padded row by row, then every outer axis
+ * copies whole padded slabs, so each axis maps on its own.  mode 0 constant, 1 edge, 2 reflect.  Written here the
+ * way the reference works, axis by axis from the innermost outwards on a growing buffer.
+ */
+void espdl_oracle_pad(const void *in, const int32_t *shape, int dims, const int32_t *pads, int mode, int32_t value,
+                      int elem_size, void *out)
+{
+    int64_t cur_shape[8];
+    int64_t total = 1;
+    for (int d = 0; d < dims; d++) {
+        cur_shape[d] = shape[d];
+        total *= shape[d];
+    }
+    unsigned char *cur = (unsigned char *)malloc((size_t)(total > 0 ? total : 1) * elem_size);
+    memcpy(cur, in, (size_t)total * elem_size);
+    for (int axis = dims - 1; axis >= 0; axis--) {
+        const int64_t before = pads[axis], after = pads[axis + dims], n = cur_shape[axis], m = n + before + after;
+        int64_t outer = 1, inner = elem_size;
+        for (int d = 0; d < axis; d++)
+            outer *= cur_shape[d];
+        for (int d = axis + 1; d < dims; d++)
+            inner *= cur_shape[d];
+        unsigned char *next = (unsigned char *)malloc((size_t)(outer * m * inner > 0 ? outer * m * inner : 1));
+        for (int64_t o = 0; o < outer; o++) {
+            const unsigned char *src = cur + o * n * inner;
+            unsigned char *dst = next + o * m * inner;
+            memcpy(dst + before * inner, src, (size_t)(n * inner));
+            for (int64_t i = 0; i < before + after; i++) {
+                const int64_t pos = i < before ? i : n + i;      /* position in the padded axis */
+                unsigned char *line = dst + pos * inner;
+                if (mode == 0) {
+                    for (int64_t k = 0; k < inner; k += elem_size)
+                        memcpy(line + k, &value, (size_t)elem_size); /* little endian: the low bytes */
+                } else {
+                    int64_t from;
+                    if (mode == 1)
+                        from = i < before ? 0 : n - 1;
+                    else
+                        from = i < before ? before - i : n - 2 - (i - before);
+                    memcpy(line, src + from * inner, (size_t)inner);
+                }
+            }
+        }
+        free(cur);
+        cur = next;
+        cur_shape[axis] = m;
+    }
+    total = elem_size;
+    for (int d = 0; d < dims; d++)
+        total *= cur_shape[d];
+    memcpy(out, cur, (size_t)total);
+    free(cur);
+}
+
 /* Sub, int8 (c_impl_sub_n_n<int8_t>, esp-dl/dl/base/dl_base_sub.cpp:33-43): saturating integer subtraction. */
 void espdl_oracle_sub_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size, int8_t *out)
 {

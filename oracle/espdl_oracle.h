@@ -77,6 +77,8 @@
  *                                HardSwish and sigmoid against numpy operations of those widths; expf / logf
  *                                are the host libm's, which may differ from the target's in the last bit
  *                                                                       PARITY UNPINNED (libm last-bit, near-ties)
+ *   espdl_oracle_pad             equality with numpy.pad (constant / edge / reflect) on random shapes, ranks 1-5,
+ *                                all three element sizes                                             PINNED
  *   espdl_oracle_sub_s8          numpy saturating subtraction                                        PINNED
  *   espdl_oracle_div_s8          as _div_s16 for the three loop forms; the table forms against a table built in
  *                                numpy float32 from the reference's two expressions, entry by entry   PINNED
@@ -179,6 +181,8 @@ void espdl_oracle_unary_s8(int kind, const int8_t *in, int64_t size, int in_exp,
                            int round_mode, int8_t *out);
 void espdl_oracle_unary_s16(int kind, const int16_t *in, int64_t size, int in_exp, int out_exp, float alpha, float beta,
                             int round_mode, int16_t *out);
+void espdl_oracle_pad(const void *in, const int32_t *shape, int dims, const int32_t *pads, int mode, int32_t value,
+                      int elem_size, void *out);
 void espdl_oracle_sub_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size, int8_t *out);
 void espdl_oracle_div_s8(const int8_t *in0, const int8_t *in1, int64_t size, int shift, int form, int table_operand,
                          int8_t *out);

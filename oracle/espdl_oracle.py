@@ -73,6 +73,8 @@ def lib():
         L.espdl_oracle_unary_s8.argtypes = [i32, vp, i64, i32, i32, ctypes.c_float, ctypes.c_float, i32, vp]
         L.espdl_oracle_unary_s16.restype = None
         L.espdl_oracle_unary_s16.argtypes = [i32, vp, i64, i32, i32, ctypes.c_float, ctypes.c_float, i32, vp]
+        L.espdl_oracle_pad.restype = None
+        L.espdl_oracle_pad.argtypes = [vp, vp, i32, vp, i32, i32, i32, vp]
         L.espdl_oracle_sub_s8.restype = None
         L.espdl_oracle_sub_s8.argtypes = [vp, i64, vp, i64, i64, vp]
         L.espdl_oracle_div_s8.restype = None
@@ -367,6 +369,21 @@ def unary(op_type, x, in_exp, out_exp, alpha=None, beta=None, round_mode=ROUND_H
     fn = lib().espdl_oracle_unary_s8 if x.dtype == np.int8 else lib().espdl_oracle_unary_s16
     fn(UNARY_KINDS[op_type], _ptr(x), x.size, int(in_exp), int(out_exp), float(alpha), float(beta), int(round_mode),
        _ptr(out))
+    return out
+
+
+PAD_MODES = {"constant": 0, "edge": 1, "reflect": 2}
+
+
+def pad(x, pads, mode="constant", value=0):
+    """pads: the leading pad of every axis, then the trailing pad of every axis."""
+    x = np.ascontiguousarray(x)
+    nd = x.ndim
+    assert len(pads) == 2 * nd and x.dtype.itemsize in (1, 2, 4)
+    shape = np.asarray(x.shape, dtype=np.int32)
+    p = np.asarray(pads, dtype=np.int32)
+    out = np.empty([x.shape[i] + int(p[i]) + int(p[i + nd]) for i in range(nd)], dtype=x.dtype)
+    lib().espdl_oracle_pad(_ptr(x), _ptr(shape), nd, _ptr(p), PAD_MODES[mode], int(value), x.dtype.itemsize, _ptr(out))
     return out
 
 

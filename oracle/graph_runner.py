@@ -108,6 +108,10 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None
             y = oracle.unary(op, x, exponent_of(ins[0]), spec.exponent(y_name), a.get("alpha"), a.get("beta"), round_mode)
         elif op == "Identity":  # output->assign(input): a requantize when the exponents differ
             y = requantize(x, spec.exponent(ins[0]), spec.exponent(y_name), spec.dtype(y_name))
+        elif op == "Pad":
+            pads = [int(v) for v in spec.initializers[ins[1]][2].ravel()]
+            value = int(spec.initializers[ins[2]][2].ravel()[0]) if len(ins) > 2 and ins[2] else 0
+            y = oracle.pad(x, pads, a.get("mode", "constant"), value)
         elif op == "Sub":
             b = operand(ins[1])
             if x.shape != b.shape:

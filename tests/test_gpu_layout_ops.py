@@ -181,3 +181,37 @@ def test_insert_zeros_one_spatial_dim(oracle):
     x = _rand(np.random.default_rng(30), (3, 11, 5))
     got = to_host(espdl().insert_zeros(to_dev(x), (3,), (2,)))
     np.testing.assert_array_equal(got, oracle.insert_zeros(x[:, :, None], (3, 1), (2, 0))[:, :, 0])
+
+
+@pytest.mark.parametrize("mode", ["constant", "edge", "reflect"])
+@pytest.mark.parametrize("dtype", [np.int8, np.int16, np.int32])
+def test_pad(oracle, mode, dtype):
+    announce(f"pad {mode} {np.dtype(dtype).name}")
+    rng = np.random.default_rng(72)
+    shapes = [(37,), (5, 9), (2, 7, 11), (3, 14, 14, 32), (2, 3, 4, 5, 6), (1, 56, 56, 24)]
+    for shape in shapes:
+        nd = len(shape)
+        info = np.iinfo(dtype)
+        x = rng.integers(info.min, info.max, size=shape, dtype=dtype, endpoint=True)
+        before = [int(rng.integers(0, min(s, 4))) for s in shape]
+        after = [int(rng.integers(0, min(s, 4))) for s in shape]
+        value = int(rng.integers(-100, 100))
+        got = to_host(espdl().pad(to_dev(x), before + after, mode, value))
+        np.testing.assert_array_equal(got, oracle.pad(x, before + after, mode, value))
+        kw = {"constant_values": value} if mode == "constant" else {}
+        np.testing.assert_array_equal(got, np.pad(x, list(zip(before, after)), mode=mode, **kw))
+
+
+def test_pad_rejects_what_the_reference_cannot_do(oracle):
+    announce("pad error paths")
+    import torch
+    x = torch.zeros((2, 3), dtype=torch.int8, device="cuda")
+    with pytest.raises(espdl().EspdlHipError):
+        espdl().pad(x, [0, 3, 0, 0], "reflect")          # reflected pad as long as the axis
+    with pytest.raises(espdl().EspdlHipError):
+        espdl().pad(x, [0, -1, 0, 0], "constant")
+    empty = torch.zeros((2, 0), dtype=torch.int8, device="cuda")
+    with pytest.raises(espdl().EspdlHipError):
+        espdl().pad(empty, [0, 1, 0, 0], "edge")
+    got = espdl().pad(empty, [0, 1, 0, 2], "constant", 5)
+    assert got.shape == (2, 3) and bool((got == 5).all())

@@ -287,6 +287,18 @@ def test_activation_chain(oracle, s16, round_mode):
     mdl.close()
 
 
+def test_padded_convs(oracle):
+    """Pad nodes (reflect, edge, constant with a value) in front of unpadded convolutions."""
+    announce("model padded_convs")
+    _, zoo, _, _ = _mods()
+    spec = zoo.padded_convs()
+    mdl, want, _ = _run_config(spec, 3, 43)
+    got = mdl.get_tensor(spec.outputs[0])
+    np.testing.assert_array_equal(got, want[spec.outputs[0]])
+    assert len(np.unique(want[spec.outputs[0]])) > 20
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()

@@ -201,3 +201,27 @@ def test_insert_zeros_is_strided_assignment(oracle, dtype, stride, pad):
     want[:, :(5 - 1) * stride[0] + 1:stride[0], :(4 - 1) * stride[1] + 1:stride[1]] = x
     np.testing.assert_array_equal(got, want)
     np.testing.assert_array_equal(got[:, ::stride[0], ::stride[1]][:, :5, :4], x)
+
+
+@pytest.mark.parametrize("mode", ["constant", "edge", "reflect"])
+@pytest.mark.parametrize("dtype", [np.int8, np.int16, np.int32])
+def test_pad_is_numpy_pad(oracle, mode, dtype):
+    """numpy.pad is the textbook routine for all three modes; random ranks 1..5, unequal sides, zero pads."""
+    rng = np.random.default_rng(71)
+    for _ in range(30):
+        nd = int(rng.integers(1, 6))
+        shape = [int(rng.integers(2, 7)) for _ in range(nd)]
+        info = np.iinfo(dtype)
+        x = rng.integers(info.min, info.max, size=shape, dtype=dtype, endpoint=True)
+        before = [int(rng.integers(0, s if mode == "reflect" else 4)) for s in shape]
+        after = [int(rng.integers(0, s if mode == "reflect" else 4)) for s in shape]
+        value = int(rng.integers(-100, 100))
+        kw = {"constant_values": value} if mode == "constant" else {}
+        want = np.pad(x, list(zip(before, after)), mode=mode, **kw)
+        np.testing.assert_array_equal(oracle.pad(x, before + after, mode, value), want)
+
+
+def test_pad_of_an_empty_axis_is_all_constant(oracle):
+    x = np.zeros((2, 0, 3), np.int8)
+    got = oracle.pad(x, [0, 2, 0, 0, 1, 0], "constant", 7)
+    assert got.shape == (2, 3, 3) and np.all(got == 7)
