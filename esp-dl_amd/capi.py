@@ -92,6 +92,8 @@ def lib():
         L.espdl_hip_insert_zeros.restype = ctypes.c_int
         L.espdl_hip_pad.argtypes = [vp, vp, i32, vp, i32, i32, i32, vp, vp]
         L.espdl_hip_pad.restype = ctypes.c_int
+        L.espdl_hip_reduce_int.argtypes = [vp, i32, vp, i32, vp, i32, i32, i32, vp, vp]
+        L.espdl_hip_reduce_int.restype = ctypes.c_int
         L.espdl_hip_lut_s16.argtypes = [vp, i64, vp, i32, i32, vp, vp]
         L.espdl_hip_lut_s16.restype = ctypes.c_int
         L.espdl_hip_softmax_s8.argtypes = [vp, i64, i64, i64, i32, vp, vp]
@@ -518,6 +520,23 @@ def sub_s16(a, b, stream=None):
     _check(lib().espdl_hip_sub_s16(ctypes.byref(dims), ctypes.byref(s0), ctypes.byref(s1), _p(a), _p(b), _p(out),
                                    _stream(stream)))
     return out
+
+
+REDUCE_OPS = {"ReduceMax": 0, "ReduceMin": 1, "ReduceSum": 2}
+
+
+def reduce_int(op_type, x, axes, keepdims=True, shift=0, round_mode=ROUND_HALF_UP, stream=None):
+    """ReduceMax / ReduceMin / ReduceSum of an int8 or int16 tensor (espdl_hip_reduce_int); shift = out_exp - in_exp."""
+    import torch
+    nd = x.dim()
+    axes = [a + nd if a < 0 else a for a in (axes if len(axes) else range(nd))]
+    flags = [1 if i in axes else 0 for i in range(nd)]
+    kept = [int(x.shape[i]) for i in range(nd) if not flags[i]]
+    out = torch.empty(kept if kept else [1], dtype=x.dtype, device=x.device)
+    _check(lib().espdl_hip_reduce_int(_p(x), S8 if x.dtype == torch.int8 else S16, (ctypes.c_int32 * nd)(*x.shape), nd,
+                                      (ctypes.c_int32 * nd)(*flags), REDUCE_OPS[op_type], int(shift), round_mode, _p(out),
+                                      _stream(stream)))
+    return out.reshape([1 if flags[i] else int(x.shape[i]) for i in range(nd)]) if keepdims else out
 
 
 PAD_MODES = {"constant": 0, "edge": 1, "reflect": 2}

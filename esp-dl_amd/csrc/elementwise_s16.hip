@@ -150,6 +150,50 @@ __global__ __launch_bounds__(kThreads) void reduce_mean_s16_kernel(const Reduce1
     }
 }
 
+// ReduceMax / ReduceMin / ReduceSum (esp-dl/dl/module/include/dl_module_reduce_max.hpp:14-52,
+// dl_module_reduce_min.hpp:15-53, dl_module_reduce_sum.hpp:13-56): max and min return the stored integer, the sum
+// (int32 for int8, int64 for int16) goes through shift_and_round(sum, out_exp - in_exp) and truncate.
+template <typename T>
+struct ReduceIntArgs {
+    const T *in;
+    T *out;
+    int n_kept, n_red;
+    int kept_shape[8], red_shape[8];
+    long long kept_stride[8], red_stride[8];
+    long long n_out, count;
+    int shift, half_even;
+};
+
+// OP: 0 max, 1 min, 2 sum
+template <typename T, int OP>
+__global__ __launch_bounds__(kThreads) void reduce_int_kernel(const ReduceIntArgs<T> a)
+{
+    constexpr int lo = sizeof(T) == 1 ? -128 : -32768, hi = sizeof(T) == 1 ? 127 : 32767;
+    for (long long o = (long long)blockIdx.x * kThreads + threadIdx.x; o < a.n_out; o += (long long)gridDim.x * kThreads) {
+        long long rem = o, base = 0;
+        for (int d = a.n_kept - 1; d >= 0; d--) {
+            const long long q = rem / a.kept_shape[d];
+            base += (rem - q * a.kept_shape[d]) * a.kept_stride[d];
+            rem = q;
+        }
+        long long acc = OP == 0 ? lo : (OP == 1 ? hi : 0);
+        for (long long r = 0; r < a.count; r++) {
+            long long rr = r, off = base;
+            for (int d = a.n_red - 1; d >= 0; d--) {
+                const long long q = rr / a.red_shape[d];
+                off += (rr - q * a.red_shape[d]) * a.red_stride[d];
+                rr = q;
+            }
+            const long long v = a.in[off];
+            acc = OP == 0 ? max(acc, v) : (OP == 1 ? min(acc, v) : acc + v);
+        }
+        if (OP == 2)
+            acc = sizeof(T) == 1 ? requant_s8((int)acc, a.shift, false, a.half_even)
+                                 : requant_s16(acc, a.shift, false, a.half_even);
+        a.out[o] = (T)acc;
+    }
+}
+
 unsigned blocks_for(long long total, int cu_count)
 {
     return (unsigned)max(1ll, min((total + kThreads - 1) / kThreads, (long long)max(1, cu_count) * 16));
@@ -280,6 +324,58 @@ hipError_t launch_reduce_mean_s16(const int16_t *in, const int *shape, int dims,
     a.output_scale = dl_rescale(out_exp);
     reduce_mean_s16_kernel<<<dim3(blocks_for(a.n_out, cu_count)), dim3(kThreads), 0, stream>>>(a);
     return hipGetLastError();
+}
+
+namespace {
+
+template <typename T>
+hipError_t launch_reduce_int_t(const T *in, const int *shape, int dims, const int *reduce_flag, int op, int shift,
+                               bool half_even, T *out, int cu_count, hipStream_t stream)
+{
+    ReduceIntArgs<T> a = {};
+    a.in = in;
+    a.out = out;
+    long long stride[8];
+    stride[dims - 1] = 1;
+    for (int i = dims - 2; i >= 0; i--)
+        stride[i] = stride[i + 1] * shape[i + 1];
+    a.n_out = 1;
+    a.count = 1;
+    for (int i = 0; i < dims; i++) {
+        if (reduce_flag[i]) {
+            a.red_shape[a.n_red] = shape[i];
+            a.red_stride[a.n_red++] = stride[i];
+            a.count *= shape[i];
+        } else {
+            a.kept_shape[a.n_kept] = shape[i];
+            a.kept_stride[a.n_kept++] = stride[i];
+            a.n_out *= shape[i];
+        }
+    }
+    if (a.n_out <= 0)
+        return hipSuccess;
+    a.shift = shift;
+    a.half_even = half_even;
+    const dim3 grid(blocks_for(a.n_out, cu_count)), block(kThreads);
+    if (op == 0)
+        reduce_int_kernel<T, 0><<<grid, block, 0, stream>>>(a);
+    else if (op == 1)
+        reduce_int_kernel<T, 1><<<grid, block, 0, stream>>>(a);
+    else
+        reduce_int_kernel<T, 2><<<grid, block, 0, stream>>>(a);
+    return hipGetLastError();
+}
+
+} // namespace
+
+hipError_t launch_reduce_int(const void *in, int bits, const int *shape, int dims, const int *reduce_flag, int op,
+                             int shift, bool half_even, void *out, int cu_count, hipStream_t stream)
+{
+    if (bits == 8)
+        return launch_reduce_int_t<int8_t>(static_cast<const int8_t *>(in), shape, dims, reduce_flag, op, shift, half_even,
+                                           static_cast<int8_t *>(out), cu_count, stream);
+    return launch_reduce_int_t<int16_t>(static_cast<const int16_t *>(in), shape, dims, reduce_flag, op, shift, half_even,
+                                        static_cast<int16_t *>(out), cu_count, stream);
 }
 
 } // namespace espdl

@@ -540,6 +540,47 @@ int espdl_hip_slice(const void *in, const int32_t *shape, int32_t dims, const in
                          "slice");
 }
 
+int espdl_hip_reduce_int(const void *in, int32_t dtype, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
+                         int32_t op, int32_t shift, int32_t round_mode, void *out, void *stream)
+{
+    if (dtype != ESPDL_HIP_S8 && dtype != ESPDL_HIP_S16)
+        return fail(ESPDL_HIP_EINVAL, "dtype must be ESPDL_HIP_S8 or ESPDL_HIP_S16");
+    if (dims < 1 || dims > 8 || shape == nullptr || reduce_flag == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "reduce handles 1..8 dims");
+    if (op != ESPDL_HIP_REDUCE_MAX && op != ESPDL_HIP_REDUCE_MIN && op != ESPDL_HIP_REDUCE_SUM)
+        return fail(ESPDL_HIP_EINVAL, "unknown reduce op %d", op);
+    if (round_mode != ESPDL_HIP_ROUND_HALF_UP && round_mode != ESPDL_HIP_ROUND_HALF_EVEN)
+        return fail(ESPDL_HIP_EINVAL, "bad round_mode %d", round_mode);
+    if (shift < -30 || shift > 62)
+        return fail(ESPDL_HIP_EINVAL, "shift %d outside [-30, 62]", shift);
+    int sh[8], fl[8];
+    long long n_out = 1, count = 1;
+    for (int i = 0; i < dims; i++) {
+        if (shape[i] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative extent in dim %d", i);
+        sh[i] = shape[i];
+        fl[i] = reduce_flag[i] ? 1 : 0;
+        if (fl[i])
+            count *= shape[i];
+        else
+            n_out *= shape[i];
+        if (n_out > (1ll << 40) || count > (1ll << 40))
+            return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
+    }
+    if (n_out == 0)
+        return ESPDL_HIP_OK;
+    if (dtype == ESPDL_HIP_S8 && op == ESPDL_HIP_REDUCE_SUM && count > (1ll << 24))
+        return fail(ESPDL_HIP_ENOTSUP, "an int8 sum over more than 2^24 elements leaves the reference's int32");
+    if (out == nullptr || (in == nullptr && count > 0))
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    if (dtype == ESPDL_HIP_S16 && (misaligned(in, 2) || misaligned(out, 2)))
+        return fail(ESPDL_HIP_EINVAL, "int16 tensors must be 2-byte aligned");
+    return device_status(espdl::launch_reduce_int(in, dtype == ESPDL_HIP_S8 ? 8 : 16, sh, dims, fl, op, shift,
+                                                  round_mode == ESPDL_HIP_ROUND_HALF_EVEN, out, cu_count_cached(),
+                                                  reinterpret_cast<hipStream_t>(stream)),
+                         "reduce_int");
+}
+
 int espdl_hip_pad(const void *in, const int32_t *shape, int32_t dims, const int32_t *pads, int32_t mode,
                   int32_t constant_value, int32_t elem_size, void *out, void *stream)
 {

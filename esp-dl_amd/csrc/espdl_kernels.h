@@ -155,6 +155,8 @@ hipError_t launch_binary_s16(int op, const int32_t dims[4], const int64_t s0[4],
                              const int16_t *in1, int shift, bool half_even, int16_t *out, int cu_count, hipStream_t stream);
 hipError_t launch_subdiv_s8(bool div, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,
                             const int8_t *in1, int shift, int8_t *out, int cu_count, hipStream_t stream);
+hipError_t launch_reduce_int(const void *in, int bits, const int *shape, int dims, const int *reduce_flag, int op,
+                             int shift, bool half_even, void *out, int cu_count, hipStream_t stream);
 hipError_t launch_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                                int stride_w, int pad_top, int pad_left, int out_h, int out_w, int in_exp, int out_exp,
                                int16_t *out, int cu_count, hipStream_t stream);

@@ -75,6 +75,9 @@ public:
         register_module("AveragePool", AveragePool::deserialize);
         register_module("Slice", Slice::deserialize);
         register_module("ReduceMean", ReduceMean::deserialize);
+        register_module("ReduceMax", ReduceMean::deserialize_max);
+        register_module("ReduceMin", ReduceMean::deserialize_min);
+        register_module("ReduceSum", ReduceMean::deserialize_sum);
         register_module("InsertZeros", InsertZeros::deserialize);
         register_module("Pad", Pad::deserialize);
         register_module("StreamingCache", StreamingCache::deserialize);

@@ -569,6 +569,8 @@ private:
     int m_keepdims;
     std::vector<int64_t> m_axes;
     int m_noop_with_empty_axes;
+    int m_int_op; ///< -1: mean; else ESPDL_HIP_REDUCE_MAX / _MIN / _SUM (the modules of dl_module_reduce_max.hpp,
+                  ///< dl_module_reduce_min.hpp and dl_module_reduce_sum.hpp share the axes handling)
 
     std::vector<int32_t> flags_for(size_t rank) const
     {
@@ -588,9 +590,9 @@ private:
 
 public:
     ReduceMean(const char *name = nullptr, int keepdims = 1, const std::vector<int64_t> &axes = {},
-               int noop_with_empty_axes = 0, quant_type_t quant_type = QUANT_TYPE_NONE) :
+               int noop_with_empty_axes = 0, quant_type_t quant_type = QUANT_TYPE_NONE, int int_op = -1) :
         Module(name, MODULE_NON_INPLACE, quant_type), m_keepdims(keepdims), m_axes(axes),
-        m_noop_with_empty_axes(noop_with_empty_axes)
+        m_noop_with_empty_axes(noop_with_empty_axes), m_int_op(int_op)
     {
     }
     std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
@@ -619,6 +621,16 @@ public:
             return;
         }
         const std::vector<int32_t> f = flags_for(input->shape.size());
+        if (m_int_op >= 0) {
+            const int rc = espdl_hip_reduce_int(
+                input->data, quant_type == QUANT_TYPE_SYMM_16BIT ? ESPDL_HIP_S16 : ESPDL_HIP_S8, input->shape.data(),
+                (int32_t)input->shape.size(), f.data(), m_int_op, output->exponent.get() - input->exponent.get(),
+                context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP,
+                output->data, context->stream);
+            if (rc != ESPDL_HIP_OK)
+                DL_LOGE("Reduce", "%s: %s", name.c_str(), espdl_hip_last_error());
+            return;
+        }
         const int rc = quant_type == QUANT_TYPE_SYMM_16BIT
             ? espdl_hip_reduce_mean_s16(static_cast<const int16_t *>(input->data), input->shape.data(),
                                         (int32_t)input->shape.size(), f.data(), input->exponent.get(),
@@ -629,7 +641,20 @@ public:
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("ReduceMean", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
-    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name) { return make(fbs_model, node_name, -1); }
+    static Module *deserialize_max(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        return make(fbs_model, node_name, ESPDL_HIP_REDUCE_MAX);
+    }
+    static Module *deserialize_min(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        return make(fbs_model, node_name, ESPDL_HIP_REDUCE_MIN);
+    }
+    static Module *deserialize_sum(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        return make(fbs_model, node_name, ESPDL_HIP_REDUCE_SUM);
+    }
+    static Module *make(fbs::FbsModel *fbs_model, const std::string &node_name, int int_op)
     {
         quant_type_t quant_type = QUANT_TYPE_NONE;
         int keepdims = 1, noop = 0;
@@ -652,7 +677,7 @@ public:
             if (fbs_model->get_operation_attribute(node_name, "axes", attr_axes) == ESP_OK)
                 axes.assign(attr_axes.begin(), attr_axes.end());
         }
-        return new ReduceMean(node_name.c_str(), keepdims, axes, noop, quant_type);
+        return new ReduceMean(node_name.c_str(), keepdims, axes, noop, quant_type, int_op);
     }
     void print() { DL_LOGI("ReduceMean", "keepdims: %d, quant_type: %s.", m_keepdims, quant_type_to_string(quant_type)); }
 };

@@ -829,6 +829,34 @@ def padded_convs(seed=0xE5DC):
     return g
 
 
+def reduce_heads(seed=0xE5DD, s16=False):
+    """ReduceMax over the image, ReduceMin over channels and ReduceSum over the image (coarser output exponent)
+    on one feature map, int8 or int16."""
+    g = GraphSpec("reduce_heads_s16" if s16 else "reduce_heads")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    qt, dt = ("S16", INT16) if s16 else ("S8", INT8)
+    x = b.input("input", [1, 10, 12, 16], -5)
+    f = b.conv(x, 32, k=3, name="features")
+    if s16:
+        f16 = "features_s16"
+        g.add_value(f16, g.shape(f), g.exponent(f) - 8, INT16)
+        g.add_node("to_s16", "RequantizeLinear", [f], [f16], quant_type="S16")
+        f = b.conv(f16, 32, k=1, s16=True, out_exp=g.exponent(f16), name="mixed")
+    n, h, w, c = g.shape(f)
+
+    def reduce(op, axes, out_shape, out_exp, name, keepdims=1):
+        y = name + "_out"
+        g.add_init(name + ".axes", [len(axes)], INT64, axes, [0])
+        g.add_value(y, out_shape, out_exp, dt)
+        g.add_node(name, op, [f, name + ".axes"], [y], keepdims=keepdims, noop_with_empty_axes=0, quant_type=qt)
+        g.outputs.append(y)
+
+    reduce("ReduceMax", [1, 2], [1, 1, 1, c], g.exponent(f), "image_max")
+    reduce("ReduceMin", [-1], [1, h, w], g.exponent(f), "channel_min", keepdims=0)
+    reduce("ReduceSum", [1, 2], [1, 1, 1, c], g.exponent(f) + 5, "image_sum")
+    return g
+
+
 def int16_tail(seed=0xE5D9):
     """int8 Conv -> RequantizeLinear to int16 -> int16 Conv -> int16 table (SiLU) -> int16 Add (residual) ->
     int16 Mul by a constant -> int16 AveragePool -> int16 ReduceMean -> int16 Gemm: the operator mix of the

@@ -251,6 +251,15 @@ int espdl_hip_insert_zeros(const void *in, int32_t elem_size, int32_t batch, int
                            int32_t stride_h, int32_t stride_w, int32_t output_padding_h, int32_t output_padding_w,
                            void *out, void *stream);
 
+/* module::ReduceMax, ReduceMin, ReduceSum for int8 / int16 (esp-dl/dl/module/include/dl_module_reduce_max.hpp:14-52,
+ * dl_module_reduce_min.hpp:15-53, dl_module_reduce_sum.hpp:13-56; loop nest dl_module_reduce_base.hpp).  dtype is
+ * ESPDL_HIP_S8 or ESPDL_HIP_S16; shape / reduce_flag as espdl_hip_reduce_mean_s8.  Max and min return stored
+ * integers and ignore shift; the sum (int32 for int8, int64 for int16) is shift_and_round(sum, shift) with
+ * shift = out_exp - in_exp, then saturated.  An empty reduction gives the identity (type minimum, maximum, 0). */
+enum { ESPDL_HIP_REDUCE_MAX = 0, ESPDL_HIP_REDUCE_MIN = 1, ESPDL_HIP_REDUCE_SUM = 2 };
+int espdl_hip_reduce_int(const void *in, int32_t dtype, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
+                         int32_t op, int32_t shift, int32_t round_mode, void *out, void *stream);
+
 /* module::Pad = TensorBase::pad (esp-dl/dl/module/include/dl_module_pad.hpp:33-40;
  * esp-dl/dl/tensor/src/dl_tensor_base.cpp:1225-1299; base::pad1D..pad4D, esp-dl/dl/base/dl_base_pad.cpp:19-260).
  * `shape` has `dims` (1..8) extents, `pads` 2 * dims entries: the leading pad of every axis, then the trailing pad

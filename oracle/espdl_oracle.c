@@ -756,6 +756,63 @@ void espdl_oracle_div_s16(const int16_t *in0, const int16_t *in1, int64_t size, 
 }
 
 /*
+ * ReduceMax, ReduceMin, ReduceSum for int8 / int16 (esp-dl/dl/module/include/dl_module_reduce_max.hpp:14-52,
+ * dl_module_reduce_min.hpp:15-53, dl_module_reduce_sum.hpp:13-56): max and min of the stored integers from the
+ * type's minimum / maximum; the sum is accumulated in int32 (int8) or int64 (int16), then
+ * shift_and_round(sum, out_exp - in_exp) and truncate.  Written as one walk over the input that folds every
+ * element into its output slot.  op: 0 max, 1 min, 2 sum.
+ */
+int espdl_oracle_reduce_int(const void *in, int bits, const int32_t *shape, int dims, const int32_t *reduce_flag, int op,
+                            int shift, int round_mode, void *out)
+{
+    if (dims < 1 || dims > 8 || (bits != 8 && bits != 16))
+        return -1;
+    const int lo = bits == 8 ? INT8_MIN : INT16_MIN, hi = bits == 8 ? INT8_MAX : INT16_MAX;
+    int64_t out_stride[8], n_out = 1, total = 1;
+    for (int d = dims - 1; d >= 0; d--) {
+        out_stride[d] = reduce_flag[d] ? 0 : n_out;
+        if (!reduce_flag[d])
+            n_out *= shape[d];
+        total *= shape[d];
+    }
+    int64_t *acc = (int64_t *)malloc(sizeof(int64_t) * (size_t)(n_out > 0 ? n_out : 1));
+    for (int64_t o = 0; o < n_out; o++)
+        acc[o] = op == 0 ? lo : (op == 1 ? hi : 0);
+    int32_t idx[8] = {0};
+    for (int64_t i = 0; i < total; i++) {
+        int64_t o = 0;
+        for (int d = 0; d < dims; d++)
+            o += idx[d] * out_stride[d];
+        const int64_t v = bits == 8 ? ((const int8_t *)in)[i] : ((const int16_t *)in)[i];
+        if (op == 0)
+            acc[o] = v > acc[o] ? v : acc[o];
+        else if (op == 1)
+            acc[o] = v < acc[o] ? v : acc[o];
+        else
+            acc[o] += v;
+        for (int d = dims - 1; d >= 0; d--) {
+            if (++idx[d] < shape[d])
+                break;
+            idx[d] = 0;
+        }
+    }
+    for (int64_t o = 0; o < n_out; o++) {
+        int64_t r = acc[o];
+        if (op == 2) {
+            r = bits == 8 ? (int64_t)espdl_oracle_shift_round_s32((int32_t)r, shift, round_mode)
+                          : espdl_oracle_shift_round_s64(r, shift, round_mode);
+            r = clamp_i64(r, lo, hi);
+        }
+        if (bits == 8)
+            ((int8_t *)out)[o] = (int8_t)r;
+        else
+            ((int16_t *)out)[o] = (int16_t)r;
+    }
+    free(acc);
+    return 0;
+}
+
+/*
  * Pad (TensorBase::pad, esp-dl/dl/tensor/src/dl_tensor_base.cpp:1225-1299; base::pad1D and pad_head_and_tail,
  * esp-dl/dl/base/dl_base_pad.cpp:19-64, 108-183): the innermost axis is padded row by row, then every outer axis
  * copies whole padded slabs, so each axis maps on its own.  mode 0 constant, 1 edge, 2 reflect.  Written here the

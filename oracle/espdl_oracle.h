@@ -77,6 +77,8 @@
  *                                HardSwish and sigmoid against numpy operations of those widths; expf / logf
  *                                are the host libm's, which may differ from the target's in the last bit
  *                                                                       PARITY UNPINNED (libm last-bit, near-ties)
+ *   espdl_oracle_reduce_int      numpy max / min / sum over the same axes; the sum followed by the pinned
+ *                                shift-round and saturation                                          PINNED
  *   espdl_oracle_pad             equality with numpy.pad (constant / edge / reflect) on random shapes, ranks 1-5,
  *                                all three element sizes                                             PINNED
  *   espdl_oracle_sub_s8          numpy saturating subtraction                                        PINNED
@@ -181,6 +183,8 @@ void espdl_oracle_unary_s8(int kind, const int8_t *in, int64_t size, int in_exp,
                            int round_mode, int8_t *out);
 void espdl_oracle_unary_s16(int kind, const int16_t *in, int64_t size, int in_exp, int out_exp, float alpha, float beta,
                             int round_mode, int16_t *out);
+int espdl_oracle_reduce_int(const void *in, int bits, const int32_t *shape, int dims, const int32_t *reduce_flag, int op,
+                            int shift, int round_mode, void *out);
 void espdl_oracle_pad(const void *in, const int32_t *shape, int dims, const int32_t *pads, int mode, int32_t value,
                       int elem_size, void *out);
 void espdl_oracle_sub_s8(const int8_t *in0, int64_t len0, const int8_t *in1, int64_t len1, int64_t size, int8_t *out);

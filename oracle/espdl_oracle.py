@@ -73,6 +73,8 @@ def lib():
         L.espdl_oracle_unary_s8.argtypes = [i32, vp, i64, i32, i32, ctypes.c_float, ctypes.c_float, i32, vp]
         L.espdl_oracle_unary_s16.restype = None
         L.espdl_oracle_unary_s16.argtypes = [i32, vp, i64, i32, i32, ctypes.c_float, ctypes.c_float, i32, vp]
+        L.espdl_oracle_reduce_int.restype = ctypes.c_int
+        L.espdl_oracle_reduce_int.argtypes = [vp, i32, vp, i32, vp, i32, i32, i32, vp]
         L.espdl_oracle_pad.restype = None
         L.espdl_oracle_pad.argtypes = [vp, vp, i32, vp, i32, i32, i32, vp]
         L.espdl_oracle_sub_s8.restype = None
@@ -369,6 +371,27 @@ def unary(op_type, x, in_exp, out_exp, alpha=None, beta=None, round_mode=ROUND_H
     fn = lib().espdl_oracle_unary_s8 if x.dtype == np.int8 else lib().espdl_oracle_unary_s16
     fn(UNARY_KINDS[op_type], _ptr(x), x.size, int(in_exp), int(out_exp), float(alpha), float(beta), int(round_mode),
        _ptr(out))
+    return out
+
+
+REDUCE_OPS = {"ReduceMax": 0, "ReduceMin": 1, "ReduceSum": 2}
+
+
+def reduce_int(op_type, x, axes, keepdims=True, shift=0, round_mode=ROUND_HALF_UP):
+    """ReduceMax / ReduceMin / ReduceSum of an int8 or int16 tensor; shift = out_exp - in_exp (sum only)."""
+    x = np.ascontiguousarray(x)
+    assert x.dtype in (np.int8, np.int16)
+    nd = x.ndim
+    axes = [a + nd if a < 0 else a for a in (axes if len(axes) else range(nd))]
+    flags = np.array([1 if i in axes else 0 for i in range(nd)], dtype=np.int32)
+    kept = [x.shape[i] for i in range(nd) if not flags[i]]
+    out = np.empty(kept if kept else [1], dtype=x.dtype)
+    shape = np.array(x.shape, dtype=np.int32)
+    rc = lib().espdl_oracle_reduce_int(_ptr(x), 8 * x.dtype.itemsize, _ptr(shape), nd, _ptr(flags), REDUCE_OPS[op_type],
+                                       int(shift), int(round_mode), _ptr(out))
+    assert rc == 0
+    if keepdims:
+        out = out.reshape([1 if flags[i] else x.shape[i] for i in range(nd)])
     return out
 
 

@@ -165,6 +165,13 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None
                 reduce_mean = oracle.reduce_mean_s16 if x.dtype == np.int16 else oracle.reduce_mean_s8
                 y = reduce_mean(x, [int(v) for v in axes], bool(a.get("keepdims", 1)), spec.exponent(ins[0]),
                                 spec.exponent(y_name))
+        elif op in oracle.REDUCE_OPS:
+            axes = spec.initializers[ins[1]][2].ravel() if len(ins) > 1 and ins[1] in spec.initializers else a.get("axes", [])
+            if len(axes) == 0 and a.get("noop_with_empty_axes", 0):
+                y = x
+            else:
+                y = oracle.reduce_int(op, x, [int(v) for v in axes], bool(a.get("keepdims", 1)),
+                                      spec.exponent(y_name) - spec.exponent(ins[0]), round_mode)
         elif op == "Slice":
             par = [spec.initializers[n][2].ravel() if n in spec.initializers else None for n in (ins[1:5] + [None] * 4)[:4]]
             y = oracle.slice_(x, par[0], par[1], par[2], par[3])

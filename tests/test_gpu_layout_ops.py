@@ -215,3 +215,18 @@ def test_pad_rejects_what_the_reference_cannot_do(oracle):
         espdl().pad(empty, [0, 1, 0, 0], "edge")
     got = espdl().pad(empty, [0, 1, 0, 2], "constant", 5)
     assert got.shape == (2, 3) and bool((got == 5).all())
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("op", ["ReduceMax", "ReduceMin", "ReduceSum"])
+def test_reduce_int(oracle, op, dtype):
+    announce(f"reduce_int {op} {np.dtype(dtype).name}")
+    rng = np.random.default_rng(74)
+    info = np.iinfo(dtype)
+    cases = [((3, 14, 14, 32), [1, 2], True), ((3, 14, 14, 32), [3], True), ((2, 40, 97), [-1], False),
+             ((2, 5, 6, 7), [], True), ((4, 300), [0], False), ((2, 3, 4, 5, 6), [1, 3], True)]
+    for shape, axes, keep in cases:
+        x = rng.integers(info.min, info.max, size=shape, dtype=dtype, endpoint=True)
+        for shift, rm in ([(0, 0)] if op != "ReduceSum" else [(-1, 0), (0, 0), (4, 0), (4, 1), (7, 1)]):
+            got = to_host(espdl().reduce_int(op, to_dev(x), axes, keep, shift, rm))
+            np.testing.assert_array_equal(got, oracle.reduce_int(op, x, axes, keep, shift, rm))

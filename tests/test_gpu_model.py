@@ -299,6 +299,21 @@ def test_padded_convs(oracle):
     mdl.close()
 
 
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+@pytest.mark.parametrize("s16", [False, True], ids=["s8", "s16"])
+def test_reduce_heads(oracle, s16, round_mode):
+    """ReduceMax, ReduceMin and ReduceSum nodes through dl::Model."""
+    announce(f"model reduce_heads s16={s16} round_mode={round_mode}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.reduce_heads(s16=s16)
+    mdl, want, _ = _run_config(spec, 3, 45, round_mode=round_mode)
+    for name in spec.outputs:
+        got = mdl.get_tensor(name, np.int16) if s16 else mdl.get_tensor(name)
+        np.testing.assert_array_equal(got, want[name], err_msg=name)
+        assert len(np.unique(want[name])) > 8, name
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()

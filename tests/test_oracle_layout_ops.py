@@ -225,3 +225,31 @@ def test_pad_of_an_empty_axis_is_all_constant(oracle):
     x = np.zeros((2, 0, 3), np.int8)
     got = oracle.pad(x, [0, 2, 0, 0, 1, 0], "constant", 7)
     assert got.shape == (2, 3, 3) and np.all(got == 7)
+
+
+@pytest.mark.parametrize("dtype", [np.int8, np.int16])
+@pytest.mark.parametrize("op", ["ReduceMax", "ReduceMin", "ReduceSum"])
+def test_reduce_int_is_numpy(oracle, op, dtype):
+    """numpy max / min / sum over the same axes; the sum then takes the pinned shift-round and saturates."""
+    rng = np.random.default_rng(73)
+    info = np.iinfo(dtype)
+    for axes, keep in [([1, 2], True), ([3], False), ([0, 2], True), ([], True), ([-1], True), ([1], False)]:
+        x = rng.integers(info.min, info.max, size=(2, 5, 6, 7), dtype=dtype, endpoint=True)
+        ax = tuple(a % 4 for a in axes) if axes else None
+        if op == "ReduceSum":
+            for shift in (-1, 0, 3, 6):
+                for rm in (0, 1):
+                    s = x.astype(np.int64).sum(axis=ax, keepdims=keep)
+                    if shift <= 0:
+                        q = s << -shift
+                    elif rm == 0:
+                        q = (s + (1 << (shift - 1))) >> shift          # floor((s + half) / 2^shift)
+                    else:
+                        q = np.round(s / 2.0 ** shift).astype(np.int64)  # exact in float64; numpy rounds half to even
+                    want = np.clip(q, info.min, info.max).astype(dtype)
+                    got = oracle.reduce_int(op, x, axes, keep, shift, rm)
+                    np.testing.assert_array_equal(got.reshape(want.shape), want)
+        else:
+            want = (x.max if op == "ReduceMax" else x.min)(axis=ax, keepdims=keep)
+            got = oracle.reduce_int(op, x, axes, keep)
+            np.testing.assert_array_equal(got.reshape(np.shape(want)), want)
