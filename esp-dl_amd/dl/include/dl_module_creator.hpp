@@ -80,6 +80,8 @@ public:
         register_module("ReduceSum", ReduceMean::deserialize_sum);
         register_module("InsertZeros", InsertZeros::deserialize);
         register_module("Pad", Pad::deserialize);
+        register_module("SpaceToDepth", SpaceDepth::deserialize_space_to_depth);
+        register_module("DepthToSpace", SpaceDepth::deserialize_depth_to_space);
         register_module("StreamingCache", StreamingCache::deserialize);
         register_module("Softmax", Softmax::deserialize);
         // both are TensorBase::assign between a float32 and a quantized tensor

@@ -860,6 +860,99 @@ public:
     void print() { DL_LOGI("InsertZeros", "stride: %s, quant_type: %s.", vector_to_string(m_stride).c_str(), quant_type_to_string(quant_type)); }
 };
 
+/// SpaceToDepth and DepthToSpace on NHWC tensors (esp-dl/dl/module/include/dl_module_space_to_depth.hpp:17-44,
+/// dl_module_depth_to_space.hpp:17-67).  Both are permutations of a six-axis view of the tensor, so they run
+/// on the transpose kernel:
+///   SpaceToDepth      [N, H/b, b, W/b, b, C] -> [N, H/b, W/b, C, b, b]      out_c = c * b^2 + (h % b) * b + w % b
+///   DepthToSpace CRD  [N, H, W, C', b, b]    -> [N, H, b, W, b, C']         c = out_c * b^2 + hb * b + wb
+///   DepthToSpace DCR  [N, H, W, b, b, C']    -> [N, H, b, W, b, C']         c = (hb * b + wb) * C' + out_c
+/// The reference's DCR loop takes out_c = c % b, which is this permutation when C' == b and not a permutation
+/// otherwise (output elements are written twice or never); the ONNX definition is used for every C'.
+class SpaceDepth : public Module {
+public:
+    enum kind_t { SPACE_TO_DEPTH, DEPTH_TO_SPACE_CRD, DEPTH_TO_SPACE_DCR };
+
+private:
+    kind_t m_kind;
+    int m_blocksize;
+
+public:
+    SpaceDepth(kind_t kind, int blocksize, const char *name = nullptr, quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_kind(kind), m_blocksize(blocksize)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        const int b = m_blocksize;
+        if (in.size() != 4 || b < 1)
+            return {{}};
+        if (m_kind == SPACE_TO_DEPTH) {
+            if (in[1] % b || in[2] % b)
+                return {{}};
+            return {{in[0], in[1] / b, in[2] / b, in[3] * b * b}};
+        }
+        if (in[3] % (b * b))
+            return {{}};
+        return {{in[0], in[1] * b, in[2] * b, in[3] / (b * b)}};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        const char *tag = m_kind == SPACE_TO_DEPTH ? "SpaceToDepth" : "DepthToSpace";
+        if (!on_device_all({input, output}) || input->shape.size() != 4 || input->dtype != output->dtype ||
+            input->get_size() != output->get_size()) {
+            DL_LOGE(tag, "%s: needs NHWC device tensors of one type", name.c_str());
+            return;
+        }
+        const int b = m_blocksize, n = input->shape[0], h = input->shape[1], w = input->shape[2], c = input->shape[3];
+        int32_t view[6], perm[6];
+        if (m_kind == SPACE_TO_DEPTH) {
+            const int32_t v[6] = {n, h / b, b, w / b, b, c}, p[6] = {0, 1, 3, 5, 2, 4};
+            std::copy(v, v + 6, view);
+            std::copy(p, p + 6, perm);
+        } else if (m_kind == DEPTH_TO_SPACE_CRD) {
+            const int32_t v[6] = {n, h, w, c / (b * b), b, b}, p[6] = {0, 1, 4, 2, 5, 3};
+            std::copy(v, v + 6, view);
+            std::copy(p, p + 6, perm);
+        } else {
+            const int32_t v[6] = {n, h, w, b, b, c / (b * b)}, p[6] = {0, 1, 3, 2, 4, 5};
+            std::copy(v, v + 6, view);
+            std::copy(p, p + 6, perm);
+        }
+        const int rc = espdl_hip_transpose(input->data, view, 6, perm, 6, (int32_t)input->get_dtype_bytes(), output->data,
+                                           context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE(tag, "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    static Module *deserialize_space_to_depth(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        int blocksize = 2;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "blocksize", blocksize);
+        return new SpaceDepth(SPACE_TO_DEPTH, blocksize, node_name.c_str(), quant_type);
+    }
+    static Module *deserialize_depth_to_space(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        int blocksize = 2;
+        std::string mode_name = "DCR";
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "blocksize", blocksize);
+        fbs_model->get_operation_attribute(node_name, "mode", mode_name);
+        return new SpaceDepth(mode_name == "CRD" ? DEPTH_TO_SPACE_CRD : DEPTH_TO_SPACE_DCR, blocksize, node_name.c_str(),
+                              quant_type);
+    }
+    void print()
+    {
+        DL_LOGI(m_kind == SPACE_TO_DEPTH ? "SpaceToDepth" : "DepthToSpace", "blocksize: %d, quant_type: %s.", m_blocksize,
+                quant_type_to_string(quant_type));
+    }
+};
+
 /// Pad (esp-dl/dl/module/include/dl_module_pad.hpp:12-100): pads and the optional constant are initializer
 /// operands; the constant is read as the tensor's element type, whatever its own exponent says
 /// (TensorBase::pad, esp-dl/dl/tensor/src/dl_tensor_base.cpp:1231-1234).

@@ -857,6 +857,28 @@ def reduce_heads(seed=0xE5DD, s16=False):
     return g
 
 
+def pixel_shuffle(seed=0xE5DE):
+    """SpaceToDepth in front of a convolution (a stride-2 stem without losing pixels), then DepthToSpace in both
+    channel orders as sub-pixel upsampling heads."""
+    g = GraphSpec("pixel_shuffle")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 12, 16, 8], -5)
+
+    def shuffle(op, src, out_shape, name, **attrs):
+        y = name + "_out"
+        g.add_value(y, out_shape, g.exponent(src))
+        g.add_node(name, op, [src], [y], quant_type="S8", **attrs)
+        return y
+
+    s = shuffle("SpaceToDepth", x, [1, 6, 8, 32], "fold", blocksize=2)
+    f = b.conv(s, 48, k=3, relu=True, name="features")
+    up_crd = shuffle("DepthToSpace", f, [1, 12, 16, 12], "unfold_crd", blocksize=2, mode="CRD")
+    up_dcr = shuffle("DepthToSpace", f, [1, 12, 16, 12], "unfold_dcr", blocksize=2, mode="DCR")
+    b.output(b.conv(up_crd, 8, k=3, name="head_crd"))
+    b.output(b.conv(up_dcr, 8, k=3, name="head_dcr"))
+    return g
+
+
 def int16_tail(seed=0xE5D9):
     """int8 Conv -> RequantizeLinear to int16 -> int16 Conv -> int16 table (SiLU) -> int16 Add (residual) ->
     int16 Mul by a constant -> int16 AveragePool -> int16 ReduceMean -> int16 Gemm: the operator mix of the

@@ -374,6 +374,39 @@ def unary(op_type, x, in_exp, out_exp, alpha=None, beta=None, round_mode=ROUND_H
     return out
 
 
+def space_to_depth(x, blocksize):
+    """SpaceToDepth on NHWC as the reference's loop scatters it
+    (esp-dl/dl/module/include/dl_module_space_to_depth.hpp:17-44): input element (n, h, w, c) lands at
+    (n, h // b, w // b, c * b^2 + (h % b) * b + w % b)."""
+    x = np.ascontiguousarray(x)
+    n, h, w, c = x.shape
+    b = int(blocksize)
+    out = np.empty((n, h // b, w // b, c * b * b), dtype=x.dtype)
+    hh, ww, cc = np.meshgrid(np.arange(h), np.arange(w), np.arange(c), indexing="ij")
+    out[:, hh // b, ww // b, cc * b * b + (hh % b) * b + ww % b] = x[:, hh, ww, cc]
+    return out
+
+
+def depth_to_space(x, blocksize, mode="DCR"):
+    """DepthToSpace on NHWC, a scatter like the reference's loops
+    (esp-dl/dl/module/include/dl_module_depth_to_space.hpp:17-67).  CRD: channel c goes to out channel c // b^2 at
+    row offset (c % b^2) // b and column offset c % b.  DCR: the reference takes out channel c % b, row offset
+    c // b^2, column offset (c % b^2) // b, which is a permutation only when the output has b channels; the ONNX
+    definition c = (row * b + col) * C' + out_c agrees with it there and is used for every C'."""
+    x = np.ascontiguousarray(x)
+    n, h, w, c = x.shape
+    b = int(blocksize)
+    oc = c // (b * b)
+    out = np.empty((n, h * b, w * b, oc), dtype=x.dtype)
+    hh, ww, cc = np.meshgrid(np.arange(h), np.arange(w), np.arange(c), indexing="ij")
+    if mode == "CRD":
+        k, row, col = cc // (b * b), (cc % (b * b)) // b, cc % b
+    else:
+        k, row, col = cc % oc, cc // (b * oc), (cc // oc) % b
+    out[:, hh * b + row, ww * b + col, k] = x[:, hh, ww, cc]
+    return out
+
+
 REDUCE_OPS = {"ReduceMax": 0, "ReduceMin": 1, "ReduceSum": 2}
 
 

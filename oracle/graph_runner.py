@@ -108,6 +108,10 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None
             y = oracle.unary(op, x, exponent_of(ins[0]), spec.exponent(y_name), a.get("alpha"), a.get("beta"), round_mode)
         elif op == "Identity":  # output->assign(input): a requantize when the exponents differ
             y = requantize(x, spec.exponent(ins[0]), spec.exponent(y_name), spec.dtype(y_name))
+        elif op == "SpaceToDepth":
+            y = oracle.space_to_depth(x, a.get("blocksize", 2))
+        elif op == "DepthToSpace":
+            y = oracle.depth_to_space(x, a.get("blocksize", 2), a.get("mode", "DCR"))
         elif op == "Pad":
             pads = [int(v) for v in spec.initializers[ins[1]][2].ravel()]
             value = int(spec.initializers[ins[2]][2].ravel()[0]) if len(ins) > 2 and ins[2] else 0

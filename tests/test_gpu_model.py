@@ -314,6 +314,19 @@ def test_reduce_heads(oracle, s16, round_mode):
     mdl.close()
 
 
+def test_pixel_shuffle(oracle):
+    """SpaceToDepth and DepthToSpace (CRD and DCR) nodes through dl::Model."""
+    announce("model pixel_shuffle")
+    _, zoo, _, _ = _mods()
+    spec = zoo.pixel_shuffle()
+    mdl, want, _ = _run_config(spec, 3, 47)
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
+        assert len(np.unique(want[name])) > 20, name
+    assert not np.array_equal(want[spec.outputs[0]], want[spec.outputs[1]])
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()

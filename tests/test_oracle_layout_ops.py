@@ -253,3 +253,38 @@ def test_reduce_int_is_numpy(oracle, op, dtype):
             want = (x.max if op == "ReduceMax" else x.min)(axis=ax, keepdims=keep)
             got = oracle.reduce_int(op, x, axes, keep)
             np.testing.assert_array_equal(got.reshape(np.shape(want)), want)
+
+
+@pytest.mark.parametrize("b", [2, 3])
+def test_space_to_depth_and_depth_to_space_are_the_onnx_permutations(oracle, b):
+    """The ONNX operator definitions are reshape / transpose recipes (NCHW there, NHWC here); the oracle scatters
+    with the reference's index arithmetic.  CRD DepthToSpace inverts SpaceToDepth."""
+    rng = np.random.default_rng(75)
+    for c in (1, 4, 5):
+        x = rng.integers(-128, 128, size=(2, 2 * b, 3 * b, c), dtype=np.int8)
+        n, h, w, _ = x.shape
+        want = x.reshape(n, h // b, b, w // b, b, c).transpose(0, 1, 3, 5, 2, 4).reshape(n, h // b, w // b, c * b * b)
+        got = oracle.space_to_depth(x, b)
+        np.testing.assert_array_equal(got, want)
+        np.testing.assert_array_equal(oracle.depth_to_space(got, b, "CRD"), x)
+    for oc in (1, b, 5):
+        x = rng.integers(-128, 128, size=(2, 3, 4, oc * b * b), dtype=np.int16)
+        n, h, w, _ = x.shape
+        crd = x.reshape(n, h, w, oc, b, b).transpose(0, 1, 4, 2, 5, 3).reshape(n, h * b, w * b, oc)
+        dcr = x.reshape(n, h, w, b, b, oc).transpose(0, 1, 3, 2, 4, 5).reshape(n, h * b, w * b, oc)
+        np.testing.assert_array_equal(oracle.depth_to_space(x, b, "CRD"), crd)
+        np.testing.assert_array_equal(oracle.depth_to_space(x, b, "DCR"), dcr)
+
+
+def test_depth_to_space_dcr_is_the_reference_loop_when_it_is_a_permutation(oracle):
+    """dl_module_depth_to_space.hpp:45-67 with C' == b: out channel c % b, row offset c // b^2, column offset
+    (c % b^2) // b, replayed element by element."""
+    rng = np.random.default_rng(76)
+    b = 2
+    x = rng.integers(-128, 128, size=(1, 3, 2, b * b * b), dtype=np.int8)
+    want = np.zeros((1, 3 * b, 2 * b, b), dtype=np.int8)
+    for h in range(3):
+        for w in range(2):
+            for c in range(b * b * b):
+                want[0, h * b + c // (b * b), w * b + (c % (b * b)) // b, c % b] = x[0, h, w, c]
+    np.testing.assert_array_equal(oracle.depth_to_space(x, b, "DCR"), want)
