@@ -80,6 +80,7 @@ public:
         register_module("ReduceSum", ReduceMean::deserialize_sum);
         register_module("InsertZeros", InsertZeros::deserialize);
         register_module("Pad", Pad::deserialize);
+        register_module("Gather", Gather::deserialize);
         register_module("SpaceToDepth", SpaceDepth::deserialize_space_to_depth);
         register_module("DepthToSpace", SpaceDepth::deserialize_depth_to_space);
         register_module("StreamingCache", StreamingCache::deserialize);

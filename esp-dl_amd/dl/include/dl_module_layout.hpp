@@ -953,6 +953,100 @@ public:
     }
 };
 
+/// Gather with constant indices (esp-dl/dl/module/include/dl_module_gather.hpp:13-170): for every outer index, the
+/// rows named by `indices` along `axis` are copied in order.  Runs of consecutive indices are one strided copy
+/// (espdl_hip_copy_rows), so a single index or a range costs one launch.  Indices outside [0, extent) read
+/// outside the tensor in the reference; they are rejected here.
+class Gather : public Module {
+private:
+    std::vector<int64_t> m_indices;
+    std::vector<int> m_indices_shape;
+    int m_axis;
+
+public:
+    Gather(const std::vector<int64_t> &indices, const std::vector<int> &indices_shape, int axis, const char *name = nullptr,
+           quant_type_t quant_type = QUANT_TYPE_NONE) :
+        Module(name, MODULE_NON_INPLACE, quant_type), m_indices(indices), m_indices_shape(indices_shape), m_axis(axis)
+    {
+    }
+    std::vector<std::vector<int>> get_output_shape(std::vector<std::vector<int>> &input_shapes)
+    {
+        const std::vector<int> &in = input_shapes[0];
+        const int axis = m_axis < 0 ? m_axis + (int)in.size() : m_axis;
+        if (axis < 0 || axis >= (int)in.size())
+            return {{}};
+        for (int64_t i : m_indices)
+            if (i < 0 || i >= in[axis])
+                return {{}};
+        std::vector<int> out(in.begin(), in.begin() + axis);
+        out.insert(out.end(), m_indices_shape.begin(), m_indices_shape.end());
+        out.insert(out.end(), in.begin() + axis + 1, in.end());
+        if (out.empty())
+            out.push_back(1);
+        return {out};
+    }
+    void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
+    {
+        (void)mode;
+        TensorBase *input = context->get_tensor(m_inputs_index[0]);
+        TensorBase *output = context->get_tensor(m_outputs_index[0]);
+        const int rank = (int)input->shape.size(), axis = m_axis < 0 ? m_axis + rank : m_axis;
+        if (!on_device_all({input, output}) || input->dtype != output->dtype || axis < 0 || axis >= rank) {
+            DL_LOGE("Gather", "%s: needs device tensors of one type and an axis inside the tensor", name.c_str());
+            return;
+        }
+        int64_t outer = 1, inner = input->get_dtype_bytes();
+        for (int i = 0; i < axis; i++)
+            outer *= input->shape[i];
+        for (int i = axis + 1; i < rank; i++)
+            inner *= input->shape[i];
+        const int64_t extent = input->shape[axis], count = (int64_t)m_indices.size();
+        if (output->get_size() * (int64_t)output->get_dtype_bytes() != outer * count * inner) {
+            DL_LOGE("Gather", "%s: output size does not match", name.c_str());
+            return;
+        }
+        const char *src = static_cast<const char *>(input->data);
+        char *dst = static_cast<char *>(output->data);
+        for (int64_t i = 0; i < count;) {
+            int64_t run = 1;
+            while (i + run < count && m_indices[i + run] == m_indices[i] + run)
+                run++;
+            if (m_indices[i] < 0 || m_indices[i] + run > extent) {
+                DL_LOGE("Gather", "%s: index outside the axis", name.c_str());
+                return;
+            }
+            const int rc = espdl_hip_copy_rows(src + m_indices[i] * inner, extent * inner, dst + i * inner, count * inner,
+                                               run * inner, outer, context->stream);
+            if (rc != ESPDL_HIP_OK) {
+                DL_LOGE("Gather", "%s: %s", name.c_str(), espdl_hip_last_error());
+                return;
+            }
+            i += run;
+        }
+    }
+    static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        quant_type_t quant_type = QUANT_TYPE_NONE;
+        int axis = 0;
+        fbs_model->get_operation_attribute(node_name, "quant_type", quant_type);
+        fbs_model->get_operation_attribute(node_name, "axis", axis);
+        TensorBase *t = fbs_model->get_operation_parameter(node_name, 1);
+        if (!t || (t->dtype != DATA_TYPE_INT64 && t->dtype != DATA_TYPE_INT32)) {
+            DL_LOGE("Gather", "%s: indices must be an int64 or int32 initializer", node_name.c_str());
+            delete t;
+            return nullptr;
+        }
+        std::vector<int64_t> indices;
+        for (int i = 0; i < t->get_size(); i++)
+            indices.push_back(t->dtype == DATA_TYPE_INT64 ? t->get_element_ptr<int64_t>()[i]
+                                                          : (int64_t)t->get_element_ptr<int32_t>()[i]);
+        const std::vector<int> shape = t->shape;
+        delete t;
+        return new Gather(indices, shape, axis, node_name.c_str(), quant_type);
+    }
+    void print() { DL_LOGI("Gather", "axis: %d, indices: %d, quant_type: %s.", m_axis, (int)m_indices.size(), quant_type_to_string(quant_type)); }
+};
+
 /// Pad (esp-dl/dl/module/include/dl_module_pad.hpp:12-100): pads and the optional constant are initializer
 /// operands; the constant is read as the tensor's element type, whatever its own exponent says
 /// (TensorBase::pad, esp-dl/dl/tensor/src/dl_tensor_base.cpp:1231-1234).

@@ -879,6 +879,28 @@ def pixel_shuffle(seed=0xE5DE):
     return g
 
 
+def gathered_rows(seed=0xE5DF):
+    """Gather with constant indices along three axes: one time step of a sequence (the usual exported form), a
+    reordering with repeats along channels, and a 2-D index tensor along the width."""
+    g = GraphSpec("gathered_rows")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 8, 10, 16], -5)
+    f = b.conv(x, 24, k=3, name="features")
+
+    def gather(src, indices, idx_shape, axis, out_shape, name):
+        y = name + "_out"
+        g.add_init(name + ".indices", idx_shape, INT64, indices, [0])
+        g.add_value(y, out_shape, g.exponent(src))
+        g.add_node(name, "Gather", [src, name + ".indices"], [y], axis=axis, quant_type="S8")
+        g.outputs.append(y)
+        return y
+
+    gather(f, [7], [1], 1, [1, 1, 10, 24], "last_row")
+    gather(f, [5, 6, 7, 0, 0, 23, 1, 2, 3], [9], -1, [1, 8, 10, 9], "channels")
+    gather(f, [0, 9, 4, 5, 6, 2], [2, 3], 2, [1, 8, 2, 3, 24], "columns")
+    return g
+
+
 def int16_tail(seed=0xE5D9):
     """int8 Conv -> RequantizeLinear to int16 -> int16 Conv -> int16 table (SiLU) -> int16 Add (residual) ->
     int16 Mul by a constant -> int16 AveragePool -> int16 ReduceMean -> int16 Gemm: the operator mix of the

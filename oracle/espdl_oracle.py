@@ -374,6 +374,25 @@ def unary(op_type, x, in_exp, out_exp, alpha=None, beta=None, round_mode=ROUND_H
     return out
 
 
+def gather(x, indices, axis=0):
+    """Gather with constant indices as the reference copies it
+    (esp-dl/dl/module/include/dl_module_gather.hpp:56-66): per outer index, one inner row per index, in order."""
+    x = np.ascontiguousarray(x)
+    indices = np.asarray(indices, dtype=np.int64)
+    axis = axis + x.ndim if axis < 0 else axis
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    extent = x.shape[axis]
+    flat_in = x.reshape(outer, extent, inner)
+    flat_idx = indices.ravel()
+    assert flat_idx.size == 0 or (flat_idx.min() >= 0 and flat_idx.max() < extent)
+    out = np.empty((outer, flat_idx.size, inner), dtype=x.dtype)
+    for o in range(outer):
+        for i, idx in enumerate(flat_idx):
+            out[o, i] = flat_in[o, int(idx)]
+    return out.reshape(list(x.shape[:axis]) + list(indices.shape) + list(x.shape[axis + 1:]))
+
+
 def space_to_depth(x, blocksize):
     """SpaceToDepth on NHWC as the reference's loop scatters it
     (esp-dl/dl/module/include/dl_module_space_to_depth.hpp:17-44): input element (n, h, w, c) lands at

@@ -112,6 +112,9 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None
             y = oracle.space_to_depth(x, a.get("blocksize", 2))
         elif op == "DepthToSpace":
             y = oracle.depth_to_space(x, a.get("blocksize", 2), a.get("mode", "DCR"))
+        elif op == "Gather":
+            dims, _, data, _ = spec.initializers[ins[1]]
+            y = oracle.gather(x, np.asarray(data).reshape(dims), a.get("axis", 0))
         elif op == "Pad":
             pads = [int(v) for v in spec.initializers[ins[1]][2].ravel()]
             value = int(spec.initializers[ins[2]][2].ravel()[0]) if len(ins) > 2 and ins[2] else 0

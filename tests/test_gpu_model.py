@@ -327,6 +327,18 @@ def test_pixel_shuffle(oracle):
     mdl.close()
 
 
+def test_gathered_rows(oracle):
+    """Gather with constant indices (single index, repeats, a 2-D index tensor) through dl::Model."""
+    announce("model gathered_rows")
+    _, zoo, _, _ = _mods()
+    spec = zoo.gathered_rows()
+    mdl, want, _ = _run_config(spec, 3, 49)
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
+        assert len(np.unique(want[name])) > 20, name
+    mdl.close()
+
+
 def test_config5_ocr_style(oracle):
     announce("model config5 batch 3")
     _, zoo, _, _ = _mods()

@@ -288,3 +288,12 @@ def test_depth_to_space_dcr_is_the_reference_loop_when_it_is_a_permutation(oracl
             for c in range(b * b * b):
                 want[0, h * b + c // (b * b), w * b + (c % (b * b)) // b, c % b] = x[0, h, w, c]
     np.testing.assert_array_equal(oracle.depth_to_space(x, b, "DCR"), want)
+
+
+def test_gather_is_numpy_take(oracle):
+    rng = np.random.default_rng(77)
+    x = rng.integers(-128, 128, size=(3, 5, 6, 7), dtype=np.int8)
+    for axis, idx in [(0, [2]), (1, [4, 0, 0, 3]), (-1, [[0, 6], [3, 3]]), (2, list(range(6)))]:
+        np.testing.assert_array_equal(oracle.gather(x, idx, axis), np.take(x, np.asarray(idx), axis=axis))
+    x16 = rng.integers(-32768, 32767, size=(4, 9), dtype=np.int16)
+    np.testing.assert_array_equal(oracle.gather(x16, [8, 1], 1), np.take(x16, [8, 1], axis=1))
