@@ -152,7 +152,8 @@ __global__ __launch_bounds__(kThreads) void reduce_mean_s16_kernel(const Reduce1
 
 // ReduceMax / ReduceMin / ReduceSum (esp-dl/dl/module/include/dl_module_reduce_max.hpp:14-52,
 // dl_module_reduce_min.hpp:15-53, dl_module_reduce_sum.hpp:13-56): max and min return the stored integer, the sum
-// (int32 for int8, int64 for int16) goes through shift_and_round(sum, out_exp - in_exp) and truncate.
+// (int32 for int8, int64 for int16) goes through shift_and_round(sum, out_exp - in_exp) and truncate.  ReduceL1 and
+// ReduceSumSquare (dl_module_reduce_l1.hpp:14-50, dl_module_reduce_sum_square.hpp:14-46) sum |x| and x * x the same way.
 template <typename T>
 struct ReduceIntArgs {
     const T *in;
@@ -164,7 +165,7 @@ struct ReduceIntArgs {
     int shift, half_even;
 };
 
-// OP: 0 max, 1 min, 2 sum
+// OP: 0 max, 1 min, 2 sum, 3 sum of magnitudes (ReduceL1), 4 sum of squares (ReduceSumSquare)
 template <typename T, int OP>
 __global__ __launch_bounds__(kThreads) void reduce_int_kernel(const ReduceIntArgs<T> a)
 {
@@ -185,9 +186,9 @@ __global__ __launch_bounds__(kThreads) void reduce_int_kernel(const ReduceIntArg
                 rr = q;
             }
             const long long v = a.in[off];
-            acc = OP == 0 ? max(acc, v) : (OP == 1 ? min(acc, v) : acc + v);
+            acc = OP == 0 ? max(acc, v) : (OP == 1 ? min(acc, v) : (OP == 2 ? acc + v : (OP == 3 ? acc + (v < 0 ? -v : v) : acc + v * v)));
         }
-        if (OP == 2)
+        if (OP >= 2)
             acc = sizeof(T) == 1 ? requant_s8((int)acc, a.shift, false, a.half_even)
                                  : requant_s16(acc, a.shift, false, a.half_even);
         a.out[o] = (T)acc;
@@ -361,8 +362,12 @@ hipError_t launch_reduce_int_t(const T *in, const int *shape, int dims, const in
         reduce_int_kernel<T, 0><<<grid, block, 0, stream>>>(a);
     else if (op == 1)
         reduce_int_kernel<T, 1><<<grid, block, 0, stream>>>(a);
-    else
+    else if (op == 2)
         reduce_int_kernel<T, 2><<<grid, block, 0, stream>>>(a);
+    else if (op == 3)
+        reduce_int_kernel<T, 3><<<grid, block, 0, stream>>>(a);
+    else
+        reduce_int_kernel<T, 4><<<grid, block, 0, stream>>>(a);
     return hipGetLastError();
 }
 

@@ -547,7 +547,7 @@ int espdl_hip_reduce_int(const void *in, int32_t dtype, const int32_t *shape, in
         return fail(ESPDL_HIP_EINVAL, "dtype must be ESPDL_HIP_S8 or ESPDL_HIP_S16");
     if (dims < 1 || dims > 8 || shape == nullptr || reduce_flag == nullptr)
         return fail(ESPDL_HIP_EINVAL, "reduce handles 1..8 dims");
-    if (op != ESPDL_HIP_REDUCE_MAX && op != ESPDL_HIP_REDUCE_MIN && op != ESPDL_HIP_REDUCE_SUM)
+    if (op < ESPDL_HIP_REDUCE_MAX || op > ESPDL_HIP_REDUCE_SUM_SQUARE)
         return fail(ESPDL_HIP_EINVAL, "unknown reduce op %d", op);
     if (round_mode != ESPDL_HIP_ROUND_HALF_UP && round_mode != ESPDL_HIP_ROUND_HALF_EVEN)
         return fail(ESPDL_HIP_EINVAL, "bad round_mode %d", round_mode);
@@ -569,8 +569,9 @@ int espdl_hip_reduce_int(const void *in, int32_t dtype, const int32_t *shape, in
     }
     if (n_out == 0)
         return ESPDL_HIP_OK;
-    if (dtype == ESPDL_HIP_S8 && op == ESPDL_HIP_REDUCE_SUM && count > (1ll << 24))
-        return fail(ESPDL_HIP_ENOTSUP, "an int8 sum over more than 2^24 elements leaves the reference's int32");
+    if (dtype == ESPDL_HIP_S8 && op >= ESPDL_HIP_REDUCE_SUM &&
+        count > (op == ESPDL_HIP_REDUCE_SUM_SQUARE ? (1ll << 17) - 1 : (1ll << 24) - 1))
+        return fail(ESPDL_HIP_ENOTSUP, "this int8 sum can leave the reference's int32 accumulator");
     if (out == nullptr || (in == nullptr && count > 0))
         return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
     if (dtype == ESPDL_HIP_S16 && (misaligned(in, 2) || misaligned(out, 2)))

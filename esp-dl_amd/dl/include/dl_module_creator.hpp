@@ -78,6 +78,8 @@ public:
         register_module("ReduceMax", ReduceMean::deserialize_max);
         register_module("ReduceMin", ReduceMean::deserialize_min);
         register_module("ReduceSum", ReduceMean::deserialize_sum);
+        register_module("ReduceL1", ReduceMean::deserialize_l1);
+        register_module("ReduceSumSquare", ReduceMean::deserialize_sum_square);
         register_module("InsertZeros", InsertZeros::deserialize);
         register_module("Pad", Pad::deserialize);
         register_module("Gather", Gather::deserialize);

@@ -624,7 +624,8 @@ public:
         if (m_int_op >= 0) {
             const int rc = espdl_hip_reduce_int(
                 input->data, quant_type == QUANT_TYPE_SYMM_16BIT ? ESPDL_HIP_S16 : ESPDL_HIP_S8, input->shape.data(),
-                (int32_t)input->shape.size(), f.data(), m_int_op, output->exponent.get() - input->exponent.get(),
+                (int32_t)input->shape.size(), f.data(), m_int_op,
+                output->exponent.get() - input->exponent.get() * (m_int_op == ESPDL_HIP_REDUCE_SUM_SQUARE ? 2 : 1),
                 context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP,
                 output->data, context->stream);
             if (rc != ESPDL_HIP_OK)
@@ -653,6 +654,14 @@ public:
     static Module *deserialize_sum(fbs::FbsModel *fbs_model, std::string node_name)
     {
         return make(fbs_model, node_name, ESPDL_HIP_REDUCE_SUM);
+    }
+    static Module *deserialize_l1(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        return make(fbs_model, node_name, ESPDL_HIP_REDUCE_L1);
+    }
+    static Module *deserialize_sum_square(fbs::FbsModel *fbs_model, std::string node_name)
+    {
+        return make(fbs_model, node_name, ESPDL_HIP_REDUCE_SUM_SQUARE);
     }
     static Module *make(fbs::FbsModel *fbs_model, const std::string &node_name, int int_op)
     {

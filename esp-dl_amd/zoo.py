@@ -830,8 +830,8 @@ def padded_convs(seed=0xE5DC):
 
 
 def reduce_heads(seed=0xE5DD, s16=False):
-    """ReduceMax over the image, ReduceMin over channels and ReduceSum over the image (coarser output exponent)
-    on one feature map, int8 or int16."""
+    """ReduceMax over the image, ReduceMin over channels, ReduceSum and ReduceSumSquare over the image and ReduceL1
+    over channels (coarser output exponents for the sums) on one feature map, int8 or int16."""
     g = GraphSpec("reduce_heads_s16" if s16 else "reduce_heads")
     b = Builder(g, seed, per_channel=True, w_exp_range=None)
     qt, dt = ("S16", INT16) if s16 else ("S8", INT8)
@@ -854,6 +854,8 @@ def reduce_heads(seed=0xE5DD, s16=False):
     reduce("ReduceMax", [1, 2], [1, 1, 1, c], g.exponent(f), "image_max")
     reduce("ReduceMin", [-1], [1, h, w], g.exponent(f), "channel_min", keepdims=0)
     reduce("ReduceSum", [1, 2], [1, 1, 1, c], g.exponent(f) + 5, "image_sum")
+    reduce("ReduceL1", [-1], [1, h, w, 1], g.exponent(f) + 4, "channel_l1")
+    reduce("ReduceSumSquare", [1, 2], [1, 1, 1, c], 2 * g.exponent(f) + (20 if s16 else 12), "image_energy")
     return g
 
 

@@ -255,8 +255,16 @@ int espdl_hip_insert_zeros(const void *in, int32_t elem_size, int32_t batch, int
  * dl_module_reduce_min.hpp:15-53, dl_module_reduce_sum.hpp:13-56; loop nest dl_module_reduce_base.hpp).  dtype is
  * ESPDL_HIP_S8 or ESPDL_HIP_S16; shape / reduce_flag as espdl_hip_reduce_mean_s8.  Max and min return stored
  * integers and ignore shift; the sum (int32 for int8, int64 for int16) is shift_and_round(sum, shift) with
- * shift = out_exp - in_exp, then saturated.  An empty reduction gives the identity (type minimum, maximum, 0). */
-enum { ESPDL_HIP_REDUCE_MAX = 0, ESPDL_HIP_REDUCE_MIN = 1, ESPDL_HIP_REDUCE_SUM = 2 };
+ * shift = out_exp - in_exp, then saturated.  ReduceL1 and ReduceSumSquare (dl_module_reduce_l1.hpp:14-50,
+ * dl_module_reduce_sum_square.hpp:14-46) sum |x| and x * x the same way, the latter with
+ * shift = out_exp - 2 * in_exp.  An empty reduction gives the identity (type minimum, maximum, 0). */
+enum {
+    ESPDL_HIP_REDUCE_MAX = 0,
+    ESPDL_HIP_REDUCE_MIN = 1,
+    ESPDL_HIP_REDUCE_SUM = 2,
+    ESPDL_HIP_REDUCE_L1 = 3,        /* sum of |x|, shift = out_exp - in_exp */
+    ESPDL_HIP_REDUCE_SUM_SQUARE = 4 /* sum of x * x, shift = out_exp - 2 * in_exp */
+};
 int espdl_hip_reduce_int(const void *in, int32_t dtype, const int32_t *shape, int32_t dims, const int32_t *reduce_flag,
                          int32_t op, int32_t shift, int32_t round_mode, void *out, void *stream);
 

@@ -760,7 +760,9 @@ void espdl_oracle_div_s16(const int16_t *in0, const int16_t *in1, int64_t size, 
  * dl_module_reduce_min.hpp:15-53, dl_module_reduce_sum.hpp:13-56): max and min of the stored integers from the
  * type's minimum / maximum; the sum is accumulated in int32 (int8) or int64 (int16), then
  * shift_and_round(sum, out_exp - in_exp) and truncate.  Written as one walk over the input that folds every
- * element into its output slot.  op: 0 max, 1 min, 2 sum.
+ * element into its output slot.  ReduceL1 and ReduceSumSquare (dl_module_reduce_l1.hpp:14-50,
+ * dl_module_reduce_sum_square.hpp:14-46) accumulate |x| and x * x the same way; the caller passes
+ * shift = out_exp - 2 * in_exp for the squares.  op: 0 max, 1 min, 2 sum, 3 L1, 4 sum of squares.
  */
 int espdl_oracle_reduce_int(const void *in, int bits, const int32_t *shape, int dims, const int32_t *reduce_flag, int op,
                             int shift, int round_mode, void *out)
@@ -788,8 +790,12 @@ int espdl_oracle_reduce_int(const void *in, int bits, const int32_t *shape, int 
             acc[o] = v > acc[o] ? v : acc[o];
         else if (op == 1)
             acc[o] = v < acc[o] ? v : acc[o];
-        else
+        else if (op == 2)
             acc[o] += v;
+        else if (op == 3)
+            acc[o] += v < 0 ? -v : v;
+        else
+            acc[o] += v * v;
         for (int d = dims - 1; d >= 0; d--) {
             if (++idx[d] < shape[d])
                 break;
@@ -798,7 +804,7 @@ int espdl_oracle_reduce_int(const void *in, int bits, const int32_t *shape, int 
     }
     for (int64_t o = 0; o < n_out; o++) {
         int64_t r = acc[o];
-        if (op == 2) {
+        if (op >= 2) {
             r = bits == 8 ? (int64_t)espdl_oracle_shift_round_s32((int32_t)r, shift, round_mode)
                           : espdl_oracle_shift_round_s64(r, shift, round_mode);
             r = clamp_i64(r, lo, hi);

@@ -426,7 +426,7 @@ def depth_to_space(x, blocksize, mode="DCR"):
     return out
 
 
-REDUCE_OPS = {"ReduceMax": 0, "ReduceMin": 1, "ReduceSum": 2}
+REDUCE_OPS = {"ReduceMax": 0, "ReduceMin": 1, "ReduceSum": 2, "ReduceL1": 3, "ReduceSumSquare": 4}
 
 
 def reduce_int(op_type, x, axes, keepdims=True, shift=0, round_mode=ROUND_HALF_UP):

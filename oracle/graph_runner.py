@@ -178,7 +178,8 @@ def run(spec, inputs, round_mode=oracle.ROUND_HALF_UP, keep_all=True, state=None
                 y = x
             else:
                 y = oracle.reduce_int(op, x, [int(v) for v in axes], bool(a.get("keepdims", 1)),
-                                      spec.exponent(y_name) - spec.exponent(ins[0]), round_mode)
+                                      spec.exponent(y_name) - spec.exponent(ins[0]) * (2 if op == "ReduceSumSquare" else 1),
+                                      round_mode)
         elif op == "Slice":
             par = [spec.initializers[n][2].ravel() if n in spec.initializers else None for n in (ins[1:5] + [None] * 4)[:4]]
             y = oracle.slice_(x, par[0], par[1], par[2], par[3])

@@ -218,7 +218,7 @@ def test_pad_rejects_what_the_reference_cannot_do(oracle):
 
 
 @pytest.mark.parametrize("dtype", [np.int8, np.int16])
-@pytest.mark.parametrize("op", ["ReduceMax", "ReduceMin", "ReduceSum"])
+@pytest.mark.parametrize("op", ["ReduceMax", "ReduceMin", "ReduceSum", "ReduceL1", "ReduceSumSquare"])
 def test_reduce_int(oracle, op, dtype):
     announce(f"reduce_int {op} {np.dtype(dtype).name}")
     rng = np.random.default_rng(74)
@@ -227,6 +227,8 @@ def test_reduce_int(oracle, op, dtype):
              ((2, 5, 6, 7), [], True), ((4, 300), [0], False), ((2, 3, 4, 5, 6), [1, 3], True)]
     for shape, axes, keep in cases:
         x = rng.integers(info.min, info.max, size=shape, dtype=dtype, endpoint=True)
-        for shift, rm in ([(0, 0)] if op != "ReduceSum" else [(-1, 0), (0, 0), (4, 0), (4, 1), (7, 1)]):
+        shifts = {"ReduceSum": [(-1, 0), (0, 0), (4, 0), (4, 1), (7, 1)], "ReduceL1": [(0, 0), (5, 0), (9, 1)],
+                  "ReduceSumSquare": [(0, 0), (12, 0), (15, 1), (24, 0), (27, 1)]}.get(op, [(0, 0)])
+        for shift, rm in shifts:
             got = to_host(espdl().reduce_int(op, to_dev(x), axes, keep, shift, rm))
             np.testing.assert_array_equal(got, oracle.reduce_int(op, x, axes, keep, shift, rm))

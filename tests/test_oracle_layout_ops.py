@@ -228,7 +228,7 @@ def test_pad_of_an_empty_axis_is_all_constant(oracle):
 
 
 @pytest.mark.parametrize("dtype", [np.int8, np.int16])
-@pytest.mark.parametrize("op", ["ReduceMax", "ReduceMin", "ReduceSum"])
+@pytest.mark.parametrize("op", ["ReduceMax", "ReduceMin", "ReduceSum", "ReduceL1", "ReduceSumSquare"])
 def test_reduce_int_is_numpy(oracle, op, dtype):
     """numpy max / min / sum over the same axes; the sum then takes the pinned shift-round and saturates."""
     rng = np.random.default_rng(73)
@@ -236,10 +236,12 @@ def test_reduce_int_is_numpy(oracle, op, dtype):
     for axes, keep in [([1, 2], True), ([3], False), ([0, 2], True), ([], True), ([-1], True), ([1], False)]:
         x = rng.integers(info.min, info.max, size=(2, 5, 6, 7), dtype=dtype, endpoint=True)
         ax = tuple(a % 4 for a in axes) if axes else None
-        if op == "ReduceSum":
-            for shift in (-1, 0, 3, 6):
+        if op in ("ReduceSum", "ReduceL1", "ReduceSumSquare"):
+            wide = x.astype(np.int64)
+            terms = wide if op == "ReduceSum" else (np.abs(wide) if op == "ReduceL1" else wide * wide)
+            for shift in ((-1, 0, 3, 6) if op != "ReduceSumSquare" else (0, 9, 14, 22)):
                 for rm in (0, 1):
-                    s = x.astype(np.int64).sum(axis=ax, keepdims=keep)
+                    s = terms.sum(axis=ax, keepdims=keep)
                     if shift <= 0:
                         q = s << -shift
                     elif rm == 0:
