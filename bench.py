@@ -10,6 +10,8 @@ input batch already resident in HBM.  Prints ONE JSON line:
   roofline     the kernel family that takes the most GPU time in a step: algorithmic bytes (or
                operations) of its launches divided by their HIP-event time, against MI355X's peak
   kernels      the same for every kernel family (conv/gemm on MFMA, depthwise, element-wise)
+  parity_checked  true when every output of the timed batch equals the CPU oracle's bit for bit (checked
+               after the timed region; the program exits with status 3 when it does not)
   cpu_baseline the CPU oracle (a port of the reference's portable C path) timed on this host's
                cores on a bounded sample of the same workload
 Synthetic data: seeded uniform int8 images, random-init int8 weights with per-channel exponents.
@@ -103,6 +105,25 @@ def cpu_baseline(pkg, spec, threads_all):
     }
 
 
+def check_against_oracle(spec, x, got, chunk=32):
+    """True when every graph output equals the oracle's, bit for bit."""
+    import numpy as np
+    import espdl_oracle as oracle
+    import graph_runner
+    oracle.set_threads(min(16, os.cpu_count() or 1))
+    ok = True
+    for i in range(0, x.shape[0], chunk):
+        want = graph_runner.run(spec, {spec.inputs[0]: x[i:i + chunk]}, keep_all=False)
+        for name in spec.outputs:
+            g = got[name][i:i + chunk]
+            if not np.array_equal(g.reshape(want[name].shape), want[name]):
+                bad = int((g.reshape(want[name].shape) != want[name]).sum())
+                print("bench.py: output %s of images %d..%d differs from the oracle in %d elements"
+                      % (name, i, i + chunk - 1, bad), file=sys.stderr)
+                ok = False
+    return ok
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -111,6 +132,7 @@ def main():
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--config", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-parity", action="store_true", help="skip the comparison of the timed batch with the oracle")
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of HIP-graph replay")
     ap.add_argument("--profile-repeats", type=int, default=5)
     ap.add_argument("--layers", action="store_true", help="print the per-module timing table to stderr")
@@ -162,8 +184,13 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
     images_per_s = batch * args.steps / elapsed
-    checksum = int(mdl.get_tensor(spec.outputs[0], np.int16 if spec.dtype(spec.outputs[0]) == 5 else np.int8)
-                   .astype(np.int64).sum())
+    out_np = {name: mdl.get_tensor(name, np.int16 if spec.dtype(name) == 5 else np.int8) for name in spec.outputs}
+    checksum = int(sum(int(v.astype(np.int64).sum()) for v in out_np.values()))
+    parity_checked = None
+    if not args.no_parity:
+        # outside the timed region: every output of the batch that was just timed (the result of the last
+        # timed step) against the CPU oracle on the same seeded input, in chunks of images
+        parity_checked = check_against_oracle(spec, x, out_np)
 
     # per-kernel timing with HIP events on the model's stream (eager launches of the same plan)
     mdl.disable_graph()
@@ -195,6 +222,7 @@ def main():
                       "ops_per_byte": round(ai, 1)}
     dom = max(kernels, key=lambda k: kernels[k]["us_per_step"])
     kd = kernels[dom]
+    # time per family comes from whole passes in plan order, so the family times add up to a step
     if dom in ("conv2d_s8",) and kd["ops_per_byte"] > MACHINE_BALANCE:
         roofline = {"kernel": dom, "bound": "mfma", "achieved": kd["TOPs"], "peak": PEAK_INT8_TOPS,
                     "unit": "TOP/s", "frac": kd["mfma_frac"], "traffic": None}
@@ -203,6 +231,8 @@ def main():
                     "frac": kd["hbm_frac"], "traffic": None}
     if args.config == 3 and batch == 256:
         roofline["traffic"] = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(dom)
+    roofline["frac_hbm"] = kd["hbm_frac"]
+    roofline["frac_mfma"] = kd["mfma_frac"]
     roofline["launches_per_step"] = kd["launches_per_step"]
     roofline["avg_launch_us"] = kd["avg_launch_us"]
     roofline["algorithmic_per_launch"] = (kd["algorithmic_ops_per_step"] if roofline["bound"] == "mfma"
@@ -210,7 +240,9 @@ def main():
 
     conv_macs = spec.macs_per_image * batch
     result = {
-        "metric": "images/sec + int8 TOPS (% roofline), MobileNetV2-224 int8, batch 256",
+        "metric": ("images/sec + int8 TOPS (% roofline), MobileNetV2-224 int8, batch 256"
+                   if args.config == 3 and batch == 256 else
+                   "images/sec + int8 TOPS (%% roofline), %s, batch %d" % (spec.name, batch)),
         "value": round(images_per_s, 1), "unit": "images/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "s8", "data": "synthetic",
@@ -220,6 +252,7 @@ def main():
         "int8_tops": round(2.0 * conv_macs / (ms_per_step * 1e-3) / 1e12, 2),
         "int8_mfma_frac": round(2.0 * conv_macs / (ms_per_step * 1e-3) / 1e12 / PEAK_INT8_TOPS, 4),
         "output_checksum": checksum,
+        "parity_checked": parity_checked,
         "roofline": roofline,
         "kernels": kernels,
     }
@@ -228,6 +261,8 @@ def main():
         result["cpu_baseline"] = cpu_baseline(pkg, spec, threads)
     mdl.close()
     print(json.dumps(result))
+    if parity_checked is False:
+        sys.exit(3)
 
 
 if __name__ == "__main__":

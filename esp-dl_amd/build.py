@@ -86,21 +86,24 @@ def build_host_layer(verbose=True):
 
 
 def build_api_check(verbose=True):
-    """lib/espdl_api_check: a small C++ program written against the host layer's public headers
-    (tests/cpp/api_check.cpp); the GPU tests run it on the `.espdl` fixtures."""
-    src = os.path.join(os.path.dirname(HERE), "tests", "cpp", "api_check.cpp")
-    out = os.path.join(LIB_DIR, "espdl_api_check")
-    warn = _run([HIPCC, "-x", "hip", "--offload-arch=" + ARCH, "-O1", "-std=c++17", "-Wall",
-                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                 "-I" + os.path.join(DL_DIR, "include"), "-I" + INCLUDE_DIR, src, "-o", out,
-                 "-L" + LIB_DIR, "-lespdl_dl", "-lespdl_hip", "-Wl,-rpath,$ORIGIN"])
-    if warn.strip() and verbose:
-        print("[api_check.cpp]\n%s" % warn, file=sys.stderr)
-    return out
+    """lib/espdl_api_check and lib/espdl_module_api_check: small C++ programs written against the host
+    layer's public headers (tests/cpp/*.cpp); the tests run them."""
+    outs = []
+    for stem in ("api_check", "module_api_check"):
+        src = os.path.join(os.path.dirname(HERE), "tests", "cpp", stem + ".cpp")
+        out = os.path.join(LIB_DIR, "espdl_" + stem)
+        warn = _run([HIPCC, "-x", "hip", "--offload-arch=" + ARCH, "-O1", "-std=c++17", "-Wall",
+                     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                     "-I" + os.path.join(DL_DIR, "include"), "-I" + INCLUDE_DIR, src, "-o", out,
+                     "-L" + LIB_DIR, "-lespdl_dl", "-lespdl_hip", "-Wl,-rpath,$ORIGIN"])
+        if warn.strip() and verbose:
+            print("[%s.cpp]\n%s" % (stem, warn), file=sys.stderr)
+        outs.append(out)
+    return outs
 
 
 def build_all(verbose=True):
-    return [build_kernels(verbose), build_host_layer(verbose), build_api_check(verbose)]
+    return [build_kernels(verbose), build_host_layer(verbose), *build_api_check(verbose)]
 
 
 if __name__ == "__main__":

@@ -6,6 +6,7 @@
 // "capabilities" describe host RAM vs device HBM instead of internal RAM vs PSRAM.
 #pragma once
 
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <string>
@@ -17,7 +18,20 @@ typedef int esp_err_t;
 #define ESP_FAIL (-1)
 #endif
 
-#define DL_LOGE(tag, fmt, ...) std::fprintf(stderr, "E (%s) " fmt "\n", tag, ##__VA_ARGS__)
+namespace dl {
+/// Number of errors logged by this process so far.  Module::forward returns void, as in the reference,
+/// so a launch that a kernel rejects can only log; dl::Model compares this count before and after a
+/// pass to report the failure to its caller (Model::last_run_failed).  The count is process-wide: an
+/// error logged by another thread during the pass is attributed to the pass as well.
+inline std::atomic<long> &error_log_count()
+{
+    static std::atomic<long> count{0};
+    return count;
+}
+} // namespace dl
+
+#define DL_LOGE(tag, fmt, ...) \
+    (dl::error_log_count().fetch_add(1), std::fprintf(stderr, "E (%s) " fmt "\n", tag, ##__VA_ARGS__))
 #define DL_LOGW(tag, fmt, ...) std::fprintf(stderr, "W (%s) " fmt "\n", tag, ##__VA_ARGS__)
 #define DL_LOGI(tag, fmt, ...) std::fprintf(stdout, "I (%s) " fmt "\n", tag, ##__VA_ARGS__)
 

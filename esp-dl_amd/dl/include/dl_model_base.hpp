@@ -60,6 +60,10 @@ public:
     bool enable_graph();
     void disable_graph();
     bool graph_enabled() const { return m_graph_exec != nullptr; }
+    /// True when a module logged an error (a rejected kernel launch, a host tensor handed to a device
+    /// module) or a HIP call failed since the last run / run_async / enable_graph / test began.  The
+    /// tensors a failed pass leaves behind are not valid results.
+    bool last_run_failed() const { return m_failed || error_log_count().load() != m_errors_at_start; }
 
     /// Compare every tensor that has a test vector in the FbsModel (int8 exact, int16 within 1).
     esp_err_t test();
@@ -102,6 +106,13 @@ private:
     void *m_graph = nullptr;      // hipGraph_t
     void *m_graph_exec = nullptr; // hipGraphExec_t
     bool m_built = false;
+    bool m_failed = false;
+    long m_errors_at_start = 0;
+    void begin_pass()
+    {
+        m_failed = false;
+        m_errors_at_start = error_log_count().load();
+    }
 };
 
 } // namespace dl

@@ -615,7 +615,9 @@ public:
                 for (int a : m_arg)
                     if ((a < 0 ? a + rank : a) == i && in[i] == 1)
                         drop = true;
-                if (m_arg.empty() && in[i] == 1 && i != 0)
+                // no axes: every extent-1 dimension goes, the leading one included when the batch is 1
+                // (esp-dl/dl/module/include/dl_module_squeeze.hpp:37-41)
+                if (m_arg.empty() && in[i] == 1)
                     drop = true;
                 if (!drop)
                     out.push_back(in[i]);
@@ -631,26 +633,39 @@ public:
                 out.push_back(ins ? 1 : in[src++]);
             }
         } else {
+            // The target shape is used as written, with the reference's two rules: a 0 copies the
+            // input extent unless allowzero is set, one -1 is inferred from the element count
+            // (esp-dl/dl/module/include/dl_module_reshape.hpp:36-75).  Exported targets describe one
+            // image (leading 1); only that leading 1 is replaced by the batch.  A target that folds the
+            // leading dimension into something else is valid for a batch of one only; anything whose
+            // element count differs from the input's has no output shape, so that build() fails.
             int64_t total = 1, known = 1;
             for (int d : in)
                 total *= d;
             out = m_arg;
-            // a 0 copies the input extent unless allowzero is set
-            // (esp-dl/dl/module/include/dl_module_reshape.hpp:46-61)
             for (size_t i = 0; i < out.size(); i++)
                 if (out[i] == 0 && !m_allowzero && i < in.size())
                     out[i] = in[i];
-            if (!out.empty())
-                out[0] = in[0]; // the batch dimension is kept
+            if (!out.empty() && out[0] == 1 && !in.empty())
+                out[0] = in[0];
             int infer = -1;
             for (size_t i = 0; i < out.size(); i++) {
-                if (out[i] == -1)
+                if (out[i] == -1) {
+                    if (infer >= 0)
+                        return {{}};
                     infer = (int)i;
-                else
+                } else {
                     known *= out[i];
+                }
             }
-            if (infer >= 0)
+            if (infer >= 0) {
+                if (known <= 0 || total % known != 0)
+                    return {{}};
                 out[infer] = (int)(total / known);
+                known *= out[infer];
+            }
+            if (known != total)
+                return {{}};
         }
         return {out};
     }

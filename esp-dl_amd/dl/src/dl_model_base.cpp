@@ -588,8 +588,11 @@ esp_err_t Model::build(int batch)
 
 void Model::run_async(runtime_mode_t mode)
 {
-    if (!m_built)
+    begin_pass();
+    if (!m_built) {
+        m_failed = true;
         return;
+    }
     if (m_graph_exec) {
         (void)hip_ok(hipGraphLaunch(static_cast<hipGraphExec_t>(m_graph_exec), static_cast<hipStream_t>(m_stream)),
                      "hipGraphLaunch");
@@ -656,6 +659,7 @@ void Model::run(int stage_num, int stage_index, runtime_mode_t mode)
         DL_LOGE(TAG, "Invalid stage_index(%d), it should be in range [0, %d).", stage_index, stage_num);
         return;
     }
+    begin_pass();
     const int start = stage_index * plan_size / stage_num;
     const int end = (stage_index + 1) * plan_size / stage_num;
     for (int i = start; i < end; i++)
@@ -667,6 +671,7 @@ bool Model::enable_graph()
 {
     if (!m_built || m_graph_exec)
         return m_graph_exec != nullptr;
+    begin_pass();
     hipStream_t s = static_cast<hipStream_t>(m_stream);
     // one eager pass so that every module has uploaded its shifts / tables before capture starts; modules that
     // carry data between passes (StreamingCache) get it back afterwards, the pass counts for nothing
@@ -676,8 +681,8 @@ bool Model::enable_graph()
         module->forward(m_model_context, RUNTIME_MODE_AUTO);
     for (auto *module : m_execution_plan)
         module->restore_state(m_stream);
-    if (!hip_ok(hipStreamSynchronize(s), "hipStreamSynchronize"))
-        return false;
+    if (!hip_ok(hipStreamSynchronize(s), "hipStreamSynchronize") || last_run_failed())
+        return false; // a plan with a rejected module must not be captured: the graph would miss its kernels
     if (!hip_ok(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture"))
         return false;
     for (auto *module : m_execution_plan)
@@ -685,6 +690,10 @@ bool Model::enable_graph()
     hipGraph_t graph = nullptr;
     if (!hip_ok(hipStreamEndCapture(s, &graph), "hipStreamEndCapture") || !graph)
         return false;
+    if (last_run_failed()) {
+        (void)hipGraphDestroy(graph);
+        return false;
+    }
     hipGraphExec_t exec = nullptr;
     if (!hip_ok(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0), "hipGraphInstantiate")) {
         (void)hipGraphDestroy(graph);
@@ -712,6 +721,7 @@ esp_err_t Model::test()
 {
     if (!m_built)
         return ESP_FAIL;
+    begin_pass();
     for (auto &kv : m_inputs) {
         TensorBase *test_input = m_fbs_model->get_test_input_tensor(kv.first);
         if (!test_input) {
@@ -739,6 +749,10 @@ esp_err_t Model::test()
     for (auto *module : m_execution_plan) {
         module->forward(m_model_context, RUNTIME_MODE_SINGLE_CORE);
         synchronize();
+        if (last_run_failed()) {
+            DL_LOGE(TAG, "Module %s failed", module->name.c_str());
+            return ESP_FAIL;
+        }
         for (int index : module->get_outputs_index()) {
             const std::string out_name = m_model_context->get_tensor_name(index);
             if (std::find(names.begin(), names.end(), out_name) == names.end())
@@ -760,31 +774,53 @@ esp_err_t Model::test()
 
 std::vector<module_info> Model::get_module_info(int repeats)
 {
+    // Whole passes of the plan in execution order with one event between consecutive modules: every
+    // module is timed with the cache state an ordinary run gives it (its input was just written by the
+    // module before, not by an earlier repeat of itself), the per-module times add up to the time of a
+    // pass, and the tensors hold an ordinary pass's results afterwards.
     std::vector<module_info> info;
     if (!m_built)
         return info;
     hipStream_t s = static_cast<hipStream_t>(m_stream);
-    hipEvent_t e0, e1;
-    if (!hip_ok(hipEventCreate(&e0), "hipEventCreate") || !hip_ok(hipEventCreate(&e1), "hipEventCreate"))
-        return info;
     if (repeats < 1)
         repeats = 1;
-    for (auto *module : m_execution_plan) {
-        module->hold_state(m_stream); // timing passes leave no trace in modules that carry data between passes
-        module->forward(m_model_context, RUNTIME_MODE_AUTO); // warm
-        (void)hipEventRecord(e0, s);
-        for (int r = 0; r < repeats; r++)
-            module->forward(m_model_context, RUNTIME_MODE_AUTO);
-        (void)hipEventRecord(e1, s);
-        module->restore_state(m_stream);
-        (void)hipEventSynchronize(e1);
-        float ms = 0.f;
-        (void)hipEventElapsedTime(&ms, e0, e1);
+    const size_t n = m_execution_plan.size();
+    std::vector<hipEvent_t> ev(n + 1, nullptr);
+    bool ok = true;
+    for (auto &e : ev)
+        ok = ok && hip_ok(hipEventCreate(&e), "hipEventCreate");
+    std::vector<double> total_ms(n, 0.0);
+    if (ok) {
+        for (auto *module : m_execution_plan)
+            module->hold_state(m_stream); // timing passes leave no trace in modules that carry data between passes
+        for (int r = -1; r < repeats; r++) { // pass -1 warms up and is not counted
+            (void)hipEventRecord(ev[0], s);
+            for (size_t i = 0; i < n; i++) {
+                m_execution_plan[i]->forward(m_model_context, RUNTIME_MODE_AUTO);
+                (void)hipEventRecord(ev[i + 1], s);
+            }
+            (void)hipEventSynchronize(ev[n]);
+            for (size_t i = 0; i < n && r >= 0; i++) {
+                float ms = 0.f;
+                (void)hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
+                total_ms[i] += ms;
+            }
+        }
+        for (auto *module : m_execution_plan)
+            module->restore_state(m_stream);
+        synchronize();
+    }
+    for (auto &e : ev)
+        if (e)
+            (void)hipEventDestroy(e);
+    if (!ok)
+        return info;
+    for (size_t i = 0; i < n; i++) {
+        dl::module::Module *module = m_execution_plan[i];
         module_info mi;
         mi.name = module->name;
-        const std::string op = m_fbs_model->get_operation_type(module->name);
-        mi.type = op;
-        mi.latency_us = ms * 1000.f / repeats;
+        mi.type = m_fbs_model->get_operation_type(module->name);
+        mi.latency_us = (float)(total_ms[i] * 1000.0 / repeats);
         std::vector<std::vector<int>> in_shapes;
         mi.bytes = 0;
         for (int idx : module->m_inputs_index) {
@@ -801,8 +837,6 @@ std::vector<module_info> Model::get_module_info(int repeats)
         mi.macs = module->get_macs(in_shapes);
         info.push_back(mi);
     }
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
     return info;
 }
 

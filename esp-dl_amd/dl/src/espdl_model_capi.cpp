@@ -282,7 +282,7 @@ int espdl_model_run(espdl_model *m)
     if (!m)
         return -1;
     m->model->run();
-    return 0;
+    return m->model->last_run_failed() ? -2 : 0;
 }
 
 int espdl_model_run_async(espdl_model *m)
@@ -290,7 +290,7 @@ int espdl_model_run_async(espdl_model *m)
     if (!m)
         return -1;
     m->model->run_async();
-    return 0;
+    return m->model->last_run_failed() ? -2 : 0;
 }
 
 int espdl_model_synchronize(espdl_model *m)
@@ -298,7 +298,7 @@ int espdl_model_synchronize(espdl_model *m)
     if (!m)
         return -1;
     m->model->synchronize();
-    return 0;
+    return m->model->last_run_failed() ? -2 : 0;
 }
 
 int espdl_model_enable_graph(espdl_model *m)

@@ -211,13 +211,15 @@ class Model:
 
     def run(self):
         if lib().espdl_model_run(self.h) != 0:
-            raise EspdlModelError("run failed")
+            raise EspdlModelError("run failed: a module rejected its launch or a HIP call failed (see stderr)")
 
     def run_async(self):
-        lib().espdl_model_run_async(self.h)
+        if lib().espdl_model_run_async(self.h) != 0:
+            raise EspdlModelError("run_async failed: a module rejected its launch (see stderr)")
 
     def synchronize(self):
-        lib().espdl_model_synchronize(self.h)
+        if lib().espdl_model_synchronize(self.h) != 0:
+            raise EspdlModelError("the pass failed: a module rejected its launch or a HIP call failed (see stderr)")
 
     def enable_graph(self):
         return lib().espdl_model_enable_graph(self.h) == 0

@@ -675,6 +675,26 @@ def gated_block(seed=0xE5D6):
     return g
 
 
+def activation_modules(seed=0xE5E0):
+    """The activation operators as graph nodes of their own rather than fused into a Conv: Conv (Linear) ->
+    PRelu with a per-channel int8 slope -> Conv (Linear) -> standalone Relu -> Conv -> PRelu whose result
+    is requantized to another exponent -> Add with the Relu branch.  This is how the reference's face /
+    landmark models carry PReLU (esp-dl/dl/module/include/dl_module_prelu.hpp:109-121, dl_module_relu.hpp:65-93)."""
+    g = GraphSpec("activation_modules")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 18, 22, 16], -5)
+    h = b.conv(x, 48, k=3, name="c1")
+    h = b.prelu(h, name="c1_prelu")
+    h = b.conv(h, 32, k=1, name="c2")
+    r = b.relu(h, name="c2_relu")
+    h = b.conv(r, 32, k=3, depthwise=True, name="c3")
+    h = b.prelu(h, name="c3_prelu", alpha_exp=-6, out_exp=g.exponent(h) + 1)
+    r2 = b.requantize(r, g.exponent(h), name="r_align")
+    y = b.add(r2, h, name="join")
+    b.output(y)
+    return g
+
+
 def pooled_embedding(seed=0xE5D7):
     """Conv -> AveragePool -> Conv -> ReduceMean over H x W (axes as an initializer operand) -> Transpose to
     N,C,1,1 -> Reshape [1,-1] (shape as an initializer operand) -> Gemm: the tail of the reference's exported

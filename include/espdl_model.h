@@ -82,6 +82,11 @@ int espdl_graph_add_test_output(espdl_graph *g, const char *name, const int32_t 
  * conv epilogue (7 = all).  The graph must outlive the model. */
 espdl_model *espdl_model_create(espdl_graph *g, int32_t batch, int32_t round_mode, void *stream, int32_t fuse);
 void espdl_model_destroy(espdl_model *m);
+/* Module::forward returns void, as in the reference, so a module whose launch is rejected (an operand
+ * that is not on the device, a shape a kernel refuses) can only log.  The model counts what is logged
+ * during a pass: run / run_async / synchronize return -2 when a module of the current pass logged an
+ * error or a HIP call failed; the tensors of such a pass are not valid results.  enable_graph refuses to
+ * capture a plan with a failing module. */
 int espdl_model_run(espdl_model *m);       /* enqueue + wait */
 int espdl_model_run_async(espdl_model *m); /* enqueue only   */
 int espdl_model_synchronize(espdl_model *m);

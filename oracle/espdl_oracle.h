@@ -35,19 +35,22 @@
  *                                scales every intermediate is exactly representable, so the
  *                                result is fixed by the mathematics: checked exhaustively
  *                                against round-half-up in exact rationals                 PINNED
- *   espdl_oracle_global_avg_pool_s8   float32 mean times a float scale under -ffast-math in the
- *                                reference; the restatement is checked against exact rational
- *                                round-half-up, which fixes every case whose exact value is not
- *                                within float rounding error of a tie; the reference itself
- *                                cannot be built here (every translation unit needs ESP-IDF
- *                                headers that are absent)                   PARITY UNPINNED (near-ties)
+ *   espdl_oracle_global_avg_pool_s8, _avg_pool_s8, _avg_pool_s16   float32-defined in the reference:
+ *                                (DL_SCALE(in) * (1.f / area)) * DL_RESCALE(out), one multiply of float(sum),
+ *                                tool::round.  Every reachable int8 sum for areas 49, 9, 6, 4, 2, 100, 196, 5 (a
+ *                                dense sample plus all tie multiples for int16) x twelve exponent pairs, ties and
+ *                                near-ties included, against the same IEEE float32 sequence replayed operation by
+ *                                operation with numpy scalars, and against round-half-up in exact rationals (no
+ *                                enumerated sum differs between the two).  The reference itself cannot be built
+ *                                here (every translation unit needs ESP-IDF headers that are absent); it is
+ *                                compiled with -ffast-math, which for int8 can only matter on exact ties of areas
+ *                                that are not powers of two, where the order as written is followed   PINNED
  *   espdl_oracle_mul_s8          exhaustive over all int8 operand pairs and shifts -4..14 against round-half-up
  *                                (and the half-even table) of the exact product in rationals        PINNED
- *   espdl_oracle_avg_pool_s8     float32 scale as espdl_oracle_global_avg_pool_s8: exact rational round-half-up away
- *                                from ties; the reference's streaming-model fixtures (S3 and P4 exports with
- *                                embedded outputs) pass through it                  PARITY UNPINNED (near-ties)
- *   espdl_oracle_reduce_mean_s8  float32 as the two above: exact rational mean, round half up, away from ties
- *                                                                                   PARITY UNPINNED (near-ties)
+ *   espdl_oracle_reduce_mean_s8, _s16   ((float(sum) * DL_SCALE(in)) / float(count)) * DL_RESCALE(out): every
+ *                                reachable int8 sum for counts 49, 9, 6, 4, 2, 100, 40, 3 (dense + tie multiples
+ *                                for int16) against the numpy float32 replay and exact rationals, as above; the
+ *                                reference's streaming-model fixtures pass through AveragePool        PINNED
  *   espdl_oracle_slice           equality with numpy basic slicing                                   PINNED
  *   espdl_oracle_softmax_s8      float32: within 2e-6 relative of scipy.special.softmax of the dequantized values;
  *                                the order-sensitive part (the float32 row sum in index order, one IEEE division
@@ -72,11 +75,15 @@
  *   espdl_oracle_div_s16         numpy float32 arithmetic in the same order for each of the three forms (IEEE
  *                                operations, so the order is the whole content), and within one unit of the exact
  *                                rational quotient                                                   PINNED
- *   espdl_oracle_unary_s8, _s16  every function against its closed form in numpy float64 (within one output unit
- *                                everywhere, equal away from rounding ties), the float / double promotions of
- *                                HardSwish and sigmoid against numpy operations of those widths; expf / logf
- *                                are the host libm's, which may differ from the target's in the last bit
- *                                                                       PARITY UNPINNED (libm last-bit, near-ties)
+ *   espdl_oracle_unary_s8, _s16  every table entry (256 / 65536) of every function against the reference's
+ *                                float / double sequence replayed with numpy scalars of the same widths and the
+ *                                host C library's expf / logf / sqrtf, and against the float64 closed form rounded
+ *                                half up on every entry that is not within 4 float32 ulps of a tie.  int8: no entry
+ *                                of a libm-dependent function is that close to a tie, so any C library decides the
+ *                                same table.  int16: 123 to 4012 of 65536 entries per libm-dependent function are
+ *                                (counted in tests/test_oracle_float_pins.py); on those a C library that differs
+ *                                from this host's in the last places of expf / logf could move the entry by one
+ *                                unit, which no restatement can settle             PINNED (int16: to the host libm)
  *   espdl_oracle_reduce_int      numpy max / min / sum over the same axes; the sum followed by the pinned
  *                                shift-round and saturation                                          PINNED
  *   espdl_oracle_pad             equality with numpy.pad (constant / edge / reflect) on random shapes, ranks 1-5,
@@ -84,8 +91,6 @@
  *   espdl_oracle_sub_s8          numpy saturating subtraction                                        PINNED
  *   espdl_oracle_div_s8          as _div_s16 for the three loop forms; the table forms against a table built in
  *                                numpy float32 from the reference's two expressions, entry by entry   PINNED
- *   espdl_oracle_avg_pool_s16, _reduce_mean_s16   as their int8 forms: exact rationals away from ties
- *                                                                                   PARITY UNPINNED (near-ties)
  *   espdl_oracle_concat, _split_slice, _transpose   pure copies: equality with numpy.concatenate /
  *                                numpy.split / numpy.transpose on random shapes           PINNED
  *   espdl_oracle_max_pool        equality with scipy.ndimage.maximum_filter (minimum-value border)

@@ -402,3 +402,51 @@ def test_mobilenetv2_conv_add_fusion(oracle):
     assert mdl.module_count() < plain.module_count()
     mdl.close()
     plain.close()
+
+
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+def test_activation_modules_prelu_relu_nodes(oracle, round_mode):
+    """PRelu and Relu as graph nodes of their own (dl::module::PRelu::forward, dl::module::Relu::forward
+    through dl::Model), every tensor compared; also under HIP-graph replay."""
+    announce(f"model activation_modules round_mode={round_mode}")
+    m, zoo, model, runner = _mods()
+    spec = zoo.activation_modules()
+    assert [n["op_type"] for n in spec.nodes].count("PRelu") == 2 and "Relu" in [n["op_type"] for n in spec.nodes]
+    batch = 5
+    x = spec.make_input(np.random.default_rng(31), batch)
+    import espdl_oracle as oracle_mod
+    want = runner.run(spec, {"input": x}, oracle_mod.ROUND_HALF_EVEN if round_mode else oracle_mod.ROUND_HALF_UP)
+    outs = {k: v for k, v in want.items() if k != "input"}
+    g = model.Graph.from_spec(spec, test_input={"input": x}, test_outputs=outs)
+    mdl = model.Model(g, batch, round_mode=round_mode)
+    assert mdl.test()  # module by module, every tensor
+    mdl.set_input("input", x)
+    assert mdl.enable_graph()
+    for _ in range(2):
+        mdl.run()
+        np.testing.assert_array_equal(mdl.get_tensor(spec.outputs[0]), want[spec.outputs[0]])
+    assert (want["c1_prelu_out"] < 0).any() and (want["c2_relu_out"] == 0).any()
+    mdl.close()
+
+
+def test_failed_forward_is_reported(oracle):
+    """A module whose launch is rejected on the host (a Conv with an activation no kernel fuses) makes
+    run() fail instead of returning stale bytes, and its plan is not captured into a HIP graph."""
+    announce("model run reports a rejected module")
+    m, zoo, model, runner = _mods()
+    spec = zoo.config1_single_conv()
+    spec.nodes[0]["attrs"]["activation"] = "LeakyRelu"
+    mdl = model.Model(model.Graph.from_spec(spec), 1)
+    mdl.set_input("input", spec.make_input(np.random.default_rng(1), 1))
+    with pytest.raises(model.EspdlModelError):
+        mdl.run()
+    assert not mdl.enable_graph()
+    with pytest.raises(model.EspdlModelError):
+        mdl.run()
+    mdl.close()
+    # the same graph with a supported activation runs
+    spec = zoo.config1_single_conv()
+    mdl = model.Model(model.Graph.from_spec(spec), 1)
+    mdl.set_input("input", spec.make_input(np.random.default_rng(1), 1))
+    mdl.run()
+    mdl.close()
