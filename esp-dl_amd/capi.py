@@ -107,7 +107,8 @@ def lib():
         L.espdl_hip_mbconv_out_shape.argtypes = [mp, ctypes.POINTER(i32), ctypes.POINTER(i32)]
         L.espdl_hip_mbconv_s8_supported.argtypes = [mp]
         L.espdl_hip_mbconv_s8.argtypes = [mp, vp, ctypes.POINTER(MbconvWeights), vp, vp, vp]
-        for name in ("mbconv_out_shape", "mbconv_s8_supported", "mbconv_s8"):
+        L.espdl_hip_mbconv_s8_staged.argtypes = L.espdl_hip_mbconv_s8.argtypes
+        for name in ("mbconv_out_shape", "mbconv_s8_supported", "mbconv_s8", "mbconv_s8_staged"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         for name in ("conv_out_shape", "conv2d", "lut_s8", "prelu_s8", "relu_s8", "clip_s8", "add_s8",
                      "global_avg_pool_s8", "requantize_s8", "requantize", "device_cu_count"):
@@ -166,8 +167,9 @@ def conv2d(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 
 
 
 def mbconv_s8(x, expand, dw, project, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), relus=(True, True, False),
-              residual=None, round_mode=ROUND_HALF_UP, out=None, stream=None):
-    """Fused inverted-residual block.  expand / dw / project are (filter, bias, shift) triples of CUDA
+              residual=None, round_mode=ROUND_HALF_UP, out=None, stream=None, staged=False):
+    """Fused inverted-residual block (staged=True: espdl_hip_mbconv_s8_staged, the separate stages with the
+    intermediates in the library's own device array; `out` must then be given, nothing is allocated).  expand / dw / project are (filter, bias, shift) triples of CUDA
     tensors (expand may be None); filters as for conv2d: [E][C], [kH][kW][E], [OC][E]."""
     import torch
     n, h, w, c = x.shape
@@ -185,8 +187,8 @@ def mbconv_s8(x, expand, dw, project, k, stride=(1, 1), dilation=(1, 1), pads=(0
     if out is None:
         out = torch.empty((n, oh.value, ow.value, out_c), dtype=torch.int8, device=x.device)
     wts = MbconvWeights(_p(we), _p(be), _p(se), _p(wd), _p(bd), _p(sd), _p(wp), _p(bp), _p(sp))
-    _check(lib().espdl_hip_mbconv_s8(ctypes.byref(desc), _p(x), ctypes.byref(wts), _p(residual), _p(out),
-                                     _stream(stream)))
+    fn = lib().espdl_hip_mbconv_s8_staged if staged else lib().espdl_hip_mbconv_s8
+    _check(fn(ctypes.byref(desc), _p(x), ctypes.byref(wts), _p(residual), _p(out), _stream(stream)))
     return out
 
 

@@ -10,10 +10,11 @@
 #include <vector>
 
 namespace {
-
 thread_local char g_last_error[256] = "";
+}
 
-int fail(int code, const char *fmt, ...)
+// Records the message espdl_hip_last_error() returns on this thread and hands `code` back.
+int espdl::set_error(int code, const char *fmt, ...)
 {
     va_list ap;
     va_start(ap, fmt);
@@ -21,6 +22,10 @@ int fail(int code, const char *fmt, ...)
     va_end(ap);
     return code;
 }
+
+#define fail(...) espdl::set_error(__VA_ARGS__)
+
+namespace {
 
 int device_status(hipError_t e, const char *what)
 {

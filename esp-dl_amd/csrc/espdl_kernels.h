@@ -6,6 +6,9 @@
 
 namespace espdl {
 
+// Sets the calling thread's espdl_hip_last_error() text; returns `code` (defined in espdl_hip_api.hip).
+int set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
 // Geometry every convolution kernel works from (derived once on the host by the C ABI).
 struct ConvGeom {
     int batch, in_h, in_w, in_c;

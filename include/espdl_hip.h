@@ -360,6 +360,25 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc);
 int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *weights,
                         const int8_t *residual, int8_t *out, void *stream);
 
+/*
+ * The same block as espdl_hip_mbconv_s8, run as its separate stages ([1x1 Conv] -> depthwise Conv ->
+ * 1x1 Conv [+ Add]: espdl_hip_conv2d, espdl_hip_conv2d, espdl_hip_conv2d_add on `stream`) with the two
+ * intermediate activations in device memory that belongs to the library.  It has no counterpart in the
+ * reference; it exists for callers that cannot allocate device memory and whose block shape the
+ * single-launch kernels do not cover (espdl_hip_mbconv_s8_supported() == 0): code under HIP-graph
+ * capture, serving loops, harnesses that forbid hipMalloc.  It allocates nothing and accepts every shape
+ * espdl_hip_conv2d accepts.  Results are bit-identical to espdl_hip_mbconv_s8 and to the separate calls.
+ * The intermediates (batch*in_h*in_w*exp_c bytes when has_expand, plus batch*out_h*out_w*exp_c bytes, each
+ * rounded up to 256) must fit ESPDL_HIP_MBCONV_STAGED_MAX_BYTES, else ESPDL_HIP_ENOTSUP: split the batch.
+ * Every call on a device uses the same array: calls that overlap on one device (two streams, two threads)
+ * race; calls ordered on one stream are safe.  The array stays allocated on every device the library
+ * has been used on until the process ends.
+ */
+#define ESPDL_HIP_MBCONV_STAGED_MAX_BYTES (64u << 20)
+int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *desc, const int8_t *in,
+                               const espdl_hip_mbconv_weights *weights, const int8_t *residual, int8_t *out,
+                               void *stream);
+
 /* Library / device information. */
 const char *espdl_hip_last_error(void);
 const char *espdl_hip_version(void);
