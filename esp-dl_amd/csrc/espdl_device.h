@@ -126,6 +126,34 @@ __device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const 
                                       0x07050301u);
 }
 
+// pack_fast4 followed by the saturating int8 Add of `res` (four packed int8, esp-dl/dl/base/dl_base_add.cpp:34-44).
+// The int16 pairs hold q_sat * 256 + fraction after the saturating convert (and the ReLU max), so adding
+// res * 256 with int16 saturation leaves saturate_int8(q_sat + res) in the high byte: the fraction (0..255)
+// cannot carry across a saturation bound.  Two byte permutes spread `res` into the high bytes.
+template <int MODE>
+__device__ __forceinline__ int pack_fast4_add(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk, int res)
+{
+    int t[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int v = MODE != 0 ? (int)((unsigned)acc[r] << lsh[r]) : acc[r];
+        t[r] = v >> rsh[r];
+        if (MODE == 2) {
+            const bool tie = (int)((unsigned)(t[r] & ~0xff) << rsh[r]) == v;
+            t[r] -= tie ? (t[r] & 0x100) : 0;
+        }
+    }
+    const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
+    const v2s r01 = __builtin_bit_cast(v2s, (int)__builtin_amdgcn_perm(0u, (unsigned)res, 0x010c000cu));
+    const v2s r23 = __builtin_bit_cast(v2s, (int)__builtin_amdgcn_perm(0u, (unsigned)res, 0x030c020cu));
+    v2s p01 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(t[0], t[1]), floor2);
+    v2s p23 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(t[2], t[3]), floor2);
+    p01 = __builtin_elementwise_add_sat(p01, r01);
+    p23 = __builtin_elementwise_add_sat(p23, r23);
+    return (int)__builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, p23), (unsigned)__builtin_bit_cast(int, p01),
+                                      0x07050301u);
+}
+
 // int8 x 4 saturating add of two packed dwords
 __device__ __forceinline__ int sat_add4_s8(int x, int y)
 {

@@ -790,6 +790,8 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
         if (espdl::depthwise_project_s8_supports(g, p.in, pj))
             return 2;
     }
+    if (desc->has_expand && espdl::mbconv_s8_wave_supports(p))
+        return 4;
     if (desc->has_expand) {
         espdl::ConvGeom g;
         espdl::DwProject pj;
@@ -838,6 +840,9 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
                                                                     reinterpret_cast<hipStream_t>(stream)),
                                  "depthwise_project_s8");
     }
+    if (desc->has_expand && espdl::mbconv_s8_wave_supports(p))
+        return device_status(espdl::launch_mbconv_s8_wave(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                             "mbconv_s8_wave");
     if (desc->has_expand) {
         espdl::ConvGeom g;
         espdl::DwProject pj;

@@ -85,6 +85,11 @@ struct MbconvParams {
 bool mbconv_s8_fused_supports(const MbconvParams &p);
 hipError_t launch_mbconv_s8_fused(const MbconvParams &p, int cu_count, hipStream_t stream);
 
+// The same block with one wavefront per output tile and no workgroup barriers (mbconv_s8_wave.hip): 3x3
+// depthwise stage with stride 1 or 2, at most 64 block-input channels and 64 project filters.
+bool mbconv_s8_wave_supports(const MbconvParams &p);
+hipError_t launch_mbconv_s8_wave(const MbconvParams &p, int cu_count, hipStream_t stream);
+
 // Depthwise -> 1x1 project [-> Add] in one launch of the LDS-tile depthwise kernel: the depthwise
 // result never leaves LDS.  Needs at most 256 depthwise channels.
 bool depthwise_project_s8_supports(const ConvGeom &g, const void *in, const DwProject &pj);

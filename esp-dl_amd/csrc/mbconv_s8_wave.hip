@@ -1,0 +1,666 @@
+// Inverted-residual block (1x1 expand conv -> 3x3 depthwise conv -> 1x1 project conv [-> Add]) for int8
+// on gfx950 with ONE WAVEFRONT PER TILE and no workgroup barriers.
+//
+// Every stage computes exactly what the separate operators compute, in the same integer arithmetic,
+// with the int8 result of each stage materialized before the next one reads it:
+//   expand / project  conv2d_11cn + n_wise epilogue (esp-dl/dl/base/dl_base_conv2d.cpp:9-33;
+//                     esp-dl/dl/base/dl_base_activate_buffer.hpp:10-74, 162-212)
+//   depthwise         depthwise_conv2d_33c1 under dwconv_operation_shell's window clipping
+//                     (esp-dl/dl/base/dl_base_depthwise_conv2d.cpp:19-65; esp-dl/dl/base/dl_base.hpp:1852-2102)
+//   Add               saturating int8 add without rescale (esp-dl/dl/base/dl_base_add.cpp:34-44)
+// so a fused block is bit-identical to running Conv, Conv, Conv, Add modules one after the other.
+//
+// Why one wavefront per tile: the block is a chain of small dependent stages (a matrix product, a
+// requantization on the vector ALU, a trip through LDS, the next matrix product ...).  A workgroup that
+// walks the chain with barriers between the stages leaves every pipe idle most of the time.  Here a
+// workgroup IS one wavefront: it owns a th x tw tile of the block's output in one image and runs the
+// whole chain on its own, ordered only by its own LDS accesses; eight to sixteen such wavefronts per
+// compute unit sit at different points of the chain, so the matrix pipe, the vector ALU, LDS and the
+// memory pipeline of the unit are all busy at once.
+//
+// Per tile:
+//   * the (th*s + 2) x (tw*s + 2) patch of the block input is loaded ONCE, straight into the registers
+//     that are operand B of the expand products (lane = patch pixel x 16 input channels), and stays
+//     there for all expanded channels;
+//   * the expanded channels are walked in chunks of 16:
+//       expand     v_mfma_i32_16x16x64_i8 (rows = 16 expanded channels, columns = 16 patch pixels), fused
+//                  shift-round-saturate, zeros for patch pixels outside the image (the depthwise zero
+//                  padding pads the EXPANDED activation), int8 result to LDS as [patch pixel][16 ch];
+//       depthwise  the same instruction with a diagonal operand A whose reduction axis is
+//                  (input row, channel): the four 16-lane groups of a wavefront hold four consecutive
+//                  patch rows, so one set of three operand-B reads (kx = 0, 1, 2) serves TWO output rows
+//                  through two operand-A sets (rows 0-2 and rows 1-3); result to LDS as [pixel][64 ch];
+//     and after every 64 expanded channels the project product accumulates into registers
+//     (rows = 16 project filters, columns = one output row of the tile);
+//   * project epilogue, residual add, stores.
+// Filters, biases and shifts are read from global memory (L2) as they are needed: 16-byte pieces in
+// operand order, no staging.
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <type_traits>
+
+#include "espdl_device.h"
+#include "espdl_kernels.h"
+
+namespace espdl {
+
+namespace {
+
+constexpr int kDws = 80; // LDS pixel stride of the depthwise result: 64 channels + 16 (odd number of 16-byte units)
+
+struct WaveArgs {
+    MbconvParams p;
+    int th, tw, ph, pw;
+    int n_xpt; // pixel tiles of 16 in the patch
+    int tiles_x, tiles_y, n_tiles;
+    int n_sub; // chunks of 16 expanded channels
+    int rt;    // project row tiles of 16 filters
+    int x_vec16, we_vec16;
+    int off_exp, off_dw, off_tab;
+    FastDiv fd_pw, fd_tiles_x, fd_tiles_yx;
+};
+
+// 16 bytes at p + off of which the first `nvalid` exist (nvalid a multiple of 4, possibly <= 0); the rest
+// are zeros.  Branch-free: a piece that does not exist is read from offset 0 of `p` instead (always a valid
+// address) and replaced by zero, so that every lane issues the same loads and the wait counters of loads
+// requested ahead of their use stay exact.  VEC16: p + off is 16-byte aligned whenever nvalid >= 16 and
+// nvalid is then never in 1..15.
+template <bool VEC16>
+__device__ __forceinline__ v4i load16_partial(const int8_t *p, unsigned off, int nvalid)
+{
+    // `p` is the same in every lane and `off` is an unsigned 32-bit byte offset: one scalar base plus one
+    // vector offset per load, no 64-bit address arithmetic on the vector ALU
+    v4i r;
+    if constexpr (VEC16) {
+        const bool ok = nvalid >= 16;
+        r = *reinterpret_cast<const v4i *>(p + (size_t)(ok ? off : 0u));
+        r = ok ? r : v4i{0, 0, 0, 0};
+    } else {
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const bool ok = 4 * d < nvalid;
+            const int v = *reinterpret_cast<const int *>(p + (size_t)(ok ? off + 4u * d : 0u));
+            r[d] = ok ? v : 0;
+        }
+    }
+    return r;
+}
+
+// Orders the LDS accesses of the wavefront's lanes among each other.  LDS executes the instructions of one
+// wavefront in order, so nothing has to be waited for; the compiler must not move accesses across.
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Is the short epilogue (pack_fast4) exact for this channel?  The shift must be in 1..31 and
+// |bias| + 2^(s-1) + mac_bound (the largest magnitude the accumulator can reach) must stay below
+// 2^(31 - max(0, 8 - s)), so that neither the accumulator nor its left-shifted form overflows.
+// mac_bound < 2^30 (checked on the host); everything fits unsigned 32-bit arithmetic.
+__device__ __forceinline__ bool short_ok(int s, int bias, unsigned mac_bound)
+{
+    if (s < 1 || s > 31)
+        return false;
+    const unsigned lim = 1u << (31 - max(0, 8 - s));
+    const unsigned t = mac_bound + (1u << (s - 1));
+    const unsigned ub = bias < 0 ? 0u - (unsigned)bias : (unsigned)bias;
+    return t < lim && ub < lim - t;
+}
+
+// Requantization constants of four consecutive channels of one stage, and which epilogue the whole
+// wavefront takes for them: pack_fast4 mode 0 (every shift >= 8), 1 (some shift below 8), 2 (half-even),
+// or -1 for the general shift_and_round restatement (a shift outside 1..31, or an accumulator that could
+// overflow the short form).
+struct StageConsts {
+    v4i init, rsh, lsh;
+    int mode;
+};
+
+// b, sh: bias and shift of the lane's four channels (channels that do not exist: 0 and 8).
+__device__ __forceinline__ StageConsts stage_consts(const v4i &b, const v4i &sh, unsigned mac_bound, bool half_even)
+{
+    StageConsts c;
+    bool ok = true;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+        ok = ok && short_ok(sh[r], b[r], mac_bound);
+    if (__all(ok)) {
+        bool any_lsh = false;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            c.init[r] = b[r] + (1 << (sh[r] - 1));
+            c.rsh[r] = max(0, sh[r] - 8);
+            c.lsh[r] = max(0, 8 - sh[r]);
+            any_lsh = any_lsh || sh[r] < 8;
+        }
+        c.mode = half_even ? 2 : (__any(any_lsh) ? 1 : 0);
+    } else {
+        c.init = b;
+        c.rsh = sh;
+        c.lsh = v4i{0, 0, 0, 0};
+        c.mode = -1;
+    }
+    return c;
+}
+
+// Per-channel constants of a stage for every channel of the block, built once per tile in LDS by all lanes
+// (channel = lane + 64 i) as [init | right shift | left shift][n_ch], in the form the stage's epilogue
+// `mode` wants (see StageConsts); returns that mode, one for the whole stage.
+__device__ __forceinline__ int build_stage_table(int *tab, const int32_t *bias, const int32_t *shift, int n_shift,
+                                                 int n_ch, unsigned mac_bound, bool half_even, int lane)
+{
+    bool ok = true, any_lsh = false;
+    for (int c = lane; c < n_ch; c += 64) {
+        const int b = bias != nullptr ? bias[c] : 0;
+        const int sh = shift[n_shift == 1 ? 0 : c];
+        ok = ok && short_ok(sh, b, mac_bound);
+        any_lsh = any_lsh || sh < 8;
+        tab[c] = b;
+        tab[n_ch + c] = sh;
+    }
+    const bool fast = __all(ok) != 0;
+    const int mode = !fast ? -1 : (half_even ? 2 : (__any(any_lsh) ? 1 : 0));
+    for (int c = lane; c < n_ch; c += 64) { // each lane revisits the channels it wrote
+        const int b = tab[c], sh = tab[n_ch + c];
+        if (fast) {
+            tab[c] = b + (1 << (sh - 1));
+            tab[n_ch + c] = max(0, sh - 8);
+            tab[2 * n_ch + c] = max(0, 8 - sh);
+        } else {
+            tab[2 * n_ch + c] = 0;
+        }
+    }
+    return mode;
+}
+
+__device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch, int ch, int mode)
+{
+    StageConsts c;
+    c.init = *reinterpret_cast<const v4i *>(tab + ch);
+    c.rsh = *reinterpret_cast<const v4i *>(tab + n_ch + ch);
+    c.lsh = v4i{0, 0, 0, 0};
+    if (mode == 1 || mode == 2)
+        c.lsh = *reinterpret_cast<const v4i *>(tab + 2 * n_ch + ch);
+    c.mode = mode;
+    return c;
+}
+
+// Bias and shift of four consecutive channels starting at `ch` (a multiple of 4), straight from memory,
+// branch-free (see load16_partial): channels that do not exist give bias 0 and shift 8.
+__device__ __forceinline__ void load_bias_shift(const int32_t *bias, const int32_t *shift, int n_shift, int ch, int n_ch,
+                                                v4i &b, v4i &sh)
+{
+    const bool exists = ch < n_ch; // channel counts are multiples of 4: all four exist or none
+    const int32_t *bp = bias != nullptr ? bias : shift;
+    const int cb = (exists && bias != nullptr) ? ch : 0;
+    const int cs = (exists && n_shift != 1) ? ch : 0;
+    const int step = n_shift != 1 ? 1 : 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int bv = bp[cb + (bias != nullptr ? r : 0)];
+        const int sv = shift[cs + step * r];
+        b[r] = (exists && bias != nullptr) ? bv : 0;
+        sh[r] = exists ? sv : 8;
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ int wave_pack(const v4i &acc, const StageConsts &c, int floor_pk, bool relu, bool half_even)
+{
+    if constexpr (MODE >= 0) {
+        return pack_fast4<MODE>(acc, c.lsh, c.rsh, floor_pk);
+    } else {
+        int q[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            q[r] = requant_s8(acc[r], c.rsh[r], relu, half_even);
+        return pack4_s8(q[0], q[1], q[2], q[3]);
+    }
+}
+
+// Expand stage of one chunk of 16 channels: every patch pixel tile through one MFMA and the epilogue, four
+// tiles at a time so that four independent MFMA -> requantize -> store chains are in flight (tiles past
+// n_xpt inside the last group of four have zero operands and a zero mask and land in slack).
+template <int MODE, int NXPT, bool EXACT>
+__device__ __forceinline__ void expand_chunk(const v4i (&xb)[NXPT], int n_xpt, unsigned xmask, const v4i &aop,
+                                             const StageConsts &c, int floor_pk, bool relu, bool half_even,
+                                             unsigned char *dst /* exp_l + col * 16 + 4 * quad */)
+{
+#pragma unroll
+    for (int g0 = 0; g0 < NXPT; g0 += 4) {
+        if (EXACT || g0 < n_xpt) { // uniform
+            v4i acc[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (g0 + j < NXPT)
+                    acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, xb[g0 + j], c.init, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (g0 + j < NXPT) {
+                    int word = wave_pack<MODE>(acc[j], c, floor_pk, relu, half_even);
+                    word &= __builtin_amdgcn_sbfe((int)xmask, g0 + j, 1); // all ones or zero
+                    *reinterpret_cast<int *>(dst + (g0 + j) * 256) = word;
+                }
+            }
+        }
+    }
+}
+
+// Depthwise stage of one chunk of 16 channels.  S == 1: output rows in pairs, four patch rows per read.
+template <int MODE, int PT, int S, bool EXACT>
+__device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_l + (quad * pw + S * col) * 16 */,
+                                                int th, int pw, const v4i (&a0)[3], const v4i (&a1)[3],
+                                                const StageConsts &c, int floor_pk, bool relu, bool half_even,
+                                                unsigned char *dst /* dw_l + col * kDws + 16 * (sub & 3) + 4 * quad */)
+{
+    if constexpr (S == 1) {
+#pragma unroll
+        for (int j = 0; j < (PT + 1) / 2; j++) {
+            if (EXACT || 2 * j < th) { // uniform
+                const unsigned char *s = src + 2 * j * pw * 16;
+                const v4i b0 = *reinterpret_cast<const v4i *>(s);
+                const v4i b1 = *reinterpret_cast<const v4i *>(s + 16);
+                const v4i b2 = *reinterpret_cast<const v4i *>(s + 32);
+                v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b0, c.init, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b1, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[2], b2, acc, 0, 0, 0);
+                *reinterpret_cast<int *>(dst + (2 * j) * 16 * kDws) = wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+                if (EXACT ? 2 * j + 1 < PT : 2 * j + 1 < th) {
+                    v4i acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[0], b0, c.init, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[1], b1, acc1, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[2], b2, acc1, 0, 0, 0);
+                    *reinterpret_cast<int *>(dst + (2 * j + 1) * 16 * kDws) =
+                        wave_pack<MODE>(acc1, c, floor_pk, relu, half_even);
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < PT; t++) {
+            if (EXACT || t < th) { // uniform
+                const unsigned char *s = src + S * t * pw * 16;
+                const v4i b0 = *reinterpret_cast<const v4i *>(s);
+                const v4i b1 = *reinterpret_cast<const v4i *>(s + 16);
+                const v4i b2 = *reinterpret_cast<const v4i *>(s + 32);
+                v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b0, c.init, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b1, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[2], b2, acc, 0, 0, 0);
+                *reinterpret_cast<int *>(dst + t * 16 * kDws) = wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+            }
+        }
+    }
+}
+
+// One dword of a diagonal operand A: weight byte `w` of channel row i sits at byte i of the lane's 16.
+__device__ __forceinline__ v4i diag_operand(int w, int i)
+{
+    const int d = (w & 0xff) << (8 * (i & 3));
+    const int sel = i >> 2;
+    return v4i{sel == 0 ? d : 0, sel == 1 ? d : 0, sel == 2 ? d : 0, sel == 3 ? d : 0};
+}
+
+// EXACT: the tile plan is exactly (NXPT pixel tiles, RT project row tiles, PT rows): no run-time guards in
+// the stage loops, so each stage of a chunk is one straight-line block the scheduler can interleave.  Rows
+// of a ragged last tile that do not exist are computed from whatever the patch area holds and never stored.
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT>
+__global__ __launch_bounds__(64) void mbconv_s8_wave_kernel(const WaveArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const MbconvParams &p = a.p;
+    const int lane = threadIdx.x & 63, col = lane & 15, quad = lane >> 4;
+    unsigned char *exp_l = smem + a.off_exp;
+    unsigned char *dw_l = smem + a.off_dw;
+    int *tab_e = reinterpret_cast<int *>(smem + a.off_tab);
+    int *tab_d = tab_e + 3 * a.p.exp_c;
+
+    // tile of this wavefront; consecutive tiles of an image stay on one XCD (its L2 holds the shared halo rows)
+    int tile = blockIdx.x;
+    if ((gridDim.x & 7u) == 0) {
+        const int per = gridDim.x >> 3;
+        tile = (int)(blockIdx.x & 7u) * per + (int)(blockIdx.x >> 3);
+    }
+    const unsigned n = fastdiv((unsigned)tile, a.fd_tiles_yx);
+    const unsigned rem = (unsigned)tile - n * a.fd_tiles_yx.d;
+    const unsigned ty = fastdiv(rem, a.fd_tiles_x);
+    const int oy0 = (int)ty * a.th, ox0 = (int)(rem - ty * a.fd_tiles_x.d) * a.tw;
+    const int iy0 = oy0 * S - p.pad_top, ix0 = ox0 * S - p.pad_left;
+    const int th_real = min(a.th, p.out_h - oy0); // rows of this tile that exist
+    const int th = EXACT ? PT : th_real;
+    const int n_xpt = EXACT ? NXPT : a.n_xpt;
+    const int n_rt = EXACT ? RT : a.rt;
+
+    // block-input patch -> operand B registers of the expand stage; xmask: patch pixels inside the image
+    const int c0 = p.in_c;
+    v4i xb[NXPT];
+    unsigned xmask = 0;
+    {
+        const int8_t *img = p.in + (long long)n * p.in_h * p.in_w * c0;
+#pragma unroll
+        for (int pt = 0; pt < NXPT; pt++) {
+            xb[pt] = v4i{0, 0, 0, 0};
+            if (pt < n_xpt) { // uniform
+                const unsigned pp = (unsigned)(pt * 16 + col);
+                const unsigned prow = fastdiv(pp, a.fd_pw);
+                const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
+                const bool valid = (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
+                xmask |= valid ? 1u << pt : 0u;
+                xb[pt] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
+                                               valid ? c0 - 16 * quad : 0);
+            }
+        }
+    }
+
+    v4i accp[RT][PT];
+#pragma unroll
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < PT; t++)
+            accp[r][t] = v4i{0, 0, 0, 0};
+
+    const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
+    const int floor_d = p.relu_dw ? 0 : (int)0x80008000u;
+    const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
+    unsigned char *exp_dst = exp_l + col * 16 + 4 * quad;
+    const unsigned char *exp_src = exp_l + (quad * a.pw + S * col) * 16;
+
+    const int mode_e = build_stage_table(tab_e, p.b_expand, p.s_expand, p.n_s_expand, p.exp_c, bound_e, HE, lane);
+    const int mode_d = build_stage_table(tab_d, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_d, HE, lane);
+    wave_lds_sync();
+
+    // Filters of a chunk are requested one chunk ahead (ChunkW), the project filters of a group of four
+    // chunks at the start of the group: their latency hides behind the chunk in between.
+    struct ChunkW {
+        v4i aop;
+        int wd0[3], wd1[3];
+    };
+    auto load_chunk = [&](int sub) {
+        ChunkW w;
+        const int ch0 = 16 * sub;
+        w.aop = load16_partial<VEC16>(p.w_expand, (unsigned)((ch0 + col) * c0 + 16 * quad), c0 - 16 * quad);
+        const unsigned wd = (unsigned)(ch0 + col);
+#pragma unroll
+        for (int kx = 0; kx < 3; kx++) {
+            const int v0 = (int)p.w_dw[(size_t)(wd + (unsigned)((min(quad, 2) * 3 + kx) * p.exp_c))];
+            w.wd0[kx] = quad < 3 ? v0 : 0;
+            w.wd1[kx] = 0;
+            if constexpr (S == 1) {
+                const int v1 = (int)p.w_dw[(size_t)(wd + (unsigned)((max(quad - 1, 0) * 3 + kx) * p.exp_c))];
+                w.wd1[kx] = quad >= 1 ? v1 : 0;
+            }
+        }
+        return w;
+    };
+    v4i ap[RT];
+    auto load_project = [&](int sub) {
+        const int kc = (sub & ~3) * 16;
+        const int nk = p.exp_c - kc - 16 * quad; // valid bytes of this lane's 16 k positions
+#pragma unroll
+        for (int r = 0; r < RT; r++) {
+            ap[r] = load16_partial<true>(p.w_project, (unsigned)((16 * r + col) * p.exp_c + kc + 16 * quad),
+                                         (r < n_rt && 16 * r + col < p.out_c) ? nk : 0);
+        }
+    };
+
+    ChunkW cur = load_chunk(0);
+    for (int sub = 0; sub < a.n_sub; sub++) {
+        if ((sub & 3) == 0)
+            load_project(sub);
+        const ChunkW nxt = load_chunk(min(sub + 1, a.n_sub - 1));
+        // ---- expand: 16 channels x every patch pixel
+        {
+            const StageConsts ce = read_stage_table(tab_e, p.exp_c, 16 * sub + 4 * quad, mode_e);
+            if (ce.mode == 0)
+                expand_chunk<0, NXPT, EXACT>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+            else if (ce.mode == 1)
+                expand_chunk<1, NXPT, EXACT>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+            else if (ce.mode == 2)
+                expand_chunk<2, NXPT, EXACT>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+            else
+                expand_chunk<-1, NXPT, EXACT>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+        }
+        wave_lds_sync();
+
+        // ---- depthwise: diagonal operands for patch rows quad (a0) and quad - 1 (a1)
+        {
+            v4i a0[3], a1[3];
+#pragma unroll
+            for (int kx = 0; kx < 3; kx++) {
+                a0[kx] = diag_operand(cur.wd0[kx], col);
+                a1[kx] = diag_operand(cur.wd1[kx], col);
+            }
+            const StageConsts cd = read_stage_table(tab_d, p.exp_c, 16 * sub + 4 * quad, mode_d);
+            unsigned char *dst = dw_l + col * kDws + 16 * (sub & 3) + 4 * quad;
+            if (cd.mode == 0)
+                depthwise_chunk<0, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+            else if (cd.mode == 1)
+                depthwise_chunk<1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+            else if (cd.mode == 2)
+                depthwise_chunk<2, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+            else
+                depthwise_chunk<-1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+        }
+        wave_lds_sync();
+
+        // ---- project: accumulate over the 64 (or last few) expanded channels gathered so far
+        if ((sub & 3) == 3 || sub == a.n_sub - 1) {
+            const unsigned char *bsrc = dw_l + col * kDws + 16 * quad;
+#pragma unroll
+            for (int t = 0; t < PT; t++) {
+                if (EXACT || t < th) { // uniform
+                    const v4i b = *reinterpret_cast<const v4i *>(bsrc + t * 16 * kDws);
+#pragma unroll
+                    for (int r = 0; r < RT; r++)
+                        if (EXACT || r < n_rt) // uniform
+                            accp[r][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ap[r], b, accp[r][t], 0, 0, 0);
+                }
+            }
+            wave_lds_sync();
+        }
+        cur = nxt;
+    }
+
+    // ---- project epilogue, residual Add, stores: lane = output pixel (oy0 + t, ox0 + col) x 4 filters
+    const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
+    const unsigned bound_p = (unsigned)p.exp_c * 16384u;
+    const int ox = ox0 + col;
+    const bool col_ok = col < a.tw && ox < p.out_w;
+    const long long img_off = (long long)n * p.out_h * p.out_w * p.out_c;
+    const int8_t *res_img = p.residual != nullptr ? p.residual + img_off : nullptr;
+    int8_t *out_img = p.out + img_off;
+#pragma unroll
+    for (int r = 0; r < RT; r++) {
+        if (r < n_rt) { // uniform
+            const int c = 16 * r + 4 * quad;
+            v4i bp, sp;
+            load_bias_shift(p.b_project, p.s_project, p.n_s_project, c, p.out_c, bp, sp);
+            const StageConsts cp = stage_consts(bp, sp, bound_p, HE);
+            const bool live = col_ok && c < p.out_c;
+            const unsigned off0 = (unsigned)((oy0 * p.out_w + ox) * p.out_c + c);
+            auto rows = [&](auto mode_tag) {
+                constexpr int MODE = decltype(mode_tag)::value;
+#pragma unroll
+                for (int t = 0; t < PT; t++) {
+                    if (t < th_real) { // uniform
+                        v4i acc = accp[r][t];
+#pragma unroll
+                        for (int k = 0; k < 4; k++)
+                            acc[k] += cp.init[k];
+                        const unsigned off = off0 + (unsigned)(t * p.out_w * p.out_c);
+                        int word;
+                        if (res_img != nullptr) { // uniform
+                            const int rv = *reinterpret_cast<const int *>(res_img + (size_t)(live ? off : 0u));
+                            if constexpr (MODE >= 0)
+                                word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, rv);
+                            else
+                                word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), rv);
+                        } else {
+                            word = wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE);
+                        }
+                        if (live)
+                            *reinterpret_cast<int *>(out_img + (size_t)off) = word;
+                    }
+                }
+            };
+            if (cp.mode == 0)
+                rows(std::integral_constant<int, 0>{});
+            else if (cp.mode == 1)
+                rows(std::integral_constant<int, 1>{});
+            else if (cp.mode == 2)
+                rows(std::integral_constant<int, 2>{});
+            else
+                rows(std::integral_constant<int, -1>{});
+        }
+    }
+}
+
+struct WavePlan {
+    bool ok;
+    WaveArgs a;
+    size_t lds;
+    int nxpt_max, rt_max;
+};
+
+constexpr int kPtMax = 8;
+
+WavePlan wave_plan(const MbconvParams &p)
+{
+    WavePlan plan;
+    plan.ok = false;
+    if (p.w_expand == nullptr || p.k_h != 3 || p.k_w != 3 || p.dil_h != 1 || p.dil_w != 1 || p.stride_h != p.stride_w ||
+        (p.stride_h != 1 && p.stride_h != 2))
+        return plan;
+    if (p.in_c % 4 != 0 || p.in_c > 64 || p.exp_c % 16 != 0 || p.out_c % 4 != 0 || p.out_c > 64)
+        return plan;
+    if ((long long)p.in_h * p.in_w * p.in_c >= (1ll << 30) || (long long)p.out_h * p.out_w * p.out_c >= (1ll << 30) ||
+        p.exp_c >= 65536)
+        return plan;
+    const int s = p.stride_h;
+    WaveArgs a = {};
+    a.p = p;
+    // columns: the fewest column tiles, then the narrowest tile that gives them (less halo to expand)
+    const int n_cols = (p.out_w + 15) / 16;
+    a.tw = (p.out_w + n_cols - 1) / n_cols;
+    a.pw = (a.tw - 1) * s + 3;
+    a.tiles_x = n_cols;
+    // rows: cheapest total of expand tiles (x 1.5: MFMA + the longer epilogue) and depthwise MFMAs
+    const int nxpt_limit = 17;
+    double best = 1e30;
+    a.th = 0;
+    for (int th = 1; th <= kPtMax; th++) {
+        const int ph = (th - 1) * s + 3;
+        const int n_xpt = (ph * a.pw + 15) / 16;
+        if (n_xpt > nxpt_limit)
+            break;
+        const int tiles_y = (p.out_h + th - 1) / th;
+        const double cost = (double)tiles_y * (1.5 * n_xpt + 3.0 * th + 2.0);
+        if (cost < best) {
+            best = cost;
+            a.th = th;
+        }
+    }
+    if (a.th == 0)
+        return plan;
+    a.ph = (a.th - 1) * s + 3;
+    a.n_xpt = (a.ph * a.pw + 15) / 16;
+    a.tiles_y = (p.out_h + a.th - 1) / a.th;
+    a.n_sub = p.exp_c / 16;
+    a.rt = (p.out_c + 15) / 16;
+    a.x_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.in) & 15) == 0) ? 1 : 0;
+    a.we_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.w_expand) & 15) == 0) ? 1 : 0;
+    // LDS: expanded patch of one chunk (16 bytes per pixel; the depthwise reads run up to three rows and a
+    // few pixels past the patch, into products with zero weights or into discarded columns) and the
+    // depthwise result of 64 channels
+    const int exp_px = std::max(((a.n_xpt + 3) & ~3) * 16, (a.ph + 3) * a.pw + 64);
+    a.off_exp = 0;
+    a.off_dw = exp_px * 16;
+    a.off_tab = a.off_dw + kPtMax * 16 * kDws;
+    plan.lds = (size_t)a.off_tab + (size_t)p.exp_c * 24; // two stages x [init | rsh | lsh] x int32
+    if (plan.lds > 40 * 1024)
+        return plan;
+    a.fd_pw = make_fastdiv((unsigned)a.pw);
+    a.fd_tiles_x = make_fastdiv((unsigned)a.tiles_x);
+    a.fd_tiles_yx = make_fastdiv((unsigned)(a.tiles_y * a.tiles_x));
+    plan.a = a;
+    plan.nxpt_max = a.n_xpt <= 10 ? 10 : 17;
+    plan.rt_max = a.rt <= 2 ? 2 : 4;
+    plan.ok = true;
+    return plan;
+}
+
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT>
+hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
+{
+    const WaveArgs &a = plan.a;
+    hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT>), dim3((unsigned)a.n_tiles), dim3(64),
+                       plan.lds, stream, a);
+    return hipGetLastError();
+}
+
+// Guarded builds that take any plan within (17 pixel tiles, 4 row tiles, 8 rows).
+template <int S, bool HE>
+hipError_t launch_generic(const WavePlan &plan, hipStream_t stream)
+{
+    return (plan.a.x_vec16 && plan.a.we_vec16) ? launch_one<17, 4, kPtMax, S, HE, true, false>(plan, stream)
+                                               : launch_one<17, 4, kPtMax, S, HE, false, false>(plan, stream);
+}
+
+hipError_t launch_planned(const WavePlan &plan, hipStream_t stream)
+{
+    const WaveArgs &a = plan.a;
+    const bool vec16 = a.x_vec16 && a.we_vec16;
+    const int s = a.p.stride_h;
+    if (!a.p.half_even) {
+        // guard-free builds for the tile plans of MobileNetV2-style blocks (round half up)
+        const auto is = [&](int nxpt, int rt, int th, int stride, bool v) {
+            return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v;
+        };
+        if (is(17, 2, 4, 2, true))
+            return launch_one<17, 2, 4, 2, false, true, true>(plan, stream);
+        if (is(17, 2, 4, 2, false))
+            return launch_one<17, 2, 4, 2, false, false, true>(plan, stream);
+        if (is(10, 2, 8, 1, false))
+            return launch_one<10, 2, 8, 1, false, false, true>(plan, stream);
+        if (is(10, 2, 8, 1, true))
+            return launch_one<10, 2, 8, 1, false, true, true>(plan, stream);
+        if (is(9, 2, 7, 1, true))
+            return launch_one<9, 2, 7, 1, false, true, true>(plan, stream);
+        if (is(13, 4, 3, 2, true))
+            return launch_one<13, 4, 3, 2, false, true, true>(plan, stream);
+        if (is(9, 4, 7, 1, true))
+            return launch_one<9, 4, 7, 1, false, true, true>(plan, stream);
+        return s == 1 ? launch_generic<1, false>(plan, stream) : launch_generic<2, false>(plan, stream);
+    }
+    return s == 1 ? launch_generic<1, true>(plan, stream) : launch_generic<2, true>(plan, stream);
+}
+
+} // namespace
+
+bool mbconv_s8_wave_supports(const MbconvParams &p)
+{
+    return wave_plan(p).ok;
+}
+
+hipError_t launch_mbconv_s8_wave(const MbconvParams &p, int cu_count, hipStream_t stream)
+{
+    (void)cu_count;
+    if ((long long)p.batch * p.out_h * p.out_w == 0)
+        return hipSuccess;
+    WavePlan plan = wave_plan(p);
+    if (!plan.ok)
+        return hipErrorInvalidValue;
+    const long long tiles = (long long)p.batch * plan.a.tiles_y * plan.a.tiles_x;
+    if (tiles > 0x7fffffff)
+        return hipErrorInvalidValue;
+    plan.a.n_tiles = (int)tiles;
+    static const bool trace = getenv("ESPDL_HIP_TRACE") != nullptr;
+    if (trace)
+        fprintf(stderr, "mbconv_s8_wave: %dx%d in %d exp %d out %d s%d tile %dx%d patch %dx%d n_xpt %d rt %d lds %zu tiles %lld\n",
+                p.in_h, p.in_w, p.in_c, p.exp_c, p.out_c, p.stride_h, plan.a.th, plan.a.tw, plan.a.ph, plan.a.pw,
+                plan.a.n_xpt, plan.a.rt, plan.lds, tiles);
+    return launch_planned(plan, stream);
+}
+
+} // namespace espdl
