@@ -46,6 +46,10 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
 def kernel_family(info, spec_nodes):
     """Map a module to the kernel that runs it."""
     node = spec_nodes.get(info["name"])
+    if info["type"] == "Conv>DepthwiseConv>Conv":
+        return "mbconv_s8"  # expand + depthwise + project (+ Add) in one launch
+    if info["type"] == "DepthwiseConv>Conv":
+        return "depthwise_s8"  # depthwise + project (+ Add) in one launch of the depthwise kernel
     if info["type"] in ("Gemm", "MatMul"):
         return "conv2d_s8"
     if info["type"] == "Conv":
@@ -223,7 +227,7 @@ def main():
     dom = max(kernels, key=lambda k: kernels[k]["us_per_step"])
     kd = kernels[dom]
     # time per family comes from whole passes in plan order, so the family times add up to a step
-    if dom in ("conv2d_s8",) and kd["ops_per_byte"] > MACHINE_BALANCE:
+    if dom in ("conv2d_s8", "mbconv_s8") and kd["ops_per_byte"] > MACHINE_BALANCE:
         roofline = {"kernel": dom, "bound": "mfma", "achieved": kd["TOPs"], "peak": PEAK_INT8_TOPS,
                     "unit": "TOP/s", "frac": kd["mfma_frac"], "traffic": None}
     else:

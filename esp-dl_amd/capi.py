@@ -108,7 +108,8 @@ def lib():
         L.espdl_hip_mbconv_s8_supported.argtypes = [mp]
         L.espdl_hip_mbconv_s8.argtypes = [mp, vp, ctypes.POINTER(MbconvWeights), vp, vp, vp]
         L.espdl_hip_mbconv_s8_staged.argtypes = L.espdl_hip_mbconv_s8.argtypes
-        for name in ("mbconv_out_shape", "mbconv_s8_supported", "mbconv_s8", "mbconv_s8_staged"):
+        L.espdl_hip_mbconv_s8_preferred.argtypes = [mp]
+        for name in ("mbconv_out_shape", "mbconv_s8_supported", "mbconv_s8_preferred", "mbconv_s8", "mbconv_s8_staged"):
             getattr(L, "espdl_hip_" + name).restype = ctypes.c_int
         for name in ("conv_out_shape", "conv2d", "lut_s8", "prelu_s8", "relu_s8", "clip_s8", "add_s8",
                      "global_avg_pool_s8", "requantize_s8", "requantize", "device_cu_count"):

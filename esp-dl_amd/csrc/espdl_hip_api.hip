@@ -790,6 +790,10 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
         if (espdl::depthwise_project_s8_supports(g, p.in, pj))
             return 2;
     }
+    if (desc->has_expand && desc->in_h >= 28 && espdl::mbconv_s8_wave_supports(p))
+        return 4;
+    if (desc->has_expand && espdl::mbconv_s8_group_supports(p))
+        return 5;
     if (desc->has_expand && espdl::mbconv_s8_wave_supports(p))
         return 4;
     if (desc->has_expand) {
@@ -801,6 +805,28 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
             return 3;
     }
     return espdl::mbconv_s8_fused_supports(p) ? 1 : 0;
+}
+
+int espdl_hip_mbconv_s8_preferred(const espdl_hip_mbconv_desc *desc)
+{
+    const int kind = espdl_hip_mbconv_s8_supported(desc);
+    if (kind == 2)
+        return 1;
+    if (kind == 5) // a workgroup per tile of a small image: at least one workgroup per compute unit
+        return (long long)desc->batch >= (cu_count_cached() > 0 ? cu_count_cached() : 256) ? 1 : 0;
+    if (kind != 4)
+        return 0;
+    // one wavefront per tile: it needs several tiles per SIMD to keep the pipes busy, and at small images
+    // the separate kernels (which also split the channels) are as fast
+    espdl::MbconvParams p = {};
+    if (mbconv_geometry(desc, &p) != ESPDL_HIP_OK)
+        return 0;
+    static const int8_t *const aligned = reinterpret_cast<const int8_t *>(uintptr_t(256));
+    p.in = aligned;
+    p.w_expand = aligned;
+    const long long tiles = espdl::mbconv_s8_wave_tiles(p);
+    const int cus = cu_count_cached() > 0 ? cu_count_cached() : 256;
+    return (desc->in_h >= 28 && desc->in_w >= 28 && tiles >= 4ll * cus) ? 1 : 0;
 }
 
 int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *w,
@@ -840,6 +866,9 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
                                                                     reinterpret_cast<hipStream_t>(stream)),
                                  "depthwise_project_s8");
     }
+    if (desc->has_expand && !(desc->in_h >= 28 && espdl::mbconv_s8_wave_supports(p)) && espdl::mbconv_s8_group_supports(p))
+        return device_status(espdl::launch_mbconv_s8_group(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                             "mbconv_s8_group");
     if (desc->has_expand && espdl::mbconv_s8_wave_supports(p))
         return device_status(espdl::launch_mbconv_s8_wave(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
                              "mbconv_s8_wave");

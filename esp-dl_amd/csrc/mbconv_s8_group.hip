@@ -1,0 +1,438 @@
+// Inverted-residual block (1x1 expand conv -> 3x3 depthwise conv -> 1x1 project conv [-> Add]) for int8
+// on gfx950 at SMALL spatial sizes (14 x 14, 7 x 7 images with hundreds of expanded channels), where a
+// batch has too few output tiles to give every SIMD a tile of its own: a workgroup of eight wavefronts
+// shares one tile and splits the EXPANDED CHANNELS instead.
+//
+// The stages compute exactly what the separate operators compute (see mbconv_s8_stages.h for the reference
+// functions), with the int8 result of every stage materialized before the next one reads it, so the block
+// is bit-identical to running Conv, Conv, Conv, Add modules one after the other.
+//
+// Per tile (th x tw output pixels of one image, tw = whole image width):
+//   phase 0  all lanes build the per-channel requantization tables of the expand and depthwise stages in
+//            LDS; every wavefront loads the block-input patch of the tile into the registers that are
+//            operand B of its expand products (lane = patch pixel x 16 input channels per k step);
+//   phase 1  wavefront w takes the chunks of 16 expanded channels w, w + 8, ... and, on its own (no barrier,
+//            private LDS area), runs expand -> depthwise for them as the one-wavefront-per-tile kernel does;
+//            the depthwise result goes to an LDS tile [pixel][all expanded channels] shared by the group;
+//   barrier
+//   phase 2  the project product: (16 filters x 16 pixels) accumulator tiles are dealt to the wavefronts,
+//            operand B straight from the shared depthwise tile, operand A straight from the filter in
+//            global memory (L2); epilogue, residual add, stores.
+// Two barriers per tile in all; between them eight independent instruction streams per workgroup keep the
+// matrix pipe, the vector ALU and LDS busy.
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <type_traits>
+
+#include "mbconv_s8_stages.h"
+
+namespace espdl {
+
+namespace {
+
+using namespace mbstage;
+
+constexpr int kGroupWaves = 8;
+constexpr int kGroupThreads = 64 * kGroupWaves;
+constexpr int kMaxT = 7; // project pixel tiles per wavefront and row tile
+
+struct GroupArgs {
+    MbconvParams p;
+    int th, tw, ph, pw;
+    int twp;   // pixel slots per output row in the shared depthwise tile: 8 or 16
+    int n_xpt; // pixel tiles of 16 in the patch
+    int kse;   // expand k steps of 64 block-input channels
+    int tiles_y, n_tiles;
+    int n_sub; // chunks of 16 expanded channels
+    int rt;    // project row tiles of 16 filters
+    int npt;   // project pixel tiles of 16 slots
+    int ds;    // LDS pixel stride of the shared depthwise tile, bytes
+    int exp_bytes; // private expand area per wavefront
+    int off_tab, off_exp, off_dw;
+    FastDiv fd_pw, fd_tiles_y, fd_npt;
+};
+
+// EXACT: the plan is exactly (NXPT patch pixel tiles, KSE k steps, PT rows): no guards in the stage loops.
+template <int NXPT, int KSE, int PT, int S, bool HE, bool EXACT>
+__global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mbconv_s8_group_kernel(const GroupArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const MbconvParams &p = a.p;
+    const int tid = threadIdx.x, lane = tid & 63, col = lane & 15, quad = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int *tab_e = reinterpret_cast<int *>(smem + a.off_tab);
+    int *tab_d = tab_e + 3 * p.exp_c;
+    unsigned char *exp_l = smem + a.off_exp + wave * a.exp_bytes;
+    unsigned char *dw_l = smem + a.off_dw;
+
+    int tile = blockIdx.x;
+    if ((gridDim.x & 7u) == 0) {
+        const int per = gridDim.x >> 3;
+        tile = (int)(blockIdx.x & 7u) * per + (int)(blockIdx.x >> 3);
+    }
+    const unsigned n = fastdiv((unsigned)tile, a.fd_tiles_y);
+    const int oy0 = (int)((unsigned)tile - n * a.fd_tiles_y.d) * a.th;
+    const int iy0 = oy0 * S - p.pad_top, ix0 = -p.pad_left;
+    const int th_real = min(a.th, p.out_h - oy0);
+    const int th = EXACT ? PT : th_real;
+    const int n_xpt = EXACT ? NXPT : a.n_xpt;
+    const int kse = EXACT ? KSE : a.kse;
+    const int c0 = p.in_c;
+
+    // ---- phase 0: tables (all lanes of the group), block-input patch -> operand B registers (per wavefront)
+    const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
+    int ok_e = 1, ok_d = 1, lsh_e = 0, lsh_d = 0;
+    for (int c = tid; c < p.exp_c; c += kGroupThreads) {
+        const int be = p.b_expand != nullptr ? p.b_expand[c] : 0, se = p.s_expand[p.n_s_expand == 1 ? 0 : c];
+        const int bd = p.b_dw != nullptr ? p.b_dw[c] : 0, sd = p.s_dw[p.n_s_dw == 1 ? 0 : c];
+        ok_e &= short_ok(se, be, bound_e) ? 1 : 0;
+        ok_d &= short_ok(sd, bd, bound_d) ? 1 : 0;
+        lsh_e |= se < 8 ? 1 : 0;
+        lsh_d |= sd < 8 ? 1 : 0;
+        tab_e[c] = be;
+        tab_e[p.exp_c + c] = se;
+        tab_d[c] = bd;
+        tab_d[p.exp_c + c] = sd;
+    }
+    const bool fast_e = __syncthreads_and(ok_e) != 0, fast_d = __syncthreads_and(ok_d) != 0;
+    const bool any_le = __syncthreads_or(lsh_e) != 0, any_ld = __syncthreads_or(lsh_d) != 0;
+    const int mode_e = !fast_e ? -1 : (HE ? 2 : (any_le ? 1 : 0));
+    const int mode_d = !fast_d ? -1 : (HE ? 2 : (any_ld ? 1 : 0));
+    for (int c = tid; c < p.exp_c; c += kGroupThreads) { // every lane revisits the channels it wrote
+        const int be = tab_e[c], se = tab_e[p.exp_c + c], bd = tab_d[c], sd = tab_d[p.exp_c + c];
+        if (fast_e) {
+            tab_e[c] = be + (1 << (se - 1));
+            tab_e[p.exp_c + c] = max(0, se - 8);
+        }
+        tab_e[2 * p.exp_c + c] = fast_e ? max(0, 8 - se) : 0;
+        if (fast_d) {
+            tab_d[c] = bd + (1 << (sd - 1));
+            tab_d[p.exp_c + c] = max(0, sd - 8);
+        }
+        tab_d[2 * p.exp_c + c] = fast_d ? max(0, 8 - sd) : 0;
+    }
+
+    v4i xb[NXPT * KSE];
+    unsigned xmask = 0;
+    {
+        const int8_t *img = p.in + (long long)n * p.in_h * p.in_w * c0;
+#pragma unroll
+        for (int pt = 0; pt < NXPT; pt++) {
+            const unsigned pp = (unsigned)(pt * 16 + col);
+            const unsigned prow = fastdiv(pp, a.fd_pw);
+            const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
+            const bool valid = pt < n_xpt && (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h &&
+                (unsigned)ix < (unsigned)p.in_w;
+            xmask |= valid ? 1u << pt : 0u;
+#pragma unroll
+            for (int ks = 0; ks < KSE; ks++) {
+                xb[pt * KSE + ks] = v4i{0, 0, 0, 0};
+                if (EXACT || (pt < n_xpt && ks < kse)) // uniform
+                    xb[pt * KSE + ks] = load16_partial<true>(img, (unsigned)((iy * p.in_w + ix) * c0 + 64 * ks + 16 * quad),
+                                                             valid ? c0 - 64 * ks - 16 * quad : 0);
+            }
+        }
+    }
+    __syncthreads(); // tables complete
+
+    // ---- phase 1: this wavefront's chunks of 16 expanded channels, expand -> depthwise, no barriers
+    const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
+    const int floor_d = p.relu_dw ? 0 : (int)0x80008000u;
+    unsigned char *exp_dst = exp_l + col * 16 + 4 * quad;
+    const unsigned char *exp_src = exp_l + (quad * a.pw + S * col) * 16;
+    const int row_bytes = a.twp * a.ds;
+    const bool write_ok = col < a.twp;
+
+    struct ChunkW {
+        v4i aop[KSE];
+        int wd0[3], wd1[3];
+    };
+    auto load_chunk = [&](int sub) {
+        ChunkW w;
+        const int ch0 = 16 * sub;
+#pragma unroll
+        for (int ks = 0; ks < KSE; ks++) {
+            w.aop[ks] = v4i{0, 0, 0, 0};
+            if (EXACT || ks < kse) // uniform
+                w.aop[ks] = load16_partial<true>(p.w_expand, (unsigned)((ch0 + col) * c0 + 64 * ks + 16 * quad),
+                                                 c0 - 64 * ks - 16 * quad);
+        }
+        const unsigned wd = (unsigned)(ch0 + col);
+#pragma unroll
+        for (int kx = 0; kx < 3; kx++) {
+            const int v0 = (int)p.w_dw[(size_t)(wd + (unsigned)((min(quad, 2) * 3 + kx) * p.exp_c))];
+            w.wd0[kx] = quad < 3 ? v0 : 0;
+            w.wd1[kx] = 0;
+            if constexpr (S == 1) {
+                const int v1 = (int)p.w_dw[(size_t)(wd + (unsigned)((max(quad - 1, 0) * 3 + kx) * p.exp_c))];
+                w.wd1[kx] = quad >= 1 ? v1 : 0;
+            }
+        }
+        return w;
+    };
+
+    if (wave < a.n_sub) {
+        ChunkW cur = load_chunk(wave);
+        for (int sub = wave; sub < a.n_sub; sub += kGroupWaves) {
+            const ChunkW nxt = load_chunk(min(sub + kGroupWaves, a.n_sub - 1));
+            {
+                const StageConsts ce = read_stage_table(tab_e, p.exp_c, 16 * sub + 4 * quad, mode_e);
+                if (ce.mode == 0)
+                    expand_chunk<0, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                else if (ce.mode == 1)
+                    expand_chunk<1, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                else if (ce.mode == 2)
+                    expand_chunk<2, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                else
+                    expand_chunk<-1, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+            }
+            wave_lds_sync();
+            {
+                v4i a0[3], a1[3];
+#pragma unroll
+                for (int kx = 0; kx < 3; kx++) {
+                    a0[kx] = diag_operand(cur.wd0[kx], col);
+                    a1[kx] = diag_operand(cur.wd1[kx], col);
+                }
+                const StageConsts cd = read_stage_table(tab_d, p.exp_c, 16 * sub + 4 * quad, mode_d);
+                unsigned char *dst = dw_l + col * a.ds + 16 * sub + 4 * quad;
+                if (cd.mode == 0)
+                    depthwise_chunk<0, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
+                else if (cd.mode == 1)
+                    depthwise_chunk<1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
+                else if (cd.mode == 2)
+                    depthwise_chunk<2, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
+                else
+                    depthwise_chunk<-1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
+            }
+            wave_lds_sync();
+            cur = nxt;
+        }
+    }
+    __syncthreads(); // the shared depthwise tile is complete
+
+    // ---- phase 2: project.  A wavefront owns one row tile of 16 filters at a time (all of them when there
+    // are at least eight, otherwise the row tiles are shared by 8 / rt wavefronts that split the pixel tiles),
+    // so operand A is loaded once per k step and used for up to kMaxT pixel tiles; eight k steps of operand A
+    // are requested together, which is what hides the latency of these loads.
+    const int ksp = (p.exp_c + 63) / 64;
+    int rt_first, rt_step, t0, t1;
+    if (a.rt >= kGroupWaves) {
+        rt_first = wave;
+        rt_step = kGroupWaves;
+        t0 = 0;
+        t1 = a.npt;
+    } else {
+        const int wpr = kGroupWaves / a.rt; // wavefronts per row tile
+        const int part = wave % wpr, per = (a.npt + wpr - 1) / wpr;
+        rt_first = wave / wpr; // >= a.rt for the wavefronts left over: they have nothing to do
+        rt_step = a.rt;        // one row tile per wavefront
+        t0 = min(a.npt, part * per);
+        t1 = min(a.npt, t0 + per);
+    }
+    const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
+    const unsigned bound_p = (unsigned)p.exp_c * 16384u;
+    const long long img_off = (long long)n * p.out_h * p.out_w * p.out_c;
+    const int8_t *res_img = p.residual != nullptr ? p.residual + img_off : nullptr;
+    int8_t *out_img = p.out + img_off;
+    for (int rt = rt_first; rt < a.rt; rt += rt_step) {
+        v4i accp[kMaxT];
+#pragma unroll
+        for (int i = 0; i < kMaxT; i++)
+            accp[i] = v4i{0, 0, 0, 0};
+        const bool row_ok = 16 * rt + col < p.out_c;
+        const unsigned a_off = (unsigned)((16 * rt + col) * p.exp_c + 16 * quad);
+        const unsigned char *bsrc = dw_l + (t0 * 16 + col) * a.ds + 16 * quad;
+        for (int k0 = 0; k0 < ksp; k0 += 8) {
+            v4i ap[8];
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++) // lanes past the last channel read offset 0 and get zeros
+                ap[kk] = load16_partial<true>(p.w_project, a_off + 64u * (unsigned)(k0 + kk),
+                                              row_ok ? p.exp_c - 64 * (k0 + kk) - 16 * quad : 0);
+#pragma unroll
+            for (int kk = 0; kk < 8; kk++) {
+                if (k0 + kk < ksp) { // uniform
+                    const bool k_ok = p.exp_c - 64 * (k0 + kk) - 16 * quad > 0;
+#pragma unroll
+                    for (int i = 0; i < kMaxT; i++) {
+                        if (t0 + i < t1) { // uniform
+                            v4i bv = *reinterpret_cast<const v4i *>(bsrc + i * 16 * a.ds + 64 * (k0 + kk));
+                            bv = k_ok ? bv : v4i{0, 0, 0, 0};
+                            accp[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ap[kk], bv, accp[i], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+        const int c = 16 * rt + 4 * quad;
+        v4i bp, sp;
+        load_bias_shift(p.b_project, p.s_project, p.n_s_project, c, p.out_c, bp, sp);
+        const StageConsts cp = stage_consts(bp, sp, bound_p, HE);
+#pragma unroll
+        for (int i = 0; i < kMaxT; i++) {
+            if (t0 + i < t1) { // uniform
+                // pixel slot -> (row, column) of the tile: twp slots per output row
+                const int slot = (t0 + i) * 16 + col;
+                const int oy = a.twp == 16 ? t0 + i : (slot >> 3), ox = a.twp == 16 ? col : (slot & 7);
+                const bool live = oy < th_real && ox < p.out_w && c < p.out_c;
+                const unsigned off = (unsigned)(((oy0 + oy) * p.out_w + ox) * p.out_c + c);
+                v4i acc = accp[i];
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    acc[k] += cp.init[k];
+                const int rv = res_img != nullptr ? *reinterpret_cast<const int *>(res_img + (size_t)(live ? off : 0u)) : 0;
+                int word;
+                if (cp.mode == 0)
+                    word = res_img != nullptr ? pack_fast4_add<0>(acc, cp.lsh, cp.rsh, floor_p, rv)
+                                              : wave_pack<0>(acc, cp, floor_p, false, HE);
+                else if (cp.mode == 1)
+                    word = res_img != nullptr ? pack_fast4_add<1>(acc, cp.lsh, cp.rsh, floor_p, rv)
+                                              : wave_pack<1>(acc, cp, floor_p, false, HE);
+                else if (cp.mode == 2)
+                    word = res_img != nullptr ? pack_fast4_add<2>(acc, cp.lsh, cp.rsh, floor_p, rv)
+                                              : wave_pack<2>(acc, cp, floor_p, false, HE);
+                else {
+                    word = wave_pack<-1>(acc, cp, floor_p, p.relu_project != 0, HE);
+                    if (res_img != nullptr)
+                        word = sat_add4_s8(word, rv);
+                }
+                if (live)
+                    *reinterpret_cast<int *>(out_img + (size_t)off) = word;
+            }
+        }
+    }
+}
+
+struct GroupPlan {
+    bool ok;
+    GroupArgs a;
+    size_t lds;
+};
+
+constexpr int kGroupPtMax = 8;
+constexpr size_t kGroupLdsMax = 156 * 1024;
+
+GroupPlan group_plan(const MbconvParams &p)
+{
+    GroupPlan plan;
+    plan.ok = false;
+    if (p.w_expand == nullptr || p.k_h != 3 || p.k_w != 3 || p.dil_h != 1 || p.dil_w != 1 || p.stride_h != p.stride_w ||
+        (p.stride_h != 1 && p.stride_h != 2))
+        return plan;
+    if (p.in_c % 16 != 0 || p.in_c > 192 || p.exp_c % 16 != 0 || p.exp_c >= 65536 || p.out_c % 4 != 0 || p.out_w > 16 ||
+        (reinterpret_cast<uintptr_t>(p.in) & 15) != 0 || (reinterpret_cast<uintptr_t>(p.w_expand) & 15) != 0)
+        return plan;
+    if ((long long)p.in_h * p.in_w * p.in_c >= (1ll << 30) || (long long)p.out_h * p.out_w * p.out_c >= (1ll << 30) ||
+        (long long)p.out_c * p.exp_c >= (1ll << 31))
+        return plan;
+    const int s = p.stride_h;
+    GroupArgs a = {};
+    a.p = p;
+    a.tw = p.out_w;
+    a.pw = (a.tw - 1) * s + 3;
+    a.twp = p.out_w <= 8 ? 8 : 16;
+    a.kse = (p.in_c + 63) / 64;
+    a.n_sub = p.exp_c / 16;
+    a.rt = (p.out_c + 15) / 16;
+    a.ds = p.exp_c + 16; // exp_c is a multiple of 16: an odd number of 16-byte units when exp_c / 16 is even ...
+    if ((a.ds / 16) % 2 == 0)
+        a.ds += 16;      // ... and made odd otherwise, so that operand-B reads of 16 pixels spread over the banks
+    // rows per tile: as many as fit the register and LDS budgets (fewer tiles, less halo to expand)
+    a.th = 0;
+    for (int th = 1; th <= std::min(kGroupPtMax - 1, p.out_h); th++) {
+        const int ph = (th - 1) * s + 3;
+        const int n_xpt = (ph * a.pw + 15) / 16;
+        if (n_xpt > 9)
+            break;
+        const int npt = (th * a.twp + 15) / 16;
+        if (npt > kMaxT)
+            break;
+        const size_t exp_bytes = (size_t)((ph * a.pw + 48 + 15) & ~15) * 16;
+        const size_t lds = (size_t)p.exp_c * 24 + kGroupWaves * std::max(exp_bytes, (size_t)((n_xpt + 3) & ~3) * 256) +
+            (size_t)npt * 16 * a.ds;
+        if (lds > kGroupLdsMax)
+            break;
+        a.th = th;
+    }
+    if (a.th == 0)
+        return plan;
+    a.ph = (a.th - 1) * s + 3;
+    a.n_xpt = (a.ph * a.pw + 15) / 16;
+    a.npt = (a.th * a.twp + 15) / 16;
+    a.tiles_y = (p.out_h + a.th - 1) / a.th;
+    a.exp_bytes = (int)std::max((size_t)((a.ph * a.pw + 48 + 15) & ~15) * 16, (size_t)((a.n_xpt + 3) & ~3) * 256);
+    a.off_tab = 0;
+    a.off_exp = p.exp_c * 24;
+    a.off_dw = a.off_exp + kGroupWaves * a.exp_bytes;
+    plan.lds = (size_t)a.off_dw + (size_t)a.npt * 16 * a.ds;
+    a.fd_pw = make_fastdiv((unsigned)a.pw);
+    a.fd_tiles_y = make_fastdiv((unsigned)a.tiles_y);
+    a.fd_npt = make_fastdiv((unsigned)a.npt);
+    plan.a = a;
+    plan.ok = true;
+    return plan;
+}
+
+template <int NXPT, int KSE, int PT, int S, bool HE, bool EXACT>
+hipError_t launch_group_one(const GroupPlan &plan, hipStream_t stream)
+{
+    auto kernel = mbconv_s8_group_kernel<NXPT, KSE, PT, S, HE, EXACT>;
+    static bool raised = false; // the dynamic LDS limit of a kernel is raised once per process
+    if (!raised) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGroupLdsMax);
+        if (e != hipSuccess)
+            return e;
+        raised = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)plan.a.n_tiles), dim3(kGroupThreads), plan.lds, stream, plan.a);
+    return hipGetLastError();
+}
+
+} // namespace
+
+bool mbconv_s8_group_supports(const MbconvParams &p)
+{
+    return group_plan(p).ok;
+}
+
+hipError_t launch_mbconv_s8_group(const MbconvParams &p, int cu_count, hipStream_t stream)
+{
+    (void)cu_count;
+    if ((long long)p.batch * p.out_h * p.out_w == 0)
+        return hipSuccess;
+    GroupPlan plan = group_plan(p);
+    if (!plan.ok)
+        return hipErrorInvalidValue;
+    const long long tiles = (long long)p.batch * plan.a.tiles_y;
+    if (tiles > 0x7fffffff)
+        return hipErrorInvalidValue;
+    plan.a.n_tiles = (int)tiles;
+    const GroupArgs &a = plan.a;
+    static const bool trace = getenv("ESPDL_HIP_TRACE") != nullptr;
+    if (trace)
+        fprintf(stderr, "mbconv_s8_group: %dx%d in %d exp %d out %d s%d tile %dx%d patch %dx%d n_xpt %d kse %d rt %d npt %d lds %zu tiles %lld\n",
+                p.in_h, p.in_w, p.in_c, p.exp_c, p.out_c, p.stride_h, a.th, a.tw, a.ph, a.pw, a.n_xpt, a.kse, a.rt, a.npt,
+                plan.lds, tiles);
+    const int s = p.stride_h;
+    if (!p.half_even) {
+        const auto is = [&](int nxpt, int kse, int th, int stride) {
+            return a.n_xpt == nxpt && a.kse == kse && a.th == th && s == stride;
+        };
+        if (is(9, 1, 7, 1))
+            return launch_group_one<9, 1, 7, 1, false, true>(plan, stream);
+        if (is(9, 2, 7, 1))
+            return launch_group_one<9, 2, 7, 1, false, true>(plan, stream);
+        if (is(6, 3, 7, 1))
+            return launch_group_one<6, 3, 7, 1, false, true>(plan, stream);
+        if (is(9, 2, 4, 2))
+            return launch_group_one<9, 2, 4, 2, false, true>(plan, stream);
+        return s == 1 ? launch_group_one<9, 3, kGroupPtMax, 1, false, false>(plan, stream)
+                      : launch_group_one<9, 3, kGroupPtMax, 2, false, false>(plan, stream);
+    }
+    return s == 1 ? launch_group_one<9, 3, kGroupPtMax, 1, true, false>(plan, stream)
+                  : launch_group_one<9, 3, kGroupPtMax, 2, true, false>(plan, stream);
+}
+
+} // namespace espdl

@@ -1,0 +1,270 @@
+// Stage building blocks of the inverted-residual kernels that run expand -> depthwise -> project with
+// wavefronts working on their own (mbconv_s8_wave.hip: one wavefront per tile; mbconv_s8_group.hip: a
+// workgroup of wavefronts that split the expanded channels of one tile).  The arithmetic is that of the
+// separate operators: conv2d_11cn + n_wise epilogue (esp-dl/dl/base/dl_base_conv2d.cpp:9-33;
+// esp-dl/dl/base/dl_base_activate_buffer.hpp:10-74, 162-212), depthwise_conv2d_33c1 under the shell's
+// window clipping (esp-dl/dl/base/dl_base_depthwise_conv2d.cpp:19-65; esp-dl/dl/base/dl_base.hpp:1852-2102).
+#pragma once
+
+#include <type_traits>
+
+#include "espdl_device.h"
+#include "espdl_kernels.h"
+
+namespace espdl {
+namespace mbstage {
+
+constexpr int kDws = 80; // LDS pixel stride of a 64-channel depthwise result: 64 + 16 (odd number of 16-byte units)
+
+// 16 bytes at p + off of which the first `nvalid` exist (nvalid a multiple of 4, possibly <= 0); the rest
+// are zeros.  Branch-free: a piece that does not exist is read from offset 0 of `p` instead (always a valid
+// address) and replaced by zero, so that every lane issues the same loads and the wait counters of loads
+// requested ahead of their use stay exact.  VEC16: p + off is 16-byte aligned whenever nvalid >= 16 and
+// nvalid is then never in 1..15.
+template <bool VEC16>
+__device__ __forceinline__ v4i load16_partial(const int8_t *p, unsigned off, int nvalid)
+{
+    // `p` is the same in every lane and `off` is an unsigned 32-bit byte offset: one scalar base plus one
+    // vector offset per load, no 64-bit address arithmetic on the vector ALU
+    v4i r;
+    if constexpr (VEC16) {
+        const bool ok = nvalid >= 16;
+        r = *reinterpret_cast<const v4i *>(p + (size_t)(ok ? off : 0u));
+        r = ok ? r : v4i{0, 0, 0, 0};
+    } else {
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const bool ok = 4 * d < nvalid;
+            const int v = *reinterpret_cast<const int *>(p + (size_t)(ok ? off + 4u * d : 0u));
+            r[d] = ok ? v : 0;
+        }
+    }
+    return r;
+}
+
+// Orders the LDS accesses of the wavefront's lanes among each other.  LDS executes the instructions of one
+// wavefront in order, so nothing has to be waited for; the compiler must not move accesses across.
+__device__ __forceinline__ void wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Is the short epilogue (pack_fast4) exact for this channel?  The shift must be in 1..31 and
+// |bias| + 2^(s-1) + mac_bound (the largest magnitude the accumulator can reach) must stay below
+// 2^(31 - max(0, 8 - s)), so that neither the accumulator nor its left-shifted form overflows.
+// mac_bound < 2^30 (checked on the host); everything fits unsigned 32-bit arithmetic.
+__device__ __forceinline__ bool short_ok(int s, int bias, unsigned mac_bound)
+{
+    if (s < 1 || s > 31)
+        return false;
+    const unsigned lim = 1u << (31 - max(0, 8 - s));
+    const unsigned t = mac_bound + (1u << (s - 1));
+    const unsigned ub = bias < 0 ? 0u - (unsigned)bias : (unsigned)bias;
+    return t < lim && ub < lim - t;
+}
+
+// Requantization constants of four consecutive channels of one stage, and which epilogue the whole
+// wavefront takes for them: pack_fast4 mode 0 (every shift >= 8), 1 (some shift below 8), 2 (half-even),
+// or -1 for the general shift_and_round restatement (a shift outside 1..31, or an accumulator that could
+// overflow the short form).
+struct StageConsts {
+    v4i init, rsh, lsh;
+    int mode;
+};
+
+// b, sh: bias and shift of the lane's four channels (channels that do not exist: 0 and 8).
+__device__ __forceinline__ StageConsts stage_consts(const v4i &b, const v4i &sh, unsigned mac_bound, bool half_even)
+{
+    StageConsts c;
+    bool ok = true;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+        ok = ok && short_ok(sh[r], b[r], mac_bound);
+    if (__all(ok)) {
+        bool any_lsh = false;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            c.init[r] = b[r] + (1 << (sh[r] - 1));
+            c.rsh[r] = max(0, sh[r] - 8);
+            c.lsh[r] = max(0, 8 - sh[r]);
+            any_lsh = any_lsh || sh[r] < 8;
+        }
+        c.mode = half_even ? 2 : (__any(any_lsh) ? 1 : 0);
+    } else {
+        c.init = b;
+        c.rsh = sh;
+        c.lsh = v4i{0, 0, 0, 0};
+        c.mode = -1;
+    }
+    return c;
+}
+
+// Per-channel constants of a stage for every channel of the block, built once per tile in LDS by all lanes
+// (channel = lane + 64 i) as [init | right shift | left shift][n_ch], in the form the stage's epilogue
+// `mode` wants (see StageConsts); returns that mode, one for the whole stage.
+__device__ __forceinline__ int build_stage_table(int *tab, const int32_t *bias, const int32_t *shift, int n_shift,
+                                                 int n_ch, unsigned mac_bound, bool half_even, int lane)
+{
+    bool ok = true, any_lsh = false;
+    for (int c = lane; c < n_ch; c += 64) {
+        const int b = bias != nullptr ? bias[c] : 0;
+        const int sh = shift[n_shift == 1 ? 0 : c];
+        ok = ok && short_ok(sh, b, mac_bound);
+        any_lsh = any_lsh || sh < 8;
+        tab[c] = b;
+        tab[n_ch + c] = sh;
+    }
+    const bool fast = __all(ok) != 0;
+    const int mode = !fast ? -1 : (half_even ? 2 : (__any(any_lsh) ? 1 : 0));
+    for (int c = lane; c < n_ch; c += 64) { // each lane revisits the channels it wrote
+        const int b = tab[c], sh = tab[n_ch + c];
+        if (fast) {
+            tab[c] = b + (1 << (sh - 1));
+            tab[n_ch + c] = max(0, sh - 8);
+            tab[2 * n_ch + c] = max(0, 8 - sh);
+        } else {
+            tab[2 * n_ch + c] = 0;
+        }
+    }
+    return mode;
+}
+
+__device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch, int ch, int mode)
+{
+    StageConsts c;
+    c.init = *reinterpret_cast<const v4i *>(tab + ch);
+    c.rsh = *reinterpret_cast<const v4i *>(tab + n_ch + ch);
+    c.lsh = v4i{0, 0, 0, 0};
+    if (mode == 1 || mode == 2)
+        c.lsh = *reinterpret_cast<const v4i *>(tab + 2 * n_ch + ch);
+    c.mode = mode;
+    return c;
+}
+
+// Bias and shift of four consecutive channels starting at `ch` (a multiple of 4), straight from memory,
+// branch-free (see load16_partial): channels that do not exist give bias 0 and shift 8.
+__device__ __forceinline__ void load_bias_shift(const int32_t *bias, const int32_t *shift, int n_shift, int ch, int n_ch,
+                                                v4i &b, v4i &sh)
+{
+    const bool exists = ch < n_ch; // channel counts are multiples of 4: all four exist or none
+    const int32_t *bp = bias != nullptr ? bias : shift;
+    const int cb = (exists && bias != nullptr) ? ch : 0;
+    const int cs = (exists && n_shift != 1) ? ch : 0;
+    const int step = n_shift != 1 ? 1 : 0;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int bv = bp[cb + (bias != nullptr ? r : 0)];
+        const int sv = shift[cs + step * r];
+        b[r] = (exists && bias != nullptr) ? bv : 0;
+        sh[r] = exists ? sv : 8;
+    }
+}
+
+template <int MODE>
+__device__ __forceinline__ int wave_pack(const v4i &acc, const StageConsts &c, int floor_pk, bool relu, bool half_even)
+{
+    if constexpr (MODE >= 0) {
+        return pack_fast4<MODE>(acc, c.lsh, c.rsh, floor_pk);
+    } else {
+        int q[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            q[r] = requant_s8(acc[r], c.rsh[r], relu, half_even);
+        return pack4_s8(q[0], q[1], q[2], q[3]);
+    }
+}
+
+// Expand stage of one chunk of 16 channels: every patch pixel tile through one MFMA and the epilogue, four
+// tiles at a time so that four independent MFMA -> requantize -> store chains are in flight (tiles past
+// n_xpt inside the last group of four have zero operands and a zero mask and land in slack).
+template <int MODE, int NXPT, bool EXACT, int KSE = 1>
+__device__ __forceinline__ void expand_chunk(const v4i (&xb)[NXPT * KSE], int n_xpt, unsigned xmask,
+                                             const v4i (&aop)[KSE], const StageConsts &c, int floor_pk, bool relu,
+                                             bool half_even, unsigned char *dst /* exp_l + col * 16 + 4 * quad */)
+{
+#pragma unroll
+    for (int g0 = 0; g0 < NXPT; g0 += 4) {
+        if (EXACT || g0 < n_xpt) { // uniform
+            v4i acc[4];
+#pragma unroll
+            for (int ks = 0; ks < KSE; ks++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (g0 + j < NXPT)
+                        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], xb[(g0 + j) * KSE + ks],
+                                                                       ks == 0 ? c.init : acc[j], 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if (g0 + j < NXPT) {
+                    int word = wave_pack<MODE>(acc[j], c, floor_pk, relu, half_even);
+                    word &= __builtin_amdgcn_sbfe((int)xmask, g0 + j, 1); // all ones or zero
+                    *reinterpret_cast<int *>(dst + (g0 + j) * 256) = word;
+                }
+            }
+        }
+    }
+}
+
+// Depthwise stage of one chunk of 16 channels.  S == 1: output rows in pairs, four patch rows per read.
+template <int MODE, int PT, int S, bool EXACT>
+__device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_l + (quad * pw + S * col) * 16 */,
+                                                int th, int pw, const v4i (&a0)[3], const v4i (&a1)[3],
+                                                const StageConsts &c, int floor_pk, bool relu, bool half_even,
+                                                unsigned char *dst /* lane's slot in output row 0 of the result */,
+                                                int row_bytes = 16 * kDws, bool write_ok = true)
+{
+    if constexpr (S == 1) {
+#pragma unroll
+        for (int j = 0; j < (PT + 1) / 2; j++) {
+            if (EXACT || 2 * j < th) { // uniform
+                const unsigned char *s = src + 2 * j * pw * 16;
+                const v4i b0 = *reinterpret_cast<const v4i *>(s);
+                const v4i b1 = *reinterpret_cast<const v4i *>(s + 16);
+                const v4i b2 = *reinterpret_cast<const v4i *>(s + 32);
+                v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b0, c.init, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b1, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[2], b2, acc, 0, 0, 0);
+                const int w0 = wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+                if (write_ok)
+                    *reinterpret_cast<int *>(dst + (2 * j) * row_bytes) = w0;
+                if (EXACT ? 2 * j + 1 < PT : 2 * j + 1 < th) {
+                    v4i acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[0], b0, c.init, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[1], b1, acc1, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[2], b2, acc1, 0, 0, 0);
+                    const int w1 = wave_pack<MODE>(acc1, c, floor_pk, relu, half_even);
+                    if (write_ok)
+                        *reinterpret_cast<int *>(dst + (2 * j + 1) * row_bytes) = w1;
+                }
+            }
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < PT; t++) {
+            if (EXACT || t < th) { // uniform
+                const unsigned char *s = src + S * t * pw * 16;
+                const v4i b0 = *reinterpret_cast<const v4i *>(s);
+                const v4i b1 = *reinterpret_cast<const v4i *>(s + 16);
+                const v4i b2 = *reinterpret_cast<const v4i *>(s + 32);
+                v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b0, c.init, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b1, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[2], b2, acc, 0, 0, 0);
+                const int w0 = wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+                if (write_ok)
+                    *reinterpret_cast<int *>(dst + t * row_bytes) = w0;
+            }
+        }
+    }
+}
+
+// One dword of a diagonal operand A: weight byte `w` of channel row i sits at byte i of the lane's 16.
+__device__ __forceinline__ v4i diag_operand(int w, int i)
+{
+    const int d = (w & 0xff) << (8 * (i & 3));
+    const int sel = i >> 2;
+    return v4i{sel == 0 ? d : 0, sel == 1 ? d : 0, sel == 2 ? d : 0, sel == 3 ? d : 0};
+}
+
+} // namespace mbstage
+} // namespace espdl

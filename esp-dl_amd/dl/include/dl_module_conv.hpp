@@ -55,6 +55,13 @@ private:
     bool m_has_pre_add_exponent = false;
     int m_pre_add_exponent = 0; ///< exponent of the tensor an absorbed Add used to read from this module
     DeviceInts m_shift_project;
+    // A depthwise Conv that absorbed its project Conv may also absorb the 1x1 Conv in front of it: its first
+    // input is then the block input and the expanded tensor is never materialized.
+    bool m_has_expand = false;
+    activation_type_t m_expand_activation = Linear;
+    int m_expand_exponent = 0; ///< exponent of the (no longer materialized) expanded tensor
+    int m_expand_filter_pos = -1, m_expand_bias_pos = -1;
+    DeviceInts m_shift_expand;
 
 public:
     Conv(activation_type_t activation = Linear, std::vector<int> pads = {}, std::vector<int> dilations = {},
@@ -111,6 +118,22 @@ public:
             m_inputs_index.push_back(residual_index);
         }
     }
+    /// Absorb the 1x1 Conv in front (after fuse_project): `input_index` is that Conv's input, which becomes
+    /// this module's first input; `expand_exponent` the exponent of the tensor it used to write.
+    void fuse_expand(int input_index, int filter_index, int bias_index, activation_type_t act, int expand_exponent)
+    {
+        m_has_expand = true;
+        m_expand_activation = act;
+        m_expand_exponent = expand_exponent;
+        m_inputs_index[0] = input_index;
+        m_expand_filter_pos = (int)m_inputs_index.size();
+        m_inputs_index.push_back(filter_index);
+        if (bias_index >= 0) {
+            m_expand_bias_pos = (int)m_inputs_index.size();
+            m_inputs_index.push_back(bias_index);
+        }
+    }
+    bool has_fused_expand() const { return m_has_expand; }
     /// Absorb the Add that follows a dense Conv: `residual_index` is the Add's other operand and
     /// `own_out_exponent` the exponent of the tensor the Conv used to write.  The Add sums stored integers
     /// whatever the exponents of its operands and result are (esp-dl/dl/base/dl_base_add.cpp:35-44), so the
@@ -167,8 +190,13 @@ public:
             pixels *= out[i];
         const int64_t taps = out.size() == 3 ? f[0] : (int64_t)f[0] * f[1];
         const int64_t in_c = m_group == 1 ? input_shapes[0].back() : 1;
-        if (m_has_project) // depthwise over the input channels + 1x1 over them
-            return pixels * input_shapes[0].back() * taps + pixels * out.back() * input_shapes[0].back();
+        if (m_has_project) { // [1x1 over the block input +] depthwise + 1x1 over the depthwise channels
+            const int64_t dw_c = input_shapes[m_project_filter_pos][2];
+            int64_t macs = pixels * dw_c * taps + pixels * out.back() * dw_c;
+            if (m_has_expand)
+                macs += (int64_t)input_shapes[0][0] * input_shapes[0][1] * input_shapes[0][2] * input_shapes[0][3] * dw_c;
+            return macs;
+        }
         return pixels * out.back() * taps * in_c;
     }
 
@@ -262,9 +290,12 @@ public:
         TensorBase *pfilter = context->get_tensor(m_inputs_index[m_project_filter_pos]);
         TensorBase *pbias = m_project_bias_pos >= 0 ? context->get_tensor(m_inputs_index[m_project_bias_pos]) : nullptr;
         TensorBase *residual = m_residual_pos >= 0 ? context->get_tensor(m_inputs_index[m_residual_pos]) : nullptr;
+        TensorBase *efilter = m_has_expand ? context->get_tensor(m_inputs_index[m_expand_filter_pos]) : nullptr;
+        TensorBase *ebias = m_expand_bias_pos >= 0 ? context->get_tensor(m_inputs_index[m_expand_bias_pos]) : nullptr;
         if (!input || !filter || !output || !pfilter || !input->on_device() || !filter->on_device() ||
             !output->on_device() || !pfilter->on_device() || (bias && !bias->on_device()) ||
-            (pbias && !pbias->on_device()) || (residual && !residual->on_device()) || input->shape.size() != 4) {
+            (pbias && !pbias->on_device()) || (residual && !residual->on_device()) || input->shape.size() != 4 ||
+            (m_has_expand && (!efilter || !efilter->on_device())) || (ebias && !ebias->on_device())) {
             DL_LOGE("Conv", "%s: fused depthwise+project needs 4-D device tensors", name.c_str());
             return;
         }
@@ -273,9 +304,10 @@ public:
         d.in_h = input->shape[1];
         d.in_w = input->shape[2];
         d.in_c = input->shape[3];
-        d.exp_c = d.in_c;
+        d.exp_c = m_has_expand ? pfilter->shape[2] : d.in_c;
         d.out_c = output->shape[3];
-        d.has_expand = 0;
+        d.has_expand = m_has_expand ? 1 : 0;
+        d.act_expand = m_expand_activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR;
         d.k_h = filter->shape[0];
         d.k_w = filter->shape[1];
         d.stride_h = m_strides[0];
@@ -289,12 +321,21 @@ public:
         d.act_dw = activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR;
         d.act_project = m_project_activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR;
         d.round_mode = context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP;
-        std::vector<int32_t> s_dw, s_pj;
+        std::vector<int32_t> s_dw, s_pj, s_ex;
+        const int dw_in_exponent = m_has_expand ? m_expand_exponent : input->exponent.get();
         if (filter->exponent.is_per_channel()) {
-            for (int c = 0; c < d.in_c; c++)
-                s_dw.push_back(m_mid_exponent - filter->exponent.get(c) - input->exponent.get());
+            for (int c = 0; c < d.exp_c; c++)
+                s_dw.push_back(m_mid_exponent - filter->exponent.get(c) - dw_in_exponent);
         } else {
-            s_dw.push_back(m_mid_exponent - filter->exponent.get() - input->exponent.get());
+            s_dw.push_back(m_mid_exponent - filter->exponent.get() - dw_in_exponent);
+        }
+        if (m_has_expand) {
+            if (efilter->exponent.is_per_channel()) {
+                for (int c = 0; c < d.exp_c; c++)
+                    s_ex.push_back(m_expand_exponent - efilter->exponent.get(c) - input->exponent.get());
+            } else {
+                s_ex.push_back(m_expand_exponent - efilter->exponent.get() - input->exponent.get());
+            }
         }
         const int pj_out_exponent = m_has_pre_add_exponent ? m_pre_add_exponent : output->exponent.get();
         if (pfilter->exponent.is_per_channel()) {
@@ -303,10 +344,15 @@ public:
         } else {
             s_pj.push_back(pj_out_exponent - pfilter->exponent.get() - m_mid_exponent);
         }
-        d.n_shift_expand = 1;
+        d.n_shift_expand = m_has_expand ? (int32_t)s_ex.size() : 1;
         d.n_shift_dw = (int32_t)s_dw.size();
         d.n_shift_project = (int32_t)s_pj.size();
         espdl_hip_mbconv_weights w = {};
+        if (m_has_expand) {
+            w.w_expand = static_cast<const int8_t *>(efilter->data);
+            w.b_expand = ebias ? static_cast<const int32_t *>(ebias->data) : nullptr;
+            w.s_expand = m_shift_expand.sync(s_ex);
+        }
         w.w_dw = static_cast<const int8_t *>(filter->data);
         w.b_dw = bias ? static_cast<const int32_t *>(bias->data) : nullptr;
         w.s_dw = m_shift.sync(s_dw);

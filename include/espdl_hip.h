@@ -332,7 +332,10 @@ int espdl_hip_slice(const void *in, const int32_t *shape, int32_t dims, const in
  * Needs exp_c % 16 == 0, in_c % 16 == 0, out_c % 4 == 0, at most 12 depthwise taps, in_c <= 192,
  * exp_c <= 1024, out_c <= 384, 16-byte aligned input and filters; espdl_hip_mbconv_s8_supported() answers for a descriptor: 0 = no, 1 = yes (general
  * fused kernel), 2 = yes, through the depthwise+project kernel (no expand stage, at most 256
- * channels), which is the form that is faster than separate launches today.
+ * channels), 3 = yes, expand stage inside the LDS-tile depthwise kernel, 4 = yes, one wavefront per tile
+ * (3x3 depthwise stage, at most 64 block-input channels and 64 project filters), 5 = yes, a workgroup of
+ * wavefronts per tile of a small image (output at most 16 pixels wide, block-input channels a multiple of
+ * 16 and at most 192).
  * espdl_hip_mbconv_s8 returns ESPDL_HIP_ENOTSUP where it does not apply.
  */
 typedef struct espdl_hip_mbconv_desc {
@@ -357,6 +360,11 @@ typedef struct espdl_hip_mbconv_weights {
 
 int espdl_hip_mbconv_out_shape(const espdl_hip_mbconv_desc *desc, int32_t *out_h, int32_t *out_w);
 int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc);
+/* 1 when the single launch is expected to be faster than the separate launches for this descriptor,
+ * batch included (the rule follows measurements on MI355X: the one-wavefront-per-tile kernel, answer 4
+ * of espdl_hip_mbconv_s8_supported, on images of at least 28 x 28 with enough tiles to fill the device;
+ * the depthwise+project form, answer 2, always); 0 otherwise.  dl::Model fuses blocks by this answer. */
+int espdl_hip_mbconv_s8_preferred(const espdl_hip_mbconv_desc *desc);
 int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *weights,
                         const int8_t *residual, int8_t *out, void *stream);
 
