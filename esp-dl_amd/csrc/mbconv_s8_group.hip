@@ -82,36 +82,9 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
 
     // ---- phase 0: tables (all lanes of the group), block-input patch -> operand B registers (per wavefront)
     const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
-    int ok_e = 1, ok_d = 1, lsh_e = 0, lsh_d = 0;
-    for (int c = tid; c < p.exp_c; c += kGroupThreads) {
-        const int be = p.b_expand != nullptr ? p.b_expand[c] : 0, se = p.s_expand[p.n_s_expand == 1 ? 0 : c];
-        const int bd = p.b_dw != nullptr ? p.b_dw[c] : 0, sd = p.s_dw[p.n_s_dw == 1 ? 0 : c];
-        ok_e &= short_ok(se, be, bound_e) ? 1 : 0;
-        ok_d &= short_ok(sd, bd, bound_d) ? 1 : 0;
-        lsh_e |= se < 8 ? 1 : 0;
-        lsh_d |= sd < 8 ? 1 : 0;
-        tab_e[c] = be;
-        tab_e[p.exp_c + c] = se;
-        tab_d[c] = bd;
-        tab_d[p.exp_c + c] = sd;
-    }
-    const bool fast_e = __syncthreads_and(ok_e) != 0, fast_d = __syncthreads_and(ok_d) != 0;
-    const bool any_le = __syncthreads_or(lsh_e) != 0, any_ld = __syncthreads_or(lsh_d) != 0;
-    const int mode_e = !fast_e ? -1 : (HE ? 2 : (any_le ? 1 : 0));
-    const int mode_d = !fast_d ? -1 : (HE ? 2 : (any_ld ? 1 : 0));
-    for (int c = tid; c < p.exp_c; c += kGroupThreads) { // every lane revisits the channels it wrote
-        const int be = tab_e[c], se = tab_e[p.exp_c + c], bd = tab_d[c], sd = tab_d[p.exp_c + c];
-        if (fast_e) {
-            tab_e[c] = be + (1 << (se - 1));
-            tab_e[p.exp_c + c] = max(0, se - 8);
-        }
-        tab_e[2 * p.exp_c + c] = fast_e ? max(0, 8 - se) : 0;
-        if (fast_d) {
-            tab_d[c] = bd + (1 << (sd - 1));
-            tab_d[p.exp_c + c] = max(0, sd - 8);
-        }
-        tab_d[2 * p.exp_c + c] = fast_d ? max(0, 8 - sd) : 0;
-    }
+    const int mode_e = build_stage_table_group(tab_e, p.b_expand, p.s_expand, p.n_s_expand, p.exp_c, bound_e, HE, tid,
+                                               kGroupThreads);
+    const int mode_d = build_stage_table_group(tab_d, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_d, HE, tid, kGroupThreads);
 
     v4i xb[NXPT * KSE];
     unsigned xmask = 0;

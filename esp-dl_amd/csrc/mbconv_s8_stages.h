@@ -131,6 +131,37 @@ __device__ __forceinline__ int build_stage_table(int *tab, const int32_t *bias, 
     return mode;
 }
 
+// The same tables built by all `nthreads` lanes of a workgroup (thread = channel + nthreads * i); the mode
+// is agreed on with workgroup votes, so every lane of the workgroup must call this.  The tables are
+// complete for other wavefronts only after the caller's next barrier.
+__device__ __forceinline__ int build_stage_table_group(int *tab, const int32_t *bias, const int32_t *shift, int n_shift,
+                                                       int n_ch, unsigned mac_bound, bool half_even, int tid,
+                                                       int nthreads)
+{
+    int ok = 1, any_lsh = 0;
+    const unsigned step = n_shift == 1 ? 0u : 1u;
+    for (int c = tid; c < n_ch; c += nthreads) {
+        const int b = bias != nullptr ? bias[(size_t)(unsigned)c] : 0;
+        const int sh = shift[(size_t)(step * (unsigned)c)];
+        ok &= short_ok(sh, b, mac_bound) ? 1 : 0;
+        any_lsh |= sh < 8 ? 1 : 0;
+        tab[c] = b;
+        tab[n_ch + c] = sh;
+    }
+    const bool fast = __syncthreads_and(ok) != 0;
+    const bool lsh = __syncthreads_or(any_lsh) != 0;
+    const int mode = !fast ? -1 : (half_even ? 2 : (lsh ? 1 : 0));
+    for (int c = tid; c < n_ch; c += nthreads) { // every lane revisits the channels it wrote
+        const int b = tab[c], sh = tab[n_ch + c];
+        if (fast) {
+            tab[c] = b + (1 << (sh - 1));
+            tab[n_ch + c] = max(0, sh - 8);
+        }
+        tab[2 * n_ch + c] = fast ? max(0, 8 - sh) : 0;
+    }
+    return mode;
+}
+
 __device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch, int ch, int mode)
 {
     StageConsts c;
@@ -179,43 +210,120 @@ __device__ __forceinline__ int wave_pack(const v4i &acc, const StageConsts &c, i
 // Expand stage of one chunk of 16 channels: every patch pixel tile through one MFMA and the epilogue, four
 // tiles at a time so that four independent MFMA -> requantize -> store chains are in flight (tiles past
 // n_xpt inside the last group of four have zero operands and a zero mask and land in slack).
-template <int MODE, int NXPT, bool EXACT, int KSE = 1>
-__device__ __forceinline__ void expand_chunk(const v4i (&xb)[NXPT * KSE], int n_xpt, unsigned xmask,
+template <int MODE, int NXPT, bool EXACT, int KSE = 1, bool XLDS = false, bool PIPE = false>
+__device__ __forceinline__ void expand_chunk(const v4i (&xb)[XLDS ? 1 : NXPT * KSE], int n_xpt, unsigned xmask,
                                              const v4i (&aop)[KSE], const StageConsts &c, int floor_pk, bool relu,
-                                             bool half_even, unsigned char *dst /* exp_l + col * 16 + 4 * quad */)
+                                             bool half_even, unsigned char *dst /* exp_l + col * 16 + 4 * quad */,
+                                             const unsigned char *xsrc = nullptr, int x_tile_bytes = 0)
 {
+    // XLDS: operand B of pixel tile pt and k step ks sits in LDS at xsrc + (pt * KSE + ks) * x_tile_bytes
+    // (where this lane put it), not in registers
+    auto operand = [&](int pt, int ks) -> v4i {
+        if constexpr (XLDS)
+            return *reinterpret_cast<const v4i *>(xsrc + (pt * KSE + ks) * x_tile_bytes);
+        else
+            return xb[pt * KSE + ks];
+    };
+    auto product = [&](int pt) -> v4i {
+        v4i acc = c.init;
 #pragma unroll
-    for (int g0 = 0; g0 < NXPT; g0 += 4) {
-        if (EXACT || g0 < n_xpt) { // uniform
-            v4i acc[4];
+        for (int ks = 0; ks < KSE; ks++)
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], operand(pt, ks), acc, 0, 0, 0);
+        return acc;
+    };
+    auto finish = [&](const v4i &acc, int pt) {
+        int word = wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+        word &= __builtin_amdgcn_sbfe((int)xmask, pt, 1); // all ones or zero
+        *reinterpret_cast<int *>(dst + pt * 256) = word;
+    };
+    if constexpr (EXACT && PIPE) {
+        // software pipeline: the matrix product of the next pixel tile is issued before the requantization of
+        // the current one, so the matrix pipe works while the vector ALU requantizes (the scheduling barriers
+        // keep the compiler from putting the two back in source order of dependence)
+        v4i acc[2];
+        acc[0] = product(0);
 #pragma unroll
-            for (int ks = 0; ks < KSE; ks++)
+        for (int pt = 0; pt < NXPT; pt++) {
+            if (pt + 1 < NXPT)
+                acc[(pt + 1) & 1] = product(pt + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            finish(acc[pt & 1], pt);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+#pragma unroll
+        for (int g0 = 0; g0 < NXPT; g0 += 4) {
+            if (EXACT || g0 < n_xpt) { // uniform
+                v4i acc[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++)
                     if (g0 + j < NXPT)
-                        acc[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], xb[(g0 + j) * KSE + ks],
-                                                                       ks == 0 ? c.init : acc[j], 0, 0, 0);
+                        acc[j] = product(g0 + j);
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                if (g0 + j < NXPT) {
-                    int word = wave_pack<MODE>(acc[j], c, floor_pk, relu, half_even);
-                    word &= __builtin_amdgcn_sbfe((int)xmask, g0 + j, 1); // all ones or zero
-                    *reinterpret_cast<int *>(dst + (g0 + j) * 256) = word;
-                }
+                for (int j = 0; j < 4; j++)
+                    if (g0 + j < NXPT)
+                        finish(acc[j], g0 + j);
             }
         }
     }
 }
 
 // Depthwise stage of one chunk of 16 channels.  S == 1: output rows in pairs, four patch rows per read.
-template <int MODE, int PT, int S, bool EXACT>
+template <int MODE, int PT, int S, bool EXACT, bool PIPE = false>
 __device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_l + (quad * pw + S * col) * 16 */,
                                                 int th, int pw, const v4i (&a0)[3], const v4i (&a1)[3],
                                                 const StageConsts &c, int floor_pk, bool relu, bool half_even,
                                                 unsigned char *dst /* lane's slot in output row 0 of the result */,
                                                 int row_bytes = 16 * kDws, bool write_ok = true)
 {
-    if constexpr (S == 1) {
+    if constexpr (EXACT && PIPE) {
+        // software pipeline over units (S == 1: a pair of output rows, S == 2: one output row): operand-B
+        // reads two units ahead, matrix products one unit ahead of the requantization
+        constexpr int UNITS = S == 1 ? (PT + 1) / 2 : PT;
+        constexpr int ROWS = S == 1 ? 2 : 1;
+        v4i b[3][3], acc[2][2];
+        auto read = [&](int u) {
+            const unsigned char *sp = src + (S == 1 ? 2 * u : S * u) * pw * 16;
+#pragma unroll
+            for (int kx = 0; kx < 3; kx++)
+                b[u % 3][kx] = *reinterpret_cast<const v4i *>(sp + 16 * kx);
+        };
+        auto products = [&](int u) {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                if (ROWS * u + r < PT) {
+                    const v4i(&aw)[3] = r == 0 ? a0 : a1;
+                    v4i v = __builtin_amdgcn_mfma_i32_16x16x64_i8(aw[0], b[u % 3][0], c.init, 0, 0, 0);
+                    v = __builtin_amdgcn_mfma_i32_16x16x64_i8(aw[1], b[u % 3][1], v, 0, 0, 0);
+                    acc[u & 1][r] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aw[2], b[u % 3][2], v, 0, 0, 0);
+                }
+            }
+        };
+        auto finish = [&](int u) {
+#pragma unroll
+            for (int r = 0; r < ROWS; r++) {
+                if (ROWS * u + r < PT) {
+                    const int w = wave_pack<MODE>(acc[u & 1][r], c, floor_pk, relu, half_even);
+                    if (write_ok)
+                        *reinterpret_cast<int *>(dst + (ROWS * u + r) * row_bytes) = w;
+                }
+            }
+        };
+        read(0);
+        if (UNITS > 1)
+            read(1);
+        products(0);
+#pragma unroll
+        for (int u = 0; u < UNITS; u++) {
+            if (u + 2 < UNITS)
+                read(u + 2);
+            if (u + 1 < UNITS)
+                products(u + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            finish(u);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else if constexpr (S == 1) {
 #pragma unroll
         for (int j = 0; j < (PT + 1) / 2; j++) {
             if (EXACT || 2 * j < th) { // uniform

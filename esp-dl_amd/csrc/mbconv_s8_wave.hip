@@ -48,6 +48,8 @@ namespace {
 
 using namespace mbstage;
 
+constexpr int kWavesPerGroup = 4;
+
 struct WaveArgs {
     MbconvParams p;
     int th, tw, ph, pw;
@@ -56,30 +58,49 @@ struct WaveArgs {
     int n_sub; // chunks of 16 expanded channels
     int rt;    // project row tiles of 16 filters
     int x_vec16, we_vec16;
-    int off_exp, off_dw, off_tab;
+    int off_exp, off_dw, off_tab, off_x;
+    int xlds;
+    int wave_bytes; // LDS of one wavefront (expanded patch + depthwise result); the tables are shared
     FastDiv fd_pw, fd_tiles_x, fd_tiles_yx;
 };
 
 // EXACT: the tile plan is exactly (NXPT pixel tiles, RT project row tiles, PT rows): no run-time guards in
 // the stage loops, so each stage of a chunk is one straight-line block the scheduler can interleave.  Rows
 // of a ragged last tile that do not exist are computed from whatever the patch area holds and never stored.
-template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT>
-__global__ __launch_bounds__(64) void mbconv_s8_wave_kernel(const WaveArgs a)
+// A workgroup is kWavesPerGroup wavefronts with a tile each; all they share is the requantization tables of
+// the expand and depthwise stages, which they build together (one barrier) before going their own ways.
+// XLDS: the block-input operands wait in LDS (each lane keeps its own 16 bytes per pixel tile there) instead of
+// in registers, and the project product runs after every chunk of 16 channels on a 16-byte-per-pixel depthwise
+// tile instead of after every 64: fewer registers and less LDS per wavefront, i.e. more wavefronts per SIMD,
+// for a quarter-filled project MFMA.
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool XLDS>
+__global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) void mbconv_s8_wave_kernel(const WaveArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const MbconvParams &p = a.p;
     const int lane = threadIdx.x & 63, col = lane & 15, quad = lane >> 4;
-    unsigned char *exp_l = smem + a.off_exp;
-    unsigned char *dw_l = smem + a.off_dw;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    unsigned char *exp_l = smem + a.off_exp + wave * a.wave_bytes;
+    unsigned char *dw_l = smem + a.off_dw + wave * a.wave_bytes;
     int *tab_e = reinterpret_cast<int *>(smem + a.off_tab);
     int *tab_d = tab_e + 3 * a.p.exp_c;
+    const int c0 = p.in_c;
+    const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
+    const int mode_e = build_stage_table_group(tab_e, p.b_expand, p.s_expand, p.n_s_expand, p.exp_c, bound_e, HE,
+                                               (int)threadIdx.x, 64 * kWavesPerGroup);
+    const int mode_d = build_stage_table_group(tab_d, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_d, HE, (int)threadIdx.x,
+                                               64 * kWavesPerGroup);
+    __syncthreads(); // tables complete; no barrier after this one
 
     // tile of this wavefront; consecutive tiles of an image stay on one XCD (its L2 holds the shared halo rows)
-    int tile = blockIdx.x;
+    int group = blockIdx.x;
     if ((gridDim.x & 7u) == 0) {
         const int per = gridDim.x >> 3;
-        tile = (int)(blockIdx.x & 7u) * per + (int)(blockIdx.x >> 3);
+        group = (int)(blockIdx.x & 7u) * per + (int)(blockIdx.x >> 3);
     }
+    const int tile = group * kWavesPerGroup + wave;
+    if (tile >= a.n_tiles)
+        return;
     const unsigned n = fastdiv((unsigned)tile, a.fd_tiles_yx);
     const unsigned rem = (unsigned)tile - n * a.fd_tiles_yx.d;
     const unsigned ty = fastdiv(rem, a.fd_tiles_x);
@@ -90,23 +111,33 @@ __global__ __launch_bounds__(64) void mbconv_s8_wave_kernel(const WaveArgs a)
     const int n_xpt = EXACT ? NXPT : a.n_xpt;
     const int n_rt = EXACT ? RT : a.rt;
 
-    // block-input patch -> operand B registers of the expand stage; xmask: patch pixels inside the image
-    const int c0 = p.in_c;
-    v4i xb[NXPT];
+    // block-input patch -> operand B of the expand stage (registers, or this lane's slots in LDS); xmask: patch
+    // pixels inside the image
+    v4i xb[XLDS ? 1 : NXPT];
     unsigned xmask = 0;
+    const int nq = (c0 + 15) >> 4; // 16-lane groups whose 16 k positions hold block-input channels
+    unsigned char *x_l = smem + a.off_x + wave * a.wave_bytes + (min(quad, nq - 1) * 16 + col) * 16;
+    const int x_tile_bytes = nq * 256;
     {
         const int8_t *img = p.in + (long long)n * p.in_h * p.in_w * c0;
 #pragma unroll
         for (int pt = 0; pt < NXPT; pt++) {
-            xb[pt] = v4i{0, 0, 0, 0};
+            if constexpr (!XLDS)
+                xb[pt] = v4i{0, 0, 0, 0};
             if (pt < n_xpt) { // uniform
                 const unsigned pp = (unsigned)(pt * 16 + col);
                 const unsigned prow = fastdiv(pp, a.fd_pw);
                 const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
                 const bool valid = (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
                 xmask |= valid ? 1u << pt : 0u;
-                xb[pt] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
-                                               valid ? c0 - 16 * quad : 0);
+                const v4i xv = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
+                                                     valid ? c0 - 16 * quad : 0);
+                if constexpr (XLDS) {
+                    if (quad < nq) // the other groups multiply zero filter bytes: whatever they read back is fine
+                        *reinterpret_cast<v4i *>(x_l + pt * x_tile_bytes) = xv;
+                } else {
+                    xb[pt] = xv;
+                }
             }
         }
     }
@@ -120,19 +151,15 @@ __global__ __launch_bounds__(64) void mbconv_s8_wave_kernel(const WaveArgs a)
 
     const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
     const int floor_d = p.relu_dw ? 0 : (int)0x80008000u;
-    const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
     unsigned char *exp_dst = exp_l + col * 16 + 4 * quad;
     const unsigned char *exp_src = exp_l + (quad * a.pw + S * col) * 16;
-
-    const int mode_e = build_stage_table(tab_e, p.b_expand, p.s_expand, p.n_s_expand, p.exp_c, bound_e, HE, lane);
-    const int mode_d = build_stage_table(tab_d, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_d, HE, lane);
-    wave_lds_sync();
 
     // Filters of a chunk are requested one chunk ahead (ChunkW), the project filters of a group of four
     // chunks at the start of the group: their latency hides behind the chunk in between.
     struct ChunkW {
         v4i aop[1];
         int wd0[3], wd1[3];
+        v4i ap[XLDS ? RT : 1]; // XLDS: project filter bytes of these 16 channels (k positions of lanes 0-15)
     };
     auto load_chunk = [&](int sub) {
         ChunkW w;
@@ -149,6 +176,12 @@ __global__ __launch_bounds__(64) void mbconv_s8_wave_kernel(const WaveArgs a)
                 w.wd1[kx] = quad >= 1 ? v1 : 0;
             }
         }
+        if constexpr (XLDS) {
+#pragma unroll
+            for (int r = 0; r < RT; r++)
+                w.ap[r] = load16_partial<true>(p.w_project, (unsigned)((16 * r + col) * p.exp_c + ch0),
+                                               (quad == 0 && r < n_rt && 16 * r + col < p.out_c) ? 16 : 0);
+        }
         return w;
     };
     v4i ap[RT];
@@ -164,20 +197,24 @@ __global__ __launch_bounds__(64) void mbconv_s8_wave_kernel(const WaveArgs a)
 
     ChunkW cur = load_chunk(0);
     for (int sub = 0; sub < a.n_sub; sub++) {
-        if ((sub & 3) == 0)
+        if (!XLDS && (sub & 3) == 0)
             load_project(sub);
         const ChunkW nxt = load_chunk(min(sub + 1, a.n_sub - 1));
         // ---- expand: 16 channels x every patch pixel
         {
             const StageConsts ce = read_stage_table(tab_e, p.exp_c, 16 * sub + 4 * quad, mode_e);
             if (ce.mode == 0)
-                expand_chunk<0, NXPT, EXACT>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<0, NXPT, EXACT, 1, XLDS, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, x_l,
+                                                       x_tile_bytes);
             else if (ce.mode == 1)
-                expand_chunk<1, NXPT, EXACT>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<1, NXPT, EXACT, 1, XLDS, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, x_l,
+                                                       x_tile_bytes);
             else if (ce.mode == 2)
-                expand_chunk<2, NXPT, EXACT>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<2, NXPT, EXACT, 1, XLDS, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, x_l,
+                                                       x_tile_bytes);
             else
-                expand_chunk<-1, NXPT, EXACT>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<-1, NXPT, EXACT, 1, XLDS, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, x_l,
+                                                       x_tile_bytes);
         }
         wave_lds_sync();
 
@@ -190,20 +227,37 @@ __global__ __launch_bounds__(64) void mbconv_s8_wave_kernel(const WaveArgs a)
                 a1[kx] = diag_operand(cur.wd1[kx], col);
             }
             const StageConsts cd = read_stage_table(tab_d, p.exp_c, 16 * sub + 4 * quad, mode_d);
-            unsigned char *dst = dw_l + col * kDws + 16 * (sub & 3) + 4 * quad;
+            unsigned char *dst = XLDS ? dw_l + col * 16 + 4 * quad : dw_l + col * kDws + 16 * (sub & 3) + 4 * quad;
             if (cd.mode == 0)
-                depthwise_chunk<0, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<0, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst,
+                                                  XLDS ? 256 : 16 * kDws);
             else if (cd.mode == 1)
-                depthwise_chunk<1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst,
+                                                  XLDS ? 256 : 16 * kDws);
             else if (cd.mode == 2)
-                depthwise_chunk<2, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<2, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst,
+                                                  XLDS ? 256 : 16 * kDws);
             else
-                depthwise_chunk<-1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<-1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst,
+                                                  XLDS ? 256 : 16 * kDws);
         }
         wave_lds_sync();
 
         // ---- project: accumulate over the 64 (or last few) expanded channels gathered so far
-        if ((sub & 3) == 3 || sub == a.n_sub - 1) {
+        if constexpr (XLDS) {
+            const unsigned char *bsrc = dw_l + col * 16; // the 16 channels of the chunk; lanes 16-63 multiply zeros
+#pragma unroll
+            for (int t = 0; t < PT; t++) {
+                if (EXACT || t < th) { // uniform
+                    const v4i b = *reinterpret_cast<const v4i *>(bsrc + t * 256);
+#pragma unroll
+                    for (int r = 0; r < RT; r++)
+                        if (EXACT || r < n_rt) // uniform
+                            accp[r][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.ap[r], b, accp[r][t], 0, 0, 0);
+                }
+            }
+            wave_lds_sync();
+        } else if ((sub & 3) == 3 || sub == a.n_sub - 1) {
             const unsigned char *bsrc = dw_l + col * kDws + 16 * quad;
 #pragma unroll
             for (int t = 0; t < PT; t++) {
@@ -283,6 +337,23 @@ struct WavePlan {
 
 constexpr int kPtMax = 8;
 
+// LDS layout: the tables (shared by the wavefronts of a group), then per wavefront the expanded patch of one
+// chunk (16 bytes per pixel; the depthwise reads run up to one row and a few pixels past the patch, into
+// products with zero weights or into discarded columns), the depthwise result and, in the XLDS form, the
+// block-input operands.
+void wave_layout(WaveArgs &a, bool xlds, size_t *lds)
+{
+    const int exp_px = std::max(((a.n_xpt + 3) & ~3) * 16, (a.ph * a.pw + 48 + 15) & ~15);
+    a.off_tab = 0; // two stages x [init | rsh | lsh] x int32
+    a.off_exp = a.p.exp_c * 24;
+    a.off_dw = a.off_exp + exp_px * 16;
+    a.xlds = xlds ? 1 : 0;
+    const int dw_bytes = xlds ? a.th * 256 : a.th * 16 * kDws;
+    a.off_x = a.off_dw + dw_bytes;
+    a.wave_bytes = exp_px * 16 + dw_bytes + (xlds ? a.n_xpt * ((a.p.in_c + 15) / 16) * 256 : 0);
+    *lds = (size_t)a.off_exp + (size_t)kWavesPerGroup * a.wave_bytes;
+}
+
 WavePlan wave_plan(const MbconvParams &p)
 {
     WavePlan plan;
@@ -328,15 +399,8 @@ WavePlan wave_plan(const MbconvParams &p)
     a.rt = (p.out_c + 15) / 16;
     a.x_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.in) & 15) == 0) ? 1 : 0;
     a.we_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.w_expand) & 15) == 0) ? 1 : 0;
-    // LDS: expanded patch of one chunk (16 bytes per pixel; the depthwise reads run up to three rows and a
-    // few pixels past the patch, into products with zero weights or into discarded columns) and the
-    // depthwise result of 64 channels
-    const int exp_px = std::max(((a.n_xpt + 3) & ~3) * 16, (a.ph + 3) * a.pw + 64);
-    a.off_exp = 0;
-    a.off_dw = exp_px * 16;
-    a.off_tab = a.off_dw + kPtMax * 16 * kDws;
-    plan.lds = (size_t)a.off_tab + (size_t)p.exp_c * 24; // two stages x [init | rsh | lsh] x int32
-    if (plan.lds > 40 * 1024)
+    wave_layout(a, false, &plan.lds);
+    if (plan.lds > 64 * 1024)
         return plan;
     a.fd_pw = make_fastdiv((unsigned)a.pw);
     a.fd_tiles_x = make_fastdiv((unsigned)a.tiles_x);
@@ -352,8 +416,13 @@ template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT>
 hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
 {
     const WaveArgs &a = plan.a;
-    hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT>), dim3((unsigned)a.n_tiles), dim3(64),
-                       plan.lds, stream, a);
+    const unsigned groups = (unsigned)((a.n_tiles + kWavesPerGroup - 1) / kWavesPerGroup);
+    if (EXACT && a.xlds)
+        hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, EXACT>), dim3(groups),
+                           dim3(64 * kWavesPerGroup), plan.lds, stream, a);
+    else
+        hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, false>), dim3(groups),
+                           dim3(64 * kWavesPerGroup), plan.lds, stream, a);
     return hipGetLastError();
 }
 
@@ -365,15 +434,19 @@ hipError_t launch_generic(const WavePlan &plan, hipStream_t stream)
                                                : launch_one<17, 4, kPtMax, S, HE, false, false>(plan, stream);
 }
 
-hipError_t launch_planned(const WavePlan &plan, hipStream_t stream)
+hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
 {
-    const WaveArgs &a = plan.a;
+    static const bool use_xlds = getenv("ESPDL_HIP_WAVE_XLDS") != nullptr && atoi(getenv("ESPDL_HIP_WAVE_XLDS")) != 0;
+    WaveArgs &a = plan.a;
     const bool vec16 = a.x_vec16 && a.we_vec16;
     const int s = a.p.stride_h;
     if (!a.p.half_even) {
         // guard-free builds for the tile plans of MobileNetV2-style blocks (round half up)
         const auto is = [&](int nxpt, int rt, int th, int stride, bool v) {
-            return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v;
+            const bool hit = a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v;
+            if (hit && use_xlds)
+                wave_layout(a, true, &plan.lds); // the guard-free builds exist in the XLDS form
+            return hit;
         };
         if (is(17, 2, 4, 2, true))
             return launch_one<17, 2, 4, 2, false, true, true>(plan, stream);
@@ -387,8 +460,6 @@ hipError_t launch_planned(const WavePlan &plan, hipStream_t stream)
             return launch_one<9, 2, 7, 1, false, true, true>(plan, stream);
         if (is(13, 4, 3, 2, true))
             return launch_one<13, 4, 3, 2, false, true, true>(plan, stream);
-        if (is(9, 4, 7, 1, true))
-            return launch_one<9, 4, 7, 1, false, true, true>(plan, stream);
         return s == 1 ? launch_generic<1, false>(plan, stream) : launch_generic<2, false>(plan, stream);
     }
     return s == 1 ? launch_generic<1, true>(plan, stream) : launch_generic<2, true>(plan, stream);
