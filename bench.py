@@ -46,9 +46,12 @@ MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
 def kernel_family(info, spec_nodes):
     """Map a module to the kernel that runs it."""
     node = spec_nodes.get(info["name"])
-    if info["type"] == "Conv>DepthwiseConv>Conv":
-        return "mbconv_s8"  # expand + depthwise + project (+ Add) in one launch
-    if info["type"] == "DepthwiseConv>Conv":
+    kind, _, kernel = info["type"].partition(":")
+    if kind == "Conv>DepthwiseConv>Conv":
+        # expand + depthwise + project (+ Add) in one launch: the one-wavefront-per-tile kernel for the large
+        # images, the workgroup-per-tile kernel for the small ones
+        return "mbconv_s8_" + kernel if kernel in ("wave", "group") else "mbconv_s8"
+    if kind == "DepthwiseConv>Conv":
         return "depthwise_s8"  # depthwise + project (+ Add) in one launch of the depthwise kernel
     if info["type"] in ("Gemm", "MatMul"):
         return "conv2d_s8"
@@ -227,7 +230,7 @@ def main():
     dom = max(kernels, key=lambda k: kernels[k]["us_per_step"])
     kd = kernels[dom]
     # time per family comes from whole passes in plan order, so the family times add up to a step
-    if dom in ("conv2d_s8", "mbconv_s8") and kd["ops_per_byte"] > MACHINE_BALANCE:
+    if (dom == "conv2d_s8" or dom.startswith("mbconv_s8")) and kd["ops_per_byte"] > MACHINE_BALANCE:
         roofline = {"kernel": dom, "bound": "mfma", "achieved": kd["TOPs"], "peak": PEAK_INT8_TOPS,
                     "unit": "TOP/s", "frac": kd["mfma_frac"], "traffic": None}
     else:

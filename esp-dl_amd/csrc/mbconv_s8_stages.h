@@ -210,25 +210,16 @@ __device__ __forceinline__ int wave_pack(const v4i &acc, const StageConsts &c, i
 // Expand stage of one chunk of 16 channels: every patch pixel tile through one MFMA and the epilogue, four
 // tiles at a time so that four independent MFMA -> requantize -> store chains are in flight (tiles past
 // n_xpt inside the last group of four have zero operands and a zero mask and land in slack).
-template <int MODE, int NXPT, bool EXACT, int KSE = 1, bool XLDS = false, bool PIPE = false>
-__device__ __forceinline__ void expand_chunk(const v4i (&xb)[XLDS ? 1 : NXPT * KSE], int n_xpt, unsigned xmask,
+template <int MODE, int NXPT, bool EXACT, int KSE = 1, bool PIPE = false>
+__device__ __forceinline__ void expand_chunk(const v4i (&xb)[NXPT * KSE], int n_xpt, unsigned xmask,
                                              const v4i (&aop)[KSE], const StageConsts &c, int floor_pk, bool relu,
-                                             bool half_even, unsigned char *dst /* exp_l + col * 16 + 4 * quad */,
-                                             const unsigned char *xsrc = nullptr, int x_tile_bytes = 0)
+                                             bool half_even, unsigned char *dst /* exp_l + col * 16 + 4 * quad */)
 {
-    // XLDS: operand B of pixel tile pt and k step ks sits in LDS at xsrc + (pt * KSE + ks) * x_tile_bytes
-    // (where this lane put it), not in registers
-    auto operand = [&](int pt, int ks) -> v4i {
-        if constexpr (XLDS)
-            return *reinterpret_cast<const v4i *>(xsrc + (pt * KSE + ks) * x_tile_bytes);
-        else
-            return xb[pt * KSE + ks];
-    };
     auto product = [&](int pt) -> v4i {
         v4i acc = c.init;
 #pragma unroll
         for (int ks = 0; ks < KSE; ks++)
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], operand(pt, ks), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], xb[pt * KSE + ks], acc, 0, 0, 0);
         return acc;
     };
     auto finish = [&](const v4i &acc, int pt) {

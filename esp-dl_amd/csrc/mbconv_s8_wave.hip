@@ -58,8 +58,7 @@ struct WaveArgs {
     int n_sub; // chunks of 16 expanded channels
     int rt;    // project row tiles of 16 filters
     int x_vec16, we_vec16;
-    int off_exp, off_dw, off_tab, off_x;
-    int xlds;
+    int off_exp, off_dw, off_tab;
     int wave_bytes; // LDS of one wavefront (expanded patch + depthwise result); the tables are shared
     FastDiv fd_pw, fd_tiles_x, fd_tiles_yx;
 };
@@ -69,12 +68,11 @@ struct WaveArgs {
 // of a ragged last tile that do not exist are computed from whatever the patch area holds and never stored.
 // A workgroup is kWavesPerGroup wavefronts with a tile each; all they share is the requantization tables of
 // the expand and depthwise stages, which they build together (one barrier) before going their own ways.
-// XLDS: the block-input operands wait in LDS (each lane keeps its own 16 bytes per pixel tile there) instead of
-// in registers, and the project product runs after every chunk of 16 channels on a 16-byte-per-pixel depthwise
-// tile instead of after every 64: fewer registers and less LDS per wavefront, i.e. more wavefronts per SIMD,
-// for a quarter-filled project MFMA.
-template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool XLDS>
-__global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) void mbconv_s8_wave_kernel(const WaveArgs a)
+// Everything a tile reads from memory up front (its block-input patch, the residual words it will add at the
+// very end, the filters of its first chunk) is requested BEFORE the tables are built, so that one memory
+// round trip covers all of it.
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT>
+__global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_wave_kernel(const WaveArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const MbconvParams &p = a.p;
@@ -85,22 +83,16 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) vo
     int *tab_e = reinterpret_cast<int *>(smem + a.off_tab);
     int *tab_d = tab_e + 3 * a.p.exp_c;
     const int c0 = p.in_c;
-    const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
-    const int mode_e = build_stage_table_group(tab_e, p.b_expand, p.s_expand, p.n_s_expand, p.exp_c, bound_e, HE,
-                                               (int)threadIdx.x, 64 * kWavesPerGroup);
-    const int mode_d = build_stage_table_group(tab_d, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_d, HE, (int)threadIdx.x,
-                                               64 * kWavesPerGroup);
-    __syncthreads(); // tables complete; no barrier after this one
 
-    // tile of this wavefront; consecutive tiles of an image stay on one XCD (its L2 holds the shared halo rows)
+    // tile of this wavefront; consecutive tiles of an image stay on one XCD (its L2 holds the shared halo rows).
+    // A wavefront past the last tile works on the last tile again and stores nothing.
     int group = blockIdx.x;
     if ((gridDim.x & 7u) == 0) {
         const int per = gridDim.x >> 3;
         group = (int)(blockIdx.x & 7u) * per + (int)(blockIdx.x >> 3);
     }
-    const int tile = group * kWavesPerGroup + wave;
-    if (tile >= a.n_tiles)
-        return;
+    const bool has_tile = group * kWavesPerGroup + wave < a.n_tiles; // uniform
+    const int tile = min(group * kWavesPerGroup + wave, a.n_tiles - 1);
     const unsigned n = fastdiv((unsigned)tile, a.fd_tiles_yx);
     const unsigned rem = (unsigned)tile - n * a.fd_tiles_yx.d;
     const unsigned ty = fastdiv(rem, a.fd_tiles_x);
@@ -111,55 +103,38 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) vo
     const int n_xpt = EXACT ? NXPT : a.n_xpt;
     const int n_rt = EXACT ? RT : a.rt;
 
-    // block-input patch -> operand B of the expand stage (registers, or this lane's slots in LDS); xmask: patch
-    // pixels inside the image
-    v4i xb[XLDS ? 1 : NXPT];
+    // block-input patch -> operand B registers of the expand stage; xmask: patch pixels inside the image
+    v4i xb[NXPT];
     unsigned xmask = 0;
-    const int nq = (c0 + 15) >> 4; // 16-lane groups whose 16 k positions hold block-input channels
-    unsigned char *x_l = smem + a.off_x + wave * a.wave_bytes + (min(quad, nq - 1) * 16 + col) * 16;
-    const int x_tile_bytes = nq * 256;
     {
         const int8_t *img = p.in + (long long)n * p.in_h * p.in_w * c0;
 #pragma unroll
         for (int pt = 0; pt < NXPT; pt++) {
-            if constexpr (!XLDS)
-                xb[pt] = v4i{0, 0, 0, 0};
+            xb[pt] = v4i{0, 0, 0, 0};
             if (pt < n_xpt) { // uniform
                 const unsigned pp = (unsigned)(pt * 16 + col);
                 const unsigned prow = fastdiv(pp, a.fd_pw);
                 const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
                 const bool valid = (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
                 xmask |= valid ? 1u << pt : 0u;
-                const v4i xv = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
-                                                     valid ? c0 - 16 * quad : 0);
-                if constexpr (XLDS) {
-                    if (quad < nq) // the other groups multiply zero filter bytes: whatever they read back is fine
-                        *reinterpret_cast<v4i *>(x_l + pt * x_tile_bytes) = xv;
-                } else {
-                    xb[pt] = xv;
-                }
+                xb[pt] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
+                                               valid ? c0 - 16 * quad : 0);
             }
         }
     }
 
-    v4i accp[RT][PT];
-#pragma unroll
-    for (int r = 0; r < RT; r++)
-#pragma unroll
-        for (int t = 0; t < PT; t++)
-            accp[r][t] = v4i{0, 0, 0, 0};
-
-    const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
-    const int floor_d = p.relu_dw ? 0 : (int)0x80008000u;
-    unsigned char *exp_dst = exp_l + col * 16 + 4 * quad;
-    const unsigned char *exp_src = exp_l + (quad * a.pw + S * col) * 16;
-
+    // output words of this lane: pixel (oy0 + t, ox0 + col), filters 16 r + 4 quad ...
+    const int ox = ox0 + col;
+    const bool col_ok = has_tile && col < a.tw && ox < p.out_w;
+    const long long img_off = (long long)n * p.out_h * p.out_w * p.out_c;
+    const int8_t *res_img = p.residual != nullptr ? p.residual + img_off : nullptr;
+    int8_t *out_img = p.out + img_off;
+    const unsigned off0 = (unsigned)((oy0 * p.out_w + ox) * p.out_c + 4 * quad);
     // Filters of a chunk are requested one chunk ahead (ChunkW), the project filters of a group of four
     // chunks at the start of the group: their latency hides behind the chunk in between.
     struct ChunkW {
         v4i aop[1];
         int wd0[3], wd1[3];
-        v4i ap[XLDS ? RT : 1]; // XLDS: project filter bytes of these 16 channels (k positions of lanes 0-15)
     };
     auto load_chunk = [&](int sub) {
         ChunkW w;
@@ -176,12 +151,6 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) vo
                 w.wd1[kx] = quad >= 1 ? v1 : 0;
             }
         }
-        if constexpr (XLDS) {
-#pragma unroll
-            for (int r = 0; r < RT; r++)
-                w.ap[r] = load16_partial<true>(p.w_project, (unsigned)((16 * r + col) * p.exp_c + ch0),
-                                               (quad == 0 && r < n_rt && 16 * r + col < p.out_c) ? 16 : 0);
-        }
         return w;
     };
     v4i ap[RT];
@@ -189,32 +158,47 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) vo
         const int kc = (sub & ~3) * 16;
         const int nk = p.exp_c - kc - 16 * quad; // valid bytes of this lane's 16 k positions
 #pragma unroll
-        for (int r = 0; r < RT; r++) {
+        for (int r = 0; r < RT; r++)
             ap[r] = load16_partial<true>(p.w_project, (unsigned)((16 * r + col) * p.exp_c + kc + 16 * quad),
                                          (r < n_rt && 16 * r + col < p.out_c) ? nk : 0);
-        }
     };
-
     ChunkW cur = load_chunk(0);
+
+    // the stage tables, by the whole group
+    const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
+    const int mode_e = build_stage_table_group(tab_e, p.b_expand, p.s_expand, p.n_s_expand, p.exp_c, bound_e, HE,
+                                               (int)threadIdx.x, 64 * kWavesPerGroup);
+    const int mode_d = build_stage_table_group(tab_d, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_d, HE, (int)threadIdx.x,
+                                               64 * kWavesPerGroup);
+    __syncthreads(); // tables complete; no barrier after this one
+
+    v4i accp[RT][PT];
+#pragma unroll
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < PT; t++)
+            accp[r][t] = v4i{0, 0, 0, 0};
+
+    const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
+    const int floor_d = p.relu_dw ? 0 : (int)0x80008000u;
+    unsigned char *exp_dst = exp_l + col * 16 + 4 * quad;
+    const unsigned char *exp_src = exp_l + (quad * a.pw + S * col) * 16;
+
     for (int sub = 0; sub < a.n_sub; sub++) {
-        if (!XLDS && (sub & 3) == 0)
+        if ((sub & 3) == 0)
             load_project(sub);
         const ChunkW nxt = load_chunk(min(sub + 1, a.n_sub - 1));
         // ---- expand: 16 channels x every patch pixel
         {
             const StageConsts ce = read_stage_table(tab_e, p.exp_c, 16 * sub + 4 * quad, mode_e);
             if (ce.mode == 0)
-                expand_chunk<0, NXPT, EXACT, 1, XLDS, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, x_l,
-                                                       x_tile_bytes);
+                expand_chunk<0, NXPT, EXACT, 1, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else if (ce.mode == 1)
-                expand_chunk<1, NXPT, EXACT, 1, XLDS, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, x_l,
-                                                       x_tile_bytes);
+                expand_chunk<1, NXPT, EXACT, 1, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else if (ce.mode == 2)
-                expand_chunk<2, NXPT, EXACT, 1, XLDS, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, x_l,
-                                                       x_tile_bytes);
+                expand_chunk<2, NXPT, EXACT, 1, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else
-                expand_chunk<-1, NXPT, EXACT, 1, XLDS, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, x_l,
-                                                       x_tile_bytes);
+                expand_chunk<-1, NXPT, EXACT, 1, true>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
         }
         wave_lds_sync();
 
@@ -227,37 +211,20 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) vo
                 a1[kx] = diag_operand(cur.wd1[kx], col);
             }
             const StageConsts cd = read_stage_table(tab_d, p.exp_c, 16 * sub + 4 * quad, mode_d);
-            unsigned char *dst = XLDS ? dw_l + col * 16 + 4 * quad : dw_l + col * kDws + 16 * (sub & 3) + 4 * quad;
+            unsigned char *dst = dw_l + col * kDws + 16 * (sub & 3) + 4 * quad;
             if (cd.mode == 0)
-                depthwise_chunk<0, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst,
-                                                  XLDS ? 256 : 16 * kDws);
+                depthwise_chunk<0, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
             else if (cd.mode == 1)
-                depthwise_chunk<1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst,
-                                                  XLDS ? 256 : 16 * kDws);
+                depthwise_chunk<1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
             else if (cd.mode == 2)
-                depthwise_chunk<2, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst,
-                                                  XLDS ? 256 : 16 * kDws);
+                depthwise_chunk<2, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
             else
-                depthwise_chunk<-1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst,
-                                                  XLDS ? 256 : 16 * kDws);
+                depthwise_chunk<-1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
         }
         wave_lds_sync();
 
         // ---- project: accumulate over the 64 (or last few) expanded channels gathered so far
-        if constexpr (XLDS) {
-            const unsigned char *bsrc = dw_l + col * 16; // the 16 channels of the chunk; lanes 16-63 multiply zeros
-#pragma unroll
-            for (int t = 0; t < PT; t++) {
-                if (EXACT || t < th) { // uniform
-                    const v4i b = *reinterpret_cast<const v4i *>(bsrc + t * 256);
-#pragma unroll
-                    for (int r = 0; r < RT; r++)
-                        if (EXACT || r < n_rt) // uniform
-                            accp[r][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(cur.ap[r], b, accp[r][t], 0, 0, 0);
-                }
-            }
-            wave_lds_sync();
-        } else if ((sub & 3) == 3 || sub == a.n_sub - 1) {
+        if ((sub & 3) == 3 || sub == a.n_sub - 1) {
             const unsigned char *bsrc = dw_l + col * kDws + 16 * quad;
 #pragma unroll
             for (int t = 0; t < PT; t++) {
@@ -274,14 +241,21 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) vo
         cur = nxt;
     }
 
-    // ---- project epilogue, residual Add, stores: lane = output pixel (oy0 + t, ox0 + col) x 4 filters
+    // ---- project epilogue, residual Add, stores; every residual word is requested before the first is used
+    int resw[RT][PT];
+#pragma unroll
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < PT; t++) {
+            resw[r][t] = 0;
+            if (res_img != nullptr) { // uniform
+                const bool live = col_ok && t < th_real && 16 * r + 4 * quad < p.out_c;
+                resw[r][t] = *reinterpret_cast<const int *>(
+                    res_img + (size_t)(live ? off0 + (unsigned)(t * p.out_w * p.out_c + 16 * r) : 0u));
+            }
+        }
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
     const unsigned bound_p = (unsigned)p.exp_c * 16384u;
-    const int ox = ox0 + col;
-    const bool col_ok = col < a.tw && ox < p.out_w;
-    const long long img_off = (long long)n * p.out_h * p.out_w * p.out_c;
-    const int8_t *res_img = p.residual != nullptr ? p.residual + img_off : nullptr;
-    int8_t *out_img = p.out + img_off;
 #pragma unroll
     for (int r = 0; r < RT; r++) {
         if (r < n_rt) { // uniform
@@ -290,7 +264,6 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) vo
             load_bias_shift(p.b_project, p.s_project, p.n_s_project, c, p.out_c, bp, sp);
             const StageConsts cp = stage_consts(bp, sp, bound_p, HE);
             const bool live = col_ok && c < p.out_c;
-            const unsigned off0 = (unsigned)((oy0 * p.out_w + ox) * p.out_c + c);
             auto rows = [&](auto mode_tag) {
                 constexpr int MODE = decltype(mode_tag)::value;
 #pragma unroll
@@ -300,19 +273,17 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, XLDS ? 3 : (EXACT ? 2 : 1)) vo
 #pragma unroll
                         for (int k = 0; k < 4; k++)
                             acc[k] += cp.init[k];
-                        const unsigned off = off0 + (unsigned)(t * p.out_w * p.out_c);
                         int word;
                         if (res_img != nullptr) { // uniform
-                            const int rv = *reinterpret_cast<const int *>(res_img + (size_t)(live ? off : 0u));
                             if constexpr (MODE >= 0)
-                                word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, rv);
+                                word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, resw[r][t]);
                             else
-                                word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), rv);
+                                word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), resw[r][t]);
                         } else {
                             word = wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE);
                         }
                         if (live)
-                            *reinterpret_cast<int *>(out_img + (size_t)off) = word;
+                            *reinterpret_cast<int *>(out_img + (size_t)(off0 + (unsigned)(t * p.out_w * p.out_c + 16 * r))) = word;
                     }
                 }
             };
@@ -339,18 +310,14 @@ constexpr int kPtMax = 8;
 
 // LDS layout: the tables (shared by the wavefronts of a group), then per wavefront the expanded patch of one
 // chunk (16 bytes per pixel; the depthwise reads run up to one row and a few pixels past the patch, into
-// products with zero weights or into discarded columns), the depthwise result and, in the XLDS form, the
-// block-input operands.
-void wave_layout(WaveArgs &a, bool xlds, size_t *lds)
+// products with zero weights or into discarded columns) and the depthwise result of 64 channels.
+void wave_layout(WaveArgs &a, size_t *lds)
 {
     const int exp_px = std::max(((a.n_xpt + 3) & ~3) * 16, (a.ph * a.pw + 48 + 15) & ~15);
     a.off_tab = 0; // two stages x [init | rsh | lsh] x int32
     a.off_exp = a.p.exp_c * 24;
     a.off_dw = a.off_exp + exp_px * 16;
-    a.xlds = xlds ? 1 : 0;
-    const int dw_bytes = xlds ? a.th * 256 : a.th * 16 * kDws;
-    a.off_x = a.off_dw + dw_bytes;
-    a.wave_bytes = exp_px * 16 + dw_bytes + (xlds ? a.n_xpt * ((a.p.in_c + 15) / 16) * 256 : 0);
+    a.wave_bytes = exp_px * 16 + a.th * 16 * kDws;
     *lds = (size_t)a.off_exp + (size_t)kWavesPerGroup * a.wave_bytes;
 }
 
@@ -399,7 +366,7 @@ WavePlan wave_plan(const MbconvParams &p)
     a.rt = (p.out_c + 15) / 16;
     a.x_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.in) & 15) == 0) ? 1 : 0;
     a.we_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.w_expand) & 15) == 0) ? 1 : 0;
-    wave_layout(a, false, &plan.lds);
+    wave_layout(a, &plan.lds);
     if (plan.lds > 64 * 1024)
         return plan;
     a.fd_pw = make_fastdiv((unsigned)a.pw);
@@ -417,12 +384,8 @@ hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
 {
     const WaveArgs &a = plan.a;
     const unsigned groups = (unsigned)((a.n_tiles + kWavesPerGroup - 1) / kWavesPerGroup);
-    if (EXACT && a.xlds)
-        hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, EXACT>), dim3(groups),
-                           dim3(64 * kWavesPerGroup), plan.lds, stream, a);
-    else
-        hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, false>), dim3(groups),
-                           dim3(64 * kWavesPerGroup), plan.lds, stream, a);
+    hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT>), dim3(groups),
+                       dim3(64 * kWavesPerGroup), plan.lds, stream, a);
     return hipGetLastError();
 }
 
@@ -436,17 +399,13 @@ hipError_t launch_generic(const WavePlan &plan, hipStream_t stream)
 
 hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
 {
-    static const bool use_xlds = getenv("ESPDL_HIP_WAVE_XLDS") != nullptr && atoi(getenv("ESPDL_HIP_WAVE_XLDS")) != 0;
     WaveArgs &a = plan.a;
     const bool vec16 = a.x_vec16 && a.we_vec16;
     const int s = a.p.stride_h;
     if (!a.p.half_even) {
         // guard-free builds for the tile plans of MobileNetV2-style blocks (round half up)
         const auto is = [&](int nxpt, int rt, int th, int stride, bool v) {
-            const bool hit = a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v;
-            if (hit && use_xlds)
-                wave_layout(a, true, &plan.lds); // the guard-free builds exist in the XLDS form
-            return hit;
+            return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v;
         };
         if (is(17, 2, 4, 2, true))
             return launch_one<17, 2, 4, 2, false, true, true>(plan, stream);

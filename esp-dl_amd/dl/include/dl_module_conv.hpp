@@ -58,6 +58,7 @@ private:
     // A depthwise Conv that absorbed its project Conv may also absorb the 1x1 Conv in front of it: its first
     // input is then the block input and the expanded tensor is never materialized.
     bool m_has_expand = false;
+    int m_fused_kernel = 0;
     activation_type_t m_expand_activation = Linear;
     int m_expand_exponent = 0; ///< exponent of the (no longer materialized) expanded tensor
     int m_expand_filter_pos = -1, m_expand_bias_pos = -1;
@@ -134,6 +135,9 @@ public:
         }
     }
     bool has_fused_expand() const { return m_has_expand; }
+    /// answer of espdl_hip_mbconv_s8_supported for the fused form at its last forward (0 before the first):
+    /// which single-launch kernel runs it
+    int fused_kernel() const { return m_fused_kernel; }
     /// Absorb the Add that follows a dense Conv: `residual_index` is the Add's other operand and
     /// `own_out_exponent` the exponent of the tensor the Conv used to write.  The Add sums stored integers
     /// whatever the exponents of its operands and result are (esp-dl/dl/base/dl_base_add.cpp:35-44), so the
@@ -347,6 +351,7 @@ public:
         d.n_shift_expand = m_has_expand ? (int32_t)s_ex.size() : 1;
         d.n_shift_dw = (int32_t)s_dw.size();
         d.n_shift_project = (int32_t)s_pj.size();
+        m_fused_kernel = espdl_hip_mbconv_s8_supported(&d);
         espdl_hip_mbconv_weights w = {};
         if (m_has_expand) {
             w.w_expand = static_cast<const int8_t *>(efilter->data);

@@ -882,10 +882,14 @@ std::vector<module_info> Model::get_module_info(int repeats)
         mi.type = m_fbs_model->get_operation_type(module->name);
         if (auto *conv = dynamic_cast<dl::module::Conv *>(module)) {
             // a Conv that absorbed its neighbours reports what it runs
+            // and, after a colon, which single-launch kernel took it (the espdl_hip_mbconv_s8_supported answer)
+            static const char *const kKernel[] = {"", ":fused", ":lds", ":lds", ":wave", ":group"};
+            const int k = conv->fused_kernel();
+            const char *suffix = k >= 0 && k <= 5 ? kKernel[k] : "";
             if (conv->has_fused_expand())
-                mi.type = "Conv>DepthwiseConv>Conv";
+                mi.type = std::string("Conv>DepthwiseConv>Conv") + suffix;
             else if (conv->has_fused_project())
-                mi.type = "DepthwiseConv>Conv";
+                mi.type = std::string("DepthwiseConv>Conv") + suffix;
         }
         mi.latency_us = (float)std::max(0.0, (total_ms[i] / repeats - gap_ms) * 1000.0);
         std::vector<std::vector<int>> in_shapes;
