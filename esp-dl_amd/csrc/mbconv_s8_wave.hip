@@ -13,10 +13,11 @@
 // Why one wavefront per tile: the block is a chain of small dependent stages (a matrix product, a
 // requantization on the vector ALU, a trip through LDS, the next matrix product ...).  A workgroup that
 // walks the chain with barriers between the stages leaves every pipe idle most of the time.  Here a
-// workgroup IS one wavefront: it owns a th x tw tile of the block's output in one image and runs the
-// whole chain on its own, ordered only by its own LDS accesses; eight to sixteen such wavefronts per
-// compute unit sit at different points of the chain, so the matrix pipe, the vector ALU, LDS and the
-// memory pipeline of the unit are all busy at once.
+// wavefront owns a th x tw tile of the block's output in one image and runs the whole chain on its own,
+// ordered only by its own LDS accesses; the wavefronts of a compute unit sit at different points of the
+// chain, so the matrix pipe, the vector ALU, LDS and the memory pipeline of the unit are busy at once.
+// Four wavefronts form a workgroup for one reason only: they share the per-channel requantization tables
+// of the two inner stages, built once in LDS before the single barrier of the kernel.
 //
 // Per tile:
 //   * the (th*s + 2) x (tw*s + 2) patch of the block input is loaded ONCE, straight into the registers
