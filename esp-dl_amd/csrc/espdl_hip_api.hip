@@ -673,16 +673,41 @@ int mbconv_geometry(const espdl_hip_mbconv_desc *d, espdl::MbconvParams *p)
         return fail(ESPDL_HIP_EINVAL, "bad mbconv geometry");
     if (!d->has_expand && d->exp_c != d->in_c)
         return fail(ESPDL_HIP_EINVAL, "without an expand stage exp_c must equal in_c");
+    // expand stage with a window: the depthwise stage reads that convolution's output
+    const bool windowed = d->exp_k_h != 0 || d->exp_k_w != 0 || d->exp_stride_h != 0 || d->exp_stride_w != 0 ||
+        d->exp_pad_top != 0 || d->exp_pad_bottom != 0 || d->exp_pad_left != 0 || d->exp_pad_right != 0;
+    int mid_h = d->in_h, mid_w = d->in_w;
+    if (windowed) {
+        if (!d->has_expand)
+            return fail(ESPDL_HIP_EINVAL, "exp_k_* / exp_stride_* / exp_pad_* describe the expand stage: has_expand must be set");
+        if (d->exp_k_h <= 0 || d->exp_k_w <= 0 || d->exp_stride_h <= 0 || d->exp_stride_w <= 0 || d->exp_pad_top < 0 ||
+            d->exp_pad_bottom < 0 || d->exp_pad_left < 0 || d->exp_pad_right < 0)
+            return fail(ESPDL_HIP_EINVAL, "bad expand-stage geometry");
+        const int eh = d->in_h + d->exp_pad_top + d->exp_pad_bottom - d->exp_k_h;
+        const int ew = d->in_w + d->exp_pad_left + d->exp_pad_right - d->exp_k_w;
+        if (eh < 0 || ew < 0)
+            return fail(ESPDL_HIP_EINVAL, "expand filter larger than the padded input");
+        mid_h = eh / d->exp_stride_h + 1;
+        mid_w = ew / d->exp_stride_w + 1;
+    }
     const int eff_h = (d->k_h - 1) * d->dil_h + 1, eff_w = (d->k_w - 1) * d->dil_w + 1;
-    const int span_h = d->in_h + d->pad_top + d->pad_bottom - eff_h, span_w = d->in_w + d->pad_left + d->pad_right - eff_w;
+    const int span_h = mid_h + d->pad_top + d->pad_bottom - eff_h, span_w = mid_w + d->pad_left + d->pad_right - eff_w;
     if (span_h < 0 || span_w < 0)
         return fail(ESPDL_HIP_EINVAL, "depthwise filter larger than the padded input");
     if ((d->has_expand && d->n_shift_expand != 1 && d->n_shift_expand != d->exp_c) ||
         (d->n_shift_dw != 1 && d->n_shift_dw != d->exp_c) || (d->n_shift_project != 1 && d->n_shift_project != d->out_c))
         return fail(ESPDL_HIP_EINVAL, "n_shift_* must be 1 or the channel count of the stage");
     p->batch = d->batch;
-    p->in_h = d->in_h;
-    p->in_w = d->in_w;
+    p->in_h = mid_h;
+    p->in_w = mid_w;
+    p->img_h = d->in_h;
+    p->img_w = d->in_w;
+    p->ek_h = windowed ? d->exp_k_h : 1;
+    p->ek_w = windowed ? d->exp_k_w : 1;
+    p->es_h = windowed ? d->exp_stride_h : 1;
+    p->es_w = windowed ? d->exp_stride_w : 1;
+    p->epad_top = d->exp_pad_top;
+    p->epad_left = d->exp_pad_left;
     p->in_c = d->in_c;
     p->exp_c = d->exp_c;
     p->out_c = d->out_c;
@@ -706,6 +731,13 @@ int mbconv_geometry(const espdl_hip_mbconv_desc *d, espdl::MbconvParams *p)
     if ((long long)p->batch * p->out_h * p->out_w > 0x7fffffffll - 65536)
         return fail(ESPDL_HIP_EINVAL, "too many output pixels");
     return ESPDL_HIP_OK;
+}
+
+// Only the one-wavefront-per-tile kernel takes an expand stage with a window; every other form reads the
+// block input as the depthwise stage's input grid.
+bool pointwise_expand(const espdl::MbconvParams &p)
+{
+    return espdl::mbconv_expand_is_pointwise(p);
 }
 
 // Depthwise geometry and project description of a block without expand stage.
@@ -790,7 +822,9 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
         if (espdl::depthwise_project_s8_supports(g, p.in, pj))
             return 2;
     }
-    if (desc->has_expand && desc->in_h >= 28 && espdl::mbconv_s8_wave_supports(p))
+    if (desc->has_expand && !pointwise_expand(p))
+        return espdl::mbconv_s8_wave_supports(p) ? 4 : 0;
+    if (desc->has_expand && p.in_h >= 28 && espdl::mbconv_s8_wave_supports(p))
         return 4;
     if (desc->has_expand && espdl::mbconv_s8_group_supports(p))
         return 5;
@@ -826,7 +860,7 @@ int espdl_hip_mbconv_s8_preferred(const espdl_hip_mbconv_desc *desc)
     p.w_expand = aligned;
     const long long tiles = espdl::mbconv_s8_wave_tiles(p);
     const int cus = cu_count_cached() > 0 ? cu_count_cached() : 256;
-    return (desc->in_h >= 28 && desc->in_w >= 28 && tiles >= 4ll * cus) ? 1 : 0;
+    return (p.in_h >= 28 && p.in_w >= 28 && tiles >= 4ll * cus) ? 1 : 0;
 }
 
 int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *w,
@@ -866,7 +900,13 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
                                                                     reinterpret_cast<hipStream_t>(stream)),
                                  "depthwise_project_s8");
     }
-    if (desc->has_expand && !(desc->in_h >= 28 && espdl::mbconv_s8_wave_supports(p)) && espdl::mbconv_s8_group_supports(p))
+    if (desc->has_expand && !pointwise_expand(p)) {
+        if (!espdl::mbconv_s8_wave_supports(p))
+            return fail(ESPDL_HIP_ENOTSUP, "an expand stage with a window needs a 3x3 depthwise stage, at most 4 filter rows of at most 16 bytes (exp_k_w * in_c) and at most 64 project filters");
+        return device_status(espdl::launch_mbconv_s8_wave(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                             "mbconv_s8_wave");
+    }
+    if (desc->has_expand && !(p.in_h >= 28 && espdl::mbconv_s8_wave_supports(p)) && espdl::mbconv_s8_group_supports(p))
         return device_status(espdl::launch_mbconv_s8_group(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
                              "mbconv_s8_group");
     if (desc->has_expand && espdl::mbconv_s8_wave_supports(p))

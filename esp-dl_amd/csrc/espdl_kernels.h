@@ -81,7 +81,16 @@ struct MbconvParams {
     int batch, in_h, in_w, in_c, exp_c, out_c, out_h, out_w;
     int k_h, k_w, stride_h, stride_w, dil_h, dil_w, pad_top, pad_left;
     int relu_expand, relu_dw, relu_project, half_even;
+    // Expand stage with a window (ek_h x ek_w not 1 x 1, or a stride, or padding): in_h / in_w above stay the
+    // extents of the DEPTHWISE stage's input (the expand convolution's output), img_h / img_w are those of
+    // the block input, w_expand is [exp_c][ek_h][ek_w][in_c].  For the 1x1 expand img == in and ek == es == 1.
+    int img_h, img_w, ek_h, ek_w, es_h, es_w, epad_top, epad_left;
 };
+inline bool mbconv_expand_is_pointwise(const MbconvParams &p)
+{
+    return p.ek_h == 1 && p.ek_w == 1 && p.es_h == 1 && p.es_w == 1 && p.epad_top == 0 && p.epad_left == 0 &&
+        p.img_h == p.in_h && p.img_w == p.in_w;
+}
 bool mbconv_s8_fused_supports(const MbconvParams &p);
 hipError_t launch_mbconv_s8_fused(const MbconvParams &p, int cu_count, hipStream_t stream);
 

@@ -82,9 +82,6 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
 
     // ---- phase 0: tables (all lanes of the group), block-input patch -> operand B registers (per wavefront)
     const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
-    const int mode_e = build_stage_table_group(tab_e, p.b_expand, p.s_expand, p.n_s_expand, p.exp_c, bound_e, HE, tid,
-                                               kGroupThreads);
-    const int mode_d = build_stage_table_group(tab_d, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_d, HE, tid, kGroupThreads);
 
     v4i xb[NXPT * KSE];
     unsigned xmask = 0;
@@ -107,7 +104,9 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
             }
         }
     }
-    __syncthreads(); // tables complete
+    int mode_e, mode_d;
+    build_stage_tables_pair(reinterpret_cast<int *>(smem + a.off_tab + p.exp_c * 24), tab_e, tab_d, p.b_expand, p.s_expand, p.n_s_expand, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_e,
+                            bound_d, HE, tid, kGroupThreads, mode_e, mode_d); // tables complete
 
     // ---- phase 1: this wavefront's chunks of 16 expanded channels, expand -> depthwise, no barriers
     const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
@@ -322,7 +321,7 @@ GroupPlan group_plan(const MbconvParams &p)
         if (npt > kMaxT)
             break;
         const size_t exp_bytes = (size_t)((ph * a.pw + 48 + 15) & ~15) * 16;
-        const size_t lds = (size_t)p.exp_c * 24 + kGroupWaves * std::max(exp_bytes, (size_t)((n_xpt + 3) & ~3) * 256) +
+        const size_t lds = (size_t)p.exp_c * 24 + kStageVoteBytes + kGroupWaves * std::max(exp_bytes, (size_t)((n_xpt + 3) & ~3) * 256) +
             (size_t)npt * 16 * a.ds;
         if (lds > kGroupLdsMax)
             break;
@@ -336,7 +335,7 @@ GroupPlan group_plan(const MbconvParams &p)
     a.tiles_y = (p.out_h + a.th - 1) / a.th;
     a.exp_bytes = (int)std::max((size_t)((a.ph * a.pw + 48 + 15) & ~15) * 16, (size_t)((a.n_xpt + 3) & ~3) * 256);
     a.off_tab = 0;
-    a.off_exp = p.exp_c * 24;
+    a.off_exp = p.exp_c * 24 + kStageVoteBytes; // the workgroup's vote words sit behind the tables
     a.off_dw = a.off_exp + kGroupWaves * a.exp_bytes;
     plan.lds = (size_t)a.off_dw + (size_t)a.npt * 16 * a.ds;
     a.fd_pw = make_fastdiv((unsigned)a.pw);

@@ -65,7 +65,11 @@ extern "C" int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *d, const 
         return ESPDL_HIP_OK;
     if (in == nullptr || out == nullptr || w == nullptr)
         return espdl::set_error(ESPDL_HIP_EINVAL, "in, out and weights must not be NULL");
-    const size_t expanded = d->has_expand ? align256((size_t)d->batch * d->in_h * d->in_w * d->exp_c) : 0;
+    // extents of the depthwise stage's input: the block input's, or those of an expand stage with a window
+    const bool windowed = d->exp_k_h > 0;
+    const int mid_h = windowed ? (d->in_h + d->exp_pad_top + d->exp_pad_bottom - d->exp_k_h) / d->exp_stride_h + 1 : d->in_h;
+    const int mid_w = windowed ? (d->in_w + d->exp_pad_left + d->exp_pad_right - d->exp_k_w) / d->exp_stride_w + 1 : d->in_w;
+    const size_t expanded = d->has_expand ? align256((size_t)d->batch * mid_h * mid_w * d->exp_c) : 0;
     const size_t dw_out = align256((size_t)d->batch * out_h * out_w * d->exp_c);
     if (expanded + dw_out > kScratchBytes)
         return espdl::set_error(ESPDL_HIP_ENOTSUP,
@@ -89,6 +93,16 @@ extern "C" int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *d, const 
         c.in_c = d->in_c;
         c.out_c = d->exp_c;
         c.k_h = c.k_w = c.stride_h = c.stride_w = c.dil_h = c.dil_w = 1;
+        if (windowed) {
+            c.k_h = d->exp_k_h;
+            c.k_w = d->exp_k_w;
+            c.stride_h = d->exp_stride_h;
+            c.stride_w = d->exp_stride_w;
+            c.pad_top = d->exp_pad_top;
+            c.pad_bottom = d->exp_pad_bottom;
+            c.pad_left = d->exp_pad_left;
+            c.pad_right = d->exp_pad_right;
+        }
         c.group = 1;
         c.activation = d->act_expand;
         c.round_mode = d->round_mode;
@@ -102,8 +116,8 @@ extern "C" int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *d, const 
         espdl_hip_conv_desc c = {};
         c.dtype = ESPDL_HIP_S8;
         c.batch = d->batch;
-        c.in_h = d->in_h;
-        c.in_w = d->in_w;
+        c.in_h = mid_h;
+        c.in_w = mid_w;
         c.in_c = d->exp_c;
         c.out_c = d->exp_c;
         c.k_h = d->k_h;

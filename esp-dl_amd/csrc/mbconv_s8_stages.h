@@ -162,6 +162,69 @@ __device__ __forceinline__ int build_stage_table_group(int *tab, const int32_t *
     return mode;
 }
 
+// The tables of both inner stages (expand and depthwise: the same n_ch channels) with ONE memory round trip
+// and ONE workgroup vote, which is also the barrier after which the tables are complete: every lane writes
+// the short-epilogue form of its channels straight away and the vote tells whether some channel of a stage
+// cannot take it; only then (rare) that stage's table is rewritten with the plain bias and shift, behind a
+// second barrier.  `votes` is one LDS word per wavefront of the workgroup (kStageVoteBytes in all; a wavefront
+// stores the OR of its lanes' flags, every lane ORs the words after the barrier).  Every lane of the workgroup
+// must call this.
+constexpr int kStageVoteBytes = 64; // up to 16 wavefronts
+__device__ __forceinline__ void build_stage_tables_pair(int *votes, int *tab_e, int *tab_d, const int32_t *b_e, const int32_t *s_e,
+                                                        int n_s_e, const int32_t *b_d, const int32_t *s_d, int n_s_d,
+                                                        int n_ch, unsigned bound_e, unsigned bound_d, bool half_even,
+                                                        int tid, int nthreads, int &mode_e, int &mode_d)
+{
+    const unsigned step_e = n_s_e == 1 ? 0u : 1u, step_d = n_s_d == 1 ? 0u : 1u;
+    int flags = 0; // bit 0 / 1: expand / depthwise needs the general form; bit 2 / 3: a shift below 8
+    for (int c = tid; c < n_ch; c += nthreads) {
+        const int be = b_e != nullptr ? b_e[(size_t)(unsigned)c] : 0;
+        const int bd = b_d != nullptr ? b_d[(size_t)(unsigned)c] : 0;
+        const int se = s_e[(size_t)(step_e * (unsigned)c)];
+        const int sd = s_d[(size_t)(step_d * (unsigned)c)];
+        flags |= short_ok(se, be, bound_e) ? 0 : 1;
+        flags |= short_ok(sd, bd, bound_d) ? 0 : 2;
+        flags |= se < 8 ? 4 : 0;
+        flags |= sd < 8 ? 8 : 0;
+        const int se1 = min(max(se, 1), 31), sd1 = min(max(sd, 1), 31); // defined shifts where the form does not apply
+        tab_e[c] = be + (1 << (se1 - 1));
+        tab_e[n_ch + c] = max(0, se - 8);
+        tab_e[2 * n_ch + c] = max(0, 8 - se);
+        tab_d[c] = bd + (1 << (sd1 - 1));
+        tab_d[n_ch + c] = max(0, sd - 8);
+        tab_d[2 * n_ch + c] = max(0, 8 - sd);
+    }
+    {
+        int wf = 0; // OR over the wavefront's lanes, bit by bit
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+            wf |= __any(flags & (1 << b)) ? 1 << b : 0;
+        if ((tid & 63) == 0)
+            votes[tid >> 6] = wf;
+    }
+    __syncthreads();
+    int all = 0;
+    for (int w = 0; w < (nthreads >> 6); w++)
+        all |= votes[w];
+    if (all & 3) { // uniform
+        for (int c = tid; c < n_ch; c += nthreads) {
+            if (all & 1) {
+                tab_e[c] = b_e != nullptr ? b_e[(size_t)(unsigned)c] : 0;
+                tab_e[n_ch + c] = s_e[(size_t)(step_e * (unsigned)c)];
+                tab_e[2 * n_ch + c] = 0;
+            }
+            if (all & 2) {
+                tab_d[c] = b_d != nullptr ? b_d[(size_t)(unsigned)c] : 0;
+                tab_d[n_ch + c] = s_d[(size_t)(step_d * (unsigned)c)];
+                tab_d[2 * n_ch + c] = 0;
+            }
+        }
+        __syncthreads();
+    }
+    mode_e = (all & 1) ? -1 : (half_even ? 2 : ((all & 4) ? 1 : 0));
+    mode_d = (all & 2) ? -1 : (half_even ? 2 : ((all & 8) ? 1 : 0));
+}
+
 __device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch, int ch, int mode)
 {
     StageConsts c;

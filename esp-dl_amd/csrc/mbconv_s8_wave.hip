@@ -36,6 +36,14 @@
 //   * project epilogue, residual add, stores.
 // Filters, biases and shifts are read from global memory (L2) as they are needed: 16-byte pieces in
 // operand order, no staging.
+//
+// ROWCONV builds: the expand stage is a dense convolution with a window (a network's stem in front of its
+// first depthwise stage: conv2d_hwcn, esp-dl/dl/base/dl_base_conv2d.cpp:35-68) whose filter rows are at
+// most 9 bytes (k_w * in_c) and at most 4.  The reduction axis of the expand product is then
+// (filter row = 16-lane group, 16 bytes of that row): operand B of a patch pixel is the window's row as it
+// lies in memory (k_w * in_c consecutive bytes, cut out of three aligned dwords with v_alignbyte_b32),
+// operand A the filter row padded with zeros, prepared once per workgroup in LDS.  Everything behind the
+// expand product is the same code.
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -60,6 +68,7 @@ struct WaveArgs {
     int rt;    // project row tiles of 16 filters
     int x_vec16, we_vec16;
     int off_exp, off_dw, off_tab;
+    int off_aop; // ROWCONV: operand A of the expand stage for every expanded channel, [exp_c][4 rows][16 bytes]
     int wave_bytes; // LDS of one wavefront (expanded patch + depthwise result); the tables are shared
     FastDiv fd_pw, fd_tiles_x, fd_tiles_yx;
 };
@@ -72,7 +81,20 @@ struct WaveArgs {
 // Everything a tile reads from memory up front (its block-input patch, the residual words it will add at the
 // very end, the filters of its first chunk) is requested BEFORE the tables are built, so that one memory
 // round trip covers all of it.
-template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT>
+// Byte masks of three dwords from a 12-bit byte-validity mask (bit j: byte j is kept).
+__device__ __forceinline__ void byte_masks3(unsigned bm, int (&m)[3])
+{
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        int v = __builtin_amdgcn_sbfe((int)bm, 4 * k, 1) & 0xff;
+        v |= __builtin_amdgcn_sbfe((int)bm, 4 * k + 1, 1) & 0xff00;
+        v |= __builtin_amdgcn_sbfe((int)bm, 4 * k + 2, 1) & 0xff0000;
+        v |= __builtin_amdgcn_sbfe((int)bm, 4 * k + 3, 1) & (int)0xff000000u;
+        m[k] = v;
+    }
+}
+
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false>
 __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_wave_kernel(const WaveArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -107,7 +129,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
     // block-input patch -> operand B registers of the expand stage; xmask: patch pixels inside the image
     v4i xb[NXPT];
     unsigned xmask = 0;
-    {
+    if constexpr (!ROWCONV) {
         const int8_t *img = p.in + (long long)n * p.in_h * p.in_w * c0;
 #pragma unroll
         for (int pt = 0; pt < NXPT; pt++) {
@@ -121,6 +143,106 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
                 xb[pt] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
                                                valid ? c0 - 16 * quad : 0);
             }
+        }
+    } else {
+        // Lane (col, quad) of pixel tile pt: row `quad` of the window of patch pixel pt * 16 + col, i.e. the
+        // wb = ek_w * c0 bytes of input row ry from column rx on, as bytes 0 .. wb-1 of the lane's 16 (bytes
+        // from wb on meet zero weights).  They are cut out of the three aligned dwords around them; dword
+        // addresses are clamped to the image, bytes outside the image (the convolution's zero padding) and
+        // whole rows that do not exist are masked.  A tile whose windows all lie inside the image skips the masks.
+        const int rowb = p.img_w * c0;
+        const long long img_bytes = (long long)p.img_h * rowb;
+        const int8_t *img = p.in + (long long)n * img_bytes;
+        const int delta = (int)(reinterpret_cast<uintptr_t>(img) & 3u);
+        const int8_t *base = img - delta; // 4-byte aligned; offsets below are relative to it
+        const int off_max = (delta + (int)img_bytes - 1) & ~3; // the dword that holds the image's last byte
+        const int wy0 = iy0 * p.es_h - p.epad_top, wx0 = ix0 * p.es_w - p.epad_left;
+        const bool interior = iy0 >= 0 && ix0 >= 0 && iy0 + a.ph <= p.in_h && ix0 + a.pw <= p.in_w && wy0 >= 0 && wx0 >= 0 &&
+            wy0 + (a.ph - 1) * p.es_h + p.ek_h <= p.img_h && wx0 + (a.pw - 1) * p.es_w + p.ek_w <= p.img_w; // uniform
+        // byte-validity mask of a window row that starts at input column rx: the columns inside the image
+        auto x_bytes = [&](int rx) -> unsigned {
+            const int lo = max(0, -rx) * c0, hi = max(0, min(p.ek_w, p.img_w - rx)) * c0;
+            return hi > lo ? ((1u << hi) - 1u) & ~((1u << lo) - 1u) : 0u;
+        };
+        // phase 1: every load of the patch is requested before any of them is used
+        int d[NXPT][3];
+        unsigned shs = 0;   // two bits per pixel tile: where the row starts inside its first dword
+        unsigned rowok = 0; // one bit per pixel tile: the lane's window row exists (filter row, image row, pixel)
+        auto request = [&](int pt, int o) {
+            const int ab = o & ~3;
+            shs |= (unsigned)(o & 3) << (2 * pt);
+#pragma unroll
+            for (int k = 0; k < 3; k++)
+                d[pt][k] = *reinterpret_cast<const int *>(base + (size_t)(unsigned)min(max(ab + 4 * k, 0), off_max));
+        };
+        int rx_lane = 0; // EXACT: the lane's window column, the same for every pixel tile
+        if constexpr (EXACT) {
+            // guard-free builds have 16-pixel-wide patches: pixel tile = patch row, lane column = patch column,
+            // so everything about the column is computed once and a row costs one addition
+            const int mx = ix0 + col;
+            rx_lane = mx * p.es_w - p.epad_left;
+            const bool col_valid = (unsigned)mx < (unsigned)p.in_w;
+            const int ry0 = wy0 + quad;
+            const int o0 = ry0 * rowb + rx_lane * c0 + delta, o_step = p.es_h * rowb;
+            unsigned rows = 0; // uniform: patch rows inside the depthwise stage's input
+#pragma unroll
+            for (int pt = 0; pt < NXPT; pt++)
+                rows |= (pt < a.ph && (unsigned)(iy0 + pt) < (unsigned)p.in_h) ? 1u << pt : 0u;
+            xmask = col_valid ? rows : 0u;
+#pragma unroll
+            for (int pt = 0; pt < NXPT; pt++) {
+                request(pt, o0 + pt * o_step);
+                const bool ok = quad < p.ek_h && (unsigned)(ry0 + pt * p.es_h) < (unsigned)p.img_h;
+                rowok |= ok ? 1u << pt : 0u;
+            }
+            rowok &= xmask;
+        } else {
+#pragma unroll
+            for (int pt = 0; pt < NXPT; pt++) {
+#pragma unroll
+                for (int k = 0; k < 3; k++)
+                    d[pt][k] = 0;
+                if (pt < n_xpt) { // uniform
+                    const unsigned pp = (unsigned)(pt * 16 + col);
+                    const unsigned prow = fastdiv(pp, a.fd_pw);
+                    const int my = iy0 + (int)prow, mx = ix0 + (int)(pp - prow * a.fd_pw.d);
+                    const bool valid = (int)prow < a.ph && (unsigned)my < (unsigned)p.in_h && (unsigned)mx < (unsigned)p.in_w;
+                    xmask |= valid ? 1u << pt : 0u;
+                    const int ry = my * p.es_h - p.epad_top + quad, rx = mx * p.es_w - p.epad_left;
+                    request(pt, ry * rowb + rx * c0 + delta); // may lie outside the image; only masked bytes then
+                    rowok |= (valid && quad < p.ek_h && (unsigned)ry < (unsigned)p.img_h) ? 1u << pt : 0u;
+                }
+            }
+        }
+        // phase 2: cut the rows out of their dwords; border tiles mask what lies outside the image
+        int mx3[3] = {-1, -1, -1};
+        if (EXACT && !interior)
+            byte_masks3(x_bytes(rx_lane), mx3);
+#pragma unroll
+        for (int pt = 0; pt < NXPT; pt++) {
+            const unsigned sh = (shs >> (2 * pt)) & 3u;
+            int r[3];
+            r[0] = (int)__builtin_amdgcn_alignbyte((unsigned)d[pt][1], (unsigned)d[pt][0], sh);
+            r[1] = (int)__builtin_amdgcn_alignbyte((unsigned)d[pt][2], (unsigned)d[pt][1], sh);
+            r[2] = (int)__builtin_amdgcn_alignbyte(0u, (unsigned)d[pt][2], sh);
+            if (!interior) { // uniform
+                int m[3];
+                if constexpr (EXACT) {
+#pragma unroll
+                    for (int k = 0; k < 3; k++)
+                        m[k] = mx3[k];
+                } else {
+                    const unsigned pp = (unsigned)(pt * 16 + col);
+                    const unsigned prow = fastdiv(pp, a.fd_pw);
+                    const int mx = ix0 + (int)(pp - prow * a.fd_pw.d);
+                    byte_masks3(x_bytes(mx * p.es_w - p.epad_left), m);
+                }
+                const int keep = __builtin_amdgcn_sbfe((int)rowok, pt, 1); // all ones or zero
+#pragma unroll
+                for (int k = 0; k < 3; k++)
+                    r[k] &= m[k] & keep;
+            }
+            xb[pt] = v4i{r[0], r[1], r[2], 0};
         }
     }
 
@@ -140,7 +262,10 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
     auto load_chunk = [&](int sub) {
         ChunkW w;
         const int ch0 = 16 * sub;
-        w.aop[0] = load16_partial<VEC16>(p.w_expand, (unsigned)((ch0 + col) * c0 + 16 * quad), c0 - 16 * quad);
+        if constexpr (ROWCONV)
+            w.aop[0] = *reinterpret_cast<const v4i *>(smem + a.off_aop + ((ch0 + col) * 4 + quad) * 16);
+        else
+            w.aop[0] = load16_partial<VEC16>(p.w_expand, (unsigned)((ch0 + col) * c0 + 16 * quad), c0 - 16 * quad);
         const unsigned wd = (unsigned)(ch0 + col);
 #pragma unroll
         for (int kx = 0; kx < 3; kx++) {
@@ -163,15 +288,36 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
             ap[r] = load16_partial<true>(p.w_project, (unsigned)((16 * r + col) * p.exp_c + kc + 16 * quad),
                                          (r < n_rt && 16 * r + col < p.out_c) ? nk : 0);
     };
-    ChunkW cur = load_chunk(0);
+    ChunkW cur;
+    if constexpr (!ROWCONV)
+        cur = load_chunk(0);
+
+    if constexpr (ROWCONV) {
+        // operand A of the expand stage: filter row `q` of expanded channel f, zero-padded to 16 bytes
+        const int wb = p.ek_w * c0;
+        for (int i = (int)threadIdx.x; i < p.exp_c * 4; i += 64 * kWavesPerGroup) {
+            const int f = i >> 2, q = i & 3;
+            const bool row = q < p.ek_h;
+            const unsigned src = (unsigned)((f * p.ek_h + (row ? q : 0)) * wb);
+            int w[3] = {0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 9; j++) {
+                const bool ok = row && j < wb;
+                const int v = (int)(unsigned char)p.w_expand[(size_t)(src + (unsigned)(ok ? j : 0))];
+                w[j >> 2] |= ok ? v << (8 * (j & 3)) : 0;
+            }
+            *reinterpret_cast<v4i *>(smem + a.off_aop + i * 16) = v4i{w[0], w[1], w[2], 0};
+        }
+    }
 
     // the stage tables, by the whole group
-    const unsigned bound_e = (unsigned)c0 * 16384u, bound_d = 9u * 16384u;
-    const int mode_e = build_stage_table_group(tab_e, p.b_expand, p.s_expand, p.n_s_expand, p.exp_c, bound_e, HE,
-                                               (int)threadIdx.x, 64 * kWavesPerGroup);
-    const int mode_d = build_stage_table_group(tab_d, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_d, HE, (int)threadIdx.x,
-                                               64 * kWavesPerGroup);
-    __syncthreads(); // tables complete; no barrier after this one
+    const unsigned bound_e = (unsigned)(ROWCONV ? p.ek_h * p.ek_w * c0 : c0) * 16384u, bound_d = 9u * 16384u;
+    int mode_e, mode_d;
+    build_stage_tables_pair(reinterpret_cast<int *>(smem + a.off_tab + p.exp_c * 24), tab_e, tab_d, p.b_expand, p.s_expand, p.n_s_expand, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_e,
+                            bound_d, HE, (int)threadIdx.x, 64 * kWavesPerGroup, mode_e, mode_d);
+    // tables (and, in ROWCONV builds, the expand operands) complete; no barrier after this one
+    if constexpr (ROWCONV)
+        cur = load_chunk(0);
 
     v4i accp[RT][PT];
 #pragma unroll
@@ -316,7 +462,8 @@ void wave_layout(WaveArgs &a, size_t *lds)
 {
     const int exp_px = std::max(((a.n_xpt + 3) & ~3) * 16, (a.ph * a.pw + 48 + 15) & ~15);
     a.off_tab = 0; // two stages x [init | rsh | lsh] x int32
-    a.off_exp = a.p.exp_c * 24;
+    a.off_aop = a.p.exp_c * 24 + kStageVoteBytes; // the workgroup's vote words sit behind the tables
+    a.off_exp = a.off_aop + (mbconv_expand_is_pointwise(a.p) ? 0 : a.p.exp_c * 64);
     a.off_dw = a.off_exp + exp_px * 16;
     a.wave_bytes = exp_px * 16 + a.th * 16 * kDws;
     *lds = (size_t)a.off_exp + (size_t)kWavesPerGroup * a.wave_bytes;
@@ -329,7 +476,16 @@ WavePlan wave_plan(const MbconvParams &p)
     if (p.w_expand == nullptr || p.k_h != 3 || p.k_w != 3 || p.dil_h != 1 || p.dil_w != 1 || p.stride_h != p.stride_w ||
         (p.stride_h != 1 && p.stride_h != 2))
         return plan;
-    if (p.in_c % 4 != 0 || p.in_c > 64 || p.exp_c % 16 != 0 || p.out_c % 4 != 0 || p.out_c > 64)
+    const bool rowconv = !mbconv_expand_is_pointwise(p);
+    if (rowconv) {
+        // filter rows of at most 9 bytes cut out of three aligned dwords, one 16-lane group per row
+        if (p.ek_h < 1 || p.ek_h > 4 || p.ek_w < 1 || p.ek_w * p.in_c > 9 || p.es_h < 1 || p.es_w < 1 ||
+            (long long)p.img_h * p.img_w * p.in_c >= (1ll << 30) || (reinterpret_cast<uintptr_t>(p.in) & 3) != 0)
+            return plan;
+    } else if (p.in_c % 4 != 0 || p.in_c > 64) {
+        return plan;
+    }
+    if (p.exp_c % 16 != 0 || p.out_c % 4 != 0 || p.out_c > 64)
         return plan;
     if ((long long)p.in_h * p.in_w * p.in_c >= (1ll << 30) || (long long)p.out_h * p.out_w * p.out_c >= (1ll << 30) ||
         p.exp_c >= 65536)
@@ -338,8 +494,11 @@ WavePlan wave_plan(const MbconvParams &p)
     WaveArgs a = {};
     a.p = p;
     // columns: the fewest column tiles, then the narrowest tile that gives them (less halo to expand)
-    const int n_cols = (p.out_w + 15) / 16;
-    a.tw = (p.out_w + n_cols - 1) / n_cols;
+    // (an expand stage with a window at depthwise stride 1: patches of exactly 16 columns, where the patch
+    // column of a lane does not change from pixel tile to pixel tile and its window address costs one addition)
+    const int tw_max = (rowconv && s == 1 && p.out_w > 14) ? 14 : 16;
+    const int n_cols = (p.out_w + tw_max - 1) / tw_max;
+    a.tw = (rowconv && tw_max == 14) ? 14 : (p.out_w + n_cols - 1) / n_cols;
     a.pw = (a.tw - 1) * s + 3;
     a.tiles_x = n_cols;
     // rows: cheapest total of expand tiles (x 1.5: MFMA + the longer epilogue) and depthwise MFMAs
@@ -380,12 +539,12 @@ WavePlan wave_plan(const MbconvParams &p)
     return plan;
 }
 
-template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT>
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false>
 hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
 {
     const WaveArgs &a = plan.a;
     const unsigned groups = (unsigned)((a.n_tiles + kWavesPerGroup - 1) / kWavesPerGroup);
-    hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT>), dim3(groups),
+    hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV>), dim3(groups),
                        dim3(64 * kWavesPerGroup), plan.lds, stream, a);
     return hipGetLastError();
 }
@@ -403,6 +562,16 @@ hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
     WaveArgs &a = plan.a;
     const bool vec16 = a.x_vec16 && a.we_vec16;
     const int s = a.p.stride_h;
+    if (!mbconv_expand_is_pointwise(a.p)) {
+        // expand stage with a window: one guard-free build (the stem + first block of MobileNetV2 at 224 x 224)
+        if (!a.p.half_even && a.n_xpt == 10 && a.pw == 16 && a.rt == 1 && a.th == 8 && s == 1)
+            return launch_one<10, 1, 8, 1, false, false, true, true>(plan, stream);
+        if (a.p.half_even)
+            return s == 1 ? launch_one<17, 4, kPtMax, 1, true, false, false, true>(plan, stream)
+                          : launch_one<17, 4, kPtMax, 2, true, false, false, true>(plan, stream);
+        return s == 1 ? launch_one<17, 4, kPtMax, 1, false, false, false, true>(plan, stream)
+                      : launch_one<17, 4, kPtMax, 2, false, false, false, true>(plan, stream);
+    }
     if (!a.p.half_even) {
         // guard-free builds for the tile plans of MobileNetV2-style blocks (round half up)
         const auto is = [&](int nxpt, int rt, int th, int stride, bool v) {

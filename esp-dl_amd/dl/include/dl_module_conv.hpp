@@ -63,6 +63,9 @@ private:
     int m_expand_exponent = 0; ///< exponent of the (no longer materialized) expanded tensor
     int m_expand_filter_pos = -1, m_expand_bias_pos = -1;
     DeviceInts m_shift_expand;
+    // the absorbed Conv's own window: {1, 1} / {1, 1} / no padding for the usual 1x1 expand, anything else
+    // for a stem convolution that took the expand stage's place
+    std::vector<int> m_expand_kernel = {1, 1}, m_expand_strides = {1, 1}, m_expand_pads = {0, 0, 0, 0};
 
 public:
     Conv(activation_type_t activation = Linear, std::vector<int> pads = {}, std::vector<int> dilations = {},
@@ -119,10 +122,16 @@ public:
             m_inputs_index.push_back(residual_index);
         }
     }
-    /// Absorb the 1x1 Conv in front (after fuse_project): `input_index` is that Conv's input, which becomes
-    /// this module's first input; `expand_exponent` the exponent of the tensor it used to write.
-    void fuse_expand(int input_index, int filter_index, int bias_index, activation_type_t act, int expand_exponent)
+    /// Absorb the Conv in front (after fuse_project): `input_index` is that Conv's input, which becomes
+    /// this module's first input; `expand_exponent` the exponent of the tensor it used to write.  kernel /
+    /// strides / pads ({top, bottom, left, right}) describe that Conv when it is not a plain 1x1.
+    void fuse_expand(int input_index, int filter_index, int bias_index, activation_type_t act, int expand_exponent,
+                     std::vector<int> kernel = {1, 1}, std::vector<int> strides = {1, 1},
+                     std::vector<int> pads = {0, 0, 0, 0})
     {
+        m_expand_kernel = kernel;
+        m_expand_strides = strides;
+        m_expand_pads = pads;
         m_has_expand = true;
         m_expand_activation = act;
         m_expand_exponent = expand_exponent;
@@ -135,6 +144,12 @@ public:
         }
     }
     bool has_fused_expand() const { return m_has_expand; }
+    bool expand_has_window() const
+    {
+        return m_has_expand &&
+            (m_expand_kernel != std::vector<int>{1, 1} || m_expand_strides != std::vector<int>{1, 1} ||
+             m_expand_pads != std::vector<int>{0, 0, 0, 0});
+    }
     /// answer of espdl_hip_mbconv_s8_supported for the fused form at its last forward (0 before the first):
     /// which single-launch kernel runs it
     int fused_kernel() const { return m_fused_kernel; }
@@ -164,6 +179,11 @@ public:
         assert(input_shapes[0].size() == 3 || input_shapes[0].size() == 4);
         std::vector<int> input_shape = input_shapes[0];
         std::vector<int> filter_shape = input_shapes[1];
+        if (expand_has_window() && input_shape.size() == 4) {
+            // the depthwise stage reads the absorbed convolution's output
+            input_shape[1] = (input_shape[1] + m_expand_pads[0] + m_expand_pads[1] - m_expand_kernel[0]) / m_expand_strides[0] + 1;
+            input_shape[2] = (input_shape[2] + m_expand_pads[2] + m_expand_pads[3] - m_expand_kernel[1]) / m_expand_strides[1] + 1;
+        }
         std::vector<int> output_shape = input_shape;
         if (input_shape.size() == 3) {
             // [N, W, C], filter [kW, Cin, Cout] (dense) / [kW, 1, C] (depthwise)
@@ -197,8 +217,12 @@ public:
         if (m_has_project) { // [1x1 over the block input +] depthwise + 1x1 over the depthwise channels
             const int64_t dw_c = input_shapes[m_project_filter_pos][2];
             int64_t macs = pixels * dw_c * taps + pixels * out.back() * dw_c;
-            if (m_has_expand)
-                macs += (int64_t)input_shapes[0][0] * input_shapes[0][1] * input_shapes[0][2] * input_shapes[0][3] * dw_c;
+            if (m_has_expand) {
+                // absorbed convolution: its output pixels x window x input channels x expanded channels
+                const int64_t eh = (input_shapes[0][1] + m_expand_pads[0] + m_expand_pads[1] - m_expand_kernel[0]) / m_expand_strides[0] + 1;
+                const int64_t ew = (input_shapes[0][2] + m_expand_pads[2] + m_expand_pads[3] - m_expand_kernel[1]) / m_expand_strides[1] + 1;
+                macs += (int64_t)input_shapes[0][0] * eh * ew * m_expand_kernel[0] * m_expand_kernel[1] * input_shapes[0][3] * dw_c;
+            }
             return macs;
         }
         return pixels * out.back() * taps * in_c;
@@ -311,6 +335,16 @@ public:
         d.exp_c = m_has_expand ? pfilter->shape[2] : d.in_c;
         d.out_c = output->shape[3];
         d.has_expand = m_has_expand ? 1 : 0;
+        if (expand_has_window()) {
+            d.exp_k_h = m_expand_kernel[0];
+            d.exp_k_w = m_expand_kernel[1];
+            d.exp_stride_h = m_expand_strides[0];
+            d.exp_stride_w = m_expand_strides[1];
+            d.exp_pad_top = m_expand_pads[0];
+            d.exp_pad_bottom = m_expand_pads[1];
+            d.exp_pad_left = m_expand_pads[2];
+            d.exp_pad_right = m_expand_pads[3];
+        }
         d.act_expand = m_expand_activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR;
         d.k_h = filter->shape[0];
         d.k_w = filter->shape[1];

@@ -310,6 +310,7 @@ void Model::fuse_dw_project()
         // fuse where the depthwise+project kernel applies.
         dl::module::Conv *ex = nullptr;
         size_t ex_pos = 0;
+        int ex_kernel[2] = {1, 1};
         {
             const int dw_in = dw->m_inputs_index[0];
             size_t reader = 0;
@@ -323,17 +324,25 @@ void Model::fuse_dw_project()
                        ex->get_pads().size() != 4))
                 ex = nullptr;
             TensorBase *ef = ex ? m_model_context->get_tensor(ex->m_inputs_index[1]) : nullptr;
-            if (ex && (!ef || ef->shape.size() != 4 || ef->shape[0] != 1 || ef->shape[1] != 1 || ef->shape[3] != d.in_c))
+            if (ex && (!ef || ef->shape.size() != 4 || ef->shape[3] != d.in_c))
                 ex = nullptr;
+            bool plain_ex = true; // 1x1, stride 1, no padding
             if (ex) {
-                bool plain_ex = true;
+                plain_ex = ef->shape[0] == 1 && ef->shape[1] == 1;
                 for (int v : ex->get_pads())
                     plain_ex = plain_ex && v == 0;
                 for (int v : ex->get_strides())
                     plain_ex = plain_ex && v == 1;
                 for (int v : ex->get_dilations())
-                    plain_ex = plain_ex && v == 1;
-                if (!plain_ex)
+                    if (v != 1)
+                        ex = nullptr; // no kernel takes a dilated expand stage
+            }
+            std::vector<int> ex_in_shape;
+            if (ex) {
+                ex_kernel[0] = ef->shape[0];
+                ex_kernel[1] = ef->shape[1];
+                ex_in_shape = m_fbs_model->get_value_info_shape(m_model_context->get_tensor_name(ex->m_inputs_index[0]));
+                if (ex_in_shape.size() != 4 || ex->get_strides().size() != 2)
                     ex = nullptr;
             }
             if (ex) {
@@ -342,6 +351,19 @@ void Model::fuse_dw_project()
                 de.has_expand = 1;
                 de.exp_c = d.in_c;
                 de.in_c = ef->shape[2];
+                if (!plain_ex) {
+                    // a convolution with a window (a stem) as the expand stage: the block input is its input
+                    de.in_h = ex_in_shape[1];
+                    de.in_w = ex_in_shape[2];
+                    de.exp_k_h = ef->shape[0];
+                    de.exp_k_w = ef->shape[1];
+                    de.exp_stride_h = ex->get_strides()[0];
+                    de.exp_stride_w = ex->get_strides()[1];
+                    de.exp_pad_top = ex->get_pads()[0];
+                    de.exp_pad_bottom = ex->get_pads()[1];
+                    de.exp_pad_left = ex->get_pads()[2];
+                    de.exp_pad_right = ex->get_pads()[3];
+                }
                 if (espdl_hip_mbconv_s8_preferred(&de) != 1)
                     ex = nullptr;
             }
@@ -381,7 +403,8 @@ void Model::fuse_dw_project()
         if (ex)
             dw->fuse_expand(ex->m_inputs_index[0], ex->m_inputs_index[1],
                             ex->m_inputs_index.size() == 3 ? ex->m_inputs_index[2] : -1, ex->get_activation(),
-                            m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(ex->m_outputs_index[0])));
+                            m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(ex->m_outputs_index[0])),
+                            {ex_kernel[0], ex_kernel[1]}, ex->get_strides(), ex->get_pads());
         // the fused module moves to the slot of the last absorbed module
         m_execution_plan[last_pos] = dw;
         if (add) {

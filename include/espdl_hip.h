@@ -335,7 +335,8 @@ int espdl_hip_slice(const void *in, const int32_t *shape, int32_t dims, const in
  * channels), 3 = yes, expand stage inside the LDS-tile depthwise kernel, 4 = yes, one wavefront per tile
  * (3x3 depthwise stage, at most 64 block-input channels and 64 project filters), 5 = yes, a workgroup of
  * wavefronts per tile of a small image (output at most 16 pixels wide, block-input channels a multiple of
- * 16 and at most 192).
+ * 16 and at most 192).  An expand stage with a window (exp_k_h, exp_k_w not 1: at most 4 rows of at most
+ * 16 bytes, i.e. exp_k_w * in_c <= 16) is taken by the one-wavefront-per-tile kernel only.
  * espdl_hip_mbconv_s8 returns ESPDL_HIP_ENOTSUP where it does not apply.
  */
 typedef struct espdl_hip_mbconv_desc {
@@ -347,6 +348,12 @@ typedef struct espdl_hip_mbconv_desc {
     int32_t act_expand, act_dw, act_project;                          /* ESPDL_HIP_LINEAR / ESPDL_HIP_RELU */
     int32_t round_mode;
     int32_t n_shift_expand, n_shift_dw, n_shift_project;              /* 1 or channels of the stage */
+    /* Expand stage other than a 1x1 convolution (a stem convolution in front of the first depthwise stage):
+     * window, stride and padding of a dense convolution over the block input; in_h / in_w are then the
+     * extents of the block input and the depthwise stage works on that convolution's output.  All eight
+     * zero: the 1x1 stride-1 convolution.  Filter layout [exp_c][exp_k_h][exp_k_w][in_c]. */
+    int32_t exp_k_h, exp_k_w, exp_stride_h, exp_stride_w;
+    int32_t exp_pad_top, exp_pad_bottom, exp_pad_left, exp_pad_right;
 } espdl_hip_mbconv_desc;
 
 typedef struct espdl_hip_mbconv_weights {

@@ -1,5 +1,7 @@
 """GPU parity: every C-ABI entry point against the CPU oracle on the same seeded inputs.
 Bit-exact equality is the bar for all of them (integer / byte work)."""
+import ctypes
+
 import numpy as np
 import pytest
 
@@ -569,6 +571,96 @@ def test_mbconv_s8_fused(oracle, case):
     got = m.mbconv_s8(to_dev(x), dev(expand), dev(dw), dev(proj), k, stride, (1, 1), pads, (True, True, False),
                       residual=to_dev(res), round_mode=rm_g)
     np.testing.assert_array_equal(to_host(got), cur)
+
+
+# Expand stage with a window: a stem convolution in front of the first depthwise stage, in the block's launch.
+# (name, (N, H, W, Cin), expand (kernel, stride, pads), Ce, Cout, depthwise stride, depthwise pads, residual, half_even)
+ROWCONV_CASES = [
+    ("stem_64x64_rgb_s2_32_16", (2, 64, 64, 3), ((3, 3), (2, 2), (1, 1, 1, 1)), 32, 16, (1, 1), (1, 1, 1, 1), False, False),
+    ("stem_224x224_rgb_s2_32_16", (1, 224, 224, 3), ((3, 3), (2, 2), (1, 1, 1, 1)), 32, 16, (1, 1), (1, 1, 1, 1), False, False),
+    ("stem_tailpad_65x47_rgb_s2", (2, 65, 47, 3), ((3, 3), (2, 2), (0, 1, 0, 1)), 32, 24, (1, 1), (1, 1, 1, 1), False, False),
+    ("stem_gray_33x40_s1_16_8", (2, 33, 40, 1), ((3, 3), (1, 1), (1, 1, 1, 1)), 16, 8, (2, 2), (0, 1, 0, 1), False, False),
+    ("stem_2ch_4x2window_30x31", (3, 30, 31, 2), ((4, 2), (2, 1), (1, 2, 0, 1)), 48, 48, (1, 1), (1, 1, 1, 1), True, False),
+    ("stem_halfeven_50x50_rgb_s2", (2, 50, 50, 3), ((3, 3), (2, 2), (1, 1, 1, 1)), 32, 16, (1, 1), (1, 1, 1, 1), False, True),
+    ("stem_nopad_21x21_rgb_s1_res", (2, 21, 21, 3), ((2, 3), (1, 1), (0, 0, 0, 0)), 32, 32, (1, 1), (1, 1, 1, 1), True, False),
+    ("stem_tiny_5x5_rgb", (3, 5, 5, 3), ((3, 3), (2, 2), (1, 1, 1, 1)), 16, 4, (1, 1), (1, 1, 1, 1), False, False),
+]
+
+
+@pytest.mark.parametrize("staged", [False, True], ids=["single_launch", "staged"])
+@pytest.mark.parametrize("case", ROWCONV_CASES, ids=lambda c: c[0])
+def test_mbconv_s8_expand_with_window(oracle, case, staged):
+    announce(f"mbconv_s8 expand stage with a window: {case[0]} staged={staged}")
+    name, (n, h, w, cin), (ek, es, ep), ce, cout, stride, pads, with_res, half_even = case
+    m = espdl()
+    import torch
+    rng = np.random.default_rng(0x57E4 + len(name))
+    rm_o = oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP
+    rm_g = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
+
+    def stage(oc, kk, fshape):
+        f = rng_int8(rng, fshape)
+        b = rng.integers(-4096, 4097, size=oc).astype(np.int32)
+        s = (typical_shift(kk) + rng.integers(-2, 3, size=oc)).astype(np.int32)
+        return f, b, s
+
+    x = rng_int8(rng, (n, h, w, cin))
+    x[:, 0, :, :] = 127   # make the borders count: a wrongly placed or unmasked byte changes the result
+    x[:, :, 0, :] = -128
+    expand = stage(ce, ek[0] * ek[1] * cin, (ce, ek[0], ek[1], cin))
+    cur = oracle.conv2d_s8(x, expand[0], expand[1], expand[2], ek, es, (1, 1), ep, oracle.RELU, rm_o)
+    dw = stage(ce, 9, (3, 3, ce))
+    cur = oracle.depthwise_s8(cur, dw[0], dw[1], dw[2], (3, 3), stride, (1, 1), pads, oracle.RELU, rm_o)
+    proj = stage(cout, ce, (cout, 1, 1, ce))
+    cur = oracle.conv2d_s8(cur, proj[0], proj[1], proj[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.LINEAR, rm_o)
+    res = None
+    if with_res:
+        res = rng_int8(rng, cur.shape)
+        cur = oracle.add_s8(cur, res)
+    dev = lambda t: tuple(to_dev(a) for a in t)  # noqa: E731
+    out = torch.empty(cur.shape, dtype=torch.int8, device="cuda")
+    got = m.mbconv_s8(to_dev(x), dev(expand), dev(dw), dev(proj), (3, 3), stride, (1, 1), pads, (True, True, False),
+                      residual=to_dev(res), round_mode=rm_g, out=out, staged=staged, expand_conv=(ek, es, ep))
+    np.testing.assert_array_equal(to_host(got), cur)
+
+
+def test_mbconv_s8_expand_with_window_unaligned_images(oracle):
+    """Image sizes whose byte count is not a multiple of four: every image but the first starts at an odd address."""
+    announce("mbconv_s8 expand stage with a window, images at unaligned addresses")
+    m = espdl()
+    rng = np.random.default_rng(0xA11)
+    n, h, w, cin, ce, cout = 5, 9, 7, 3, 16, 8
+    x = rng_int8(rng, (n, h, w, cin))
+    f = lambda oc, kk, shape: (rng_int8(rng, shape), rng.integers(-999, 999, size=oc).astype(np.int32),  # noqa: E731
+                               (typical_shift(kk) + rng.integers(-2, 3, size=oc)).astype(np.int32))
+    ex, dw, pj = f(ce, 27, (ce, 3, 3, cin)), f(ce, 9, (3, 3, ce)), f(cout, ce, (cout, 1, 1, ce))
+    cur = oracle.conv2d_s8(x, ex[0], ex[1], ex[2], (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), oracle.RELU)
+    cur = oracle.depthwise_s8(cur, dw[0], dw[1], dw[2], (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), oracle.RELU)
+    want = oracle.conv2d_s8(cur, pj[0], pj[1], pj[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.LINEAR)
+    dev = lambda t: tuple(to_dev(a) for a in t)  # noqa: E731
+    got = m.mbconv_s8(to_dev(x), dev(ex), dev(dw), dev(pj), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), (True, True, False),
+                      expand_conv=((3, 3), (1, 1), (1, 1, 1, 1)))
+    np.testing.assert_array_equal(to_host(got), want)
+
+
+def test_mbconv_s8_expand_with_window_is_refused_where_not_covered():
+    announce("mbconv_s8 expand stage with a window: unsupported shapes are refused")
+    m = espdl()
+    d = m.capi.MbconvDesc()
+    d.batch, d.in_h, d.in_w, d.in_c, d.exp_c, d.out_c, d.has_expand = 2, 32, 32, 8, 32, 16, 1
+    d.k_h = d.k_w = 3
+    d.stride_h = d.stride_w = d.dil_h = d.dil_w = 1
+    d.pad_top = d.pad_bottom = d.pad_left = d.pad_right = 1
+    d.n_shift_expand = d.n_shift_dw = d.n_shift_project = 1
+    d.exp_k_h = d.exp_k_w = 3
+    d.exp_stride_h = d.exp_stride_w = 2
+    d.exp_pad_top = d.exp_pad_bottom = d.exp_pad_left = d.exp_pad_right = 1
+    assert m.capi.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == 0  # filter rows of 24 bytes
+    d.in_c = 3
+    assert m.capi.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == 4
+    d.has_expand = 0
+    d.exp_c = 3
+    assert m.capi.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == 0  # a window without an expand stage
 
 
 @pytest.mark.parametrize("ce", [320, 192], ids=["e320_block_kernel", "e192_lds_tile_kernel"])
