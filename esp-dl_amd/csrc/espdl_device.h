@@ -102,9 +102,32 @@ typedef short v2s __attribute__((ext_vector_type(2)));
 // acc = value + 2^(s-1) is a tie iff its low s bits are zero, so the half-even result is the half-up
 // result minus one when that holds and the half-up result is odd (the rule of
 // esp-dl/dl/tool/src/dl_tool.cpp:95-119, stated on acc instead of the value).
+// Saturating packed multiply of two int16 by two int16 (v_pk_mad_i16 with the clamp bit: the products are
+// formed exactly and saturated to int16).
+__device__ __forceinline__ v2s pk_mul_sat_i16(v2s a, int m)
+{
+    int d;
+    asm("v_pk_mad_i16 %0, %1, %2, 0 clamp" : "=v"(d) : "v"(__builtin_bit_cast(int, a)), "v"(m));
+    return __builtin_bit_cast(v2s, d);
+}
+
+// MODE 4 is MODE 1 with the left shifts moved behind the saturating convert, two values per instruction:
+// lsh[0] and lsh[1] hold the multipliers 2^max(0, 8-s) of the channel pairs (0, 1) and (2, 3) as packed
+// int16.  A channel has either a right shift (s > 8) or a multiplier (s < 8), never both.  Saturating
+// acc to int16 first and the product to int16 again gives the same high byte as saturating acc * 2^l once:
+// where the first saturation acts (|acc| >= 2^15, l >= 0) the second one does too.
 template <int MODE>
 __device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk, bool he = false)
 {
+    if constexpr (MODE == 4) {
+        const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
+        v2s p01 = __builtin_amdgcn_cvt_pk_i16(acc[0] >> rsh[0], acc[1] >> rsh[1]);
+        v2s p23 = __builtin_amdgcn_cvt_pk_i16(acc[2] >> rsh[2], acc[3] >> rsh[3]);
+        p01 = __builtin_elementwise_max(pk_mul_sat_i16(p01, lsh[0]), floor2);
+        p23 = __builtin_elementwise_max(pk_mul_sat_i16(p23, lsh[1]), floor2);
+        return (int)__builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, p23), (unsigned)__builtin_bit_cast(int, p01),
+                                          0x07050301u);
+    }
     int t[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {

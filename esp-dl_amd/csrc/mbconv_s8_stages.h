@@ -233,6 +233,8 @@ __device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch
     c.lsh = v4i{0, 0, 0, 0};
     if (mode == 1 || mode == 2)
         c.lsh = *reinterpret_cast<const v4i *>(tab + 2 * n_ch + ch);
+    if (mode == 1) // the multiplier form of pack_fast4<4>: 2^lsh of the channel pairs as packed int16
+        c.lsh = v4i{(1 << c.lsh[0]) | (65536 << c.lsh[1]), (1 << c.lsh[2]) | (65536 << c.lsh[3]), 0, 0};
     c.mode = mode;
     return c;
 }
@@ -270,6 +272,16 @@ __device__ __forceinline__ int wave_pack(const v4i &acc, const StageConsts &c, i
     }
 }
 
+// The same for constants that came from read_stage_table: in mode 1 they carry multipliers, not shift counts.
+template <int MODE>
+__device__ __forceinline__ int wave_pack_tab(const v4i &acc, const StageConsts &c, int floor_pk, bool relu, bool half_even)
+{
+    if constexpr (MODE == 1)
+        return pack_fast4<4>(acc, c.lsh, c.rsh, floor_pk);
+    else
+        return wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+}
+
 // Expand stage of one chunk of 16 channels: every patch pixel tile through one MFMA and the epilogue, four
 // tiles at a time so that four independent MFMA -> requantize -> store chains are in flight (tiles past
 // n_xpt inside the last group of four have zero operands and a zero mask and land in slack).
@@ -286,7 +298,7 @@ __device__ __forceinline__ void expand_chunk(const v4i (&xb)[NXPT * KSE], int n_
         return acc;
     };
     auto finish = [&](const v4i &acc, int pt) {
-        int word = wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+        int word = wave_pack_tab<MODE>(acc, c, floor_pk, relu, half_even);
         word &= __builtin_amdgcn_sbfe((int)xmask, pt, 1); // all ones or zero
         *reinterpret_cast<int *>(dst + pt * 256) = word;
     };
@@ -357,7 +369,7 @@ __device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
                 if (ROWS * u + r < PT) {
-                    const int w = wave_pack<MODE>(acc[u & 1][r], c, floor_pk, relu, half_even);
+                    const int w = wave_pack_tab<MODE>(acc[u & 1][r], c, floor_pk, relu, half_even);
                     if (write_ok)
                         *reinterpret_cast<int *>(dst + (ROWS * u + r) * row_bytes) = w;
                 }
@@ -388,14 +400,14 @@ __device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_
                 v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b0, c.init, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b1, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[2], b2, acc, 0, 0, 0);
-                const int w0 = wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+                const int w0 = wave_pack_tab<MODE>(acc, c, floor_pk, relu, half_even);
                 if (write_ok)
                     *reinterpret_cast<int *>(dst + (2 * j) * row_bytes) = w0;
                 if (EXACT ? 2 * j + 1 < PT : 2 * j + 1 < th) {
                     v4i acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[0], b0, c.init, 0, 0, 0);
                     acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[1], b1, acc1, 0, 0, 0);
                     acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[2], b2, acc1, 0, 0, 0);
-                    const int w1 = wave_pack<MODE>(acc1, c, floor_pk, relu, half_even);
+                    const int w1 = wave_pack_tab<MODE>(acc1, c, floor_pk, relu, half_even);
                     if (write_ok)
                         *reinterpret_cast<int *>(dst + (2 * j + 1) * row_bytes) = w1;
                 }
@@ -412,7 +424,7 @@ __device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_
                 v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b0, c.init, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b1, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[2], b2, acc, 0, 0, 0);
-                const int w0 = wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+                const int w0 = wave_pack_tab<MODE>(acc, c, floor_pk, relu, half_even);
                 if (write_ok)
                     *reinterpret_cast<int *>(dst + t * row_bytes) = w0;
             }
