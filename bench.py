@@ -36,16 +36,10 @@ MACHINE_BALANCE = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)  # OP per byte
 # rocprofv3 counter runs of this program (FETCH_SIZE scaled by 2.0, WRITE_SIZE by 1.0: the factors a
 # 256 MiB element-wise kernel of known traffic gave in the same runs).  Only valid for config 3 at
 # batch 256; any other workload reports null.
-_KIB = 1024
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    # six launches: 2 x FETCH_SIZE + WRITE_SIZE of the five kernel variants (one of them runs twice)
-    "mbconv_s8_wave": (2 * (25311.0 + 9665.5 + 9687.5 + 2 * 4965.0 + 3472.5)
-                       + (18816.0 + 18816.0 + 6272.0 + 2 * 6272.0 + 3136.0)) / 6 * _KIB,
-    # ten launches of four kernel variants (4 + 2 + 1 + 3)
-    "mbconv_s8_group": (2 * (4 * 6430.7 + 2 * 3049.0 + 3188.0 + 3 * 2680.7)
-                        + (4 * 11720.0 + 2 * 4704.0 + 1960.0 + 3 * 2613.3)) / 10 * _KIB,
-    "depthwise_s8": (2 * 50333.7 + 50176.0) * _KIB,                       # the first block's depthwise+project
-    "conv2d_s8": (2 * (19034.0 + 9600.1 + 2917.5) + (100352.0 + 15680.0 + 346.0)) / 3 * _KIB,  # stem, head, classifier
+    "mbconv_s8_wave": 38590363.0,   # 7 launches (the stem convolution rides in the first block's launch)
+    "mbconv_s8_group": 14708848.0,  # 10 launches
+    "conv2d_s8": 21020144.0,        # head convolution and classifier
     "elementwise_s8": None,
 }
 
