@@ -47,6 +47,7 @@ struct GroupArgs {
     int n_sub; // chunks of 16 expanded channels
     int rt;    // project row tiles of 16 filters
     int npt;   // project pixel tiles of 16 slots
+    int wr, wp, nt; // phase 2: wavefront grid (row groups x pixel groups, wr * wp <= 8), pixel tiles per wavefront
     int ds;    // LDS pixel stride of the shared depthwise tile, bytes
     int exp_bytes; // private expand area per wavefront
     int off_tab, off_exp, off_dw;
@@ -182,96 +183,132 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
             cur = nxt;
         }
     }
+    // operand A of the first project step does not depend on this tile's data: requested before the barrier
+    const int ksp = (p.exp_c + 63) / 64;
+    const int wrow = wave / a.wp, wpix = wave - wrow * a.wp;
+    auto load_a = [&](int rt, int k0, v4i(&ap)[8]) {
+        const bool row_ok = rt < a.rt && 16 * rt + col < p.out_c;
+        const unsigned a_off = (unsigned)((16 * rt + col) * p.exp_c + 16 * quad);
+#pragma unroll
+        for (int kk = 0; kk < 8; kk++) // lanes past the last channel read offset 0 and get zeros
+            ap[kk] = load16_partial<true>(p.w_project, a_off + 64u * (unsigned)(k0 + kk),
+                                          row_ok ? p.exp_c - 64 * (k0 + kk) - 16 * quad : 0);
+    };
+    // (not in the build that is held to 128 registers so that two workgroups share a compute unit)
+    constexpr bool kPrefetchA = !(KSE == 1 && EXACT);
+    v4i ap_first[8];
+    if constexpr (kPrefetchA)
+        load_a(wrow, 0, ap_first);
     __syncthreads(); // the shared depthwise tile is complete
 
-    // ---- phase 2: project.  A wavefront owns one row tile of 16 filters at a time (all of them when there
-    // are at least eight, otherwise the row tiles are shared by 8 / rt wavefronts that split the pixel tiles),
-    // so operand A is loaded once per k step and used for up to kMaxT pixel tiles; eight k steps of operand A
-    // are requested together, which is what hides the latency of these loads.
-    const int ksp = (p.exp_c + 63) / 64;
-    int rt_first, rt_step, t0, t1;
-    if (a.rt >= kGroupWaves) {
-        rt_first = wave;
-        rt_step = kGroupWaves;
-        t0 = 0;
-        t1 = a.npt;
-    } else {
-        const int wpr = kGroupWaves / a.rt; // wavefronts per row tile
-        const int part = wave % wpr, per = (a.npt + wpr - 1) / wpr;
-        rt_first = wave / wpr; // >= a.rt for the wavefronts left over: they have nothing to do
-        rt_step = a.rt;        // one row tile per wavefront
-        t0 = min(a.npt, part * per);
-        t1 = min(a.npt, t0 + per);
-    }
+    // ---- phase 2: project.  The (row tile of 16 filters) x (pixel tile of 16 slots) accumulator tiles are dealt
+    // to the wavefronts as a grid of a.wr row groups x a.wp pixel groups (chosen on the host): a wavefront
+    // walks the row tiles of its row group and holds nt = ceil(npt / wp) pixel tiles at a time.  nt is a compile-time count here, so the operand-B reads of a k step are issued together and the
+    // products follow back to back; a pixel tile past the last one reads the last tile again and stores
+    // nothing.  Eight k steps of operand A are requested together, which hides the latency of those loads.
+    // Reduction positions past exp_c meet zeros in operand A, whatever operand B holds there.
+    const int t0 = wpix * a.nt;
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
     const unsigned bound_p = (unsigned)p.exp_c * 16384u;
     const long long img_off = (long long)n * p.out_h * p.out_w * p.out_c;
     const int8_t *res_img = p.residual != nullptr ? p.residual + img_off : nullptr;
     int8_t *out_img = p.out + img_off;
-    for (int rt = rt_first; rt < a.rt; rt += rt_step) {
-        v4i accp[kMaxT];
+    auto project = [&](auto nt_tag) {
+        constexpr int NT = decltype(nt_tag)::value;
+        const unsigned char *bsrc[NT];
 #pragma unroll
-        for (int i = 0; i < kMaxT; i++)
-            accp[i] = v4i{0, 0, 0, 0};
-        const bool row_ok = 16 * rt + col < p.out_c;
-        const unsigned a_off = (unsigned)((16 * rt + col) * p.exp_c + 16 * quad);
-        const unsigned char *bsrc = dw_l + (t0 * 16 + col) * a.ds + 16 * quad;
-        for (int k0 = 0; k0 < ksp; k0 += 8) {
-            v4i ap[8];
+        for (int i = 0; i < NT; i++)
+            bsrc[i] = dw_l + (min(t0 + i, a.npt - 1) * 16 + col) * a.ds + 16 * quad;
+        v4i ap[8];
+        if constexpr (kPrefetchA) {
 #pragma unroll
-            for (int kk = 0; kk < 8; kk++) // lanes past the last channel read offset 0 and get zeros
-                ap[kk] = load16_partial<true>(p.w_project, a_off + 64u * (unsigned)(k0 + kk),
-                                              row_ok ? p.exp_c - 64 * (k0 + kk) - 16 * quad : 0);
+            for (int kk = 0; kk < 8; kk++)
+                ap[kk] = ap_first[kk];
+        }
+        for (int rt = wrow; rt < a.rt; rt += a.wr) {
+            v4i accp[NT];
 #pragma unroll
-            for (int kk = 0; kk < 8; kk++) {
-                if (k0 + kk < ksp) { // uniform
-                    const bool k_ok = p.exp_c - 64 * (k0 + kk) - 16 * quad > 0;
+            for (int i = 0; i < NT; i++)
+                accp[i] = v4i{0, 0, 0, 0};
+            for (int k0 = 0; k0 < ksp; k0 += 8) {
+                // the next block of operand A (the next k steps, or the first ones of the next row tile) is
+                // requested before this block's products
+                v4i an[8];
+                const bool more_k = k0 + 8 < ksp;
+                if constexpr (kPrefetchA)
+                    load_a(more_k ? rt : rt + a.wr, more_k ? k0 + 8 : 0, an);
+                else
+                    load_a(rt, k0, ap);
 #pragma unroll
-                    for (int i = 0; i < kMaxT; i++) {
-                        if (t0 + i < t1) { // uniform
-                            v4i bv = *reinterpret_cast<const v4i *>(bsrc + i * 16 * a.ds + 64 * (k0 + kk));
-                            bv = k_ok ? bv : v4i{0, 0, 0, 0};
-                            accp[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ap[kk], bv, accp[i], 0, 0, 0);
-                        }
+                for (int kk = 0; kk < 8; kk++) {
+                    if (k0 + kk < ksp) { // uniform
+                        v4i bv[NT];
+#pragma unroll
+                        for (int i = 0; i < NT; i++)
+                            bv[i] = *reinterpret_cast<const v4i *>(bsrc[i] + 64 * (k0 + kk));
+#pragma unroll
+                        for (int i = 0; i < NT; i++)
+                            accp[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ap[kk], bv[i], accp[i], 0, 0, 0);
                     }
                 }
-            }
-        }
-        const int c = 16 * rt + 4 * quad;
-        v4i bp, sp;
-        load_bias_shift(p.b_project, p.s_project, p.n_s_project, c, p.out_c, bp, sp);
-        const StageConsts cp = stage_consts(bp, sp, bound_p, HE);
+                if constexpr (kPrefetchA) {
 #pragma unroll
-        for (int i = 0; i < kMaxT; i++) {
-            if (t0 + i < t1) { // uniform
+                    for (int kk = 0; kk < 8; kk++)
+                        ap[kk] = an[kk];
+                }
+            }
+            const int c = 16 * rt + 4 * quad;
+            v4i bp, sp;
+            load_bias_shift(p.b_project, p.s_project, p.n_s_project, c, p.out_c, bp, sp);
+            const StageConsts cp = stage_consts(bp, sp, bound_p, HE);
+            // residual words of all pixel tiles first, then the epilogues
+            bool live[NT];
+            unsigned off[NT];
+            int rv[NT];
+#pragma unroll
+            for (int i = 0; i < NT; i++) {
                 // pixel slot -> (row, column) of the tile: twp slots per output row
                 const int slot = (t0 + i) * 16 + col;
                 const int oy = a.twp == 16 ? t0 + i : (slot >> 3), ox = a.twp == 16 ? col : (slot & 7);
-                const bool live = oy < th_real && ox < p.out_w && c < p.out_c;
-                const unsigned off = (unsigned)(((oy0 + oy) * p.out_w + ox) * p.out_c + c);
+                live[i] = t0 + i < a.npt && oy < th_real && ox < p.out_w && c < p.out_c;
+                off[i] = (unsigned)(((oy0 + oy) * p.out_w + ox) * p.out_c + c);
+                rv[i] = res_img != nullptr ? *reinterpret_cast<const int *>(res_img + (size_t)(live[i] ? off[i] : 0u)) : 0;
+            }
+#pragma unroll
+            for (int i = 0; i < NT; i++) {
                 v4i acc = accp[i];
 #pragma unroll
                 for (int k = 0; k < 4; k++)
                     acc[k] += cp.init[k];
-                const int rv = res_img != nullptr ? *reinterpret_cast<const int *>(res_img + (size_t)(live ? off : 0u)) : 0;
                 int word;
                 if (cp.mode == 0)
-                    word = res_img != nullptr ? pack_fast4_add<0>(acc, cp.lsh, cp.rsh, floor_p, rv)
+                    word = res_img != nullptr ? pack_fast4_add<0>(acc, cp.lsh, cp.rsh, floor_p, rv[i])
                                               : wave_pack<0>(acc, cp, floor_p, false, HE);
                 else if (cp.mode == 1)
-                    word = res_img != nullptr ? pack_fast4_add<1>(acc, cp.lsh, cp.rsh, floor_p, rv)
+                    word = res_img != nullptr ? pack_fast4_add<1>(acc, cp.lsh, cp.rsh, floor_p, rv[i])
                                               : wave_pack<1>(acc, cp, floor_p, false, HE);
                 else if (cp.mode == 2)
-                    word = res_img != nullptr ? pack_fast4_add<2>(acc, cp.lsh, cp.rsh, floor_p, rv)
+                    word = res_img != nullptr ? pack_fast4_add<2>(acc, cp.lsh, cp.rsh, floor_p, rv[i])
                                               : wave_pack<2>(acc, cp, floor_p, false, HE);
                 else {
                     word = wave_pack<-1>(acc, cp, floor_p, p.relu_project != 0, HE);
                     if (res_img != nullptr)
-                        word = sat_add4_s8(word, rv);
+                        word = sat_add4_s8(word, rv[i]);
                 }
-                if (live)
-                    *reinterpret_cast<int *>(out_img + (size_t)off) = word;
+                if (live[i])
+                    *reinterpret_cast<int *>(out_img + (size_t)off[i]) = word;
             }
+        }
+    };
+    if (wrow < a.wr) { // uniform: wavefronts beyond the grid have no share
+        switch (a.nt) {
+        case 1: project(std::integral_constant<int, 1>{}); break;
+        case 2: project(std::integral_constant<int, 2>{}); break;
+        case 3: project(std::integral_constant<int, 3>{}); break;
+        case 4: project(std::integral_constant<int, 4>{}); break;
+        case 5: project(std::integral_constant<int, 5>{}); break;
+        case 6: project(std::integral_constant<int, 6>{}); break;
+        default: project(std::integral_constant<int, kMaxT>{}); break;
         }
     }
 }
@@ -322,7 +359,7 @@ GroupPlan group_plan(const MbconvParams &p)
             break;
         const size_t exp_bytes = (size_t)((ph * a.pw + 48 + 15) & ~15) * 16;
         const size_t lds = (size_t)p.exp_c * 24 + kStageVoteBytes + kGroupWaves * std::max(exp_bytes, (size_t)((n_xpt + 3) & ~3) * 256) +
-            (size_t)npt * 16 * a.ds;
+            (size_t)npt * 16 * a.ds + 64;
         if (lds > kGroupLdsMax)
             break;
         a.th = th;
@@ -337,7 +374,18 @@ GroupPlan group_plan(const MbconvParams &p)
     a.off_tab = 0;
     a.off_exp = p.exp_c * 24 + kStageVoteBytes; // the workgroup's vote words sit behind the tables
     a.off_dw = a.off_exp + kGroupWaves * a.exp_bytes;
-    plan.lds = (size_t)a.off_dw + (size_t)a.npt * 16 * a.ds;
+    plan.lds = (size_t)a.off_dw + (size_t)a.npt * 16 * a.ds + 64; // k steps read whole 64-byte pieces
+    // phase-2 grid: a row tile of filters belongs to one wavefront where there are at least eight of them
+    // (operand A comes from global memory: loading it once per workgroup matters more than an even share);
+    // with fewer row tiles 8 / rt wavefronts share one and split the pixel tiles
+    if (a.rt >= kGroupWaves) {
+        a.wr = kGroupWaves;
+        a.wp = 1;
+    } else {
+        a.wr = a.rt;
+        a.wp = kGroupWaves / a.rt;
+    }
+    a.nt = (a.npt + a.wp - 1) / a.wp;
     a.fd_pw = make_fastdiv((unsigned)a.pw);
     a.fd_tiles_y = make_fastdiv((unsigned)a.tiles_y);
     a.fd_npt = make_fastdiv((unsigned)a.npt);

@@ -45,6 +45,7 @@
 // operand A the filter row padded with zeros, prepared once per workgroup in LDS.  Everything behind the
 // expand product is the same code.
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <type_traits>
@@ -454,6 +455,7 @@ struct WavePlan {
 };
 
 constexpr int kPtMax = 8;
+constexpr int kPlanCus = 256; // compute units the tile plan is balanced for
 
 // LDS layout: the tables (shared by the wavefronts of a group), then per wavefront the expanded patch of one
 // chunk (16 bytes per pixel; the depthwise reads run up to one row and a few pixels past the patch, into
@@ -501,8 +503,11 @@ WavePlan wave_plan(const MbconvParams &p)
     a.tw = (rowconv && tw_max == 14) ? 14 : (p.out_w + n_cols - 1) / n_cols;
     a.pw = (a.tw - 1) * s + 3;
     a.tiles_x = n_cols;
-    // rows: cheapest total of expand tiles (x 1.5: MFMA + the longer epilogue) and depthwise MFMAs
+    // rows: cheapest total of expand tiles (x 1.5: MFMA + the longer epilogue) and depthwise MFMAs.  A launch
+    // that does not fill the device once (two resident workgroups per compute unit) takes one tile's time
+    // whatever its tile count, so there a lower tile that brings more workgroups wins.
     const int nxpt_limit = 17;
+    const double slots = 2.0 * kPlanCus;
     double best = 1e30;
     a.th = 0;
     for (int th = 1; th <= kPtMax; th++) {
@@ -511,7 +516,10 @@ WavePlan wave_plan(const MbconvParams &p)
         if (n_xpt > nxpt_limit)
             break;
         const int tiles_y = (p.out_h + th - 1) / th;
-        const double cost = (double)tiles_y * (1.5 * n_xpt + 3.0 * th + 2.0);
+        const double tile_cost = 1.5 * n_xpt + 3.0 * th + 2.0;
+        const double groups = std::ceil((double)std::max(1, p.batch) * tiles_y * a.tiles_x / kWavesPerGroup);
+        const double rounds = groups / slots;
+        const double cost = tile_cost * std::max(1.0, rounds);
         if (cost < best) {
             best = cost;
             a.th = th;
@@ -587,6 +595,8 @@ hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
             return launch_one<10, 2, 8, 1, false, true, true>(plan, stream);
         if (is(9, 2, 7, 1, true))
             return launch_one<9, 2, 7, 1, false, true, true>(plan, stream);
+        if (is(10, 4, 2, 2, true))
+            return launch_one<10, 4, 2, 2, false, true, true>(plan, stream);
         if (is(13, 4, 3, 2, true))
             return launch_one<13, 4, 3, 2, false, true, true>(plan, stream);
         return s == 1 ? launch_generic<1, false>(plan, stream) : launch_generic<2, false>(plan, stream);
