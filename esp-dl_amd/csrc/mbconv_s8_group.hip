@@ -105,9 +105,31 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
             }
         }
     }
-    int mode_e, mode_d;
-    build_stage_tables_pair(reinterpret_cast<int *>(smem + a.off_tab + p.exp_c * 24), tab_e, tab_d, p.b_expand, p.s_expand, p.n_s_expand, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_e,
-                            bound_d, HE, tid, kGroupThreads, mode_e, mode_d); // tables complete
+    int mode_e, mode_d, mode_p;
+    int *tab_p = tab_d + 3 * p.exp_c; // 3 x 16 rt entries
+    {
+        StageTablesArgs t;
+        t.tab_e = tab_e;
+        t.tab_d = tab_d;
+        t.tab_p = tab_p;
+        t.votes = tab_p + 3 * 16 * a.rt;
+        t.b_e = p.b_expand;
+        t.s_e = p.s_expand;
+        t.b_d = p.b_dw;
+        t.s_d = p.s_dw;
+        t.b_p = p.b_project;
+        t.s_p = p.s_project;
+        t.n_s_e = p.n_s_expand;
+        t.n_s_d = p.n_s_dw;
+        t.n_s_p = p.n_s_project;
+        t.n_ch = p.exp_c;
+        t.n_ch_p = p.out_c;
+        t.n_pad_p = 16 * a.rt;
+        t.bound_e = bound_e;
+        t.bound_d = bound_d;
+        t.bound_p = (unsigned)p.exp_c * 16384u;
+        build_stage_tables(t, HE, tid, kGroupThreads, mode_e, mode_d, mode_p); // tables complete
+    }
 
     // ---- phase 1: this wavefront's chunks of 16 expanded channels, expand -> depthwise, no barriers
     const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
@@ -209,7 +231,6 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
     // Reduction positions past exp_c meet zeros in operand A, whatever operand B holds there.
     const int t0 = wpix * a.nt;
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
-    const unsigned bound_p = (unsigned)p.exp_c * 16384u;
     const long long img_off = (long long)n * p.out_h * p.out_w * p.out_c;
     const int8_t *res_img = p.residual != nullptr ? p.residual + img_off : nullptr;
     int8_t *out_img = p.out + img_off;
@@ -258,9 +279,7 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
                 }
             }
             const int c = 16 * rt + 4 * quad;
-            v4i bp, sp;
-            load_bias_shift(p.b_project, p.s_project, p.n_s_project, c, p.out_c, bp, sp);
-            const StageConsts cp = stage_consts(bp, sp, bound_p, HE);
+            const StageConsts cp = read_stage_table<false>(tab_p, 16 * a.rt, c, mode_p);
             // residual words of all pixel tiles first, then the epilogues
             bool live[NT];
             unsigned off[NT];
@@ -358,7 +377,7 @@ GroupPlan group_plan(const MbconvParams &p)
         if (npt > kMaxT)
             break;
         const size_t exp_bytes = (size_t)((ph * a.pw + 48 + 15) & ~15) * 16;
-        const size_t lds = (size_t)p.exp_c * 24 + kStageVoteBytes + kGroupWaves * std::max(exp_bytes, (size_t)((n_xpt + 3) & ~3) * 256) +
+        const size_t lds = (size_t)p.exp_c * 24 + (size_t)a.rt * 16 * 12 + kStageVoteBytes + kGroupWaves * std::max(exp_bytes, (size_t)((n_xpt + 3) & ~3) * 256) +
             (size_t)npt * 16 * a.ds + 64;
         if (lds > kGroupLdsMax)
             break;
@@ -372,7 +391,7 @@ GroupPlan group_plan(const MbconvParams &p)
     a.tiles_y = (p.out_h + a.th - 1) / a.th;
     a.exp_bytes = (int)std::max((size_t)((a.ph * a.pw + 48 + 15) & ~15) * 16, (size_t)((a.n_xpt + 3) & ~3) * 256);
     a.off_tab = 0;
-    a.off_exp = p.exp_c * 24 + kStageVoteBytes; // the workgroup's vote words sit behind the tables
+    a.off_exp = p.exp_c * 24 + a.rt * 16 * 12 + kStageVoteBytes; // expand, depthwise and project tables, vote words
     a.off_dw = a.off_exp + kGroupWaves * a.exp_bytes;
     plan.lds = (size_t)a.off_dw + (size_t)a.npt * 16 * a.ds + 64; // k steps read whole 64-byte pieces
     // phase-2 grid: a row tile of filters belongs to one wavefront where there are at least eight of them

@@ -162,7 +162,7 @@ __device__ __forceinline__ int build_stage_table_group(int *tab, const int32_t *
     return mode;
 }
 
-// The tables of both inner stages (expand and depthwise: the same n_ch channels) with ONE memory round trip
+// The tables of the three stages (expand and depthwise: the same n_ch channels; project: see below) with ONE memory round trip
 // and ONE workgroup vote, which is also the barrier after which the tables are complete: every lane writes
 // the short-epilogue form of its channels straight away and the vote tells whether some channel of a stage
 // cannot take it; only then (rare) that stage's table is rewritten with the plain bias and shift, behind a
@@ -170,61 +170,96 @@ __device__ __forceinline__ int build_stage_table_group(int *tab, const int32_t *
 // stores the OR of its lanes' flags, every lane ORs the words after the barrier).  Every lane of the workgroup
 // must call this.
 constexpr int kStageVoteBytes = 64; // up to 16 wavefronts
-__device__ __forceinline__ void build_stage_tables_pair(int *votes, int *tab_e, int *tab_d, const int32_t *b_e, const int32_t *s_e,
-                                                        int n_s_e, const int32_t *b_d, const int32_t *s_d, int n_s_d,
-                                                        int n_ch, unsigned bound_e, unsigned bound_d, bool half_even,
-                                                        int tid, int nthreads, int &mode_e, int &mode_d)
+// The project stage has its own table of n_pad_p channels (out_c rounded up to 16; channels that do not
+// exist get bias 0 and shift 8), in the same three-row layout; its epilogue reads it with
+// read_stage_table<false> (shift counts, not multipliers).
+struct StageTablesArgs {
+    int *votes, *tab_e, *tab_d, *tab_p;
+    const int32_t *b_e, *s_e, *b_d, *s_d, *b_p, *s_p;
+    int n_s_e, n_s_d, n_s_p;
+    int n_ch, n_ch_p, n_pad_p;
+    unsigned bound_e, bound_d, bound_p;
+};
+__device__ __forceinline__ void build_stage_tables(const StageTablesArgs &t, bool half_even, int tid, int nthreads,
+                                                   int &mode_e, int &mode_d, int &mode_p)
 {
-    const unsigned step_e = n_s_e == 1 ? 0u : 1u, step_d = n_s_d == 1 ? 0u : 1u;
-    int flags = 0; // bit 0 / 1: expand / depthwise needs the general form; bit 2 / 3: a shift below 8
+    const unsigned step_e = t.n_s_e == 1 ? 0u : 1u, step_d = t.n_s_d == 1 ? 0u : 1u, step_p = t.n_s_p == 1 ? 0u : 1u;
+    const int n_ch = t.n_ch;
+    // bits 0 / 1 / 2: expand / depthwise / project needs the general form; bits 3 / 4 / 5: a shift below 8
+    int flags = 0;
     for (int c = tid; c < n_ch; c += nthreads) {
-        const int be = b_e != nullptr ? b_e[(size_t)(unsigned)c] : 0;
-        const int bd = b_d != nullptr ? b_d[(size_t)(unsigned)c] : 0;
-        const int se = s_e[(size_t)(step_e * (unsigned)c)];
-        const int sd = s_d[(size_t)(step_d * (unsigned)c)];
-        flags |= short_ok(se, be, bound_e) ? 0 : 1;
-        flags |= short_ok(sd, bd, bound_d) ? 0 : 2;
-        flags |= se < 8 ? 4 : 0;
-        flags |= sd < 8 ? 8 : 0;
+        const int be = t.b_e != nullptr ? t.b_e[(size_t)(unsigned)c] : 0;
+        const int bd = t.b_d != nullptr ? t.b_d[(size_t)(unsigned)c] : 0;
+        const int se = t.s_e[(size_t)(step_e * (unsigned)c)];
+        const int sd = t.s_d[(size_t)(step_d * (unsigned)c)];
+        flags |= short_ok(se, be, t.bound_e) ? 0 : 1;
+        flags |= short_ok(sd, bd, t.bound_d) ? 0 : 2;
+        flags |= se < 8 ? 8 : 0;
+        flags |= sd < 8 ? 16 : 0;
         const int se1 = min(max(se, 1), 31), sd1 = min(max(sd, 1), 31); // defined shifts where the form does not apply
-        tab_e[c] = be + (1 << (se1 - 1));
-        tab_e[n_ch + c] = max(0, se - 8);
-        tab_e[2 * n_ch + c] = max(0, 8 - se);
-        tab_d[c] = bd + (1 << (sd1 - 1));
-        tab_d[n_ch + c] = max(0, sd - 8);
-        tab_d[2 * n_ch + c] = max(0, 8 - sd);
+        t.tab_e[c] = be + (1 << (se1 - 1));
+        t.tab_e[n_ch + c] = max(0, se - 8);
+        t.tab_e[2 * n_ch + c] = max(0, 8 - se);
+        t.tab_d[c] = bd + (1 << (sd1 - 1));
+        t.tab_d[n_ch + c] = max(0, sd - 8);
+        t.tab_d[2 * n_ch + c] = max(0, 8 - sd);
+    }
+    // the project channels are few: the last lanes of the workgroup take them, so that with up to
+    // nthreads - n_pad_p expanded channels no lane does both
+    for (int c = nthreads - 1 - tid; c < t.n_pad_p; c += nthreads) {
+        const bool exists = c < t.n_ch_p;
+        const int bp = (exists && t.b_p != nullptr) ? t.b_p[(size_t)(unsigned)c] : 0;
+        const int sp = exists ? t.s_p[(size_t)(step_p * (unsigned)c)] : 8;
+        flags |= short_ok(sp, bp, t.bound_p) ? 0 : 4;
+        flags |= sp < 8 ? 32 : 0;
+        const int sp1 = min(max(sp, 1), 31);
+        t.tab_p[c] = bp + (1 << (sp1 - 1));
+        t.tab_p[t.n_pad_p + c] = max(0, sp - 8);
+        t.tab_p[2 * t.n_pad_p + c] = max(0, 8 - sp);
     }
     {
         int wf = 0; // OR over the wavefront's lanes, bit by bit
 #pragma unroll
-        for (int b = 0; b < 4; b++)
+        for (int b = 0; b < 6; b++)
             wf |= __any(flags & (1 << b)) ? 1 << b : 0;
         if ((tid & 63) == 0)
-            votes[tid >> 6] = wf;
+            t.votes[tid >> 6] = wf;
     }
     __syncthreads();
     int all = 0;
     for (int w = 0; w < (nthreads >> 6); w++)
-        all |= votes[w];
-    if (all & 3) { // uniform
+        all |= t.votes[w];
+    if (all & 7) { // uniform
         for (int c = tid; c < n_ch; c += nthreads) {
             if (all & 1) {
-                tab_e[c] = b_e != nullptr ? b_e[(size_t)(unsigned)c] : 0;
-                tab_e[n_ch + c] = s_e[(size_t)(step_e * (unsigned)c)];
-                tab_e[2 * n_ch + c] = 0;
+                t.tab_e[c] = t.b_e != nullptr ? t.b_e[(size_t)(unsigned)c] : 0;
+                t.tab_e[n_ch + c] = t.s_e[(size_t)(step_e * (unsigned)c)];
+                t.tab_e[2 * n_ch + c] = 0;
             }
             if (all & 2) {
-                tab_d[c] = b_d != nullptr ? b_d[(size_t)(unsigned)c] : 0;
-                tab_d[n_ch + c] = s_d[(size_t)(step_d * (unsigned)c)];
-                tab_d[2 * n_ch + c] = 0;
+                t.tab_d[c] = t.b_d != nullptr ? t.b_d[(size_t)(unsigned)c] : 0;
+                t.tab_d[n_ch + c] = t.s_d[(size_t)(step_d * (unsigned)c)];
+                t.tab_d[2 * n_ch + c] = 0;
+            }
+        }
+        if (all & 4) {
+            for (int c = tid; c < t.n_pad_p; c += nthreads) {
+                const bool exists = c < t.n_ch_p;
+                t.tab_p[c] = (exists && t.b_p != nullptr) ? t.b_p[(size_t)(unsigned)c] : 0;
+                t.tab_p[t.n_pad_p + c] = exists ? t.s_p[(size_t)(step_p * (unsigned)c)] : 8;
+                t.tab_p[2 * t.n_pad_p + c] = 0;
             }
         }
         __syncthreads();
     }
-    mode_e = (all & 1) ? -1 : (half_even ? 2 : ((all & 4) ? 1 : 0));
-    mode_d = (all & 2) ? -1 : (half_even ? 2 : ((all & 8) ? 1 : 0));
+    mode_e = (all & 1) ? -1 : (half_even ? 2 : ((all & 8) ? 1 : 0));
+    mode_d = (all & 2) ? -1 : (half_even ? 2 : ((all & 16) ? 1 : 0));
+    mode_p = (all & 4) ? -1 : (half_even ? 2 : ((all & 32) ? 1 : 0));
 }
 
+// MULTIPLIERS: in mode 1 turn the left-shift counts into the packed multipliers of pack_fast4<4>
+// (wave_pack_tab); false leaves the counts (wave_pack, pack_fast4_add).
+template <bool MULTIPLIERS = true>
 __device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch, int ch, int mode)
 {
     StageConsts c;
@@ -233,7 +268,7 @@ __device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch
     c.lsh = v4i{0, 0, 0, 0};
     if (mode == 1 || mode == 2)
         c.lsh = *reinterpret_cast<const v4i *>(tab + 2 * n_ch + ch);
-    if (mode == 1) // the multiplier form of pack_fast4<4>: 2^lsh of the channel pairs as packed int16
+    if (MULTIPLIERS && mode == 1) // the multiplier form of pack_fast4<4>: 2^lsh of the channel pairs as packed int16
         c.lsh = v4i{(1 << c.lsh[0]) | (65536 << c.lsh[1]), (1 << c.lsh[2]) | (65536 << c.lsh[3]), 0, 0};
     c.mode = mode;
     return c;

@@ -106,6 +106,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
     unsigned char *dw_l = smem + a.off_dw + wave * a.wave_bytes;
     int *tab_e = reinterpret_cast<int *>(smem + a.off_tab);
     int *tab_d = tab_e + 3 * a.p.exp_c;
+    int *tab_p = tab_d + 3 * a.p.exp_c; // 3 x 16 rt entries
     const int c0 = p.in_c;
 
     // tile of this wavefront; consecutive tiles of an image stay on one XCD (its L2 holds the shared halo rows).
@@ -313,9 +314,30 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
 
     // the stage tables, by the whole group
     const unsigned bound_e = (unsigned)(ROWCONV ? p.ek_h * p.ek_w * c0 : c0) * 16384u, bound_d = 9u * 16384u;
-    int mode_e, mode_d;
-    build_stage_tables_pair(reinterpret_cast<int *>(smem + a.off_tab + p.exp_c * 24), tab_e, tab_d, p.b_expand, p.s_expand, p.n_s_expand, p.b_dw, p.s_dw, p.n_s_dw, p.exp_c, bound_e,
-                            bound_d, HE, (int)threadIdx.x, 64 * kWavesPerGroup, mode_e, mode_d);
+    int mode_e, mode_d, mode_p;
+    {
+        StageTablesArgs t;
+        t.tab_e = tab_e;
+        t.tab_d = tab_d;
+        t.tab_p = tab_p;
+        t.votes = tab_p + 3 * 16 * a.rt;
+        t.b_e = p.b_expand;
+        t.s_e = p.s_expand;
+        t.b_d = p.b_dw;
+        t.s_d = p.s_dw;
+        t.b_p = p.b_project;
+        t.s_p = p.s_project;
+        t.n_s_e = p.n_s_expand;
+        t.n_s_d = p.n_s_dw;
+        t.n_s_p = p.n_s_project;
+        t.n_ch = p.exp_c;
+        t.n_ch_p = p.out_c;
+        t.n_pad_p = 16 * a.rt;
+        t.bound_e = bound_e;
+        t.bound_d = bound_d;
+        t.bound_p = (unsigned)p.exp_c * 16384u;
+        build_stage_tables(t, HE, (int)threadIdx.x, 64 * kWavesPerGroup, mode_e, mode_d, mode_p);
+    }
     // tables (and, in ROWCONV builds, the expand operands) complete; no barrier after this one
     if constexpr (ROWCONV)
         cur = load_chunk(0);
@@ -403,14 +425,11 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
             }
         }
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
-    const unsigned bound_p = (unsigned)p.exp_c * 16384u;
 #pragma unroll
     for (int r = 0; r < RT; r++) {
         if (r < n_rt) { // uniform
             const int c = 16 * r + 4 * quad;
-            v4i bp, sp;
-            load_bias_shift(p.b_project, p.s_project, p.n_s_project, c, p.out_c, bp, sp);
-            const StageConsts cp = stage_consts(bp, sp, bound_p, HE);
+            const StageConsts cp = read_stage_table<false>(tab_p, 16 * a.rt, c, mode_p);
             const bool live = col_ok && c < p.out_c;
             auto rows = [&](auto mode_tag) {
                 constexpr int MODE = decltype(mode_tag)::value;
@@ -464,7 +483,7 @@ void wave_layout(WaveArgs &a, size_t *lds)
 {
     const int exp_px = std::max(((a.n_xpt + 3) & ~3) * 16, (a.ph * a.pw + 48 + 15) & ~15);
     a.off_tab = 0; // two stages x [init | rsh | lsh] x int32
-    a.off_aop = a.p.exp_c * 24 + kStageVoteBytes; // the workgroup's vote words sit behind the tables
+    a.off_aop = a.p.exp_c * 24 + a.rt * 16 * 12 + kStageVoteBytes; // expand, depthwise and project tables, vote words
     a.off_exp = a.off_aop + (mbconv_expand_is_pointwise(a.p) ? 0 : a.p.exp_c * 64);
     a.off_dw = a.off_exp + exp_px * 16;
     a.wave_bytes = exp_px * 16 + a.th * 16 * kDws;
