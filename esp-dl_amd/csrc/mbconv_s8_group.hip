@@ -251,6 +251,20 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
 #pragma unroll
             for (int i = 0; i < NT; i++)
                 accp[i] = v4i{0, 0, 0, 0};
+            // the residual words of this row tile are requested now and used after the products
+            const int c = 16 * rt + 4 * quad;
+            bool live[NT];
+            unsigned off[NT];
+            int rv[NT];
+#pragma unroll
+            for (int i = 0; i < NT; i++) {
+                // pixel slot -> (row, column) of the tile: twp slots per output row
+                const int slot = (t0 + i) * 16 + col;
+                const int oy = a.twp == 16 ? t0 + i : (slot >> 3), ox = a.twp == 16 ? col : (slot & 7);
+                live[i] = t0 + i < a.npt && oy < th_real && ox < p.out_w && c < p.out_c;
+                off[i] = (unsigned)(((oy0 + oy) * p.out_w + ox) * p.out_c + c);
+                rv[i] = res_img != nullptr ? *reinterpret_cast<const int *>(res_img + (size_t)(live[i] ? off[i] : 0u)) : 0;
+            }
             for (int k0 = 0; k0 < ksp; k0 += 8) {
                 // the next block of operand A (the next k steps, or the first ones of the next row tile) is
                 // requested before this block's products
@@ -278,21 +292,7 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
                         ap[kk] = an[kk];
                 }
             }
-            const int c = 16 * rt + 4 * quad;
             const StageConsts cp = read_stage_table<false>(tab_p, 16 * a.rt, c, mode_p);
-            // residual words of all pixel tiles first, then the epilogues
-            bool live[NT];
-            unsigned off[NT];
-            int rv[NT];
-#pragma unroll
-            for (int i = 0; i < NT; i++) {
-                // pixel slot -> (row, column) of the tile: twp slots per output row
-                const int slot = (t0 + i) * 16 + col;
-                const int oy = a.twp == 16 ? t0 + i : (slot >> 3), ox = a.twp == 16 ? col : (slot & 7);
-                live[i] = t0 + i < a.npt && oy < th_real && ox < p.out_w && c < p.out_c;
-                off[i] = (unsigned)(((oy0 + oy) * p.out_w + ox) * p.out_c + c);
-                rv[i] = res_img != nullptr ? *reinterpret_cast<const int *>(res_img + (size_t)(live[i] ? off[i] : 0u)) : 0;
-            }
 #pragma unroll
             for (int i = 0; i < NT; i++) {
                 v4i acc = accp[i];
