@@ -65,6 +65,7 @@ struct WaveArgs {
     int th, tw, ph, pw;
     int n_xpt; // pixel tiles of 16 in the patch
     int tiles_x, tiles_y, n_tiles;
+    int tpw; // ROWCONV: consecutive tiles per wavefront
     int n_sub; // chunks of 16 expanded channels
     int rt;    // project row tiles of 16 filters
     int x_vec16, we_vec16;
@@ -116,8 +117,14 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
         const int per = gridDim.x >> 3;
         group = (int)(blockIdx.x & 7u) * per + (int)(blockIdx.x >> 3);
     }
-    const bool has_tile = group * kWavesPerGroup + wave < a.n_tiles; // uniform
-    const int tile = min(group * kWavesPerGroup + wave, a.n_tiles - 1);
+    // ROWCONV builds: a wavefront takes a.tpw consecutive tiles (their tiles are short: two chunks of expanded
+    // channels), so that the workgroup's set-up serves several tiles
+    int mode_e = 0, mode_d = 0, mode_p = 0;
+    const int tpw = ROWCONV ? a.tpw : 1;
+    for (int it = 0; it < tpw; it++) {
+    const int tile_id = (group * kWavesPerGroup + wave) * tpw + it;
+    const bool has_tile = tile_id < a.n_tiles; // uniform
+    const int tile = min(tile_id, a.n_tiles - 1);
     const unsigned n = fastdiv((unsigned)tile, a.fd_tiles_yx);
     const unsigned rem = (unsigned)tile - n * a.fd_tiles_yx.d;
     const unsigned ty = fastdiv(rem, a.fd_tiles_x);
@@ -294,7 +301,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
     if constexpr (!ROWCONV)
         cur = load_chunk(0);
 
-    if constexpr (ROWCONV) {
+    if (ROWCONV && it == 0) {
         // operand A of the expand stage: filter row `q` of expanded channel f, zero-padded to 16 bytes
         const int wb = p.ek_w * c0;
         for (int i = (int)threadIdx.x; i < p.exp_c * 4; i += 64 * kWavesPerGroup) {
@@ -314,8 +321,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
 
     // the stage tables, by the whole group
     const unsigned bound_e = (unsigned)(ROWCONV ? p.ek_h * p.ek_w * c0 : c0) * 16384u, bound_d = 9u * 16384u;
-    int mode_e, mode_d, mode_p;
-    {
+    if (it == 0) { // uniform over the workgroup: every wavefront is in its first tile
         StageTablesArgs t;
         t.tab_e = tab_e;
         t.tab_d = tab_d;
@@ -337,6 +343,8 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
         t.bound_d = bound_d;
         t.bound_p = (unsigned)p.exp_c * 16384u;
         build_stage_tables(t, HE, (int)threadIdx.x, 64 * kWavesPerGroup, mode_e, mode_d, mode_p);
+    } else {
+        wave_lds_sync(); // the previous tile's reads of the wavefront's LDS areas come before this tile's writes
     }
     // tables (and, in ROWCONV builds, the expand operands) complete; no barrier after this one
     if constexpr (ROWCONV)
@@ -464,6 +472,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
                 rows(std::integral_constant<int, -1>{});
         }
     }
+    } // tiles of this wavefront
 }
 
 struct WavePlan {
@@ -471,6 +480,7 @@ struct WavePlan {
     WaveArgs a;
     size_t lds;
     int nxpt_max, rt_max;
+    int cus; // compute units of the device the launch goes to
 };
 
 constexpr int kPtMax = 8;
@@ -569,10 +579,23 @@ WavePlan wave_plan(const MbconvParams &p)
 template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false>
 hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
 {
-    const WaveArgs &a = plan.a;
-    const unsigned groups = (unsigned)((a.n_tiles + kWavesPerGroup - 1) / kWavesPerGroup);
-    hipLaunchKernelGGL((mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV>), dim3(groups),
-                       dim3(64 * kWavesPerGroup), plan.lds, stream, a);
+    WaveArgs a = plan.a;
+    auto kernel = mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV>;
+    a.tpw = 1;
+    if (ROWCONV) {
+        // Tiles per wavefront: these tiles are short (two chunks of expanded channels for a 32-filter stem), so
+        // a workgroup's set-up weighs on them.  Up to 16 rounds over the device the launch becomes one round of
+        // resident workgroups that walk ceil(tiles / resident wavefronts) tiles each (measured on MobileNetV2's
+        // stem at batch 256: 14 tiles per wavefront 0.742 ms per step, 7: 0.746, 10: 0.765, 1: 0.777); beyond
+        // that the rounds balance themselves and eight tiles per wavefront amortize the set-up.
+        const long long resident = (long long)plan.cus * resident_workgroups_per_cu(kernel, 64 * kWavesPerGroup, plan.lds) *
+            kWavesPerGroup;
+        const long long per_wave = (a.n_tiles + resident - 1) / resident;
+        a.tpw = per_wave <= 16 ? (int)std::max<long long>(1, per_wave) : 8;
+    }
+    const int per_group = kWavesPerGroup * a.tpw;
+    const unsigned groups = (unsigned)((a.n_tiles + per_group - 1) / per_group);
+    hipLaunchKernelGGL(kernel, dim3(groups), dim3(64 * kWavesPerGroup), plan.lds, stream, a);
     return hipGetLastError();
 }
 
@@ -638,7 +661,6 @@ long long mbconv_s8_wave_tiles(const MbconvParams &p)
 
 hipError_t launch_mbconv_s8_wave(const MbconvParams &p, int cu_count, hipStream_t stream)
 {
-    (void)cu_count;
     if ((long long)p.batch * p.out_h * p.out_w == 0)
         return hipSuccess;
     WavePlan plan = wave_plan(p);
@@ -648,6 +670,7 @@ hipError_t launch_mbconv_s8_wave(const MbconvParams &p, int cu_count, hipStream_
     if (tiles > 0x7fffffff)
         return hipErrorInvalidValue;
     plan.a.n_tiles = (int)tiles;
+    plan.cus = cu_count > 0 ? cu_count : kPlanCus;
     static const bool trace = getenv("ESPDL_HIP_TRACE") != nullptr;
     if (trace)
         fprintf(stderr, "mbconv_s8_wave: %dx%d in %d exp %d out %d s%d tile %dx%d patch %dx%d n_xpt %d rt %d lds %zu tiles %lld\n",
