@@ -37,9 +37,9 @@ MACHINE_BALANCE = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)  # OP per byte
 # 256 MiB element-wise kernel of known traffic gave in the same runs).  Only valid for config 3 at
 # batch 256; any other workload reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "mbconv_s8_wave": 38590363.0,   # 7 launches (the stem convolution rides in the first block's launch)
-    "mbconv_s8_group": 14708848.0,  # 10 launches
-    "conv2d_s8": 21020144.0,        # head convolution and classifier
+    "mbconv_s8_wave": 42326313.0,   # 7 launches (the stem convolution rides in the first block's launch)
+    "mbconv_s8_group": 13716755.0,  # 10 launches
+    "conv2d_s8": 21020512.0,        # head convolution and classifier
     "elementwise_s8": None,
 }
 
@@ -135,8 +135,8 @@ def check_against_oracle(spec, x, got, chunk=32):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--batch", type=int, default=256)
     ap.add_argument("--config", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
