@@ -74,96 +74,10 @@ struct StageConsts {
     int mode;
 };
 
-// b, sh: bias and shift of the lane's four channels (channels that do not exist: 0 and 8).
-__device__ __forceinline__ StageConsts stage_consts(const v4i &b, const v4i &sh, unsigned mac_bound, bool half_even)
-{
-    StageConsts c;
-    bool ok = true;
-#pragma unroll
-    for (int r = 0; r < 4; r++)
-        ok = ok && short_ok(sh[r], b[r], mac_bound);
-    if (__all(ok)) {
-        bool any_lsh = false;
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            c.init[r] = b[r] + (1 << (sh[r] - 1));
-            c.rsh[r] = max(0, sh[r] - 8);
-            c.lsh[r] = max(0, 8 - sh[r]);
-            any_lsh = any_lsh || sh[r] < 8;
-        }
-        c.mode = half_even ? 2 : (__any(any_lsh) ? 1 : 0);
-    } else {
-        c.init = b;
-        c.rsh = sh;
-        c.lsh = v4i{0, 0, 0, 0};
-        c.mode = -1;
-    }
-    return c;
-}
-
-// Per-channel constants of a stage for every channel of the block, built once per tile in LDS by all lanes
-// (channel = lane + 64 i) as [init | right shift | left shift][n_ch], in the form the stage's epilogue
-// `mode` wants (see StageConsts); returns that mode, one for the whole stage.
-__device__ __forceinline__ int build_stage_table(int *tab, const int32_t *bias, const int32_t *shift, int n_shift,
-                                                 int n_ch, unsigned mac_bound, bool half_even, int lane)
-{
-    bool ok = true, any_lsh = false;
-    for (int c = lane; c < n_ch; c += 64) {
-        const int b = bias != nullptr ? bias[c] : 0;
-        const int sh = shift[n_shift == 1 ? 0 : c];
-        ok = ok && short_ok(sh, b, mac_bound);
-        any_lsh = any_lsh || sh < 8;
-        tab[c] = b;
-        tab[n_ch + c] = sh;
-    }
-    const bool fast = __all(ok) != 0;
-    const int mode = !fast ? -1 : (half_even ? 2 : (__any(any_lsh) ? 1 : 0));
-    for (int c = lane; c < n_ch; c += 64) { // each lane revisits the channels it wrote
-        const int b = tab[c], sh = tab[n_ch + c];
-        if (fast) {
-            tab[c] = b + (1 << (sh - 1));
-            tab[n_ch + c] = max(0, sh - 8);
-            tab[2 * n_ch + c] = max(0, 8 - sh);
-        } else {
-            tab[2 * n_ch + c] = 0;
-        }
-    }
-    return mode;
-}
-
-// The same tables built by all `nthreads` lanes of a workgroup (thread = channel + nthreads * i); the mode
-// is agreed on with workgroup votes, so every lane of the workgroup must call this.  The tables are
-// complete for other wavefronts only after the caller's next barrier.
-__device__ __forceinline__ int build_stage_table_group(int *tab, const int32_t *bias, const int32_t *shift, int n_shift,
-                                                       int n_ch, unsigned mac_bound, bool half_even, int tid,
-                                                       int nthreads)
-{
-    int ok = 1, any_lsh = 0;
-    const unsigned step = n_shift == 1 ? 0u : 1u;
-    for (int c = tid; c < n_ch; c += nthreads) {
-        const int b = bias != nullptr ? bias[(size_t)(unsigned)c] : 0;
-        const int sh = shift[(size_t)(step * (unsigned)c)];
-        ok &= short_ok(sh, b, mac_bound) ? 1 : 0;
-        any_lsh |= sh < 8 ? 1 : 0;
-        tab[c] = b;
-        tab[n_ch + c] = sh;
-    }
-    const bool fast = __syncthreads_and(ok) != 0;
-    const bool lsh = __syncthreads_or(any_lsh) != 0;
-    const int mode = !fast ? -1 : (half_even ? 2 : (lsh ? 1 : 0));
-    for (int c = tid; c < n_ch; c += nthreads) { // every lane revisits the channels it wrote
-        const int b = tab[c], sh = tab[n_ch + c];
-        if (fast) {
-            tab[c] = b + (1 << (sh - 1));
-            tab[n_ch + c] = max(0, sh - 8);
-        }
-        tab[2 * n_ch + c] = fast ? max(0, 8 - sh) : 0;
-    }
-    return mode;
-}
-
-// The tables of the three stages (expand and depthwise: the same n_ch channels; project: see below) with ONE memory round trip
-// and ONE workgroup vote, which is also the barrier after which the tables are complete: every lane writes
+// Per-channel constants of a stage live in LDS as three rows of n_ch int32: [bias + rounding constant |
+// right shift | left shift] in the form the short epilogue wants, or [bias | shift | 0] for the general one.
+// build_stage_tables fills the tables of the three stages (expand and depthwise: the same n_ch channels;
+// project: see below) with ONE memory round trip and ONE workgroup vote, which is also the barrier after which the tables are complete: every lane writes
 // the short-epilogue form of its channels straight away and the vote tells whether some channel of a stage
 // cannot take it; only then (rare) that stage's table is rewritten with the plain bias and shift, behind a
 // second barrier.  `votes` is one LDS word per wavefront of the workgroup (kStageVoteBytes in all; a wavefront
@@ -272,25 +186,6 @@ __device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch
         c.lsh = v4i{(1 << c.lsh[0]) | (65536 << c.lsh[1]), (1 << c.lsh[2]) | (65536 << c.lsh[3]), 0, 0};
     c.mode = mode;
     return c;
-}
-
-// Bias and shift of four consecutive channels starting at `ch` (a multiple of 4), straight from memory,
-// branch-free (see load16_partial): channels that do not exist give bias 0 and shift 8.
-__device__ __forceinline__ void load_bias_shift(const int32_t *bias, const int32_t *shift, int n_shift, int ch, int n_ch,
-                                                v4i &b, v4i &sh)
-{
-    const bool exists = ch < n_ch; // channel counts are multiples of 4: all four exist or none
-    const int32_t *bp = bias != nullptr ? bias : shift;
-    const int cb = (exists && bias != nullptr) ? ch : 0;
-    const int cs = (exists && n_shift != 1) ? ch : 0;
-    const int step = n_shift != 1 ? 1 : 0;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int bv = bp[cb + (bias != nullptr ? r : 0)];
-        const int sv = shift[cs + step * r];
-        b[r] = (exists && bias != nullptr) ? bv : 0;
-        sh[r] = exists ? sv : 8;
-    }
 }
 
 template <int MODE>
