@@ -140,17 +140,34 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
     unsigned xmask = 0;
     if constexpr (!ROWCONV) {
         const int8_t *img = p.in + (long long)n * p.in_h * p.in_w * c0;
+        if constexpr (EXACT && S == 1) {
+            // guard-free builds at stride 1 have patches of exactly 16 columns: pixel tile = patch row and lane
+            // column = patch column, so the column part of the address and of the validity test is formed once
+            // and a patch row costs one addition (rows are uniform: one scalar bit mask)
+            const int ix = ix0 + col;
+            const bool col_valid = (unsigned)ix < (unsigned)p.in_w;
+            const int o0 = (iy0 * p.in_w + ix) * c0 + 16 * quad, o_step = p.in_w * c0;
+            unsigned rows = 0;
 #pragma unroll
-        for (int pt = 0; pt < NXPT; pt++) {
-            xb[pt] = v4i{0, 0, 0, 0};
-            if (pt < n_xpt) { // uniform
-                const unsigned pp = (unsigned)(pt * 16 + col);
-                const unsigned prow = fastdiv(pp, a.fd_pw);
-                const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
-                const bool valid = (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
-                xmask |= valid ? 1u << pt : 0u;
-                xb[pt] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
-                                               valid ? c0 - 16 * quad : 0);
+            for (int pt = 0; pt < NXPT; pt++)
+                rows |= (unsigned)(iy0 + pt) < (unsigned)p.in_h ? 1u << pt : 0u;
+            xmask = col_valid ? rows : 0u;
+#pragma unroll
+            for (int pt = 0; pt < NXPT; pt++)
+                xb[pt] = load16_partial<VEC16>(img, (unsigned)(o0 + pt * o_step), ((xmask >> pt) & 1u) ? c0 - 16 * quad : 0);
+        } else {
+#pragma unroll
+            for (int pt = 0; pt < NXPT; pt++) {
+                xb[pt] = v4i{0, 0, 0, 0};
+                if (pt < n_xpt) { // uniform
+                    const unsigned pp = (unsigned)(pt * 16 + col);
+                    const unsigned prow = fastdiv(pp, a.fd_pw);
+                    const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
+                    const bool valid = (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
+                    xmask |= valid ? 1u << pt : 0u;
+                    xb[pt] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
+                                                   valid ? c0 - 16 * quad : 0);
+                }
             }
         }
     } else {
@@ -625,7 +642,7 @@ hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
     if (!a.p.half_even) {
         // guard-free builds for the tile plans of MobileNetV2-style blocks (round half up)
         const auto is = [&](int nxpt, int rt, int th, int stride, bool v) {
-            return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v;
+            return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v && (stride != 1 || a.pw == 16);
         };
         if (is(17, 2, 4, 2, true))
             return launch_one<17, 2, 4, 2, false, true, true>(plan, stream);
