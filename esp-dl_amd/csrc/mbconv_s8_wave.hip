@@ -279,6 +279,25 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
     const int8_t *res_img = p.residual != nullptr ? p.residual + img_off : nullptr;
     int8_t *out_img = p.out + img_off;
     const unsigned off0 = (unsigned)((oy0 * p.out_w + ox) * p.out_c + 4 * quad);
+    // The residual words (the guard-free builds have the registers for it) are requested now, with the patch,
+    // and used after the last chunk: in the epilogue their round trip would be fully exposed.
+    constexpr bool kEarlyResidual = EXACT;
+    int resw[RT][PT];
+    auto request_residual = [&]() {
+#pragma unroll
+        for (int r = 0; r < RT; r++)
+#pragma unroll
+            for (int t = 0; t < PT; t++) {
+                resw[r][t] = 0;
+                if (res_img != nullptr) { // uniform
+                    const bool live = col_ok && t < th_real && 16 * r + 4 * quad < p.out_c;
+                    resw[r][t] = *reinterpret_cast<const int *>(
+                        res_img + (size_t)(live ? off0 + (unsigned)(t * p.out_w * p.out_c + 16 * r) : 0u));
+                }
+            }
+    };
+    if constexpr (kEarlyResidual)
+        request_residual();
     // Filters of a chunk are requested one chunk ahead (ChunkW), the project filters of a group of four
     // chunks at the start of the group: their latency hides behind the chunk in between.
     struct ChunkW {
@@ -436,59 +455,57 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
         cur = nxt;
     }
 
-    // ---- project epilogue, residual Add, stores; every residual word is requested before the first is used
-    int resw[RT][PT];
-#pragma unroll
-    for (int r = 0; r < RT; r++)
-#pragma unroll
-        for (int t = 0; t < PT; t++) {
-            resw[r][t] = 0;
-            if (res_img != nullptr) { // uniform
-                const bool live = col_ok && t < th_real && 16 * r + 4 * quad < p.out_c;
-                resw[r][t] = *reinterpret_cast<const int *>(
-                    res_img + (size_t)(live ? off0 + (unsigned)(t * p.out_w * p.out_c + 16 * r) : 0u));
-            }
-        }
+    // ---- project epilogue, residual Add, stores
+    if constexpr (!kEarlyResidual)
+        request_residual(); // every residual word is requested before the first is used
+    // The uniform choices (epilogue form, residual or not) are made once, outside the loops over the words, and
+    // a row of a ragged last tile that does not exist is a store that no lane takes: the words of a tile are
+    // one straight-line block.
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
+    auto words = [&](auto mode_tag, auto res_tag) {
+        constexpr int MODE = decltype(mode_tag)::value;
+        constexpr bool RES = decltype(res_tag)::value;
 #pragma unroll
-    for (int r = 0; r < RT; r++) {
-        if (r < n_rt) { // uniform
-            const int c = 16 * r + 4 * quad;
-            const StageConsts cp = read_stage_table<false>(tab_p, 16 * a.rt, c, mode_p);
-            const bool live = col_ok && c < p.out_c;
-            auto rows = [&](auto mode_tag) {
-                constexpr int MODE = decltype(mode_tag)::value;
+        for (int r = 0; r < RT; r++) {
+            if (EXACT || r < n_rt) { // uniform
+                const int c = 16 * r + 4 * quad;
+                const StageConsts cp = read_stage_table<false>(tab_p, 16 * a.rt, c, mode_p);
+                const bool live = col_ok && c < p.out_c;
 #pragma unroll
                 for (int t = 0; t < PT; t++) {
-                    if (t < th_real) { // uniform
-                        v4i acc = accp[r][t];
+                    v4i acc = accp[r][t];
 #pragma unroll
-                        for (int k = 0; k < 4; k++)
-                            acc[k] += cp.init[k];
-                        int word;
-                        if (res_img != nullptr) { // uniform
-                            if constexpr (MODE >= 0)
-                                word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, resw[r][t]);
-                            else
-                                word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), resw[r][t]);
-                        } else {
-                            word = wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE);
-                        }
-                        if (live)
-                            *reinterpret_cast<int *>(out_img + (size_t)(off0 + (unsigned)(t * p.out_w * p.out_c + 16 * r))) = word;
+                    for (int k = 0; k < 4; k++)
+                        acc[k] += cp.init[k];
+                    int word;
+                    if constexpr (RES) {
+                        if constexpr (MODE >= 0)
+                            word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, resw[r][t]);
+                        else
+                            word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), resw[r][t]);
+                    } else {
+                        word = wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE);
                     }
+                    if (live && t < th_real)
+                        *reinterpret_cast<int *>(out_img + (size_t)(off0 + (unsigned)(t * p.out_w * p.out_c + 16 * r))) = word;
                 }
-            };
-            if (cp.mode == 0)
-                rows(std::integral_constant<int, 0>{});
-            else if (cp.mode == 1)
-                rows(std::integral_constant<int, 1>{});
-            else if (cp.mode == 2)
-                rows(std::integral_constant<int, 2>{});
-            else
-                rows(std::integral_constant<int, -1>{});
+            }
         }
-    }
+    };
+    auto with_mode = [&](auto mode_tag) {
+        if (res_img != nullptr)
+            words(mode_tag, std::true_type{});
+        else
+            words(mode_tag, std::false_type{});
+    };
+    if (mode_p == -1)
+        with_mode(std::integral_constant<int, -1>{});
+    else if constexpr (HE)
+        with_mode(std::integral_constant<int, 2>{});
+    else if (mode_p == 0)
+        with_mode(std::integral_constant<int, 0>{});
+    else
+        with_mode(std::integral_constant<int, 1>{});
     } // tiles of this wavefront
 }
 
