@@ -846,21 +846,23 @@ int espdl_hip_mbconv_s8_preferred(const espdl_hip_mbconv_desc *desc)
     const int kind = espdl_hip_mbconv_s8_supported(desc);
     if (kind == 2)
         return 1;
-    if (kind == 5) // a workgroup per tile of a small image: at least one workgroup per compute unit
-        return (long long)desc->batch >= (cu_count_cached() > 0 ? cu_count_cached() : 256) ? 1 : 0;
-    if (kind != 4)
+    if (kind != 4 && kind != 5)
         return 0;
-    // one wavefront per tile: it needs several tiles per SIMD to keep the pipes busy, and at small images
-    // the separate kernels (which also split the channels) are as fast
     espdl::MbconvParams p = {};
     if (mbconv_geometry(desc, &p) != ESPDL_HIP_OK)
         return 0;
     static const int8_t *const aligned = reinterpret_cast<const int8_t *>(uintptr_t(256));
     p.in = aligned;
     p.w_expand = aligned;
-    const long long tiles = espdl::mbconv_s8_wave_tiles(p);
     const int cus = cu_count_cached() > 0 ? cu_count_cached() : 256;
-    return (p.in_h >= 28 && p.in_w >= 28 && tiles >= 4ll * cus) ? 1 : 0;
+    // Both single-launch kernels win with their guard-free builds only (one per tile plan of MobileNetV2-style
+    // blocks); the guarded builds cover every shape but are no faster than the separate launches.
+    if (kind == 5) // a workgroup per tile of a small image: at least one workgroup per compute unit
+        return (espdl::mbconv_s8_group_has_fast_build(p) && (long long)desc->batch >= cus) ? 1 : 0;
+    // one wavefront per tile: it needs several tiles per SIMD to keep the pipes busy, and at small images
+    // the separate kernels (which also split the channels) are as fast
+    const long long tiles = espdl::mbconv_s8_wave_tiles(p);
+    return (espdl::mbconv_s8_wave_has_fast_build(p) && p.in_h >= 28 && p.in_w >= 28 && tiles >= 4ll * cus) ? 1 : 0;
 }
 
 int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *w,

@@ -429,6 +429,34 @@ hipError_t launch_group_one(const GroupPlan &plan, hipStream_t stream)
     return hipGetLastError();
 }
 
+// The guard-free builds: the tile plans of MobileNetV2's 14 x 14 and 7 x 7 blocks, in both rounding modes.
+// Returns false when the plan has none; with `dry` nothing is launched.
+template <bool HE>
+bool launch_group_exact(const GroupPlan &plan, hipStream_t stream, bool dry, hipError_t *err)
+{
+    const GroupArgs &a = plan.a;
+    const int s = a.p.stride_h;
+    const auto is = [&](int nxpt, int kse, int th, int stride) {
+        return a.n_xpt == nxpt && a.kse == kse && a.th == th && s == stride;
+    };
+#define ESPDL_GROUP_EXACT(NXPT, KSE, PT, S)                                        \
+    do {                                                                            \
+        if (!dry)                                                                   \
+            *err = launch_group_one<NXPT, KSE, PT, S, HE, true>(plan, stream);      \
+        return true;                                                                \
+    } while (0)
+    if (is(9, 1, 7, 1))
+        ESPDL_GROUP_EXACT(9, 1, 7, 1);
+    if (is(9, 2, 7, 1))
+        ESPDL_GROUP_EXACT(9, 2, 7, 1);
+    if (is(6, 3, 7, 1))
+        ESPDL_GROUP_EXACT(6, 3, 7, 1);
+    if (is(9, 2, 4, 2))
+        ESPDL_GROUP_EXACT(9, 2, 4, 2);
+#undef ESPDL_GROUP_EXACT
+    return false;
+}
+
 } // namespace
 
 bool mbconv_s8_group_supports(const MbconvParams &p)
@@ -455,23 +483,22 @@ hipError_t launch_mbconv_s8_group(const MbconvParams &p, int cu_count, hipStream
                 p.in_h, p.in_w, p.in_c, p.exp_c, p.out_c, p.stride_h, a.th, a.tw, a.ph, a.pw, a.n_xpt, a.kse, a.rt, a.npt,
                 plan.lds, tiles);
     const int s = p.stride_h;
-    if (!p.half_even) {
-        const auto is = [&](int nxpt, int kse, int th, int stride) {
-            return a.n_xpt == nxpt && a.kse == kse && a.th == th && s == stride;
-        };
-        if (is(9, 1, 7, 1))
-            return launch_group_one<9, 1, 7, 1, false, true>(plan, stream);
-        if (is(9, 2, 7, 1))
-            return launch_group_one<9, 2, 7, 1, false, true>(plan, stream);
-        if (is(6, 3, 7, 1))
-            return launch_group_one<6, 3, 7, 1, false, true>(plan, stream);
-        if (is(9, 2, 4, 2))
-            return launch_group_one<9, 2, 4, 2, false, true>(plan, stream);
+    hipError_t err = hipSuccess;
+    if (p.half_even ? launch_group_exact<true>(plan, stream, false, &err) : launch_group_exact<false>(plan, stream, false, &err))
+        return err;
+    if (!p.half_even)
         return s == 1 ? launch_group_one<9, 3, kGroupPtMax, 1, false, false>(plan, stream)
                       : launch_group_one<9, 3, kGroupPtMax, 2, false, false>(plan, stream);
-    }
     return s == 1 ? launch_group_one<9, 3, kGroupPtMax, 1, true, false>(plan, stream)
                   : launch_group_one<9, 3, kGroupPtMax, 2, true, false>(plan, stream);
+}
+
+bool mbconv_s8_group_has_fast_build(const MbconvParams &p)
+{
+    const GroupPlan plan = group_plan(p);
+    hipError_t err = hipSuccess;
+    return plan.ok &&
+        (p.half_even ? launch_group_exact<true>(plan, nullptr, true, &err) : launch_group_exact<false>(plan, nullptr, true, &err));
 }
 
 } // namespace espdl

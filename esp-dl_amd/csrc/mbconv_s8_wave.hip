@@ -641,42 +641,62 @@ hipError_t launch_generic(const WavePlan &plan, hipStream_t stream)
                                                : launch_one<17, 4, kPtMax, S, HE, false, false>(plan, stream);
 }
 
+// The guard-free builds: one per tile plan of MobileNetV2-style blocks, in both rounding modes.  Returns
+// false when the plan has none; with `dry` nothing is launched (the question is only whether one exists).
+template <bool HE>
+bool launch_exact(const WavePlan &plan, hipStream_t stream, bool dry, hipError_t *err)
+{
+    const WaveArgs &a = plan.a;
+    const bool vec16 = a.x_vec16 && a.we_vec16;
+    const int s = a.p.stride_h;
+#define ESPDL_WAVE_EXACT(NXPT, RT, PT, S, V, ROWCONV)                                     \
+    do {                                                                                   \
+        if (!dry)                                                                          \
+            *err = launch_one<NXPT, RT, PT, S, HE, V, true, ROWCONV>(plan, stream);        \
+        return true;                                                                       \
+    } while (0)
+    if (!mbconv_expand_is_pointwise(a.p)) {
+        // expand stage with a window: the stem + first block of MobileNetV2 at 224 x 224
+        if (a.n_xpt == 10 && a.pw == 16 && a.rt == 1 && a.th == 8 && s == 1)
+            ESPDL_WAVE_EXACT(10, 1, 8, 1, false, true);
+        return false;
+    }
+    const auto is = [&](int nxpt, int rt, int th, int stride, bool v) {
+        return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v && (stride != 1 || a.pw == 16);
+    };
+    if (is(17, 2, 4, 2, true))
+        ESPDL_WAVE_EXACT(17, 2, 4, 2, true, false);
+    if (is(17, 2, 4, 2, false))
+        ESPDL_WAVE_EXACT(17, 2, 4, 2, false, false);
+    if (is(10, 2, 8, 1, false))
+        ESPDL_WAVE_EXACT(10, 2, 8, 1, false, false);
+    if (is(10, 2, 8, 1, true))
+        ESPDL_WAVE_EXACT(10, 2, 8, 1, true, false);
+    if (is(9, 2, 7, 1, true))
+        ESPDL_WAVE_EXACT(9, 2, 7, 1, true, false);
+    if (is(10, 4, 2, 2, true))
+        ESPDL_WAVE_EXACT(10, 4, 2, 2, true, false);
+#undef ESPDL_WAVE_EXACT
+    return false;
+}
+
 hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
 {
     WaveArgs &a = plan.a;
-    const bool vec16 = a.x_vec16 && a.we_vec16;
     const int s = a.p.stride_h;
+    hipError_t err = hipSuccess;
+    if (a.p.half_even ? launch_exact<true>(plan, stream, false, &err) : launch_exact<false>(plan, stream, false, &err))
+        return err;
+    // guarded builds
     if (!mbconv_expand_is_pointwise(a.p)) {
-        // expand stage with a window: one guard-free build (the stem + first block of MobileNetV2 at 224 x 224)
-        if (!a.p.half_even && a.n_xpt == 10 && a.pw == 16 && a.rt == 1 && a.th == 8 && s == 1)
-            return launch_one<10, 1, 8, 1, false, false, true, true>(plan, stream);
         if (a.p.half_even)
             return s == 1 ? launch_one<17, 4, kPtMax, 1, true, false, false, true>(plan, stream)
                           : launch_one<17, 4, kPtMax, 2, true, false, false, true>(plan, stream);
         return s == 1 ? launch_one<17, 4, kPtMax, 1, false, false, false, true>(plan, stream)
                       : launch_one<17, 4, kPtMax, 2, false, false, false, true>(plan, stream);
     }
-    if (!a.p.half_even) {
-        // guard-free builds for the tile plans of MobileNetV2-style blocks (round half up)
-        const auto is = [&](int nxpt, int rt, int th, int stride, bool v) {
-            return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v && (stride != 1 || a.pw == 16);
-        };
-        if (is(17, 2, 4, 2, true))
-            return launch_one<17, 2, 4, 2, false, true, true>(plan, stream);
-        if (is(17, 2, 4, 2, false))
-            return launch_one<17, 2, 4, 2, false, false, true>(plan, stream);
-        if (is(10, 2, 8, 1, false))
-            return launch_one<10, 2, 8, 1, false, false, true>(plan, stream);
-        if (is(10, 2, 8, 1, true))
-            return launch_one<10, 2, 8, 1, false, true, true>(plan, stream);
-        if (is(9, 2, 7, 1, true))
-            return launch_one<9, 2, 7, 1, false, true, true>(plan, stream);
-        if (is(10, 4, 2, 2, true))
-            return launch_one<10, 4, 2, 2, false, true, true>(plan, stream);
-        if (is(13, 4, 3, 2, true))
-            return launch_one<13, 4, 3, 2, false, true, true>(plan, stream);
+    if (!a.p.half_even)
         return s == 1 ? launch_generic<1, false>(plan, stream) : launch_generic<2, false>(plan, stream);
-    }
     return s == 1 ? launch_generic<1, true>(plan, stream) : launch_generic<2, true>(plan, stream);
 }
 
@@ -685,6 +705,13 @@ hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
 bool mbconv_s8_wave_supports(const MbconvParams &p)
 {
     return wave_plan(p).ok;
+}
+
+bool mbconv_s8_wave_has_fast_build(const MbconvParams &p)
+{
+    const WavePlan plan = wave_plan(p);
+    hipError_t err = hipSuccess;
+    return plan.ok && (p.half_even ? launch_exact<true>(plan, nullptr, true, &err) : launch_exact<false>(plan, nullptr, true, &err));
 }
 
 long long mbconv_s8_wave_tiles(const MbconvParams &p)
