@@ -876,7 +876,7 @@ std::vector<module_info> Model::get_module_info(int repeats)
         }
         for (auto *module : m_execution_plan)
             module->hold_state(m_stream); // timing passes leave no trace in modules that carry data between passes
-        for (int r = -1; r < repeats; r++) { // pass -1 warms up and is not counted
+        for (int r = -3; r < repeats; r++) { // three passes warm up (caches, clocks) and are not counted
             (void)hipEventRecord(ev[0], s);
             for (size_t i = 0; i < n; i++) {
                 m_execution_plan[i]->forward(m_model_context, RUNTIME_MODE_AUTO);
