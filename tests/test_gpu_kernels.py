@@ -663,6 +663,41 @@ def test_mbconv_s8_expand_with_window_is_refused_where_not_covered():
     assert m.capi.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == 0  # a window without an expand stage
 
 
+def _block_desc(m, batch, hw, cin, ce, cout, stride, half_even=False):
+    d = m.capi.MbconvDesc()
+    d.batch, d.in_h, d.in_w, d.in_c, d.exp_c, d.out_c, d.has_expand = batch, hw, hw, cin, ce, cout, 1
+    d.k_h = d.k_w = 3
+    d.stride_h = d.stride_w = stride
+    d.dil_h = d.dil_w = 1
+    d.pad_top = d.pad_bottom = d.pad_left = d.pad_right = 1
+    d.act_expand = d.act_dw = m.capi.RELU
+    d.round_mode = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
+    d.n_shift_expand, d.n_shift_dw, d.n_shift_project = ce, ce, cout
+    return d
+
+
+def test_mbconv_s8_preferred_follows_the_fast_builds():
+    """dl::Model fuses a block where espdl_hip_mbconv_s8_preferred says so: yes for MobileNetV2's block shapes
+    at a batch that fills the device, in both rounding modes; no for a small batch, and no for a shape that
+    only the guarded builds take (they cover it, but the separate launches are as fast)."""
+    announce("mbconv_s8_preferred")
+    m = espdl()
+    L = m.capi.lib()
+    pref = lambda d: L.espdl_hip_mbconv_s8_preferred(ctypes.byref(d))  # noqa: E731
+    kind = lambda d: L.espdl_hip_mbconv_s8_supported(ctypes.byref(d))  # noqa: E731
+    blocks = [(112, 16, 96, 24, 2, 4), (56, 24, 144, 24, 1, 4), (56, 24, 144, 32, 2, 4), (28, 32, 192, 32, 1, 4),
+              (28, 32, 192, 64, 2, 4), (14, 64, 384, 64, 1, 5), (14, 96, 576, 96, 1, 5), (14, 96, 576, 160, 2, 5),
+              (7, 160, 960, 160, 1, 5), (7, 160, 960, 320, 1, 5)]
+    for hw, cin, ce, cout, stride, want_kind in blocks:
+        for he in (False, True):
+            d = _block_desc(m, 256, hw, cin, ce, cout, stride, he)
+            assert kind(d) == want_kind, (hw, cin, ce, cout, stride)
+            assert pref(d) == 1, (hw, cin, ce, cout, stride, he)
+        assert pref(_block_desc(m, 4, hw, cin, ce, cout, stride)) == 0  # too few tiles to fill the device
+    odd = _block_desc(m, 256, 50, 24, 144, 24, 1)  # 50 x 50: a tile plan without a guard-free build
+    assert kind(odd) == 4 and pref(odd) == 0
+
+
 @pytest.mark.parametrize("ce", [320, 192], ids=["e320_block_kernel", "e192_lds_tile_kernel"])
 @pytest.mark.parametrize("general_stage", [0, 1, 2], ids=["expand_general", "dw_general", "project_general"])
 def test_mbconv_s8_mixed_epilogues(oracle, general_stage, ce):
