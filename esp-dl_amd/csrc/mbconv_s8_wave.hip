@@ -17,7 +17,7 @@
 // ordered only by its own LDS accesses; the wavefronts of a compute unit sit at different points of the
 // chain, so the matrix pipe, the vector ALU, LDS and the memory pipeline of the unit are busy at once.
 // Four wavefronts form a workgroup for one reason only: they share the per-channel requantization tables
-// of the two inner stages, built once in LDS before the single barrier of the kernel.
+// of the three stages, built once in LDS before the single barrier of the kernel.
 //
 // Per tile:
 //   * the (th*s + 2) x (tw*s + 2) patch of the block input is loaded ONCE, straight into the registers
@@ -33,9 +33,9 @@
 //                  through two operand-A sets (rows 0-2 and rows 1-3); result to LDS as [pixel][64 ch];
 //     and after every 64 expanded channels the project product accumulates into registers
 //     (rows = 16 project filters, columns = one output row of the tile);
-//   * project epilogue, residual add, stores.
-// Filters, biases and shifts are read from global memory (L2) as they are needed: 16-byte pieces in
-// operand order, no staging.
+//   * project epilogue (constants from the LDS table), residual add, stores.
+// Filters are read from global memory (L2) as they are needed, one chunk ahead of their use: 16-byte pieces
+// in operand order, no staging.
 //
 // ROWCONV builds: the expand stage is a dense convolution with a window (a network's stem in front of its
 // first depthwise stage: conv2d_hwcn, esp-dl/dl/base/dl_base_conv2d.cpp:35-68) whose filter rows are at
@@ -43,7 +43,8 @@
 // (filter row = 16-lane group, 16 bytes of that row): operand B of a patch pixel is the window's row as it
 // lies in memory (k_w * in_c consecutive bytes, cut out of three aligned dwords with v_alignbyte_b32),
 // operand A the filter row padded with zeros, prepared once per workgroup in LDS.  Everything behind the
-// expand product is the same code.
+// expand product is the same code.  These tiles are short (two chunks for a 32-filter stem), so a wavefront
+// walks several consecutive tiles and the workgroup's set-up is paid once.
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
