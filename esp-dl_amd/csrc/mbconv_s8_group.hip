@@ -51,7 +51,7 @@ struct GroupArgs {
     int ds;    // LDS pixel stride of the shared depthwise tile, bytes
     int exp_bytes; // private expand area per wavefront
     int off_tab, off_exp, off_dw;
-    FastDiv fd_pw, fd_tiles_y, fd_npt;
+    FastDiv fd_pw, fd_tiles_y;
 };
 
 // EXACT: the plan is exactly (NXPT patch pixel tiles, KSE k steps, PT rows): no guards in the stage loops.
@@ -407,7 +407,6 @@ GroupPlan group_plan(const MbconvParams &p)
     a.nt = (a.npt + a.wp - 1) / a.wp;
     a.fd_pw = make_fastdiv((unsigned)a.pw);
     a.fd_tiles_y = make_fastdiv((unsigned)a.tiles_y);
-    a.fd_npt = make_fastdiv((unsigned)a.npt);
     plan.a = a;
     plan.ok = true;
     return plan;

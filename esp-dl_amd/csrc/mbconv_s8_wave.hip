@@ -514,7 +514,6 @@ struct WavePlan {
     bool ok;
     WaveArgs a;
     size_t lds;
-    int nxpt_max, rt_max;
     int cus; // compute units of the device the launch goes to
 };
 
@@ -605,8 +604,6 @@ WavePlan wave_plan(const MbconvParams &p)
     a.fd_tiles_x = make_fastdiv((unsigned)a.tiles_x);
     a.fd_tiles_yx = make_fastdiv((unsigned)(a.tiles_y * a.tiles_x));
     plan.a = a;
-    plan.nxpt_max = a.n_xpt <= 10 ? 10 : 17;
-    plan.rt_max = a.rt <= 2 ? 2 : 4;
     plan.ok = true;
     return plan;
 }
