@@ -269,6 +269,39 @@ __global__ __launch_bounds__(kBlock) void global_avg_pool_s8_kernel(const int8_t
     }
 }
 
+// The same operator for small windows (hw <= 64: a 7 x 7 head): one lane owns FOUR consecutive channels of one
+// image and walks all pixels itself (one 4-byte load per pixel, adjacent lanes adjacent dwords, every load
+// requested before the first is used), so there is no exchange between lanes at all.
+__global__ __launch_bounds__(kBlock) void global_avg_pool_s8_small_kernel(const int8_t *in, int8_t *out, int hw, int c,
+                                                                          float scale)
+{
+    const int ch = (blockIdx.x * kBlock + threadIdx.x) * 4;
+    if (ch >= c)
+        return;
+    const int8_t *img = in + (long long)blockIdx.y * hw * c + ch;
+    int sum[4] = {0, 0, 0, 0};
+    constexpr int kStep = 16; // loads in flight per lane
+    for (int p0 = 0; p0 < hw; p0 += kStep) {
+        int v[kStep];
+#pragma unroll
+        for (int j = 0; j < kStep; j++)
+            v[j] = *reinterpret_cast<const int *>(img + (size_t)(unsigned)(min(p0 + j, hw - 1) * c));
+#pragma unroll
+        for (int j = 0; j < kStep; j++) {
+            if (p0 + j < hw) { // uniform
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+                    sum[k] += (int)(int8_t)(v[j] >> (8 * k));
+            }
+        }
+    }
+    int q[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        q[k] = clamp_s8(round_half_up_f32((float)sum[k] * scale));
+    *reinterpret_cast<int *>(out + (long long)blockIdx.y * c + ch) = pack4_s8(q[0], q[1], q[2], q[3]);
+}
+
 } // namespace
 
 hipError_t launch_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out, hipStream_t stream)
@@ -366,7 +399,10 @@ hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, 
         return hipSuccess;
     const float area_inv = 1.f / (float)(h * w);
     const float scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
-    if ((c & 15) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0)
+    if ((c & 3) == 0 && h * w <= 64 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 3) == 0)
+        hipLaunchKernelGGL(global_avg_pool_s8_small_kernel, dim3((unsigned)((c / 4 + kBlock - 1) / kBlock), (unsigned)batch),
+                           dim3(kBlock), 0, stream, in, out, h * w, c, scale);
+    else if ((c & 15) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0)
         hipLaunchKernelGGL(global_avg_pool_s8_kernel<16>, dim3((unsigned)((c + 1023) / 1024), (unsigned)batch), dim3(kBlock),
                            0, stream, in, out, h * w, c, scale);
     else
