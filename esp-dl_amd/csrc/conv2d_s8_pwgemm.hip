@@ -92,8 +92,12 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
         }
     };
 
-    v4i pb[kPiecesB], pa[kPiecesA];
+    // two register sets: the operands of k step s+2 are requested while step s computes and are stored to LDS
+    // at the end of step s+1, so a load has a whole k step (not just one step's few products) to arrive
+    v4i pb[kPiecesB], pa[kPiecesA], pb2[kPiecesB], pa2[kPiecesA];
     fetch(0, pb, pa);
+    if (a.ksteps > 1)
+        fetch(1, pb2, pa2);
 
     // epilogue constants of the workgroup's filters; the short form needs every shift in 1..31 and no
     // possible overflow of bias + 2^(s-1) + K products
@@ -124,6 +128,8 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
         cst[2][tid] = fast ? max(0, 8 - my_s) : 0;
     }
     stash(0, pb, pa);
+    if (a.ksteps > 2)
+        fetch(2, pb, pa);
     __syncthreads();
 
     // accumulators: 2 pixel tiles x 4*NG filter tiles, started at bias (+ rounding constant)
@@ -141,10 +147,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
 
     // operand A row of this lane in tile t of group g: filter 64*g + 16*(col/4) + 4*t + col%4
     const int a_row0 = 16 * (col >> 2) + (col & 3);
-    for (int ks = 0; ks < a.ksteps; ks++) {
-        const int buf = ks & 1;
-        if (ks + 1 < a.ksteps)
-            fetch(ks + 1, pb, pa); // in flight during this step's MFMAs
+    auto products = [&](int buf) {
         v4i b[PT];
 #pragma unroll
         for (int c = 0; c < PT; c++)
@@ -158,11 +161,25 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
                 for (int c = 0; c < PT; c++)
                     acc[c][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[c], acc[c][4 * g + t], 0, 0, 0);
             }
+    };
+    // Step ks reads LDS buffer ks & 1.  At its end the operands of step ks + 1 (held in registers since step
+    // ks - 1) go to the other buffer, which was last read in step ks - 1 (every wavefront finished that before
+    // the barrier at its end), and the registers they leave take the request for step ks + 3 ... the loop is
+    // unrolled by two so that the two register sets keep their names.
+    for (int ks = 0; ks < a.ksteps; ks += 2) {
+        products(0);
         if (ks + 1 < a.ksteps) {
-            // the other buffer was last read in step ks - 1, which every wavefront finished before
-            // the barrier at the end of that step
-            stash(buf ^ 1, pb, pa);
+            stash(1, pb2, pa2);
+            if (ks + 3 < a.ksteps)
+                fetch(ks + 3, pb2, pa2);
             __syncthreads();
+            products(1);
+            if (ks + 2 < a.ksteps) {
+                stash(0, pb, pa);
+                if (ks + 4 < a.ksteps)
+                    fetch(ks + 4, pb, pa);
+                __syncthreads();
+            }
         }
     }
 
