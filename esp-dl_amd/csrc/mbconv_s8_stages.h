@@ -215,20 +215,20 @@ __device__ __forceinline__ int wave_pack_tab(const v4i &acc, const StageConsts &
 // Expand stage of one chunk of 16 channels: every patch pixel tile through one MFMA and the epilogue, four
 // tiles at a time so that four independent MFMA -> requantize -> store chains are in flight (tiles past
 // n_xpt inside the last group of four have zero operands and a zero mask and land in slack).
-// PACK4 (block inputs of 16 channels): the four 16-lane groups of an operand-B register set hold FOUR pixel
-// tiles (tile 4 g + q in group q), so the patch takes a quarter of the registers and of the loads; operand A
-// comes in four copies, copy q holding the filter in group q and zeros elsewhere, which picks tile q out of the
-// reduction.
-template <int MODE, int NXPT, bool EXACT, int KSE = 1, bool PIPE = false, bool PACK4 = false>
-__device__ __forceinline__ void expand_chunk(const v4i (&xb)[PACK4 ? (NXPT + 3) / 4 : NXPT * KSE], int n_xpt, unsigned xmask,
-                                             const v4i (&aop)[PACK4 ? 4 : KSE], const StageConsts &c, int floor_pk,
-                                             bool relu, bool half_even,
+// PACK = 2 or 4 (block inputs of at most 32 / 16 channels): the four 16-lane groups of an operand-B register set
+// hold PACK pixel tiles (tile PACK g + t in the groups t * 4 / PACK ...), so the patch takes 1 / PACK of the
+// registers and of the loads; operand A comes in PACK copies, copy t holding the filter in the groups of tile t
+// and zeros elsewhere, which picks tile t out of the reduction.
+template <int MODE, int NXPT, bool EXACT, int KSE = 1, bool PIPE = false, int PACK = 1>
+__device__ __forceinline__ void expand_chunk(const v4i (&xb)[PACK > 1 ? (NXPT + PACK - 1) / PACK : NXPT * KSE], int n_xpt,
+                                             unsigned xmask, const v4i (&aop)[PACK > 1 ? PACK : KSE], const StageConsts &c,
+                                             int floor_pk, bool relu, bool half_even,
                                              unsigned char *dst /* exp_l + col * 16 + 4 * quad */)
 {
     auto product = [&](int pt) -> v4i {
         v4i acc = c.init;
-        if constexpr (PACK4) {
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[pt & 3], xb[pt >> 2], acc, 0, 0, 0);
+        if constexpr (PACK > 1) {
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[pt % PACK], xb[pt / PACK], acc, 0, 0, 0);
         } else {
 #pragma unroll
             for (int ks = 0; ks < KSE; ks++)

@@ -97,7 +97,7 @@ __device__ __forceinline__ void byte_masks3(unsigned bm, int (&m)[3])
     }
 }
 
-template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, bool PACK4 = false>
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, int PACK = 1>
 __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_wave_kernel(const WaveArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -137,24 +137,27 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
     const int n_rt = EXACT ? RT : a.rt;
 
     // block-input patch -> operand B registers of the expand stage; xmask: patch pixels inside the image
-    v4i xb[PACK4 ? (NXPT + 3) / 4 : NXPT];
+    v4i xb[(NXPT + PACK - 1) / PACK];
     unsigned xmask = 0;
-    if constexpr (PACK4) {
-        // 16 input channels: lane (col, quad) of register set g loads patch pixel (4 g + quad) * 16 + col, every lane
-        // a whole pixel; the validity bits of all pixel tiles of a column come from the wavefront's votes
+    if constexpr (PACK > 1) {
+        // at most 64 / PACK input channels: the 4 / PACK 16-lane groups `sub` of tile slot `tsel` of register set
+        // g load the 16-byte pieces of patch pixel (PACK g + tsel) * 16 + col; the validity bits of all pixel
+        // tiles of a column come from the wavefront's votes
+        constexpr int kSubs = 4 / PACK;
+        const int tsel = quad / kSubs, sub = quad % kSubs;
         const int8_t *img = p.in + (long long)n * p.in_h * p.in_w * c0;
 #pragma unroll
-        for (int g = 0; g < (NXPT + 3) / 4; g++) {
-            const int pt = 4 * g + quad;
+        for (int g = 0; g < (NXPT + PACK - 1) / PACK; g++) {
+            const int pt = PACK * g + tsel;
             const unsigned pp = (unsigned)(pt * 16 + col);
             const unsigned prow = fastdiv(pp, a.fd_pw);
             const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
             const bool valid = pt < NXPT && (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
-            xb[g] = load16_partial<true>(img, (unsigned)((iy * p.in_w + ix) * 16), valid ? 16 : 0);
-            const unsigned long long votes = __ballot(valid); // bit 16 q + col: tile 4 g + q, column col
+            xb[g] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * sub), valid ? c0 - 16 * sub : 0);
+            const unsigned long long votes = __ballot(valid); // bit 16 quad + col
 #pragma unroll
-            for (int q = 0; q < 4; q++)
-                xmask |= (unsigned)((votes >> (16 * q + col)) & 1ull) << (4 * g + q);
+            for (int t = 0; t < PACK; t++)
+                xmask |= (unsigned)((votes >> (16 * kSubs * t + col)) & 1ull) << (PACK * g + t);
         }
     } else if constexpr (!ROWCONV) {
         const int8_t *img = p.in + (long long)n * p.in_h * p.in_w * c0;
@@ -319,18 +322,20 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
     // Filters of a chunk are requested one chunk ahead (ChunkW), the project filters of a group of four
     // chunks at the start of the group: their latency hides behind the chunk in between.
     struct ChunkW {
-        v4i aop[PACK4 ? 4 : 1];
+        v4i aop[PACK];
         int wd0[3], wd1[3];
     };
     auto load_chunk = [&](int sub) {
         ChunkW w;
         const int ch0 = 16 * sub;
-        if constexpr (PACK4) {
-            // the filter's 16 bytes in every 16-lane group; copy q keeps them in group q only
-            const v4i wq = *reinterpret_cast<const v4i *>(p.w_expand + (size_t)(unsigned)((ch0 + col) * 16));
+        if constexpr (PACK > 1) {
+            // the filter's bytes in every tile slot; copy t keeps them in the groups of slot t only
+            constexpr int kSubs = 4 / PACK;
+            const v4i wq = load16_partial<VEC16>(p.w_expand, (unsigned)((ch0 + col) * c0 + 16 * (quad % kSubs)),
+                                                 c0 - 16 * (quad % kSubs));
 #pragma unroll
-            for (int q = 0; q < 4; q++)
-                w.aop[q] = quad == q ? wq : v4i{0, 0, 0, 0};
+            for (int t = 0; t < PACK; t++)
+                w.aop[t] = quad / kSubs == t ? wq : v4i{0, 0, 0, 0};
         } else if constexpr (ROWCONV) {
             w.aop[0] = *reinterpret_cast<const v4i *>(smem + a.off_aop + ((ch0 + col) * 4 + quad) * 16);
         } else {
@@ -431,13 +436,13 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_
         {
             const StageConsts ce = read_stage_table(tab_e, p.exp_c, 16 * sub + 4 * quad, mode_e);
             if (ce.mode == 0)
-                expand_chunk<0, NXPT, EXACT, 1, true, PACK4>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<0, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else if (ce.mode == 1)
-                expand_chunk<1, NXPT, EXACT, 1, true, PACK4>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<1, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else if (ce.mode == 2)
-                expand_chunk<2, NXPT, EXACT, 1, true, PACK4>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<2, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else
-                expand_chunk<-1, NXPT, EXACT, 1, true, PACK4>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<-1, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
         }
         wave_lds_sync();
 
@@ -632,11 +637,11 @@ WavePlan wave_plan(const MbconvParams &p)
     return plan;
 }
 
-template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, bool PACK4 = false>
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, int PACK = 1>
 hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
 {
     WaveArgs a = plan.a;
-    auto kernel = mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV, PACK4>;
+    auto kernel = mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV, PACK>;
     a.tpw = 1;
     if (ROWCONV) {
         // Tiles per wavefront: these tiles are short (two chunks of expanded channels for a 32-filter stem), so
@@ -686,11 +691,25 @@ bool launch_exact(const WavePlan &plan, hipStream_t stream, bool dry, hipError_t
     const auto is = [&](int nxpt, int rt, int th, int stride, bool v) {
         return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v && (stride != 1 || a.pw == 16);
     };
-    if (is(17, 2, 4, 2, true) && a.p.in_c == 16) { // four pixel tiles per operand-B register set
-        if (!dry)
-            *err = launch_one<17, 2, 4, 2, HE, true, true, false, true>(plan, stream);
-        return true;
-    }
+    // block inputs of at most 16 / 32 channels: four / two pixel tiles per operand-B register set
+#define ESPDL_WAVE_PACKED(NXPT, RT, PT, S, V, PACK)                                           \
+    do {                                                                                       \
+        if (!dry)                                                                              \
+            *err = launch_one<NXPT, RT, PT, S, HE, V, true, false, PACK>(plan, stream);        \
+        return true;                                                                           \
+    } while (0)
+    const int c0 = a.p.in_c;
+    if (is(17, 2, 4, 2, true) && c0 == 16)
+        ESPDL_WAVE_PACKED(17, 2, 4, 2, true, 4);
+    if (is(17, 2, 4, 2, false) && c0 <= 32)
+        ESPDL_WAVE_PACKED(17, 2, 4, 2, false, 2);
+    if (is(10, 2, 8, 1, false) && c0 <= 32)
+        ESPDL_WAVE_PACKED(10, 2, 8, 1, false, 2);
+    if (is(9, 2, 7, 1, true) && c0 == 32)
+        ESPDL_WAVE_PACKED(9, 2, 7, 1, true, 2);
+    if (is(10, 4, 2, 2, true) && c0 == 32)
+        ESPDL_WAVE_PACKED(10, 4, 2, 2, true, 2);
+#undef ESPDL_WAVE_PACKED
     if (is(17, 2, 4, 2, true))
         ESPDL_WAVE_EXACT(17, 2, 4, 2, true, false);
     if (is(17, 2, 4, 2, false))
