@@ -98,7 +98,7 @@ __device__ __forceinline__ void byte_masks3(unsigned bm, int (&m)[3])
 }
 
 template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, int PACK = 1>
-__global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? 2 : 1) void mbconv_s8_wave_kernel(const WaveArgs a)
+__global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) ? 3 : 2) : 1) void mbconv_s8_wave_kernel(const WaveArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const MbconvParams &p = a.p;
