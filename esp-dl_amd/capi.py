@@ -45,6 +45,18 @@ class MbconvWeights(ctypes.Structure):
 _lib = None
 
 
+def torch_device_first():
+    """PyTorch wheels carry their own copy of the HIP runtime.  The copy that initializes first owns the device for
+    the process, and the buffers handed to this library come from torch: so before the library makes its first
+    HIP call, torch's runtime is brought up (nothing happens without torch or without a GPU)."""
+    try:
+        import torch
+    except ImportError:
+        return
+    if torch.cuda.is_available():
+        torch.cuda.init()
+
+
 def lib():
     """Load libespdl_hip.so; fails loudly when it has not been built."""
     global _lib
@@ -52,6 +64,7 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise EspdlHipError(
                 f"{LIB_PATH} is missing: build it with `python esp-dl_amd/build.py` (no CPU fallback exists)")
+        torch_device_first()
         L = ctypes.CDLL(LIB_PATH)
         vp, i32, i64 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64
         dp = ctypes.POINTER(ConvDesc)

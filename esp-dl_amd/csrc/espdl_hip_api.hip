@@ -39,12 +39,16 @@ int cu_count_cached()
     static thread_local int cached_dev = -1;
     static thread_local int cached_cus = 0;
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess)
+    if (hipGetDevice(&dev) != hipSuccess) {
+        (void)hipGetLastError(); // a failed query must not surface as the error of a later launch
         return 0;
+    }
     if (dev != cached_dev) {
         int cus = 0;
-        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
-            cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+            (void)hipGetLastError();
+            return 0; // not remembered: the next call asks again
+        }
         cached_dev = dev;
         cached_cus = cus;
     }

@@ -20,6 +20,8 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise EspdlModelError(f"{LIB_PATH} is missing: build it with `python esp-dl_amd/build.py`")
         # libespdl_dl.so links libespdl_hip.so through $ORIGIN
+        from . import capi
+        capi.torch_device_first()
         L = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
         vp, cp, i32, i64 = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int32, ctypes.c_int64
         pi32 = ctypes.POINTER(i32)

@@ -663,6 +663,49 @@ def test_mbconv_s8_expand_with_window_is_refused_where_not_covered():
     assert m.capi.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == 0  # a window without an expand stage
 
 
+# The guard-free builds are picked at batches that fill the device; here with image sizes that leave ragged
+# last tiles in both directions (rows computed and not stored, columns masked).
+# (name, (N, H, W, Cin), Ce, Cout, stride, residual, half_even)
+GUARD_FREE_RAGGED = [
+    ("pack4_110x110_16_96_24_s2", (80, 110, 110, 16), 96, 24, 2, False, False),
+    ("pack2_54x54_24_144_24_s1_res", (80, 54, 54, 24), 144, 24, 1, True, False),
+    ("pack2_54x54_24_144_32_s2_halfeven", (96, 54, 54, 24), 144, 32, 2, False, True),
+    ("pack2_27x27_32_192_32_s1_res", (300, 27, 27, 32), 192, 32, 1, True, False),
+]
+
+
+@pytest.mark.parametrize("case", GUARD_FREE_RAGGED, ids=lambda c: c[0])
+def test_mbconv_s8_guard_free_builds_ragged_tiles(oracle, case):
+    announce(f"mbconv_s8 guard-free build, ragged tiles: {case[0]}")
+    name, (n, h, w, cin), ce, cout, stride, with_res, half_even = case
+    m = espdl()
+    d = _block_desc(m, n, h, cin, ce, cout, stride, half_even)
+    assert m.capi.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == 4
+    rng = np.random.default_rng(0x9A6 + len(name))
+    rm_o = oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP
+    rm_g = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
+    oracle.set_threads(16)
+
+    def stage(oc, kk, fshape):
+        return (rng_int8(rng, fshape), rng.integers(-4096, 4097, size=oc).astype(np.int32),
+                (typical_shift(kk) + rng.integers(-2, 3, size=oc)).astype(np.int32))
+
+    x = rng_int8(rng, (n, h, w, cin))
+    ex, dw, pj = stage(ce, cin, (ce, 1, 1, cin)), stage(ce, 9, (3, 3, ce)), stage(cout, ce, (cout, 1, 1, ce))
+    pads = (1, 1, 1, 1)
+    cur = oracle.conv2d_s8(x, ex[0], ex[1], ex[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.RELU, rm_o)
+    cur = oracle.depthwise_s8(cur, dw[0], dw[1], dw[2], (3, 3), (stride, stride), (1, 1), pads, oracle.RELU, rm_o)
+    cur = oracle.conv2d_s8(cur, pj[0], pj[1], pj[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.LINEAR, rm_o)
+    res = None
+    if with_res:
+        res = rng_int8(rng, cur.shape)
+        cur = oracle.add_s8(cur, res)
+    dev = lambda t: tuple(to_dev(a) for a in t)  # noqa: E731
+    got = m.mbconv_s8(to_dev(x), dev(ex), dev(dw), dev(pj), (3, 3), (stride, stride), (1, 1), pads, (True, True, False),
+                      residual=to_dev(res), round_mode=rm_g)
+    np.testing.assert_array_equal(to_host(got), cur)
+
+
 def _block_desc(m, batch, hw, cin, ce, cout, stride, half_even=False):
     d = m.capi.MbconvDesc()
     d.batch, d.in_h, d.in_w, d.in_c, d.exp_c, d.out_c, d.has_expand = batch, hw, hw, cin, ce, cout, 1
