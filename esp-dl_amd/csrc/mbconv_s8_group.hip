@@ -55,7 +55,10 @@ struct GroupArgs {
 };
 
 // EXACT: the plan is exactly (NXPT patch pixel tiles, KSE k steps, PT rows): no guards in the stage loops.
-template <int NXPT, int KSE, int PT, int S, bool HE, bool EXACT>
+// KSP > 0: the project stage has exactly KSP k steps of 64 expanded channels and a wavefront holds operand A of
+// a whole row tile of filters in registers (KSP = 0: any count, operand A in blocks of eight k steps).
+// NTX > 0: a wavefront holds exactly NTX project pixel tiles at a time (no code for other counts: fewer registers).
+template <int NXPT, int KSE, int PT, int S, bool HE, bool EXACT, int KSP = 0, int NTX = 0>
 __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mbconv_s8_group_kernel(const GroupArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -105,6 +108,35 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
             }
         }
     }
+    // filters of a chunk of 16 expanded channels, requested one chunk ahead
+    struct ChunkW {
+        v4i aop[KSE];
+        int wd0[3], wd1[3];
+    };
+    auto load_chunk = [&](int sub) {
+        ChunkW w;
+        const int ch0 = 16 * sub;
+#pragma unroll
+        for (int ks = 0; ks < KSE; ks++) {
+            w.aop[ks] = v4i{0, 0, 0, 0};
+            if (EXACT || ks < kse) // uniform
+                w.aop[ks] = load16_partial<true>(p.w_expand, (unsigned)((ch0 + col) * c0 + 64 * ks + 16 * quad),
+                                                 c0 - 64 * ks - 16 * quad);
+        }
+        const unsigned wd = (unsigned)(ch0 + col);
+#pragma unroll
+        for (int kx = 0; kx < 3; kx++) {
+            const int v0 = (int)p.w_dw[(size_t)(wd + (unsigned)((min(quad, 2) * 3 + kx) * p.exp_c))];
+            w.wd0[kx] = quad < 3 ? v0 : 0;
+            w.wd1[kx] = 0;
+            if constexpr (S == 1) {
+                const int v1 = (int)p.w_dw[(size_t)(wd + (unsigned)((max(quad - 1, 0) * 3 + kx) * p.exp_c))];
+                w.wd1[kx] = quad >= 1 ? v1 : 0;
+            }
+        }
+        return w;
+    };
+
     int mode_e, mode_d, mode_p;
     int *tab_p = tab_d + 3 * p.exp_c; // 3 x 16 rt entries
     {
@@ -138,34 +170,6 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
     const unsigned char *exp_src = exp_l + (quad * a.pw + S * col) * 16;
     const int row_bytes = a.twp * a.ds;
     const bool write_ok = col < a.twp;
-
-    struct ChunkW {
-        v4i aop[KSE];
-        int wd0[3], wd1[3];
-    };
-    auto load_chunk = [&](int sub) {
-        ChunkW w;
-        const int ch0 = 16 * sub;
-#pragma unroll
-        for (int ks = 0; ks < KSE; ks++) {
-            w.aop[ks] = v4i{0, 0, 0, 0};
-            if (EXACT || ks < kse) // uniform
-                w.aop[ks] = load16_partial<true>(p.w_expand, (unsigned)((ch0 + col) * c0 + 64 * ks + 16 * quad),
-                                                 c0 - 64 * ks - 16 * quad);
-        }
-        const unsigned wd = (unsigned)(ch0 + col);
-#pragma unroll
-        for (int kx = 0; kx < 3; kx++) {
-            const int v0 = (int)p.w_dw[(size_t)(wd + (unsigned)((min(quad, 2) * 3 + kx) * p.exp_c))];
-            w.wd0[kx] = quad < 3 ? v0 : 0;
-            w.wd1[kx] = 0;
-            if constexpr (S == 1) {
-                const int v1 = (int)p.w_dw[(size_t)(wd + (unsigned)((max(quad - 1, 0) * 3 + kx) * p.exp_c))];
-                w.wd1[kx] = quad >= 1 ? v1 : 0;
-            }
-        }
-        return w;
-    };
 
     if (wave < a.n_sub) {
         ChunkW cur = load_chunk(wave);
@@ -216,11 +220,24 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
             ap[kk] = load16_partial<true>(p.w_project, a_off + 64u * (unsigned)(k0 + kk),
                                           row_ok ? p.exp_c - 64 * (k0 + kk) - 16 * quad : 0);
     };
-    // (not in the build that is held to 128 registers so that two workgroups share a compute unit)
+    auto load_a_step = [&](int rt, int k) {
+        const bool row_ok = rt < a.rt && 16 * rt + col < p.out_c;
+        return load16_partial<true>(p.w_project, (unsigned)((16 * rt + col) * p.exp_c + 16 * quad) + 64u * (unsigned)k,
+                                    row_ok ? p.exp_c - 64 * k - 16 * quad : 0);
+    };
+    // (the blocked form does not prefetch in the build that is held to 128 registers so that two workgroups
+    // share a compute unit)
     constexpr bool kPrefetchA = !(KSE == 1 && EXACT);
-    v4i ap_first[8];
-    if constexpr (kPrefetchA)
+    v4i ap_first[KSP > 0 ? KSP : 8];
+    if constexpr (KSP > 0) {
+        if (wrow < a.wr) { // uniform
+#pragma unroll
+            for (int kk = 0; kk < KSP; kk++)
+                ap_first[kk] = load_a_step(wrow, kk);
+        }
+    } else if constexpr (kPrefetchA) {
         load_a(wrow, 0, ap_first);
+    }
     __syncthreads(); // the shared depthwise tile is complete
 
     // ---- phase 2: project.  The (row tile of 16 filters) x (pixel tile of 16 slots) accumulator tiles are dealt
@@ -240,10 +257,10 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
 #pragma unroll
         for (int i = 0; i < NT; i++)
             bsrc[i] = dw_l + (min(t0 + i, a.npt - 1) * 16 + col) * a.ds + 16 * quad;
-        v4i ap[8];
-        if constexpr (kPrefetchA) {
+        v4i ap[KSP > 0 ? KSP : 8];
+        if constexpr (KSP > 0 || kPrefetchA) {
 #pragma unroll
-            for (int kk = 0; kk < 8; kk++)
+            for (int kk = 0; kk < (KSP > 0 ? KSP : 8); kk++)
                 ap[kk] = ap_first[kk];
         }
         for (int rt = wrow; rt < a.rt; rt += a.wr) {
@@ -265,31 +282,55 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
                 off[i] = (unsigned)(((oy0 + oy) * p.out_w + ox) * p.out_c + c);
                 rv[i] = res_img != nullptr ? *reinterpret_cast<const int *>(res_img + (size_t)(live[i] ? off[i] : 0u)) : 0;
             }
-            for (int k0 = 0; k0 < ksp; k0 += 8) {
-                // the next block of operand A (the next k steps, or the first ones of the next row tile) is
-                // requested before this block's products
-                v4i an[8];
-                const bool more_k = k0 + 8 < ksp;
-                if constexpr (kPrefetchA)
-                    load_a(more_k ? rt : rt + a.wr, more_k ? k0 + 8 : 0, an);
-                else
-                    load_a(rt, k0, ap);
+            if constexpr (KSP > 0) {
+                // operand A of the whole row tile is in registers; each register is requested again, for the
+                // wavefront's next row tile, as soon as its products are issued (the compiler gives the new
+                // values registers of their own, so this form is for short reductions)
+                auto steps = [&](auto more_tag) {
 #pragma unroll
-                for (int kk = 0; kk < 8; kk++) {
-                    if (k0 + kk < ksp) { // uniform
+                    for (int kk = 0; kk < KSP; kk++) {
                         v4i bv[NT];
 #pragma unroll
                         for (int i = 0; i < NT; i++)
-                            bv[i] = *reinterpret_cast<const v4i *>(bsrc[i] + 64 * (k0 + kk));
+                            bv[i] = *reinterpret_cast<const v4i *>(bsrc[i] + 64 * kk);
 #pragma unroll
                         for (int i = 0; i < NT; i++)
                             accp[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ap[kk], bv[i], accp[i], 0, 0, 0);
+                        if constexpr (decltype(more_tag)::value)
+                            ap[kk] = load_a_step(rt + a.wr, kk);
                     }
-                }
-                if constexpr (kPrefetchA) {
+                };
+                if (rt + a.wr < a.rt) // uniform
+                    steps(std::true_type{});
+                else
+                    steps(std::false_type{});
+            } else {
+                for (int k0 = 0; k0 < ksp; k0 += 8) {
+                    // the next block of operand A (the next k steps, or the first ones of the next row tile) is
+                    // requested before this block's products
+                    v4i an[8];
+                    const bool more_k = k0 + 8 < ksp;
+                    if constexpr (kPrefetchA)
+                        load_a(more_k ? rt : rt + a.wr, more_k ? k0 + 8 : 0, an);
+                    else
+                        load_a(rt, k0, ap);
 #pragma unroll
-                    for (int kk = 0; kk < 8; kk++)
-                        ap[kk] = an[kk];
+                    for (int kk = 0; kk < 8; kk++) {
+                        if (k0 + kk < ksp) { // uniform
+                            v4i bv[NT];
+#pragma unroll
+                            for (int i = 0; i < NT; i++)
+                                bv[i] = *reinterpret_cast<const v4i *>(bsrc[i] + 64 * (k0 + kk));
+#pragma unroll
+                            for (int i = 0; i < NT; i++)
+                                accp[i] = __builtin_amdgcn_mfma_i32_16x16x64_i8(ap[kk], bv[i], accp[i], 0, 0, 0);
+                        }
+                    }
+                    if constexpr (kPrefetchA) {
+#pragma unroll
+                        for (int kk = 0; kk < 8; kk++)
+                            ap[kk] = an[kk];
+                    }
                 }
             }
             const StageConsts cp = read_stage_table<false>(tab_p, 16 * a.rt, c, mode_p);
@@ -320,14 +361,18 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
         }
     };
     if (wrow < a.wr) { // uniform: wavefronts beyond the grid have no share
+        const auto run = [&](auto nt_tag) {
+            if constexpr (NTX == 0 || decltype(nt_tag)::value == NTX)
+                project(nt_tag);
+        };
         switch (a.nt) {
-        case 1: project(std::integral_constant<int, 1>{}); break;
-        case 2: project(std::integral_constant<int, 2>{}); break;
-        case 3: project(std::integral_constant<int, 3>{}); break;
-        case 4: project(std::integral_constant<int, 4>{}); break;
-        case 5: project(std::integral_constant<int, 5>{}); break;
-        case 6: project(std::integral_constant<int, 6>{}); break;
-        default: project(std::integral_constant<int, kMaxT>{}); break;
+        case 1: run(std::integral_constant<int, 1>{}); break;
+        case 2: run(std::integral_constant<int, 2>{}); break;
+        case 3: run(std::integral_constant<int, 3>{}); break;
+        case 4: run(std::integral_constant<int, 4>{}); break;
+        case 5: run(std::integral_constant<int, 5>{}); break;
+        case 6: run(std::integral_constant<int, 6>{}); break;
+        default: run(std::integral_constant<int, kMaxT>{}); break;
         }
     }
 }
@@ -412,10 +457,10 @@ GroupPlan group_plan(const MbconvParams &p)
     return plan;
 }
 
-template <int NXPT, int KSE, int PT, int S, bool HE, bool EXACT>
+template <int NXPT, int KSE, int PT, int S, bool HE, bool EXACT, int KSP = 0, int NTX = 0>
 hipError_t launch_group_one(const GroupPlan &plan, hipStream_t stream)
 {
-    auto kernel = mbconv_s8_group_kernel<NXPT, KSE, PT, S, HE, EXACT>;
+    auto kernel = mbconv_s8_group_kernel<NXPT, KSE, PT, S, HE, EXACT, KSP, NTX>;
     static bool raised = false; // the dynamic LDS limit of a kernel is raised once per process
     if (!raised) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
@@ -435,23 +480,32 @@ bool launch_group_exact(const GroupPlan &plan, hipStream_t stream, bool dry, hip
 {
     const GroupArgs &a = plan.a;
     const int s = a.p.stride_h;
-    const auto is = [&](int nxpt, int kse, int th, int stride) {
-        return a.n_xpt == nxpt && a.kse == kse && a.th == th && s == stride;
+    const int ksp = (a.p.exp_c + 63) / 64;
+    // k_project / nt: the project stage's k steps and pixel tiles per wavefront the build is made for (0: any)
+    const auto is = [&](int nxpt, int kse, int th, int stride, int k_project, int nt) {
+        return a.n_xpt == nxpt && a.kse == kse && a.th == th && s == stride && (k_project == 0 || ksp == k_project) &&
+            (nt == 0 || a.nt == nt);
     };
-#define ESPDL_GROUP_EXACT(NXPT, KSE, PT, S)                                        \
-    do {                                                                            \
-        if (!dry)                                                                   \
-            *err = launch_group_one<NXPT, KSE, PT, S, HE, true>(plan, stream);      \
-        return true;                                                                \
+#define ESPDL_GROUP_EXACT(NXPT, KSE, PT, S, KSP, NTX)                                    \
+    do {                                                                                 \
+        if (is(NXPT, KSE, PT, S, KSP, NTX)) {                                            \
+            if (!dry)                                                                    \
+                *err = launch_group_one<NXPT, KSE, PT, S, HE, true, KSP, NTX>(plan, stream); \
+            return true;                                                                 \
+        }                                                                                \
     } while (0)
-    if (is(9, 1, 7, 1))
-        ESPDL_GROUP_EXACT(9, 1, 7, 1);
-    if (is(9, 2, 7, 1))
-        ESPDL_GROUP_EXACT(9, 2, 7, 1);
-    if (is(6, 3, 7, 1))
-        ESPDL_GROUP_EXACT(6, 3, 7, 1);
-    if (is(9, 2, 4, 2))
-        ESPDL_GROUP_EXACT(9, 2, 4, 2);
+    // MobileNetV2-1.0's blocks, each with the one pixel-tile count and reduction length it has there ...
+    ESPDL_GROUP_EXACT(9, 1, 7, 1, 0, 4); // 14 x 14, 64 -> 384 -> 64 (held to 128 registers: operand A in blocks)
+    ESPDL_GROUP_EXACT(9, 1, 7, 1, 0, 7); // 14 x 14, 64 -> 384 -> 96
+    ESPDL_GROUP_EXACT(9, 2, 7, 1, 9, 7); // 14 x 14, 96 -> 576 -> 96
+    ESPDL_GROUP_EXACT(9, 2, 4, 2, 9, 2); // 14 x 14, 96 -> 576 -> 160, stride 2
+    ESPDL_GROUP_EXACT(6, 3, 7, 1, 0, 4); // 7 x 7, 160 -> 960 -> 160 / 320 (several row tiles per wavefront:
+                                         // operand A in blocks hides their loads better)
+    // ... and the same tile plans with any output channel count
+    ESPDL_GROUP_EXACT(9, 1, 7, 1, 0, 0);
+    ESPDL_GROUP_EXACT(9, 2, 7, 1, 0, 0);
+    ESPDL_GROUP_EXACT(6, 3, 7, 1, 0, 0);
+    ESPDL_GROUP_EXACT(9, 2, 4, 2, 0, 0);
 #undef ESPDL_GROUP_EXACT
     return false;
 }

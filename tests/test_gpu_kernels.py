@@ -665,22 +665,32 @@ def test_mbconv_s8_expand_with_window_is_refused_where_not_covered():
 
 # The guard-free builds are picked at batches that fill the device; here with image sizes that leave ragged
 # last tiles in both directions (rows computed and not stored, columns masked).
-# (name, (N, H, W, Cin), Ce, Cout, stride, residual, half_even)
+# The eight-wavefront kernel (answer 5 of espdl_hip_mbconv_s8_supported) has builds for one count of project pixel
+# tiles per wavefront (MobileNetV2's output channel counts) and builds for any count: other output channel
+# counts below, and a 13 x 13 image whose second tile has six rows.
+# (name, (N, H, W, Cin), Ce, Cout, stride, residual, half_even, answer of espdl_hip_mbconv_s8_supported)
 GUARD_FREE_RAGGED = [
-    ("pack4_110x110_16_96_24_s2", (80, 110, 110, 16), 96, 24, 2, False, False),
-    ("pack2_54x54_24_144_24_s1_res", (80, 54, 54, 24), 144, 24, 1, True, False),
-    ("pack2_54x54_24_144_32_s2_halfeven", (96, 54, 54, 24), 144, 32, 2, False, True),
-    ("pack2_27x27_32_192_32_s1_res", (300, 27, 27, 32), 192, 32, 1, True, False),
+    ("pack4_110x110_16_96_24_s2", (80, 110, 110, 16), 96, 24, 2, False, False, 4),
+    ("pack2_54x54_24_144_24_s1_res", (80, 54, 54, 24), 144, 24, 1, True, False, 4),
+    ("pack2_54x54_24_144_32_s2_halfeven", (96, 54, 54, 24), 144, 32, 2, False, True, 4),
+    ("pack2_27x27_32_192_32_s1_res", (300, 27, 27, 32), 192, 32, 1, True, False, 4),
+    ("group_13x13_64_384_64_s1_res", (70, 13, 13, 64), 384, 64, 1, True, False, 5),
+    ("group_14x14_64_384_32_s1", (66, 14, 14, 64), 384, 32, 1, False, False, 5),
+    ("group_14x14_96_576_64_s1_halfeven", (66, 14, 14, 96), 576, 64, 1, False, True, 5),
+    ("group_13x13_96_576_96_s1_res", (40, 13, 13, 96), 576, 96, 1, True, False, 5),
+    ("group_14x14_96_576_48_s2", (70, 14, 14, 96), 576, 48, 2, False, False, 5),
+    ("group_7x7_160_960_64_s1", (130, 7, 7, 160), 960, 64, 1, False, False, 5),
+    ("group_7x7_160_960_96_s1_halfeven", (130, 7, 7, 160), 960, 96, 1, False, True, 5),
 ]
 
 
 @pytest.mark.parametrize("case", GUARD_FREE_RAGGED, ids=lambda c: c[0])
 def test_mbconv_s8_guard_free_builds_ragged_tiles(oracle, case):
     announce(f"mbconv_s8 guard-free build, ragged tiles: {case[0]}")
-    name, (n, h, w, cin), ce, cout, stride, with_res, half_even = case
+    name, (n, h, w, cin), ce, cout, stride, with_res, half_even, answer = case
     m = espdl()
     d = _block_desc(m, n, h, cin, ce, cout, stride, half_even)
-    assert m.capi.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == 4
+    assert m.capi.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == answer
     rng = np.random.default_rng(0x9A6 + len(name))
     rm_o = oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP
     rm_g = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
