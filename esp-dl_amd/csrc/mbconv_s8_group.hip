@@ -177,11 +177,11 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
             const ChunkW nxt = load_chunk(min(sub + kGroupWaves, a.n_sub - 1));
             {
                 const StageConsts ce = read_stage_table(tab_e, p.exp_c, 16 * sub + 4 * quad, mode_e);
-                if (ce.mode == 0)
+                if (!HE && ce.mode == 0) // a build meets the forms of its rounding mode only
                     expand_chunk<0, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
-                else if (ce.mode == 1)
+                else if (!HE && ce.mode == 1)
                     expand_chunk<1, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
-                else if (ce.mode == 2)
+                else if (HE && ce.mode == 2)
                     expand_chunk<2, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
                 else
                     expand_chunk<-1, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
@@ -196,11 +196,11 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
                 }
                 const StageConsts cd = read_stage_table(tab_d, p.exp_c, 16 * sub + 4 * quad, mode_d);
                 unsigned char *dst = dw_l + col * a.ds + 16 * sub + 4 * quad;
-                if (cd.mode == 0)
+                if (!HE && cd.mode == 0) // a build meets the forms of its rounding mode only
                     depthwise_chunk<0, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
-                else if (cd.mode == 1)
+                else if (!HE && cd.mode == 1)
                     depthwise_chunk<1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
-                else if (cd.mode == 2)
+                else if (HE && cd.mode == 2)
                     depthwise_chunk<2, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
                 else
                     depthwise_chunk<-1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
@@ -334,30 +334,44 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
                 }
             }
             const StageConsts cp = read_stage_table<false>(tab_p, 16 * a.rt, c, mode_p);
+            // the uniform choices (epilogue form, residual or not) are made once per row tile, outside the loop
+            // over the words
+            auto words = [&](auto mode_tag, auto res_tag) {
+                constexpr int MODE = decltype(mode_tag)::value;
+                constexpr bool RES = decltype(res_tag)::value;
 #pragma unroll
-            for (int i = 0; i < NT; i++) {
-                v4i acc = accp[i];
+                for (int i = 0; i < NT; i++) {
+                    v4i acc = accp[i];
 #pragma unroll
-                for (int k = 0; k < 4; k++)
-                    acc[k] += cp.init[k];
-                int word;
-                if (cp.mode == 0)
-                    word = res_img != nullptr ? pack_fast4_add<0>(acc, cp.lsh, cp.rsh, floor_p, rv[i])
-                                              : wave_pack<0>(acc, cp, floor_p, false, HE);
-                else if (cp.mode == 1)
-                    word = res_img != nullptr ? pack_fast4_add<1>(acc, cp.lsh, cp.rsh, floor_p, rv[i])
-                                              : wave_pack<1>(acc, cp, floor_p, false, HE);
-                else if (cp.mode == 2)
-                    word = res_img != nullptr ? pack_fast4_add<2>(acc, cp.lsh, cp.rsh, floor_p, rv[i])
-                                              : wave_pack<2>(acc, cp, floor_p, false, HE);
-                else {
-                    word = wave_pack<-1>(acc, cp, floor_p, p.relu_project != 0, HE);
-                    if (res_img != nullptr)
-                        word = sat_add4_s8(word, rv[i]);
+                    for (int k = 0; k < 4; k++)
+                        acc[k] += cp.init[k];
+                    int word;
+                    if constexpr (RES) {
+                        if constexpr (MODE >= 0)
+                            word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, rv[i]);
+                        else
+                            word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), rv[i]);
+                    } else {
+                        word = wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE);
+                    }
+                    if (live[i])
+                        *reinterpret_cast<int *>(out_img + (size_t)off[i]) = word;
                 }
-                if (live[i])
-                    *reinterpret_cast<int *>(out_img + (size_t)off[i]) = word;
-            }
+            };
+            auto with_mode = [&](auto mode_tag) {
+                if (res_img != nullptr)
+                    words(mode_tag, std::true_type{});
+                else
+                    words(mode_tag, std::false_type{});
+            };
+            if (cp.mode == -1)
+                with_mode(std::integral_constant<int, -1>{});
+            else if constexpr (HE)
+                with_mode(std::integral_constant<int, 2>{});
+            else if (cp.mode == 0)
+                with_mode(std::integral_constant<int, 0>{});
+            else
+                with_mode(std::integral_constant<int, 1>{});
         }
     };
     if (wrow < a.wr) { // uniform: wavefronts beyond the grid have no share

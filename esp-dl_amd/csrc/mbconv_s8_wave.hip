@@ -435,11 +435,11 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
         // ---- expand: 16 channels x every patch pixel
         {
             const StageConsts ce = read_stage_table(tab_e, p.exp_c, 16 * sub + 4 * quad, mode_e);
-            if (ce.mode == 0)
+            if (!HE && ce.mode == 0) // a build meets the forms of its rounding mode only
                 expand_chunk<0, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
-            else if (ce.mode == 1)
+            else if (!HE && ce.mode == 1)
                 expand_chunk<1, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
-            else if (ce.mode == 2)
+            else if (HE && ce.mode == 2)
                 expand_chunk<2, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else
                 expand_chunk<-1, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
@@ -456,11 +456,11 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
             }
             const StageConsts cd = read_stage_table(tab_d, p.exp_c, 16 * sub + 4 * quad, mode_d);
             unsigned char *dst = dw_l + col * kDws + 16 * (sub & 3) + 4 * quad;
-            if (cd.mode == 0)
+            if (!HE && cd.mode == 0) // a build meets the forms of its rounding mode only
                 depthwise_chunk<0, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
-            else if (cd.mode == 1)
+            else if (!HE && cd.mode == 1)
                 depthwise_chunk<1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
-            else if (cd.mode == 2)
+            else if (HE && cd.mode == 2)
                 depthwise_chunk<2, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
             else
                 depthwise_chunk<-1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
