@@ -858,15 +858,11 @@ int espdl_hip_mbconv_s8_preferred(const espdl_hip_mbconv_desc *desc)
     static const int8_t *const aligned = reinterpret_cast<const int8_t *>(uintptr_t(256));
     p.in = aligned;
     p.w_expand = aligned;
-    const int cus = cu_count_cached() > 0 ? cu_count_cached() : 256;
-    // Both single-launch kernels win with their guard-free builds only (one per tile plan of MobileNetV2-style
-    // blocks); the guarded builds cover every shape but are no faster than the separate launches.
-    if (kind == 5) // a workgroup per tile of a small image: at least one workgroup per compute unit
-        return (espdl::mbconv_s8_group_has_fast_build(p) && (long long)desc->batch >= cus) ? 1 : 0;
-    // one wavefront per tile: it needs several tiles per SIMD to keep the pipes busy, and at small images
-    // the separate kernels (which also split the channels) are as fast
-    const long long tiles = espdl::mbconv_s8_wave_tiles(p);
-    return (espdl::mbconv_s8_wave_has_fast_build(p) && p.in_h >= 28 && p.in_w >= 28 && tiles >= 4ll * cus) ? 1 : 0;
+    // Both single-launch kernels win with their guard-free builds (one per tile plan of MobileNetV2-style blocks)
+    // and then at every batch size, from one image (fewer launches, no round trip of the expanded tensor) to
+    // several rounds over the device; the guarded builds cover every shape but are no faster than the separate
+    // launches.
+    return (kind == 5 ? espdl::mbconv_s8_group_has_fast_build(p) : espdl::mbconv_s8_wave_has_fast_build(p)) ? 1 : 0;
 }
 
 int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *w,

@@ -97,7 +97,6 @@ hipError_t launch_mbconv_s8_fused(const MbconvParams &p, int cu_count, hipStream
 // The same block with one wavefront per output tile and no workgroup barriers (mbconv_s8_wave.hip): 3x3
 // depthwise stage with stride 1 or 2, at most 64 block-input channels and 64 project filters.
 bool mbconv_s8_wave_supports(const MbconvParams &p);
-long long mbconv_s8_wave_tiles(const MbconvParams &p); // wavefronts a launch would start (0: not supported)
 // Does the launch take one of the guard-free builds (compiled for the tile plans of MobileNetV2-style blocks)?
 // The guarded builds cover every supported shape but do not beat the separate launches.
 bool mbconv_s8_wave_has_fast_build(const MbconvParams &p);
@@ -106,7 +105,7 @@ hipError_t launch_mbconv_s8_wave(const MbconvParams &p, int cu_count, hipStream_
 // The same block for small images (output at most 16 pixels wide): a workgroup of eight wavefronts per tile
 // splits the expanded channels (mbconv_s8_group.hip); block-input channels a multiple of 16, at most 192.
 bool mbconv_s8_group_supports(const MbconvParams &p);
-bool mbconv_s8_group_has_fast_build(const MbconvParams &p); // as for the wave kernel
+bool mbconv_s8_group_has_fast_build(const MbconvParams &p);
 hipError_t launch_mbconv_s8_group(const MbconvParams &p, int cu_count, hipStream_t stream);
 
 // Depthwise -> 1x1 project [-> Add] in one launch of the LDS-tile depthwise kernel: the depthwise

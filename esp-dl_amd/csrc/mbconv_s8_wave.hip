@@ -563,6 +563,9 @@ void wave_layout(WaveArgs &a, size_t *lds)
     *lds = (size_t)a.off_exp + (size_t)kWavesPerGroup * a.wave_bytes;
 }
 
+// Whether a guard-free build exists for a plan (tile geometry, row tiles, alignment, rounding mode of a.p).
+bool wave_plan_has_exact_build(const WaveArgs &a);
+
 WavePlan wave_plan(const MbconvParams &p)
 {
     WavePlan plan;
@@ -597,35 +600,42 @@ WavePlan wave_plan(const MbconvParams &p)
     a.tiles_x = n_cols;
     // rows: cheapest total of expand tiles (x 1.5: MFMA + the longer epilogue) and depthwise MFMAs.  A launch
     // that does not fill the device once (two resident workgroups per compute unit) takes one tile's time
-    // whatever its tile count, so there a lower tile that brings more workgroups wins.
+    // whatever its tile count, so there a lower tile that brings more workgroups wins.  Heights whose plan has a
+    // guard-free build come first: the guarded builds take about three times as long per tile, and a caller
+    // that fuses by espdl_hip_mbconv_s8_preferred gets the same answer at every batch size.
     const int nxpt_limit = 17;
     const double slots = 2.0 * kPlanCus;
-    double best = 1e30;
-    a.th = 0;
-    for (int th = 1; th <= kPtMax; th++) {
-        const int ph = (th - 1) * s + 3;
-        const int n_xpt = (ph * a.pw + 15) / 16;
-        if (n_xpt > nxpt_limit)
-            break;
-        const int tiles_y = (p.out_h + th - 1) / th;
-        const double tile_cost = 1.5 * n_xpt + 3.0 * th + 2.0;
-        const double groups = std::ceil((double)std::max(1, p.batch) * tiles_y * a.tiles_x / kWavesPerGroup);
-        const double rounds = groups / slots;
-        const double cost = tile_cost * std::max(1.0, rounds);
-        if (cost < best) {
-            best = cost;
-            a.th = th;
-        }
-    }
-    if (a.th == 0)
-        return plan;
-    a.ph = (a.th - 1) * s + 3;
-    a.n_xpt = (a.ph * a.pw + 15) / 16;
-    a.tiles_y = (p.out_h + a.th - 1) / a.th;
     a.n_sub = p.exp_c / 16;
     a.rt = (p.out_c + 15) / 16;
     a.x_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.in) & 15) == 0) ? 1 : 0;
     a.we_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.w_expand) & 15) == 0) ? 1 : 0;
+    double best = 1e30;
+    int best_th = 0;
+    bool best_exact = false;
+    for (int th = 1; th <= kPtMax; th++) {
+        a.th = th;
+        a.ph = (th - 1) * s + 3;
+        a.n_xpt = (a.ph * a.pw + 15) / 16;
+        if (a.n_xpt > nxpt_limit)
+            break;
+        a.tiles_y = (p.out_h + th - 1) / th;
+        const bool exact = wave_plan_has_exact_build(a);
+        const double tile_cost = 1.5 * a.n_xpt + 3.0 * th + 2.0;
+        const double groups = std::ceil((double)std::max(1, p.batch) * a.tiles_y * a.tiles_x / kWavesPerGroup);
+        const double rounds = groups / slots;
+        const double cost = tile_cost * std::max(1.0, rounds);
+        if ((exact && !best_exact) || (exact == best_exact && cost < best)) {
+            best = cost;
+            best_th = th;
+            best_exact = exact;
+        }
+    }
+    if (best_th == 0)
+        return plan;
+    a.th = best_th;
+    a.ph = (a.th - 1) * s + 3;
+    a.n_xpt = (a.ph * a.pw + 15) / 16;
+    a.tiles_y = (p.out_h + a.th - 1) / a.th;
     wave_layout(a, &plan.lds);
     if (plan.lds > 64 * 1024)
         return plan;
@@ -726,6 +736,17 @@ bool launch_exact(const WavePlan &plan, hipStream_t stream, bool dry, hipError_t
     return false;
 }
 
+bool wave_plan_has_exact_build(const WaveArgs &a)
+{
+    WavePlan plan;
+    plan.ok = true;
+    plan.a = a;
+    plan.lds = 0;
+    plan.cus = kPlanCus;
+    hipError_t err = hipSuccess;
+    return a.p.half_even ? launch_exact<true>(plan, nullptr, true, &err) : launch_exact<false>(plan, nullptr, true, &err);
+}
+
 hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
 {
     WaveArgs &a = plan.a;
@@ -756,14 +777,7 @@ bool mbconv_s8_wave_supports(const MbconvParams &p)
 bool mbconv_s8_wave_has_fast_build(const MbconvParams &p)
 {
     const WavePlan plan = wave_plan(p);
-    hipError_t err = hipSuccess;
-    return plan.ok && (p.half_even ? launch_exact<true>(plan, nullptr, true, &err) : launch_exact<false>(plan, nullptr, true, &err));
-}
-
-long long mbconv_s8_wave_tiles(const MbconvParams &p)
-{
-    const WavePlan plan = wave_plan(p);
-    return plan.ok ? (long long)p.batch * plan.a.tiles_y * plan.a.tiles_x : 0;
+    return plan.ok && wave_plan_has_exact_build(plan.a);
 }
 
 hipError_t launch_mbconv_s8_wave(const MbconvParams &p, int cu_count, hipStream_t stream)

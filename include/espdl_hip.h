@@ -368,12 +368,11 @@ typedef struct espdl_hip_mbconv_weights {
 int espdl_hip_mbconv_out_shape(const espdl_hip_mbconv_desc *desc, int32_t *out_h, int32_t *out_w);
 int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc);
 /* 1 when the single launch is expected to be faster than the separate launches for this descriptor,
- * batch and rounding mode included (the rule follows measurements on MI355X: the one-wavefront-per-tile
- * kernel, answer 4 of espdl_hip_mbconv_s8_supported, on images of at least 28 x 28 with enough tiles to fill
- * the device; the workgroup-per-tile kernel, answer 5, with at least one image per compute unit; both only
- * where the tile plan has one of the guard-free builds, which exist for the block shapes of MobileNetV2-style
- * networks in both rounding modes; the depthwise+project form, answer 2, always); 0 otherwise.  dl::Model
- * fuses blocks by this answer. */
+ * rounding mode included (the rule follows measurements on MI355X at batch sizes from 1 to 512: the
+ * one-wavefront-per-tile kernel, answer 4 of espdl_hip_mbconv_s8_supported, and the workgroup-per-tile kernel,
+ * answer 5, where the tile plan has one of the guard-free builds, which exist for the block shapes of
+ * MobileNetV2-style networks in both rounding modes; the depthwise+project form, answer 2, always); 0
+ * otherwise.  dl::Model fuses blocks by this answer. */
 int espdl_hip_mbconv_s8_preferred(const espdl_hip_mbconv_desc *desc);
 int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, const espdl_hip_mbconv_weights *weights,
                         const int8_t *residual, int8_t *out, void *stream);

@@ -731,8 +731,9 @@ def _block_desc(m, batch, hw, cin, ce, cout, stride, half_even=False):
 
 def test_mbconv_s8_preferred_follows_the_fast_builds():
     """dl::Model fuses a block where espdl_hip_mbconv_s8_preferred says so: yes for MobileNetV2's block shapes
-    at a batch that fills the device, in both rounding modes; no for a small batch, and no for a shape that
-    only the guarded builds take (they cover it, but the separate launches are as fast)."""
+    in both rounding modes, at a batch that fills the device and at a small one (the tile plan keeps the height
+    that has a guard-free build); no for a shape that only the guarded builds take (they cover it, but the
+    separate launches are as fast)."""
     announce("mbconv_s8_preferred")
     m = espdl()
     L = m.capi.lib()
@@ -746,7 +747,8 @@ def test_mbconv_s8_preferred_follows_the_fast_builds():
             d = _block_desc(m, 256, hw, cin, ce, cout, stride, he)
             assert kind(d) == want_kind, (hw, cin, ce, cout, stride)
             assert pref(d) == 1, (hw, cin, ce, cout, stride, he)
-        assert pref(_block_desc(m, 4, hw, cin, ce, cout, stride)) == 0  # too few tiles to fill the device
+        for small in (1, 4, 64):
+            assert pref(_block_desc(m, small, hw, cin, ce, cout, stride)) == 1, (small, hw, cin, ce, cout, stride)
     odd = _block_desc(m, 256, 50, 24, 144, 24, 1)  # 50 x 50: a tile plan without a guard-free build
     assert kind(odd) == 4 and pref(odd) == 0
 
