@@ -102,9 +102,14 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
 #pragma unroll
             for (int ks = 0; ks < KSE; ks++) {
                 xb[pt * KSE + ks] = v4i{0, 0, 0, 0};
-                if (EXACT || (pt < n_xpt && ks < kse)) // uniform
-                    xb[pt * KSE + ks] = load16_partial<true>(img, (unsigned)((iy * p.in_w + ix) * c0 + 64 * ks + 16 * quad),
-                                                             valid ? c0 - 64 * ks - 16 * quad : 0);
+                if (EXACT || (pt < n_xpt && ks < kse)) { // uniform
+                    // nothing is zeroed here: a pixel outside the image gets its expand OUTPUT zeroed through
+                    // xmask, reduction positions past in_c (a multiple of 16) meet zeros in operand A; such
+                    // lanes read the image's first bytes
+                    const bool ok = valid && c0 - 64 * ks - 16 * quad >= 16;
+                    xb[pt * KSE + ks] = *reinterpret_cast<const v4i *>(
+                        img + (size_t)(ok ? (unsigned)((iy * p.in_w + ix) * c0 + 64 * ks + 16 * quad) : 0u));
+                }
             }
         }
     }
@@ -220,10 +225,12 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
             ap[kk] = load16_partial<true>(p.w_project, a_off + 64u * (unsigned)(k0 + kk),
                                           row_ok ? p.exp_c - 64 * (k0 + kk) - 16 * quad : 0);
     };
+    // KSP builds take whole row tiles and whole k steps only (out_c a multiple of 16, exp_c of 64), so this load
+    // needs no mask: nothing touches the value between the load and its product, and a request for a row tile
+    // past the last one reads the last one again
     auto load_a_step = [&](int rt, int k) {
-        const bool row_ok = rt < a.rt && 16 * rt + col < p.out_c;
-        return load16_partial<true>(p.w_project, (unsigned)((16 * rt + col) * p.exp_c + 16 * quad) + 64u * (unsigned)k,
-                                    row_ok ? p.exp_c - 64 * k - 16 * quad : 0);
+        return *reinterpret_cast<const v4i *>(
+            p.w_project + (size_t)((unsigned)((16 * min(rt, a.rt - 1) + col) * p.exp_c + 16 * quad) + 64u * (unsigned)k));
     };
     // (the blocked form does not prefetch in the build that is held to 128 registers so that two workgroups
     // share a compute unit)
@@ -497,8 +504,8 @@ bool launch_group_exact(const GroupPlan &plan, hipStream_t stream, bool dry, hip
     const int ksp = (a.p.exp_c + 63) / 64;
     // k_project / nt: the project stage's k steps and pixel tiles per wavefront the build is made for (0: any)
     const auto is = [&](int nxpt, int kse, int th, int stride, int k_project, int nt) {
-        return a.n_xpt == nxpt && a.kse == kse && a.th == th && s == stride && (k_project == 0 || ksp == k_project) &&
-            (nt == 0 || a.nt == nt);
+        return a.n_xpt == nxpt && a.kse == kse && a.th == th && s == stride &&
+            (k_project == 0 || (ksp == k_project && a.p.exp_c % 64 == 0 && a.p.out_c % 16 == 0)) && (nt == 0 || a.nt == nt);
     };
 #define ESPDL_GROUP_EXACT(NXPT, KSE, PT, S, KSP, NTX)                                    \
     do {                                                                                 \

@@ -42,6 +42,24 @@ __device__ __forceinline__ v4i load16_partial(const int8_t *p, unsigned off, int
     return r;
 }
 
+// The same addresses, nothing zeroed: pieces that do not exist read the first bytes at `p` and keep them.  For
+// operand B of the expand products, where such bytes never count: a pixel outside the image has its expand
+// OUTPUT zeroed, and reduction positions past the last input channel meet zeros in operand A.  Without the
+// select between a load and its product, the loads of a patch stay in flight behind the set-up that follows.
+template <bool VEC16>
+__device__ __forceinline__ v4i load16_clamped(const int8_t *p, unsigned off, int nvalid)
+{
+    v4i r;
+    if constexpr (VEC16) {
+        r = *reinterpret_cast<const v4i *>(p + (size_t)(nvalid >= 16 ? off : 0u));
+    } else {
+#pragma unroll
+        for (int d = 0; d < 4; d++)
+            r[d] = *reinterpret_cast<const int *>(p + (size_t)(4 * d < nvalid ? off + 4u * d : 0u));
+    }
+    return r;
+}
+
 // Orders the LDS accesses of the wavefront's lanes among each other.  LDS executes the instructions of one
 // wavefront in order, so nothing has to be waited for; the compiler must not move accesses across.
 __device__ __forceinline__ void wave_lds_sync()

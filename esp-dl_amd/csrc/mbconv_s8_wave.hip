@@ -153,7 +153,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
             const unsigned prow = fastdiv(pp, a.fd_pw);
             const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
             const bool valid = pt < NXPT && (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
-            xb[g] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * sub), valid ? c0 - 16 * sub : 0);
+            xb[g] = load16_clamped<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * sub), valid ? c0 - 16 * sub : 0);
             const unsigned long long votes = __ballot(valid); // bit 16 quad + col
 #pragma unroll
             for (int t = 0; t < PACK; t++)
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
             xmask = col_valid ? rows : 0u;
 #pragma unroll
             for (int pt = 0; pt < NXPT; pt++)
-                xb[pt] = load16_partial<VEC16>(img, (unsigned)(o0 + pt * o_step), ((xmask >> pt) & 1u) ? c0 - 16 * quad : 0);
+                xb[pt] = load16_clamped<VEC16>(img, (unsigned)(o0 + pt * o_step), ((xmask >> pt) & 1u) ? c0 - 16 * quad : 0);
         } else {
 #pragma unroll
             for (int pt = 0; pt < NXPT; pt++) {
@@ -186,7 +186,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
                     const int iy = iy0 + (int)prow, ix = ix0 + (int)(pp - prow * a.fd_pw.d);
                     const bool valid = (int)prow < a.ph && (unsigned)iy < (unsigned)p.in_h && (unsigned)ix < (unsigned)p.in_w;
                     xmask |= valid ? 1u << pt : 0u;
-                    xb[pt] = load16_partial<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
+                    xb[pt] = load16_clamped<VEC16>(img, (unsigned)((iy * p.in_w + ix) * c0 + 16 * quad),
                                                    valid ? c0 - 16 * quad : 0);
                 }
             }
