@@ -33,7 +33,7 @@ class MbconvDesc(ctypes.Structure):
         "dil_h", "dil_w", "pad_top", "pad_bottom", "pad_left", "pad_right", "act_expand", "act_dw", "act_project",
         "round_mode", "n_shift_expand", "n_shift_dw", "n_shift_project",
         "exp_k_h", "exp_k_w", "exp_stride_h", "exp_stride_w", "exp_pad_top", "exp_pad_bottom", "exp_pad_left",
-        "exp_pad_right")]
+        "exp_pad_right", "residual_shift")]
 
 
 class MbconvWeights(ctypes.Structure):
@@ -183,7 +183,8 @@ def conv2d(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 
 
 
 def mbconv_s8(x, expand, dw, project, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), relus=(True, True, False),
-              residual=None, round_mode=ROUND_HALF_UP, out=None, stream=None, staged=False, expand_conv=None):
+              residual=None, round_mode=ROUND_HALF_UP, out=None, stream=None, staged=False, expand_conv=None,
+              residual_shift=0):
     """Fused inverted-residual block (staged=True: espdl_hip_mbconv_s8_staged, the separate stages with the
     intermediates in the library's own device array; `out` must then be given, nothing is allocated).  expand / dw / project are (filter, bias, shift) triples of CUDA
     tensors (expand may be None); filters as for conv2d: [E][C], [kH][kW][E], [OC][E].
@@ -204,6 +205,7 @@ def mbconv_s8(x, expand, dw, project, k, stride=(1, 1), dilation=(1, 1), pads=(0
         ek, es, ep = expand_conv
         (desc.exp_k_h, desc.exp_k_w, desc.exp_stride_h, desc.exp_stride_w) = (ek[0], ek[1], es[0], es[1])
         (desc.exp_pad_top, desc.exp_pad_bottom, desc.exp_pad_left, desc.exp_pad_right) = ep
+    desc.residual_shift = residual_shift
     oh, ow = ctypes.c_int32(), ctypes.c_int32()
     _check(lib().espdl_hip_mbconv_out_shape(ctypes.byref(desc), ctypes.byref(oh), ctypes.byref(ow)))
     if out is None:

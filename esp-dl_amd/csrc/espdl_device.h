@@ -177,6 +177,38 @@ __device__ __forceinline__ int pack_fast4_add(const v4i &acc, const v4i &lsh, co
                                       0x07050301u);
 }
 
+// Four packed int8 requantized by 2^d, d in [-7, 7]: what RequantizeLinear / TensorBase::assign does between two
+// int8 exponents (esp-dl/dl/tensor/src/dl_tensor_base.cpp:362-371: round(x * 2^d) half up, saturated).  The
+// bytes are spread into the high bytes of int16 pairs (x * 256).  d > 0: a saturating multiply by 2^d.  d < 0:
+// x * 128 (one shift, so that the rounding constant cannot overflow), + 2^(6-d), arithmetic shift by -d - 1.
+// The result's high bytes are the answer.
+struct Requant4 {
+    int mul, pre, rnd, sh;
+};
+__device__ __forceinline__ Requant4 make_requant4(int d)
+{
+    Requant4 q;
+    q.mul = (1 << max(d, 0)) * 0x00010001;
+    q.pre = d < 0 ? 1 : 0;
+    q.rnd = d < 0 ? (1 << (6 - d)) * 0x00010001 : 0;
+    q.sh = d < 0 ? -d - 1 : 0;
+    return q;
+}
+__device__ __forceinline__ int requant4_s8(int word, const Requant4 &q)
+{
+    int out[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const int hi = (int)__builtin_amdgcn_perm(0u, (unsigned)word, h == 0 ? 0x010c000cu : 0x030c020cu);
+        v2s v = pk_mul_sat_i16(__builtin_bit_cast(v2s, hi), q.mul);
+        v = v >> (short)q.pre;
+        v = v + __builtin_bit_cast(v2s, q.rnd);
+        v = v >> (short)q.sh;
+        out[h] = __builtin_bit_cast(int, v);
+    }
+    return (int)__builtin_amdgcn_perm((unsigned)out[1], (unsigned)out[0], 0x07050301u);
+}
+
 // int8 x 4 saturating add of two packed dwords
 __device__ __forceinline__ int sat_add4_s8(int x, int y)
 {

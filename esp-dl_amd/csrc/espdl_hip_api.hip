@@ -732,6 +732,9 @@ int mbconv_geometry(const espdl_hip_mbconv_desc *d, espdl::MbconvParams *p)
     p->n_s_expand = d->n_shift_expand;
     p->n_s_dw = d->n_shift_dw;
     p->n_s_project = d->n_shift_project;
+    if (d->residual_shift < -7 || d->residual_shift > 7)
+        return fail(ESPDL_HIP_EINVAL, "residual_shift %d outside [-7, 7]", d->residual_shift);
+    p->residual_shift = d->residual_shift;
     if ((long long)p->batch * p->out_h * p->out_w > 0x7fffffffll - 65536)
         return fail(ESPDL_HIP_EINVAL, "too many output pixels");
     return ESPDL_HIP_OK;
@@ -807,7 +810,18 @@ int espdl_hip_mbconv_out_shape(const espdl_hip_mbconv_desc *desc, int32_t *out_h
     return ESPDL_HIP_OK;
 }
 
+static int mbconv_kernel_choice(const espdl_hip_mbconv_desc *desc);
+
 int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
+{
+    const int kind = mbconv_kernel_choice(desc);
+    // a requantized residual operand is built into the two kernels that carry MobileNetV2-style networks
+    if (kind != 0 && desc->residual_shift != 0 && kind != 4 && kind != 5)
+        return 0;
+    return kind;
+}
+
+static int mbconv_kernel_choice(const espdl_hip_mbconv_desc *desc)
 {
     espdl::MbconvParams p = {};
     if (mbconv_geometry(desc, &p) != ESPDL_HIP_OK)
@@ -874,6 +888,12 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
         return rc;
     if (p.batch == 0)
         return ESPDL_HIP_OK;
+    if (p.residual_shift != 0) {
+        const int kind = espdl_hip_mbconv_s8_supported(desc);
+        if (kind != 4 && kind != 5)
+            return fail(ESPDL_HIP_ENOTSUP, "a requantized residual operand (residual_shift %d) is not covered for this block shape",
+                        p.residual_shift);
+    }
     if (in == nullptr || out == nullptr || w == nullptr || w->w_dw == nullptr || w->s_dw == nullptr ||
         w->w_project == nullptr || w->s_project == nullptr || (desc->has_expand && (w->w_expand == nullptr || w->s_expand == nullptr)))
         return fail(ESPDL_HIP_EINVAL, "in, out, filters and shifts must not be NULL");

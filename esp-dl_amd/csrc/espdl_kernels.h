@@ -85,6 +85,10 @@ struct MbconvParams {
     // extents of the DEPTHWISE stage's input (the expand convolution's output), img_h / img_w are those of
     // the block input, w_expand is [exp_c][ek_h][ek_w][in_c].  For the 1x1 expand img == in and ek == es == 1.
     int img_h, img_w, ek_h, ek_w, es_h, es_w, epad_top, epad_left;
+    // The residual operand is requantized by 2^residual_shift (round half up, saturated) before the Add:
+    // a RequantizeLinear between two int8 exponents in front of the Add.  -7 .. 7; only the one-wavefront-per-tile
+    // and the workgroup-per-tile kernels take a value other than 0.
+    int residual_shift;
 };
 inline bool mbconv_expand_is_pointwise(const MbconvParams &p)
 {

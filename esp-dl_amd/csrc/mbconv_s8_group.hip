@@ -255,6 +255,7 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
     // Reduction positions past exp_c meet zeros in operand A, whatever operand B holds there.
     const int t0 = wpix * a.nt;
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
+    const Requant4 res_q = make_requant4(p.residual_shift);
     const long long img_off = (long long)n * p.out_h * p.out_w * p.out_c;
     const int8_t *res_img = p.residual != nullptr ? p.residual + img_off : nullptr;
     int8_t *out_img = p.out + img_off;
@@ -354,10 +355,13 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
                         acc[k] += cp.init[k];
                     int word;
                     if constexpr (RES) {
+                        int res = rv[i];
+                        if (p.residual_shift != 0) // uniform
+                            res = requant4_s8(res, res_q);
                         if constexpr (MODE >= 0)
-                            word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, rv[i]);
+                            word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, res);
                         else
-                            word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), rv[i]);
+                            word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), res);
                     } else {
                         word = wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE);
                     }

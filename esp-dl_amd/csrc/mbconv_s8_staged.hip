@@ -65,6 +65,9 @@ extern "C" int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *d, const 
         return ESPDL_HIP_OK;
     if (in == nullptr || out == nullptr || w == nullptr)
         return espdl::set_error(ESPDL_HIP_EINVAL, "in, out and weights must not be NULL");
+    if (d->residual_shift != 0 && residual != nullptr)
+        return espdl::set_error(ESPDL_HIP_ENOTSUP, "the staged form adds the residual operand as it is (residual_shift %d): "
+                                                   "requantize it first with espdl_hip_requantize_s8", d->residual_shift);
     // extents of the depthwise stage's input: the block input's, or those of an expand stage with a window
     const bool windowed = d->exp_k_h > 0;
     const int mid_h = windowed ? (d->in_h + d->exp_pad_top + d->exp_pad_bottom - d->exp_k_h) / d->exp_stride_h + 1 : d->in_h;

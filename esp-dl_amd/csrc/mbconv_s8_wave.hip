@@ -492,6 +492,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
     // a row of a ragged last tile that does not exist is a store that no lane takes: the words of a tile are
     // one straight-line block.
     const int floor_p = p.relu_project ? 0 : (int)0x80008000u;
+    const Requant4 res_q = make_requant4(p.residual_shift);
     auto words = [&](auto mode_tag, auto res_tag) {
         constexpr int MODE = decltype(mode_tag)::value;
         constexpr bool RES = decltype(res_tag)::value;
@@ -509,10 +510,13 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
                         acc[k] += cp.init[k];
                     int word;
                     if constexpr (RES) {
+                        int res = resw[r][t];
+                        if (p.residual_shift != 0) // uniform
+                            res = requant4_s8(res, res_q);
                         if constexpr (MODE >= 0)
-                            word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, resw[r][t]);
+                            word = pack_fast4_add<MODE>(acc, cp.lsh, cp.rsh, floor_p, res);
                         else
-                            word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), resw[r][t]);
+                            word = sat_add4_s8(wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE), res);
                     } else {
                         word = wave_pack<MODE>(acc, cp, floor_p, p.relu_project != 0, HE);
                     }

@@ -354,6 +354,12 @@ typedef struct espdl_hip_mbconv_desc {
      * zero: the 1x1 stride-1 convolution.  Filter layout [exp_c][exp_k_h][exp_k_w][in_c]. */
     int32_t exp_k_h, exp_k_w, exp_stride_h, exp_stride_w;
     int32_t exp_pad_top, exp_pad_bottom, exp_pad_left, exp_pad_right;
+    /* The residual operand stands at another exponent than the block output: it is requantized by
+     * 2^residual_shift first (residual exponent - output exponent, -7 .. 7; round half up and saturate, as
+     * TensorBase::assign does for the RequantizeLinear node that an exporter puts in front of such an Add,
+     * esp-dl/dl/tensor/src/dl_tensor_base.cpp:362-371).  0: the operand is added as it is.  Taken by the
+     * single-launch kernels of answers 4 and 5 only; espdl_hip_mbconv_s8_supported answers 0 elsewhere. */
+    int32_t residual_shift;
 } espdl_hip_mbconv_desc;
 
 typedef struct espdl_hip_mbconv_weights {

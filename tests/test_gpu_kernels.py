@@ -716,6 +716,37 @@ def test_mbconv_s8_guard_free_builds_ragged_tiles(oracle, case):
     np.testing.assert_array_equal(to_host(got), cur)
 
 
+# A residual operand at another exponent than the block output: the kernels requantize it in registers, as the
+# RequantizeLinear node in front of the Add would (every shift the descriptor allows; wave and group kernels).
+@pytest.mark.parametrize("shape", [(40, 28, 28, 32, 192, 32), (40, 14, 14, 64, 384, 64), (3, 20, 20, 8, 48, 8)],
+                         ids=["wave_28x28", "group_14x14", "wave_guarded_20x20"])
+@pytest.mark.parametrize("shift", [-7, -3, -1, 1, 2, 7])
+def test_mbconv_s8_requantized_residual(oracle, shape, shift):
+    announce(f"mbconv_s8 residual requantized by 2^{shift}, {shape}")
+    n, h, w, cin, ce, cout = shape
+    m = espdl()
+    rng = np.random.default_rng(0x5E51 + shift + h)
+    oracle.set_threads(16)
+
+    def stage(oc, kk, fshape):
+        return (rng_int8(rng, fshape), rng.integers(-4096, 4097, size=oc).astype(np.int32),
+                (typical_shift(kk) + rng.integers(-2, 3, size=oc)).astype(np.int32))
+
+    x = rng_int8(rng, (n, h, w, cin))
+    ex, dw, pj = stage(ce, cin, (ce, 1, 1, cin)), stage(ce, 9, (3, 3, ce)), stage(cout, ce, (cout, 1, 1, ce))
+    pads = (1, 1, 1, 1)
+    cur = oracle.conv2d_s8(x, ex[0], ex[1], ex[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.RELU)
+    cur = oracle.depthwise_s8(cur, dw[0], dw[1], dw[2], (3, 3), (1, 1), (1, 1), pads, oracle.RELU)
+    cur = oracle.conv2d_s8(cur, pj[0], pj[1], pj[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.LINEAR)
+    res = rng_int8(rng, cur.shape)
+    res[0, 0, 0, :8] = [-128, -127, -1, 0, 1, 63, 64, 127][:min(8, cout)]
+    want = oracle.add_s8(cur, oracle.requantize_s8(res, shift, 0))
+    dev = lambda t: tuple(to_dev(a) for a in t)  # noqa: E731
+    got = m.mbconv_s8(to_dev(x), dev(ex), dev(dw), dev(pj), (3, 3), (1, 1), (1, 1), pads, (True, True, False),
+                      residual=to_dev(res), residual_shift=shift)
+    np.testing.assert_array_equal(to_host(got), want)
+
+
 def _block_desc(m, batch, hw, cin, ce, cout, stride, half_even=False):
     d = m.capi.MbconvDesc()
     d.batch, d.in_h, d.in_w, d.in_c, d.exp_c, d.out_c, d.has_expand = batch, hw, hw, cin, ce, cout, 1

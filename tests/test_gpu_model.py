@@ -106,6 +106,11 @@ def test_config3_mobilenetv2_full_resolution(oracle):
     assert mdl.shape(spec.outputs[0]) == [2, 1000]
     logits = want[spec.outputs[0]]
     assert logits.min() < 0 < logits.max() and len(np.unique(logits)) > 50  # not degenerate
+    # every inverted-residual block is one module (the stem inside the first), and the two RequantizeLinear
+    # nodes that only align a residual operand's exponent ride in their block's launch: 17 blocks + head
+    # convolution + GlobalAveragePool + the view + Gemm
+    n_requant = sum(1 for n in spec.nodes if n["op_type"] == "RequantizeLinear")
+    assert n_requant == 2 and mdl.module_count() == 21
     mdl.close()
 
 
