@@ -144,6 +144,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch kernels eagerly instead of HIP-graph replay")
     ap.add_argument("--profile-repeats", type=int, default=5)
     ap.add_argument("--layers", action="store_true", help="print the per-module timing table to stderr")
+    ap.add_argument("--no-fuse-gap", action="store_true",
+                    help="run GlobalAveragePool as a module of its own instead of inside the 1x1 convolution before it")
     ap.add_argument("--no-fuse-add", action="store_true",
                     help="keep residual Adds as separate kernels instead of folding them into the conv before them")
     ap.add_argument("--copy-mib", type=int, default=0,
@@ -174,7 +176,7 @@ def main():
     spec = pkg.zoo.CONFIGS[args.config]()
     batch = args.batch
     graph = pkg.model.Graph.from_spec(spec)
-    mdl = pkg.model.Model(graph, batch, fuse_add=not args.no_fuse_add)
+    mdl = pkg.model.Model(graph, batch, fuse_add=not args.no_fuse_add, fuse_gap=not args.no_fuse_gap)
     x = spec.make_input(np.random.default_rng(0xE5D10003), batch)
     mdl.set_input(spec.inputs[0], x)  # resident in HBM from here on
     mdl.run()

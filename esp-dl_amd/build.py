@@ -18,6 +18,9 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             # the float-defined operators (pooling, requantize, table builders) round every product to float
+             # before the next operation, as the reference's C code does: no fused multiply-add
+             "-ffp-contract=off",
              # keep MFMA accumulators in ordinary VGPRs: no v_accvgpr_read/write around the epilogue
              "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 

@@ -72,6 +72,10 @@ def lib():
         L.espdl_hip_conv2d.argtypes = [dp, vp, vp, vp, vp, vp, vp, vp]
         L.espdl_hip_conv2d_add.argtypes = [dp, vp, vp, vp, vp, vp, vp, vp, vp]
         L.espdl_hip_conv2d_add.restype = ctypes.c_int
+        L.espdl_hip_conv2d_gap_s8.argtypes = [dp, vp, vp, vp, vp, i32, i32, vp, vp]
+        L.espdl_hip_conv2d_gap_s8.restype = ctypes.c_int
+        L.espdl_hip_conv2d_gap_s8_supported.argtypes = [dp]
+        L.espdl_hip_conv2d_gap_s8_supported.restype = ctypes.c_int
         L.espdl_hip_lut_s8.argtypes = [vp, i64, vp, vp, vp]
         L.espdl_hip_prelu_s8.argtypes = [vp, i64, i32, vp, i32, vp, vp]
         L.espdl_hip_relu_s8.argtypes = [vp, i64, i32, i32, vp, vp]
@@ -179,6 +183,21 @@ def conv2d(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 
         out = torch.empty((n, oh, ow, out_c), dtype=x.dtype, device=x.device)
     _check(lib().espdl_hip_conv2d_add(ctypes.byref(desc), _p(x), _p(filt), _p(bias), _p(shift), _p(lut), _p(residual),
                                       _p(out), _stream(stream)))
+    return out
+
+
+def conv2d_gap_s8(x, filt, bias, shift, conv_out_exp, pool_out_exp, activation=LINEAR, round_mode=ROUND_HALF_UP,
+                  out=None, stream=None):
+    """1x1 convolution followed by GlobalAveragePool in one launch: x [N,H,W,C] int8 with H*W <= 64, filt [OC][C];
+    returns the pooled [N][OC] int8 tensor (espdl_hip_conv2d_gap_s8)."""
+    import torch
+    n, h, w, c = x.shape
+    out_c = filt.numel() // c
+    desc = make_desc(x.shape, out_c, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), 1, activation, round_mode, shift.numel(), S8)
+    if out is None:
+        out = torch.empty((n, out_c), dtype=torch.int8, device=x.device)
+    _check(lib().espdl_hip_conv2d_gap_s8(ctypes.byref(desc), _p(x), _p(filt), _p(bias), _p(shift), conv_out_exp,
+                                         pool_out_exp, _p(out), _stream(stream)))
     return out
 
 

@@ -41,11 +41,20 @@ struct PwArgs {
     int ksteps;
     int relu, half_even, n_shift;
     int out_vec; // 16, 4 or 1
+    int hw;          // GAP builds: pixels per image (at most 64)
+    float gap_scale; // GAP builds: 2^in_exp / (h w) * 2^-out_exp of the pooling operator
 };
 
-template <int NG, int PT>
+// GAP: the convolution is followed by a GlobalAveragePool (base::avgpool2d_hwc with the filter covering the whole
+// image, esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54) and only the pooled tensor [image][filter] is written.  A
+// workgroup's pixel tile is then PT images of at most 64 pixels, 64 tile rows each: the convolution's int8
+// results (requantized, activation applied, exactly what the separate operator would have stored) are summed
+// over the image's pixels - over the 16 lanes of a pixel tile by rotations inside the row, over the four
+// wavefronts through LDS - and the sum goes through the pooling operator's float scale and rounding.
+template <int NG, int PT, bool GAP = false>
 __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs a)
 {
+    static_assert(!GAP || NG == 1, "the pooled form works on 64 filters per workgroup");
     constexpr int TN = 64 * NG;
     constexpr int kTileM = 64 * PT; // pixels per workgroup, 16 * PT per wavefront
     constexpr int kPiecesB = kTileM * 4 / kThreads; // 16-byte pieces of the pixel tile per thread and k step (2)
@@ -54,10 +63,22 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     __shared__ __align__(16) unsigned char a_l[2][TN * kRow];
     __shared__ int cst[3][TN]; // start value | shift | left shift
     __shared__ int8_t lut_l[256];
+    __shared__ int pool_l[GAP ? 4 * PT : 1][GAP ? 64 : 1]; // [wavefront x pixel tile][filter]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 15, quad = lane >> 4;
     const long long m0 = (long long)blockIdx.x * kTileM;
+    // tile row -> pixel of the flat [M][K] input, or -1.  Pooled form: rows 64 i .. 64 i + hw - 1 are image
+    // PT * blockIdx.x + i.
+    auto row_pixel = [&](int r) -> long long {
+        if constexpr (GAP) {
+            const long long img = (long long)blockIdx.x * PT + (r >> 6);
+            const int pix = r & 63;
+            return (pix < a.hw && img * a.hw < a.M) ? img * a.hw + pix : -1;
+        } else {
+            return m0 + r < a.M ? m0 + r : -1;
+        }
+    };
     const int n0 = blockIdx.y * TN;
     const bool relu = a.relu != 0, half_even = a.half_even != 0, has_lut = a.lut != nullptr;
 
@@ -67,9 +88,9 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
 #pragma unroll
         for (int j = 0; j < kPiecesB; j++) {
             const int p = tid + j * kThreads;
-            const long long m = m0 + (p >> 2);
+            const long long m = row_pixel(p >> 2);
             const int k = k0 + 16 * (p & 3);
-            pb[j] = (m < a.M && k < a.K) ? *reinterpret_cast<const v4i *>(a.in + m * a.K + k) : v4i{0, 0, 0, 0};
+            pb[j] = (m >= 0 && k < a.K) ? *reinterpret_cast<const v4i *>(a.in + m * a.K + k) : v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int j = 0; j < kPiecesA; j++) {
@@ -213,6 +234,24 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
                                             lut_l[(int)(int8_t)(v >> 16) + 128], lut_l[(v >> 24) + 128]);
                     }
                 }
+                if constexpr (GAP) {
+                    // this lane's 16 filters of its pixel: sum over the 16 pixels of the tile
+                    const bool pixel = row_pixel(16 * PT * wave + 16 * c + col) >= 0;
+#pragma unroll
+                    for (int t = 0; t < 4; t++)
+#pragma unroll
+                        for (int r = 0; r < 4; r++) {
+                            int v = pixel ? (int)(int8_t)(words[t] >> (8 * r)) : 0;
+                            // rotations by 8, 4, 2, 1 inside the row of 16 lanes: every lane ends with the row's sum
+                            v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false);
+                            v += __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false);
+                            v += __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false);
+                            v += __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false);
+                            if (col == 0)
+                                pool_l[wave * PT + c][16 * quad + 4 * t + r] = v;
+                        }
+                    continue;
+                }
                 if (m >= a.M || n >= a.N)
                     continue;
                 const long long goff = m * a.N + n;
@@ -252,6 +291,18 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
         epilogue(std::integral_constant<int, 2>{});
     else
         epilogue(std::integral_constant<int, 1>{});
+    if constexpr (GAP) {
+        __syncthreads();
+        const int img_l = tid >> 6, flt = tid & 63; // image of the tile, filter of the group
+        const long long img = (long long)blockIdx.x * PT + img_l;
+        if (img_l < PT && img * a.hw < a.M && n0 + flt < a.N) {
+            int sum = 0;
+#pragma unroll
+            for (int i = 0; i < 4 * PT; i++) // pixel tile i holds tile rows 16 i ..: image i / 4
+                sum += (i >> 2) == img_l ? pool_l[i][flt] : 0;
+            a.out[img * a.N + n0 + flt] = (int8_t)clamp_s8(round_half_up_f32((float)sum * a.gap_scale));
+        }
+    }
 }
 
 } // namespace
@@ -289,6 +340,8 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
     a.relu = g.relu;
     a.half_even = g.half_even;
     a.n_shift = g.n_shift;
+    a.hw = 0;
+    a.gap_scale = 0.f;
     const uintptr_t oaddr = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(residual);
     a.out_vec = ((a.N & 15) == 0 && (oaddr & 15) == 0) ? 16 : (((a.N & 3) == 0 && (oaddr & 3) == 0) ? 4 : 1);
     if (a.M == 0)
@@ -302,6 +355,48 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
         hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1>), dim3((unsigned)((a.M + 63) / 64), gy), dim3(kThreads), 0, stream, a);
     else
         hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2>), dim3((unsigned)tiles128, gy), dim3(kThreads), 0, stream, a);
+    return hipGetLastError();
+}
+
+// The same convolution followed by GlobalAveragePool, pooled tensor only: images of at most 64 pixels.
+bool conv2d_gap_s8_supports(const ConvGeom &g, const void *in, const void *filter)
+{
+    const bool flat = g.k_h == 1 && g.k_w == 1 && g.stride_h == 1 && g.stride_w == 1 && g.pad_top == 0 &&
+        g.pad_left == 0 && g.out_h == g.in_h && g.out_w == g.in_w;
+    return flat && (g.in_c & 15) == 0 && g.in_c >= 64 && g.out_c >= 32 && g.out_h * g.out_w <= 64 && g.batch <= 0x7fffffff &&
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) == 0;
+}
+
+hipError_t launch_conv2d_gap_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                const int32_t *shift, float gap_scale, int8_t *out, int cu_count, hipStream_t stream)
+{
+    const int cus = cu_count > 0 ? cu_count : 256;
+    PwArgs a;
+    a.in = in;
+    a.w = filter;
+    a.bias = bias;
+    a.shift = shift;
+    a.lut = nullptr;
+    a.res = nullptr;
+    a.out = out;
+    a.hw = g.out_h * g.out_w;
+    a.M = (long long)g.batch * a.hw;
+    a.K = g.in_c;
+    a.N = g.out_c;
+    a.ksteps = (a.K + 63) / 64;
+    a.relu = g.relu;
+    a.half_even = g.half_even;
+    a.n_shift = g.n_shift;
+    a.out_vec = 1;
+    a.gap_scale = gap_scale;
+    if (a.M == 0)
+        return hipSuccess;
+    // two images per workgroup (each filter tile is then read half as often) unless that leaves compute units idle
+    const unsigned gy = (unsigned)((a.N + 63) / 64);
+    if ((long long)((g.batch + 1) / 2) * gy >= 2ll * cus)
+        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2, true>), dim3((unsigned)((g.batch + 1) / 2), gy), dim3(kThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1, true>), dim3((unsigned)g.batch, gy), dim3(kThreads), 0, stream, a);
     return hipGetLastError();
 }
 

@@ -392,13 +392,19 @@ hipError_t launch_mul_s8(const int32_t dims[4], const int64_t s0[4], const int64
     return launch_binary_s8(dims, s0, s1, in0, in1, out, MulOp{shift, half_even != 0}, stream);
 }
 
+// the float factor of the pooling operator, formed as the reference forms it
+float global_avg_pool_scale(int h, int w, int in_exp, int out_exp)
+{
+    const float area_inv = 1.f / (float)(h * w);
+    return dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
+}
+
 hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
                                      int8_t *out, hipStream_t stream)
 {
     if (batch <= 0)
         return hipSuccess;
-    const float area_inv = 1.f / (float)(h * w);
-    const float scale = dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
+    const float scale = global_avg_pool_scale(h, w, in_exp, out_exp);
     if ((c & 3) == 0 && h * w <= 64 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 3) == 0)
         hipLaunchKernelGGL(global_avg_pool_s8_small_kernel, dim3((unsigned)((c / 4 + kBlock - 1) / kBlock), (unsigned)batch),
                            dim3(kBlock), 0, stream, in, out, h * w, c, scale);

@@ -206,6 +206,42 @@ int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const 
     return device_status(espdl::launch_conv2d_s16(g, i16, f16, b64, shift, o16, s), "conv2d_s16");
 }
 
+static int check_exps(int32_t in_exp, int32_t out_exp);
+
+int espdl_hip_conv2d_gap_s8_supported(const espdl_hip_conv_desc *desc)
+{
+    espdl::ConvGeom g;
+    if (desc == nullptr || desc->dtype != ESPDL_HIP_S8 || desc->group != 1 || derive_geometry(desc, &g) != ESPDL_HIP_OK)
+        return 0;
+    static const int8_t *const aligned = reinterpret_cast<const int8_t *>(uintptr_t(256));
+    return espdl::conv2d_gap_s8_supports(g, aligned, aligned) ? 1 : 0;
+}
+
+int espdl_hip_conv2d_gap_s8(const espdl_hip_conv_desc *desc, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                            const int32_t *shift, int32_t conv_out_exp, int32_t pool_out_exp, int8_t *out, void *stream)
+{
+    espdl::ConvGeom g;
+    const int rc = derive_geometry(desc, &g);
+    if (rc != ESPDL_HIP_OK)
+        return rc;
+    if (desc->dtype != ESPDL_HIP_S8 || desc->group != 1)
+        return fail(ESPDL_HIP_ENOTSUP, "the pooled form exists for dense int8 convolutions only");
+    if (check_exps(conv_out_exp, pool_out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (g.batch == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || filter == nullptr || shift == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in, filter, shift and out must not be NULL");
+    if (misaligned(bias, 4) || misaligned(shift, 4))
+        return fail(ESPDL_HIP_EINVAL, "bias and shift must be 4-byte aligned");
+    if (!espdl::conv2d_gap_s8_supports(g, in, filter))
+        return fail(ESPDL_HIP_ENOTSUP, "the pooled form takes 1x1 stride-1 convolutions over images of at most 64 pixels, "
+                                       "input channels a multiple of 16 (at least 64), 16-byte aligned input and filter");
+    const float scale = espdl::global_avg_pool_scale(g.out_h, g.out_w, conv_out_exp, pool_out_exp);
+    return device_status(espdl::launch_conv2d_gap_s8(g, in, filter, bias, shift, scale, out, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                         "conv2d_gap_s8");
+}
+
 int espdl_hip_lut_s8(const int8_t *in, int64_t size, const int8_t *table, int8_t *out, void *stream)
 {
     if (size < 0)

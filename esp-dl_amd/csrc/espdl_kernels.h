@@ -28,6 +28,12 @@ bool conv2d_s8_pwgemm_supports(const ConvGeom &g, const void *in, const void *fi
 hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                    const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
                                    int cu_count, hipStream_t stream);
+// The pointwise convolution followed by GlobalAveragePool, writing only the pooled [batch][out_c] tensor (images
+// of at most 64 pixels); gap_scale from global_avg_pool_scale.
+bool conv2d_gap_s8_supports(const ConvGeom &g, const void *in, const void *filter);
+hipError_t launch_conv2d_gap_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                const int32_t *shift, float gap_scale, int8_t *out, int cu_count, hipStream_t stream);
+float global_avg_pool_scale(int h, int w, int in_exp, int out_exp);
 
 hipError_t launch_depthwise_s8(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                const int32_t *shift, const int8_t *lut, int8_t *out, hipStream_t stream);

@@ -52,6 +52,8 @@ private:
     int m_lut_in_exponent = 0;   ///< exponent of the conv result that indexes a fused LUT
     int m_project_filter_pos = -1, m_project_bias_pos = -1, m_residual_pos = -1;
     bool m_residual_requantized = false;
+    bool m_has_gap = false;      // a GlobalAveragePool behind this (1x1) convolution runs in its launch
+    int m_gap_in_exponent = 0;   // exponent of the tensor the convolution used to write
     int m_own_inputs = 0; ///< inputs of the Conv itself when a plain residual Add was absorbed
     bool m_has_pre_add_exponent = false;
     int m_pre_add_exponent = 0; ///< exponent of the tensor an absorbed Add used to read from this module
@@ -170,6 +172,15 @@ public:
         m_inputs_index.push_back(residual_index);
     }
     bool has_fused_residual() const { return m_residual_pos >= 0; }
+    /// Absorb the GlobalAveragePool that is the only reader of this convolution's output: the module then
+    /// writes the pooled tensor [N, 1, 1, C] (espdl_hip_conv2d_gap_s8); `conv_out_exponent` is the exponent of
+    /// the tensor the convolution used to write.
+    void fuse_gap(int conv_out_exponent)
+    {
+        m_has_gap = true;
+        m_gap_in_exponent = conv_out_exponent;
+    }
+    bool has_fused_gap() const { return m_has_gap; }
     /// Position of the depthwise bias in m_inputs_index, or -1.
     int own_bias_pos() const
     {
@@ -205,6 +216,8 @@ public:
             output_shape[3] = m_group == 1 ? filter_shape[3] : input_shape[3];
             if (m_has_project)
                 output_shape[3] = input_shapes[m_project_filter_pos][3];
+            if (m_has_gap)
+                output_shape[1] = output_shape[2] = 1;
         }
         return {output_shape};
     }
@@ -213,6 +226,10 @@ public:
     {
         std::vector<int> out = get_output_shape(input_shapes)[0];
         const std::vector<int> &f = input_shapes[1];
+        if (m_has_gap) { // a 1x1 stride-1 convolution: as many output pixels as input pixels
+            out[1] = input_shapes[0][1];
+            out[2] = input_shapes[0][2];
+        }
         int64_t pixels = 1;
         for (size_t i = 0; i + 1 < out.size(); i++)
             pixels *= out[i];
@@ -291,6 +308,18 @@ public:
             return;
         }
         d.round_mode = context->round_mode == ROUND_MODE_HALF_EVEN ? ESPDL_HIP_ROUND_HALF_EVEN : ESPDL_HIP_ROUND_HALF_UP;
+        if (m_has_gap) {
+            const std::vector<int32_t> gs = conv_shifts(m_gap_in_exponent, input, filter, d.out_c);
+            d.n_shift = (int32_t)gs.size();
+            const int rc = espdl_hip_conv2d_gap_s8(&d, static_cast<const int8_t *>(input->data),
+                                                   static_cast<const int8_t *>(filter->data),
+                                                   bias ? static_cast<const int32_t *>(bias->data) : nullptr, m_shift.sync(gs),
+                                                   m_gap_in_exponent, output->exponent.get(),
+                                                   static_cast<int8_t *>(output->data), context->stream);
+            if (rc != ESPDL_HIP_OK)
+                DL_LOGE("Conv", "%s: %s", name.c_str(), espdl_hip_last_error());
+            return;
+        }
         const std::vector<int32_t> shifts =
             conv_shifts(m_fused_lut ? m_lut_in_exponent
                                     : (m_has_pre_add_exponent ? m_pre_add_exponent : output->exponent.get()),

@@ -186,6 +186,8 @@ esp_err_t Model::load(fbs::FbsModel *fbs_model)
         fuse_dw_project();
     if (ret == ESP_OK && (m_fuse & FUSE_CONV_ADD))
         fuse_conv_add();
+    if (ret == ESP_OK && (m_fuse & FUSE_CONV_GAP))
+        fuse_conv_gap();
     return ret;
 }
 
@@ -457,6 +459,69 @@ void Model::fuse_dw_project()
             if (rq_pos <= i + 1) // it stood before the module the loop looks at next
                 i--;
         }
+    }
+}
+
+// 1x1 Conv -> GlobalAveragePool with no other reader of the conv output (the head of a classification
+// network): one kernel forms the convolution's int8 results, sums them per image and filter and writes the
+// pooled tensor only (espdl_hip_conv2d_gap_s8); the convolution's output tensor disappears from the plan.
+void Model::fuse_conv_gap()
+{
+    std::set<std::string> pinned;
+    for (auto &n : m_fbs_model->get_graph_outputs())
+        pinned.insert(n);
+    for (auto &n : m_fbs_model->get_test_outputs_name())
+        pinned.insert(n);
+    for (size_t i = 0; i < m_execution_plan.size(); i++) {
+        auto *conv = dynamic_cast<dl::module::Conv *>(m_execution_plan[i]);
+        if (!conv || conv->quant_type != QUANT_TYPE_SYMM_8BIT || conv->get_group() != 1 || conv->has_fused_lut() ||
+            conv->has_fused_project() || conv->has_fused_residual() || conv->has_fused_gap() || conv->get_pads().size() != 4 ||
+            (conv->get_activation() != Linear && conv->get_activation() != ReLU))
+            continue;
+        const int mid = conv->m_outputs_index[0];
+        const std::string mid_name = m_model_context->get_tensor_name(mid);
+        if (pinned.count(mid_name))
+            continue;
+        int readers = 0;
+        size_t gap_pos = 0;
+        for (size_t j = 0; j < m_execution_plan.size(); j++)
+            for (int in : m_execution_plan[j]->m_inputs_index)
+                if (in == mid) {
+                    readers++;
+                    gap_pos = j;
+                }
+        if (readers != 1 || gap_pos <= i)
+            continue;
+        auto *gap = dynamic_cast<dl::module::GlobalAveragePool *>(m_execution_plan[gap_pos]);
+        TensorBase *filter = m_model_context->get_tensor(conv->m_inputs_index[1]);
+        const std::vector<int> in_shape = m_fbs_model->get_value_info_shape(m_model_context->get_tensor_name(conv->m_inputs_index[0]));
+        if (!gap || gap->quant_type != QUANT_TYPE_SYMM_8BIT || !filter || filter->shape.size() != 4 || in_shape.size() != 4)
+            continue;
+        espdl_hip_conv_desc d = {};
+        d.dtype = ESPDL_HIP_S8;
+        d.batch = 1;
+        d.in_h = in_shape[1];
+        d.in_w = in_shape[2];
+        d.in_c = in_shape[3];
+        d.out_c = filter->shape[3];
+        d.k_h = filter->shape[0];
+        d.k_w = filter->shape[1];
+        d.stride_h = conv->get_strides()[0];
+        d.stride_w = conv->get_strides()[1];
+        d.dil_h = conv->get_dilations()[0];
+        d.dil_w = conv->get_dilations()[1];
+        d.pad_top = conv->get_pads()[0];
+        d.pad_bottom = conv->get_pads()[1];
+        d.pad_left = conv->get_pads()[2];
+        d.pad_right = conv->get_pads()[3];
+        d.group = 1;
+        d.n_shift = 1;
+        if (espdl_hip_conv2d_gap_s8_supported(&d) != 1)
+            continue;
+        conv->fuse_gap(m_fbs_model->get_value_info_exponent(mid_name));
+        conv->m_outputs_index[0] = gap->m_outputs_index[0];
+        delete gap;
+        m_execution_plan.erase(m_execution_plan.begin() + gap_pos);
     }
 }
 

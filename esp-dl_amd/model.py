@@ -194,10 +194,12 @@ def is_registered(op_type):
 class Model:
     """dl::Model handle.  `stream` is a raw hipStream_t value (e.g. torch.cuda.Stream().cuda_stream) or None."""
 
-    def __init__(self, graph, batch, round_mode=0, stream=None, fuse_lut=True, fuse_blocks=True, fuse_add=True):
+    def __init__(self, graph, batch, round_mode=0, stream=None, fuse_lut=True, fuse_blocks=True, fuse_add=True,
+                 fuse_gap=True):
         self.graph = graph  # keep alive: the native model references it
         self.h = lib().espdl_model_create(graph.h, batch, round_mode, ctypes.c_void_p(stream) if stream else None,
-                                          (1 if fuse_lut else 0) | (2 if fuse_blocks else 0) | (4 if fuse_add else 0))
+                                          (1 if fuse_lut else 0) | (2 if fuse_blocks else 0) | (4 if fuse_add else 0) |
+                                          (8 if fuse_gap else 0))
         if not self.h:
             raise EspdlModelError("espdl_model_create failed (see stderr)")
         self.batch = batch

@@ -133,6 +133,18 @@ int espdl_hip_mul_s8(const int32_t out_dims[4], const int64_t in0_strides[4], co
                      const int8_t *in0, const int8_t *in1, int32_t mul_shift, int32_t round_mode, int8_t *out,
                      void *stream);
 
+/* A 1x1 stride-1 module::Conv followed by GlobalAveragePool in one launch (the head of a classification network:
+ * Conv::forward, esp-dl/dl/module/include/dl_module_conv.hpp, then the pooling of
+ * esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54 over the whole image): the convolution's int8 results - at exponent
+ * conv_out_exp, activation applied, exactly what espdl_hip_conv2d would store - are summed per image and filter
+ * inside the kernel and only the pooled tensor out[batch][out_c] (exponent pool_out_exp) is written.  desc as for
+ * espdl_hip_conv2d (ESPDL_HIP_S8, group 1, ESPDL_HIP_LINEAR / _RELU); images of at most 64 pixels, in_c a
+ * multiple of 16 and at least 64, in and filter 16-byte aligned; ESPDL_HIP_ENOTSUP otherwise
+ * (espdl_hip_conv2d_gap_s8_supported answers 1 / 0 for a descriptor). */
+int espdl_hip_conv2d_gap_s8_supported(const espdl_hip_conv_desc *desc);
+int espdl_hip_conv2d_gap_s8(const espdl_hip_conv_desc *desc, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                            const int32_t *shift, int32_t conv_out_exp, int32_t pool_out_exp, int8_t *out, void *stream);
+
 /* GlobalAveragePool over H x W per image and channel: base::avgpool2d_hwc with the filter covering
  * the whole image (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54). out is [batch][1][1][c]. */
 int espdl_hip_global_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t in_exp,

@@ -79,7 +79,8 @@ int espdl_graph_add_test_output(espdl_graph *g, const char *name, const int32_t 
 /* round_mode: 0 half-up (portable C path), 1 half-even.  stream: hipStream_t or NULL (own stream).
  * fuse: bit mask of graph fusions, all exact: 1 folds Conv -> LUT pairs into the conv epilogue, 2 runs
  * depthwise Conv -> 1x1 Conv [-> Add] chains as one kernel, 4 folds the Add behind a dense Conv into the
- * conv epilogue (7 = all).  The graph must outlive the model. */
+ * conv epilogue, 8 runs a 1x1 Conv and the GlobalAveragePool behind it as one kernel (15 = all).  The graph
+ * must outlive the model. */
 espdl_model *espdl_model_create(espdl_graph *g, int32_t batch, int32_t round_mode, void *stream, int32_t fuse);
 void espdl_model_destroy(espdl_model *m);
 /* Module::forward returns void, as in the reference, so a module whose launch is rejected (an operand

@@ -489,6 +489,29 @@ def test_global_avg_pool_s8(oracle):
     np.testing.assert_array_equal(got, oracle.global_avg_pool_s8(x, -4, -4))
 
 
+@pytest.mark.parametrize("hw", [(3, 3), (7, 7), (2, 5)], ids=["3x3", "7x7", "2x5"])
+def test_global_avg_pool_s8_every_sum(oracle, hw):
+    """Every sum an image can have, ties included: the operator is float(sum) * scale rounded in float and THEN
+    given to round(), so a product that rounds to k + 0.5 in float must not be fused with the + 0.5 (sum -18 over
+    3 x 3 at exponents -5 -> -3: the float product is exactly -0.5 and the result 0; a fused multiply-add gives -1)."""
+    announce(f"global_avg_pool_s8 every sum {hw}")
+    m = espdl()
+    h, w = hw
+    area = h * w
+    sums = np.arange(-128 * area, 127 * area + 1)
+    c = (len(sums) + 3) // 4 * 4
+    x = np.zeros((1, area, c), dtype=np.int64)
+    for i, t in enumerate(sums):  # spread the sum over the pixels, every value within int8
+        q, r = divmod(int(t), area)
+        x[0, :, i] = q
+        x[0, :r, i] += 1
+    assert x.min() >= -128 and x.max() <= 127
+    x = x.reshape(1, h, w, c).astype(np.int8)
+    for in_exp, out_exp in ((-5, -3), (-4, -4), (-4, -5), (-6, -3), (-3, -6)):
+        got = to_host(m.global_avg_pool_s8(to_dev(x), in_exp, out_exp))
+        np.testing.assert_array_equal(got, oracle.global_avg_pool_s8(x, in_exp, out_exp), err_msg=f"{in_exp} -> {out_exp}")
+
+
 def test_bad_arguments_are_rejected():
     announce("argument validation")
     m = espdl()
@@ -714,6 +737,44 @@ def test_mbconv_s8_guard_free_builds_ragged_tiles(oracle, case):
     got = m.mbconv_s8(to_dev(x), dev(ex), dev(dw), dev(pj), (3, 3), (stride, stride), (1, 1), pads, (True, True, False),
                       residual=to_dev(res), round_mode=rm_g)
     np.testing.assert_array_equal(to_host(got), cur)
+
+
+# 1x1 convolution followed by GlobalAveragePool in one launch against the two operators of the oracle: the head of
+# MobileNetV2 (7 x 7 x 320 -> 1280), an image of 64 pixels, one of 1 pixel, a filter count that is no multiple of
+# 64, both rounding modes, a linear convolution, shifts outside the short epilogue's range, and a batch large
+# enough for the build that takes two images per workgroup (odd, so that the last workgroup has one).
+GAP_CASES = [
+    ("head_7x7_320_1280", (37, 7, 7, 320), 1280, True, False, 0),
+    ("head_two_images_per_group_odd_batch", (53, 7, 7, 320), 1280, True, False, 0),
+    ("full_8x8_64_96", (5, 8, 8, 64), 96, True, False, 0),
+    ("one_pixel_128_40", (9, 1, 1, 128), 40, False, False, 0),
+    ("half_even_5x5_80_100", (6, 5, 5, 80), 100, True, True, 0),
+    ("general_shifts_3x3_64_64", (4, 3, 3, 64), 64, False, False, 1),
+]
+
+
+@pytest.mark.parametrize("case", GAP_CASES, ids=lambda c: c[0])
+@pytest.mark.parametrize("exps", [(-4, -4), (-5, -3), (-3, -6)], ids=["same_exp", "coarser", "finer"])
+def test_conv2d_gap_s8(oracle, case, exps):
+    announce(f"conv2d_gap_s8 {case[0]} exponents {exps}")
+    name, (n, h, w, cin), cout, relu, half_even, odd_shifts = case
+    m = espdl()
+    rng = np.random.default_rng(0x6A9 + len(name) + exps[1])
+    x = rng_int8(rng, (n, h, w, cin))
+    f = rng_int8(rng, (cout, 1, 1, cin))
+    b = rng.integers(-4096, 4097, size=cout).astype(np.int32)
+    s = (typical_shift(cin) + rng.integers(-2, 3, size=cout)).astype(np.int32)
+    if odd_shifts:
+        s[::5] = 0
+        s[2::9] = 33
+    rm_o = oracle.ROUND_HALF_EVEN if half_even else oracle.ROUND_HALF_UP
+    rm_g = m.capi.ROUND_HALF_EVEN if half_even else m.capi.ROUND_HALF_UP
+    conv = oracle.conv2d_s8(x, f, b, s, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.RELU if relu else oracle.LINEAR, rm_o)
+    want = oracle.global_avg_pool_s8(conv, exps[0], exps[1]).reshape(n, cout)
+    got = m.conv2d_gap_s8(to_dev(x), to_dev(f), to_dev(b), to_dev(s), exps[0], exps[1],
+                          activation=m.capi.RELU if relu else m.capi.LINEAR, round_mode=rm_g)
+    np.testing.assert_array_equal(to_host(got), want)
+    assert len(np.unique(want)) > 3  # not degenerate
 
 
 # A residual operand at another exponent than the block output: the kernels requantize it in registers, as the

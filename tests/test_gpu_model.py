@@ -35,14 +35,16 @@ def _check_all(spec, mdl, want, skip_missing=True):
     return checked
 
 
-def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fuse_blocks=True, fuse_add=True):
+def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fuse_blocks=True, fuse_add=True,
+                fuse_gap=True):
     m, zoo, model, runner = _mods()
     import espdl_oracle as oracle
     rng = np.random.default_rng(seed)
     x = spec.make_input(rng, batch)
     want = runner.run(spec, {spec.inputs[0]: x}, oracle.ROUND_HALF_EVEN if round_mode else oracle.ROUND_HALF_UP)
     g = model.Graph.from_spec(spec)
-    mdl = model.Model(g, batch, round_mode=round_mode, fuse_lut=fuse_lut, fuse_blocks=fuse_blocks, fuse_add=fuse_add)
+    mdl = model.Model(g, batch, round_mode=round_mode, fuse_lut=fuse_lut, fuse_blocks=fuse_blocks, fuse_add=fuse_add,
+                      fuse_gap=fuse_gap)
     mdl.set_input(spec.inputs[0], x)
     if graph:
         assert mdl.enable_graph()
@@ -106,11 +108,11 @@ def test_config3_mobilenetv2_full_resolution(oracle):
     assert mdl.shape(spec.outputs[0]) == [2, 1000]
     logits = want[spec.outputs[0]]
     assert logits.min() < 0 < logits.max() and len(np.unique(logits)) > 50  # not degenerate
-    # every inverted-residual block is one module (the stem inside the first), and the two RequantizeLinear
-    # nodes that only align a residual operand's exponent ride in their block's launch: 17 blocks + head
-    # convolution + GlobalAveragePool + the view + Gemm
+    # every inverted-residual block is one module (the stem inside the first), the two RequantizeLinear nodes
+    # that only align a residual operand's exponent ride in their block's launch, and the head convolution
+    # pools its own output: 17 blocks + head convolution with GlobalAveragePool + the view + Gemm
     n_requant = sum(1 for n in spec.nodes if n["op_type"] == "RequantizeLinear")
-    assert n_requant == 2 and mdl.module_count() == 21
+    assert n_requant == 2 and mdl.module_count() == 20
     mdl.close()
 
 
@@ -384,7 +386,7 @@ def test_mobilenetv2_block_fusion(oracle, fuse_blocks):
     announce(f"model config3 96px fuse_blocks={fuse_blocks}")
     _, zoo, _, _ = _mods()
     spec = zoo.config3_mobilenetv2(resolution=96, num_classes=100)
-    mdl, want, _ = _run_config(spec, 3, 21, fuse_blocks=fuse_blocks, fuse_add=fuse_blocks)
+    mdl, want, _ = _run_config(spec, 3, 21, fuse_blocks=fuse_blocks, fuse_add=fuse_blocks, fuse_gap=fuse_blocks)
     for name in spec.outputs:
         np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
     if fuse_blocks:
