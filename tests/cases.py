@@ -62,3 +62,20 @@ def typical_shift(k_total):
     """A requantization shift that keeps outputs spread over the int8 range for uniform int8 operands."""
     import math
     return max(1, int(round(math.log2(5461 * math.sqrt(k_total) / 40))))
+
+
+def every_sum_image(h, w):
+    """int8 [1, h, w, C]: channel i sums to the i-th of all the sums h * w int8 values can have (C padded to a
+    multiple of 4 with zeros) - for the operators that average in float, where a tie in the rounding of
+    float(sum) * scale is a single value of the sum."""
+    import numpy as np
+    area = h * w
+    sums = np.arange(-128 * area, 127 * area + 1)
+    c = (len(sums) + 3) // 4 * 4
+    x = np.zeros((1, area, c), dtype=np.int64)
+    for i, t in enumerate(sums):
+        q, r = divmod(int(t), area)
+        x[0, :, i] = q
+        x[0, :r, i] += 1
+    assert x.min() >= -128 and x.max() <= 127
+    return x.reshape(1, h, w, c).astype(np.int8)

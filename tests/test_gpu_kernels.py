@@ -5,7 +5,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, rng_int8, typical_shift
+from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, every_sum_image, rng_int8, typical_shift
 from gpu_util import announce, espdl, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
@@ -496,17 +496,7 @@ def test_global_avg_pool_s8_every_sum(oracle, hw):
     3 x 3 at exponents -5 -> -3: the float product is exactly -0.5 and the result 0; a fused multiply-add gives -1)."""
     announce(f"global_avg_pool_s8 every sum {hw}")
     m = espdl()
-    h, w = hw
-    area = h * w
-    sums = np.arange(-128 * area, 127 * area + 1)
-    c = (len(sums) + 3) // 4 * 4
-    x = np.zeros((1, area, c), dtype=np.int64)
-    for i, t in enumerate(sums):  # spread the sum over the pixels, every value within int8
-        q, r = divmod(int(t), area)
-        x[0, :, i] = q
-        x[0, :r, i] += 1
-    assert x.min() >= -128 and x.max() <= 127
-    x = x.reshape(1, h, w, c).astype(np.int8)
+    x = every_sum_image(*hw)
     for in_exp, out_exp in ((-5, -3), (-4, -4), (-4, -5), (-6, -3), (-3, -6)):
         got = to_host(m.global_avg_pool_s8(to_dev(x), in_exp, out_exp))
         np.testing.assert_array_equal(got, oracle.global_avg_pool_s8(x, in_exp, out_exp), err_msg=f"{in_exp} -> {out_exp}")

@@ -129,6 +129,21 @@ def test_reduce_mean_s8(oracle, shape, axes, keepdims, exps):
     np.testing.assert_array_equal(got, oracle.reduce_mean_s8(x, axes, keepdims, exps[0], exps[1]))
 
 
+@pytest.mark.parametrize("hw", [(3, 3), (2, 5)], ids=["3x3", "2x5"])
+def test_avg_pool_and_reduce_mean_s8_every_sum(oracle, hw):
+    """Every sum a window can have, exponent pairs with and without ties: float(sum) * scale is rounded to float
+    before round() adds its 0.5 (no fused multiply-add on the device)."""
+    from cases import every_sum_image
+    announce(f"avg_pool / reduce_mean every sum {hw}")
+    x = every_sum_image(*hw)
+    m = espdl()
+    for exps in ((-5, -3), (-4, -4), (-4, -5), (-6, -3)):
+        got = to_host(m.avg_pool_s8(to_dev(x), hw, (1, 1), (0, 0, 0, 0), exps[0], exps[1]))
+        np.testing.assert_array_equal(got, oracle.avg_pool_s8(x, hw, (1, 1), (0, 0, 0, 0), exps[0], exps[1]), err_msg=str(exps))
+        got = to_host(m.reduce_mean_s8(to_dev(x), [1, 2], True, exps[0], exps[1]))
+        np.testing.assert_array_equal(got, oracle.reduce_mean_s8(x, [1, 2], True, exps[0], exps[1]), err_msg=str(exps))
+
+
 def test_sppf_pool_chain_idempotence():
     """Size-independent property at full batch: three chained 5x5/1 pools equal one 13x13/1 pool, and
     pooling is monotone (output >= input)."""
