@@ -51,7 +51,7 @@ private:
     int m_mid_exponent = 0;      ///< exponent of the (no longer materialized) depthwise output
     int m_lut_in_exponent = 0;   ///< exponent of the conv result that indexes a fused LUT
     int m_project_filter_pos = -1, m_project_bias_pos = -1, m_residual_pos = -1;
-    bool m_residual_requantized = false;
+    int m_residual_shift = 0;
     bool m_has_gap = false;      // a GlobalAveragePool behind this (1x1) convolution runs in its launch
     int m_gap_in_exponent = 0;   // exponent of the tensor the convolution used to write
     int m_own_inputs = 0; ///< inputs of the Conv itself when a plain residual Add was absorbed
@@ -104,12 +104,12 @@ public:
     const std::vector<int> &get_dilations() const { return m_dilations; }
     /// Absorb a following 1x1 Conv (filter / bias indices, activation) and optionally the other
     /// operand of the Add after it.  The caller re-points m_outputs_index at the final tensor.
-    /// `residual_requantized`: the residual operand stands at its own exponent and is brought to
-    /// `project_out_exponent` inside the kernel (the pass absorbed the RequantizeLinear that did it).
+    /// `residual_shift`: the residual operand is requantized by that power of two inside the kernel (the pass
+    /// absorbed the RequantizeLinear that did it: exponent of its input - exponent of its output).
     void fuse_project(int filter_index, int bias_index, activation_type_t act, int mid_exponent, int residual_index,
-                      int project_out_exponent = 0, bool residual_requantized = false)
+                      int project_out_exponent = 0, int residual_shift = 0)
     {
-        m_residual_requantized = residual_requantized && residual_index >= 0;
+        m_residual_shift = residual_index >= 0 ? residual_shift : 0;
         if (residual_index >= 0) {
             m_has_pre_add_exponent = true;
             m_pre_add_exponent = project_out_exponent;
@@ -418,9 +418,8 @@ public:
         d.n_shift_expand = m_has_expand ? (int32_t)s_ex.size() : 1;
         d.n_shift_dw = (int32_t)s_dw.size();
         d.n_shift_project = (int32_t)s_pj.size();
-        // a residual operand at another exponent than the Add's (the fusion pass absorbed the RequantizeLinear
-        // in front of the Add) is requantized inside the kernel
-        d.residual_shift = (residual && m_residual_requantized) ? residual->exponent.get() - pj_out_exponent : 0;
+        // a residual operand whose RequantizeLinear the fusion pass absorbed is requantized inside the kernel
+        d.residual_shift = residual ? m_residual_shift : 0;
         m_fused_kernel = espdl_hip_mbconv_s8_supported(&d);
         espdl_hip_mbconv_weights w = {};
         if (m_has_expand) {

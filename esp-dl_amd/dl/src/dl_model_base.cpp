@@ -399,26 +399,31 @@ void Model::fuse_dw_project()
         }
         const int mid_exp = m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(mid));
         const int pj_out_exp = m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(pj->m_outputs_index[0]));
-        // A RequantizeLinear whose only job is to bring the residual operand to the Add's exponent joins the
-        // launch of a whole block: the kernel requantizes the operand in registers (residual_shift of the
-        // descriptor, which Conv::forward derives from the two exponents).
+        // A RequantizeLinear whose only reader is the Add (the exporter's way of re-scaling the residual operand)
+        // joins the launch of a whole block: the kernel requantizes the operand in registers (residual_shift
+        // of the descriptor = exponent of the node's input - exponent of its output; the Add itself adds raw
+        // values whatever the exponents say, as the reference's does).
         dl::module::Module *rq = nullptr;
+        int rq_shift = 0;
         if (ex && residual >= 0) {
             size_t rq_reader = 0;
             for (size_t j = 0; j < add_pos; j++)
                 if (m_execution_plan[j]->m_outputs_index.size() == 1 && m_execution_plan[j]->m_outputs_index[0] == residual)
                     rq = dynamic_cast<dl::module::RequantizeLinear *>(m_execution_plan[j]);
-            if (rq && (rq->m_inputs_index.size() != 1 || rq->m_inputs_index[0] >= CONTEXT_PARAMETER_OFFSET ||
+            // (exported files give the node its scale and zero point as further, constant inputs)
+            if (rq && (rq->m_inputs_index.empty() || rq->m_inputs_index[0] >= CONTEXT_PARAMETER_OFFSET ||
                        !single_reader(residual, &rq_reader)))
                 rq = nullptr;
             if (rq) {
                 const std::string src_name = m_model_context->get_tensor_name(rq->m_inputs_index[0]);
                 const std::string res_name = m_model_context->get_tensor_name(residual);
-                const int shift = m_fbs_model->has_value_info(src_name) ? m_fbs_model->get_value_info_exponent(src_name) - pj_out_exp : 0;
+                const int shift = m_fbs_model->has_value_info(src_name)
+                    ? m_fbs_model->get_value_info_exponent(src_name) - m_fbs_model->get_value_info_exponent(res_name)
+                    : 0;
                 de.residual_shift = shift;
+                rq_shift = shift;
                 if (!m_fbs_model->has_value_info(src_name) || m_fbs_model->get_value_info_dtype(src_name) != DATA_TYPE_INT8 ||
                     m_fbs_model->get_value_info_dtype(res_name) != DATA_TYPE_INT8 ||
-                    m_fbs_model->get_value_info_exponent(res_name) != pj_out_exp ||
                     m_fbs_model->get_value_info_shape(src_name) != m_fbs_model->get_value_info_shape(res_name) || shift == 0 ||
                     shift < -7 || shift > 7 || espdl_hip_mbconv_s8_preferred(&de) != 1)
                     rq = nullptr;
@@ -427,7 +432,7 @@ void Model::fuse_dw_project()
             }
         }
         dw->fuse_project(pj->m_inputs_index[1], pj->m_inputs_index.size() == 3 ? pj->m_inputs_index[2] : -1,
-                         pj->get_activation(), mid_exp, residual, pj_out_exp, rq != nullptr);
+                         pj->get_activation(), mid_exp, residual, pj_out_exp, rq != nullptr ? rq_shift : 0);
         dw->m_outputs_index[0] = out_index;
         if (ex)
             dw->fuse_expand(ex->m_inputs_index[0], ex->m_inputs_index[1],

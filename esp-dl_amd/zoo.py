@@ -234,12 +234,19 @@ class Builder:
         g.add_node(name, "PRelu", [x, name + ".slope"], [y], quant_type="S8")
         return y
 
-    def requantize(self, x, out_exp, name=None):
+    def requantize(self, x, out_exp, name=None, with_scale_input=False):
+        """with_scale_input: the node carries its scale as a second, constant input, as exported files do (the
+        operator itself works from the two tensors' exponents)."""
         g = self.g
         name = name or self._name("requant")
         y = name + "_out"
         g.add_value(y, g.shape(x), out_exp, g.dtype(x))
-        g.add_node(name, "RequantizeLinear", [x], [y], quant_type="S8")
+        inputs = [x]
+        if with_scale_input:
+            sname = name + ".scale"
+            g.add_init(sname, [1], FLOAT, [2.0 ** out_exp], [0])
+            inputs.append(sname)
+        g.add_node(name, "RequantizeLinear", inputs, [y], quant_type="S8")
         return y
 
     def add(self, a, b, name=None, out_exp=None):
@@ -493,9 +500,12 @@ def config2_mbv2_block(seed=0xE5D2):
 MBV2_TABLE = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]
 
 
-def config3_mobilenetv2(seed=0xE5D3, resolution=224, num_classes=1000, width=1.0):
+def config3_mobilenetv2(seed=0xE5D3, resolution=224, num_classes=1000, width=1.0, relabel_residual=False):
     """MobileNetV2-1.0 as ESP-DL runs it: ReLU fused into Conv (ReLU6 was replaced by ReLU before
-    quantization), project convs Linear, residual Adds, GlobalAveragePool, Flatten, Gemm head."""
+    quantization), project convs Linear, residual Adds, GlobalAveragePool, Flatten, Gemm head.
+    relabel_residual: as in the exported files of the reference, some residual operands pass through a
+    RequantizeLinear (with its scale as a second, constant input) to an exponent that is NOT the project
+    convolution's; the Add sums the stored integers whatever the exponents say."""
     g = GraphSpec("config3_mobilenetv2_%d" % resolution)
     b = Builder(g, seed, per_channel=True, w_exp_range=None)
     x = b.input("input", [1, resolution, resolution, 3], -6)
@@ -514,7 +524,18 @@ def config3_mobilenetv2(seed=0xE5D3, resolution=224, num_classes=1000, width=1.0
             h = b.conv(h, cin * t, k=3, stride=stride, depthwise=True, relu=True, name="b%d_dw" % blk)
             h = b.conv(h, c, k=1, relu=False, name="b%d_project" % blk)
             if stride == 1 and cin == c:
-                h = b.add(skip, h, name="b%d_add" % blk)
+                if relabel_residual and blk % 2 == 0:
+                    # exponent one or two off the project output's, never equal to it
+                    e = g.exponent(h) + (1 if blk % 4 == 0 else -2)
+                    if e == g.exponent(skip):
+                        e += 1
+                    skip = b.requantize(skip, e, name="b%d_skip_requant" % blk, with_scale_input=True)
+                    y = "b%d_add_out" % blk
+                    g.add_value(y, g.shape(h), g.exponent(h))
+                    g.add_node("b%d_add" % blk, "Add", [skip, h], [y], quant_type="S8")
+                    h = y
+                else:
+                    h = b.add(skip, h, name="b%d_add" % blk)
             x = h
             cin = c
     x = b.conv(x, int(1280 * max(1.0, width)), k=1, relu=True, name="head_conv")

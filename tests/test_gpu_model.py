@@ -130,6 +130,24 @@ def test_config3_mobilenetv2_all_intermediates(oracle):
     mdl.close()
 
 
+@pytest.mark.parametrize("round_mode", [0, 1], ids=["half_up", "half_even"])
+def test_mobilenetv2_requantized_residuals_at_other_exponents(oracle, round_mode):
+    """The pattern of the reference's exported MobileNetV2 files: the residual operand goes through a
+    RequantizeLinear (scale as a constant second input) to an exponent that differs from the project convolution's,
+    and the Add sums the stored integers.  Each such node rides in its block's launch (residual_shift = its input
+    exponent - its output exponent); same logits as the node-by-node run of the oracle."""
+    announce(f"model config3 224px with relabelled residual RequantizeLinear, round mode {round_mode}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.config3_mobilenetv2(num_classes=100, relabel_residual=True)
+    n_requant = sum(1 for n in spec.nodes if n["op_type"] == "RequantizeLinear")
+    assert n_requant >= 5
+    mdl, want, _ = _run_config(spec, 2, 23, round_mode=round_mode)
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
+    assert mdl.module_count() == 20  # 17 blocks, head convolution, the view, Gemm: no RequantizeLinear module left
+    mdl.close()
+
+
 def test_config3_half_even(oracle):
     announce("model config3 96px half-even")
     _, zoo, _, _ = _mods()
