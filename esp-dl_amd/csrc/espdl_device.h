@@ -116,6 +116,18 @@ __device__ __forceinline__ v2s pk_mul_sat_i16(v2s a, int m)
 // int16.  A channel has either a right shift (s > 8) or a multiplier (s < 8), never both.  Saturating
 // acc to int16 first and the product to int16 again gives the same high byte as saturating acc * 2^l once:
 // where the first saturation acts (|acc| >= 2^15, l >= 0) the second one does too.
+// Round half to even on an accumulator that already holds v + 2^(s-1) (the round-half-up start value): the two
+// roundings differ only on an exact tie with an odd result, i.e. where the low s bits of the accumulator are zero
+// and bit s is set, and there one less shifts down to the even neighbour.  s = rsh + 8 - lsh (one of the two is
+// zero).  Three instructions per value; the two constants depend on the channel only and are formed once per
+// group of pixel tiles by the compiler.
+__device__ __forceinline__ int half_even_fix(int acc, int lsh, int rsh)
+{
+    const unsigned pow_s = 1u << (rsh + 8 - lsh);
+    const unsigned mask = (pow_s << 1) - 1u;
+    return acc - ((((unsigned)acc) & mask) == pow_s ? 1 : 0);
+}
+
 template <int MODE>
 __device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk, bool he = false)
 {
@@ -131,15 +143,11 @@ __device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const 
     int t[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        const int v = MODE != 0 ? (int)((unsigned)acc[r] << lsh[r]) : acc[r];
+        int a = acc[r];
+        if (MODE == 2 || (MODE == 3 && he))
+            a = half_even_fix(a, lsh[r], rsh[r]);
+        const int v = MODE != 0 ? (int)((unsigned)a << lsh[r]) : a;
         t[r] = v >> rsh[r];
-        if (MODE == 2 || (MODE == 3 && he)) {
-            // t = q * 256 + (top 8 fraction bits); the other fraction bits left with the shift by rsh.
-            // All fraction bits are zero iff putting q back in place gives v again.  Written with rsh
-            // only, so that no further per-channel constant has to live across the pixel loop.
-            const bool tie = (int)((unsigned)(t[r] & ~0xff) << rsh[r]) == v;
-            t[r] -= tie ? (t[r] & 0x100) : 0;
-        }
     }
     // floor_pk holds the lower clamp twice as int16: 0 for ReLU, -32768 (no effect) otherwise
     const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
@@ -159,12 +167,9 @@ __device__ __forceinline__ int pack_fast4_add(const v4i &acc, const v4i &lsh, co
     int t[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        const int v = MODE != 0 ? (int)((unsigned)acc[r] << lsh[r]) : acc[r];
+        const int a = MODE == 2 ? half_even_fix(acc[r], lsh[r], rsh[r]) : acc[r];
+        const int v = MODE != 0 ? (int)((unsigned)a << lsh[r]) : a;
         t[r] = v >> rsh[r];
-        if (MODE == 2) {
-            const bool tie = (int)((unsigned)(t[r] & ~0xff) << rsh[r]) == v;
-            t[r] -= tie ? (t[r] & 0x100) : 0;
-        }
     }
     const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
     const v2s r01 = __builtin_bit_cast(v2s, (int)__builtin_amdgcn_perm(0u, (unsigned)res, 0x010c000cu));
