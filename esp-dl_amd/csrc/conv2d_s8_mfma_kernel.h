@@ -603,7 +603,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
         if (oc < OC) {
             const int s = a.shift[g.n_shift == 1 ? 0 : oc];
             const int b = a.bias != nullptr ? a.bias[oc] : 0;
-            init = fast ? b + (1 << (s - 1)) : b;
+            init = fast ? b + (1 << (s - 1)) - (HE ? 1 : 0) : b; // the half-even form starts one lower
             sh = fast ? max(0, s - 8) : s;
             lsh = fast ? max(0, 8 - s) : 0;
         }
@@ -628,11 +628,11 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_mfma_kernel(const MfmaConv
     w.has_lut = has_lut;
     w.floor_pk = w.relu ? 0 : (int)0x80008000u;
     w.stage_out = a.stage_out != 0;
-    // epilogue mode of pack_fast4: 0 plain (every shift >= 8), 1 with the left shift, 2 the same with
+    // epilogue mode of pack_fast4: 0 plain (every shift >= 8), 1 with the left shift, 5 the same with
     // round-half-even
     if (HE) {
         if (fast)
-            run_sets<BMODE, PT, KSC, true, 2>(a, w, wave, g_first, g_count, seq, px, bc);
+            run_sets<BMODE, PT, KSC, true, 5>(a, w, wave, g_first, g_count, seq, px, bc);
         else
             run_sets<BMODE, PT, KSC, false, 0>(a, w, wave, g_first, g_count, seq, px, bc);
     } else {

@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     const bool fast = __syncthreads_and(ok_local) != 0;
     if (tid < TN) {
         const bool valid = n0 + tid < a.N;
-        cst[0][tid] = (fast && valid) ? my_b + (1 << (my_s - 1)) : my_b;
+        cst[0][tid] = (fast && valid) ? my_b + (1 << (my_s - 1)) - (half_even ? 1 : 0) : my_b; // mode 5 starts one lower
         cst[1][tid] = fast ? max(0, my_s - 8) : my_s;
         cst[2][tid] = fast ? max(0, 8 - my_s) : 0;
     }
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
 
     // epilogue: lane (col, quad) holds, per pixel tile and group, filters 64*g + 16*quad + [0, 16)
     const int floor_pk = relu ? 0 : (int)0x80008000u;
-    // one straight-line copy per rounding mode (pack_fast4 mode 1: half up, 2: half even)
+    // one straight-line copy per rounding mode (pack_fast4 mode 1: half up, 5: half even)
     auto epilogue = [&](auto mode) {
     #pragma unroll
         for (int c = 0; c < PT; c++) {
@@ -288,7 +288,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
         }
     };
     if (half_even)
-        epilogue(std::integral_constant<int, 2>{});
+        epilogue(std::integral_constant<int, 5>{});
     else
         epilogue(std::integral_constant<int, 1>{});
     if constexpr (GAP) {

@@ -418,7 +418,7 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
     const bool use_lsh = __syncthreads_or(lsh_local) != 0;
     {
         if (tid < cw) {
-            reinterpret_cast<int *>(smem + a.off_init)[tid] = fast ? my_b + (1 << (my_s - 1)) : my_b;
+            reinterpret_cast<int *>(smem + a.off_init)[tid] = fast ? my_b + (1 << (my_s - 1)) - (HE ? 1 : 0) : my_b; // half-even forms start one lower
             reinterpret_cast<int *>(smem + a.off_ss)[tid] = fast ? max(0, my_s - 8) : my_s;
             reinterpret_cast<int *>(smem + a.off_ls)[tid] = fast ? max(0, 8 - my_s) : 0;
         }
@@ -481,7 +481,7 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
         fast_p = __syncthreads_and(okp) != 0;
         int *cp = reinterpret_cast<int *>(smem + a.off_cp);
         if (tid < ocp) {
-            cp[tid] = (fast_p && tid < pj.out_c) ? pb + (1 << (ps - 1)) : pb;
+            cp[tid] = (fast_p && tid < pj.out_c) ? pb + (1 << (ps - 1)) - (HE ? 1 : 0) : pb;
             cp[ocp + tid] = fast_p ? max(0, ps - 8) : ps;
             cp[2 * ocp + tid] = fast_p ? max(0, 8 - ps) : 0;
         }
@@ -518,7 +518,7 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
         fast_e = __syncthreads_and(oke) != 0;
         int *ce = reinterpret_cast<int *>(smem + a.off_ce);
         if (tid < cw) {
-            ce[tid] = fast_e ? eb + (1 << (es - 1)) : eb;
+            ce[tid] = fast_e ? eb + (1 << (es - 1)) - (HE ? 1 : 0) : eb;
             ce[cw + tid] = fast_e ? max(0, es - 8) : es;
             ce[2 * cw + tid] = fast_e ? max(0, 8 - es) : 0;
         }
@@ -564,18 +564,18 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
             const int py0 = u_cur.y0 * g.stride_h - g.pad_top, px0 = u_cur.x0 * g.stride_w - g.pad_left;
             const bool interior = py0 >= 0 && px0 >= 0 && py0 + a.ph <= g.in_h && px0 + a.pw <= g.in_w;
             if (fast_e && interior)
-                dw_expand<HE ? 2 : 1, true>(a, smem, wave, lane, u_cur, floor_e);
+                dw_expand<HE ? 5 : 1, true>(a, smem, wave, lane, u_cur, floor_e);
             else if (fast_e)
-                dw_expand<HE ? 2 : 1, false>(a, smem, wave, lane, u_cur, floor_e);
+                dw_expand<HE ? 5 : 1, false>(a, smem, wave, lane, u_cur, floor_e);
             else
                 dw_expand<-1, false>(a, smem, wave, lane, u_cur, floor_e);
             __syncthreads();
         }
 
-        // epilogue mode of pack_fast4: 0 plain (every shift >= 8), 1 with the left shift, 2 the same with
+        // epilogue mode of pack_fast4: 0 plain (every shift >= 8), 1 with the left shift, 5 the same with
         // round-half-even
         if (fast && HE)
-            dw_compute<true, 2>(a, smem, wave, lane, tapoff, floor_pk);
+            dw_compute<true, 5>(a, smem, wave, lane, tapoff, floor_pk);
         else if (fast && !use_lsh)
             dw_compute<true, 0>(a, smem, wave, lane, tapoff, floor_pk);
         else if (fast)
@@ -608,7 +608,7 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
                 int word;
                 if (fast_p) {
                     const v4i ls = *reinterpret_cast<const v4i *>(cp + 2 * ocp + c);
-                    word = pack_fast4<HE ? 2 : 1>(r, ls, ss, floor_p);
+                    word = pack_fast4<HE ? 5 : 1>(r, ls, ss, floor_p);
                 } else {
                     int q[4];
 #pragma unroll

@@ -160,7 +160,7 @@ __device__ __forceinline__ void dw_block(const DwMfmaArgs &a, unsigned char *sme
     for (int c = tid; c < 16 * NT; c += kThreads) {
         const int s = a.shift[g.n_shift == 1 ? 0 : cb + c];
         const int bv = a.bias != nullptr ? a.bias[cb + c] : 0;
-        init_l[c] = fast ? bv + (1 << (s - 1)) : bv;
+        init_l[c] = fast ? bv + (1 << (s - 1)) - (half_even ? 1 : 0) : bv; // pack_fast4<5> starts one lower
         shift_l[c] = fast ? max(0, s - 8) : s;
         lsh_l[c] = fast ? max(0, 8 - s) : 0;
     }
@@ -212,7 +212,7 @@ __device__ __forceinline__ void dw_block(const DwMfmaArgs &a, unsigned char *sme
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 if (fast) {
-                    words[t] = half_even ? pack_fast4<2>(acc[t], ls[t], ss[t], floor_pk) : pack_fast4<1>(acc[t], ls[t], ss[t], floor_pk);
+                    words[t] = half_even ? pack_fast4<5>(acc[t], ls[t], ss[t], floor_pk) : pack_fast4<1>(acc[t], ls[t], ss[t], floor_pk);
                 } else {
                     int q[4];
 #pragma unroll

@@ -95,13 +95,7 @@ typedef short v2s __attribute__((ext_vector_type(2)));
 // result q sits in bits 8.. of t; v_cvt_pk_i16_i32 saturates t to int16, which saturates q to int8
 // in the high byte; ReLU is one packed max on the int16 pairs; v_perm_b32 gathers the four high bytes.
 // MODE 0: every shift is at least 8, round half up.  MODE 1: some shift is below 8, so the value is
-// first shifted left by max(0, 8-s).  MODE 2: as 1 with round-half-even.  MODE 3: as 1, half-even
-// when `he` is set (a run-time choice, for kernels whose register budget rules out one more
-// compiled copy of their main loop).  Half-up and half-even
-// differ only at exact ties, where half-up gives q + 1 and half-even the even one of q, q + 1;
-// acc = value + 2^(s-1) is a tie iff its low s bits are zero, so the half-even result is the half-up
-// result minus one when that holds and the half-up result is odd (the rule of
-// esp-dl/dl/tool/src/dl_tool.cpp:95-119, stated on acc instead of the value).
+// first shifted left by max(0, 8-s).  MODES 4, 5 and 6 are described at pack_fast4.
 // Saturating packed multiply of two int16 by two int16 (v_pk_mad_i16 with the clamp bit: the products are
 // formed exactly and saturated to int16).
 __device__ __forceinline__ v2s pk_mul_sat_i16(v2s a, int m)
@@ -111,25 +105,26 @@ __device__ __forceinline__ v2s pk_mul_sat_i16(v2s a, int m)
     return __builtin_bit_cast(v2s, d);
 }
 
+// Round half to even on an accumulator that holds v + 2^(s-1) - 1, one less than the round-half-up start value:
+// adding bit s of that accumulator gives the value whose arithmetic shift by s is the half-even result (the rule
+// of esp-dl/dl/tool/src/dl_tool.cpp:95-119).  With f the low s bits of v and q the bits above: if f <= 2^(s-1)
+// the sum f + 2^(s-1) - 1 does not carry, bit s of the accumulator is the parity of q, and adding it carries into
+// bit s exactly when f = 2^(s-1) and q is odd; if f > 2^(s-1) the sum has carried already and one more cannot
+// carry again.  Two instructions per value (v_bfe_u32, v_add).
+__device__ __forceinline__ int half_even_add(int acc, int s)
+{
+    return acc + (int)__builtin_amdgcn_ubfe((unsigned)acc, (unsigned)s, 1u);
+}
+
 // MODE 4 is MODE 1 with the left shifts moved behind the saturating convert, two values per instruction:
 // lsh[0] and lsh[1] hold the multipliers 2^max(0, 8-s) of the channel pairs (0, 1) and (2, 3) as packed
 // int16.  A channel has either a right shift (s > 8) or a multiplier (s < 8), never both.  Saturating
 // acc to int16 first and the product to int16 again gives the same high byte as saturating acc * 2^l once:
 // where the first saturation acts (|acc| >= 2^15, l >= 0) the second one does too.
-// Round half to even on an accumulator that already holds v + 2^(s-1) (the round-half-up start value): the two
-// roundings differ only on an exact tie with an odd result, i.e. where the low s bits of the accumulator are zero
-// and bit s is set, and there one less shifts down to the even neighbour.  s = rsh + 8 - lsh (one of the two is
-// zero).  Three instructions per value; the two constants depend on the channel only and are formed once per
-// group of pixel tiles by the compiler.
-__device__ __forceinline__ int half_even_fix(int acc, int lsh, int rsh)
-{
-    const unsigned pow_s = 1u << (rsh + 8 - lsh);
-    const unsigned mask = (pow_s << 1) - 1u;
-    return acc - ((((unsigned)acc) & mask) == pow_s ? 1 : 0);
-}
-
+// MODE 5: half-even for accumulators that hold bias + 2^(s-1) - 1 (half_even_add), with the left shift.
+// MODE 6: the same where every shift is at least 8.
 template <int MODE>
-__device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk, bool he = false)
+__device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk)
 {
     if constexpr (MODE == 4) {
         const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
@@ -144,9 +139,11 @@ __device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const 
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         int a = acc[r];
-        if (MODE == 2 || (MODE == 3 && he))
-            a = half_even_fix(a, lsh[r], rsh[r]);
-        const int v = MODE != 0 ? (int)((unsigned)a << lsh[r]) : a;
+        if (MODE == 5)
+            a = half_even_add(a, rsh[r] + 8 - lsh[r]);
+        if (MODE == 6)
+            a = half_even_add(a, rsh[r] + 8);
+        const int v = (MODE != 0 && MODE != 6) ? (int)((unsigned)a << lsh[r]) : a;
         t[r] = v >> rsh[r];
     }
     // floor_pk holds the lower clamp twice as int16: 0 for ReLU, -32768 (no effect) otherwise
@@ -167,8 +164,12 @@ __device__ __forceinline__ int pack_fast4_add(const v4i &acc, const v4i &lsh, co
     int t[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        const int a = MODE == 2 ? half_even_fix(acc[r], lsh[r], rsh[r]) : acc[r];
-        const int v = MODE != 0 ? (int)((unsigned)a << lsh[r]) : a;
+        int a = acc[r];
+        if (MODE == 5)
+            a = half_even_add(a, rsh[r] + 8 - lsh[r]);
+        if (MODE == 6)
+            a = half_even_add(a, rsh[r] + 8);
+        const int v = (MODE != 0 && MODE != 6) ? (int)((unsigned)a << lsh[r]) : a;
         t[r] = v >> rsh[r];
     }
     const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);

@@ -91,7 +91,7 @@ __device__ __forceinline__ int mb_pack_r(const v4i &acc, const v4i &ss, const v4
                                          bool half_even, int floor_pk)
 {
     if (fast)
-        return half_even ? pack_fast4<2>(acc, ls, ss, floor_pk) : pack_fast4<1>(acc, ls, ss, floor_pk);
+        return half_even ? pack_fast4<5>(acc, ls, ss, floor_pk) : pack_fast4<1>(acc, ls, ss, floor_pk);
     int q[4];
 #pragma unroll
     for (int r = 0; r < 4; r++)
@@ -109,9 +109,10 @@ __device__ __forceinline__ bool mb_short_ok(int s, int bias, long long mac_bound
     return (start < 0 ? -start : start) + mac_bound < (1ll << (31 - max(0, 8 - s)));
 }
 
-__device__ __forceinline__ void mb_put_consts(int *cst, int stride, int c, bool valid, bool fast, int s, int b)
+// The half-even short form (pack_fast4<5>) starts one below the half-up rounding constant.
+__device__ __forceinline__ void mb_put_consts(int *cst, int stride, int c, bool valid, bool fast, int s, int b, bool half_even)
 {
-    cst[c] = (fast && valid) ? b + (1 << (s - 1)) : b;
+    cst[c] = (fast && valid) ? b + (1 << (s - 1)) - (half_even ? 1 : 0) : b;
     cst[stride + c] = fast ? max(0, s - 8) : s;
     cst[2 * stride + c] = fast ? max(0, 8 - s) : 0;
 }
@@ -192,11 +193,11 @@ __global__ __launch_bounds__(kThreads) void mbconv_s8_fused_kernel(const MbArgs 
         fast_p = __syncthreads_or(bad & 4) == 0;
         if (tid < ec_pad) {
             if (a.has_expand)
-                mb_put_consts(cst_e, ec_pad, tid, tid < p.exp_c, fast_e, s_e, b_e);
-            mb_put_consts(cst_d, ec_pad, tid, tid < p.exp_c, fast_d, s_d, b_d);
+                mb_put_consts(cst_e, ec_pad, tid, tid < p.exp_c, fast_e, s_e, b_e, half_even);
+            mb_put_consts(cst_d, ec_pad, tid, tid < p.exp_c, fast_d, s_d, b_d, half_even);
         }
         if (tid < oc_pad)
-            mb_put_consts(cst_p, oc_pad, tid, tid < p.out_c, fast_p, s_p, b_p);
+            mb_put_consts(cst_p, oc_pad, tid, tid < p.out_c, fast_p, s_p, b_p, half_even);
     }
     // the depthwise stage reads from E (stride kEs) or, without expand, from the input patch (stride xs)
     const int dw_stride = a.has_expand ? kEs : a.xs;

@@ -186,8 +186,10 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
                     expand_chunk<0, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
                 else if (!HE && ce.mode == 1)
                     expand_chunk<1, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
-                else if (HE && ce.mode == 2)
-                    expand_chunk<2, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                else if (HE && ce.mode == 6)
+                    expand_chunk<6, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                else if (HE && ce.mode == 5)
+                    expand_chunk<5, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
                 else
                     expand_chunk<-1, NXPT, EXACT, KSE>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             }
@@ -205,8 +207,10 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
                     depthwise_chunk<0, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
                 else if (!HE && cd.mode == 1)
                     depthwise_chunk<1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
-                else if (HE && cd.mode == 2)
-                    depthwise_chunk<2, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
+                else if (HE && cd.mode == 6)
+                    depthwise_chunk<6, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
+                else if (HE && cd.mode == 5)
+                    depthwise_chunk<5, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
                 else
                     depthwise_chunk<-1, PT, S, EXACT>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, row_bytes, write_ok);
             }
@@ -377,8 +381,10 @@ __global__ __launch_bounds__(kGroupThreads, (KSE == 1 && EXACT) ? 4 : 2) void mb
             };
             if (cp.mode == -1)
                 with_mode(std::integral_constant<int, -1>{});
+            else if (HE && cp.mode == 6)
+                with_mode(std::integral_constant<int, 6>{});
             else if constexpr (HE)
-                with_mode(std::integral_constant<int, 2>{});
+                with_mode(std::integral_constant<int, 5>{});
             else if (cp.mode == 0)
                 with_mode(std::integral_constant<int, 0>{});
             else

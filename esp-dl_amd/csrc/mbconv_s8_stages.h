@@ -84,15 +84,15 @@ __device__ __forceinline__ bool short_ok(int s, int bias, unsigned mac_bound)
 }
 
 // Requantization constants of four consecutive channels of one stage, and which epilogue the whole
-// wavefront takes for them: pack_fast4 mode 0 (every shift >= 8), 1 (some shift below 8), 2 (half-even),
-// or -1 for the general shift_and_round restatement (a shift outside 1..31, or an accumulator that could
+// wavefront takes for them: pack_fast4 mode 0 (every shift >= 8), 1 (some shift below 8), 6 and 5 (the
+// same two in half-even), or -1 for the general shift_and_round restatement (a shift outside 1..31, or an accumulator that could
 // overflow the short form).
 struct StageConsts {
     v4i init, rsh, lsh;
     int mode;
 };
 
-// Per-channel constants of a stage live in LDS as three rows of n_ch int32: [bias + rounding constant |
+// Per-channel constants of a stage live in LDS as three rows of n_ch int32: [bias + rounding constant (2^(s-1), one less in half-even) |
 // right shift | left shift] in the form the short epilogue wants, or [bias | shift | 0] for the general one.
 // build_stage_tables fills the tables of the three stages (expand and depthwise: the same n_ch channels;
 // project: see below) with ONE memory round trip and ONE workgroup vote, which is also the barrier after which the tables are complete: every lane writes
@@ -117,6 +117,7 @@ __device__ __forceinline__ void build_stage_tables(const StageTablesArgs &t, boo
 {
     const unsigned step_e = t.n_s_e == 1 ? 0u : 1u, step_d = t.n_s_d == 1 ? 0u : 1u, step_p = t.n_s_p == 1 ? 0u : 1u;
     const int n_ch = t.n_ch;
+    const int he1 = half_even ? 1 : 0; // the half-even forms start one below the half-up rounding constant
     // bits 0 / 1 / 2: expand / depthwise / project needs the general form; bits 3 / 4 / 5: a shift below 8
     int flags = 0;
     for (int c = tid; c < n_ch; c += nthreads) {
@@ -129,10 +130,10 @@ __device__ __forceinline__ void build_stage_tables(const StageTablesArgs &t, boo
         flags |= se < 8 ? 8 : 0;
         flags |= sd < 8 ? 16 : 0;
         const int se1 = min(max(se, 1), 31), sd1 = min(max(sd, 1), 31); // defined shifts where the form does not apply
-        t.tab_e[c] = be + (1 << (se1 - 1));
+        t.tab_e[c] = be + (1 << (se1 - 1)) - he1;
         t.tab_e[n_ch + c] = max(0, se - 8);
         t.tab_e[2 * n_ch + c] = max(0, 8 - se);
-        t.tab_d[c] = bd + (1 << (sd1 - 1));
+        t.tab_d[c] = bd + (1 << (sd1 - 1)) - he1;
         t.tab_d[n_ch + c] = max(0, sd - 8);
         t.tab_d[2 * n_ch + c] = max(0, 8 - sd);
     }
@@ -145,7 +146,7 @@ __device__ __forceinline__ void build_stage_tables(const StageTablesArgs &t, boo
         flags |= short_ok(sp, bp, t.bound_p) ? 0 : 4;
         flags |= sp < 8 ? 32 : 0;
         const int sp1 = min(max(sp, 1), 31);
-        t.tab_p[c] = bp + (1 << (sp1 - 1));
+        t.tab_p[c] = bp + (1 << (sp1 - 1)) - he1;
         t.tab_p[t.n_pad_p + c] = max(0, sp - 8);
         t.tab_p[2 * t.n_pad_p + c] = max(0, 8 - sp);
     }
@@ -184,9 +185,9 @@ __device__ __forceinline__ void build_stage_tables(const StageTablesArgs &t, boo
         }
         __syncthreads();
     }
-    mode_e = (all & 1) ? -1 : (half_even ? 2 : ((all & 8) ? 1 : 0));
-    mode_d = (all & 2) ? -1 : (half_even ? 2 : ((all & 16) ? 1 : 0));
-    mode_p = (all & 4) ? -1 : (half_even ? 2 : ((all & 32) ? 1 : 0));
+    mode_e = (all & 1) ? -1 : (half_even ? ((all & 8) ? 5 : 6) : ((all & 8) ? 1 : 0));
+    mode_d = (all & 2) ? -1 : (half_even ? ((all & 16) ? 5 : 6) : ((all & 16) ? 1 : 0));
+    mode_p = (all & 4) ? -1 : (half_even ? ((all & 32) ? 5 : 6) : ((all & 32) ? 1 : 0));
 }
 
 // MULTIPLIERS: in mode 1 turn the left-shift counts into the packed multipliers of pack_fast4<4>
@@ -198,7 +199,7 @@ __device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch
     c.init = *reinterpret_cast<const v4i *>(tab + ch);
     c.rsh = *reinterpret_cast<const v4i *>(tab + n_ch + ch);
     c.lsh = v4i{0, 0, 0, 0};
-    if (mode == 1 || mode == 2)
+    if (mode == 1 || mode == 5)
         c.lsh = *reinterpret_cast<const v4i *>(tab + 2 * n_ch + ch);
     if (MULTIPLIERS && mode == 1) // the multiplier form of pack_fast4<4>: 2^lsh of the channel pairs as packed int16
         c.lsh = v4i{(1 << c.lsh[0]) | (65536 << c.lsh[1]), (1 << c.lsh[2]) | (65536 << c.lsh[3]), 0, 0};

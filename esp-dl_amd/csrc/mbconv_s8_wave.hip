@@ -439,8 +439,10 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
                 expand_chunk<0, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else if (!HE && ce.mode == 1)
                 expand_chunk<1, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
-            else if (HE && ce.mode == 2)
-                expand_chunk<2, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+            else if (HE && ce.mode == 6)
+                expand_chunk<6, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+            else if (HE && ce.mode == 5)
+                expand_chunk<5, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
             else
                 expand_chunk<-1, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
         }
@@ -460,8 +462,10 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
                 depthwise_chunk<0, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
             else if (!HE && cd.mode == 1)
                 depthwise_chunk<1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
-            else if (HE && cd.mode == 2)
-                depthwise_chunk<2, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+            else if (HE && cd.mode == 6)
+                depthwise_chunk<6, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+            else if (HE && cd.mode == 5)
+                depthwise_chunk<5, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
             else
                 depthwise_chunk<-1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
         }
@@ -534,8 +538,10 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
     };
     if (mode_p == -1)
         with_mode(std::integral_constant<int, -1>{});
+    else if (HE && mode_p == 6)
+        with_mode(std::integral_constant<int, 6>{});
     else if constexpr (HE)
-        with_mode(std::integral_constant<int, 2>{});
+        with_mode(std::integral_constant<int, 5>{});
     else if (mode_p == 0)
         with_mode(std::integral_constant<int, 0>{});
     else
