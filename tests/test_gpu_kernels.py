@@ -798,6 +798,40 @@ def test_mbconv_s8_requantized_residual(oracle, shape, shift):
     np.testing.assert_array_equal(to_host(got), want)
 
 
+# Half-even in the block kernels: small operands and small shifts put exact ties in a large share of the outputs of
+# every stage; shifts below 8 take the epilogue form with the left shift, a range across 8 mixes both in one stage.
+@pytest.mark.parametrize("shape", [(3, 28, 28, 32, 192, 32), (3, 14, 14, 64, 384, 64), (2, 7, 7, 160, 960, 160)],
+                         ids=["wave_28x28", "group_14x14", "group_7x7"])
+@pytest.mark.parametrize("shift_lo,shift_hi", [(1, 3), (2, 9)])
+def test_mbconv_s8_half_even_ties(oracle, shape, shift_lo, shift_hi):
+    announce(f"mbconv_s8 half-even ties {shape} shifts {shift_lo}..{shift_hi}")
+    n, h, w, cin, ce, cout = shape
+    m = espdl()
+    rng = np.random.default_rng(0x71E5 + shift_lo + h)
+
+    def stage(oc, fshape):
+        return (rng.integers(-2, 3, size=fshape).astype(np.int8), rng.integers(-8, 9, size=oc).astype(np.int32),
+                rng.integers(shift_lo, shift_hi + 1, size=oc).astype(np.int32))
+
+    x = rng.integers(-6, 7, size=(n, h, w, cin)).astype(np.int8)
+    ex, dw, pj = stage(ce, (ce, 1, 1, cin)), stage(ce, (3, 3, ce)), stage(cout, (cout, 1, 1, ce))
+    res = rng.integers(-6, 7, size=(n, h, w, cout)).astype(np.int8)
+    pads = (1, 1, 1, 1)
+    dev = lambda t: tuple(to_dev(a) for a in t)  # noqa: E731
+    results = {}
+    for name, rm_o, rm_g in (("even", oracle.ROUND_HALF_EVEN, m.capi.ROUND_HALF_EVEN),
+                             ("up", oracle.ROUND_HALF_UP, m.capi.ROUND_HALF_UP)):
+        cur = oracle.conv2d_s8(x, ex[0], ex[1], ex[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.RELU, rm_o)
+        cur = oracle.depthwise_s8(cur, dw[0], dw[1], dw[2], (3, 3), (1, 1), (1, 1), pads, oracle.RELU, rm_o)
+        cur = oracle.conv2d_s8(cur, pj[0], pj[1], pj[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.LINEAR, rm_o)
+        want = oracle.add_s8(cur, res)
+        got = m.mbconv_s8(to_dev(x), dev(ex), dev(dw), dev(pj), (3, 3), (1, 1), (1, 1), pads, (True, True, False),
+                          residual=to_dev(res), round_mode=rm_g)
+        np.testing.assert_array_equal(to_host(got), want)
+        results[name] = want
+    assert (results["even"] != results["up"]).mean() > 0.01  # the two modes really differ on this input
+
+
 def _block_desc(m, batch, hw, cin, ce, cout, stride, half_even=False):
     d = m.capi.MbconvDesc()
     d.batch, d.in_h, d.in_w, d.in_c, d.exp_c, d.out_c, d.has_expand = batch, hw, hw, cin, ce, cout, 1
