@@ -213,6 +213,16 @@ public:
                 m_perm[i] += dims;
             out.push_back(input_shapes[0][m_perm[i]]);
         }
+        // a permutation that keeps the axes longer than 1 in their order moves no byte (the [N, 1, 1, C] -> [N, C, 1, 1]
+        // in front of an exported classifier): the output is then a view of the input, as with Reshape
+        int last = -1;
+        bool view = true;
+        for (int i = 0; i < dims; i++)
+            if (input_shapes[0][m_perm[i]] > 1) {
+                view = view && m_perm[i] > last;
+                last = m_perm[i];
+            }
+        inplace = view ? MODULE_INPLACE_UNCHANGED_BUFFER : MODULE_NON_INPLACE;
         return {out};
     }
     void forward(ModelContext *context, runtime_mode_t mode = RUNTIME_MODE_AUTO)
@@ -224,6 +234,8 @@ public:
             DL_LOGE("Transpose", "%s: needs device tensors of one type", name.c_str());
             return;
         }
+        if (inplace == MODULE_INPLACE_UNCHANGED_BUFFER && input->data == output->data)
+            return; // a view
         const int rc = espdl_hip_transpose(input->data, input->shape.data(), (int32_t)input->shape.size(), m_perm.data(),
                                            (int32_t)m_perm.size(), (int32_t)input->get_dtype_bytes(), output->data,
                                            context->stream);
