@@ -305,6 +305,80 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     }
 }
 
+// The same product for a handful of rows (a classifier Gemm over one batch: 256 x 1280 x 1000): the tiled kernel
+// above would run on a few dozen compute units and spend its time in twenty barrier-separated k steps.  Here a
+// wavefront owns a 16-row x 16-filter tile for the whole reduction and reads both operands straight from
+// global memory / L2 in the MFMA operand layout (lane (col, quad): 16 bytes of row col at k = 64 step + 16 quad),
+// G k steps per batch of loads, the next batch in flight under the current one's MFMAs; a workgroup is four row
+// tiles under one filter tile, so N / 16 x M / 64 workgroups fill the device and a workgroup's time is a few memory
+// round trips.  K must be a multiple of 64.  The epilogue is the general one (any shift, either rounding).
+template <int G>
+__global__ __launch_bounds__(kThreads) void conv2d_s8_rows_kernel(const PwArgs a)
+{
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 15, quad = lane >> 4;
+    const long long m0 = ((long long)blockIdx.x * 4 + wave) * 16;
+    const int n0 = blockIdx.y * 16;
+    if (m0 >= a.M) // uniform per wavefront; the kernel has no barrier
+        return;
+    const long long row = min(m0 + col, a.M - 1);
+    const int flt = min(n0 + col, a.N - 1);
+    const v4i *pa = reinterpret_cast<const v4i *>(a.w + (long long)flt * a.K + 16 * quad);
+    const v4i *pb = reinterpret_cast<const v4i *>(a.in + row * a.K + 16 * quad);
+    v4i ca[G], cb[G], na[G], nb[G];
+#pragma unroll
+    for (int i = 0; i < G; i++) {
+        const int ks = min(i, a.ksteps - 1);
+        ca[i] = pa[4 * ks];
+        cb[i] = pb[4 * ks];
+    }
+    v4i acc = {0, 0, 0, 0};
+    for (int g0 = 0; g0 < a.ksteps; g0 += G) {
+        const bool more = g0 + G < a.ksteps; // uniform
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < G; i++) {
+                const int ks = min(g0 + G + i, a.ksteps - 1);
+                na[i] = pa[4 * ks];
+                nb[i] = pb[4 * ks];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < G; i++)
+            if (g0 + i < a.ksteps) // uniform
+                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ca[i], cb[i], acc, 0, 0, 0);
+        if (more) {
+#pragma unroll
+            for (int i = 0; i < G; i++) {
+                ca[i] = na[i];
+                cb[i] = nb[i];
+            }
+        }
+    }
+    // lane (col, quad) holds filters n0 + 4 quad + [0, 4) of row m0 + col
+    const long long m = m0 + col;
+    const int n = n0 + 4 * quad;
+    const bool relu = a.relu != 0, half_even = a.half_even != 0;
+    int q[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const int nn = min(n + r, a.N - 1);
+        const int b = a.bias != nullptr ? a.bias[nn] : 0;
+        q[r] = requant_s8(acc[r] + b, a.shift[a.n_shift == 1 ? 0 : nn], relu, half_even);
+    }
+    if (m >= a.M || n >= a.N)
+        return;
+    int8_t *dst = a.out + m * a.N + n;
+    if (a.out_vec >= 4 && n + 4 <= a.N) {
+        *reinterpret_cast<int *>(dst) = pack4_s8(q[0], q[1], q[2], q[3]);
+    } else {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+            if (n + r < a.N)
+                dst[r] = (int8_t)q[r];
+    }
+}
+
 } // namespace
 
 // Flat pointwise geometry with 16-byte aligned rows; worth it when a workgroup of the implicit-GEMM
@@ -351,6 +425,12 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
     const unsigned gy = (unsigned)((a.N + 63) / 64);
     const long long tiles128 = (a.M + 127) / 128;
     const int cus = cu_count > 0 ? cu_count : 256;
+    // fewer 64 x 64 tiles than compute units: one wavefront per 16 x 16 tile, operands straight from global memory
+    if (lut == nullptr && residual == nullptr && (a.K & 63) == 0 && (a.M + 63) / 64 * gy < cus) {
+        hipLaunchKernelGGL((conv2d_s8_rows_kernel<10>), dim3((unsigned)((a.M + 63) / 64), (unsigned)((a.N + 15) / 16)),
+                           dim3(kThreads), 0, stream, a);
+        return hipGetLastError();
+    }
     if (tiles128 * gy * 2 < 3ll * cus)
         hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1>), dim3((unsigned)((a.M + 63) / 64), gy), dim3(kThreads), 0, stream, a);
     else

@@ -195,6 +195,28 @@ def test_gemm_s8(oracle, m, k, n, has_bias, relu):
     np.testing.assert_array_equal(got, want)
 
 
+# Products with so few rows that the tiled kernels would leave most of the device idle go to a kernel with one
+# wavefront per 16 x 16 tile: ragged row and filter counts, byte stores (N not a multiple of 4), one shift for all
+# filters, shifts outside 1..31, both roundings.
+@pytest.mark.parametrize("m,k,n", [(256, 1280, 1000), (1, 1280, 1000), (70, 64, 37), (33, 576, 129), (512, 128, 32)])
+@pytest.mark.parametrize("variant", ["per_channel", "per_tensor", "half_even", "wide_shifts"])
+def test_conv2d_s8_few_rows(oracle, m, k, n, variant):
+    announce(f"conv2d_s8 few rows M={m} K={k} N={n} {variant}")
+    rng = np.random.default_rng(0xF3 + m + n)
+    x = rng_int8(rng, (m, 1, 1, k))
+    f = rng_int8(rng, (n, 1, 1, k))
+    bias = rng.integers(-4096, 4097, size=n).astype(np.int32)
+    if variant == "per_tensor":
+        shift = np.full(1, typical_shift(k), np.int32)
+    elif variant == "wide_shifts":
+        shift = rng.choice(np.array([-2, 0, 1, 5, typical_shift(k), 20, 31, 33], np.int32), size=n)
+    else:
+        shift = (typical_shift(k) + rng.integers(-2, 3, size=n)).astype(np.int32)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), variant == "per_tensor",
+                             half_even=variant == "half_even")
+    np.testing.assert_array_equal(got, want)
+
+
 def test_gemm_reference_known_answers_on_gpu():
     """The reference-held Gemm vectors, straight through the C ABI."""
     import json
