@@ -54,7 +54,6 @@ struct PwArgs {
 template <int NG, int PT, bool GAP = false>
 __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs a)
 {
-    static_assert(!GAP || NG == 1, "the pooled form works on 64 filters per workgroup");
     constexpr int TN = 64 * NG;
     constexpr int kTileM = 64 * PT; // pixels per workgroup, 16 * PT per wavefront
     constexpr int kPiecesB = kTileM * 4 / kThreads; // 16-byte pieces of the pixel tile per thread and k step (2)
@@ -63,7 +62,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     __shared__ __align__(16) unsigned char a_l[2][TN * kRow];
     __shared__ int cst[3][TN]; // start value | shift | left shift
     __shared__ int8_t lut_l[256];
-    __shared__ int pool_l[GAP ? 4 * PT : 1][GAP ? 64 : 1]; // [wavefront x pixel tile][filter]
+    __shared__ int pool_l[GAP ? 4 : 1][GAP ? TN : 1]; // [wavefront][filter]: the wavefront's share of its image's sum
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 15, quad = lane >> 4;
@@ -160,7 +159,11 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
 #pragma unroll
         for (int t = 0; t < 4; t++) {
             // rows 4*quad .. 4*quad+3 of tile t are filters 64*g + 16*quad + 4*t + r
-            const v4i init = *reinterpret_cast<const v4i *>(&cst[0][64 * g + 16 * quad + 4 * t]);
+            v4i init = *reinterpret_cast<const v4i *>(&cst[0][64 * g + 16 * quad + 4 * t]);
+            if constexpr (GAP) { // pooled form: the operands swap roles, a lane holds four pixels of ONE filter
+                const int i1 = cst[0][64 * g + 16 * (col >> 2) + (col & 3) + 4 * t];
+                init = v4i{i1, i1, i1, i1};
+            }
 #pragma unroll
             for (int c = 0; c < PT; c++)
                 acc[c][4 * g + t] = init;
@@ -179,8 +182,12 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
             for (int t = 0; t < 4; t++) {
                 const v4i aop = *reinterpret_cast<const v4i *>(&a_l[buf][(64 * g + a_row0 + 4 * t) * kRow + 16 * quad]);
 #pragma unroll
-                for (int c = 0; c < PT; c++)
-                    acc[c][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[c], acc[c][4 * g + t], 0, 0, 0);
+                for (int c = 0; c < PT; c++) {
+                    if constexpr (GAP) // rows = pixels, columns = filters: the sum over pixels stays inside a lane
+                        acc[c][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(b[c], aop, acc[c][4 * g + t], 0, 0, 0);
+                    else
+                        acc[c][4 * g + t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop, b[c], acc[c][4 * g + t], 0, 0, 0);
+                }
             }
     };
     // Step ks reads LDS buffer ks & 1.  At its end the operands of step ks + 1 (held in registers since step
@@ -234,24 +241,6 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
                                             lut_l[(int)(int8_t)(v >> 16) + 128], lut_l[(v >> 24) + 128]);
                     }
                 }
-                if constexpr (GAP) {
-                    // this lane's 16 filters of its pixel: sum over the 16 pixels of the tile
-                    const bool pixel = row_pixel(16 * PT * wave + 16 * c + col) >= 0;
-#pragma unroll
-                    for (int t = 0; t < 4; t++)
-#pragma unroll
-                        for (int r = 0; r < 4; r++) {
-                            int v = pixel ? (int)(int8_t)(words[t] >> (8 * r)) : 0;
-                            // rotations by 8, 4, 2, 1 inside the row of 16 lanes: every lane ends with the row's sum
-                            v += __builtin_amdgcn_update_dpp(0, v, 0x128, 0xf, 0xf, false);
-                            v += __builtin_amdgcn_update_dpp(0, v, 0x124, 0xf, 0xf, false);
-                            v += __builtin_amdgcn_update_dpp(0, v, 0x122, 0xf, 0xf, false);
-                            v += __builtin_amdgcn_update_dpp(0, v, 0x121, 0xf, 0xf, false);
-                            if (col == 0)
-                                pool_l[wave * PT + c][16 * quad + 4 * t + r] = v;
-                        }
-                    continue;
-                }
                 if (m >= a.M || n >= a.N)
                     continue;
                 const long long goff = m * a.N + n;
@@ -287,21 +276,93 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
             }
         }
     };
-    if (half_even)
-        epilogue(std::integral_constant<int, 5>{});
-    else
-        epilogue(std::integral_constant<int, 1>{});
+    // Pooled form: lane (col, quad) holds pixels 4 quad + [0, 4) of every pixel tile for filter a_row0 + 4 t of the
+    // group.  The four results of a tile are requantized with the lane's one set of constants, brought down to
+    // their int8 value inside the int16 pairs (packed shift by 8), masked where the tile row is past the image,
+    // and summed as packed int16 (at most 8 PT values of magnitude <= 128 per half).
+    auto pooled = [&](auto mode) {
+        constexpr int MODE = decltype(mode)::value; // 1: half up, 5: half even, -1: the general epilogue
+        const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
+        const long long img = (long long)blockIdx.x * PT + ((16 * PT * wave) >> 6);
+        const bool img_ok = img * a.hw < a.M;
+        int sums[4 * NG];
+#pragma unroll
+        for (int t = 0; t < 4 * NG; t++)
+            sums[t] = 0;
+#pragma unroll
+        for (int c = 0; c < PT; c++) {
+            const int pix0 = (16 * PT * wave + 16 * c) & 63;
+            const int rows = img_ok ? min(max(a.hw - pix0, 0), 16) : 0; // uniform: tile rows inside the image
+            if (rows == 0)
+                continue;
+            const int mine = rows - 4 * quad; // this lane's rows r < mine count
+            const int m01 = (mine > 0 ? 0xffff : 0) | (mine > 1 ? (int)0xffff0000u : 0);
+            const int m23 = (mine > 2 ? 0xffff : 0) | (mine > 3 ? (int)0xffff0000u : 0);
+#pragma unroll
+            for (int t = 0; t < 4 * NG; t++) {
+                const int f = 64 * (t >> 2) + a_row0 + 4 * (t & 3); // tile t = 4 g + t' holds filters of group g
+                const int ss = cst[1][f], ls = cst[2][f];
+                const v4i v = acc[c][t];
+                if constexpr (MODE >= 0) {
+                    int w[4];
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        int x = v[r];
+                        if (MODE == 5)
+                            x = half_even_add(x, ss + 8 - ls);
+                        w[r] = (int)((unsigned)x << ls) >> ss;
+                    }
+                    v2s p01 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(w[0], w[1]), floor2);
+                    v2s p23 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(w[2], w[3]), floor2);
+                    int q01 = __builtin_bit_cast(int, p01 >> 8), q23 = __builtin_bit_cast(int, p23 >> 8);
+                    if (rows < 16) { // uniform
+                        q01 &= m01;
+                        q23 &= m23;
+                    }
+                    const v2s both = __builtin_bit_cast(v2s, q01) + __builtin_bit_cast(v2s, q23);
+                    sums[t] = __builtin_bit_cast(int, __builtin_bit_cast(v2s, sums[t]) + both);
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        sums[t] += r < mine ? requant_s8(v[r], ss, relu, half_even) : 0;
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4 * NG; t++) {
+            int total = MODE >= 0 ? (int)(short)(sums[t] & 0xffff) + (sums[t] >> 16) : sums[t];
+            total += __shfl_xor(total, 16);
+            total += __shfl_xor(total, 32);
+            if (quad == 0)
+                pool_l[wave][64 * (t >> 2) + a_row0 + 4 * (t & 3)] = total;
+        }
+    };
+    if constexpr (GAP) {
+        if (!fast)
+            pooled(std::integral_constant<int, -1>{});
+        else if (half_even)
+            pooled(std::integral_constant<int, 5>{});
+        else
+            pooled(std::integral_constant<int, 1>{});
+    } else {
+        if (half_even)
+            epilogue(std::integral_constant<int, 5>{});
+        else
+            epilogue(std::integral_constant<int, 1>{});
+    }
     if constexpr (GAP) {
         __syncthreads();
         const int img_l = tid >> 6, flt = tid & 63; // image of the tile, filter of the group
         const long long img = (long long)blockIdx.x * PT + img_l;
-        if (img_l < PT && img * a.hw < a.M && n0 + flt < a.N) {
-            int sum = 0;
 #pragma unroll
-            for (int i = 0; i < 4 * PT; i++) // pixel tile i holds tile rows 16 i ..: image i / 4
-                sum += (i >> 2) == img_l ? pool_l[i][flt] : 0;
-            a.out[img * a.N + n0 + flt] = (int8_t)clamp_s8(round_half_up_f32((float)sum * a.gap_scale));
-        }
+        for (int g = 0; g < NG; g++)
+            if (img_l < PT && img * a.hw < a.M && n0 + 64 * g + flt < a.N) {
+                int sum = 0;
+#pragma unroll
+                for (int w = 0; w < 4; w++) // wavefront w holds tile rows 16 PT w ..: image PT w / 4
+                    sum += ((PT * w) >> 2) == img_l ? pool_l[w][64 * g + flt] : 0;
+                a.out[img * a.N + n0 + 64 * g + flt] = (int8_t)clamp_s8(round_half_up_f32((float)sum * a.gap_scale));
+            }
     }
 }
 
@@ -471,9 +532,13 @@ hipError_t launch_conv2d_gap_s8(const ConvGeom &g, const int8_t *in, const int8_
     a.gap_scale = gap_scale;
     if (a.M == 0)
         return hipSuccess;
-    // two images per workgroup (each filter tile is then read half as often) unless that leaves compute units idle
+    // else two images per workgroup (each filter tile is then read half as often) unless that leaves compute units idle
     const unsigned gy = (unsigned)((a.N + 63) / 64);
-    if ((long long)((g.batch + 1) / 2) * gy >= 2ll * cus)
+    // four images per workgroup while that leaves four workgroups per compute unit: a wavefront then reads each
+    // filter tile from LDS once for four pixel tiles (the kernel is bound by LDS reads, not by the matrix pipe)
+    if ((long long)((g.batch + 3) / 4) * gy >= 4ll * cus)
+        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 4, true>), dim3((unsigned)((g.batch + 3) / 4), gy), dim3(kThreads), 0, stream, a);
+    else     if ((long long)((g.batch + 1) / 2) * gy >= 2ll * cus)
         hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2, true>), dim3((unsigned)((g.batch + 1) / 2), gy), dim3(kThreads), 0, stream, a);
     else
         hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1, true>), dim3((unsigned)g.batch, gy), dim3(kThreads), 0, stream, a);

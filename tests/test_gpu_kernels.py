@@ -762,6 +762,10 @@ GAP_CASES = [
     ("one_pixel_128_40", (9, 1, 1, 128), 40, False, False, 0),
     ("half_even_5x5_80_100", (6, 5, 5, 80), 100, True, True, 0),
     ("general_shifts_3x3_64_64", (4, 3, 3, 64), 64, False, False, 1),
+    # enough images for four per workgroup, the last workgroup holding three
+    ("four_images_per_group_7x7_64_1280", (207, 7, 7, 64), 1280, True, False, 0),
+    ("four_images_per_group_half_even_6x6_128_1300", (210, 6, 6, 128), 1300, False, True, 0),
+    ("four_images_per_group_general_shifts_8x8", (206, 8, 8, 64), 1290, True, False, 1),
 ]
 
 
