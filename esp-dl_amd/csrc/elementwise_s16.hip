@@ -13,6 +13,7 @@
 // ReduceMean: reduce<int64_t, int16_t> (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:18-56).
 #include "espdl_device.h"
 #include "espdl_kernels.h"
+#include "reduce_mid.h"
 
 namespace espdl {
 namespace {
@@ -296,6 +297,18 @@ hipError_t launch_avg_pool_s16(const int16_t *in, int batch, int h, int w, int c
     return hipGetLastError();
 }
 
+namespace {
+// ReduceMean's float expression on the integer sum, left to right as in the reference
+struct MeanFinish16 {
+    int16_t *out;
+    float input_scale, count, output_scale;
+    __device__ void operator()(long long o, int total) const
+    {
+        out[o] = (int16_t)clamp_s16(round_half_up_f32((float)total * input_scale / count * output_scale));
+    }
+};
+} // namespace
+
 hipError_t launch_reduce_mean_s16(const int16_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
                                   int out_exp, int16_t *out, int cu_count, hipStream_t stream)
 {
@@ -323,6 +336,11 @@ hipError_t launch_reduce_mean_s16(const int16_t *in, const int *shape, int dims,
         return hipSuccess;
     a.input_scale = dl_scale(in_exp);
     a.output_scale = dl_rescale(out_exp);
+    // the reduced axes are neighbours and the sum fits int32: contiguous loads, every lane busy
+    long long outer, r_count, inner;
+    if (reduce_mid::mid_view(shape, dims, reduce_flag, &outer, &r_count, &inner) && r_count >= 8 &&
+        reduce_mid::fits<int16_t>(outer, r_count, inner))
+        return reduce_mid::launch(in, outer, r_count, inner, MeanFinish16{out, a.input_scale, (float)a.count, a.output_scale}, stream);
     reduce_mean_s16_kernel<<<dim3(blocks_for(a.n_out, cu_count)), dim3(kThreads), 0, stream>>>(a);
     return hipGetLastError();
 }

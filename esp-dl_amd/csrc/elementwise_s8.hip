@@ -3,6 +3,7 @@
 // 16-byte aligned; a byte tail (and unaligned tensors) take the scalar path of the same kernel.
 #include "espdl_device.h"
 #include "espdl_kernels.h"
+#include "reduce_mid.h"
 
 namespace espdl {
 
@@ -399,6 +400,18 @@ float global_avg_pool_scale(int h, int w, int in_exp, int out_exp)
     return dl_scale(in_exp) * area_inv * dl_rescale(out_exp);
 }
 
+namespace {
+// what GlobalAveragePool does with the sum of an image's pixels
+struct GapFinish {
+    int8_t *out;
+    float scale;
+    __device__ void operator()(long long o, int total) const
+    {
+        out[o] = (int8_t)clamp_s8(round_half_up_f32((float)total * scale));
+    }
+};
+} // namespace
+
 hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
                                      int8_t *out, hipStream_t stream)
 {
@@ -408,6 +421,8 @@ hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, 
     if ((c & 3) == 0 && h * w <= 64 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 3) == 0)
         hipLaunchKernelGGL(global_avg_pool_s8_small_kernel, dim3((unsigned)((c / 4 + kBlock - 1) / kBlock), (unsigned)batch),
                            dim3(kBlock), 0, stream, in, out, h * w, c, scale);
+    else if (reduce_mid::fits<int8_t>(batch, (long long)h * w, c)) // every lane busy whatever the channel count
+        return reduce_mid::launch(in, batch, (long long)h * w, c, GapFinish{out, scale}, stream);
     else if ((c & 15) == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0)
         hipLaunchKernelGGL(global_avg_pool_s8_kernel<16>, dim3((unsigned)((c + 1023) / 1024), (unsigned)batch), dim3(kBlock),
                            0, stream, in, out, h * w, c, scale);

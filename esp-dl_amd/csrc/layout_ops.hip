@@ -10,6 +10,7 @@
 //   MaxPool    esp-dl/dl/base/dl_base_max_pool2d.cpp:9-29 on the window clipped to the image
 #include "espdl_device.h"
 #include "espdl_kernels.h"
+#include "reduce_mid.h"
 
 namespace espdl {
 
@@ -804,6 +805,18 @@ hipError_t launch_pad(const void *in, const int *shape, int dims, const int *pad
     return hipGetLastError();
 }
 
+namespace {
+// ReduceMean's float expression on the integer sum, left to right as in the reference
+struct MeanFinish8 {
+    int8_t *out;
+    float input_scale, count, output_scale;
+    __device__ void operator()(long long o, int total) const
+    {
+        out[o] = (int8_t)clamp_s8(round_half_up_f32((float)total * input_scale / count * output_scale));
+    }
+};
+} // namespace
+
 hipError_t launch_reduce_mean_s8(const int8_t *in, const int *shape, int dims, const int *reduce_flag, int in_exp,
                                  int out_exp, int8_t *out, int cu_count, hipStream_t stream)
 {
@@ -831,6 +844,11 @@ hipError_t launch_reduce_mean_s8(const int8_t *in, const int *shape, int dims, c
     a.out = out;
     a.input_scale = dl_scale(in_exp);
     a.output_scale = dl_rescale(out_exp);
+    // the reduced axes are neighbours (a pooled embedding, a mean over time): contiguous loads, every lane busy
+    long long outer, r_count, inner;
+    if (reduce_mid::mid_view(shape, dims, reduce_flag, &outer, &r_count, &inner) && r_count >= 8 &&
+        reduce_mid::fits<int8_t>(outer, r_count, inner))
+        return reduce_mid::launch(in, outer, r_count, inner, MeanFinish8{out, a.input_scale, (float)a.count, a.output_scale}, stream);
     // enough lanes per output to occupy the device when there are few outputs and long sums
     a.lanes = 1;
     while (a.lanes < 64 && a.n_out * a.lanes < (long long)max(1, cu_count) * 2048 && a.count >= 4ll * a.lanes)

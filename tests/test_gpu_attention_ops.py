@@ -196,6 +196,20 @@ def test_avg_pool_and_reduce_mean_s16(oracle):
         np.testing.assert_array_equal(got, oracle.reduce_mean_s16(x, axes, keep, -10, -12))
 
 
+# int16 means over long runs of neighbouring axes (the pooling of a speaker-embedding or text-recognition graph):
+# inner sizes of one 16-byte piece, several slabs, odd (single-element loads), 1; extreme inputs.
+@pytest.mark.parametrize("shape,axes,keepdims", [
+    ((4, 300, 8), [1], False), ((2, 40, 50, 520), [1, 2], True), ((3, 97, 1, 37), [1, 2], True), ((6, 1500), [1], True),
+    ((2, 3, 200, 24), [2], False),
+])
+def test_reduce_mean_s16_long_runs(oracle, shape, axes, keepdims):
+    announce(f"reduce_mean_s16 long runs {shape} axes {axes}")
+    rng = np.random.default_rng(63)
+    for x in (_rand(rng, shape, np.int16), np.full(shape, 32767, np.int16), np.full(shape, -32768, np.int16)):
+        got = to_host(espdl().reduce_mean_s16(to_dev(x), axes, keepdims, -10, -12))
+        np.testing.assert_array_equal(got, oracle.reduce_mean_s16(x, axes, keepdims, -10, -12))
+
+
 def test_sub_s16(oracle):
     announce("sub_s16")
     rng = np.random.default_rng(63)

@@ -129,6 +129,34 @@ def test_reduce_mean_s8(oracle, shape, axes, keepdims, exps):
     np.testing.assert_array_equal(got, oracle.reduce_mean_s8(x, axes, keepdims, exps[0], exps[1]))
 
 
+# Reductions over a run of neighbouring axes with many elements per output go through the kernel that sums the
+# middle axis of an [outer][R][inner] view: inner sizes that are one 16-byte piece, several slabs with a ragged
+# last one, not a multiple of 16 (single-element loads), 1 (a mean over the last axis); R not a multiple of the
+# positions in flight; a reduced run split by an axis of length 1; extreme inputs (the largest sums).
+@pytest.mark.parametrize("shape,axes,keepdims,exps", [
+    ((2, 50, 60, 96), [1, 2], True, (-4, -5)), ((3, 33, 31, 20), [1, 2], False, (-5, -5)),
+    ((2, 19, 23, 1040), [1, 2], True, (-3, -4)), ((5, 301, 16), [1], False, (-6, -6)),
+    ((7, 1000), [1], True, (-4, -4)), ((3, 257, 1, 48), [1, 2], True, (-5, -6)), ((4, 6, 13, 1, 11, 24), [2, 3, 4], False, (-5, -5)),
+])
+def test_reduce_mean_s8_long_runs(oracle, shape, axes, keepdims, exps):
+    announce(f"reduce_mean long runs {shape} axes {axes}")
+    rng = np.random.default_rng(281)
+    for x in (_rand(rng, shape), np.full(shape, 127, np.int8), np.full(shape, -128, np.int8)):
+        got = to_host(espdl().reduce_mean_s8(to_dev(x), axes, keepdims, exps[0], exps[1]))
+        np.testing.assert_array_equal(got, oracle.reduce_mean_s8(x, axes, keepdims, exps[0], exps[1]))
+
+
+@pytest.mark.parametrize("shape", [(2, 50, 60, 96), (3, 33, 31, 20), (2, 19, 23, 1040), (1, 120, 160, 16), (4, 9, 9, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_global_avg_pool_s8_large_images(oracle, shape):
+    announce(f"global_avg_pool_s8 large image {shape}")
+    rng = np.random.default_rng(282)
+    for x in (_rand(rng, shape), np.full(shape, 127, np.int8), np.full(shape, -128, np.int8)):
+        for exps in ((-4, -5), (-5, -3)):
+            got = to_host(espdl().global_avg_pool_s8(to_dev(x), exps[0], exps[1]))
+            np.testing.assert_array_equal(got, oracle.global_avg_pool_s8(x, exps[0], exps[1]))
+
+
 @pytest.mark.parametrize("hw", [(3, 3), (2, 5)], ids=["3x3", "2x5"])
 def test_avg_pool_and_reduce_mean_s8_every_sum(oracle, hw):
     """Every sum a window can have, exponent pairs with and without ties: float(sum) * scale is rounded to float
