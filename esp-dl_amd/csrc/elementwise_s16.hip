@@ -13,6 +13,7 @@
 // ReduceMean: reduce<int64_t, int16_t> (esp-dl/dl/module/include/dl_module_reduce_mean.hpp:18-56).
 #include "espdl_device.h"
 #include "espdl_kernels.h"
+#include "binary_vec.h"
 #include "reduce_mid.h"
 
 namespace espdl {
@@ -205,10 +206,46 @@ unsigned blocks_for(long long total, int cu_count)
 
 namespace {
 
+// The element operations of binary_kernel as functors for the 16-bytes-per-thread form (Div stays element-wise).
+struct Add16 {
+    __device__ __forceinline__ int apply(int x, int y) const { return clamp_s16(x + y); }
+};
+template <typename T>
+struct SubOp {
+    __device__ __forceinline__ int apply(int x, int y) const
+    {
+        constexpr int lo = sizeof(T) == 1 ? -128 : -32768, hi = sizeof(T) == 1 ? 127 : 32767;
+        return min(max(x - y, lo), hi);
+    }
+};
+struct Mul16 {
+    int shift, half_even;
+    float rescale;
+    __device__ __forceinline__ int apply(int x, int y) const
+    {
+        const int prod = x * y; // at most 2^30 in magnitude
+        if (half_even && shift > 0) {
+            const long long q = (long long)prod >> shift;
+            const long long frac = (long long)prod & ((1ll << shift) - 1), half = 1ll << (shift - 1);
+            return (int)min(max(q + ((frac > half || (frac == half && (q & 1))) ? 1 : 0), -32768ll), 32767ll);
+        }
+        return clamp_s16(round_half_up_f32((float)prod * rescale));
+    }
+};
+
 template <typename T>
 hipError_t launch_binary(int op, const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const T *in0, const T *in1,
                          int shift, bool half_even, T *out, int cu_count, hipStream_t stream)
 {
+    if (binary_vec::Args va; op != 3 && binary_vec::plan(dims, s0, s1, in0, in1, out, &va)) {
+        if (op == 2)
+            return binary_vec::launch(in0, in1, out, va, SubOp<T>{}, cu_count, stream);
+        if constexpr (sizeof(T) == 2) {
+            if (op == 1)
+                return binary_vec::launch(in0, in1, out, va, Mul16{shift, half_even ? 1 : 0, dl_rescale(shift)}, cu_count, stream);
+            return binary_vec::launch(in0, in1, out, va, Add16{}, cu_count, stream);
+        }
+    }
     BinaryArgs<T> a = {};
     a.in0 = in0;
     a.in1 = in1;

@@ -3,6 +3,7 @@
 // 16-byte aligned; a byte tail (and unaligned tensors) take the scalar path of the same kernel.
 #include "espdl_device.h"
 #include "espdl_kernels.h"
+#include "binary_vec.h"
 #include "reduce_mid.h"
 
 namespace espdl {
@@ -214,6 +215,9 @@ hipError_t launch_binary_s8(const int32_t dims[4], const int64_t s0[4], const in
         int64_t vecs;
         const dim3 grid = grid_for(size, vec_ok, &vecs);
         hipLaunchKernelGGL(binary_s8_dense_kernel<Op>, grid, dim3(kBlock), 0, stream, in0, in1, out, size, vecs, op);
+    } else if (binary_vec::Args va; binary_vec::plan(dims, s0, s1, in0, in1, out, &va)) {
+        // innermost axis dense or constant in each operand (a channel-wise scale, a per-row offset): 16 bytes per thread
+        return binary_vec::launch(in0, in1, out, va, op, 0, stream);
     } else {
         BroadcastArgs a;
         for (int i = 0; i < 4; i++) {

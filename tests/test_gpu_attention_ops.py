@@ -210,6 +210,29 @@ def test_reduce_mean_s16_long_runs(oracle, shape, axes, keepdims):
         np.testing.assert_array_equal(got, oracle.reduce_mean_s16(x, axes, keepdims, -10, -12))
 
 
+# int16 Add / Mul / Sub and int8 Sub where the innermost axis is dense or constant in each operand and a multiple of
+# a 16-byte piece long (8 int16, 16 int8): the 16-bytes-per-thread form, dense and with broadcasting.
+@pytest.mark.parametrize("sa,sb", [((3, 20, 20, 64), (3, 1, 1, 64)), ((3, 1, 1, 64), (3, 20, 20, 64)), ((2, 75, 40), (2, 75, 40)),
+                                   ((4, 7, 32), (1, 7, 1)), ((2, 9, 16), (16,)), ((6, 1, 5, 32), (1, 4, 1, 1))],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_binary_s16_and_sub_s8_wide_form(oracle, sa, sb):
+    announce(f"binary s16 / sub s8 wide form {sa} {sb}")
+    rng = np.random.default_rng(66)
+    a, b = _rand(rng, sa, np.int16), _rand(rng, sb, np.int16)
+    a.reshape(-1)[:2], b.reshape(-1)[:2] = [-32768, 32767], [32767, -32768]
+    wide = lambda t: t.astype(np.int64)  # noqa: E731
+    np.testing.assert_array_equal(to_host(espdl().add_s16(to_dev(a), to_dev(b))),
+                                  np.clip(wide(a) + wide(b), -32768, 32767).astype(np.int16))
+    np.testing.assert_array_equal(to_host(espdl().sub_s16(to_dev(a), to_dev(b))),
+                                  np.clip(wide(a) - wide(b), -32768, 32767).astype(np.int16))
+    af, bf = (np.ascontiguousarray(t) for t in np.broadcast_arrays(a, b))  # the oracle multiplies equal shapes
+    for shift, rm in ((14, 0), (15, 1), (3, 1)):
+        np.testing.assert_array_equal(to_host(espdl().mul_s16(to_dev(a), to_dev(b), shift, rm)), oracle.mul_s16(af, bf, shift, rm))
+    a8, b8 = _rand(rng, sa, np.int8), _rand(rng, sb, np.int8)
+    np.testing.assert_array_equal(to_host(espdl().sub_s8(to_dev(a8), to_dev(b8))),
+                                  np.clip(wide(a8) - wide(b8), -128, 127).astype(np.int8))
+
+
 def test_sub_s16(oracle):
     announce("sub_s16")
     rng = np.random.default_rng(63)

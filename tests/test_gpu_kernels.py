@@ -466,6 +466,9 @@ ADD_SHAPES = [
     ((1, 1, 4, 5), (2, 3, 1, 1)), ((10, 1, 5, 5), (1, 1, 5, 5)), ((1, 512, 7, 7), (1, 512, 7, 7)),
     ((5,), (1,)), ((2, 5), (2, 1)), ((8, 2, 5), (2, 1)), ((1, 96, 5, 49), (1, 96, 5, 49)),
     ((4, 56, 56, 24), (4, 56, 56, 24)),
+    # innermost axis dense or constant in each operand, a multiple of 16 long: 16 bytes per thread
+    ((3, 20, 20, 64), (3, 1, 1, 64)), ((3, 1, 1, 64), (3, 20, 20, 64)), ((2, 286, 800), (2, 1, 800)),
+    ((4, 7, 32), (1, 7, 1)), ((5, 3, 9, 48), (1, 3, 1, 48)), ((2, 9, 16), (16,)), ((6, 1, 5, 32), (1, 4, 1, 1)),
 ]
 
 
