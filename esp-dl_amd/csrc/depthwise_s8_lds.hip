@@ -40,7 +40,8 @@ namespace {
 
 constexpr int kThreads = 512; // 8 wavefronts share one patch: fewer chunks (registers) per thread
 constexpr int kWaves = kThreads / 64;
-constexpr int kKs = 3;     // k steps of 4 taps
+constexpr int kKs = 3;     // k steps of 4 taps: windows of up to 12 taps (3 x 3) ...
+constexpr int kKsWide = 7; // ... and of up to 28 (5 x 5), in builds of their own (plain depthwise only)
 constexpr int kMaxIn = 5;  // 16-byte patch chunks per thread
 constexpr int kMaxOut = 4; // 16-byte output chunks per thread
 constexpr int kMaxX = 4;   // dwords of the expand stage's input patch per thread
@@ -210,9 +211,9 @@ __device__ __forceinline__ void dw_expand(const DwLdsArgs &a, unsigned char *sme
     }
 }
 
-template <bool FAST, int USE_LSH>
+template <bool FAST, int USE_LSH, int KS>
 __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *smem, int wave, int lane,
-                                           const int (&tapoff)[kKs], int floor_pk)
+                                           const int (&tapoff)[KS], int floor_pk)
 {
     const ConvGeom &g = a.g;
     const int col = lane & 15, quad = lane >> 4;
@@ -231,11 +232,11 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
     int p = t - grp * a.np;
 
     const int sel = col >> 2; // dword of the 16-byte operand A vector that holds this row's weight
-    v4i aop[kKs], init, ss, ls;
+    v4i aop[KS], init, ss, ls;
     auto load_group = [&](int gi) {
 #pragma unroll
-        for (int ks = 0; ks < kKs; ks++) {
-            const int d = a_l[(gi * kKs + ks) * 64 + lane];
+        for (int ks = 0; ks < KS; ks++) {
+            const int d = a_l[(gi * KS + ks) * 64 + lane];
             aop[ks] = v4i{sel == 0 ? d : 0, sel == 1 ? d : 0, sel == 2 ? d : 0, sel == 3 ? d : 0};
         }
         const int ch = 16 * gi + 4 * quad;
@@ -245,11 +246,11 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
     };
     int grp_loaded = -1;
 
-    v4i b[kKs];
+    v4i b[KS];
     {
         const int po = pixtab[p * 16 + col] + 16 * grp;
 #pragma unroll
-        for (int ks = 0; ks < kKs; ks++)
+        for (int ks = 0; ks < KS; ks++)
             b[ks] = *reinterpret_cast<const v4i *>(patch + po + tapoff[ks]);
     }
     const int out_lane = col * a.cso + 4 * quad;
@@ -266,14 +267,14 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
         const int out_off = out_lane + p * 16 * a.cso + 16 * grp;
         v4i acc = init;
 #pragma unroll
-        for (int ks = 0; ks < kKs; ks++)
+        for (int ks = 0; ks < KS; ks++)
             if (4 * ks < a.taps)
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], acc, 0, 0, 0);
         // operand B of the next tile of this wavefront is read while this one is in the matrix pipe
         if (t + 1 < t_end) {
             const int po = pixtab[p_next * 16 + col] + 16 * grp_next;
 #pragma unroll
-            for (int ks = 0; ks < kKs; ks++)
+            for (int ks = 0; ks < KS; ks++)
                 b[ks] = *reinterpret_cast<const v4i *>(patch + po + tapoff[ks]);
         }
         int word;
@@ -296,8 +297,9 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
 }
 
 // HE: the round-half-even build (a separate kernel so that the half-up build keeps its register count).
-template <bool PROJ, bool HE, bool EXP>
-__global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwLdsArgs a)
+// KS: k steps of 4 taps the build holds operands for (kKs, or kKsWide for windows of 13 to 28 taps).
+template <bool PROJ, bool HE, bool EXP, int KS = kKs>
+__global__ __launch_bounds__(kThreads, KS > kKs ? 2 : 4) void depthwise_s8_lds_kernel(const DwLdsArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const ConvGeom &g = a.g;
@@ -388,8 +390,8 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
     // tables: diagonal operand A as one dword per (group, k step, lane); start values and shifts;
     // patch offset of every output pixel of the tile; the LUT
     int *a_l = reinterpret_cast<int *>(smem + a.off_a);
-    for (int e = tid; e < a.gc * kKs * 64; e += kThreads) {
-        const int l = e & 63, ks = (e >> 6) % kKs, gi = e / (64 * kKs);
+    for (int e = tid; e < a.gc * KS * 64; e += kThreads) {
+        const int l = e & 63, ks = (e >> 6) % KS, gi = e / (64 * KS);
         const int i = l & 15, tap = 4 * ks + (l >> 4);
         int d = 0;
         if (tap < a.taps)
@@ -436,9 +438,9 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
             reinterpret_cast<int8_t *>(smem + a.off_lut)[tid] = a.lut[tid];
     }
     // tap offsets of this lane's quad inside the patch
-    int tapoff[kKs];
+    int tapoff[KS];
 #pragma unroll
-    for (int ks = 0; ks < kKs; ks++) {
+    for (int ks = 0; ks < KS; ks++) {
         const int tap = 4 * ks + quad;
         tapoff[ks] = 0;
         if (tap < a.taps) {
@@ -575,13 +577,13 @@ __global__ __launch_bounds__(kThreads, 4) void depthwise_s8_lds_kernel(const DwL
         // epilogue mode of pack_fast4: 0 plain (every shift >= 8), 1 with the left shift, 5 the same with
         // round-half-even
         if (fast && HE)
-            dw_compute<true, 5>(a, smem, wave, lane, tapoff, floor_pk);
+            dw_compute<true, 5, KS>(a, smem, wave, lane, tapoff, floor_pk);
         else if (fast && !use_lsh)
-            dw_compute<true, 0>(a, smem, wave, lane, tapoff, floor_pk);
+            dw_compute<true, 0, KS>(a, smem, wave, lane, tapoff, floor_pk);
         else if (fast)
-            dw_compute<true, 1>(a, smem, wave, lane, tapoff, floor_pk);
+            dw_compute<true, 1, KS>(a, smem, wave, lane, tapoff, floor_pk);
         else
-            dw_compute<false, 0>(a, smem, wave, lane, tapoff, floor_pk);
+            dw_compute<false, 0, KS>(a, smem, wave, lane, tapoff, floor_pk);
         __syncthreads();
 
         if (PROJ) {
@@ -690,6 +692,7 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr, const Dw
     best.ok = false;
     const int G = g.in_c / 16;
     const int taps = g.k_h * g.k_w;
+    const int ks_steps = taps > 4 * kKs ? kKsWide : kKs;
     const int halo_h = (g.k_h - 1) * g.dil_h + 1, halo_w = (g.k_w - 1) * g.dil_w + 1;
     double best_cost = 1e30;
     static const int sizes[] = {1, 2, 3, 4, 6, 7, 8, 12, 14, 16, 24, 28, 32, 56, 64, 112};
@@ -748,7 +751,7 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr, const Dw
                 const long long n_pout = (long long)the * twe * p_vecs;
                 if (proj && n_pout > kMaxOut * kThreads)
                     continue;
-                const size_t tables = (size_t)gc * kKs * 64 * 4 + (size_t)gc * 16 * 12 + (size_t)np * 16 * 4 + 256;
+                const size_t tables = (size_t)gc * ks_steps * 64 * 4 + (size_t)gc * 16 * 12 + (size_t)np * 16 * 4 + 256;
                 const size_t lds = patch + outb + tables + pbytes + xbytes + 64;
                 if (lds > (size_t)kLdsBudget)
                     continue;
@@ -789,7 +792,7 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr, const Dw
                     a.off_out = (int)off;
                     off += outb;
                     a.off_a = (int)off;
-                    off += (size_t)gc * kKs * 64 * 4;
+                    off += (size_t)gc * ks_steps * 64 * 4;
                     a.off_init = (int)off;
                     off += (size_t)gc * 16 * 4;
                     a.off_ss = (int)off;
@@ -838,7 +841,7 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr, const Dw
 
 bool depthwise_s8_lds_supports(const ConvGeom &g, const void *in, const void *out)
 {
-    if ((g.in_c & 15) != 0 || g.k_h * g.k_w > 4 * kKs ||
+    if ((g.in_c & 15) != 0 || g.k_h * g.k_w > 4 * kKsWide ||
         ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) != 0)
         return false;
     // 32-bit offsets inside one image
@@ -849,7 +852,7 @@ bool depthwise_s8_lds_supports(const ConvGeom &g, const void *in, const void *ou
 
 namespace {
 
-template <bool PROJ, bool EXP = false>
+template <bool PROJ, bool EXP = false, int KS = kKs>
 hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
 {
     DwLdsArgs &a = plan.a;
@@ -870,17 +873,17 @@ hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
     a.fd_nxg = make_fastdiv((unsigned)max(1, (a.n_xpt + 3) / 4));
     const int cus = cu_count > 0 ? cu_count : 256;
     static const hipError_t lds_opt_in = [] {
-        const hipError_t e0 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, false, EXP>),
+        const hipError_t e0 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, false, EXP, KS>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
-        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, true, EXP>),
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(depthwise_s8_lds_kernel<PROJ, true, EXP, KS>),
                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBudget);
         return e0 != hipSuccess ? e0 : e1;
     }();
     if (lds_opt_in != hipSuccess)
         return lds_opt_in;
     const bool he = g.half_even != 0;
-    const int per_cu = he ? resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, true, EXP>, kThreads, plan.lds)
-                          : resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, false, EXP>, kThreads, plan.lds);
+    const int per_cu = he ? resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, true, EXP, KS>, kThreads, plan.lds)
+                          : resident_workgroups_per_cu(depthwise_s8_lds_kernel<PROJ, false, EXP, KS>, kThreads, plan.lds);
     int gx = max(1, (cus * per_cu) / plan.n_cchunk);
     if (gx > a.n_units)
         gx = a.n_units;
@@ -892,10 +895,10 @@ hipError_t dw_lds_launch(DwLdsPlan &plan, int cu_count, hipStream_t stream)
                 EXP ? "expand+" : "", PROJ ? "+project" : "", g.in_h, g.in_w, g.in_c, g.stride_h, a.th, a.tw, a.ph, a.pw, a.gc, a.np, plan.lds,
                 per_cu, gx, plan.n_cchunk, a.n_units);
     if (he)
-        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, true, EXP>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
+        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, true, EXP, KS>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
                            dim3(kThreads), plan.lds, stream, a);
     else
-        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, false, EXP>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
+        hipLaunchKernelGGL((depthwise_s8_lds_kernel<PROJ, false, EXP, KS>), dim3((unsigned)gx, (unsigned)plan.n_cchunk),
                            dim3(kThreads), plan.lds, stream, a);
     return hipGetLastError();
 }
@@ -921,6 +924,8 @@ hipError_t launch_depthwise_s8_lds(const ConvGeom &g, const int8_t *in, const in
     a.g = g;
     a.pj = DwProject{};
     a.ex = DwExpand{};
+    if (a.taps > 4 * kKs) // a 5 x 5 window: the build with seven k steps of taps
+        return dw_lds_launch<false, false, kKsWide>(plan, cu_count, stream);
     return dw_lds_launch<false>(plan, cu_count, stream);
 }
 

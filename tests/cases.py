@@ -44,6 +44,12 @@ DW_CASES = [
     ("dw144_14x14_k3p1_relu", (14, 14, 144), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
     ("dw96_15x15_k3s2p1", (15, 15, 96), (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, False),
     ("dw8_7x9_k3s2_tailpad", (7, 9, 8), (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), True, False),
+    # windows of 13 to 28 taps (5 x 5 and others): the matrix-pipe depthwise kernel's build with seven k steps of taps
+    ("dw64_60x60_k5p2_relu", (60, 60, 64), (5, 5), (1, 1), (1, 1), (2, 2, 2, 2), True, True),
+    ("dw32_31x29_k5s2p2", (31, 29, 32), (5, 5), (2, 2), (1, 1), (2, 2, 2, 2), True, False),
+    ("dw48_20x20_k4x6", (20, 20, 48), (4, 6), (1, 1), (1, 1), (1, 2, 2, 3), True, True),
+    ("dw16_12x40_k1x25", (12, 40, 16), (1, 25), (1, 1), (1, 1), (0, 0, 12, 12), True, False),
+    ("dw80_17x17_k7x4_nobias", (17, 17, 80), (7, 4), (1, 1), (1, 1), (3, 3, 1, 2), False, False),
 ]
 
 GEMM_CASES = [  # (M, K, N, bias, relu)

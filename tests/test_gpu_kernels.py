@@ -156,7 +156,7 @@ def test_conv2d_s8_pointwise_tiled_gemm(oracle, case, variant):
 
 # Round-half-even differs from half-up only at exact ties; small operands and small shifts make ties
 # frequent (a quarter to a half of all outputs), on every kernel route that has the short epilogue.
-@pytest.mark.parametrize("route", ["dense3x3", "pointwise_tiled", "pointwise_large", "depthwise", "depthwise_s2"])
+@pytest.mark.parametrize("route", ["dense3x3", "pointwise_tiled", "pointwise_large", "depthwise", "depthwise_s2", "depthwise_5x5"])
 @pytest.mark.parametrize("shift_lo,shift_hi", [(1, 3), (2, 9), (8, 10)])
 def test_half_even_ties(oracle, route, shift_lo, shift_hi):
     announce(f"half-even ties {route} shifts {shift_lo}..{shift_hi}")
@@ -168,6 +168,8 @@ def test_half_even_ties(oracle, route, shift_lo, shift_hi):
         shape, oc, k, stride, pads = (2, 9, 9, 64), 48, (1, 1), (1, 1), (0, 0, 0, 0)
     elif route == "pointwise_large":
         shape, oc, k, stride, pads = (2, 9, 9, 24), 40, (1, 1), (1, 1), (0, 0, 0, 0)
+    elif route == "depthwise_5x5":
+        shape, oc, k, stride, pads = (2, 18, 18, 32), 32, (5, 5), (1, 1), (2, 2, 2, 2)
     elif route == "depthwise":
         shape, oc, k, stride, pads = (2, 14, 14, 32), 32, (3, 3), (1, 1), (1, 1, 1, 1)
     else:
