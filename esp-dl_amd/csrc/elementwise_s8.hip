@@ -331,6 +331,29 @@ hipError_t launch_clip_s8(const int8_t *in, int64_t size, int min_q, int max_q, 
     return launch_map(in, out, size, ClipFn{min_q, max_q, dl_scale(in_exp) * dl_rescale(out_exp)}, stream);
 }
 
+namespace {
+// int8 -> int8 between exponents at most 7 apart: four values per packed-int16 sequence (requant4_s8: round half
+// up of x * 2^d, saturated - what RequantFn computes in float, where both scales are powers of two and every step
+// is exact); bytes past the last 16-byte vector take RequantFn itself.
+__global__ __launch_bounds__(kBlock) void requantize_pow2_s8_kernel(const int8_t *in, int8_t *out, int64_t size, int64_t vecs,
+                                                                    int d, RequantFn tail)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const Requant4 q = make_requant4(d);
+    if (i < vecs) {
+        const v4i v = reinterpret_cast<const v4i *>(in)[i];
+        v4i r;
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+            r[w] = requant4_s8(v[w], q);
+        reinterpret_cast<v4i *>(out)[i] = r;
+    }
+    const int64_t t = vecs * 16 + i;
+    if (t < size)
+        out[t] = (int8_t)tail((int)in[t], t);
+}
+} // namespace
+
 hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out,
                                 hipStream_t stream)
 {
@@ -340,26 +363,67 @@ hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int 
         return hipMemcpyAsync(out, in, (size_t)size, hipMemcpyDeviceToDevice, stream);
     }
     const float inv = (float)(1.0 / (double)dl_scale(out_exp));
+    const int d = in_exp - out_exp;
+    if (d >= -7 && d <= 7 && aligned16(in, out) && size >= 16) {
+        int64_t vecs;
+        const dim3 grid = grid_for(size, true, &vecs);
+        hipLaunchKernelGGL(requantize_pow2_s8_kernel, grid, dim3(kBlock), 0, stream, in, out, size, vecs, d,
+                           RequantFn{dl_scale(in_exp), inv});
+        return hipGetLastError();
+    }
     return launch_map(in, out, size, RequantFn{dl_scale(in_exp), inv}, stream);
 }
 
 // TensorBase::assign between int8 / int16 (esp-dl/dl/tensor/src/dl_tensor_base.cpp:321-392).
+// Eight elements per thread (one 8- or 16-byte access each way) when both pointers allow; the last size % 8 elements,
+// or everything when a pointer is unaligned, one element per thread.
+template <typename T>
+struct alignas(8 * sizeof(T)) Eight {
+    T v[8];
+};
+
 template <typename ST, typename DT>
-__global__ __launch_bounds__(kBlock) void requantize_any_kernel(const ST *in, DT *out, int64_t size, int same_exp,
-                                                                float src_scale, float inv_scale)
+__device__ __forceinline__ DT requantize_one(ST x, int same_exp, float src_scale, float inv_scale)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= size)
-        return;
     const int lo = sizeof(DT) == 1 ? -128 : -32768, hi = sizeof(DT) == 1 ? 127 : 32767;
     int q;
     if (same_exp) {
-        q = (int)in[i];
+        q = (int)x;
     } else {
-        const float tmp = (float)in[i] * src_scale;
+        const float tmp = (float)x * src_scale;
         q = round_half_up_f32(tmp * inv_scale);
     }
-    out[i] = (DT)min(max(q, lo), hi);
+    return (DT)min(max(q, lo), hi);
+}
+
+template <typename ST, typename DT>
+__global__ __launch_bounds__(kBlock) void requantize_any_kernel(const ST *in, DT *out, int64_t size, int64_t vecs, int same_exp,
+                                                                float src_scale, float inv_scale)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < vecs) {
+        const Eight<ST> x = reinterpret_cast<const Eight<ST> *>(in)[i];
+        Eight<DT> r;
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+            r.v[k] = requantize_one<ST, DT>(x.v[k], same_exp, src_scale, inv_scale);
+        reinterpret_cast<Eight<DT> *>(out)[i] = r;
+    }
+    const int64_t t = vecs * 8 + i;
+    if (t < size)
+        out[t] = requantize_one<ST, DT>(in[t], same_exp, src_scale, inv_scale);
+}
+
+template <typename ST, typename DT>
+hipError_t launch_requantize_any_t(const void *in, void *out, int64_t size, int same, float src, float inv, hipStream_t stream)
+{
+    const bool vec_ok = (reinterpret_cast<uintptr_t>(in) % (8 * sizeof(ST))) == 0 && (reinterpret_cast<uintptr_t>(out) % (8 * sizeof(DT))) == 0;
+    const int64_t vecs = vec_ok ? size / 8 : 0;
+    const int64_t tail = size - vecs * 8;
+    const int64_t threads = vecs > tail ? vecs : tail;
+    hipLaunchKernelGGL((requantize_any_kernel<ST, DT>), dim3((unsigned)((threads + kBlock - 1) / kBlock)), dim3(kBlock), 0, stream,
+                       static_cast<const ST *>(in), static_cast<DT *>(out), size, vecs, same, src, inv);
+    return hipGetLastError();
 }
 
 hipError_t launch_requantize_any(const void *in, int in_bits, int64_t size, int in_exp, int out_exp, void *out,
@@ -367,22 +431,15 @@ hipError_t launch_requantize_any(const void *in, int in_bits, int64_t size, int 
 {
     if (size <= 0)
         return hipSuccess;
-    const dim3 grid((unsigned)((size + kBlock - 1) / kBlock));
     const int same = in_exp == out_exp;
     const float src = dl_scale(in_exp), inv = (float)(1.0 / (double)dl_scale(out_exp));
     if (in_bits == 8 && out_bits == 16)
-        hipLaunchKernelGGL((requantize_any_kernel<int8_t, int16_t>), grid, dim3(kBlock), 0, stream,
-                           static_cast<const int8_t *>(in), static_cast<int16_t *>(out), size, same, src, inv);
-    else if (in_bits == 16 && out_bits == 8)
-        hipLaunchKernelGGL((requantize_any_kernel<int16_t, int8_t>), grid, dim3(kBlock), 0, stream,
-                           static_cast<const int16_t *>(in), static_cast<int8_t *>(out), size, same, src, inv);
-    else if (in_bits == 16 && out_bits == 16)
-        hipLaunchKernelGGL((requantize_any_kernel<int16_t, int16_t>), grid, dim3(kBlock), 0, stream,
-                           static_cast<const int16_t *>(in), static_cast<int16_t *>(out), size, same, src, inv);
-    else
-        hipLaunchKernelGGL((requantize_any_kernel<int8_t, int8_t>), grid, dim3(kBlock), 0, stream,
-                           static_cast<const int8_t *>(in), static_cast<int8_t *>(out), size, same, src, inv);
-    return hipGetLastError();
+        return launch_requantize_any_t<int8_t, int16_t>(in, out, size, same, src, inv, stream);
+    if (in_bits == 16 && out_bits == 8)
+        return launch_requantize_any_t<int16_t, int8_t>(in, out, size, same, src, inv, stream);
+    if (in_bits == 16 && out_bits == 16)
+        return launch_requantize_any_t<int16_t, int16_t>(in, out, size, same, src, inv, stream);
+    return launch_requantize_any_t<int8_t, int8_t>(in, out, size, same, src, inv, stream);
 }
 
 hipError_t launch_add_s8(const int32_t dims[4], const int64_t s0[4], const int64_t s1[4], const int8_t *in0,

@@ -441,6 +441,20 @@ def test_relu_clip_requantize_s8(oracle):
                                       oracle.requantize_s8(x, in_exp, out_exp))
 
 
+def test_requantize_s8_every_byte_every_shift(oracle):
+    """int8 -> int8 for every byte value and every exponent difference from -9 to 9: differences up to 7 take the
+    packed-int16 form, larger ones the float expression; sizes with and without a tail of single bytes."""
+    announce("requantize_s8 every byte, every shift")
+    m = espdl()
+    rng = np.random.default_rng(55)
+    for size in (256, 256 + 16 * 7 + 5, 4096 + 3):
+        x = np.concatenate([np.arange(-128, 128), rng.integers(-128, 128, size=size - 256)]).astype(np.int8)
+        xd = to_dev(x)
+        for d in range(-9, 10):
+            got = to_host(m.requantize_s8(xd, -6, -6 - d))
+            np.testing.assert_array_equal(got, oracle.requantize_s8(x, -6, -6 - d), err_msg=f"size {size} d {d}")
+
+
 @pytest.mark.parametrize("src,dst", [("s8", "s16"), ("s16", "s8"), ("s16", "s16")])
 def test_requantize_across_widths(oracle, src, dst):
     """TensorBase::assign between int8 and int16 tensors: same exponent widens / saturates, different
