@@ -110,14 +110,15 @@ struct PreluFn {
     const int8_t *alpha;
     int channels, shift;
     __device__ void prepare() {}
-    __device__ int operator()(int x, int64_t idx) const
+    __device__ __forceinline__ int one(int x, int slope) const
     {
         if (x >= 0)
             return x;
-        const int prod = x * (int)alpha[idx % channels];
+        const int prod = x * slope;
         const int shifted = shift > 0 ? (prod >> shift) : (int)((unsigned)prod << -shift);
         return clamp_s8((int)(int16_t)shifted);
     }
+    __device__ int operator()(int x, int64_t idx) const { return x >= 0 ? x : one(x, (int)alpha[idx % channels]); }
 };
 
 template <typename F>
@@ -314,9 +315,42 @@ hipError_t launch_lut_s8(const int8_t *in, int64_t size, const int8_t *table, in
     return launch_map(in, out, size, LutFn{table, nullptr}, stream);
 }
 
+namespace {
+// PReLU with a channel count that is a multiple of 16 and 16-byte aligned tensors: a thread's 16 bytes are 16
+// consecutive channels of one pixel, so the slopes are one 16-byte load and the channel index is one division per
+// thread (the per-byte functor form divides a 64-bit index for every byte).
+__global__ __launch_bounds__(kBlock) void prelu_s8_vec_kernel(const int8_t *in, const int8_t *alpha, int8_t *out, int64_t vecs,
+                                                              unsigned vecs_per_pixel, int shift)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= vecs)
+        return;
+    const unsigned cv = (unsigned)((uint64_t)i % vecs_per_pixel);
+    const v4i x = reinterpret_cast<const v4i *>(in)[i];
+    const v4i s = reinterpret_cast<const v4i *>(alpha)[cv];
+    const PreluFn f{nullptr, 1, shift};
+    v4i r;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        int o = 0;
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+            o |= (f.one((int)(int8_t)(x[w] >> (8 * b)), (int)(int8_t)(s[w] >> (8 * b))) & 0xff) << (8 * b);
+        r[w] = o;
+    }
+    reinterpret_cast<v4i *>(out)[i] = r;
+}
+} // namespace
+
 hipError_t launch_prelu_s8(const int8_t *in, int64_t pixels, int channels, const int8_t *alpha, int shift,
                            int8_t *out, hipStream_t stream)
 {
+    if (pixels > 0 && channels > 0 && (channels & 15) == 0 && aligned16(in, out) && aligned16(alpha, alpha)) {
+        const int64_t vecs = pixels * (channels / 16);
+        hipLaunchKernelGGL(prelu_s8_vec_kernel, dim3((unsigned)((vecs + kBlock - 1) / kBlock)), dim3(kBlock), 0, stream, in, alpha,
+                           out, vecs, (unsigned)(channels / 16), shift);
+        return hipGetLastError();
+    }
     return launch_map(in, out, pixels * channels, PreluFn{alpha, channels, shift}, stream);
 }
 

@@ -418,10 +418,12 @@ def test_prelu_s8(oracle, shift):
     got = to_host(m.prelu_s8(to_dev(x), to_dev(alpha), shift))
     np.testing.assert_array_equal(got, oracle.prelu_s8(x, alpha, shift))
     rng = np.random.default_rng(3)
-    x = rng_int8(rng, (1, 20, 20, 20))
-    alpha = rng_int8(rng, (20,))
-    got = to_host(m.prelu_s8(to_dev(x), to_dev(alpha), shift))
-    np.testing.assert_array_equal(got, oracle.prelu_s8(x, alpha, shift))
+    # 20 channels: the per-byte form; 48 and 256: 16 consecutive channels per thread
+    for shape in ((1, 20, 20, 20), (3, 9, 11, 48), (2, 5, 5, 256)):
+        x = rng_int8(rng, shape)
+        alpha = rng_int8(rng, (shape[-1],))
+        got = to_host(m.prelu_s8(to_dev(x), to_dev(alpha), shift))
+        np.testing.assert_array_equal(got, oracle.prelu_s8(x, alpha, shift))
 
 
 def test_relu_clip_requantize_s8(oracle):
