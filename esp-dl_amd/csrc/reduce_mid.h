@@ -8,7 +8,9 @@
 // t % G of the slab and the reduced positions t / G, t / G + PS, ... (PS = 256 / G): consecutive threads read
 // consecutive 16-byte pieces of one reduced position, then the next position, so a wavefront's loads are whole
 // contiguous runs whatever the inner size is - 16 channels or 1024 - and every lane has work when R is large.
-// Four loads are in flight per thread.  The partial sums of the PS position classes meet in LDS.
+// Four loads are in flight per thread.  The partial sums of the PS position classes meet in LDS.  With few outer
+// indices the slabs are made narrower (down to 8 pieces, one 128-byte line per position) until the grid has two
+// workgroups per compute unit: more workgroups, and more position classes in each, so fewer loads in a row per thread.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -19,7 +21,7 @@ namespace espdl {
 namespace reduce_mid {
 
 constexpr int kThreads = 256;
-constexpr int kSlabGroups = 64;
+constexpr int kSlabGroups = 64; // widest slab, in pieces
 
 template <typename T, int VEC>
 struct alignas(sizeof(T) * VEC) Piece { // one load instruction: 16 bytes in the wide form
@@ -27,15 +29,15 @@ struct alignas(sizeof(T) * VEC) Piece { // one load instruction: 16 bytes in the
 };
 
 template <typename T, int VEC, typename Fin>
-__global__ __launch_bounds__(kThreads) void sum_mid_kernel(const T *in, long long r_count, long long inner, Fin fin)
+__global__ __launch_bounds__(kThreads) void sum_mid_kernel(const T *in, long long r_count, long long inner, int slab, Fin fin)
 {
     __shared__ int partial[kThreads * VEC];
     const int tid = threadIdx.x;
     const long long groups_total = inner / VEC;
-    const int g_count = (int)min((long long)kSlabGroups, groups_total - (long long)blockIdx.x * kSlabGroups);
+    const int g_count = (int)min((long long)slab, groups_total - (long long)blockIdx.x * slab);
     const int ps = kThreads / g_count; // position classes
     const int g = tid % g_count, pl = tid / g_count;
-    const long long e0 = ((long long)blockIdx.x * kSlabGroups + g) * VEC; // first inner element of this thread
+    const long long e0 = ((long long)blockIdx.x * slab + g) * VEC; // first inner element of this thread
     const T *base = in + (long long)blockIdx.y * r_count * inner + e0;
     int sum[VEC];
 #pragma unroll
@@ -66,7 +68,7 @@ __global__ __launch_bounds__(kThreads) void sum_mid_kernel(const T *in, long lon
         int total = 0;
         for (int c = 0; c < ps; c++)
             total += partial[c * width + e];
-        fin((long long)blockIdx.y * inner + (long long)blockIdx.x * kSlabGroups * VEC + e, total);
+        fin((long long)blockIdx.y * inner + (long long)blockIdx.x * slab * VEC + e, total);
     }
 }
 
@@ -81,18 +83,24 @@ inline bool fits(long long outer, long long r_count, long long inner)
 
 // Launches the widest form the inner size and the address allow (16-byte pieces, else single elements).
 template <typename T, typename Fin>
-inline hipError_t launch(const T *in, long long outer, long long r_count, long long inner, Fin fin, hipStream_t stream)
+inline hipError_t launch(const T *in, long long outer, long long r_count, long long inner, Fin fin, hipStream_t stream,
+                         int cu_count = 256)
 {
     constexpr int kWide = 16 / (int)sizeof(T);
-    if (inner % kWide == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0) {
-        const long long slabs = (inner / kWide + kSlabGroups - 1) / kSlabGroups;
+    const bool wide = inner % kWide == 0 && (reinterpret_cast<uintptr_t>(in) & 15) == 0;
+    const long long groups = wide ? inner / kWide : inner;
+    // narrower slabs while the grid is under two workgroups per compute unit; a slab keeps whole 128-byte lines
+    int slab = kSlabGroups;
+    const int narrowest = wide ? 8 : kSlabGroups;
+    while (slab > narrowest && outer * ((groups + slab - 1) / slab) < 2ll * cu_count && groups > slab / 2)
+        slab /= 2;
+    const long long slabs = (groups + slab - 1) / slab;
+    if (wide)
         hipLaunchKernelGGL((sum_mid_kernel<T, kWide, Fin>), dim3((unsigned)slabs, (unsigned)outer), dim3(kThreads), 0, stream, in,
-                           r_count, inner, fin);
-    } else {
-        const long long slabs = (inner + kSlabGroups - 1) / kSlabGroups;
+                           r_count, inner, slab, fin);
+    else
         hipLaunchKernelGGL((sum_mid_kernel<T, 1, Fin>), dim3((unsigned)slabs, (unsigned)outer), dim3(kThreads), 0, stream, in,
-                           r_count, inner, fin);
-    }
+                           r_count, inner, slab, fin);
     return hipGetLastError();
 }
 
