@@ -23,7 +23,8 @@ struct SoftmaxArgs {
     long long outer, len, inner;
     int rows_per_block; // rows staged per workgroup (softmax axis innermost)
     int row_stride;     // padded LDS bytes per row
-    FastDiv fd_len;     // element index -> row, without an integer division per element
+    FastDiv fd_len;     // element (or dword, see vec4) index -> row, without an integer division per element
+    int vec4;           // rows are whole dwords at dword-aligned addresses: staged and stored four elements at a time
     float table[256];
 };
 
@@ -43,10 +44,19 @@ __global__ __launch_bounds__(kThreads) void softmax_s8_rows_kernel(const Softmax
          row0 += (long long)gridDim.x * a.rows_per_block) {
         const int rows_here = (int)min((long long)a.rows_per_block, n_rows - row0);
         const int8_t *src = a.in + row0 * len;
+        float *dst = a.out + row0 * len;
         __syncthreads(); // table ready / previous span consumed
-        for (int e = tid; e < rows_here * len; e += kThreads) {
-            const int r = (int)fastdiv((unsigned)e, a.fd_len);
-            rows[r * a.row_stride + (e - r * len)] = src[e];
+        if (a.vec4) { // rows of whole dwords at dword-aligned addresses: four elements per access
+            const int len4 = len >> 2;
+            for (int e = tid; e < rows_here * len4; e += kThreads) {
+                const int r = (int)fastdiv((unsigned)e, a.fd_len);
+                *reinterpret_cast<int *>(rows + r * a.row_stride + 4 * (e - r * len4)) = reinterpret_cast<const int *>(src)[e];
+            }
+        } else {
+            for (int e = tid; e < rows_here * len; e += kThreads) {
+                const int r = (int)fastdiv((unsigned)e, a.fd_len);
+                rows[r * a.row_stride + (e - r * len)] = src[e];
+            }
         }
         __syncthreads();
         if (tid < rows_here) {
@@ -70,10 +80,24 @@ __global__ __launch_bounds__(kThreads) void softmax_s8_rows_kernel(const Softmax
             sums[tid] = sum;
         }
         __syncthreads();
-        float *dst = a.out + row0 * len;
-        for (int e = tid; e < rows_here * len; e += kThreads) {
-            const int r = (int)fastdiv((unsigned)e, a.fd_len);
-            dst[e] = table[(int)rows[r * a.row_stride + (e - r * len)] + 128] / sums[r];
+        if (a.vec4) {
+            const int len4 = len >> 2;
+            for (int e = tid; e < rows_here * len4; e += kThreads) {
+                const int r = (int)fastdiv((unsigned)e, a.fd_len);
+                const int q = *reinterpret_cast<const int *>(rows + r * a.row_stride + 4 * (e - r * len4));
+                const float s = sums[r];
+                float4 o;
+                o.x = table[(int)(int8_t)q + 128] / s;
+                o.y = table[(int)(int8_t)(q >> 8) + 128] / s;
+                o.z = table[(int)(int8_t)(q >> 16) + 128] / s;
+                o.w = table[(q >> 24) + 128] / s;
+                reinterpret_cast<float4 *>(dst)[e] = o;
+            }
+        } else {
+            for (int e = tid; e < rows_here * len; e += kThreads) {
+                const int r = (int)fastdiv((unsigned)e, a.fd_len);
+                dst[e] = table[(int)rows[r * a.row_stride + (e - r * len)] + 128] / sums[r];
+            }
         }
     }
 }
@@ -275,9 +299,14 @@ hipError_t launch_softmax_s8(const int8_t *in, long long outer, long long len, l
     if (inner == 1 && (long long)stride * 8 <= lds_budget) {
         int rows = (int)min((long long)kThreads, lds_budget / stride);
         rows = (int)min((long long)rows, outer);
+        // fewer rows per workgroup while that leaves under two workgroups per compute unit (down to one wavefront
+        // of row sums): the staging and the divisions of several workgroups then overlap on a compute unit
+        while (rows > 64 && (outer + rows - 1) / rows < 2ll * max(1, cu_count))
+            rows = (rows + 1) / 2;
         a.rows_per_block = rows;
         a.row_stride = stride;
-        a.fd_len = make_fastdiv((unsigned)len);
+        a.vec4 = (len & 3) == 0 && (reinterpret_cast<uintptr_t>(in) & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+        a.fd_len = make_fastdiv((unsigned)(a.vec4 ? len / 4 : len));
         const size_t lds = 256 * sizeof(float) + (size_t)rows * sizeof(float) + (size_t)rows * stride;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(softmax_s8_rows_kernel),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
