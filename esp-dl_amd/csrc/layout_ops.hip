@@ -503,6 +503,20 @@ hipError_t launch_transpose(const void *in, const int *shape, int dims, const in
     if (n <= 1) // identity
         return hipMemcpyAsync(out, in, (size_t)(total * elem_size), hipMemcpyDeviceToDevice, stream);
 
+    if (s_perm[n - 1] == n - 1) {
+        // the innermost axis stays innermost: its runs move in the widest pieces their length and the addresses
+        // allow (one index decomposition per 16 bytes instead of per element)
+        const uintptr_t addr = reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out);
+        for (int wide = 16; wide > elem_size; wide >>= 1) {
+            const long long run = (long long)s_shape[n - 1] * elem_size;
+            if (run % wide == 0 && (addr & (uintptr_t)(wide - 1)) == 0) {
+                s_shape[n - 1] = (int)(run / wide);
+                total = total * elem_size / wide;
+                elem_size = wide;
+                break;
+            }
+        }
+    }
     TransposeArgs a = {};
     a.in = static_cast<const char *>(in);
     a.out = static_cast<char *>(out);
@@ -561,8 +575,12 @@ hipError_t launch_transpose(const void *in, const int *shape, int dims, const in
         hipLaunchKernelGGL(transpose_general_kernel<int8_t>, grid, dim3(kBlock), 0, stream, a);
     else if (elem_size == 2)
         hipLaunchKernelGGL(transpose_general_kernel<int16_t>, grid, dim3(kBlock), 0, stream, a);
-    else
+    else if (elem_size == 4)
         hipLaunchKernelGGL(transpose_general_kernel<int32_t>, grid, dim3(kBlock), 0, stream, a);
+    else if (elem_size == 8)
+        hipLaunchKernelGGL(transpose_general_kernel<long long>, grid, dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL(transpose_general_kernel<v4i>, grid, dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -730,8 +748,12 @@ hipError_t launch_slice(const void *in, const int *shape, int dims, const int *s
         hipLaunchKernelGGL(transpose_general_kernel<int8_t>, grid, dim3(kBlock), 0, stream, a);
     else if (elem_size == 2)
         hipLaunchKernelGGL(transpose_general_kernel<int16_t>, grid, dim3(kBlock), 0, stream, a);
-    else
+    else if (elem_size == 4)
         hipLaunchKernelGGL(transpose_general_kernel<int32_t>, grid, dim3(kBlock), 0, stream, a);
+    else if (elem_size == 8)
+        hipLaunchKernelGGL(transpose_general_kernel<long long>, grid, dim3(kBlock), 0, stream, a);
+    else
+        hipLaunchKernelGGL(transpose_general_kernel<v4i>, grid, dim3(kBlock), 0, stream, a);
     return hipGetLastError();
 }
 

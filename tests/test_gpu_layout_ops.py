@@ -58,6 +58,9 @@ def test_split(oracle, shape, axis, sizes, dtype):
     ((2, 20, 20, 64), (0, 3, 1, 2)), ((2, 64, 20, 20), (0, 2, 3, 1)), ((3, 5, 7, 9), None), ((37, 65), (1, 0)),
     ((4, 1, 1, 1280), (0, 3, 1, 2)), ((2, 3, 4, 5), (0, 1, 2, 3)), ((2, 3, 4, 5), (1, 0, 2, 3)),
     ((2, 2, 3, 2, 5), (4, 0, 3, 1, 2)), ((2, 3, 33, 40), (0, 1, 3, 2)), ((6,), (0,)), ((2, 3, 4), (-1, 0, 1)),
+    # the innermost axis stays innermost: its runs move in pieces of 16, 8, 4 or 2 bytes, by length and address
+    ((2, 6, 10, 16), (0, 2, 1, 3)), ((3, 4, 5, 24), (0, 2, 1, 3)), ((2, 5, 7, 12), (1, 0, 2, 3)), ((2, 2, 25, 40, 16), (0, 1, 3, 2, 4)),
+    ((2, 9, 3, 6), (2, 0, 1, 3)),
 ])
 def test_transpose(oracle, shape, perm, dtype):
     announce(f"transpose {shape} {perm} {dtype.__name__}")
