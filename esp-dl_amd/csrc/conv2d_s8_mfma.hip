@@ -86,7 +86,9 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     int ksc = a.n_kchunks == 1 ? pick_ksc(a.ksteps) : 0;
     if (bmode == B_GATHER)
         ksc = 0;
-    const int pt = (a.npix >= (long long)cus * 8 * 128 && ksc <= 12) ? 2 : 1;
+    // (with six or more resident k steps two pixel tiles take every register and leave one wavefront per SIMD:
+    // measured 2 to 4 % slower on whole YOLO11n graphs than one tile at two wavefronts per SIMD)
+    const int pt = (a.npix >= (long long)cus * 8 * 128 && ksc < 6) ? 2 : 1;
     a.n_sets = (int)((a.npix + 64 * pt - 1) / (64 * pt));
     // contiguous output: needs every filter group in one chunk, 4-byte aligned rows and room in LDS
     const size_t out_tiles = (size_t)4 * 16 * pt * g.out_c;
