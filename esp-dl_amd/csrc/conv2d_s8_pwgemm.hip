@@ -456,6 +456,20 @@ bool conv2d_s8_pwgemm_supports(const ConvGeom &g, const void *in, const void *fi
     return npix > 0 && (npix + 63) / 64 < (long long)cus * 16 && (npix + 63) / 64 <= 0x7fffffffll;
 }
 
+// The one-wavefront-per-tile kernel on its own: any filter count (a classifier with a handful of classes), K a
+// multiple of 64, fewer 64 x 64 tiles than compute units.
+bool conv2d_s8_rows_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count)
+{
+    const bool flat = g.k_h == 1 && g.k_w == 1 && g.stride_h == 1 && g.stride_w == 1 && g.pad_top == 0 &&
+        g.pad_left == 0 && g.out_h == g.in_h && g.out_w == g.in_w;
+    if (!flat || (g.in_c & 63) != 0 || g.out_c < 1 ||
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) != 0)
+        return false;
+    const long long npix = (long long)g.batch * g.out_h * g.out_w;
+    const int cus = cu_count > 0 ? cu_count : 256;
+    return npix > 0 && (npix + 63) / 64 * ((g.out_c + 63) / 64) < cus;
+}
+
 hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                    const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
                                    int cu_count, hipStream_t stream)

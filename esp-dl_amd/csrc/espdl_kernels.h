@@ -25,6 +25,7 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
 // Pointwise int8 convolution / Gemm as a tiled GEMM with both operands streamed through LDS; for layers
 // with few pixels per compute unit, where the implicit-GEMM kernel's filter staging dominates.
 bool conv2d_s8_pwgemm_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count);
+bool conv2d_s8_rows_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count);
 hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                    const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
                                    int cu_count, hipStream_t stream);

@@ -200,7 +200,8 @@ def test_gemm_s8(oracle, m, k, n, has_bias, relu):
 # Products with so few rows that the tiled kernels would leave most of the device idle go to a kernel with one
 # wavefront per 16 x 16 tile: ragged row and filter counts, byte stores (N not a multiple of 4), one shift for all
 # filters, shifts outside 1..31, both roundings.
-@pytest.mark.parametrize("m,k,n", [(256, 1280, 1000), (1, 1280, 1000), (70, 64, 37), (33, 576, 129), (512, 128, 32)])
+@pytest.mark.parametrize("m,k,n", [(256, 1280, 1000), (1, 1280, 1000), (70, 64, 37), (33, 576, 129), (512, 128, 32),
+                                   (32, 1280, 8), (5, 64, 1), (40, 128, 20)])
 @pytest.mark.parametrize("variant", ["per_channel", "per_tensor", "half_even", "wide_shifts"])
 def test_conv2d_s8_few_rows(oracle, m, k, n, variant):
     announce(f"conv2d_s8 few rows M={m} K={k} N={n} {variant}")
