@@ -8,7 +8,7 @@
 // t % G of the slab and the reduced positions t / G, t / G + PS, ... (PS = 256 / G): consecutive threads read
 // consecutive 16-byte pieces of one reduced position, then the next position, so a wavefront's loads are whole
 // contiguous runs whatever the inner size is - 16 channels or 1024 - and every lane has work when R is large.
-// Four loads are in flight per thread.  The partial sums of the PS position classes meet in LDS.  With few outer
+// Four loads are in flight per thread (eight where the grid is small and the sums long).  The partial sums of the PS position classes meet in LDS.  With few outer
 // indices the slabs are made narrower (down to 8 pieces, one 128-byte line per position) until the grid has two
 // workgroups per compute unit: more workgroups, and more position classes in each, so fewer loads in a row per thread.
 #pragma once
@@ -28,7 +28,8 @@ struct alignas(sizeof(T) * VEC) Piece { // one load instruction: 16 bytes in the
     T v[VEC];
 };
 
-template <typename T, int VEC, typename Fin>
+// U: loads in flight per thread (4; 8 when the grid has fewer workgroups than compute units and each has far to go).
+template <typename T, int VEC, int U, typename Fin>
 __global__ __launch_bounds__(kThreads) void sum_mid_kernel(const T *in, long long r_count, long long inner, int slab, Fin fin)
 {
     __shared__ int partial[kThreads * VEC];
@@ -45,13 +46,13 @@ __global__ __launch_bounds__(kThreads) void sum_mid_kernel(const T *in, long lon
         sum[k] = 0;
     if (pl < ps) {
         using P = Piece<T, VEC>;
-        for (long long r = pl; r < r_count; r += 4ll * ps) {
-            P p[4];
+        for (long long r = pl; r < r_count; r += (long long)U * ps) {
+            P p[U];
 #pragma unroll
-            for (int j = 0; j < 4; j++) // a position past the end reads the last one again and is not added
+            for (int j = 0; j < U; j++) // a position past the end reads the last one again and is not added
                 p[j] = *reinterpret_cast<const P *>(base + min(r + (long long)j * ps, r_count - 1) * inner);
 #pragma unroll
-            for (int j = 0; j < 4; j++)
+            for (int j = 0; j < U; j++)
                 if (r + (long long)j * ps < r_count) {
 #pragma unroll
                     for (int k = 0; k < VEC; k++)
@@ -95,12 +96,14 @@ inline hipError_t launch(const T *in, long long outer, long long r_count, long l
     while (slab > narrowest && outer * ((groups + slab - 1) / slab) < 2ll * cu_count && groups > slab / 2)
         slab /= 2;
     const long long slabs = (groups + slab - 1) / slab;
-    if (wide)
-        hipLaunchKernelGGL((sum_mid_kernel<T, kWide, Fin>), dim3((unsigned)slabs, (unsigned)outer), dim3(kThreads), 0, stream, in,
-                           r_count, inner, slab, fin);
+    const dim3 grid((unsigned)slabs, (unsigned)outer);
+    const bool deep = wide && outer * slabs < cu_count && r_count >= 64ll * kThreads; // few workgroups, long sums
+    if (deep)
+        hipLaunchKernelGGL((sum_mid_kernel<T, kWide, 8, Fin>), grid, dim3(kThreads), 0, stream, in, r_count, inner, slab, fin);
+    else if (wide)
+        hipLaunchKernelGGL((sum_mid_kernel<T, kWide, 4, Fin>), grid, dim3(kThreads), 0, stream, in, r_count, inner, slab, fin);
     else
-        hipLaunchKernelGGL((sum_mid_kernel<T, 1, Fin>), dim3((unsigned)slabs, (unsigned)outer), dim3(kThreads), 0, stream, in,
-                           r_count, inner, slab, fin);
+        hipLaunchKernelGGL((sum_mid_kernel<T, 1, 4, Fin>), grid, dim3(kThreads), 0, stream, in, r_count, inner, slab, fin);
     return hipGetLastError();
 }
 

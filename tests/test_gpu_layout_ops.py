@@ -149,7 +149,8 @@ def test_reduce_mean_s8_long_runs(oracle, shape, axes, keepdims, exps):
         np.testing.assert_array_equal(got, oracle.reduce_mean_s8(x, axes, keepdims, exps[0], exps[1]))
 
 
-@pytest.mark.parametrize("shape", [(2, 50, 60, 96), (3, 33, 31, 20), (2, 19, 23, 1040), (1, 120, 160, 16), (4, 9, 9, 8)],
+@pytest.mark.parametrize("shape", [(2, 50, 60, 96), (3, 33, 31, 20), (2, 19, 23, 1040), (1, 120, 160, 16), (4, 9, 9, 8),
+                                   (2, 131, 127, 64)],  # few workgroups and a long sum: eight loads in flight per thread
                          ids=lambda s: "x".join(map(str, s)))
 def test_global_avg_pool_s8_large_images(oracle, shape):
     announce(f"global_avg_pool_s8 large image {shape}")
