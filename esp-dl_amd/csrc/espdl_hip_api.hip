@@ -189,6 +189,10 @@ int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const 
             (lut == nullptr && residual == nullptr && espdl::conv2d_s8_rows_supports(g, in, filter, cu_count_cached())))
             return device_status(espdl::launch_conv2d_s8_pwgemm(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
                                  "conv2d_s8_pwgemm");
+        static const bool no_tiled = getenv("ESPDL_HIP_NO_TILED") != nullptr;
+        if (!no_tiled && espdl::conv2d_s8_tiled_supports(g, in, filter, cu_count_cached()))
+            return device_status(espdl::launch_conv2d_s8_tiled(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
+                                 "conv2d_s8_tiled");
         return device_status(espdl::launch_conv2d_s8_mfma(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
                              "conv2d_s8");
     }
@@ -926,12 +930,6 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
         return rc;
     if (p.batch == 0)
         return ESPDL_HIP_OK;
-    if (p.residual_shift != 0) {
-        const int kind = espdl_hip_mbconv_s8_supported(desc);
-        if (kind != 4 && kind != 5)
-            return fail(ESPDL_HIP_ENOTSUP, "a requantized residual operand (residual_shift %d) is not covered for this block shape",
-                        p.residual_shift);
-    }
     if (in == nullptr || out == nullptr || w == nullptr || w->w_dw == nullptr || w->s_dw == nullptr ||
         w->w_project == nullptr || w->s_project == nullptr || (desc->has_expand && (w->w_expand == nullptr || w->s_expand == nullptr)))
         return fail(ESPDL_HIP_EINVAL, "in, out, filters and shifts must not be NULL");
@@ -955,7 +953,7 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
         espdl::ConvGeom g;
         espdl::DwProject pj;
         dwproject_from(p, &g, &pj);
-        if (espdl::depthwise_project_s8_supports(g, p.in, pj))
+        if (p.residual_shift == 0 && espdl::depthwise_project_s8_supports(g, p.in, pj))
             return device_status(espdl::launch_depthwise_project_s8(g, p.in, p.w_dw, p.b_dw, p.s_dw, pj, cu_count_cached(),
                                                                     reinterpret_cast<hipStream_t>(stream)),
                                  "depthwise_project_s8");
@@ -972,6 +970,11 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
     if (desc->has_expand && espdl::mbconv_s8_wave_supports(p))
         return device_status(espdl::launch_mbconv_s8_wave(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
                              "mbconv_s8_wave");
+    // Only the two kernels above requantize the residual operand.  The answer comes from the real pointers: a
+    // block whose operands are merely 4-byte aligned can be refused by both although the shape alone passes.
+    if (p.residual_shift != 0)
+        return fail(ESPDL_HIP_ENOTSUP, "a requantized residual operand (residual_shift %d) is not covered for this block shape and operand alignment",
+                    p.residual_shift);
     if (desc->has_expand) {
         espdl::ConvGeom g;
         espdl::DwProject pj;

@@ -29,6 +29,27 @@ CONV_CASES = [
     ("c32_10x10_k3p1_oc64_relu", (10, 10, 32), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
 ]
 
+# Windowed convolutions whose channel count is a multiple of 16: the kernel that stages the input tile and the
+# filters in LDS.  Strides 1 to 3, dilation, reduction steps that span several taps (16, 32, 48 channels), several
+# groups of 64 filters in one and in several chunks, filter counts that are not a multiple of 64 / 16 / 4, images
+# wider than one column tile, ragged last tiles, padding on one side only, a window larger than the image.
+TILED_CASES = [
+    ("t64_30x30_k3p1_oc64", (30, 30, 64), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
+    ("t16_37x41_k3p1_oc16", (37, 41, 16), 16, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False),
+    ("t32_33x35_k3s2p1_oc64", (33, 35, 32), 64, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, True),
+    ("t48_20x20_k3p1_oc40", (20, 20, 48), 40, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False),
+    ("t128_18x18_k3p1_oc128", (18, 18, 128), 128, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
+    ("t64_24x24_k3p1_oc160", (24, 24, 64), 160, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False),
+    ("t16_21x300_k3s2p1_oc32", (21, 300, 16), 32, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, True),
+    ("t32_40x40_k5d2p4_oc33", (40, 40, 32), 33, (5, 5), (1, 1), (2, 2), (4, 4, 4, 4), True, False),
+    ("t16_26x26_k3s3_oc7", (26, 26, 16), 7, (3, 3), (3, 3), (1, 1), (0, 0, 0, 0), False, False),
+    ("t32_9x70_k1x7p3_oc64", (9, 70, 32), 64, (1, 7), (1, 1), (1, 1), (0, 0, 3, 3), True, True),
+    ("t64_5x5_k7p3_oc64", (5, 5, 64), 64, (7, 7), (1, 1), (1, 1), (3, 3, 3, 3), True, False),
+    ("t32_17x19_k3s2_tailpad_oc20", (17, 19, 32), 20, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), True, True),
+    ("t256_12x12_k3p1_oc64", (12, 12, 256), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False),
+    ("t16_64x200_k3p1_oc16", (64, 200, 16), 16, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
+]
+
 # BASELINE config 1: 1x56x56x64 -> 64, 3x3, s1, p1, bias, ReLU, shift 9
 CONFIG1 = ("config1_56x56x64_k3p1_relu", (56, 56, 64), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True)
 

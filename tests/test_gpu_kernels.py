@@ -5,7 +5,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, every_sum_image, rng_int8, typical_shift
+from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
 from gpu_util import announce, espdl, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
@@ -75,6 +75,32 @@ def test_conv2d_s8_config1_batched(oracle):
     announce("conv2d_s8 config1 batch 16")
     x, f, bias, _, k, stride, dil, pads, relu = _conv_inputs(CONFIG1, 0xE5D2, 16, False)
     got, want = _run_conv_s8(oracle, x, f, bias, 9, k, stride, dil, pads, True)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", TILED_CASES, ids=lambda c: c[0])
+@pytest.mark.parametrize("flavour", ["per_tensor", "per_channel", "half_even", "lut_residual", "general_epilogue"])
+def test_conv2d_s8_lds_tiled(oracle, case, flavour):
+    """Windowed convolutions with a multiple of 16 channels (input tile and filters staged in LDS): both exponent
+    forms, round-half-even, table + residual in the epilogue, and shifts outside 1..31 mixed with large biases
+    (the general shift-and-round form)."""
+    announce(f"conv2d_s8 lds-tiled {case[0]} {flavour}")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 211, 3, flavour != "per_tensor")
+    kw = {}
+    if flavour == "half_even":
+        kw["half_even"] = True
+    if flavour == "lut_residual":
+        kw["lut"] = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8)
+        kw["residual_seed"] = 9
+        relu = False
+    if flavour == "general_epilogue":
+        shift = np.array(shift, dtype=np.int32)
+        shift[::3] = 0
+        shift[1::5] = 33
+        if bias is not None:
+            bias = bias.copy()
+            bias[::2] = (1 << 30) - 7
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
     np.testing.assert_array_equal(got, want)
 
 
