@@ -108,8 +108,18 @@ __device__ __forceinline__ v4i weight_unit(const MfmaConvArgs &a, int gbase, int
     const int8_t *src = a.w + (size_t)oc * K + k;
     if ((K & 15) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15) == 0)
         return *reinterpret_cast<const v4i *>(src);
-    unsigned int words[4] = {0, 0, 0, 0};
     const int n = min(16, K - k);
+    if ((long long)oc * K + k + 16 <= (long long)OC * K) {
+        // 16 bytes from any address in one load; what lies past the filter's last position is cut off
+        v4i v = *reinterpret_cast<const v4i_unaligned *>(src);
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const int keep = min(max(n - 4 * d, 0), 4);
+            v[d] = keep >= 4 ? v[d] : (int)((unsigned)v[d] & ((1u << (8 * keep)) - 1u));
+        }
+        return v;
+    }
+    unsigned int words[4] = {0, 0, 0, 0};
     for (int b = 0; b < n; b++)
         words[b >> 2] |= (unsigned int)(unsigned char)src[b] << ((b & 3) * 8);
     return v4i{(int)words[0], (int)words[1], (int)words[2], (int)words[3]};
@@ -410,34 +420,36 @@ __device__ __forceinline__ void run_group(const MfmaConvArgs &a, const WaveCtx &
             continue;
         const long long goff = (long long)px[p].pix * OC + c_lane;
         int8_t *dst = a.out + goff;
-        if (NT == 4 && a.out_vec == 16) {
+        // Stores (and residual loads) take the widest piece that exists: 16 bytes when the lane's 16 channels do,
+        // else 4 bytes per filter tile, single bytes only for the last channels of a row.  No piece needs an
+        // aligned address, so a channel count that is not a multiple of 4 costs nothing but the row tails.
+        if (NT == 4 && c_lane + 16 <= OC) {
             v4i v = {words[0], words[NT > 1 ? 1 : 0], words[NT > 2 ? 2 : 0], words[NT > 3 ? 3 : 0]};
             if (a.res != nullptr) {
-                const v4i r = *reinterpret_cast<const v4i *>(a.res + goff);
+                const v4i r = *reinterpret_cast<const v4i_unaligned *>(a.res + goff);
 #pragma unroll
                 for (int d = 0; d < 4; d++)
                     v[d] = sat_add4_s8(v[d], r[d]);
             }
-            *reinterpret_cast<v4i *>(dst) = v;
-        } else if (a.out_vec >= 4) {
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-                if (c_lane + 4 * t < OC) {
-                    int v = words[t];
-                    if (a.res != nullptr)
-                        v = sat_add4_s8(v, *reinterpret_cast<const int *>(a.res + goff + 4 * t));
-                    *reinterpret_cast<int *>(dst + 4 * t) = v;
-                }
+            *reinterpret_cast<v4i_unaligned *>(dst) = v;
         } else {
 #pragma unroll
-            for (int t = 0; t < NT; t++)
-                for (int r = 0; r < 4; r++)
-                    if (c_lane + 4 * t + r < OC) {
-                        int v = (int)(int8_t)(words[t] >> (8 * r));
-                        if (a.res != nullptr)
-                            v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
-                        dst[4 * t + r] = (int8_t)v;
-                    }
+            for (int t = 0; t < NT; t++) {
+                if (c_lane + 4 * t + 4 <= OC) {
+                    int v = words[t];
+                    if (a.res != nullptr)
+                        v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(a.res + goff + 4 * t));
+                    *reinterpret_cast<int_unaligned *>(dst + 4 * t) = v;
+                } else {
+                    for (int r = 0; r < 4; r++)
+                        if (c_lane + 4 * t + r < OC) {
+                            int v = (int)(int8_t)(words[t] >> (8 * r));
+                            if (a.res != nullptr)
+                                v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
+                            dst[4 * t + r] = (int8_t)v;
+                        }
+                }
+            }
         }
     }
 }

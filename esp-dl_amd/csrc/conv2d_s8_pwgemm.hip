@@ -12,7 +12,9 @@
 // k steps of 64 with a register/LDS double buffer, so the first MFMA starts after one k step:
 //   workgroup tile = 64*PT pixels x 64*NG filters, 4 wavefronts, wavefront = 16*PT pixels x all filters;
 //   per k step: 64*PT x 64 B of pixels and 64*NG x 64 B of filters go global -> registers (one step
-//   ahead) -> LDS rows of 80 bytes (odd number of 16-byte units: conflict-free operand reads);
+//   ahead) -> LDS rows of 96 bytes (a 16-byte-per-lane read is served in groups of 8 rows x 2 neighbouring
+//   quarters; with a row pitch of twice an odd number of 16-byte units the 16 pieces of a group fall into
+//   different bank sets, which a pitch of 80 bytes does not achieve);
 //   one barrier per k step; MFMA operands are plain 16-byte LDS reads.
 // The filter -> tile-row permutation (row i of tile t is filter 16*(i/4) + 4*t + i%4 of the group)
 // leaves every lane with 16 consecutive output channels per pixel: one 16-byte store.
@@ -26,7 +28,7 @@ namespace espdl {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kRow = 80;    // LDS row: 64 k bytes + 16
+constexpr int kRow = 96;    // LDS row: 64 k bytes + 32
 
 struct PwArgs {
     const int8_t *in;  // [M][K]
@@ -81,22 +83,49 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     const int n0 = blockIdx.y * TN;
     const bool relu = a.relu != 0, half_even = a.half_even != 0, has_lut = a.lut != nullptr;
 
-    // piece p of a tile: row p / 4, 16-byte quarter p % 4 of the 64-byte k step
+    // piece p of a tile: row p / 4, 16-byte quarter p % 4 of the 64-byte k step.  Rows whose length is not a
+    // multiple of 16 (a Gemm over 120 features) are read with loads that need no alignment; the one piece that
+    // holds a row's last n < 16 bytes is read as the 16 bytes that END at the row's end and shifted down, so
+    // that nothing past a row (and so nothing past the tensor) is touched and the piece ends in zeros.
+    const bool k16 = (a.K & 15) == 0; // uniform
+    auto piece = [&](const int8_t *row, int k) -> v4i {
+        if (k16)
+            return k < a.K ? *reinterpret_cast<const v4i *>(row + k) : v4i{0, 0, 0, 0};
+        if (k >= a.K)
+            return v4i{0, 0, 0, 0};
+        if (k + 16 <= a.K)
+            return *reinterpret_cast<const v4i_unaligned *>(row + k);
+        const v4i v = *reinterpret_cast<const v4i_unaligned *>(row + a.K - 16);
+        const int sh = 16 - (a.K & 15); // uniform: bytes to shift down, 1..15
+        const int d = sh >> 2;
+        const unsigned b = (unsigned)(sh & 3);
+        const int w[8] = {v[0], v[1], v[2], v[3], 0, 0, 0, 0};
+        v4i r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int lo = 0, hi = 0;
+#pragma unroll
+            for (int j = 0; j < 4; j++) { // d is uniform: these are scalar choices
+                lo = d == j ? w[i + j] : lo;
+                hi = d == j ? w[i + j + 1] : hi;
+            }
+            r[i] = (int)__builtin_amdgcn_alignbyte((unsigned)hi, (unsigned)lo, b);
+        }
+        return r;
+    };
     auto fetch = [&](int ks, v4i(&pb)[kPiecesB], v4i(&pa)[kPiecesA]) {
         const int k0 = 64 * ks;
 #pragma unroll
         for (int j = 0; j < kPiecesB; j++) {
             const int p = tid + j * kThreads;
             const long long m = row_pixel(p >> 2);
-            const int k = k0 + 16 * (p & 3);
-            pb[j] = (m >= 0 && k < a.K) ? *reinterpret_cast<const v4i *>(a.in + m * a.K + k) : v4i{0, 0, 0, 0};
+            pb[j] = m >= 0 ? piece(a.in + m * a.K, k0 + 16 * (p & 3)) : v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int j = 0; j < kPiecesA; j++) {
             const int p = tid + j * kThreads;
             const int n = n0 + (p >> 2);
-            const int k = k0 + 16 * (p & 3);
-            pa[j] = (n < a.N && k < a.K) ? *reinterpret_cast<const v4i *>(a.w + (long long)n * a.K + k) : v4i{0, 0, 0, 0};
+            pa[j] = n < a.N ? piece(a.w + (long long)n * a.K, k0 + 16 * (p & 3)) : v4i{0, 0, 0, 0};
         }
     };
     auto stash = [&](int buf, const v4i(&pb)[kPiecesB], const v4i(&pa)[kPiecesA]) {
@@ -244,34 +273,38 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
                 if (m >= a.M || n >= a.N)
                     continue;
                 const long long goff = m * a.N + n;
-                if (a.out_vec == 16 && n + 16 <= a.N) {
+                // the widest piece that exists, at any byte address: 16 bytes, else 4 per filter tile, bytes for
+                // the last channels of a row (a row length that is not a multiple of 4 costs only those)
+                if (n + 16 <= a.N) {
                     v4i v = {words[0], words[1], words[2], words[3]};
                     if (a.res != nullptr) {
-                        const v4i r = *reinterpret_cast<const v4i *>(a.res + goff);
+                        const v4i r = *reinterpret_cast<const v4i_unaligned *>(a.res + goff);
     #pragma unroll
                         for (int d = 0; d < 4; d++)
                             v[d] = sat_add4_s8(v[d], r[d]);
                     }
-                    __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(a.out + goff));
-                } else if (a.out_vec >= 4) {
+                    if (a.out_vec == 16)
+                        __builtin_nontemporal_store(v, reinterpret_cast<v4i *>(a.out + goff));
+                    else
+                        *reinterpret_cast<v4i_unaligned *>(a.out + goff) = v;
+                } else {
     #pragma unroll
-                    for (int t = 0; t < 4; t++)
+                    for (int t = 0; t < 4; t++) {
                         if (n + 4 * t + 4 <= a.N) {
                             int v = words[t];
                             if (a.res != nullptr)
-                                v = sat_add4_s8(v, *reinterpret_cast<const int *>(a.res + goff + 4 * t));
-                            *reinterpret_cast<int *>(a.out + goff + 4 * t) = v;
+                                v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(a.res + goff + 4 * t));
+                            *reinterpret_cast<int_unaligned *>(a.out + goff + 4 * t) = v;
+                        } else {
+                            for (int r = 0; r < 4; r++)
+                                if (n + 4 * t + r < a.N) {
+                                    int v = (int)(int8_t)(words[t] >> (8 * r));
+                                    if (a.res != nullptr)
+                                        v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
+                                    a.out[goff + 4 * t + r] = (int8_t)v;
+                                }
                         }
-                } else {
-    #pragma unroll
-                    for (int t = 0; t < 4; t++)
-                        for (int r = 0; r < 4; r++)
-                            if (n + 4 * t + r < a.N) {
-                                int v = (int)(int8_t)(words[t] >> (8 * r));
-                                if (a.res != nullptr)
-                                    v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
-                                a.out[goff + 4 * t + r] = (int8_t)v;
-                            }
+                    }
                 }
             }
         }
@@ -442,17 +475,24 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_rows_kernel(const PwArgs a
 
 } // namespace
 
-// Flat pointwise geometry with 16-byte aligned rows; worth it when a workgroup of the implicit-GEMM
+// Flat pointwise geometry; worth it when a workgroup of the implicit-GEMM
 // kernel would see only a few pixel sets.
 bool conv2d_s8_pwgemm_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count)
 {
     const bool flat = g.k_h == 1 && g.k_w == 1 && g.stride_h == 1 && g.stride_w == 1 && g.pad_top == 0 &&
         g.pad_left == 0 && g.out_h == g.in_h && g.out_w == g.in_w;
-    if (!flat || (g.in_c & 15) != 0 || g.in_c < 64 || g.out_c < 32 ||
-        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) != 0)
+    if (!flat || g.in_c < 64 || g.out_c < 32)
+        return false;
+    // rows of a multiple of 16 bytes are read with aligned loads; any other length with loads that need none
+    if ((g.in_c & 15) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) != 0)
         return false;
     const long long npix = (long long)g.batch * g.out_h * g.out_w;
     const int cus = cu_count > 0 ? cu_count : 256;
+    // A short reduction under thousands of filters (a recognizer's 120 -> 6625 classifier) is bound by writing
+    // the output: the implicit-GEMM kernel, whose wavefronts keep their pixels' operands in registers and write
+    // several hundred contiguous bytes per pixel, does that faster (76 against 112 us on 20480 x 120 x 6625).
+    if (g.in_c <= 128 && g.out_c >= 2048 && npix >= 64ll * cus)
+        return false;
     return npix > 0 && (npix + 63) / 64 < (long long)cus * 16 && (npix + 63) / 64 <= 0x7fffffffll;
 }
 

@@ -221,34 +221,34 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
         if (!ok)
             continue;
         int8_t *dst = out_img + (size_t)go;
-        if (EPI == 1 || (NT == 4 && a.out_vec == 16)) {
+        // the widest piece that exists, at any byte address: 16 bytes, else 4 per filter tile, bytes for a row's tail
+        if (EPI == 1 || (NT == 4 && c_lane + 16 <= OC)) {
             v4i v = {words[0], words[NT > 1 ? 1 : 0], words[NT > 2 ? 2 : 0], words[NT > 3 ? 3 : 0]};
             if (res_img != nullptr) {
-                const v4i r = *reinterpret_cast<const v4i *>(res_img + (size_t)go);
+                const v4i r = *reinterpret_cast<const v4i_unaligned *>(res_img + (size_t)go);
 #pragma unroll
                 for (int d = 0; d < 4; d++)
                     v[d] = sat_add4_s8(v[d], r[d]);
             }
-            *reinterpret_cast<v4i *>(dst) = v;
-        } else if (a.out_vec >= 4) {
-#pragma unroll
-            for (int t = 0; t < NT; t++)
-                if (c_lane + 4 * t < OC) {
-                    int v = words[t];
-                    if (res_img != nullptr)
-                        v = sat_add4_s8(v, *reinterpret_cast<const int *>(res_img + (size_t)go + 4 * t));
-                    *reinterpret_cast<int *>(dst + 4 * t) = v;
-                }
+            *reinterpret_cast<v4i_unaligned *>(dst) = v;
         } else {
 #pragma unroll
-            for (int t = 0; t < NT; t++)
-                for (int r = 0; r < 4; r++)
-                    if (c_lane + 4 * t + r < OC) {
-                        int v = (int)(int8_t)(words[t] >> (8 * r));
-                        if (res_img != nullptr)
-                            v = clamp_s8(v + (int)res_img[(size_t)go + 4 * t + r]);
-                        dst[4 * t + r] = (int8_t)v;
-                    }
+            for (int t = 0; t < NT; t++) {
+                if (c_lane + 4 * t + 4 <= OC) {
+                    int v = words[t];
+                    if (res_img != nullptr)
+                        v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(res_img + (size_t)go + 4 * t));
+                    *reinterpret_cast<int_unaligned *>(dst + 4 * t) = v;
+                } else {
+                    for (int r = 0; r < 4; r++)
+                        if (c_lane + 4 * t + r < OC) {
+                            int v = (int)(int8_t)(words[t] >> (8 * r));
+                            if (res_img != nullptr)
+                                v = clamp_s8(v + (int)res_img[(size_t)go + 4 * t + r]);
+                            dst[4 * t + r] = (int8_t)v;
+                        }
+                }
+            }
         }
     }
 }

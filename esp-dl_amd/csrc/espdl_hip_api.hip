@@ -185,7 +185,8 @@ int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const 
             return device_status(espdl::launch_depthwise_s8(g, i8, f8, b32, shift, lut, o8, s), "depthwise_s8");
         }
         // (the second test admits products with fewer than 32 filters, which only the few-rows kernel inside takes)
-        if (espdl::conv2d_s8_pwgemm_supports(g, in, filter, cu_count_cached()) ||
+        static const bool no_pw = getenv("ESPDL_HIP_NO_PWGEMM") != nullptr;
+        if (!no_pw && espdl::conv2d_s8_pwgemm_supports(g, in, filter, cu_count_cached()) ||
             (lut == nullptr && residual == nullptr && espdl::conv2d_s8_rows_supports(g, in, filter, cu_count_cached())))
             return device_status(espdl::launch_conv2d_s8_pwgemm(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
                                  "conv2d_s8_pwgemm");
