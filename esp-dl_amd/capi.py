@@ -33,7 +33,8 @@ class MbconvDesc(ctypes.Structure):
         "dil_h", "dil_w", "pad_top", "pad_bottom", "pad_left", "pad_right", "act_expand", "act_dw", "act_project",
         "round_mode", "n_shift_expand", "n_shift_dw", "n_shift_project",
         "exp_k_h", "exp_k_w", "exp_stride_h", "exp_stride_w", "exp_pad_top", "exp_pad_bottom", "exp_pad_left",
-        "exp_pad_right", "residual_shift")]
+        "exp_pad_right", "residual_shift", "clip_expand", "clip_expand_min", "clip_expand_max", "clip_dw",
+        "clip_dw_min", "clip_dw_max")]
 
 
 class MbconvWeights(ctypes.Structure):
@@ -203,7 +204,7 @@ def conv2d_gap_s8(x, filt, bias, shift, conv_out_exp, pool_out_exp, activation=L
 
 def mbconv_s8(x, expand, dw, project, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), relus=(True, True, False),
               residual=None, round_mode=ROUND_HALF_UP, out=None, stream=None, staged=False, expand_conv=None,
-              residual_shift=0):
+              residual_shift=0, clip_expand=None, clip_dw=None):
     """Fused inverted-residual block (staged=True: espdl_hip_mbconv_s8_staged, the separate stages with the
     intermediates in the library's own device array; `out` must then be given, nothing is allocated).  expand / dw / project are (filter, bias, shift) triples of CUDA
     tensors (expand may be None); filters as for conv2d: [E][C], [kH][kW][E], [OC][E].
@@ -225,6 +226,10 @@ def mbconv_s8(x, expand, dw, project, k, stride=(1, 1), dilation=(1, 1), pads=(0
         (desc.exp_k_h, desc.exp_k_w, desc.exp_stride_h, desc.exp_stride_w) = (ek[0], ek[1], es[0], es[1])
         (desc.exp_pad_top, desc.exp_pad_bottom, desc.exp_pad_left, desc.exp_pad_right) = ep
     desc.residual_shift = residual_shift
+    if clip_expand is not None:  # (min, max): Clip with equal exponents behind the expand stage
+        desc.clip_expand, desc.clip_expand_min, desc.clip_expand_max = 1, clip_expand[0], clip_expand[1]
+    if clip_dw is not None:
+        desc.clip_dw, desc.clip_dw_min, desc.clip_dw_max = 1, clip_dw[0], clip_dw[1]
     oh, ow = ctypes.c_int32(), ctypes.c_int32()
     _check(lib().espdl_hip_mbconv_out_shape(ctypes.byref(desc), ctypes.byref(oh), ctypes.byref(ow)))
     if out is None:

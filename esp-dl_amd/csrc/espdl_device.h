@@ -126,8 +126,12 @@ __device__ __forceinline__ int half_even_add(int acc, int s)
 // where the first saturation acts (|acc| >= 2^15, l >= 0) the second one does too.
 // MODE 5: half-even for accumulators that hold bias + 2^(s-1) - 1 (half_even_add), with the left shift.
 // MODE 6: the same where every shift is at least 8.
-template <int MODE>
-__device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk)
+// CEIL: the int8 result is also clamped from above (a Clip between two stages): ceil_pk holds the upper bound
+// twice as int16 in the same fixed-point form, (max << 8) | 0xff, one packed minimum per pair.  floor_pk is
+// then (max(lower bound, 0 for ReLU) << 8) & 0xffff twice.
+template <int MODE, bool CEIL = false>
+__device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const v4i &rsh, int floor_pk,
+                                          int ceil_pk = 0x7fff7fff)
 {
     if constexpr (MODE == 4) {
         const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
@@ -135,6 +139,10 @@ __device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const 
         v2s p23 = __builtin_amdgcn_cvt_pk_i16(acc[2] >> rsh[2], acc[3] >> rsh[3]);
         p01 = __builtin_elementwise_max(pk_mul_sat_i16(p01, lsh[0]), floor2);
         p23 = __builtin_elementwise_max(pk_mul_sat_i16(p23, lsh[1]), floor2);
+        if constexpr (CEIL) {
+            p01 = __builtin_elementwise_min(p01, __builtin_bit_cast(v2s, ceil_pk));
+            p23 = __builtin_elementwise_min(p23, __builtin_bit_cast(v2s, ceil_pk));
+        }
         return (int)__builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, p23), (unsigned)__builtin_bit_cast(int, p01),
                                           0x07050301u);
     }
@@ -151,8 +159,12 @@ __device__ __forceinline__ int pack_fast4(const v4i &acc, const v4i &lsh, const 
     }
     // floor_pk holds the lower clamp twice as int16: 0 for ReLU, -32768 (no effect) otherwise
     const v2s floor2 = __builtin_bit_cast(v2s, floor_pk);
-    const v2s p01 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(t[0], t[1]), floor2);
-    const v2s p23 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(t[2], t[3]), floor2);
+    v2s p01 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(t[0], t[1]), floor2);
+    v2s p23 = __builtin_elementwise_max(__builtin_amdgcn_cvt_pk_i16(t[2], t[3]), floor2);
+    if constexpr (CEIL) {
+        p01 = __builtin_elementwise_min(p01, __builtin_bit_cast(v2s, ceil_pk));
+        p23 = __builtin_elementwise_min(p23, __builtin_bit_cast(v2s, ceil_pk));
+    }
     return (int)__builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, p23), (unsigned)__builtin_bit_cast(int, p01),
                                       0x07050301u);
 }

@@ -778,6 +778,21 @@ int mbconv_geometry(const espdl_hip_mbconv_desc *d, espdl::MbconvParams *p)
     if (d->residual_shift < -7 || d->residual_shift > 7)
         return fail(ESPDL_HIP_EINVAL, "residual_shift %d outside [-7, 7]", d->residual_shift);
     p->residual_shift = d->residual_shift;
+    for (int st = 0; st < 2; st++) {
+        const int on = st == 0 ? d->clip_expand : d->clip_dw;
+        const int lo = st == 0 ? d->clip_expand_min : d->clip_dw_min, hi = st == 0 ? d->clip_expand_max : d->clip_dw_max;
+        if (on != 0 && (lo < -128 || hi > 127 || lo > hi))
+            return fail(ESPDL_HIP_EINVAL, "clip bounds [%d, %d] of the %s stage outside int8 or empty", lo, hi,
+                        st == 0 ? "expand" : "depthwise");
+    }
+    if (d->clip_expand != 0 && !d->has_expand)
+        return fail(ESPDL_HIP_EINVAL, "clip_expand without an expand stage");
+    p->clip_e = d->clip_expand != 0;
+    p->clip_e_lo = d->clip_expand_min;
+    p->clip_e_hi = d->clip_expand_max;
+    p->clip_d = d->clip_dw != 0;
+    p->clip_d_lo = d->clip_dw_min;
+    p->clip_d_hi = d->clip_dw_max;
     if ((long long)p->batch * p->out_h * p->out_w > 0x7fffffffll - 65536)
         return fail(ESPDL_HIP_EINVAL, "too many output pixels");
     return ESPDL_HIP_OK;
@@ -876,6 +891,9 @@ static int mbconv_kernel_choice(const espdl_hip_mbconv_desc *desc)
     p.w_expand = desc->has_expand ? aligned : nullptr;
     p.w_dw = aligned;
     p.w_project = aligned;
+    // a clamp between the stages: the guard-free builds of the one-wavefront-per-tile kernel only
+    if (espdl::mbconv_has_clip(p))
+        return (desc->has_expand && espdl::mbconv_s8_wave_has_fast_build(p)) ? 4 : 0;
     if (!desc->has_expand) {
         espdl::ConvGeom g;
         espdl::DwProject pj;
@@ -950,6 +968,12 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
     p.w_project = w->w_project;
     p.b_project = w->b_project;
     p.s_project = w->s_project;
+    if (espdl::mbconv_has_clip(p)) {
+        if (!desc->has_expand || !espdl::mbconv_s8_wave_has_fast_build(p))
+            return fail(ESPDL_HIP_ENOTSUP, "a Clip between the stages is covered for the block shapes with a guard-free build of the one-wavefront-per-tile kernel, round half up");
+        return device_status(espdl::launch_mbconv_s8_wave(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
+                             "mbconv_s8_wave");
+    }
     if (!desc->has_expand) {
         espdl::ConvGeom g;
         espdl::DwProject pj;
@@ -961,7 +985,7 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
     }
     if (desc->has_expand && !pointwise_expand(p)) {
         if (!espdl::mbconv_s8_wave_supports(p))
-            return fail(ESPDL_HIP_ENOTSUP, "an expand stage with a window needs a 3x3 depthwise stage, at most 4 filter rows of at most 16 bytes (exp_k_w * in_c) and at most 64 project filters");
+            return fail(ESPDL_HIP_ENOTSUP, "an expand stage with a window needs a 3x3 depthwise stage, at most 4 filter rows of at most 9 bytes (exp_k_w * in_c) and at most 64 project filters");
         return device_status(espdl::launch_mbconv_s8_wave(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
                              "mbconv_s8_wave");
     }

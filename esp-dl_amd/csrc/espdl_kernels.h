@@ -102,7 +102,14 @@ struct MbconvParams {
     // a RequantizeLinear between two int8 exponents in front of the Add.  -7 .. 7; only the one-wavefront-per-tile
     // and the workgroup-per-tile kernels take a value other than 0.
     int residual_shift;
+    // Clamp of a stage's int8 result before the next stage reads it (a Clip with equal exponents between the
+    // stages); only the guard-free builds of the one-wavefront-per-tile kernel take it.
+    int clip_e, clip_e_lo, clip_e_hi, clip_d, clip_d_lo, clip_d_hi;
 };
+inline bool mbconv_has_clip(const MbconvParams &p)
+{
+    return p.clip_e != 0 || p.clip_d != 0;
+}
 inline bool mbconv_expand_is_pointwise(const MbconvParams &p)
 {
     return p.ek_h == 1 && p.ek_w == 1 && p.es_h == 1 && p.es_w == 1 && p.epad_top == 0 && p.epad_left == 0 &&

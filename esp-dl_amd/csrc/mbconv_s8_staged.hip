@@ -80,6 +80,18 @@ extern "C" int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *d, const 
                                 "(ESPDL_HIP_MBCONV_STAGED_MAX_BYTES): use a smaller batch per call",
                                 expanded + dw_out, kScratchBytes);
     hipError_t err = hipSuccess;
+    {
+        // The array's address is looked up on the first call on a device, which may load the code object: not
+        // something to do while `stream` records a graph.  One call (or espdl_hip_mbconv_s8_staged_init) outside
+        // capture comes first.
+        int dev = -1;
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < kMaxDevices && g_scratch_ptr[dev] == nullptr &&
+            hipStreamIsCapturing(reinterpret_cast<hipStream_t>(stream), &capturing) == hipSuccess &&
+            capturing != hipStreamCaptureStatusNone)
+            return espdl::set_error(ESPDL_HIP_ENOTSUP, "the first espdl_hip_mbconv_s8_staged call on a device must not be "
+                                                       "under stream capture: call espdl_hip_mbconv_s8_staged_init first");
+    }
     unsigned char *base = scratch_of_current_device(&err);
     if (base == nullptr)
         return espdl::set_error(ESPDL_HIP_EDEVICE, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(err));
@@ -111,6 +123,9 @@ extern "C" int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *d, const 
         c.round_mode = d->round_mode;
         c.n_shift = d->n_shift_expand;
         rc = espdl_hip_conv2d(&c, in, w->w_expand, w->b_expand, w->s_expand, nullptr, t_expand, stream);
+        if (rc == ESPDL_HIP_OK && d->clip_expand != 0) // a Clip with equal exponents: in place on the intermediate
+            rc = espdl_hip_clip_s8(t_expand, (int64_t)d->batch * mid_h * mid_w * d->exp_c, d->clip_expand_min,
+                                   d->clip_expand_max, 0, 0, t_expand, stream);
         if (rc != ESPDL_HIP_OK)
             return rc;
         dw_in = t_expand;
@@ -138,6 +153,9 @@ extern "C" int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *d, const 
         c.round_mode = d->round_mode;
         c.n_shift = d->n_shift_dw;
         rc = espdl_hip_conv2d(&c, dw_in, w->w_dw, w->b_dw, w->s_dw, nullptr, t_dw, stream);
+        if (rc == ESPDL_HIP_OK && d->clip_dw != 0)
+            rc = espdl_hip_clip_s8(t_dw, (int64_t)d->batch * out_h * out_w * d->exp_c, d->clip_dw_min, d->clip_dw_max, 0, 0,
+                                   t_dw, stream);
         if (rc != ESPDL_HIP_OK)
             return rc;
     }
@@ -154,4 +172,12 @@ extern "C" int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *d, const 
     c.round_mode = d->round_mode;
     c.n_shift = d->n_shift_project;
     return espdl_hip_conv2d_add(&c, t_dw, w->w_project, w->b_project, w->s_project, nullptr, residual, out, stream);
+}
+
+extern "C" int espdl_hip_mbconv_s8_staged_init(void)
+{
+    hipError_t err = hipSuccess;
+    if (scratch_of_current_device(&err) == nullptr)
+        return espdl::set_error(ESPDL_HIP_EDEVICE, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(err));
+    return ESPDL_HIP_OK;
 }

@@ -207,28 +207,35 @@ __device__ __forceinline__ StageConsts read_stage_table(const int *tab, int n_ch
     return c;
 }
 
-template <int MODE>
-__device__ __forceinline__ int wave_pack(const v4i &acc, const StageConsts &c, int floor_pk, bool relu, bool half_even)
+// CLIP: a Clip sits behind the stage; floor_pk / ceil_pk carry its bounds (see pack_fast4), the general form
+// reads them back out of the packed words.
+template <int MODE, bool CLIP = false>
+__device__ __forceinline__ int wave_pack(const v4i &acc, const StageConsts &c, int floor_pk, bool relu, bool half_even,
+                                         int ceil_pk = 0x7fff7fff)
 {
     if constexpr (MODE >= 0) {
-        return pack_fast4<MODE>(acc, c.lsh, c.rsh, floor_pk);
+        return pack_fast4<MODE, CLIP>(acc, c.lsh, c.rsh, floor_pk, ceil_pk);
     } else {
         int q[4];
 #pragma unroll
-        for (int r = 0; r < 4; r++)
+        for (int r = 0; r < 4; r++) {
             q[r] = requant_s8(acc[r], c.rsh[r], relu, half_even);
+            if constexpr (CLIP)
+                q[r] = min(max(q[r], (int)(short)(floor_pk & 0xffff) >> 8), (int)(short)(ceil_pk & 0xffff) >> 8);
+        }
         return pack4_s8(q[0], q[1], q[2], q[3]);
     }
 }
 
 // The same for constants that came from read_stage_table: in mode 1 they carry multipliers, not shift counts.
-template <int MODE>
-__device__ __forceinline__ int wave_pack_tab(const v4i &acc, const StageConsts &c, int floor_pk, bool relu, bool half_even)
+template <int MODE, bool CLIP = false>
+__device__ __forceinline__ int wave_pack_tab(const v4i &acc, const StageConsts &c, int floor_pk, bool relu, bool half_even,
+                                             int ceil_pk = 0x7fff7fff)
 {
     if constexpr (MODE == 1)
-        return pack_fast4<4>(acc, c.lsh, c.rsh, floor_pk);
+        return pack_fast4<4, CLIP>(acc, c.lsh, c.rsh, floor_pk, ceil_pk);
     else
-        return wave_pack<MODE>(acc, c, floor_pk, relu, half_even);
+        return wave_pack<MODE, CLIP>(acc, c, floor_pk, relu, half_even, ceil_pk);
 }
 
 // Expand stage of one chunk of 16 channels: every patch pixel tile through one MFMA and the epilogue, four
@@ -238,11 +245,11 @@ __device__ __forceinline__ int wave_pack_tab(const v4i &acc, const StageConsts &
 // hold PACK pixel tiles (tile PACK g + t in the groups t * 4 / PACK ...), so the patch takes 1 / PACK of the
 // registers and of the loads; operand A comes in PACK copies, copy t holding the filter in the groups of tile t
 // and zeros elsewhere, which picks tile t out of the reduction.
-template <int MODE, int NXPT, bool EXACT, int KSE = 1, bool PIPE = false, int PACK = 1>
+template <int MODE, int NXPT, bool EXACT, int KSE = 1, bool PIPE = false, int PACK = 1, bool CLIP = false>
 __device__ __forceinline__ void expand_chunk(const v4i (&xb)[PACK > 1 ? (NXPT + PACK - 1) / PACK : NXPT * KSE], int n_xpt,
                                              unsigned xmask, const v4i (&aop)[PACK > 1 ? PACK : KSE], const StageConsts &c,
                                              int floor_pk, bool relu, bool half_even,
-                                             unsigned char *dst /* exp_l + col * 16 + 4 * quad */)
+                                             unsigned char *dst /* exp_l + col * 16 + 4 * quad */, int ceil_pk = 0x7fff7fff)
 {
     auto product = [&](int pt) -> v4i {
         v4i acc = c.init;
@@ -256,7 +263,7 @@ __device__ __forceinline__ void expand_chunk(const v4i (&xb)[PACK > 1 ? (NXPT + 
         return acc;
     };
     auto finish = [&](const v4i &acc, int pt) {
-        int word = wave_pack_tab<MODE>(acc, c, floor_pk, relu, half_even);
+        int word = wave_pack_tab<MODE, CLIP>(acc, c, floor_pk, relu, half_even, ceil_pk);
         word &= __builtin_amdgcn_sbfe((int)xmask, pt, 1); // all ones or zero
         *reinterpret_cast<int *>(dst + pt * 256) = word;
     };
@@ -293,12 +300,12 @@ __device__ __forceinline__ void expand_chunk(const v4i (&xb)[PACK > 1 ? (NXPT + 
 }
 
 // Depthwise stage of one chunk of 16 channels.  S == 1: output rows in pairs, four patch rows per read.
-template <int MODE, int PT, int S, bool EXACT, bool PIPE = false>
+template <int MODE, int PT, int S, bool EXACT, bool PIPE = false, bool CLIP = false>
 __device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_l + (quad * pw + S * col) * 16 */,
                                                 int th, int pw, const v4i (&a0)[3], const v4i (&a1)[3],
                                                 const StageConsts &c, int floor_pk, bool relu, bool half_even,
                                                 unsigned char *dst /* lane's slot in output row 0 of the result */,
-                                                int row_bytes = 16 * kDws, bool write_ok = true)
+                                                int row_bytes = 16 * kDws, bool write_ok = true, int ceil_pk = 0x7fff7fff)
 {
     if constexpr (EXACT && PIPE) {
         // software pipeline over units (S == 1: a pair of output rows, S == 2: one output row): operand-B
@@ -327,7 +334,7 @@ __device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_
 #pragma unroll
             for (int r = 0; r < ROWS; r++) {
                 if (ROWS * u + r < PT) {
-                    const int w = wave_pack_tab<MODE>(acc[u & 1][r], c, floor_pk, relu, half_even);
+                    const int w = wave_pack_tab<MODE, CLIP>(acc[u & 1][r], c, floor_pk, relu, half_even, ceil_pk);
                     if (write_ok)
                         *reinterpret_cast<int *>(dst + (ROWS * u + r) * row_bytes) = w;
                 }
@@ -358,14 +365,14 @@ __device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_
                 v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b0, c.init, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b1, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[2], b2, acc, 0, 0, 0);
-                const int w0 = wave_pack_tab<MODE>(acc, c, floor_pk, relu, half_even);
+                const int w0 = wave_pack_tab<MODE, CLIP>(acc, c, floor_pk, relu, half_even, ceil_pk);
                 if (write_ok)
                     *reinterpret_cast<int *>(dst + (2 * j) * row_bytes) = w0;
                 if (EXACT ? 2 * j + 1 < PT : 2 * j + 1 < th) {
                     v4i acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[0], b0, c.init, 0, 0, 0);
                     acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[1], b1, acc1, 0, 0, 0);
                     acc1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1[2], b2, acc1, 0, 0, 0);
-                    const int w1 = wave_pack_tab<MODE>(acc1, c, floor_pk, relu, half_even);
+                    const int w1 = wave_pack_tab<MODE, CLIP>(acc1, c, floor_pk, relu, half_even, ceil_pk);
                     if (write_ok)
                         *reinterpret_cast<int *>(dst + (2 * j + 1) * row_bytes) = w1;
                 }
@@ -382,7 +389,7 @@ __device__ __forceinline__ void depthwise_chunk(const unsigned char *src /* exp_
                 v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[0], b0, c.init, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[1], b1, acc, 0, 0, 0);
                 acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0[2], b2, acc, 0, 0, 0);
-                const int w0 = wave_pack_tab<MODE>(acc, c, floor_pk, relu, half_even);
+                const int w0 = wave_pack_tab<MODE, CLIP>(acc, c, floor_pk, relu, half_even, ceil_pk);
                 if (write_ok)
                     *reinterpret_cast<int *>(dst + t * row_bytes) = w0;
             }

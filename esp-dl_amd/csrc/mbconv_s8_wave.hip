@@ -97,7 +97,10 @@ __device__ __forceinline__ void byte_masks3(unsigned bm, int (&m)[3])
     }
 }
 
-template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, int PACK = 1>
+// CLIP: a Clip with equal exponents sits behind the expand and / or the depthwise stage (a ReLU6 exported as
+// Clip): the stage's int8 result is clamped to the Clip's bounds before it goes to LDS, one packed minimum
+// per pair of values on top of the packed maximum the ReLU floor already costs.
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, int PACK = 1, bool CLIP = false>
 __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) ? 3 : 2) : 1) void mbconv_s8_wave_kernel(const WaveArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -423,8 +426,14 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
         for (int t = 0; t < PT; t++)
             accp[r][t] = v4i{0, 0, 0, 0};
 
-    const int floor_e = p.relu_expand ? 0 : (int)0x80008000u;
-    const int floor_d = p.relu_dw ? 0 : (int)0x80008000u;
+    // lower / upper clamp of a stage as two int16 in the fixed-point form of the short epilogue: ReLU and a Clip's
+    // lower bound share the packed maximum, a Clip's upper bound is the packed minimum of the CLIP builds
+    const int lo_e = max(p.relu_expand ? 0 : -128, (CLIP && p.clip_e) ? p.clip_e_lo : -128);
+    const int lo_d = max(p.relu_dw ? 0 : -128, (CLIP && p.clip_d) ? p.clip_d_lo : -128);
+    const int floor_e = ((lo_e << 8) & 0xffff) * 0x10001;
+    const int floor_d = ((lo_d << 8) & 0xffff) * 0x10001;
+    const int ceil_e = (CLIP && p.clip_e) ? (((p.clip_e_hi << 8) | 0xff) & 0xffff) * 0x10001 : 0x7fff7fff;
+    const int ceil_d = (CLIP && p.clip_d) ? (((p.clip_d_hi << 8) | 0xff) & 0xffff) * 0x10001 : 0x7fff7fff;
     unsigned char *exp_dst = exp_l + col * 16 + 4 * quad;
     const unsigned char *exp_src = exp_l + (quad * a.pw + S * col) * 16;
 
@@ -436,15 +445,15 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
         {
             const StageConsts ce = read_stage_table(tab_e, p.exp_c, 16 * sub + 4 * quad, mode_e);
             if (!HE && ce.mode == 0) // a build meets the forms of its rounding mode only
-                expand_chunk<0, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<0, NXPT, EXACT, 1, true, PACK, CLIP>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, ceil_e);
             else if (!HE && ce.mode == 1)
-                expand_chunk<1, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<1, NXPT, EXACT, 1, true, PACK, CLIP>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, ceil_e);
             else if (HE && ce.mode == 6)
-                expand_chunk<6, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<6, NXPT, EXACT, 1, true, PACK, CLIP>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, ceil_e);
             else if (HE && ce.mode == 5)
-                expand_chunk<5, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<5, NXPT, EXACT, 1, true, PACK, CLIP>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, ceil_e);
             else
-                expand_chunk<-1, NXPT, EXACT, 1, true, PACK>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst);
+                expand_chunk<-1, NXPT, EXACT, 1, true, PACK, CLIP>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, ceil_e);
         }
         wave_lds_sync();
 
@@ -459,15 +468,15 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
             const StageConsts cd = read_stage_table(tab_d, p.exp_c, 16 * sub + 4 * quad, mode_d);
             unsigned char *dst = dw_l + col * kDws + 16 * (sub & 3) + 4 * quad;
             if (!HE && cd.mode == 0) // a build meets the forms of its rounding mode only
-                depthwise_chunk<0, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<0, PT, S, EXACT, true, CLIP>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, 16 * kDws, true, ceil_d);
             else if (!HE && cd.mode == 1)
-                depthwise_chunk<1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<1, PT, S, EXACT, true, CLIP>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, 16 * kDws, true, ceil_d);
             else if (HE && cd.mode == 6)
-                depthwise_chunk<6, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<6, PT, S, EXACT, true, CLIP>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, 16 * kDws, true, ceil_d);
             else if (HE && cd.mode == 5)
-                depthwise_chunk<5, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<5, PT, S, EXACT, true, CLIP>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, 16 * kDws, true, ceil_d);
             else
-                depthwise_chunk<-1, PT, S, EXACT, true>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst);
+                depthwise_chunk<-1, PT, S, EXACT, true, CLIP>(exp_src, th, a.pw, a0, a1, cd, floor_d, p.relu_dw != 0, HE, dst, 16 * kDws, true, ceil_d);
         }
         wave_lds_sync();
 
@@ -657,11 +666,11 @@ WavePlan wave_plan(const MbconvParams &p)
     return plan;
 }
 
-template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, int PACK = 1>
+template <int NXPT, int RT, int PT, int S, bool HE, bool VEC16, bool EXACT, bool ROWCONV = false, int PACK = 1, bool CLIP = false>
 hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
 {
     WaveArgs a = plan.a;
-    auto kernel = mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV, PACK>;
+    auto kernel = mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV, PACK, CLIP>;
     a.tpw = 1;
     if (ROWCONV) {
         // Tiles per wavefront: these tiles are short (two chunks of expanded channels for a 32-filter stem), so
@@ -696,11 +705,22 @@ bool launch_exact(const WavePlan &plan, hipStream_t stream, bool dry, hipError_t
     const WaveArgs &a = plan.a;
     const bool vec16 = a.x_vec16 && a.we_vec16;
     const int s = a.p.stride_h;
-#define ESPDL_WAVE_EXACT(NXPT, RT, PT, S, V, ROWCONV)                                     \
-    do {                                                                                   \
-        if (!dry)                                                                          \
-            *err = launch_one<NXPT, RT, PT, S, HE, V, true, ROWCONV>(plan, stream);        \
-        return true;                                                                       \
+    // a Clip between the stages: the half-up builds exist with the clamp compiled in, nothing else takes it
+    const bool clip = mbconv_has_clip(a.p);
+    if (clip && HE)
+        return false;
+#define ESPDL_WAVE_EXACT(NXPT, RT, PT, S, V, ROWCONV)                                                 \
+    do {                                                                                               \
+        if constexpr (!HE) {                                                                           \
+            if (clip) {                                                                                \
+                if (!dry)                                                                              \
+                    *err = launch_one<NXPT, RT, PT, S, false, V, true, ROWCONV, 1, true>(plan, stream); \
+                return true;                                                                           \
+            }                                                                                          \
+        }                                                                                              \
+        if (!dry)                                                                                      \
+            *err = launch_one<NXPT, RT, PT, S, HE, V, true, ROWCONV>(plan, stream);                    \
+        return true;                                                                                   \
     } while (0)
     if (!mbconv_expand_is_pointwise(a.p)) {
         // expand stage with a window: the stem + first block of MobileNetV2 at 224 x 224
@@ -712,11 +732,18 @@ bool launch_exact(const WavePlan &plan, hipStream_t stream, bool dry, hipError_t
         return a.n_xpt == nxpt && a.rt == rt && a.th == th && s == stride && vec16 == v && (stride != 1 || a.pw == 16);
     };
     // block inputs of at most 16 / 32 channels: four / two pixel tiles per operand-B register set
-#define ESPDL_WAVE_PACKED(NXPT, RT, PT, S, V, PACK)                                           \
-    do {                                                                                       \
-        if (!dry)                                                                              \
-            *err = launch_one<NXPT, RT, PT, S, HE, V, true, false, PACK>(plan, stream);        \
-        return true;                                                                           \
+#define ESPDL_WAVE_PACKED(NXPT, RT, PT, S, V, PACK)                                                       \
+    do {                                                                                                   \
+        if constexpr (!HE) {                                                                               \
+            if (clip) {                                                                                    \
+                if (!dry)                                                                                  \
+                    *err = launch_one<NXPT, RT, PT, S, false, V, true, false, PACK, true>(plan, stream);   \
+                return true;                                                                               \
+            }                                                                                              \
+        }                                                                                                  \
+        if (!dry)                                                                                          \
+            *err = launch_one<NXPT, RT, PT, S, HE, V, true, false, PACK>(plan, stream);                    \
+        return true;                                                                                       \
     } while (0)
     const int c0 = a.p.in_c;
     if (is(17, 2, 4, 2, true) && c0 == 16)
@@ -764,6 +791,8 @@ hipError_t launch_planned(WavePlan &plan, hipStream_t stream)
     hipError_t err = hipSuccess;
     if (a.p.half_even ? launch_exact<true>(plan, stream, false, &err) : launch_exact<false>(plan, stream, false, &err))
         return err;
+    if (mbconv_has_clip(a.p))
+        return hipErrorInvalidValue; // the guarded builds have no clamp
     // guarded builds
     if (!mbconv_expand_is_pointwise(a.p)) {
         if (a.p.half_even)

@@ -69,6 +69,8 @@ private:
     // the absorbed Conv's own window: {1, 1} / {1, 1} / no padding for the usual 1x1 expand, anything else
     // for a stem convolution that took the expand stage's place
     std::vector<int> m_expand_kernel = {1, 1}, m_expand_strides = {1, 1}, m_expand_pads = {0, 0, 0, 0};
+    // Clip modules with equal exponents that stood between the stages of the fused block: {on, min, max}
+    int m_clip_expand[3] = {0, -128, 127}, m_clip_dw[3] = {0, -128, 127};
 
 public:
     Conv(activation_type_t activation = Linear, std::vector<int> pads = {}, std::vector<int> dilations = {},
@@ -148,6 +150,15 @@ public:
             m_expand_bias_pos = (int)m_inputs_index.size();
             m_inputs_index.push_back(bias_index);
         }
+    }
+    /// A Clip (equal exponents: a clamp of the stored value) that stood behind the absorbed expand Conv
+    /// (`stage` 0) or behind this depthwise Conv (`stage` 1) runs inside the fused launch.
+    void fuse_clip(int stage, int min_q, int max_q)
+    {
+        int *c = stage == 0 ? m_clip_expand : m_clip_dw;
+        c[0] = 1;
+        c[1] = min_q;
+        c[2] = max_q;
     }
     bool has_fused_expand() const { return m_has_expand; }
     bool expand_has_window() const
@@ -420,6 +431,12 @@ public:
         d.n_shift_project = (int32_t)s_pj.size();
         // a residual operand whose RequantizeLinear the fusion pass absorbed is requantized inside the kernel
         d.residual_shift = residual ? m_residual_shift : 0;
+        d.clip_expand = m_has_expand ? m_clip_expand[0] : 0;
+        d.clip_expand_min = m_clip_expand[1];
+        d.clip_expand_max = m_clip_expand[2];
+        d.clip_dw = m_clip_dw[0];
+        d.clip_dw_min = m_clip_dw[1];
+        d.clip_dw_max = m_clip_dw[2];
         m_fused_kernel = espdl_hip_mbconv_s8_supported(&d);
         espdl_hip_mbconv_weights w = {};
         if (m_has_expand) {

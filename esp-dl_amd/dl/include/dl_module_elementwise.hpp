@@ -266,21 +266,7 @@ public:
             DL_LOGE("Clip", "%s: needs int8 device tensors", name.c_str());
             return;
         }
-        // min / max are quantized scalars held as parameters (read once on the host)
-        if (!m_bounds_read) {
-            m_min = std::numeric_limits<int8_t>::min();
-            m_max = std::numeric_limits<int8_t>::max();
-            for (size_t i = 1; i < m_inputs_index.size() && i < 3; i++) {
-                TensorBase *b = context->get_tensor(m_inputs_index[i]);
-                if (!b)
-                    continue;
-                TensorBase *host = b->on_device() ? b->to_host(context->stream) : b;
-                (i == 1 ? m_min : m_max) = host->get_element<int8_t>(0);
-                if (host != b)
-                    delete host;
-            }
-            m_bounds_read = true;
-        }
+        read_bounds(context);
         const int rc = espdl_hip_clip_s8(static_cast<const int8_t *>(input->data), input->get_size(), m_min, m_max,
                                          input->exponent.get(), output->exponent.get(),
                                          static_cast<int8_t *>(output->data), context->stream);
@@ -295,6 +281,28 @@ public:
         return op ? op : new Clip(node_name.c_str(), MODULE_INPLACE_CHANGED_BUFFER, quant_type);
     }
     void print() { DL_LOGI("Clip", "quant_type: %s.", quant_type_to_string(quant_type)); }
+
+    /// min / max are quantized scalars held as parameters (read once, on the host); also what a fusion pass
+    /// asks for when it folds the clamp into the convolution in front
+    void read_bounds(ModelContext *context)
+    {
+        if (m_bounds_read)
+            return;
+        m_min = std::numeric_limits<int8_t>::min();
+        m_max = std::numeric_limits<int8_t>::max();
+        for (size_t i = 1; i < m_inputs_index.size() && i < 3; i++) {
+            TensorBase *b = context->get_tensor(m_inputs_index[i]);
+            if (!b)
+                continue;
+            TensorBase *host = b->on_device() ? b->to_host(context->stream) : b;
+            (i == 1 ? m_min : m_max) = host->get_element<int8_t>(0);
+            if (host != b)
+                delete host;
+        }
+        m_bounds_read = true;
+    }
+    int get_min() const { return m_min; }
+    int get_max() const { return m_max; }
 
 private:
     bool m_bounds_read = false;

@@ -259,18 +259,41 @@ void Model::fuse_dw_project()
                 }
         return readers == 1 && !pinned.count(m_model_context->get_tensor_name(tensor));
     };
+    // A Clip whose input and output exponents are equal is a clamp of the stored value
+    // (esp-dl/dl/module/include/dl_module_clip.hpp:78-90 with a rescale factor of 1): between two stages of the
+    // block it can run inside the launch.  Returns the module when `m` is such a Clip with one data input.
+    auto clamp_only = [&](dl::module::Module *m) -> dl::module::Clip * {
+        auto *clip = dynamic_cast<dl::module::Clip *>(m);
+        if (!clip || clip->quant_type != QUANT_TYPE_SYMM_8BIT || clip->m_inputs_index.empty() || clip->m_outputs_index.size() != 1 ||
+            clip->m_inputs_index[0] >= CONTEXT_PARAMETER_OFFSET)
+            return nullptr;
+        const std::string in_name = m_model_context->get_tensor_name(clip->m_inputs_index[0]);
+        const std::string out_name = m_model_context->get_tensor_name(clip->m_outputs_index[0]);
+        if (!m_fbs_model->has_value_info(in_name) || !m_fbs_model->has_value_info(out_name) ||
+            m_fbs_model->get_value_info_exponent(in_name) != m_fbs_model->get_value_info_exponent(out_name))
+            return nullptr;
+        clip->read_bounds(m_model_context);
+        return clip->get_min() <= clip->get_max() ? clip : nullptr;
+    };
+    auto plain_act = [](dl::module::Conv *c) { return c->get_activation() == Linear || c->get_activation() == ReLU; };
     for (size_t i = 0; i < m_execution_plan.size(); i++) {
         auto *dw = dynamic_cast<dl::module::Conv *>(m_execution_plan[i]);
         if (!dw || dw->quant_type != QUANT_TYPE_SYMM_8BIT || dw->get_group() == 1 || dw->has_fused_lut() ||
-            dw->has_fused_project() || dw->get_pads().size() != 4)
+            dw->has_fused_project() || dw->get_pads().size() != 4 || !plain_act(dw))
             continue;
-        const int mid = dw->m_outputs_index[0];
+        int mid = dw->m_outputs_index[0]; // the tensor the project Conv reads
         size_t pj_pos = 0;
         if (!single_reader(mid, &pj_pos) || pj_pos <= i)
             continue;
+        dl::module::Clip *clip_d = clamp_only(m_execution_plan[pj_pos]);
+        if (clip_d) {
+            mid = clip_d->m_outputs_index[0];
+            if (!single_reader(mid, &pj_pos) || pj_pos <= i)
+                continue;
+        }
         auto *pj = dynamic_cast<dl::module::Conv *>(m_execution_plan[pj_pos]);
         if (!pj || pj->quant_type != QUANT_TYPE_SYMM_8BIT || pj->get_group() != 1 || pj->has_fused_lut() ||
-            pj->has_fused_project() || pj->m_inputs_index[0] != mid)
+            pj->has_fused_project() || pj->m_inputs_index[0] != mid || !plain_act(pj))
             continue;
         TensorBase *pf = m_model_context->get_tensor(pj->m_inputs_index[1]);
         TensorBase *df = m_model_context->get_tensor(dw->m_inputs_index[1]);
@@ -305,26 +328,43 @@ void Model::fuse_dw_project()
         d.pad_left = dw->get_pads()[2];
         d.pad_right = dw->get_pads()[3];
         d.n_shift_expand = d.n_shift_dw = d.n_shift_project = 1;
+        if (clip_d) {
+            d.clip_dw = 1;
+            d.clip_dw_min = clip_d->get_min();
+            d.clip_dw_max = clip_d->get_max();
+        }
         if (pf->shape[2] != d.in_c)
             continue;
         // The 1x1 Conv in front (the expand stage of an inverted-residual block) joins when the single
         // launch of the whole block is the preferred form for this batch; otherwise depthwise + project
-        // fuse where the depthwise+project kernel applies.
+        // fuse where the depthwise+project kernel applies.  A clamp-only Clip may stand between the two.
         dl::module::Conv *ex = nullptr;
-        size_t ex_pos = 0;
+        dl::module::Clip *clip_e = nullptr;
         int ex_kernel[2] = {1, 1};
         espdl_hip_mbconv_desc de = d; // the whole block, when a Conv in front joins
         {
-            const int dw_in = dw->m_inputs_index[0];
+            int dw_in = dw->m_inputs_index[0];
             size_t reader = 0;
+            dl::module::Module *producer = nullptr;
             for (size_t j = 0; j < i; j++)
-                if (m_execution_plan[j]->m_outputs_index.size() == 1 && m_execution_plan[j]->m_outputs_index[0] == dw_in) {
-                    ex = dynamic_cast<dl::module::Conv *>(m_execution_plan[j]);
-                    ex_pos = j;
+                if (m_execution_plan[j]->m_outputs_index.size() == 1 && m_execution_plan[j]->m_outputs_index[0] == dw_in)
+                    producer = m_execution_plan[j];
+            if (producer && (clip_e = clamp_only(producer)) != nullptr) {
+                if (!single_reader(dw_in, &reader)) {
+                    clip_e = nullptr;
+                    producer = nullptr;
+                } else {
+                    dw_in = clip_e->m_inputs_index[0];
+                    producer = nullptr;
+                    for (size_t j = 0; j < i; j++)
+                        if (m_execution_plan[j]->m_outputs_index.size() == 1 && m_execution_plan[j]->m_outputs_index[0] == dw_in)
+                            producer = m_execution_plan[j];
                 }
+            }
+            ex = dynamic_cast<dl::module::Conv *>(producer);
             if (ex && (ex->quant_type != QUANT_TYPE_SYMM_8BIT || ex->get_group() != 1 || ex->has_fused_lut() ||
                        ex->has_fused_project() || ex->has_fused_residual() || !single_reader(dw_in, &reader) ||
-                       ex->get_pads().size() != 4))
+                       ex->get_pads().size() != 4 || !plain_act(ex)))
                 ex = nullptr;
             TensorBase *ef = ex ? m_model_context->get_tensor(ex->m_inputs_index[1]) : nullptr;
             if (ex && (!ef || ef->shape.size() != 4 || ef->shape[3] != d.in_c))
@@ -353,6 +393,11 @@ void Model::fuse_dw_project()
                 de.has_expand = 1;
                 de.exp_c = d.in_c;
                 de.in_c = ef->shape[2];
+                if (clip_e) {
+                    de.clip_expand = 1;
+                    de.clip_expand_min = clip_e->get_min();
+                    de.clip_expand_max = clip_e->get_max();
+                }
                 if (!plain_ex) {
                     // a convolution with a window (a stem) as the expand stage: the block input is its input
                     de.in_h = ex_in_shape[1];
@@ -369,6 +414,8 @@ void Model::fuse_dw_project()
                 if (espdl_hip_mbconv_s8_preferred(&de) != 1)
                     ex = nullptr;
             }
+            if (!ex)
+                clip_e = nullptr; // a Clip in front of a depthwise Conv that stays on its own stays too
         }
         if (!ex && espdl_hip_mbconv_s8_supported(&d) != 2)
             continue;
@@ -376,7 +423,7 @@ void Model::fuse_dw_project()
         // optional Add behind the project conv
         int out_index = pj->m_outputs_index[0];
         int residual = -1;
-        size_t last_pos = pj_pos, add_pos = 0;
+        size_t add_pos = 0;
         dl::module::Add *add = nullptr;
         if (single_reader(out_index, &add_pos) && add_pos > pj_pos) {
             add = plain_add(m_execution_plan[add_pos]);
@@ -389,7 +436,6 @@ void Model::fuse_dw_project()
                     m_fbs_model->get_value_info_shape(other_name) == m_fbs_model->get_value_info_shape(out_name)) {
                     residual = other;
                     out_index = add->m_outputs_index[0];
-                    last_pos = add_pos;
                 } else {
                     add = nullptr;
                 }
@@ -434,36 +480,34 @@ void Model::fuse_dw_project()
         dw->fuse_project(pj->m_inputs_index[1], pj->m_inputs_index.size() == 3 ? pj->m_inputs_index[2] : -1,
                          pj->get_activation(), mid_exp, residual, pj_out_exp, rq != nullptr ? rq_shift : 0);
         dw->m_outputs_index[0] = out_index;
-        if (ex)
+        if (clip_d)
+            dw->fuse_clip(1, clip_d->get_min(), clip_d->get_max());
+        if (ex) {
             dw->fuse_expand(ex->m_inputs_index[0], ex->m_inputs_index[1],
                             ex->m_inputs_index.size() == 3 ? ex->m_inputs_index[2] : -1, ex->get_activation(),
                             m_fbs_model->get_value_info_exponent(m_model_context->get_tensor_name(ex->m_outputs_index[0])),
                             {ex_kernel[0], ex_kernel[1]}, ex->get_strides(), ex->get_pads());
-        // the fused module moves to the slot of the last absorbed module
-        m_execution_plan[last_pos] = dw;
-        if (add) {
-            delete add;
-            if (last_pos != pj_pos) {
-                delete pj;
-                m_execution_plan.erase(m_execution_plan.begin() + pj_pos);
-            }
-        } else {
-            delete pj;
+            if (clip_e)
+                dw->fuse_clip(0, clip_e->get_min(), clip_e->get_max());
         }
-        m_execution_plan.erase(m_execution_plan.begin() + i);
-        i--;
-        if (ex) { // ex_pos < i + 1: erasing it shifts the modules behind it down by one more
-            delete ex;
-            m_execution_plan.erase(m_execution_plan.begin() + ex_pos);
-            i--;
+        // The fused module takes the slot of the last module it absorbs (everything it reads, the residual
+        // operand included, is produced before that); the absorbed modules leave the plan.  The scan then starts
+        // over: positions have moved, and modules already fused are skipped by their flag.
+        dl::module::Module *last = add ? static_cast<dl::module::Module *>(add) : static_cast<dl::module::Module *>(pj);
+        std::vector<dl::module::Module *> gone = {pj, add, ex, rq, clip_e, clip_d};
+        std::vector<dl::module::Module *> plan;
+        for (dl::module::Module *m : m_execution_plan) {
+            if (m == dw)
+                continue;
+            if (m == last)
+                plan.push_back(dw);
+            if (std::find(gone.begin(), gone.end(), m) == gone.end())
+                plan.push_back(m);
         }
-        if (rq) {
-            const size_t rq_pos = std::find(m_execution_plan.begin(), m_execution_plan.end(), rq) - m_execution_plan.begin();
-            m_execution_plan.erase(m_execution_plan.begin() + rq_pos);
-            delete rq;
-            if (rq_pos <= i + 1) // it stood before the module the loop looks at next
-                i--;
-        }
+        for (dl::module::Module *m : gone)
+            delete m;
+        m_execution_plan.swap(plan);
+        i = (size_t)-1;
     }
 }
 

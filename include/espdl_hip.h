@@ -139,7 +139,7 @@ int espdl_hip_mul_s8(const int32_t out_dims[4], const int64_t in0_strides[4], co
  * conv_out_exp, activation applied, exactly what espdl_hip_conv2d would store - are summed per image and filter
  * inside the kernel and only the pooled tensor out[batch][out_c] (exponent pool_out_exp) is written.  desc as for
  * espdl_hip_conv2d (ESPDL_HIP_S8, group 1, ESPDL_HIP_LINEAR / _RELU); images of at most 64 pixels, in_c a
- * multiple of 16 and at least 64, in and filter 16-byte aligned; ESPDL_HIP_ENOTSUP otherwise
+ * multiple of 16 and at least 64, at least 32 filters, in and filter 16-byte aligned; ESPDL_HIP_ENOTSUP otherwise
  * (espdl_hip_conv2d_gap_s8_supported answers 1 / 0 for a descriptor). */
 int espdl_hip_conv2d_gap_s8_supported(const espdl_hip_conv_desc *desc);
 int espdl_hip_conv2d_gap_s8(const espdl_hip_conv_desc *desc, const int8_t *in, const int8_t *filter, const int32_t *bias,
@@ -348,7 +348,7 @@ int espdl_hip_slice(const void *in, const int32_t *shape, int32_t dims, const in
  * (3x3 depthwise stage, at most 64 block-input channels and 64 project filters), 5 = yes, a workgroup of
  * wavefronts per tile of a small image (output at most 16 pixels wide, block-input channels a multiple of
  * 16 and at most 192).  An expand stage with a window (exp_k_h, exp_k_w not 1: at most 4 rows of at most
- * 16 bytes, i.e. exp_k_w * in_c <= 16) is taken by the one-wavefront-per-tile kernel only.
+ * 9 bytes, i.e. exp_k_w * in_c <= 9) is taken by the one-wavefront-per-tile kernel only.
  * espdl_hip_mbconv_s8 returns ESPDL_HIP_ENOTSUP where it does not apply.
  */
 typedef struct espdl_hip_mbconv_desc {
@@ -372,6 +372,16 @@ typedef struct espdl_hip_mbconv_desc {
      * esp-dl/dl/tensor/src/dl_tensor_base.cpp:362-371).  0: the operand is added as it is.  Taken by the
      * single-launch kernels of answers 4 and 5 only; espdl_hip_mbconv_s8_supported answers 0 elsewhere. */
     int32_t residual_shift;
+    /* A Clip between two stages whose input and output exponents are equal (module::Clip::forward,
+     * esp-dl/dl/module/include/dl_module_clip.hpp:78-90: the rescale factor is 1 and the operator is a clamp of
+     * the stored int8 value; a ReLU6 exported as Clip): clip_expand != 0 clamps the expand stage's int8 result
+     * to [clip_expand_min, clip_expand_max] before the depthwise stage reads it (the zero padding of the
+     * depthwise window pads the CLAMPED activation, as with separate operators), clip_dw != 0 the depthwise
+     * stage's result before the project stage.  Bounds in -128 .. 127, min <= max.  Taken by the
+     * one-wavefront-per-tile kernel (answer 4) where its tile plan has a guard-free build, round half up;
+     * espdl_hip_mbconv_s8_supported answers 0 elsewhere. */
+    int32_t clip_expand, clip_expand_min, clip_expand_max;
+    int32_t clip_dw, clip_dw_min, clip_dw_max;
 } espdl_hip_mbconv_desc;
 
 typedef struct espdl_hip_mbconv_weights {
@@ -402,7 +412,12 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
  * reference; it exists for callers that cannot allocate device memory and whose block shape the
  * single-launch kernels do not cover (espdl_hip_mbconv_s8_supported() == 0): code under HIP-graph
  * capture, serving loops, harnesses that forbid hipMalloc.  It allocates nothing and accepts every shape
- * espdl_hip_conv2d accepts.  Results are bit-identical to espdl_hip_mbconv_s8 and to the separate calls.
+ * espdl_hip_conv2d accepts, with or without Clips between the stages; a requantized residual operand
+ * (residual_shift != 0) is refused with ESPDL_HIP_ENOTSUP (requantize it first).  Results are bit-identical to
+ * espdl_hip_mbconv_s8 and to the separate calls.
+ * The first call on a device looks up the array's address, which must not happen while `stream` records a
+ * graph: call espdl_hip_mbconv_s8_staged_init() (or the entry point itself) once per device outside capture;
+ * a first call under capture returns ESPDL_HIP_ENOTSUP.
  * The intermediates (batch*in_h*in_w*exp_c bytes when has_expand, plus batch*out_h*out_w*exp_c bytes, each
  * rounded up to 256) must fit ESPDL_HIP_MBCONV_STAGED_MAX_BYTES, else ESPDL_HIP_ENOTSUP: split the batch.
  * Every call on a device uses the same array: calls that overlap on one device (two streams, two threads)
@@ -413,6 +428,9 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
 int espdl_hip_mbconv_s8_staged(const espdl_hip_mbconv_desc *desc, const int8_t *in,
                                const espdl_hip_mbconv_weights *weights, const int8_t *residual, int8_t *out,
                                void *stream);
+/* Set-up of espdl_hip_mbconv_s8_staged on the current device (address of the library's array); allocates
+ * nothing, launches nothing.  No counterpart in the reference. */
+int espdl_hip_mbconv_s8_staged_init(void);
 
 /* Library / device information. */
 const char *espdl_hip_last_error(void);

@@ -656,6 +656,82 @@ def test_mbconv_s8_fused(oracle, case):
     np.testing.assert_array_equal(to_host(got), cur)
 
 
+# A Clip with equal exponents between the stages (ReLU6 exported as Clip), inside the launch: the block shapes of
+# MobileNetV2 that the one-wavefront-per-tile kernel covers, linear convolutions followed by clamps with a lower
+# bound of 0 / below 0 / above 0, one clamp only, a ragged last tile, a requantized residual operand.
+# (name, (N, H, W, Cin), Ce, Cout, stride, clip_expand, clip_dw, relus, residual, residual_shift)
+CLIP_CASES = [
+    ("c2_56x56_24_144_24_relu6", (3, 56, 56, 24), 144, 24, (1, 1), (0, 48), (0, 96), (False, False, False), True, 0),
+    ("c2_56x56_24_144_24_relu6_rq", (2, 56, 56, 24), 144, 24, (1, 1), (0, 48), (0, 96), (False, False, False), True, -1),
+    ("b2_112x112_16_96_24_s2", (1, 112, 112, 16), 96, 24, (2, 2), (-20, 100), (5, 90), (False, False, False), False, 0),
+    ("b4_56x56_24_144_32_s2", (2, 56, 56, 24), 144, 32, (2, 2), (0, 127), None, (True, True, False), False, 0),
+    ("b5_28x28_32_192_32_only_dw", (2, 28, 28, 32), 192, 32, (1, 1), None, (-128, 20), (True, False, False), True, 0),
+    ("b7_28x28_32_192_64_s2", (3, 28, 28, 32), 192, 64, (2, 2), (0, 31), (0, 31), (False, False, False), False, 0),
+    ("ragged_50x56_24_144_24", (2, 50, 56, 24), 144, 24, (1, 1), (0, 48), (0, 96), (False, False, False), True, 0),
+]
+
+
+@pytest.mark.parametrize("staged", [False, True], ids=["single_launch", "staged"])
+@pytest.mark.parametrize("case", CLIP_CASES, ids=lambda c: c[0])
+def test_mbconv_s8_clip_between_stages(oracle, case, staged):
+    announce(f"mbconv_s8 with Clip between the stages: {case[0]} staged={staged}")
+    name, (n, h, w, cin), ce, cout, stride, clip_e, clip_d, relus, with_res, res_shift = case
+    if staged and res_shift != 0:
+        pytest.skip("the staged form adds the residual operand as it is")
+    m = espdl()
+    import torch
+    rng = np.random.default_rng(0xC11F + len(name))
+
+    def stage(oc, kk, fshape):
+        f = rng_int8(rng, fshape)
+        b = rng.integers(-4096, 4097, size=oc).astype(np.int32)
+        s = (typical_shift(kk) + rng.integers(-2, 3, size=oc)).astype(np.int32)
+        return f, b, s
+
+    act = lambda r: oracle.RELU if r else oracle.LINEAR  # noqa: E731
+    x = rng_int8(rng, (n, h, w, cin))
+    expand = stage(ce, cin, (ce, 1, 1, cin))
+    cur = oracle.conv2d_s8(x, expand[0], expand[1], expand[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), act(relus[0]))
+    if clip_e is not None:
+        cur = oracle.clip_s8(cur, clip_e[0], clip_e[1], 0, 0)
+    dw = stage(ce, 9, (3, 3, ce))
+    pads = (1, 1, 1, 1) if stride == (1, 1) else (0, 1, 0, 1)
+    cur = oracle.depthwise_s8(cur, dw[0], dw[1], dw[2], (3, 3), stride, (1, 1), pads, act(relus[1]))
+    if clip_d is not None:
+        cur = oracle.clip_s8(cur, clip_d[0], clip_d[1], 0, 0)
+    proj = stage(cout, ce, (cout, 1, 1, ce))
+    cur = oracle.conv2d_s8(cur, proj[0], proj[1], proj[2], (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), act(relus[2]))
+    res = None
+    if with_res:
+        res = rng_int8(rng, cur.shape)
+        cur = oracle.add_s8(cur, oracle.requantize_s8(res, res_shift, 0) if res_shift else res)
+    dev = lambda t: tuple(to_dev(a) for a in t)  # noqa: E731
+    out = torch.empty(cur.shape, dtype=torch.int8, device="cuda")
+    got = m.mbconv_s8(to_dev(x), dev(expand), dev(dw), dev(proj), (3, 3), stride, (1, 1), pads, relus,
+                      residual=to_dev(res), residual_shift=res_shift, clip_expand=clip_e, clip_dw=clip_d, out=out,
+                      staged=staged)
+    np.testing.assert_array_equal(to_host(got), cur)
+
+
+def test_mbconv_s8_clip_is_refused_where_not_covered():
+    """Shapes without a guard-free build of the one-wavefront-per-tile kernel, and round half even, answer 0 /
+    ESPDL_HIP_ENOTSUP when a Clip sits between the stages."""
+    m = espdl()
+    import torch
+    for shape, ce, cout, rm in (((1, 14, 14, 96), 576, 96, m.capi.ROUND_HALF_UP), ((1, 50, 50, 24), 144, 24, m.capi.ROUND_HALF_UP),
+                                ((1, 56, 56, 24), 144, 24, m.capi.ROUND_HALF_EVEN)):
+        n, h, w, c = shape
+        d = m.capi.MbconvDesc(n, h, w, c, ce, cout, 1, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0, rm, 1, 1, 1)
+        d.clip_expand, d.clip_expand_min, d.clip_expand_max = 1, 0, 48
+        assert m.lib().espdl_hip_mbconv_s8_supported(ctypes.byref(d)) == 0, shape
+        x = torch.zeros(shape, dtype=torch.int8, device="cuda")
+        z = lambda *s: torch.zeros(s, dtype=torch.int8, device="cuda")  # noqa: E731
+        sh = torch.full((1,), 8, dtype=torch.int32, device="cuda")
+        with pytest.raises(m.EspdlHipError, match="Clip"):
+            m.mbconv_s8(x, (z(ce, c), None, sh), (z(3, 3, ce), None, sh), (z(cout, ce), None, sh), (3, 3), (1, 1), (1, 1),
+                        (1, 1, 1, 1), (False, False, False), round_mode=rm, clip_expand=(0, 48))
+
+
 # Expand stage with a window: a stem convolution in front of the first depthwise stage, in the block's launch.
 # (name, (N, H, W, Cin), expand (kernel, stride, pads), Ce, Cout, depthwise stride, depthwise pads, residual, half_even)
 ROWCONV_CASES = [
