@@ -28,7 +28,10 @@ namespace espdl {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kRow = 96;    // LDS row: 64 k bytes + 32
+// LDS row of a tile: 64 k bytes + padding.  96 where LDS capacity allows it (conflict-free operand reads, see the
+// head of the file); 80 for the four-image pooled build, whose 256-row pixel tile would otherwise leave two
+// workgroups per compute unit instead of three (measured: 16.5 us at 80, 26.9 us at 96 on MobileNetV2's head).
+template <int PT> constexpr int row_pitch = PT >= 4 ? 80 : 96;
 
 struct PwArgs {
     const int8_t *in;  // [M][K]
@@ -53,10 +56,11 @@ struct PwArgs {
 // results (requantized, activation applied, exactly what the separate operator would have stored) are summed
 // over the image's pixels - over the 16 lanes of a pixel tile by rotations inside the row, over the four
 // wavefronts through LDS - and the sum goes through the pooling operator's float scale and rounding.
-template <int NG, int PT, bool GAP = false>
+template <int NG, int PT, bool GAP = false, bool K16 = true>
 __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs a)
 {
     constexpr int TN = 64 * NG;
+    constexpr int kRow = row_pitch<PT>;
     constexpr int kTileM = 64 * PT; // pixels per workgroup, 16 * PT per wavefront
     constexpr int kPiecesB = kTileM * 4 / kThreads; // 16-byte pieces of the pixel tile per thread and k step (2)
     constexpr int kPiecesA = TN * 4 / kThreads;     // ... of the filter tile (1 or 2)
@@ -87,9 +91,9 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
     // multiple of 16 (a Gemm over 120 features) are read with loads that need no alignment; the one piece that
     // holds a row's last n < 16 bytes is read as the 16 bytes that END at the row's end and shifted down, so
     // that nothing past a row (and so nothing past the tensor) is touched and the piece ends in zeros.
-    const bool k16 = (a.K & 15) == 0; // uniform
+    // (K16 builds: rows of whole 16-byte pieces at aligned addresses)
     auto piece = [&](const int8_t *row, int k) -> v4i {
-        if (k16)
+        if constexpr (K16)
             return k < a.K ? *reinterpret_cast<const v4i *>(row + k) : v4i{0, 0, 0, 0};
         if (k >= a.K)
             return v4i{0, 0, 0, 0};
@@ -546,10 +550,18 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
                            dim3(kThreads), 0, stream, a);
         return hipGetLastError();
     }
-    if (tiles128 * gy * 2 < 3ll * cus)
-        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1>), dim3((unsigned)((a.M + 63) / 64), gy), dim3(kThreads), 0, stream, a);
-    else
-        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2>), dim3((unsigned)tiles128, gy), dim3(kThreads), 0, stream, a);
+    const bool k16 = (a.K & 15) == 0;
+    if (tiles128 * gy * 2 < 3ll * cus) {
+        if (k16)
+            hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1>), dim3((unsigned)((a.M + 63) / 64), gy), dim3(kThreads), 0, stream, a);
+        else
+            hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1, false, false>), dim3((unsigned)((a.M + 63) / 64), gy), dim3(kThreads), 0, stream, a);
+    } else {
+        if (k16)
+            hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2>), dim3((unsigned)tiles128, gy), dim3(kThreads), 0, stream, a);
+        else
+            hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2, false, false>), dim3((unsigned)tiles128, gy), dim3(kThreads), 0, stream, a);
+    }
     return hipGetLastError();
 }
 

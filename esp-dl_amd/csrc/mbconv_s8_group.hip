@@ -439,9 +439,14 @@ GroupPlan group_plan(const MbconvParams &p)
     a.kse = (p.in_c + 63) / 64;
     a.n_sub = p.exp_c / 16;
     a.rt = (p.out_c + 15) / 16;
-    a.ds = p.exp_c + 16; // exp_c is a multiple of 16: an odd number of 16-byte units when exp_c / 16 is even ...
-    if ((a.ds / 16) % 2 == 0)
-        a.ds += 16;      // ... and made odd otherwise, so that operand-B reads of 16 pixels spread over the banks
+    // Pixel pitch of the depthwise result: twice an odd number of 16-byte units.  A 16-byte-per-lane LDS read is
+    // served in groups of 8 consecutive pixels x 2 neighbouring 16-byte quarters; with such a pitch the 16 pieces
+    // of a group fall into 16 different bank sets (an odd number of units, the earlier choice, leaves half of the
+    // project stage's operand-B reads in two passes).  The 4-byte stores of the depthwise stage then take two
+    // passes, but the project stage reads every piece once per wavefront: eight times as many LDS cycles.
+    a.ds = p.exp_c + 16;
+    while ((a.ds / 16) % 4 != 2)
+        a.ds += 16;
     // rows per tile: as many as fit the register and LDS budgets (fewer tiles, less halo to expand)
     a.th = 0;
     for (int th = 1; th <= std::min(kGroupPtMax - 1, p.out_h); th++) {
