@@ -359,9 +359,49 @@ hipError_t launch_relu_s8(const int8_t *in, int64_t size, int in_exp, int out_ex
     return launch_map(in, out, size, ReluFn{in_exp == out_exp, dl_scale(in_exp), dl_rescale(out_exp)}, stream);
 }
 
+namespace {
+// Clip between equal exponents: the rescale factor is 1 and the operator is a clamp of the stored value.  Four
+// bytes per packed-int16 sequence: the bytes go to the high bytes of two int16 pairs (x * 256), one packed
+// maximum and minimum against (lo << 8) and (hi << 8) | 0xff, the high bytes are gathered again.
+__global__ __launch_bounds__(kBlock) void clamp_s8_kernel(const int8_t *in, int8_t *out, int64_t size, int64_t vecs, int lo,
+                                                          int hi)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const v2s lo2 = __builtin_bit_cast(v2s, ((lo << 8) & 0xffff) * 0x10001);
+    const v2s hi2 = __builtin_bit_cast(v2s, (((hi << 8) | 0xff) & 0xffff) * 0x10001);
+    if (i < vecs) {
+        const v4i v = reinterpret_cast<const v4i *>(in)[i];
+        v4i r;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            v2s p01 = __builtin_bit_cast(v2s, (int)__builtin_amdgcn_perm(0u, (unsigned)v[w], 0x010c000cu));
+            v2s p23 = __builtin_bit_cast(v2s, (int)__builtin_amdgcn_perm(0u, (unsigned)v[w], 0x030c020cu));
+            p01 = __builtin_elementwise_min(__builtin_elementwise_max(p01, lo2), hi2);
+            p23 = __builtin_elementwise_min(__builtin_elementwise_max(p23, lo2), hi2);
+            r[w] = (int)__builtin_amdgcn_perm((unsigned)__builtin_bit_cast(int, p23), (unsigned)__builtin_bit_cast(int, p01),
+                                              0x07050301u);
+        }
+        reinterpret_cast<v4i *>(out)[i] = r;
+    }
+    const int64_t t = vecs * 16 + i;
+    if (t < size)
+        out[t] = (int8_t)min(max((int)in[t], lo), hi);
+}
+} // namespace
+
 hipError_t launch_clip_s8(const int8_t *in, int64_t size, int min_q, int max_q, int in_exp, int out_exp, int8_t *out,
                           hipStream_t stream)
 {
+    const bool aligned = ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    if (in_exp == out_exp && aligned && min_q >= -128 && max_q <= 127 && min_q <= max_q) {
+        const int64_t vecs = size / 16;
+        const int64_t work = std::max<int64_t>(vecs, size - vecs * 16);
+        if (work <= 0)
+            return hipSuccess;
+        hipLaunchKernelGGL(clamp_s8_kernel, dim3((unsigned)((work + kBlock - 1) / kBlock)), dim3(kBlock), 0, stream, in, out,
+                           size, vecs, min_q, max_q);
+        return hipGetLastError();
+    }
     return launch_map(in, out, size, ClipFn{min_q, max_q, dl_scale(in_exp) * dl_rescale(out_exp)}, stream);
 }
 

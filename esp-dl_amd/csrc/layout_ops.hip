@@ -34,28 +34,56 @@ struct RowCopyArgs {
     long long rows;
 };
 
+// Four pieces per thread and pass: the four loads are requested before the first store, so that enough bytes are
+// in flight to cover the memory latency (one piece per thread moved 4.3 TB/s, a plain copy's rate is above 6).
 __global__ __launch_bounds__(kBlock) void copy_rows_kernel(const RowCopyArgs a)
 {
     const RowSeg &s = a.seg[blockIdx.y];
     const long long total = a.rows * s.per_row.d;
-    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < total; i += (long long)gridDim.x * kBlock) {
+    const long long stride = (long long)gridDim.x * kBlock;
+    const bool small = total <= 0x7fffffffll; // range in which fastdiv is exact
+    auto locate = [&](long long i, const char *&sp, char *&dp) {
         long long r;
         unsigned c;
-        if (total <= 0x7fffffffll) { // range in which fastdiv is exact
+        if (small) {
             r = fastdiv((unsigned)i, s.per_row);
             c = (unsigned)i - (unsigned)r * s.per_row.d;
         } else {
             r = i / s.per_row.d;
             c = (unsigned)(i - r * s.per_row.d);
         }
-        const char *sp = s.src + r * s.src_pitch + (long long)c * s.vec;
-        char *dp = s.dst + r * s.dst_pitch + (long long)c * s.vec;
-        if (s.vec == 16)
-            *reinterpret_cast<v4i *>(dp) = *reinterpret_cast<const v4i *>(sp);
-        else if (s.vec == 4)
-            *reinterpret_cast<int *>(dp) = *reinterpret_cast<const int *>(sp);
-        else
-            *dp = *sp;
+        sp = s.src + r * s.src_pitch + (long long)c * s.vec;
+        dp = s.dst + r * s.dst_pitch + (long long)c * s.vec;
+    };
+    for (long long i0 = (long long)blockIdx.x * kBlock + threadIdx.x; i0 < total; i0 += 4 * stride) {
+        if (s.vec == 16) {
+            v4i v[4];
+            char *dp[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const long long i = i0 + j * stride;
+                const char *sp;
+                locate(i < total ? i : i0, sp, dp[j]);
+                v[j] = *reinterpret_cast<const v4i *>(sp);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (i0 + j * stride < total)
+                    *reinterpret_cast<v4i *>(dp[j]) = v[j];
+        } else {
+            for (int j = 0; j < 4; j++) {
+                const long long i = i0 + j * stride;
+                if (i >= total)
+                    break;
+                const char *sp;
+                char *dp;
+                locate(i, sp, dp);
+                if (s.vec == 4)
+                    *reinterpret_cast<int *>(dp) = *reinterpret_cast<const int *>(sp);
+                else
+                    *dp = *sp;
+            }
+        }
     }
 }
 
@@ -83,7 +111,7 @@ inline bool fill_seg(RowSeg &s, const void *src, long long src_pitch, void *dst,
 
 inline unsigned blocks_for(long long work, int cu_count)
 {
-    const long long want = (work + kBlock - 1) / kBlock;
+    const long long want = (work + 4 * kBlock - 1) / (4 * kBlock); // four pieces per thread and pass
     const long long cap = (long long)(cu_count > 0 ? cu_count : 256) * 32; // grid-stride beyond this
     return (unsigned)std::max<long long>(1, std::min(want, cap));
 }
@@ -429,6 +457,46 @@ hipError_t launch_copy_rows(const void *src, long long src_pitch, void *dst, lon
     return hipGetLastError();
 }
 
+namespace {
+// Concat walked in OUTPUT order: piece o of the output (16 bytes) lies in row o / per_row at column o % per_row,
+// and the column says which input it comes from.  Every store of a wavefront is then a run of whole cache lines;
+// with one pass per input the two halves of a 128-byte line arrive from different workgroups at different times
+// (measured on 64 + 64 channels: 4.2 TB/s per-input, see the table in the kernel list for this form).
+struct ConcatArgs {
+    const char *src[kMaxSeg];
+    unsigned first[kMaxSeg + 1]; // first output piece (of a row) of input j; first[n] = pieces per row
+    unsigned pieces[kMaxSeg];    // pieces per row of input j
+    int n;
+    char *dst;
+    long long rows;
+    FastDiv per_row;
+};
+
+__global__ __launch_bounds__(kBlock) void concat_rows_kernel(const ConcatArgs a)
+{
+    const long long total = a.rows * a.per_row.d; // below 2^31 (checked on the host)
+    const long long stride = (long long)gridDim.x * kBlock;
+    for (long long i0 = (long long)blockIdx.x * kBlock + threadIdx.x; i0 < total; i0 += 4 * stride) {
+        v4i v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const long long i = i0 + j * stride < total ? i0 + j * stride : i0;
+            const unsigned r = fastdiv((unsigned)i, a.per_row);
+            const unsigned c = (unsigned)i - r * a.per_row.d;
+            int seg = 0;
+#pragma unroll
+            for (int k = 1; k < kMaxSeg; k++)
+                seg += (k < a.n && c >= a.first[k]) ? 1 : 0;
+            v[j] = *reinterpret_cast<const v4i *>(a.src[seg] + ((long long)r * a.pieces[seg] + (c - a.first[seg])) * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (i0 + j * stride < total)
+                reinterpret_cast<v4i *>(a.dst)[i0 + j * stride] = v[j];
+    }
+}
+} // namespace
+
 hipError_t launch_concat(int n_inputs, const void *const *inputs, const long long *copy_bytes, long long loop_times,
                          void *out, int cu_count, hipStream_t stream)
 {
@@ -437,6 +505,34 @@ hipError_t launch_concat(int n_inputs, const void *const *inputs, const long lon
         total += copy_bytes[j];
     if (loop_times <= 0 || total <= 0)
         return hipSuccess;
+    {
+        // output-order form: up to kMaxSeg inputs, everything in whole aligned 16-byte pieces
+        bool ok = n_inputs <= kMaxSeg && (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (total & 15) == 0 &&
+            loop_times * (total / 16) <= 0x7fffffffll;
+        ConcatArgs a = {};
+        unsigned first = 0;
+        int n = 0;
+        for (int j = 0; ok && j < n_inputs; j++) {
+            if (copy_bytes[j] == 0)
+                continue;
+            ok = (copy_bytes[j] & 15) == 0 && (reinterpret_cast<uintptr_t>(inputs[j]) & 15) == 0;
+            a.src[n] = static_cast<const char *>(inputs[j]);
+            a.first[n] = first;
+            a.pieces[n] = (unsigned)(copy_bytes[j] / 16);
+            first += a.pieces[n];
+            n++;
+        }
+        if (ok && n > 0) {
+            for (int k = n; k <= kMaxSeg; k++)
+                a.first[k] = first;
+            a.n = n;
+            a.dst = static_cast<char *>(out);
+            a.rows = loop_times;
+            a.per_row = make_fastdiv(first);
+            hipLaunchKernelGGL(concat_rows_kernel, dim3(blocks_for(loop_times * first, cu_count)), dim3(kBlock), 0, stream, a);
+            return hipGetLastError();
+        }
+    }
     long long prefix = 0;
     for (int j0 = 0; j0 < n_inputs; j0 += kMaxSeg) {
         RowCopyArgs a;
