@@ -23,7 +23,8 @@ class ConvDesc(ctypes.Structure):
     """espdl_hip_conv_desc"""
     _fields_ = [(n, ctypes.c_int32) for n in (
         "dtype", "batch", "in_h", "in_w", "in_c", "out_c", "k_h", "k_w", "stride_h", "stride_w", "dil_h", "dil_w",
-        "pad_top", "pad_bottom", "pad_left", "pad_right", "group", "activation", "round_mode", "n_shift")]
+        "pad_top", "pad_bottom", "pad_left", "pad_right", "group", "activation", "round_mode", "n_shift",
+        "in_pitch", "out_pitch", "res_pitch")]
 
 
 class MbconvDesc(ctypes.Structure):
@@ -169,16 +170,30 @@ def conv_out_shape(desc):
     return oh.value, ow.value
 
 
+def _channel_pitch(t):
+    """0 for a dense NHWC tensor; the pixel pitch for a channel slice t = wide[..., a:b] of a dense tensor."""
+    if t is None or t.is_contiguous():
+        return 0
+    n, h, w, c = t.shape
+    st = t.stride()
+    if st[3] != 1 or st[1] != w * st[2] or st[0] != h * st[1] or st[2] < c:
+        raise ValueError("only channel slices of dense NHWC tensors can be passed without a copy")
+    return st[2]
+
+
 def conv2d(x, filt, bias, shift, k, stride=(1, 1), dilation=(1, 1), pads=(0, 0, 0, 0), depthwise=False,
            activation=LINEAR, round_mode=ROUND_HALF_UP, lut=None, out=None, stream=None, residual=None):
     """x [N,H,W,C] int8|int16 CUDA tensor; filt dense [OC][kH][kW][C] or depthwise [kH][kW][C];
-    bias int32|int64 [OC] or None; shift int32 tensor with 1 or OC entries (device)."""
+    bias int32|int64 [OC] or None; shift int32 tensor with 1 or OC entries (device).  x, out and residual may be
+    channel slices of wider NHWC tensors (wide[..., a:b]): they are read / written in place through the
+    descriptor's pitches."""
     import torch
     dtype = S8 if x.dtype == torch.int8 else S16
     n, h, w, c = x.shape
     out_c = c if depthwise else filt.numel() // (k[0] * k[1] * c)
     desc = make_desc(x.shape, out_c, k, stride, dilation, pads, c if depthwise else 1, activation, round_mode,
                      shift.numel(), dtype)
+    desc.in_pitch, desc.out_pitch, desc.res_pitch = _channel_pitch(x), _channel_pitch(out), _channel_pitch(residual)
     oh, ow = conv_out_shape(desc)
     if out is None:
         out = torch.empty((n, oh, ow, out_c), dtype=x.dtype, device=x.device)

@@ -26,7 +26,8 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     a.out = out;
     a.g = g;
     a.npix = (long long)g.batch * g.out_h * g.out_w;
-    a.in_bytes = (long long)g.batch * g.in_h * g.in_w * g.in_c;
+    // bytes a load may touch: up to the last channel of the last pixel of the (possibly pitched) input
+    a.in_bytes = ((long long)g.batch * g.in_h * g.in_w - 1) * g.in_pitch + g.in_c;
     if (a.npix == 0)
         return hipSuccess;
 
@@ -38,9 +39,9 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
         g.pad_left == 0 && g.out_h == g.in_h && g.out_w == g.in_w;
     if (flat)
         bmode = B_POINT;
-    else if ((g.in_c & 15) == 0 && aligned16)
+    else if ((g.in_c & 15) == 0 && (g.in_pitch & 15) == 0 && aligned16)
         bmode = B_VEC16;
-    else if (g.dil_w == 1)
+    else if (g.dil_w == 1 && g.in_pitch == g.in_c) // a filter row's bytes are contiguous in a dense input only
         bmode = B_ROWSEG;
     a.seg_len = a.seg_pad = 0;
     a.K = g.k_h * g.k_w * g.in_c;
@@ -92,7 +93,7 @@ hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8
     a.n_sets = (int)((a.npix + 64 * pt - 1) / (64 * pt));
     // contiguous output: needs every filter group in one chunk, 4-byte aligned rows and room in LDS
     const size_t out_tiles = (size_t)4 * 16 * pt * g.out_c;
-    a.stage_out = (n_chunks == 1 && a.out_vec >= 4 && (out_addr & 15) == 0 &&
+    a.stage_out = (n_chunks == 1 && a.out_vec >= 4 && (out_addr & 15) == 0 && g.out_pitch == g.out_c && g.res_pitch == g.out_c &&
                    lds + out_tiles <= 40 * 1024) ? 1 : 0;
     if (a.stage_out)
         lds += out_tiles;

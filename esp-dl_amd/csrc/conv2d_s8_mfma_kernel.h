@@ -177,7 +177,7 @@ __device__ __forceinline__ v4i load_b(const MfmaConvArgs &a, bool valid, long lo
         const int ky = (int)fastdiv((unsigned)tap, a.fd_k_w), kx = tap - ky * g.k_w;
         const int iy = iy0 + ky * g.dil_h, ix = ix0 + kx * g.dil_w;
         if ((unsigned)iy < (unsigned)g.in_h && (unsigned)ix < (unsigned)g.in_w)
-            r = *reinterpret_cast<const v4i *>(a.in + img_off + ((long long)iy * g.in_w + ix) * g.in_c + c0);
+            r = *reinterpret_cast<const v4i *>(a.in + img_off + ((long long)iy * g.in_w + ix) * g.in_pitch + c0);
         return r;
     }
     if (BMODE == B_ROWSEG) {
@@ -219,7 +219,7 @@ __device__ __forceinline__ v4i load_b(const MfmaConvArgs &a, bool valid, long lo
     for (int b = 0; b < n; b++) {
         const int iy = iy0 + ky * g.dil_h, ix = ix0 + kx * g.dil_w;
         if ((unsigned)iy < (unsigned)g.in_h && (unsigned)ix < (unsigned)g.in_w) {
-            const unsigned char v = (unsigned char)a.in[img_off + ((long long)iy * g.in_w + ix) * g.in_c + c];
+            const unsigned char v = (unsigned char)a.in[img_off + ((long long)iy * g.in_w + ix) * g.in_pitch + c];
             words[b >> 2] |= (unsigned int)v << ((b & 3) * 8);
         }
         if (++c == g.in_c) {
@@ -245,7 +245,7 @@ template <int BMODE, int PT>
 __device__ __forceinline__ void decode_set(const MfmaConvArgs &a, int set, int wave, int col, PixelRef (&px)[PT])
 {
     const ConvGeom &g = a.g;
-    const long long img_bytes = (long long)g.in_h * g.in_w * g.in_c;
+    const long long img_bytes = (long long)g.in_h * g.in_w * g.in_pitch;
 #pragma unroll
     for (int p = 0; p < PT; p++) {
         const unsigned int pix = ((unsigned)set * 4u + (unsigned)wave) * (16u * PT) + p * 16 + col;
@@ -253,7 +253,7 @@ __device__ __forceinline__ void decode_set(const MfmaConvArgs &a, int set, int w
         px[p].valid = (long long)pix < a.npix;
         if (BMODE == B_POINT) {
             // flat pointwise: output pixel i reads input pixel i, no coordinates needed
-            px[p].img_off = (long long)pix * g.in_c;
+            px[p].img_off = (long long)pix * g.in_pitch;
             px[p].iy0 = px[p].ix0 = 0;
             continue;
         }
@@ -418,7 +418,8 @@ __device__ __forceinline__ void run_group(const MfmaConvArgs &a, const WaveCtx &
         }
         if (!px[p].valid)
             continue;
-        const long long goff = (long long)px[p].pix * OC + c_lane;
+        const long long goff = (long long)px[p].pix * a.g.out_pitch + c_lane;  // output and residual operand may be
+        const long long roff = (long long)px[p].pix * a.g.res_pitch + c_lane; // channel slices of wider tensors
         int8_t *dst = a.out + goff;
         // Stores (and residual loads) take the widest piece that exists: 16 bytes when the lane's 16 channels do,
         // else 4 bytes per filter tile, single bytes only for the last channels of a row.  No piece needs an
@@ -426,7 +427,7 @@ __device__ __forceinline__ void run_group(const MfmaConvArgs &a, const WaveCtx &
         if (NT == 4 && c_lane + 16 <= OC) {
             v4i v = {words[0], words[NT > 1 ? 1 : 0], words[NT > 2 ? 2 : 0], words[NT > 3 ? 3 : 0]};
             if (a.res != nullptr) {
-                const v4i r = *reinterpret_cast<const v4i_unaligned *>(a.res + goff);
+                const v4i r = *reinterpret_cast<const v4i_unaligned *>(a.res + roff);
 #pragma unroll
                 for (int d = 0; d < 4; d++)
                     v[d] = sat_add4_s8(v[d], r[d]);
@@ -438,14 +439,14 @@ __device__ __forceinline__ void run_group(const MfmaConvArgs &a, const WaveCtx &
                 if (c_lane + 4 * t + 4 <= OC) {
                     int v = words[t];
                     if (a.res != nullptr)
-                        v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(a.res + goff + 4 * t));
+                        v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(a.res + roff + 4 * t));
                     *reinterpret_cast<int_unaligned *>(dst + 4 * t) = v;
                 } else {
                     for (int r = 0; r < 4; r++)
                         if (c_lane + 4 * t + r < OC) {
                             int v = (int)(int8_t)(words[t] >> (8 * r));
                             if (a.res != nullptr)
-                                v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
+                                v = clamp_s8(v + (int)a.res[roff + 4 * t + r]);
                             dst[4 * t + r] = (int8_t)v;
                         }
                 }

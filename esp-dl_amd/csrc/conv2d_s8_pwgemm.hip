@@ -43,6 +43,7 @@ struct PwArgs {
     int8_t *out;       // [M][N]
     long long M;
     int K, N;
+    int in_pitch, out_pitch, res_pitch; // bytes between consecutive rows of in, out and res (K, N, N when dense)
     int ksteps;
     int relu, half_even, n_shift;
     int out_vec; // 16, 4 or 1
@@ -123,7 +124,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
         for (int j = 0; j < kPiecesB; j++) {
             const int p = tid + j * kThreads;
             const long long m = row_pixel(p >> 2);
-            pb[j] = m >= 0 ? piece(a.in + m * a.K, k0 + 16 * (p & 3)) : v4i{0, 0, 0, 0};
+            pb[j] = m >= 0 ? piece(a.in + m * a.in_pitch, k0 + 16 * (p & 3)) : v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int j = 0; j < kPiecesA; j++) {
@@ -276,13 +277,13 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
                 }
                 if (m >= a.M || n >= a.N)
                     continue;
-                const long long goff = m * a.N + n;
+                const long long goff = m * a.out_pitch + n, roff = m * a.res_pitch + n;
                 // the widest piece that exists, at any byte address: 16 bytes, else 4 per filter tile, bytes for
                 // the last channels of a row (a row length that is not a multiple of 4 costs only those)
                 if (n + 16 <= a.N) {
                     v4i v = {words[0], words[1], words[2], words[3]};
                     if (a.res != nullptr) {
-                        const v4i r = *reinterpret_cast<const v4i_unaligned *>(a.res + goff);
+                        const v4i r = *reinterpret_cast<const v4i_unaligned *>(a.res + roff);
     #pragma unroll
                         for (int d = 0; d < 4; d++)
                             v[d] = sat_add4_s8(v[d], r[d]);
@@ -297,14 +298,14 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
                         if (n + 4 * t + 4 <= a.N) {
                             int v = words[t];
                             if (a.res != nullptr)
-                                v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(a.res + goff + 4 * t));
+                                v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(a.res + roff + 4 * t));
                             *reinterpret_cast<int_unaligned *>(a.out + goff + 4 * t) = v;
                         } else {
                             for (int r = 0; r < 4; r++)
                                 if (n + 4 * t + r < a.N) {
                                     int v = (int)(int8_t)(words[t] >> (8 * r));
                                     if (a.res != nullptr)
-                                        v = clamp_s8(v + (int)a.res[goff + 4 * t + r]);
+                                        v = clamp_s8(v + (int)a.res[roff + 4 * t + r]);
                                     a.out[goff + 4 * t + r] = (int8_t)v;
                                 }
                         }
@@ -422,7 +423,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_rows_kernel(const PwArgs a
     const long long row = min(m0 + col, a.M - 1);
     const int flt = min(n0 + col, a.N - 1);
     const v4i *pa = reinterpret_cast<const v4i *>(a.w + (long long)flt * a.K + 16 * quad);
-    const v4i *pb = reinterpret_cast<const v4i *>(a.in + row * a.K + 16 * quad);
+    const v4i *pb = reinterpret_cast<const v4i *>(a.in + row * a.in_pitch + 16 * quad);
     v4i ca[G], cb[G], na[G], nb[G];
 #pragma unroll
     for (int i = 0; i < G; i++) {
@@ -466,7 +467,7 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_rows_kernel(const PwArgs a
     }
     if (m >= a.M || n >= a.N)
         return;
-    int8_t *dst = a.out + m * a.N + n;
+    int8_t *dst = a.out + m * a.out_pitch + n;
     if (a.out_vec >= 4 && n + 4 <= a.N) {
         *reinterpret_cast<int *>(dst) = pack4_s8(q[0], q[1], q[2], q[3]);
     } else {
@@ -488,7 +489,8 @@ bool conv2d_s8_pwgemm_supports(const ConvGeom &g, const void *in, const void *fi
     if (!flat || g.in_c < 64 || g.out_c < 32)
         return false;
     // rows of a multiple of 16 bytes are read with aligned loads; any other length with loads that need none
-    if ((g.in_c & 15) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) != 0)
+    if ((g.in_c & 15) == 0 && (g.in_pitch & 15) == 0 &&
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) != 0)
         return false;
     const long long npix = (long long)g.batch * g.out_h * g.out_w;
     const int cus = cu_count > 0 ? cu_count : 256;
@@ -506,7 +508,7 @@ bool conv2d_s8_rows_supports(const ConvGeom &g, const void *in, const void *filt
 {
     const bool flat = g.k_h == 1 && g.k_w == 1 && g.stride_h == 1 && g.stride_w == 1 && g.pad_top == 0 &&
         g.pad_left == 0 && g.out_h == g.in_h && g.out_w == g.in_w;
-    if (!flat || (g.in_c & 63) != 0 || g.out_c < 1 ||
+    if (!flat || (g.in_c & 63) != 0 || g.out_c < 1 || (g.in_pitch & 15) != 0 ||
         ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) != 0)
         return false;
     const long long npix = (long long)g.batch * g.out_h * g.out_w;
@@ -529,6 +531,9 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
     a.M = (long long)g.batch * g.out_h * g.out_w;
     a.K = g.in_c;
     a.N = g.out_c;
+    a.in_pitch = g.in_pitch;
+    a.out_pitch = g.out_pitch;
+    a.res_pitch = g.res_pitch;
     a.ksteps = (a.K + 63) / 64;
     a.relu = g.relu;
     a.half_even = g.half_even;
@@ -536,7 +541,8 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
     a.hw = 0;
     a.gap_scale = 0.f;
     const uintptr_t oaddr = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(residual);
-    a.out_vec = ((a.N & 15) == 0 && (oaddr & 15) == 0) ? 16 : (((a.N & 3) == 0 && (oaddr & 3) == 0) ? 4 : 1);
+    a.out_vec = ((a.N & 15) == 0 && (oaddr & 15) == 0 && (a.out_pitch & 15) == 0) ? 16
+        : (((a.N & 3) == 0 && (oaddr & 3) == 0 && (a.out_pitch & 3) == 0) ? 4 : 1);
     if (a.M == 0)
         return hipSuccess;
     // 64-filter tiles: measured faster than 128 on every MobileNetV2 layer (more, shorter workgroups).
@@ -545,12 +551,12 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
     const long long tiles128 = (a.M + 127) / 128;
     const int cus = cu_count > 0 ? cu_count : 256;
     // fewer 64 x 64 tiles than compute units: one wavefront per 16 x 16 tile, operands straight from global memory
-    if (lut == nullptr && residual == nullptr && (a.K & 63) == 0 && (a.M + 63) / 64 * gy < cus) {
+    if (lut == nullptr && residual == nullptr && (a.K & 63) == 0 && (a.in_pitch & 15) == 0 && (a.M + 63) / 64 * gy < cus) {
         hipLaunchKernelGGL((conv2d_s8_rows_kernel<10>), dim3((unsigned)((a.M + 63) / 64), (unsigned)((a.N + 15) / 16)),
                            dim3(kThreads), 0, stream, a);
         return hipGetLastError();
     }
-    const bool k16 = (a.K & 15) == 0;
+    const bool k16 = (a.K & 15) == 0 && (a.in_pitch & 15) == 0;
     if (tiles128 * gy * 2 < 3ll * cus) {
         if (k16)
             hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1>), dim3((unsigned)((a.M + 63) / 64), gy), dim3(kThreads), 0, stream, a);
@@ -570,7 +576,7 @@ bool conv2d_gap_s8_supports(const ConvGeom &g, const void *in, const void *filte
 {
     const bool flat = g.k_h == 1 && g.k_w == 1 && g.stride_h == 1 && g.stride_w == 1 && g.pad_top == 0 &&
         g.pad_left == 0 && g.out_h == g.in_h && g.out_w == g.in_w;
-    return flat && (g.in_c & 15) == 0 && g.in_c >= 64 && g.out_c >= 32 && g.out_h * g.out_w <= 64 && g.batch <= 0x7fffffff &&
+    return flat && g.in_pitch == g.in_c && (g.in_c & 15) == 0 && g.in_c >= 64 && g.out_c >= 32 && g.out_h * g.out_w <= 64 && g.batch <= 0x7fffffff &&
         ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) == 0;
 }
 
@@ -590,6 +596,8 @@ hipError_t launch_conv2d_gap_s8(const ConvGeom &g, const int8_t *in, const int8_
     a.M = (long long)g.batch * a.hw;
     a.K = g.in_c;
     a.N = g.out_c;
+    a.in_pitch = g.in_c;
+    a.out_pitch = a.res_pitch = g.out_c;
     a.ksteps = (a.K + 63) / 64;
     a.relu = g.relu;
     a.half_even = g.half_even;

@@ -78,7 +78,7 @@ __device__ __forceinline__ int group_tiles(int out_c, int gbase)
 }
 
 struct TileRef {
-    long long img_in, img_out; // byte offsets of the tile's image in the input and output tensors
+    long long img_in, img_out, img_res; // byte offsets of the tile's image in the input, output and residual tensors
     int oy0, ox0, iy0, ix0, th_real, tw_real;
 };
 
@@ -90,8 +90,9 @@ __device__ __forceinline__ TileRef decode_tile(const TiledArgs &a, int tile)
     const unsigned ty = fastdiv(rem, a.fd_tiles_x);
     const unsigned tx = rem - ty * a.fd_tiles_x.d;
     TileRef t;
-    t.img_in = (long long)n * g.in_h * g.in_w * g.in_c;
-    t.img_out = (long long)n * g.out_h * g.out_w * g.out_c;
+    t.img_in = (long long)n * g.in_h * g.in_w * g.in_pitch;
+    t.img_out = (long long)n * g.out_h * g.out_w * g.out_pitch;
+    t.img_res = (long long)n * g.out_h * g.out_w * g.res_pitch;
     t.oy0 = (int)ty * a.th;
     t.ox0 = (int)tx * a.tw;
     t.iy0 = t.oy0 * g.stride_h - g.pad_top;
@@ -117,7 +118,7 @@ struct Ctx {
 // product and the store; 1 - 64 filters, 16-byte stores, table and / or residual; 2 - anything else.
 template <int PT, int NT, int MODE, bool HE, int EPI>
 __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t *out_img, const int8_t *res_img,
-                                        const int (&pixoff)[PT], const int (&ooff)[PT], unsigned okmask, int gi, int gbase)
+                                        const int (&pixoff)[PT], const int (&opix)[PT], unsigned okmask, int gi, int gbase)
 {
     const int OC = a.g.out_c;
     const int c_local = gi * 64 + 4 * NT * c.quad;
@@ -203,7 +204,10 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
                 words[t] = pack4_s8(q[0], q[1], q[2], q[3]);
             }
         }
-        const unsigned go = (unsigned)(ooff[p] + c_lane); // inside the image: below 2^31
+        // pixel index inside the image times the channel pitch of the output (and of the residual operand, which
+        // may be a channel slice of another tensor): below 2^31
+        const unsigned go = (unsigned)(opix[p] * a.g.out_pitch + c_lane);
+        const unsigned ro = (unsigned)(opix[p] * a.g.res_pitch + c_lane);
         const bool ok = (okmask >> p) & 1u;
         if constexpr (EPI == 0) {
             if (ok)
@@ -225,7 +229,7 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
         if (EPI == 1 || (NT == 4 && c_lane + 16 <= OC)) {
             v4i v = {words[0], words[NT > 1 ? 1 : 0], words[NT > 2 ? 2 : 0], words[NT > 3 ? 3 : 0]};
             if (res_img != nullptr) {
-                const v4i r = *reinterpret_cast<const v4i_unaligned *>(res_img + (size_t)go);
+                const v4i r = *reinterpret_cast<const v4i_unaligned *>(res_img + (size_t)ro);
 #pragma unroll
                 for (int d = 0; d < 4; d++)
                     v[d] = sat_add4_s8(v[d], r[d]);
@@ -237,14 +241,14 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
                 if (c_lane + 4 * t + 4 <= OC) {
                     int v = words[t];
                     if (res_img != nullptr)
-                        v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(res_img + (size_t)go + 4 * t));
+                        v = sat_add4_s8(v, *reinterpret_cast<const int_unaligned *>(res_img + (size_t)ro + 4 * t));
                     *reinterpret_cast<int_unaligned *>(dst + 4 * t) = v;
                 } else {
                     for (int r = 0; r < 4; r++)
                         if (c_lane + 4 * t + r < OC) {
                             int v = (int)(int8_t)(words[t] >> (8 * r));
                             if (res_img != nullptr)
-                                v = clamp_s8(v + (int)res_img[(size_t)go + 4 * t + r]);
+                                v = clamp_s8(v + (int)res_img[(size_t)ro + 4 * t + r]);
                             dst[4 * t + r] = (int8_t)v;
                         }
                 }
@@ -261,11 +265,11 @@ __device__ __forceinline__ void run_tile(const TiledArgs &a, const Ctx &c, const
     const ConvGeom &g = a.g;
     const int OC = g.out_c;
     int8_t *out_img = a.out + tr.img_out;
-    const int8_t *res_img = a.res != nullptr ? a.res + tr.img_out : nullptr;
-    const int org_out = (tr.oy0 * g.out_w + tr.ox0) * OC;
+    const int8_t *res_img = a.res != nullptr ? a.res + tr.img_res : nullptr;
+    const int org_out = tr.oy0 * g.out_w + tr.ox0; // in pixels
     for (int set = wave; set < a.n_sets; set += n_waves) {
         int pixoff[PT];
-        int ooff[PT];
+        int opix[PT];
         unsigned okmask = 0;
 #pragma unroll
         for (int p = 0; p < PT; p++) {
@@ -288,25 +292,25 @@ __device__ __forceinline__ void run_tile(const TiledArgs &a, const Ctx &c, const
             }
             const bool ok = live && oy_l < tr.th_real && ox_l < tr.tw_real;
             okmask |= ok ? 1u << p : 0u;
-            ooff[p] = org_out + (oy_l * g.out_w + ox_l) * OC;
+            opix[p] = org_out + oy_l * g.out_w + ox_l;
         }
         for (int gi = 0; gi < g_count; gi++) {
             const int gbase = (g_first + gi) * 64;
             if constexpr (EPI != 2) {
-                run_set<PT, 4, MODE, HE, EPI>(a, c, out_img, res_img, pixoff, ooff, okmask, gi, gbase);
+                run_set<PT, 4, MODE, HE, EPI>(a, c, out_img, res_img, pixoff, opix, okmask, gi, gbase);
             } else {
                 switch (group_tiles(OC, gbase)) { // uniform
                 case 4:
-                    run_set<PT, 4, MODE, HE, 2>(a, c, out_img, res_img, pixoff, ooff, okmask, gi, gbase);
+                    run_set<PT, 4, MODE, HE, 2>(a, c, out_img, res_img, pixoff, opix, okmask, gi, gbase);
                     break;
                 case 3:
-                    run_set<PT, 3, MODE, HE, 2>(a, c, out_img, res_img, pixoff, ooff, okmask, gi, gbase);
+                    run_set<PT, 3, MODE, HE, 2>(a, c, out_img, res_img, pixoff, opix, okmask, gi, gbase);
                     break;
                 case 2:
-                    run_set<PT, 2, MODE, HE, 2>(a, c, out_img, res_img, pixoff, ooff, okmask, gi, gbase);
+                    run_set<PT, 2, MODE, HE, 2>(a, c, out_img, res_img, pixoff, opix, okmask, gi, gbase);
                     break;
                 default:
-                    run_set<PT, 1, MODE, HE, 2>(a, c, out_img, res_img, pixoff, ooff, okmask, gi, gbase);
+                    run_set<PT, 1, MODE, HE, 2>(a, c, out_img, res_img, pixoff, opix, okmask, gi, gbase);
                     break;
                 }
             }
@@ -357,7 +361,7 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     const int st_cu = ru - (int)st_px * a.cu16;
     const unsigned st_pxq = fastdiv(st_px, a.fd_sw);
     const int st_phase = (int)st_px - (int)st_pxq * g.stride_w;
-    const int st_src0 = ((int)r0 * g.in_w + (int)st_px) * g.in_c + 16 * st_cu;
+    const int st_src0 = ((int)r0 * g.in_w + (int)st_px) * g.in_pitch + 16 * st_cu;
     const int st_dst0 = (((int)r0 * g.stride_w + st_phase) * a.pwp + (int)st_pxq) * a.cs + 16 * st_cu;
     // rows of this thread: r0, r0 + row_par, ... below ph
     const int st_rows = st_active ? (a.ph - (int)r0 + a.row_par - 1) / a.row_par : 0;
@@ -373,7 +377,7 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
         return y_in && (x_in || one_col);
     };
     auto request = [&](const TileRef &t) {
-        const int org = (t.iy0 * g.in_w + t.ix0) * g.in_c;
+        const int org = (t.iy0 * g.in_w + t.ix0) * g.in_pitch;
         pre_short = tile_short(t);
         const int8_t *img = a.in + t.img_in;
         if (pre_short) {
@@ -587,7 +591,8 @@ TiledPlan tiled_plan(const ConvGeom &g, const void *in, const void *filter, int 
         return best;
     if ((reinterpret_cast<uintptr_t>(in) & 15) != 0 || (reinterpret_cast<uintptr_t>(filter) & 15) != 0)
         return best;
-    if ((long long)g.in_h * g.in_w * g.in_c >= (1ll << 31) || (long long)g.out_h * g.out_w * g.out_c >= (1ll << 31))
+    if ((long long)g.in_h * g.in_w * g.in_pitch >= (1ll << 31) || (long long)g.out_h * g.out_w * g.out_pitch >= (1ll << 31) ||
+        (long long)g.out_h * g.out_w * g.res_pitch >= (1ll << 31) || (g.in_pitch & 15) != 0)
         return best;
     if (g.stride_h != g.stride_w || g.stride_w > 4)
         return best;
@@ -698,7 +703,7 @@ TiledPlan tiled_plan(const ConvGeom &g, const void *in, const void *filter, int 
                         a.n_tiles = (int)std::min<long long>(n_tiles, 0x7fffffff);
                         a.row_units = row_units;
                         a.row_par = row_par;
-                        a.src_row_step = row_par * g.in_w * g.in_c;
+                        a.src_row_step = row_par * g.in_w * g.in_pitch;
                         a.lds_row_step = row_par * s * pwp * cs;
                         a.off_tabs = w_bytes;
                         a.off_koff = w_bytes + gpc * 768;
@@ -785,7 +790,10 @@ hipError_t launch_conv2d_s8_tiled(const ConvGeom &g, const int8_t *in, const int
     a.out = out;
     const uintptr_t out_addr = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(residual);
     a.out_vec = ((g.out_c & 15) == 0 && (out_addr & 15) == 0) ? 16 : (((g.out_c & 3) == 0 && (out_addr & 3) == 0) ? 4 : 1);
-    a.epi = (g.out_c % 64 == 0 && a.out_vec == 16) ? ((lut == nullptr && residual == nullptr) ? 0 : 1) : 2;
+    // the 16-byte-store forms need every store (and residual load) aligned: pitches of whole 16-byte pieces
+    a.epi = (g.out_c % 64 == 0 && a.out_vec == 16 && (g.out_pitch & 15) == 0 && (g.res_pitch & 15) == 0)
+        ? ((lut == nullptr && residual == nullptr) ? 0 : 1)
+        : 2;
     a.fd_cu16 = make_fastdiv((unsigned)a.cu16);
     a.fd_row_units = make_fastdiv((unsigned)a.row_units);
     a.fd_sw = make_fastdiv((unsigned)g.stride_w);

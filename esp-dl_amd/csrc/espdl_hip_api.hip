@@ -107,6 +107,15 @@ int derive_geometry(const espdl_hip_conv_desc *d, espdl::ConvGeom *g)
     g->relu = d->activation == ESPDL_HIP_RELU;
     g->half_even = d->round_mode == ESPDL_HIP_ROUND_HALF_EVEN;
     g->n_shift = d->n_shift;
+    if (d->in_pitch < 0 || d->out_pitch < 0 || d->res_pitch < 0 || (d->in_pitch != 0 && d->in_pitch < d->in_c) ||
+        (d->out_pitch != 0 && d->out_pitch < d->out_c) || (d->res_pitch != 0 && d->res_pitch < d->out_c))
+        return fail(ESPDL_HIP_EINVAL, "channel pitches %d / %d / %d must be 0 or at least the channel counts", d->in_pitch,
+                    d->out_pitch, d->res_pitch);
+    g->in_pitch = d->in_pitch != 0 ? d->in_pitch : d->in_c;
+    g->out_pitch = d->out_pitch != 0 ? d->out_pitch : d->out_c;
+    g->res_pitch = d->res_pitch != 0 ? d->res_pitch : d->out_c;
+    if ((long long)d->batch * d->in_h * d->in_w * g->in_pitch > (1ll << 40) || (long long)d->batch * oh * ow * g->out_pitch > (1ll << 40))
+        return fail(ESPDL_HIP_ENOTSUP, "tensor too large for this build");
     return ESPDL_HIP_OK;
 }
 
@@ -166,6 +175,8 @@ int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const 
         return fail(ESPDL_HIP_EINVAL, "in, filter, shift and out must not be NULL");
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const bool depthwise = desc->group != 1;
+    if (!espdl::conv_is_dense(g) && (depthwise || desc->dtype != ESPDL_HIP_S8))
+        return fail(ESPDL_HIP_ENOTSUP, "channel pitches exist for dense int8 convolutions (group 1) only");
     if (desc->dtype == ESPDL_HIP_S8) {
         if (misaligned(bias, 4) || misaligned(shift, 4))
             return fail(ESPDL_HIP_EINVAL, "bias and shift must be 4-byte aligned");
@@ -826,6 +837,8 @@ void dwproject_from(const espdl::MbconvParams &p, espdl::ConvGeom *g, espdl::DwP
     g->relu = p.relu_dw;
     g->half_even = p.half_even;
     g->n_shift = p.n_s_dw;
+    g->in_pitch = g->in_c;
+    g->out_pitch = g->res_pitch = g->out_c;
     pj->w = p.w_project;
     pj->bias = p.b_project;
     pj->shift = p.s_project;
@@ -842,6 +855,7 @@ void expand_dwproject_from(const espdl::MbconvParams &p, espdl::ConvGeom *g, esp
     dwproject_from(p, g, pj);
     g->in_c = p.exp_c;
     g->out_c = p.exp_c;
+    g->in_pitch = g->out_pitch = g->res_pitch = p.exp_c;
     ex->x = p.in;
     ex->w = p.w_expand;
     ex->bias = p.b_expand;

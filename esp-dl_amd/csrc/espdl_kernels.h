@@ -15,7 +15,13 @@ struct ConvGeom {
     int out_c, out_h, out_w;
     int k_h, k_w, stride_h, stride_w, dil_h, dil_w, pad_top, pad_left;
     int relu, half_even, n_shift;
+    // channel pitches of input, output and residual operand in elements (>= the channel count; equal: dense)
+    int in_pitch, out_pitch, res_pitch;
 };
+inline bool conv_is_dense(const ConvGeom &g)
+{
+    return g.in_pitch == g.in_c && g.out_pitch == g.out_c && g.res_pitch == g.out_c;
+}
 
 // Dense int8 convolution / Gemm as an implicit GEMM on v_mfma_i32_16x16x64_i8.
 hipError_t launch_conv2d_s8_mfma(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,

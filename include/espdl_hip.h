@@ -65,6 +65,13 @@ typedef struct espdl_hip_conv_desc {
     int32_t activation; /* ESPDL_HIP_LINEAR / ESPDL_HIP_RELU */
     int32_t round_mode; /* ESPDL_HIP_ROUND_HALF_UP / ESPDL_HIP_ROUND_HALF_EVEN */
     int32_t n_shift;    /* 1 or out_c */
+    /* Channel pitches, in elements; 0 = dense (the tensor's own channel count).  A pitch larger than the channel
+     * count means the operand is a channel slice of a wider NHWC tensor: `in` / `out` / `residual` point at the
+     * slice's first channel of the first pixel and consecutive pixels lie pitch elements apart.  This is how a
+     * Conv reads one output of a Split (esp-dl/dl/module/include/dl_module_split.hpp:84-152) or writes its part
+     * of a Concat result (dl_module_concat.hpp:86-108) without the copy those operators make.  Dense int8
+     * convolutions (group 1) only; ESPDL_HIP_ENOTSUP elsewhere. */
+    int32_t in_pitch, out_pitch, res_pitch;
 } espdl_hip_conv_desc;
 
 /* Output spatial size, Conv::get_output_shape (esp-dl/dl/module/include/dl_module_conv.hpp:81-102). */

@@ -104,6 +104,56 @@ def test_conv2d_s8_lds_tiled(oracle, case, flavour):
     np.testing.assert_array_equal(got, want)
 
 
+# Operands that are channel slices of wider NHWC tensors (what a Conv reads from a Split output and writes into its
+# part of a Concat result), on every dense route: (name, (N, H, W), in_c, out_c, k, stride, pads,
+# (input offset, input width), (output offset, output width), (residual offset, residual width) or None, lut)
+PITCH_CASES = [
+    ("pw_few_pixels_64_64", (2, 7, 9), 64, 64, (1, 1), (1, 1), (0, 0, 0, 0), (32, 128), (64, 192), None, False),
+    ("pw_few_pixels_120_48_unaligned", (2, 5, 8), 120, 48, (1, 1), (1, 1), (0, 0, 0, 0), (8, 136), (5, 61), (3, 55), False),
+    ("pw_rows_64_32", (1, 1, 16), 64, 32, (1, 1), (1, 1), (0, 0, 0, 0), (64, 128), (32, 96), None, False),
+    ("pw_many_pixels_32_32", (2, 150, 160), 32, 32, (1, 1), (1, 1), (0, 0, 0, 0), (16, 64), (0, 96), (32, 64), True),
+    ("c3_tiled_32_32_residual", (2, 40, 40), 32, 32, (3, 3), (1, 1), (1, 1, 1, 1), (32, 64), (64, 96), (32, 64), True),
+    ("c3_tiled_64_64", (3, 30, 30), 64, 64, (3, 3), (1, 1), (1, 1, 1, 1), (0, 128), (64, 128), None, False),
+    ("c3s2_tiled_16_40", (2, 33, 35), 16, 40, (3, 3), (2, 2), (1, 1, 1, 1), (16, 48), (8, 56), (0, 40), False),
+    ("c3_gather_22_33", (2, 19, 23), 22, 33, (3, 3), (1, 1), (1, 1, 1, 1), (5, 40), (7, 47), (1, 34), False),
+    ("c3_direct_256_64", (1, 12, 12), 256, 64, (3, 3), (1, 1), (1, 1, 1, 1), (256, 512), (64, 192), None, True),
+]
+
+
+@pytest.mark.parametrize("case", PITCH_CASES, ids=lambda c: c[0])
+def test_conv2d_s8_channel_slices(oracle, case):
+    announce(f"conv2d_s8 on channel slices: {case[0]}")
+    name, (n, h, w), cin, cout, k, stride, pads, (io, iw), (oo, ow_), res, with_lut = case
+    m = espdl()
+    import torch
+    rng = np.random.default_rng(0x517C + len(name))
+    wide_in = rng_int8(rng, (n, h, w, iw))
+    x = np.ascontiguousarray(wide_in[..., io:io + cin])
+    f = rng_int8(rng, (cout, k[0], k[1], cin))
+    bias = rng.integers(-4096, 4097, size=cout).astype(np.int32)
+    shift = (typical_shift(k[0] * k[1] * cin) + rng.integers(-2, 3, size=cout)).astype(np.int32)
+    want = oracle.conv2d_s8(x, f, bias, shift, k, stride, (1, 1), pads, oracle.RELU, oracle.ROUND_HALF_UP)
+    lut = None
+    if with_lut:
+        lut = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8)
+        want = oracle.lut_s8(want, lut)
+    wide_res = None
+    if res is not None:
+        wide_res = rng_int8(rng, want.shape[:3] + (res[1],))
+        want = oracle.add_s8(want, np.ascontiguousarray(wide_res[..., res[0]:res[0] + cout]))
+    before = rng_int8(rng, want.shape[:3] + (ow_,))
+    d_in, d_out = to_dev(wide_in), to_dev(before)
+    d_res = to_dev(wide_res)
+    m.conv2d(d_in[..., io:io + cin], to_dev(f), to_dev(bias), to_dev(shift), k, stride, (1, 1), pads, activation=m.capi.RELU,
+             lut=to_dev(lut), out=d_out[..., oo:oo + cout], residual=None if res is None else d_res[..., res[0]:res[0] + cout])
+    got = to_host(d_out)
+    np.testing.assert_array_equal(got[..., oo:oo + cout], want)
+    # nothing outside the slice was touched
+    keep = np.ones(ow_, dtype=bool)
+    keep[oo:oo + cout] = False
+    np.testing.assert_array_equal(got[..., keep], before[..., keep])
+
+
 @pytest.mark.parametrize("shift", [-3, -1, 0, 1, 31, 33])
 def test_conv2d_s8_shift_range(oracle, shift):
     announce(f"conv2d_s8 shift={shift}")
