@@ -27,7 +27,7 @@ struct module_info {
     int64_t bytes;    ///< bytes of the tensors it reads and writes (each counted once)
 };
 
-enum { FUSE_CONV_LUT = 1, FUSE_DW_PROJECT = 2, FUSE_CONV_ADD = 4, FUSE_CONV_GAP = 8 };
+enum { FUSE_CONV_LUT = 1, FUSE_DW_PROJECT = 2, FUSE_CONV_ADD = 4, FUSE_CONV_GAP = 8, FUSE_CHANNEL_SLICES = 16 };
 
 class Model {
 public:
@@ -35,9 +35,12 @@ public:
     /// model creates its own).  `fuse` is a bit mask of graph fusions: FUSE_CONV_LUT folds a LUT that directly follows a Conv
     /// into its epilogue, FUSE_DW_PROJECT runs depthwise Conv -> 1x1 Conv [-> Add] as one kernel,
     /// FUSE_CONV_ADD folds the Add behind a dense Conv into its epilogue, FUSE_CONV_GAP runs a 1x1 Conv and the
-    /// GlobalAveragePool behind it as one kernel that writes the pooled tensor only.  All are exact and on by default.
+    /// GlobalAveragePool behind it as one kernel that writes the pooled tensor only, FUSE_CHANNEL_SLICES leaves the
+    /// outputs of a Split along the last axis inside its input and lets dense 8-bit Convs write straight into the
+    /// output of a Concat along the last axis (the modules stay in the plan and copy only what is not in place).
+    /// All are exact and on by default.
     Model(fbs::FbsModel *fbs_model, int batch = 1, round_mode_t round_mode = ROUND_MODE_HALF_UP, void *stream = nullptr,
-          int fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT | FUSE_CONV_ADD | FUSE_CONV_GAP);
+          int fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT | FUSE_CONV_ADD | FUSE_CONV_GAP | FUSE_CHANNEL_SLICES);
     virtual ~Model();
     Model(const Model &) = delete;
     Model &operator=(const Model &) = delete;
@@ -102,7 +105,7 @@ private:
     std::string m_name, m_doc_string;
     int64_t m_version = 0;
     int m_batch = 1;
-    int m_fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT | FUSE_CONV_ADD | FUSE_CONV_GAP;
+    int m_fuse = FUSE_CONV_LUT | FUSE_DW_PROJECT | FUSE_CONV_ADD | FUSE_CONV_GAP | FUSE_CHANNEL_SLICES;
     void *m_stream = nullptr;
     bool m_own_stream = false;
     void *m_graph = nullptr;      // hipGraph_t

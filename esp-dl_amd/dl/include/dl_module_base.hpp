@@ -56,6 +56,20 @@ public:
     /// capture, profiling passes) with the two calls, on `stream`.
     virtual void hold_state(void *stream) { (void)stream; }
     virtual void restore_state(void *stream) { (void)stream; }
+    /// Whether forward handles input `slot` (a position in m_inputs_index) / output `slot` being a channel
+    /// slice of a wider tensor (TensorBase::channel_pitch).  A model only leaves the output of a channel Split
+    /// inside the Split's input, or lets a producer write straight into the output of a channel Concat, when
+    /// every module that touches the tensor says yes here.
+    virtual bool reads_channel_slice(int slot) const
+    {
+        (void)slot;
+        return false;
+    }
+    virtual bool writes_channel_slice(int slot) const
+    {
+        (void)slot;
+        return false;
+    }
     /// Multiply-accumulates one forward performs for the given input shapes (0 for data movement);
     /// used by Model::profile to report achieved int8 OP/s.
     virtual int64_t get_macs(std::vector<std::vector<int>> &input_shapes)

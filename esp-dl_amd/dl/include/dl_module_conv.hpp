@@ -183,6 +183,14 @@ public:
         m_inputs_index.push_back(residual_index);
     }
     bool has_fused_residual() const { return m_residual_pos >= 0; }
+    /// A dense 8-bit convolution on its own (with or without a folded table or residual Add) passes channel
+    /// pitches to the kernels for its data input, its residual and its output.
+    bool handles_channel_slices() const
+    {
+        return quant_type == QUANT_TYPE_SYMM_8BIT && m_group == 1 && !m_has_project && !m_has_gap;
+    }
+    bool reads_channel_slice(int slot) const { return handles_channel_slices() && (slot == 0 || slot == m_residual_pos); }
+    bool writes_channel_slice(int slot) const { return handles_channel_slices() && slot == 0; }
     /// Absorb the GlobalAveragePool that is the only reader of this convolution's output: the module then
     /// writes the pooled tensor [N, 1, 1, C] (espdl_hip_conv2d_gap_s8); `conv_out_exponent` is the exponent of
     /// the tensor the convolution used to write.
@@ -313,6 +321,8 @@ public:
             return;
         }
         d.group = m_group == 1 ? 1 : d.in_c;
+        d.in_pitch = input->is_dense() ? 0 : input->channel_pitch;
+        d.out_pitch = output->is_dense() ? 0 : output->channel_pitch;
         d.activation = activation == ReLU ? ESPDL_HIP_RELU : ESPDL_HIP_LINEAR;
         if (activation != Linear && activation != ReLU) {
             DL_LOGE("Conv", "%s: only Linear and ReLU can be fused into Conv", name.c_str());
@@ -347,6 +357,7 @@ public:
             DL_LOGE("Conv", "%s: the residual must be a device tensor", name.c_str());
             return;
         }
+        d.res_pitch = residual && !residual->is_dense() ? residual->channel_pitch : 0;
         const int rc = espdl_hip_conv2d_add(&d, input->data, filter->data, bias ? bias->data : nullptr, shift_dev,
                                             m_fused_lut ? static_cast<const int8_t *>(m_fused_lut->data) : nullptr,
                                             residual ? static_cast<const int8_t *>(residual->data) : nullptr, output->data,

@@ -59,6 +59,7 @@ public:
         std::vector<const void *> ptrs;
         std::vector<int64_t> bytes;
         int64_t loop_times = 1;
+        bool sliced = false; // an input is a channel slice (possibly of the output itself)
         for (size_t j = 0; j < m_inputs_index.size(); j++) {
             TensorBase *input = context->get_tensor(m_inputs_index[j]);
             if (!input || !input->on_device() || input->dtype != output->dtype) {
@@ -73,11 +74,40 @@ public:
                     loop_times *= input->shape[i];
             ptrs.push_back(input->data);
             bytes.push_back(n * (int64_t)esize);
+            sliced = sliced || !input->is_dense();
+        }
+        if (sliced) {
+            // along the last axis only (the model makes no other slices): inputs that already lie in their
+            // place inside the output were written there by their producers; the others are copied row by row
+            if (m_axis != (int)output->shape.size() - 1 || !output->is_dense()) {
+                DL_LOGE("Concat", "%s: channel slices along another axis than the last", name.c_str());
+                return;
+            }
+            const int64_t out_row = (int64_t)output->shape.back() * (int64_t)esize;
+            int64_t at = 0;
+            for (size_t j = 0; j < ptrs.size(); j++) {
+                TensorBase *input = context->get_tensor(m_inputs_index[j]);
+                char *dst = static_cast<char *>(output->data) + at;
+                at += bytes[j];
+                if (ptrs[j] == dst && (int64_t)input->get_channel_pitch() * (int64_t)esize == out_row)
+                    continue;
+                const int rc = espdl_hip_copy_rows(ptrs[j], (int64_t)input->get_channel_pitch() * (int64_t)esize, dst, out_row,
+                                                   bytes[j], loop_times, context->stream);
+                if (rc != ESPDL_HIP_OK)
+                    DL_LOGE("Concat", "%s: %s", name.c_str(), espdl_hip_last_error());
+            }
+            return;
         }
         const int rc =
             espdl_hip_concat((int32_t)ptrs.size(), ptrs.data(), bytes.data(), loop_times, output->data, context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("Concat", "%s: %s", name.c_str(), espdl_hip_last_error());
+    }
+    int get_axis() const { return m_axis; }
+    bool reads_channel_slice(int slot) const
+    {
+        (void)slot;
+        return true; // along the last axis, which is the only one a model slices
     }
     static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
     {
@@ -146,6 +176,12 @@ public:
             slice_size *= input->shape[i];
         const int64_t esize = (int64_t)input->get_dtype_bytes();
         const int64_t in_axis = input->shape[m_axis];
+        if (!input->is_dense() && m_axis != (int)input->shape.size() - 1) {
+            DL_LOGE("Split", "%s: the input is a channel slice and the axis is not the last", name.c_str());
+            return;
+        }
+        // bytes between consecutive runs of the input (a channel slice of a wider tensor has a larger pitch)
+        const int64_t in_pitch = input->is_dense() ? slice_size * in_axis * esize : (int64_t)input->channel_pitch * esize;
         int64_t slice_index = 0;
         for (size_t i = 0; i < m_outputs_index.size(); i++) {
             TensorBase *output = context->get_tensor(m_outputs_index[i]);
@@ -155,14 +191,22 @@ public:
             }
             const int64_t out_axis = output->shape[m_axis];
             const int64_t row = slice_size * out_axis * esize;
-            const int rc = espdl_hip_copy_rows(static_cast<const char *>(input->data) + slice_index * slice_size * esize,
-                                               slice_size * in_axis * esize, output->data, row, row, num_slices,
-                                               context->stream);
+            const char *src = static_cast<const char *>(input->data) + slice_index * slice_size * esize;
+            slice_index += out_axis;
+            // an output the model left inside the input is already there
+            if (output->data == src && !output->is_dense() && (int64_t)output->channel_pitch * esize == in_pitch)
+                continue;
+            if (!output->is_dense()) {
+                DL_LOGE("Split", "%s: output %d is a channel slice of another tensor than the input", name.c_str(), (int)i);
+                return;
+            }
+            const int rc = espdl_hip_copy_rows(src, in_pitch, output->data, row, row, num_slices, context->stream);
             if (rc != ESPDL_HIP_OK)
                 DL_LOGE("Split", "%s: %s", name.c_str(), espdl_hip_last_error());
-            slice_index += out_axis;
         }
     }
+    int get_axis() const { return m_axis; }
+    bool reads_channel_slice(int slot) const { return slot == 0; }
     static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
     {
         int axis = 0, num_outputs = -1;

@@ -82,6 +82,12 @@ public:
     bool auto_free; ///< free `data` on destruction
     void *data;     ///< host or device pointer, see `caps`
     uint32_t caps;  ///< MALLOC_CAP_HOST / MALLOC_CAP_DEVICE
+    /// Elements from one position of the last axis run to the next one in memory; 0 = shape.back() (dense).
+    /// A model gives a device activation a larger pitch when it lives inside a wider tensor (an output of a
+    /// channel Split that stays in its input, an input of a channel Concat that is written in place).  Only
+    /// the copies to and from dense tensors below and the modules that say so (Module::reads_channel_slice /
+    /// writes_channel_slice) understand such a tensor.
+    int channel_pitch = 0;
 
     /// deep = true: allocate (host or device by `caps`) and copy `element` (a HOST pointer, may be
     /// null -> zero filled).  deep = false: wrap `element`, which must already live where `caps` says.
@@ -94,6 +100,9 @@ public:
     TensorBase &operator=(const TensorBase &) = delete;
 
     bool on_device() const { return (caps & MALLOC_CAP_DEVICE) != 0; }
+    bool is_dense() const { return channel_pitch == 0 || shape.empty() || channel_pitch == shape.back(); }
+    /// elements between consecutive runs of the last axis
+    int get_channel_pitch() const { return is_dense() ? (shape.empty() ? 1 : shape.back()) : channel_pitch; }
     int64_t get_size() const { return size; }
     size_t get_dtype_bytes() const { return dtype_sizeof(dtype); }
     size_t get_bytes() const { return (size_t)size * get_dtype_bytes(); }

@@ -645,6 +645,8 @@ esp_err_t Model::build(int batch)
         int first = -1, last = -1; // producing module, last reading module
         bool known = false;
         int alias_of = -1; // view of another variable's bytes
+        int slice_of = -1; // channel slice of this (wider) variable, starting at channel slice_at of it
+        int slice_at = 0;
     };
     std::vector<VarInfo> vars(n_var);
     const int plan_size = (int)m_execution_plan.size();
@@ -723,11 +725,140 @@ esp_err_t Model::build(int batch)
         if (idx >= 0)
             vars[idx].last = plan_size;
     }
+    // 1b. channel slices.  The outputs of a Split along the last axis stay inside its input when every module
+    // that reads them takes a channel pitch; an input of a Concat along the last axis is written in its place
+    // inside the Concat's output when its producer can write with a pitch and every reader can read with one.
+    // The three outputs of [Split -> ... -> Concat of all pieces and more] (the C2f / C3k2 pattern) compose:
+    // the Split's input itself then lives inside the Concat's output.  int8 only (pitches count elements).
+    if (m_fuse & FUSE_CHANNEL_SLICES) {
+        std::set<int> fixed; // tensors a caller may look at: stay dense
+        for (const std::string &name : m_fbs_model->get_graph_inputs())
+            fixed.insert(ctx->get_variable_index(name));
+        for (const std::string &name : m_fbs_model->get_graph_outputs())
+            fixed.insert(ctx->get_variable_index(name));
+        for (const std::string &name : m_fbs_model->get_test_outputs_name())
+            fixed.insert(ctx->get_variable_index(name));
+        std::vector<std::vector<std::pair<int, int>>> readers(n_var); // (module, input slot)
+        std::vector<bool> aliased(n_var, false);
+        for (int i = 0; i < plan_size; i++) {
+            dl::module::Module *m = m_execution_plan[i];
+            for (size_t sidx = 0; sidx < m->m_inputs_index.size(); sidx++)
+                if (m->m_inputs_index[sidx] > 0 && m->m_inputs_index[sidx] < CONTEXT_PARAMETER_OFFSET)
+                    readers[m->m_inputs_index[sidx]].push_back({i, (int)sidx});
+        }
+        for (int v = 1; v < n_var; v++)
+            if (vars[v].alias_of >= 0)
+                aliased[vars[v].alias_of] = aliased[v] = true;
+        auto sliceable = [&](int v) {
+            return v > 0 && v < CONTEXT_PARAMETER_OFFSET && vars[v].known && vars[v].dtype == DATA_TYPE_INT8 &&
+                vars[v].shape.size() >= 2 && !aliased[v];
+        };
+        // every reader but module `except` takes the tensor with a pitch
+        auto readers_take_pitch = [&](int v, int except) {
+            for (auto &r : readers[v])
+                if (r.first != except && !m_execution_plan[r.first]->reads_channel_slice(r.second))
+                    return false;
+            return true;
+        };
+        auto last_axis = [&](int axis, const VarInfo &v) {
+            return axis == (int)v.shape.size() - 1 || axis == -1;
+        };
+        for (int i = 0; i < plan_size; i++) {
+            auto *split = dynamic_cast<dl::module::Split *>(m_execution_plan[i]);
+            if (!split || split->m_inputs_index.empty())
+                continue;
+            const int x = split->m_inputs_index[0];
+            if (!sliceable(x) || !last_axis(split->get_axis(), vars[x]))
+                continue;
+            int at = 0;
+            for (size_t j = 0; j < split->m_outputs_index.size(); j++) {
+                const int o = split->m_outputs_index[j];
+                if (sliceable(o) && !fixed.count(o) && readers_take_pitch(o, -1)) {
+                    vars[o].slice_of = x;
+                    vars[o].slice_at = at;
+                }
+                at += vars[o].shape.back();
+            }
+        }
+        for (int i = 0; i < plan_size; i++) {
+            auto *cat = dynamic_cast<dl::module::Concat *>(m_execution_plan[i]);
+            if (!cat || cat->m_outputs_index.empty())
+                continue;
+            const int c = cat->m_outputs_index[0];
+            if (!sliceable(c) || !last_axis(cat->get_axis(), vars[c]))
+                continue;
+            // a tensor with storage of its own that may move into the Concat's output
+            auto movable = [&](int v) {
+                if (!sliceable(v) || fixed.count(v) || vars[v].slice_of >= 0 || vars[v].first < 0)
+                    return false;
+                dl::module::Module *producer = m_execution_plan[vars[v].first];
+                int slot = -1;
+                for (size_t k = 0; k < producer->m_outputs_index.size(); k++)
+                    if (producer->m_outputs_index[k] == v)
+                        slot = (int)k;
+                if (slot < 0 || !producer->writes_channel_slice(slot) || !readers_take_pitch(v, i))
+                    return false;
+                // an in-place producer may already have been promised its input's bytes
+                return producer->inplace == MODULE_NON_INPLACE;
+            };
+            const std::vector<int> &in = cat->m_inputs_index;
+            int at = 0;
+            for (size_t j = 0; j < in.size();) {
+                const int v = in[j];
+                if (v <= 0 || v >= CONTEXT_PARAMETER_OFFSET)
+                    break; // a constant input: it and what follows are copied
+                const int count_in_cat = (int)std::count(in.begin(), in.end(), v);
+                if (count_in_cat == 1 && movable(v)) {
+                    vars[v].slice_of = c;
+                    vars[v].slice_at = at;
+                    at += vars[v].shape.back();
+                    j++;
+                    continue;
+                }
+                // consecutive inputs that are, in order, all the slices of one tensor x: x moves
+                const int x = vars[v].slice_of;
+                if (x >= 0 && x != c && vars[v].slice_at == 0 && count_in_cat == 1) {
+                    size_t k = j;
+                    int covered = 0;
+                    while (k < in.size() && in[k] > 0 && in[k] < CONTEXT_PARAMETER_OFFSET && vars[in[k]].slice_of == x &&
+                           vars[in[k]].slice_at == covered && std::count(in.begin(), in.end(), in[k]) == 1) {
+                        covered += vars[in[k]].shape.back();
+                        k++;
+                    }
+                    if (covered == vars[x].shape.back() && movable(x)) {
+                        vars[x].slice_of = c;
+                        vars[x].slice_at = at;
+                        at += covered;
+                        j = k;
+                        continue;
+                    }
+                }
+                at += vars[v].shape.back();
+                j++;
+            }
+        }
+        // resolve chains (a Split output inside a tensor that moved into a Concat output)
+        for (int v = 1; v < n_var; v++) {
+            int hops = 0;
+            while (vars[v].slice_of >= 0 && vars[vars[v].slice_of].slice_of >= 0 && hops++ < 8) {
+                const int mid = vars[v].slice_of;
+                vars[v].slice_at += vars[mid].slice_at;
+                vars[v].slice_of = vars[mid].slice_of;
+            }
+        }
+        // the wider tensor lives from its first writer to its last reader
+        for (int v = 1; v < n_var; v++)
+            if (vars[v].slice_of >= 0) {
+                VarInfo &w = vars[vars[v].slice_of];
+                w.last = std::max(w.last, vars[v].last);
+                if (vars[v].first >= 0 && w.first >= 0 && vars[v].first < w.first)
+                    w.first = vars[v].first; // a Concat output that a producer writes into before the Concat runs
+            }
+    }
     // a view keeps its source alive
     for (int i = n_var - 1; i >= 1; i--)
         if (vars[i].alias_of >= 0)
             vars[vars[i].alias_of].last = std::max(vars[vars[i].alias_of].last, vars[i].last);
-
     // 2. placement
     auto bytes_of = [&](const VarInfo &v) {
         size_t n = dtype_sizeof(v.dtype);
@@ -763,6 +894,17 @@ esp_err_t Model::build(int batch)
                 offset[idx] = offset[v.alias_of];
                 continue;
             }
+            if (placed[idx])
+                continue; // the output of a Concat that an earlier producer already writes into
+            if (v.slice_of >= 0) {
+                // lives inside the wider tensor, which is placed when its first slice is written
+                const int w = v.slice_of;
+                if (!placed[w]) {
+                    offset[w] = arena.alloc(bytes_of(vars[w]));
+                    placed[w] = true;
+                }
+                continue;
+            }
             // an in-place module may overwrite its first input when nobody reads that input later
             const int in0 = m->m_inputs_index.empty() ? -1 : m->m_inputs_index[0];
             if (m->inplace == MODULE_INPLACE_CHANGED_BUFFER && j == 0 && in0 > 0 && in0 < CONTEXT_PARAMETER_OFFSET &&
@@ -770,7 +912,7 @@ esp_err_t Model::build(int batch)
                 bytes_of(vars[in0]) == bytes_of(v)) {
                 bool aliased_elsewhere = false;
                 for (int k = 1; k < n_var; k++)
-                    if (vars[k].alias_of == in0)
+                    if (vars[k].alias_of == in0 || vars[k].slice_of == in0)
                         aliased_elsewhere = true;
                 if (!aliased_elsewhere) {
                     offset[idx] = offset[in0];
@@ -793,6 +935,13 @@ esp_err_t Model::build(int batch)
     for (int i = 1; i < n_var; i++) {
         if (!vars[i].known)
             continue;
+        if (vars[i].slice_of >= 0) {
+            const VarInfo &w = vars[vars[i].slice_of];
+            ctx->m_variables[i] = new TensorBase(vars[i].shape, root + offset[vars[i].slice_of] + vars[i].slice_at, vars[i].exponent,
+                                                 vars[i].dtype, false, MALLOC_CAP_DEVICE);
+            ctx->m_variables[i]->channel_pitch = w.shape.back();
+            continue;
+        }
         ctx->m_variables[i] =
             new TensorBase(vars[i].shape, root + offset[i], vars[i].exponent, vars[i].dtype, false, MALLOC_CAP_DEVICE);
     }

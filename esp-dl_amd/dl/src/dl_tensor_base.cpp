@@ -192,10 +192,33 @@ TensorBase &TensorBase::set_shape(const std::vector<int> &new_shape)
     return *this;
 }
 
+namespace {
+// rows of a tensor (positions of all axes but the last) and the bytes of one row / between rows
+struct RowView {
+    size_t rows, row_bytes, pitch_bytes;
+};
+RowView row_view(const TensorBase *t)
+{
+    const size_t e = t->get_dtype_bytes();
+    const size_t c = t->shape.empty() ? 1 : (size_t)t->shape.back();
+    return {c ? (size_t)t->size / c : 0, c * e, (size_t)t->get_channel_pitch() * e};
+}
+} // namespace
+
 bool TensorBase::copy_from_host(const void *host, size_t bytes, void *stream)
 {
     if (!data || !host || bytes > get_bytes())
         return false;
+    if (!is_dense()) {
+        // a channel slice of a wider device tensor: whole tensors only, row by row
+        const RowView v = row_view(this);
+        if (!on_device() || bytes != get_bytes())
+            return false;
+        hipStream_t s2 = static_cast<hipStream_t>(stream);
+        return hip_ok(hipMemcpy2DAsync(data, v.pitch_bytes, host, v.row_bytes, v.row_bytes, v.rows, hipMemcpyHostToDevice, s2),
+                      "hipMemcpy2DAsync H2D") &&
+            hip_ok(hipStreamSynchronize(s2), "hipStreamSynchronize");
+    }
     if (!on_device()) {
         memcpy(data, host, bytes);
         return true;
@@ -209,6 +232,15 @@ bool TensorBase::copy_to_host(void *host, size_t bytes, void *stream) const
 {
     if (!data || !host || bytes > get_bytes())
         return false;
+    if (!is_dense()) {
+        const RowView v = row_view(this);
+        if (!on_device() || bytes != get_bytes())
+            return false;
+        hipStream_t s2 = static_cast<hipStream_t>(stream);
+        return hip_ok(hipMemcpy2DAsync(host, v.row_bytes, data, v.pitch_bytes, v.row_bytes, v.rows, hipMemcpyDeviceToHost, s2),
+                      "hipMemcpy2DAsync D2H") &&
+            hip_ok(hipStreamSynchronize(s2), "hipStreamSynchronize");
+    }
     if (!on_device()) {
         memcpy(host, data, bytes);
         return true;
@@ -226,6 +258,13 @@ bool TensorBase::copy_from(const TensorBase *tensor, void *stream)
         return copy_from_host(tensor->data, get_bytes(), stream);
     if (!on_device())
         return tensor->copy_to_host(data, get_bytes(), stream);
+    if (!is_dense() || !tensor->is_dense()) {
+        const RowView d = row_view(this), v = row_view(tensor);
+        if (d.row_bytes != v.row_bytes)
+            return false;
+        return espdl_hip_copy_rows(tensor->data, (int64_t)v.pitch_bytes, data, (int64_t)d.pitch_bytes, (int64_t)v.row_bytes,
+                                   (int64_t)v.rows, stream) == ESPDL_HIP_OK;
+    }
     return hip_ok(hipMemcpyAsync(data, tensor->data, get_bytes(), hipMemcpyDeviceToDevice,
                                  static_cast<hipStream_t>(stream)),
                   "hipMemcpyAsync D2D");
@@ -255,6 +294,12 @@ void TensorBase::memset(int value, void *stream)
         return;
     if (on_device()) {
         hipStream_t s = static_cast<hipStream_t>(stream);
+        if (!is_dense()) {
+            const RowView v = row_view(this);
+            (void)hip_ok(hipMemset2DAsync(data, v.pitch_bytes, value, v.row_bytes, v.rows, s), "hipMemset2DAsync");
+            (void)hipStreamSynchronize(s);
+            return;
+        }
         (void)hip_ok(hipMemsetAsync(data, value, get_bytes(), s), "hipMemsetAsync");
         (void)hipStreamSynchronize(s);
     } else {
@@ -269,6 +314,16 @@ bool TensorBase::assign(TensorBase *tensor, void *stream)
     const bool per_channel = exponent.is_per_channel() || tensor->exponent.is_per_channel();
     if (exponent == tensor->exponent && dtype == tensor->dtype)
         return copy_from(tensor, stream);
+    if (!is_dense()) {
+        DL_LOGE("TensorBase::assign", "a channel slice of a wider tensor can only be copied to, not requantized to");
+        return false;
+    }
+    if (!tensor->is_dense()) {
+        // requantize from a dense copy of the slice
+        TensorBase dense(tensor->shape, nullptr, 0, tensor->dtype, true, tensor->caps);
+        dense.exponent = tensor->exponent;
+        return dense.copy_from(tensor, stream) && assign(&dense, stream);
+    }
     if (per_channel) {
         DL_LOGE("TensorBase::assign", "per-channel tensors can only be copied, not requantized");
         return false;

@@ -384,6 +384,12 @@ int espdl_model_tensor_exponent(espdl_model *m, const char *name, int32_t *expon
     return 0;
 }
 
+int espdl_model_tensor_channel_pitch(espdl_model *m, const char *name)
+{
+    dl::TensorBase *t = (m && name) ? m->model->get_intermediate(name) : nullptr;
+    return t ? t->get_channel_pitch() : -1;
+}
+
 int espdl_model_set_input(espdl_model *m, const char *name, const void *host_data, int64_t bytes)
 {
     dl::TensorBase *t = (m && name) ? m->model->get_input(name) : nullptr;

@@ -50,6 +50,7 @@ def lib():
                                           ctypes.POINTER(ctypes.c_float), ctypes.POINTER(i64), ctypes.POINTER(i64)]
         L.espdl_model_print_profile.argtypes = [vp]
         L.espdl_model_print_profile.restype = None
+        L.espdl_model_tensor_channel_pitch.argtypes = [vp, cp]
         L.espdl_model_tensor_device_ptr.restype = vp
         L.espdl_model_tensor_device_ptr.argtypes = [vp, cp]
         L.espdl_model_tensor_bytes.restype = i64
@@ -195,11 +196,11 @@ class Model:
     """dl::Model handle.  `stream` is a raw hipStream_t value (e.g. torch.cuda.Stream().cuda_stream) or None."""
 
     def __init__(self, graph, batch, round_mode=0, stream=None, fuse_lut=True, fuse_blocks=True, fuse_add=True,
-                 fuse_gap=True):
+                 fuse_gap=True, channel_slices=True):
         self.graph = graph  # keep alive: the native model references it
         self.h = lib().espdl_model_create(graph.h, batch, round_mode, ctypes.c_void_p(stream) if stream else None,
                                           (1 if fuse_lut else 0) | (2 if fuse_blocks else 0) | (4 if fuse_add else 0) |
-                                          (8 if fuse_gap else 0))
+                                          (8 if fuse_gap else 0) | (16 if channel_slices else 0))
         if not self.h:
             raise EspdlModelError("espdl_model_create failed (see stderr)")
         self.batch = batch
@@ -233,6 +234,10 @@ class Model:
 
     def test(self):
         return lib().espdl_model_test(self.h) == 0
+
+    def channel_pitch(self, name):
+        """Elements between consecutive positions of the last axis in device memory (the last dim when dense)."""
+        return lib().espdl_model_tensor_channel_pitch(self.h, name.encode())
 
     def module_count(self):
         return lib().espdl_model_module_count(self.h)

@@ -696,6 +696,42 @@ def gated_block(seed=0xE5D6):
     return g
 
 
+def channel_slices(seed=0xE5E7):
+    """Splits and Concats along channels in every combination a model has to tell apart when it leaves Split
+    outputs inside the Split's input and lets Convs write into Concat outputs: pieces of 16 / 20 / 12
+    channels (rows that are not multiples of 16 bytes), a piece read by a module that takes no channel
+    pitch (Relu), a residual Add on a piece, a Concat of all pieces of a Split plus more (the C2f pattern),
+    one tensor twice in a Concat, one tensor in two Concats, a Concat input that is a graph output, a Concat
+    with the graph input, a strided 3x3 Conv on a piece and a depthwise Conv (no pitches) on another."""
+    g = GraphSpec("channel_slices")
+    b = Builder(g, seed, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 14, 18, 24], -5)
+    e = -4
+    h = b.conv(x, 48, k=1, out_exp=e, name="s1_cv1")
+    a, c, d = b.split(h, [16, 20, 12], name="s1_split")
+    m = b.conv(c, 20, k=3, out_exp=e, relu=True, name="s1_m1")
+    m = b.conv(m, 20, k=3, out_exp=e, name="s1_m2")
+    m = b.add(c, m, name="s1_add")
+    r = b.relu(d, name="s1_relu")                       # d must stay dense
+    cat1 = b.concat([a, c, m, r], name="s1_cat")        # 16 + 20 + 20 + 12 = 68
+    h2 = b.conv(cat1, 32, k=1, out_exp=e, name="s2_cv1")
+    p, q = b.split(h2, [16, 16], name="s2_split")
+    m2 = b.conv(q, 16, k=3, out_exp=e, name="s2_m")
+    cat2 = b.concat([p, q, m2], name="s2_cat")          # h2 itself moves into this one
+    y = b.conv(cat2, 8, k=1, out_exp=e, name="s3_y")
+    cat3 = b.concat([y, y], name="s3_twice")
+    z = b.conv(cat3, 24, k=3, out_exp=-5, name="s3_z")
+    cat4 = b.concat([z, x], name="s4_with_input")       # z in place, the graph input copied
+    out1 = b.conv(cat4, 16, k=1, out_exp=e, name="s4_out")
+    b.output(out1)
+    cat5 = b.concat([out1, y], name="s5_cat")           # out1 is a graph output: copied; y read with a pitch
+    t, u = b.split(cat5, [8, 16], name="s5_split")
+    t2 = b.conv(t, 8, k=3, stride=2, out_exp=e, name="s5_strided")
+    u2 = b.conv(u, 16, k=3, stride=2, depthwise=True, out_exp=e, name="s5_dw")
+    b.output(b.concat([t2, u2], name="s5_out"))
+    return g
+
+
 def activation_modules(seed=0xE5E0):
     """The activation operators as graph nodes of their own rather than fused into a Conv: Conv (Linear) ->
     PRelu with a per-channel int8 slope -> Conv (Linear) -> standalone Relu -> Conv -> PRelu whose result

@@ -79,8 +79,9 @@ int espdl_graph_add_test_output(espdl_graph *g, const char *name, const int32_t 
 /* round_mode: 0 half-up (portable C path), 1 half-even.  stream: hipStream_t or NULL (own stream).
  * fuse: bit mask of graph fusions, all exact: 1 folds Conv -> LUT pairs into the conv epilogue, 2 runs
  * depthwise Conv -> 1x1 Conv [-> Add] chains as one kernel, 4 folds the Add behind a dense Conv into the
- * conv epilogue, 8 runs a 1x1 Conv and the GlobalAveragePool behind it as one kernel (15 = all).  The graph
- * must outlive the model. */
+ * conv epilogue, 8 runs a 1x1 Conv and the GlobalAveragePool behind it as one kernel, 16 keeps the outputs of a
+ * Split along the last axis inside its input and lets dense 8-bit Convs write straight into the output of a
+ * Concat along the last axis, so that neither copies (31 = all).  The graph must outlive the model. */
 espdl_model *espdl_model_create(espdl_graph *g, int32_t batch, int32_t round_mode, void *stream, int32_t fuse);
 void espdl_model_destroy(espdl_model *m);
 /* Module::forward returns void, as in the reference, so a module whose launch is rejected (an operand
@@ -105,6 +106,10 @@ void *espdl_model_tensor_device_ptr(espdl_model *m, const char *name);
 int64_t espdl_model_tensor_bytes(espdl_model *m, const char *name);
 int espdl_model_tensor_shape(espdl_model *m, const char *name, int32_t *dims, int32_t capacity); /* returns rank */
 int espdl_model_tensor_exponent(espdl_model *m, const char *name, int32_t *exponent);
+/* Elements from one position of the last axis to the next at the device pointer: the last dim for a dense
+ * tensor, more for an activation the model keeps inside a wider one (fuse bit 16); -1 for an unknown name.
+ * espdl_model_get_tensor always delivers dense data. */
+int espdl_model_tensor_channel_pitch(espdl_model *m, const char *name);
 int espdl_model_set_input(espdl_model *m, const char *name, const void *host_data, int64_t bytes);
 int espdl_model_get_tensor(espdl_model *m, const char *name, void *host_data, int64_t bytes);
 int64_t espdl_model_device_bytes(espdl_model *m);

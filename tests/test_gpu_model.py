@@ -36,7 +36,7 @@ def _check_all(spec, mdl, want, skip_missing=True):
 
 
 def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fuse_blocks=True, fuse_add=True,
-                fuse_gap=True):
+                fuse_gap=True, channel_slices=True):
     m, zoo, model, runner = _mods()
     import espdl_oracle as oracle
     rng = np.random.default_rng(seed)
@@ -44,7 +44,7 @@ def _run_config(spec, batch, seed, round_mode=0, fuse_lut=True, graph=False, fus
     want = runner.run(spec, {spec.inputs[0]: x}, oracle.ROUND_HALF_EVEN if round_mode else oracle.ROUND_HALF_UP)
     g = model.Graph.from_spec(spec)
     mdl = model.Model(g, batch, round_mode=round_mode, fuse_lut=fuse_lut, fuse_blocks=fuse_blocks, fuse_add=fuse_add,
-                      fuse_gap=fuse_gap)
+                      fuse_gap=fuse_gap, channel_slices=channel_slices)
     mdl.set_input(spec.inputs[0], x)
     if graph:
         assert mdl.enable_graph()
@@ -200,6 +200,102 @@ def test_config4_yolo_style(oracle, fuse):
         assert mdl.module_count() < len(spec.nodes)  # Conv -> LUT pairs were folded
     else:
         assert mdl.module_count() == len(spec.nodes)
+    mdl.close()
+
+
+def test_channel_slices_every_case(oracle):
+    """Split outputs left inside the Split's input and Concat inputs written in place, case by case: which
+    tensors become slices (by their pitch), every tensor against the oracle, twice (the slices must survive a
+    second pass over the same arena), then under a captured graph."""
+    announce("model channel_slices")
+    _, zoo, _, runner = _mods()
+    spec = zoo.channel_slices()
+    batch = 3
+    mdl, want, x = _run_config(spec, batch, 41)
+    pitch = {n: mdl.channel_pitch(n) for n in want if n not in spec.inputs}
+    dense = lambda n: pitch[n] == want[n].shape[-1]  # noqa: E731
+    # block 1: the pieces stay in s1_cv1's output (48 wide) except the one Relu reads; the bottleneck's result
+    # (conv + folded Add) is written into the Concat (68 wide); s1_cv1's output itself cannot move
+    assert pitch["s1_split_out0"] == 48 and pitch["s1_split_out1"] == 48 and dense("s1_split_out2")
+    assert pitch["s1_add_out"] == 68 and dense("s1_relu_out") and dense("s1_cv1_out")
+    # block 2: all pieces of the Split go into the Concat -> the Split's input lives inside the Concat (48 wide)
+    assert pitch["s2_cv1_out"] == 48 and pitch["s2_split_out0"] == 48 and pitch["s2_split_out1"] == 48
+    assert pitch["s2_m_out"] == 48
+    # a tensor that appears twice in one Concat is copied there; it is in place in the later Concat (24 wide)
+    assert pitch["s3_y_out"] == 24 and pitch["s3_z_out"] == 48 and dense("s4_out_out")
+    assert pitch["s5_split_out0"] == 24 and dense("s5_split_out1")  # the depthwise Conv takes no pitch
+    assert pitch["s5_strided_out"] == 24 and dense("s5_dw_out")
+    # (intermediate tensors share arena space: only the graph outputs, which every slice feeds, outlive a pass)
+    for rep in range(2):
+        for name in spec.outputs:
+            np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=f"{name} pass {rep}")
+            assert want[name].min() < want[name].max()
+        mdl.run()
+    assert mdl.enable_graph()
+    x2 = spec.make_input(np.random.default_rng(42), batch)
+    mdl.set_input(spec.inputs[0], x2)
+    mdl.run()
+    want2 = runner.run(spec, {spec.inputs[0]: x2}, keep_all=False)
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want2[name], err_msg=name)
+    mdl.close()
+    # and with the slices switched off: everything dense, same results
+    mdl, want, _ = _run_config(spec, batch, 41, channel_slices=False)
+    for name, ref in want.items():
+        if name not in spec.inputs:
+            assert mdl.channel_pitch(name) in (ref.shape[-1], -1)  # -1: folded into a Conv, no tensor of its own
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name), want[name], err_msg=name)
+    mdl.close()
+
+
+def test_channel_slices_pinned_tensors_stay_dense(oracle):
+    """Tensors with test vectors stay dense and alive: with every Split / Concat / Conv output of the slices
+    graph pinned, each equals the oracle's and nothing is a slice."""
+    announce("model channel_slices pinned")
+    m, zoo, model, runner = _mods()
+    spec = zoo.channel_slices()
+    batch = 2
+    x = spec.make_input(np.random.default_rng(43), batch)
+    want = runner.run(spec, {spec.inputs[0]: x})
+    names = [o for n in spec.nodes for o in n["outputs"]]
+    g = model.Graph.from_spec(spec, test_outputs={n: want[n][:1] for n in names})
+    mdl = model.Model(g, batch)
+    mdl.set_input(spec.inputs[0], x)
+    mdl.run()
+    for n in names:
+        assert mdl.channel_pitch(n) == want[n].shape[-1], n
+        np.testing.assert_array_equal(mdl.get_tensor(n), want[n], err_msg=n)
+    mdl.close()
+    # pin only the Concat outputs and the Split inputs: their slices are still made, and must be right
+    keep = [o for n in spec.nodes if n["op_type"] == "Concat" for o in n["outputs"]] + ["s1_cv1_out"]
+    g = model.Graph.from_spec(spec, test_outputs={n: want[n][:1] for n in keep})
+    mdl = model.Model(g, batch)
+    mdl.set_input(spec.inputs[0], x)
+    mdl.run()
+    assert mdl.channel_pitch("s1_split_out0") == 48 and mdl.channel_pitch("s2_m_out") == 48
+    for n in keep:
+        np.testing.assert_array_equal(mdl.get_tensor(n), want[n], err_msg=n)
+    # the pieces of s1_cv1's output are views of a tensor that is still alive
+    np.testing.assert_array_equal(mdl.get_tensor("s1_split_out0"), want["s1_split_out0"])
+    np.testing.assert_array_equal(mdl.get_tensor("s1_split_out1"), want["s1_split_out1"])
+    mdl.close()
+
+
+@pytest.mark.parametrize("slices", [True, False], ids=["in_place", "copied"])
+def test_config4_channel_slices(oracle, slices):
+    """The detector graph with its C3k2 Splits / Concats in place and copied: every tensor equals the oracle's,
+    and the device arena is no larger in place."""
+    announce(f"model config4 160px channel_slices={slices}")
+    _, zoo, _, _ = _mods()
+    spec = zoo.config4_yolo_style(resolution=160)
+    mdl, want, _ = _run_config(spec, 2, 9, channel_slices=slices)
+    if slices:
+        assert mdl.channel_pitch("c2_split_out0") == 96 and mdl.channel_pitch("c2_cv1_act_out") == 96
+    else:
+        assert mdl.channel_pitch("c2_split_out0") == 32
+    for name in spec.outputs:
+        np.testing.assert_array_equal(mdl.get_tensor(name, _np_dtype(spec, name)), want[name], err_msg=name)
     mdl.close()
 
 
@@ -382,7 +478,7 @@ def test_profile_reports_every_module():
     mdl = model.Model(model.Graph.from_spec(spec), 4)
     info = mdl.profile(repeats=2)
     assert len(info) == mdl.module_count()
-    convs = [i for i in info if i["type"] == "Conv"]
+    convs = [i for i in info if "Conv" in i["type"]]  # "Conv", or "Conv>DepthwiseConv>Conv:wave" for a fused block
     assert sum(i["macs"] for i in convs) == 4 * spec.conv_macs_per_image
     assert all(i["latency_us"] > 0 for i in info)
     mdl.close()
