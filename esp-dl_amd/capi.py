@@ -96,6 +96,7 @@ def lib():
         L.espdl_hip_transpose.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
         L.espdl_hip_resize_nearest_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, vp, vp]
         L.espdl_hip_max_pool.argtypes = [vp, i32] + [i32] * 12 + [vp, vp]
+        L.espdl_hip_max_pool_pitched.argtypes = [vp, i32] + [i32] * 14 + [vp, vp]
         L.espdl_hip_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp, vp]
         L.espdl_hip_slice.argtypes = [vp, vp, i32, vp, vp, vp, i32, vp, vp]
         L.espdl_hip_reduce_mean_s8.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
@@ -418,13 +419,20 @@ def resize_nearest_s8(x, scale_h, scale_w, in_exp=0, out_exp=0, out_hw=None, out
 
 
 def max_pool(x, kernel, strides=(1, 1), pads=(0, 0, 0, 0), out=None, stream=None):
-    """pads = (top, bottom, left, right); x int8 or int16 NHWC."""
+    """pads = (top, bottom, left, right); x int8 or int16 NHWC.  x and out may be channel slices of wider
+    NHWC tensors (wide[..., a:b])."""
     import torch
     n, h, w, c = x.shape
     pt, pb, pl, pr = pads
     oh = (h + pt + pb - kernel[0]) // strides[0] + 1
     ow = (w + pl + pr - kernel[1]) // strides[1] + 1
     out = torch.empty((n, max(oh, 0), max(ow, 0), c), dtype=x.dtype, device=x.device) if out is None else out
+    ip, op = _channel_pitch(x), _channel_pitch(out)
+    if ip or op:
+        _check(lib().espdl_hip_max_pool_pitched(_p(x), S16 if x.dtype == torch.int16 else S8, n, h, w, c, kernel[0],
+                                                kernel[1], strides[0], strides[1], pt, pb, pl, pr, ip, op, _p(out),
+                                                _stream(stream)))
+        return out
     _check(lib().espdl_hip_max_pool(_p(x), S16 if x.dtype == torch.int16 else S8, n, h, w, c, kernel[0], kernel[1],
                                     strides[0], strides[1], pt, pb, pl, pr, _p(out), _stream(stream)))
     return out

@@ -101,6 +101,13 @@ typedef short v2s __attribute__((ext_vector_type(2)));
 // first shifted left by max(0, 8-s).  MODES 4, 5 and 6 are described at pack_fast4.
 // Saturating packed multiply of two int16 by two int16 (v_pk_mad_i16 with the clamp bit: the products are
 // formed exactly and saturated to int16).
+// Maximum of two int16 pairs held in dwords (v_pk_max_i16).  The operands arrive by value on purpose: a
+// __builtin_bit_cast applied directly to an element of an ext_vector (x[d]) reads element 0 whatever d is.
+__device__ __forceinline__ int pk_max_i16(int a, int b)
+{
+    return __builtin_bit_cast(int, __builtin_elementwise_max(__builtin_bit_cast(v2s, a), __builtin_bit_cast(v2s, b)));
+}
+
 __device__ __forceinline__ v2s pk_mul_sat_i16(v2s a, int m)
 {
     int d;

@@ -525,9 +525,10 @@ int espdl_hip_resize_nearest_s8(const int8_t *in, int32_t batch, int32_t h, int3
                          "resize_nearest_s8");
 }
 
-int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h,
-                       int32_t k_w, int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom,
-                       int32_t pad_left, int32_t pad_right, void *out, void *stream)
+int espdl_hip_max_pool_pitched(const void *in, int32_t dtype, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h,
+                               int32_t k_w, int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom,
+                               int32_t pad_left, int32_t pad_right, int32_t in_pitch, int32_t out_pitch, void *out,
+                               void *stream)
 {
     if (dtype != ESPDL_HIP_S8 && dtype != ESPDL_HIP_S16)
         return fail(ESPDL_HIP_EINVAL, "dtype must be ESPDL_HIP_S8 or ESPDL_HIP_S16");
@@ -536,6 +537,9 @@ int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, 
         return fail(ESPDL_HIP_EINVAL, "bad max_pool geometry");
     if (h + pad_top + pad_bottom < k_h || w + pad_left + pad_right < k_w)
         return fail(ESPDL_HIP_EINVAL, "window larger than the padded image");
+    if (in_pitch < 0 || out_pitch < 0 || (in_pitch != 0 && in_pitch < c) || (out_pitch != 0 && out_pitch < c))
+        return fail(ESPDL_HIP_EINVAL, "channel pitches %d / %d must be 0 or at least the channel count %d", in_pitch, out_pitch,
+                    c);
     const int out_h = (h + pad_top + pad_bottom - k_h) / stride_h + 1, out_w = (w + pad_left + pad_right - k_w) / stride_w + 1;
     if (batch == 0)
         return ESPDL_HIP_OK;
@@ -545,9 +549,17 @@ int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, 
     if (misaligned(in, (size_t)esize) || misaligned(out, (size_t)esize))
         return fail(ESPDL_HIP_EINVAL, "int16 tensors must be 2-byte aligned");
     return device_status(espdl::launch_max_pool(in, esize, batch, h, w, c, k_h, k_w, stride_h, stride_w, pad_top, pad_left,
-                                                out_h, out_w, out, cu_count_cached(),
-                                                reinterpret_cast<hipStream_t>(stream)),
+                                                out_h, out_w, in_pitch != 0 ? in_pitch : c, out_pitch != 0 ? out_pitch : c,
+                                                out, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
                          "max_pool");
+}
+
+int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h,
+                       int32_t k_w, int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom,
+                       int32_t pad_left, int32_t pad_right, void *out, void *stream)
+{
+    return espdl_hip_max_pool_pitched(in, dtype, batch, h, w, c, k_h, k_w, stride_h, stride_w, pad_top, pad_bottom, pad_left,
+                                      pad_right, 0, 0, out, stream);
 }
 
 int espdl_hip_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h, int32_t k_w,

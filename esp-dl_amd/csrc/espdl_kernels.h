@@ -188,9 +188,17 @@ hipError_t launch_transpose(const void *in, const int *shape, int dims, const in
 hipError_t launch_resize_nearest_s8(const int8_t *in, int batch, int h, int w, int c, int out_h, int out_w, float scale_h,
                                     float scale_w, int in_exp, int out_exp, int8_t *out, int cu_count,
                                     hipStream_t stream);
+// in_pitch / out_pitch: elements from pixel to pixel (c for dense tensors, more for channel slices)
 hipError_t launch_max_pool(const void *in, int elem_size, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
-                           int stride_w, int pad_top, int pad_left, int out_h, int out_w, void *out, int cu_count,
-                           hipStream_t stream);
+                           int stride_w, int pad_top, int pad_left, int out_h, int out_w, long long in_pitch,
+                           long long out_pitch, void *out, int cu_count, hipStream_t stream);
+// int8, square windows of 2 / 3 / 5 at stride 1, channels and pitches in multiples of 16 (max_pool_s8.hip)
+bool max_pool_s8_window_supports(const void *in, int h, int w, int c, int k_h, int k_w, int stride_h, int stride_w,
+                                 int pad_top, int pad_left, int out_h, int out_w, long long in_pitch, long long out_pitch,
+                                 const void *out);
+hipError_t launch_max_pool_s8_window(const void *in, int batch, int h, int w, int c, int k, int pad_top, int pad_left,
+                                     int out_h, int out_w, long long in_pitch, long long out_pitch, void *out,
+                                     int cu_count, hipStream_t stream);
 
 hipError_t launch_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                               int stride_w, int pad_top, int pad_left, int out_h, int out_w, int in_exp, int out_exp,

@@ -285,6 +285,7 @@ struct PoolArgs {
     int vec; // elements per thread: 16 / 8 (vector path) or 1
     FastDiv fd_cv, fd_ow, fd_oh;
     long long total;
+    long long in_pitch, out_pitch; // elements from pixel to pixel (c when dense)
 };
 
 typedef signed char v16c __attribute__((ext_vector_type(16)));
@@ -306,13 +307,35 @@ __global__ __launch_bounds__(kBlock) void max_pool_kernel(const PoolArgs a)
         const int ky0 = max(0, -iy0), ky1 = min(a.k_h, a.h - iy0);
         const int kx0 = max(0, -ix0), kx1 = min(a.k_w, a.w - ix0);
         const long long img = (long long)n * a.h * a.w;
-        const long long dst = (long long)pix * a.c + (long long)v * a.vec;
-        if (a.vec > 1) {
+        const long long dst = (long long)pix * a.out_pitch + (long long)v * a.vec;
+        if (a.vec > 1 && sizeof(T) == 1) {
+            // No byte-wise maximum exists: int16 pairs instead.  The raw dword orders like its odd bytes (the
+            // low byte of each half only breaks ties), the dword shifted left by 8 like its even bytes.
+            const v4i lowest = {(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
+            v4i odd = lowest, even = lowest;
+            bool have = false;
+            for (int ky = ky0; ky < ky1; ky++)
+                for (int kx = kx0; kx < kx1; kx++) {
+                    const v4i cur = *reinterpret_cast<const v4i *>(in + (img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.in_pitch +
+                                                                   (long long)v * a.vec);
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+                        odd[d] = pk_max_i16(odd[d], cur[d]);
+                        even[d] = pk_max_i16(even[d], cur[d] << 8);
+                    }
+                    have = true;
+                }
+            v4i res;
+#pragma unroll
+            for (int d = 0; d < 4; d++) // an empty clipped window (pads >= kernel) stores zeros
+                res[d] = have ? (int)__builtin_amdgcn_perm((unsigned)odd[d], (unsigned)even[d], 0x07030501u) : 0;
+            *reinterpret_cast<v4i *>(out + dst) = res;
+        } else if (a.vec > 1) {
             V best = {}; // an empty clipped window (pads >= kernel) stores zeros
             bool have = false;
             for (int ky = ky0; ky < ky1; ky++)
                 for (int kx = kx0; kx < kx1; kx++) {
-                    const V cur = *reinterpret_cast<const V *>(in + (img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.c +
+                    const V cur = *reinterpret_cast<const V *>(in + (img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.in_pitch +
                                                                (long long)v * a.vec);
                     best = have ? __builtin_elementwise_max(best, cur) : cur;
                     have = true;
@@ -323,7 +346,7 @@ __global__ __launch_bounds__(kBlock) void max_pool_kernel(const PoolArgs a)
             bool have = false;
             for (int ky = ky0; ky < ky1; ky++)
                 for (int kx = kx0; kx < kx1; kx++) {
-                    const int cur = in[(img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.c + v];
+                    const int cur = in[(img + (long long)(iy0 + ky) * a.w + (ix0 + kx)) * a.in_pitch + v];
                     best = have ? max(best, cur) : cur;
                     have = true;
                 }
@@ -742,9 +765,13 @@ hipError_t launch_insert_zeros(const void *in, int elem_size, int batch, int h, 
 }
 
 hipError_t launch_max_pool(const void *in, int elem_size, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
-                           int stride_w, int pad_top, int pad_left, int out_h, int out_w, void *out, int cu_count,
-                           hipStream_t stream)
+                           int stride_w, int pad_top, int pad_left, int out_h, int out_w, long long in_pitch,
+                           long long out_pitch, void *out, int cu_count, hipStream_t stream)
 {
+    if (elem_size == 1 && max_pool_s8_window_supports(in, h, w, c, k_h, k_w, stride_h, stride_w, pad_top, pad_left, out_h,
+                                                      out_w, in_pitch, out_pitch, out))
+        return launch_max_pool_s8_window(in, batch, h, w, c, k_h, pad_top, pad_left, out_h, out_w, in_pitch, out_pitch, out,
+                                         cu_count, stream);
     PoolArgs a;
     a.in = static_cast<const char *>(in);
     a.out = static_cast<char *>(out);
@@ -759,8 +786,11 @@ hipError_t launch_max_pool(const void *in, int elem_size, int batch, int h, int 
     a.stride_w = stride_w;
     a.pad_top = pad_top;
     a.pad_left = pad_left;
+    a.in_pitch = in_pitch;
+    a.out_pitch = out_pitch;
     const int per_vec = 16 / elem_size;
-    const bool vec_ok = (c % per_vec) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    const bool vec_ok = (c % per_vec) == 0 && (in_pitch % per_vec) == 0 && (out_pitch % per_vec) == 0 &&
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
     a.vec = vec_ok ? per_vec : 1;
     const int cv = c / a.vec;
     a.total = (long long)batch * out_h * out_w * cv;

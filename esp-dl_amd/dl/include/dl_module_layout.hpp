@@ -421,12 +421,17 @@ public:
         const int sh = nwc ? 1 : m_strides[0], sw = nwc ? m_strides[0] : m_strides[1];
         const int pt = nwc ? 0 : m_padding[0], pb = nwc ? 0 : m_padding[1];
         const int pl = nwc ? m_padding[0] : m_padding[2], pr = nwc ? m_padding[1] : m_padding[3];
-        const int rc = espdl_hip_max_pool(input->data, quant_type == QUANT_TYPE_SYMM_8BIT ? ESPDL_HIP_S8 : ESPDL_HIP_S16,
-                                          input->shape[0], h, w, c, kh, kw, sh, sw, pt, pb, pl, pr, output->data,
-                                          context->stream);
+        const int rc =
+            espdl_hip_max_pool_pitched(input->data, quant_type == QUANT_TYPE_SYMM_8BIT ? ESPDL_HIP_S8 : ESPDL_HIP_S16,
+                                       input->shape[0], h, w, c, kh, kw, sh, sw, pt, pb, pl, pr,
+                                       input->is_dense() ? 0 : input->channel_pitch,
+                                       output->is_dense() ? 0 : output->channel_pitch, output->data, context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("MaxPool", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
+    /// The kernels take a channel pitch on either side (the pools of an SPPF block write into its Concat).
+    bool reads_channel_slice(int slot) const { return slot == 0; }
+    bool writes_channel_slice(int slot) const { return slot == 0; }
     static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
     {
         std::vector<int> kernel_shape, pads, strides;

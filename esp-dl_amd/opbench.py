@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Achieved HBM bandwidth of the bandwidth-bound operators, one MI355X.
 
-    python esp-dl_amd/opbench.py [--mib 256] [--reps 20]
+    python esp-dl_amd/opbench.py [--mib 256] [--reps 20] [--only maxpool]
 
 Every operator runs through the C ABI on tensors of at least `--mib` MiB, timed with HIP events around `--reps`
 back-to-back launches on the current stream; bandwidth = algorithmic bytes (every input and output byte once)
@@ -24,6 +24,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--mib", type=int, default=256)
     ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--only", default="", help="run only the operators whose line contains this text")
     args = ap.parse_args()
     import torch
     m = importlib.import_module("esp-dl_amd")
@@ -35,6 +36,8 @@ def main():
         return torch.randint(-128, 128, shape, dtype=torch.int8, device=dev)
 
     def timed(name, fn, nbytes):
+        if args.only.lower() not in name.lower():
+            return
         fn()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

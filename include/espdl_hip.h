@@ -209,6 +209,14 @@ int espdl_hip_resize_nearest_s8(const int8_t *in, int32_t batch, int32_t h, int3
 int espdl_hip_max_pool(const void *in, int32_t dtype, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h,
                        int32_t k_w, int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom,
                        int32_t pad_left, int32_t pad_right, void *out, void *stream);
+/* The same on channel slices of wider NHWC tensors: in_pitch / out_pitch are the elements from one pixel to
+ * the next at `in` / `out` (0 = dense, c), as in espdl_hip_conv_desc.  This is how the chained pools of an
+ * SPPF block (MaxPool -> MaxPool -> MaxPool -> Concat of all, dl_module_concat.hpp:86-108) write their parts
+ * of the Concat result directly. */
+int espdl_hip_max_pool_pitched(const void *in, int32_t dtype, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h,
+                               int32_t k_w, int32_t stride_h, int32_t stride_w, int32_t pad_top, int32_t pad_bottom,
+                               int32_t pad_left, int32_t pad_right, int32_t in_pitch, int32_t out_pitch, void *out,
+                               void *stream);
 
 /* base::avg_pool2d<int8_t> on the portable C path (esp-dl/dl/base/dl_base_avg_pool2d.cpp:9-54 under the
  * shell of dl_base_pool2d.hpp:439-560): sum over the window clipped to the image, times

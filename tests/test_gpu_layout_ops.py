@@ -176,6 +176,53 @@ def test_avg_pool_and_reduce_mean_s8_every_sum(oracle, hw):
         np.testing.assert_array_equal(got, oracle.reduce_mean_s8(x, [1, 2], True, exps[0], exps[1]), err_msg=str(exps))
 
 
+@pytest.mark.parametrize("shape,k,pads", [
+    # the stride-1 window kernel (channels in multiples of 8): odd and even widths, images smaller than the
+    # window, one-sided padding, more rows than one strip, windows of 2 / 3 / 5
+    ((2, 20, 20, 128), 5, (2, 2, 2, 2)), ((3, 7, 9, 16), 5, (2, 2, 2, 2)), ((1, 3, 2, 32), 5, (2, 2, 2, 2)),
+    ((2, 1, 1, 16), 5, (2, 2, 2, 2)), ((1, 45, 13, 48), 5, (2, 2, 2, 2)), ((2, 9, 10, 16), 5, (4, 0, 0, 4)),
+    ((2, 12, 11, 32), 5, (0, 0, 0, 0)), ((2, 11, 12, 16), 3, (1, 1, 1, 1)), ((2, 8, 7, 64), 3, (0, 2, 2, 0)),
+    ((3, 6, 5, 16), 2, (0, 1, 0, 1)), ((1, 80, 80, 16), 5, (2, 2, 2, 2)), ((70, 20, 20, 16), 5, (2, 2, 2, 2)),
+    ((2, 9, 9, 8), 5, (2, 2, 2, 2)), ((2, 10, 7, 24), 3, (1, 1, 1, 1)),
+])
+@pytest.mark.parametrize("fill", ["random", "extremes", "low"])
+def test_max_pool_window_kernel(oracle, shape, k, pads, fill):
+    """Packed-int16 maxima must order bytes exactly like signed bytes: random data, only -128 / 127 / -1 / 0 (the
+    values where a wrong sign or a carry between neighbouring bytes shows), and all-low data (-128 / -127, where
+    the out-of-image fill value could win by mistake)."""
+    announce(f"max_pool window {shape} k{k} p{pads} {fill}")
+    rng = np.random.default_rng(26)
+    if fill == "random":
+        x = _rand(rng, shape)
+    elif fill == "extremes":
+        x = rng.choice(np.array([-128, 127, -1, 0, 1], dtype=np.int8), size=shape)
+    else:
+        x = rng.choice(np.array([-128, -127], dtype=np.int8), size=shape, p=[0.9, 0.1])
+    got = to_host(espdl().max_pool(to_dev(x), (k, k), (1, 1), pads))
+    np.testing.assert_array_equal(got, oracle.max_pool(x, (k, k), (1, 1), pads))
+
+
+@pytest.mark.parametrize("c,wide_in,wide_out,at", [(16, 64, 48, 16), (32, 32, 128, 96), (16, 40, 16, 0), (24, 72, 48, 24)])
+def test_max_pool_channel_slices(oracle, c, wide_in, wide_out, at):
+    """Input and output as channel slices of wider tensors (pitches that are and are not multiples of 16 bytes);
+    the bytes of the wide output outside the slice stay as they were."""
+    import torch
+    announce(f"max_pool slices c={c} in={wide_in} out={wide_out} at={at}")
+    m = espdl()
+    rng = np.random.default_rng(27)
+    xin = _rand(rng, (3, 13, 10, wide_in))
+    lo = min(at, wide_in - c)
+    x = np.ascontiguousarray(xin[..., lo:lo + c])
+    want = oracle.max_pool(x, (5, 5), (1, 1), (2, 2, 2, 2))
+    wide = to_dev(xin)
+    out_wide = torch.full((3, 13, 10, wide_out), 77, dtype=torch.int8, device="cuda")
+    m.max_pool(wide[..., lo:lo + c], (5, 5), (1, 1), (2, 2, 2, 2), out=out_wide[..., at:at + c])
+    got = to_host(out_wide)
+    np.testing.assert_array_equal(got[..., at:at + c], want)
+    rest = np.delete(got, np.s_[at:at + c], axis=3)
+    assert (rest == 77).all()
+
+
 def test_sppf_pool_chain_idempotence():
     """Size-independent property at full batch: three chained 5x5/1 pools equal one 13x13/1 pool, and
     pooling is monotone (output >= input)."""
