@@ -4,17 +4,22 @@
 // feature_t = int16_t, buffer_t = int64_t) under conv_operation_shell's window clipping: an exact 64-bit sum
 // of int16 x int16 products, plus the int64 bias, shifted and rounded, saturated to int16.
 //
-// There is no int16 MFMA, so both operands are cut into 7-bit digits that the int8 MFMA multiplies exactly:
-//   weight  w = 2^14 w2 + 2^7 w1 + w0,            w0, w1 in [0, 127], w2 = w >> 14 in [-2, 1]
-//   pixel   x = 2^14 x2 + 2^7 x1 + x0 - 32768,    x0, x1 in [0, 127], x2 in [0, 3]   (digits of x + 32768)
-// so  sum_k x w = sum_{i,j} 2^(7(i+j)) sum_k x_i w_j  -  32768 sum_k w.  Digit products of equal weight share
-// an int32 accumulator (five per output, none can overflow for k < 40000); the last term is a per-filter
-// constant.  Taps outside the image are x = 0, i.e. digits (0, 0, 2), which the constant accounts for.
+// There is no int16 MFMA, so both operands are cut into two signed bytes that the int8 MFMA multiplies exactly.
+// With h = the high byte of a 16-bit value v (signed) and l = its low byte xor 0x80 (signed, the low byte minus
+// 128):  v = 256 h + l + 128.  For a pixel x = A + 128 and a weight w = B + 128 (A = 256 xh + xl, B = 256 wh + wl):
+//   sum_k x w = sum_k A B + 128 sum_k A + 128 sum_k B + 16384 K
+//             = 65536 HH + 256 (HL + LH) + LL  +  128 (256 sum_k xh + sum_k xl)  +  128 sum_k w
+// with HH = sum_k xh wh and so on: four MFMA products per step into three int32 accumulators (HL and LH share
+// one; none can overflow for K < 65536), the window sums of the pixel's own bytes (two dot-product instructions
+// per loaded dword, summed over the four k slices of a tile at the end), and a per-filter constant.  Taps outside
+// the image are x = 0, i.e. bytes (0, -128), which the same formula covers; k positions that pad the last step
+// are zero bytes on both sides and add nothing.
 //
-// Layout of the work: a workgroup owns up to 64 filters, whose three digit planes it builds once in LDS in
+// Layout of the work: a workgroup owns up to 64 filters, whose two byte planes it builds once in LDS in
 // MFMA operand-A order for the whole reduction axis; each of its wavefronts then walks 16-pixel tiles,
-// loading its lane's 16 channels of one tap (32 contiguous bytes) per k step straight from memory, cutting
-// them into digits in registers and issuing nine MFMAs per 16 filters.
+// loading its lane's 16 channels of one tap (32 contiguous bytes) per k step straight from memory, sorting
+// them into the two byte operands with two permutes and one xor per dword pair and issuing four MFMAs per
+// 16 filters.
 #include "espdl_device.h"
 #include "espdl_kernels.h"
 
@@ -40,8 +45,12 @@ struct S16MfmaArgs {
     FastDiv fd_upt, fd_kw, fd_ow, fd_ohw;
 };
 
-// four consecutive k of one digit from two dwords of two int16 each
-__device__ __forceinline__ int pack_digit(int m0, int m1)
+// the high bytes / the low bytes of the four int16 held in two dwords, as one dword of four consecutive k
+__device__ __forceinline__ int high_bytes(int m0, int m1)
+{
+    return (int)__builtin_amdgcn_perm((unsigned)m1, (unsigned)m0, 0x07050301u);
+}
+__device__ __forceinline__ int low_bytes(int m0, int m1)
 {
     return (int)__builtin_amdgcn_perm((unsigned)m1, (unsigned)m0, 0x06040200u);
 }
@@ -57,9 +66,9 @@ __global__ __launch_bounds__(kThreads) void conv2d_s16_mfma_kernel(const S16Mfma
     const int n_f = a.row_tiles * 16;
     const long long ftap = (long long)g.k_h * g.k_w * C;
 
-    // LDS: digit planes [row tile][digit][k step][lane] x 16 bytes, then per filter: constant (int64), shift
+    // LDS: byte planes [row tile][high, low][k step][lane] x 16 bytes, then per filter: constant (int64), shift
     v4i *planes = reinterpret_cast<v4i *>(smem);
-    const size_t plane_bytes = (size_t)a.row_tiles * 3 * a.ksteps * 64 * 16;
+    const size_t plane_bytes = (size_t)a.row_tiles * 2 * a.ksteps * 64 * 16;
     long long *cst = reinterpret_cast<long long *>(smem + plane_bytes);
     int *shf = reinterpret_cast<int *>(cst + n_f);
 
@@ -74,32 +83,30 @@ __global__ __launch_bounds__(kThreads) void conv2d_s16_mfma_kernel(const S16Mfma
         const int l = s & 63, ks = (s >> 6) % a.ksteps, rt = (s >> 6) / a.ksteps;
         const int f = f0 + 16 * rt + (l & 15);
         const int u = 4 * ks + (l >> 4);
-        int d0[4] = {0, 0, 0, 0}, d1[4] = {0, 0, 0, 0}, d2[4] = {0, 0, 0, 0};
+        int wh[4] = {0, 0, 0, 0}, wl[4] = {0, 0, 0, 0};
         int part = 0;
         if (f < OC && u < a.n_units) {
             const int16_t *src = a.w + (long long)f * ftap + (long long)u * 16;
 #pragma unroll
             for (int e = 0; e < 16; e++) {
                 const int v = src[e];
-                d0[e >> 2] |= (v & 127) << (8 * (e & 3));
-                d1[e >> 2] |= ((v >> 7) & 127) << (8 * (e & 3));
-                d2[e >> 2] |= ((v >> 14) & 255) << (8 * (e & 3));
+                wh[e >> 2] |= ((v >> 8) & 255) << (8 * (e & 3));
+                wl[e >> 2] |= ((v & 255) ^ 128) << (8 * (e & 3));
                 part += v;
             }
             atomicAdd(&wsum[16 * rt + (l & 15)], part);
         }
-        const int base = ((rt * 3) * a.ksteps + ks) * 64 + l;
-        planes[base] = v4i{d0[0], d0[1], d0[2], d0[3]};
-        planes[base + a.ksteps * 64] = v4i{d1[0], d1[1], d1[2], d1[3]};
-        planes[base + 2 * a.ksteps * 64] = v4i{d2[0], d2[1], d2[2], d2[3]};
+        const int base = ((rt * 2) * a.ksteps + ks) * 64 + l;
+        planes[base] = v4i{wh[0], wh[1], wh[2], wh[3]};
+        planes[base + a.ksteps * 64] = v4i{wl[0], wl[1], wl[2], wl[3]};
     }
     __syncthreads();
-    // per filter: bias - 32768 * (sum of its weights), and its shift
+    // per filter: bias + 128 * (sum of its weights), and its shift
     for (int f = tid; f < n_f; f += kThreads) {
         long long c = 0;
         int sh = 0;
         if (f0 + f < OC) {
-            c = (a.bias != nullptr ? a.bias[f0 + f] : 0) - 32768ll * (long long)wsum[f];
+            c = (a.bias != nullptr ? a.bias[f0 + f] : 0) + 128ll * (long long)wsum[f];
             sh = a.shift[g.n_shift == 1 ? 0 : f0 + f];
         }
         cst[f] = c;
@@ -121,17 +128,18 @@ __global__ __launch_bounds__(kThreads) void conv2d_s16_mfma_kernel(const S16Mfma
         const int iy0 = (int)oy * g.stride_h - g.pad_top, ix0 = (int)ox * g.stride_w - g.pad_left;
         const int16_t *img = a.in + (long long)n * g.in_h * g.in_w * C;
 
-        v4i acc[kMaxRowTiles][5];
+        v4i acc[kMaxRowTiles][3]; // HH, HL + LH, LL
 #pragma unroll
         for (int rt = 0; rt < kMaxRowTiles; rt++)
 #pragma unroll
-            for (int s = 0; s < 5; s++)
+            for (int s = 0; s < 3; s++)
                 acc[rt][s] = v4i{0, 0, 0, 0};
+        int sum_h = 0, sum_l = 0; // this lane's part of sum_k xh and sum_k xl of its pixel
 
         for (int ks = 0; ks < a.ksteps; ks++) {
-            // this lane's 16 channels of one tap, as digits of x + 32768
+            // this lane's 16 channels of one tap as high bytes and low bytes - 128
             const int u = 4 * ks + quad;
-            v4i x0 = {0, 0, 0, 0}, x1 = {0, 0, 0, 0}, x2 = {0, 0, 0, 0};
+            v4i xh = {0, 0, 0, 0}, xl = {0, 0, 0, 0};
             if (u < a.n_units) {
                 const unsigned tap = fastdiv((unsigned)u, a.fd_upt);
                 const unsigned c16 = (unsigned)u - tap * a.fd_upt.d;
@@ -144,32 +152,33 @@ __global__ __launch_bounds__(kThreads) void conv2d_s16_mfma_kernel(const S16Mfma
                     lo = src[0];
                     hi = src[1];
                 }
-                int d[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const int d[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const int e0 = d[2 * q] ^ (int)0x80008000u, e1 = d[2 * q + 1] ^ (int)0x80008000u;
-                    x0[q] = pack_digit(e0 & 0x007f007f, e1 & 0x007f007f);
-                    x1[q] = pack_digit((e0 >> 7) & 0x007f007f, (e1 >> 7) & 0x007f007f);
-                    x2[q] = pack_digit((e0 >> 14) & 0x00030003, (e1 >> 14) & 0x00030003);
+                    xh[q] = high_bytes(d[2 * q], d[2 * q + 1]);
+                    xl[q] = low_bytes(d[2 * q], d[2 * q + 1]) ^ (int)0x80808080u;
+                    sum_h = __builtin_amdgcn_sdot4(xh[q], 0x01010101, sum_h, false);
+                    sum_l = __builtin_amdgcn_sdot4(xl[q], 0x01010101, sum_l, false);
                 }
             }
 #pragma unroll
             for (int rt = 0; rt < kMaxRowTiles; rt++) {
                 if (rt < a.row_tiles) { // uniform
-                    const int base = ((rt * 3) * a.ksteps + ks) * 64 + lane;
-                    const v4i w0 = planes[base], w1 = planes[base + a.ksteps * 64], w2 = planes[base + 2 * a.ksteps * 64];
-                    acc[rt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x0, acc[rt][0], 0, 0, 0);
-                    acc[rt][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x0, acc[rt][1], 0, 0, 0);
-                    acc[rt][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x1, acc[rt][1], 0, 0, 0);
-                    acc[rt][2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w2, x0, acc[rt][2], 0, 0, 0);
-                    acc[rt][2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1, acc[rt][2], 0, 0, 0);
-                    acc[rt][2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, x2, acc[rt][2], 0, 0, 0);
-                    acc[rt][3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w2, x1, acc[rt][3], 0, 0, 0);
-                    acc[rt][3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x2, acc[rt][3], 0, 0, 0);
-                    acc[rt][4] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w2, x2, acc[rt][4], 0, 0, 0);
+                    const int base = ((rt * 2) * a.ksteps + ks) * 64 + lane;
+                    const v4i wh = planes[base], wl = planes[base + a.ksteps * 64];
+                    acc[rt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wh, xh, acc[rt][0], 0, 0, 0);
+                    acc[rt][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wl, xh, acc[rt][1], 0, 0, 0);
+                    acc[rt][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wh, xl, acc[rt][1], 0, 0, 0);
+                    acc[rt][2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wl, xl, acc[rt][2], 0, 0, 0);
                 }
             }
         }
+        // the four k slices of the tile (lanes col, col + 16, col + 32, col + 48) together hold the pixel's sums
+        sum_h += __shfl_xor(sum_h, 16);
+        sum_l += __shfl_xor(sum_l, 16);
+        sum_h += __shfl_xor(sum_h, 32);
+        sum_l += __shfl_xor(sum_l, 32);
+        const long long pixel_term = 128ll * (256ll * sum_h + sum_l);
 
         // this lane: filters f0 + 16 rt + 4 quad + r of pixel `pix`
         if (pix_ok) {
@@ -180,10 +189,8 @@ __global__ __launch_bounds__(kThreads) void conv2d_s16_mfma_kernel(const S16Mfma
                     short q[4];
 #pragma unroll
                     for (int r = 0; r < 4; r++) {
-                        long long v = cst[fl + r];
-#pragma unroll
-                        for (int s = 0; s < 5; s++)
-                            v += (long long)acc[rt][s][r] << (7 * s);
+                        long long v = cst[fl + r] + pixel_term;
+                        v += ((long long)acc[rt][0][r] << 16) + ((long long)acc[rt][1][r] << 8) + (long long)acc[rt][2][r];
                         q[r] = (short)requant_s16(v, shf[fl + r], relu, half_even);
                     }
                     int16_t *dst = a.out + pix * OC + f0 + fl;
@@ -216,13 +223,14 @@ S16Plan plan_s16(const ConvGeom &g)
     if (g.in_c % 16 != 0)
         return p;
     const long long k = (long long)g.k_h * g.k_w * g.in_c;
-    if (k > 36000) // five int32 accumulators per output stay exact below this
-        return p;
+    if (k > 36000) // the int32 accumulators stay exact up to 65535; longer reductions are rare enough to leave
+        return p;  // to the 64-bit multiply-add kernel from here on
+
     p.n_units = (int)(k / 16);
     p.ksteps = (p.n_units + 3) / 4;
     int rt = min(kMaxRowTiles, (g.out_c + 15) / 16);
     for (; rt >= 1; rt--) {
-        p.lds = (size_t)rt * 3 * p.ksteps * 64 * 16 + (size_t)rt * 16 * 16;
+        p.lds = (size_t)rt * 2 * p.ksteps * 64 * 16 + (size_t)rt * 16 * 16;
         if (p.lds <= kLdsBudget)
             break;
     }
