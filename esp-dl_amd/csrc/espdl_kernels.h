@@ -151,7 +151,7 @@ hipError_t launch_expand_depthwise_project_s8(const ConvGeom &g, const DwExpand 
                                               const int32_t *bias, const int32_t *shift, const DwProject &pj,
                                               int cu_count, hipStream_t stream);
 
-// Dense int16 convolution on the int8 matrix pipe (7-bit digits); in_c % 16 == 0, reduction length < 36000.
+// Dense int16 convolution on the int8 matrix pipe (two signed bytes per operand); in_c % 16 == 0, reduction length <= 36000.
 bool conv2d_s16_mfma_supports(const ConvGeom &g, const void *in, const void *filter, const void *out);
 hipError_t launch_conv2d_s16_mfma(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,
                                   const int32_t *shift, int16_t *out, int cu_count, hipStream_t stream);

@@ -159,9 +159,9 @@ def test_fused_blocks_at_the_bounds(oracle, case, xval, he):
 @pytest.mark.parametrize("k_total", [35984, 36000, 36016])
 @pytest.mark.parametrize("value", [-32768, 32767])
 def test_conv2d_s16_digit_form_guard(oracle, k_total, value):
-    """int16 convolution as 7-bit digits on the int8 matrix pipe: its five int32 digit sums stay exact for
-    reductions of at most 36000; one case just under the guard and at it, one above it (which takes the 64-bit
-    multiply-add kernel), all operands at one extreme - the largest digit sums there are."""
+    """int16 convolution as signed-byte products on the int8 matrix pipe: its int32 sums stay exact well beyond
+    the reductions of at most 36000 it accepts; one case just under that guard and at it, one above it (which
+    takes the 64-bit multiply-add kernel), all operands at one extreme - the largest byte sums there are."""
     announce(f"conv2d_s16 K={k_total} value={value}")
     m = espdl()
     x = np.full((1, 2, 3, k_total), value, dtype=np.int16)

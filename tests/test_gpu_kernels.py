@@ -375,7 +375,7 @@ S16_MFMA_CASES = [
     ("c3s2_17x15_32_70", (2, 17, 15, 32), 70, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), True, False, "random"),
     ("c3d2_12x12_48_33", (1, 12, 12, 48), 33, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2), False, True, "random"),
     ("pw_6x6_384_256", (2, 6, 6, 384), 256, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False, "random"),
-    # every digit at its extremes: all -32768, all 32767, and the 7-bit boundaries
+    # every byte of the operands at its extremes: all -32768, all 32767, and the byte boundaries
     ("extremes_min", (1, 5, 5, 64), 32, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), False, False, "min"),
     ("extremes_max", (1, 5, 5, 64), 32, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), False, False, "max"),
     ("extremes_edges", (1, 6, 6, 32), 16, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), False, False, "edges"),
@@ -384,8 +384,8 @@ S16_MFMA_CASES = [
 
 @pytest.mark.parametrize("case", S16_MFMA_CASES, ids=lambda c: c[0])
 def test_conv2d_s16_matrix_pipe(oracle, case):
-    """int16 convolutions whose input channels are a multiple of 16 run as 7-bit digit products on the int8
-    MFMA; the 64-bit sums must come out exact whatever the digits are."""
+    """int16 convolutions whose input channels are a multiple of 16 run as products of signed bytes (high byte,
+    low byte - 128) on the int8 MFMA; the 64-bit sums must come out exact whatever the bytes are."""
     announce(f"conv2d_s16 mfma {case[0]}")
     name, (n, h, w, c), oc, k, stride, dil, pads, relu, half_even, values = case
     rng = np.random.default_rng(0x516 + len(name))
@@ -394,7 +394,8 @@ def test_conv2d_s16_matrix_pipe(oracle, case):
         f = rng.integers(-32768, 32768, size=(oc, k[0], k[1], c)).astype(np.int16)
     else:
         pool = {"min": [-32768], "max": [32767],
-                "edges": [-32768, -16385, -16384, -129, -128, -1, 0, 1, 127, 128, 16383, 16384, 32767]}[values]
+                "edges": [-32768, -32513, -32512, -16385, -16384, -257, -256, -255, -129, -128, -127, -1, 0, 1, 127, 128,
+                          255, 256, 16383, 16384, 32511, 32512, 32639, 32640, 32767]}[values]
         x = rng.choice(pool, size=(n, h, w, c)).astype(np.int16)
         f = rng.choice(pool, size=(oc, k[0], k[1], c)).astype(np.int16)
     bias = rng.integers(-2**40, 2**40, size=oc).astype(np.int64)
