@@ -26,7 +26,7 @@ HIP_FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17", "-Wall", "-
 
 KERNEL_SOURCES = ["conv2d_s8_mfma.hip", "conv2d_s8_mfma_vec16.hip", "conv2d_s8_mfma_point.hip",
                   "conv2d_s8_mfma_rowseg.hip", "conv2d_s8_mfma_gather.hip", "depthwise_s8.hip", "depthwise_s8_mfma.hip", "depthwise_s8_lds.hip",
-                  "conv2d_s8_pwgemm.hip", "conv2d_s8_tiled.hip", "mbconv_s8_fused.hip", "mbconv_s8_staged.hip", "mbconv_s8_wave.hip", "mbconv_s8_group.hip", "conv_s16.hip", "conv_s16_mfma.hip", "elementwise_s8.hip", "elementwise_s16.hip", "layout_ops.hip", "max_pool_s8.hip", "attention_ops.hip", "espdl_hip_api.hip"]
+                  "conv2d_s8_pwgemm.hip", "conv2d_s8_tiled.hip", "conv2d_s8_stem.hip", "mbconv_s8_fused.hip", "mbconv_s8_staged.hip", "mbconv_s8_wave.hip", "mbconv_s8_group.hip", "conv_s16.hip", "conv_s16_mfma.hip", "elementwise_s8.hip", "elementwise_s16.hip", "layout_ops.hip", "max_pool_s8.hip", "attention_ops.hip", "espdl_hip_api.hip"]
 
 
 def _run(cmd):

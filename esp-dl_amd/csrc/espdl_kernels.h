@@ -151,6 +151,12 @@ hipError_t launch_expand_depthwise_project_s8(const ConvGeom &g, const DwExpand 
                                               const int32_t *bias, const int32_t *shift, const DwProject &pj,
                                               int cu_count, hipStream_t stream);
 
+// Dense int8 convolution whose window rows are at most 16 contiguous bytes (k_w * in_c <= 16, k_h <= 4, at most
+// 64 filters): the first layer of a network on RGB / grey images, one MFMA step per 16 pixels (conv2d_s8_stem.hip).
+bool conv2d_s8_stem_supports(const ConvGeom &g, const void *residual);
+hipError_t launch_conv2d_s8_stem(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                 const int32_t *shift, const int8_t *lut, int8_t *out, int cu_count, hipStream_t stream);
+
 // Dense int16 convolution on the int8 matrix pipe (two signed bytes per operand); in_c % 16 == 0, reduction length <= 36000.
 bool conv2d_s16_mfma_supports(const ConvGeom &g, const void *in, const void *filter, const void *out);
 hipError_t launch_conv2d_s16_mfma(const ConvGeom &g, const int16_t *in, const int16_t *filter, const int64_t *bias,

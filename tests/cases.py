@@ -29,6 +29,23 @@ CONV_CASES = [
     ("c32_10x10_k3p1_oc64_relu", (10, 10, 32), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
 ]
 
+# Convolutions whose window rows are at most 16 contiguous bytes (k_w * C <= 16) with at most 4 rows and 64 filters:
+# the first-layer kernel that does the whole reduction in one MFMA step.  RGB / grey / RGBA / 5 and 8 channels, a
+# 1 x 2 window over 8 channels, 7 to 64 filters (1 to 4 filter tiles, ragged ones), strides 1 to 3, dilated
+# rows, padding on both / one / no side, rows longer than one 64-pixel unit, a one-row image.
+STEM_CASES = [
+    ("s3_64x96_k3s2p1_oc16", (64, 96, 3), 16, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, True),
+    ("s3_50x70_k3s1p1_oc32", (50, 70, 3), 32, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False),
+    ("s1_40x130_k4s2_oc8", (40, 130, 1), 8, (4, 4), (2, 2), (1, 1), (1, 2, 1, 2), True, True),
+    ("s4_33x65_k3s2p1_oc24", (33, 65, 4), 24, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), False, False),
+    ("s5_30x40_k3dh2_oc48", (30, 40, 5), 48, (3, 3), (1, 1), (2, 1), (2, 2, 1, 1), True, True),
+    ("s8_40x40_k1x2_oc64", (40, 40, 8), 64, (1, 2), (1, 1), (1, 1), (0, 0, 0, 1), True, False),
+    ("s8_37x41_k2s2_oc20_tailpad", (37, 41, 8), 20, (2, 2), (2, 2), (1, 1), (0, 1, 0, 1), True, True),
+    ("s3_20x200_k3s2_nopad_oc16", (20, 200, 3), 16, (3, 3), (2, 2), (1, 1), (0, 0, 0, 0), True, True),
+    ("s2_24x24_k3s3p2_oc7", (24, 24, 2), 7, (3, 3), (3, 3), (1, 1), (2, 2, 2, 2), True, False),
+    ("s3_1x700_k3s2_oc16", (1, 700, 3), 16, (1, 3), (1, 2), (1, 1), (0, 0, 1, 1), True, True),
+]
+
 # Windowed convolutions whose channel count is a multiple of 16: the kernel that stages the input tile and the
 # filters in LDS.  Strides 1 to 3, dilation, reduction steps that span several taps (16, 32, 48 channels), several
 # groups of 64 filters in one and in several chunks, filter counts that are not a multiple of 64 / 16 / 4, images

@@ -5,7 +5,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
+from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
 from gpu_util import announce, espdl, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
@@ -102,6 +102,52 @@ def test_conv2d_s8_lds_tiled(oracle, case, flavour):
             bias[::2] = (1 << 30) - 7
     got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
     np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", STEM_CASES, ids=lambda c: c[0])
+@pytest.mark.parametrize("flavour", ["per_tensor", "per_channel", "half_even", "lut", "general_epilogue"])
+def test_conv2d_s8_first_layer(oracle, case, flavour):
+    """Few-channel images through the one-MFMA-step kernel: both exponent forms, round-half-even, a table in the
+    epilogue, and shifts outside 1..31 mixed with large biases (the general shift-and-round form)."""
+    announce(f"conv2d_s8 first layer {case[0]} {flavour}")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 223, 3, flavour != "per_tensor")
+    kw = {}
+    if flavour == "half_even":
+        kw["half_even"] = True
+    if flavour == "lut":
+        kw["lut"] = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8)
+        relu = False
+    if flavour == "general_epilogue":
+        shift = np.array(shift, dtype=np.int32)
+        shift[::3] = 0
+        shift[1::5] = 33
+        if bias is not None:
+            bias = bias.copy()
+            bias[::2] = (1 << 30) - 7
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_conv2d_s8_first_layer_at_the_tensor_end(oracle):
+    """The last pixels of the last row of the last image: their 16-byte reads would end behind the tensor, so
+    they are assembled byte by byte.  The input sits at the very end of its allocation."""
+    import torch
+    announce("conv2d_s8 first layer tensor end")
+    m = espdl()
+    rng = np.random.default_rng(229)
+    n, h, w, c, oc = 2, 33, 47, 3, 16
+    x = rng_int8(rng, (n, h, w, c))
+    f = rng_int8(rng, (oc, 3, 3, c))
+    bias = rng.integers(-4096, 4097, size=oc).astype(np.int32)
+    shift = np.full(oc, 9, dtype=np.int32)
+    want = oracle.conv2d_s8(x, f, bias, shift, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), oracle.RELU, oracle.ROUND_HALF_UP)
+    # a buffer that ends exactly with the tensor (torch rounds allocations up, so the slice ends inside one; what
+    # matters is that the kernel never needs the bytes behind)
+    buf = torch.empty(x.size + 4096, dtype=torch.int8, device="cuda")
+    xd = buf[4096:].view(n, h, w, c)
+    xd.copy_(torch.from_numpy(x))
+    got = m.conv2d(xd, to_dev(f), to_dev(bias), to_dev(shift), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), activation=m.capi.RELU)
+    np.testing.assert_array_equal(to_host(got), want)
 
 
 # Operands that are channel slices of wider NHWC tensors (what a Conv reads from a Split output and writes into its
