@@ -89,12 +89,14 @@ def lib():
         L.espdl_hip_mul_s8.restype = ctypes.c_int
         L.espdl_hip_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp]
         L.espdl_hip_requantize_s8.argtypes = [vp, i64, i32, i32, vp, vp]
+        L.espdl_hip_requantize_s8_rows.argtypes = [vp, i64, vp, i64, i64, i64, i32, i32, vp]
         L.espdl_hip_requantize.argtypes = [vp, i32, i64, i32, i32, vp, i32, vp]
         f32 = ctypes.c_float
         L.espdl_hip_concat.argtypes = [i32, vp, vp, i64, vp, vp]
         L.espdl_hip_copy_rows.argtypes = [vp, i64, vp, i64, i64, i64, vp]
         L.espdl_hip_transpose.argtypes = [vp, vp, i32, vp, i32, i32, vp, vp]
         L.espdl_hip_resize_nearest_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, vp, vp]
+        L.espdl_hip_resize_nearest_s8_pitched.argtypes = [vp, i32, i32, i32, i32, i32, i32, f32, f32, i32, i32, i32, i32, vp, vp]
         L.espdl_hip_max_pool.argtypes = [vp, i32] + [i32] * 12 + [vp, vp]
         L.espdl_hip_max_pool_pitched.argtypes = [vp, i32] + [i32] * 14 + [vp, vp]
         L.espdl_hip_avg_pool_s8.argtypes = [vp] + [i32] * 14 + [vp, vp]
@@ -335,8 +337,14 @@ def global_avg_pool_s8(x, in_exp, out_exp, out=None, stream=None):
 
 
 def requantize_s8(x, in_exp, out_exp, out=None, stream=None):
+    """x and out may be channel slices of wider NHWC tensors (wide[..., a:b])."""
     import torch
-    out = torch.empty_like(x) if out is None else out
+    out = torch.empty(x.shape, dtype=torch.int8, device=x.device) if out is None else out
+    if x.dim() == 4 and (_channel_pitch(x) or _channel_pitch(out)):
+        c = x.shape[3]
+        _check(lib().espdl_hip_requantize_s8_rows(_p(x), _channel_pitch(x) or c, _p(out), _channel_pitch(out) or c, c,
+                                                  x.numel() // c, in_exp, out_exp, _stream(stream)))
+        return out
     _check(lib().espdl_hip_requantize_s8(_p(x), x.numel(), in_exp, out_exp, _p(out), _stream(stream)))
     return out
 
@@ -413,6 +421,11 @@ def resize_nearest_s8(x, scale_h, scale_w, in_exp=0, out_exp=0, out_hw=None, out
     n, h, w, c = x.shape
     oh, ow = out_hw if out_hw is not None else (int(h * np.float32(scale_h)), int(w * np.float32(scale_w)))
     out = torch.empty((n, oh, ow, c), dtype=torch.int8, device=x.device) if out is None else out
+    ip, op = _channel_pitch(x), _channel_pitch(out)
+    if ip or op:  # channel slices of wider NHWC tensors
+        _check(lib().espdl_hip_resize_nearest_s8_pitched(_p(x), n, h, w, c, oh, ow, float(scale_h), float(scale_w), in_exp,
+                                                         out_exp, ip, op, _p(out), _stream(stream)))
+        return out
     _check(lib().espdl_hip_resize_nearest_s8(_p(x), n, h, w, c, oh, ow, float(scale_h), float(scale_w), in_exp, out_exp,
                                              _p(out), _stream(stream)))
     return out

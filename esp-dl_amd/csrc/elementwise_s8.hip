@@ -448,6 +448,56 @@ hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int 
     return launch_map(in, out, size, RequantFn{dl_scale(in_exp), inv}, stream);
 }
 
+namespace {
+// The same on rows that lie `in_pitch` / `out_pitch` bytes apart (channel slices of wider NHWC tensors): a thread
+// takes one 16-byte unit of a row (VEC) or one byte of it.
+template <bool VEC>
+__global__ __launch_bounds__(kBlock) void requantize_s8_rows_kernel(const int8_t *in, int64_t in_pitch, int8_t *out,
+                                                                   int64_t out_pitch, FastDiv per_row, int64_t total, int d,
+                                                                   RequantFn f)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total)
+        return;
+    const unsigned row = fastdiv((unsigned)i, per_row);
+    const unsigned u = (unsigned)i - row * per_row.d;
+    if constexpr (VEC) {
+        const Requant4 q = make_requant4(d);
+        const v4i v = *reinterpret_cast<const v4i *>(in + (int64_t)row * in_pitch + 16 * (int64_t)u);
+        v4i r;
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+            r[w] = requant4_s8(v[w], q);
+        *reinterpret_cast<v4i *>(out + (int64_t)row * out_pitch + 16 * (int64_t)u) = r;
+    } else {
+        out[(int64_t)row * out_pitch + u] = (int8_t)f((int)in[(int64_t)row * in_pitch + u], 0);
+    }
+}
+} // namespace
+
+hipError_t launch_requantize_s8_rows(const int8_t *in, int64_t in_pitch, int8_t *out, int64_t out_pitch, int64_t row_bytes,
+                                     int64_t rows, int in_exp, int out_exp, hipStream_t stream)
+{
+    if (rows <= 0 || row_bytes <= 0)
+        return hipSuccess;
+    const int d = in_exp - out_exp;
+    const RequantFn f{dl_scale(in_exp), (float)(1.0 / (double)dl_scale(out_exp))};
+    const bool vec = d >= -7 && d <= 7 && (row_bytes & 15) == 0 && (in_pitch & 15) == 0 && (out_pitch & 15) == 0 &&
+        aligned16(in, out);
+    const int64_t per_row = vec ? row_bytes / 16 : row_bytes;
+    const int64_t total = rows * per_row;
+    if (total > 0x7fffffffll || per_row > 0x7fffffffll)
+        return hipErrorInvalidValue;
+    const dim3 grid((unsigned)((total + kBlock - 1) / kBlock));
+    if (vec)
+        hipLaunchKernelGGL(requantize_s8_rows_kernel<true>, grid, dim3(kBlock), 0, stream, in, in_pitch, out, out_pitch,
+                           make_fastdiv((unsigned)per_row), total, d, f);
+    else
+        hipLaunchKernelGGL(requantize_s8_rows_kernel<false>, grid, dim3(kBlock), 0, stream, in, in_pitch, out, out_pitch,
+                           make_fastdiv((unsigned)per_row), total, d, f);
+    return hipGetLastError();
+}
+
 // TensorBase::assign between int8 / int16 (esp-dl/dl/tensor/src/dl_tensor_base.cpp:321-392).
 // Eight elements per thread (one 8- or 16-byte access each way) when both pointers allow; the last size % 8 elements,
 // or everything when a pointer is unaligned, one element per thread.

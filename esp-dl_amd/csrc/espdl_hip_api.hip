@@ -412,6 +412,25 @@ int espdl_hip_requantize_s8(const int8_t *in, int64_t size, int32_t in_exp, int3
         "requantize_s8");
 }
 
+int espdl_hip_requantize_s8_rows(const int8_t *in, int64_t in_pitch, int8_t *out, int64_t out_pitch, int64_t row_bytes,
+                                 int64_t rows, int32_t in_exp, int32_t out_exp, void *stream)
+{
+    if (rows < 0 || row_bytes < 0 || in_pitch < row_bytes || out_pitch < row_bytes)
+        return fail(ESPDL_HIP_EINVAL, "rows of %lld bytes need pitches of at least that (got %lld / %lld) and a count >= 0",
+                    (long long)row_bytes, (long long)in_pitch, (long long)out_pitch);
+    if (check_exps(in_exp, out_exp) != ESPDL_HIP_OK)
+        return ESPDL_HIP_EINVAL;
+    if (rows == 0 || row_bytes == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr || out == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
+    if (in_exp == out_exp)
+        return espdl_hip_copy_rows(in, in_pitch, out, out_pitch, row_bytes, rows, stream);
+    return device_status(espdl::launch_requantize_s8_rows(in, in_pitch, out, out_pitch, row_bytes, rows, in_exp, out_exp,
+                                                          reinterpret_cast<hipStream_t>(stream)),
+                         "requantize_s8_rows");
+}
+
 int espdl_hip_requantize(const void *in, int32_t in_dtype, int64_t size, int32_t in_exp, int32_t out_exp, void *out,
                          int32_t out_dtype, void *stream)
 {
@@ -509,9 +528,9 @@ int espdl_hip_transpose(const void *in, const int32_t *shape, int32_t dims, cons
                          "transpose");
 }
 
-int espdl_hip_resize_nearest_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t out_h,
-                                int32_t out_w, float scale_h, float scale_w, int32_t in_exp, int32_t out_exp,
-                                int8_t *out, void *stream)
+int espdl_hip_resize_nearest_s8_pitched(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t out_h,
+                                        int32_t out_w, float scale_h, float scale_w, int32_t in_exp, int32_t out_exp,
+                                        int32_t in_pitch, int32_t out_pitch, int8_t *out, void *stream)
 {
     if (batch < 0 || h <= 0 || w <= 0 || c <= 0 || out_h < 0 || out_w < 0 || !(scale_h > 0) || !(scale_w > 0))
         return fail(ESPDL_HIP_EINVAL, "bad resize geometry");
@@ -519,14 +538,25 @@ int espdl_hip_resize_nearest_s8(const int8_t *in, int32_t batch, int32_t h, int3
         return ESPDL_HIP_EINVAL;
     if (out_exp - in_exp > 30 || in_exp - out_exp > 30)
         return fail(ESPDL_HIP_EINVAL, "exponent difference out of range");
+    if (in_pitch < 0 || out_pitch < 0 || (in_pitch != 0 && in_pitch < c) || (out_pitch != 0 && out_pitch < c))
+        return fail(ESPDL_HIP_EINVAL, "channel pitches %d / %d must be 0 or at least the channel count %d", in_pitch, out_pitch,
+                    c);
     if ((long long)batch * out_h * out_w == 0)
         return ESPDL_HIP_OK;
     if (in == nullptr || out == nullptr)
         return fail(ESPDL_HIP_EINVAL, "in and out must not be NULL");
     return device_status(espdl::launch_resize_nearest_s8(in, batch, h, w, c, out_h, out_w, scale_h, scale_w, in_exp,
-                                                         out_exp, out, cu_count_cached(),
-                                                         reinterpret_cast<hipStream_t>(stream)),
+                                                         out_exp, in_pitch != 0 ? in_pitch : c, out_pitch != 0 ? out_pitch : c,
+                                                         out, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
                          "resize_nearest_s8");
+}
+
+int espdl_hip_resize_nearest_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t out_h,
+                                int32_t out_w, float scale_h, float scale_w, int32_t in_exp, int32_t out_exp,
+                                int8_t *out, void *stream)
+{
+    return espdl_hip_resize_nearest_s8_pitched(in, batch, h, w, c, out_h, out_w, scale_h, scale_w, in_exp, out_exp, 0, 0, out,
+                                               stream);
 }
 
 int espdl_hip_max_pool_pitched(const void *in, int32_t dtype, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t k_h,

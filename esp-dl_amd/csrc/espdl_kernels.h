@@ -178,6 +178,9 @@ hipError_t launch_mul_s8(const int32_t dims[4], const int64_t s0[4], const int64
                          const int8_t *in1, int shift, int half_even, int8_t *out, hipStream_t stream);
 hipError_t launch_global_avg_pool_s8(const int8_t *in, int batch, int h, int w, int c, int in_exp, int out_exp,
                                      int8_t *out, hipStream_t stream);
+// rows of row_bytes int8 values that lie in_pitch / out_pitch bytes apart (channel slices of wider tensors)
+hipError_t launch_requantize_s8_rows(const int8_t *in, int64_t in_pitch, int8_t *out, int64_t out_pitch, int64_t row_bytes,
+                                     int64_t rows, int in_exp, int out_exp, hipStream_t stream);
 hipError_t launch_requantize_s8(const int8_t *in, int64_t size, int in_exp, int out_exp, int8_t *out,
                                 hipStream_t stream);
 
@@ -192,8 +195,8 @@ hipError_t launch_concat(int n_inputs, const void *const *inputs, const long lon
 hipError_t launch_transpose(const void *in, const int *shape, int dims, const int *perm, int elem_size, void *out,
                             int cu_count, hipStream_t stream);
 hipError_t launch_resize_nearest_s8(const int8_t *in, int batch, int h, int w, int c, int out_h, int out_w, float scale_h,
-                                    float scale_w, int in_exp, int out_exp, int8_t *out, int cu_count,
-                                    hipStream_t stream);
+                                    float scale_w, int in_exp, int out_exp, long long in_pitch, long long out_pitch,
+                                    int8_t *out, int cu_count, hipStream_t stream);
 // in_pitch / out_pitch: elements from pixel to pixel (c for dense tensors, more for channel slices)
 hipError_t launch_max_pool(const void *in, int elem_size, int batch, int h, int w, int c, int k_h, int k_w, int stride_h,
                            int stride_w, int pad_top, int pad_left, int out_h, int out_w, long long in_pitch,

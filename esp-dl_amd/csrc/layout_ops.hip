@@ -200,6 +200,7 @@ struct ResizeArgs {
     int vec;            // channels per thread: 16 or 1
     FastDiv fd_cv, fd_ow, fd_oh;
     long long total;
+    long long in_pitch, out_pitch; // elements from pixel to pixel (c when dense)
 };
 
 __device__ __forceinline__ int resize_value(int x, int rshift, int lshift)
@@ -222,8 +223,8 @@ __global__ __launch_bounds__(kBlock) void resize_nearest_s8_kernel(const ResizeA
         int in_x = a.exact2 ? (int)(x >> 1) : (int)((float)x * a.scale_w_inv);
         in_y = min(in_y, a.h - 1);
         in_x = min(in_x, a.w - 1);
-        const long long src = (((long long)n * a.h + in_y) * a.w + in_x) * a.c + (long long)v * a.vec;
-        const long long dst = (long long)pix * a.c + (long long)v * a.vec;
+        const long long src = (((long long)n * a.h + in_y) * a.w + in_x) * a.in_pitch + (long long)v * a.vec;
+        const long long dst = (long long)pix * a.out_pitch + (long long)v * a.vec;
         if (a.vec == 16) {
             v4i d = *reinterpret_cast<const v4i *>(a.in + src);
             if (a.rshift | a.lshift) {
@@ -704,12 +705,14 @@ hipError_t launch_transpose(const void *in, const int *shape, int dims, const in
 }
 
 hipError_t launch_resize_nearest_s8(const int8_t *in, int batch, int h, int w, int c, int out_h, int out_w, float scale_h,
-                                    float scale_w, int in_exp, int out_exp, int8_t *out, int cu_count,
-                                    hipStream_t stream)
+                                    float scale_w, int in_exp, int out_exp, long long in_pitch, long long out_pitch,
+                                    int8_t *out, int cu_count, hipStream_t stream)
 {
     ResizeArgs a;
     a.in = in;
     a.out = out;
+    a.in_pitch = in_pitch;
+    a.out_pitch = out_pitch;
     a.h = h;
     a.w = w;
     a.c = c;
@@ -721,7 +724,8 @@ hipError_t launch_resize_nearest_s8(const int8_t *in, int batch, int h, int w, i
     const int d = out_exp - in_exp;
     a.rshift = d > 0 ? d : 0;
     a.lshift = d < 0 ? -d : 0;
-    const bool vec_ok = (c & 15) == 0 && ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    const bool vec_ok = (c & 15) == 0 && (in_pitch & 15) == 0 && (out_pitch & 15) == 0 &&
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
     a.vec = vec_ok ? 16 : 1;
     const int cv = c / a.vec;
     a.total = (long long)batch * out_h * out_w * cv;

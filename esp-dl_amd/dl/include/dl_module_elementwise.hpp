@@ -549,6 +549,10 @@ public:
         if (!on_device_all({input, output}) || !output->assign(input, context->stream))
             DL_LOGE("RequantizeLinear", "%s: assign failed", name.c_str());
     }
+    /// int8 -> int8 goes row by row when either side is a channel slice of a wider tensor; a model only makes such
+    /// slices where both sides are int8 (TensorBase::assign handles nothing else with a pitch on the output).
+    bool reads_channel_slice(int slot) const { return slot == 0 && quant_type == QUANT_TYPE_SYMM_8BIT; }
+    bool writes_channel_slice(int slot) const { return slot == 0 && quant_type == QUANT_TYPE_SYMM_8BIT; }
     static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
     {
         quant_type_t quant_type = QUANT_TYPE_NONE;

@@ -348,12 +348,16 @@ public:
         const int c = nwc ? input->shape[2] : input->shape[3];
         const int oh = nwc ? 1 : output->shape[1], ow = nwc ? output->shape[1] : output->shape[2];
         const float sh = nwc ? 1.0f : m_scales[2], sw = nwc ? m_scales[2] : m_scales[3];
-        const int rc = espdl_hip_resize_nearest_s8(static_cast<const int8_t *>(input->data), input->shape[0], h, w, c, oh,
-                                                   ow, sh, sw, input->exponent.get(), output->exponent.get(),
-                                                   static_cast<int8_t *>(output->data), context->stream);
+        const int rc = espdl_hip_resize_nearest_s8_pitched(
+            static_cast<const int8_t *>(input->data), input->shape[0], h, w, c, oh, ow, sh, sw, input->exponent.get(),
+            output->exponent.get(), input->is_dense() ? 0 : input->channel_pitch,
+            output->is_dense() ? 0 : output->channel_pitch, static_cast<int8_t *>(output->data), context->stream);
         if (rc != ESPDL_HIP_OK)
             DL_LOGE("Resize", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
+    /// The kernel takes a channel pitch on either side (an upsampled tensor is written into the Concat behind it).
+    bool reads_channel_slice(int slot) const { return slot == 0 && quant_type == QUANT_TYPE_SYMM_8BIT; }
+    bool writes_channel_slice(int slot) const { return slot == 0 && quant_type == QUANT_TYPE_SYMM_8BIT; }
     static Module *deserialize(fbs::FbsModel *fbs_model, std::string node_name)
     {
         quant_type_t quant_type = QUANT_TYPE_NONE;

@@ -753,10 +753,23 @@ esp_err_t Model::build(int batch)
             return v > 0 && v < CONTEXT_PARAMETER_OFFSET && vars[v].known && vars[v].dtype == DATA_TYPE_INT8 &&
                 vars[v].shape.size() >= 2 && !aliased[v];
         };
+        // a RequantizeLinear handles pitches between int8 tensors only
+        auto int8_only = [&](dl::module::Module *m) {
+            if (typeid(*m) != typeid(dl::module::RequantizeLinear))
+                return true;
+            for (int idx : m->m_inputs_index)
+                if (idx > 0 && idx < CONTEXT_PARAMETER_OFFSET && vars[idx].dtype != DATA_TYPE_INT8)
+                    return false;
+            for (int idx : m->m_outputs_index)
+                if (vars[idx].dtype != DATA_TYPE_INT8)
+                    return false;
+            return true;
+        };
         // every reader but module `except` takes the tensor with a pitch
         auto readers_take_pitch = [&](int v, int except) {
             for (auto &r : readers[v])
-                if (r.first != except && !m_execution_plan[r.first]->reads_channel_slice(r.second))
+                if (r.first != except &&
+                    (!m_execution_plan[r.first]->reads_channel_slice(r.second) || !int8_only(m_execution_plan[r.first])))
                     return false;
             return true;
         };
@@ -796,10 +809,11 @@ esp_err_t Model::build(int batch)
                 for (size_t k = 0; k < producer->m_outputs_index.size(); k++)
                     if (producer->m_outputs_index[k] == v)
                         slot = (int)k;
-                if (slot < 0 || !producer->writes_channel_slice(slot) || !readers_take_pitch(v, i))
+                if (slot < 0 || !producer->writes_channel_slice(slot) || !int8_only(producer) || !readers_take_pitch(v, i))
                     return false;
-                // an in-place producer may already have been promised its input's bytes
-                return producer->inplace == MODULE_NON_INPLACE;
+                // (a producer that may work in place simply does not when its output is a slice: the placement
+                // below looks at slices first; one whose output IS its input's buffer never gets here, see aliased)
+                return producer->inplace != MODULE_INPLACE_UNCHANGED_BUFFER;
             };
             const std::vector<int> &in = cat->m_inputs_index;
             int at = 0;

@@ -314,19 +314,21 @@ bool TensorBase::assign(TensorBase *tensor, void *stream)
     const bool per_channel = exponent.is_per_channel() || tensor->exponent.is_per_channel();
     if (exponent == tensor->exponent && dtype == tensor->dtype)
         return copy_from(tensor, stream);
-    if (!is_dense()) {
-        DL_LOGE("TensorBase::assign", "a channel slice of a wider tensor can only be copied to, not requantized to");
-        return false;
-    }
-    if (!tensor->is_dense()) {
-        // requantize from a dense copy of the slice
+    if (!is_dense() || !tensor->is_dense()) {
+        // channel slices of wider device tensors: int8 -> int8 row by row; anything else from a dense copy
+        if (dtype == DATA_TYPE_INT8 && tensor->dtype == DATA_TYPE_INT8 && on_device() && tensor->on_device() && !per_channel) {
+            const RowView d = row_view(this), v = row_view(tensor);
+            return espdl_hip_requantize_s8_rows(static_cast<const int8_t *>(tensor->data), (int64_t)v.pitch_bytes,
+                                                static_cast<int8_t *>(data), (int64_t)d.pitch_bytes, (int64_t)v.row_bytes,
+                                                (int64_t)v.rows, tensor->exponent, exponent, stream) == ESPDL_HIP_OK;
+        }
+        if (!is_dense()) {
+            DL_LOGE("TensorBase::assign", "only int8 device tensors can be requantized into a channel slice");
+            return false;
+        }
         TensorBase dense(tensor->shape, nullptr, 0, tensor->dtype, true, tensor->caps);
         dense.exponent = tensor->exponent;
         return dense.copy_from(tensor, stream) && assign(&dense, stream);
-    }
-    if (per_channel) {
-        DL_LOGE("TensorBase::assign", "per-channel tensors can only be copied, not requantized");
-        return false;
     }
     const bool ints = (dtype == DATA_TYPE_INT8 || dtype == DATA_TYPE_INT16) &&
         (tensor->dtype == DATA_TYPE_INT8 || tensor->dtype == DATA_TYPE_INT16);

@@ -702,7 +702,8 @@ def channel_slices(seed=0xE5E7):
     channels (rows that are not multiples of 16 bytes), a piece read by a module that takes no channel
     pitch (Relu), a residual Add on a piece, a Concat of all pieces of a Split plus more (the C2f pattern),
     one tensor twice in a Concat, one tensor in two Concats, a Concat input that is a graph output, a Concat
-    with the graph input, a strided 3x3 Conv on a piece and a depthwise Conv (no pitches) on another."""
+    with the graph input, a strided 3x3 Conv on a piece and a depthwise Conv (no pitches) on another, a
+    RequantizeLinear and a Resize that write their places in a Concat."""
     g = GraphSpec("channel_slices")
     b = Builder(g, seed, per_channel=True, w_exp_range=None)
     x = b.input("input", [1, 14, 18, 24], -5)
@@ -729,6 +730,12 @@ def channel_slices(seed=0xE5E7):
     t2 = b.conv(t, 8, k=3, stride=2, out_exp=e, name="s5_strided")
     u2 = b.conv(u, 16, k=3, stride=2, depthwise=True, out_exp=e, name="s5_dw")
     b.output(b.concat([t2, u2], name="s5_out"))
+    # a Concat input at a finer exponent (requantized straight into its place), an upsampled one (the Resize
+    # writes its place, reading a tensor that itself lives in another Concat) and a graph output (copied)
+    fine = b.conv(out1, 16, k=1, out_exp=e - 1, name="s6_fine")
+    up = b.resize_nearest(t2, 2, name="s6_up")
+    cat6 = b.concat([fine, up, out1], name="s6_cat")    # 16 + 8 + 16 = 40
+    b.output(b.conv(cat6, 8, k=1, out_exp=e, name="s6_out"))
     return g
 
 

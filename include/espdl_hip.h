@@ -162,6 +162,12 @@ int espdl_hip_global_avg_pool_s8(const int8_t *in, int32_t batch, int32_t h, int
 int espdl_hip_requantize_s8(const int8_t *in, int64_t size, int32_t in_exp, int32_t out_exp, int8_t *out,
                             void *stream);
 
+/* int8 -> int8 requantization (TensorBase::assign, esp-dl/dl/tensor/src/dl_tensor_base.cpp:223-401) of `rows` runs
+ * of row_bytes values that lie in_pitch / out_pitch bytes apart: the channels of one tensor when it, or its
+ * destination, is a channel slice of a wider NHWC tensor (rows = pixels, row_bytes = channels). */
+int espdl_hip_requantize_s8_rows(const int8_t *in, int64_t in_pitch, int8_t *out, int64_t out_pitch, int64_t row_bytes,
+                                 int64_t rows, int32_t in_exp, int32_t out_exp, void *stream);
+
 /* TensorBase::assign between int8 / int16 tensors of any two exponents
  * (esp-dl/dl/tensor/src/dl_tensor_base.cpp:321-392): same exponent widens (int8 -> int16) or saturates
  * (int16 -> int8); different exponents run quantize(dequantize(x)) in float32 with round-half-up.
@@ -201,6 +207,11 @@ int espdl_hip_transpose(const void *in, const int32_t *shape, int32_t dims, cons
 int espdl_hip_resize_nearest_s8(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t out_h,
                                 int32_t out_w, float scale_h, float scale_w, int32_t in_exp, int32_t out_exp,
                                 int8_t *out, void *stream);
+/* The same on channel slices of wider NHWC tensors (in_pitch / out_pitch: elements from pixel to pixel, 0 = c), so
+ * that the upsampling of a top-down path writes its part of the Concat behind it (dl_module_concat.hpp:86-108). */
+int espdl_hip_resize_nearest_s8_pitched(const int8_t *in, int32_t batch, int32_t h, int32_t w, int32_t c, int32_t out_h,
+                                        int32_t out_w, float scale_h, float scale_w, int32_t in_exp, int32_t out_exp,
+                                        int32_t in_pitch, int32_t out_pitch, int8_t *out, void *stream);
 
 /* base::max_pool2d (esp-dl/dl/base/dl_base_max_pool2d.cpp:9-29) over the window clipped to the image;
  * output size (h + pad_top + pad_bottom - k_h) / stride_h + 1 and likewise for the width

@@ -223,6 +223,45 @@ def test_max_pool_channel_slices(oracle, c, wide_in, wide_out, at):
     assert (rest == 77).all()
 
 
+@pytest.mark.parametrize("c,wide_in,wide_out,at,exps", [(16, 64, 48, 16, (-4, -4)), (32, 32, 128, 96, (-4, -3)), (24, 72, 48, 24, (-5, -3)),
+                                                        (16, 16, 40, 8, (-4, -4))])
+def test_resize_nearest_channel_slices(oracle, c, wide_in, wide_out, at, exps):
+    import torch
+    announce(f"resize slices c={c} in={wide_in} out={wide_out} at={at} exps={exps}")
+    m = espdl()
+    rng = np.random.default_rng(28)
+    xin = _rand(rng, (2, 9, 7, wide_in))
+    lo = min(at, wide_in - c)
+    x = np.ascontiguousarray(xin[..., lo:lo + c])
+    want = oracle.resize_nearest_s8(x, 2, 2, exps[0], exps[1])
+    wide = to_dev(xin)
+    out_wide = torch.full((2, 18, 14, wide_out), 77, dtype=torch.int8, device="cuda")
+    m.resize_nearest_s8(wide[..., lo:lo + c], 2, 2, exps[0], exps[1], out=out_wide[..., at:at + c])
+    got = to_host(out_wide)
+    np.testing.assert_array_equal(got[..., at:at + c], want)
+    assert (np.delete(got, np.s_[at:at + c], axis=3) == 77).all()
+
+
+@pytest.mark.parametrize("c,wide_in,wide_out,at", [(16, 64, 48, 16), (32, 32, 128, 96), (24, 72, 48, 24), (20, 33, 41, 7)])
+@pytest.mark.parametrize("exps", [(-4, -5), (-3, -6), (-6, -4), (-2, -12), (-4, -4)])
+def test_requantize_s8_channel_slices(oracle, c, wide_in, wide_out, at, exps):
+    """int8 -> int8 between exponents on rows with pitches: 16-byte units, bytes, shifts beyond 7, a plain copy."""
+    import torch
+    announce(f"requantize slices c={c} in={wide_in} out={wide_out} at={at} exps={exps}")
+    m = espdl()
+    rng = np.random.default_rng(29)
+    xin = _rand(rng, (3, 5, 11, wide_in))
+    lo = min(at, wide_in - c)
+    x = np.ascontiguousarray(xin[..., lo:lo + c])
+    want = oracle.requantize_s8(x, exps[0], exps[1])
+    wide = to_dev(xin)
+    out_wide = torch.full((3, 5, 11, wide_out), 77, dtype=torch.int8, device="cuda")
+    m.requantize_s8(wide[..., lo:lo + c], exps[0], exps[1], out=out_wide[..., at:at + c])
+    got = to_host(out_wide)
+    np.testing.assert_array_equal(got[..., at:at + c], want)
+    assert (np.delete(got, np.s_[at:at + c], axis=3) == 77).all()
+
+
 def test_sppf_pool_chain_idempotence():
     """Size-independent property at full batch: three chained 5x5/1 pools equal one 13x13/1 pool, and
     pooling is monotone (output >= input)."""

@@ -225,6 +225,8 @@ def test_channel_slices_every_case(oracle):
     assert pitch["s3_y_out"] == 24 and pitch["s3_z_out"] == 48 and dense("s4_out_out")
     assert pitch["s5_split_out0"] == 24 and dense("s5_split_out1")  # the depthwise Conv takes no pitch
     assert pitch["s5_strided_out"] == 24 and dense("s5_dw_out")
+    # the requantized and the upsampled input of the last Concat are written in their places (40 wide)
+    assert pitch["s6_cat_rq0_out"] == 40 and pitch["s6_up_out"] == 40 and dense("s6_fine_out")
     # (intermediate tensors share arena space: only the graph outputs, which every slice feeds, outlive a pass)
     for rep in range(2):
         for name in spec.outputs:
