@@ -195,18 +195,15 @@ int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const 
                                      "depthwise_s8_mfma");
             return device_status(espdl::launch_depthwise_s8(g, i8, f8, b32, shift, lut, o8, s), "depthwise_s8");
         }
-        static const bool no_stem = getenv("ESPDL_HIP_NO_STEM") != nullptr;
-        if (!no_stem && espdl::conv2d_s8_stem_supports(g, residual))
+        if (espdl::conv2d_s8_stem_supports(g, residual))
             return device_status(espdl::launch_conv2d_s8_stem(g, i8, f8, b32, shift, lut, o8, cu_count_cached(), s),
                                  "conv2d_s8_stem");
         // (the second test admits products with fewer than 32 filters, which only the few-rows kernel inside takes)
-        static const bool no_pw = getenv("ESPDL_HIP_NO_PWGEMM") != nullptr;
-        if (!no_pw && espdl::conv2d_s8_pwgemm_supports(g, in, filter, cu_count_cached()) ||
+        if (espdl::conv2d_s8_pwgemm_supports(g, in, filter, cu_count_cached()) ||
             (lut == nullptr && residual == nullptr && espdl::conv2d_s8_rows_supports(g, in, filter, cu_count_cached())))
             return device_status(espdl::launch_conv2d_s8_pwgemm(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
                                  "conv2d_s8_pwgemm");
-        static const bool no_tiled = getenv("ESPDL_HIP_NO_TILED") != nullptr;
-        if (!no_tiled && espdl::conv2d_s8_tiled_supports(g, in, filter, cu_count_cached()))
+        if (espdl::conv2d_s8_tiled_supports(g, in, filter, cu_count_cached()))
             return device_status(espdl::launch_conv2d_s8_tiled(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
                                  "conv2d_s8_tiled");
         return device_status(espdl::launch_conv2d_s8_mfma(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),

@@ -203,6 +203,28 @@ def test_config4_yolo_style(oracle, fuse):
     mdl.close()
 
 
+def test_first_block_with_requantized_residual_from_the_graph_input(oracle):
+    """The very first modules of the plan form a block whose residual is the graph input behind a
+    RequantizeLinear: absorbing that node must not end the scan, so the second block fuses as well."""
+    announce("model two blocks, first residual requantized from the graph input")
+    _, zoo, model, runner = _mods()
+    g = zoo.GraphSpec("first_block_requantized_residual")
+    b = zoo.Builder(g, 0xE5F1, per_channel=True, w_exp_range=None)
+    x = b.input("input", [1, 14, 14, 32], -5)
+    cur = x
+    for i in range(2):
+        h = b.conv(cur, 192, k=1, relu=True, name="b%d_expand" % i)
+        h = b.conv(h, None, k=3, depthwise=True, relu=True, name="b%d_dw" % i)
+        p = b.conv(h, 32, k=1, out_exp=-4, name="b%d_project" % i)
+        cur = b.add(cur, p, name="b%d_add" % i)  # the first operand is at -5: requantized to -4 in front of the Add
+    b.output(cur)
+    assert sum(1 for n in g.nodes if n["op_type"] == "RequantizeLinear") == 1
+    mdl, want, _ = _run_config(g, 3, 47)
+    np.testing.assert_array_equal(mdl.get_tensor(g.outputs[0]), want[g.outputs[0]])
+    assert mdl.module_count() == 2
+    mdl.close()
+
+
 def test_channel_slices_every_case(oracle):
     """Split outputs left inside the Split's input and Concat inputs written in place, case by case: which
     tensors become slices (by their pitch), every tensor against the oracle, twice (the slices must survive a

@@ -88,3 +88,46 @@ def test_staged_block_without_expand_and_the_size_limit(oracle):
         m.mbconv_s8(big, dev(expand), dev(dwb), dev(projb), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), (True, True, False),
                     out=torch.empty((80, 56, 56, 24), dtype=torch.int8, device="cuda"), staged=True)
     assert "ESPDL_HIP_MBCONV_STAGED_MAX_BYTES" in str(err.value)
+
+
+def test_staged_block_allocates_nothing_and_replays_under_a_captured_graph(oracle):
+    """Free device memory is the same before and after staged calls, and the entry point can be recorded into a
+    HIP graph once it has been called (or initialised) outside capture: three replays with new inputs in
+    between, each compared with the eager result of the single-launch entry point."""
+    import torch
+    m = espdl()
+    rng = np.random.default_rng(0x57A6EF)
+    dev = lambda t: None if t is None else tuple(to_dev(a) for a in t)  # noqa: E731
+    n, h, w, cin, ce, cout = 4, 28, 28, 32, 192, 32
+    x, expand, dw, proj = _block(rng, n, h, w, cin, ce, cout)
+    assert m.lib().espdl_hip_mbconv_s8_staged_init() == 0
+    geom = ((3, 3), (1, 1), (1, 1), (1, 1, 1, 1), (True, True, False))
+    xd, ed, dd, pd = to_dev(x), dev(expand), dev(dw), dev(proj)
+    res = to_dev(rng_int8(rng, (n, h, w, cout)))
+    out = torch.empty((n, h, w, cout), dtype=torch.int8, device="cuda")
+    announce("mbconv_s8_staged warm call, then free-memory check")
+    m.mbconv_s8(xd, ed, dd, pd, *geom, residual=res, out=out, staged=True)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        m.mbconv_s8(xd, ed, dd, pd, *geom, residual=res, out=out, staged=True)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    # capture on a side stream, replay with new inputs
+    announce("mbconv_s8_staged under a captured graph")
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.graph(graph, stream=side):
+        m.mbconv_s8(xd, ed, dd, pd, *geom, residual=res, out=out, staged=True, stream=side.cuda_stream)
+    for rep in range(3):
+        x2 = rng_int8(rng, (n, h, w, cin))
+        xd.copy_(torch.from_numpy(x2))
+        out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = m.mbconv_s8(xd, ed, dd, pd, *geom, residual=res)
+        np.testing.assert_array_equal(to_host(out), to_host(eager), err_msg="replay %d" % rep)
+        want = _oracle_block(oracle, x2, expand, dw, proj, (1, 1), (1, 1, 1, 1), to_host(res))
+        np.testing.assert_array_equal(to_host(out), want, err_msg="replay %d vs oracle" % rep)
