@@ -936,6 +936,18 @@ int espdl_hip_mbconv_s8_supported(const espdl_hip_mbconv_desc *desc)
     return kind;
 }
 
+// Blocks on large images go to the one-wavefront-per-tile kernel, small ones to the workgroup-per-tile kernel -
+// unless only the former has a guard-free build for the shape (a third of the time of a guarded one).
+static bool wave_before_group(const espdl::MbconvParams &p)
+{
+    if (!espdl::mbconv_s8_wave_supports(p))
+        return false;
+    if (p.in_h >= 28)
+        return true;
+    return espdl::mbconv_s8_wave_has_fast_build(p) &&
+        !(espdl::mbconv_s8_group_supports(p) && espdl::mbconv_s8_group_has_fast_build(p));
+}
+
 static int mbconv_kernel_choice(const espdl_hip_mbconv_desc *desc)
 {
     espdl::MbconvParams p = {};
@@ -960,7 +972,7 @@ static int mbconv_kernel_choice(const espdl_hip_mbconv_desc *desc)
     }
     if (desc->has_expand && !pointwise_expand(p))
         return espdl::mbconv_s8_wave_supports(p) ? 4 : 0;
-    if (desc->has_expand && p.in_h >= 28 && espdl::mbconv_s8_wave_supports(p))
+    if (desc->has_expand && wave_before_group(p))
         return 4;
     if (desc->has_expand && espdl::mbconv_s8_group_supports(p))
         return 5;
@@ -1046,7 +1058,7 @@ int espdl_hip_mbconv_s8(const espdl_hip_mbconv_desc *desc, const int8_t *in, con
         return device_status(espdl::launch_mbconv_s8_wave(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
                              "mbconv_s8_wave");
     }
-    if (desc->has_expand && !(p.in_h >= 28 && espdl::mbconv_s8_wave_supports(p)) && espdl::mbconv_s8_group_supports(p))
+    if (desc->has_expand && !wave_before_group(p) && espdl::mbconv_s8_group_supports(p))
         return device_status(espdl::launch_mbconv_s8_group(p, cu_count_cached(), reinterpret_cast<hipStream_t>(stream)),
                              "mbconv_s8_group");
     if (desc->has_expand && espdl::mbconv_s8_wave_supports(p))

@@ -417,6 +417,9 @@ struct GroupPlan {
 constexpr int kGroupPtMax = 8;
 constexpr size_t kGroupLdsMax = 156 * 1024;
 
+// Whether a guard-free build exists for a plan (defined behind the builds).
+bool group_plan_has_exact_build(const GroupPlan &plan);
+
 GroupPlan group_plan(const MbconvParams &p)
 {
     GroupPlan plan;
@@ -431,65 +434,81 @@ GroupPlan group_plan(const MbconvParams &p)
         (long long)p.out_c * p.exp_c >= (1ll << 31))
         return plan;
     const int s = p.stride_h;
-    GroupArgs a = {};
-    a.p = p;
-    a.tw = p.out_w;
-    a.pw = (a.tw - 1) * s + 3;
-    a.twp = p.out_w <= 8 ? 8 : 16;
-    a.kse = (p.in_c + 63) / 64;
-    a.n_sub = p.exp_c / 16;
-    a.rt = (p.out_c + 15) / 16;
-    // Pixel pitch of the depthwise result: twice an odd number of 16-byte units.  A 16-byte-per-lane LDS read is
-    // served in groups of 8 consecutive pixels x 2 neighbouring 16-byte quarters; with such a pitch the 16 pieces
-    // of a group fall into 16 different bank sets (an odd number of units, the earlier choice, leaves half of the
-    // project stage's operand-B reads in two passes).  The 4-byte stores of the depthwise stage then take two
-    // passes, but the project stage reads every piece once per wavefront: eight times as many LDS cycles.
-    a.ds = p.exp_c + 16;
-    while ((a.ds / 16) % 4 != 2)
-        a.ds += 16;
-    // rows per tile: as many as fit the register and LDS budgets (fewer tiles, less halo to expand)
-    a.th = 0;
-    for (int th = 1; th <= std::min(kGroupPtMax - 1, p.out_h); th++) {
-        const int ph = (th - 1) * s + 3;
-        const int n_xpt = (ph * a.pw + 15) / 16;
-        if (n_xpt > 9)
-            break;
-        const int npt = (th * a.twp + 15) / 16;
-        if (npt > kMaxT)
-            break;
-        const size_t exp_bytes = (size_t)((ph * a.pw + 48 + 15) & ~15) * 16;
-        const size_t lds = (size_t)p.exp_c * 24 + (size_t)a.rt * 16 * 12 + kStageVoteBytes + kGroupWaves * std::max(exp_bytes, (size_t)((n_xpt + 3) & ~3) * 256) +
-            (size_t)npt * 16 * a.ds + 64;
-        if (lds > kGroupLdsMax)
-            break;
-        a.th = th;
+    // The tile a workgroup takes is the whole width and as many rows as fit.  The guard-free builds are made for
+    // widths of 14 (7 at depthwise stride 2 and for images up to 7 wide) and 7 rows (4 at stride 2): a narrower
+    // or lower image is first tried rounded up to that tile - the columns and rows that do not exist load as
+    // padding and their stores are dropped - and keeps the rounded plan when a guard-free build takes it (a third
+    // of the time of a guarded build, which more than pays for the idle part of the tile).
+    const int tw_class = (p.out_w <= 7) ? 7 : (p.out_w <= 14 ? 14 : p.out_w);
+    const int th_class = s == 1 ? 7 : 4;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        const bool rounded = attempt == 0;
+        if (rounded && tw_class == p.out_w && th_class <= p.out_h)
+            continue; // nothing to round: the natural plan below is the same or better
+        GroupArgs a = {};
+        a.p = p;
+        a.tw = rounded ? tw_class : p.out_w;
+        a.pw = (a.tw - 1) * s + 3;
+        a.twp = a.tw <= 8 ? 8 : 16;
+        a.kse = (p.in_c + 63) / 64;
+        a.n_sub = p.exp_c / 16;
+        a.rt = (p.out_c + 15) / 16;
+        // Pixel pitch of the depthwise result: twice an odd number of 16-byte units.  A 16-byte-per-lane LDS read is
+        // served in groups of 8 consecutive pixels x 2 neighbouring 16-byte quarters; with such a pitch the 16 pieces
+        // of a group fall into 16 different bank sets (an odd number of units, the earlier choice, leaves half of the
+        // project stage's operand-B reads in two passes).  The 4-byte stores of the depthwise stage then take two
+        // passes, but the project stage reads every piece once per wavefront: eight times as many LDS cycles.
+        a.ds = p.exp_c + 16;
+        while ((a.ds / 16) % 4 != 2)
+            a.ds += 16;
+        // rows per tile: as many as fit the register and LDS budgets (fewer tiles, less halo to expand)
+        a.th = 0;
+        const int th_max = rounded ? th_class : std::min(kGroupPtMax - 1, p.out_h);
+        for (int th = rounded ? th_class : 1; th <= th_max; th++) {
+            const int ph = (th - 1) * s + 3;
+            const int n_xpt = (ph * a.pw + 15) / 16;
+            if (n_xpt > 9)
+                break;
+            const int npt = (th * a.twp + 15) / 16;
+            if (npt > kMaxT)
+                break;
+            const size_t exp_bytes = (size_t)((ph * a.pw + 48 + 15) & ~15) * 16;
+            const size_t lds = (size_t)p.exp_c * 24 + (size_t)a.rt * 16 * 12 + kStageVoteBytes + kGroupWaves * std::max(exp_bytes, (size_t)((n_xpt + 3) & ~3) * 256) +
+                (size_t)npt * 16 * a.ds + 64;
+            if (lds > kGroupLdsMax)
+                break;
+            a.th = th;
+        }
+        if (a.th == 0)
+            continue;
+        a.ph = (a.th - 1) * s + 3;
+        a.n_xpt = (a.ph * a.pw + 15) / 16;
+        a.npt = (a.th * a.twp + 15) / 16;
+        a.tiles_y = (p.out_h + a.th - 1) / a.th;
+        a.exp_bytes = (int)std::max((size_t)((a.ph * a.pw + 48 + 15) & ~15) * 16, (size_t)((a.n_xpt + 3) & ~3) * 256);
+        a.off_tab = 0;
+        a.off_exp = p.exp_c * 24 + a.rt * 16 * 12 + kStageVoteBytes; // expand, depthwise and project tables, vote words
+        a.off_dw = a.off_exp + kGroupWaves * a.exp_bytes;
+        plan.lds = (size_t)a.off_dw + (size_t)a.npt * 16 * a.ds + 64; // k steps read whole 64-byte pieces
+        // phase-2 grid: a row tile of filters belongs to one wavefront where there are at least eight of them
+        // (operand A comes from global memory: loading it once per workgroup matters more than an even share);
+        // with fewer row tiles 8 / rt wavefronts share one and split the pixel tiles
+        if (a.rt >= kGroupWaves) {
+            a.wr = kGroupWaves;
+            a.wp = 1;
+        } else {
+            a.wr = a.rt;
+            a.wp = kGroupWaves / a.rt;
+        }
+        a.nt = (a.npt + a.wp - 1) / a.wp;
+        a.fd_pw = make_fastdiv((unsigned)a.pw);
+        a.fd_tiles_y = make_fastdiv((unsigned)a.tiles_y);
+        plan.a = a;
+        plan.ok = true;
+        if (!rounded || group_plan_has_exact_build(plan))
+            return plan;
+        plan.ok = false; // the rounded tile has no guard-free build: take the natural one
     }
-    if (a.th == 0)
-        return plan;
-    a.ph = (a.th - 1) * s + 3;
-    a.n_xpt = (a.ph * a.pw + 15) / 16;
-    a.npt = (a.th * a.twp + 15) / 16;
-    a.tiles_y = (p.out_h + a.th - 1) / a.th;
-    a.exp_bytes = (int)std::max((size_t)((a.ph * a.pw + 48 + 15) & ~15) * 16, (size_t)((a.n_xpt + 3) & ~3) * 256);
-    a.off_tab = 0;
-    a.off_exp = p.exp_c * 24 + a.rt * 16 * 12 + kStageVoteBytes; // expand, depthwise and project tables, vote words
-    a.off_dw = a.off_exp + kGroupWaves * a.exp_bytes;
-    plan.lds = (size_t)a.off_dw + (size_t)a.npt * 16 * a.ds + 64; // k steps read whole 64-byte pieces
-    // phase-2 grid: a row tile of filters belongs to one wavefront where there are at least eight of them
-    // (operand A comes from global memory: loading it once per workgroup matters more than an even share);
-    // with fewer row tiles 8 / rt wavefronts share one and split the pixel tiles
-    if (a.rt >= kGroupWaves) {
-        a.wr = kGroupWaves;
-        a.wp = 1;
-    } else {
-        a.wr = a.rt;
-        a.wp = kGroupWaves / a.rt;
-    }
-    a.nt = (a.npt + a.wp - 1) / a.wp;
-    a.fd_pw = make_fastdiv((unsigned)a.pw);
-    a.fd_tiles_y = make_fastdiv((unsigned)a.tiles_y);
-    plan.a = a;
-    plan.ok = true;
     return plan;
 }
 
@@ -544,6 +563,13 @@ bool launch_group_exact(const GroupPlan &plan, hipStream_t stream, bool dry, hip
     ESPDL_GROUP_EXACT(9, 2, 4, 2, 0, 0);
 #undef ESPDL_GROUP_EXACT
     return false;
+}
+
+bool group_plan_has_exact_build(const GroupPlan &plan)
+{
+    hipError_t err = hipSuccess;
+    return plan.a.p.half_even ? launch_group_exact<true>(plan, nullptr, true, &err)
+                              : launch_group_exact<false>(plan, nullptr, true, &err);
 }
 
 } // namespace

@@ -609,14 +609,11 @@ WavePlan wave_plan(const MbconvParams &p)
     const int s = p.stride_h;
     WaveArgs a = {};
     a.p = p;
-    // columns: the fewest column tiles, then the narrowest tile that gives them (less halo to expand)
-    // (an expand stage with a window at depthwise stride 1: patches of exactly 16 columns, where the patch
-    // column of a lane does not change from pixel tile to pixel tile and its window address costs one addition)
-    const int tw_max = (rowconv && s == 1 && p.out_w > 14) ? 14 : 16;
-    const int n_cols = (p.out_w + tw_max - 1) / tw_max;
-    a.tw = (rowconv && tw_max == 14) ? 14 : (p.out_w + n_cols - 1) / n_cols;
-    a.pw = (a.tw - 1) * s + 3;
-    a.tiles_x = n_cols;
+    // columns: the fewest column tiles and the narrowest tile that gives them (less halo to expand), or tiles of
+    // 14 columns, the width every guard-free build is made for (patches of 16 columns at depthwise stride 1,
+    // where the patch column of a lane does not change from pixel tile to pixel tile, and of 29 at stride 2).
+    // A plan rounded up to that width computes columns that do not exist (their loads are masked, their stores
+    // dropped) and still takes a third of the time of a guarded build.
     // rows: cheapest total of expand tiles (x 1.5: MFMA + the longer epilogue) and depthwise MFMAs.  A launch
     // that does not fill the device once (two resident workgroups per compute unit) takes one tile's time
     // whatever its tile count, so there a lower tile that brings more workgroups wins.  Heights whose plan has a
@@ -629,28 +626,40 @@ WavePlan wave_plan(const MbconvParams &p)
     a.x_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.in) & 15) == 0) ? 1 : 0;
     a.we_vec16 = (p.in_c % 16 == 0 && (reinterpret_cast<uintptr_t>(p.w_expand) & 15) == 0) ? 1 : 0;
     double best = 1e30;
-    int best_th = 0;
+    int best_th = 0, best_tw = 0;
     bool best_exact = false;
-    for (int th = 1; th <= kPtMax; th++) {
-        a.th = th;
-        a.ph = (th - 1) * s + 3;
-        a.n_xpt = (a.ph * a.pw + 15) / 16;
-        if (a.n_xpt > nxpt_limit)
-            break;
-        a.tiles_y = (p.out_h + th - 1) / th;
-        const bool exact = wave_plan_has_exact_build(a);
-        const double tile_cost = 1.5 * a.n_xpt + 3.0 * th + 2.0;
-        const double groups = std::ceil((double)std::max(1, p.batch) * a.tiles_y * a.tiles_x / kWavesPerGroup);
-        const double rounds = groups / slots;
-        const double cost = tile_cost * std::max(1.0, rounds);
-        if ((exact && !best_exact) || (exact == best_exact && cost < best)) {
-            best = cost;
-            best_th = th;
-            best_exact = exact;
+    const int n_cols16 = (p.out_w + 15) / 16;
+    const int tw_narrow = (rowconv && s == 1 && p.out_w > 14) ? 14 : (p.out_w + n_cols16 - 1) / n_cols16;
+    const int tw_candidates[2] = {tw_narrow, 14};
+    for (int ci = 0; ci < (tw_narrow == 14 ? 1 : 2); ci++) {
+        a.tw = tw_candidates[ci];
+        a.pw = (a.tw - 1) * s + 3;
+        a.tiles_x = (p.out_w + a.tw - 1) / a.tw;
+        for (int th = 1; th <= kPtMax; th++) {
+            a.th = th;
+            a.ph = (th - 1) * s + 3;
+            a.n_xpt = (a.ph * a.pw + 15) / 16;
+            if (a.n_xpt > nxpt_limit)
+                break;
+            a.tiles_y = (p.out_h + th - 1) / th;
+            const bool exact = wave_plan_has_exact_build(a);
+            const double tile_cost = 1.5 * a.n_xpt + 3.0 * th + 2.0;
+            const double groups = std::ceil((double)std::max(1, p.batch) * a.tiles_y * a.tiles_x / kWavesPerGroup);
+            const double rounds = groups / slots;
+            const double cost = tile_cost * std::max(1.0, rounds);
+            if ((exact && !best_exact) || (exact == best_exact && cost < best)) {
+                best = cost;
+                best_th = th;
+                best_tw = a.tw;
+                best_exact = exact;
+            }
         }
     }
     if (best_th == 0)
         return plan;
+    a.tw = best_tw;
+    a.pw = (a.tw - 1) * s + 3;
+    a.tiles_x = (p.out_w + a.tw - 1) / a.tw;
     a.th = best_th;
     a.ph = (a.th - 1) * s + 3;
     a.n_xpt = (a.ph * a.pw + 15) / 16;

@@ -815,7 +815,7 @@ def test_mbconv_s8_clip_is_refused_where_not_covered():
     ESPDL_HIP_ENOTSUP when a Clip sits between the stages."""
     m = espdl()
     import torch
-    for shape, ce, cout, rm in (((1, 14, 14, 96), 576, 96, m.capi.ROUND_HALF_UP), ((1, 50, 50, 24), 144, 24, m.capi.ROUND_HALF_UP),
+    for shape, ce, cout, rm in (((1, 14, 14, 96), 576, 96, m.capi.ROUND_HALF_UP), ((1, 50, 50, 24), 144, 40, m.capi.ROUND_HALF_UP),
                                 ((1, 56, 56, 24), 144, 24, m.capi.ROUND_HALF_EVEN)):
         n, h, w, c = shape
         d = m.capi.MbconvDesc(n, h, w, c, ce, cout, 1, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0, rm, 1, 1, 1)
@@ -937,6 +937,20 @@ GUARD_FREE_RAGGED = [
     ("group_14x14_96_576_48_s2", (70, 14, 14, 96), 576, 48, 2, False, False, 5),
     ("group_7x7_160_960_64_s1", (130, 7, 7, 160), 960, 64, 1, False, False, 5),
     ("group_7x7_160_960_96_s1_halfeven", (130, 7, 7, 160), 960, 96, 1, False, True, 5),
+    # image sizes of MobileNetV2 at 192 and 160 pixels and a 50 x 50 block: tile plans rounded up to the widths
+    # and heights the guard-free builds are made for (14 or 7 columns, 8 / 7 / 4 rows)
+    ("wave_96x96_16_96_24_s2", (8, 96, 96, 16), 96, 24, 2, False, False, 4),
+    ("wave_48x48_24_144_24_s1_res", (12, 48, 48, 24), 144, 24, 1, True, False, 4),
+    ("wave_50x50_24_144_24_s1_res", (12, 50, 50, 24), 144, 24, 1, True, True, 4),
+    ("wave_40x40_24_144_32_s2", (12, 40, 40, 24), 144, 32, 2, False, False, 4),
+    ("wave_24x24_32_192_32_s1_res", (30, 24, 24, 32), 192, 32, 1, True, False, 4),
+    ("wave_20x20_32_192_64_s2", (30, 20, 20, 32), 192, 64, 2, False, False, 4),
+    ("group_12x12_64_384_64_s1_res", (40, 12, 12, 64), 384, 64, 1, True, False, 5),
+    ("group_10x10_96_576_96_s1_res_halfeven", (40, 10, 10, 96), 576, 96, 1, True, True, 5),
+    ("group_12x12_96_576_160_s2", (40, 12, 12, 96), 576, 160, 2, False, False, 5),
+    ("group_10x10_96_576_160_s2", (40, 10, 10, 96), 576, 160, 2, False, False, 5),
+    ("group_6x6_160_960_160_s1_res", (60, 6, 6, 160), 960, 160, 1, True, False, 5),
+    ("group_5x5_160_960_320_s1", (60, 5, 5, 160), 960, 320, 1, False, False, 5),
 ]
 
 
@@ -1095,7 +1109,8 @@ def _block_desc(m, batch, hw, cin, ce, cout, stride, half_even=False):
 def test_mbconv_s8_preferred_follows_the_fast_builds():
     """dl::Model fuses a block where espdl_hip_mbconv_s8_preferred says so: yes for MobileNetV2's block shapes
     in both rounding modes, at a batch that fills the device and at a small one (the tile plan keeps the height
-    that has a guard-free build); no for a shape that only the guarded builds take (they cover it, but the
+    that has a guard-free build), and for the same blocks at other image sizes (their tiles are rounded up to the
+    ones the builds are made for); no for a shape that only the guarded builds take (they cover it, but the
     separate launches are as fast)."""
     announce("mbconv_s8_preferred")
     m = espdl()
@@ -1112,7 +1127,17 @@ def test_mbconv_s8_preferred_follows_the_fast_builds():
             assert pref(d) == 1, (hw, cin, ce, cout, stride, he)
         for small in (1, 4, 64):
             assert pref(_block_desc(m, small, hw, cin, ce, cout, stride)) == 1, (small, hw, cin, ce, cout, stride)
-    odd = _block_desc(m, 256, 50, 24, 144, 24, 1)  # 50 x 50: a tile plan without a guard-free build
+    # other image sizes are rounded up to the tiles the guard-free builds are made for: a 50 x 50 block, and the
+    # blocks of MobileNetV2 at 192 and 160 pixels
+    for hw, cin, ce, cout, stride, want_kind in [(50, 24, 144, 24, 1, 4), (96, 16, 96, 24, 2, 4), (48, 24, 144, 24, 1, 4),
+                                                 (48, 24, 144, 32, 2, 4), (24, 32, 192, 32, 1, 4), (24, 32, 192, 64, 2, 4),
+                                                 (12, 64, 384, 64, 1, 5), (12, 96, 576, 96, 1, 5), (12, 96, 576, 160, 2, 5),
+                                                 (6, 160, 960, 160, 1, 5), (80, 16, 96, 24, 2, 4), (40, 24, 144, 24, 1, 4),
+                                                 (20, 32, 192, 32, 1, 4), (10, 64, 384, 96, 1, 5), (5, 160, 960, 320, 1, 5)]:
+        for he in (False, True):
+            d = _block_desc(m, 256, hw, cin, ce, cout, stride, he)
+            assert kind(d) == want_kind and pref(d) == 1, (hw, cin, ce, cout, stride, he)
+    odd = _block_desc(m, 256, 50, 24, 144, 40, 1)  # three project row tiles: no guard-free build has them
     assert kind(odd) == 4 and pref(odd) == 0
 
 
