@@ -89,6 +89,7 @@ def lib():
         L.espdl_hip_mul_s8.restype = ctypes.c_int
         L.espdl_hip_global_avg_pool_s8.argtypes = [vp, i32, i32, i32, i32, i32, i32, vp, vp]
         L.espdl_hip_requantize_s8.argtypes = [vp, i64, i32, i32, vp, vp]
+        L.espdl_hip_split.argtypes = [vp, i64, i32, ctypes.POINTER(vp), ctypes.POINTER(i64), i64, vp]
         L.espdl_hip_requantize_s8_rows.argtypes = [vp, i64, vp, i64, i64, i64, i32, i32, vp]
         L.espdl_hip_requantize.argtypes = [vp, i32, i64, i32, i32, vp, i32, vp]
         f32 = ctypes.c_float
@@ -383,24 +384,26 @@ def concat(tensors, axis, out=None, stream=None):
     return out
 
 
-def split(x, axis, sizes, stream=None):
-    """Consecutive pieces of the given sizes along axis, each a new contiguous tensor."""
+def split(x, axis, sizes, stream=None, outs=None):
+    """Consecutive pieces of the given sizes along axis, each a new contiguous tensor (or the tensors of `outs`;
+    a None entry there skips that piece), in one pass over x (espdl_hip_split)."""
     import torch
     axis = axis + x.dim() if axis < 0 else axis
     esize = x.element_size()
     num_slices, slice_size = _prod(x.shape[:axis]), _prod(x.shape[axis + 1:])
-    outs, start = [], 0
-    for sz in sizes:
+    results = []
+    for j, sz in enumerate(sizes):
         shape = list(x.shape)
         shape[axis] = int(sz)
-        out = torch.empty(shape, dtype=x.dtype, device=x.device)
-        row = slice_size * int(sz) * esize
-        _check(lib().espdl_hip_copy_rows(ctypes.c_void_p(x.data_ptr() + start * slice_size * esize),
-                                         slice_size * int(x.shape[axis]) * esize, _p(out), row, row, num_slices,
-                                         _stream(stream)))
-        outs.append(out)
-        start += int(sz)
-    return outs
+        if outs is not None:
+            results.append(outs[j])
+        else:
+            results.append(torch.empty(shape, dtype=x.dtype, device=x.device))
+    n = len(sizes)
+    ptrs = (ctypes.c_void_p * n)(*[None if t is None else t.data_ptr() for t in results])
+    sizes_b = (ctypes.c_int64 * n)(*[slice_size * int(sz) * esize for sz in sizes])
+    _check(lib().espdl_hip_split(_p(x), slice_size * int(x.shape[axis]) * esize, n, ptrs, sizes_b, num_slices, _stream(stream)))
+    return results
 
 
 def transpose(x, perm=None, out=None, stream=None):

@@ -489,6 +489,31 @@ int espdl_hip_copy_rows(const void *src, int64_t src_pitch, void *dst, int64_t d
                          "copy_rows");
 }
 
+int espdl_hip_split(const void *in, int64_t in_pitch, int32_t n_outputs, void *const *outputs, const int64_t *copy_bytes,
+                    int64_t rows, void *stream)
+{
+    if (n_outputs < 1 || outputs == nullptr || copy_bytes == nullptr || rows < 0 || in_pitch < 0)
+        return fail(ESPDL_HIP_EINVAL, "split needs at least one output, sizes and a row count >= 0");
+    long long total = 0;
+    std::vector<long long> bytes((size_t)n_outputs);
+    for (int j = 0; j < n_outputs; j++) {
+        if (copy_bytes[j] < 0)
+            return fail(ESPDL_HIP_EINVAL, "negative size of output %d", j);
+        bytes[(size_t)j] = copy_bytes[j];
+        total += copy_bytes[j];
+    }
+    if (rows == 0 || total == 0)
+        return ESPDL_HIP_OK;
+    if (in == nullptr)
+        return fail(ESPDL_HIP_EINVAL, "in must not be NULL");
+    if (rows > 1 && in_pitch < total)
+        return fail(ESPDL_HIP_EINVAL, "the input pitch %lld is smaller than the pieces together (%lld)", (long long)in_pitch,
+                    total);
+    return device_status(espdl::launch_split(in, in_pitch, n_outputs, outputs, bytes.data(), rows, cu_count_cached(),
+                                             reinterpret_cast<hipStream_t>(stream)),
+                         "split");
+}
+
 int espdl_hip_transpose(const void *in, const int32_t *shape, int32_t dims, const int32_t *perm, int32_t n_perm,
                         int32_t elem_size, void *out, void *stream)
 {

@@ -188,6 +188,10 @@ hipError_t launch_requantize_any(const void *in, int in_bits, int64_t size, int 
                                  int out_bits, hipStream_t stream);
 
 // Data-movement operators (layout_ops.hip).
+// Split: `rows` runs of the input, in_pitch bytes apart, cut into n_outputs consecutive pieces of copy_bytes[j] bytes;
+// piece j of run r goes to outputs[j] + r * copy_bytes[j] (a null output is skipped).  One pass in input order.
+hipError_t launch_split(const void *in, long long in_pitch, int n_outputs, void *const *outputs, const long long *copy_bytes,
+                        long long rows, int cu_count, hipStream_t stream);
 hipError_t launch_copy_rows(const void *src, long long src_pitch, void *dst, long long dst_pitch, long long row_bytes,
                             long long rows, int cu_count, hipStream_t stream);
 hipError_t launch_concat(int n_inputs, const void *const *inputs, const long long *copy_bytes, long long loop_times,

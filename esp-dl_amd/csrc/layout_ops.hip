@@ -519,7 +519,94 @@ __global__ __launch_bounds__(kBlock) void concat_rows_kernel(const ConcatArgs a)
                 reinterpret_cast<v4i *>(a.dst)[i0 + j * stride] = v[j];
     }
 }
+
+// Split walked in input order: the mirror image.  Piece i of the input (row r, column c) goes to the output the
+// column belongs to; every load of a wavefront is a run of whole cache lines of the input, which one pass per
+// output reads as half lines twice (measured on 128 -> 64 + 64 channels: 0.44 of the HBM rate per output).
+struct SplitArgs {
+    char *dst[kMaxSeg];
+    unsigned first[kMaxSeg + 1]; // first input piece (of a row) of output j; first[n] = pieces per row
+    unsigned pieces[kMaxSeg];    // pieces per row of output j
+    int n;
+    const char *src;
+    long long src_pitch; // bytes from row to row of the input
+    long long rows;
+    FastDiv per_row;
+};
+
+__global__ __launch_bounds__(kBlock) void split_rows_kernel(const SplitArgs a)
+{
+    const long long total = a.rows * a.per_row.d; // below 2^31 (checked on the host)
+    const long long stride = (long long)gridDim.x * kBlock;
+    for (long long i0 = (long long)blockIdx.x * kBlock + threadIdx.x; i0 < total; i0 += 4 * stride) {
+        v4i v[4];
+        unsigned rr[4], cc[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const long long i = i0 + j * stride < total ? i0 + j * stride : i0;
+            rr[j] = fastdiv((unsigned)i, a.per_row);
+            cc[j] = (unsigned)i - rr[j] * a.per_row.d;
+            v[j] = *reinterpret_cast<const v4i *>(a.src + (long long)rr[j] * a.src_pitch + (long long)cc[j] * 16);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            if (i0 + j * stride >= total)
+                continue;
+            int seg = 0;
+#pragma unroll
+            for (int k = 1; k < kMaxSeg; k++)
+                seg += (k < a.n && cc[j] >= a.first[k]) ? 1 : 0;
+            if (a.dst[seg] != nullptr) // an output that already lies in the input is not written
+                *reinterpret_cast<v4i *>(a.dst[seg] + ((long long)rr[j] * a.pieces[seg] + (cc[j] - a.first[seg])) * 16) = v[j];
+        }
+    }
+}
 } // namespace
+
+hipError_t launch_split(const void *in, long long in_pitch, int n_outputs, void *const *outputs, const long long *copy_bytes,
+                        long long rows, int cu_count, hipStream_t stream)
+{
+    long long total = 0;
+    for (int j = 0; j < n_outputs; j++)
+        total += copy_bytes[j];
+    if (rows <= 0 || total <= 0)
+        return hipSuccess;
+    // input-order form: up to kMaxSeg outputs, everything in whole aligned 16-byte pieces
+    bool ok = n_outputs <= kMaxSeg && (reinterpret_cast<uintptr_t>(in) & 15) == 0 && (in_pitch & 15) == 0 &&
+        rows * (total / 16) <= 0x7fffffffll;
+    SplitArgs a = {};
+    unsigned first = 0;
+    for (int j = 0; ok && j < n_outputs; j++) {
+        ok = (copy_bytes[j] & 15) == 0 && copy_bytes[j] > 0 && (reinterpret_cast<uintptr_t>(outputs[j]) & 15) == 0;
+        a.dst[j] = static_cast<char *>(outputs[j]);
+        a.first[j] = first;
+        a.pieces[j] = (unsigned)(copy_bytes[j] / 16);
+        first += a.pieces[j];
+    }
+    if (ok) {
+        for (int k = n_outputs; k <= kMaxSeg; k++)
+            a.first[k] = first;
+        a.n = n_outputs;
+        a.src = static_cast<const char *>(in);
+        a.src_pitch = in_pitch;
+        a.rows = rows;
+        a.per_row = make_fastdiv(first);
+        hipLaunchKernelGGL(split_rows_kernel, dim3(blocks_for(rows * first, cu_count)), dim3(kBlock), 0, stream, a);
+        return hipGetLastError();
+    }
+    // one pass per output
+    long long prefix = 0;
+    for (int j = 0; j < n_outputs; j++) {
+        if (outputs[j] != nullptr && copy_bytes[j] > 0) {
+            const hipError_t e = launch_copy_rows(static_cast<const char *>(in) + prefix, in_pitch, outputs[j], copy_bytes[j],
+                                                  copy_bytes[j], rows, cu_count, stream);
+            if (e != hipSuccess)
+                return e;
+        }
+        prefix += copy_bytes[j];
+    }
+    return hipSuccess;
+}
 
 hipError_t launch_concat(int n_inputs, const void *const *inputs, const long long *copy_bytes, long long loop_times,
                          void *out, int cu_count, hipStream_t stream)

@@ -183,6 +183,9 @@ public:
         // bytes between consecutive runs of the input (a channel slice of a wider tensor has a larger pitch)
         const int64_t in_pitch = input->is_dense() ? slice_size * in_axis * esize : (int64_t)input->channel_pitch * esize;
         int64_t slice_index = 0;
+        std::vector<void *> dsts;
+        std::vector<int64_t> bytes;
+        bool any = false;
         for (size_t i = 0; i < m_outputs_index.size(); i++) {
             TensorBase *output = context->get_tensor(m_outputs_index[i]);
             if (!output || !output->on_device() || output->dtype != input->dtype) {
@@ -190,20 +193,27 @@ public:
                 return;
             }
             const int64_t out_axis = output->shape[m_axis];
-            const int64_t row = slice_size * out_axis * esize;
             const char *src = static_cast<const char *>(input->data) + slice_index * slice_size * esize;
             slice_index += out_axis;
+            bytes.push_back(slice_size * out_axis * esize);
             // an output the model left inside the input is already there
-            if (output->data == src && !output->is_dense() && (int64_t)output->channel_pitch * esize == in_pitch)
+            if (output->data == src && !output->is_dense() && (int64_t)output->channel_pitch * esize == in_pitch) {
+                dsts.push_back(nullptr);
                 continue;
+            }
             if (!output->is_dense()) {
                 DL_LOGE("Split", "%s: output %d is a channel slice of another tensor than the input", name.c_str(), (int)i);
                 return;
             }
-            const int rc = espdl_hip_copy_rows(src, in_pitch, output->data, row, row, num_slices, context->stream);
-            if (rc != ESPDL_HIP_OK)
-                DL_LOGE("Split", "%s: %s", name.c_str(), espdl_hip_last_error());
+            dsts.push_back(output->data);
+            any = true;
         }
+        if (!any)
+            return;
+        const int rc = espdl_hip_split(input->data, in_pitch, (int32_t)dsts.size(), dsts.data(), bytes.data(), num_slices,
+                                       context->stream);
+        if (rc != ESPDL_HIP_OK)
+            DL_LOGE("Split", "%s: %s", name.c_str(), espdl_hip_last_error());
     }
     int get_axis() const { return m_axis; }
     bool reads_channel_slice(int slot) const { return slot == 0; }

@@ -70,7 +70,7 @@ def main():
     # Concat / Split along channels: two halves of 64 channels <-> 128 channels
     cat = torch.empty((n, 64, 64, 128), dtype=torch.int8, device=dev)
     timed("Concat 64 + 64 channels (espdl_hip_concat)", lambda: m.concat([x, out], 3, out=cat), 2 * cat.numel())
-    timed("Split 128 -> 64 + 64 channels (espdl_hip_copy_rows x 2)", lambda: m.split(cat, 3, [64, 64]), 2 * cat.numel())
+    timed("Split 128 -> 64 + 64 channels (espdl_hip_split)", lambda: m.split(cat, 3, [64, 64]), 2 * cat.numel())
     del cat
 
     # MaxPool 5x5 stride 1 (SPPF), Resize nearest x2, on 80 x 80 x 128 images

@@ -193,6 +193,14 @@ int espdl_hip_concat(int32_t n_inputs, const void *const *inputs, const int64_t 
 int espdl_hip_copy_rows(const void *src, int64_t src_pitch, void *dst, int64_t dst_pitch, int64_t row_bytes,
                         int64_t rows, void *stream);
 
+/* All outputs of module::Split (esp-dl/dl/module/include/dl_module_split.hpp:84-152) in one pass over the input:
+ * `rows` runs (num_slices) that lie in_pitch bytes apart are cut into n_outputs consecutive pieces of copy_bytes[j]
+ * bytes (slice_size * out_axis_j * sizeof(T)); piece j of run r goes to outputs[j] + r * copy_bytes[j].  A NULL
+ * output is skipped (a piece the caller reads in place).  `outputs` and `copy_bytes` are host arrays read during
+ * the call. */
+int espdl_hip_split(const void *in, int64_t in_pitch, int32_t n_outputs, void *const *outputs, const int64_t *copy_bytes,
+                    int64_t rows, void *stream);
+
 /* TensorBase::transpose (esp-dl/dl/tensor/src/dl_tensor_base.cpp:722-812): out.shape[i] =
  * shape[perm[i]].  1..8 dims, elem_size 1, 2 or 4 bytes; perm entries may be negative (counted from
  * the end) and n_perm = 0 reverses the dims.  shape and perm are host arrays. */

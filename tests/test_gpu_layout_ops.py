@@ -41,7 +41,8 @@ def test_concat(oracle, case, dtype):
 @pytest.mark.parametrize("dtype", [np.int8, np.int16])
 @pytest.mark.parametrize("shape,axis,sizes", [
     ((2, 20, 20, 128), 3, [64, 64]), ((2, 9, 9, 48), 3, [5, 20, 23]), ((4, 6, 5, 8), 1, [1, 2, 3]),
-    ((5, 3, 3, 4), 0, [2, 3]), ((1, 1, 1, 32), -1, [16, 16]),
+    ((5, 3, 3, 4), 0, [2, 3]), ((1, 1, 1, 32), -1, [16, 16]), ((3, 7, 11, 160), 3, [32, 16, 64, 48]),
+    ((2, 5, 5, 144), 3, [16] * 9), ((3, 4, 64, 16), 1, [1, 3]),
 ])
 def test_split(oracle, shape, axis, sizes, dtype):
     announce(f"split {shape} axis {axis} {sizes} {dtype.__name__}")
@@ -51,6 +52,19 @@ def test_split(oracle, shape, axis, sizes, dtype):
     assert len(got) == len(want)
     for g, w in zip(got, want):
         np.testing.assert_array_equal(to_host(g), w)
+
+
+def test_split_skips_pieces_without_a_destination(oracle):
+    """A NULL output is a piece the caller reads in place: the others are written, nothing else is touched."""
+    import torch
+    announce("split with a skipped piece")
+    m = espdl()
+    x = _rand(np.random.default_rng(30), (2, 6, 7, 96))
+    a = torch.full((2, 6, 7, 32), 55, dtype=torch.int8, device="cuda")
+    c = torch.full((2, 6, 7, 48), 55, dtype=torch.int8, device="cuda")
+    m.split(to_dev(x), 3, [32, 16, 48], outs=[a, None, c])
+    np.testing.assert_array_equal(to_host(a), x[..., :32])
+    np.testing.assert_array_equal(to_host(c), x[..., 48:])
 
 
 @pytest.mark.parametrize("dtype", [np.int8, np.int16, np.int32])
