@@ -244,6 +244,38 @@ __global__ __launch_bounds__(kBlock) void resize_nearest_s8_kernel(const ResizeA
     }
 }
 
+// Exactly 2 x 2 on 16-byte channel vectors: a thread reads one input piece and writes the four output pixels that
+// replicate it (one load instead of four; the value is rescaled once).
+__global__ __launch_bounds__(kBlock) void resize_nearest2x_s8_kernel(const ResizeArgs a)
+{
+    // a.total counts INPUT pieces here: i = ((n * h + y) * w + x) * cv + v
+    for (long long i = (long long)blockIdx.x * kBlock + threadIdx.x; i < a.total; i += (long long)gridDim.x * kBlock) {
+        const unsigned pix = fastdiv((unsigned)i, a.fd_cv);
+        const unsigned v = (unsigned)i - pix * a.fd_cv.d;
+        const unsigned row = fastdiv(pix, a.fd_ow); // fd_ow / fd_oh hold the INPUT width / height in this kernel
+        const unsigned x = pix - row * a.fd_ow.d;
+        const unsigned n = fastdiv(row, a.fd_oh);
+        const unsigned y = row - n * a.fd_oh.d;
+        v4i d = *reinterpret_cast<const v4i *>(a.in + (long long)pix * a.in_pitch + (long long)v * 16);
+        if (a.rshift | a.lshift) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                int o = 0;
+#pragma unroll
+                for (int b = 0; b < 4; b++)
+                    o |= (resize_value((int)(int8_t)(d[k] >> (8 * b)), a.rshift, a.lshift) & 0xff) << (8 * b);
+                d[k] = o;
+            }
+        }
+        int8_t *dst = a.out + (((long long)n * a.out_h + 2 * y) * a.out_w + 2 * x) * a.out_pitch + (long long)v * 16;
+        const long long down = (long long)a.out_w * a.out_pitch;
+        *reinterpret_cast<v4i *>(dst) = d;
+        *reinterpret_cast<v4i *>(dst + a.out_pitch) = d;
+        *reinterpret_cast<v4i *>(dst + down) = d;
+        *reinterpret_cast<v4i *>(dst + down + a.out_pitch) = d;
+    }
+}
+
 struct InsertZerosArgs {
     const char *in;
     char *out;
@@ -821,6 +853,13 @@ hipError_t launch_resize_nearest_s8(const int8_t *in, int batch, int h, int w, i
     if (a.total > 0x7fffffffll) // fastdiv range
         return hipErrorInvalidValue;
     a.fd_cv = make_fastdiv((unsigned)cv);
+    if (a.exact2 && a.vec == 16 && out_h == 2 * h && out_w == 2 * w) {
+        a.total = (long long)batch * h * w * cv;
+        a.fd_ow = make_fastdiv((unsigned)w);
+        a.fd_oh = make_fastdiv((unsigned)h);
+        hipLaunchKernelGGL(resize_nearest2x_s8_kernel, dim3(blocks_for(a.total, cu_count)), dim3(kBlock), 0, stream, a);
+        return hipGetLastError();
+    }
     a.fd_ow = make_fastdiv((unsigned)out_w);
     a.fd_oh = make_fastdiv((unsigned)out_h);
     hipLaunchKernelGGL(resize_nearest_s8_kernel, dim3(blocks_for(a.total, cu_count)), dim3(kBlock), 0, stream, a);
