@@ -19,8 +19,10 @@
 //     reduction axis (tap, channel) in steps of 64: PT + 4 operand reads of 16 bytes per lane from LDS feed
 //     4 * PT matrix instructions, the operands of the next step being read while the current products run.
 // LDS layout of the patch: [row][column phase = column % stride_w][column / stride_w][channels + pad], the
-// pixel pitch an odd number of 16-byte units.  Splitting the columns by phase makes the 16 pixels of a tile
-// neighbours in LDS for every tap also at stride 2, so operand-B reads are conflict-free.  With stride 1
+// pixel pitch twice an odd number of 16-byte units (the pitch at which 16-byte-per-lane reads of 16 neighbouring
+// pixels meet no bank twice).  Splitting the columns by phase makes the 16 pixels of a tile neighbours in LDS for
+// every tap also at stride 2.  (The kernel keeps that strided form, but the planner hands it stride-1 layers
+// only: strided layers re-read little and measured as fast or faster through the direct kernel.)  With stride 1
 // the "pixels" of a tile are 16 consecutive positions of the patch's flattened (row, column) space: a tap is
 // then a constant offset, tiles run across row ends, and only the (k-1)*d positions per row that wrap are
 // wasted instead of the padding of every row to a multiple of 16.

@@ -46,6 +46,21 @@ STEM_CASES = [
     ("s3_1x700_k3s2_oc16", (1, 700, 3), 16, (1, 3), (1, 2), (1, 1), (0, 0, 1, 1), True, True),
 ]
 
+# Pointwise products with at most 128 input channels over enough pixels to fill the device (3 x 80 x 80: the routes
+# the dispatcher takes for many pixels, which the small cases above never reach).  One and two reduction steps,
+# reductions that end inside a step (72, 100, 120), filter counts that are no multiple of 64 / 16 / 4, many filters.
+POINTWISE_MANY_PIXELS = [
+    ("p16_32", (80, 80, 16), 32, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
+    ("p32_64", (80, 80, 32), 64, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("p48_40", (80, 80, 48), 40, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), False, True),
+    ("p64_120", (80, 80, 64), 120, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
+    ("p72_33", (80, 80, 72), 33, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("p96_64", (80, 80, 96), 64, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
+    ("p100_70", (80, 80, 100), 70, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("p120_1100", (80, 80, 120), 1100, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("p128_128", (80, 80, 128), 128, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
+]
+
 # Windowed convolutions whose channel count is a multiple of 16: the kernel that stages the input tile and the
 # filters in LDS.  Strides 1 to 3, dilation, reduction steps that span several taps (16, 32, 48 channels), several
 # groups of 64 filters in one and in several chunks, filter counts that are not a multiple of 64 / 16 / 4, images

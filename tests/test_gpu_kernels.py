@@ -5,7 +5,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
+from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, POINTWISE_MANY_PIXELS, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
 from gpu_util import announce, espdl, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
@@ -124,6 +124,31 @@ def test_conv2d_s8_first_layer(oracle, case, flavour):
         if bias is not None:
             bias = bias.copy()
             bias[::2] = (1 << 30) - 7
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", POINTWISE_MANY_PIXELS, ids=lambda c: c[0])
+@pytest.mark.parametrize("flavour", ["per_tensor", "per_channel", "half_even", "lut", "general_epilogue"])
+def test_conv2d_s8_pointwise_short_reduction(oracle, case, flavour):
+    """Pointwise products over many pixels with at most 128 input channels: both exponent forms, round-half-even,
+    a table in the epilogue, the general shift-and-round form."""
+    announce(f"conv2d_s8 pointwise short reduction {case[0]} {flavour}")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 227, 3, flavour != "per_tensor")
+    kw = {}
+    if flavour == "half_even":
+        kw["half_even"] = True
+    if flavour == "lut":
+        kw["lut"] = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8)
+        relu = False
+    if flavour == "general_epilogue":
+        shift = np.array(shift, dtype=np.int32)
+        shift[::3] = 0
+        shift[1::5] = 33
+        if bias is not None:
+            bias = bias.copy()
+            bias[::2] = (1 << 30) - 7
+    oracle.set_threads(16)
     got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
     np.testing.assert_array_equal(got, want)
 
