@@ -65,6 +65,8 @@ def kernel_family(info, spec_nodes):
         return "depthwise_s8" if node and node["attrs"].get("group", 1) != 1 else "conv2d_s8"
     if info["type"] in ("Flatten", "Squeeze", "Reshape", "Unsqueeze"):
         return "view"
+    if info["type"] in ("Concat", "Split") and info["bytes"] == 0:
+        return "view"  # every piece is a channel slice of the wide tensor: nothing is launched
     return "elementwise_s8"
 
 

@@ -1239,6 +1239,27 @@ std::vector<module_info> Model::get_module_info(int repeats)
             if (t)
                 mi.bytes += (int64_t)t->get_bytes();
         }
+        if (mi.type == "Concat" || mi.type == "Split") {
+            // pieces that already lie in their place inside the wide tensor (channel slices) are not moved:
+            // only the copied pieces count, once read and once written
+            const bool concat = mi.type == "Concat";
+            const auto &wide_ids = concat ? module->m_outputs_index : module->m_inputs_index;
+            const auto &piece_ids = concat ? module->m_inputs_index : module->m_outputs_index;
+            TensorBase *wide = wide_ids.empty() ? nullptr : m_model_context->get_tensor(wide_ids[0]);
+            if (wide && wide->data) {
+                const char *lo = static_cast<const char *>(wide->data);
+                const char *hi = lo + wide->get_bytes();
+                mi.bytes = 0;
+                for (int idx : piece_ids) {
+                    TensorBase *t = m_model_context->get_tensor(idx);
+                    if (!t || !t->data)
+                        continue;
+                    const char *p = static_cast<const char *>(t->data);
+                    if (!(p >= lo && p < hi))
+                        mi.bytes += 2 * (int64_t)t->get_bytes();
+                }
+            }
+        }
         mi.macs = module->get_macs(in_shapes);
         info.push_back(mi);
     }
