@@ -17,7 +17,9 @@
 //     reduction axis = (tap, channel), A[i][(tap, c)] = w[tap][i] if c == i): three MFMAs finish 16
 //     pixels x 16 channels x up to 12 taps, and operand B is one 16-byte LDS read per lane and k
 //     step, at patch offset (pixel) + (tap) + 16 * group.  The vector ALU is left with three adds
-//     and the epilogue per MFMA tile.
+//     and the epilogue per MFMA tile.  Windows of three columns take one k step per window row (slots
+//     kx 0, 1, 2 and 2 again with zero weights): lane groups that read LDS together then address pieces
+//     one pixel pitch apart or the same piece, which is free of bank conflicts at an odd pitch.
 //   * MFMA tiles are taken group-major and split evenly over the four wavefronts; a wavefront
 //     rebuilds operand A and its per-channel constants only when the channel group changes.
 //   * Results go to an LDS copy of the output tile and leave as 16-byte stores of consecutive
@@ -55,6 +57,8 @@ struct DwLdsArgs {
     int8_t *out;
     ConvGeom g;
     int taps;
+    int row3;           // 1: windows of 3 columns and at most 3 rows take one k step per window row (slots kx 0, 1, 2, 2)
+    int ks_used;        // k steps that hold taps
     int th, tw;         // output tile, pixels
     int ph, pw;         // input patch, pixels
     int gc;             // channel groups of 16 per workgroup (divides in_c / 16)
@@ -211,6 +215,22 @@ __device__ __forceinline__ void dw_expand(const DwLdsArgs &a, unsigned char *sme
     }
 }
 
+// Tap of k slot `slot` (k step slot / 4, lane group slot % 4), or -1 for a slot without one; `*twin` is the tap
+// whose patch offset an empty slot reads (its weights are zero).  Lane groups 0 / 1 and 2 / 3 read LDS
+// together: their pieces must lie an odd number of 16-byte units apart or coincide, or the read takes two
+// passes.  With one k step per window row (3-column windows) the pairs are (kx 0, kx 1) and (kx 2, kx 2 again):
+// one pixel pitch apart, and identical.
+__device__ __forceinline__ int dw_slot_tap(const DwLdsArgs &a, int slot, int *twin)
+{
+    if (a.row3) {
+        const int ky = slot >> 2, q = slot & 3;
+        *twin = ky < a.g.k_h ? ky * 3 + min(q, 2) : 0;
+        return (q < 3 && ky < a.g.k_h) ? ky * 3 + q : -1;
+    }
+    *twin = slot < a.taps ? slot : 0;
+    return slot < a.taps ? slot : -1;
+}
+
 template <bool FAST, int USE_LSH, int KS>
 __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *smem, int wave, int lane,
                                            const int (&tapoff)[KS], int floor_pk)
@@ -219,64 +239,25 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
     const int col = lane & 15, quad = lane >> 4;
     const bool relu = g.relu != 0, half_even = g.half_even != 0, has_lut = a.lut != nullptr;
     const int *a_l = reinterpret_cast<const int *>(smem + a.off_a);
-    const int *pixtab = reinterpret_cast<const int *>(smem + a.off_pixtab);
     const int8_t *lut_l = reinterpret_cast<const int8_t *>(smem + a.off_lut);
     const unsigned char *patch = smem + a.off_patch;
     unsigned char *out_l = smem + a.off_out;
+    const int *pixtab = reinterpret_cast<const int *>(smem + a.off_pixtab) + col;
 
-    const int t_end = min((wave + 1) * a.tiles_per_wave, a.gc * a.np);
+    // this wavefront's run of tiles, group-major: [t, t_end) = tiles [p, ...) of group grp, then whole
+    // groups, then the head of a last one.  Everything that steers the walk is wave-uniform.
+    const int npt = a.np;
+    const int t_end = min((wave + 1) * a.tiles_per_wave, a.gc * npt);
     int t = wave * a.tiles_per_wave;
     if (t >= t_end)
         return;
     int grp = (int)fastdiv((unsigned)t, a.fd_np);
-    int p = t - grp * a.np;
+    int p = t - grp * npt;
+    const bool all_k = a.ks_used == KS; // the usual case: no test per k step
 
     const int sel = col >> 2; // dword of the 16-byte operand A vector that holds this row's weight
-    v4i aop[KS], init, ss, ls;
-    auto load_group = [&](int gi) {
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const int d = a_l[(gi * KS + ks) * 64 + lane];
-            aop[ks] = v4i{sel == 0 ? d : 0, sel == 1 ? d : 0, sel == 2 ? d : 0, sel == 3 ? d : 0};
-        }
-        const int ch = 16 * gi + 4 * quad;
-        init = *reinterpret_cast<const v4i *>(smem + a.off_init + 4 * ch);
-        ss = *reinterpret_cast<const v4i *>(smem + a.off_ss + 4 * ch);
-        ls = *reinterpret_cast<const v4i *>(smem + a.off_ls + 4 * ch);
-    };
-    int grp_loaded = -1;
-
-    v4i b[KS];
-    {
-        const int po = pixtab[p * 16 + col] + 16 * grp;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++)
-            b[ks] = *reinterpret_cast<const v4i *>(patch + po + tapoff[ks]);
-    }
     const int out_lane = col * a.cso + 4 * quad;
-    for (; t < t_end; t++) {
-        if (grp != grp_loaded) { // uniform; once per np tiles
-            load_group(grp);
-            grp_loaded = grp;
-        }
-        int p_next = p + 1, grp_next = grp;
-        if (p_next == a.np) {
-            p_next = 0;
-            grp_next = grp + 1;
-        }
-        const int out_off = out_lane + p * 16 * a.cso + 16 * grp;
-        v4i acc = init;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++)
-            if (4 * ks < a.taps)
-                acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], acc, 0, 0, 0);
-        // operand B of the next tile of this wavefront is read while this one is in the matrix pipe
-        if (t + 1 < t_end) {
-            const int po = pixtab[p_next * 16 + col] + 16 * grp_next;
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++)
-                b[ks] = *reinterpret_cast<const v4i *>(patch + po + tapoff[ks]);
-        }
+    auto finish = [&](const v4i &acc, const v4i &ls, const v4i &ss, unsigned char *dst) {
         int word;
         if (FAST) {
             word = pack_fast4<USE_LSH>(acc, ls, ss, floor_pk);
@@ -290,9 +271,55 @@ __device__ __forceinline__ void dw_compute(const DwLdsArgs &a, unsigned char *sm
         if (has_lut)
             word = pack4_s8(lut_l[(int)(int8_t)word + 128], lut_l[(int)(int8_t)(word >> 8) + 128],
                             lut_l[(int)(int8_t)(word >> 16) + 128], lut_l[(word >> 24) + 128]);
-        *reinterpret_cast<int *>(out_l + out_off) = word;
-        p = p_next;
-        grp = grp_next;
+        *reinterpret_cast<int *>(dst) = word;
+    };
+    while (t < t_end) {
+        // constants of the channel group; they are waited for here, outside the tile loop, so that the loop's own
+        // waits count only its operand reads
+        v4i aop[KS], init, ss, ls;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int d = a_l[(grp * KS + ks) * 64 + lane];
+            aop[ks] = v4i{sel == 0 ? d : 0, sel == 1 ? d : 0, sel == 2 ? d : 0, sel == 3 ? d : 0};
+        }
+        const int ch = 16 * grp + 4 * quad;
+        init = *reinterpret_cast<const v4i *>(smem + a.off_init + 4 * ch);
+        ss = *reinterpret_cast<const v4i *>(smem + a.off_ss + 4 * ch);
+        ls = *reinterpret_cast<const v4i *>(smem + a.off_ls + 4 * ch);
+        const int p_end = min(npt, p + (t_end - t)); // uniform
+        const unsigned char *pg = patch + 16 * grp;
+        unsigned char *og = out_l + out_lane + 16 * grp;
+        // operand B one tile ahead, its patch offset two tiles ahead
+        int po = pixtab[p * 16];
+        int po_next = pixtab[min(p + 1, npt - 1) * 16];
+        v4i b[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+            b[ks] = *reinterpret_cast<const v4i *>(pg + po + tapoff[ks]);
+        t += p_end - p;
+        for (; p < p_end; p++) {
+            v4i acc = init;
+            if (all_k) {
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++)
+                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], acc, 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int ks = 0; ks < KS; ks++)
+                    if (ks < a.ks_used)
+                        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(aop[ks], b[ks], acc, 0, 0, 0);
+            }
+            // the next tile's operand B is read while this one is in the matrix pipe and the epilogue (past the
+            // last tile of the run the reads repeat a valid offset and are dropped)
+            po = po_next;
+            po_next = pixtab[min(p + 2, npt - 1) * 16];
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++)
+                b[ks] = *reinterpret_cast<const v4i *>(pg + po + tapoff[ks]);
+            finish(acc, ls, ss, og + p * 16 * a.cso);
+        }
+        p = 0;
+        grp++;
     }
 }
 
@@ -303,7 +330,8 @@ __global__ __launch_bounds__(kThreads, KS > kKs ? 2 : 4) void depthwise_s8_lds_k
 {
     extern __shared__ __align__(16) unsigned char smem[];
     const ConvGeom &g = a.g;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // the same in every lane: loops over it are scalar
     const int quad = lane >> 4;
     const int C = g.in_c;
     const int cc0 = blockIdx.y * a.gc * 16; // first channel of this workgroup's chunk
@@ -392,9 +420,11 @@ __global__ __launch_bounds__(kThreads, KS > kKs ? 2 : 4) void depthwise_s8_lds_k
     int *a_l = reinterpret_cast<int *>(smem + a.off_a);
     for (int e = tid; e < a.gc * KS * 64; e += kThreads) {
         const int l = e & 63, ks = (e >> 6) % KS, gi = e / (64 * KS);
-        const int i = l & 15, tap = 4 * ks + (l >> 4);
+        const int i = l & 15;
+        int twin;
+        const int tap = dw_slot_tap(a, 4 * ks + (l >> 4), &twin);
         int d = 0;
-        if (tap < a.taps)
+        if (tap >= 0)
             d = (int)(unsigned char)a.w[(long long)tap * C + cc0 + 16 * gi + i] << (8 * (i & 3));
         a_l[e] = d;
     }
@@ -441,12 +471,10 @@ __global__ __launch_bounds__(kThreads, KS > kKs ? 2 : 4) void depthwise_s8_lds_k
     int tapoff[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
-        const int tap = 4 * ks + quad;
-        tapoff[ks] = 0;
-        if (tap < a.taps) {
-            const int ky = tap / g.k_w, kx = tap - ky * g.k_w;
-            tapoff[ks] = (ky * g.dil_h * a.pw + kx * g.dil_w) * a.cs;
-        }
+        int twin; // empty slots read where a neighbour reads: no bank conflict, no read outside the patch
+        (void)dw_slot_tap(a, 4 * ks + quad, &twin);
+        const int ky = twin / g.k_w, kx = twin - ky * g.k_w;
+        tapoff[ks] = (ky * g.dil_h * a.pw + kx * g.dil_w) * a.cs;
     }
     const int floor_pk = g.relu ? 0 : (int)0x80008000u;
 
@@ -773,6 +801,8 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr, const Dw
                     best.ok = true;
                     DwLdsArgs &a = best.a;
                     a.taps = taps;
+                    a.row3 = (g.k_w == 3 && g.k_h <= kKs && ks_steps == kKs) ? 1 : 0;
+                    a.ks_used = a.row3 ? g.k_h : (taps + 3) / 4;
                     a.th = the;
                     a.tw = twe;
                     a.ph = ph;
