@@ -61,6 +61,19 @@ POINTWISE_MANY_PIXELS = [
     ("p128_128", (80, 80, 128), 128, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
 ]
 
+# Gemm-like products with a short reduction axis under a thousand or more filters over many rows (a recognizer's
+# classifier), the output too large for the caches.  Row lengths that are odd (every output row starts at another
+# alignment), even but not a multiple of 4, a multiple of 64; reduction lengths that are and are not multiples of
+# 16, with one and two steps of 64; a last group of a single filter; row counts that are not a multiple of 64.
+WIDE_ROWS = [
+    ("w120_2049", (80, 81, 120), 2049, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("w128_1792", (80, 80, 128), 1792, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
+    ("w64_2050", (80, 81, 64), 2050, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), False, True),
+    ("w40_1801", (83, 80, 40), 1801, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+    ("w100_1777", (80, 80, 100), 1777, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, True),
+    ("w16_1900", (81, 81, 16), 1900, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), True, False),
+]
+
 # Windowed convolutions whose channel count is a multiple of 16: the kernel that stages the input tile and the
 # filters in LDS.  Strides 1 to 3, dilation, reduction steps that span several taps (16, 32, 48 channels), several
 # groups of 64 filters in one and in several chunks, filter counts that are not a multiple of 64 / 16 / 4, images

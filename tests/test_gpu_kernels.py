@@ -5,7 +5,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, POINTWISE_MANY_PIXELS, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
+from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, POINTWISE_MANY_PIXELS, WIDE_ROWS, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
 from gpu_util import announce, espdl, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
@@ -151,6 +151,58 @@ def test_conv2d_s8_pointwise_short_reduction(oracle, case, flavour):
     oracle.set_threads(16)
     got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
     np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", WIDE_ROWS, ids=lambda c: c[0])
+@pytest.mark.parametrize("flavour", ["per_tensor", "per_channel", "half_even", "lut", "general_epilogue", "mixed_epilogue"])
+def test_conv2d_s8_wide_rows(oracle, case, flavour):
+    """Short reduction under thousands of filters over many rows (a recognizer's classifier): both exponent forms,
+    round-half-even, a table in the epilogue, the general shift-and-round form for every group of 64 filters and for
+    some of them only."""
+    announce(f"conv2d_s8 wide rows {case[0]} {flavour}")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 233, 3, flavour != "per_tensor")
+    kw = {}
+    if flavour == "half_even":
+        kw["half_even"] = True
+    if flavour == "lut":
+        kw["lut"] = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8)
+        relu = False
+    if flavour in ("general_epilogue", "mixed_epilogue"):
+        lim = len(shift) if flavour == "general_epilogue" else 700
+        shift = np.array(shift, dtype=np.int32)
+        shift[:lim:3] = 0
+        shift[1:lim:5] = 33
+        if bias is not None:
+            bias = bias.copy()
+            bias[:lim:2] = (1 << 30) - 7
+    oracle.set_threads(16)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_conv2d_s8_wide_rows_views(oracle):
+    """The same product with an output that starts at an odd address, an input that is a channel slice of a wider
+    tensor, and the recognizer's own shape (120 -> 6625) at a sequence count that is not a multiple of 64."""
+    import torch
+    announce("conv2d_s8 wide rows views")
+    m = espdl()
+    rng = np.random.default_rng(239)
+    rows, c, oc = 16 * 4 * 256 + 37, 120, 6625
+    x = rng_int8(rng, (1, 1, rows, c))
+    f = rng_int8(rng, (oc, 1, 1, c))
+    bias = rng.integers(-4096, 4097, size=oc).astype(np.int32)
+    shift = (typical_shift(c) + rng.integers(-2, 3, size=oc)).astype(np.int32)
+    oracle.set_threads(16)
+    want = oracle.conv2d_s8(x, f, bias, shift, (1, 1), (1, 1), (1, 1), (0, 0, 0, 0), oracle.LINEAR, oracle.ROUND_HALF_UP)
+    wide = torch.zeros((1, 1, rows, c + 24), dtype=torch.int8, device="cuda")
+    wide[..., 8:8 + c].copy_(torch.from_numpy(x))
+    for offset in (0, 1, 7, 13):
+        buf = torch.full((rows * oc + 64,), 77, dtype=torch.int8, device="cuda")
+        out = buf[offset:offset + rows * oc].view(1, 1, rows, oc)
+        m.conv2d(wide[..., 8:8 + c], to_dev(f), to_dev(bias), to_dev(shift), (1, 1), out=out)
+        np.testing.assert_array_equal(to_host(out), want)
+        # nothing outside the tensor was written
+        assert bool((buf[:offset] == 77).all()) and bool((buf[offset + rows * oc:] == 77).all())
 
 
 def test_conv2d_s8_first_layer_at_the_tensor_end(oracle):
