@@ -40,9 +40,9 @@ MACHINE_BALANCE = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)  # OP per byte
 # 256 MiB element-wise kernel of known traffic gave in the same runs).  Only valid for config 3 at
 # batch 256; any other workload reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "mbconv_s8_wave": 43233941.0,   # 7 launches (the stem convolution rides in the first block's launch)
-    "mbconv_s8_group": 8492449.0,   # 10 launches
-    "conv2d_s8": 7164469.0,         # head convolution with GlobalAveragePool, classifier
+    "mbconv_s8_wave": 43231559.0,   # 7 launches (the stem convolution rides in the first block's launch)
+    "mbconv_s8_group": 8491849.0,   # 10 launches
+    "conv2d_s8": 7172235.0,         # head convolution with GlobalAveragePool, classifier
     "elementwise_s8": None,
 }
 
