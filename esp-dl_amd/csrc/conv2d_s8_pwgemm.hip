@@ -47,6 +47,10 @@ struct PwArgs {
     int ksteps;
     int relu, half_even, n_shift;
     int out_vec; // 16, 4 or 1
+    // WIN builds: a convolution with a window as the same product over gathered rows (im2col on the fly): row m is
+    // output pixel m, its k bytes [tap][channel] come from the input pixels under the window (zeros outside the image)
+    int w_in_h, w_in_w, w_in_c, w_k_w, w_stride_h, w_stride_w, w_dil_h, w_dil_w, w_pad_top, w_pad_left;
+    FastDiv fd_ohw, fd_ow, fd_inc, fd_kw;
     int hw;          // GAP builds: pixels per image (at most 64)
     float gap_scale; // GAP builds: 2^in_exp / (h w) * 2^-out_exp of the pooling operator
 };
@@ -57,7 +61,12 @@ struct PwArgs {
 // results (requantized, activation applied, exactly what the separate operator would have stored) are summed
 // over the image's pixels - over the 16 lanes of a pixel tile by rotations inside the row, over the four
 // wavefronts through LDS - and the sum goes through the pooling operator's float scale and rounding.
-template <int NG, int PT, bool GAP = false, bool K16 = true>
+// WIN: rows are gathered from under a convolution window (channels a multiple of 64, so that a k step of 64 lies
+// inside one tap): what conv2d_33cn / conv2d_hwcn compute (esp-dl/dl/base/dl_base_conv2d.cpp:35-163) under
+// conv_operation_shell's window clipping (esp-dl/dl/base/dl_base.hpp:940-1191).  For layers with few output pixels
+// and a long reduction axis (the strided 3 x 3 convolutions deep in a detector's backbone), where a workgroup of
+// the other kernels spends its time staging filters it uses for a handful of pixel sets.
+template <int NG, int PT, bool GAP = false, bool K16 = true, bool WIN = false>
 __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs a)
 {
     constexpr int TN = 64 * NG;
@@ -118,13 +127,49 @@ __global__ __launch_bounds__(kThreads) void conv2d_s8_pwgemm_kernel(const PwArgs
         }
         return r;
     };
-    auto fetch = [&](int ks, v4i(&pb)[kPiecesB], v4i(&pa)[kPiecesA]) {
-        const int k0 = 64 * ks;
+    // WIN: where the window of this thread's rows starts in the input (row of piece slot j: (tid + j * kThreads) / 4)
+    long long win_base[WIN ? kPiecesB : 1];
+    int win_iy[WIN ? kPiecesB : 1], win_ix[WIN ? kPiecesB : 1];
+    if constexpr (WIN) {
 #pragma unroll
         for (int j = 0; j < kPiecesB; j++) {
-            const int p = tid + j * kThreads;
-            const long long m = row_pixel(p >> 2);
-            pb[j] = m >= 0 ? piece(a.in + m * a.in_pitch, k0 + 16 * (p & 3)) : v4i{0, 0, 0, 0};
+            const long long m = row_pixel((tid + j * kThreads) >> 2);
+            win_iy[j] = -0x40000000; // a row past the last: every tap is outside
+            win_ix[j] = 0;
+            win_base[j] = 0;
+            if (m >= 0) {
+                const unsigned n = fastdiv((unsigned)m, a.fd_ohw);
+                const unsigned rem = (unsigned)m - n * a.fd_ohw.d;
+                const unsigned oy = fastdiv(rem, a.fd_ow);
+                const unsigned ox = rem - oy * a.fd_ow.d;
+                win_iy[j] = (int)oy * a.w_stride_h - a.w_pad_top;
+                win_ix[j] = (int)ox * a.w_stride_w - a.w_pad_left;
+                win_base[j] = (((long long)n * a.w_in_h + win_iy[j]) * a.w_in_w + win_ix[j]) * a.in_pitch;
+            }
+        }
+    }
+    auto fetch = [&](int ks, v4i(&pb)[kPiecesB], v4i(&pa)[kPiecesA]) {
+        const int k0 = 64 * ks;
+        if constexpr (WIN) {
+            // the tap and first channel of this k step (uniform)
+            const unsigned tap = fastdiv((unsigned)k0, a.fd_inc);
+            const int c0 = k0 - (int)tap * a.w_in_c;
+            const unsigned ky = fastdiv(tap, a.fd_kw);
+            const int dy = (int)ky * a.w_dil_h, dx = (int)(tap - ky * a.fd_kw.d) * a.w_dil_w;
+            const long long tap_off = ((long long)dy * a.w_in_w + dx) * a.in_pitch + c0;
+#pragma unroll
+            for (int j = 0; j < kPiecesB; j++) {
+                const int p = tid + j * kThreads;
+                const bool ok = (unsigned)(win_iy[j] + dy) < (unsigned)a.w_in_h && (unsigned)(win_ix[j] + dx) < (unsigned)a.w_in_w;
+                pb[j] = ok ? *reinterpret_cast<const v4i *>(a.in + win_base[j] + tap_off + 16 * (p & 3)) : v4i{0, 0, 0, 0};
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < kPiecesB; j++) {
+                const int p = tid + j * kThreads;
+                const long long m = row_pixel(p >> 2);
+                pb[j] = m >= 0 ? piece(a.in + m * a.in_pitch, k0 + 16 * (p & 3)) : v4i{0, 0, 0, 0};
+            }
         }
 #pragma unroll
         for (int j = 0; j < kPiecesA; j++) {
@@ -568,6 +613,71 @@ hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const in
         else
             hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2, false, false>), dim3((unsigned)tiles128, gy), dim3(kThreads), 0, stream, a);
     }
+    return hipGetLastError();
+}
+
+// A convolution with a window through the same kernel, rows gathered from under the window: channels a multiple of
+// 64, few output pixels per compute unit and a long reduction axis.
+bool conv2d_s8_wingemm_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count)
+{
+    if (g.k_h * g.k_w < 2 || (g.in_c & 63) != 0 || (g.in_pitch & 15) != 0 || g.out_c < 64 ||
+        ((reinterpret_cast<uintptr_t>(in) | reinterpret_cast<uintptr_t>(filter)) & 15) != 0)
+        return false;
+    const long long npix = (long long)g.batch * g.out_h * g.out_w;
+    const int cus = cu_count > 0 ? cu_count : 256;
+    // the workgroups of the other kernels stage a filter group for every few pixel sets here: at most sixteen
+    // 64-pixel tiles per compute unit, and a reduction axis of nine k steps or more
+    return npix > 0 && npix < 0x7fffffffll && (npix + 63) / 64 < (long long)cus * 32 && g.k_h * g.k_w * g.in_c >= 576;
+}
+
+hipError_t launch_conv2d_s8_wingemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                    const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
+                                    int cu_count, hipStream_t stream)
+{
+    PwArgs a = {};
+    a.in = in;
+    a.w = filter;
+    a.bias = bias;
+    a.shift = shift;
+    a.lut = lut;
+    a.res = residual;
+    a.out = out;
+    a.M = (long long)g.batch * g.out_h * g.out_w;
+    a.K = g.k_h * g.k_w * g.in_c;
+    a.N = g.out_c;
+    a.in_pitch = g.in_pitch;
+    a.out_pitch = g.out_pitch;
+    a.res_pitch = g.res_pitch;
+    a.ksteps = a.K / 64;
+    a.relu = g.relu;
+    a.half_even = g.half_even;
+    a.n_shift = g.n_shift;
+    a.w_in_h = g.in_h;
+    a.w_in_w = g.in_w;
+    a.w_in_c = g.in_c;
+    a.w_k_w = g.k_w;
+    a.w_stride_h = g.stride_h;
+    a.w_stride_w = g.stride_w;
+    a.w_dil_h = g.dil_h;
+    a.w_dil_w = g.dil_w;
+    a.w_pad_top = g.pad_top;
+    a.w_pad_left = g.pad_left;
+    a.fd_ohw = make_fastdiv((unsigned)(g.out_h * g.out_w));
+    a.fd_ow = make_fastdiv((unsigned)g.out_w);
+    a.fd_inc = make_fastdiv((unsigned)g.in_c);
+    a.fd_kw = make_fastdiv((unsigned)g.k_w);
+    const uintptr_t oaddr = reinterpret_cast<uintptr_t>(out) | reinterpret_cast<uintptr_t>(residual);
+    a.out_vec = ((a.N & 15) == 0 && (oaddr & 15) == 0 && (a.out_pitch & 15) == 0) ? 16
+        : (((a.N & 3) == 0 && (oaddr & 3) == 0 && (a.out_pitch & 3) == 0) ? 4 : 1);
+    if (a.M == 0)
+        return hipSuccess;
+    const unsigned gy = (unsigned)((a.N + 63) / 64);
+    const long long tiles128 = (a.M + 127) / 128;
+    const int cus = cu_count > 0 ? cu_count : 256;
+    if (tiles128 * gy * 2 < 3ll * cus)
+        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 1, false, true, true>), dim3((unsigned)((a.M + 63) / 64), gy), dim3(kThreads), 0, stream, a);
+    else
+        hipLaunchKernelGGL((conv2d_s8_pwgemm_kernel<1, 2, false, true, true>), dim3((unsigned)tiles128, gy), dim3(kThreads), 0, stream, a);
     return hipGetLastError();
 }
 

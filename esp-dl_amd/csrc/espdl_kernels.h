@@ -35,6 +35,12 @@ bool conv2d_s8_rows_supports(const ConvGeom &g, const void *in, const void *filt
 hipError_t launch_conv2d_s8_pwgemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
                                    const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
                                    int cu_count, hipStream_t stream);
+// A convolution with a window through the pointwise GEMM kernel, rows gathered from under the window (channels a
+// multiple of 64, few output pixels per compute unit, a long reduction axis).
+bool conv2d_s8_wingemm_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count);
+hipError_t launch_conv2d_s8_wingemm(const ConvGeom &g, const int8_t *in, const int8_t *filter, const int32_t *bias,
+                                    const int32_t *shift, const int8_t *lut, const int8_t *residual, int8_t *out,
+                                    int cu_count, hipStream_t stream);
 // Dense int8 convolution with a window, input tile and filters staged in LDS (conv2d_s8_tiled.hip): channel
 // count a multiple of 16, 16-byte aligned input and filter.
 bool conv2d_s8_tiled_supports(const ConvGeom &g, const void *in, const void *filter, int cu_count);

@@ -96,6 +96,22 @@ TILED_CASES = [
 ]
 
 # BASELINE config 1: 1x56x56x64 -> 64, 3x3, s1, p1, bias, ReLU, shift 9
+# Strided windows over 64 channels or more on few pixels: rows gathered from under the window for the pointwise
+# GEMM kernel.  Strides 2, 3 and mixed, 3 x 3 / 5 x 5 / 2 x 4 windows, dilation, asymmetric padding, windows that
+# hang over every border, 64 / 128 / 192 / 320 channels, filter counts that are not a multiple of 64 / 16 / 4, pixel
+# counts that are not a multiple of 64 or 128.
+WINDOW_GEMM_CASES = [
+    ("g64_40x40_k3s2p1_oc64", (40, 40, 64), 64, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, True),
+    ("g128_33x35_k3s2p1_oc128", (33, 35, 128), 128, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, True),
+    ("g128_20x20_k3s2p1_oc256", (20, 20, 128), 256, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, False),
+    ("g192_17x19_k3s2_tailpad_oc70", (17, 19, 192), 70, (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), True, True),
+    ("g64_31x29_k5s2p2_oc65", (31, 29, 64), 65, (5, 5), (2, 2), (1, 1), (2, 2, 2, 2), False, True),
+    ("g64_26x26_k3s3_oc130", (26, 26, 64), 130, (3, 3), (3, 3), (1, 1), (0, 0, 0, 0), True, False),
+    ("g64_30x44_k3s12d2p2_oc64", (30, 44, 64), 64, (3, 3), (1, 2), (2, 2), (2, 2, 2, 2), True, True),
+    ("g320_9x9_k3s2p1_oc96", (9, 9, 320), 96, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, False),
+    ("g128_12x50_k24s21p0312_oc64", (12, 50, 128), 64, (2, 4), (2, 1), (1, 1), (0, 3, 1, 2), True, True),
+]
+
 CONFIG1 = ("config1_56x56x64_k3p1_relu", (56, 56, 64), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True)
 
 DW_CASES = [

@@ -5,7 +5,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, POINTWISE_MANY_PIXELS, WIDE_ROWS, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
+from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, POINTWISE_MANY_PIXELS, WIDE_ROWS, WINDOW_GEMM_CASES, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
 from gpu_util import announce, espdl, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
@@ -151,6 +151,54 @@ def test_conv2d_s8_pointwise_short_reduction(oracle, case, flavour):
     oracle.set_threads(16)
     got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
     np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", WINDOW_GEMM_CASES, ids=lambda c: c[0])
+@pytest.mark.parametrize("flavour", ["per_tensor", "per_channel", "half_even", "lut", "residual", "general_epilogue"])
+def test_conv2d_s8_strided_window_on_few_pixels(oracle, case, flavour):
+    """Strided windows over many channels on few pixels (the downsampling convolutions deep in a detector): both
+    exponent forms, round-half-even, a table and a residual Add in the epilogue, the general shift-and-round form."""
+    announce(f"conv2d_s8 strided window {case[0]} {flavour}")
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 241, 5, flavour != "per_tensor")
+    kw = {}
+    if flavour == "half_even":
+        kw["half_even"] = True
+    if flavour == "lut":
+        kw["lut"] = np.array([(i * 109 + 37) & 0xFF for i in range(256)], dtype=np.uint8).view(np.int8)
+        relu = False
+    if flavour == "residual":
+        kw["residual_seed"] = 7
+    if flavour == "general_epilogue":
+        shift = np.array(shift, dtype=np.int32)
+        shift[::3] = 0
+        shift[1::5] = 33
+        if bias is not None:
+            bias = bias.copy()
+            bias[::2] = (1 << 30) - 7
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_conv2d_s8_strided_window_channel_slices(oracle):
+    """The same route reading a channel slice of a wider tensor and writing into one (the operands of a Concat)."""
+    import torch
+    announce("conv2d_s8 strided window channel slices")
+    m = espdl()
+    rng = np.random.default_rng(251)
+    n, h, w, c, oc = 4, 30, 34, 128, 96
+    x = rng_int8(rng, (n, h, w, c))
+    f = rng_int8(rng, (oc, 3, 3, c))
+    bias = rng.integers(-4096, 4097, size=oc).astype(np.int32)
+    shift = (typical_shift(9 * c) + rng.integers(-2, 3, size=oc)).astype(np.int32)
+    want = oracle.conv2d_s8(x, f, bias, shift, (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), oracle.RELU, oracle.ROUND_HALF_UP)
+    wide_in = torch.full((n, h, w, c + 64), 55, dtype=torch.int8, device="cuda")
+    wide_in[..., 32:32 + c].copy_(torch.from_numpy(x))
+    wide_out = torch.full((n, want.shape[1], want.shape[2], oc + 48), 66, dtype=torch.int8, device="cuda")
+    m.conv2d(wide_in[..., 32:32 + c], to_dev(f), to_dev(bias), to_dev(shift), (3, 3), (2, 2), (1, 1), (1, 1, 1, 1),
+             activation=m.capi.RELU, out=wide_out[..., 16:16 + oc])
+    got = to_host(wide_out)
+    np.testing.assert_array_equal(got[..., 16:16 + oc], want)
+    assert (got[..., :16] == 66).all() and (got[..., 16 + oc:] == 66).all()
 
 
 @pytest.mark.parametrize("case", WIDE_ROWS, ids=lambda c: c[0])
