@@ -26,7 +26,7 @@
 namespace espdl {
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 256; // per workgroup, or twice that (see the launch)
 constexpr int kMaxRowTiles = 4;
 constexpr size_t kLdsBudget = 140 * 1024;
 
@@ -55,8 +55,10 @@ __device__ __forceinline__ int low_bytes(int m0, int m1)
     return (int)__builtin_amdgcn_perm((unsigned)m1, (unsigned)m0, 0x06040200u);
 }
 
-__global__ __launch_bounds__(kThreads) void conv2d_s16_mfma_kernel(const S16MfmaArgs a)
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void conv2d_s16_mfma_kernel(const S16MfmaArgs a)
 {
+    constexpr int kThreads = THREADS;
     extern __shared__ __align__(16) unsigned char smem[];
     const ConvGeom &g = a.g;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -279,8 +281,13 @@ hipError_t launch_conv2d_s16_mfma(const ConvGeom &g, const int16_t *in, const in
     a.fd_kw = make_fastdiv((unsigned)g.k_w);
     a.fd_ow = make_fastdiv((unsigned)g.out_w);
     a.fd_ohw = make_fastdiv((unsigned)(g.out_h * g.out_w));
-    static const hipError_t lds_opt_in = hipFuncSetAttribute(reinterpret_cast<const void *>(conv2d_s16_mfma_kernel),
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBudget);
+    static const hipError_t lds_opt_in = [] {
+        const hipError_t e0 = hipFuncSetAttribute(reinterpret_cast<const void *>(conv2d_s16_mfma_kernel<kThreads>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBudget);
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(conv2d_s16_mfma_kernel<2 * kThreads>),
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBudget);
+        return e0 != hipSuccess ? e0 : e1;
+    }();
     if (lds_opt_in != hipSuccess)
         return lds_opt_in;
     const int gy = (g.out_c + p.row_tiles * 16 - 1) / (p.row_tiles * 16);
@@ -288,8 +295,16 @@ hipError_t launch_conv2d_s16_mfma(const ConvGeom &g, const int16_t *in, const in
     const size_t fit = (size_t)(160 * 1024) / (p.lds > 0 ? p.lds : 1);
     const int per_cu = fit < 1 ? 1 : (fit > 4 ? 4 : (int)fit);
     int gx = max(1, (cus * per_cu) / gy);
-    gx = min(gx, (a.n_pixel_tiles + 3) / 4);
-    conv2d_s16_mfma_kernel<<<dim3((unsigned)gx, (unsigned)gy), dim3(kThreads), p.lds, stream>>>(a);
+    // Filter planes of a long reduction axis (72 KB for 3 x 3 x 64 channels) leave room for two workgroups per
+    // compute unit; eight wavefronts each then keep the vector ALU, which sorts the pixels' bytes, busy where four
+    // leave it idle half of the time (80 x 80 x 64 -> 64, 3 x 3, batch 64: 123 -> 88 us).
+    const bool wide = per_cu <= 2;
+    const int waves = (wide ? 2 * kThreads : kThreads) / 64;
+    gx = min(gx, (a.n_pixel_tiles + waves - 1) / waves);
+    if (wide)
+        conv2d_s16_mfma_kernel<2 * kThreads><<<dim3((unsigned)gx, (unsigned)gy), dim3(2 * kThreads), p.lds, stream>>>(a);
+    else
+        conv2d_s16_mfma_kernel<kThreads><<<dim3((unsigned)gx, (unsigned)gy), dim3(kThreads), p.lds, stream>>>(a);
     return hipGetLastError();
 }
 
