@@ -237,6 +237,16 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
                     v[d] = sat_add4_s8(v[d], r[d]);
             }
             *reinterpret_cast<v4i_unaligned *>(dst) = v;
+        } else if (NT == 2 && c_lane + 8 <= OC) {
+            // two filter tiles: the lane's eight channels as one piece (half the store instructions of a layer with
+            // 32 filters, which the memory pipeline serves lane by lane either way)
+            v2i v = {words[0], words[NT > 1 ? 1 : 0]};
+            if (res_img != nullptr) {
+                const v2i r = *reinterpret_cast<const v2i_unaligned *>(res_img + (size_t)ro);
+                v[0] = sat_add4_s8(v[0], r[0]);
+                v[1] = sat_add4_s8(v[1], r[1]);
+            }
+            *reinterpret_cast<v2i_unaligned *>(dst) = v;
         } else {
 #pragma unroll
             for (int t = 0; t < NT; t++) {

@@ -16,6 +16,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 // The same values at any byte address: gfx950 global loads and stores need no alignment, one instruction each.
 typedef v4i v4i_unaligned __attribute__((aligned(1)));
+typedef v2i v2i_unaligned __attribute__((aligned(1)));
 typedef int int_unaligned __attribute__((aligned(1)));
 
 __device__ __forceinline__ int clamp_s8(int v)
