@@ -203,9 +203,14 @@ int espdl_hip_conv2d_add(const espdl_hip_conv_desc *desc, const void *in, const 
             (lut == nullptr && residual == nullptr && espdl::conv2d_s8_rows_supports(g, in, filter, cu_count_cached())))
             return device_status(espdl::launch_conv2d_s8_pwgemm(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
                                  "conv2d_s8_pwgemm");
-        // strided windows over 64 channels or more on few pixels: the pointwise GEMM kernel over gathered rows
-        // (80 x 80 x 128 -> 128 at stride 2, batch 64: 91 -> 41 us; at stride 1 the LDS-tiled kernel below is faster)
-        if ((g.stride_h != 1 || g.stride_w != 1) && espdl::conv2d_s8_wingemm_supports(g, in, filter, cu_count_cached()))
+        // Windows over 64 channels or more on few pixels: the pointwise GEMM kernel over gathered rows.  Strided
+        // windows (80 x 80 x 128 -> 128 at stride 2, batch 64: 91 -> 41 us); at stride 1 up to 128 K output pixels
+        // (40 x 40 x 128 -> 64, batch 64: 26 -> 22 us; 20 x 20 x 256 -> 256: 93 -> 38 us) or with a reduction axis of
+        // 2048 or more, whose filters the LDS-tiled kernel below cannot keep resident (80 x 80 x 256 -> 256: 732 ->
+        // 472 us); with more pixels and fewer channels that kernel is faster (80 x 80 x 64 -> 64: 30 against 41 us).
+        const bool few_pixels = (long long)g.batch * g.out_h * g.out_w <= 128 * 1024;
+        if ((g.stride_h != 1 || g.stride_w != 1 || few_pixels || g.k_h * g.k_w * g.in_c >= 2048) &&
+            espdl::conv2d_s8_wingemm_supports(g, in, filter, cu_count_cached()))
             return device_status(espdl::launch_conv2d_s8_wingemm(g, i8, f8, b32, shift, lut, residual, o8, cu_count_cached(), s),
                                  "conv2d_s8_wingemm");
         if (espdl::conv2d_s8_tiled_supports(g, in, filter, cu_count_cached()))

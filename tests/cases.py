@@ -112,6 +112,14 @@ WINDOW_GEMM_CASES = [
     ("g128_12x50_k24s21p0312_oc64", (12, 50, 128), 64, (2, 4), (2, 1), (1, 1), (0, 3, 1, 2), True, True),
 ]
 
+# Stride-1 windows over 64 and 128 channels on more than 128 K output pixels (with the batch the test gives them):
+# the shapes that stay with the LDS-tiled kernel when the few-pixel route takes the smaller ones.
+TILED_MANY_PIXELS = [
+    ("tm64_56x56_k3p1_oc64", (56, 56, 64), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True),
+    ("tm128_40x44_k3p1_oc96", (40, 44, 128), 96, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False),
+    ("tm64_50x60_k3d2p2_oc72", (50, 60, 64), 72, (3, 3), (1, 1), (2, 2), (2, 2, 2, 2), False, True),
+]
+
 CONFIG1 = ("config1_56x56x64_k3p1_relu", (56, 56, 64), 64, (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True)
 
 DW_CASES = [

@@ -5,7 +5,7 @@ import ctypes
 import numpy as np
 import pytest
 
-from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, POINTWISE_MANY_PIXELS, WIDE_ROWS, WINDOW_GEMM_CASES, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
+from cases import CONFIG1, CONV_CASES, DW_CASES, GEMM_CASES, POINTWISE_MANY_PIXELS, WIDE_ROWS, WINDOW_GEMM_CASES, TILED_MANY_PIXELS, STEM_CASES, TILED_CASES, every_sum_image, rng_int8, typical_shift
 from gpu_util import announce, espdl, to_dev, to_host
 
 pytestmark = pytest.mark.gpu
@@ -148,6 +148,24 @@ def test_conv2d_s8_pointwise_short_reduction(oracle, case, flavour):
         if bias is not None:
             bias = bias.copy()
             bias[::2] = (1 << 30) - 7
+    oracle.set_threads(16)
+    got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("case", TILED_MANY_PIXELS, ids=lambda c: c[0])
+@pytest.mark.parametrize("flavour", ["per_channel", "half_even", "residual"])
+def test_conv2d_s8_window_on_many_pixels(oracle, case, flavour):
+    """Stride-1 windows over 64 channels or more at a batch that puts them above 128 K output pixels."""
+    announce(f"conv2d_s8 window on many pixels {case[0]} {flavour}")
+    h, w = case[1][0], case[1][1]
+    n = (128 * 1024) // (h * w) + 2
+    x, f, bias, shift, k, stride, dil, pads, relu = _conv_inputs(case, 257, n, True)
+    kw = {}
+    if flavour == "half_even":
+        kw["half_even"] = True
+    if flavour == "residual":
+        kw["residual_seed"] = 11
     oracle.set_threads(16)
     got, want = _run_conv_s8(oracle, x, f, bias, shift, k, stride, dil, pads, relu, **kw)
     np.testing.assert_array_equal(got, want)
