@@ -40,9 +40,9 @@ MACHINE_BALANCE = PEAK_INT8_TOPS * 1e12 / (PEAK_HBM_GBS * 1e9)  # OP per byte
 # 256 MiB element-wise kernel of known traffic gave in the same runs).  Only valid for config 3 at
 # batch 256; any other workload reports null.
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {
-    "mbconv_s8_wave": 43231559.0,   # 7 launches (the stem convolution rides in the first block's launch)
+    "mbconv_s8_wave": 43231581.0,   # 7 launches (the stem convolution rides in the first block's launch)
     "mbconv_s8_group": 8491849.0,   # 10 launches
-    "conv2d_s8": 7172235.0,         # head convolution with GlobalAveragePool, classifier
+    "conv2d_s8": 7173205.0,         # head convolution with GlobalAveragePool, classifier
     "elementwise_s8": None,
 }
 
@@ -352,7 +352,9 @@ def main():
         # the other four BASELINE configs, same procedure, fewer steps; the CPU leg stays on the headline workload
         configs = {}
         for cfg, b in OTHER_CONFIGS:
-            o = measure(pkg, args, cfg, b, max(20, args.steps // 4), max(5, args.warmup // 2), parity=not args.no_parity)
+            # (the single image is a 15 us step: many more of them, or the clock is reading launch jitter)
+            k = args.steps * 5 if b == 1 else max(20, args.steps // 4)
+            o = measure(pkg, args, cfg, b, k, max(5, args.warmup // 2) * (10 if b == 1 else 1), parity=not args.no_parity)
             r = dominant_roofline(o["kernels"])
             configs["config%d_batch%d" % (cfg, b)] = {
                 "workload": "%s, batch %d" % (o["spec"].name, b), "ms_per_step": round(o["ms_per_step"], 4),
