@@ -352,9 +352,10 @@ def main():
         # the other four BASELINE configs, same procedure, fewer steps; the CPU leg stays on the headline workload
         configs = {}
         for cfg, b in OTHER_CONFIGS:
-            # (the single image is a 15 us step: many more of them, or the clock is reading launch jitter)
-            k = args.steps * 5 if b == 1 else max(20, args.steps // 4)
-            o = measure(pkg, args, cfg, b, k, max(5, args.warmup // 2) * (10 if b == 1 else 1), parity=not args.no_parity)
+            # (steps of config 1 take 15 and 50 us: many more of them, or the clock reads launch jitter and the
+            # ramp of the GPU's clocks)
+            k = args.steps * 5 if cfg == 1 else max(20, args.steps // 4)
+            o = measure(pkg, args, cfg, b, k, max(5, args.warmup // 2) * (10 if cfg == 1 else 1), parity=not args.no_parity)
             r = dominant_roofline(o["kernels"])
             configs["config%d_batch%d" % (cfg, b)] = {
                 "workload": "%s, batch %d" % (o["spec"].name, b), "ms_per_step": round(o["ms_per_step"], 4),

@@ -6,6 +6,7 @@ The GPU box runs the prebuilt .so files that travel with the tree; nothing is co
 """
 import concurrent.futures
 import os
+import re
 import subprocess
 import sys
 
@@ -40,8 +41,79 @@ def _run(cmd):
 
 def _compile(src, extra=()):
     obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
+    if os.path.basename(src) in CHECKED_ASM:
+        extra = (*extra, "-save-temps=obj")
     warn = _run([HIPCC, *HIP_FLAGS, *extra, "-c", src, "-o", obj])
+    if os.path.basename(src) in CHECKED_ASM:
+        stem = os.path.splitext(os.path.basename(src))[0]
+        CHECKED_ASM[os.path.basename(src)](os.path.join(OBJ_DIR, stem + "-hip-amdgcn-amd-amdhsa-%s.s" % ARCH))
     return obj, warn
+
+
+def _vgprs(text):
+    """Vector registers an instruction line names (vN and v[a:b])."""
+    text = text.split(";")[0]
+    regs = set()
+    for a, b in re.findall(r"\bv\[(\d+):(\d+)\]", text):
+        regs.update(range(int(a), int(b) + 1))
+    regs.update(int(a) for a in re.findall(r"\bv(\d+)\b", text))
+    return regs
+
+
+def check_tiled_patch_registers(asm_path):
+    """conv2d_s8_tiled.hip loads the pieces of the next input patch with buffer loads written as asm statements
+    and waits for them by hand, so the compiler does not know that the destination registers are in flight.
+    This reads the generated code of every conv2d_s8_tiled_kernel instance and fails the build unless
+      * the kernel has no vector register spills, and
+      * from the first load into a piece register to the end of the kernel that register is named only by the
+        loads of the piece, by the LDS write of the piece (as data) and by the few instructions right in front of
+        a load that compute its address in the load's own destination (the piece in it was written to LDS before).
+    """
+    lines = open(asm_path).read().splitlines()
+    starts = [i for i, l in enumerate(lines) if re.match(r"^_ZN5espdl\S*conv2d_s8_tiled_kernel\S*:", l)]
+    if not starts:
+        raise RuntimeError("%s: no conv2d_s8_tiled_kernel in the generated code" % asm_path)
+    spills = re.findall(r"\.vgpr_spill_count:\s*(\d+)", "\n".join(lines))
+    problems = []
+    if any(int(n) for n in spills):
+        problems.append("vector register spills: %s" % spills)
+    for st in starts:
+        end = next(i for i in range(st, len(lines)) if "s_endpgm" in lines[i])
+        body = lines[st:end]
+        loads, first = {}, {}
+        for i, l in enumerate(body):
+            m = re.search(r"buffer_load_dwordx4 v\[(\d+):(\d+)\], v(\d+)", l)
+            if m:
+                loads[i] = set(range(int(m.group(1)), int(m.group(2)) + 1))
+                for r in loads[i]:
+                    first.setdefault(r, i)
+        if len(first) != 32:
+            problems.append("%s: %d piece registers, expected 32" % (lines[st].split(":")[0], len(first)))
+        load_lines = sorted(loads)
+        for i, l in enumerate(body):
+            if not l.startswith("\t") or l.lstrip().startswith((";", ".")):
+                continue
+            named = {r for r in _vgprs(l) if r in first and i > first[r]}
+            if not named:
+                continue
+            op = l.split()[0]
+            if op == "buffer_load_dwordx4":
+                continue
+            if op == "ds_write_b128":
+                m = re.search(r"ds_write_b128 v(\d+), v\[(\d+):(\d+)\]", l)
+                if m and int(m.group(1)) not in named:
+                    continue
+            # address arithmetic in the destination of a load that follows within sixteen lines
+            ahead = [j for j in load_lines if i < j <= i + 16]
+            if ahead and all(any(r in loads[j] for j in ahead) for r in named):
+                continue
+            problems.append("%s line %d touches a piece register: %s" % (os.path.basename(asm_path), st + i + 1, l.strip()))
+    if problems:
+        raise RuntimeError("conv2d_s8_tiled.hip: generated code breaks what its hand-placed waits assume:\n  " +
+                           "\n  ".join(problems[:20]))
+
+
+CHECKED_ASM = {"conv2d_s8_tiled.hip": check_tiled_patch_registers}
 
 
 def build_kernels(verbose=True):

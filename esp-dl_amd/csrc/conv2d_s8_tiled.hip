@@ -1,4 +1,4 @@
-// Dense int8 convolution with a window (3x3, 5x5, strided, dilated ...) for gfx950: implicit GEMM on
+// Dense int8 convolution with a window (3x3, 5x5, dilated ...) at stride 1 for gfx950: implicit GEMM on
 // v_mfma_i32_16x16x64_i8 with the NHWC input tile AND the filters staged in LDS.
 //
 // It computes what conv2d_33cn / conv2d_hwcn compute (esp-dl/dl/base/dl_base_conv2d.cpp:35-163) for every
@@ -10,7 +10,7 @@
 // Why a second kernel next to conv2d_s8_mfma_kernel.h: that one reads operand B (the pixels) straight from
 // global memory, once per filter tap, so a 3x3 convolution fetches every input byte nine times from L2 and
 // pays address arithmetic per tap and pixel.  Here a workgroup owns a th x tw tile of ONE image's output:
-//   * the (th*s + (k-1)*d) x (tw*s + (k-1)*d) input patch with all channels is copied to LDS once, with
+//   * the (th + (k-1)*d) x (tw + (k-1)*d) input patch with all channels is copied to LDS once, with
 //     16-byte loads of consecutive addresses and zeros for positions outside the image; the copy of the
 //     NEXT tile's patch is in flight in registers while the current tile is computed;
 //   * the filters of the workgroup's chunk (up to all of them) sit in LDS in MFMA operand-A order for the
@@ -18,14 +18,12 @@
 //   * a wavefront takes sets of PT pixel tiles (16 pixels each) and, per group of 64 filters, walks the
 //     reduction axis (tap, channel) in steps of 64: PT + 4 operand reads of 16 bytes per lane from LDS feed
 //     4 * PT matrix instructions, the operands of the next step being read while the current products run.
-// LDS layout of the patch: [row][column phase = column % stride_w][column / stride_w][channels + pad], the
-// pixel pitch twice an odd number of 16-byte units (the pitch at which 16-byte-per-lane reads of 16 neighbouring
-// pixels meet no bank twice).  Splitting the columns by phase makes the 16 pixels of a tile neighbours in LDS for
-// every tap also at stride 2.  (The kernel keeps that strided form, but the planner hands it stride-1 layers
-// only: strided layers re-read little and measured as fast or faster through the direct kernel.)  With stride 1
-// the "pixels" of a tile are 16 consecutive positions of the patch's flattened (row, column) space: a tap is
-// then a constant offset, tiles run across row ends, and only the (k-1)*d positions per row that wrap are
-// wasted instead of the padding of every row to a multiple of 16.
+// LDS layout of the patch: [row][column][channels + pad], the pixel pitch twice an odd number of 16-byte units
+// (the pitch at which 16-byte-per-lane reads of 16 neighbouring pixels meet no bank twice).  The kernel is for
+// stride 1 (strided layers re-read little and measured as fast or faster through the direct kernel, so the
+// planner refuses them): the "pixels" of a tile are 16 consecutive positions of the patch's flattened
+// (row, column) space, a tap is then a constant offset, tiles run across row ends, and only the (k-1)*d positions
+// per row that wrap are wasted instead of the padding of every row to a multiple of 16.
 // The offset of reduction step ks for lane group q (tap and first channel of k = 64 ks + 16 q) comes from a
 // small LDS table, so any channel count that is a multiple of 16 works, also when a step of 64 spans taps.
 #include <algorithm>
@@ -55,22 +53,22 @@ struct TiledArgs {
     int K, ksteps;
     int n_groups, groups_per_chunk;
     int th, tw;          // output tile
-    int ph, pw, pwp;     // patch rows, columns, columns per phase plane
+    int ph, pw;          // patch rows and columns
     int cs;              // LDS bytes per patch pixel
     int cu16;            // in_c / 16
-    int flat;            // stride 1 x 1: pixel tiles run over the flattened patch
-    int vrow;            // virtual pixels per output row (flat: pw, else tw rounded up to 16)
     int n_ptiles, n_sets;
     int tiles_x, tiles_y, n_tiles;
     int row_units;       // pw * cu16: 16-byte pieces of one patch row
     int row_par;         // patch rows the workgroup's threads copy at a time (threads / row_units)
+    int row_groups;      // pieces per thread: patch rows / row_par, rounded up (the LDS patch holds that many rows)
     int src_row_step;    // bytes between the input rows of a thread's consecutive pieces (row_par rows)
     int lds_row_step;    // the same in the LDS patch
+    int img_bytes;       // bytes of one image of the input tensor
     int off_tabs, off_koff, off_lut, off_patch; // LDS offsets (filters at 0)
     int out_vec;
     int epi;             // epilogue form: 0 plain 16-byte stores, 1 the same with table / residual, 2 general
     int koff_pitch;      // ints per lane-group row of the step-offset table
-    FastDiv fd_cu16, fd_sw, fd_vrow, fd_tiles_x, fd_tiles_yx, fd_vrow16, fd_row_units;
+    FastDiv fd_cu16, fd_pw, fd_tiles_x, fd_tiles_yx, fd_row_units;
 };
 
 __device__ __forceinline__ int group_tiles(int out_c, int gbase)
@@ -97,11 +95,19 @@ __device__ __forceinline__ TileRef decode_tile(const TiledArgs &a, int tile)
     t.img_res = (long long)n * g.out_h * g.out_w * g.res_pitch;
     t.oy0 = (int)ty * a.th;
     t.ox0 = (int)tx * a.tw;
-    t.iy0 = t.oy0 * g.stride_h - g.pad_top;
-    t.ix0 = t.ox0 * g.stride_w - g.pad_left;
+    t.iy0 = t.oy0 - g.pad_top;
+    t.ix0 = t.ox0 - g.pad_left;
     t.th_real = min(a.th, g.out_h - t.oy0);
     t.tw_real = min(a.tw, g.out_w - t.ox0);
     return t;
+}
+
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
+
+// Wait for the wavefront's outstanding vector-memory instructions, as an instruction of its own.
+__device__ __forceinline__ void settle()
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 struct Ctx {
@@ -183,6 +189,7 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
         if (ks < ksteps)
             products(0);
     }
+    settle(); // the pieces of the next patch, before the first store after their request
     // epilogue: this lane owns output channels [c_lane, c_lane + 4 * NT) of pixel p * 16 + col of the set
     const int c_lane = gbase + 4 * NT * c.quad;
     v4i ss[NT], ls[NT];
@@ -269,7 +276,7 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
     }
 }
 
-// All sets of the wavefront for one tile, with one epilogue form compiled in.
+// All sets of a wavefront that has at least one (wave < n_sets) for one tile, with one epilogue form compiled in.
 template <int PT, int MODE, bool HE, int EPI>
 __device__ __forceinline__ void run_tile(const TiledArgs &a, const Ctx &c, const TileRef &tr, int wave, int n_waves,
                                          int g_first, int g_count)
@@ -279,7 +286,9 @@ __device__ __forceinline__ void run_tile(const TiledArgs &a, const Ctx &c, const
     int8_t *out_img = a.out + tr.img_out;
     const int8_t *res_img = a.res != nullptr ? a.res + tr.img_res : nullptr;
     const int org_out = tr.oy0 * g.out_w + tr.ox0; // in pixels
-    for (int set = wave; set < a.n_sets; set += n_waves) {
+    int set = wave;
+    do {
+        // the pixels of a set: 16 consecutive positions of the flattened patch per pixel tile
         int pixoff[PT];
         int opix[PT];
         unsigned okmask = 0;
@@ -288,25 +297,17 @@ __device__ __forceinline__ void run_tile(const TiledArgs &a, const Ctx &c, const
             const int tp = set * PT + p;
             const bool live = tp < a.n_ptiles; // uniform
             const int tpc = live ? tp : 0;
-            int oy_l, ox_l;
-            if (a.flat) {
-                const unsigned v = (unsigned)(tpc * 16 + c.col);
-                const unsigned row = fastdiv(v, a.fd_vrow);
-                oy_l = (int)row;
-                ox_l = (int)(v - row * a.fd_vrow.d);
-                pixoff[p] = (int)v * a.cs;
-            } else {
-                const unsigned row = fastdiv((unsigned)tpc, a.fd_vrow16);
-                const int xt = tpc - (int)row * (int)a.fd_vrow16.d;
-                oy_l = (int)row;
-                ox_l = xt * 16 + c.col;
-                pixoff[p] = ((int)row * g.stride_h * g.stride_w * a.pwp + ox_l) * a.cs;
-            }
+            const unsigned v = (unsigned)(tpc * 16 + c.col);
+            const unsigned row = fastdiv(v, a.fd_pw);
+            const int oy_l = (int)row;
+            const int ox_l = (int)(v - row * a.fd_pw.d);
+            pixoff[p] = (int)v * a.cs;
             const bool ok = live && oy_l < tr.th_real && ox_l < tr.tw_real;
             okmask |= ok ? 1u << p : 0u;
             opix[p] = org_out + oy_l * g.out_w + ox_l;
         }
-        for (int gi = 0; gi < g_count; gi++) {
+        int gi = 0;
+        do {
             const int gbase = (g_first + gi) * 64;
             if constexpr (EPI != 2) {
                 run_set<PT, 4, MODE, HE, EPI>(a, c, out_img, res_img, pixoff, opix, okmask, gi, gbase);
@@ -326,8 +327,9 @@ __device__ __forceinline__ void run_tile(const TiledArgs &a, const Ctx &c, const
                     break;
                 }
             }
-        }
-    }
+        } while (++gi < g_count); // g_count >= 1
+        set += n_waves;
+    } while (set < a.n_sets);
 }
 
 // PT: pixel tiles per set; UMAX: 16-byte pieces of the next patch a thread holds in registers; MAXT / MINB:
@@ -358,84 +360,63 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     const TileSeq seq = xcd_tile_sequence(a.n_tiles);
     int tile = seq.first;
 
-    // Copying a patch: a thread owns ONE 16-byte column piece (patch column px, channels 16 cu ...) and walks
-    // the patch rows r0, r0 + row_par, ...; everything about the column is computed once per kernel.  Pieces
-    // outside the image become zeros (the reference's window clipping).  The pieces of the NEXT tile are
-    // requested before the current tile is computed and written to LDS after it.
-    // Two forms.  A tile whose patch rows all lie inside the image, and whose columns outside the image are the
-    // same for every tile (one column tile: the left / right padding) or do not exist, takes the short one: the
-    // padding columns were zeroed once and are never written, a piece costs one address and one load.  Tiles
-    // at the top / bottom border (and border column tiles) test every piece.
+    // Copying a patch: a thread owns ONE 16-byte column piece (patch column st_px, channels 16 st_cu ...) and
+    // walks the patch rows r0, r0 + row_par, ...: row_groups pieces, the same count for every thread (the LDS
+    // patch is that many rows tall; rows past the patch are never read).  Everything about the column is computed
+    // once per kernel.  The loads go through a buffer descriptor of the tile's image: a piece outside the image
+    // gets an offset past the descriptor's end and comes back as zeros (the reference's window clipping), so
+    // there is one form for inner and border tiles and nothing to patch up when the pieces are written to LDS.
+    // The pieces of the NEXT tile are requested before the current tile is computed and written to LDS after it.
+    //
+    // The loads and the wait for them are written as instructions.  The pieces are used after the tile's stores; a
+    // wavefront's loads and stores share one counter, and the compiler, for which the two kinds may complete in
+    // any order, waits for that counter to reach zero where the pieces are written to LDS - for the stores just
+    // issued as well - or, when the set loop reuses a piece register, in front of that loop, right after the
+    // request (measured on 56 x 56 x 64 -> 64 at batch 256: 48.8 and 46.9 us per launch; this form 43.3 us).
+    // settle() waits before the first store that follows a request instead - by then the loads have had the
+    // products of a set to arrive - and nothing waits where the pieces are used.  What the compiler does not
+    // know any more has to hold by construction:
+    //   * between a request and settle() nothing may read or move a piece.  The compiler sees the pieces as
+    //     values defined by request() and used by deposit(), keeps them in their registers over the tile and has no
+    //     reason to touch them; the build checks in the generated code that it did not, and that the kernels have
+    //     no register spills (build.py: check_tiled_patch_registers);
+    //   * the descriptor may have been moved into its scalar registers by vector instructions right before a load,
+    //     and a memory instruction may read such a register five wait states later at the earliest: the
+    //     compiler pads its own instructions, not the text of an asm statement, hence the s_nop.
     const unsigned r0 = fastdiv((unsigned)tid, a.fd_row_units);
     const int ru = tid - (int)r0 * a.row_units;
     const bool st_active = (int)r0 < a.row_par;
     const unsigned st_px = fastdiv((unsigned)ru, a.fd_cu16);
     const int st_cu = ru - (int)st_px * a.cu16;
-    const unsigned st_pxq = fastdiv(st_px, a.fd_sw);
-    const int st_phase = (int)st_px - (int)st_pxq * g.stride_w;
     const int st_src0 = ((int)r0 * g.in_w + (int)st_px) * g.in_pitch + 16 * st_cu;
-    const int st_dst0 = (((int)r0 * g.stride_w + st_phase) * a.pwp + (int)st_pxq) * a.cs + 16 * st_cu;
-    // rows of this thread: r0, r0 + row_par, ... below ph
-    const int st_rows = st_active ? (a.ph - (int)r0 + a.row_par - 1) / a.row_par : 0;
-    const bool one_col = a.tiles_x == 1;
-    const bool st_col_static = (unsigned)((int)st_px - g.pad_left) < (unsigned)g.in_w; // one column tile: inside the image
-    const int st_rows_short = (one_col && !st_col_static) ? 0 : st_rows;
-    v4i pre[kUnitsMax];
-    unsigned pre_ok = 0; // long form, bit j: piece j of the requested patch lies inside the image
-    bool pre_short = false;
-    auto tile_short = [&](const TileRef &t) -> bool { // uniform
-        const bool y_in = t.iy0 >= 0 && t.iy0 + a.ph <= g.in_h;
-        const bool x_in = t.ix0 >= 0 && t.ix0 + a.pw <= g.in_w;
-        return y_in && (x_in || one_col);
-    };
-    auto request = [&](const TileRef &t) {
+    const int st_dst0 = ((int)r0 * a.pw + (int)st_px) * a.cs + 16 * st_cu;
+    v4u pre[kUnitsMax];
+    auto request = [&](const TileRef &t, int row_groups) {
+        // buffer descriptor: base, stride 0, bytes, 32-bit raw format
+        const __amdgpu_buffer_rsrc_t img = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<int8_t *>(a.in + t.img_in), (short)0, a.img_bytes, 0x00020000);
         const int org = (t.iy0 * g.in_w + t.ix0) * g.in_pitch;
-        pre_short = tile_short(t);
-        const int8_t *img = a.in + t.img_in;
-        if (pre_short) {
-            if (st_rows_short > 0) {
+        const bool xok = st_active && (unsigned)(t.ix0 + (int)st_px) < (unsigned)g.in_w;
+        const int row = t.iy0 + (int)r0;
+        const int src = org + st_src0;
 #pragma unroll
-                for (int j = 0; j < kUnitsMax; j++) {
-                    const unsigned off = (unsigned)(org + st_src0 + min(j, st_rows_short - 1) * a.src_row_step);
-                    pre[j] = *reinterpret_cast<const v4i *>(img + (size_t)off);
-                }
+        for (int j = 0; j < kUnitsMax; j++)
+            if (j < row_groups) { // uniform
+                const bool ok = xok && (unsigned)(row + j * a.row_par) < (unsigned)g.in_h;
+                const int off = ok ? src + j * a.src_row_step : (int)0x80000000u;
+                asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(pre[j]) : "v"(off), "s"(img));
             }
-        } else {
-            const bool xok = st_active && (unsigned)(t.ix0 + (int)st_px) < (unsigned)g.in_w;
-            const int lo = max(0, -t.iy0), span = min(a.ph, g.in_h - t.iy0) - lo; // patch rows inside the image
-            const int pyv = (int)r0 - lo;
-            pre_ok = 0;
-#pragma unroll
-            for (int j = 0; j < kUnitsMax; j++) {
-                const bool ok = xok && (unsigned)(pyv + j * a.row_par) < (unsigned)span;
-                pre_ok |= ok ? 1u << j : 0u;
-                const unsigned off = ok ? (unsigned)(org + st_src0 + j * a.src_row_step) : 0u;
-                pre[j] = *reinterpret_cast<const v4i *>(img + (size_t)off);
-            }
-        }
     };
-    auto deposit = [&]() {
-        if (pre_short) {
+    auto deposit = [&](int row_groups) {
+        if (st_active) {
 #pragma unroll
             for (int j = 0; j < kUnitsMax; j++)
-                if (j < st_rows_short)
-                    *reinterpret_cast<v4i *>(patch + st_dst0 + j * a.lds_row_step) = pre[j];
-        } else {
-#pragma unroll
-            for (int j = 0; j < kUnitsMax; j++)
-                if (j < st_rows) {
-                    const v4i v = ((pre_ok >> j) & 1u) ? pre[j] : v4i{0, 0, 0, 0};
-                    *reinterpret_cast<v4i *>(patch + st_dst0 + j * a.lds_row_step) = v;
-                }
+                if (j < row_groups) // uniform
+                    *reinterpret_cast<v4u *>(patch + st_dst0 + j * a.lds_row_step) = pre[j];
         }
     };
-    // the padding columns of the short form: zero once
-    if (one_col && !st_col_static)
-        for (int j = 0; j < st_rows; j++)
-            *reinterpret_cast<v4i *>(patch + st_dst0 + j * a.lds_row_step) = v4i{0, 0, 0, 0};
-    TileRef cur = decode_tile(a, min(tile, a.n_tiles - 1));
     if (tile < seq.end)
-        request(cur);
+        request(decode_tile(a, tile), a.row_groups);
 
     // filters of this workgroup's chunk -> LDS in operand-A order: unit (group, k step, tile, lane) holds the 16
     // k positions [64 ks + 16 (lane / 16), +16) of filter row (lane % 16) of tile t; filter rows are permuted
@@ -476,8 +457,7 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
         if (k < a.K) {
             const int tap = k / g.in_c, c0 = k - tap * g.in_c;
             const int ky = tap / g.k_w, kx = tap - ky * g.k_w;
-            const int pxo = kx * g.dil_w;
-            off = ((ky * g.dil_h * g.stride_w + pxo % g.stride_w) * a.pwp + pxo / g.stride_w) * a.cs + c0;
+            off = (ky * g.dil_h * a.pw + kx * g.dil_w) * a.cs + c0;
         }
         koff_l[e] = off;
     }
@@ -505,8 +485,9 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     if (has_lut)
         for (int i = tid; i < 256; i += nthreads)
             lut_l[i] = a.lut[i];
-    const bool fast = __syncthreads_and(ok_local) != 0;
-    const bool use_lsh = __syncthreads_or(lsh_local) != 0;
+    // (the votes are the same in every lane; readfirstlane lets the compiler branch on them as scalars)
+    const bool fast = __builtin_amdgcn_readfirstlane(__syncthreads_and(ok_local)) != 0;
+    const bool use_lsh = __builtin_amdgcn_readfirstlane(__syncthreads_or(lsh_local)) != 0;
     for (int c = tid; c < g_count * 64; c += nthreads) {
         const int oc = g_first * 64 + c;
         int init = 0, sh = fast ? 8 : 0, lsh = 0;
@@ -537,15 +518,21 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     c.has_lut = has_lut;
     c.floor_pk = c.relu ? 0 : (int)0x80008000u;
 
+    settle(); // the first patch
     for (; tile < seq.end; tile += seq.step) {
-        deposit();
+        // The piece count goes through an empty asm statement, so that the compiler compares it where it is used:
+        // a comparison per piece that is the same for every tile gets computed in front of the loop otherwise, as
+        // a lane mask in a pair of scalar registers, and with more scalars alive over the tile loop than
+        // registers to hold them, each mask then costs two vector instructions per tile to fetch back.
+        int row_groups = a.row_groups;
+        asm volatile("" : "+s"(row_groups));
+        deposit(row_groups);
         __syncthreads(); // patch (and, the first time, filters and tables) complete
-        const TileRef now = cur;
+        // tile coordinates are scalar arithmetic: recomputed rather than carried over the loop
+        const TileRef now = decode_tile(a, tile);
         const int next = tile + seq.step;
-        if (next < seq.end) {
-            cur = decode_tile(a, next);
-            request(cur);
-        }
+        if (next < seq.end)
+            request(decode_tile(a, next), row_groups);
         const auto go = [&](auto mode_tag) {
             constexpr int MODE = decltype(mode_tag)::value;
             if (a.epi == 0)
@@ -555,7 +542,11 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
             else
                 run_tile<PT, MODE, HE, 2>(a, c, now, wave, n_waves, g_first, g_count);
         };
-        if (!fast)
+        // every path to the end of the tile settles the request: a set does before its stores, a wavefront
+        // without a set does here
+        if (wave >= a.n_sets)
+            settle();
+        else if (!fast)
             go(std::integral_constant<int, -1>{});
         else if (HE)
             use_lsh ? go(std::integral_constant<int, 5>{}) : go(std::integral_constant<int, 6>{});
@@ -624,20 +615,14 @@ TiledPlan tiled_plan(const ConvGeom &g, const void *in, const void *filter, int 
         while (cs_units % 4 != 2)
             cs_units++;
     const int cs = 16 * cs_units;
-    const bool flat = g.stride_h == 1 && g.stride_w == 1;
-    const int s = g.stride_w;
     const int span_h = (g.k_h - 1) * g.dil_h, span_w = (g.k_w - 1) * g.dil_w;
 
     for (int chunks = 1; chunks <= n_groups; chunks++) {
         const int gpc = (n_groups + chunks - 1) / chunks;
         if ((n_groups + gpc - 1) / gpc != chunks)
             continue;
-        // Filters in several chunks mean every chunk's workgroups copy the same patch again.  At stride 1 that
-        // still beats reading operand B from global memory tap by tap; a strided convolution reads each input
-        // byte about twice there, and the direct kernel is faster (measured on 80 x 80 x 64 -> 128 and
-        // 40 x 40 x 128 -> 256 at stride 2: 28 and 51 us against 35 and 61 us at batch 64).
-        if (chunks > 1 && s > 1)
-            break;
+        // (filters in several chunks mean every chunk's workgroups copy the same patch again; that still beats
+        // reading operand B from global memory tap by tap)
         const int w_bytes = gpc * ksteps * 4096;
         const int koff_pitch = round_up(ksteps + 4, 4);
         const int tab_bytes = gpc * 768 + koff_pitch * 16 + 256;
@@ -648,37 +633,34 @@ TiledPlan tiled_plan(const ConvGeom &g, const void *in, const void *filter, int 
             const int tw = (g.out_w + ncol - 1) / ncol;
             if (ncol > 1 && tw < 16)
                 break;
-            const int pw = (tw - 1) * s + span_w + 1;
-            const int pwp = (pw + s - 1) / s;
-            const int vrow = flat ? pw : round_up(tw, 16);
+            const int pw = tw + span_w;
             for (int th = 1; th <= g.out_h; th++) {
-                const int ph = (th - 1) * g.stride_h + span_h + 1;
-                const int px_alloc = ph * s * pwp + 16 + span_w + 1;
-                const long long patch_bytes = (long long)px_alloc * cs;
-                const long long lds = w_bytes + tab_bytes + patch_bytes;
-                if (lds > kLdsLimit)
+                const int ph = th + span_h;
+                if ((long long)w_bytes + tab_bytes + (long long)(ph * pw + 16 + span_w + 1) * cs > kLdsLimit)
                     break;
-                const int n_ptiles = (th * vrow + 15) / 16;
+                const int n_ptiles = (th * pw + 15) / 16;
                 const int tiles_y = (g.out_h + th - 1) / th;
                 const long long n_tiles = (long long)g.batch * tiles_y * ncol;
                 const int row_units = pw * cu16;
                 for (int vi = 0; vi < kNumVariants; vi++) {
                     const Variant &var = kVariants[vi];
-                    // a strided convolution re-reads little through the direct kernel; the staged form only wins
-                    // there with two workgroups per compute unit (160 x 160 x 64 -> 64 at stride 2, batch 64:
-                    // 47 us direct, 63 us with one workgroup of eight wavefronts)
-                    if (s > 1 && var.max_per_cu < 2)
-                        continue;
                     const int PT = var.pt, threads = var.threads, kUnitsMax = var.umax;
                     const int n_sets = (n_ptiles + PT - 1) / PT;
                     const int waves = threads / 64;
                     if (row_units > threads)
                         continue;
                     const int row_par = std::min(threads / row_units, ph);
-                    if ((ph + row_par - 1) / row_par > kUnitsMax)
+                    const int row_groups = (ph + row_par - 1) / row_par;
+                    if (row_groups > kUnitsMax)
+                        continue;
+                    // the patch in LDS: every thread writes row_groups rows, and the pixel tiles of the flattened
+                    // patch run up to 16 + span_w positions past its last row
+                    const int px_alloc = std::max(row_groups * row_par, ph) * pw + 16 + span_w + 1;
+                    const long long lds = (long long)w_bytes + tab_bytes + (long long)px_alloc * cs;
+                    if (lds > kLdsLimit)
                         continue;
                     const int per_cu = std::min<long long>(var.max_per_cu, kLdsLimit / lds);
-                    if (per_cu < 1 || (s > 1 && per_cu < 2))
+                    if (per_cu < 1)
                         continue;
                     // matrix-instruction time of a tile: the slowest wavefront's sets (k steps x 4 PT instructions
                     // per 64 filters), plus a per-set epilogue and a per-tile fixed cost (barriers, patch copy)
@@ -709,11 +691,8 @@ TiledPlan tiled_plan(const ConvGeom &g, const void *in, const void *filter, int 
                         a.tw = tw;
                         a.ph = ph;
                         a.pw = pw;
-                        a.pwp = pwp;
                         a.cs = cs;
                         a.cu16 = cu16;
-                        a.flat = flat ? 1 : 0;
-                        a.vrow = vrow;
                         a.n_ptiles = n_ptiles;
                         a.n_sets = n_sets;
                         a.tiles_x = ncol;
@@ -721,8 +700,10 @@ TiledPlan tiled_plan(const ConvGeom &g, const void *in, const void *filter, int 
                         a.n_tiles = (int)std::min<long long>(n_tiles, 0x7fffffff);
                         a.row_units = row_units;
                         a.row_par = row_par;
+                        a.row_groups = row_groups;
                         a.src_row_step = row_par * g.in_w * g.in_pitch;
-                        a.lds_row_step = row_par * s * pwp * cs;
+                        a.lds_row_step = row_par * pw * cs;
+                        a.img_bytes = g.in_h * g.in_w * g.in_pitch;
                         a.off_tabs = w_bytes;
                         a.off_koff = w_bytes + gpc * 768;
                         a.off_lut = a.off_koff + koff_pitch * 16;
@@ -814,9 +795,7 @@ hipError_t launch_conv2d_s8_tiled(const ConvGeom &g, const int8_t *in, const int
         : 2;
     a.fd_cu16 = make_fastdiv((unsigned)a.cu16);
     a.fd_row_units = make_fastdiv((unsigned)a.row_units);
-    a.fd_sw = make_fastdiv((unsigned)g.stride_w);
-    a.fd_vrow = make_fastdiv((unsigned)a.vrow);
-    a.fd_vrow16 = make_fastdiv((unsigned)std::max(1, a.vrow / 16));
+    a.fd_pw = make_fastdiv((unsigned)a.pw);
     a.fd_tiles_x = make_fastdiv((unsigned)a.tiles_x);
     a.fd_tiles_yx = make_fastdiv((unsigned)(a.tiles_y * a.tiles_x));
     static const bool trace = getenv("ESPDL_HIP_TRACE") != nullptr;
