@@ -60,24 +60,26 @@ def _vgprs(text):
     return regs
 
 
-def check_tiled_patch_registers(asm_path):
-    """conv2d_s8_tiled.hip loads the pieces of the next input patch with buffer loads written as asm statements
-    and waits for them by hand, so the compiler does not know that the destination registers are in flight.
-    This reads the generated code of every conv2d_s8_tiled_kernel instance and fails the build unless
-      * the kernel has no vector register spills, and
-      * from the first load into a piece register to the end of the kernel that register is named only by the
-        loads of the piece, by the LDS write of the piece (as data) and by the few instructions right in front of
+def check_hand_waited_loads(asm_path, kernel, expected_regs):
+    """conv2d_s8_tiled.hip and depthwise_s8_lds.hip load the pieces of the next input patch with buffer loads
+    written as asm statements and wait for them by hand, so the compiler does not know that the destination
+    registers are in flight.  This reads the generated code of every instance of `kernel` and fails the build
+    unless
+      * the instance has no vector register spills, and
+      * from the first load into a piece register to the end of the instance that register is named only by the
+        loads of the piece, by the LDS write of the piece (as data) and by the instructions shortly in front of
         a load that compute its address in the load's own destination (the piece in it was written to LDS before).
+    `expected_regs`: piece registers an instance with such loads must have (instances without any are skipped:
+    builds of the kernel that fetch their input another way).
     """
     lines = open(asm_path).read().splitlines()
-    starts = [i for i, l in enumerate(lines) if re.match(r"^_ZN5espdl\S*conv2d_s8_tiled_kernel\S*:", l)]
+    starts = [i for i, l in enumerate(lines) if re.match(r"^_ZN5espdl\S*%s\S*:" % kernel, l)]
     if not starts:
-        raise RuntimeError("%s: no conv2d_s8_tiled_kernel in the generated code" % asm_path)
-    spills = re.findall(r"\.vgpr_spill_count:\s*(\d+)", "\n".join(lines))
+        raise RuntimeError("%s: no %s in the generated code" % (asm_path, kernel))
     problems = []
-    if any(int(n) for n in spills):
-        problems.append("vector register spills: %s" % spills)
+    checked = 0
     for st in starts:
+        name = lines[st].split(":")[0]
         end = next(i for i in range(st, len(lines)) if "s_endpgm" in lines[i])
         body = lines[st:end]
         loads, first = {}, {}
@@ -87,8 +89,15 @@ def check_tiled_patch_registers(asm_path):
                 loads[i] = set(range(int(m.group(1)), int(m.group(2)) + 1))
                 for r in loads[i]:
                     first.setdefault(r, i)
-        if len(first) != 32:
-            problems.append("%s: %d piece registers, expected 32" % (lines[st].split(":")[0], len(first)))
+        if not first:
+            continue
+        checked += 1
+        meta = "\n".join(lines[next(i for i, l in enumerate(lines) if ".name:" in l and name in l):][:12])
+        m = re.search(r"\.vgpr_spill_count:\s*(\d+)", meta)
+        if m is None or int(m.group(1)) != 0:
+            problems.append("%s: vector register spills (%s)" % (name, m.group(1) if m else "count not found"))
+        if len(first) != expected_regs:
+            problems.append("%s: %d piece registers, expected %d" % (name, len(first), expected_regs))
         load_lines = sorted(loads)
         for i, l in enumerate(body):
             if not l.startswith("\t") or l.lstrip().startswith((";", ".")):
@@ -103,17 +112,22 @@ def check_tiled_patch_registers(asm_path):
                 m = re.search(r"ds_write_b128 v(\d+), v\[(\d+):(\d+)\]", l)
                 if m and int(m.group(1)) not in named:
                     continue
-            # address arithmetic in the destination of a load that follows within sixteen lines
-            ahead = [j for j in load_lines if i < j <= i + 16]
+            # address arithmetic in the destination of a load that follows within eighty lines
+            ahead = [j for j in load_lines if i < j <= i + 80]
             if ahead and all(any(r in loads[j] for j in ahead) for r in named):
                 continue
             problems.append("%s line %d touches a piece register: %s" % (os.path.basename(asm_path), st + i + 1, l.strip()))
+    if not checked:
+        problems.append("no instance of %s has hand-waited loads" % kernel)
     if problems:
-        raise RuntimeError("conv2d_s8_tiled.hip: generated code breaks what its hand-placed waits assume:\n  " +
-                           "\n  ".join(problems[:20]))
+        raise RuntimeError("%s: generated code breaks what the hand-placed waits assume:\n  %s"
+                           % (os.path.basename(asm_path), "\n  ".join(problems[:20])))
 
 
-CHECKED_ASM = {"conv2d_s8_tiled.hip": check_tiled_patch_registers}
+CHECKED_ASM = {
+    "conv2d_s8_tiled.hip": lambda path: check_hand_waited_loads(path, "conv2d_s8_tiled_kernel", 32),
+    "depthwise_s8_lds.hip": lambda path: check_hand_waited_loads(path, "depthwise_s8_lds_kernel", 20),
+}
 
 
 def build_kernels(verbose=True):

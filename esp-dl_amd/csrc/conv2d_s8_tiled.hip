@@ -379,7 +379,7 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     //   * between a request and settle() nothing may read or move a piece.  The compiler sees the pieces as
     //     values defined by request() and used by deposit(), keeps them in their registers over the tile and has no
     //     reason to touch them; the build checks in the generated code that it did not, and that the kernels have
-    //     no register spills (build.py: check_tiled_patch_registers);
+    //     no register spills (build.py: check_hand_waited_loads);
     //   * the descriptor may have been moved into its scalar registers by vector instructions right before a load,
     //     and a memory instruction may read such a register five wait states later at the earliest: the
     //     compiler pads its own instructions, not the text of an asm statement, hence the s_nop.

@@ -57,6 +57,7 @@ struct DwLdsArgs {
     int8_t *out;
     ConvGeom g;
     int taps;
+    int img_bytes;      // bytes of one image of the input tensor
     int row3;           // 1: windows of 3 columns and at most 3 rows take one k step per window row (slots kx 0, 1, 2, 2)
     int ks_used;        // k steps that hold taps
     int th, tw;         // output tile, pixels
@@ -112,20 +113,46 @@ __device__ __forceinline__ UnitPos dw_unit(const DwLdsArgs &a, int unit)
 }
 
 // Patch chunks of this thread for one tile: global -> registers (zeros outside the image).
+//
+// The loads and the wait for them (dw_settle) are written as instructions.  The chunks are used at the top of
+// the next iteration of the tile loop, after this tile's stores; a wavefront's loads and stores share one
+// counter, and the compiler, for which the two kinds may complete in any order, waits there for the counter to
+// reach zero - for the stores just issued as well, so no tile's stores would overlap the next tile's work.
+// dw_settle() waits in front of the stores instead (the loads have had the whole compute phase to arrive) and
+// nothing waits where the chunks are used.  What the compiler does not know any more has to hold by
+// construction:
+//   * between dw_fetch and dw_settle nothing may read or move a chunk.  The compiler sees the chunks as values
+//     defined here and used by the LDS writes at the top of the loop and has no reason to touch them; the build
+//     checks in the generated code that it did not (build.py: check_hand_waited_loads);
+//   * the loads go through a buffer descriptor of the tile's image, and a chunk outside the image gets an offset
+//     past the descriptor's end and comes back as zeros: no branch around a load, no select behind it;
+//   * the descriptor may have been moved into its scalar registers by vector instructions right before a load,
+//     and a memory instruction may read such a register five wait states later at the earliest: the compiler
+//     pads its own instructions, not the text of an asm statement, hence the s_nop.
 __device__ __forceinline__ void dw_fetch(const DwLdsArgs &a, const UnitPos &u, int cc0, const int (&rel)[kMaxIn],
                                          const int (&rc)[kMaxIn], v4i (&pv)[kMaxIn])
 {
     const ConvGeom &g = a.g;
     const int iy0 = u.y0 * g.stride_h - g.pad_top, ix0 = u.x0 * g.stride_w - g.pad_left;
-    const int8_t *base = a.in + (((long long)u.n * g.in_h + iy0) * g.in_w + ix0) * g.in_c + cc0;
+    // buffer descriptor: base, stride 0, bytes, 32-bit raw format
+    const __amdgpu_buffer_rsrc_t img = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<int8_t *>(a.in + (long long)u.n * a.img_bytes + cc0), (short)0, a.img_bytes - cc0, 0x00020000);
+    const int org = (iy0 * g.in_w + ix0) * g.in_c;
 #pragma unroll
     for (int i = 0; i < kMaxIn; i++) {
         if (i * kThreads < a.n_in_chunks) { // uniform
             const int iy = iy0 + (rc[i] & 0xffff), ix = ix0 + (rc[i] >> 16);
             const bool ok = rc[i] >= 0 && (unsigned)iy < (unsigned)g.in_h && (unsigned)ix < (unsigned)g.in_w;
-            pv[i] = ok ? *reinterpret_cast<const v4i *>(base + rel[i]) : v4i{0, 0, 0, 0};
+            const int off = ok ? org + rel[i] : (int)0x80000000u;
+            asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(pv[i]) : "v"(off), "s"(img));
         }
     }
+}
+
+// Wait for the wavefront's outstanding vector-memory instructions, as an instruction of its own.
+__device__ __forceinline__ void dw_settle()
+{
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 // Block-input patch dwords of this thread for one tile (expand form): global -> registers.
@@ -567,6 +594,8 @@ __global__ __launch_bounds__(kThreads, KS > kKs ? 2 : 4) void depthwise_s8_lds_k
         __syncthreads(); // the cleared patch must not overtake the first tile's stores below
     }
 
+    if (!EXP)
+        dw_settle(); // the first patch
     for (; unit < seq.end; unit += seq.step) {
         // patch of this tile: registers -> LDS
         if (EXP) {
@@ -651,7 +680,9 @@ __global__ __launch_bounds__(kThreads, KS > kKs ? 2 : 4) void depthwise_s8_lds_k
             __syncthreads();
         }
 
-        // result tile: LDS -> global, consecutive pieces
+        // result tile: LDS -> global, consecutive pieces; the next patch has arrived before the first store
+        if (!EXP)
+            dw_settle();
         const int rows = min(a.th, g.out_h - u_cur.y0), cols = min(a.tw, g.out_w - u_cur.x0);
         if (PROJ) {
             const DwProject &pj = a.pj;
@@ -733,6 +764,8 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr, const Dw
     }
     cand_h.push_back(g.out_h);
     cand_w.push_back(g.out_w);
+    if ((long long)g.in_h * g.in_w * g.in_c >= (1ll << 31)) // chunk offsets inside an image are 32-bit
+        return best;
     const bool proj = pj != nullptr && pj->w != nullptr;
     int p_nrt = 0, p_ks = 0, p_os = 0, p_vec = 16, p_vecs = 0;
     if (proj) {
@@ -801,6 +834,7 @@ DwLdsPlan dw_lds_plan(const ConvGeom &g, const DwProject *pj = nullptr, const Dw
                     best.ok = true;
                     DwLdsArgs &a = best.a;
                     a.taps = taps;
+                    a.img_bytes = g.in_h * g.in_w * g.in_c;
                     a.row3 = (g.k_w == 3 && g.k_h <= kKs && ks_steps == kKs) ? 1 : 0;
                     a.ks_used = a.row3 ? g.k_h : (taps + 3) / 4;
                     a.th = the;
