@@ -64,7 +64,7 @@ struct TiledArgs {
     int src_row_step;    // bytes between the input rows of a thread's consecutive pieces (row_par rows)
     int lds_row_step;    // the same in the LDS patch
     int img_bytes;       // bytes of one image of the input tensor
-    int off_tabs, off_koff, off_lut, off_patch; // LDS offsets (filters at 0)
+    int off_tabs, off_koff, off_lut, off_pix, off_patch; // LDS offsets (filters at 0)
     int out_vec;
     int epi;             // epilogue form: 0 plain 16-byte stores, 1 the same with table / residual, 2 general
     int koff_pitch;      // ints per lane-group row of the step-offset table
@@ -78,27 +78,22 @@ __device__ __forceinline__ int group_tiles(int out_c, int gbase)
 }
 
 struct TileRef {
-    long long img_in, img_out, img_res; // byte offsets of the tile's image in the input, output and residual tensors
-    int oy0, ox0, iy0, ix0, th_real, tw_real;
+    long long img_out, img_res; // byte offsets of the tile's image in the output and residual tensors
+    int oy0, ox0, th_real, tw_real;
 };
 
-__device__ __forceinline__ TileRef decode_tile(const TiledArgs &a, int tile)
+// Image and tile position of a tile index.
+struct TilePos {
+    int n, ty, tx;
+};
+
+__device__ __forceinline__ TilePos locate_tile(int tile, const FastDiv &fd_yx, const FastDiv &fd_x)
 {
-    const ConvGeom &g = a.g;
-    const unsigned n = fastdiv((unsigned)tile, a.fd_tiles_yx);
-    const unsigned rem = (unsigned)tile - n * a.fd_tiles_yx.d;
-    const unsigned ty = fastdiv(rem, a.fd_tiles_x);
-    const unsigned tx = rem - ty * a.fd_tiles_x.d;
-    TileRef t;
-    t.img_in = (long long)n * g.in_h * g.in_w * g.in_pitch;
-    t.img_out = (long long)n * g.out_h * g.out_w * g.out_pitch;
-    t.img_res = (long long)n * g.out_h * g.out_w * g.res_pitch;
-    t.oy0 = (int)ty * a.th;
-    t.ox0 = (int)tx * a.tw;
-    t.iy0 = t.oy0 - g.pad_top;
-    t.ix0 = t.ox0 - g.pad_left;
-    t.th_real = min(a.th, g.out_h - t.oy0);
-    t.tw_real = min(a.tw, g.out_w - t.ox0);
+    TilePos t;
+    t.n = (int)fastdiv((unsigned)tile, fd_yx);
+    const int rem = tile - t.n * (int)fd_yx.d;
+    t.ty = (int)fastdiv((unsigned)rem, fd_x);
+    t.tx = rem - t.ty * (int)fd_x.d;
     return t;
 }
 
@@ -115,6 +110,7 @@ struct Ctx {
     const int *init_l, *shift_l, *lsh_l, *koff_l;
     const int8_t *lut_l;
     const unsigned char *patch;
+    const v4i *pix_l; // per position of the flattened patch a set can cover: {patch offset, row, column, row * out_w + column}
     int lane, col, quad;
     bool relu, has_lut;
     int floor_pk;
@@ -288,23 +284,18 @@ __device__ __forceinline__ void run_tile(const TiledArgs &a, const Ctx &c, const
     const int org_out = tr.oy0 * g.out_w + tr.ox0; // in pixels
     int set = wave;
     do {
-        // the pixels of a set: 16 consecutive positions of the flattened patch per pixel tile
+        // the pixels of a set: 16 consecutive positions of the flattened patch per pixel tile, from the table
         int pixoff[PT];
         int opix[PT];
         unsigned okmask = 0;
+        const v4i *pix = c.pix_l + set * (PT * 16) + c.col;
 #pragma unroll
         for (int p = 0; p < PT; p++) {
-            const int tp = set * PT + p;
-            const bool live = tp < a.n_ptiles; // uniform
-            const int tpc = live ? tp : 0;
-            const unsigned v = (unsigned)(tpc * 16 + c.col);
-            const unsigned row = fastdiv(v, a.fd_pw);
-            const int oy_l = (int)row;
-            const int ox_l = (int)(v - row * a.fd_pw.d);
-            pixoff[p] = (int)v * a.cs;
-            const bool ok = live && oy_l < tr.th_real && ox_l < tr.tw_real;
+            const v4i e = pix[p * 16];
+            pixoff[p] = e[0];
+            const bool ok = e[1] < tr.th_real && e[2] < tr.tw_real; // (positions past the tile hold row 0x7fff)
             okmask |= ok ? 1u << p : 0u;
-            opix[p] = org_out + oy_l * g.out_w + ox_l;
+            opix[p] = org_out + e[3];
         }
         int gi = 0;
         do {
@@ -332,6 +323,171 @@ __device__ __forceinline__ void run_tile(const TiledArgs &a, const Ctx &c, const
     } while (set < a.n_sets);
 }
 
+// A value in a scalar register of its own.  Kernel arguments arrive in groups of eight or sixteen registers, and
+// a group that does not stay resident over the tile loop is fetched back whole for every use of one member.
+template <typename T>
+__device__ __forceinline__ T lone(T v)
+{
+    asm volatile("" : "+s"(v));
+    return v;
+}
+
+// Copying a patch: a thread owns ONE 16-byte column piece (patch column px, channels 16 cu ...) and walks the
+// patch rows r0, r0 + row_par, ...: row_groups pieces, the same count for every thread (the LDS patch is that
+// many rows tall; rows past the patch are never read).  Everything about the column is computed once per kernel.
+// The loads go through a buffer descriptor of the tile's image: a piece outside the image gets an offset past
+// the descriptor's end and comes back as zeros (the reference's window clipping), so there is one form for inner
+// and border tiles and nothing to patch up when the pieces are written to LDS.  The pieces of the NEXT tile are
+// requested before the current tile is computed and written to LDS after it.
+//
+// The loads and the wait for them are written as instructions.  The pieces are used after the tile's stores; a
+// wavefront's loads and stores share one counter, and the compiler, for which the two kinds may complete in
+// any order, waits for that counter to reach zero where the pieces are written to LDS - for the stores just
+// issued as well - or, when the set loop reuses a piece register, in front of that loop, right after the
+// request (measured on 56 x 56 x 64 -> 64 at batch 256: 48.8 and 46.9 us per launch; this form 43.3 us).
+// settle() waits before the first store that follows a request instead - by then the loads have had the
+// products of a set to arrive - and nothing waits where the pieces are used.  What the compiler does not
+// know any more has to hold by construction:
+//   * between a request and settle() nothing may read or move a piece.  The compiler sees the pieces as
+//     values defined by request() and used by deposit(), keeps them in their registers over the tile and has no
+//     reason to touch them; the build checks in the generated code that it did not, and that the kernels have
+//     no register spills (build.py: check_hand_waited_loads);
+//   * the descriptor may have been moved into its scalar registers by vector instructions right before a load,
+//     and a memory instruction may read such a register five wait states later at the earliest: the
+//     compiler pads its own instructions, not the text of an asm statement, hence the s_nop.
+template <int UMAX>
+struct Stager {
+    int r0, px;       // first patch row and patch column of the thread's pieces
+    bool active;      // the thread has pieces
+    int src0, dst0;   // byte offset of piece 0 from the patch origin in the image / in the LDS patch
+    v4u pre[UMAX];
+
+    __device__ __forceinline__ void init(const TiledArgs &a, int tid)
+    {
+        const ConvGeom &g = a.g;
+        r0 = (int)fastdiv((unsigned)tid, a.fd_row_units);
+        const int ru = tid - r0 * a.row_units;
+        active = r0 < a.row_par;
+        px = (int)fastdiv((unsigned)ru, a.fd_cu16);
+        const int cu = ru - px * a.cu16;
+        src0 = (r0 * g.in_w + px) * g.in_pitch + 16 * cu;
+        dst0 = (r0 * a.pw + px) * a.cs + 16 * cu;
+    }
+    // Pieces of the patch whose first pixel is (iy0, ix0) of the image at `img`.  When all patch rows lie inside the
+    // image, the row of a piece goes into the instruction's scalar offset and the pieces share one vector offset;
+    // else a piece's offset is computed and tested per thread.  Offsets handed to the hardware are never negative
+    // (a negative vector offset would not wrap against the scalar one: the unit adds them to a 48-bit base).
+    // One asm statement per piece serves both forms, so that a piece has one register whatever the form.
+    __device__ __forceinline__ void request(const int8_t *img, int img_bytes, int iy0, int ix0, int in_h, int in_w,
+                                            int in_pitch, int row_groups, int row_par, int src_row_step)
+    {
+        // buffer descriptor: base, stride 0, bytes, 32-bit raw format
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(img), (short)0, img_bytes, 0x00020000);
+        constexpr int kParked = (int)0x80000000u; // past the end of any image: the load returns zeros
+        const int org = (iy0 * in_w + ix0) * in_pitch;
+        const bool xok = active && (unsigned)(ix0 + px) < (unsigned)in_w;
+        int off[UMAX];
+        int sstep;
+        if (iy0 >= 0 && iy0 + row_groups * row_par <= in_h) { // uniform
+            const int voff = xok ? org + src0 : kParked;
+#pragma unroll
+            for (int j = 0; j < UMAX; j++)
+                off[j] = voff;
+            sstep = src_row_step;
+        } else {
+            const int row = iy0 + r0;
+#pragma unroll
+            for (int j = 0; j < UMAX; j++) {
+                const bool ok = xok && (unsigned)(row + j * row_par) < (unsigned)in_h;
+                off[j] = ok ? org + src0 + j * src_row_step : kParked;
+            }
+            sstep = 0;
+        }
+#pragma unroll
+        for (int j = 0; j < UMAX; j++)
+            if (j < row_groups) // uniform
+                asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, %3 offen"
+                             : "=v"(pre[j])
+                             : "v"(off[j]), "s"(rsrc), "s"(j * sstep));
+    }
+    __device__ __forceinline__ void deposit(unsigned char *patch, int row_groups, int lds_row_step) const
+    {
+        if (active) {
+#pragma unroll
+            for (int j = 0; j < UMAX; j++)
+                if (j < row_groups) // uniform
+                    *reinterpret_cast<v4u *>(patch + dst0 + j * lds_row_step) = pre[j];
+        }
+    }
+};
+
+// The tile loop of a workgroup.
+template <int PT, int UMAX, bool HE>
+__device__ __forceinline__ void tile_loop(const TiledArgs &a, const Ctx &c, Stager<UMAX> &st, unsigned char *patch,
+                                          const TileSeq &seq, TilePos pos, int wave, int n_waves, int g_first, int g_count,
+                                          bool fast, bool use_lsh)
+{
+    const ConvGeom &g = a.g;
+    // every scalar the loop uses, in a register of its own
+    const int8_t *const in = lone(a.in);
+    const int img_bytes = lone(a.img_bytes);
+    const int in_h = lone(g.in_h), in_w = lone(g.in_w), in_pitch = lone(g.in_pitch);
+    const int pad_top = lone(g.pad_top), pad_left = lone(g.pad_left);
+    const int th = lone(a.th), tw = lone(a.tw);
+    const int row_groups = lone(a.row_groups), row_par = lone(a.row_par);
+    const int src_row_step = lone(a.src_row_step), lds_row_step = lone(a.lds_row_step);
+    const int n_tiles_yx = lone((int)a.fd_tiles_yx.d), n_tiles_x = lone((int)a.fd_tiles_x.d);
+    const FastDiv fd_yx = {lone(a.fd_tiles_yx.m), lone(a.fd_tiles_yx.s), (unsigned)n_tiles_yx};
+    const FastDiv fd_x = {lone(a.fd_tiles_x.m), lone(a.fd_tiles_x.s), (unsigned)n_tiles_x};
+    const int step = lone(seq.step), end = lone(seq.end);
+    int tile = lone(seq.first);
+    const bool idle = wave >= a.n_sets; // a wavefront without a set in the tiles of this layer only copies
+    const int epi = lone(a.epi);
+
+    const auto request = [&](const TilePos &t) {
+        st.request(in + (long long)t.n * img_bytes, img_bytes, t.ty * th - pad_top, t.tx * tw - pad_left, in_h, in_w,
+                   in_pitch, row_groups, row_par, src_row_step);
+    };
+    settle(); // the first patch, requested before the set-up (and whatever the set-up left in flight)
+    for (; tile < end; tile += step) {
+        st.deposit(patch, row_groups, lds_row_step);
+        __syncthreads(); // patch (and, the first time, filters and tables) complete
+        TileRef now;
+        now.img_out = (long long)pos.n * g.out_h * g.out_w * g.out_pitch;
+        now.img_res = (long long)pos.n * g.out_h * g.out_w * g.res_pitch;
+        now.oy0 = pos.ty * th;
+        now.ox0 = pos.tx * tw;
+        now.th_real = min(th, g.out_h - now.oy0);
+        now.tw_real = min(tw, g.out_w - now.ox0);
+        const int next = tile + step;
+        if (next < end) {
+            pos = locate_tile(next, fd_yx, fd_x);
+            request(pos);
+        }
+        // every path to the end of the tile settles the request: a set does before its stores, a wavefront
+        // without a set does here
+        const auto go = [&](auto mode_tag) {
+            constexpr int MODE = decltype(mode_tag)::value;
+            if (epi == 0)
+                run_tile<PT, MODE, HE, 0>(a, c, now, wave, n_waves, g_first, g_count);
+            else if (epi == 1)
+                run_tile<PT, MODE, HE, 1>(a, c, now, wave, n_waves, g_first, g_count);
+            else
+                run_tile<PT, MODE, HE, 2>(a, c, now, wave, n_waves, g_first, g_count);
+        };
+        if (idle)
+            settle();
+        else if (!fast)
+            go(std::integral_constant<int, -1>{});
+        else if (HE)
+            use_lsh ? go(std::integral_constant<int, 5>{}) : go(std::integral_constant<int, 6>{});
+        else
+            use_lsh ? go(std::integral_constant<int, 1>{}) : go(std::integral_constant<int, 0>{});
+        __syncthreads(); // every wavefront is done with the patch
+    }
+}
+
 // PT: pixel tiles per set; UMAX: 16-byte pieces of the next patch a thread holds in registers; MAXT / MINB:
 // largest workgroup and how many of them share a compute unit (which caps the registers of a wavefront).
 template <int PT, int UMAX, int MAXT, int MINB, bool HE>
@@ -347,6 +503,7 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     int *lsh_l = shift_l + gpc * 64;
     int *koff_l = reinterpret_cast<int *>(smem + a.off_koff);
     int8_t *lut_l = reinterpret_cast<int8_t *>(smem + a.off_lut);
+    v4i *pix_l = reinterpret_cast<v4i *>(smem + a.off_pix);
     unsigned char *patch = smem + a.off_patch;
 
     const int tid = threadIdx.x, nthreads = blockDim.x;
@@ -358,65 +515,14 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     const bool has_lut = a.lut != nullptr;
 
     const TileSeq seq = xcd_tile_sequence(a.n_tiles);
-    int tile = seq.first;
-
-    // Copying a patch: a thread owns ONE 16-byte column piece (patch column st_px, channels 16 st_cu ...) and
-    // walks the patch rows r0, r0 + row_par, ...: row_groups pieces, the same count for every thread (the LDS
-    // patch is that many rows tall; rows past the patch are never read).  Everything about the column is computed
-    // once per kernel.  The loads go through a buffer descriptor of the tile's image: a piece outside the image
-    // gets an offset past the descriptor's end and comes back as zeros (the reference's window clipping), so
-    // there is one form for inner and border tiles and nothing to patch up when the pieces are written to LDS.
-    // The pieces of the NEXT tile are requested before the current tile is computed and written to LDS after it.
-    //
-    // The loads and the wait for them are written as instructions.  The pieces are used after the tile's stores; a
-    // wavefront's loads and stores share one counter, and the compiler, for which the two kinds may complete in
-    // any order, waits for that counter to reach zero where the pieces are written to LDS - for the stores just
-    // issued as well - or, when the set loop reuses a piece register, in front of that loop, right after the
-    // request (measured on 56 x 56 x 64 -> 64 at batch 256: 48.8 and 46.9 us per launch; this form 43.3 us).
-    // settle() waits before the first store that follows a request instead - by then the loads have had the
-    // products of a set to arrive - and nothing waits where the pieces are used.  What the compiler does not
-    // know any more has to hold by construction:
-    //   * between a request and settle() nothing may read or move a piece.  The compiler sees the pieces as
-    //     values defined by request() and used by deposit(), keeps them in their registers over the tile and has no
-    //     reason to touch them; the build checks in the generated code that it did not, and that the kernels have
-    //     no register spills (build.py: check_hand_waited_loads);
-    //   * the descriptor may have been moved into its scalar registers by vector instructions right before a load,
-    //     and a memory instruction may read such a register five wait states later at the earliest: the
-    //     compiler pads its own instructions, not the text of an asm statement, hence the s_nop.
-    const unsigned r0 = fastdiv((unsigned)tid, a.fd_row_units);
-    const int ru = tid - (int)r0 * a.row_units;
-    const bool st_active = (int)r0 < a.row_par;
-    const unsigned st_px = fastdiv((unsigned)ru, a.fd_cu16);
-    const int st_cu = ru - (int)st_px * a.cu16;
-    const int st_src0 = ((int)r0 * g.in_w + (int)st_px) * g.in_pitch + 16 * st_cu;
-    const int st_dst0 = ((int)r0 * a.pw + (int)st_px) * a.cs + 16 * st_cu;
-    v4u pre[kUnitsMax];
-    auto request = [&](const TileRef &t, int row_groups) {
-        // buffer descriptor: base, stride 0, bytes, 32-bit raw format
-        const __amdgpu_buffer_rsrc_t img = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<int8_t *>(a.in + t.img_in), (short)0, a.img_bytes, 0x00020000);
-        const int org = (t.iy0 * g.in_w + t.ix0) * g.in_pitch;
-        const bool xok = st_active && (unsigned)(t.ix0 + (int)st_px) < (unsigned)g.in_w;
-        const int row = t.iy0 + (int)r0;
-        const int src = org + st_src0;
-#pragma unroll
-        for (int j = 0; j < kUnitsMax; j++)
-            if (j < row_groups) { // uniform
-                const bool ok = xok && (unsigned)(row + j * a.row_par) < (unsigned)g.in_h;
-                const int off = ok ? src + j * a.src_row_step : (int)0x80000000u;
-                asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(pre[j]) : "v"(off), "s"(img));
-            }
-    };
-    auto deposit = [&](int row_groups) {
-        if (st_active) {
-#pragma unroll
-            for (int j = 0; j < kUnitsMax; j++)
-                if (j < row_groups) // uniform
-                    *reinterpret_cast<v4u *>(patch + st_dst0 + j * a.lds_row_step) = pre[j];
-        }
-    };
-    if (tile < seq.end)
-        request(decode_tile(a, tile), a.row_groups);
+    Stager<kUnitsMax> st;
+    st.init(a, tid);
+    TilePos first_pos = {0, 0, 0};
+    if (seq.first < seq.end) { // in flight during the set-up
+        first_pos = locate_tile(seq.first, a.fd_tiles_yx, a.fd_tiles_x);
+        st.request(a.in + (long long)first_pos.n * a.img_bytes, a.img_bytes, first_pos.ty * a.th - g.pad_top,
+                   first_pos.tx * a.tw - g.pad_left, g.in_h, g.in_w, g.in_pitch, a.row_groups, a.row_par, a.src_row_step);
+    }
 
     // filters of this workgroup's chunk -> LDS in operand-A order: unit (group, k step, tile, lane) holds the 16
     // k positions [64 ks + 16 (lane / 16), +16) of filter row (lane % 16) of tile t; filter rows are permuted
@@ -460,6 +566,14 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
             off = (ky * g.dil_h * a.pw + kx * g.dil_w) * a.cs + c0;
         }
         koff_l[e] = off;
+    }
+    // positions of the flattened patch that the sets cover: patch offset, output row and column inside the tile
+    // (0x7fff: not a pixel of any tile), pixel offset inside the image
+    for (int q = tid; q < a.n_sets * PT * 16; q += nthreads) {
+        const unsigned row = fastdiv((unsigned)q, a.fd_pw);
+        const int ox_l = q - (int)row * a.pw;
+        const bool live = q < a.n_ptiles * 16;
+        pix_l[q] = v4i{live ? q * a.cs : 0, live ? (int)row : 0x7fff, ox_l, (int)row * g.out_w + ox_l};
     }
     // Can the chunk's filters take the short epilogue?  Every shift in 1..31, and bias + 2^(s-1) plus the
     // largest sum of products must fit int32 also after the left shift by max(0, 8 - s) of the short form.
@@ -511,6 +625,7 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     c.koff_l = koff_l;
     c.lut_l = lut_l;
     c.patch = patch;
+    c.pix_l = pix_l;
     c.lane = lane;
     c.col = lane & 15;
     c.quad = lane >> 4;
@@ -518,42 +633,7 @@ __global__ __launch_bounds__(MAXT, MINB) void conv2d_s8_tiled_kernel(const Tiled
     c.has_lut = has_lut;
     c.floor_pk = c.relu ? 0 : (int)0x80008000u;
 
-    settle(); // the first patch
-    for (; tile < seq.end; tile += seq.step) {
-        // The piece count goes through an empty asm statement, so that the compiler compares it where it is used:
-        // a comparison per piece that is the same for every tile gets computed in front of the loop otherwise, as
-        // a lane mask in a pair of scalar registers, and with more scalars alive over the tile loop than
-        // registers to hold them, each mask then costs two vector instructions per tile to fetch back.
-        int row_groups = a.row_groups;
-        asm volatile("" : "+s"(row_groups));
-        deposit(row_groups);
-        __syncthreads(); // patch (and, the first time, filters and tables) complete
-        // tile coordinates are scalar arithmetic: recomputed rather than carried over the loop
-        const TileRef now = decode_tile(a, tile);
-        const int next = tile + seq.step;
-        if (next < seq.end)
-            request(decode_tile(a, next), row_groups);
-        const auto go = [&](auto mode_tag) {
-            constexpr int MODE = decltype(mode_tag)::value;
-            if (a.epi == 0)
-                run_tile<PT, MODE, HE, 0>(a, c, now, wave, n_waves, g_first, g_count);
-            else if (a.epi == 1)
-                run_tile<PT, MODE, HE, 1>(a, c, now, wave, n_waves, g_first, g_count);
-            else
-                run_tile<PT, MODE, HE, 2>(a, c, now, wave, n_waves, g_first, g_count);
-        };
-        // every path to the end of the tile settles the request: a set does before its stores, a wavefront
-        // without a set does here
-        if (wave >= a.n_sets)
-            settle();
-        else if (!fast)
-            go(std::integral_constant<int, -1>{});
-        else if (HE)
-            use_lsh ? go(std::integral_constant<int, 5>{}) : go(std::integral_constant<int, 6>{});
-        else
-            use_lsh ? go(std::integral_constant<int, 1>{}) : go(std::integral_constant<int, 0>{});
-        __syncthreads(); // every wavefront is done with the patch
-    }
+    tile_loop<PT, UMAX, HE>(a, c, st, patch, seq, first_pos, wave, n_waves, g_first, g_count, fast, use_lsh);
 }
 
 struct TiledPlan {
@@ -656,7 +736,8 @@ TiledPlan tiled_plan(const ConvGeom &g, const void *in, const void *filter, int 
                     // the patch in LDS: every thread writes row_groups rows, and the pixel tiles of the flattened
                     // patch run up to 16 + span_w positions past its last row
                     const int px_alloc = std::max(row_groups * row_par, ph) * pw + 16 + span_w + 1;
-                    const long long lds = (long long)w_bytes + tab_bytes + (long long)px_alloc * cs;
+                    const int pix_bytes = n_sets * PT * 256;
+                    const long long lds = (long long)w_bytes + tab_bytes + pix_bytes + (long long)px_alloc * cs;
                     if (lds > kLdsLimit)
                         continue;
                     const int per_cu = std::min<long long>(var.max_per_cu, kLdsLimit / lds);
@@ -708,7 +789,8 @@ TiledPlan tiled_plan(const ConvGeom &g, const void *in, const void *filter, int 
                         a.off_koff = w_bytes + gpc * 768;
                         a.off_lut = a.off_koff + koff_pitch * 16;
                         a.koff_pitch = koff_pitch;
-                        a.off_patch = a.off_lut + 256;
+                        a.off_pix = a.off_lut + 256;
+                        a.off_patch = a.off_pix + pix_bytes;
                         best.a = a;
                         best.lds = (size_t)lds;
                         best.threads = threads;
