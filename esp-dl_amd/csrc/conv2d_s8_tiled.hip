@@ -162,6 +162,10 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
             for (int p = 0; p < PT; p++)
                 acc[p][t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[0][t], B[0][p], start[t], 0, 0, 0);
     };
+    // The products run at a raised wavefront priority: the other wavefront of the SIMD is in another phase of its
+    // tile most of the time, and its vector instructions then fill the issue slots between the matrix
+    // instructions instead of alternating with them (56 x 56 x 64 -> 64 at batch 256: 41.6 -> 40.5 us).
+    __builtin_amdgcn_s_setprio(3);
     v2i pair = *reinterpret_cast<const v2i *>(kq + 2);
     load(0, 0, kq[0]);
     if (ksteps == 1) {
@@ -185,6 +189,7 @@ __device__ __forceinline__ void run_set(const TiledArgs &a, const Ctx &c, int8_t
         if (ks < ksteps)
             products(0);
     }
+    __builtin_amdgcn_s_setprio(0);
     settle(); // the pieces of the next patch, before the first store after their request
     // epilogue: this lane owns output channels [c_lane, c_lane + 4 * NT) of pixel p * 16 + col of the set
     const int c_lane = gbase + 4 * NT * c.quad;
