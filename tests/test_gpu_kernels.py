@@ -551,6 +551,12 @@ DW_TILE_CASES = [
     ("n2_56x56x144_k3p1_per_tensor", (2, 56, 56, 144), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 9, 9, False, False, True),
     ("n1_112x112x32_k3p1", (1, 112, 112, 32), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 8, 11, False, False, False),
     ("n1_112x112x96_k3s2_tailpad", (1, 112, 112, 96), (3, 3), (2, 2), (1, 1), (0, 1, 0, 1), True, True, 8, 11, False, False, False),
+    # more tiles than resident workgroups: a workgroup walks several tiles, the next patch in flight over the
+    # current tile's stores
+    ("n80_56x56x144_k3p1_many_tiles", (80, 56, 56, 144), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, True, 8, 11, False, False, False),
+    ("n80_56x56x144_k3p1_many_tiles_halfeven", (80, 56, 56, 144), (3, 3), (1, 1), (1, 1), (1, 1, 1, 1), True, False, 6, 11, True, False, False),
+    ("n96_57x57x48_k3s2_many_tiles", (96, 57, 57, 48), (3, 3), (2, 2), (1, 1), (1, 1, 1, 1), True, True, 8, 11, False, False, False),
+    ("n64_30x30x80_k5p2_many_tiles", (64, 30, 30, 80), (5, 5), (1, 1), (1, 1), (2, 2, 2, 2), True, True, 9, 12, False, False, False),
 ]
 
 
@@ -855,6 +861,9 @@ MBCONV_CASES = [
     ("dwp_28x28_192_64_s2", (3, 28, 28, 192), None, 64, (3, 3), (2, 2), (0, 1, 0, 1), False, False, False),
     ("dwp_20x20_256_48_res_halfeven", (2, 20, 20, 256), None, 48, (3, 3), (1, 1), (1, 1, 1, 1), True, True, False),
     ("dwp_112x112_32_16", (1, 112, 112, 32), None, 16, (3, 3), (1, 1), (1, 1, 1, 1), False, False, True),
+    # the same form with more tiles than resident workgroups (several tiles per workgroup)
+    ("dwp_56x56_144_24_res_many_tiles", (80, 56, 56, 144), None, 24, (3, 3), (1, 1), (1, 1, 1, 1), True, False, False),
+    ("dwp_57x41_96_24_s2_many_tiles_halfeven", (96, 57, 41, 96), None, 24, (3, 3), (2, 2), (1, 1, 1, 1), False, True, False),
 ]
 
 
