@@ -132,8 +132,10 @@ __device__ __forceinline__ void stem_units(const StemArgs &a, const v4i (&wa)[RT
         return;
     v4i pieces[2];
     fetch_rows(unit, pieces);
-    for (; unit < a.n_units; unit += unit_step) {
-        // copied rows -> LDS, then this lane's four window rows out of them (unaligned 16-byte reads)
+    // copied rows -> LDS.  The rows of the NEXT unit are written where this unit's results are about to leave (its
+    // window rows were cut out long before): the wait for their loads then stands in front of this unit's stores
+    // and not behind them, where it would wait for the stores as well.
+    const auto rows_to_lds = [&]() {
 #pragma unroll
         for (int j = 0; j < 2; j++)
             if (pr[j] < g.k_h)
@@ -141,6 +143,10 @@ __device__ __forceinline__ void stem_units(const StemArgs &a, const v4i (&wa)[RT
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+    rows_to_lds();
+    for (; unit < a.n_units; unit += unit_step) {
+        // this lane's four window rows out of the copied rows (unaligned 16-byte reads)
         const unsigned rowid = fastdiv((unsigned)unit, a.fd_xblocks);
         const int xb = unit - (int)rowid * a.xblocks;
         v4i b[kUnitTiles];
@@ -212,10 +218,8 @@ __device__ __forceinline__ void stem_units(const StemArgs &a, const v4i (&wa)[RT
                             dst[4 * r + e] = (int8_t)(words[r] >> (8 * e));
             }
         }
+        rows_to_lds(); // (its barrier also orders the slab's writes before the reads below)
         if (staged_out) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             // piece i = 16 bytes i of the slab = piece i % RT of pixel i / RT
 #pragma unroll
             for (int j = 0; j < RT; j++) {
