@@ -124,7 +124,27 @@ def check_hand_waited_loads(asm_path, kernel, expected_regs):
                            % (os.path.basename(asm_path), "\n  ".join(problems[:20])))
 
 
+def check_m0_only_for_lds_copies(asm_path):
+    """The copies from memory straight into LDS (`buffer_load ... lds`) take their LDS address from m0, which the
+    kernel source writes by hand and the compiler knows nothing about: the generated code must not use m0 for
+    anything of its own (indexed register moves, for one), or a copy in flight would land somewhere else."""
+    problems = []
+    copies = 0
+    for n, l in enumerate(open(asm_path), 1):
+        code = l.split(";")[0]
+        if re.search(r"\bbuffer_load_dwordx4\b.*\blds\b", code):
+            copies += 1
+        if re.search(r"\bm0\b", code) and not re.match(r"\s*s_mov_b32 m0, s\d+\s*$", code):
+            problems.append("line %d: %s" % (n, code.strip()))
+    if not copies:
+        problems.append("no copy into LDS found")
+    if problems:
+        raise RuntimeError("%s: m0 is used by more than the hand-written LDS copies:\n  %s"
+                           % (os.path.basename(asm_path), "\n  ".join(problems[:20])))
+
+
 CHECKED_ASM = {
+    "mbconv_s8_wave.hip": check_m0_only_for_lds_copies,
     "conv2d_s8_tiled.hip": lambda path: check_hand_waited_loads(path, "conv2d_s8_tiled_kernel", 32),
     "depthwise_s8_lds.hip": lambda path: check_hand_waited_loads(path, "depthwise_s8_lds_kernel", 20),
 }

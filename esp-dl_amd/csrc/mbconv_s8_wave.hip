@@ -60,6 +60,7 @@ namespace {
 using namespace mbstage;
 
 constexpr int kWavesPerGroup = 4;
+constexpr int kRowRounds = 4; // ROWCONV guard-free builds: at most 64 * 4 16-byte pieces of copied image rows
 
 struct WaveArgs {
     MbconvParams p;
@@ -73,7 +74,13 @@ struct WaveArgs {
     int off_exp, off_dw, off_tab;
     int off_aop; // ROWCONV: operand A of the expand stage for every expanded channel, [exp_c][4 rows][16 bytes]
     int wave_bytes; // LDS of one wavefront (expanded patch + depthwise result); the tables are shared
-    FastDiv fd_pw, fd_tiles_x, fd_tiles_yx;
+    // ROWCONV guard-free builds: the image rows under the patch's windows, copied to the wavefront's LDS as
+    // consecutive aligned 16-byte pieces (0: the plan has no room for them)
+    int rows_n;      // image rows: (ph - 1) * es_h + ek_h
+    int rows_ppr;    // 16-byte pieces per copied row
+    int rows_rounds; // load instructions per copy: pieces / 64, rounded up
+    int off_rows;    // offset of the copied rows inside the wavefront's LDS
+    FastDiv fd_pw, fd_tiles_x, fd_tiles_yx, fd_rows_ppr;
 };
 
 // EXACT: the tile plan is exactly (NXPT pixel tiles, RT project row tiles, PT rows): no run-time guards in
@@ -125,6 +132,115 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
     // channels), so that the workgroup's set-up serves several tiles
     int mode_e = 0, mode_d = 0, mode_p = 0;
     const int tpw = ROWCONV ? a.tpw : 1;
+
+    // ROWCONV guard-free builds: the image rows under the patch's windows are copied to the wavefront's LDS as
+    // consecutive aligned 16-byte pieces, by loads that write LDS directly (no registers in between), one tile
+    // ahead: the copy for tile it + 1 is requested behind the first expand stage of tile it and has the rest of
+    // the tile to arrive; settle_rows() waits for it in front of the tile's stores (a wait behind them would
+    // wait for the stores too: one counter).  Piece i of a copy = piece i % rows_ppr of row i / rows_ppr, at
+    // 16 i in the wavefront's row area; a piece whose row lies outside the image, or that would start in front of
+    // the tensor or end behind it, gets an offset past the descriptor's end and arrives as zeros.
+    constexpr bool kRowCopy = ROWCONV && EXACT;
+    struct RowPiece {
+        int wy;        // image row
+        int lo, hi;    // bytes [lo, hi) of the piece lie inside the image row
+        int po;        // byte offset of the piece from the start of the tensor (the tensor has less than 2^30 bytes)
+        bool in_row;   // the row exists and the piece has bytes of it
+        bool loadable; // the piece lies inside the tensor as a whole
+    };
+    const int rc_img_bytes = p.img_h * p.img_w * c0;
+    const int rc_total = p.batch * rc_img_bytes;
+    const int rc_rowb = p.img_w * c0;
+    // (everything per lane in 32 bits: u = offset of the first byte the tile's windows touch, the same in every lane)
+    auto row_piece = [&](int u, int wy0, int wx0, int j, int lane_now) {
+        RowPiece q;
+        const unsigned i = (unsigned)(lane_now + 64 * j);
+        const unsigned r = fastdiv(i, a.fd_rows_ppr);
+        const int pi = (int)(i - r * a.fd_rows_ppr.d);
+        q.wy = wy0 + (int)r;
+        const int first = u + (int)r * rc_rowb;  // the first byte the windows touch in this row
+        const int mis = (int)(((unsigned)reinterpret_cast<uintptr_t>(p.in) + (unsigned)first) & 15u);
+        q.po = first - mis + 16 * pi;            // 16-byte aligned as an address
+        q.lo = first - wx0 * c0 - q.po;          // the row's first byte, relative to the piece
+        q.hi = q.lo + rc_rowb;
+        q.in_row = (int)r < a.rows_n && (unsigned)q.wy < (unsigned)p.img_h && q.hi > 0 && q.lo < 16;
+        q.loadable = q.po >= 0 && q.po + 16 <= rc_total;
+        return q;
+    };
+    auto tile_origin = [&](int it_n, int &u, int &wy0, int &wx0) {
+        const int tile_id = (group * kWavesPerGroup + wave) * tpw + it_n;
+        const int tile = min(tile_id, a.n_tiles - 1);
+        const unsigned n_img = fastdiv((unsigned)tile, a.fd_tiles_yx);
+        const unsigned rem = (unsigned)tile - n_img * a.fd_tiles_yx.d;
+        const unsigned ty = fastdiv(rem, a.fd_tiles_x);
+        const int oy0 = (int)ty * a.th, ox0 = (int)(rem - ty * a.fd_tiles_x.d) * a.tw;
+        wy0 = (oy0 * S - p.pad_top) * p.es_h - p.epad_top;
+        wx0 = (ox0 * S - p.pad_left) * p.es_w - p.epad_left;
+        u = (int)n_img * rc_img_bytes + wy0 * rc_rowb + wx0 * c0;
+    };
+    unsigned char *rows_l = smem + a.off_exp + wave * a.wave_bytes + a.off_rows;
+    auto request_rows = [&](int it_n) {
+        int u, wy0, wx0;
+        tile_origin(it_n, u, wy0, wx0);
+        const int lane_now = lane; // (what depends on the lane alone is computed once, in front of the tile loop)
+        // buffer descriptor of the whole tensor: base, stride 0, bytes, 32-bit raw format
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(p.in), (short)0, rc_total, 0x00020000);
+        const unsigned lds0 = (unsigned)reinterpret_cast<uintptr_t>(rows_l); // LDS address: the low half of the pointer
+        // m0 holds the LDS address of lane 0's piece and is read when the data arrives, so it is written once per
+        // copy, when no copy is in flight (a write to it waits for the loads that still need it), and left as it is:
+        // nothing else in these kernels uses it (the build checks that).  The rounds of a copy differ in the
+        // instruction's immediate offset, which counts for the LDS address and for the memory address alike.  The
+        // s_nops are the wait states a memory instruction needs after a vector instruction wrote its scalar
+        // operands, and after m0 was written.
+        asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0" ::"s"(lds0) : "memory");
+#pragma unroll
+        for (int j = 0; j < kRowRounds; j++)
+            if (j < a.rows_rounds) { // uniform
+                const RowPiece q = row_piece(u, wy0, wx0, j, lane_now);
+                const int off = ((q.in_row && q.loadable) ? q.po : (int)0x80000000u) - 1024 * j;
+                asm volatile("s_nop 4\n\tbuffer_load_dwordx4 %0, %1, 0 offen offset:%2 lds" ::"v"(off), "s"(rsrc), "n"(1024 * j)
+                             : "memory");
+            }
+    };
+    auto settle_rows = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+    // Pieces that hang over an end of their image row carry bytes of the neighbouring row (or lie partly outside
+    // the tensor and arrived as zeros): what lies outside the row is the convolution's padding.  Only tiles at the
+    // left or right border of the image have such pieces.
+    auto fix_row_ends = [&](int u, int wy0, int wx0) {
+        // (the lane index through an empty asm statement: what depends on it is computed here, on the few tiles
+        // that come here, and not in front of the tile loop, where it would occupy registers over every tile - this
+        // kernel has none to spare)
+        int lane_now = lane;
+        asm volatile("" : "+v"(lane_now));
+#pragma unroll
+        for (int j = 0; j < kRowRounds; j++)
+            if (j < a.rows_rounds) { // uniform
+                const RowPiece q = row_piece(u, wy0, wx0, j, lane_now);
+                if (q.in_row && (q.lo > 0 || q.hi < 16 || !q.loadable)) {
+                    v4i *slot = reinterpret_cast<v4i *>(rows_l + 16 * (lane_now + 64 * j));
+                    v4i v = {0, 0, 0, 0};
+                    if (q.loadable) {
+                        v = *slot;
+                    } else { // over an end of the tensor (first or last row of the batch only): byte by byte
+#pragma unroll 1
+                        for (int k = 0; k < 16; k++)
+                            if (q.po + k >= 0 && q.po + k < rc_total)
+                                v[k >> 2] |= (int)(unsigned char)p.in[q.po + k] << (8 * (k & 3));
+                    }
+#pragma unroll
+                    for (int dd = 0; dd < 4; dd++) {
+                        const int dl = min(max(q.lo - 4 * dd, 0), 4), dh = min(max(q.hi - 4 * dd, 0), 4);
+                        const unsigned m_lo = dl >= 4 ? 0u : 0xffffffffu << (8 * dl);
+                        const unsigned m_hi = dh >= 4 ? 0xffffffffu : (1u << (8 * dh)) - 1u;
+                        v[dd] &= (int)(m_lo & m_hi);
+                    }
+                    *slot = v;
+                }
+            }
+    };
+    if constexpr (kRowCopy)
+        request_rows(0);
     for (int it = 0; it < tpw; it++) {
     const int tile_id = (group * kWavesPerGroup + wave) * tpw + it;
     const bool has_tile = tile_id < a.n_tiles; // uniform
@@ -227,25 +343,42 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
         };
         int rx_lane = 0; // EXACT: the lane's window column, the same for every pixel tile
         if constexpr (EXACT) {
-            // guard-free builds have 16-pixel-wide patches: pixel tile = patch row, lane column = patch column,
-            // so everything about the column is computed once and a row costs one addition
+            // Guard-free builds have 16-pixel-wide patches: pixel tile = patch row, lane column = patch column.
+            // The image rows under the windows are in the wavefront's LDS (request_rows, one tile ahead); a lane
+            // cuts the window row of each of its patch pixels out of them with one unaligned 16-byte read.
             const int mx = ix0 + col;
             rx_lane = mx * p.es_w - p.epad_left;
             const bool col_valid = (unsigned)mx < (unsigned)p.in_w;
-            const int ry0 = wy0 + quad;
-            const int o0 = ry0 * rowb + rx_lane * c0 + delta, o_step = p.es_h * rowb;
             unsigned rows = 0; // uniform: patch rows inside the depthwise stage's input
 #pragma unroll
             for (int pt = 0; pt < NXPT; pt++)
                 rows |= (pt < a.ph && (unsigned)(iy0 + pt) < (unsigned)p.in_h) ? 1u << pt : 0u;
             xmask = col_valid ? rows : 0u;
+            if (it == 0)
+                settle_rows(); // later copies are waited for in front of the previous tile's stores
+            // does a piece hang over an end of its row?  (uniform)
+            if (wx0 * c0 < 15 || wx0 * c0 + 16 * a.rows_ppr > rowb) {
+                fix_row_ends((int)n * rc_img_bytes + wy0 * rowb + wx0 * c0, wy0, wx0);
+                wave_lds_sync();
+            }
+            const int pitch = 16 * a.rows_ppr;
+            // the lane's window row of patch pixel (pt, col): copied row pt * es_h + quad (rows past the filter's
+            // meet zero weights: any row will do), from byte col * es_w * c0 + the row's skew against 16 bytes
+            const unsigned skew0 = (unsigned)(reinterpret_cast<uintptr_t>(img) + (uintptr_t)((long long)wy0 * rowb + wx0 * c0));
+            // (three aligned dwords and a funnel shift: neighbouring lanes read the same or neighbouring dwords, which
+            // LDS serves in one pass; an unaligned 16-byte read per lane at a 6-byte lane pitch takes several)
 #pragma unroll
             for (int pt = 0; pt < NXPT; pt++) {
-                request(pt, o0 + pt * o_step);
-                const bool ok = quad < p.ek_h && (unsigned)(ry0 + pt * p.es_h) < (unsigned)p.img_h;
-                rowok |= ok ? 1u << pt : 0u;
+                const int r = min(pt * p.es_h + quad, a.rows_n - 1);
+                const int o = r * pitch + col * p.es_w * c0 + (int)((skew0 + (unsigned)(r * rowb)) & 15u);
+                const int *src = reinterpret_cast<const int *>(rows_l + (o & ~3));
+                const unsigned sh = (unsigned)o & 3u;
+                const int d0 = src[0], d1 = src[1], d2 = src[2];
+                xb[pt] = v4i{(int)__builtin_amdgcn_alignbyte((unsigned)d1, (unsigned)d0, sh),
+                             (int)__builtin_amdgcn_alignbyte((unsigned)d2, (unsigned)d1, sh),
+                             (int)__builtin_amdgcn_alignbyte(0u, (unsigned)d2, sh), 0};
             }
-            rowok &= xmask;
+            wave_lds_sync(); // the next tile's copy comes after these reads
         } else {
 #pragma unroll
             for (int pt = 0; pt < NXPT; pt++) {
@@ -269,7 +402,7 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
         if (EXACT && !interior)
             byte_masks3(x_bytes(rx_lane), mx3);
 #pragma unroll
-        for (int pt = 0; pt < NXPT; pt++) {
+        for (int pt = 0; pt < (EXACT ? 0 : NXPT); pt++) {
             const unsigned sh = (shs >> (2 * pt)) & 3u;
             int r[3];
             r[0] = (int)__builtin_amdgcn_alignbyte((unsigned)d[pt][1], (unsigned)d[pt][0], sh);
@@ -358,13 +491,21 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
         return w;
     };
     v4i ap[RT];
+    // (through a buffer descriptor: a piece that does not exist gets an offset past the descriptor's end and comes
+    // back as zeros.  With a plain load and a select behind it the wait for the load stands at the select, right
+    // behind the request, and every group of four chunks paid a round trip for its project filters.)
+    const __amdgpu_buffer_rsrc_t wp_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t *>(p.w_project), (short)0, p.out_c * p.exp_c, 0x00020000);
     auto load_project = [&](int sub) {
         const int kc = (sub & ~3) * 16;
         const int nk = p.exp_c - kc - 16 * quad; // valid bytes of this lane's 16 k positions
 #pragma unroll
-        for (int r = 0; r < RT; r++)
-            ap[r] = load16_partial<true>(p.w_project, (unsigned)((16 * r + col) * p.exp_c + kc + 16 * quad),
-                                         (r < n_rt && 16 * r + col < p.out_c) ? nk : 0);
+        for (int r = 0; r < RT; r++) {
+            const bool ok = r < n_rt && 16 * r + col < p.out_c && nk >= 16;
+            const int off = ok ? (16 * r + col) * p.exp_c + kc + 16 * quad : (int)0x80000000u;
+            const auto v = __builtin_amdgcn_raw_buffer_load_b128(wp_rsrc, off, 0, 0);
+            ap[r] = v4i{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
+        }
     };
     ChunkW cur;
     if constexpr (!ROWCONV)
@@ -456,6 +597,15 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
                 expand_chunk<-1, NXPT, EXACT, 1, true, PACK, CLIP>(xb, n_xpt, xmask, cur.aop, ce, floor_e, p.relu_expand != 0, HE, exp_dst, ceil_e);
         }
         wave_lds_sync();
+        if constexpr (kRowCopy)
+            if (sub == 0 && it + 1 < tpw) { // uniform
+                // The compiler counts the loads it knows and waits with vmcnt(n) for all but its n youngest; the
+                // copy's loads, which it does not know, would be among the youngest, and such a wait would wait
+                // for them.  So the loads requested so far (filters, long under way) are waited for first: the
+                // compiler's counts then never reach below what is really outstanding.
+                settle_rows();
+                request_rows(it + 1);
+            }
 
         // ---- depthwise: diagonal operands for patch rows quad (a0) and quad - 1 (a1)
         {
@@ -499,6 +649,8 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
     }
 
     // ---- project epilogue, residual Add, stores
+    if constexpr (kRowCopy)
+        settle_rows(); // the next tile's rows, before this tile's first store
     if constexpr (!kEarlyResidual)
         request_residual(); // every residual word is requested before the first is used
     // The uniform choices (epilogue form, residual or not) are made once, outside the loops over the words, and
@@ -579,6 +731,23 @@ void wave_layout(WaveArgs &a, size_t *lds)
     a.off_exp = a.off_aop + (mbconv_expand_is_pointwise(a.p) ? 0 : a.p.exp_c * 64);
     a.off_dw = a.off_exp + exp_px * 16;
     a.wave_bytes = exp_px * 16 + a.th * 16 * kDws;
+    a.rows_n = a.rows_ppr = a.rows_rounds = a.off_rows = 0;
+    if (!mbconv_expand_is_pointwise(a.p)) {
+        // a lane reads 16 bytes from byte (column * es_w * c0 + skew) of a copied row, skew < 16
+        const int rows_n = (a.ph - 1) * a.p.es_h + a.p.ek_h;
+        const int ppr = ((a.pw - 1) * a.p.es_w * a.p.in_c + 15 + 16 + 15) / 16;
+        const int rounds = (rows_n * ppr + 63) / 64;
+        const long long total = (long long)a.p.batch * a.p.img_h * a.p.img_w * a.p.in_c;
+        if (rounds <= kRowRounds && total < (1ll << 30) &&
+            (size_t)a.off_exp + (size_t)kWavesPerGroup * (a.wave_bytes + rounds * 1024) <= 80 * 1024) {
+            a.rows_n = rows_n;
+            a.rows_ppr = ppr;
+            a.rows_rounds = rounds;
+            a.off_rows = a.wave_bytes;
+            a.wave_bytes += rounds * 1024; // whole rounds: lanes past the last piece write zeros
+        }
+    }
+    a.fd_rows_ppr = make_fastdiv((unsigned)std::max(1, a.rows_ppr));
     *lds = (size_t)a.off_exp + (size_t)kWavesPerGroup * a.wave_bytes;
 }
 
@@ -642,6 +811,8 @@ WavePlan wave_plan(const MbconvParams &p)
             if (a.n_xpt > nxpt_limit)
                 break;
             a.tiles_y = (p.out_h + th - 1) / th;
+            size_t lds_unused;
+            wave_layout(a, &lds_unused); // (the guard-free build of a windowed expand stage asks for its row copy)
             const bool exact = wave_plan_has_exact_build(a);
             const double tile_cost = 1.5 * a.n_xpt + 3.0 * th + 2.0;
             const double groups = std::ceil((double)std::max(1, p.batch) * a.tiles_y * a.tiles_x / kWavesPerGroup);
@@ -665,7 +836,7 @@ WavePlan wave_plan(const MbconvParams &p)
     a.n_xpt = (a.ph * a.pw + 15) / 16;
     a.tiles_y = (p.out_h + a.th - 1) / a.th;
     wave_layout(a, &plan.lds);
-    if (plan.lds > 64 * 1024)
+    if (plan.lds > (a.rows_n > 0 ? 80 : 64) * 1024)
         return plan;
     a.fd_pw = make_fastdiv((unsigned)a.pw);
     a.fd_tiles_x = make_fastdiv((unsigned)a.tiles_x);
@@ -680,6 +851,16 @@ hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
 {
     WaveArgs a = plan.a;
     auto kernel = mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV, PACK, CLIP>;
+    if (plan.lds > 64 * 1024) {
+        static bool raised = false; // the dynamic LDS limit of a kernel is raised once per process
+        if (!raised) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+            if (e != hipSuccess)
+                return e;
+            raised = true;
+        }
+    }
     a.tpw = 1;
     if (ROWCONV) {
         // Tiles per wavefront: these tiles are short (two chunks of expanded channels for a 32-filter stem), so
@@ -733,7 +914,7 @@ bool launch_exact(const WavePlan &plan, hipStream_t stream, bool dry, hipError_t
     } while (0)
     if (!mbconv_expand_is_pointwise(a.p)) {
         // expand stage with a window: the stem + first block of MobileNetV2 at 224 x 224
-        if (a.n_xpt == 10 && a.pw == 16 && a.rt == 1 && a.th == 8 && s == 1)
+        if (a.n_xpt == 10 && a.pw == 16 && a.rt == 1 && a.th == 8 && s == 1 && a.rows_n > 0)
             ESPDL_WAVE_EXACT(10, 1, 8, 1, false, true);
         return false;
     }
