@@ -73,6 +73,7 @@ struct WaveArgs {
     int x_vec16, we_vec16;
     int off_exp, off_dw, off_tab;
     int off_aop; // ROWCONV: operand A of the expand stage for every expanded channel, [exp_c][4 rows][16 bytes]
+    int off_wd;  // ROWCONV: the depthwise weights as a lane wants them, [exp_c / 16][64 lanes][8 int32]
     int wave_bytes; // LDS of one wavefront (expanded patch + depthwise result); the tables are shared
     // ROWCONV guard-free builds: the image rows under the patch's windows, copied to the wavefront's LDS as
     // consecutive aligned 16-byte pieces (0: the plan has no room for them)
@@ -477,6 +478,15 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
         } else {
             w.aop[0] = load16_partial<VEC16>(p.w_expand, (unsigned)((ch0 + col) * c0 + 16 * quad), c0 - 16 * quad);
         }
+        if constexpr (ROWCONV) {
+            // (these builds walk several short tiles per wavefront: the weights come from the workgroup's LDS copy
+            // and a tile starts without a round trip to memory for them)
+            const v4i *wl = reinterpret_cast<const v4i *>(smem + a.off_wd + (sub * 64 + lane) * 32);
+            const v4i w0 = wl[0], w1 = wl[1];
+            w.wd0[0] = w0[0], w.wd0[1] = w0[1], w.wd0[2] = w0[2];
+            w.wd1[0] = w0[3], w.wd1[1] = w1[0], w.wd1[2] = w1[1];
+            return w;
+        }
         const unsigned wd = (unsigned)(ch0 + col);
 #pragma unroll
         for (int kx = 0; kx < 3; kx++) {
@@ -526,6 +536,26 @@ __global__ __launch_bounds__(64 * kWavesPerGroup, EXACT ? ((PACK > 1 && S == 2) 
                 w[j >> 2] |= ok ? v << (8 * (j & 3)) : 0;
             }
             *reinterpret_cast<v4i *>(smem + a.off_aop + i * 16) = v4i{w[0], w[1], w[2], 0};
+        }
+        // the depthwise weights of lane l for chunk `sub`: filter rows min(quad, 2) (none for quad 3) and, at
+        // stride 1, quad - 1 (none for quad 0) of channel 16 sub + col
+        for (int i = (int)threadIdx.x; i < (p.exp_c >> 4) * 64; i += 64 * kWavesPerGroup) {
+            const int l = i & 63, l_col = l & 15, l_quad = l >> 4;
+            const unsigned wd = (unsigned)(16 * (i >> 6) + l_col);
+            int w0[3], w1[3];
+#pragma unroll
+            for (int kx = 0; kx < 3; kx++) {
+                const int v0 = (int)p.w_dw[(size_t)(wd + (unsigned)((min(l_quad, 2) * 3 + kx) * p.exp_c))];
+                w0[kx] = l_quad < 3 ? v0 : 0;
+                w1[kx] = 0;
+                if constexpr (S == 1) {
+                    const int v1 = (int)p.w_dw[(size_t)(wd + (unsigned)((max(l_quad - 1, 0) * 3 + kx) * p.exp_c))];
+                    w1[kx] = l_quad >= 1 ? v1 : 0;
+                }
+            }
+            v4i *wl = reinterpret_cast<v4i *>(smem + a.off_wd + i * 32);
+            wl[0] = v4i{w0[0], w0[1], w0[2], w1[0]};
+            wl[1] = v4i{w1[1], w1[2], 0, 0};
         }
     }
 
@@ -728,7 +758,8 @@ void wave_layout(WaveArgs &a, size_t *lds)
     const int exp_px = std::max(((a.n_xpt + 3) & ~3) * 16, (a.ph * a.pw + 48 + 15) & ~15);
     a.off_tab = 0; // two stages x [init | rsh | lsh] x int32
     a.off_aop = a.p.exp_c * 24 + a.rt * 16 * 12 + kStageVoteBytes; // expand, depthwise and project tables, vote words
-    a.off_exp = a.off_aop + (mbconv_expand_is_pointwise(a.p) ? 0 : a.p.exp_c * 64);
+    a.off_wd = a.off_aop + (mbconv_expand_is_pointwise(a.p) ? 0 : a.p.exp_c * 64);
+    a.off_exp = a.off_wd + (mbconv_expand_is_pointwise(a.p) ? 0 : a.p.exp_c * 128);
     a.off_dw = a.off_exp + exp_px * 16;
     a.wave_bytes = exp_px * 16 + a.th * 16 * kDws;
     a.rows_n = a.rows_ppr = a.rows_rounds = a.off_rows = 0;
