@@ -992,6 +992,14 @@ ROWCONV_CASES = [
     ("stem_halfeven_50x50_rgb_s2", (2, 50, 50, 3), ((3, 3), (2, 2), (1, 1, 1, 1)), 32, 16, (1, 1), (1, 1, 1, 1), False, True),
     ("stem_nopad_21x21_rgb_s1_res", (2, 21, 21, 3), ((2, 3), (1, 1), (0, 0, 0, 0)), 32, 32, (1, 1), (1, 1, 1, 1), True, False),
     ("stem_tiny_5x5_rgb", (3, 5, 5, 3), ((3, 3), (2, 2), (1, 1, 1, 1)), 16, 4, (1, 1), (1, 1, 1, 1), False, False),
+    # at most 16 project filters at depthwise stride 1: the build that copies the image rows under a tile's windows
+    # into LDS one tile ahead (other channel counts, windows, strides, paddings and odd image sizes than the stem's)
+    ("rows_gray_40x44_s1_16_8", (2, 40, 44, 1), ((3, 3), (1, 1), (1, 1, 1, 1)), 16, 8, (1, 1), (1, 1, 1, 1), False, False),
+    ("rows_2ch_4x2window_50x37_res", (2, 50, 37, 2), ((4, 2), (2, 1), (1, 2, 0, 1)), 32, 16, (1, 1), (1, 1, 1, 1), True, False),
+    ("rows_nopad_67x61_rgb_s2_halfeven", (2, 67, 61, 3), ((3, 3), (2, 2), (0, 0, 0, 0)), 32, 16, (1, 1), (1, 1, 1, 1), False, True),
+    ("rows_4ch_3x2window_36x36", (1, 36, 36, 4), ((3, 2), (1, 1), (1, 1, 0, 1)), 48, 12, (1, 1), (1, 1, 1, 1), False, False),
+    ("rows_odd_image_bytes_33x35_rgb_s2", (5, 33, 35, 3), ((3, 3), (2, 2), (1, 1, 1, 1)), 32, 16, (1, 1), (1, 1, 1, 1), False, False),
+    ("rows_many_tiles_130x126_rgb_s2", (3, 130, 126, 3), ((3, 3), (2, 2), (1, 1, 1, 1)), 32, 16, (1, 1), (1, 1, 1, 1), False, False),
 ]
 
 
