@@ -46,6 +46,7 @@
 // expand product is the same code.  These tiles are short (two chunks for a 32-filter stem), so a wavefront
 // walks several consecutive tiles and the workgroup's set-up is paid once.
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -883,13 +884,21 @@ hipError_t launch_one(const WavePlan &plan, hipStream_t stream)
     WaveArgs a = plan.a;
     auto kernel = mbconv_s8_wave_kernel<NXPT, RT, PT, S, HE, VEC16, EXACT, ROWCONV, PACK, CLIP>;
     if (plan.lds > 64 * 1024) {
-        static bool raised = false; // the dynamic LDS limit of a kernel is raised once per process
-        if (!raised) {
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+        // the dynamic LDS limit of a kernel is raised once per device (bit d: done on device d; setting it twice
+        // from two threads does no harm)
+        static std::atomic<unsigned long long> raised{0};
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess)
+            return e;
+        const unsigned long long bit = 1ull << (dev & 63);
+        if (dev >= 64 || !(raised.load(std::memory_order_relaxed) & bit)) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    80 * 1024);
             if (e != hipSuccess)
                 return e;
-            raised = true;
+            if (dev < 64)
+                raised.fetch_or(bit, std::memory_order_relaxed);
         }
     }
     a.tpw = 1;
